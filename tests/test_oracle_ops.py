@@ -1,0 +1,218 @@
+"""Pins the oracle's memory and compute ops against numpy closed forms (strided views, float64
+matmul, libm) including ragged and out-of-bounds cases."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+
+def test_mk_sv_global_arithmetic(ko):
+    buf = np.zeros(1024, dtype=np.uint16)
+    g = ko.mk_global(buf, 16, 32, 32, 1, ko.F16, dynamic_offset=64)
+    assert g.ptr == buf.ctypes.data + 128 and (g.start0, g.start1, g.end0, g.end1) == (0, 0, 16, 32)
+    s = ko.sv_global(g, 2, 10, 4, 20)
+    assert (s.start0, s.end0, s.start1, s.end1) == (2, 10, 4, 20)
+    # second-level subview: both start and end are relative to the first subview's START
+    # (SvGlobalOpToLLVM.cpp:30-33)
+    t = ko.sv_global(s, 1, 3, 2, 6)
+    assert (t.start0, t.end0, t.start1, t.end1) == (3, 5, 6, 10)
+
+
+@pytest.mark.parametrize("pad", [0, 1, 2, 3])
+def test_ld_global_padding_and_ragged_edges(ko, pad):
+    src = np.arange(10 * 12, dtype=np.uint16).reshape(10, 12) + 1000
+    g = ko.sv_global(ko.mk_global(src, 10, 12, 12, 1, ko.F16), 6, 10, 8, 12)  # 4x4 view, loaded as an 8x8 tile
+    tile = np.zeros((8, 8), dtype=np.uint16)
+    ko.lib().ko_ld_global(C.byref(g), 8, 8, pad, tile.ctypes.data_as(C.c_void_p))
+    padv = {0: 0, 1: 0x7E00, 2: 0x7C00, 3: 0xFC00}[pad]
+    want = np.full((8, 8), padv, dtype=np.uint16)
+    want[:4, :4] = src[6:10, 8:12]
+    assert np.array_equal(tile, want)
+    # column-major view of the same buffer
+    gc = ko.mk_global(src, 12, 10, 1, 12, ko.F16)
+    tile2 = np.zeros((16, 16), dtype=np.uint16)
+    ko.lib().ko_ld_global(C.byref(gc), 16, 16, pad, tile2.ctypes.data_as(C.c_void_p))
+    want2 = np.full((16, 16), padv, dtype=np.uint16)
+    want2[:12, :10] = src.T
+    assert np.array_equal(tile2, want2)
+
+
+def test_st_global_masks_out_of_bounds(ko):
+    dst = np.full((6, 6), 0xAAAA, dtype=np.uint16)
+    g = ko.sv_global(ko.mk_global(dst, 6, 6, 6, 1, ko.BF16), 1, 4, 2, 5)
+    tile = np.arange(64, dtype=np.uint16).reshape(8, 8)
+    ko.lib().ko_st_global(tile.ctypes.data_as(C.c_void_p), 8, 8, C.byref(g))
+    want = np.full((6, 6), 0xAAAA, dtype=np.uint16)
+    want[1:4, 2:5] = tile[:3, :3]
+    assert np.array_equal(dst, want)
+
+
+@pytest.mark.parametrize("dtype,np_t", [(0, np.uint16), (2, np.float32), (3, np.uint8)])
+def test_copy_transpose_forms_agree(ko, dtype, np_t):
+    rng = np.random.default_rng(0)
+    m, n = 37, 53
+    src = rng.integers(0, 250, size=(m, n)).astype(np_t)
+    # (a) relabel: transpose flag; (b) swapped strides on the source descriptor
+    out_a = np.zeros((n, m), dtype=np_t)
+    out_b = np.zeros((n, m), dtype=np_t)
+    gs = ko.mk_global(src, m, n, n, 1, dtype)
+    assert ko.lib().ko_copy(C.byref(gs), C.byref(ko.mk_global(out_a, n, m, m, 1, dtype)), 1, 0) == 0
+    gs_t = ko.mk_global(src, n, m, 1, n, dtype)
+    assert ko.lib().ko_copy(C.byref(gs_t), C.byref(ko.mk_global(out_b, n, m, m, 1, dtype)), 0, 0) == 0
+    assert np.array_equal(out_a, src.T) and np.array_equal(out_b, src.T)
+    # involution
+    back = np.zeros((m, n), dtype=np_t)
+    ko.lib().ko_copy(C.byref(ko.mk_global(out_a, n, m, m, 1, dtype)), C.byref(ko.mk_global(back, m, n, n, 1, dtype)), 1, 0)
+    assert np.array_equal(back, src)
+
+
+def test_copy_batched_is_the_bhsd_permute(ko):
+    b, h, s, d = 2, 3, 8, 16
+    src = ko.fill_bits16(b * h * s * d, 1).reshape(b, h, s, d)
+    out = np.zeros((b, s, h, d), dtype=np.uint16)
+    gs = ko.mk_global(src, s, d, d, 1, ko.BF16)
+    gd = ko.mk_global(out, s, d, h * d, 1, ko.BF16)
+    rc = ko.lib().ko_copy_batched(C.byref(gs), C.byref(gd), 0, 0, b, h, h * s * d, s * d, s * h * d, d)
+    assert rc == 0 and np.array_equal(out, src.transpose(0, 2, 1, 3))
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+def test_matmul_vs_numpy_float64(ko, dt):
+    M, N, K = 48, 40, 72
+    a = ko.fill_uniform(M * K, dt, 0, 0).reshape(M, K)
+    b = ko.fill_uniform(K * N, dt, 0, 1).reshape(K, N)
+    acc = ko.fill_normal(M * N, ko.F32, 0, 2).reshape(M, N)
+    out = np.zeros((M, N), dtype=np.float32)
+    ga, gb = ko.mk_global(a, M, K, K, 1, dt), ko.mk_global(b, K, N, N, 1, dt)
+    gacc, go = ko.mk_global(acc, M, N, N, 1, ko.F32), ko.mk_global(out, M, N, N, 1, ko.F32)
+    assert ko.lib().ko_matmul(C.byref(ga), C.byref(gb), C.byref(gacc), C.byref(go), ko.RN) == 0
+    want = ko.decode(a, dt) @ ko.decode(b, dt) + acc.astype(np.float64)
+    assert np.array_equal(out, want.astype(np.float32))
+    # column-major rhs holds the same logical matrix
+    bt = np.ascontiguousarray(b.T)
+    out2 = np.zeros((M, N), dtype=np.float32)
+    gbt = ko.mk_global(bt, K, N, 1, K, dt)
+    ko.lib().ko_matmul(C.byref(ga), C.byref(gbt), C.byref(gacc), C.byref(ko.mk_global(out2, M, N, N, 1, ko.F32)), ko.RN)
+    assert np.array_equal(out, out2)
+
+
+def test_matmul_closed_forms(ko):
+    n = 32
+    eye = np.eye(n, dtype=np.float16).view(np.uint16)
+    b = ko.fill_uniform(n * n, ko.F16, 4).reshape(n, n)
+    out = np.zeros((n, n), dtype=np.uint16)
+    g = lambda x: ko.mk_global(x, n, n, n, 1, ko.F16)
+    assert ko.lib().ko_matmul(C.byref(g(eye)), C.byref(g(b)), None, C.byref(g(out)), ko.RN) == 0
+    assert np.array_equal(out, b)                        # I·B = B, bit for bit
+    ones = np.ones((n, n), dtype=np.float16).view(np.uint16)
+    ko.lib().ko_matmul(C.byref(g(ones)), C.byref(g(ones)), None, C.byref(g(out)), ko.RN)
+    assert np.all(out.view(np.float16) == n)             # all-ones -> K
+    # rank-1: (u v^T)(w x^T) = (v·w) u x^T
+    u = np.arange(1, n + 1, dtype=np.float16)
+    a1 = np.outer(u, np.ones(n, np.float16)).astype(np.float16).view(np.uint16)
+    b1 = np.outer(np.ones(n, np.float16), u).astype(np.float16).view(np.uint16)
+    outf = np.zeros((n, n), dtype=np.float32)
+    ko.lib().ko_matmul(C.byref(g(a1)), C.byref(g(b1)), None, C.byref(ko.mk_global(outf, n, n, n, 1, ko.F32)), ko.RN)
+    assert np.array_equal(outf, n * np.outer(u, u).astype(np.float32))
+
+
+def test_matmul_verifier_rules(ko):
+    z16 = np.zeros((16, 16), dtype=np.uint16)
+    g = lambda x, dt, m=16, n=16: ko.mk_global(x, m, n, n, 1, dt)
+    L = ko.lib()
+    assert L.ko_matmul(C.byref(g(z16, ko.F16, 16, 8)), C.byref(g(z16, ko.F16)), None, C.byref(g(z16, ko.F16)), 1) == -1
+    assert L.ko_matmul(C.byref(g(z16, ko.F16)), C.byref(g(z16, ko.BF16)), None, C.byref(g(z16, ko.F16)), 1) == -4
+    assert L.ko_matmul(C.byref(g(z16, ko.BF16)), C.byref(g(z16, ko.BF16)), C.byref(g(z16, ko.F16)),
+                       C.byref(g(z16, ko.F16)), 1) == -6
+    assert L.ko_matmul(C.byref(g(z16, ko.F16)), C.byref(g(z16, ko.F8E4M3)), None, C.byref(g(z16, ko.F16)), 1) == -3
+
+
+def test_scaled_f8_matmul_vs_numpy(ko):
+    M, N, K = 16, 24, 64
+    a = ko.fill_normal(M * K, ko.F32, 0, 0).reshape(M, K)
+    w = ko.fill_normal(K * N, ko.F32, 1, 0).reshape(K, N)
+    aq, sa = np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+    wq, sb = np.zeros((K, N), np.uint8), np.zeros(N, np.float32)
+    vp = lambda x: x.ctypes.data_as(C.c_void_p)
+    ko.lib().ko_quantize_e4m3(vp(a), M, K, K, 1, 1, vp(aq), vp(sa))
+    ko.lib().ko_quantize_e4m3(vp(w), K, N, N, 1, 0, vp(wq), vp(sb))
+    assert np.array_equal(sa, np.abs(a).max(axis=1) / np.float32(448))
+    assert np.array_equal(sb, np.abs(w).max(axis=0) / np.float32(448))
+    assert np.abs(ko.decode(aq, ko.F8E4M3)).max() == 448.0
+    out = np.zeros((M, N), dtype=np.uint16)
+    ga, gw = ko.mk_global(aq, M, K, K, 1, ko.F8E4M3), ko.mk_global(wq, K, N, N, 1, ko.F8E4M3)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ga), C.byref(gw), vp(sa), vp(sb),
+                                        C.byref(ko.mk_global(out, M, N, N, 1, ko.BF16))) == 0
+    exact = (ko.decode(aq, ko.F8E4M3) @ ko.decode(wq, ko.F8E4M3)) * np.outer(sa, sb).astype(np.float64)
+    import torch
+    want = torch.from_numpy(exact).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(out, want)
+    # dequantised product approximates the unquantised one
+    rel = np.linalg.norm(ko.decode(out, ko.BF16) - a.astype(np.float64) @ w) / np.linalg.norm(a.astype(np.float64) @ w)
+    assert rel < 0.06
+
+
+def test_elementwise_gelu_vs_numpy(ko):
+    M, N = 24, 40
+    x = ko.fill_normal(M * N, ko.F16, 0, 0).reshape(M, N)
+    x.ravel()[:6] = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 60000.0], dtype=np.float16).view(np.uint16)
+    bias = ko.fill_normal(N, ko.F16, 1, 0)
+    bias[:6] = 0
+    out = np.zeros((M, N), dtype=np.uint16)
+    gx, gb = ko.mk_global(x, M, N, N, 1, ko.F16), ko.mk_global(bias, 1, N, N, 1, ko.F16)
+    assert ko.elementwise(ko.gelu_program(), [gx, gb], ko.mk_global(out, M, N, N, 1, ko.F16)) == 0
+    v = (ko.decode(x, ko.F16).astype(np.float32) * np.float32(0.5)
+         + ko.decode(bias, ko.F16).astype(np.float32)[None, :]).astype(np.float64)
+    with np.errstate(all="ignore"):
+        y = (0.5 * v * (1 + np.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))).astype(np.float32)
+        want = y.astype(np.float16)
+    got = out.view(np.float16)
+    assert np.array_equal(np.isnan(want), np.isnan(got))
+    m = ~np.isnan(want)
+    assert np.array_equal(want[m], got[m])
+    assert got[0, 0] == 0 and np.isinf(got[0, 2]) and np.isnan(got[0, 3]) and np.isnan(got[0, 4])  # -inf*0 = NaN
+
+
+def test_elementwise_typed_rounding_and_rules(ko):
+    n = 4096
+    a = ko.fill_normal(n, ko.BF16, 2, 0).reshape(1, n)
+    b = ko.fill_normal(n, ko.BF16, 2, 1).reshape(1, n)
+    out = np.zeros((1, n), dtype=np.uint16)
+    g = lambda x: ko.mk_global(x, 1, n, n, 1, ko.BF16)
+    prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_LD_GLOBAL, dst=1, a=1),
+                       dict(op=ko.EW_MULF, dst=2, a=0, b=1), dict(op=ko.EW_ADDF, dst=2, a=2, b=0),
+                       dict(op=ko.EW_ST_GLOBAL, a=2)])
+    assert ko.elementwise(prog, [g(a), g(b)], g(out)) == 0
+    import torch
+    ta = torch.from_numpy(a.view(np.int16)).view(torch.bfloat16)
+    tb = torch.from_numpy(b.view(np.int16)).view(torch.bfloat16)
+    want = ((ta * tb) + ta).view(torch.int16).numpy().view(np.uint16)   # bf16 ops, one rounding each
+    assert np.array_equal(out, want)
+    # mismatched operand dtypes and a missing store are rejected
+    bad = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_SPLAT, dst=1, dtype=ko.F32, imm=1.0),
+                      dict(op=ko.EW_ADDF, dst=2, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=2)])
+    assert ko.elementwise(bad, [g(a)], g(out)) == -10
+    assert ko.elementwise(ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0)]), [g(a)], g(out)) == -13
+    # broadcast only from size-1 axes
+    half = ko.mk_global(a, 1, n // 2, n // 2, 1, ko.BF16)
+    assert ko.elementwise(ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_ST_GLOBAL, a=0)]),
+                          [half], g(out)) == -4
+
+
+def test_reduce_vs_numpy(ko):
+    x = ko.fill_normal(2 * 256, ko.F32, 5).reshape(2, 256)
+    out = np.zeros((2, 1), dtype=np.float32)
+    rc = ko.lib().ko_reduce(C.byref(ko.mk_global(x, 2, 256, 256, 1, ko.F32)),
+                            C.byref(ko.mk_global(out, 2, 1, 1, 2, ko.F32)), 1, 0)   # column-major 2x1 target
+    assert rc == 0 and np.array_equal(out.ravel(), x.astype(np.float64).sum(axis=1).astype(np.float32))
+
+
+def test_gemm_timing_baseline_agrees_with_checker(ko):
+    M = N = K = 96
+    a = ko.fill_uniform(M * K, ko.BF16, 0, 0).reshape(M, K)
+    bt = ko.fill_uniform(N * K, ko.BF16, 0, 1).reshape(N, K)
+    o1, o2 = np.zeros((M, N), np.float32), np.zeros((M, N), np.float32)
+    ga, gb = ko.mk_global(a, M, K, K, 1, ko.BF16), ko.mk_global(bt, K, N, 1, K, ko.BF16)
+    ko.lib().ko_matmul(C.byref(ga), C.byref(gb), None, C.byref(ko.mk_global(o1, M, N, N, 1, ko.F32)), ko.RN)
+    ko.lib().ko_gemm_f32acc(C.byref(ga), C.byref(gb), C.byref(ko.mk_global(o2, M, N, N, 1, ko.F32)))
+    assert np.linalg.norm(o1 - o2) / np.linalg.norm(o1) < 1e-5

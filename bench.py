@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the kapy hot path on one MI355X.
+
+`python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]`
+
+A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM.
+The headline workload (BASELINE.json configs[1]) is the fused elementwise
+y = GELU_tanh(x*0.5 + bias) on fp16 8192x8192; the JSON line also carries every other BASELINE
+configuration under "other_workloads", each with its own roofline.  One JSON line on stdout.
+
+Timing: K launches bracketed by torch.cuda.synchronize() give ms_per_step / value; HIP events
+recorded on the stream the kernels are launched on (torch's current stream, whose handle is
+passed to the C ABI) give the per-launch duration used for roofline.achieved.  Memory-bound
+workloads rotate over buffer sets larger than the 256 MB Infinity Cache so the rate is HBM's.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "kapy-lang_amd", "python"))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f8": 5000.0}
+
+
+def _events(fn, steps, warmup):
+    """Run fn(i) warmup + steps times; return (wall ms per step, event ms per launch)."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return wall_ms, start.elapsed_time(end) / steps
+
+
+def _roof_hbm(bytes_per_launch, ev_ms):
+    a = bytes_per_launch / (ev_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(a, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(a / HBM_PEAK_GBS, 4),
+            "traffic": None}
+
+
+def _roof_mfma(flops, ev_ms, kind):
+    a = flops / (ev_ms * 1e-3) / 1e12
+    p = MFMA_PEAK_TFLOPS[kind]
+    return {"bound": "mfma", "achieved": round(a, 1), "peak": p, "unit": "TFLOP/s", "frac": round(a / p, 4), "traffic": None}
+
+
+def bench_gelu(kh, steps, warmup):
+    import torch
+    n, sets = 8192, 4
+    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    ys = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    bias = torch.randn(n, device="cuda", dtype=torch.float16)
+    prog = kh.gelu_program(kh.F16, 0.5)
+    gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
+    gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
+    gb = kh.mk_global(bias.data_ptr(), 1, n, n, 1, kh.F16)
+    wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gb], gy[i % sets]), steps, warmup)
+    nbytes = 2 * n * n * 2 + n * 2
+    return {"workload": "C2 gelu_tanh(x*0.5+bias) fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "affine_act_kernel"}
+
+
+def bench_transpose(kh, steps, warmup):
+    import torch
+    n, sets = 8192, 4
+    xs = [torch.randint(-32768, 32767, (n, n), device="cuda", dtype=torch.int16) for _ in range(sets)]
+    ys = [torch.empty(n, n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
+    gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
+    wall, ev = _events(lambda i: kh.copy(gx[i % sets], gy[i % sets], transpose=True), steps, warmup)
+    nbytes = 2 * n * n * 2
+    return {"workload": "C3a transpose fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
+            "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "transpose_kernel"}
+
+
+def bench_permute(kh, steps, warmup):
+    import torch
+    b, h, s, d, sets = 8, 32, 2048, 128, 4
+    xs = [torch.randint(-32768, 32767, (b * h * s * d,), device="cuda", dtype=torch.int16) for _ in range(sets)]
+    ys = [torch.empty(b * h * s * d, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    gx = [kh.mk_global(x.data_ptr(), s, d, d, 1, kh.BF16) for x in xs]
+    gy = [kh.mk_global(y.data_ptr(), s, d, h * d, 1, kh.BF16) for y in ys]
+    grid = (b, h, h * s * d, s * d, s * h * d, d)
+    wall, ev = _events(lambda i: kh.copy_batched(gx[i % sets], gy[i % sets], grid), steps, warmup)
+    nbytes = 2 * b * h * s * d * 2
+    return {"workload": "C3b permute bf16 [8,32,2048,128] bhsd->bshd", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
+
+
+def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel):
+    import torch
+    tdt = torch.bfloat16 if dtype == kh.BF16 else torch.float16
+    std = 0.02 if dtype == kh.BF16 else 0.5
+    a = (torch.randn(M, K, device="cuda") * std).to(tdt)
+    b = (torch.randn(N, K, device="cuda") * std).to(tdt) if b_col_major else (torch.randn(K, N, device="cuda") * std).to(tdt)
+    d = torch.empty(M, N, device="cuda", dtype=tdt)
+    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, dtype)
+    gb = kh.mk_global(b.data_ptr(), K, N, 1, K, dtype) if b_col_major else kh.mk_global(b.data_ptr(), K, N, N, 1, dtype)
+    gd = kh.mk_global(d.data_ptr(), M, N, N, 1, dtype)
+    wall, ev = _events(lambda i: kh.matmul(ga, gb, gd), steps, warmup)
+    flops = 2.0 * M * N * K
+    kind = "bf16" if dtype == kh.BF16 else "f16"
+    return {"workload": name, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "kernel_ms": ev,
+            "dtype": kind, "roofline": _roof_mfma(flops, ev, kind), "kernel": kernel}
+
+
+def bench_f8(kh, steps, warmup, M):
+    import torch
+    N = K = 8192
+    a = torch.randint(0, 120, (M, K), device="cuda", dtype=torch.uint8)      # finite e4m3 patterns
+    w = torch.randint(0, 120, (N, K), device="cuda", dtype=torch.uint8)
+    sa = torch.rand(M, device="cuda") * 0.01 + 0.001
+    sb = torch.rand(N, device="cuda") * 0.01 + 0.001
+    d = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, kh.F8E4M3)
+    gw = kh.mk_global(w.data_ptr(), K, N, 1, K, kh.F8E4M3)
+    gd = kh.mk_global(d.data_ptr(), M, N, N, 1, kh.BF16)
+    wall, ev = _events(lambda i: kh.matmul_scaled_f8(ga, gw, sa.data_ptr(), sb.data_ptr(), gd), steps, warmup)
+    flops = 2.0 * M * N * K
+    nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
+    out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192" % M, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_kernel"}
+    out["roofline"] = _roof_hbm(nbytes, ev) if M <= 64 else _roof_mfma(flops, ev, "f8")
+    return out
+
+
+def cpu_baseline_gelu(sample_rows=256):
+    """The oracle's elementwise program on a bounded sample (sample_rows x 8192) of the same workload,
+    on this box's host cores.  Reported, never the optimisation target."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import ko
+    n = 8192
+    x = ko.fill_normal(sample_rows * n, ko.F16, 0, 0).reshape(sample_rows, n)
+    bias = ko.fill_normal(n, ko.F16, 1, 0)
+    out = np.zeros((sample_rows, n), dtype=np.uint16)
+    prog = ko.gelu_program()
+    gx, gb, go = ko.mk_global(x, sample_rows, n, n, 1, ko.F16), ko.mk_global(bias, 1, n, n, 1, ko.F16), ko.mk_global(out, sample_rows, n, n, 1, ko.F16)
+    ko.elementwise(prog, [gx, gb], go)  # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ko.elementwise(prog, [gx, gb], go)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or reps >= 50:
+            break
+    nbytes = (2 * sample_rows * n * 2 + n * 2) * reps
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": ko.lib().ko_num_threads(), "kind": "port",
+            "sample": "%d of 8192 rows of the same workload, %d repetitions, %.1f s" % (sample_rows, reps, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (every path here runs on a single MI355X)" % args.gpus)
+    import torch
+    import kapy_hip as kh
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the library has no CPU fallback to time")
+    torch.cuda.set_device(0)
+    kh.lib()
+    table = {
+        "gelu": lambda s, w: bench_gelu(kh, s, w),
+        "transpose": lambda s, w: bench_transpose(kh, s, w),
+        "permute": lambda s, w: bench_permute(kh, s, w),
+        "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
+        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "staged_kernel"),
+        "f8_m16": lambda s, w: bench_f8(kh, s, w, 16),
+        "f8_m4096": lambda s, w: bench_f8(kh, s, w, 4096),
+    }
+    main_res = table[args.workload](args.steps, args.warmup)
+    others = []
+    if not args.no_others:
+        for name, fn in table.items():
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            r = fn(min(args.steps, 20), min(args.warmup, 5))
+            r["value"] = round(r["value"], 2)
+            r["ms_per_step"] = round(r["ms_per_step"], 4)
+            r["kernel_ms"] = round(r["kernel_ms"], 4)
+            others.append(r)
+    line = {
+        "metric": "GEMM TFLOP/s + % MFMA peak; elementwise/transpose GB/s + % HBM peak (1 GPU)",
+        "value": round(main_res["value"], 2), "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(main_res["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_res["dtype"], "data": "synthetic",
+        "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "kernel_ms": round(main_res["kernel_ms"], 4),
+                   "buffers": "4 rotating sets (1 GiB) so reads miss the Infinity Cache" if main_res["unit"] == "GB/s" else "single set"},
+        "roofline": main_res["roofline"],
+        "cpu_baseline": None if args.no_cpu else cpu_baseline_gelu(),
+        "other_workloads": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

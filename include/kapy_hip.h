@@ -1,0 +1,218 @@
+/*
+ * kapy_hip.h — C ABI of the MI355X (gfx950) implementation of kapy-lang's hot op path.
+ *
+ * kapy-lang is a compiler: it has no FFI of its own.  The boundary kept here is its op-level
+ * surface — the op builders of python/src/ir.cc:480-1181 and the kernel ABI that
+ * lib/Conversion/KgpuToLLVM/FuncOpToLLVM.cpp:55-92 produces (global pointers + i32 scalars, one
+ * stream-ordered launch) — at whole-tensor granularity: one call runs the op over the full
+ * extent of its descriptors instead of over one warp tile, and the library chooses the tiling.
+ * Every entry point cites the reference interface it stands in for.
+ *
+ * Conventions: plain C types only; all pointers in descriptors are DEVICE pointers owned by the
+ * caller (the reference never allocates global memory either); device entry points are
+ * asynchronous on the given HIP stream (a hipStream_t passed as void*, NULL = default stream);
+ * every function returns KAPY_OK or a negative kapy_status and never throws; the text of the
+ * last failure on the calling thread is available from kapy_last_error().  There is no CPU
+ * fallback: device entry points fail with KAPY_ERR_HIP when no gfx950 device is usable.
+ */
+#ifndef KAPY_HIP_H
+#define KAPY_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum kapy_status {
+  KAPY_OK = 0,
+  KAPY_ERR_INVALID = -1,     /* null pointer, unknown enum value, malformed program            */
+  KAPY_ERR_VERIFY = -2,      /* an op verifier of the reference rejects the operands           */
+  KAPY_ERR_UNSUPPORTED = -3, /* legal in kapy, not implemented on this device                  */
+  KAPY_ERR_HIP = -4          /* HIP runtime failure (including "no device")                    */
+} kapy_status;
+
+/* Element types of Kapy tensors (include/kapy/Dialect/Kapy/IR/Types.td; f8 = OCP E4M3FN / E5M2). */
+typedef enum kapy_dtype {
+  KAPY_F16 = 0, KAPY_BF16 = 1, KAPY_F32 = 2, KAPY_F8E4M3 = 3, KAPY_F8E5M2 = 4,
+  KAPY_I8 = 5, KAPY_I16 = 6, KAPY_I32 = 7
+} kapy_dtype;
+
+/* Enum values equal include/kapy/Dialect/Kapy/IR/Enums.td (python/src/ir.cc:125-156). */
+typedef enum kapy_padding_option { KAPY_PAD_ZERO = 0, KAPY_PAD_QNAN = 1, KAPY_PAD_PINF = 2, KAPY_PAD_NINF = 3 } kapy_padding_option;
+typedef enum kapy_cache_modifier {
+  KAPY_CACHE_NONE = 0, KAPY_CACHE_CA = 1, KAPY_CACHE_CG = 2, KAPY_CACHE_CS = 3,
+  KAPY_CACHE_WB = 4, KAPY_CACHE_WT = 5, KAPY_CACHE_LU = 6, KAPY_CACHE_CV = 7
+} kapy_cache_modifier;
+typedef enum kapy_rounding_mode { KAPY_RZ = 0, KAPY_RN = 1 } kapy_rounding_mode;
+/* MatmulImplWay: values 1..4 are the reference's (mma.sync shapes); on gfx950 they only select the
+ * operand class (f16/bf16, tf32 — unsupported: CDNA4 has no tf32 MFMA —, f8).  0 lets the library
+ * choose; 16..18 name the MFMA shape explicitly. */
+typedef enum kapy_matmul_impl_way {
+  KAPY_MATMUL_AUTO = 0,
+  KAPY_MMA_M16N8K8_F16 = 1, KAPY_MMA_M16N8K16_F16 = 2, KAPY_MMA_M16N8K8_TF32 = 3, KAPY_MMA_M16N8K16_F8 = 4,
+  KAPY_MFMA_32X32X16_16B = 16, KAPY_MFMA_16X16X32_16B = 17, KAPY_MFMA_16X16X128_F8 = 18, KAPY_MFMA_32X32X64_F8 = 19
+} kapy_matmul_impl_way;
+
+/* Global-memory tensor descriptor: the struct of lib/Conversion/KgpuToLLVM/TypeConverter.cpp:65-73
+ * {ptr, start0, start1, end0, end1, stride0, stride1} plus the element type and the kapy.alignment
+ * attribute (bytes) that the reference carries on the IR.  Element (i,j) of the view lives at
+ * ptr + ((start0+i)*stride0 + (start1+j)*stride1) elements and is in bounds iff
+ * (start0+i) <u end0 && (start1+j) <u end1. */
+typedef struct kapy_global {
+  void *ptr;
+  int32_t start0, start1, end0, end1, stride0, stride1;
+  int32_t dtype;     /* kapy_dtype */
+  int32_t alignment; /* bytes the base pointer and every row start are aligned to */
+} kapy_global;
+
+/* #kgpu.fragments<[a0,a1],[l0,l1],(minor,major)> (include/kapy/Dialect/Kgpu/IR/Attrs.td:12-135).
+ * The lane count is a0*a1: 64 on gfx950 (32 in the reference). */
+typedef struct kapy_fragments {
+  int32_t lane_array[2];
+  int32_t lane_loops[2];
+  int32_t minor_axis, major_axis;
+} kapy_fragments;
+
+/* #kapy.swizzling<[stride0,stride1],(bank_param,line_param)> (include/kapy/Dialect/Kapy/IR/Attrs.td:54-81). */
+typedef struct kapy_swizzling {
+  int32_t stride0, stride1, bank_param, line_param;
+} kapy_swizzling;
+
+/* ---------------------------------------------------------------- library */
+int kapy_version(void);
+/* Text of the last error on this thread; mirrors the reference's emitOpError messages. */
+const char *kapy_last_error(void);
+/* Device facts used for dispatch: CU count, wavefront size, LDS bytes per workgroup, arch name. */
+int kapy_device_info(int32_t *num_cus, int32_t *wave_size, int32_t *lds_bytes, char *arch, int32_t arch_len);
+
+/* ---------------------------------------------------------------- descriptors (host only) */
+/* kapy.mk_global — create_mk_global, python/src/ir.cc:1013-1025; MkGlobalOpToLLVM.cpp:23-47. */
+int kapy_mk_global(kapy_global *out, void *ptr, int32_t dynamic_offset, int32_t size0, int32_t size1,
+                   int32_t stride0, int32_t stride1, int32_t dtype, int32_t alignment);
+/* kapy.sv_global — create_sv_global(src, start0, end0, start1, end1), python/src/ir.cc:1026-1034;
+ * SvGlobalOpToLLVM.cpp:22-40: both new bounds are offsets from the source view's start. */
+int kapy_sv_global(kapy_global *out, const kapy_global *src, int32_t start0, int32_t end0, int32_t start1, int32_t end1);
+
+/* ---------------------------------------------------------------- layout engine (host only) */
+/* FragmentsLayoutAttr::getWarpLoops / getLoopSpace — lib/Dialect/Kgpu/IR/Kgpu.cpp:164-184. */
+int kapy_fragments_loops(const kapy_fragments *layout, const int64_t shape[2], int64_t warp_loops[2], int64_t loop_space[2]);
+/* FragmentsLayoutAttr::getAffineMap(shape, option) — Kgpu.cpp:186-251.  option 1/2: in = (lane, iv),
+ * out = (i0, i1); option 3: in = (i0, i1), out = (lane, iv). */
+int kapy_fragments_map(const kapy_fragments *layout, const int64_t shape[2], int32_t option, const int64_t in[2], int64_t out[2]);
+/* FragmentsLayoutAttr::transpose / exchangeAxes — Kgpu.cpp:253-263. */
+int kapy_fragments_transpose(const kapy_fragments *layout, kapy_fragments *out);
+int kapy_fragments_exchange_axes(const kapy_fragments *layout, kapy_fragments *out);
+/* getFragmentsLayout(laneLoops, type, rowMajor) — lib/Support/LayoutUtils.cpp:92-104, 64 lanes. */
+int kapy_fragments_default(const int64_t lane_loops[2], const int64_t shape[2], int32_t row_major, kapy_fragments *out);
+/* getGlobalSimdSize — lib/Dialect/Kgpu/Transforms/CoalesceAccess.cpp:18-27, 64 lanes. */
+int64_t kapy_access_simd_size(int64_t alignment, int64_t bits, int64_t numel);
+/* ChangeOpHelper::getShflIdxMap / getNumShfls — LayoutUtils.cpp:61-90. */
+int kapy_change_source(const kapy_fragments *src, const kapy_fragments *dst, const int64_t shape[2], int64_t lane,
+                       int64_t iv, int64_t *src_lane, int64_t *src_iv);
+int64_t kapy_change_num_shuffles(const kapy_fragments *src, const kapy_fragments *dst, const int64_t shape[2]);
+/* Swizzled element offset — CpAsyncOpToLLVM.cpp:124-139 (same in LdMatrix/LdShared/StShared), for
+ * the 64-bank x 4-byte LDS of gfx950 (a line is 256 bytes). */
+int64_t kapy_swizzle_offset(const kapy_swizzling *layout, int64_t bits, int64_t i0, int64_t i1);
+/* getSwizzlingLayouts — LayoutUtils.cpp:167-225 re-parameterised for 64 banks and 64 lanes: writes
+ * up to max_pairs (bank_param, line_param) candidates in the reference's search order, returns the count. */
+int kapy_swizzle_search(const kapy_fragments *access, const int64_t shape[2], int64_t stride0, int64_t stride1,
+                        int64_t bits, int64_t alignment, int32_t *pairs, int32_t max_pairs);
+/* getDefaultLayouts(MatmulOp) — LayoutUtils.cpp:123-149 for the MFMA shapes of gfx950:
+ * which = 0 lhs, 1 rhs, 2 acc; also reports the MFMA tile (m, n, k). */
+int kapy_matmul_layouts(int32_t impl_way, int32_t which, kapy_fragments *out, int32_t mnk[3]);
+/* The LDS layout the tiled matmul stages its operands in (result of kapy_swizzle_search on the
+ * MFMA operand layout), so callers and tests can check it is conflict-free by construction. */
+int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out);
+
+/* ---------------------------------------------------------------- device ops */
+typedef struct kapy_copy_cfg {
+  int32_t transpose;      /* 1: kapy.transpose between the load and the store (dst[i,j] = src[j,i]) */
+  int32_t padding_option; /* kapy_padding_option of the ld_global                                   */
+  int32_t cache_modifier; /* kapy_cache_modifier; CS / CG select non-temporal access                */
+  int32_t reserved;
+} kapy_copy_cfg;
+
+/* ld_global -> [transpose] -> st_global over the destination view's full extent.
+ * Stands in for create_ld_global / create_transpose / create_st_global, python/src/ir.cc:1035-1049,
+ * 1087-1090 (LdGlobalOpToLLVM.cpp:60-145, TransposeOpToLLVM.cpp:21-26, StGlobalOpToLLVM.cpp:60-139).
+ * Source elements out of bounds read as padding; destination elements out of bounds are not written.
+ * Element types must have equal width; bits move untouched. cfg may be NULL (no transpose, zero padding). */
+int kapy_copy(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, void *stream);
+
+/* A 2-D grid of programs (kapy.program_id axes 0 and 1, ParallelIdOpToLLVM.cpp:28-38), program (p0,p1)
+ * running kapy_copy on views displaced by p0*off0 + p1*off1 ELEMENTS, i.e. mk_global's dynamic_offset
+ * affine in the program ids.  (b,h,s,d)->(b,s,h,d) is grid (b,h) over [s x d] views. */
+typedef struct kapy_grid2 {
+  int32_t n0, n1;
+  int64_t src_off0, src_off1, dst_off0, dst_off1;
+} kapy_grid2;
+int kapy_copy_batched(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, const kapy_grid2 *grid, void *stream);
+
+/* Elementwise programs: a straight-line list of kapy/arith/math ops over at most 16 virtual
+ * registers, evaluated for every element of `out`'s extent (create_{addf,mulf,fma,exp,...},
+ * create_fptofp, create_splat, create_broadcast, python/src/ir.cc:744-1157; lowering
+ * ElementwiseOpToLLVM.cpp:424-1238).  A register has a dtype; arithmetic on f16/bf16/f32 registers
+ * rounds once to that dtype after every op.  LD_GLOBAL of an input whose extent is 1 along an axis
+ * broadcasts along it (kapy.broadcast, Kapy.cpp:686-698). */
+typedef enum kapy_ew_op {
+  KAPY_EW_LD_GLOBAL = 0, /* dst <- ins[a]            (c = kapy_padding_option)                  */
+  KAPY_EW_SPLAT,         /* dst <- imm as `dtype`    (kapy.splat)                               */
+  KAPY_EW_FPTOFP,        /* dst <- cast(a) to `dtype`, `rmode` on down-casts (kapy.fptofp/extf/truncf) */
+  KAPY_EW_ADDF, KAPY_EW_SUBF, KAPY_EW_MULF, KAPY_EW_DIVF,
+  KAPY_EW_FMA,           /* dst <- a*b + c                                                     */
+  KAPY_EW_MAXIMUMF, KAPY_EW_MINIMUMF, KAPY_EW_NEGF, KAPY_EW_ABSF,
+  KAPY_EW_EXP, KAPY_EW_EXP2, KAPY_EW_LOG, KAPY_EW_LOG2, KAPY_EW_SQRT, KAPY_EW_RSQRT,
+  KAPY_EW_TANH, KAPY_EW_ERF, /* the extern-lib calls of create_elementwise_extern_lib, ir.cc:1168-1174 */
+  KAPY_EW_GELU_TANH,     /* dst <- 0.5*a*(1+tanh(sqrt(2/pi)*(a+0.044715*a^3))), one rounding       */
+  KAPY_EW_ST_GLOBAL,     /* out <- a                                                              */
+  KAPY_EW_NUM_OPS
+} kapy_ew_op;
+typedef struct kapy_ew_inst {
+  int32_t op, dst, a, b, c;
+  int32_t dtype, rmode;
+  float imm;
+} kapy_ew_inst;
+int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
+                     const kapy_global *out, void *stream);
+
+/* kapy.fptofp over whole tensors (create_fptofp, python/src/ir.cc:744-754; verifier
+ * lib/Dialect/Kapy/IR/Kapy.cpp:272-287): dst[i,j] = cast(src[i,j]), rounding per `rmode`. */
+int kapy_fptofp(const kapy_global *src, const kapy_global *dst, int32_t rmode, void *stream);
+
+typedef struct kapy_matmul_cfg {
+  int32_t impl_way;              /* kapy_matmul_impl_way                                         */
+  int32_t tile_m, tile_n, tile_k; /* workgroup tile; 0 = library's choice                          */
+  int32_t rmode;                 /* rounding of the final cast to result dtype (default RN)      */
+  int32_t reserved[3];
+} kapy_matmul_cfg;
+
+/* kapy.matmul — create_matmul(lhs, rhs, acc, implWay), python/src/ir.cc:1101-1105; verifier
+ * lib/Dialect/Kapy/IR/Kapy.cpp:451-574; lowering MatmulOpToLLVM.cpp:58-311 with the
+ * cp_async/ld_matrix pipeline of CpAsyncOpToLLVM.cpp and LdMatrixOpToLLVM.cpp.
+ * result[M,N] = lhs[M,K]·rhs[K,N] (+ acc[M,N]), fp32 accumulate, one final cast to result->dtype.
+ * Operand layouts come from the descriptor strides (row- or column-major, either operand).
+ * acc may be NULL (zero).  cfg may be NULL. */
+int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
+                const kapy_matmul_cfg *cfg, void *stream);
+
+/* W8A8: result[m,n] = cast( (sum_k a8[m,k]·w8[k,n]) · row_scale[m] · col_scale[n] ).
+ * In kapy terms: matmul (mma f8, f32 acc) -> mulf with broadcast(row_scale [Mx1]) and
+ * broadcast(col_scale [1xN]) -> fptofp rn.  Scales are dense fp32 device arrays. */
+int kapy_matmul_scaled_f8(const kapy_global *a8, const kapy_global *w8, const float *row_scale, const float *col_scale,
+                          const kapy_global *result, const kapy_matmul_cfg *cfg, void *stream);
+
+/* kgpu.change on one wavefront's registers (lib/Conversion/KgpuToLLVM/ChangeOpToLLVM.cpp:21-93):
+ * lane_values_in[lane*n_src + iv] under `src` is re-distributed to lane_values_out[lane*n_dst + iv]
+ * under `dst`, 32-bit values, moved with wave64 ds_bpermute shuffles.  n_* = loop-space sizes. */
+int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const kapy_fragments *dst,
+                const int64_t shape[2], uint32_t *lane_values_out, void *stream);
+
+/* kapy.reduce with an addf / maximumf combiner along `axis` (Ops.td:441-457, ReduceOpToLLVM.cpp:51-172).
+ * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`. */
+int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KAPY_HIP_H */

@@ -1,0 +1,62 @@
+// common.hpp — shared host-side helpers of the library: error reporting, descriptor arithmetic,
+// HIP call checking.  No device code here.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/kapy_hip.h"
+
+namespace kapy {
+
+// Thread-local text of the last failure; the counterpart of the reference's emitOpError
+// diagnostics (e.g. lib/Dialect/Kapy/IR/Kapy.cpp:272-287).
+char *last_error_buffer();
+int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define KAPY_HIP_CHECK(expr)                                                                   \
+  do {                                                                                         \
+    hipError_t e_ = (expr);                                                                    \
+    if (e_ != hipSuccess) return ::kapy::fail(KAPY_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+inline int dtype_bytes(int32_t dtype) {
+  switch (dtype) {
+  case KAPY_F16: case KAPY_BF16: case KAPY_I16: return 2;
+  case KAPY_F32: case KAPY_I32: return 4;
+  case KAPY_F8E4M3: case KAPY_F8E5M2: case KAPY_I8: return 1;
+  }
+  return 0;
+}
+inline bool is_float(int32_t d) { return d == KAPY_F16 || d == KAPY_BF16 || d == KAPY_F32 || d == KAPY_F8E4M3 || d == KAPY_F8E5M2; }
+inline bool is_f8(int32_t d) { return d == KAPY_F8E4M3 || d == KAPY_F8E5M2; }
+inline const char *dtype_name(int32_t d) {
+  static const char *names[] = {"f16", "bf16", "f32", "f8E4M3", "f8E5M2", "i8", "i16", "i32"};
+  return d >= 0 && d < 8 ? names[d] : "?";
+}
+
+inline int64_t extent0(const kapy_global *g) { return int64_t(g->end0) - g->start0; }
+inline int64_t extent1(const kapy_global *g) { return int64_t(g->end1) - g->start1; }
+// Address (in elements, relative to g->ptr) of view element (0,0).
+inline int64_t origin(const kapy_global *g) { return int64_t(g->start0) * g->stride0 + int64_t(g->start1) * g->stride1; }
+inline const char *view_base(const kapy_global *g) { return (const char *)g->ptr + origin(g) * dtype_bytes(g->dtype); }
+
+// Largest power-of-two byte count (<= 16) that divides the address of every row/column start of
+// the view: what a vector access along the contiguous axis may assume.
+inline int vector_bytes(const kapy_global *g, int contiguous_axis) {
+  int b = dtype_bytes(g->dtype);
+  uint64_t bits = (uint64_t)(uintptr_t)view_base(g);
+  int64_t pitch = (contiguous_axis == 1 ? int64_t(g->stride0) : int64_t(g->stride1)) * b;
+  int64_t rows = contiguous_axis == 1 ? extent0(g) : extent1(g);
+  if (rows > 1) bits |= (uint64_t)(pitch < 0 ? -pitch : pitch);
+  int v = 16;
+  while (v > b && (bits & (uint64_t)(v - 1))) v >>= 1;
+  return v;
+}
+
+int check_global(const kapy_global *g, const char *what);
+int ensure_device();
+int device_cus();
+
+}  // namespace kapy

@@ -1,0 +1,328 @@
+// copy.hip — ld_global -> [transpose] -> st_global over whole views: the affine-map-described
+// layout moves of kapy (strided copies, (i,j)->(j,i) transposes, batched permutes).
+//
+// Reference semantics: LdGlobalOpToLLVM.cpp:60-145 (addressing, unsigned-compare predicate,
+// padding pre-initialisation), StGlobalOpToLLVM.cpp:60-139, TransposeOpToLLVM.cpp:21-26 (a
+// transpose is a relabel of the register layout: values never pass through an FP unit), and the
+// lane re-distribution of ChangeOpToLLVM.cpp:43-78 for the in-register transpose.
+//
+// Three kernels, chosen from the descriptor strides:
+//   rows_kernel       source and destination contiguous along the same axis: 16-byte vectors,
+//                     consecutive lanes on consecutive vectors, every byte read and written once.
+//   transpose_kernel  contiguous axes differ: a wavefront owns a (8V x 8V) tile (V = elements per
+//                     16 bytes).  Each lane loads a V x V block as V 16-byte vectors along the
+//                     source's contiguous axis, transposes it in registers, then the 8x8 grid of
+//                     lanes is itself transposed with ds_bpermute so that consecutive lanes again
+//                     hold consecutive 16-byte vectors for the store.  Both sides of HBM see full
+//                     128-byte segments; no LDS allocation, no barrier.
+//   generic_kernel    anything else (no contiguous axis, misaligned rows): one element per lane.
+#include "common.hpp"
+
+namespace kapy {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// All quantities are in the destination's index space (i over d0, j over d1) after the host has
+// folded the transpose flag into the source strides; strides are in elements.
+struct CopyParams {
+  const char *src;
+  char *dst;
+  int64_t es0, es1;  // source element strides along i and j
+  int64_t ds0, ds1;  // destination element strides
+  int32_t d0, d1;    // destination extent: elements outside are not written
+  int32_t sb0, sb1;  // source bounds: elements at i >= sb0 or j >= sb1 read as padding
+  uint32_t pad;      // 32-bit padding word (element pattern replicated)
+  int32_t n1;        // second grid dimension; program (p0,p1) = (z / n1, z % n1)
+  int64_t s_off0, s_off1, d_off0, d_off1;  // per-program displacement in elements
+};
+
+template <int B> struct ElemOf;
+template <> struct ElemOf<1> { typedef uint8_t type; };
+template <> struct ElemOf<2> { typedef uint16_t type; };
+template <> struct ElemOf<4> { typedef uint32_t type; };
+
+template <int B>
+__device__ __forceinline__ void program_base(const CopyParams &p, const char *&src, char *&dst) {
+  int32_t z = blockIdx.z, p0 = z / p.n1, p1 = z - p0 * p.n1;
+  src = p.src + (p0 * p.s_off0 + p1 * p.s_off1) * B;
+  dst = p.dst + (p0 * p.d_off0 + p1 * p.d_off1) * B;
+}
+
+template <int B>
+__device__ __forceinline__ void copy_one(const CopyParams &p, const char *src, char *dst, int32_t i, int32_t j) {
+  typedef typename ElemOf<B>::type T;
+  if (i >= p.d0 || j >= p.d1) return;
+  T v = (T)p.pad;
+  if (i < p.sb0 && j < p.sb1) v = *(const T *)(src + (i * p.es0 + j * p.es1) * B);
+  *(T *)(dst + (i * p.ds0 + j * p.ds1) * B) = v;
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int B>
+__global__ __launch_bounds__(256) void generic_kernel(CopyParams p, int j_fastest) {
+  const char *src;
+  char *dst;
+  program_base<B>(p, src, dst);
+  int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  int64_t total = (int64_t)p.d0 * p.d1;
+  if (t >= total) return;
+  int32_t i, j;
+  if (j_fastest) { i = (int32_t)(t / p.d1); j = (int32_t)(t - (int64_t)i * p.d1); }
+  else { j = (int32_t)(t / p.d0); i = (int32_t)(t - (int64_t)j * p.d0); }
+  copy_one<B>(p, src, dst, i, j);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rows: es1 == ds1 == 1.  A slot is one VB-byte vector of one row; a thread serves UNROLL slots a
+// block-stride apart, all loads issued before the first store.
+template <int VB> struct VecOf;
+template <> struct VecOf<16> { typedef u32x4 type; };
+template <> struct VecOf<8> { typedef u32x2 type; };
+template <> struct VecOf<4> { typedef uint32_t type; };
+
+template <int B, int VB, bool NT, bool RAGGED>
+__global__ __launch_bounds__(256) void rows_kernel(CopyParams p, int32_t vec_per_row) {
+  typedef typename VecOf<VB>::type Vec;
+  constexpr int E = VB / B;  // elements per vector
+  constexpr int UNROLL = 4;
+  const char *src;
+  char *dst;
+  program_base<B>(p, src, dst);
+  const uint32_t total = (uint32_t)p.d0 * (uint32_t)vec_per_row;  // the host keeps this below 2^31
+  const uint32_t first = blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  Vec v[UNROLL];
+  int32_t row[UNROLL], col[UNROLL];
+  bool whole[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    uint32_t slot = first + u * 256;
+    row[u] = -1;
+    whole[u] = false;
+    if (slot < total) {
+      row[u] = (int32_t)(slot / (uint32_t)vec_per_row);
+      col[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)vec_per_row) * E;
+      whole[u] = !RAGGED || (row[u] < p.sb0 && col[u] + E <= p.sb1 && col[u] + E <= p.d1);
+      if (whole[u]) {
+        const Vec *s = (const Vec *)(src + ((int64_t)row[u] * p.es0 + col[u]) * B);
+        v[u] = NT ? __builtin_nontemporal_load(s) : *s;
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    if (row[u] < 0) continue;
+    if (whole[u]) {
+      Vec *d = (Vec *)(dst + ((int64_t)row[u] * p.ds0 + col[u]) * B);
+      if (NT) __builtin_nontemporal_store(v[u], d);
+      else *d = v[u];
+    } else {
+#pragma unroll 1
+      for (int e = 0; e < E; ++e) copy_one<B>(p, src, dst, row[u], col[u] + e);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Transpose: es0 == 1 (source contiguous along i) and ds1 == 1 (destination contiguous along j).
+template <int B, bool NT>
+__global__ __launch_bounds__(256) void transpose_kernel(CopyParams p) {
+  typedef typename ElemOf<B>::type T;
+  constexpr int V = 16 / B;  // lane block is V x V elements
+  constexpr int TILE = 8 * V;
+  const char *src;
+  char *dst;
+  program_base<B>(p, src, dst);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int32_t ti = (blockIdx.x * 2 + (wave & 1)) * TILE;
+  const int32_t tj = (blockIdx.y * 2 + (wave >> 1)) * TILE;
+  if (ti >= p.d0 || tj >= p.d1) return;
+  const bool interior = ti + TILE <= p.d0 && ti + TILE <= p.sb0 && tj + TILE <= p.d1 && tj + TILE <= p.sb1;
+  if (!interior) {  // ragged edge: element-wise with the ld/st predicates
+    for (int e = lane; e < TILE * TILE; e += 64) copy_one<B>(p, src, dst, ti + e / TILE, tj + e % TILE);
+    return;
+  }
+  const int la = lane & 7, lb = lane >> 3;
+  union Block {
+    u32x4 vec[V];
+    T el[V][V];
+  };
+  Block in, out;
+  const char *s = src + ((int64_t)(ti + V * la) + (int64_t)(tj + V * lb) * p.es1) * B;
+#pragma unroll
+  for (int c = 0; c < V; ++c) {
+    const u32x4 *ptr = (const u32x4 *)(s + (int64_t)c * p.es1 * B);
+    in.vec[c] = NT ? __builtin_nontemporal_load(ptr) : *ptr;
+  }
+  // in.el[c][r] = S(i = ti + V*la + r, j = tj + V*lb + c)  ->  out.el[r][c]
+#pragma unroll
+  for (int r = 0; r < V; ++r)
+#pragma unroll
+    for (int c = 0; c < V; ++c) out.el[r][c] = in.el[c][r];
+  // Transpose the 8x8 grid of lanes: lane (la', lb') takes the block of lane (la = lb', lb = la'),
+  // i.e. the registers of source lane lb' ... the same permutation kgpu.change would derive for
+  // <[8,8],[V,V],(0,1)> -> <[8,8],[V,V],(1,0)> on the transposed tile.
+  const int from = (la << 3) | lb;
+#pragma unroll
+  for (int r = 0; r < V; ++r)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) out.vec[r][w] = (uint32_t)__builtin_amdgcn_ds_bpermute(from << 2, (int)out.vec[r][w]);
+  // now this lane holds rows i = ti + V*lb + r, columns tj + V*la .. + V-1
+  char *d = dst + ((int64_t)(ti + V * lb) * p.ds0 + (int64_t)(tj + V * la)) * B;
+#pragma unroll
+  for (int r = 0; r < V; ++r) {
+    u32x4 *ptr = (u32x4 *)(d + (int64_t)r * p.ds0 * B);
+    if (NT) __builtin_nontemporal_store(out.vec[r], ptr);
+    else *ptr = out.vec[r];
+  }
+}
+
+uint32_t padding_word(int32_t dtype, int32_t padding) {
+  // ConvertUtils.cpp:267-334; e4m3 is OCP E4M3FN here (no infinities): +-inf -> +-448, qnan -> 0x7F.
+  static const uint32_t f32[4] = {0, 0x7FC00000u, 0x7F800000u, 0xFF800000u};
+  static const uint32_t f16[4] = {0, 0x7E007E00u, 0x7C007C00u, 0xFC00FC00u};
+  static const uint32_t bf16[4] = {0, 0x7FC07FC0u, 0x7F807F80u, 0xFF80FF80u};
+  static const uint32_t e4m3[4] = {0, 0x7F7F7F7Fu, 0x7E7E7E7Eu, 0xFEFEFEFEu};
+  static const uint32_t e5m2[4] = {0, 0x7E7E7E7Eu, 0x7C7C7C7Cu, 0xFCFCFCFCu};
+  switch (dtype) {
+  case KAPY_F32: return f32[padding];
+  case KAPY_F16: return f16[padding];
+  case KAPY_BF16: return bf16[padding];
+  case KAPY_F8E4M3: return e4m3[padding];
+  case KAPY_F8E5M2: return e5m2[padding];
+  }
+  return 0;
+}
+
+template <int B>
+int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch, hipStream_t stream) {
+  CopyParams p = p0;
+  if (p.d0 <= 0 || p.d1 <= 0 || batch <= 0) return KAPY_OK;
+  // Make "destination contiguous along j" the canonical orientation.
+  if (p.ds1 != 1 && p.ds0 == 1) {
+    std::swap(p.es0, p.es1);
+    std::swap(p.ds0, p.ds1);
+    std::swap(p.d0, p.d1);
+    std::swap(p.sb0, p.sb1);
+  }
+  if (batch > 65535) return fail(KAPY_ERR_UNSUPPORTED, "copy: more than 65535 programs in one launch");
+  if (p.ds1 == 1 && p.es1 == 1) {
+    int vb = std::min(vb_src, vb_dst);
+    int64_t slots_at_vb = (int64_t)p.d0 * ((p.d1 + vb / B - 1) / (vb / B));
+    if (vb >= 4 && slots_at_vb < (int64_t(1) << 31) - 1024) {
+      int e = vb / B;
+      int32_t vpr = (p.d1 + e - 1) / e;
+      int64_t slots = slots_at_vb;
+      dim3 grid((unsigned)((slots + 1023) / 1024), 1, (unsigned)batch);
+      // no ragged vector anywhere: every slot is a whole in-bounds vector on both sides
+      bool ragged = p.d1 % e != 0 || p.sb1 < p.d1 || p.sb0 < p.d0;
+      if (vb == 16 && !ragged) {
+        if (nt) rows_kernel<B, 16, true, false><<<grid, 256, 0, stream>>>(p, vpr);
+        else rows_kernel<B, 16, false, false><<<grid, 256, 0, stream>>>(p, vpr);
+      } else if (vb == 16) {
+        rows_kernel<B, 16, false, true><<<grid, 256, 0, stream>>>(p, vpr);
+      } else if (vb == 8) {
+        rows_kernel<B, 8, false, true><<<grid, 256, 0, stream>>>(p, vpr);
+      } else {
+        rows_kernel<B, 4, false, true><<<grid, 256, 0, stream>>>(p, vpr);
+      }
+      KAPY_HIP_CHECK(hipGetLastError());
+      return KAPY_OK;
+    }
+  } else if (p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16) {
+    constexpr int TILE = 8 * (16 / B);
+    unsigned gx = (unsigned)((p.d0 + 2 * TILE - 1) / (2 * TILE)), gy = (unsigned)((p.d1 + 2 * TILE - 1) / (2 * TILE));
+    if (gy <= 65535) {
+      dim3 grid(gx, gy, (unsigned)batch);
+      if (nt) transpose_kernel<B, true><<<grid, 256, 0, stream>>>(p);
+      else transpose_kernel<B, false><<<grid, 256, 0, stream>>>(p);
+      KAPY_HIP_CHECK(hipGetLastError());
+      return KAPY_OK;
+    }
+  }
+  int64_t total = (int64_t)p.d0 * p.d1;
+  int j_fastest = p.ds1 <= p.ds0;
+  dim3 grid((unsigned)((total + 255) / 256), 1, (unsigned)batch);
+  generic_kernel<B><<<grid, 256, 0, stream>>>(p, j_fastest);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
+int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, const kapy_grid2 *grid, void *stream) {
+  int rc = check_global(src, "copy source");
+  if (!rc) rc = check_global(dst, "copy target");
+  if (rc) return rc;
+  int B = dtype_bytes(src->dtype);
+  // st_global carries SameOperandsElementType (Ops.td:163-170); a move only needs equal widths, so
+  // re-typed views of the same bits (f16 <-> i16 ...) are let through.
+  if (B != dtype_bytes(dst->dtype))
+    return fail(KAPY_ERR_VERIFY, "copy: source (%s) and target (%s) must have the same element width", dtype_name(src->dtype),
+                dtype_name(dst->dtype));
+  kapy_copy_cfg c = {0, KAPY_PAD_ZERO, KAPY_CACHE_NONE, 0};
+  if (cfg) c = *cfg;
+  if (c.padding_option < 0 || c.padding_option > 3) return fail(KAPY_ERR_INVALID, "copy: unknown padding option %d", c.padding_option);
+  if (c.padding_option != KAPY_PAD_ZERO && !is_float(src->dtype))
+    return fail(KAPY_ERR_VERIFY, "copy: integer tensors only take zero padding");
+  if (src->start0 < 0 || src->start1 < 0 || dst->start0 < 0 || dst->start1 < 0)
+    return fail(KAPY_ERR_INVALID, "copy: negative view start");
+  kapy_grid2 g = {1, 1, 0, 0, 0, 0};
+  if (grid) g = *grid;
+  if (g.n0 < 0 || g.n1 < 0) return fail(KAPY_ERR_INVALID, "copy: negative grid size");
+  rc = ensure_device();
+  if (rc) return rc;
+
+  CopyParams p;
+  p.src = view_base(src);
+  p.dst = (char *)view_base(dst);
+  bool t = c.transpose != 0;
+  p.es0 = t ? src->stride1 : src->stride0;
+  p.es1 = t ? src->stride0 : src->stride1;
+  p.ds0 = dst->stride0;
+  p.ds1 = dst->stride1;
+  p.d0 = (int32_t)extent0(dst);
+  p.d1 = (int32_t)extent1(dst);
+  p.sb0 = (int32_t)(t ? extent1(src) : extent0(src));
+  p.sb1 = (int32_t)(t ? extent0(src) : extent1(src));
+  p.pad = padding_word(src->dtype, c.padding_option);
+  p.n1 = g.n1 > 0 ? g.n1 : 1;
+  p.s_off0 = g.src_off0;
+  p.s_off1 = g.src_off1;
+  p.d_off0 = g.dst_off0;
+  p.d_off1 = g.dst_off1;
+  // vector width each side may use along its contiguous axis, also honouring the batch displacements
+  auto side_vb = [&](const kapy_global *v, int64_t o0, int64_t o1) {
+    int axis = v->stride1 == 1 ? 1 : (v->stride0 == 1 ? 0 : -1);
+    if (axis < 0) return B;
+    int vb = vector_bytes(v, axis);
+    uint64_t bits = (uint64_t)((o0 < 0 ? -o0 : o0) * B) | (uint64_t)((o1 < 0 ? -o1 : o1) * B);
+    while (vb > B && (bits & (uint64_t)(vb - 1))) vb >>= 1;
+    return vb;
+  };
+  int vb_src = side_vb(src, g.n0 > 1 ? g.src_off0 : 0, g.n1 > 1 ? g.src_off1 : 0);
+  int vb_dst = side_vb(dst, g.n0 > 1 ? g.dst_off0 : 0, g.n1 > 1 ? g.dst_off1 : 0);
+  bool nt = c.cache_modifier == KAPY_CACHE_CS || c.cache_modifier == KAPY_CACHE_CG;
+  int32_t batch = g.n0 * g.n1;
+  hipStream_t s = (hipStream_t)stream;
+  switch (B) {
+  case 1: return launch<1>(p, vb_src, vb_dst, nt, batch, s);
+  case 2: return launch<2>(p, vb_src, vb_dst, nt, batch, s);
+  default: return launch<4>(p, vb_src, vb_dst, nt, batch, s);
+  }
+}
+
+}  // namespace
+}  // namespace kapy
+
+extern "C" {
+
+int kapy_copy(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, void *stream) {
+  return kapy::copy_impl(src, dst, cfg, nullptr, stream);
+}
+
+int kapy_copy_batched(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, const kapy_grid2 *grid, void *stream) {
+  if (!grid) return kapy::fail(KAPY_ERR_INVALID, "copy_batched: null grid");
+  return kapy::copy_impl(src, dst, cfg, grid, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,511 @@
+// elementwise.hip — fused elementwise programs over whole views.
+//
+// Reference: the per-lane, per-element application of arith/math ops by
+// lib/Conversion/KgpuToLLVM/ElementwiseOpToLLVM.cpp (generic conversion :424-534, fptofp
+// :536-661, bf16 single-rounding arithmetic :771-892, exp :1039-1073, extern-lib calls
+// :1100-1166) fed by ld_global / broadcast / splat and drained by st_global.  In the reference
+// a fused chain is one straight-line kernel body; here the host recognises the common chain
+//     out = cast( act( x * splat(scale) + bias ) )
+// and runs it in one pass with 16-byte accesses (affine_act_kernel); any other program runs on a
+// small register machine (interpreter_kernel) whose register file lives in LDS.
+#include <math.h>
+#include <string.h>
+
+#include <vector>
+
+#include "common.hpp"
+#include "numeric.hpp"
+
+namespace kapy {
+namespace {
+
+constexpr int kMaxRegs = 16;
+constexpr int kMaxInst = 48;
+constexpr int kMaxInputs = 8;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct DevView {
+  const char *base;  // address of view element (0,0)
+  int64_t stride0, stride1;
+  int32_t ext0, ext1;
+  int32_t dtype;
+  uint32_t pad;
+};
+
+struct Program {
+  kapy_ew_inst inst[kMaxInst];
+  int32_t n_inst;
+  int32_t n_ins;
+  DevView in[kMaxInputs];
+  DevView out;
+};
+
+// 0.5*v*(1+tanh(sqrt(2/pi)*(v+0.044715*v^3))) == v * sigmoid(2u): no cancellation for v << 0.
+__device__ __forceinline__ float gelu_tanh_f32(float v) {
+  float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+  return v / (1.0f + __expf(-2.0f * u));
+}
+
+__device__ __forceinline__ float apply_unary(int op, float a) {
+  switch (op) {
+  case KAPY_EW_NEGF: return -a;
+  case KAPY_EW_ABSF: return fabsf(a);
+  case KAPY_EW_EXP: return expf(a);
+  case KAPY_EW_EXP2: return exp2f(a);
+  case KAPY_EW_LOG: return logf(a);
+  case KAPY_EW_LOG2: return log2f(a);
+  case KAPY_EW_SQRT: return sqrtf(a);
+  case KAPY_EW_RSQRT: return 1.0f / sqrtf(a);
+  case KAPY_EW_TANH: return tanhf(a);
+  case KAPY_EW_ERF: return erff(a);
+  case KAPY_EW_GELU_TANH: return gelu_tanh_f32(a);
+  }
+  return a;
+}
+
+// arith.maximumf / minimumf: NaN if either operand is NaN.
+__device__ __forceinline__ float max_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ __forceinline__ float min_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+
+// ---------------------------------------------------------------------------------------------
+// Register machine: one output element per lane per pass; register r of lane t is regs[r][t], so
+// every access is conflict-free.  Values are fp32 images of the register's dtype.
+__global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_fastest) {
+  __shared__ float regs[kMaxRegs][256];
+  const int tid = threadIdx.x;
+  const int64_t total = (int64_t)P.out.ext0 * P.out.ext1;
+  const int64_t t = (int64_t)blockIdx.x * 256 + tid;
+  const bool active = t < total;
+  int32_t i = 0, j = 0;
+  if (active) {
+    if (j_fastest) { i = (int32_t)(t / P.out.ext1); j = (int32_t)(t - (int64_t)i * P.out.ext1); }
+    else { j = (int32_t)(t / P.out.ext0); i = (int32_t)(t - (int64_t)j * P.out.ext0); }
+  }
+  // The host has written every instruction's result dtype into I.dtype.
+  for (int k = 0; k < P.n_inst; ++k) {
+    const kapy_ew_inst I = P.inst[k];
+    float r = 0.f;
+    const int dt = I.dtype;
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: {
+      const DevView &g = P.in[I.a];
+      int32_t gi = g.ext0 == 1 ? 0 : i, gj = g.ext1 == 1 ? 0 : j;
+      if (active && gi < g.ext0 && gj < g.ext1) r = load_as_f32(g.base, g.dtype, gi * g.stride0 + gj * g.stride1);
+      else {
+        uint32_t w = I.c == KAPY_PAD_ZERO ? 0u : g.pad;
+        r = load_as_f32(&w, g.dtype, 0);
+      }
+      break;
+    }
+    case KAPY_EW_SPLAT:
+      r = round_to_dtype(I.imm, dt, true);
+      break;
+    case KAPY_EW_FPTOFP:
+      r = round_to_dtype(regs[I.a][tid], dt, I.rmode != KAPY_RZ);
+      break;
+    case KAPY_EW_ST_GLOBAL:
+      if (active) store_from_f32((void *)P.out.base, P.out.dtype, i * P.out.stride0 + j * P.out.stride1, regs[I.a][tid]);
+      continue;
+    default: {
+      const float a = regs[I.a][tid];
+      switch (I.op) {
+      case KAPY_EW_ADDF: r = __fadd_rn(a, regs[I.b][tid]); break;
+      case KAPY_EW_SUBF: r = __fsub_rn(a, regs[I.b][tid]); break;
+      case KAPY_EW_MULF: r = __fmul_rn(a, regs[I.b][tid]); break;
+      case KAPY_EW_DIVF: r = __fdiv_rn(a, regs[I.b][tid]); break;
+      case KAPY_EW_FMA: r = __fmaf_rn(a, regs[I.b][tid], regs[I.c][tid]); break;
+      case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
+      case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
+      default: r = apply_unary(I.op, a);
+      }
+      if (dt != KAPY_F32) r = round_to_dtype(r, dt, true);
+    }
+    }
+    regs[I.dst][tid] = r;  // regs[*][tid] is private to the lane: no barrier needed
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[i,j] = cast_out( act( f32(x[i,j]) * scale + f32(bias) ) ), x/out contiguous along j.
+enum BiasMode { kNoBias = 0, kBiasRow = 1 /* bias[0,j] */, kBiasCol = 2 /* bias[i,0] */, kBiasFull = 3 };
+
+struct AffineActParams {
+  const char *x, *bias;
+  char *out;
+  int64_t x_stride0, out_stride0, bias_stride0;  // elements
+  int32_t rows, vec_per_row;
+  int32_t has_scale, bias_mode, act;  // act: a unary kapy_ew_op, or -1
+  float scale;
+};
+
+template <typename T> struct Codec;
+template <> struct Codec<_Float16> {
+  static __device__ __forceinline__ float up(uint16_t h) { return f16_to_f32(h); }
+  static __device__ __forceinline__ uint16_t down(float v) { return f32_to_f16_rn(v); }
+};
+struct Bf16Tag {};
+template <> struct Codec<Bf16Tag> {
+  static __device__ __forceinline__ float up(uint16_t h) { return bf16_to_f32(h); }
+  static __device__ __forceinline__ uint16_t down(float v) { return f32_to_bf16_rn(v); }
+};
+
+template <typename T>
+__device__ __forceinline__ void unpack8(u32x4 v, float f[8]) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    f[2 * w] = Codec<T>::up((uint16_t)(v[w] & 0xFFFFu));
+    f[2 * w + 1] = Codec<T>::up((uint16_t)(v[w] >> 16));
+  }
+}
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float f[8]) {
+  u32x4 v;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) v[w] = (uint32_t)Codec<T>::down(f[2 * w]) | ((uint32_t)Codec<T>::down(f[2 * w + 1]) << 16);
+  return v;
+}
+
+// 16-bit in, 16-bit out (same type), 8 elements per 16-byte vector, UNROLL vectors per lane.
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
+  constexpr int UNROLL = 4;
+  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;
+  const uint32_t first = blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  u32x4 xv[UNROLL], bv[UNROLL];
+  int32_t row[UNROLL], col[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    uint32_t slot = first + u * 256;
+    row[u] = -1;
+    if (slot < total) {
+      row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);
+      col[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row) * 8;
+      xv[u] = __builtin_nontemporal_load((const u32x4 *)(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2));
+      if (p.bias_mode == kBiasRow) bv[u] = *(const u32x4 *)(p.bias + (int64_t)col[u] * 2);
+      else if (p.bias_mode == kBiasFull) bv[u] = *(const u32x4 *)(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2);
+      else if (p.bias_mode == kBiasCol) {
+        uint32_t h = *(const uint16_t *)(p.bias + (int64_t)row[u] * p.bias_stride0 * 2);
+        h |= h << 16;
+        bv[u] = u32x4{h, h, h, h};
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    if (row[u] < 0) continue;
+    float f[8], b[8];
+    unpack8<T>(xv[u], f);
+    if (p.bias_mode != kNoBias) unpack8<T>(bv[u], b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float v = f[e];
+      if (p.has_scale) v = __fmul_rn(v, p.scale);
+      if (p.bias_mode != kNoBias) v = __fadd_rn(v, b[e]);
+      if (ACT == KAPY_EW_GELU_TANH) v = gelu_tanh_f32(v);
+      else if (ACT >= 0) v = apply_unary(p.act, v);
+      f[e] = v;
+    }
+    __builtin_nontemporal_store(pack8<T>(f), (u32x4 *)(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side: verification (the op verifiers of the reference), pattern matching, launch.
+struct Node {
+  int kind;  // kapy_ew_op
+  int a = -1, b = -1, c = -1;
+  int dtype = -1, rmode = KAPY_RN, input = -1;
+  float imm = 0.f;
+};
+
+int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                   int result_dtype[kMaxInst]) {
+  if (!prog || n_inst <= 0) return fail(KAPY_ERR_INVALID, "elementwise: empty program");
+  if (n_inst > kMaxInst) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: more than %d instructions", kMaxInst);
+  if (n_ins < 0 || n_ins > kMaxInputs) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: more than %d inputs", kMaxInputs);
+  int rc = check_global(out, "elementwise result");
+  if (rc) return rc;
+  for (int k = 0; k < n_ins; ++k) {
+    if (!ins || (rc = check_global(ins[k], "elementwise operand"))) return rc ? rc : fail(KAPY_ERR_INVALID, "elementwise: null operand list");
+    if (ins[k]->start0 < 0 || ins[k]->start1 < 0) return fail(KAPY_ERR_INVALID, "elementwise: negative view start");
+  }
+  if (out->start0 < 0 || out->start1 < 0) return fail(KAPY_ERR_INVALID, "elementwise: negative view start");
+  int reg_dtype[kMaxRegs];
+  for (int r = 0; r < kMaxRegs; ++r) reg_dtype[r] = -1;
+  const int64_t o0 = extent0(out), o1 = extent1(out);
+  bool has_store = false;
+  auto reg_ok = [&](int r) { return r >= 0 && r < kMaxRegs && reg_dtype[r] >= 0; };
+  for (int k = 0; k < n_inst; ++k) {
+    const kapy_ew_inst &I = prog[k];
+    if (I.op < 0 || I.op >= KAPY_EW_NUM_OPS) return fail(KAPY_ERR_INVALID, "elementwise: unknown op %d at %d", I.op, k);
+    if (I.op != KAPY_EW_ST_GLOBAL && (I.dst < 0 || I.dst >= kMaxRegs))
+      return fail(KAPY_ERR_INVALID, "elementwise: result register out of range at %d", k);
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: {
+      if (I.a < 0 || I.a >= n_ins) return fail(KAPY_ERR_INVALID, "elementwise: ld_global of unknown operand at %d", k);
+      if (I.c < 0 || I.c > 3) return fail(KAPY_ERR_INVALID, "elementwise: unknown padding option at %d", k);
+      int64_t e0 = extent0(ins[I.a]), e1 = extent1(ins[I.a]);
+      if ((e0 != o0 && e0 != 1) || (e1 != o1 && e1 != 1))
+        return fail(KAPY_ERR_VERIFY, "broadcast: source shape must be 1 on the axes it is broadcast along");
+      reg_dtype[I.dst] = ins[I.a]->dtype;
+      break;
+    }
+    case KAPY_EW_SPLAT:
+      if (I.dtype != KAPY_F16 && I.dtype != KAPY_BF16 && I.dtype != KAPY_F32)
+        return fail(KAPY_ERR_VERIFY, "splat: only f16, bf16 and f32 splats are supported");
+      reg_dtype[I.dst] = I.dtype;
+      break;
+    case KAPY_EW_FPTOFP: {
+      if (!reg_ok(I.a)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      int sd = reg_dtype[I.a], dd = I.dtype;
+      if (!is_float(sd) || !is_float(dd)) return fail(KAPY_ERR_VERIFY, "fptofp: operands must have float element type");
+      bool down = dtype_bytes(dd) < dtype_bytes(sd);
+      if (down && I.rmode != KAPY_RN && I.rmode != KAPY_RZ) return fail(KAPY_ERR_VERIFY, "fptofp: rounding mode is required for down cast");
+      if (sd == KAPY_BF16 && is_f8(dd) && I.rmode == KAPY_RZ)
+        return fail(KAPY_ERR_VERIFY, "fptofp: unsupported rounding mode when convert bf16 to f8");
+      if (is_f8(sd) && is_f8(dd)) return fail(KAPY_ERR_VERIFY, "fptofp: convert f8 to f8 is not supported");
+      reg_dtype[I.dst] = dd;
+      break;
+    }
+    case KAPY_EW_FMA:
+      if (!reg_ok(I.a) || !reg_ok(I.b) || !reg_ok(I.c)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      if (reg_dtype[I.a] != reg_dtype[I.b] || reg_dtype[I.a] != reg_dtype[I.c])
+        return fail(KAPY_ERR_VERIFY, "elementwise: operands must have the same element type at %d", k);
+      reg_dtype[I.dst] = reg_dtype[I.a];
+      break;
+    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+      if (!reg_ok(I.a) || !reg_ok(I.b)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      if (reg_dtype[I.a] != reg_dtype[I.b])
+        return fail(KAPY_ERR_VERIFY, "elementwise: operands must have the same element type at %d", k);
+      reg_dtype[I.dst] = reg_dtype[I.a];
+      break;
+    case KAPY_EW_ST_GLOBAL:
+      if (!reg_ok(I.a)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      if (reg_dtype[I.a] != out->dtype) return fail(KAPY_ERR_VERIFY, "st_global: source and target must have the same element type");
+      has_store = true;
+      break;
+    default:
+      if (!reg_ok(I.a)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      reg_dtype[I.dst] = reg_dtype[I.a];
+    }
+    if (result_dtype) result_dtype[k] = I.op == KAPY_EW_ST_GLOBAL ? out->dtype : reg_dtype[I.dst];
+    if (I.op != KAPY_EW_ST_GLOBAL && I.op != KAPY_EW_LD_GLOBAL && I.op != KAPY_EW_FPTOFP) {
+      int d = reg_dtype[I.dst];
+      if (d != KAPY_F16 && d != KAPY_BF16 && d != KAPY_F32)
+        return fail(KAPY_ERR_VERIFY, "elementwise: arithmetic needs f16, bf16 or f32 operands at %d", k);
+    }
+  }
+  if (!has_store) return fail(KAPY_ERR_INVALID, "elementwise: program has no st_global");
+  return KAPY_OK;
+}
+
+uint32_t padding_word_of(int32_t dtype, int32_t padding);
+
+// Symbolic evaluation into a DAG, then a structural match of
+//   st( fptofp_rn[T]( act?( addf( mulf(extf(ld x), splat s), extf(ld bias) ) ) ) )   (operands in either order;
+//   the scale and the bias optional; fma(x, s, bias) is NOT matched: it rounds once, mulf+addf twice).
+bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *const *ins, const kapy_global *out,
+                      AffineActParams *p, int *elem_dtype) {
+  std::vector<Node> nodes;
+  int reg[kMaxRegs];
+  for (int r = 0; r < kMaxRegs; ++r) reg[r] = -1;
+  int stored = -1, n_store = 0;
+  for (int k = 0; k < n_inst; ++k) {
+    const kapy_ew_inst &I = prog[k];
+    Node n;
+    n.kind = I.op;
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: n.input = I.a; if (I.c != KAPY_PAD_ZERO) return false; break;
+    case KAPY_EW_SPLAT: n.imm = I.imm; n.dtype = I.dtype; break;
+    case KAPY_EW_FPTOFP: n.a = reg[I.a]; n.dtype = I.dtype; n.rmode = I.rmode; break;
+    case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; ++n_store; continue;
+    case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
+    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+      n.a = reg[I.a]; n.b = reg[I.b]; break;
+    default: n.a = reg[I.a];
+    }
+    nodes.push_back(n);
+    reg[I.dst] = (int)nodes.size() - 1;
+  }
+  if (n_store != 1 || stored < 0) return false;
+  const int T = out->dtype;
+  if (T != KAPY_F16 && T != KAPY_BF16) return false;
+  auto is_kind = [&](int id, int kind) { return id >= 0 && nodes[id].kind == kind; };
+  // x: extf(ld in) with in of the output's type and full extent
+  auto as_input_f32 = [&](int id) -> int {
+    if (!is_kind(id, KAPY_EW_FPTOFP) || nodes[id].dtype != KAPY_F32) return -1;
+    int s = nodes[id].a;
+    return is_kind(s, KAPY_EW_LD_GLOBAL) ? nodes[s].input : -1;
+  };
+  auto as_splat_f32 = [&](int id, float *v) {
+    if (!is_kind(id, KAPY_EW_SPLAT) || nodes[id].dtype != KAPY_F32) return false;
+    *v = nodes[id].imm;
+    return true;
+  };
+  int cur = stored;
+  if (!is_kind(cur, KAPY_EW_FPTOFP) || nodes[cur].dtype != T || nodes[cur].rmode != KAPY_RN) return false;
+  cur = nodes[cur].a;
+  if (cur < 0) return false;
+  p->act = -1;
+  int k = nodes[cur].kind;
+  if (k >= KAPY_EW_NEGF && k <= KAPY_EW_GELU_TANH) {
+    p->act = k;
+    cur = nodes[cur].a;
+    if (cur < 0) return false;
+  }
+  int x_in = -1, bias_in = -1;
+  p->has_scale = 0;
+  p->scale = 1.f;
+  auto match_scaled = [&](int id) -> int {  // mulf(x, s) | mulf(s, x) | x
+    if (is_kind(id, KAPY_EW_MULF)) {
+      float s;
+      int xa = as_input_f32(nodes[id].a), xb = as_input_f32(nodes[id].b);
+      if (xa >= 0 && as_splat_f32(nodes[id].b, &s)) { p->has_scale = 1; p->scale = s; return xa; }
+      if (xb >= 0 && as_splat_f32(nodes[id].a, &s)) { p->has_scale = 1; p->scale = s; return xb; }
+      return -1;
+    }
+    return as_input_f32(id);
+  };
+  if (is_kind(cur, KAPY_EW_ADDF)) {
+    int l = nodes[cur].a, r = nodes[cur].b;
+    int xl = match_scaled(l);
+    if (xl >= 0 && as_input_f32(r) >= 0) { x_in = xl; bias_in = as_input_f32(r); }
+    else {
+      p->has_scale = 0;
+      int xr = match_scaled(r);
+      if (xr >= 0 && as_input_f32(l) >= 0) { x_in = xr; bias_in = as_input_f32(l); }
+      else return false;
+    }
+  } else {
+    x_in = match_scaled(cur);
+    if (x_in < 0) return false;
+  }
+  const kapy_global *x = ins[x_in];
+  if (x->dtype != T || x->stride1 != 1 || out->stride1 != 1) return false;
+  const int64_t o0 = extent0(out), o1 = extent1(out);
+  if (extent0(x) != o0 || extent1(x) != o1 || o1 % 8 != 0) return false;
+  if (vector_bytes(x, 1) != 16 || vector_bytes(out, 1) != 16) return false;
+  if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  p->bias_mode = kNoBias;
+  p->bias = nullptr;
+  p->bias_stride0 = 0;
+  if (bias_in >= 0) {
+    const kapy_global *b = ins[bias_in];
+    if (b->dtype != T) return false;
+    int64_t b0 = extent0(b), b1 = extent1(b);
+    if (b1 == o1 && b->stride1 == 1 && vector_bytes(b, 1) == 16) p->bias_mode = (b0 == 1 && o0 != 1) ? kBiasRow : kBiasFull;
+    else if (b1 == 1 && o1 != 1 && b0 == o0) p->bias_mode = kBiasCol;
+    else return false;
+    p->bias = view_base(b);
+    p->bias_stride0 = b->stride0;
+  }
+  p->x = view_base(x);
+  p->out = (char *)view_base(out);
+  p->x_stride0 = x->stride0;
+  p->out_stride0 = out->stride0;
+  p->rows = (int32_t)o0;
+  p->vec_per_row = (int32_t)(o1 / 8);
+  *elem_dtype = T;
+  return true;
+}
+
+uint32_t padding_word_of(int32_t dtype, int32_t padding) {
+  static const uint32_t f32[4] = {0, 0x7FC00000u, 0x7F800000u, 0xFF800000u};
+  static const uint32_t f16[4] = {0, 0x7E00u, 0x7C00u, 0xFC00u};
+  static const uint32_t bf16[4] = {0, 0x7FC0u, 0x7F80u, 0xFF80u};
+  static const uint32_t e4m3[4] = {0, 0x7Fu, 0x7Eu, 0xFEu};
+  static const uint32_t e5m2[4] = {0, 0x7Eu, 0x7Cu, 0xFCu};
+  switch (dtype) {
+  case KAPY_F32: return f32[padding];
+  case KAPY_F16: return f16[padding];
+  case KAPY_BF16: return bf16[padding];
+  case KAPY_F8E4M3: return e4m3[padding];
+  case KAPY_F8E5M2: return e5m2[padding];
+  }
+  return 0;
+}
+
+DevView to_dev(const kapy_global *g) {
+  DevView v;
+  v.base = view_base(g);
+  v.stride0 = g->stride0;
+  v.stride1 = g->stride1;
+  v.ext0 = (int32_t)extent0(g);
+  v.ext1 = (int32_t)extent1(g);
+  v.dtype = g->dtype;
+  v.pad = 0;
+  return v;
+}
+
+}  // namespace
+}  // namespace kapy
+
+using namespace kapy;
+
+extern "C" {
+
+int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
+                     const kapy_global *out, void *stream) {
+  int result_dtype[kMaxInst];
+  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype);
+  if (rc) return rc;
+  rc = ensure_device();
+  if (rc) return rc;
+  const int64_t o0 = extent0(out), o1 = extent1(out);
+  if (o0 <= 0 || o1 <= 0) return KAPY_OK;
+  hipStream_t s = (hipStream_t)stream;
+
+  AffineActParams ap;
+  int T = -1;
+  if (match_affine_act(prog, n_inst, ins, out, &ap, &T)) {
+    uint32_t slots = (uint32_t)ap.rows * (uint32_t)ap.vec_per_row;
+    dim3 grid((slots + 1023) / 1024);
+    if (T == KAPY_F16) {
+      if (ap.act == KAPY_EW_GELU_TANH) affine_act_kernel<_Float16, KAPY_EW_GELU_TANH><<<grid, 256, 0, s>>>(ap);
+      else if (ap.act < 0) affine_act_kernel<_Float16, -1><<<grid, 256, 0, s>>>(ap);
+      else affine_act_kernel<_Float16, 0><<<grid, 256, 0, s>>>(ap);
+    } else {
+      if (ap.act == KAPY_EW_GELU_TANH) affine_act_kernel<Bf16Tag, KAPY_EW_GELU_TANH><<<grid, 256, 0, s>>>(ap);
+      else if (ap.act < 0) affine_act_kernel<Bf16Tag, -1><<<grid, 256, 0, s>>>(ap);
+      else affine_act_kernel<Bf16Tag, 0><<<grid, 256, 0, s>>>(ap);
+    }
+    KAPY_HIP_CHECK(hipGetLastError());
+    return KAPY_OK;
+  }
+
+  Program P;
+  memset(&P, 0, sizeof P);
+  P.n_inst = n_inst;
+  P.n_ins = n_ins;
+  for (int k = 0; k < n_inst; ++k) {
+    P.inst[k] = prog[k];
+    P.inst[k].dtype = result_dtype[k];
+  }
+  for (int k = 0; k < n_ins; ++k) P.in[k] = to_dev(ins[k]);
+  // padding pattern per input: taken from the (single) ld_global that names it
+  for (int k = 0; k < n_inst; ++k)
+    if (prog[k].op == KAPY_EW_LD_GLOBAL) P.in[prog[k].a].pad = padding_word_of(ins[prog[k].a]->dtype, prog[k].c);
+  P.out = to_dev(out);
+  int64_t total = o0 * o1;
+  int j_fastest = out->stride1 <= out->stride0;
+  dim3 grid((unsigned)((total + 255) / 256));
+  interpreter_kernel<<<grid, 256, 0, s>>>(P, j_fastest);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
+int kapy_fptofp(const kapy_global *src, const kapy_global *dst, int32_t rmode, void *stream) {
+  int rc = check_global(src, "fptofp source");
+  if (!rc) rc = check_global(dst, "fptofp result");
+  if (rc) return rc;
+  if (extent0(src) != extent0(dst) || extent1(src) != extent1(dst))
+    return fail(KAPY_ERR_VERIFY, "fptofp: source and result must have the same shape");
+  kapy_ew_inst prog[3] = {{KAPY_EW_LD_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f},
+                          {KAPY_EW_FPTOFP, 1, 0, 0, 0, dst->dtype, rmode, 0.f},
+                          {KAPY_EW_ST_GLOBAL, 0, 1, 0, 0, 0, KAPY_RN, 0.f}};
+  const kapy_global *ins[1] = {src};
+  return kapy_elementwise(prog, 3, ins, 1, dst, stream);
+}
+
+}  // extern "C"

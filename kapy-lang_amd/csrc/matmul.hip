@@ -1,0 +1,638 @@
+// matmul.hip — kapy.matmul over whole views on CDNA4 matrix cores (f16 / bf16 operands).
+//
+// Reference: kapy.matmul (include/kapy/Dialect/Kapy/IR/Ops.td:416-439, verifier
+// lib/Dialect/Kapy/IR/Kapy.cpp:451-574) lowered by MatmulOpToLLVM.cpp:58-311 to mma.sync, fed by
+// the cp.async ring of CpAsyncOpToLLVM.cpp:22-186 and ldmatrix (LdMatrixOpToLLVM.cpp:21-174);
+// the kernel shape is the fixture test/Conversion/KapyToKgpu/matmul.mlir: a 2-stage shared-memory
+// ring, fragments prefetched one k-slice ahead, one barrier per wait.
+//
+// gfx950 counterparts used here:
+//   mma.sync m16n8k16          -> v_mfma_f32_32x32x16_{f16,bf16} (fp32 accumulate)
+//   cp.async + wait_group      -> global_load_lds_dwordx4 (16 B per lane, written straight into
+//                                 LDS) + s_waitcnt vmcnt
+//   per-lane swizzled cp.async destination (CpAsyncOpToLLVM.cpp:124-139)
+//                              -> the destination of an LDS-direct load is wave-contiguous, so the
+//                                 XOR swizzle is applied to WHICH global chunk a lane fetches; the
+//                                 LDS image is the same swizzled one
+//   ldmatrix                   -> ds_read_b128 of 8 K-contiguous elements per lane
+//   swizzle (4,8) for 32 banks -> searched at compile time for 64 banks from the MFMA operand
+//                                 layout (layout.hpp first_swizzle)
+//
+// Two kernels:
+//   tn_kernel      both operands contiguous along K (lhs row-major, rhs column-major), extents
+//                  multiples of the tile: the roofline path.
+//   staged_kernel  any strides, ragged extents: tiles go global -> registers -> LDS, transposing
+//                  on the way when an operand is contiguous along M/N.  128x128x32 tiles.
+#include <algorithm>
+#include <type_traits>
+
+#include "common.hpp"
+#include "layout.hpp"
+#include "numeric.hpp"
+
+namespace kapy {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+struct Bf16 {};
+struct F16 {};
+template <typename T> struct Mfma32x32x16;
+template <> struct Mfma32x32x16<Bf16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma32x32x16<F16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+// LDS image of an operand tile: [rows][BK] 16-bit elements, K contiguous, 16-byte chunks XOR-ed
+// with the line index.  LP comes from the compile-time search over the MFMA operand layout.
+template <int BK>
+struct TileLayout {
+  static constexpr int kRowBytes = BK * 2;
+  static constexpr Swizzle kSwizzle = first_swizzle(mfma_lhs(kMfma32x32x16), {32, 16}, BK, 1, 16, 1024);
+  static_assert(kSwizzle.bank_param == 4, "MFMA operand reads are 16-byte: the search must return 16-byte atoms");
+  static constexpr int kLineParam = kSwizzle.line_param;
+  // byte offset of 16-byte chunk `chunk` of row `row`
+  static __device__ __forceinline__ uint32_t offset(uint32_t row, uint32_t chunk) {
+    uint32_t o = row * kRowBytes + chunk * 16;
+    return o ^ (((o >> 8) & (kLineParam - 1)) << 4);
+  }
+  // inverse on a linear LDS byte offset: which (row, chunk) of the tile lives there
+  static __device__ __forceinline__ void locate(uint32_t lds_off, uint32_t &row, uint32_t &chunk) {
+    uint32_t o = lds_off ^ (((lds_off >> 8) & (kLineParam - 1)) << 4);
+    row = o / kRowBytes;
+    chunk = (o % kRowBytes) / 16;
+  }
+};
+
+// s_waitcnt immediate that waits only on vmcnt <= n (gfx9 encoding: vmcnt in bits [3:0] and [15:14],
+// expcnt [6:4] and lgkmcnt [11:8] left at "no wait").
+constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+// Same, and also lgkmcnt(0): this wave's LDS reads have returned.  Used in front of a barrier after
+// which other waves overwrite the LDS stage this wave has been reading.
+constexpr int vmcnt_lgkm0_imm(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
+
+struct GemmParams {
+  const char *a, *b, *acc;
+  char *d;
+  int64_t a_sm, a_sk;  // lhs element strides along M and K
+  int64_t b_sn, b_sk;  // rhs element strides along N and K
+  int64_t acc_sm, acc_sn, d_sm, d_sn;
+  int32_t M, N, K;
+  int32_t acc_dtype;  // -1: no accumulator input
+  int32_t d_dtype;
+  int32_t rz;         // final cast rounds toward zero
+  int32_t tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ void store_result(const GemmParams &p, int32_t m, int32_t n, float v) {
+  if (m >= p.M || n >= p.N) return;
+  if (p.acc_dtype >= 0) v += load_as_f32(p.acc, p.acc_dtype, m * p.acc_sm + n * p.acc_sn);
+  int64_t idx = m * p.d_sm + n * p.d_sn;
+  switch (p.d_dtype) {
+  case KAPY_F32: ((float *)p.d)[idx] = v; break;
+  case KAPY_F16: ((uint16_t *)p.d)[idx] = p.rz ? f32_to_f16_rz(v) : f32_to_f16_rn(v); break;
+  default: ((uint16_t *)p.d)[idx] = p.rz ? f32_to_bf16_rz(v) : f32_to_bf16_rn(v); break;
+  }
+}
+
+// Epilogue of one 32x32 accumulator block.  The MFMA is issued with the operands swapped
+// (rhs fragment first), so register v of lane l holds D[m = l%32][n = 8*(v/4) + 4*(l/32) + v%4]:
+// four consecutive n per register quad, the transposed form of the <[2,32],[4,1],(0,1)>
+// accumulator fragments.
+// Packed form: 16-bit row-major result, block fully in range, no accumulator input, RN: one
+// 8-byte store per quad.
+__device__ __forceinline__ void store_block_packed(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, const f32x16 &acc) {
+  char *row = p.d + ((int64_t)(m_base + (lane & 31)) * p.d_sm + n_base + 4 * (lane >> 5)) * 2;
+  const bool f16 = p.d_dtype == KAPY_F16;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    uint16_t h[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = f16 ? f32_to_f16_rn(acc[4 * q + e]) : f32_to_bf16_rn(acc[4 * q + e]);
+    u32x2 w = {h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16)};
+    *(u32x2 *)(row + 16 * q) = w;
+  }
+}
+// General form: any result type and strides, accumulator input, ragged edges.  Out of line: it is
+// large and off the roofline path.
+__device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, f32x16 acc) {
+  const int32_t m = m_base + (lane & 31);
+  for (int v = 0; v < 16; ++v) store_result(p, m, n_base + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), acc[v]);
+}
+
+// Workgroup id -> output tile.  Consecutive workgroup ids land on different XCDs (8 of them, each
+// with its own L2), so ids are first regrouped per XCD, then each XCD walks a compact band of
+// tiles GROUP_M tall so that the operand panels it streams stay in its L2.
+__device__ __forceinline__ void tile_of_block(const GemmParams &p, int32_t &tm, int32_t &tn) {
+  constexpr int kXcds = 8, kGroupM = 8;
+  int32_t total = p.tiles_m * p.tiles_n, id = blockIdx.x;
+  if (total % kXcds == 0) id = (id % kXcds) * (total / kXcds) + id / kXcds;
+  int32_t per_group = kGroupM * p.tiles_n;
+  int32_t g = id / per_group, first_m = g * kGroupM;
+  int32_t rows = std::min(p.tiles_m - first_m, kGroupM);
+  int32_t in_group = id - g * per_group;
+  tm = first_m + in_group % rows;
+  tn = in_group / rows;
+}
+
+// ---------------------------------------------------------------------------------------------
+// TN kernel.  BM x BN x BK workgroup tile, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN)
+// block of 32x32 accumulators.  STAGES-deep LDS ring filled by LDS-direct loads.
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
+struct TnConfig {
+  static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves;
+  static constexpr int kWtm = BM / WM, kWtn = BN / WN;       // wave tile
+  static constexpr int kTm = kWtm / 32, kTn = kWtn / 32;     // 32x32 accumulators per wave
+  static constexpr int kRowBytes = BK * 2;
+  static constexpr int kRowsPerLoad = 1024 / kRowBytes;      // rows one LDS-direct wave instruction fills
+  static constexpr int kLoadsA = BM / kRowsPerLoad, kLoadsB = BN / kRowsPerLoad;
+  static constexpr int kLoadsAPerWave = kLoadsA / kWaves, kLoadsBPerWave = kLoadsB / kWaves;
+  static constexpr int kStageBytes = (BM + BN) * kRowBytes;
+  static constexpr int kLdsBytes = STAGES * kStageBytes;
+  static_assert(kLoadsA % kWaves == 0 && kLoadsB % kWaves == 0, "loads must divide evenly over the wavefronts");
+  static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % 16 == 0, "wave tile must be a multiple of the MFMA tile");
+};
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
+__global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
+  using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
+  using L = TileLayout<BK>;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+  int32_t tm, tn;
+  tile_of_block(p, tm, tn);
+  const int32_t m0 = tm * BM, n0 = tn * BN;
+
+  // Per-lane global byte offsets of the chunks this lane fetches, one per load instruction.
+  // Instruction q of an operand fills LDS bytes [q*1024, q*1024+1024); this lane's 16 bytes sit at
+  // q*1024 + lane*16, which the (inverse) swizzle maps back to a (row, chunk) of the tile.
+  uint32_t a_goff[C::kLoadsAPerWave], b_goff[C::kLoadsBPerWave];
+#pragma unroll
+  for (int i = 0; i < C::kLoadsAPerWave; ++i) {
+    uint32_t row, chunk;
+    L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
+    a_goff[i] = (uint32_t)((row * p.a_sm + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < C::kLoadsBPerWave; ++i) {
+    uint32_t row, chunk;
+    L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
+    b_goff[i] = (uint32_t)((row * p.b_sn + chunk * 8) * 2);
+  }
+  const char *a_tile = p.a + (int64_t)m0 * p.a_sm * 2;
+  const char *b_tile = p.b + (int64_t)n0 * p.b_sn * 2;
+
+  // Load instruction `idx` (0 .. loads per tile - 1) of this wavefront for K-tile kt into `stage`.
+  auto issue_load = [&](int stage, int kt, int idx) {
+    char *sa = lds + stage * C::kStageBytes, *sb = sa + BM * C::kRowBytes;
+    if (idx < C::kLoadsAPerWave) {
+      const char *ga = a_tile + (int64_t)kt * BK * 2;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ga + a_goff[idx]),
+                                       (__attribute__((address_space(3))) void *)(sa + (wave + idx * C::kWaves) * 1024), 16, 0, 0);
+    } else {
+      const int i = idx - C::kLoadsAPerWave;
+      const char *gb = b_tile + (int64_t)kt * BK * 2;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb + b_goff[i]),
+                                       (__attribute__((address_space(3))) void *)(sb + (wave + i * C::kWaves) * 1024), 16, 0, 0);
+    }
+  };
+  auto issue_loads = [&](int stage, int kt) {
+#pragma unroll
+    for (int idx = 0; idx < C::kLoadsAPerWave + C::kLoadsBPerWave; ++idx) issue_load(stage, kt, idx);
+  };
+
+  // LDS byte offsets of this lane's operand reads: row (lane % 32) of each 32-row block, 16-byte
+  // chunk (2*kk + lane/32) of the K slice kk.
+  const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
+
+  f32x16 acc[C::kTm][C::kTn];
+  {
+    f32x16 zero;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+#pragma unroll
+    for (int i = 0; i < C::kTm; ++i)
+#pragma unroll
+      for (int j = 0; j < C::kTn; ++j) acc[i][j] = zero;
+  }
+
+  const int KT = p.K / BK;
+  constexpr int KK = BK / 16;                                          // MFMA K-slices per tile
+  constexpr int kLoadsPerTile = C::kLoadsAPerWave + C::kLoadsBPerWave;  // per wavefront
+  // Per-lane LDS offsets of the operand reads of slice kk, relative to the wave's rows of a stage.
+  uint32_t frag_off[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) frag_off[kk] = L::offset(frag_row, 2 * kk + frag_half);
+  const uint32_t a_rows = (wm * C::kWtm) * C::kRowBytes, b_rows = BM * C::kRowBytes + (wn * C::kWtn) * C::kRowBytes;
+  // 32-row blocks are whole multiples of the swizzle period, so block i only adds i*32*rowBytes.
+  static_assert((32 * C::kRowBytes) % (256 * L::kLineParam) == 0, "a 32-row block must span whole swizzle periods");
+  // Fragment `idx` of slice kk: the first kTm are lhs row blocks, the rest rhs column blocks.
+  auto read_frag = [&](int stage, int kk, int idx, u32x4 *af, u32x4 *bf) {
+    const char *base = lds + stage * C::kStageBytes + frag_off[kk];
+    if (idx < C::kTm) af[idx] = *(const u32x4 *)(base + a_rows + idx * 32 * C::kRowBytes);
+    else bf[idx - C::kTm] = *(const u32x4 *)(base + b_rows + (idx - C::kTm) * 32 * C::kRowBytes);
+  };
+  auto read_frags = [&](int stage, int kk, u32x4 *af, u32x4 *bf) {
+#pragma unroll
+    for (int idx = 0; idx < C::kTm + C::kTn; ++idx) read_frag(stage, kk, idx, af, bf);
+  };
+  auto multiply = [&](const u32x4 *af, const u32x4 *bf) {
+#pragma unroll
+    for (int i = 0; i < C::kTm; ++i)
+#pragma unroll
+      for (int j = 0; j < C::kTn; ++j) acc[i][j] = Mfma32x32x16<T>::run(bf[j], af[i], acc[i][j]);
+  };
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < KT) issue_loads(s, s);
+
+  if constexpr (STAGES == 2) {
+    // Two stages: the tile multiplied in iteration kt was requested in iteration kt-1.
+    for (int kt = 0; kt < KT; ++kt) {
+      __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+      __builtin_amdgcn_s_barrier();  // tile kt visible to all; all done reading the stage refilled next
+      if (kt + 1 < KT) issue_loads((kt + 1) & 1, kt + 1);
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        u32x4 af[C::kTm], bf[C::kTn];
+        read_frags(kt & 1, kk, af, bf);
+        multiply(af, bf);
+      }
+    }
+  } else {
+    // Three or more stages: the barrier at the top of iteration kt publishes tile kt+1, so the
+    // fragments of the next K-slice are always fetched one slice ahead, across tile boundaries
+    // (the register double-buffering of the reference fixture, matmul.mlir:51-91).
+    static_assert(KK % 2 == 0, "fragment double-buffering needs an even number of K-slices per tile");
+    u32x4 af[2][C::kTm], bf[2][C::kTn];
+    if (KT > STAGES - 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsPerTile * (STAGES - 2)));
+    else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    __builtin_amdgcn_s_barrier();  // tile 0 published
+    read_frags(0, 0, af[0], bf[0]);
+    int stage = 0;  // stage of tile kt
+    // One tile.  HAS_NEXT: tile kt+1 exists (publish it, prefetch its first fragments).
+    // LOADS: tile kt+STAGES-1 exists (request it).  The flags are compile-time so that the
+    // steady-state body is branch-free and the scheduler can interleave LDS reads with MFMAs.
+    auto tile_step = [&](int kt, auto has_next, auto loads) {
+      const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+      if constexpr (has_next.value) {
+        // own loads of tile kt+1 have landed once only the younger tiles' loads remain in flight
+        if constexpr (loads.value) __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kLoadsPerTile * (STAGES - 3)));
+        else __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+        __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
+      }
+      // Source order is issue order (sched_barrier pins it): behind each of the first matrix
+      // instructions of a slice goes one LDS read of the next slice's fragments and, in the first
+      // slice, one LDS-direct global load, so reads have the rest of the slice to land.
+      constexpr int kReads = C::kTm + C::kTn, kMfmas = C::kTm * C::kTn;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        u32x4 *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
+#pragma unroll
+        for (int g = 0; g < kMfmas; ++g) {
+          const int i = g / C::kTn, j = g % C::kTn;
+          acc[i][j] = Mfma32x32x16<T>::run(b_cur[j], a_cur[i], acc[i][j]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (g < kReads) {
+            if (kk + 1 < KK) read_frag(stage, kk + 1, g, a_nxt, b_nxt);
+            else if constexpr (has_next.value) read_frag(next_stage, 0, g, a_nxt, b_nxt);
+          }
+          if constexpr (has_next.value && loads.value)
+            if (kk == 0 && g < kLoadsPerTile) issue_load(stage == 0 ? STAGES - 1 : stage - 1, kt + STAGES - 1, g);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      stage = next_stage;
+    };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+    int kt = 0;
+    for (; kt + STAGES - 1 < KT; ++kt) tile_step(kt, Yes{}, Yes{});
+    for (; kt + 1 < KT; ++kt) tile_step(kt, Yes{}, No{});
+    tile_step(kt, No{}, No{});
+  }
+
+#pragma unroll
+  for (int i = 0; i < C::kTm; ++i)
+#pragma unroll
+    for (int j = 0; j < C::kTn; ++j)
+      if (PACKED) store_block_packed(p, m0 + wm * C::kWtm + i * 32, n0 + wn * C::kWtn + j * 32, lane, acc[i][j]);
+      else store_block_generic(p, m0 + wm * C::kWtm + i * 32, n0 + wn * C::kWtn + j * 32, lane, acc[i][j]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Staged kernel: 128x128x32 tile, 4 wavefronts (2x2), wave tile 64x64.  Any operand strides, ragged
+// extents (out-of-range elements read as zero: the padding-ZERO ld_global of the reference).
+constexpr int kSBM = 128, kSBN = 128, kSBK = 32;
+
+// One operand tile [128 rows][32 k] is 512 16-byte vectors: 2 per thread.  In "k contiguous" mode a
+// vector is 8 consecutive k of one row; in "row contiguous" mode it is 8 consecutive rows at one k
+// and is scattered into the K-contiguous LDS image element by element.
+struct StagedRegs {
+  u32x4 v[2];
+};
+
+__device__ __forceinline__ u32x4 load_vec8(const char *base, int64_t s_row, int64_t s_k, int32_t row, int32_t k, int32_t rows,
+                                           int32_t K, bool k_contig) {
+  u32x4 r = {0, 0, 0, 0};
+  const uint16_t *e = (const uint16_t *)base;
+  if (k_contig) {
+    if (row >= rows || k >= K) return r;
+    const uint16_t *ptr = e + row * s_row + k;
+    if (k + 8 <= K && (((uintptr_t)ptr) & 15) == 0) return *(const u32x4 *)ptr;
+    uint16_t t[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = (k + i < K) ? ptr[i] : (uint16_t)0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) r[w] = t[2 * w] | ((uint32_t)t[2 * w + 1] << 16);
+    return r;
+  }
+  if (row >= rows || k >= K) return r;
+  const uint16_t *ptr = e + row + k * s_k;  // s_row == 1
+  if (row + 8 <= rows && (((uintptr_t)ptr) & 15) == 0) return *(const u32x4 *)ptr;
+  uint16_t t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t[i] = (row + i < rows) ? ptr[i] : (uint16_t)0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) r[w] = t[2 * w] | ((uint32_t)t[2 * w + 1] << 16);
+  return r;
+}
+
+// Fully strided operand (no contiguous axis): element-wise gather of 8 consecutive k of one row.
+__device__ __forceinline__ u32x4 gather_vec8(const char *base, int64_t s_row, int64_t s_k, int32_t row, int32_t k, int32_t rows,
+                                             int32_t K) {
+  u32x4 r = {0, 0, 0, 0};
+  if (row >= rows) return r;
+  const uint16_t *e = (const uint16_t *)base + row * s_row;
+  uint16_t t[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t[i] = (k + i < K) ? e[(k + i) * s_k] : (uint16_t)0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) r[w] = t[2 * w] | ((uint32_t)t[2 * w + 1] << 16);
+  return r;
+}
+
+enum OperandMode { kKContig = 0, kRowContig = 1, kStrided = 2 };
+
+template <typename T, bool PACKED>
+__global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, int b_mode) {
+  using L = TileLayout<kSBK>;
+  __shared__ __attribute__((aligned(1024))) char lds[(kSBM + kSBN) * kSBK * 2];
+  char *sa = lds, *sb = lds + kSBM * kSBK * 2;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  int32_t tm, tn;
+  tile_of_block(p, tm, tn);
+  const int32_t m0 = tm * kSBM, n0 = tn * kSBN;
+
+  auto fetch = [&](const char *base, int64_t s_row, int64_t s_k, int32_t row0, int32_t rows, int mode, int kt, StagedRegs &r) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int v = tid + h * 256;
+      if (mode == kRowContig) {
+        int k = v >> 4, rchunk = v & 15;  // 16 chunks of 8 rows at each of 32 k
+        r.v[h] = load_vec8(base, s_row, s_k, row0 + rchunk * 8, kt * kSBK + k, rows, p.K, false);
+      } else {
+        int row = v >> 2, kchunk = v & 3;  // 4 chunks of 8 k in each of 128 rows
+        r.v[h] = mode == kKContig ? load_vec8(base, s_row, s_k, row0 + row, kt * kSBK + kchunk * 8, rows, p.K, true)
+                                  : gather_vec8(base, s_row, s_k, row0 + row, kt * kSBK + kchunk * 8, rows, p.K);
+      }
+    }
+  };
+  auto stash = [&](char *tile, int mode, const StagedRegs &r) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int v = tid + h * 256;
+      if (mode == kRowContig) {
+        int k = v >> 4, rchunk = v & 15;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          uint16_t x = (uint16_t)(r.v[h][e >> 1] >> ((e & 1) * 16));
+          *(uint16_t *)(tile + L::offset(rchunk * 8 + e, k >> 3) + (k & 7) * 2) = x;
+        }
+      } else {
+        int row = v >> 2, kchunk = v & 3;
+        *(u32x4 *)(tile + L::offset(row, kchunk)) = r.v[h];
+      }
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int KT = (p.K + kSBK - 1) / kSBK;
+  StagedRegs ra, rb;
+  fetch(p.a, p.a_sm, p.a_sk, m0, p.M, a_mode, 0, ra);
+  fetch(p.b, p.b_sn, p.b_sk, n0, p.N, b_mode, 0, rb);
+  const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
+  for (int kt = 0; kt < KT; ++kt) {
+    __syncthreads();  // every wave has finished reading the previous tile
+    stash(sa, a_mode, ra);
+    stash(sb, b_mode, rb);
+    __syncthreads();
+    if (kt + 1 < KT) {  // next tile's global loads fly while this one is multiplied
+      fetch(p.a, p.a_sm, p.a_sk, m0, p.M, a_mode, kt + 1, ra);
+      fetch(p.b, p.b_sn, p.b_sk, n0, p.N, b_mode, kt + 1, rb);
+    }
+#pragma unroll
+    for (int kk = 0; kk < kSBK / 16; ++kk) {
+      u32x4 af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = *(const u32x4 *)(sa + L::offset(wm * 64 + i * 32 + frag_row, 2 * kk + frag_half));
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bf[j] = *(const u32x4 *)(sb + L::offset(wn * 64 + j * 32 + frag_row, 2 * kk + frag_half));
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32x32x16<T>::run(bf[j], af[i], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int32_t mb = m0 + wm * 64 + i * 32, nb = n0 + wn * 64 + j * 32;
+      if (PACKED && mb + 32 <= p.M && nb + 32 <= p.N) store_block_packed(p, mb, nb, lane, acc[i][j]);
+      else store_block_generic(p, mb, nb, lane, acc[i][j]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side.
+// 16-bit row-major result with 8-byte aligned rows, no accumulator input, RN: the packed epilogue.
+bool packed_epilogue(const GemmParams &p) {
+  return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16) && p.d_sn == 1 && p.acc_dtype < 0 && !p.rz &&
+         ((uintptr_t)p.d & 7) == 0 && (p.d_sm * 2) % 8 == 0;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
+int launch_tn_epi(GemmParams p, hipStream_t s) {
+  using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
+  auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED>;
+  static bool configured = false;  // raising the dynamic LDS limit is idempotent; a race only repeats it
+  if (!configured) {
+    KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes));
+    configured = true;
+  }
+  p.tiles_m = p.M / BM;
+  p.tiles_n = p.N / BN;
+  kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(C::kThreads), C::kLdsBytes, s>>>(p);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
+int launch_tn(const GemmParams &p, hipStream_t s) {
+  return packed_epilogue(p) ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s)
+                            : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
+}
+
+template <typename T>
+int launch_staged(GemmParams p, int a_mode, int b_mode, hipStream_t s) {
+  p.tiles_m = (p.M + kSBM - 1) / kSBM;
+  p.tiles_n = (p.N + kSBN - 1) / kSBN;
+  dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  if (packed_epilogue(p)) staged_kernel<T, true><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
+  else staged_kernel<T, false><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
+// Kapy.cpp:451-487 (shape / element type rules) and :491-564 (minimum tile sizes).
+int verify_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *res, int impl_way) {
+  int rc = check_global(lhs, "matmul lhs");
+  if (!rc) rc = check_global(rhs, "matmul rhs");
+  if (!rc) rc = check_global(res, "matmul result");
+  if (!rc && acc) rc = check_global(acc, "matmul acc");
+  if (rc) return rc;
+  if (extent1(lhs) != extent0(rhs))
+    return fail(KAPY_ERR_VERIFY, "matmul: number of columns of lhs must be equal to number of rows of rhs");
+  if (extent0(res) != extent0(lhs) || (acc && extent0(acc) != extent0(lhs)))
+    return fail(KAPY_ERR_VERIFY, "matmul: number of rows of acc must be equal to number of rows of lhs");
+  if (extent1(res) != extent1(rhs) || (acc && extent1(acc) != extent1(rhs)))
+    return fail(KAPY_ERR_VERIFY, "matmul: number of columns of acc must be equal to number of columns of rhs");
+  if (dtype_bytes(lhs->dtype) != dtype_bytes(rhs->dtype))
+    return fail(KAPY_ERR_VERIFY, "matmul: lhs and rhs must have same element bit width");
+  if (acc && acc->dtype != KAPY_F16 && acc->dtype != KAPY_F32)
+    return fail(KAPY_ERR_VERIFY, "matmul: result must have f16 or f32 element type");
+  if (acc && lhs->dtype == KAPY_BF16 && rhs->dtype == KAPY_BF16 && acc->dtype == KAPY_F16)
+    return fail(KAPY_ERR_VERIFY, "matmul: result must have f32 element type when operands are bf16 element type");
+  if (!is_f8(lhs->dtype) && lhs->dtype != rhs->dtype)
+    return fail(KAPY_ERR_VERIFY, "matmul: lhs and rhs must have same element type unless they have f8 element type");
+  bool f16ish = lhs->dtype == KAPY_F16 || lhs->dtype == KAPY_BF16;
+  switch (impl_way) {
+  case KAPY_MATMUL_AUTO: break;
+  case KAPY_MMA_M16N8K8_F16: case KAPY_MMA_M16N8K16_F16: case KAPY_MFMA_32X32X16_16B: case KAPY_MFMA_16X16X32_16B:
+    if (!f16ish) return fail(KAPY_ERR_VERIFY, "matmul: mma f16 operands must have f16 or bf16 element type");
+    break;
+  case KAPY_MMA_M16N8K8_TF32:
+    if (lhs->dtype != KAPY_F32) return fail(KAPY_ERR_VERIFY, "matmul: mma_m16n8k8_tf32 operands must have f32 element type");
+    return fail(KAPY_ERR_UNSUPPORTED, "matmul: mma_m16n8k8_tf32 has no counterpart on gfx950 (no tf32 matrix instruction)");
+  case KAPY_MMA_M16N8K16_F8: case KAPY_MFMA_16X16X128_F8: case KAPY_MFMA_32X32X64_F8:
+    if (!is_f8(lhs->dtype) || !is_f8(rhs->dtype))
+      return fail(KAPY_ERR_VERIFY, "matmul: mma f8 operands must have f8E4M3 or f8E5M2 element type");
+    break;
+  default: return fail(KAPY_ERR_INVALID, "matmul: unknown implement way %d", impl_way);
+  }
+  for (const kapy_global *g : {lhs, rhs, res, acc})
+    if (g && (g->start0 < 0 || g->start1 < 0)) return fail(KAPY_ERR_INVALID, "matmul: negative view start");
+  return KAPY_OK;
+}
+
+int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
+
+}  // namespace
+
+// Implemented in matmul_f8.hip.
+int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale, const float *col_scale, const kapy_global *acc,
+              const kapy_global *result, const kapy_matmul_cfg *cfg, hipStream_t s);
+
+}  // namespace kapy
+
+using namespace kapy;
+
+extern "C" {
+
+int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
+                const kapy_matmul_cfg *cfg, void *stream) {
+  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, {0, 0, 0}};
+  if (cfg) c = *cfg;
+  int rc = verify_matmul(lhs, rhs, acc, result, c.impl_way);
+  if (rc) return rc;
+  if (c.rmode != KAPY_RN && c.rmode != KAPY_RZ) return fail(KAPY_ERR_INVALID, "matmul: unknown rounding mode %d", c.rmode);
+  if (result->dtype != KAPY_F16 && result->dtype != KAPY_BF16 && result->dtype != KAPY_F32)
+    return fail(KAPY_ERR_VERIFY, "matmul: result must have f16, bf16 or f32 element type");
+  rc = ensure_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_f8(lhs->dtype)) return matmul_f8(lhs, rhs, nullptr, nullptr, acc, result, &c, s);
+  if (lhs->dtype != KAPY_F16 && lhs->dtype != KAPY_BF16)
+    return fail(KAPY_ERR_UNSUPPORTED, "matmul: %s operands have no matrix instruction on gfx950", dtype_name(lhs->dtype));
+
+  GemmParams p;
+  p.a = view_base(lhs);
+  p.b = view_base(rhs);
+  p.acc = acc ? view_base(acc) : nullptr;
+  p.d = (char *)view_base(result);
+  p.a_sm = lhs->stride0; p.a_sk = lhs->stride1;
+  p.b_sk = rhs->stride0; p.b_sn = rhs->stride1;
+  p.acc_sm = acc ? acc->stride0 : 0; p.acc_sn = acc ? acc->stride1 : 0;
+  p.d_sm = result->stride0; p.d_sn = result->stride1;
+  p.M = (int32_t)extent0(lhs); p.K = (int32_t)extent1(lhs); p.N = (int32_t)extent1(rhs);
+  p.acc_dtype = acc ? acc->dtype : -1;
+  p.d_dtype = result->dtype;
+  p.rz = c.rmode == KAPY_RZ;
+  p.tiles_m = p.tiles_n = 0;
+  if (p.M == 0 || p.N == 0) return KAPY_OK;
+  const bool bf16 = lhs->dtype == KAPY_BF16;
+
+  // Roofline path: both operands K-contiguous, 16-byte aligned rows, extents multiples of the tile,
+  // and offsets that fit the 32-bit per-lane address arithmetic of the loader.
+  bool tn = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 0) == 16 && p.K > 0 &&
+            p.a_sm * 2 * 256 < (int64_t(1) << 31) && p.b_sn * 2 * 256 < (int64_t(1) << 31) && p.a_sm > 0 && p.b_sn > 0;
+  int bm = c.tile_m, bn = c.tile_n, bk = c.tile_k;
+  if (tn && (bm == 0 || bm == 256) && (bn == 0 || bn == 256) && (bk == 0 || bk == 32) && p.M % 256 == 0 && p.N % 256 == 0 &&
+      p.K % 32 == 0)
+    return bf16 ? launch_tn<Bf16, 256, 256, 32, 2, 2, 4>(p, s) : launch_tn<F16, 256, 256, 32, 2, 2, 4>(p, s);
+  if ((bm != 0 && bm != kSBM) || (bn != 0 && bn != kSBN) || (bk != 0 && bk != kSBK))
+    return fail(KAPY_ERR_UNSUPPORTED, "matmul: tile %dx%dx%d is not available for these operands (128x128x32 is)", bm, bn, bk);
+  int a_mode = operand_mode(p.a_sm, p.a_sk), b_mode = operand_mode(p.b_sn, p.b_sk);
+  return bf16 ? launch_staged<Bf16>(p, a_mode, b_mode, s) : launch_staged<F16>(p, a_mode, b_mode, s);
+}
+
+int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out) {
+  if (!out) return fail(KAPY_ERR_INVALID, "matmul_lds_layout: null result");
+  if (operand_dtype != KAPY_F16 && operand_dtype != KAPY_BF16)
+    return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: only f16 / bf16 operand tiles are described here");
+  Swizzle s;
+  switch (tile_k) {
+  case 32: s = TileLayout<32>::kSwizzle; break;
+  case 64: s = TileLayout<64>::kSwizzle; break;
+  default: return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: tile_k must be 32 or 64");
+  }
+  out->stride0 = s.stride0;
+  out->stride1 = s.stride1;
+  out->bank_param = s.bank_param;
+  out->line_param = s.line_param;
+  return KAPY_OK;
+}
+
+}  // extern "C"

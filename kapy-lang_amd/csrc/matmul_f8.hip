@@ -1,0 +1,177 @@
+// matmul_f8.hip — kapy.matmul on OCP fp8 operands (E4M3FN / E5M2, mixable) with fp32 accumulate,
+// and the W8A8 form with fp32 row/column scales applied in the epilogue.
+//
+// Reference: MatmulImplWay::MMA_M16N8K16_F8 (lib/Dialect/Kapy/IR/Kapy.cpp:545-564 verifier,
+// MatmulOpToLLVM.cpp:269-311 mma.sync.m16n8k16 e4m3/e5m2 strings, operand layouts
+// LayoutUtils.cpp:141-147) followed by mulf with broadcast scales and fptofp rn.
+// gfx950: v_mfma_scale_f32_16x16x128_f8f6f4 with unit E8M0 block scales (2^0); the operand format
+// selectors (cbsz / blgp: 0 = E4M3, 1 = E5M2) carry kapy's mixed-f8 rule.
+//
+//   skinny_kernel  few rows of lhs (decode shape): HBM-bound on the weight.  One workgroup per 16
+//                  output columns, its 4 wavefronts split K; every weight byte is read once,
+//                  straight from global memory into the MFMA operand registers (each lane's 32
+//                  K-contiguous bytes are exactly its operand), partial sums meet in LDS.
+//   naive_kernel   any strides / ragged K: one output element per lane, software decode.
+#include "common.hpp"
+#include "layout.hpp"
+#include "numeric.hpp"
+
+namespace kapy {
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct F8Params {
+  const uint8_t *a, *b;
+  const char *acc;
+  char *d;
+  const float *row_scale, *col_scale;
+  int64_t a_sm, a_sk, b_sn, b_sk, acc_sm, acc_sn, d_sm, d_sn;
+  int32_t M, N, K;
+  int32_t a_dtype, b_dtype, acc_dtype, d_dtype, rz;
+};
+
+__device__ __forceinline__ void finish(const F8Params &p, int32_t m, int32_t n, float v) {
+  if (m >= p.M || n >= p.N) return;
+  if (p.row_scale) v *= __fmul_rn(p.row_scale[m], p.col_scale[n]);
+  if (p.acc_dtype >= 0) v += load_as_f32(p.acc, p.acc_dtype, m * p.acc_sm + n * p.acc_sn);
+  int64_t idx = m * p.d_sm + n * p.d_sn;
+  switch (p.d_dtype) {
+  case KAPY_F32: ((float *)p.d)[idx] = v; break;
+  case KAPY_F16: ((uint16_t *)p.d)[idx] = p.rz ? f32_to_f16_rz(v) : f32_to_f16_rn(v); break;
+  default: ((uint16_t *)p.d)[idx] = p.rz ? f32_to_bf16_rz(v) : f32_to_bf16_rn(v); break;
+  }
+}
+
+__global__ __launch_bounds__(256) void naive_kernel(F8Params p) {
+  int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= (int64_t)p.M * p.N) return;
+  int32_t m = (int32_t)(t / p.N), n = (int32_t)(t - (int64_t)m * p.N);
+  float s = 0.f;
+  for (int32_t k = 0; k < p.K; ++k) {
+    float x = load_as_f32(p.a, p.a_dtype, m * p.a_sm + k * p.a_sk);
+    float y = load_as_f32(p.b, p.b_dtype, n * p.b_sn + k * p.b_sk);
+    s = __fmaf_rn(x, y, s);
+  }
+  finish(p, m, n, s);
+}
+
+// 32 K-contiguous bytes of one row/column as the 8-dword MFMA operand; rows past the end read zero.
+__device__ __forceinline__ i32x8 load_k32(const uint8_t *base, int64_t stride, int32_t row, int32_t rows, int32_t k) {
+  i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (row < rows) {
+    const i32x4 *ptr = (const i32x4 *)(base + row * stride + k);
+    i32x4 lo = ptr[0], hi = ptr[1];
+    r = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  }
+  return r;
+}
+
+template <int A_FMT, int B_FMT>
+__global__ __launch_bounds__(256) void skinny_kernel(F8Params p) {
+  __shared__ float partial[4][16][16 + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int32_t n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+  const int32_t row = lane & 15, kq = (lane >> 4) * 32;  // this lane's row/column and its 32-byte K quarter
+  // K is split in 4 contiguous ranges of whole 128-element MFMA steps
+  const int32_t steps = p.K / 128, per_wave = (steps + 3) / 4;
+  const int32_t s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  constexpr int UNROLL = 4;
+  int32_t s = s_begin;
+  for (; s + UNROLL <= s_end; s += UNROLL) {
+    i32x8 bw[UNROLL], aw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) bw[u] = load_k32(p.b, p.b_sn, n0 + row, p.N, (s + u) * 128 + kq);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) aw[u] = load_k32(p.a, p.a_sm, m0 + row, p.M, (s + u) * 128 + kq);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aw[u], bw[u], acc, A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  }
+  for (; s < s_end; ++s) {
+    i32x8 bw = load_k32(p.b, p.b_sn, n0 + row, p.N, s * 128 + kq);
+    i32x8 aw = load_k32(p.a, p.a_sm, m0 + row, p.M, s * 128 + kq);
+    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aw, bw, acc, A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  }
+  // accumulator register v of lane l: row 4*(l/16) + v, column l%16
+#pragma unroll
+  for (int v = 0; v < 4; ++v) partial[wave][4 * (lane >> 4) + v][lane & 15] = acc[v];
+  __syncthreads();
+  const int m = threadIdx.x >> 4, n = threadIdx.x & 15;
+  float sum = (partial[0][m][n] + partial[1][m][n]) + (partial[2][m][n] + partial[3][m][n]);
+  finish(p, m0 + m, n0 + n, sum);
+}
+
+int fmt_of(int dtype) { return dtype == KAPY_F8E5M2 ? 1 : 0; }
+
+}  // namespace
+
+int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale, const float *col_scale, const kapy_global *acc,
+              const kapy_global *result, const kapy_matmul_cfg *cfg, hipStream_t s) {
+  F8Params p;
+  p.a = (const uint8_t *)view_base(a);
+  p.b = (const uint8_t *)view_base(b);
+  p.acc = acc ? view_base(acc) : nullptr;
+  p.d = (char *)view_base(result);
+  p.row_scale = row_scale;
+  p.col_scale = col_scale;
+  p.a_sm = a->stride0; p.a_sk = a->stride1;
+  p.b_sk = b->stride0; p.b_sn = b->stride1;
+  p.acc_sm = acc ? acc->stride0 : 0; p.acc_sn = acc ? acc->stride1 : 0;
+  p.d_sm = result->stride0; p.d_sn = result->stride1;
+  p.M = (int32_t)extent0(a); p.K = (int32_t)extent1(a); p.N = (int32_t)extent1(b);
+  p.a_dtype = a->dtype; p.b_dtype = b->dtype;
+  p.acc_dtype = acc ? acc->dtype : -1;
+  p.d_dtype = result->dtype;
+  p.rz = cfg && cfg->rmode == KAPY_RZ;
+  if (p.M == 0 || p.N == 0) return KAPY_OK;
+  bool k_contig = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(a, 1) == 16 && vector_bytes(b, 0) == 16 && p.K % 128 == 0 && p.K > 0;
+  if (k_contig) {
+    dim3 grid((unsigned)((p.N + 15) / 16), (unsigned)((p.M + 15) / 16));
+    if (grid.y <= 65535) {
+      int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
+      if (fa == 0 && fb == 0) skinny_kernel<0, 0><<<grid, 256, 0, s>>>(p);
+      else if (fa == 0) skinny_kernel<0, 1><<<grid, 256, 0, s>>>(p);
+      else if (fb == 0) skinny_kernel<1, 0><<<grid, 256, 0, s>>>(p);
+      else skinny_kernel<1, 1><<<grid, 256, 0, s>>>(p);
+      KAPY_HIP_CHECK(hipGetLastError());
+      return KAPY_OK;
+    }
+  }
+  int64_t total = (int64_t)p.M * p.N;
+  naive_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(p);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
+}  // namespace kapy
+
+using namespace kapy;
+
+extern "C" int kapy_matmul_scaled_f8(const kapy_global *a8, const kapy_global *w8, const float *row_scale, const float *col_scale,
+                                     const kapy_global *result, const kapy_matmul_cfg *cfg, void *stream) {
+  int rc = check_global(a8, "matmul lhs");
+  if (!rc) rc = check_global(w8, "matmul rhs");
+  if (!rc) rc = check_global(result, "matmul result");
+  if (rc) return rc;
+  if (!row_scale || !col_scale) return fail(KAPY_ERR_INVALID, "matmul_scaled_f8: null scale array");
+  if (!is_f8(a8->dtype) || !is_f8(w8->dtype))
+    return fail(KAPY_ERR_VERIFY, "matmul: mma f8 operands must have f8E4M3 or f8E5M2 element type");
+  if (extent1(a8) != extent0(w8))
+    return fail(KAPY_ERR_VERIFY, "matmul: number of columns of lhs must be equal to number of rows of rhs");
+  if (extent0(result) != extent0(a8))
+    return fail(KAPY_ERR_VERIFY, "matmul: number of rows of acc must be equal to number of rows of lhs");
+  if (extent1(result) != extent1(w8))
+    return fail(KAPY_ERR_VERIFY, "matmul: number of columns of acc must be equal to number of columns of rhs");
+  if (result->dtype != KAPY_F16 && result->dtype != KAPY_BF16 && result->dtype != KAPY_F32)
+    return fail(KAPY_ERR_VERIFY, "matmul: result must have f16, bf16 or f32 element type");
+  for (const kapy_global *g : {a8, w8, result})
+    if (g->start0 < 0 || g->start1 < 0) return fail(KAPY_ERR_INVALID, "matmul: negative view start");
+  if (cfg && cfg->rmode != KAPY_RN && cfg->rmode != KAPY_RZ) return fail(KAPY_ERR_INVALID, "matmul: unknown rounding mode %d", cfg->rmode);
+  rc = ensure_device();
+  if (rc) return rc;
+  return matmul_f8(a8, w8, row_scale, col_scale, nullptr, result, cfg, (hipStream_t)stream);
+}

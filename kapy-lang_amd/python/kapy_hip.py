@@ -1,0 +1,244 @@
+"""ctypes binding of libkapy_hip.so for the test and benchmark harness.
+
+The product is the C ABI in include/kapy_hip.h; this module only loads it, declares argument
+types and offers a few conveniences around torch tensors (device memory and streams).  It never
+computes anything itself and has no fallback: a missing library is an ImportError, a failing call
+raises KapyError with the library's own message.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libkapy_hip.so")
+
+F16, BF16, F32, F8E4M3, F8E5M2, I8, I16, I32 = range(8)
+RZ, RN = 0, 1
+PAD_ZERO, PAD_QNAN, PAD_PINF, PAD_NINF = range(4)
+CACHE_NONE, CACHE_CA, CACHE_CG, CACHE_CS = 0, 1, 2, 3
+OK, ERR_INVALID, ERR_VERIFY, ERR_UNSUPPORTED, ERR_HIP = 0, -1, -2, -3, -4
+MATMUL_AUTO, MMA_M16N8K8_F16, MMA_M16N8K16_F16, MMA_M16N8K8_TF32, MMA_M16N8K16_F8 = 0, 1, 2, 3, 4
+MFMA_32X32X16_16B, MFMA_16X16X32_16B, MFMA_16X16X128_F8, MFMA_32X32X64_F8 = 16, 17, 18, 19
+DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, F8E4M3: 1, F8E5M2: 1, I8: 1, I16: 2, I32: 4}
+
+(EW_LD_GLOBAL, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
+ EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH,
+ EW_ST_GLOBAL) = range(22)
+
+EXPORTS = [
+    "kapy_version", "kapy_last_error", "kapy_device_info", "kapy_mk_global", "kapy_sv_global",
+    "kapy_fragments_loops", "kapy_fragments_map", "kapy_fragments_transpose", "kapy_fragments_exchange_axes",
+    "kapy_fragments_default", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
+    "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
+    "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
+    "kapy_change", "kapy_reduce",
+]
+
+
+class KapyError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("kapy status %d: %s" % (status, message))
+        self.status = status
+        self.message = message
+
+
+class Global(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("start0", C.c_int32), ("start1", C.c_int32), ("end0", C.c_int32),
+                ("end1", C.c_int32), ("stride0", C.c_int32), ("stride1", C.c_int32), ("dtype", C.c_int32),
+                ("alignment", C.c_int32)]
+
+
+class Fragments(C.Structure):
+    _fields_ = [("lane_array", C.c_int32 * 2), ("lane_loops", C.c_int32 * 2), ("minor_axis", C.c_int32),
+                ("major_axis", C.c_int32)]
+
+    @classmethod
+    def make(cls, lane_array, lane_loops, minor, major):
+        f = cls()
+        f.lane_array[:] = lane_array
+        f.lane_loops[:] = lane_loops
+        f.minor_axis, f.major_axis = minor, major
+        return f
+
+    def astuple(self):
+        return (list(self.lane_array), list(self.lane_loops), self.minor_axis, self.major_axis)
+
+
+class Swizzling(C.Structure):
+    _fields_ = [("stride0", C.c_int32), ("stride1", C.c_int32), ("bank_param", C.c_int32), ("line_param", C.c_int32)]
+
+
+class CopyCfg(C.Structure):
+    _fields_ = [("transpose", C.c_int32), ("padding_option", C.c_int32), ("cache_modifier", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
+class Grid2(C.Structure):
+    _fields_ = [("n0", C.c_int32), ("n1", C.c_int32), ("src_off0", C.c_int64), ("src_off1", C.c_int64),
+                ("dst_off0", C.c_int64), ("dst_off1", C.c_int64)]
+
+
+class EwInst(C.Structure):
+    _fields_ = [("op", C.c_int32), ("dst", C.c_int32), ("a", C.c_int32), ("b", C.c_int32), ("c", C.c_int32),
+                ("dtype", C.c_int32), ("rmode", C.c_int32), ("imm", C.c_float)]
+
+
+class MatmulCfg(C.Structure):
+    _fields_ = [("impl_way", C.c_int32), ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
+                ("rmode", C.c_int32), ("reserved", C.c_int32 * 3)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises ImportError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("%s is missing: build it with `make -C kapy-lang_amd` (there is no fallback path)" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    i64, i32, vp = C.c_int64, C.c_int32, C.c_void_p
+    P = C.POINTER
+    A2 = i64 * 2
+    L.kapy_version.restype = C.c_int
+    L.kapy_last_error.restype = C.c_char_p
+    L.kapy_device_info.argtypes = [P(i32), P(i32), P(i32), C.c_char_p, i32]
+    L.kapy_mk_global.argtypes = [P(Global), vp, i32, i32, i32, i32, i32, i32, i32]
+    L.kapy_sv_global.argtypes = [P(Global), P(Global), i32, i32, i32, i32]
+    L.kapy_fragments_loops.argtypes = [P(Fragments), A2, A2, A2]
+    L.kapy_fragments_map.argtypes = [P(Fragments), A2, i32, A2, A2]
+    L.kapy_fragments_transpose.argtypes = [P(Fragments), P(Fragments)]
+    L.kapy_fragments_exchange_axes.argtypes = [P(Fragments), P(Fragments)]
+    L.kapy_fragments_default.argtypes = [A2, A2, i32, P(Fragments)]
+    L.kapy_access_simd_size.restype = i64
+    L.kapy_access_simd_size.argtypes = [i64, i64, i64]
+    L.kapy_change_source.argtypes = [P(Fragments), P(Fragments), A2, i64, i64, P(i64), P(i64)]
+    L.kapy_change_num_shuffles.restype = i64
+    L.kapy_change_num_shuffles.argtypes = [P(Fragments), P(Fragments), A2]
+    L.kapy_swizzle_offset.restype = i64
+    L.kapy_swizzle_offset.argtypes = [P(Swizzling), i64, i64, i64]
+    L.kapy_swizzle_search.argtypes = [P(Fragments), A2, i64, i64, i64, i64, P(i32), i32]
+    L.kapy_matmul_layouts.argtypes = [i32, i32, P(Fragments), P(i32)]
+    L.kapy_matmul_lds_layout.argtypes = [i32, i32, P(Swizzling)]
+    L.kapy_copy.argtypes = [P(Global), P(Global), P(CopyCfg), vp]
+    L.kapy_copy_batched.argtypes = [P(Global), P(Global), P(CopyCfg), P(Grid2), vp]
+    L.kapy_elementwise.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), vp]
+    L.kapy_fptofp.argtypes = [P(Global), P(Global), i32, vp]
+    L.kapy_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
+    L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
+    L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
+    L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
+    for name in EXPORTS:
+        f = getattr(L, name)
+        if name not in ("kapy_last_error", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
+            f.restype = C.c_int
+    _lib = L
+    return L
+
+
+def last_error():
+    return lib().kapy_last_error().decode()
+
+
+def check(status):
+    if status < 0:
+        raise KapyError(status, last_error())
+    return status
+
+
+def A2(a, b):
+    return (C.c_int64 * 2)(a, b)
+
+
+# ---------------------------------------------------------------- descriptors
+def mk_global(ptr, size0, size1, stride0, stride1, dtype, dynamic_offset=0, alignment=16):
+    g = Global()
+    check(lib().kapy_mk_global(C.byref(g), C.c_void_p(ptr), dynamic_offset, size0, size1, stride0, stride1, dtype, alignment))
+    return g
+
+
+def sv_global(g, start0, end0, start1, end1):
+    r = Global()
+    check(lib().kapy_sv_global(C.byref(r), C.byref(g), start0, end0, start1, end1))
+    return r
+
+
+def tensor_global(t, dtype, size0=None, size1=None, stride0=None, stride1=None, dynamic_offset=0, alignment=16):
+    """Descriptor over a 2-D torch tensor's storage (any torch dtype of the right width)."""
+    if size0 is None:
+        size0, size1 = t.shape
+        stride0, stride1 = t.stride()
+    return mk_global(t.data_ptr(), size0, size1, stride0, stride1, dtype, dynamic_offset, alignment)
+
+
+def current_stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+# ---------------------------------------------------------------- ops
+def copy(src, dst, transpose=False, padding=PAD_ZERO, cache=CACHE_NONE, stream=None):
+    cfg = CopyCfg(int(transpose), padding, cache, 0)
+    check(lib().kapy_copy(C.byref(src), C.byref(dst), C.byref(cfg), stream if stream is not None else current_stream()))
+
+
+def copy_batched(src, dst, grid, transpose=False, padding=PAD_ZERO, cache=CACHE_NONE, stream=None):
+    cfg = CopyCfg(int(transpose), padding, cache, 0)
+    g = Grid2(*grid)
+    check(lib().kapy_copy_batched(C.byref(src), C.byref(dst), C.byref(cfg), C.byref(g),
+                                  stream if stream is not None else current_stream()))
+
+
+def program(insts):
+    arr = (EwInst * len(insts))()
+    for k, d in enumerate(insts):
+        arr[k] = EwInst(d["op"], d.get("dst", 0), d.get("a", 0), d.get("b", 0), d.get("c", 0), d.get("dtype", 0),
+                        d.get("rmode", RN), d.get("imm", 0.0))
+    return arr
+
+
+def gelu_program(out_dtype=F16, scale=0.5):
+    """y = GELU_tanh(x*scale + bias): ld x, ld bias, extf both, mulf by splat, addf, gelu, fptofp rn, st."""
+    return program([
+        dict(op=EW_LD_GLOBAL, dst=0, a=0),
+        dict(op=EW_LD_GLOBAL, dst=1, a=1),
+        dict(op=EW_FPTOFP, dst=2, a=0, dtype=F32),
+        dict(op=EW_FPTOFP, dst=3, a=1, dtype=F32),
+        dict(op=EW_SPLAT, dst=4, dtype=F32, imm=scale),
+        dict(op=EW_MULF, dst=2, a=2, b=4),
+        dict(op=EW_ADDF, dst=2, a=2, b=3),
+        dict(op=EW_GELU_TANH, dst=2, a=2),
+        dict(op=EW_FPTOFP, dst=5, a=2, dtype=out_dtype, rmode=RN),
+        dict(op=EW_ST_GLOBAL, a=5),
+    ])
+
+
+def elementwise(prog, ins, out, stream=None):
+    arr = (C.POINTER(Global) * max(len(ins), 1))(*[C.pointer(g) for g in ins])
+    check(lib().kapy_elementwise(prog, len(prog), arr, len(ins), C.byref(out),
+                                 stream if stream is not None else current_stream()))
+
+
+def fptofp(src, dst, rmode=RN, stream=None):
+    check(lib().kapy_fptofp(C.byref(src), C.byref(dst), rmode, stream if stream is not None else current_stream()))
+
+
+def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stream=None):
+    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode)
+    check(lib().kapy_matmul(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
+                            C.byref(cfg), stream if stream is not None else current_stream()))
+
+
+def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, stream=None):
+    check(lib().kapy_matmul_scaled_f8(C.byref(a8), C.byref(w8), C.c_void_p(row_scale_ptr), C.c_void_p(col_scale_ptr),
+                                      C.byref(result), None, stream if stream is not None else current_stream()))
+
+
+def reduce(src, dst, axis, kind=0, stream=None):
+    check(lib().kapy_reduce(C.byref(src), C.byref(dst), axis, kind, stream if stream is not None else current_stream()))
+
+
+def change(in_ptr, src, dst, shape, out_ptr, stream=None):
+    check(lib().kapy_change(C.c_void_p(in_ptr), C.byref(src), C.byref(dst), A2(*shape), C.c_void_p(out_ptr),
+                            stream if stream is not None else current_stream()))

@@ -1,0 +1,166 @@
+"""GPU parity for the layout moves (ld_global -> [transpose] -> st_global): bit-exact against the
+oracle on small / ragged / strided cases and against closed forms at the BASELINE sizes."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+NP = {1: np.uint8, 2: np.uint16, 4: np.uint32}
+
+
+def _rand(n, itemsize, seed):
+    rng = np.random.default_rng(seed)
+    return rng.integers(0, 2 ** (8 * itemsize), size=n, dtype=np.uint64).astype(NP[itemsize])
+
+
+CASES = [
+    # (dtype, src_shape(m,n), transpose, use swapped strides, view (s0,e0,s1,e1) or None)
+    (kh.F16, (64, 64), True, False, None),
+    (kh.F16, (128, 192), True, False, None),
+    (kh.BF16, (37, 53), True, False, None),           # ragged: generic + edge tiles
+    (kh.F16, (200, 136), True, False, None),          # interior tiles + ragged edges (136 % 8 == 0)
+    (kh.F16, (128, 128), False, True, None),          # transpose expressed by swapped source strides
+    (kh.F32, (96, 160), True, False, None),
+    (kh.F8E4M3, (256, 384), True, False, None),
+    (kh.I8, (130, 70), True, False, None),
+    (kh.F16, (77, 129), False, False, None),          # plain ragged row copy
+    (kh.F32, (64, 256), False, False, (3, 60, 8, 200)),  # sub-view copy
+    (kh.F16, (256, 256), True, False, (64, 192, 32, 160)),
+]
+
+
+@pytest.mark.parametrize("dtype,shape,transpose,swapped,view", CASES)
+def test_copy_matches_oracle(ko, dtype, shape, transpose, swapped, view):
+    b = kh.DTYPE_BYTES[dtype]
+    m, n = shape
+    src = _rand(m * n, b, 7).reshape(m, n)
+    if swapped:
+        ssz, sst = (n, m), (1, n)
+    else:
+        ssz, sst = (m, n), (n, 1)
+    logical = (ssz[1], ssz[0]) if transpose else ssz
+    dm, dn = logical
+    d_src = to_dev(src)
+    want = np.full((dm, dn), 0x5A, dtype=NP[b]) if b == 1 else np.full((dm, dn), 0x5A5A, dtype=NP[b])
+    d_dst = to_dev(want)
+    gs_o, gd_o = ko.mk_global(src, ssz[0], ssz[1], sst[0], sst[1], dtype), ko.mk_global(want, dm, dn, dn, 1, dtype)
+    gs_d, gd_d = dglobal(d_src, ssz[0], ssz[1], sst[0], sst[1], dtype), dglobal(d_dst, dm, dn, dn, 1, dtype)
+    if view:
+        s0, e0, s1, e1 = view
+        vs = (s1, e1, s0, e0) if transpose else view
+        gs_o, gs_d = ko.sv_global(gs_o, *vs), kh.sv_global(gs_d, *vs)
+        gd_o, gd_d = ko.sv_global(gd_o, *view), kh.sv_global(gd_d, *view)
+    assert ko.lib().ko_copy(C.byref(gs_o), C.byref(gd_o), int(transpose), 0) == 0
+    kh.copy(gs_d, gd_d, transpose=transpose)
+    sync()
+    got = to_host(d_dst, NP[b], (dm, dn))
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("pad", [kh.PAD_ZERO, kh.PAD_QNAN, kh.PAD_PINF, kh.PAD_NINF])
+def test_padding_for_out_of_bounds_source(ko, pad):
+    """Destination larger than the source view: the excess reads as the padding pattern."""
+    src = _rand(40 * 48, 2, 3).reshape(40, 48)
+    want = np.zeros((64, 64), dtype=np.uint16)
+    d_src, d_dst = to_dev(src), dev_zeros(64 * 64, 2, 0x1111)
+    for tr in (False, True):
+        ssz = (48, 40) if tr else (40, 48)
+        so = ko.mk_global(src, 40, 48, 48, 1, ko.BF16)
+        sd = dglobal(d_src, 40, 48, 48, 1, kh.BF16)
+        assert ko.lib().ko_copy(C.byref(so), C.byref(ko.mk_global(want, 64, 64, 64, 1, ko.BF16)), int(tr), pad) == 0
+        kh.copy(sd, dglobal(d_dst, 64, 64, 64, 1, kh.BF16), transpose=tr, padding=pad)
+        sync()
+        assert np.array_equal(to_host(d_dst, np.uint16, (64, 64)), want)
+        assert want[ssz[0]:, :].min() == want[ssz[0]:, :].max() == {0: 0, 1: 0x7FC0, 2: 0x7F80, 3: 0xFF80}[pad]
+
+
+def test_column_major_destination_and_no_contiguous_axis(ko):
+    src = _rand(96 * 80, 2, 11).reshape(96, 80)
+    d_src = to_dev(src)
+    # destination column-major (stride0 == 1): same-axis copy in the transposed orientation
+    want = np.zeros((80, 96), dtype=np.uint16)   # holds dst^T
+    d_dst = dev_zeros(80 * 96, 2)
+    ko.lib().ko_copy(C.byref(ko.mk_global(src, 96, 80, 80, 1, 0)), C.byref(ko.mk_global(want, 96, 80, 1, 96, 0)), 0, 0)
+    kh.copy(dglobal(d_src, 96, 80, 80, 1, kh.F16), dglobal(d_dst, 96, 80, 1, 96, kh.F16))
+    sync()
+    assert np.array_equal(to_host(d_dst, np.uint16, (80, 96)), want) and np.array_equal(want, src.T)
+    # every-other-element destination: no contiguous axis -> generic kernel
+    want2 = np.zeros(96 * 80 * 2, dtype=np.uint16)
+    d_dst2 = dev_zeros(96 * 80 * 2, 2)
+    ko.lib().ko_copy(C.byref(ko.mk_global(src, 96, 80, 80, 1, 0)), C.byref(ko.mk_global(want2, 96, 80, 160, 2, 0)), 0, 0)
+    kh.copy(dglobal(d_src, 96, 80, 80, 1, kh.F16), dglobal(d_dst2, 96, 80, 160, 2, kh.F16))
+    sync()
+    assert np.array_equal(to_host(d_dst2, np.uint16), want2)
+
+
+def test_empty_views_are_no_ops():
+    d = dev_zeros(64, 2, 0x7777)
+    g = dglobal(d, 8, 8, 8, 1, kh.F16)
+    kh.copy(kh.sv_global(g, 2, 2, 0, 8), kh.sv_global(g, 4, 4, 0, 8))
+    kh.copy(g, kh.sv_global(g, 0, 8, 3, 3), transpose=True)
+    sync()
+    assert np.all(to_host(d, np.uint16) == 0x7777)
+
+
+def test_bhsd_permute_small_matches_oracle(ko):
+    b, h, s, d = 2, 3, 40, 64
+    src = ko.fill_bits16(b * h * s * d, 1).reshape(b, h, s, d)
+    want = np.zeros((b, s, h, d), dtype=np.uint16)
+    ko.lib().ko_copy_batched(C.byref(ko.mk_global(src, s, d, d, 1, ko.BF16)), C.byref(ko.mk_global(want, s, d, h * d, 1, ko.BF16)),
+                             0, 0, b, h, h * s * d, s * d, s * h * d, d)
+    d_src, d_dst = to_dev(src), dev_zeros(b * s * h * d, 2)
+    kh.copy_batched(dglobal(d_src, s, d, d, 1, kh.BF16), dglobal(d_dst, s, d, h * d, 1, kh.BF16),
+                    (b, h, h * s * d, s * d, s * h * d, d))
+    sync()
+    got = to_host(d_dst, np.uint16, (b, s, h, d))
+    assert np.array_equal(got, want) and np.array_equal(got, src.transpose(0, 2, 1, 3))
+
+
+def test_config3a_transpose_8192_bit_exact(ko):
+    """BASELINE config 3a: fp16 8192x8192 (i,j)->(j,i), random 16-bit patterns from seed 0."""
+    n = 8192
+    src = ko.fill_bits16(n * n, 0).reshape(n, n)
+    d_src, d_dst = to_dev(src), dev_zeros(n * n, 2)
+    gs, gd = dglobal(d_src, n, n, n, 1, kh.F16), dglobal(d_dst, n, n, n, 1, kh.F16)
+    kh.copy(gs, gd, transpose=True)
+    sync()
+    got = to_host(d_dst, np.uint16, (n, n))
+    assert np.array_equal(got, src.T)                      # closed form: out[j,i] = in[i,j]
+    assert int(np.bitwise_xor.reduce(got.ravel())) == int(np.bitwise_xor.reduce(src.ravel()))
+    # oracle on a band of destination rows (sub-views of both sides)
+    want = np.zeros((64, n), dtype=np.uint16)
+    so = ko.sv_global(ko.mk_global(src, n, n, n, 1, ko.F16), 0, n, 4096, 4160)
+    assert ko.lib().ko_copy(C.byref(so), C.byref(ko.mk_global(want, 64, n, n, 1, ko.F16)), 1, 0) == 0
+    assert np.array_equal(got[4096:4160], want)
+    # involution: transposing again restores the input bit for bit
+    kh.copy(gd, gs, transpose=True)
+    sync()
+    assert np.array_equal(to_host(d_src, np.uint16, (n, n)), src)
+    # the same move expressed with swapped source strides
+    d_dst.zero_()
+    kh.copy(dglobal(d_src, n, n, 1, n, kh.F16), gd)
+    sync()
+    assert np.array_equal(to_host(d_dst, np.uint16, (n, n)), src.T)
+
+
+def test_config3b_permute_bhsd_bit_exact(ko):
+    """BASELINE config 3b: bf16 [8,32,2048,128] (b,h,s,d)->(b,s,h,d), random bits from seed 1."""
+    b, h, s, d = 8, 32, 2048, 128
+    src = ko.fill_bits16(b * h * s * d, 1).reshape(b, h, s, d)
+    d_src, d_dst = to_dev(src), dev_zeros(b * h * s * d, 2)
+    kh.copy_batched(dglobal(d_src, s, d, d, 1, kh.BF16), dglobal(d_dst, s, d, h * d, 1, kh.BF16),
+                    (b, h, h * s * d, s * d, s * h * d, d))
+    sync()
+    got = to_host(d_dst, np.uint16, (b, s, h, d))
+    assert np.array_equal(got, src.transpose(0, 2, 1, 3))
+    # and back: (b,s,h,d) -> (b,h,s,d)
+    d_back = dev_zeros(b * h * s * d, 2)
+    kh.copy_batched(dglobal(d_dst, s, d, h * d, 1, kh.BF16), dglobal(d_back, s, d, d, 1, kh.BF16),
+                    (b, h, s * h * d, d, h * s * d, s * d))
+    sync()
+    assert np.array_equal(to_host(d_back, np.uint16, (b, h, s, d)), src)

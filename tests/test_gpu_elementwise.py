@@ -1,0 +1,184 @@
+"""GPU parity for fused elementwise programs: max |err| <= 2 ulp of the 16-bit result type against
+the oracle (tolerance stated by BASELINE north_star), bit-exact where the op is exactly rounded."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host, ulp_diff_f16
+
+pytestmark = pytest.mark.gpu
+ULP_TOL = 2
+
+
+def _check_ulp(got, want, dtype):
+    f = (lambda a: a.view(np.float16).astype(np.float64)) if dtype == kh.F16 else \
+        (lambda a: (a.astype(np.uint32) << 16).view(np.float32).astype(np.float64))
+    gn, wn = np.isnan(f(got)), np.isnan(f(want))
+    assert np.array_equal(gn, wn)
+    d = ulp_diff_f16(got[~gn], want[~wn])
+    assert d.max(initial=0) <= ULP_TOL, "max ulp error %d" % d.max()
+    return d
+
+
+def _gelu_case(ko, dtype, m, n, seed, specials=False):
+    x = ko.fill_normal(m * n, dtype, seed, 0).reshape(m, n)
+    bias = ko.fill_normal(n, dtype, seed + 1, 0)
+    if specials:
+        enc = (lambda v: np.array(v, dtype=np.float16).view(np.uint16)) if dtype == kh.F16 else \
+            (lambda v: (np.array(v, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16))
+        sp = enc([0.0, -0.0, np.inf, -np.inf, np.nan, 60000.0, -60000.0, 1e-7, -8.0, 8.0, -3.0, 3.0])
+        x.ravel()[:len(sp)] = sp
+        bias[:len(sp)] = 0
+    want = np.zeros((m, n), dtype=np.uint16)
+    go = ko.mk_global(want, m, n, n, 1, dtype)
+    assert ko.elementwise(ko.gelu_program(dtype, dtype), [ko.mk_global(x, m, n, n, 1, dtype), ko.mk_global(bias, 1, n, n, 1, dtype)], go) == 0
+    dx, db, dy = to_dev(x), to_dev(bias), dev_zeros(m * n, 2)
+    kh.elementwise(kh.gelu_program(dtype), [dglobal(dx, m, n, n, 1, dtype), dglobal(db, 1, n, n, 1, dtype)], dglobal(dy, m, n, n, 1, dtype))
+    sync()
+    return to_host(dy, np.uint16, (m, n)), want
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(64, 256), (33, 1000), (7, 24)])
+def test_gelu_bias_scale_fused(ko, dtype, m, n):
+    got, want = _gelu_case(ko, dtype, m, n, 0, specials=True)
+    _check_ulp(got, want, dtype)
+
+
+def test_gelu_unaligned_shape_takes_the_interpreter(ko):
+    got, want = _gelu_case(ko, kh.F16, 19, 37, 5)   # 37 % 8 != 0: not the vector path
+    _check_ulp(got, want, kh.F16)
+
+
+def test_config2_gelu_8192_sampled_against_oracle(ko):
+    """BASELINE config 2: y = GELU_tanh(x*0.5 + bias), x fp16 8192x8192 normal(0,1) seed 0, bias seed 1.
+    The whole result is produced on the GPU; the oracle checks 64 full rows spread over the matrix, and
+    a row-broadcast invariant (rows with equal x rows give equal y rows) covers the rest."""
+    n = 8192
+    x = ko.fill_normal(n * n, ko.F16, 0, 0).reshape(n, n)
+    bias = ko.fill_normal(n, ko.F16, 1, 0)
+    x[5000] = x[17]                                    # planted duplicate row
+    dx, db, dy = to_dev(x), to_dev(bias), dev_zeros(n * n, 2)
+    kh.elementwise(kh.gelu_program(kh.F16), [dglobal(dx, n, n, n, 1, kh.F16), dglobal(db, 1, n, n, 1, kh.F16)],
+                   dglobal(dy, n, n, n, 1, kh.F16))
+    sync()
+    got = to_host(dy, np.uint16, (n, n))
+    rows = np.unique(np.concatenate([np.arange(0, n, 131), [n - 1, 17, 5000]]))
+    xs = np.ascontiguousarray(x[rows])
+    want = np.zeros_like(xs)
+    m = len(rows)
+    assert ko.elementwise(ko.gelu_program(), [ko.mk_global(xs, m, n, n, 1, ko.F16), ko.mk_global(bias, 1, n, n, 1, ko.F16)],
+                          ko.mk_global(want, m, n, n, 1, ko.F16)) == 0
+    d = _check_ulp(got[rows], want, kh.F16)
+    assert (d > 0).mean() < 0.02                       # almost every element is bit-identical
+    assert np.array_equal(got[5000], got[17])
+    assert not np.any(np.isnan(got.view(np.float16)))
+
+
+def _run_prog(ko, insts, ins_np, in_dtypes, out_dtype, m, n, in_shapes=None):
+    outb = kh.DTYPE_BYTES[out_dtype]
+    np_out = {1: np.uint8, 2: np.uint16, 4: np.uint32}[outb]
+    want = np.zeros((m, n), dtype=np_out)
+    in_shapes = in_shapes or [(m, n)] * len(ins_np)
+    gos = [ko.mk_global(a, s[0], s[1], s[1], 1, dt) for a, s, dt in zip(ins_np, in_shapes, in_dtypes)]
+    assert ko.elementwise(ko.program(insts), gos, ko.mk_global(want, m, n, n, 1, out_dtype)) == 0
+    devs = [to_dev(a) for a in ins_np]
+    dout = dev_zeros(m * n, outb)
+    kh.elementwise(kh.program(insts), [dglobal(t, s[0], s[1], s[1], 1, dt) for t, s, dt in zip(devs, in_shapes, in_dtypes)],
+                   dglobal(dout, m, n, n, 1, out_dtype))
+    sync()
+    return to_host(dout, np_out, (m, n)), want
+
+
+def test_bf16_and_f16_arithmetic_is_exactly_rounded(ko):
+    m, n = 32, 96
+    for dt in (kh.BF16, kh.F16):
+        a = ko.fill_normal(m * n, dt, 2, 0).reshape(m, n)
+        b = ko.fill_normal(m * n, dt, 2, 1).reshape(m, n)
+        insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1),
+                 dict(op=kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ADDF, dst=2, a=2, b=0),
+                 dict(op=kh.EW_SUBF, dst=3, a=2, b=1), dict(op=kh.EW_MAXIMUMF, dst=3, a=3, b=0),
+                 dict(op=kh.EW_FMA, dst=3, a=3, b=1, c=0), dict(op=kh.EW_ST_GLOBAL, a=3)]
+        got, want = _run_prog(ko, insts, [a, b], [dt, dt], dt, m, n)
+        assert np.array_equal(got, want)       # +,-,*,max,fma: one rounding each, bit-exact
+
+
+def test_explicit_tanh_chain_equals_the_fused_gelu_within_tolerance(ko):
+    """GELU written out in kapy ops (mulf/addf/fma/tanh) against the oracle of the same chain."""
+    m, n = 16, 256
+    x = ko.fill_normal(m * n, kh.F16, 9, 0).reshape(m, n)
+    c = lambda r, v: dict(op=kh.EW_SPLAT, dst=r, dtype=kh.F32, imm=v)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_FPTOFP, dst=1, a=0, dtype=kh.F32),
+             dict(op=kh.EW_MULF, dst=2, a=1, b=1), dict(op=kh.EW_MULF, dst=2, a=2, b=1),     # v^3
+             c(3, 0.044715), dict(op=kh.EW_FMA, dst=2, a=2, b=3, c=1),                       # v + 0.044715 v^3
+             c(3, 0.7978845608028654), dict(op=kh.EW_MULF, dst=2, a=2, b=3),
+             dict(op=kh.EW_TANH, dst=2, a=2), c(3, 1.0), dict(op=kh.EW_ADDF, dst=2, a=2, b=3),
+             c(3, 0.5), dict(op=kh.EW_MULF, dst=4, a=1, b=3), dict(op=kh.EW_MULF, dst=2, a=2, b=4),
+             dict(op=kh.EW_FPTOFP, dst=5, a=2, dtype=kh.F16, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=5)]
+    got, want = _run_prog(ko, insts, [x], [kh.F16], kh.F16, m, n)
+    _check_ulp(got, want, kh.F16)
+
+
+@pytest.mark.parametrize("op", [kh.EW_EXP, kh.EW_EXP2, kh.EW_LOG, kh.EW_LOG2, kh.EW_SQRT, kh.EW_RSQRT, kh.EW_TANH,
+                                kh.EW_ERF, kh.EW_ABSF, kh.EW_NEGF, kh.EW_GELU_TANH])
+def test_unary_math_ops_within_2_ulp_of_16bit_result(ko, op):
+    m, n = 8, 512
+    x = ko.fill_uniform(m * n, kh.F16, 4, 0, 0.01 if op in (kh.EW_LOG, kh.EW_LOG2, kh.EW_SQRT, kh.EW_RSQRT) else -6.0, 6.0).reshape(m, n)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_FPTOFP, dst=1, a=0, dtype=kh.F32),
+             dict(op=op, dst=1, a=1), dict(op=kh.EW_FPTOFP, dst=2, a=1, dtype=kh.F16, rmode=kh.RN),
+             dict(op=kh.EW_ST_GLOBAL, a=2)]
+    got, want = _run_prog(ko, insts, [x], [kh.F16], kh.F16, m, n)
+    _check_ulp(got, want, kh.F16)
+
+
+@pytest.mark.parametrize("src,dst,rmode", [(kh.F32, kh.F16, kh.RN), (kh.F32, kh.F16, kh.RZ), (kh.F32, kh.BF16, kh.RN),
+                                           (kh.F32, kh.BF16, kh.RZ), (kh.F32, kh.F8E4M3, kh.RN), (kh.F32, kh.F8E5M2, kh.RN),
+                                           (kh.F16, kh.F8E4M3, kh.RN), (kh.F16, kh.F8E5M2, kh.RZ), (kh.BF16, kh.F8E4M3, kh.RN),
+                                           (kh.F8E4M3, kh.F16, kh.RN), (kh.F8E5M2, kh.BF16, kh.RN), (kh.F8E4M3, kh.F32, kh.RN),
+                                           (kh.F16, kh.F32, kh.RN), (kh.BF16, kh.F32, kh.RN)])
+def test_fptofp_bit_exact(ko, src, dst, rmode):
+    """kapy.fptofp over whole tensors: every cast is an exactly-rounded op, so results are bit-exact."""
+    m, n = 64, 1024
+    sb, db = kh.DTYPE_BYTES[src], kh.DTYPE_BYTES[dst]
+    if sb == 1:
+        x = (np.arange(m * n) % 256).astype(np.uint8)
+    elif sb == 2:
+        x = np.arange(m * n, dtype=np.uint32).astype(np.uint16)            # every 16-bit pattern
+    else:
+        rng = np.random.default_rng(0)
+        x = np.concatenate([rng.normal(0, 1, m * n // 2), rng.normal(0, 300, m * n // 4),
+                            rng.normal(0, 1e-3, m * n // 4)]).astype(np.float32)
+        x[:8] = [0, -0.0, np.inf, -np.inf, np.nan, 448.0, 464.0, 57344.0]
+        h = np.arange(0, 0x7F, dtype=np.uint8)                             # e4m3 midpoints: ties
+        v = np.array([ko.lib().ko_e4m3_to_f64(int(b)) for b in h])
+        x[8:8 + len(v) - 1] = ((v[:-1] + v[1:]) / 2).astype(np.float32)
+    want = ko.fptofp(x, src, dst, rmode)
+    dx, dy = to_dev(x), dev_zeros(m * n, db)
+    kh.fptofp(dglobal(dx, m, n, n, 1, src), dglobal(dy, m, n, n, 1, dst), rmode)
+    sync()
+    got = to_host(dy, want.dtype)
+    if dst in (kh.F16, kh.BF16, kh.F32) and src != kh.F32:
+        pass
+    wf, gf = ko.decode(want, dst), ko.decode(got.view(want.dtype), dst)
+    nan = np.isnan(wf)
+    assert np.array_equal(np.isnan(gf), nan)
+    assert np.array_equal(got.view(want.dtype)[~nan], want[~nan])
+
+
+def test_broadcast_column_vector_and_padding(ko):
+    m, n = 48, 64
+    x = ko.fill_normal(m * n, kh.F16, 1, 0).reshape(m, n)
+    col = ko.fill_normal(m, kh.F16, 1, 1)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1),
+             dict(op=kh.EW_ADDF, dst=2, a=0, b=1), dict(op=kh.EW_ST_GLOBAL, a=2)]
+    got, want = _run_prog(ko, insts, [x, col], [kh.F16, kh.F16], kh.F16, m, n, in_shapes=[(m, n), (m, 1)])
+    assert np.array_equal(got, want)
+    # column-broadcast bias through the fused path
+    prog = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1),
+            dict(op=kh.EW_FPTOFP, dst=2, a=0, dtype=kh.F32), dict(op=kh.EW_FPTOFP, dst=3, a=1, dtype=kh.F32),
+            dict(op=kh.EW_ADDF, dst=2, a=2, b=3), dict(op=kh.EW_EXP, dst=2, a=2),
+            dict(op=kh.EW_FPTOFP, dst=4, a=2, dtype=kh.F16, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=4)]
+    got, want = _run_prog(ko, prog, [x, col], [kh.F16, kh.F16], kh.F16, m, n, in_shapes=[(m, n), (m, 1)])
+    _check_ulp(got, want, kh.F16)

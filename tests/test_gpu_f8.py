@@ -1,0 +1,107 @@
+"""GPU parity for fp8 (OCP E4M3FN / E5M2) matmuls with fp32 row/column scales (BASELINE config 5)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+FROB_TOL = 1e-3
+vp = lambda x: x.ctypes.data_as(C.c_void_p)
+
+
+def _quantised(ko, M, N, K, seed=0):
+    a = ko.fill_normal(M * K, ko.F32, seed, 0).reshape(M, K)
+    w = ko.fill_normal(N * K, ko.F32, seed + 1, 0).reshape(N, K)   # W stored K-contiguous per output column
+    aq, sa = np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+    wq, sb = np.zeros((N, K), np.uint8), np.zeros(N, np.float32)
+    ko.lib().ko_quantize_e4m3(vp(a), M, K, K, 1, 1, vp(aq), vp(sa))
+    ko.lib().ko_quantize_e4m3(vp(w), N, K, K, 1, 1, vp(wq), vp(sb))
+    return aq, sa, wq, sb
+
+
+def _frob(ko, got, want, dt=kh.BF16):
+    g, w = ko.decode(got, dt), ko.decode(want, dt)
+    assert np.all(np.isfinite(g))
+    return np.linalg.norm(g - w) / np.linalg.norm(w)
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 64, 128), (16, 256, 1024), (5, 48, 256), (33, 100, 384), (64, 64, 512)])
+def test_scaled_f8_small(ko, M, N, K):
+    aq, sa, wq, sb = _quantised(ko, M, N, K)
+    want = np.zeros((M, N), dtype=np.uint16)
+    rc = ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                      vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16)))
+    assert rc == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N, 2)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    assert _frob(ko, to_host(dd, np.uint16, (M, N)), want) <= FROB_TOL
+
+
+def test_plain_f8_matmul_mixed_formats_and_fallback(ko):
+    """kapy.matmul on f8 operands without scales: e4m3 x e5m2 mix (Kapy.cpp:484-487), f32 result; and an
+    operand layout only the element-wise kernel serves (row-major rhs)."""
+    M, N, K = 32, 48, 256
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    a[(a & 0x7F) == 0x7F] = 0x30                      # no NaN patterns (e4m3fn)
+    b = rng.integers(0, 256, size=(N, K)).astype(np.uint8)
+    b[(b & 0x7C) == 0x7C] = 0x3C                      # no inf/NaN patterns (e5m2)
+    want = np.zeros((M, N), dtype=np.float32)
+    assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(b, K, N, 1, K, ko.F8E5M2)), None,
+                              C.byref(ko.mk_global(want, M, N, N, 1, ko.F32)), ko.RN) == 0
+    da, db, dd = to_dev(a), to_dev(b), dev_zeros(M * N, 4)
+    kh.matmul(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(db, K, N, 1, K, kh.F8E5M2), dglobal(dd, M, N, N, 1, kh.F32))
+    sync()
+    got = to_host(dd, np.float32, (M, N))
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-5
+    # rhs row-major (N contiguous): naive kernel
+    bk = np.ascontiguousarray(b.T)                     # [K, N] row-major, same logical matrix
+    dbk = to_dev(bk)
+    dd.zero_()
+    kh.matmul(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dbk, K, N, N, 1, kh.F8E5M2), dglobal(dd, M, N, N, 1, kh.F32))
+    sync()
+    got2 = to_host(dd, np.float32, (M, N))
+    assert np.linalg.norm(got2 - want) / np.linalg.norm(want) <= 1e-5
+
+
+def test_config5_decode_shape_m16(ko):
+    """BASELINE config 5, M = 16: N = K = 8192, scales amax/448, bf16 out; full oracle check."""
+    M, N, K = 16, 8192, 8192
+    aq, sa, wq, sb = _quantised(ko, M, N, K)
+    want = np.zeros((M, N), dtype=np.uint16)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                        vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16))) == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N, 2)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    assert _frob(ko, to_host(dd, np.uint16, (M, N)), want) <= FROB_TOL
+
+
+def test_config5_m4096_sampled(ko):
+    """BASELINE config 5, M = 4096: oracle on 64x64 blocks spread over the result."""
+    M, N, K = 4096, 8192, 8192
+    aq, sa, wq, sb = _quantised(ko, M, N, K)
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N, 2)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    got = to_host(dd, np.uint16, (M, N))
+    goa, gow = ko.mk_global(aq, M, K, K, 1, ko.F8E4M3), ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)
+    num = den = 0.0
+    blk = 64
+    for t in range(16):
+        r0, c0 = (t * 256 + 29 * t) % (M - blk), ((15 - t) * 512 + 71 * t) % (N - blk)
+        want = np.zeros((blk, blk), dtype=np.uint16)
+        rs, cs = np.ascontiguousarray(sa[r0:r0 + blk]), np.ascontiguousarray(sb[c0:c0 + blk])
+        assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.sv_global(goa, r0, r0 + blk, 0, K)), C.byref(ko.sv_global(gow, 0, K, c0, c0 + blk)),
+                                            vp(rs), vp(cs), C.byref(ko.mk_global(want, blk, blk, blk, 1, ko.BF16))) == 0
+        g, w = ko.decode(got[r0:r0 + blk, c0:c0 + blk], ko.BF16), ko.decode(want, ko.BF16)
+        num += ((g - w) ** 2).sum()
+        den += (w ** 2).sum()
+    assert np.sqrt(num / den) <= FROB_TOL

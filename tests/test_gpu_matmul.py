@@ -1,0 +1,164 @@
+"""GPU parity for kapy.matmul: relative Frobenius error <= 1e-3 against the oracle's fp64-accumulated
+result (tolerance stated by BASELINE north_star), closed forms bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+FROB_TOL = 1e-3
+
+
+def _frob(ko, got, want, dtype):
+    g, w = ko.decode(got, dtype), ko.decode(want, dtype)
+    assert np.all(np.isfinite(g))
+    return np.linalg.norm(g - w) / max(np.linalg.norm(w), 1e-30)
+
+
+def _np_store(dtype):
+    return {1: np.uint8, 2: np.uint16, 4: np.float32}[kh.DTYPE_BYTES[dtype]]
+
+
+def _run(ko, dt, M, N, K, a_row_major=True, b_row_major=True, out_dtype=None, with_acc=None, d_col_major=False,
+         seed=0, gen="uniform", rmode=kh.RN, tile=(0, 0, 0)):
+    out_dtype = dt if out_dtype is None else out_dtype
+    fill = (lambda n, s: ko.fill_uniform(n, dt, seed, s)) if gen == "uniform" else (lambda n, s: ko.fill_normal(n, dt, seed, s, 0.0, 0.02))
+    a, b = fill(M * K, 0), fill(K * N, 1)
+    a_str = (K, 1) if a_row_major else (1, M)
+    b_str = (N, 1) if b_row_major else (1, K)
+    d_str = (1, M) if d_col_major else (N, 1)
+    want = np.zeros(M * N, dtype=_np_store(out_dtype))
+    acc = None
+    da, db, dd = to_dev(a), to_dev(b), dev_zeros(M * N, kh.DTYPE_BYTES[out_dtype])
+    go_acc = gd_acc = None
+    if with_acc is not None:
+        acc = ko.fill_normal(M * N, with_acc, seed, 2)
+        dacc = to_dev(acc)
+        go_acc, gd_acc = ko.mk_global(acc, M, N, N, 1, with_acc), dglobal(dacc, M, N, N, 1, with_acc)
+    rc = ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, *a_str, dt)), C.byref(ko.mk_global(b, K, N, *b_str, dt)),
+                            C.byref(go_acc) if go_acc is not None else None, C.byref(ko.mk_global(want, M, N, *d_str, out_dtype)), rmode)
+    assert rc == 0
+    kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(dd, M, N, *d_str, out_dtype), acc=gd_acc,
+              rmode=rmode, tile=tile)
+    sync()
+    return to_host(dd, want.dtype), want
+
+
+def test_config1_fp16_1024_row_major_128x128x32_tiles(ko):
+    """BASELINE config 1: fp16 GEMM 1024^3, row-major A and B, fp32 accumulate, fp16 out, uniform[-1,1) seed 0."""
+    got, want = _run(ko, kh.F16, 1024, 1024, 1024, True, True, tile=(128, 128, 32))
+    assert _frob(ko, got, want, kh.F16) <= FROB_TOL
+    assert (got != want).mean() < 0.05    # fp32 vs fp64 accumulation flips few roundings
+
+
+@pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("a_rm,b_rm", [(True, True), (True, False), (False, True), (False, False)])
+def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):
+    for (M, N, K) in ((128, 128, 64), (200, 136, 72), (16, 8, 16), (130, 257, 100)):
+        got, want = _run(ko, dt, M, N, K, a_rm, b_rm, seed=3)
+        assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
+
+
+def test_tn_roofline_kernel_small(ko):
+    """lhs row-major, rhs column-major, multiples of the 256x256x32 tile: the LDS-direct kernel."""
+    for dt in (kh.BF16, kh.F16):
+        for (M, N, K) in ((256, 256, 32), (256, 256, 64), (256, 512, 96), (512, 256, 128), (768, 512, 1024)):
+            got, want = _run(ko, dt, M, N, K, True, False, seed=5)
+            assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
+            got32, want32 = _run(ko, dt, M, N, K, True, False, out_dtype=kh.F32, seed=5)
+            assert _frob(ko, got32, want32, kh.F32) <= 1e-5, (M, N, K)
+
+
+def test_closed_forms_identity_ones_rank1(ko):
+    n = 256
+    eye = np.eye(n, dtype=np.float16).view(np.uint16)
+    b = ko.fill_uniform(n * n, kh.F16, 4)
+    d_eye, d_b, d_out = to_dev(eye), to_dev(b), dev_zeros(n * n, 2)
+    g = lambda t, s=(n, 1): dglobal(t, n, n, s[0], s[1], kh.F16)
+    kh.matmul(g(d_eye), g(d_b), g(d_out))                           # staged kernel: I·B = B
+    sync()
+    assert np.array_equal(to_host(d_out, np.uint16), b)
+    kh.matmul(g(d_eye), g(d_b, (1, n)), g(d_out))                   # TN kernel: I·(B^T as col-major) = B^T
+    sync()
+    assert np.array_equal(to_host(d_out, np.uint16, (n, n)), b.reshape(n, n).T)
+    ones = np.ones(n * n, dtype=np.float16).view(np.uint16)
+    d_ones = to_dev(ones)
+    kh.matmul(g(d_ones), g(d_ones, (1, n)), g(d_out))
+    sync()
+    assert np.all(to_host(d_out, np.uint16).view(np.float16) == n)  # all-ones -> K
+    u = (np.arange(n) % 7 + 1).astype(np.float16)
+    a1 = np.outer(u, np.ones(n)).astype(np.float16).view(np.uint16)
+    b1t = np.outer(u, np.ones(n)).astype(np.float16).view(np.uint16)  # column-major rhs: (k,n) at n*K+k -> rhs[k,n] = u[n]
+    d32 = dev_zeros(n * n, 4)
+    kh.matmul(g(to_dev(a1)), g(to_dev(b1t), (1, n)), dglobal(d32, n, n, n, 1, kh.F32))
+    sync()
+    assert np.array_equal(to_host(d32, np.float32, (n, n)), n * np.outer(u, u).astype(np.float32))
+
+
+def test_accumulator_input_f32_out_and_column_major_result(ko):
+    got, want = _run(ko, kh.BF16, 256, 256, 128, True, False, out_dtype=kh.F32, with_acc=kh.F32, seed=8)
+    assert _frob(ko, got, want, kh.F32) <= 1e-5
+    got, want = _run(ko, kh.F16, 192, 160, 64, True, True, out_dtype=kh.F16, with_acc=kh.F16, seed=8)
+    assert _frob(ko, got, want, kh.F16) <= FROB_TOL
+    got, want = _run(ko, kh.F16, 256, 256, 64, True, False, d_col_major=True, seed=9)
+    assert _frob(ko, got, want, kh.F16) <= FROB_TOL
+    got, want = _run(ko, kh.BF16, 128, 128, 256, True, False, rmode=kh.RZ, seed=9)
+    assert _frob(ko, got, want, kh.BF16) <= 2e-3   # RZ against RZ oracle; accumulation order differs
+
+
+def test_subview_operands(ko):
+    """matmul on sv_global views of larger buffers (start offsets, same strides)."""
+    M, N, K = 128, 128, 96
+    big_a = ko.fill_uniform(256 * 256, kh.F16, 6, 0)
+    big_b = ko.fill_uniform(256 * 256, kh.F16, 6, 1)
+    want = np.zeros((M, N), dtype=np.uint16)
+    va = ko.sv_global(ko.mk_global(big_a, 256, 256, 256, 1, ko.F16), 64, 64 + M, 32, 32 + K)
+    vb = ko.sv_global(ko.mk_global(big_b, 256, 256, 256, 1, ko.F16), 16, 16 + K, 100, 100 + N)
+    assert ko.lib().ko_matmul(C.byref(va), C.byref(vb), None, C.byref(ko.mk_global(want, M, N, N, 1, ko.F16)), ko.RN) == 0
+    da, db, dd = to_dev(big_a), to_dev(big_b), dev_zeros(M * N, 2)
+    kh.matmul(kh.sv_global(dglobal(da, 256, 256, 256, 1, kh.F16), 64, 64 + M, 32, 32 + K),
+              kh.sv_global(dglobal(db, 256, 256, 256, 1, kh.F16), 16, 16 + K, 100, 100 + N), dglobal(dd, M, N, N, 1, kh.F16))
+    sync()
+    assert _frob(ko, to_host(dd, np.uint16), want.ravel(), kh.F16) <= FROB_TOL
+
+
+def test_config4_bf16_8192_sampled_against_oracle(ko):
+    """BASELINE config 4: bf16 8192^3, A row-major, B column-major, normal(0,0.02) seeds 0/1, bf16 out.
+    The GPU computes the whole product; the fp64 oracle recomputes 64x64 blocks spread over the
+    result (every block row and column of the 256-tile grid is hit), and linearity in A covers the rest:
+    (A + A)·B must equal 2·(A·B) exactly, element by element, in bf16."""
+    n = 8192
+    a = ko.fill_normal(n * n, ko.BF16, 0, 0, 0.0, 0.02)
+    bt = ko.fill_normal(n * n, ko.BF16, 1, 0, 0.0, 0.02)      # column-major rhs: element (k, j) at j*n + k
+    da, db, dd = to_dev(a), to_dev(bt), dev_zeros(n * n, 2)
+    ga, gb, gd = dglobal(da, n, n, n, 1, kh.BF16), dglobal(db, n, n, 1, n, kh.BF16), dglobal(dd, n, n, n, 1, kh.BF16)
+    kh.matmul(ga, gb, gd)
+    sync()
+    got = to_host(dd, np.uint16, (n, n))
+    goa, gob = ko.mk_global(a, n, n, n, 1, ko.BF16), ko.mk_global(bt, n, n, 1, n, ko.BF16)
+    num = den = 0.0
+    blk = 64
+    for t in range(32):
+        r0, c0 = (t * 256 + (t * 37) % 192) % n, ((31 - t) * 256 + (t * 53) % 192) % n
+        want = np.zeros((blk, blk), dtype=np.uint16)
+        rc = ko.lib().ko_matmul(C.byref(ko.sv_global(goa, r0, r0 + blk, 0, n)), C.byref(ko.sv_global(gob, 0, n, c0, c0 + blk)), None,
+                                C.byref(ko.mk_global(want, blk, blk, blk, 1, ko.BF16)), ko.RN)
+        assert rc == 0
+        g, w = ko.decode(got[r0:r0 + blk, c0:c0 + blk], ko.BF16), ko.decode(want, ko.BF16)
+        num += ((g - w) ** 2).sum()
+        den += (w ** 2).sum()
+    assert np.sqrt(num / den) <= FROB_TOL
+    # linearity: doubling A (exact in bf16) doubles every output bit-exactly (exponent + 1)
+    import torch
+    a2 = (torch.from_numpy(a.view(np.int16)).view(torch.bfloat16) * 2).view(torch.int16).numpy().view(np.uint16)
+    da.copy_(torch.from_numpy(a2.view(np.int16)).cuda())
+    dd2 = dev_zeros(n * n, 2)
+    kh.matmul(ga, gb, dglobal(dd2, n, n, n, 1, kh.BF16))
+    sync()
+    got2 = to_host(dd2, np.uint16, (n, n))
+    g1 = (got.astype(np.uint32) << 16).view(np.float32)
+    g2 = (got2.astype(np.uint32) << 16).view(np.float32)
+    assert np.array_equal(g2, 2 * g1)

@@ -184,7 +184,9 @@ typedef struct kapy_matmul_cfg {
   int32_t impl_way;              /* kapy_matmul_impl_way                                         */
   int32_t tile_m, tile_n, tile_k; /* workgroup tile; 0 = library's choice                          */
   int32_t rmode;                 /* rounding of the final cast to result dtype (default RN)      */
-  int32_t reserved[3];
+  int32_t stages;                /* depth of the LDS ring (the reference fixture uses 2); 0 = library's choice */
+  int32_t waves;                 /* wavefronts per workgroup (num_warps of the reference); 0 = library's choice */
+  int32_t reserved;
 } kapy_matmul_cfg;
 
 /* kapy.matmul — create_matmul(lhs, rhs, acc, implWay), python/src/ir.cc:1101-1105; verifier

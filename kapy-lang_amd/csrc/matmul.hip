@@ -74,6 +74,10 @@ struct TileLayout {
   }
 };
 
+#ifndef KAPY_TOUCH_AHEAD
+#define KAPY_TOUCH_AHEAD 3
+#endif
+
 // s_waitcnt immediate that waits only on vmcnt <= n (gfx9 encoding: vmcnt in bits [3:0] and [15:14],
 // expcnt [6:4] and lgkmcnt [11:8] left at "no wait").
 constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
@@ -158,7 +162,9 @@ struct TnConfig {
   static constexpr int kLoadsA = BM / kRowsPerLoad, kLoadsB = BN / kRowsPerLoad;
   static constexpr int kLoadsAPerWave = kLoadsA / kWaves, kLoadsBPerWave = kLoadsB / kWaves;
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
-  static constexpr int kLdsBytes = STAGES * kStageBytes;
+  static constexpr int kRingBytes = STAGES * kStageBytes;
+  static constexpr int kTouchBytes = KAPY_TOUCH_AHEAD > 0 ? 256 * kWaves : 0;  // landing area of the L2-warming loads (data unused)
+  static constexpr int kLdsBytes = kRingBytes + kTouchBytes;
   static_assert(kLoadsA % kWaves == 0 && kLoadsB % kWaves == 0, "loads must divide evenly over the wavefronts");
   static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % 16 == 0, "wave tile must be a multiple of the MFMA tile");
 };
@@ -255,29 +261,95 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       for (int j = 0; j < C::kTn; ++j) acc[i][j] = Mfma32x32x16<T>::run(bf[j], af[i], acc[i][j]);
   };
 
-#pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s)
-    if (s < KT) issue_loads(s, s);
+  using Yes = std::integral_constant<bool, true>;
+  using No = std::integral_constant<bool, false>;
+  constexpr int kReads = C::kTm + C::kTn, kMfmas = C::kTm * C::kTn;
+  static_assert(kMfmas >= kReads, "not enough matrix instructions per slice to pace the LDS reads");
 
   if constexpr (STAGES == 2) {
-    // Two stages: the tile multiplied in iteration kt was requested in iteration kt-1.
-    for (int kt = 0; kt < KT; ++kt) {
-      __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
-      __builtin_amdgcn_s_barrier();  // tile kt visible to all; all done reading the stage refilled next
-      if (kt + 1 < KT) issue_loads((kt + 1) & 1, kt + 1);
+    // Two stages (the ring depth of the reference fixture, matmul.mlir:19-22).  The one barrier per
+    // tile sits BEFORE the tile's last K-slice: by then every wave has fetched the fragments of that
+    // last slice, so the stage is free to be refilled, and the next tile (requested one tile ago)
+    // is waited for and published.  The last slice's matrix instructions then cover the first
+    // fragment reads of the next tile and the issue of the loads for the tile after it.
+    static_assert(KK >= 2 && KK % 2 == 0, "needs an even number of K-slices per tile");
+    constexpr int kLoadsPerMfma = (kLoadsPerTile + kMfmas - 1) / kMfmas;
+    u32x4 af[2][C::kTm], bf[2][C::kTn];
+    issue_loads(0, 0);
+    if (KT > 1) {
+      issue_loads(1, 1);
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsPerTile));
+    } else {
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    __builtin_amdgcn_s_barrier();  // tile 0 published
+    read_frags(0, 0, af[0], bf[0]);
+    // L2 warming: kTouchAhead tiles beyond the tile being requested, every lane reads 4 bytes of
+    // one operand row (one 128-byte line per row and K-tile), LDS-direct into a landing area nobody
+    // reads.  The first requester of a line pays the HBM / Infinity Cache latency; with two stages
+    // a real load only has one tile of time to land, a touched line is an L2 hit by then.
+    constexpr int kTouchAhead = KAPY_TOUCH_AHEAD;
+    const int touch_row = wave * 64 + lane;
+    const char *a_touch = a_tile + (int64_t)(touch_row % BM) * p.a_sm * 2;
+    const char *b_touch = b_tile + (int64_t)(touch_row % BN) * p.b_sn * 2;
+    char *touch_lds = lds + C::kRingBytes + wave * 256;
+    bool touched = false;  // were touches issued after the loads we wait for next?
+    auto tile_step = [&](int kt, auto has_next, auto loads) {
+      const int stage = kt & 1;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
-        u32x4 af[C::kTm], bf[C::kTn];
-        read_frags(kt & 1, kk, af, bf);
-        multiply(af, bf);
+        u32x4 *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
+        if (kk == KK - 1) {
+          if constexpr (has_next.value) {
+            // own loads of tile kt+1 landed (younger touches may still fly); own reads of this stage returned
+            if (kTouchAhead > 0 && touched) __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(2));
+            else __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+            __builtin_amdgcn_s_barrier();
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < kMfmas; ++g) {
+          const int i = g / C::kTn, j = g % C::kTn;
+          acc[i][j] = Mfma32x32x16<T>::run(b_cur[j], a_cur[i], acc[i][j]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (g < kReads) {
+            if (kk + 1 < KK) read_frag(stage, kk + 1, g, a_nxt, b_nxt);
+            else if constexpr (has_next.value) read_frag(stage ^ 1, 0, g, a_nxt, b_nxt);
+          }
+          if constexpr (loads.value)
+            if (kk == KK - 1) {
+#pragma unroll
+              for (int t = 0; t < kLoadsPerMfma; ++t)
+                if (g * kLoadsPerMfma + t < kLoadsPerTile) issue_load(stage, kt + 2, g * kLoadsPerMfma + t);
+            }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
-    }
+      if constexpr (has_next.value && kTouchAhead > 0) {
+        touched = false;
+        if (loads.value && kt + 2 + kTouchAhead < KT) {
+          const int64_t k_off = (int64_t)(kt + 2 + kTouchAhead) * BK * 2;
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(a_touch + k_off),
+                                           (__attribute__((address_space(3))) void *)touch_lds, 4, 0, 0);
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(b_touch + k_off),
+                                           (__attribute__((address_space(3))) void *)touch_lds, 4, 0, 0);
+          touched = true;
+        }
+      }
+    };
+    int kt = 0;
+    for (; kt + 2 < KT; ++kt) tile_step(kt, Yes{}, Yes{});
+    for (; kt + 1 < KT; ++kt) tile_step(kt, Yes{}, No{});
+    tile_step(kt, No{}, No{});
   } else {
     // Three or more stages: the barrier at the top of iteration kt publishes tile kt+1, so the
     // fragments of the next K-slice are always fetched one slice ahead, across tile boundaries
     // (the register double-buffering of the reference fixture, matmul.mlir:51-91).
     static_assert(KK % 2 == 0, "fragment double-buffering needs an even number of K-slices per tile");
     u32x4 af[2][C::kTm], bf[2][C::kTn];
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+      if (s < KT) issue_loads(s, s);
     if (KT > STAGES - 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsPerTile * (STAGES - 2)));
     else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __builtin_amdgcn_s_barrier();  // tile 0 published
@@ -297,7 +369,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       // Source order is issue order (sched_barrier pins it): behind each of the first matrix
       // instructions of a slice goes one LDS read of the next slice's fragments and, in the first
       // slice, one LDS-direct global load, so reads have the rest of the slice to land.
-      constexpr int kReads = C::kTm + C::kTn, kMfmas = C::kTm * C::kTn;
+      static_assert(KK * kMfmas >= kLoadsPerTile, "not enough matrix instructions per tile to pace the global loads");
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         u32x4 *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
@@ -310,15 +382,14 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
             if (kk + 1 < KK) read_frag(stage, kk + 1, g, a_nxt, b_nxt);
             else if constexpr (has_next.value) read_frag(next_stage, 0, g, a_nxt, b_nxt);
           }
+          // the tile's LDS-direct loads are spread one per matrix instruction over the whole tile
           if constexpr (has_next.value && loads.value)
-            if (kk == 0 && g < kLoadsPerTile) issue_load(stage == 0 ? STAGES - 1 : stage - 1, kt + STAGES - 1, g);
+            if (kk * kMfmas + g < kLoadsPerTile) issue_load(stage == 0 ? STAGES - 1 : stage - 1, kt + STAGES - 1, kk * kMfmas + g);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
       stage = next_stage;
     };
-    using Yes = std::integral_constant<bool, true>;
-    using No = std::integral_constant<bool, false>;
     int kt = 0;
     for (; kt + STAGES - 1 < KT; ++kt) tile_step(kt, Yes{}, Yes{});
     for (; kt + 1 < KT; ++kt) tile_step(kt, Yes{}, No{});
@@ -487,9 +558,22 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool P
 int launch_tn_epi(GemmParams p, hipStream_t s) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
   auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED>;
-  static bool configured = false;  // raising the dynamic LDS limit is idempotent; a race only repeats it
+  // The kernel addresses kLdsBytes of dynamic LDS (more than the 64 KiB default limit), also through
+  // LDS-direct loads, which fault when they land outside the allocation.  Make sure the limit has
+  // really been raised before the first launch: query first (this also forces the code object to be
+  // loaded, so the attribute is not set on a function the runtime has not materialised yet), set,
+  // and read back.
+  static bool configured = false;  // idempotent; a race only repeats the calls
   if (!configured) {
-    KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes));
+    hipFuncAttributes fa;
+    KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, (const void *)kernel));
+    if (fa.maxDynamicSharedSizeBytes < C::kLdsBytes) {
+      KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes));
+      KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, (const void *)kernel));
+      if (fa.maxDynamicSharedSizeBytes < C::kLdsBytes)
+        return fail(KAPY_ERR_HIP, "matmul: could not raise the dynamic LDS limit to %d bytes (runtime reports %d)", C::kLdsBytes,
+                    (int)fa.maxDynamicSharedSizeBytes);
+    }
     configured = true;
   }
   p.tiles_m = p.M / BM;
@@ -557,6 +641,23 @@ int verify_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_glo
   return KAPY_OK;
 }
 
+// Compiled configurations of the TN kernel, in order of preference.
+struct TnVariant {
+  int bm, bn, bk, waves, stages;
+  int (*launch_bf16)(const GemmParams &, hipStream_t);
+  int (*launch_f16)(const GemmParams &, hipStream_t);
+};
+#define KAPY_TN(BM, BN, BK, WM, WN, S) \
+  { BM, BN, BK, (WM) * (WN), S, launch_tn<Bf16, BM, BN, BK, WM, WN, S>, launch_tn<F16, BM, BN, BK, WM, WN, S> }
+const TnVariant kTnVariants[] = {
+    KAPY_TN(256, 256, 32, 2, 2, 4),
+#ifdef KAPY_TUNING
+    KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2),
+    KAPY_TN(256, 128, 64, 2, 2, 3), KAPY_TN(128, 256, 64, 2, 2, 3), KAPY_TN(128, 128, 64, 2, 2, 4), KAPY_TN(128, 128, 32, 2, 2, 4),
+    KAPY_TN(256, 256, 32, 2, 2, 5), KAPY_TN(256, 128, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2),
+#endif
+};
+
 int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
 
 }  // namespace
@@ -573,7 +674,7 @@ extern "C" {
 
 int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                 const kapy_matmul_cfg *cfg, void *stream) {
-  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, {0, 0, 0}};
+  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0};
   if (cfg) c = *cfg;
   int rc = verify_matmul(lhs, rhs, acc, result, c.impl_way);
   if (rc) return rc;
@@ -608,12 +709,20 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   // and offsets that fit the 32-bit per-lane address arithmetic of the loader.
   bool tn = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 0) == 16 && p.K > 0 &&
             p.a_sm * 2 * 256 < (int64_t(1) << 31) && p.b_sn * 2 * 256 < (int64_t(1) << 31) && p.a_sm > 0 && p.b_sn > 0;
-  int bm = c.tile_m, bn = c.tile_n, bk = c.tile_k;
-  if (tn && (bm == 0 || bm == 256) && (bn == 0 || bn == 256) && (bk == 0 || bk == 32) && p.M % 256 == 0 && p.N % 256 == 0 &&
-      p.K % 32 == 0)
-    return bf16 ? launch_tn<Bf16, 256, 256, 32, 2, 2, 4>(p, s) : launch_tn<F16, 256, 256, 32, 2, 2, 4>(p, s);
-  if ((bm != 0 && bm != kSBM) || (bn != 0 && bn != kSBN) || (bk != 0 && bk != kSBK))
-    return fail(KAPY_ERR_UNSUPPORTED, "matmul: tile %dx%dx%d is not available for these operands (128x128x32 is)", bm, bn, bk);
+  if (tn) {
+    for (const TnVariant &v : kTnVariants) {
+      if ((c.tile_m && c.tile_m != v.bm) || (c.tile_n && c.tile_n != v.bn) || (c.tile_k && c.tile_k != v.bk) ||
+          (c.stages && c.stages != v.stages) || (c.waves && c.waves != v.waves))
+        continue;
+      if (p.M % v.bm || p.N % v.bn || p.K % v.bk) continue;
+      return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
+    }
+  }
+  if ((c.tile_m && c.tile_m != kSBM) || (c.tile_n && c.tile_n != kSBN) || (c.tile_k && c.tile_k != kSBK) || (c.stages && c.stages != 1) ||
+      (c.waves && c.waves != 4))
+    return fail(KAPY_ERR_UNSUPPORTED, "matmul: no kernel with tile %dx%dx%d, %d stages, %d waves serves these operands "
+                                      "(the general kernel is 128x128x32, 1 stage, 4 waves)",
+                c.tile_m, c.tile_n, c.tile_k, c.stages, c.waves);
   int a_mode = operand_mode(p.a_sm, p.a_sk), b_mode = operand_mode(p.b_sn, p.b_sk);
   return bf16 ? launch_staged<Bf16>(p, a_mode, b_mode, s) : launch_staged<F16>(p, a_mode, b_mode, s);
 }

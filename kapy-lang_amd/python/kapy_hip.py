@@ -84,7 +84,7 @@ class EwInst(C.Structure):
 
 class MatmulCfg(C.Structure):
     _fields_ = [("impl_way", C.c_int32), ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
-                ("rmode", C.c_int32), ("reserved", C.c_int32 * 3)]
+                ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("reserved", C.c_int32)]
 
 
 _lib = None
@@ -224,8 +224,8 @@ def fptofp(src, dst, rmode=RN, stream=None):
     check(lib().kapy_fptofp(C.byref(src), C.byref(dst), rmode, stream if stream is not None else current_stream()))
 
 
-def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stream=None):
-    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode)
+def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stages=0, waves=0, stream=None):
+    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, 0)
     check(lib().kapy_matmul(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
                             C.byref(cfg), stream if stream is not None else current_stream()))
 

@@ -12,9 +12,9 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("src,dst,shape", [
     (([8, 8], [1, 2], 0, 1), ([16, 4], [1, 8], 0, 1), (16, 32)),
-    (([2, 32], [4, 1], 0, 1), ([8, 8], [1, 8], 0, 1), (32, 32)),      # MFMA accumulator -> 16-byte store layout
+    (([2, 32], [4, 1], 0, 1), ([8, 8], [1, 4], 0, 1), (32, 32)),      # MFMA accumulator -> 8-byte store layout
     (([8, 8], [2, 2], 0, 1), ([8, 8], [2, 2], 1, 0), (16, 16)),       # exchange axes: a lane-grid transpose
-    (([32, 2], [1, 8], 1, 0), ([2, 32], [8, 1], 0, 1), (32, 16)),
+    (([32, 2], [1, 8], 1, 0), ([8, 8], [4, 2], 0, 1), (32, 16)),       # MFMA lhs operand -> row-major 4x2 blocks
 ])
 def test_change_matches_oracle(ko, src, dst, shape):
     fs, fd = kh.Fragments.make(*src), kh.Fragments.make(*dst)

@@ -74,10 +74,6 @@ struct TileLayout {
   }
 };
 
-#ifndef KAPY_TOUCH_AHEAD
-#define KAPY_TOUCH_AHEAD 3
-#endif
-
 // s_waitcnt immediate that waits only on vmcnt <= n (gfx9 encoding: vmcnt in bits [3:0] and [15:14],
 // expcnt [6:4] and lgkmcnt [11:8] left at "no wait").
 constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
@@ -162,9 +158,7 @@ struct TnConfig {
   static constexpr int kLoadsA = BM / kRowsPerLoad, kLoadsB = BN / kRowsPerLoad;
   static constexpr int kLoadsAPerWave = kLoadsA / kWaves, kLoadsBPerWave = kLoadsB / kWaves;
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
-  static constexpr int kRingBytes = STAGES * kStageBytes;
-  static constexpr int kTouchBytes = KAPY_TOUCH_AHEAD > 0 ? 256 * kWaves : 0;  // landing area of the L2-warming loads (data unused)
-  static constexpr int kLdsBytes = kRingBytes + kTouchBytes;
+  static constexpr int kLdsBytes = STAGES * kStageBytes;
   static_assert(kLoadsA % kWaves == 0 && kLoadsB % kWaves == 0, "loads must divide evenly over the wavefronts");
   static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % 16 == 0, "wave tile must be a multiple of the MFMA tile");
 };
@@ -269,11 +263,24 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   if constexpr (STAGES == 2) {
     // Two stages (the ring depth of the reference fixture, matmul.mlir:19-22).  The one barrier per
     // tile sits BEFORE the tile's last K-slice: by then every wave has fetched the fragments of that
-    // last slice, so the stage is free to be refilled, and the next tile (requested one tile ago)
-    // is waited for and published.  The last slice's matrix instructions then cover the first
-    // fragment reads of the next tile and the issue of the loads for the tile after it.
+    // last slice, so the stage is free to be refilled, and the next tile is waited for and published.
+    // The last slice's matrix instructions then cover the first fragment reads of the next tile.
+    //
+    // Pacing of the LDS-direct loads: the CU's texture path moves 64 bytes per clock, i.e. one 1 KiB
+    // wave-load per 16 clocks, 64 clocks for one load from each of the 4 waves - two matrix
+    // instructions.  Issued any faster the loads back up, a wave blocks at the load instruction and
+    // its matrix pipe starves.  So one load goes behind every kLoadSpacing-th matrix instruction:
+    // the first ones (tile kt+2) in the last slice of tile kt, right after the barrier, the rest in
+    // the first slices of tile kt+1.
     static_assert(KK >= 2 && KK % 2 == 0, "needs an even number of K-slices per tile");
-    constexpr int kLoadsPerMfma = (kLoadsPerTile + kMfmas - 1) / kMfmas;
+#ifndef KAPY_LOAD_SPACING
+#define KAPY_LOAD_SPACING 2
+#endif
+    // (narrower tiles have fewer matrix instructions per load: they fall back to a denser spacing)
+    constexpr int kFit = ((KK - 1) * kMfmas) / kLoadsPerTile;
+    constexpr int kLoadSpacing = kFit < 1 ? 1 : (kFit < KAPY_LOAD_SPACING ? kFit : KAPY_LOAD_SPACING);
+    constexpr int kEarly = kMfmas / kLoadSpacing < kLoadsPerTile ? kMfmas / kLoadSpacing : kLoadsPerTile;  // issued in the last slice
+    static_assert((kLoadsPerTile - kEarly) * kLoadSpacing <= (KK - 1) * kMfmas, "late loads must go out before the barrier that waits for them");
     u32x4 af[2][C::kTm], bf[2][C::kTn];
     issue_loads(0, 0);
     if (KT > 1) {
@@ -284,26 +291,16 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     }
     __builtin_amdgcn_s_barrier();  // tile 0 published
     read_frags(0, 0, af[0], bf[0]);
-    // L2 warming: kTouchAhead tiles beyond the tile being requested, every lane reads 4 bytes of
-    // one operand row (one 128-byte line per row and K-tile), LDS-direct into a landing area nobody
-    // reads.  The first requester of a line pays the HBM / Infinity Cache latency; with two stages
-    // a real load only has one tile of time to land, a touched line is an L2 hit by then.
-    constexpr int kTouchAhead = KAPY_TOUCH_AHEAD;
-    const int touch_row = wave * 64 + lane;
-    const char *a_touch = a_tile + (int64_t)(touch_row % BM) * p.a_sm * 2;
-    const char *b_touch = b_tile + (int64_t)(touch_row % BN) * p.b_sn * 2;
-    char *touch_lds = lds + C::kRingBytes + wave * 256;
-    bool touched = false;  // were touches issued after the loads we wait for next?
-    auto tile_step = [&](int kt, auto has_next, auto loads) {
+    // has_next: tile kt+1 exists.  early: tile kt+2 exists (its first loads go out in the last slice).
+    // late: the remaining loads of tile kt+1 are still to be issued (false for tile 1: the prologue did).
+    auto tile_step = [&](int kt, auto has_next, auto early, auto late) {
       const int stage = kt & 1;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         u32x4 *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
         if (kk == KK - 1) {
           if constexpr (has_next.value) {
-            // own loads of tile kt+1 landed (younger touches may still fly); own reads of this stage returned
-            if (kTouchAhead > 0 && touched) __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(2));
-            else __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+            __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));  // own loads of tile kt+1 landed; own reads of this stage returned
             __builtin_amdgcn_s_barrier();
           }
         }
@@ -316,31 +313,27 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
             if (kk + 1 < KK) read_frag(stage, kk + 1, g, a_nxt, b_nxt);
             else if constexpr (has_next.value) read_frag(stage ^ 1, 0, g, a_nxt, b_nxt);
           }
-          if constexpr (loads.value)
-            if (kk == KK - 1) {
-#pragma unroll
-              for (int t = 0; t < kLoadsPerMfma; ++t)
-                if (g * kLoadsPerMfma + t < kLoadsPerTile) issue_load(stage, kt + 2, g * kLoadsPerMfma + t);
-            }
+          if (g % kLoadSpacing == 0) {
+            const int slot = (kk * kMfmas + g) / kLoadSpacing;  // load slots counted from the start of the tile
+            if constexpr (early.value)
+              if (kk == KK - 1 && g / kLoadSpacing < kEarly) issue_load(stage, kt + 2, g / kLoadSpacing);
+            if constexpr (late.value)
+              if (kk < KK - 1 && kEarly + slot < kLoadsPerTile) issue_load(stage ^ 1, kt + 1, kEarly + slot);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      if constexpr (has_next.value && kTouchAhead > 0) {
-        touched = false;
-        if (loads.value && kt + 2 + kTouchAhead < KT) {
-          const int64_t k_off = (int64_t)(kt + 2 + kTouchAhead) * BK * 2;
-          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(a_touch + k_off),
-                                           (__attribute__((address_space(3))) void *)touch_lds, 4, 0, 0);
-          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(b_touch + k_off),
-                                           (__attribute__((address_space(3))) void *)touch_lds, 4, 0, 0);
-          touched = true;
-        }
-      }
     };
-    int kt = 0;
-    for (; kt + 2 < KT; ++kt) tile_step(kt, Yes{}, Yes{});
-    for (; kt + 1 < KT; ++kt) tile_step(kt, Yes{}, No{});
-    tile_step(kt, No{}, No{});
+    if (KT == 1) {
+      tile_step(0, No{}, No{}, No{});
+    } else {
+      if (KT > 2) tile_step(0, Yes{}, Yes{}, No{});
+      else tile_step(0, Yes{}, No{}, No{});
+      int kt = 1;
+      for (; kt + 2 < KT; ++kt) tile_step(kt, Yes{}, Yes{}, Yes{});
+      if (KT > 2) tile_step(KT - 2, Yes{}, No{}, Yes{});
+      tile_step(KT - 1, No{}, No{}, No{});
+    }
   } else {
     // Three or more stages: the barrier at the top of iteration kt publishes tile kt+1, so the
     // fragments of the next K-slice are always fetched one slice ahead, across tile boundaries
@@ -650,11 +643,10 @@ struct TnVariant {
 #define KAPY_TN(BM, BN, BK, WM, WN, S) \
   { BM, BN, BK, (WM) * (WN), S, launch_tn<Bf16, BM, BN, BK, WM, WN, S>, launch_tn<F16, BM, BN, BK, WM, WN, S> }
 const TnVariant kTnVariants[] = {
-    KAPY_TN(256, 256, 32, 2, 2, 4),
+    KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
 #ifdef KAPY_TUNING
-    KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2),
-    KAPY_TN(256, 128, 64, 2, 2, 3), KAPY_TN(128, 256, 64, 2, 2, 3), KAPY_TN(128, 128, 64, 2, 2, 4), KAPY_TN(128, 128, 32, 2, 2, 4),
-    KAPY_TN(256, 256, 32, 2, 2, 5), KAPY_TN(256, 128, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2),
+    KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2), KAPY_TN(256, 128, 64, 2, 2, 3),
+    KAPY_TN(128, 256, 64, 2, 2, 3), KAPY_TN(128, 128, 64, 2, 2, 4), KAPY_TN(256, 256, 32, 2, 2, 5), KAPY_TN(256, 128, 32, 2, 2, 4),
 #endif
 };
 
@@ -708,13 +700,17 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   // Roofline path: both operands K-contiguous, 16-byte aligned rows, extents multiples of the tile,
   // and offsets that fit the 32-bit per-lane address arithmetic of the loader.
   bool tn = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 0) == 16 && p.K > 0 &&
-            p.a_sm * 2 * 256 < (int64_t(1) << 31) && p.b_sn * 2 * 256 < (int64_t(1) << 31) && p.a_sm > 0 && p.b_sn > 0;
+            p.a_sm * 2 * 256 < (int64_t(1) << 31) && p.b_sn * 2 * 256 < (int64_t(1) << 31) && p.a_sm >= 0 && p.b_sn >= 0;
   if (tn) {
+    const bool free_choice = !c.tile_m && !c.tile_n && !c.tile_k && !c.stages && !c.waves;
     for (const TnVariant &v : kTnVariants) {
       if ((c.tile_m && c.tile_m != v.bm) || (c.tile_n && c.tile_n != v.bn) || (c.tile_k && c.tile_k != v.bk) ||
           (c.stages && c.stages != v.stages) || (c.waves && c.waves != v.waves))
         continue;
       if (p.M % v.bm || p.N % v.bn || p.K % v.bk) continue;
+      // with a free choice, a 256x256 tiling that cannot occupy half of the CUs yields to 128x128
+      if (free_choice && v.bm == 256 && (int64_t)(p.M / v.bm) * (p.N / v.bn) * 2 < device_cus() && p.M % 128 == 0 && p.N % 128 == 0)
+        continue;
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }
@@ -726,6 +722,7 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   int a_mode = operand_mode(p.a_sm, p.a_sk), b_mode = operand_mode(p.b_sn, p.b_sk);
   return bf16 ? launch_staged<Bf16>(p, a_mode, b_mode, s) : launch_staged<F16>(p, a_mode, b_mode, s);
 }
+
 
 int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out) {
   if (!out) return fail(KAPY_ERR_INVALID, "matmul_lds_layout: null result");

@@ -23,7 +23,7 @@ def _np_store(dtype):
 
 
 def _run(ko, dt, M, N, K, a_row_major=True, b_row_major=True, out_dtype=None, with_acc=None, d_col_major=False,
-         seed=0, gen="uniform", rmode=kh.RN, tile=(0, 0, 0)):
+         seed=0, gen="uniform", rmode=kh.RN, tile=(0, 0, 0), stages=0):
     out_dtype = dt if out_dtype is None else out_dtype
     fill = (lambda n, s: ko.fill_uniform(n, dt, seed, s)) if gen == "uniform" else (lambda n, s: ko.fill_normal(n, dt, seed, s, 0.0, 0.02))
     a, b = fill(M * K, 0), fill(K * N, 1)
@@ -42,7 +42,7 @@ def _run(ko, dt, M, N, K, a_row_major=True, b_row_major=True, out_dtype=None, wi
                             C.byref(go_acc) if go_acc is not None else None, C.byref(ko.mk_global(want, M, N, *d_str, out_dtype)), rmode)
     assert rc == 0
     kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(dd, M, N, *d_str, out_dtype), acc=gd_acc,
-              rmode=rmode, tile=tile)
+              rmode=rmode, tile=tile, stages=stages)
     sync()
     return to_host(dd, want.dtype), want
 
@@ -62,14 +62,26 @@ def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):
         assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
 
 
-def test_tn_roofline_kernel_small(ko):
-    """lhs row-major, rhs column-major, multiples of the 256x256x32 tile: the LDS-direct kernel."""
+TN_VARIANTS = [((256, 256, 64), 2), ((256, 256, 32), 4), ((128, 128, 64), 2), ((128, 128, 32), 4)]
+
+
+@pytest.mark.parametrize("tile,stages", TN_VARIANTS)
+def test_tn_roofline_kernel_every_variant(ko, tile, stages):
+    """lhs row-major, rhs column-major, extents multiples of the tile: the LDS-direct kernels, each compiled
+    configuration forced through kapy_matmul_cfg, including K of 1, 2, 3 and many tiles (pipeline prologue / tail)."""
+    bm, bn, bk = tile
     for dt in (kh.BF16, kh.F16):
-        for (M, N, K) in ((256, 256, 32), (256, 256, 64), (256, 512, 96), (512, 256, 128), (768, 512, 1024)):
-            got, want = _run(ko, dt, M, N, K, True, False, seed=5)
+        for (M, N, K) in ((bm, bn, bk), (bm, bn, 2 * bk), (bm, 2 * bn, 3 * bk), (2 * bm, bn, 4 * bk), (3 * bm, 2 * bn, 16 * bk)):
+            got, want = _run(ko, dt, M, N, K, True, False, seed=5, tile=tile, stages=stages)
             assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
-            got32, want32 = _run(ko, dt, M, N, K, True, False, out_dtype=kh.F32, seed=5)
-            assert _frob(ko, got32, want32, kh.F32) <= 1e-5, (M, N, K)
+    got32, want32 = _run(ko, kh.BF16, 2 * bm, 2 * bn, 8 * bk, True, False, out_dtype=kh.F32, seed=5, tile=tile, stages=stages)
+    assert _frob(ko, got32, want32, kh.F32) <= 1e-5
+
+
+def test_tn_default_choice(ko):
+    for (M, N, K) in ((256, 256, 64), (512, 768, 1024), (1024, 1024, 96), (384, 640, 160)):
+        got, want = _run(ko, kh.BF16, M, N, K, True, False, seed=6)
+        assert _frob(ko, got, want, kh.BF16) <= FROB_TOL, (M, N, K)
 
 
 def test_closed_forms_identity_ones_rank1(ko):

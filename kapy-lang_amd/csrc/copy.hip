@@ -18,6 +18,13 @@
 //   generic_kernel    anything else (no contiguous axis, misaligned rows): one element per lane.
 #include "common.hpp"
 
+#ifndef KAPY_TRANSPOSE_MAP
+#define KAPY_TRANSPOSE_MAP 2
+#endif
+#ifndef KAPY_TRANSPOSE_LDS
+#define KAPY_TRANSPOSE_LDS 1
+#endif
+
 namespace kapy {
 namespace {
 
@@ -35,6 +42,7 @@ struct CopyParams {
   int32_t sb0, sb1;  // source bounds: elements at i >= sb0 or j >= sb1 read as padding
   uint32_t pad;      // 32-bit padding word (element pattern replicated)
   int32_t n1;        // second grid dimension; program (p0,p1) = (z / n1, z % n1)
+  int32_t map_mode;  // transpose kernel: how workgroup ids walk the tile grid
   int64_t s_off0, s_off1, d_off0, d_off1;  // per-program displacement in elements
 };
 
@@ -82,11 +90,14 @@ template <> struct VecOf<16> { typedef u32x4 type; };
 template <> struct VecOf<8> { typedef u32x2 type; };
 template <> struct VecOf<4> { typedef uint32_t type; };
 
+#ifndef KAPY_ROWS_UNROLL
+#define KAPY_ROWS_UNROLL 1
+#endif
 template <int B, int VB, bool NT, bool RAGGED>
 __global__ __launch_bounds__(256) void rows_kernel(CopyParams p, int32_t vec_per_row) {
   typedef typename VecOf<VB>::type Vec;
   constexpr int E = VB / B;  // elements per vector
-  constexpr int UNROLL = 4;
+  constexpr int UNROLL = KAPY_ROWS_UNROLL;
   const char *src;
   char *dst;
   program_base<B>(p, src, dst);
@@ -135,8 +146,19 @@ __global__ __launch_bounds__(256) void transpose_kernel(CopyParams p) {
   char *dst;
   program_base<B>(p, src, dst);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int32_t ti = (blockIdx.x * 2 + (wave & 1)) * TILE;
-  const int32_t tj = (blockIdx.y * 2 + (wave >> 1)) * TILE;
+  // Workgroup id -> 2x2 block of wave tiles.  mode 0: x walks the source's contiguous axis; 1: x walks
+  // the destination's; 2: diagonal (consecutive workgroups differ in both), which spreads the
+  // pitch-strided side of the transpose over the memory channels.
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  if (p.map_mode == 1) {
+    uint32_t lin = by * gridDim.x + bx;
+    by = lin % gridDim.y;
+    bx = lin / gridDim.y;
+  } else if (p.map_mode == 2) {
+    by = (by + bx) % gridDim.y;
+  }
+  const int32_t ti = (bx * 2 + (wave & 1)) * TILE;
+  const int32_t tj = (by * 2 + (wave >> 1)) * TILE;
   if (ti >= p.d0 || tj >= p.d1) return;
   const bool interior = ti + TILE <= p.d0 && ti + TILE <= p.sb0 && tj + TILE <= p.d1 && tj + TILE <= p.sb1;
   if (!interior) {  // ragged edge: element-wise with the ld/st predicates
@@ -178,6 +200,95 @@ __global__ __launch_bounds__(256) void transpose_kernel(CopyParams p) {
   }
 }
 
+// Transpose of 16-bit elements through LDS: a workgroup owns a TI x TJ tile.  Each lane still
+// transposes 8x8 blocks in registers, but the lane re-distribution goes through LDS, which frees
+// the lane->block assignment on each side: consecutive lanes cover TI*2 contiguous bytes of a
+// source line when loading and TJ*2 contiguous bytes of a destination line when storing.
+// LDS image: [TI rows][TJ/8 chunks of 16 bytes], chunk index XOR-ed with (row/8) % 16: the 16
+// lanes of an access phase differ in row/8 on the write side and in the chunk on the read side,
+// so either way they land on 16 distinct chunks = all 64 banks once.
+template <int TI, int TJ, bool NT>
+__global__ __launch_bounds__(256) void transpose_lds_kernel(CopyParams p) {
+  constexpr int NI = TI / 8, NJ = TJ / 8, ROW = TJ * 2, PER_LANE = NI * NJ / 256;
+  static_assert(NI >= 16 && NJ >= 16 && (NI * NJ) % 256 == 0, "tile must hold whole 16-lane phases");
+  extern __shared__ __attribute__((aligned(16))) char tile[];
+  const char *src;
+  char *dst;
+  program_base<2>(p, src, dst);
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  if (p.map_mode == 1) {
+    uint32_t lin = by * gridDim.x + bx;
+    by = lin % gridDim.y;
+    bx = lin / gridDim.y;
+  } else if (p.map_mode == 2) {
+    by = (by + bx) % gridDim.y;
+  }
+  const int32_t ti = bx * TI, tj = by * TJ;
+  const int t = threadIdx.x;
+  const bool interior = ti + TI <= p.d0 && ti + TI <= p.sb0 && tj + TJ <= p.d1 && tj + TJ <= p.sb1;
+  if (!interior) {
+    for (int e = t; e < TI * TJ; e += 256) copy_one<2>(p, src, dst, ti + e / TJ, tj + e % TJ);
+    return;
+  }
+  union Block {
+    u32x4 vec[8];
+    uint16_t el[8][8];
+  };
+  Block in[PER_LANE];
+#pragma unroll
+  for (int k = 0; k < PER_LANE; ++k) {
+    const int q = t + 256 * k, bi = q % NI, bj = q / NI;  // consecutive lanes along the source's contiguous axis
+    const char *s = src + ((int64_t)(ti + 8 * bi) + (int64_t)(tj + 8 * bj) * p.es1) * 2;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const u32x4 *ptr = (const u32x4 *)(s + (int64_t)c * p.es1 * 2);
+      in[k].vec[c] = NT ? __builtin_nontemporal_load(ptr) : *ptr;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < PER_LANE; ++k) {
+    const int q = t + 256 * k, bi = q % NI, bj = q / NI;
+    Block out;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) out.el[r][c] = in[k].el[c][r];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) *(u32x4 *)(tile + (8 * bi + r) * ROW + ((bj ^ (bi & 15)) << 4)) = out.vec[r];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < PER_LANE; ++k) {
+    const int q = t + 256 * k, bj = q % NJ, bi = q / NJ;  // consecutive lanes along the destination's contiguous axis
+    char *d = dst + ((int64_t)(ti + 8 * bi) * p.ds0 + (int64_t)(tj + 8 * bj)) * 2;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      u32x4 v = *(const u32x4 *)(tile + (8 * bi + r) * ROW + ((bj ^ (bi & 15)) << 4));
+      u32x4 *ptr = (u32x4 *)(d + (int64_t)r * p.ds0 * 2);
+      if (NT) __builtin_nontemporal_store(v, ptr);
+      else *ptr = v;
+    }
+  }
+}
+
+template <int TI, int TJ>
+int launch_transpose_lds(const CopyParams &p, bool nt, int32_t batch, hipStream_t stream) {
+  constexpr int kLds = TI * TJ * 2;
+  dim3 grid((unsigned)((p.d0 + TI - 1) / TI), (unsigned)((p.d1 + TJ - 1) / TJ), (unsigned)batch);
+  if (kLds > 65536) {
+    static bool configured = false;
+    if (!configured) {
+      KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)transpose_lds_kernel<TI, TJ, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+      KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)transpose_lds_kernel<TI, TJ, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+      configured = true;
+    }
+  }
+  if (nt) transpose_lds_kernel<TI, TJ, true><<<grid, 256, kLds, stream>>>(p);
+  else transpose_lds_kernel<TI, TJ, false><<<grid, 256, kLds, stream>>>(p);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 uint32_t padding_word(int32_t dtype, int32_t padding) {
   // ConvertUtils.cpp:267-334; e4m3 is OCP E4M3FN here (no infinities): +-inf -> +-448, qnan -> 0x7F.
   static const uint32_t f32[4] = {0, 0x7FC00000u, 0x7F800000u, 0xFF800000u};
@@ -214,7 +325,7 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
       int e = vb / B;
       int32_t vpr = (p.d1 + e - 1) / e;
       int64_t slots = slots_at_vb;
-      dim3 grid((unsigned)((slots + 1023) / 1024), 1, (unsigned)batch);
+      dim3 grid((unsigned)((slots + 256 * KAPY_ROWS_UNROLL - 1) / (256 * KAPY_ROWS_UNROLL)), 1, (unsigned)batch);
       // no ragged vector anywhere: every slot is a whole in-bounds vector on both sides
       bool ragged = p.d1 % e != 0 || p.sb1 < p.d1 || p.sb0 < p.d0;
       if (vb == 16 && !ragged) {
@@ -230,7 +341,15 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
       KAPY_HIP_CHECK(hipGetLastError());
       return KAPY_OK;
     }
+  } else if (B == 2 && KAPY_TRANSPOSE_LDS && p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16 && p.d0 >= 128 && p.d1 >= 128 &&
+             (p.d1 + 127) / 128 <= 65535 && !(p.map_mode & 16)) {
+    const int shape = (p.map_mode >> 5) & 3;  // tuning builds select the tile; 0 = default
+    p.map_mode &= 15;
+    if (shape == 1) return launch_transpose_lds<256, 128>(p, nt, batch, stream);
+    if (shape == 2) return launch_transpose_lds<128, 256>(p, nt, batch, stream);
+    return launch_transpose_lds<128, 128>(p, nt, batch, stream);
   } else if (p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16) {
+    p.map_mode &= 15;
     constexpr int TILE = 8 * (16 / B);
     unsigned gx = (unsigned)((p.d0 + 2 * TILE - 1) / (2 * TILE)), gy = (unsigned)((p.d1 + 2 * TILE - 1) / (2 * TILE));
     if (gy <= 65535) {
@@ -286,6 +405,10 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   p.sb1 = (int32_t)(t ? extent0(src) : extent1(src));
   p.pad = padding_word(src->dtype, c.padding_option);
   p.n1 = g.n1 > 0 ? g.n1 : 1;
+  p.map_mode = KAPY_TRANSPOSE_MAP;
+#ifdef KAPY_TUNING
+  if (c.reserved) p.map_mode = c.reserved - 1;
+#endif
   p.s_off0 = g.src_off0;
   p.s_off1 = g.src_off1;
   p.d_off0 = g.dst_off0;
@@ -301,7 +424,11 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   };
   int vb_src = side_vb(src, g.n0 > 1 ? g.src_off0 : 0, g.n1 > 1 ? g.src_off1 : 0);
   int vb_dst = side_vb(dst, g.n0 > 1 ? g.dst_off0 : 0, g.n1 > 1 ? g.dst_off1 : 0);
-  bool nt = c.cache_modifier == KAPY_CACHE_CS || c.cache_modifier == KAPY_CACHE_CG;
+  // Streaming (non-temporal) access when asked for (cs / cg), and by default for moves too large to
+  // be re-read from the 256 MB Infinity Cache anyway.
+  const int64_t moved = (int64_t)p.d0 * p.d1 * B * (g.n0 > 0 ? g.n0 : 1) * (g.n1 > 0 ? g.n1 : 1);
+  bool nt = c.cache_modifier == KAPY_CACHE_CS || c.cache_modifier == KAPY_CACHE_CG ||
+            (c.cache_modifier == KAPY_CACHE_NONE && moved >= (int64_t(32) << 20));
   int32_t batch = g.n0 * g.n1;
   hipStream_t s = (hipStream_t)stream;
   switch (B) {

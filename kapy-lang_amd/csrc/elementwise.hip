@@ -11,6 +11,7 @@
 #include <math.h>
 #include <string.h>
 
+#include <type_traits>
 #include <vector>
 
 #include "common.hpp"
@@ -41,10 +42,14 @@ struct Program {
   DevView out;
 };
 
-// 0.5*v*(1+tanh(sqrt(2/pi)*(v+0.044715*v^3))) == v * sigmoid(2u): no cancellation for v << 0.
+// 0.5*v*(1+tanh(u)) with u = sqrt(2/pi)*(v+0.044715*v^3) equals v*sigmoid(2u) = v / (1 + 2^(-2u*log2 e)):
+// no cancellation for v << 0, and only three slow-rate operations per element (exp2, rcp and
+// their operand prep).  The constants fold -2*log2(e)*sqrt(2/pi) into the cubic.
 __device__ __forceinline__ float gelu_tanh_f32(float v) {
-  float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-  return v / (1.0f + __expf(-2.0f * u));
+  constexpr float kC1 = -2.0f * 1.4426950408889634f * 0.7978845608028654f;
+  constexpr float kC3 = kC1 * 0.044715f;
+  float t = v * (kC1 + kC3 * v * v);
+  return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
 }
 
 __device__ __forceinline__ float apply_unary(int op, float a) {
@@ -147,11 +152,23 @@ template <> struct Codec<_Float16> {
 struct Bf16Tag {};
 template <> struct Codec<Bf16Tag> {
   static __device__ __forceinline__ float up(uint16_t h) { return bf16_to_f32(h); }
-  static __device__ __forceinline__ uint16_t down(float v) { return f32_to_bf16_rn(v); }
+  static __device__ __forceinline__ uint16_t down(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }  // v_cvt_pk_bf16_f32: RN-even
 };
 
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 template <typename T>
 __device__ __forceinline__ void unpack8(u32x4 v, float f[8]) {
+  if constexpr (std::is_same<T, _Float16>::value) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t word = v[w];  // bit_cast needs a scalar object, not a vector-element lvalue
+      float2_t x = __builtin_convertvector(__builtin_bit_cast(half2_t, word), float2_t);
+      f[2 * w] = x[0];
+      f[2 * w + 1] = x[1];
+    }
+    return;
+  }
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
     f[2 * w] = Codec<T>::up((uint16_t)(v[w] & 0xFFFFu));
@@ -161,15 +178,22 @@ __device__ __forceinline__ void unpack8(u32x4 v, float f[8]) {
 template <typename T>
 __device__ __forceinline__ u32x4 pack8(const float f[8]) {
   u32x4 v;
+
 #pragma unroll
   for (int w = 0; w < 4; ++w) v[w] = (uint32_t)Codec<T>::down(f[2 * w]) | ((uint32_t)Codec<T>::down(f[2 * w + 1]) << 16);
   return v;
 }
 
 // 16-bit in, 16-bit out (same type), 8 elements per 16-byte vector, UNROLL vectors per lane.
+#ifndef KAPY_EW_UNROLL
+#define KAPY_EW_UNROLL 2
+#endif
+#ifndef KAPY_EW_NT
+#define KAPY_EW_NT 1
+#endif
 template <typename T, int ACT>
 __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
-  constexpr int UNROLL = 4;
+  constexpr int UNROLL = KAPY_EW_UNROLL;
   const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;
   const uint32_t first = blockIdx.x * (256 * UNROLL) + threadIdx.x;
   u32x4 xv[UNROLL], bv[UNROLL];
@@ -181,7 +205,8 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
     if (slot < total) {
       row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);
       col[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row) * 8;
-      xv[u] = __builtin_nontemporal_load((const u32x4 *)(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2));
+      const u32x4 *xp = (const u32x4 *)(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2);
+      xv[u] = KAPY_EW_NT ? __builtin_nontemporal_load(xp) : *xp;
       if (p.bias_mode == kBiasRow) bv[u] = *(const u32x4 *)(p.bias + (int64_t)col[u] * 2);
       else if (p.bias_mode == kBiasFull) bv[u] = *(const u32x4 *)(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2);
       else if (p.bias_mode == kBiasCol) {
@@ -206,7 +231,50 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
       else if (ACT >= 0) v = apply_unary(p.act, v);
       f[e] = v;
     }
-    __builtin_nontemporal_store(pack8<T>(f), (u32x4 *)(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2));
+    u32x4 *op = (u32x4 *)(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2);
+    if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
+    else *op = pack8<T>(f);
+  }
+}
+
+// Same chain when the bias is broadcast along rows (bias[0, j]) or absent: a lane keeps one
+// 8-column chunk and walks ROWS consecutive rows, so its bias vector is fetched and widened once
+// and no index division is needed.  Grid: x over column chunks, y over groups of ROWS rows.
+#ifndef KAPY_EW_ROWS
+#define KAPY_EW_ROWS 2
+#endif
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p) {
+  constexpr int ROWS = KAPY_EW_ROWS;
+  const int32_t chunk = blockIdx.x * 256 + threadIdx.x;
+  if (chunk >= p.vec_per_row) return;
+  const int32_t col = chunk * 8, row0 = blockIdx.y * ROWS;
+  float b[8];
+  if (p.bias_mode == kBiasRow) unpack8<T>(*(const u32x4 *)(p.bias + (int64_t)col * 2), b);
+  u32x4 xv[ROWS];
+#pragma unroll
+  for (int u = 0; u < ROWS; ++u)
+    if (row0 + u < p.rows) {
+      const u32x4 *xp = (const u32x4 *)(p.x + ((int64_t)(row0 + u) * p.x_stride0 + col) * 2);
+      xv[u] = KAPY_EW_NT ? __builtin_nontemporal_load(xp) : *xp;
+    }
+#pragma unroll
+  for (int u = 0; u < ROWS; ++u) {
+    if (row0 + u >= p.rows) break;
+    float f[8];
+    unpack8<T>(xv[u], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float v = f[e];
+      if (p.has_scale) v = __fmul_rn(v, p.scale);
+      if (p.bias_mode == kBiasRow) v = __fadd_rn(v, b[e]);
+      if (ACT == KAPY_EW_GELU_TANH) v = gelu_tanh_f32(v);
+      else if (ACT >= 0) v = apply_unary(p.act, v);
+      f[e] = v;
+    }
+    u32x4 *op = (u32x4 *)(p.out + ((int64_t)(row0 + u) * p.out_stride0 + col) * 2);
+    if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
+    else *op = pack8<T>(f);
   }
 }
 
@@ -460,16 +528,24 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   int T = -1;
   if (match_affine_act(prog, n_inst, ins, out, &ap, &T)) {
     uint32_t slots = (uint32_t)ap.rows * (uint32_t)ap.vec_per_row;
-    dim3 grid((slots + 1023) / 1024);
+    const bool cols = (ap.bias_mode == kBiasRow || ap.bias_mode == kNoBias) && (ap.rows + KAPY_EW_ROWS - 1) / KAPY_EW_ROWS <= 65535;
+    dim3 grid = cols ? dim3((ap.vec_per_row + 255) / 256, (ap.rows + KAPY_EW_ROWS - 1) / KAPY_EW_ROWS)
+                     : dim3((slots + 256 * KAPY_EW_UNROLL - 1) / (256 * KAPY_EW_UNROLL));
+#define KAPY_LAUNCH_AFFINE(TT, AA)                                                     \
+  do {                                                                                 \
+    if (cols) affine_act_cols_kernel<TT, AA><<<grid, 256, 0, s>>>(ap);                 \
+    else affine_act_kernel<TT, AA><<<grid, 256, 0, s>>>(ap);                           \
+  } while (0)
     if (T == KAPY_F16) {
-      if (ap.act == KAPY_EW_GELU_TANH) affine_act_kernel<_Float16, KAPY_EW_GELU_TANH><<<grid, 256, 0, s>>>(ap);
-      else if (ap.act < 0) affine_act_kernel<_Float16, -1><<<grid, 256, 0, s>>>(ap);
-      else affine_act_kernel<_Float16, 0><<<grid, 256, 0, s>>>(ap);
+      if (ap.act == KAPY_EW_GELU_TANH) KAPY_LAUNCH_AFFINE(_Float16, KAPY_EW_GELU_TANH);
+      else if (ap.act < 0) KAPY_LAUNCH_AFFINE(_Float16, -1);
+      else KAPY_LAUNCH_AFFINE(_Float16, 0);
     } else {
-      if (ap.act == KAPY_EW_GELU_TANH) affine_act_kernel<Bf16Tag, KAPY_EW_GELU_TANH><<<grid, 256, 0, s>>>(ap);
-      else if (ap.act < 0) affine_act_kernel<Bf16Tag, -1><<<grid, 256, 0, s>>>(ap);
-      else affine_act_kernel<Bf16Tag, 0><<<grid, 256, 0, s>>>(ap);
+      if (ap.act == KAPY_EW_GELU_TANH) KAPY_LAUNCH_AFFINE(Bf16Tag, KAPY_EW_GELU_TANH);
+      else if (ap.act < 0) KAPY_LAUNCH_AFFINE(Bf16Tag, -1);
+      else KAPY_LAUNCH_AFFINE(Bf16Tag, 0);
     }
+#undef KAPY_LAUNCH_AFFINE
     KAPY_HIP_CHECK(hipGetLastError());
     return KAPY_OK;
   }

@@ -16,7 +16,9 @@ def _check_ulp(got, want, dtype):
     f = (lambda a: a.view(np.float16).astype(np.float64)) if dtype == kh.F16 else \
         (lambda a: (a.astype(np.uint32) << 16).view(np.float32).astype(np.float64))
     gn, wn = np.isnan(f(got)), np.isnan(f(want))
-    assert np.array_equal(gn, wn)
+    bad = np.argwhere(gn != wn)
+    assert len(bad) == 0, "NaN pattern differs at %s: got %s want %s" % (bad[:8].tolist(), [hex(int(got[tuple(b)])) for b in bad[:8]],
+                                                                       [hex(int(want[tuple(b)])) for b in bad[:8]])
     d = ulp_diff_f16(got[~gn], want[~wn])
     assert d.max(initial=0) <= ULP_TOL, "max ulp error %d" % d.max()
     return d

@@ -144,43 +144,65 @@ struct AffineActParams {
   float scale;
 };
 
-template <typename T> struct Codec;
-template <> struct Codec<_Float16> {
-  static __device__ __forceinline__ float up(uint16_t h) { return f16_to_f32(h); }
-  static __device__ __forceinline__ uint16_t down(float v) { return f32_to_f16_rn(v); }
-};
+// Two 16-bit elements of a 32-bit word <-> two fp32.  For f16 the widening is left as a plain cast
+// so that the compiler can fold it into v_fma_mix_f32 (conversion + multiply + add in one
+// instruction), and the narrowing pairs up into v_cvt_pk_f16_f32; bf16 widens with a shift and
+// narrows with v_cvt_pk_bf16_f32.  All narrowing is round-to-nearest-even.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 struct Bf16Tag {};
-template <> struct Codec<Bf16Tag> {
-  static __device__ __forceinline__ float up(uint16_t h) { return bf16_to_f32(h); }
-  static __device__ __forceinline__ uint16_t down(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }  // v_cvt_pk_bf16_f32: RN-even
+template <typename T> struct Pair;
+template <> struct Pair<_Float16> {
+  static __device__ __forceinline__ void widen(uint32_t word, float &lo, float &hi) {
+    half2_t h = __builtin_bit_cast(half2_t, word);
+    lo = (float)h[0];
+    hi = (float)h[1];
+  }
+  static __device__ __forceinline__ uint32_t narrow(float lo, float hi) {
+    half2_t h;
+    h[0] = (_Float16)lo;
+    h[1] = (_Float16)hi;
+    return __builtin_bit_cast(uint32_t, h);
+  }
+};
+template <> struct Pair<Bf16Tag> {
+  static __device__ __forceinline__ void widen(uint32_t word, float &lo, float &hi) {
+    lo = bits_f32(word << 16);
+    hi = bits_f32(word & 0xFFFF0000u);
+  }
+  static __device__ __forceinline__ uint32_t narrow(float lo, float hi) {
+    bf16x2_t h;
+    h[0] = (__bf16)lo;
+    h[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, h);
+  }
 };
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef float float2_t __attribute__((ext_vector_type(2)));
 template <typename T>
 __device__ __forceinline__ void unpack8(u32x4 v, float f[8]) {
-  if constexpr (std::is_same<T, _Float16>::value) {
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const uint32_t word = v[w];  // bit_cast needs a scalar object, not a vector-element lvalue
-      float2_t x = __builtin_convertvector(__builtin_bit_cast(half2_t, word), float2_t);
-      f[2 * w] = x[0];
-      f[2 * w + 1] = x[1];
-    }
-    return;
-  }
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    f[2 * w] = Codec<T>::up((uint16_t)(v[w] & 0xFFFFu));
-    f[2 * w + 1] = Codec<T>::up((uint16_t)(v[w] >> 16));
+    const uint32_t word = v[w];  // bit_cast needs a scalar object, not a vector-element lvalue
+    Pair<T>::widen(word, f[2 * w], f[2 * w + 1]);
   }
 }
 template <typename T>
 __device__ __forceinline__ u32x4 pack8(const float f[8]) {
   u32x4 v;
-
 #pragma unroll
-  for (int w = 0; w < 4; ++w) v[w] = (uint32_t)Codec<T>::down(f[2 * w]) | ((uint32_t)Codec<T>::down(f[2 * w + 1]) << 16);
+  for (int w = 0; w < 4; ++w) v[w] = Pair<T>::narrow(f[2 * w], f[2 * w + 1]);
+  return v;
+}
+
+// One element of the fused chain.  x*scale + bias is written as a plain expression: the compiler
+// may contract it into one FMA (for f16 inputs the mixed-precision v_fma_mix_f32), i.e. one
+// rounding where mulf-then-addf has two; the difference is at most half an ulp of fp32, five
+// orders of magnitude inside the 2-ulp tolerance of the 16-bit result.
+template <int ACT>
+__device__ __forceinline__ float affine_act(float x, float scale, float bias, int act) {
+  float v = x * scale + bias;
+  if (ACT == KAPY_EW_GELU_TANH) return gelu_tanh_f32(v);
+  if (ACT >= 0) return apply_unary(act, v);
   return v;
 }
 
@@ -196,6 +218,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
   constexpr int UNROLL = KAPY_EW_UNROLL;
   const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;
   const uint32_t first = blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  const float scale = p.has_scale ? p.scale : 1.0f;
   u32x4 xv[UNROLL], bv[UNROLL];
   int32_t row[UNROLL], col[UNROLL];
 #pragma unroll
@@ -223,14 +246,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
     unpack8<T>(xv[u], f);
     if (p.bias_mode != kNoBias) unpack8<T>(bv[u], b);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float v = f[e];
-      if (p.has_scale) v = __fmul_rn(v, p.scale);
-      if (p.bias_mode != kNoBias) v = __fadd_rn(v, b[e]);
-      if (ACT == KAPY_EW_GELU_TANH) v = gelu_tanh_f32(v);
-      else if (ACT >= 0) v = apply_unary(p.act, v);
-      f[e] = v;
-    }
+    for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, p.bias_mode != kNoBias ? b[e] : 0.f, p.act);
     u32x4 *op = (u32x4 *)(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2);
     if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
     else *op = pack8<T>(f);
@@ -249,7 +265,8 @@ __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p)
   const int32_t chunk = blockIdx.x * 256 + threadIdx.x;
   if (chunk >= p.vec_per_row) return;
   const int32_t col = chunk * 8, row0 = blockIdx.y * ROWS;
-  float b[8];
+  const float scale = p.has_scale ? p.scale : 1.0f;
+  float b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (p.bias_mode == kBiasRow) unpack8<T>(*(const u32x4 *)(p.bias + (int64_t)col * 2), b);
   u32x4 xv[ROWS];
 #pragma unroll
@@ -264,14 +281,7 @@ __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p)
     float f[8];
     unpack8<T>(xv[u], f);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float v = f[e];
-      if (p.has_scale) v = __fmul_rn(v, p.scale);
-      if (p.bias_mode == kBiasRow) v = __fadd_rn(v, b[e]);
-      if (ACT == KAPY_EW_GELU_TANH) v = gelu_tanh_f32(v);
-      else if (ACT >= 0) v = apply_unary(p.act, v);
-      f[e] = v;
-    }
+    for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, b[e], p.act);
     u32x4 *op = (u32x4 *)(p.out + ((int64_t)(row0 + u) * p.out_stride0 + col) * 2);
     if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
     else *op = pack8<T>(f);

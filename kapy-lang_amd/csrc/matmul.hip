@@ -28,6 +28,7 @@
 
 #include "common.hpp"
 #include "layout.hpp"
+#include "matmul_params.hpp"
 #include "numeric.hpp"
 
 namespace kapy {
@@ -36,29 +37,48 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-struct Bf16 {};
-struct F16 {};
-template <typename T> struct Mfma32x32x16;
-template <> struct Mfma32x32x16<Bf16> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// Operand element policies: bytes per element, the K extent of one matrix instruction, how many
+// 16-byte LDS chunks a lane feeds it per operand, and its duration in clocks (4 per pass).
+struct Bf16 {
+  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32;
+  static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
   }
 };
-template <> struct Mfma32x32x16<F16> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+struct F16 {
+  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32;
+  static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
+  }
+};
+// OCP fp8, v_mfma_scale_f32_32x32x64_f8f6f4 with unit block scales (E8M0 127 = 2^0).  AF / BF are the
+// format selectors of the first / second instruction operand: 0 = E4M3, 1 = E5M2 (kapy lets the two
+// f8 types mix, Kapy.cpp:484-487).  A lane feeds 32 K-contiguous bytes per operand: two chunks.
+template <int AF, int BF>
+struct F8 {
+  static constexpr int kBytes = 1, kSliceK = 64, kChunks = 2, kMfmaClocks = 64;
+  static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
+    i32x8 av = {(int)a[0][0], (int)a[0][1], (int)a[0][2], (int)a[0][3], (int)a[1][0], (int)a[1][1], (int)a[1][2], (int)a[1][3]};
+    i32x8 bv = {(int)b[0][0], (int)b[0][1], (int)b[0][2], (int)b[0][3], (int)b[1][0], (int)b[1][1], (int)b[1][2], (int)b[1][3]};
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AF, BF, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
   }
 };
 
-// LDS image of an operand tile: [rows][BK] 16-bit elements, K contiguous, 16-byte chunks XOR-ed
-// with the line index.  LP comes from the compile-time search over the MFMA operand layout.
-template <int BK>
+// LDS image of an operand tile: [rows][ROWBYTES] bytes, K contiguous, 16-byte chunks XOR-ed with the
+// line index.  The parameters come from the compile-time search (the reference's getSwizzlingLayouts
+// for 64 banks) run on the access layout of an MFMA operand read: 32 lanes down the rows, 2 across,
+// 16 contiguous bytes per lane.
+constexpr Fragments kOperandRead16B{32, 2, 1, 16, 0};
+template <int ROWBYTES>
 struct TileLayout {
-  static constexpr int kRowBytes = BK * 2;
-  static constexpr Swizzle kSwizzle = first_swizzle(mfma_lhs(kMfma32x32x16), {32, 16}, BK, 1, 16, 1024);
+  static constexpr int kRowBytes = ROWBYTES;
+  static constexpr Swizzle kSwizzle = first_swizzle(kOperandRead16B, {32, 32}, ROWBYTES, 1, 8, 1024);
   static_assert(kSwizzle.bank_param == 4, "MFMA operand reads are 16-byte: the search must return 16-byte atoms");
   static constexpr int kLineParam = kSwizzle.line_param;
   // byte offset of 16-byte chunk `chunk` of row `row`
@@ -81,21 +101,10 @@ constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // which other waves overwrite the LDS stage this wave has been reading.
 constexpr int vmcnt_lgkm0_imm(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
-struct GemmParams {
-  const char *a, *b, *acc;
-  char *d;
-  int64_t a_sm, a_sk;  // lhs element strides along M and K
-  int64_t b_sn, b_sk;  // rhs element strides along N and K
-  int64_t acc_sm, acc_sn, d_sm, d_sn;
-  int32_t M, N, K;
-  int32_t acc_dtype;  // -1: no accumulator input
-  int32_t d_dtype;
-  int32_t rz;         // final cast rounds toward zero
-  int32_t tiles_m, tiles_n;
-};
 
 __device__ __forceinline__ void store_result(const GemmParams &p, int32_t m, int32_t n, float v) {
   if (m >= p.M || n >= p.N) return;
+  if (p.row_scale) v = __fmul_rn(v, __fmul_rn(p.row_scale[m], p.col_scale[n]));
   if (p.acc_dtype >= 0) v += load_as_f32(p.acc, p.acc_dtype, m * p.acc_sm + n * p.acc_sn);
   int64_t idx = m * p.d_sm + n * p.d_sn;
   switch (p.d_dtype) {
@@ -114,11 +123,18 @@ __device__ __forceinline__ void store_result(const GemmParams &p, int32_t m, int
 __device__ __forceinline__ void store_block_packed(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, const f32x16 &acc) {
   char *row = p.d + ((int64_t)(m_base + (lane & 31)) * p.d_sm + n_base + 4 * (lane >> 5)) * 2;
   const bool f16 = p.d_dtype == KAPY_F16;
+  const float rs = p.row_scale ? p.row_scale[m_base + (lane & 31)] : 1.0f;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     uint16_t h[4];
+    f32x4 cs = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (p.row_scale) cs = *(const f32x4 *)(p.col_scale + n_base + 4 * (lane >> 5) + 8 * q);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) h[e] = f16 ? f32_to_f16_rn(acc[4 * q + e]) : f32_to_bf16_rn(acc[4 * q + e]);
+    for (int e = 0; e < 4; ++e) {
+      float v = acc[4 * q + e];
+      if (p.row_scale) v = __fmul_rn(v, __fmul_rn(rs, cs[e]));
+      h[e] = f16 ? f32_to_f16_rn(v) : f32_to_bf16_rn(v);
+    }
     u32x2 w = {h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16)};
     *(u32x2 *)(row + 16 * q) = w;
   }
@@ -153,20 +169,21 @@ struct TnConfig {
   static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves;
   static constexpr int kWtm = BM / WM, kWtn = BN / WN;       // wave tile
   static constexpr int kTm = kWtm / 32, kTn = kWtn / 32;     // 32x32 accumulators per wave
-  static constexpr int kRowBytes = BK * 2;
+  static constexpr int kRowBytes = BK * T::kBytes;
   static constexpr int kRowsPerLoad = 1024 / kRowBytes;      // rows one LDS-direct wave instruction fills
   static constexpr int kLoadsA = BM / kRowsPerLoad, kLoadsB = BN / kRowsPerLoad;
   static constexpr int kLoadsAPerWave = kLoadsA / kWaves, kLoadsBPerWave = kLoadsB / kWaves;
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
   static constexpr int kLdsBytes = STAGES * kStageBytes;
   static_assert(kLoadsA % kWaves == 0 && kLoadsB % kWaves == 0, "loads must divide evenly over the wavefronts");
-  static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % 16 == 0, "wave tile must be a multiple of the MFMA tile");
+  static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % T::kSliceK == 0, "wave tile must be a multiple of the MFMA tile");
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
 __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
-  using L = TileLayout<BK>;
+  using L = TileLayout<C::kRowBytes>;
+  constexpr int EB = T::kBytes, CH = T::kChunks;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -183,27 +200,27 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   for (int i = 0; i < C::kLoadsAPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
-    a_goff[i] = (uint32_t)((row * p.a_sm + chunk * 8) * 2);
+    a_goff[i] = (uint32_t)((row * p.a_sm + chunk * (16 / EB)) * EB);
   }
 #pragma unroll
   for (int i = 0; i < C::kLoadsBPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
-    b_goff[i] = (uint32_t)((row * p.b_sn + chunk * 8) * 2);
+    b_goff[i] = (uint32_t)((row * p.b_sn + chunk * (16 / EB)) * EB);
   }
-  const char *a_tile = p.a + (int64_t)m0 * p.a_sm * 2;
-  const char *b_tile = p.b + (int64_t)n0 * p.b_sn * 2;
+  const char *a_tile = p.a + (int64_t)m0 * p.a_sm * EB;
+  const char *b_tile = p.b + (int64_t)n0 * p.b_sn * EB;
 
   // Load instruction `idx` (0 .. loads per tile - 1) of this wavefront for K-tile kt into `stage`.
   auto issue_load = [&](int stage, int kt, int idx) {
     char *sa = lds + stage * C::kStageBytes, *sb = sa + BM * C::kRowBytes;
     if (idx < C::kLoadsAPerWave) {
-      const char *ga = a_tile + (int64_t)kt * BK * 2;
+      const char *ga = a_tile + (int64_t)kt * BK * EB;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ga + a_goff[idx]),
                                        (__attribute__((address_space(3))) void *)(sa + (wave + idx * C::kWaves) * 1024), 16, 0, 0);
     } else {
       const int i = idx - C::kLoadsAPerWave;
-      const char *gb = b_tile + (int64_t)kt * BK * 2;
+      const char *gb = b_tile + (int64_t)kt * BK * EB;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb + b_goff[i]),
                                        (__attribute__((address_space(3))) void *)(sb + (wave + i * C::kWaves) * 1024), 16, 0, 0);
     }
@@ -229,36 +246,38 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   }
 
   const int KT = p.K / BK;
-  constexpr int KK = BK / 16;                                          // MFMA K-slices per tile
+  constexpr int KK = BK / T::kSliceK;                                   // matrix-instruction K-slices per tile
   constexpr int kLoadsPerTile = C::kLoadsAPerWave + C::kLoadsBPerWave;  // per wavefront
-  // Per-lane LDS offsets of the operand reads of slice kk, relative to the wave's rows of a stage.
-  uint32_t frag_off[KK];
+  // A fragment: the CH 16-byte chunks one lane feeds a matrix instruction for one operand block.
+  struct Frag {
+    u32x4 c[CH];
+  };
+  // Per-lane LDS offsets of the operand reads of slice kk, relative to the wave's rows of a stage:
+  // row (lane % 32) of each 32-row block, chunks (2*kk + lane/32)*CH .. +CH-1 of the row.
+  uint32_t frag_off[KK][CH];
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk) frag_off[kk] = L::offset(frag_row, 2 * kk + frag_half);
+  for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+    for (int c = 0; c < CH; ++c) frag_off[kk][c] = L::offset(frag_row, (2 * kk + frag_half) * CH + c);
   const uint32_t a_rows = (wm * C::kWtm) * C::kRowBytes, b_rows = BM * C::kRowBytes + (wn * C::kWtn) * C::kRowBytes;
   // 32-row blocks are whole multiples of the swizzle period, so block i only adds i*32*rowBytes.
   static_assert((32 * C::kRowBytes) % (256 * L::kLineParam) == 0, "a 32-row block must span whole swizzle periods");
-  // Fragment `idx` of slice kk: the first kTm are lhs row blocks, the rest rhs column blocks.
-  auto read_frag = [&](int stage, int kk, int idx, u32x4 *af, u32x4 *bf) {
-    const char *base = lds + stage * C::kStageBytes + frag_off[kk];
-    if (idx < C::kTm) af[idx] = *(const u32x4 *)(base + a_rows + idx * 32 * C::kRowBytes);
-    else bf[idx - C::kTm] = *(const u32x4 *)(base + b_rows + (idx - C::kTm) * 32 * C::kRowBytes);
+  // Read `idx` of slice kk (0 .. kReads-1): the first kTm*CH are lhs row blocks, the rest rhs column blocks.
+  auto read_frag = [&](int stage, int kk, int idx, Frag *af, Frag *bf) {
+    const int blk = idx / CH, c = idx % CH;
+    const char *base = lds + stage * C::kStageBytes + frag_off[kk][c];
+    if (blk < C::kTm) af[blk].c[c] = *(const u32x4 *)(base + a_rows + blk * 32 * C::kRowBytes);
+    else bf[blk - C::kTm].c[c] = *(const u32x4 *)(base + b_rows + (blk - C::kTm) * 32 * C::kRowBytes);
   };
-  auto read_frags = [&](int stage, int kk, u32x4 *af, u32x4 *bf) {
+  auto read_frags = [&](int stage, int kk, Frag *af, Frag *bf) {
 #pragma unroll
-    for (int idx = 0; idx < C::kTm + C::kTn; ++idx) read_frag(stage, kk, idx, af, bf);
-  };
-  auto multiply = [&](const u32x4 *af, const u32x4 *bf) {
-#pragma unroll
-    for (int i = 0; i < C::kTm; ++i)
-#pragma unroll
-      for (int j = 0; j < C::kTn; ++j) acc[i][j] = Mfma32x32x16<T>::run(bf[j], af[i], acc[i][j]);
+    for (int idx = 0; idx < (C::kTm + C::kTn) * CH; ++idx) read_frag(stage, kk, idx, af, bf);
   };
 
   using Yes = std::integral_constant<bool, true>;
   using No = std::integral_constant<bool, false>;
-  constexpr int kReads = C::kTm + C::kTn, kMfmas = C::kTm * C::kTn;
-  static_assert(kMfmas >= kReads, "not enough matrix instructions per slice to pace the LDS reads");
+  constexpr int kReads = (C::kTm + C::kTn) * CH, kMfmas = C::kTm * C::kTn;
+  constexpr int kReadsPerMfma = (kReads + kMfmas - 1) / kMfmas;  // LDS reads issued behind each matrix instruction
 
   if constexpr (STAGES == 2) {
     // Two stages (the ring depth of the reference fixture, matmul.mlir:19-22).  The one barrier per
@@ -273,15 +292,12 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     // the first ones (tile kt+2) in the last slice of tile kt, right after the barrier, the rest in
     // the first slices of tile kt+1.
     static_assert(KK >= 2 && KK % 2 == 0, "needs an even number of K-slices per tile");
-#ifndef KAPY_LOAD_SPACING
-#define KAPY_LOAD_SPACING 2
-#endif
     // (narrower tiles have fewer matrix instructions per load: they fall back to a denser spacing)
-    constexpr int kFit = ((KK - 1) * kMfmas) / kLoadsPerTile;
-    constexpr int kLoadSpacing = kFit < 1 ? 1 : (kFit < KAPY_LOAD_SPACING ? kFit : KAPY_LOAD_SPACING);
+    constexpr int kWanted = 64 / T::kMfmaClocks, kFit = ((KK - 1) * kMfmas) / kLoadsPerTile;
+    constexpr int kLoadSpacing = kFit < 1 ? 1 : (kFit < kWanted ? kFit : kWanted);
     constexpr int kEarly = kMfmas / kLoadSpacing < kLoadsPerTile ? kMfmas / kLoadSpacing : kLoadsPerTile;  // issued in the last slice
     static_assert((kLoadsPerTile - kEarly) * kLoadSpacing <= (KK - 1) * kMfmas, "late loads must go out before the barrier that waits for them");
-    u32x4 af[2][C::kTm], bf[2][C::kTn];
+    Frag af[2][C::kTm], bf[2][C::kTn];
     issue_loads(0, 0);
     if (KT > 1) {
       issue_loads(1, 1);
@@ -297,7 +313,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       const int stage = kt & 1;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
-        u32x4 *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
+        Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
         if (kk == KK - 1) {
           if constexpr (has_next.value) {
             __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));  // own loads of tile kt+1 landed; own reads of this stage returned
@@ -307,11 +323,15 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
         for (int g = 0; g < kMfmas; ++g) {
           const int i = g / C::kTn, j = g % C::kTn;
-          acc[i][j] = Mfma32x32x16<T>::run(b_cur[j], a_cur[i], acc[i][j]);
+          acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
           __builtin_amdgcn_sched_barrier(0);
-          if (g < kReads) {
-            if (kk + 1 < KK) read_frag(stage, kk + 1, g, a_nxt, b_nxt);
-            else if constexpr (has_next.value) read_frag(stage ^ 1, 0, g, a_nxt, b_nxt);
+#pragma unroll
+          for (int t = 0; t < kReadsPerMfma; ++t) {
+            const int idx = g * kReadsPerMfma + t;
+            if (idx < kReads) {
+              if (kk + 1 < KK) read_frag(stage, kk + 1, idx, a_nxt, b_nxt);
+              else if constexpr (has_next.value) read_frag(stage ^ 1, 0, idx, a_nxt, b_nxt);
+            }
           }
           if (g % kLoadSpacing == 0) {
             const int slot = (kk * kMfmas + g) / kLoadSpacing;  // load slots counted from the start of the tile
@@ -339,7 +359,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     // fragments of the next K-slice are always fetched one slice ahead, across tile boundaries
     // (the register double-buffering of the reference fixture, matmul.mlir:51-91).
     static_assert(KK % 2 == 0, "fragment double-buffering needs an even number of K-slices per tile");
-    u32x4 af[2][C::kTm], bf[2][C::kTn];
+    Frag af[2][C::kTm], bf[2][C::kTn];
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
       if (s < KT) issue_loads(s, s);
@@ -365,15 +385,19 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       static_assert(KK * kMfmas >= kLoadsPerTile, "not enough matrix instructions per tile to pace the global loads");
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
-        u32x4 *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
+        Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
 #pragma unroll
         for (int g = 0; g < kMfmas; ++g) {
           const int i = g / C::kTn, j = g % C::kTn;
-          acc[i][j] = Mfma32x32x16<T>::run(b_cur[j], a_cur[i], acc[i][j]);
+          acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
           __builtin_amdgcn_sched_barrier(0);
-          if (g < kReads) {
-            if (kk + 1 < KK) read_frag(stage, kk + 1, g, a_nxt, b_nxt);
-            else if constexpr (has_next.value) read_frag(next_stage, 0, g, a_nxt, b_nxt);
+#pragma unroll
+          for (int t = 0; t < kReadsPerMfma; ++t) {
+            const int idx = g * kReadsPerMfma + t;
+            if (idx < kReads) {
+              if (kk + 1 < KK) read_frag(stage, kk + 1, idx, a_nxt, b_nxt);
+              else if constexpr (has_next.value) read_frag(next_stage, 0, idx, a_nxt, b_nxt);
+            }
           }
           // the tile's LDS-direct loads are spread one per matrix instruction over the whole tile
           if constexpr (has_next.value && loads.value)
@@ -453,7 +477,7 @@ enum OperandMode { kKContig = 0, kRowContig = 1, kStrided = 2 };
 
 template <typename T, bool PACKED>
 __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, int b_mode) {
-  using L = TileLayout<kSBK>;
+  using L = TileLayout<kSBK * 2>;
   __shared__ __attribute__((aligned(1024))) char lds[(kSBM + kSBN) * kSBK * 2];
   char *sa = lds, *sb = lds + kSBM * kSBK * 2;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -526,7 +550,7 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma32x32x16<T>::run(bf[j], af[i], acc[i][j]);
+        for (int j = 0; j < 2; ++j) acc[i][j] = T::mfma(&bf[j], &af[i], acc[i][j]);
     }
   }
 #pragma unroll
@@ -544,7 +568,7 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
 // 16-bit row-major result with 8-byte aligned rows, no accumulator input, RN: the packed epilogue.
 bool packed_epilogue(const GemmParams &p) {
   return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16) && p.d_sn == 1 && p.acc_dtype < 0 && !p.rz &&
-         ((uintptr_t)p.d & 7) == 0 && (p.d_sm * 2) % 8 == 0;
+         ((uintptr_t)p.d & 7) == 0 && (p.d_sm * 2) % 8 == 0 && (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
@@ -652,6 +676,28 @@ const TnVariant kTnVariants[] = {
 
 int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
 
+template <int BM, int BN, int BK, int WM, int WN, int S>
+int launch_f8(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
+  // the kernel issues mfma(rhs fragment, lhs fragment): the first format selector is the rhs's
+  switch (rhs_fmt * 2 + lhs_fmt) {
+  case 0: return launch_tn<F8<0, 0>, BM, BN, BK, WM, WN, S>(p, s);
+  case 1: return launch_tn<F8<0, 1>, BM, BN, BK, WM, WN, S>(p, s);
+  case 2: return launch_tn<F8<1, 0>, BM, BN, BK, WM, WN, S>(p, s);
+  default: return launch_tn<F8<1, 1>, BM, BN, BK, WM, WN, S>(p, s);
+  }
+}
+
+}  // namespace
+
+int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
+  if (p.a_sm * 256 >= (int64_t(1) << 31) || p.b_sn * 256 >= (int64_t(1) << 31)) return KAPY_ERR_UNSUPPORTED;
+  if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
+    return launch_f8<256, 256, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
+  if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
+  return KAPY_ERR_UNSUPPORTED;
+}
+
+namespace {
 }  // namespace
 
 // Implemented in matmul_f8.hip.
@@ -685,6 +731,7 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   p.b = view_base(rhs);
   p.acc = acc ? view_base(acc) : nullptr;
   p.d = (char *)view_base(result);
+  p.row_scale = p.col_scale = nullptr;
   p.a_sm = lhs->stride0; p.a_sk = lhs->stride1;
   p.b_sk = rhs->stride0; p.b_sn = rhs->stride1;
   p.acc_sm = acc ? acc->stride0 : 0; p.acc_sn = acc ? acc->stride1 : 0;
@@ -730,10 +777,11 @@ int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling
     return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: only f16 / bf16 operand tiles are described here");
   Swizzle s;
   switch (tile_k) {
-  case 32: s = TileLayout<32>::kSwizzle; break;
-  case 64: s = TileLayout<64>::kSwizzle; break;
+  case 32: s = TileLayout<64>::kSwizzle; break;
+  case 64: s = TileLayout<128>::kSwizzle; break;
   default: return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: tile_k must be 32 or 64");
   }
+  s.stride0 = tile_k;  // the search runs on bytes; report the row stride in elements
   out->stride0 = s.stride0;
   out->stride1 = s.stride1;
   out->bank_param = s.bank_param;

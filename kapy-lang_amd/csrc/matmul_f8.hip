@@ -14,6 +14,7 @@
 //   naive_kernel   any strides / ragged K: one output element per lane, software decode.
 #include "common.hpp"
 #include "layout.hpp"
+#include "matmul_params.hpp"
 #include "numeric.hpp"
 
 namespace kapy {
@@ -129,6 +130,18 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   p.rz = cfg && cfg->rmode == KAPY_RZ;
   if (p.M == 0 || p.N == 0) return KAPY_OK;
   bool k_contig = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(a, 1) == 16 && vector_bytes(b, 0) == 16 && p.K % 128 == 0 && p.K > 0;
+  // Many rows: the tiled LDS-direct kernel (MFMA-bound).  Few rows: the skinny kernel (HBM-bound).
+  if (k_contig && p.M >= 128 && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
+    GemmParams g;
+    g.a = (const char *)p.a; g.b = (const char *)p.b; g.acc = nullptr; g.d = p.d;
+    g.row_scale = row_scale; g.col_scale = col_scale;
+    g.a_sm = p.a_sm; g.a_sk = 1; g.b_sn = p.b_sn; g.b_sk = 1;
+    g.acc_sm = g.acc_sn = 0; g.d_sm = p.d_sm; g.d_sn = p.d_sn;
+    g.M = p.M; g.N = p.N; g.K = p.K;
+    g.acc_dtype = -1; g.d_dtype = p.d_dtype; g.rz = p.rz; g.tiles_m = g.tiles_n = 0;
+    int rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), s);
+    if (rc != KAPY_ERR_UNSUPPORTED) return rc;
+  }
   if (k_contig) {
     dim3 grid((unsigned)((p.N + 15) / 16), (unsigned)((p.M + 15) / 16));
     if (grid.y <= 65535) {

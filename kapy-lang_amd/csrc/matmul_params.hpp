@@ -1,0 +1,27 @@
+// matmul_params.hpp — kernel argument block shared by the 16-bit and fp8 matmul paths.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace kapy {
+
+struct GemmParams {
+  const char *a, *b, *acc;
+  char *d;
+  const float *row_scale, *col_scale;  // optional fp32 scales applied to the accumulator (both or neither)
+  int64_t a_sm, a_sk;  // lhs element strides along M and K
+  int64_t b_sn, b_sk;  // rhs element strides along N and K
+  int64_t acc_sm, acc_sn, d_sm, d_sn;
+  int32_t M, N, K;
+  int32_t acc_dtype;  // -1: no accumulator input
+  int32_t d_dtype;
+  int32_t rz;         // final cast rounds toward zero
+  int32_t tiles_m, tiles_n;
+};
+
+// Tiled LDS-direct MFMA kernel on fp8 operands (both K-contiguous, extents multiples of the tile).
+// lhs_fmt / rhs_fmt: 0 = E4M3, 1 = E5M2.  Returns KAPY_ERR_UNSUPPORTED when no compiled tile fits,
+// without having launched anything.
+int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s);
+
+}  // namespace kapy

@@ -42,6 +42,38 @@ def test_scaled_f8_small(ko, M, N, K):
     assert _frob(ko, to_host(dd, np.uint16, (M, N)), want) <= FROB_TOL
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (128, 256, 384), (256, 256, 256), (384, 128, 512), (512, 768, 1024), (1024, 2560, 256)])
+def test_scaled_f8_tiled_kernel(ko, M, N, K):
+    """Rows >= 128 and extents multiples of the tile: the LDS-direct MFMA kernel (128- and 256-wide tiles)."""
+    aq, sa, wq, sb = _quantised(ko, M, N, K, seed=3)
+    want = np.zeros((M, N), dtype=np.uint16)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                        vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16))) == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N, 2)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    assert _frob(ko, to_host(dd, np.uint16, (M, N)), want) <= FROB_TOL
+
+
+def test_f8_tiled_mixed_formats_f32_result(ko):
+    """e4m3 x e5m2 and e5m2 x e4m3 through the tiled kernel, fp32 result, no scales: checks the operand format
+    selectors of the matrix instruction on both sides."""
+    M, N, K = 256, 128, 256
+    rng = np.random.default_rng(1)
+    e4 = rng.integers(0x20, 0x50, size=(M, K)).astype(np.uint8) | (rng.integers(0, 2, size=(M, K)).astype(np.uint8) << 7)
+    e5 = rng.integers(0x30, 0x48, size=(N, K)).astype(np.uint8) | (rng.integers(0, 2, size=(N, K)).astype(np.uint8) << 7)
+    for (a, adt, b, bdt, m, n) in ((e4, ko.F8E4M3, e5, ko.F8E5M2, M, N), (e5, ko.F8E5M2, e4, ko.F8E4M3, N, M)):
+        want = np.zeros((m, n), dtype=np.float32)
+        assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, m, K, K, 1, adt)), C.byref(ko.mk_global(b, K, n, 1, K, bdt)), None,
+                                  C.byref(ko.mk_global(want, m, n, n, 1, ko.F32)), ko.RN) == 0
+        da, db, dd = to_dev(a), to_dev(b), dev_zeros(m * n, 4)
+        kh.matmul(dglobal(da, m, K, K, 1, adt), dglobal(db, K, n, 1, K, bdt), dglobal(dd, m, n, n, 1, kh.F32))
+        sync()
+        got = to_host(dd, np.float32, (m, n))
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-4
+
+
 def test_plain_f8_matmul_mixed_formats_and_fallback(ko):
     """kapy.matmul on f8 operands without scales: e4m3 x e5m2 mix (Kapy.cpp:484-487), f32 result; and an
     operand layout only the element-wise kernel serves (row-major rhs)."""

@@ -7,8 +7,8 @@
 // gfx950: v_mfma_scale_f32_16x16x128_f8f6f4 with unit E8M0 block scales (2^0); the operand format
 // selectors (cbsz / blgp: 0 = E4M3, 1 = E5M2) carry kapy's mixed-f8 rule.
 //
-//   skinny_kernel  few rows of lhs (decode shape): HBM-bound on the weight.  One workgroup per 16
-//                  output columns, its 4 wavefronts split K; every weight byte is read once,
+//   skinny_kernel  few rows of lhs (decode shape): HBM-bound on the weight.  One workgroup per 16*NG
+//                  output columns, its 8 wavefronts split K; every weight byte is read once,
 //                  straight from global memory into the MFMA operand registers (each lane's 32
 //                  K-contiguous bytes are exactly its operand), partial sums meet in LDS.
 //   naive_kernel   any strides / ragged K: one output element per lane, software decode.
@@ -70,40 +70,57 @@ __device__ __forceinline__ i32x8 load_k32(const uint8_t *base, int64_t stride, i
   return r;
 }
 
-template <int A_FMT, int B_FMT>
-__global__ __launch_bounds__(256) void skinny_kernel(F8Params p) {
-  __shared__ float partial[4][16][16 + 1];
+// Skinny kernel.  Workgroup = 8 wavefronts = 8 contiguous K ranges, NG groups of 16 output columns.
+// A wave first requests everything it will multiply in a chunk of CH K-steps - the weight bytes of
+// its NG column groups and the activation bytes they share - and only then starts the matrix
+// instructions, so that a CU keeps >100 KiB of HBM reads in flight with only 8 resident waves.
+#ifndef KAPY_SKINNY_NG
+#define KAPY_SKINNY_NG 1
+#endif
+#ifndef KAPY_SKINNY_CH
+#define KAPY_SKINNY_CH 8
+#endif
+constexpr int kSkinnyWaves = 8;
+template <int A_FMT, int B_FMT, int NG, int CH>
+__global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
+  __shared__ float partial[kSkinnyWaves][NG][16][16 + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int32_t n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+  const int32_t n0 = blockIdx.x * 16 * NG, m0 = blockIdx.y * 16;
   const int32_t row = lane & 15, kq = (lane >> 4) * 32;  // this lane's row/column and its 32-byte K quarter
-  // K is split in 4 contiguous ranges of whole 128-element MFMA steps
-  const int32_t steps = p.K / 128, per_wave = (steps + 3) / 4;
+  const int32_t steps = p.K / 128, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
   const int32_t s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  constexpr int UNROLL = 4;
-  int32_t s = s_begin;
-  for (; s + UNROLL <= s_end; s += UNROLL) {
-    i32x8 bw[UNROLL], aw[UNROLL];
+  f32x4 acc[NG];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) bw[u] = load_k32(p.b, p.b_sn, n0 + row, p.N, (s + u) * 128 + kq);
+  for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int32_t s = s_begin; s < s_end; s += CH) {
+    i32x8 bw[NG][CH], aw[CH];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) aw[u] = load_k32(p.a, p.a_sm, m0 + row, p.M, (s + u) * 128 + kq);
+    for (int u = 0; u < CH; ++u) {
+      const bool live = s + u < s_end;
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aw[u], bw[u], acc, A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
-  }
-  for (; s < s_end; ++s) {
-    i32x8 bw = load_k32(p.b, p.b_sn, n0 + row, p.N, s * 128 + kq);
-    i32x8 aw = load_k32(p.a, p.a_sm, m0 + row, p.M, s * 128 + kq);
-    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aw, bw, acc, A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+      for (int g = 0; g < NG; ++g) bw[g][u] = load_k32(p.b, p.b_sn, n0 + 16 * g + row, live ? p.N : 0, (s + u) * 128 + kq);
+    }
+#pragma unroll
+    for (int u = 0; u < CH; ++u) aw[u] = load_k32(p.a, p.a_sm, m0 + row, s + u < s_end ? p.M : 0, (s + u) * 128 + kq);
+#pragma unroll
+    for (int u = 0; u < CH; ++u)
+#pragma unroll
+      for (int g = 0; g < NG; ++g)
+        acc[g] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aw[u], bw[g][u], acc[g], A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
   }
   // accumulator register v of lane l: row 4*(l/16) + v, column l%16
 #pragma unroll
-  for (int v = 0; v < 4; ++v) partial[wave][4 * (lane >> 4) + v][lane & 15] = acc[v];
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) partial[wave][g][4 * (lane >> 4) + v][lane & 15] = acc[g][v];
   __syncthreads();
-  const int m = threadIdx.x >> 4, n = threadIdx.x & 15;
-  float sum = (partial[0][m][n] + partial[1][m][n]) + (partial[2][m][n] + partial[3][m][n]);
-  finish(p, m0 + m, n0 + n, sum);
+  for (int e = threadIdx.x; e < NG * 256; e += 64 * kSkinnyWaves) {
+    const int g = e >> 8, m = (e >> 4) & 15, n = e & 15;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kSkinnyWaves; ++w) sum += partial[w][g][m][n];
+    finish(p, m0 + m, n0 + 16 * g + n, sum);
+  }
 }
 
 int fmt_of(int dtype) { return dtype == KAPY_F8E5M2 ? 1 : 0; }
@@ -143,13 +160,14 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
   }
   if (k_contig) {
-    dim3 grid((unsigned)((p.N + 15) / 16), (unsigned)((p.M + 15) / 16));
+    constexpr int NG = KAPY_SKINNY_NG, CH = KAPY_SKINNY_CH;
+    dim3 grid((unsigned)((p.N + 16 * NG - 1) / (16 * NG)), (unsigned)((p.M + 15) / 16));
     if (grid.y <= 65535) {
       int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
-      if (fa == 0 && fb == 0) skinny_kernel<0, 0><<<grid, 256, 0, s>>>(p);
-      else if (fa == 0) skinny_kernel<0, 1><<<grid, 256, 0, s>>>(p);
-      else if (fb == 0) skinny_kernel<1, 0><<<grid, 256, 0, s>>>(p);
-      else skinny_kernel<1, 1><<<grid, 256, 0, s>>>(p);
+      if (fa == 0 && fb == 0) skinny_kernel<0, 0, NG, CH><<<grid, 64 * kSkinnyWaves, 0, s>>>(p);
+      else if (fa == 0) skinny_kernel<0, 1, NG, CH><<<grid, 64 * kSkinnyWaves, 0, s>>>(p);
+      else if (fb == 0) skinny_kernel<1, 0, NG, CH><<<grid, 64 * kSkinnyWaves, 0, s>>>(p);
+      else skinny_kernel<1, 1, NG, CH><<<grid, 64 * kSkinnyWaves, 0, s>>>(p);
       KAPY_HIP_CHECK(hipGetLastError());
       return KAPY_OK;
     }

@@ -56,7 +56,7 @@ def _events(fn, steps, warmup):
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the
 # same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {"gelu": 268406784, "transpose": 268450816}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -185,7 +185,7 @@ def cpu_baseline_gelu(sample_rows=256):
         ko.elementwise(prog, [gx, gb], go)
         reps += 1
         dt = time.perf_counter() - t0
-        if dt > 10.0 or reps >= 50:
+        if dt > 10.0:
             break
     nbytes = (2 * sample_rows * n * 2 + n * 2) * reps
     return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": ko.lib().ko_num_threads(), "kind": "port",

@@ -184,7 +184,8 @@ typedef struct kapy_matmul_cfg {
   int32_t impl_way;              /* kapy_matmul_impl_way                                         */
   int32_t tile_m, tile_n, tile_k; /* workgroup tile; 0 = library's choice                          */
   int32_t rmode;                 /* rounding of the final cast to result dtype (default RN)      */
-  int32_t stages;                /* depth of the LDS ring (the reference fixture uses 2); 0 = library's choice */
+  int32_t stages;                /* depth of the LDS ring in tiles (the reference fixture uses 2); 25 = the 2.5-tile
+                                    ring of half-operand units; 0 = library's choice */
   int32_t waves;                 /* wavefronts per workgroup (num_warps of the reference); 0 = library's choice */
   int32_t reserved;
 } kapy_matmul_cfg;

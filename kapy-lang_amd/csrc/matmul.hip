@@ -164,6 +164,7 @@ __device__ __forceinline__ void tile_of_block(const GemmParams &p, int32_t &tm, 
 // ---------------------------------------------------------------------------------------------
 // TN kernel.  BM x BN x BK workgroup tile, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN)
 // block of 32x32 accumulators.  STAGES-deep LDS ring filled by LDS-direct loads.
+constexpr int kRing25 = 25;  // value of STAGES (and of kapy_matmul_cfg.stages) that selects the 2.5-tile ring
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 struct TnConfig {
   static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves;
@@ -174,7 +175,9 @@ struct TnConfig {
   static constexpr int kLoadsA = BM / kRowsPerLoad, kLoadsB = BN / kRowsPerLoad;
   static constexpr int kLoadsAPerWave = kLoadsA / kWaves, kLoadsBPerWave = kLoadsB / kWaves;
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
-  static constexpr int kLdsBytes = STAGES * kStageBytes;
+  // STAGES == kRing25: a ring of ten quarter-tile units (half an operand tile each), i.e. 2.5 tiles
+  static constexpr int kUnitBytes = kStageBytes / 4;
+  static constexpr int kLdsBytes = STAGES == kRing25 ? 10 * kUnitBytes : STAGES * kStageBytes;
   static_assert(kLoadsA % kWaves == 0 && kLoadsB % kWaves == 0, "loads must divide evenly over the wavefronts");
   static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % T::kSliceK == 0, "wave tile must be a multiple of the MFMA tile");
 };
@@ -246,6 +249,20 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   }
 
   const int KT = p.K / BK;
+#ifdef KAPY_TRACE
+  // tuning builds only: clock stamps of workgroup 0 for K-tiles 32..39 (8 per tile per wave)
+  uint64_t *trace = p.row_scale ? nullptr : (uint64_t *)p.col_scale;
+  auto stamp = [&](int kt, int which) {
+    if (trace && blockIdx.x == KAPY_TRACE && kt >= 32 && kt < 40) {
+      uint64_t t = __builtin_readcyclecounter();
+      if (lane == 0) trace[(wave * 8 + (kt - 32)) * 8 + which] = t;
+    }
+  };
+#define KAPY_STAMP(kt, which) stamp(kt, which)
+  const uint64_t trace_begin = __builtin_readcyclecounter();
+#else
+#define KAPY_STAMP(kt, which)
+#endif
   constexpr int KK = BK / T::kSliceK;                                   // matrix-instruction K-slices per tile
   constexpr int kLoadsPerTile = C::kLoadsAPerWave + C::kLoadsBPerWave;  // per wavefront
   // A fragment: the CH 16-byte chunks one lane feeds a matrix instruction for one operand block.
@@ -279,7 +296,154 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   constexpr int kReads = (C::kTm + C::kTn) * CH, kMfmas = C::kTm * C::kTn;
   constexpr int kReadsPerMfma = (kReads + kMfmas - 1) / kMfmas;  // LDS reads issued behind each matrix instruction
 
-  if constexpr (STAGES == 2) {
+  if constexpr (STAGES == kRing25) {
+    // Ring of ten units, a unit being half an operand tile (unit u of tile j: 0/1 = upper/lower half
+    // of the lhs rows, 2/3 = left/right half of the rhs columns) at ring position (4j + u) mod 10:
+    // all of the 160 KiB of LDS, 2.5 tiles.  A wavefront reads exactly one lhs unit and one rhs unit.
+    // There is one barrier per tile, before the tile's last K-slice; it frees the four units of tile
+    // kt, and they are refilled in this order: rhs half of tile kt+2 (needed one tile time later),
+    // then lhs half of tile kt+3 (needed two tile times later).  That slack lets the loads be spread
+    // evenly over the whole tile time - a steady request stream into the L2 instead of every CU
+    // bursting at the L1's peak rate right after the barrier - without the last ones running late.
+    // Loads for tiles past the end of K are still issued (from the last real tile) into units nobody
+    // reads again: every tile step is then identical and the wait counts are constants.
+    //
+    // The loads are LDS-direct buffer loads: per-lane 32-bit offset (loop invariant) + scalar offset
+    // (the K position) + M0 (the LDS destination), so a load costs one scalar and one vector-memory
+    // instruction and no vector ALU work.  Ring positions repeat every five tiles; the steady-state
+    // loop is unrolled by five so that every LDS address is a constant.
+    static_assert(BM == BN && WM == 2 && WN == 2, "the unit ring assumes equal lhs / rhs halves and 2 x 2 wavefronts");
+    static_assert(KK >= 2 && KK % 2 == 0, "needs an even number of K-slices per tile");
+    constexpr int kUnit = C::kUnitBytes, kHalf = kLoadsPerTile / 2;  // loads per wavefront per operand
+    static_assert(C::kLoadsAPerWave == kHalf && C::kLoadsBPerWave == kHalf && kHalf % 2 == 0, "two equal units per operand");
+    constexpr int kPerUnit = kHalf / 2;
+#ifndef KAPY_RING_SPACING
+#define KAPY_RING_SPACING 0
+#endif
+    constexpr int kEven = (KK * kMfmas) / kLoadsPerTile;
+    constexpr int kLoadSpacing = KAPY_RING_SPACING ? KAPY_RING_SPACING : (kEven < 1 ? 1 : kEven);
+    constexpr int kEarly = kMfmas / kLoadSpacing < kLoadsPerTile ? kMfmas / kLoadSpacing : kLoadsPerTile;
+    static_assert((kLoadsPerTile - kEarly) * kLoadSpacing <= (KK - 1) * kMfmas, "late loads must go out before the barrier that waits for them");
+    // The descriptors must sit in scalar registers (a descriptor in vector registers makes every load
+    // a loop over its distinct values): pin the workgroup-uniform tile pointers with readfirstlane.
+    auto uniform_ptr = [](const char *ptr) {
+      const uint64_t v = (uint64_t)ptr;
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      return (void *)(((uint64_t)hi << 32) | lo);
+    };
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(a_tile), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(b_tile), 0, 0x7fffffff, 0x00020000);
+    const int wave_lds = wave * 1024;
+    auto wrap = [](auto pos) { return pos >= 20 ? pos - 20 : (pos >= 10 ? pos - 10 : pos); };
+    // scalar byte offset of K-tile j in a row, clamped to the last real tile
+    auto k_off = [&](int j) { return min(j, KT - 1) * (BK * EB); };
+    auto load_a = [&](int idx, int pos_of_unit0, int soff) {  // idx: 0 .. kHalf-1, unit idx / kPerUnit
+      const int u = idx / kPerUnit, i = idx % kPerUnit;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + wrap(pos_of_unit0 + u) * kUnit + i * C::kWaves * 1024 + wave_lds),
+                                               16, (int)a_goff[idx], soff, 0, 0);
+    };
+    auto load_b = [&](int idx, int pos_of_unit2, int soff) {
+      const int u = idx / kPerUnit, i = idx % kPerUnit;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + wrap(pos_of_unit2 + u) * kUnit + i * C::kWaves * 1024 + wave_lds),
+                                               16, (int)b_goff[idx], soff, 0, 0);
+    };
+    // Load `slot` (0 .. kLoadsPerTile-1) of the sequence issued after the barrier of the tile at ring
+    // position pos0: slots [0, kHalf) = rhs units of the tile two ahead (they take positions pos0,
+    // pos0+1), the rest = lhs units of the tile three ahead (positions pos0+2, pos0+3).
+    auto ring_load = [&](auto pos0, int slot, int soff_b, int soff_a) {
+      if (slot < kHalf) load_b(slot, pos0, soff_b);
+      else load_a(slot - kHalf, pos0 + 2, soff_a);
+    };
+    Frag af[2][C::kTm], bf[2][C::kTn];
+    // prologue: tiles 0 and 1 whole (lhs units first, then rhs, as the tile steps count them)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int idx = 0; idx < kHalf; ++idx) load_a(idx, 4 * t, k_off(t));
+#pragma unroll
+      for (int idx = 0; idx < kHalf; ++idx) load_b(idx, 4 * t + 2, k_off(t));
+    }
+    // ... and the part of the sequence [rhs of tile 1, lhs of tile 2] that a tile step issues in the
+    // last slice of the tile before (there is none before tile 0)
+    constexpr int kPrologueExtra = kEarly > kHalf ? kEarly - kHalf : 0;
+#pragma unroll
+    for (int slot = kHalf; slot < kHalf + kPrologueExtra; ++slot) ring_load(6, slot, 0, k_off(2));
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoadsPerTile + kPrologueExtra));
+    __builtin_amdgcn_s_barrier();  // tile 0 published
+    {
+      const uint32_t a0 = wm * kUnit, b0 = (2 + wn) * kUnit;
+#pragma unroll
+      for (int idx = 0; idx < kReads; ++idx) {
+        const int blk = idx / CH, c = idx % CH;
+        if (blk < C::kTm) af[0][blk].c[c] = *(const u32x4 *)(lds + a0 + frag_off[0][c] + blk * 32 * C::kRowBytes);
+        else bf[0][blk - C::kTm].c[c] = *(const u32x4 *)(lds + b0 + frag_off[0][c] + (blk - C::kTm) * 32 * C::kRowBytes);
+      }
+    }
+    // One tile at ring position `pos` (an int, or an integral_constant in the unrolled loop).  The
+    // sequence after the barrier of tile kt-1 is [rhs of tile kt+1, lhs of tile kt+2]; its first
+    // kEarly loads went out in the last slice of tile kt-1, the rest go out in the first slices of
+    // tile kt.  (`first`: tile 0, where the prologue has issued the rhs part of that sequence.)
+    auto tile_step = [&](int kt, auto pos, auto first) {
+      const auto prev = wrap(pos + 6), next = wrap(pos + 4);
+      // LDS bases of this wave's operand units in this tile and the next one
+      const uint32_t a_cur_base = wrap(pos + wm) * kUnit, b_cur_base = wrap(pos + 2 + wn) * kUnit;
+      const uint32_t a_nxt_base = wrap(next + wm) * kUnit, b_nxt_base = wrap(next + 2 + wn) * kUnit;
+      const int soff_late_b = k_off(kt + 1), soff_late_a = k_off(kt + 2);   // sequence of tile kt-1
+      const int soff_early_b = k_off(kt + 2), soff_early_a = k_off(kt + 3); // sequence of tile kt
+      auto ring_read = [&](uint32_t a_base, uint32_t b_base, int kk, int idx, Frag *a_dst, Frag *b_dst) {
+        const int blk = idx / CH, c = idx % CH;
+        if (blk < C::kTm) a_dst[blk].c[c] = *(const u32x4 *)(lds + (a_base + frag_off[kk][c]) + blk * 32 * C::kRowBytes);
+        else b_dst[blk - C::kTm].c[c] = *(const u32x4 *)(lds + (b_base + frag_off[kk][c]) + (blk - C::kTm) * 32 * C::kRowBytes);
+      };
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
+        KAPY_STAMP(kt, kk);
+        if (kk == KK - 1) {
+          // tile kt+1 has landed once only the kHalf youngest loads (lhs of tile kt+2) are in flight
+          __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
+          KAPY_STAMP(kt, 4);
+          __builtin_amdgcn_s_barrier();
+          KAPY_STAMP(kt, 5);
+        }
+#pragma unroll
+        for (int g = 0; g < kMfmas; ++g) {
+          const int i = g / C::kTn, j = g % C::kTn;
+          acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int t = 0; t < kReadsPerMfma; ++t) {
+            const int idx = g * kReadsPerMfma + t;
+            if (idx < kReads) {
+              if (kk + 1 < KK) ring_read(a_cur_base, b_cur_base, kk + 1, idx, a_nxt, b_nxt);
+              else ring_read(a_nxt_base, b_nxt_base, 0, idx, a_nxt, b_nxt);
+            }
+          }
+          if (g % kLoadSpacing == 0) {
+            const int slot = (kk * kMfmas + g) / kLoadSpacing;
+            if (kk == KK - 1 && g / kLoadSpacing < kEarly) ring_load(pos, g / kLoadSpacing, soff_early_b, soff_early_a);
+            if (kk < KK - 1 && kEarly + slot < kLoadsPerTile && (!first.value || kEarly + slot >= kHalf))
+              ring_load(prev, kEarly + slot, soff_late_b, soff_late_a);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    };
+    tile_step(0, std::integral_constant<int, 0>{}, Yes{});
+    int kt = 1;
+    for (; kt + 5 <= KT; kt += 5) {
+      tile_step(kt, std::integral_constant<int, 4>{}, No{});
+      tile_step(kt + 1, std::integral_constant<int, 8>{}, No{});
+      tile_step(kt + 2, std::integral_constant<int, 2>{}, No{});
+      tile_step(kt + 3, std::integral_constant<int, 6>{}, No{});
+      tile_step(kt + 4, std::integral_constant<int, 0>{}, No{});
+    }
+    for (int pos = 4; kt < KT; ++kt) {
+      tile_step(kt, pos, No{});
+      pos = wrap(pos + 4);
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // loads issued for tiles past the end still target this workgroup's LDS
+  } else if constexpr (STAGES == 2) {
     // Two stages (the ring depth of the reference fixture, matmul.mlir:19-22).  The one barrier per
     // tile sits BEFORE the tile's last K-slice: by then every wave has fetched the fragments of that
     // last slice, so the stage is free to be refilled, and the next tile is waited for and published.
@@ -314,10 +478,13 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
+        KAPY_STAMP(kt, kk);
         if (kk == KK - 1) {
           if constexpr (has_next.value) {
             __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));  // own loads of tile kt+1 landed; own reads of this stage returned
+            KAPY_STAMP(kt, 4);
             __builtin_amdgcn_s_barrier();
+            KAPY_STAMP(kt, 5);
           }
         }
 #pragma unroll
@@ -413,12 +580,81 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     tile_step(kt, No{}, No{});
   }
 
+#ifdef KAPY_TRACE
+  if (trace && blockIdx.x == KAPY_TRACE && threadIdx.x == 0) {
+    trace[256] = trace_begin;
+    trace[257] = __builtin_readcyclecounter();  // end of the K loop
+  }
+#endif
+  if constexpr (PACKED) {
+    // Packed epilogue (16-bit row-major result, 16-byte aligned rows, no accumulator input, RN), by
+    // 32-row strips of the wave's block through a wave-private LDS strip: accumulator quads (four
+    // consecutive columns of one row per lane) are narrowed and written 8 bytes at a time, read back
+    // 16 bytes per lane along rows, and stored so that one instruction writes whole 128-byte lines
+    // (64 / kChunks rows x kWtn*2 bytes) - the register layout itself would scatter 8-byte pieces
+    // over 32 rows per instruction.  Row stride kWtn*2 + 16 bytes: both the 8-byte writes down the
+    // rows and the 16-byte reads along them then use every LDS bank equally.
+    constexpr int kRowStride = C::kWtn * 2 + 16, kStrip = 32 * kRowStride;
+    constexpr int kChunks = C::kWtn * 2 / 16, kRowsPerStore = 64 / kChunks, kStores = 32 / kRowsPerStore;
+    static_assert(2 * kStrip * C::kWaves <= C::kLdsBytes, "two strips per wavefront must fit the ring");
+    __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+    __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space
+    char *strip0 = lds + wave * 2 * kStrip;
+    const int wrow = lane & 31, wcol = 4 * (lane >> 5);          // this lane's row / first column in a 32x32 block
+    const int rrow = lane / kChunks, rchunk = lane % kChunks;     // and in a read-back instruction
+    const int32_t m_wave = m0 + wm * C::kWtm, n_wave = n0 + wn * C::kWtn;
+    // result type and scaling are uniform: one specialised copy of the loop each, chosen once
+    auto epilogue = [&](auto is_f16, auto scaled) {
 #pragma unroll
-  for (int i = 0; i < C::kTm; ++i)
+      for (int i = 0; i < C::kTm; ++i) {
+        __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
+        char *strip = strip0 + (i & 1) * kStrip;
+        float rs = 1.0f;
+        if constexpr (scaled.value) rs = p.row_scale[m_wave + i * 32 + wrow];
 #pragma unroll
-    for (int j = 0; j < C::kTn; ++j)
-      if (PACKED) store_block_packed(p, m0 + wm * C::kWtm + i * 32, n0 + wn * C::kWtn + j * 32, lane, acc[i][j]);
-      else store_block_generic(p, m0 + wm * C::kWtm + i * 32, n0 + wn * C::kWtn + j * 32, lane, acc[i][j]);
+        for (int j = 0; j < C::kTn; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+            if constexpr (scaled.value) {
+              const f32x4 cs = *(const f32x4 *)(p.col_scale + n_wave + j * 32 + wcol + 8 * q);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
+            }
+            u32x2 w;
+            w[0] = is_f16.value ? pack2_f16_rn(v[0], v[1]) : pack2_bf16_rn(v[0], v[1]);
+            w[1] = is_f16.value ? pack2_f16_rn(v[2], v[3]) : pack2_bf16_rn(v[2], v[3]);
+            *(u32x2 *)(strip + wrow * kRowStride + (j * 32 + wcol + 8 * q) * 2) = w;
+          }
+        // LDS executes a wave's instructions in order: the reads below see the writes above
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < kStores; ++t) {
+          const int row = t * kRowsPerStore + rrow;
+          const u32x4 w = *(const u32x4 *)(strip + row * kRowStride + rchunk * 16);
+          *(u32x4 *)(p.d + ((int64_t)(m_wave + i * 32 + row) * p.d_sm + n_wave + rchunk * 8) * 2) = w;
+        }
+      }
+    };
+    const bool f16 = p.d_dtype == KAPY_F16;
+    if (p.row_scale) {
+      if (f16) epilogue(Yes{}, Yes{});
+      else epilogue(No{}, Yes{});
+    } else {
+      if (f16) epilogue(Yes{}, No{});
+      else epilogue(No{}, No{});
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < C::kTm; ++i)
+#pragma unroll
+      for (int j = 0; j < C::kTn; ++j) store_block_generic(p, m0 + wm * C::kWtm + i * 32, n0 + wn * C::kWtn + j * 32, lane, acc[i][j]);
+  }
+#ifdef KAPY_TRACE
+  if (trace && blockIdx.x == KAPY_TRACE && threadIdx.x == 0) trace[258] = __builtin_readcyclecounter();  // stores issued
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -565,10 +801,10 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
 
 // ---------------------------------------------------------------------------------------------
 // Host side.
-// 16-bit row-major result with 8-byte aligned rows, no accumulator input, RN: the packed epilogue.
+// 16-bit row-major result with 16-byte aligned rows, no accumulator input, RN: the packed epilogue.
 bool packed_epilogue(const GemmParams &p) {
   return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16) && p.d_sn == 1 && p.acc_dtype < 0 && !p.rz &&
-         ((uintptr_t)p.d & 7) == 0 && (p.d_sm * 2) % 8 == 0 && (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
+         ((uintptr_t)p.d & 15) == 0 && (p.d_sm * 2) % 16 == 0 && (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
@@ -667,7 +903,7 @@ struct TnVariant {
 #define KAPY_TN(BM, BN, BK, WM, WN, S) \
   { BM, BN, BK, (WM) * (WN), S, launch_tn<Bf16, BM, BN, BK, WM, WN, S>, launch_tn<F16, BM, BN, BK, WM, WN, S> }
 const TnVariant kTnVariants[] = {
-    KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
+    KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
 #ifdef KAPY_TUNING
     KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2), KAPY_TN(256, 128, 64, 2, 2, 3),
     KAPY_TN(128, 256, 64, 2, 2, 3), KAPY_TN(128, 128, 64, 2, 2, 4), KAPY_TN(256, 256, 32, 2, 2, 5), KAPY_TN(256, 128, 32, 2, 2, 4),
@@ -727,11 +963,17 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
     return fail(KAPY_ERR_UNSUPPORTED, "matmul: %s operands have no matrix instruction on gfx950", dtype_name(lhs->dtype));
 
   GemmParams p;
+#ifdef KAPY_TRACE
+  const char *trace_env = getenv("KAPY_TRACE_PTR");
+#endif
   p.a = view_base(lhs);
   p.b = view_base(rhs);
   p.acc = acc ? view_base(acc) : nullptr;
   p.d = (char *)view_base(result);
   p.row_scale = p.col_scale = nullptr;
+#ifdef KAPY_TRACE
+  if (trace_env) p.col_scale = (const float *)strtoull(trace_env, nullptr, 0);
+#endif
   p.a_sm = lhs->stride0; p.a_sk = lhs->stride1;
   p.b_sk = rhs->stride0; p.b_sn = rhs->stride1;
   p.acc_sm = acc ? acc->stride0 : 0; p.acc_sn = acc ? acc->stride1 : 0;

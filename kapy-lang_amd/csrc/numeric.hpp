@@ -29,6 +29,22 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rz(float x) {
   return (uint16_t)(u >> 16);
 }
 
+// two fp32 -> one 32-bit word of two bf16 / f16, round-to-nearest-even (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32)
+__device__ __forceinline__ uint32_t pack2_bf16_rn(float lo, float hi) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  bf16x2_t h;
+  h[0] = (__bf16)lo;
+  h[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, h);
+}
+__device__ __forceinline__ uint32_t pack2_f16_rn(float lo, float hi) {
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  half2_t h;
+  h[0] = (_Float16)lo;
+  h[1] = (_Float16)hi;
+  return __builtin_bit_cast(uint32_t, h);
+}
+
 // ---- f16 ------------------------------------------------------------------------------------
 __device__ __forceinline__ float f16_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t f32_to_f16_rn(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }

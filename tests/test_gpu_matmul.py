@@ -62,7 +62,7 @@ def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):
         assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
 
 
-TN_VARIANTS = [((256, 256, 64), 2), ((256, 256, 32), 4), ((128, 128, 64), 2), ((128, 128, 32), 4)]
+TN_VARIANTS = [((256, 256, 64), 25), ((256, 256, 64), 2), ((256, 256, 32), 4), ((128, 128, 64), 2), ((128, 128, 32), 4)]
 
 
 @pytest.mark.parametrize("tile,stages", TN_VARIANTS)
@@ -71,7 +71,7 @@ def test_tn_roofline_kernel_every_variant(ko, tile, stages):
     configuration forced through kapy_matmul_cfg, including K of 1, 2, 3 and many tiles (pipeline prologue / tail)."""
     bm, bn, bk = tile
     for dt in (kh.BF16, kh.F16):
-        for (M, N, K) in ((bm, bn, bk), (bm, bn, 2 * bk), (bm, 2 * bn, 3 * bk), (2 * bm, bn, 4 * bk), (3 * bm, 2 * bn, 16 * bk)):
+        for (M, N, K) in ((bm, bn, bk), (bm, bn, 2 * bk), (bm, 2 * bn, 3 * bk), (2 * bm, bn, 4 * bk), (bm, bn, 7 * bk), (3 * bm, 2 * bn, 16 * bk)):
             got, want = _run(ko, dt, M, N, K, True, False, seed=5, tile=tile, stages=stages)
             assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
     got32, want32 = _run(ko, kh.BF16, 2 * bm, 2 * bn, 8 * bk, True, False, out_dtype=kh.F32, seed=5, tile=tile, stages=stages)

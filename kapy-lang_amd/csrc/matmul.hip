@@ -654,6 +654,13 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   }
 #ifdef KAPY_TRACE
   if (trace && blockIdx.x == KAPY_TRACE && threadIdx.x == 0) trace[258] = __builtin_readcyclecounter();  // stores issued
+  if (trace && threadIdx.x == 0) {  // per-workgroup timeline: begin, end, where it ran
+    uint64_t *w = trace + 512 + 4 * blockIdx.x;
+    w[0] = trace_begin;
+    w[1] = __builtin_readcyclecounter();
+    w[2] = __builtin_amdgcn_s_getreg(4 | (31 << 11));    // HW_ID
+    w[3] = __builtin_amdgcn_s_getreg(20 | (31 << 11));   // XCC_ID
+  }
 #endif
 }
 
@@ -925,10 +932,13 @@ int launch_f8(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
 
 }  // namespace
 
+#ifndef KAPY_F8_STAGES
+#define KAPY_F8_STAGES kRing25
+#endif
 int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
   if (p.a_sm * 256 >= (int64_t(1) << 31) || p.b_sn * 256 >= (int64_t(1) << 31)) return KAPY_ERR_UNSUPPORTED;
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
-    return launch_f8<256, 256, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
+    return launch_f8<256, 256, 128, 2, 2, KAPY_F8_STAGES>(p, lhs_fmt, rhs_fmt, s);
   if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
   return KAPY_ERR_UNSUPPORTED;
 }

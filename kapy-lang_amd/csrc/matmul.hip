@@ -46,15 +46,35 @@ typedef int i32x8 __attribute__((ext_vector_type(8)));
 // Operand element policies: bytes per element, the K extent of one matrix instruction, how many
 // 16-byte LDS chunks a lane feeds it per operand, and its duration in clocks (4 per pass).
 struct Bf16 {
-  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32;
+  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32, kM = 32;
+  using Acc = f32x16;
   static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
   }
 };
 struct F16 {
-  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32;
+  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32, kM = 32;
+  using Acc = f32x16;
   static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
+  }
+};
+// The 16x16x32 forms: kM = 16 rows per operand block, four K-groups of lanes.  Same flops per clock
+// as 32x32x16, but each accumulator register is read and written once per 32 K instead of per 16 K;
+// under sustained load the chip holds a ~13% higher clock with them (it is power-limited), which
+// outweighs the doubled operand-register reads.
+struct Bf16M16 {
+  static constexpr int kBytes = 2, kSliceK = 32, kChunks = 1, kMfmaClocks = 16, kM = 16;
+  using Acc = f32x4;
+  static __device__ __forceinline__ f32x4 mfma(const u32x4 *a, const u32x4 *b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
+  }
+};
+struct F16M16 {
+  static constexpr int kBytes = 2, kSliceK = 32, kChunks = 1, kMfmaClocks = 16, kM = 16;
+  using Acc = f32x4;
+  static __device__ __forceinline__ f32x4 mfma(const u32x4 *a, const u32x4 *b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
   }
 };
 // OCP fp8, v_mfma_scale_f32_32x32x64_f8f6f4 with unit block scales (E8M0 127 = 2^0).  AF / BF are the
@@ -62,7 +82,8 @@ struct F16 {
 // f8 types mix, Kapy.cpp:484-487).  A lane feeds 32 K-contiguous bytes per operand: two chunks.
 template <int AF, int BF>
 struct F8 {
-  static constexpr int kBytes = 1, kSliceK = 64, kChunks = 2, kMfmaClocks = 64;
+  static constexpr int kBytes = 1, kSliceK = 64, kChunks = 2, kMfmaClocks = 64, kM = 32;
+  using Acc = f32x16;
   static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
     i32x8 av = {(int)a[0][0], (int)a[0][1], (int)a[0][2], (int)a[0][3], (int)a[1][0], (int)a[1][1], (int)a[1][2], (int)a[1][3]};
     i32x8 bv = {(int)b[0][0], (int)b[0][1], (int)b[0][2], (int)b[0][3], (int)b[1][0], (int)b[1][1], (int)b[1][2], (int)b[1][3]};
@@ -145,6 +166,11 @@ __device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_
   const int32_t m = m_base + (lane & 31);
   for (int v = 0; v < 16; ++v) store_result(p, m, n_base + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), acc[v]);
 }
+// 16x16 block: register v of lane l holds D[m = l%16][n = 4*(l/16) + v].
+__device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, f32x4 acc) {
+  const int32_t m = m_base + (lane & 15);
+  for (int v = 0; v < 4; ++v) store_result(p, m, n_base + 4 * (lane >> 4) + v, acc[v]);
+}
 
 // Workgroup id -> output tile.  Consecutive workgroup ids land on different XCDs (8 of them, each
 // with its own L2), so ids are first regrouped per XCD, then each XCD walks a compact band of
@@ -169,7 +195,7 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 struct TnConfig {
   static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves;
   static constexpr int kWtm = BM / WM, kWtn = BN / WN;       // wave tile
-  static constexpr int kTm = kWtm / 32, kTn = kWtn / 32;     // 32x32 accumulators per wave
+  static constexpr int kTm = kWtm / T::kM, kTn = kWtn / T::kM;  // accumulator blocks per wave
   static constexpr int kRowBytes = BK * T::kBytes;
   static constexpr int kRowsPerLoad = 1024 / kRowBytes;      // rows one LDS-direct wave instruction fills
   static constexpr int kLoadsA = BM / kRowsPerLoad, kLoadsB = BN / kRowsPerLoad;
@@ -179,7 +205,7 @@ struct TnConfig {
   static constexpr int kUnitBytes = kStageBytes / 4;
   static constexpr int kLdsBytes = STAGES == kRing25 ? 10 * kUnitBytes : STAGES * kStageBytes;
   static_assert(kLoadsA % kWaves == 0 && kLoadsB % kWaves == 0, "loads must divide evenly over the wavefronts");
-  static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % T::kSliceK == 0, "wave tile must be a multiple of the MFMA tile");
+  static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % T::kSliceK == 0 && 32 % T::kM == 0, "wave tile must be a multiple of the MFMA tile");
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
@@ -233,15 +259,18 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     for (int idx = 0; idx < C::kLoadsAPerWave + C::kLoadsBPerWave; ++idx) issue_load(stage, kt, idx);
   };
 
-  // LDS byte offsets of this lane's operand reads: row (lane % 32) of each 32-row block, 16-byte
-  // chunk (2*kk + lane/32) of the K slice kk.
-  const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
+  // LDS byte offsets of this lane's operand reads: row (lane % KM) of each KM-row block, 16-byte
+  // chunks of K-group (lane / KM) of the K slice kk.
+  constexpr int KM = T::kM, kGroups = 64 / KM;  // rows per operand block; K-groups of lanes
+  const uint32_t frag_row = lane % KM, frag_grp = lane / KM;
 
-  f32x16 acc[C::kTm][C::kTn];
+  using Acc = typename T::Acc;
+  constexpr int kAccRegs = KM * KM / 64;
+  Acc acc[C::kTm][C::kTn];
   {
-    f32x16 zero;
+    Acc zero;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+    for (int v = 0; v < kAccRegs; ++v) zero[v] = 0.f;
 #pragma unroll
     for (int i = 0; i < C::kTm; ++i)
 #pragma unroll
@@ -275,16 +304,16 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-    for (int c = 0; c < CH; ++c) frag_off[kk][c] = L::offset(frag_row, (2 * kk + frag_half) * CH + c);
+    for (int c = 0; c < CH; ++c) frag_off[kk][c] = L::offset(frag_row, (kGroups * kk + frag_grp) * CH + c);
   const uint32_t a_rows = (wm * C::kWtm) * C::kRowBytes, b_rows = BM * C::kRowBytes + (wn * C::kWtn) * C::kRowBytes;
   // 32-row blocks are whole multiples of the swizzle period, so block i only adds i*32*rowBytes.
-  static_assert((32 * C::kRowBytes) % (256 * L::kLineParam) == 0, "a 32-row block must span whole swizzle periods");
+  static_assert((KM * C::kRowBytes) % (256 * L::kLineParam) == 0, "an operand block must span whole swizzle periods");
   // Read `idx` of slice kk (0 .. kReads-1): the first kTm*CH are lhs row blocks, the rest rhs column blocks.
   auto read_frag = [&](int stage, int kk, int idx, Frag *af, Frag *bf) {
     const int blk = idx / CH, c = idx % CH;
     const char *base = lds + stage * C::kStageBytes + frag_off[kk][c];
-    if (blk < C::kTm) af[blk].c[c] = *(const u32x4 *)(base + a_rows + blk * 32 * C::kRowBytes);
-    else bf[blk - C::kTm].c[c] = *(const u32x4 *)(base + b_rows + (blk - C::kTm) * 32 * C::kRowBytes);
+    if (blk < C::kTm) af[blk].c[c] = *(const u32x4 *)(base + a_rows + blk * KM * C::kRowBytes);
+    else bf[blk - C::kTm].c[c] = *(const u32x4 *)(base + b_rows + (blk - C::kTm) * KM * C::kRowBytes);
   };
   auto read_frags = [&](int stage, int kk, Frag *af, Frag *bf) {
 #pragma unroll
@@ -375,8 +404,8 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
       for (int idx = 0; idx < kReads; ++idx) {
         const int blk = idx / CH, c = idx % CH;
-        if (blk < C::kTm) af[0][blk].c[c] = *(const u32x4 *)(lds + a0 + frag_off[0][c] + blk * 32 * C::kRowBytes);
-        else bf[0][blk - C::kTm].c[c] = *(const u32x4 *)(lds + b0 + frag_off[0][c] + (blk - C::kTm) * 32 * C::kRowBytes);
+        if (blk < C::kTm) af[0][blk].c[c] = *(const u32x4 *)(lds + a0 + frag_off[0][c] + blk * KM * C::kRowBytes);
+        else bf[0][blk - C::kTm].c[c] = *(const u32x4 *)(lds + b0 + frag_off[0][c] + (blk - C::kTm) * KM * C::kRowBytes);
       }
     }
     // One tile at ring position `pos` (an int, or an integral_constant in the unrolled loop).  The
@@ -392,8 +421,8 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       const int soff_early_b = k_off(kt + 2), soff_early_a = k_off(kt + 3); // sequence of tile kt
       auto ring_read = [&](uint32_t a_base, uint32_t b_base, int kk, int idx, Frag *a_dst, Frag *b_dst) {
         const int blk = idx / CH, c = idx % CH;
-        if (blk < C::kTm) a_dst[blk].c[c] = *(const u32x4 *)(lds + (a_base + frag_off[kk][c]) + blk * 32 * C::kRowBytes);
-        else b_dst[blk - C::kTm].c[c] = *(const u32x4 *)(lds + (b_base + frag_off[kk][c]) + (blk - C::kTm) * 32 * C::kRowBytes);
+        if (blk < C::kTm) a_dst[blk].c[c] = *(const u32x4 *)(lds + (a_base + frag_off[kk][c]) + blk * KM * C::kRowBytes);
+        else b_dst[blk - C::kTm].c[c] = *(const u32x4 *)(lds + (b_base + frag_off[kk][c]) + (blk - C::kTm) * KM * C::kRowBytes);
       };
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
@@ -600,34 +629,39 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
     __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space
     char *strip0 = lds + wave * 2 * kStrip;
-    const int wrow = lane & 31, wcol = 4 * (lane >> 5);          // this lane's row / first column in a 32x32 block
+    const int wrow = lane % KM, wcol = 4 * (lane / KM);           // this lane's row / first column in an accumulator block
     const int rrow = lane / kChunks, rchunk = lane % kChunks;     // and in a read-back instruction
     const int32_t m_wave = m0 + wm * C::kWtm, n_wave = n0 + wn * C::kWtn;
+    constexpr int kBlocksPerStrip = 32 / KM, kStrips = C::kWtm / 32;
+    constexpr int kQuads = kAccRegs / 4, kQuadStep = 4 * kGroups;  // register quads of a block: 4 consecutive columns each, kQuadStep apart
     // result type and scaling are uniform: one specialised copy of the loop each, chosen once
     auto epilogue = [&](auto is_f16, auto scaled) {
 #pragma unroll
-      for (int i = 0; i < C::kTm; ++i) {
+      for (int i = 0; i < kStrips; ++i) {
         __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
         char *strip = strip0 + (i & 1) * kStrip;
-        float rs = 1.0f;
-        if constexpr (scaled.value) rs = p.row_scale[m_wave + i * 32 + wrow];
 #pragma unroll
-        for (int j = 0; j < C::kTn; ++j)
+        for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
+          float rs = 1.0f;
+          if constexpr (scaled.value) rs = p.row_scale[m_wave + i * 32 + bi * KM + wrow];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float v[4];
+          for (int j = 0; j < C::kTn; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-            if constexpr (scaled.value) {
-              const f32x4 cs = *(const f32x4 *)(p.col_scale + n_wave + j * 32 + wcol + 8 * q);
+            for (int q = 0; q < kQuads; ++q) {
+              float v[4];
 #pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
+              for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
+              if constexpr (scaled.value) {
+                const f32x4 cs = *(const f32x4 *)(p.col_scale + n_wave + j * KM + wcol + kQuadStep * q);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
+              }
+              u32x2 w;
+              w[0] = is_f16.value ? pack2_f16_rn(v[0], v[1]) : pack2_bf16_rn(v[0], v[1]);
+              w[1] = is_f16.value ? pack2_f16_rn(v[2], v[3]) : pack2_bf16_rn(v[2], v[3]);
+              *(u32x2 *)(strip + (bi * KM + wrow) * kRowStride + (j * KM + wcol + kQuadStep * q) * 2) = w;
             }
-            u32x2 w;
-            w[0] = is_f16.value ? pack2_f16_rn(v[0], v[1]) : pack2_bf16_rn(v[0], v[1]);
-            w[1] = is_f16.value ? pack2_f16_rn(v[2], v[3]) : pack2_bf16_rn(v[2], v[3]);
-            *(u32x2 *)(strip + wrow * kRowStride + (j * 32 + wcol + 8 * q) * 2) = w;
-          }
+        }
         // LDS executes a wave's instructions in order: the reads below see the writes above
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -650,7 +684,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
     for (int i = 0; i < C::kTm; ++i)
 #pragma unroll
-      for (int j = 0; j < C::kTn; ++j) store_block_generic(p, m0 + wm * C::kWtm + i * 32, n0 + wn * C::kWtn + j * 32, lane, acc[i][j]);
+      for (int j = 0; j < C::kTn; ++j) store_block_generic(p, m0 + wm * C::kWtm + i * KM, n0 + wn * C::kWtn + j * KM, lane, acc[i][j]);
   }
 #ifdef KAPY_TRACE
   if (trace && blockIdx.x == KAPY_TRACE && threadIdx.x == 0) trace[258] = __builtin_readcyclecounter();  // stores issued
@@ -903,13 +937,16 @@ int verify_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_glo
 
 // Compiled configurations of the TN kernel, in order of preference.
 struct TnVariant {
-  int bm, bn, bk, waves, stages;
+  int bm, bn, bk, waves, stages, mfma;  // mfma: rows of the matrix instruction's operand block (16 or 32)
   int (*launch_bf16)(const GemmParams &, hipStream_t);
   int (*launch_f16)(const GemmParams &, hipStream_t);
 };
 #define KAPY_TN(BM, BN, BK, WM, WN, S) \
-  { BM, BN, BK, (WM) * (WN), S, launch_tn<Bf16, BM, BN, BK, WM, WN, S>, launch_tn<F16, BM, BN, BK, WM, WN, S> }
+  { BM, BN, BK, (WM) * (WN), S, 32, launch_tn<Bf16, BM, BN, BK, WM, WN, S>, launch_tn<F16, BM, BN, BK, WM, WN, S> }
+#define KAPY_TN16(BM, BN, BK, WM, WN, S) \
+  { BM, BN, BK, (WM) * (WN), S, 16, launch_tn<Bf16M16, BM, BN, BK, WM, WN, S>, launch_tn<F16M16, BM, BN, BK, WM, WN, S> }
 const TnVariant kTnVariants[] = {
+    KAPY_TN16(256, 256, 64, 2, 2, kRing25), KAPY_TN16(256, 256, 64, 2, 2, 2),
     KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
 #ifdef KAPY_TUNING
     KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2), KAPY_TN(256, 128, 64, 2, 2, 3),
@@ -1001,10 +1038,11 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   bool tn = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 0) == 16 && p.K > 0 &&
             p.a_sm * 2 * 256 < (int64_t(1) << 31) && p.b_sn * 2 * 256 < (int64_t(1) << 31) && p.a_sm >= 0 && p.b_sn >= 0;
   if (tn) {
-    const bool free_choice = !c.tile_m && !c.tile_n && !c.tile_k && !c.stages && !c.waves;
+    const bool free_choice = !c.tile_m && !c.tile_n && !c.tile_k && !c.stages && !c.waves && c.impl_way < KAPY_MFMA_32X32X16_16B;
     for (const TnVariant &v : kTnVariants) {
       if ((c.tile_m && c.tile_m != v.bm) || (c.tile_n && c.tile_n != v.bn) || (c.tile_k && c.tile_k != v.bk) ||
-          (c.stages && c.stages != v.stages) || (c.waves && c.waves != v.waves))
+          (c.stages && c.stages != v.stages) || (c.waves && c.waves != v.waves) ||
+          (c.impl_way == KAPY_MFMA_32X32X16_16B && v.mfma != 32) || (c.impl_way == KAPY_MFMA_16X16X32_16B && v.mfma != 16))
         continue;
       if (p.M % v.bm || p.N % v.bn || p.K % v.bk) continue;
       // with a free choice, a 256x256 tiling that cannot occupy half of the CUs yields to 128x128

@@ -23,7 +23,7 @@ def _np_store(dtype):
 
 
 def _run(ko, dt, M, N, K, a_row_major=True, b_row_major=True, out_dtype=None, with_acc=None, d_col_major=False,
-         seed=0, gen="uniform", rmode=kh.RN, tile=(0, 0, 0), stages=0):
+         seed=0, gen="uniform", rmode=kh.RN, tile=(0, 0, 0), stages=0, impl_way=0):
     out_dtype = dt if out_dtype is None else out_dtype
     fill = (lambda n, s: ko.fill_uniform(n, dt, seed, s)) if gen == "uniform" else (lambda n, s: ko.fill_normal(n, dt, seed, s, 0.0, 0.02))
     a, b = fill(M * K, 0), fill(K * N, 1)
@@ -42,7 +42,7 @@ def _run(ko, dt, M, N, K, a_row_major=True, b_row_major=True, out_dtype=None, wi
                             C.byref(go_acc) if go_acc is not None else None, C.byref(ko.mk_global(want, M, N, *d_str, out_dtype)), rmode)
     assert rc == 0
     kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(dd, M, N, *d_str, out_dtype), acc=gd_acc,
-              rmode=rmode, tile=tile, stages=stages)
+              rmode=rmode, tile=tile, stages=stages, impl_way=impl_way)
     sync()
     return to_host(dd, want.dtype), want
 
@@ -62,19 +62,21 @@ def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):
         assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
 
 
-TN_VARIANTS = [((256, 256, 64), 25), ((256, 256, 64), 2), ((256, 256, 32), 4), ((128, 128, 64), 2), ((128, 128, 32), 4)]
+MFMA16, MFMA32 = 17, 16   # KAPY_MFMA_16X16X32_16B, KAPY_MFMA_32X32X16_16B
+TN_VARIANTS = [((256, 256, 64), 25, MFMA16), ((256, 256, 64), 2, MFMA16), ((256, 256, 64), 25, MFMA32), ((256, 256, 64), 2, MFMA32),
+               ((256, 256, 32), 4, MFMA32), ((128, 128, 64), 2, MFMA32), ((128, 128, 32), 4, MFMA32)]
 
 
-@pytest.mark.parametrize("tile,stages", TN_VARIANTS)
-def test_tn_roofline_kernel_every_variant(ko, tile, stages):
+@pytest.mark.parametrize("tile,stages,impl_way", TN_VARIANTS)
+def test_tn_roofline_kernel_every_variant(ko, tile, stages, impl_way):
     """lhs row-major, rhs column-major, extents multiples of the tile: the LDS-direct kernels, each compiled
     configuration forced through kapy_matmul_cfg, including K of 1, 2, 3 and many tiles (pipeline prologue / tail)."""
     bm, bn, bk = tile
     for dt in (kh.BF16, kh.F16):
         for (M, N, K) in ((bm, bn, bk), (bm, bn, 2 * bk), (bm, 2 * bn, 3 * bk), (2 * bm, bn, 4 * bk), (bm, bn, 7 * bk), (3 * bm, 2 * bn, 16 * bk)):
-            got, want = _run(ko, dt, M, N, K, True, False, seed=5, tile=tile, stages=stages)
+            got, want = _run(ko, dt, M, N, K, True, False, seed=5, tile=tile, stages=stages, impl_way=impl_way)
             assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
-    got32, want32 = _run(ko, kh.BF16, 2 * bm, 2 * bn, 8 * bk, True, False, out_dtype=kh.F32, seed=5, tile=tile, stages=stages)
+    got32, want32 = _run(ko, kh.BF16, 2 * bm, 2 * bn, 8 * bk, True, False, out_dtype=kh.F32, seed=5, tile=tile, stages=stages, impl_way=impl_way)
     assert _frob(ko, got32, want32, kh.F32) <= 1e-5
 
 

@@ -190,6 +190,9 @@ __device__ __forceinline__ void tile_of_block(const GemmParams &p, int32_t &tm, 
 // ---------------------------------------------------------------------------------------------
 // TN kernel.  BM x BN x BK workgroup tile, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN)
 // block of 32x32 accumulators.  STAGES-deep LDS ring filled by LDS-direct loads.
+#ifndef KAPY_ABLATE
+#define KAPY_ABLATE 0  // timing experiments in tuning builds only: 1 no barrier, 2 no load wait, 4 no loads, 8 no LDS reads (results are wrong)
+#endif
 constexpr int kRing25 = 25;  // value of STAGES (and of kapy_matmul_cfg.stages) that selects the 2.5-tile ring
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 struct TnConfig {
@@ -430,9 +433,9 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
         KAPY_STAMP(kt, kk);
         if (kk == KK - 1) {
           // tile kt+1 has landed once only the kHalf youngest loads (lhs of tile kt+2) are in flight
-          __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
+          if (!(KAPY_ABLATE & 2)) __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
           KAPY_STAMP(kt, 4);
-          __builtin_amdgcn_s_barrier();
+          if (!(KAPY_ABLATE & 1)) __builtin_amdgcn_s_barrier();
           KAPY_STAMP(kt, 5);
         }
 #pragma unroll
@@ -443,12 +446,12 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
           for (int t = 0; t < kReadsPerMfma; ++t) {
             const int idx = g * kReadsPerMfma + t;
-            if (idx < kReads) {
+            if (idx < kReads && !(KAPY_ABLATE & 8)) {
               if (kk + 1 < KK) ring_read(a_cur_base, b_cur_base, kk + 1, idx, a_nxt, b_nxt);
               else ring_read(a_nxt_base, b_nxt_base, 0, idx, a_nxt, b_nxt);
             }
           }
-          if (g % kLoadSpacing == 0) {
+          if (g % kLoadSpacing == 0 && !(KAPY_ABLATE & 4)) {
             const int slot = (kk * kMfmas + g) / kLoadSpacing;
             if (kk == KK - 1 && g / kLoadSpacing < kEarly) ring_load(pos, g / kLoadSpacing, soff_early_b, soff_early_a);
             if (kk < KK - 1 && kEarly + slot < kLoadsPerTile && (!first.value || kEarly + slot >= kHalf))

@@ -172,6 +172,77 @@ __device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_
   for (int v = 0; v < 4; ++v) store_result(p, m, n_base + 4 * (lane >> 4) + v, acc[v]);
 }
 
+// Packed epilogue (16-bit row-major result, 16-byte aligned rows, no accumulator input, RN) of one
+// wavefront's WTM x WTN block of KM x KM accumulator blocks, by 32-row strips through a wave-private
+// LDS area: accumulator quads (four consecutive columns of one row per lane) are narrowed and written
+// 8 bytes at a time, read back 16 bytes per lane along rows, and stored so that one instruction
+// writes whole 128-byte lines (64 / kChunks rows x WTN*2 bytes) - the register layout itself would
+// scatter 8-byte pieces over KM rows per instruction.  Row stride WTN*2 + 16 bytes: both the 8-byte
+// writes down the rows and the 16-byte reads along them then use every LDS bank equally.
+// The caller makes sure (barrier) that no other wave still uses the LDS area.
+template <int KM, int WTM, int WTN>
+struct PackedEpilogue {
+  static constexpr int kRowStride = WTN * 2 + 16, kStrip = 32 * kRowStride, kBytesPerWave = 2 * kStrip;
+  static constexpr int kChunks = WTN * 2 / 16, kRowsPerStore = 64 / kChunks, kStores = 32 / kRowsPerStore;
+  static constexpr int kGroups = 64 / KM, kAccRegs = KM * KM / 64;
+  static constexpr int kBlocksPerStrip = 32 / KM, kStrips = WTM / 32, kTn = WTN / KM;
+  static constexpr int kQuads = kAccRegs / 4, kQuadStep = 4 * kGroups;  // register quads of a block: 4 consecutive columns each, kQuadStep apart
+  static_assert(WTM % 32 == 0 && 64 % kChunks == 0 && 32 % kRowsPerStore == 0, "strip geometry");
+
+  template <bool F16, bool SCALED, typename Acc>
+  static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
+    const int wrow = lane % KM, wcol = 4 * (lane / KM);        // this lane's row / first column in an accumulator block
+    const int rrow = lane / kChunks, rchunk = lane % kChunks;  // and in a read-back instruction
+#pragma unroll
+    for (int i = 0; i < kStrips; ++i) {
+      __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
+      char *strip = strip0 + (i & 1) * kStrip;
+#pragma unroll
+      for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
+        float rs = 1.0f;
+        if constexpr (SCALED) rs = p.row_scale[m_wave + i * 32 + bi * KM + wrow];
+#pragma unroll
+        for (int j = 0; j < kTn; ++j)
+#pragma unroll
+          for (int q = 0; q < kQuads; ++q) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
+            if constexpr (SCALED) {
+              const f32x4 cs = *(const f32x4 *)(p.col_scale + n_wave + j * KM + wcol + kQuadStep * q);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
+            }
+            u32x2 w;
+            w[0] = F16 ? pack2_f16_rn(v[0], v[1]) : pack2_bf16_rn(v[0], v[1]);
+            w[1] = F16 ? pack2_f16_rn(v[2], v[3]) : pack2_bf16_rn(v[2], v[3]);
+            *(u32x2 *)(strip + (bi * KM + wrow) * kRowStride + (j * KM + wcol + kQuadStep * q) * 2) = w;
+          }
+      }
+      // LDS executes a wave's instructions in order: the reads below see the writes above
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < kStores; ++t) {
+        const int row = t * kRowsPerStore + rrow;
+        const u32x4 w = *(const u32x4 *)(strip + row * kRowStride + rchunk * 16);
+        *(u32x4 *)(p.d + ((int64_t)(m_wave + i * 32 + row) * p.d_sm + n_wave + rchunk * 8) * 2) = w;
+      }
+    }
+  }
+  // result type and scaling are uniform: one specialised copy of the loop each, chosen once
+  template <typename Acc>
+  static __device__ __forceinline__ void run(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
+    const bool f16 = p.d_dtype == KAPY_F16;
+    if (p.row_scale) {
+      if (f16) strips<true, true>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<false, true>(p, acc, strip0, m_wave, n_wave, lane);
+    } else {
+      if (f16) strips<true, false>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<false, false>(p, acc, strip0, m_wave, n_wave, lane);
+    }
+  }
+};
+
 // Workgroup id -> output tile.  Consecutive workgroup ids land on different XCDs (8 of them, each
 // with its own L2), so ids are first regrouped per XCD, then each XCD walks a compact band of
 // tiles GROUP_M tall so that the operand panels it streams stay in its L2.
@@ -619,70 +690,11 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   }
 #endif
   if constexpr (PACKED) {
-    // Packed epilogue (16-bit row-major result, 16-byte aligned rows, no accumulator input, RN), by
-    // 32-row strips of the wave's block through a wave-private LDS strip: accumulator quads (four
-    // consecutive columns of one row per lane) are narrowed and written 8 bytes at a time, read back
-    // 16 bytes per lane along rows, and stored so that one instruction writes whole 128-byte lines
-    // (64 / kChunks rows x kWtn*2 bytes) - the register layout itself would scatter 8-byte pieces
-    // over 32 rows per instruction.  Row stride kWtn*2 + 16 bytes: both the 8-byte writes down the
-    // rows and the 16-byte reads along them then use every LDS bank equally.
-    constexpr int kRowStride = C::kWtn * 2 + 16, kStrip = 32 * kRowStride;
-    constexpr int kChunks = C::kWtn * 2 / 16, kRowsPerStore = 64 / kChunks, kStores = 32 / kRowsPerStore;
-    static_assert(2 * kStrip * C::kWaves <= C::kLdsBytes, "two strips per wavefront must fit the ring");
+    static_assert(PackedEpilogue<KM, C::kWtm, C::kWtn>::kBytesPerWave * C::kWaves <= C::kLdsBytes, "two strips per wavefront must fit the ring");
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
     __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space
-    char *strip0 = lds + wave * 2 * kStrip;
-    const int wrow = lane % KM, wcol = 4 * (lane / KM);           // this lane's row / first column in an accumulator block
-    const int rrow = lane / kChunks, rchunk = lane % kChunks;     // and in a read-back instruction
-    const int32_t m_wave = m0 + wm * C::kWtm, n_wave = n0 + wn * C::kWtn;
-    constexpr int kBlocksPerStrip = 32 / KM, kStrips = C::kWtm / 32;
-    constexpr int kQuads = kAccRegs / 4, kQuadStep = 4 * kGroups;  // register quads of a block: 4 consecutive columns each, kQuadStep apart
-    // result type and scaling are uniform: one specialised copy of the loop each, chosen once
-    auto epilogue = [&](auto is_f16, auto scaled) {
-#pragma unroll
-      for (int i = 0; i < kStrips; ++i) {
-        __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
-        char *strip = strip0 + (i & 1) * kStrip;
-#pragma unroll
-        for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
-          float rs = 1.0f;
-          if constexpr (scaled.value) rs = p.row_scale[m_wave + i * 32 + bi * KM + wrow];
-#pragma unroll
-          for (int j = 0; j < C::kTn; ++j)
-#pragma unroll
-            for (int q = 0; q < kQuads; ++q) {
-              float v[4];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
-              if constexpr (scaled.value) {
-                const f32x4 cs = *(const f32x4 *)(p.col_scale + n_wave + j * KM + wcol + kQuadStep * q);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
-              }
-              u32x2 w;
-              w[0] = is_f16.value ? pack2_f16_rn(v[0], v[1]) : pack2_bf16_rn(v[0], v[1]);
-              w[1] = is_f16.value ? pack2_f16_rn(v[2], v[3]) : pack2_bf16_rn(v[2], v[3]);
-              *(u32x2 *)(strip + (bi * KM + wrow) * kRowStride + (j * KM + wcol + kQuadStep * q) * 2) = w;
-            }
-        }
-        // LDS executes a wave's instructions in order: the reads below see the writes above
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < kStores; ++t) {
-          const int row = t * kRowsPerStore + rrow;
-          const u32x4 w = *(const u32x4 *)(strip + row * kRowStride + rchunk * 16);
-          *(u32x4 *)(p.d + ((int64_t)(m_wave + i * 32 + row) * p.d_sm + n_wave + rchunk * 8) * 2) = w;
-        }
-      }
-    };
-    const bool f16 = p.d_dtype == KAPY_F16;
-    if (p.row_scale) {
-      if (f16) epilogue(Yes{}, Yes{});
-      else epilogue(No{}, Yes{});
-    } else {
-      if (f16) epilogue(Yes{}, No{});
-      else epilogue(No{}, No{});
-    }
+    PackedEpilogue<KM, C::kWtm, C::kWtn>::run(p, acc, lds + wave * PackedEpilogue<KM, C::kWtm, C::kWtn>::kBytesPerWave, m0 + wm * C::kWtm,
+                                              n0 + wn * C::kWtn, lane);
   } else {
 #pragma unroll
     for (int i = 0; i < C::kTm; ++i)
@@ -699,6 +711,168 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     w[3] = __builtin_amdgcn_s_getreg(20 | (31 << 11));   // XCC_ID
   }
 #endif
+}
+
+// ---------------------------------------------------------------------------------------------
+// NN kernel: lhs row-major (K contiguous), rhs row-major (N contiguous), extents multiples of the
+// 128 x 128 x BK tile.  4 wavefronts (2x2), wave tile 64x64 = 4x4 blocks of the 16x16x32 instruction.
+// The rhs tile is staged as it lies in memory, [BK][128] with N contiguous, by the same LDS-direct
+// buffer loads as the lhs; the K-contiguous operand registers the matrix instruction wants are made
+// on the way out of LDS by ds_read_b64_tr_b16: a 16-lane group hands in 16 addresses of 8 bytes
+// (4 k-rows x 16 columns) and lane i gets column i of the four rows.  This replaces the
+// ldmatrix.trans of the reference (LdMatrixOpToLLVM.cpp:128-129).
+// STAGES-deep ring; the barrier at the top of iteration kt publishes tile kt+1 and frees the stage of
+// tile kt-1 for the loads of tile kt+STAGES-1.  Loads past the end of K re-read the last tile into
+// a stage nobody reads again, so every iteration is identical.
+constexpr int kNBM = 128, kNBN = 128;
+// rhs image: 16-byte chunk c of k-row r sits at chunk c ^ rhs_key(r).  A transposing read of a half
+// wave touches rows {0..3} + 8*{0,1} (+4) of a 32-row slice, 32 bytes of each: the key sends those
+// eight to the eight 32-byte bank groups of the 256-byte row.
+__device__ __forceinline__ uint32_t rhs_key(uint32_t row) { return ((row & 3) + 4 * ((row >> 3) & 1)) * 2; }
+
+template <typename T, int BK, int STAGES, bool PACKED>
+__global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
+  static_assert(T::kM == 16 && T::kBytes == 2 && BK % 32 == 0 && STAGES >= 3, "16x16x32 instruction, 16-bit operands");
+  using LA = TileLayout<BK * 2>;
+  constexpr int kRowA = BK * 2, kRowB = kNBN * 2;
+  constexpr int kBytesA = kNBM * kRowA, kBytesB = BK * kRowB, kStage = kBytesA + kBytesB;
+  constexpr int kLoadsA = kBytesA / 1024 / 4, kLoadsB = kBytesB / 1024 / 4, kLoads = kLoadsA + kLoadsB;  // per wavefront per tile
+  constexpr int KK = BK / 32, kTm = 4, kTn = 4, kMfmas = kTm * kTn;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  int32_t tm, tn;
+  tile_of_block(p, tm, tn);
+  const int32_t m0 = tm * kNBM, n0 = tn * kNBN;
+  const int32_t ldb = (int32_t)p.b_sk;  // elements between consecutive k-rows of the rhs
+  const int KT = p.K / BK;
+
+  uint32_t a_goff[kLoadsA], b_goff[kLoadsB];
+#pragma unroll
+  for (int i = 0; i < kLoadsA; ++i) {
+    uint32_t row, chunk;
+    LA::locate((uint32_t)(wave + i * 4) * 1024u + lane * 16u, row, chunk);
+    a_goff[i] = (uint32_t)((row * p.a_sm + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < kLoadsB; ++i) {
+    const uint32_t o = (uint32_t)(wave + i * 4) * 1024u + lane * 16u, row = o / kRowB, chunk = ((o % kRowB) / 16) ^ rhs_key(row);
+    b_goff[i] = (uint32_t)((row * ldb + chunk * 8) * 2);
+  }
+  auto uniform_ptr = [](const char *ptr) {
+    const uint64_t v = (uint64_t)ptr;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (void *)(((uint64_t)hi << 32) | lo);
+  };
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm * 2), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * 2), 0, 0x7fffffff, 0x00020000);
+  const int wave_lds = wave * 1024;
+  // load `idx` (lhs first, then rhs) of K-tile j into its stage
+  auto issue_load = [&](int j, int stage, int idx) {
+    const int jc = min(j, KT - 1);
+    if (idx < kLoadsA)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + idx * 4096 + wave_lds), 16,
+                                               (int)a_goff[idx], jc * (BK * 2), 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + kBytesA + (idx - kLoadsA) * 4096 + wave_lds),
+                                               16, (int)b_goff[idx - kLoadsA], jc * BK * ldb * 2, 0, 0);
+  };
+
+  // Operand reads.  lhs: row (lane % 16) of each 16-row block, 16-byte chunk 4*kk + lane/16.
+  // rhs: k-rows kk*32 + 8*(lane/16) + 4*h + (lane%16)/4, columns 4*((lane%16)%4).. of each 16-column block.
+  const uint32_t grp = lane >> 4, l16 = lane & 15;
+  uint32_t a_off[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) a_off[kk] = LA::offset(wm * 64 + l16, 4 * kk + grp);
+  static_assert((16 * kRowA) % (256 * LA::kLineParam) == 0, "an operand block must span whole swizzle periods");
+  const uint32_t b_row = 8 * grp + (l16 >> 2), b_key = rhs_key(b_row);  // the key is the same for every kk and h
+  uint32_t b_off[kTn];
+#pragma unroll
+  for (int j = 0; j < kTn; ++j) b_off[j] = kBytesA + b_row * kRowB + (((wn * 8 + j * 2 + ((l16 & 3) >> 1)) ^ b_key) * 16) + (l16 & 1) * 8;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  struct Frag {
+    u32x4 c[1];
+  };
+  auto read_a = [&](int stage, int kk, int i) { return *(const u32x4 *)(lds + stage * kStage + a_off[kk] + i * 16 * kRowA); };
+  auto read_b = [&](int stage, int kk, int j) {
+    const char *base = lds + stage * kStage + b_off[j] + kk * 32 * kRowB;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)base);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(base + 4 * kRowB));
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    return u32x4{l2[0], l2[1], h2[0], h2[1]};
+  };
+
+  using Acc = typename T::Acc;
+  Acc acc[kTm][kTn];
+#pragma unroll
+  for (int i = 0; i < kTm; ++i)
+#pragma unroll
+    for (int j = 0; j < kTn; ++j) acc[i][j] = Acc{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int j = 0; j < STAGES - 1; ++j)
+#pragma unroll
+    for (int idx = 0; idx < kLoads; ++idx) issue_load(j, j, idx);
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (STAGES - 2)));
+  __builtin_amdgcn_s_barrier();  // tile 0 published
+  Frag af[2][kTm], bf[2][kTn];
+#pragma unroll
+  for (int i = 0; i < kTm; ++i) af[0][i].c[0] = read_a(0, 0, i);
+#pragma unroll
+  for (int j = 0; j < kTn; ++j) bf[0][j].c[0] = read_b(0, 0, j);
+
+  constexpr int kReads = kTm + kTn;
+  constexpr int kLoadSpacing = (KK * kMfmas) / kLoads;  // matrix instructions between two loads
+  static_assert(kLoadSpacing >= 1, "");
+  int stage = 0;
+  // One K-tile.  `parity` says which fragment buffer holds slice 0 of this tile: with an odd number
+  // of slices per tile it alternates from tile to tile (compile-time, the loop is unrolled by two).
+  auto tile_step = [&](int kt, auto parity) {
+    const int next_stage = stage + 1 == STAGES ? 0 : stage + 1, free_stage = stage == 0 ? STAGES - 1 : stage - 1;
+    // own loads of tile kt+1 have landed once only the younger tiles' loads remain in flight
+    __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kLoads * (STAGES - 3)));
+    __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      constexpr int par = decltype(parity)::value;
+      Frag *a_cur = af[(kk + par) & 1], *b_cur = bf[(kk + par) & 1], *a_nxt = af[(kk + par + 1) & 1], *b_nxt = bf[(kk + par + 1) & 1];
+#pragma unroll
+      for (int g = 0; g < kMfmas; ++g) {
+        const int i = g / kTn, j = g % kTn;
+        acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g < kReads) {
+          const int rs = kk + 1 < KK ? stage : next_stage, rk = kk + 1 < KK ? kk + 1 : 0;
+          if (g < kTm) a_nxt[g].c[0] = read_a(rs, rk, g);
+          else b_nxt[g - kTm].c[0] = read_b(rs, rk, g - kTm);
+        }
+        if ((kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads)
+          issue_load(kt + STAGES - 1, free_stage, (kk * kMfmas + g) / kLoadSpacing);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    stage = next_stage;
+  };
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, KK & 1>;
+  int kt = 0;
+  for (; kt + 2 <= KT; kt += 2) {
+    tile_step(kt, P0{});
+    tile_step(kt + 1, P1{});
+  }
+  if (kt < KT) tile_step(kt, P0{});
+  __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+  __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space by the packed epilogue
+  if constexpr (PACKED) {
+    static_assert(PackedEpilogue<16, 64, 64>::kBytesPerWave * 4 <= STAGES * kStage, "two strips per wavefront must fit the ring");
+    PackedEpilogue<16, 64, 64>::run(p, acc, lds + wave * PackedEpilogue<16, 64, 64>::kBytesPerWave, m0 + wm * 64, n0 + wn * 64, lane);
+  } else {
+#pragma unroll
+    for (int i = 0; i < kTm; ++i)
+#pragma unroll
+      for (int j = 0; j < kTn; ++j) store_block_generic(p, m0 + wm * 64 + i * 16, n0 + wn * 64 + j * 16, lane, acc[i][j]);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -886,6 +1060,32 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
                             : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
 }
 
+template <typename T, int BK, int STAGES>
+int launch_nn(GemmParams p, hipStream_t s) {
+  constexpr int kLds = STAGES * BK * 512;
+  p.tiles_m = p.M / kNBM;
+  p.tiles_n = p.N / kNBN;
+  const bool packed = packed_epilogue(p);
+  const void *kernel = packed ? (const void *)nn_kernel<T, BK, STAGES, true> : (const void *)nn_kernel<T, BK, STAGES, false>;
+  static bool configured[2] = {false, false};  // idempotent; a race only repeats the calls
+  if (!configured[packed]) {
+    hipFuncAttributes fa;
+    KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, kernel));
+    if (fa.maxDynamicSharedSizeBytes < kLds) {
+      KAPY_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+      KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, kernel));
+      if (fa.maxDynamicSharedSizeBytes < kLds)
+        return fail(KAPY_ERR_HIP, "matmul: could not raise the dynamic LDS limit to %d bytes (runtime reports %d)", kLds, (int)fa.maxDynamicSharedSizeBytes);
+    }
+    configured[packed] = true;
+  }
+  dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  if (packed) nn_kernel<T, BK, STAGES, true><<<grid, dim3(256), kLds, s>>>(p);
+  else nn_kernel<T, BK, STAGES, false><<<grid, dim3(256), kLds, s>>>(p);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 template <typename T>
 int launch_staged(GemmParams p, int a_mode, int b_mode, hipStream_t s) {
   p.tiles_m = (p.M + kSBM - 1) / kSBM;
@@ -1051,6 +1251,23 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
       // with a free choice, a 256x256 tiling that cannot occupy half of the CUs yields to 128x128
       if (free_choice && v.bm == 256 && (int64_t)(p.M / v.bm) * (p.N / v.bn) * 2 < device_cus() && p.M % 128 == 0 && p.N % 128 == 0)
         continue;
+      return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
+    }
+  }
+  // Both operands row-major (the reference fixture's layout, matmul.mlir): the transposing-read kernel.
+  bool nn = p.a_sk == 1 && p.b_sn == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 1) == 16 && p.M % kNBM == 0 && p.N % kNBN == 0 &&
+            p.K > 0 && p.a_sm >= 0 && p.b_sk >= 0 && p.a_sm * 2 * kNBM < (int64_t(1) << 31) && (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31) &&
+            c.impl_way != KAPY_MFMA_32X32X16_16B && (!c.tile_m || c.tile_m == kNBM) && (!c.tile_n || c.tile_n == kNBN) && (!c.waves || c.waves == 4);
+  if (nn) {
+    struct NnVariant {
+      int bk, stages;
+      int (*launch_bf16)(GemmParams, hipStream_t);
+      int (*launch_f16)(GemmParams, hipStream_t);
+    };
+    static const NnVariant kNn[] = {{64, 4, launch_nn<Bf16M16, 64, 4>, launch_nn<F16M16, 64, 4>}, {64, 3, launch_nn<Bf16M16, 64, 3>, launch_nn<F16M16, 64, 3>},
+                                    {32, 4, launch_nn<Bf16M16, 32, 4>, launch_nn<F16M16, 32, 4>}};
+    for (const NnVariant &v : kNn) {
+      if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }

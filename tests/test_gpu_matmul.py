@@ -54,6 +54,24 @@ def test_config1_fp16_1024_row_major_128x128x32_tiles(ko):
     assert (got != want).mean() < 0.05    # fp32 vs fp64 accumulation flips few roundings
 
 
+@pytest.mark.parametrize("tile_k,stages", [(64, 4), (64, 3), (32, 4)])
+def test_nn_transposing_read_kernel_every_variant(ko, tile_k, stages):
+    """Both operands row-major, extents multiples of 128 x 128 x tile_k: the kernel that stages the rhs as it lies in
+    memory and transposes on the way out of LDS; K of 1, 2, 3, 7 and 16 tiles (prologue, ring wrap, fragment parity)."""
+    for dt in (kh.BF16, kh.F16):
+        for (M, N, K) in ((128, 128, tile_k), (128, 256, 2 * tile_k), (256, 128, 3 * tile_k), (128, 128, 7 * tile_k), (384, 256, 16 * tile_k)):
+            got, want = _run(ko, dt, M, N, K, True, True, seed=7, tile=(128, 128, tile_k), stages=stages)
+            assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
+    got32, want32 = _run(ko, kh.F16, 256, 256, 8 * tile_k, True, True, out_dtype=kh.F32, with_acc=kh.F32, seed=7, tile=(128, 128, tile_k), stages=stages)
+    assert _frob(ko, got32, want32, kh.F32) <= 1e-5
+
+
+def test_general_kernel_when_asked_for_one_stage(ko):
+    """stages=1 selects the register-staged general kernel also for shapes the faster kernels would take."""
+    got, want = _run(ko, kh.F16, 256, 256, 128, True, True, seed=9, tile=(128, 128, 32), stages=1)
+    assert _frob(ko, got, want, kh.F16) <= FROB_TOL
+
+
 @pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
 @pytest.mark.parametrize("a_rm,b_rm", [(True, True), (True, False), (False, True), (False, False)])
 def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):

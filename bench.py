@@ -129,7 +129,7 @@ def bench_permute(kh, steps, warmup):
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
 
 
-def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel):
+def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0)):
     import torch
     tdt = torch.bfloat16 if dtype == kh.BF16 else torch.float16
     std = 0.02 if dtype == kh.BF16 else 0.5
@@ -139,7 +139,7 @@ def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel):
     ga = kh.mk_global(a.data_ptr(), M, K, K, 1, dtype)
     gb = kh.mk_global(b.data_ptr(), K, N, 1, K, dtype) if b_col_major else kh.mk_global(b.data_ptr(), K, N, N, 1, dtype)
     gd = kh.mk_global(d.data_ptr(), M, N, N, 1, dtype)
-    wall, ev = _events(lambda i: kh.matmul(ga, gb, gd), steps, warmup)
+    wall, ev = _events(lambda i: kh.matmul(ga, gb, gd, tile=tile), steps, warmup)
     flops = 2.0 * M * N * K
     kind = "bf16" if dtype == kh.BF16 else "f16"
     return {"workload": name, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "kernel_ms": ev,
@@ -215,7 +215,7 @@ def main():
         "transpose": lambda s, w: bench_transpose(kh, s, w),
         "permute": lambda s, w: bench_permute(kh, s, w),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
-        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "staged_kernel"),
+        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32)),
         "f8_m16": lambda s, w: bench_f8(kh, s, w, 16),
         "f8_m4096": lambda s, w: bench_f8(kh, s, w, 4096),
     }

@@ -1266,8 +1266,11 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
     };
     static const NnVariant kNn[] = {{64, 4, launch_nn<Bf16M16, 64, 4>, launch_nn<F16M16, 64, 4>}, {64, 3, launch_nn<Bf16M16, 64, 3>, launch_nn<F16M16, 64, 3>},
                                     {32, 4, launch_nn<Bf16M16, 32, 4>, launch_nn<F16M16, 32, 4>}};
+    // more workgroups than CUs: the 64 KiB ring of the K=32 tile lets two workgroups share a CU, which
+    // hides more latency than the deeper K=64 tile does with one
+    const bool prefer_k32 = !c.tile_k && !c.stages && (int64_t)(p.M / kNBM) * (p.N / kNBN) > device_cus() && p.K % 32 == 0;
     for (const NnVariant &v : kNn) {
-      if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;
+      if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk || (prefer_k32 && v.bk != 32)) continue;
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }

@@ -102,6 +102,20 @@ def bench_copy(kh, steps, warmup):
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
 
 
+def bench_reduce(kh, steps, warmup):
+    """kapy.reduce (sum along rows) of the headline shape: the first adjacent op after the hot path proper."""
+    import torch
+    n, sets = 8192, 4
+    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    y = torch.empty(n, device="cuda", dtype=torch.float32)
+    gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
+    gy = kh.mk_global(y.data_ptr(), n, 1, 1, n, kh.F32)
+    wall, ev = _events(lambda i: kh.reduce(gx[i % sets], gy, 1, 0), steps, warmup)
+    nbytes = n * n * 2 + n * 4
+    return {"workload": "reduce_sum axis=1 fp16 8192x8192 -> f32 [8192x1]", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "reduce_rows_vec_kernel"}
+
+
 def bench_transpose(kh, steps, warmup):
     import torch
     n, sets = 8192, 4
@@ -162,7 +176,7 @@ def bench_f8(kh, steps, warmup, M):
     flops = 2.0 * M * N * K
     nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
     out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192" % M, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_kernel" if M <= 64 else "tn_kernel<F8>"}
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 64 else "tn_kernel<F8>"}
     out["roofline"] = _roof_hbm(nbytes, ev) if M <= 64 else _roof_mfma(flops, ev, "f8")
     return out
 
@@ -197,7 +211,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "copy", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "copy", "reduce", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -213,6 +227,7 @@ def main():
         "gelu": lambda s, w: bench_gelu(kh, s, w),
         "copy": lambda s, w: bench_copy(kh, s, w),
         "transpose": lambda s, w: bench_transpose(kh, s, w),
+        "reduce": lambda s, w: bench_reduce(kh, s, w),
         "permute": lambda s, w: bench_permute(kh, s, w),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32)),

@@ -7,7 +7,9 @@
 // gfx950: v_mfma_scale_f32_16x16x128_f8f6f4 with unit E8M0 block scales (2^0); the operand format
 // selectors (cbsz / blgp: 0 = E4M3, 1 = E5M2) carry kapy's mixed-f8 rule.
 //
-//   skinny_kernel  few rows of lhs (decode shape): HBM-bound on the weight.  One workgroup per 16*NG
+//   skinny_stream_kernel  few rows of lhs (decode shape), K a multiple of 1024: HBM-bound on the weight;
+//                  row-contiguous LDS-direct loads into per-wave rings, regrouped into operands by LDS reads.
+//   skinny_kernel  the same shape for other K (multiples of 128).  One workgroup per 16*NG
 //                  output columns, its 8 wavefronts split K; every weight byte is read once,
 //                  straight from global memory into the MFMA operand registers (each lane's 32
 //                  K-contiguous bytes are exactly its operand), partial sums meet in LDS.
@@ -80,6 +82,9 @@ __device__ __forceinline__ i32x8 load_k32(const uint8_t *base, int64_t stride, i
 #ifndef KAPY_SKINNY_CH
 #define KAPY_SKINNY_CH 8
 #endif
+#ifndef KAPY_SKINNY_OLD
+#define KAPY_SKINNY_OLD 0
+#endif
 constexpr int kSkinnyWaves = 8;
 template <int A_FMT, int B_FMT, int NG, int CH>
 __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
@@ -123,6 +128,96 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
   }
 }
 
+// Streaming skinny kernel (K a multiple of 1024).  Workgroup = 4 wavefronts = 4 contiguous K ranges of
+// one 16-column group; every wave works alone (no barrier until the final sum).  What decides the rate
+// of this HBM-bound shape is the shape of the load instructions: the operand layout of the matrix
+// instruction (lane = row % 16, 32 K-bytes per lane) asked for directly makes every load touch 16 rows
+// in 16-byte pieces, and the texture path takes about twice as long over it as over contiguous runs.
+// So the bytes come in as LDS-direct loads of 4 rows x 256 contiguous bytes and are regrouped on the
+// way out of LDS: a wave keeps a private ring of two 8 KiB stages (weight 4 KiB + activation 4 KiB,
+// 256 K-bytes of 16 rows each), 16-byte chunk c of row r stored at chunk c ^ r of the row's 256 bytes
+// so that the 16 rows a quarter-wave reads fall into 16 different bank groups.
+// Rows past M / N are clamped to the last valid row (never stored), so nothing is read out of range.
+constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
+template <int A_FMT, int B_FMT>
+__global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Params p) {
+  __shared__ __attribute__((aligned(1024))) char ring[kStreamWaves * kStreamStages * kStreamStage];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int32_t n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+  const int32_t k_per_wave = p.K / kStreamWaves, chunks = k_per_wave / kStreamChunk;
+  auto uniform_ptr = [](const uint8_t *ptr) {
+    const uint64_t v = (uint64_t)ptr;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (void *)(((uint64_t)hi << 32) | lo);
+  };
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * p.b_sn + (int64_t)wave * k_per_wave), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm + (int64_t)wave * k_per_wave), 0, 0x7fffffff, 0x00020000);
+  // load instruction i (0..3) of an operand: rows 4i .. 4i+3, this lane row 4i + lane/16, stored chunk lane%16
+  uint32_t w_off[4], a_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * i + (lane >> 4), c = (lane & 15) ^ r;
+    w_off[i] = (uint32_t)(min(r, p.N - 1 - n0) * p.b_sn + c * 16);
+    a_off[i] = (uint32_t)(min(r, p.M - 1 - m0) * p.a_sm + c * 16);
+  }
+  char *my_ring = ring + wave * (kStreamStages * kStreamStage);
+  auto issue_chunk = [&](int chunk, int stage) {
+    char *dst = my_ring + stage * kStreamStage;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, (int)w_off[i], chunk * kStreamChunk, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + 4096 + i * 1024), 16, (int)a_off[i], chunk * kStreamChunk, 0, 0);
+  };
+  // operand reads: row lane%16, K-group lane/16 of a 128-byte step: chunks 8*step + 2*group, +1
+  const int r16 = lane & 15, grp = lane >> 4;
+  uint32_t rd[2][2];
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) rd[st][h] = (uint32_t)(r16 * kStreamChunk + (((8 * st + 2 * grp + h) ^ r16) * 16));
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  issue_chunk(0, 0);
+  if (chunks > 1) issue_chunk(1, 1);
+  for (int32_t c = 0; c < chunks; ++c) {
+    const int stage = c & 1;
+    if (c + 1 < chunks) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);  // vmcnt(8): this chunk has landed, the next may be in flight
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
+    const char *src = my_ring + stage * kStreamStage;
+    i32x4 w[2][2], a[2][2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        w[st][h] = *(const i32x4 *)(src + rd[st][h]);
+        a[st][h] = *(const i32x4 *)(src + 4096 + rd[st][h]);
+      }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the stage has been read, it may be refilled
+    if (c + 2 < chunks) issue_chunk(c + 2, stage);
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const i32x8 av = {a[st][0][0], a[st][0][1], a[st][0][2], a[st][0][3], a[st][1][0], a[st][1][1], a[st][1][2], a[st][1][3]};
+      const i32x8 wv = {w[st][0][0], w[st][0][1], w[st][0][2], w[st][0][3], w[st][1][0], w[st][1][1], w[st][1][2], w[st][1][3]};
+      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, wv, acc, A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    }
+  }
+  // accumulator register v of lane l: row 4*(l/16) + v, column l%16; the four K ranges meet in LDS
+  __syncthreads();  // every wave is done with its ring
+  float *partial = (float *)ring;  // [wave][16][17]
+#pragma unroll
+  for (int v = 0; v < 4; ++v) partial[(wave * 16 + 4 * (lane >> 4) + v) * 17 + (lane & 15)] = acc[v];
+  __syncthreads();
+  {
+    const int m = threadIdx.x >> 4, n = threadIdx.x & 15;
+    float sum = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < kStreamWaves; ++w2) sum += partial[(w2 * 16 + m) * 17 + n];
+    finish(p, m0 + m, n0 + n, sum);
+  }
+}
+
 int fmt_of(int dtype) { return dtype == KAPY_F8E5M2 ? 1 : 0; }
 
 }  // namespace
@@ -158,6 +253,19 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     g.acc_dtype = -1; g.d_dtype = p.d_dtype; g.rz = p.rz; g.tiles_m = g.tiles_n = 0;
     int rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
+  }
+  if (k_contig && p.K % (kStreamWaves * kStreamChunk) == 0 && (p.M + 15) / 16 <= 65535 && p.a_sm * 16 < (int64_t(1) << 31) &&
+      p.b_sn * 16 < (int64_t(1) << 31) && !KAPY_SKINNY_OLD) {
+    // rows are addressed from the workgroup's first row, so the per-lane offsets stay small
+    F8Params q = p;
+    dim3 grid((unsigned)((p.N + 15) / 16), (unsigned)((p.M + 15) / 16));
+    int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
+    if (fa == 0 && fb == 0) skinny_stream_kernel<0, 0><<<grid, 64 * kStreamWaves, 0, s>>>(q);
+    else if (fa == 0) skinny_stream_kernel<0, 1><<<grid, 64 * kStreamWaves, 0, s>>>(q);
+    else if (fb == 0) skinny_stream_kernel<1, 0><<<grid, 64 * kStreamWaves, 0, s>>>(q);
+    else skinny_stream_kernel<1, 1><<<grid, 64 * kStreamWaves, 0, s>>>(q);
+    KAPY_HIP_CHECK(hipGetLastError());
+    return KAPY_OK;
   }
   if (k_contig) {
     constexpr int NG = KAPY_SKINNY_NG, CH = KAPY_SKINNY_CH;

@@ -60,6 +60,89 @@ __global__ __launch_bounds__(256) void reduce_wave_kernel(ReduceParams p) {
   if (lane == 0) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
 }
 
+// 16-bit elements, reduced axis contiguous, 16-byte aligned rows, n_red a multiple of 8: one wavefront
+// per kept index, 128-bit non-temporal loads (a wave reads 1 KiB of the row per instruction, four in
+// flight), the 8 values of a load combined in the lane first (the in-lane tree over loop ivs of
+// ReduceOpToLLVM.cpp:76-101), then the six butterfly rounds (:104-119).
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+template <bool BF16>
+__device__ __forceinline__ void widen8(u32x4_t v, float f[8]) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t word = v[w];
+    if (BF16) {
+      f[2 * w] = bits_f32(word << 16);
+      f[2 * w + 1] = bits_f32(word & 0xFFFF0000u);
+    } else {
+      f[2 * w] = f16_to_f32((uint16_t)word);
+      f[2 * w + 1] = f16_to_f32((uint16_t)(word >> 16));
+    }
+  }
+}
+template <bool BF16, int KIND>
+__global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (keep >= p.n_keep) return;
+  const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * 2);
+  const int32_t vecs = p.n_red / 8;
+  float acc = KIND == 0 ? 0.f : -__builtin_inff();
+  constexpr int U = 4;
+  int32_t v = lane;
+  for (; v + 64 * (U - 1) < vecs; v += 64 * U) {
+    u32x4_t x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(row + v + 64 * u);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float f[8];
+      widen8<BF16>(x[u], f);
+      const float t = combine(combine(combine(f[0], f[1], KIND), combine(f[2], f[3], KIND), KIND),
+                              combine(combine(f[4], f[5], KIND), combine(f[6], f[7], KIND), KIND), KIND);
+      acc = combine(acc, t, KIND);
+    }
+  }
+  for (; v < vecs; v += 64) {
+    float f[8];
+    widen8<BF16>(__builtin_nontemporal_load(row + v), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = combine(acc, f[e], KIND);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(acc)));
+    acc = combine(acc, other, KIND);
+  }
+  if (lane == 0) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
+}
+
+// 16-bit elements, kept axis contiguous: a workgroup of 512 lanes owns 32 kept indices (4 lanes x 8
+// consecutive elements, one 128-bit load each) and splits the reduced axis 128 ways; partial results
+// meet in LDS.
+template <bool BF16, int KIND>
+__global__ __launch_bounds__(512) void reduce_cols_vec_kernel(ReduceParams p) {
+  __shared__ float part[128][32 + 1];
+  const int cl = threadIdx.x & 3, rg = threadIdx.x >> 2;
+  const int64_t keep0 = (int64_t)blockIdx.x * 32 + cl * 8;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = KIND == 0 ? 0.f : -__builtin_inff();
+  for (int32_t r = rg; r < p.n_red; r += 128) {
+    float f[8];
+    widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(p.src + (r * p.s_red + keep0) * 2)), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = combine(acc[e], f[e], KIND);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) part[rg][cl * 8 + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < 32) {
+    float t = KIND == 0 ? 0.f : -__builtin_inff();
+    for (int g = 0; g < 128; ++g) t = combine(t, part[g][threadIdx.x], KIND);
+    store_from_f32(p.dst, p.dst_dtype, ((int64_t)blockIdx.x * 32 + threadIdx.x) * p.d_keep, t);
+  }
+}
+
 // One lane per kept index: used when the kept axis is the contiguous one (coalesced as is).
 __global__ __launch_bounds__(256) void reduce_lane_kernel(ReduceParams p) {
   const int64_t keep = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -132,7 +215,17 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
   p.kind = kind;
   if (p.n_keep == 0) return KAPY_OK;
   hipStream_t s = (hipStream_t)stream;
-  if (p.s_keep == 1 && p.s_red != 1) reduce_lane_kernel<<<(p.n_keep + 255) / 256, 256, 0, s>>>(p);
+  const bool b16 = src->dtype == KAPY_F16 || src->dtype == KAPY_BF16, bf = src->dtype == KAPY_BF16;
+  const bool aligned = ((uintptr_t)p.src & 15) == 0;
+  if (b16 && aligned && p.s_red == 1 && p.n_red % 8 == 0 && (p.s_keep * 2) % 16 == 0 && p.n_red >= 512) {
+    dim3 grid((unsigned)((p.n_keep + 3) / 4));
+    if (bf) { if (kind == 0) reduce_rows_vec_kernel<true, 0><<<grid, 256, 0, s>>>(p); else reduce_rows_vec_kernel<true, 1><<<grid, 256, 0, s>>>(p); }
+    else { if (kind == 0) reduce_rows_vec_kernel<false, 0><<<grid, 256, 0, s>>>(p); else reduce_rows_vec_kernel<false, 1><<<grid, 256, 0, s>>>(p); }
+  } else if (b16 && aligned && p.s_keep == 1 && p.n_keep % 32 == 0 && (p.s_red * 2) % 16 == 0 && p.n_red >= 128) {
+    dim3 grid((unsigned)(p.n_keep / 32));
+    if (bf) { if (kind == 0) reduce_cols_vec_kernel<true, 0><<<grid, 512, 0, s>>>(p); else reduce_cols_vec_kernel<true, 1><<<grid, 512, 0, s>>>(p); }
+    else { if (kind == 0) reduce_cols_vec_kernel<false, 0><<<grid, 512, 0, s>>>(p); else reduce_cols_vec_kernel<false, 1><<<grid, 512, 0, s>>>(p); }
+  } else if (p.s_keep == 1 && p.s_red != 1) reduce_lane_kernel<<<(p.n_keep + 255) / 256, 256, 0, s>>>(p);
   else reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;

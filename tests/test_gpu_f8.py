@@ -28,7 +28,8 @@ def _frob(ko, got, want, dt=kh.BF16):
     return np.linalg.norm(g - w) / np.linalg.norm(w)
 
 
-@pytest.mark.parametrize("M,N,K", [(16, 64, 128), (16, 256, 1024), (5, 48, 256), (33, 100, 384), (64, 64, 512)])
+@pytest.mark.parametrize("M,N,K", [(16, 64, 128), (16, 256, 1024), (5, 48, 256), (33, 100, 384), (64, 64, 512), (5, 40, 2048), (33, 100, 3072),
+                                   (64, 64, 4096), (1, 16, 1024)])
 def test_scaled_f8_small(ko, M, N, K):
     aq, sa, wq, sb = _quantised(ko, M, N, K)
     want = np.zeros((M, N), dtype=np.uint16)

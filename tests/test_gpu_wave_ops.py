@@ -49,7 +49,7 @@ def test_change_matches_oracle(ko, src, dst, shape):
 @pytest.mark.parametrize("dt", [kh.F32, kh.F16, kh.BF16])
 def test_reduce_matches_oracle(ko, dt):
     """reduce_sum.mlir fixture shape (2x256 -> 2x1 column-major) and larger, both axes, sum and max."""
-    for (m, n, axis) in ((2, 256, 1), (64, 1000, 1), (300, 128, 0), (4096, 64, 0)):
+    for (m, n, axis) in ((2, 256, 1), (64, 1000, 1), (300, 128, 0), (4096, 64, 0), (37, 8192, 1), (5, 520, 1), (1000, 96, 0), (130, 50, 0)):
         x = ko.fill_normal(m * n, dt, 3, 0)
         for kind in (0, 1):
             om, on = (m, 1) if axis == 1 else (1, n)

@@ -100,6 +100,10 @@ int kapy_fragments_loops(const kapy_fragments *layout, const int64_t shape[2], i
 /* FragmentsLayoutAttr::getAffineMap(shape, option) — Kgpu.cpp:186-251.  option 1/2: in = (lane, iv),
  * out = (i0, i1); option 3: in = (i0, i1), out = (lane, iv). */
 int kapy_fragments_map(const kapy_fragments *layout, const int64_t shape[2], int32_t option, const int64_t in[2], int64_t out[2]);
+/* getLayoutString — Kgpu.cpp:293-353, what bin/kapy-layout.cpp prints: for every element of a tensor of
+ * `shape`, row by row, the owning "T<lane>:<loop iv>", one block per replication round.  Writes at most
+ * out_len bytes (NUL-terminated) and returns the full length of the text, or a negative kapy_status. */
+int64_t kapy_layout_string(const kapy_fragments *layout, const int64_t shape[2], char *out, int64_t out_len);
 /* FragmentsLayoutAttr::transpose / exchangeAxes — Kgpu.cpp:253-263. */
 int kapy_fragments_transpose(const kapy_fragments *layout, kapy_fragments *out);
 int kapy_fragments_exchange_axes(const kapy_fragments *layout, kapy_fragments *out);

@@ -5,6 +5,11 @@
 #include <mutex>
 
 #include "common.hpp"
+#include <algorithm>
+#include <cstring>
+#include <string>
+#include <utility>
+#include <vector>
 #include "layout.hpp"
 
 namespace kapy {
@@ -183,6 +188,45 @@ int kapy_fragments_map(const kapy_fragments *layout, const int64_t shape[2], int
   out[0] = r.v0;
   out[1] = r.v1;
   return KAPY_OK;
+}
+
+int64_t kapy_layout_string(const kapy_fragments *layout, const int64_t shape[2], char *out, int64_t out_len) {
+  int rc = check_fragments(layout, "fragments");
+  if (rc) return rc;
+  if (!shape || shape[0] <= 0 || shape[1] <= 0) return fail(KAPY_ERR_INVALID, "layout string: shape must be positive");
+  const Fragments f = to_internal(layout);
+  const Idx2 sh{shape[0], shape[1]};
+  const int64_t lanes = f.a0 * f.a1, loop_size = f.loop_size(sh), numel = shape[0] * shape[1];
+  if (lanes > 9999 || loop_size > 9999) return fail(KAPY_ERR_UNSUPPORTED, "layout string: ids of more than four digits");
+  // owners of every element, in (lane, iv) order
+  std::vector<std::vector<std::pair<int64_t, int64_t>>> owners((size_t)numel);
+  for (int64_t lane = 0; lane < lanes; ++lane)
+    for (int64_t iv = 0; iv < loop_size; ++iv) {
+      const Idx2 at = f.to_index(sh, lane, iv, true);
+      owners[(size_t)(at.v0 * shape[1] + at.v1)].push_back({lane, iv});
+    }
+  auto width = [](int64_t id) { return id >= 1000 ? 4 : id >= 100 ? 3 : id >= 10 ? 2 : 1; };
+  const int lane_w = width(lanes - 1), iv_w = width(loop_size - 1);
+  std::string text;
+  for (size_t round = 0; round < owners[0].size(); ++round) {
+    if (round) text += "\n\n";
+    for (int64_t e = 0; e < numel; ++e) {
+      if (e % shape[1] == 0) text += e == 0 ? "[[" : "\n [";
+      if (round >= owners[(size_t)e].size()) return fail(KAPY_ERR_INVALID, "layout string: elements are not owned equally often");
+      const auto &o = owners[(size_t)e][round];
+      text.append((size_t)(lane_w - width(o.first)), ' ');
+      text += "T" + std::to_string(o.first) + ":";
+      text.append((size_t)(iv_w - width(o.second)), ' ');
+      text += std::to_string(o.second);
+      text += (e + 1) % shape[1] ? ", " : ((e + 1) == numel ? "]]" : "],");
+    }
+  }
+  if (out && out_len > 0) {
+    const size_t n = std::min(text.size(), (size_t)out_len - 1);
+    memcpy(out, text.data(), n);
+    out[n] = 0;
+  }
+  return (int64_t)text.size();
 }
 
 int kapy_fragments_transpose(const kapy_fragments *layout, kapy_fragments *out) {

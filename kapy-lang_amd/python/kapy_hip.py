@@ -27,7 +27,7 @@ DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, F8E4M3: 1, F8E5M2: 1, I8: 1, I16: 2, I32
 EXPORTS = [
     "kapy_version", "kapy_last_error", "kapy_device_info", "kapy_mk_global", "kapy_sv_global",
     "kapy_fragments_loops", "kapy_fragments_map", "kapy_fragments_transpose", "kapy_fragments_exchange_axes",
-    "kapy_fragments_default", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
+    "kapy_fragments_default", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
     "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
     "kapy_change", "kapy_reduce",
@@ -111,6 +111,8 @@ def lib():
     L.kapy_fragments_transpose.argtypes = [P(Fragments), P(Fragments)]
     L.kapy_fragments_exchange_axes.argtypes = [P(Fragments), P(Fragments)]
     L.kapy_fragments_default.argtypes = [A2, A2, i32, P(Fragments)]
+    L.kapy_layout_string.restype = i64
+    L.kapy_layout_string.argtypes = [P(Fragments), A2, C.c_char_p, i64]
     L.kapy_access_simd_size.restype = i64
     L.kapy_access_simd_size.argtypes = [i64, i64, i64]
     L.kapy_change_source.argtypes = [P(Fragments), P(Fragments), A2, i64, i64, P(i64), P(i64)]
@@ -131,10 +133,19 @@ def lib():
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
     for name in EXPORTS:
         f = getattr(L, name)
-        if name not in ("kapy_last_error", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
+        if name not in ("kapy_last_error", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
             f.restype = C.c_int
     _lib = L
     return L
+
+
+def layout_string(frag, shape):
+    n = lib().kapy_layout_string(C.byref(frag), A2(*shape), None, 0)
+    if n < 0:
+        raise KapyError(n, last_error())
+    buf = C.create_string_buffer(n + 1)
+    lib().kapy_layout_string(C.byref(frag), A2(*shape), buf, n + 1)
+    return buf.value.decode()
 
 
 def last_error():

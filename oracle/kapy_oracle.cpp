@@ -11,6 +11,7 @@
 #include <limits>
 #include <map>
 #include <set>
+#include <string>
 #include <vector>
 #ifdef _OPENMP
 #include <omp.h>
@@ -286,6 +287,45 @@ void ko_fragments_map12(const ko_fragments *l, const int64_t shape[2], int optio
   if (col_major) std::swap(out[0], out[1]);
   idx[0] = out[0];
   idx[1] = out[1];
+}
+
+// getLayoutString (Kgpu.cpp:293-353): for every element, in row-major order, the (lane, loop iv) pairs
+// that own it, printed as "T<lane>:<iv>" right-aligned to the widest lane id / iv; when an element has
+// several owners (replication) one block per round, separated by a blank line.
+// Returns the length of the text (without the terminating NUL); writes at most out_len bytes.
+static int id_width(int64_t id) { return id >= 1000 ? 4 : id >= 100 ? 3 : id >= 10 ? 2 : 1; }
+int64_t ko_layout_string(const ko_fragments *l, const int64_t shape[2], char *out, int64_t out_len) {
+  const int64_t lanes = l->lane_array[0] * l->lane_array[1], numel = shape[0] * shape[1];
+  int64_t S[2];
+  ko_fragments_loops(l, shape, nullptr, S);
+  const int64_t loop_size = S[0] * S[1];
+  std::vector<std::vector<std::pair<int64_t, int64_t>>> owners(numel);
+  for (int64_t lane = 0; lane < lanes; ++lane)
+    for (int64_t iv = 0; iv < loop_size; ++iv) {
+      int64_t idx[2];
+      ko_fragments_map12(l, shape, 1, lane, iv, idx);
+      owners[idx[0] * shape[1] + idx[1]].push_back({lane, iv});
+    }
+  const int wl = id_width(lanes - 1), wi = id_width(loop_size - 1);
+  std::string text;
+  const size_t rounds = owners[0].size();
+  for (size_t r = 0; r < rounds; ++r) {
+    if (r > 0) text += "\n\n";
+    for (int64_t e = 0; e < numel; ++e) {
+      if (e % shape[1] == 0) text += e == 0 ? "[[" : "\n [";
+      const auto pr = owners[e][r];
+      text += std::string(wl - id_width(pr.first), ' ') + "T" + std::to_string(pr.first) + ":";
+      text += std::string(wi - id_width(pr.second), ' ') + std::to_string(pr.second);
+      if ((e + 1) % shape[1] == 0) text += (e + 1) == numel ? "]]" : "],";
+      else text += ", ";
+    }
+  }
+  if (out && out_len > 0) {
+    const int64_t n = std::min<int64_t>((int64_t)text.size(), out_len - 1);
+    memcpy(out, text.data(), n);
+    out[n] = 0;
+  }
+  return (int64_t)text.size();
 }
 
 // Option 3: (i0, i1) -> (lane, iv)   (Kgpu.cpp:196-219).

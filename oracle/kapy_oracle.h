@@ -76,6 +76,7 @@ void ko_fill_bits16(uint16_t *dst, int64_t n, uint64_t seed, uint64_t stream);
 
 /* ---- layouts ---- */
 void ko_fragments_loops(const ko_fragments *l, const int64_t shape[2], int64_t warp_loops[2], int64_t loop_space[2]);
+int64_t ko_layout_string(const ko_fragments *l, const int64_t shape[2], char *out, int64_t out_len);
 void ko_fragments_map12(const ko_fragments *l, const int64_t shape[2], int option, int64_t lane, int64_t iv, int64_t idx[2]);
 void ko_fragments_map3(const ko_fragments *l, const int64_t shape[2], int64_t i0, int64_t i1, int64_t *lane, int64_t *iv);
 void ko_fragments_transpose(const ko_fragments *l, ko_fragments *out);

@@ -80,6 +80,7 @@ def lib():
         L.ko_fill_bits16.restype = None; L.ko_fill_bits16.argtypes = [vp, i64, u64, u64]
         A2 = i64 * 2
         L.ko_fragments_loops.restype = None; L.ko_fragments_loops.argtypes = [P(Fragments), A2, A2, A2]
+        L.ko_layout_string.restype = i64; L.ko_layout_string.argtypes = [P(Fragments), A2, C.c_char_p, i64]
         L.ko_fragments_map12.restype = None; L.ko_fragments_map12.argtypes = [P(Fragments), A2, C.c_int, i64, i64, A2]
         L.ko_fragments_map3.restype = None; L.ko_fragments_map3.argtypes = [P(Fragments), A2, i64, i64, P(i64), P(i64)]
         L.ko_fragments_transpose.restype = None; L.ko_fragments_transpose.argtypes = [P(Fragments), P(Fragments)]

@@ -81,6 +81,16 @@ def test_fragments_maps_agree_with_oracle(ko, shape):
         assert bytes(t1) == bytes(t2)
 
 
+def test_layout_string_agrees_with_oracle(ko):
+    for la, ll, mi, ma in LAYOUTS:
+        for shape in ((8, 8), (16, 64), (64, 4), (128, 32)):
+            f, g = kh.Fragments.make(la, ll, mi, ma), ko.Fragments.make(la, ll, mi, ma)
+            n = ko.lib().ko_layout_string(C.byref(g), kh.A2(*shape), None, 0)
+            buf = C.create_string_buffer(n + 1)
+            ko.lib().ko_layout_string(C.byref(g), kh.A2(*shape), buf, n + 1)
+            assert kh.layout_string(f, shape) == buf.value.decode()
+
+
 def test_default_layout_simd_change_agree_with_oracle(ko):
     L, O = kh.lib(), ko.lib()
     for loops, shape, rm in (((1, 8), (64, 64), 1), ((1, 1), (1, 256), 1), ((8, 1), (64, 16), 0), ((1, 4), (8, 8), 1)):

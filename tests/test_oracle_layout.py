@@ -191,3 +191,34 @@ def test_swizzle_search_matches_bruteforce_replay_64_banks(ko):
     for bp, lp in itertools.product((4,), (1, 2, 4, 8, 16)):
         ok = _replay_conflicts(ko, f, shape, 64, 1, bits, bp, lp, 64, 64 // bp) == 1
         assert ok == ((bp, lp) in found)
+
+
+def _layout_string(ko, f, shape):
+    n = ko.lib().ko_layout_string(C.byref(f), A2(*shape), None, 0)
+    buf = C.create_string_buffer(n + 1)
+    ko.lib().ko_layout_string(C.byref(f), A2(*shape), buf, n + 1)
+    return buf.value.decode()
+
+
+def test_layout_string_of_the_attrs_td_example(ko):
+    """What bin/kapy-layout.cpp prints (getLayoutString, Kgpu.cpp:293-353) for the documented example
+    #kgpu.fragments<[8,4],[1,2],(0,1)> on an 8x8 tensor: row r = lanes 4r..4r+3, two loop ivs each, ids
+    right-aligned to the widest lane id (31 -> width 2) and iv (1 -> width 1)."""
+    f = ko.Fragments.make([8, 4], [1, 2], 0, 1)
+    text = _layout_string(ko, f, (8, 8))
+    rows = text.split("\n")
+    assert len(rows) == 8
+    assert rows[0] == "[[ T0:0,  T0:1,  T1:0,  T1:1,  T2:0,  T2:1,  T3:0,  T3:1],"
+    assert rows[3] == " [T12:0, T12:1, T13:0, T13:1, T14:0, T14:1, T15:0, T15:1],"
+    assert rows[7] == " [T28:0, T28:1, T29:0, T29:1, T30:0, T30:1, T31:0, T31:1]]"
+
+
+def test_layout_string_prints_one_block_per_replication_round(ko):
+    """A layout larger than the tensor owns every element several times (Attrs.td:55-78): the 8-lane example
+    [[0,0,1,1],[2,2,3,3],...] x 4 rows on a 2x4 tensor replicates twice along rows."""
+    f = ko.Fragments.make([4, 2], [1, 2], 0, 1)
+    text = _layout_string(ko, f, (2, 4))
+    blocks = text.split("\n\n")
+    assert len(blocks) == 2
+    assert blocks[0] == "[[T0:0, T0:1, T1:0, T1:1],\n [T2:0, T2:1, T3:0, T3:1]]"
+    assert blocks[1] == "[[T4:0, T4:1, T5:0, T5:1],\n [T6:0, T6:1, T7:0, T7:1]]"

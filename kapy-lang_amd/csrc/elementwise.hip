@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include <functional>
 #include "numeric.hpp"
 
 namespace kapy {
@@ -130,6 +131,242 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
     regs[I.dst][tid] = r;  // regs[*][tid] is private to the lane: no barrier needed
   }
 }
+
+// ---------------------------------------------------------------------------------------------
+// Stack machine: any program whose expression tree needs at most three live values, on 8
+// consecutive elements per lane in registers.  The host unfolds the SSA program into postfix form
+// (a value used twice is simply evaluated twice: every op is pure) and gives every step the stack
+// depth it works at, so the three values are three fixed register arrays chosen by a uniform branch:
+// no register is ever indexed at run time and nothing is shuffled.  Values are fp32 images of the typed value, rounded to the
+// result type after every arithmetic op exactly as the register machine does.
+constexpr int kMaxPost = 40;
+enum PostKind { kPushIn = 100, kPushImm = 101, kCast = 102, kStore = 103, kRevSub = 104, kRevDiv = 105 };
+enum InKind { kInFull = 0, kInRow = 1 /* [1 x n] */, kInCol = 2 /* [m x 1] */, kInScalar = 3 };
+struct PostOp {
+  int16_t op, a, dtype, rmode;
+  int32_t slot;  // which of the three values holds the result (and the left operand)
+  float imm;
+};
+struct StackIn {
+  const char *base;
+  int64_t stride0;
+  int32_t dtype, kind;
+};
+struct StackProgram {
+  PostOp post[kMaxPost];
+  StackIn in[kMaxInputs];
+  char *out;
+  int64_t out_stride0;
+  int32_t n_post, n_ins, out_dtype, rows, vec_per_row;
+};
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void widen16x8(u32x4 v, int dtype, float f[8]) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t word = v[w];
+    if (dtype == KAPY_BF16) {
+      f[2 * w] = bits_f32(word << 16);
+      f[2 * w + 1] = bits_f32(word & 0xFFFF0000u);
+    } else {
+      f[2 * w] = f16_to_f32((uint16_t)word);
+      f[2 * w + 1] = f16_to_f32((uint16_t)(word >> 16));
+    }
+  }
+}
+// The 8 elements of vector jv of row i of a full-extent operand, as they lie in memory (16, 32 or 8 bytes).
+struct Raw8 {
+  u32x4 lo, hi;
+};
+__device__ __forceinline__ Raw8 fetch8(const StackIn &g, int32_t i, int32_t jv, bool streaming) {
+  const int eb = g.dtype == KAPY_F32 ? 4 : (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16) ? 2 : 1;
+  const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * eb;
+  Raw8 r;
+  r.lo = r.hi = u32x4{0, 0, 0, 0};
+  if (eb == 2) r.lo = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
+  else if (eb == 4) {
+    r.lo = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
+    r.hi = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr + 1) : *((const u32x4 *)ptr + 1);
+  } else {
+    const u32x2 v = *(const u32x2 *)ptr;
+    r.lo[0] = v[0];
+    r.lo[1] = v[1];
+  }
+  return r;
+}
+__device__ __forceinline__ void widen8(const Raw8 &r, int dtype, float f[8]) {
+  if (dtype == KAPY_F16 || dtype == KAPY_BF16) widen16x8(r.lo, dtype, f);
+  else if (dtype == KAPY_F32) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t a = r.lo[e], b = r.hi[e];
+      f[e] = bits_f32(a);
+      f[4 + e] = bits_f32(b);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t word = r.lo[e >> 2];
+      const uint8_t byte = (uint8_t)(word >> (8 * (e & 3)));
+      f[e] = dtype == KAPY_F8E4M3 ? e4m3_to_f32(byte) : e5m2_to_f32(byte);
+    }
+  }
+}
+template <bool NARROW>
+__device__ __forceinline__ void load8(const StackIn &g, int32_t i, int32_t jv, float f[8]) {
+  if (g.kind == kInCol || g.kind == kInScalar) {
+    const float v = load_as_f32(g.base, g.dtype, g.kind == kInCol ? i * g.stride0 : 0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = v;
+    return;
+  }
+  if (NARROW) {
+    const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * 2;
+    widen16x8(g.kind == kInFull ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr, g.dtype, f);
+  } else widen8(fetch8(g, i, jv, g.kind == kInFull), g.dtype, f);
+}
+template <bool NARROW>
+__device__ __forceinline__ void round8(float f[8], int dtype, bool rn) {
+  switch (dtype) {
+  case KAPY_F32: return;
+  case KAPY_F16:
+    if (rn) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)(_Float16)f[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = f16_to_f32(f32_to_f16_rz(f[e]));
+    }
+    return;
+  case KAPY_BF16:
+    if (rn) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)(__bf16)f[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = bf16_to_f32(f32_to_bf16_rz(f[e]));
+    }
+    return;
+  default:
+    if (!NARROW) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = round_to_dtype(f[e], dtype, rn);
+    }
+  }
+}
+template <bool NARROW>
+__device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const float f[8]) {
+  if (NARROW || dtype == KAPY_F16 || dtype == KAPY_BF16) {
+    u32x4 v;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v[w] = dtype == KAPY_F16 ? pack2_f16_rn(f[2 * w], f[2 * w + 1]) : pack2_bf16_rn(f[2 * w], f[2 * w + 1]);
+    __builtin_nontemporal_store(v, (u32x4 *)(out + elem * 2));
+  } else if (dtype == KAPY_F32) {
+    u32x4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[e] = f32_bits(f[e]);
+      hi[e] = f32_bits(f[4 + e]);
+    }
+    __builtin_nontemporal_store(lo, (u32x4 *)(out + elem * 4));
+    __builtin_nontemporal_store(hi, (u32x4 *)(out + elem * 4) + 1);
+  } else {
+    u32x2 v = {0, 0};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t byte = dtype == KAPY_F8E4M3 ? f32_to_e4m3(f[e], true) : f32_to_e5m2(f[e], true);
+      v[e >> 2] |= byte << (8 * (e & 3));
+    }
+    *(u32x2 *)(out + elem) = v;
+  }
+}
+
+// One step with its result (and left operand) in value D, the right operand in value D+1 and the
+// third operand of an fma in value D+2; D is a template parameter so that no register is indexed.
+// NARROW: every operand, every intermediate type and the result are f16 / bf16 / f32-from-16-bit
+// (no fp8, no fp32 in memory): the common case, and it needs far fewer registers.
+template <int D, bool NARROW>
+__device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &I, int32_t i, int32_t jv, float (&v)[3][8]) {
+  constexpr int R = D + 1 < 3 ? D + 1 : 2, T = D + 2 < 3 ? D + 2 : 2;
+  float *x = v[D];
+  const float *y = v[R], *z = v[T];
+  switch (I.op) {
+  case kPushIn: load8<NARROW>(P.in[I.a], i, jv, x); return;
+  case kPushImm: {
+    const float c = round_to_dtype(I.imm, I.dtype, true);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = c;
+    return;
+  }
+  case kStore: store8<NARROW>(P.out, P.out_dtype, (int64_t)i * P.out_stride0 + (int64_t)jv * 8, x); return;
+  case kCast: round8<NARROW>(x, I.dtype, I.rmode != KAPY_RZ); return;
+  case KAPY_EW_ADDF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fadd_rn(x[e], y[e]);
+    break;
+  case KAPY_EW_SUBF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fsub_rn(x[e], y[e]);
+    break;
+  case kRevSub:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fsub_rn(y[e], x[e]);
+    break;
+  case KAPY_EW_MULF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fmul_rn(x[e], y[e]);
+    break;
+  case KAPY_EW_DIVF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(x[e], y[e]);
+    break;
+  case kRevDiv:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(y[e], x[e]);
+    break;
+  case KAPY_EW_MAXIMUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = max_nan(x[e], y[e]);
+    break;
+  case KAPY_EW_MINIMUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = min_nan(x[e], y[e]);
+    break;
+  case KAPY_EW_FMA:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fmaf_rn(x[e], y[e], z[e]);
+    break;
+  default:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = apply_unary(I.op, x[e]);
+  }
+  if (I.dtype != KAPY_F32) round8<NARROW>(x, I.dtype, true);
+}
+
+template <bool NARROW>
+__device__ __forceinline__ void stack_run(const StackProgram &P) {
+  const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (slot >= (int64_t)P.rows * P.vec_per_row) return;
+  const int32_t i = (int32_t)(slot / P.vec_per_row), jv = (int32_t)(slot - (int64_t)i * P.vec_per_row);
+  float v[3][8];
+#pragma unroll
+  for (int d = 0; d < 3; ++d)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[d][e] = 0.f;
+  for (int pc = 0; pc < P.n_post; ++pc) {
+    const PostOp I = P.post[pc];
+    switch (I.slot) {
+    case 0: stack_step<0, NARROW>(P, I, i, jv, v); break;
+    case 1: stack_step<1, NARROW>(P, I, i, jv, v); break;
+    default: stack_step<2, NARROW>(P, I, i, jv, v);
+    }
+  }
+}
+
+// Throughput of this kernel follows the number of resident waves (each lane walks its program one
+// dependent step at a time), so the 16-bit-only form is held to 64 registers: 8 waves per SIMD.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void stack_kernel_narrow(StackProgram P) { stack_run<true>(P); }
+__global__ __launch_bounds__(256) void stack_kernel_any(StackProgram P) { stack_run<false>(P); }
 
 // ---------------------------------------------------------------------------------------------
 // out[i,j] = cast_out( act( f32(x[i,j]) * scale + f32(bias) ) ), x/out contiguous along j.
@@ -488,6 +725,119 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
   return true;
 }
 
+// does any ld_global of input `input` ask for a padding pattern other than zero?
+bool prog_padding_nonzero(const kapy_ew_inst *prog, int n_inst, int input) {
+  for (int k = 0; k < n_inst; ++k)
+    if (prog[k].op == KAPY_EW_LD_GLOBAL && prog[k].a == input && prog[k].c != KAPY_PAD_ZERO) return true;
+  return false;
+}
+// Postfix form of the program for the stack machine; false when the program does not fit it
+// (a tree deeper than three values, more than kMaxPost steps after unfolding shared values,
+// operands that are not full / row / column / scalar views readable 8 at a time, padding).
+bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins,
+                         const kapy_global *out, StackProgram *P) {
+  struct N {
+    int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
+    float imm = 0.f;
+  };
+  std::vector<N> nodes;
+  int reg[kMaxRegs];
+  for (int r = 0; r < kMaxRegs; ++r) reg[r] = -1;
+  int stored = -1, n_store = 0;
+  for (int k = 0; k < n_inst; ++k) {
+    const kapy_ew_inst &I = prog[k];
+    N n;
+    n.op = I.op;
+    n.dtype = result_dtype[k];
+    n.rmode = I.rmode;
+    n.imm = I.imm;
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: n.input = I.a; break;
+    case KAPY_EW_SPLAT: break;
+    case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; ++n_store; continue;
+    case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
+    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+      n.a = reg[I.a]; n.b = reg[I.b]; break;
+    default: n.a = reg[I.a];
+    }
+    nodes.push_back(n);
+    reg[I.dst] = (int)nodes.size() - 1;
+  }
+  if (n_store != 1 || stored < 0) return false;
+  // the result: rows contiguous, 8 elements at a time
+  const int64_t o0 = extent0(out), o1 = extent1(out);
+  const int ob = dtype_bytes(out->dtype);
+  if (!is_float(out->dtype) || out->stride1 != 1 || o1 % 8 != 0 || ((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
+  if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  for (int k = 0; k < n_ins; ++k) {
+    const kapy_global *g = ins[k];
+    StackIn &in = P->in[k];
+    in.base = view_base(g);
+    in.stride0 = g->stride0;
+    in.dtype = g->dtype;
+    if (!is_float(g->dtype)) return false;
+    const int64_t e0 = extent0(g), e1 = extent1(g);
+    const int eb = dtype_bytes(g->dtype);
+    const bool vec_ok = g->stride1 == 1 && ((uintptr_t)in.base % (8 * eb)) == 0 && (g->stride0 * eb) % (8 * eb) == 0;
+    if (e0 == o0 && e1 == o1 && vec_ok) in.kind = kInFull;
+    else if (e0 == 1 && e1 == o1 && vec_ok) in.kind = kInRow;
+    else if (e1 == 1 && e0 == o0) in.kind = kInCol;
+    else if (e0 == 1 && e1 == 1) in.kind = kInScalar;
+    else return false;
+  }
+  // depth of the stack an expression needs when the deeper operand is evaluated first
+  std::vector<int> need(nodes.size(), 0);
+  for (size_t id = 0; id < nodes.size(); ++id) {
+    const N &n = nodes[id];
+    if (n.op == KAPY_EW_LD_GLOBAL || n.op == KAPY_EW_SPLAT) need[id] = 1;
+    else if (n.op == KAPY_EW_FMA) need[id] = std::max(need[n.a], std::max(need[n.b] + 1, need[n.c] + 2));
+    else if (n.b >= 0) need[id] = std::min(std::max(need[n.a], need[n.b] + 1), std::max(need[n.b], need[n.a] + 1));
+    else need[id] = need[n.a];
+  }
+  if (need[stored] > 3) return false;
+  int count = 0;
+  bool ok = true;
+  auto push = [&](int op, int a, int dtype, int rmode, int slot, float imm) {
+    if (count >= kMaxPost || slot > 2) { ok = false; return; }
+    P->post[count++] = PostOp{(int16_t)op, (int16_t)a, (int16_t)dtype, (int16_t)rmode, slot, imm};
+  };
+  // evaluate node id into value d (values d+1, d+2 are free to use)
+  std::function<void(int, int)> emit = [&](int id, int d) {
+    if (!ok) return;
+    const N &n = nodes[id];
+    switch (n.op) {
+    case KAPY_EW_LD_GLOBAL:
+      if (prog_padding_nonzero(prog, n_inst, n.input)) { ok = false; return; }
+      push(kPushIn, n.input, n.dtype, 0, d, 0.f);
+      return;
+    case KAPY_EW_SPLAT: push(kPushImm, 0, n.dtype, 0, d, n.imm); return;
+    case KAPY_EW_FPTOFP: emit(n.a, d); push(kCast, 0, n.dtype, n.rmode, d, 0.f); return;
+    case KAPY_EW_FMA: emit(n.a, d); emit(n.b, d + 1); emit(n.c, d + 2); push(KAPY_EW_FMA, 0, n.dtype, 0, d, 0.f); return;
+    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF: {
+      const bool a_first = std::max(need[n.a], need[n.b] + 1) <= std::max(need[n.b], need[n.a] + 1);
+      if (a_first) { emit(n.a, d); emit(n.b, d + 1); push(n.op, 0, n.dtype, 0, d, 0.f); }
+      else {
+        emit(n.b, d); emit(n.a, d + 1);
+        push(n.op == KAPY_EW_SUBF ? kRevSub : n.op == KAPY_EW_DIVF ? kRevDiv : n.op, 0, n.dtype, 0, d, 0.f);
+      }
+      return;
+    }
+    default: emit(n.a, d); push(n.op, 0, n.dtype, 0, d, 0.f);
+    }
+  };
+  emit(stored, 0);
+  push(kStore, 0, out->dtype, 0, 0, 0.f);
+  if (!ok) return false;
+  P->n_post = count;
+  P->n_ins = n_ins;
+  P->out = (char *)view_base(out);
+  P->out_stride0 = out->stride0;
+  P->out_dtype = out->dtype;
+  P->rows = (int32_t)o0;
+  P->vec_per_row = (int32_t)(o1 / 8);
+  return true;
+}
+
 uint32_t padding_word_of(int32_t dtype, int32_t padding) {
   static const uint32_t f32[4] = {0, 0x7FC00000u, 0x7F800000u, 0xFF800000u};
   static const uint32_t f16[4] = {0, 0x7E00u, 0x7C00u, 0xFC00u};
@@ -558,6 +908,21 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 #undef KAPY_LAUNCH_AFFINE
     KAPY_HIP_CHECK(hipGetLastError());
     return KAPY_OK;
+  }
+
+  {
+    StackProgram SP;
+    memset(&SP, 0, sizeof SP);
+    if (build_stack_program(prog, n_inst, result_dtype, ins, n_ins, out, &SP)) {
+      const int64_t slots = (int64_t)SP.rows * SP.vec_per_row;
+      bool narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
+      for (int k = 0; k < n_ins; ++k) narrow = narrow && (ins[k]->dtype == KAPY_F16 || ins[k]->dtype == KAPY_BF16);
+      for (int k = 0; k < n_inst; ++k) narrow = narrow && !is_f8(result_dtype[k]);
+      if (narrow) stack_kernel_narrow<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
+      else stack_kernel_any<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
+      KAPY_HIP_CHECK(hipGetLastError());
+      return KAPY_OK;
+    }
   }
 
   Program P;

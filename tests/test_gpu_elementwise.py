@@ -184,3 +184,39 @@ def test_broadcast_column_vector_and_padding(ko):
             dict(op=kh.EW_FPTOFP, dst=4, a=2, dtype=kh.F16, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=4)]
     got, want = _run_prog(ko, prog, [x, col], [kh.F16, kh.F16], kh.F16, m, n, in_shapes=[(m, n), (m, 1)])
     _check_ulp(got, want, kh.F16)
+
+
+def test_register_stack_kernel_tree_shapes_and_operand_kinds(ko):
+    """Programs that are not the act(x*s+bias) chain run on the in-register stack machine when every operand can be
+    read 8 elements at a time: reversed subtraction / division (deeper operand on the right), a depth-3 tree, an fma
+    of three subtrees, row / column / scalar operands, f32 and fp8 operands and results; exactly rounded ops must be
+    bit-exact against the oracle, the same programs at a width that is not a multiple of 8 take the interpreter."""
+    L, ADD, SUB, MUL, DIV, FMA, MAX, ST, CAST, SPL = (kh.EW_LD_GLOBAL, kh.EW_ADDF, kh.EW_SUBF, kh.EW_MULF, kh.EW_DIVF, kh.EW_FMA,
+                                                      kh.EW_MAXIMUMF, kh.EW_ST_GLOBAL, kh.EW_FPTOFP, kh.EW_SPLAT)
+    for (m, n) in ((16, 256), (16, 252)):
+        a = ko.fill_normal(m * n, kh.F16, 21, 0).reshape(m, n)
+        b = ko.fill_uniform(m * n, kh.F16, 21, 1, 0.5, 2.0).reshape(m, n)
+        row = ko.fill_normal(n, kh.F16, 21, 2)
+        col = ko.fill_normal(m, kh.F16, 21, 3)
+        one = ko.fill_normal(1, kh.F16, 21, 4)
+        # (a - (b*row)) / ((a + col) max (b - one)), all in f16: reversed sub and div, depth 3, every operand kind
+        insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=L, dst=2, a=2), dict(op=L, dst=3, a=3), dict(op=L, dst=4, a=4),
+                 dict(op=MUL, dst=5, a=1, b=2), dict(op=SUB, dst=5, a=0, b=5), dict(op=ADD, dst=6, a=0, b=3), dict(op=SUB, dst=7, a=1, b=4),
+                 dict(op=MAX, dst=6, a=6, b=7), dict(op=DIV, dst=5, a=5, b=6), dict(op=ST, a=5)]
+        got, want = _run_prog(ko, insts, [a, b, row, col, one], [kh.F16] * 5, kh.F16, m, n, [(m, n), (m, n), (1, n), (m, 1), (1, 1)])
+        _check_ulp(got, want, kh.F16)     # division is within 2 ulp of f32 (div.full), the rest exact
+        # fma(a*b, b - a, a + b) in f32 from f16 operands, f32 result
+        insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=CAST, dst=2, a=0, dtype=kh.F32), dict(op=CAST, dst=3, a=1, dtype=kh.F32),
+                 dict(op=MUL, dst=4, a=2, b=3), dict(op=SUB, dst=5, a=3, b=2), dict(op=ADD, dst=6, a=2, b=3), dict(op=FMA, dst=7, a=4, b=5, c=6),
+                 dict(op=ST, a=7)]
+        got, want = _run_prog(ko, insts, [a, b], [kh.F16] * 2, kh.F32, m, n)
+        assert np.array_equal(got, want)
+        # quantise: f32 operand scaled by a splat, rounded to e4m3; and back: e4m3 operand widened to bf16
+        x32 = ko.fill_normal(m * n, kh.F32, 22, 0).reshape(m, n)
+        insts = [dict(op=L, dst=0, a=0), dict(op=SPL, dst=1, dtype=kh.F32, imm=37.5), dict(op=MUL, dst=0, a=0, b=1),
+                 dict(op=CAST, dst=2, a=0, dtype=kh.F8E4M3, rmode=kh.RN), dict(op=ST, a=2)]
+        q, wantq = _run_prog(ko, insts, [x32], [kh.F32], kh.F8E4M3, m, n)
+        assert np.array_equal(q, wantq)
+        insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.BF16), dict(op=ST, a=1)]
+        got, want = _run_prog(ko, insts, [wantq], [kh.F8E4M3], kh.BF16, m, n)
+        assert np.array_equal(got, want)

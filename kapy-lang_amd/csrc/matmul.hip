@@ -115,6 +115,21 @@ struct TileLayout {
   }
 };
 
+// ds_read_b64_tr_b16 issued as opaque assembly.  Through the compiler's builtin every such read is
+// preceded by s_waitcnt vmcnt(0) (it is taken to alias the LDS-direct loads in flight), which
+// serialises the whole global->LDS pipeline; ordering against those loads is established by the
+// kernel's own waits and barriers.  The result is pending until tr_reads_wait() has been called and
+// must not be touched before: the caller keeps it in a fragment buffer that is only consumed one
+// K-slice later (the kernel using this has no register spills, which would copy a pending register).
+typedef uint32_t u32x2_lds __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32x2_lds tr_read_b64(const char *lds_ptr) {
+  const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)lds_ptr;  // LDS pointers are 32-bit byte offsets
+  u32x2_lds r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+__device__ __forceinline__ void tr_reads_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
 // s_waitcnt immediate that waits only on vmcnt <= n (gfx9 encoding: vmcnt in bits [3:0] and [15:14],
 // expcnt [6:4] and lgkmcnt [11:8] left at "no wait").
 constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
@@ -790,17 +805,18 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   uint32_t b_off[kTn];
 #pragma unroll
   for (int j = 0; j < kTn; ++j) b_off[j] = kBytesA + b_row * kRowB + (((wn * 8 + j * 2 + ((l16 & 3) >> 1)) ^ b_key) * 16) + (l16 & 1) * 8;
-  typedef short s16x4 __attribute__((ext_vector_type(4)));
   struct Frag {
     u32x4 c[1];
   };
+  // an rhs fragment comes out of LDS as two 8-byte halves (k-rows +0..3 and +4..7 of the lane's K-group)
+  struct FragHalves {
+    u32x2 h[2];
+  };
   auto read_a = [&](int stage, int kk, int i) { return *(const u32x4 *)(lds + stage * kStage + a_off[kk] + i * 16 * kRowA); };
-  auto read_b = [&](int stage, int kk, int j) {
+  auto read_b = [&](int stage, int kk, int j, FragHalves &dst) {
     const char *base = lds + stage * kStage + b_off[j] + kk * 32 * kRowB;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)base);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(base + 4 * kRowB));
-    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-    return u32x4{l2[0], l2[1], h2[0], h2[1]};
+    dst.h[0] = tr_read_b64(base);
+    dst.h[1] = tr_read_b64(base + 4 * kRowB);
   };
 
   using Acc = typename T::Acc;
@@ -816,11 +832,12 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     for (int idx = 0; idx < kLoads; ++idx) issue_load(j, j, idx);
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (STAGES - 2)));
   __builtin_amdgcn_s_barrier();  // tile 0 published
-  Frag af[2][kTm], bf[2][kTn];
+  Frag af[2][kTm];
+  FragHalves bf[2][kTn];
 #pragma unroll
   for (int i = 0; i < kTm; ++i) af[0][i].c[0] = read_a(0, 0, i);
 #pragma unroll
-  for (int j = 0; j < kTn; ++j) bf[0][j].c[0] = read_b(0, 0, j);
+  for (int j = 0; j < kTn; ++j) read_b(0, 0, j, bf[0][j]);
 
   constexpr int kReads = kTm + kTn;
   constexpr int kLoadSpacing = (KK * kMfmas) / kLoads;  // matrix instructions between two loads
@@ -836,16 +853,19 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       constexpr int par = decltype(parity)::value;
-      Frag *a_cur = af[(kk + par) & 1], *b_cur = bf[(kk + par) & 1], *a_nxt = af[(kk + par + 1) & 1], *b_nxt = bf[(kk + par + 1) & 1];
+      Frag *a_cur = af[(kk + par) & 1], *a_nxt = af[(kk + par + 1) & 1];
+      FragHalves *b_cur = bf[(kk + par) & 1], *b_nxt = bf[(kk + par + 1) & 1];
+      tr_reads_wait();  // the rhs fragments of this slice were requested during the previous one
 #pragma unroll
       for (int g = 0; g < kMfmas; ++g) {
         const int i = g / kTn, j = g % kTn;
-        acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
+        const u32x4 b_op = {b_cur[j].h[0][0], b_cur[j].h[0][1], b_cur[j].h[1][0], b_cur[j].h[1][1]};
+        acc[i][j] = T::mfma(&b_op, a_cur[i].c, acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         if (g < kReads) {
           const int rs = kk + 1 < KK ? stage : next_stage, rk = kk + 1 < KK ? kk + 1 : 0;
           if (g < kTm) a_nxt[g].c[0] = read_a(rs, rk, g);
-          else b_nxt[g - kTm].c[0] = read_b(rs, rk, g - kTm);
+          else read_b(rs, rk, g - kTm, b_nxt[g - kTm]);
         }
         if ((kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads)
           issue_load(kt + STAGES - 1, free_stage, (kk * kMfmas + g) / kLoadSpacing);
@@ -1266,11 +1286,8 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
     };
     static const NnVariant kNn[] = {{64, 4, launch_nn<Bf16M16, 64, 4>, launch_nn<F16M16, 64, 4>}, {64, 3, launch_nn<Bf16M16, 64, 3>, launch_nn<F16M16, 64, 3>},
                                     {32, 4, launch_nn<Bf16M16, 32, 4>, launch_nn<F16M16, 32, 4>}};
-    // more workgroups than CUs: the 64 KiB ring of the K=32 tile lets two workgroups share a CU, which
-    // hides more latency than the deeper K=64 tile does with one
-    const bool prefer_k32 = !c.tile_k && !c.stages && (int64_t)(p.M / kNBM) * (p.N / kNBN) > device_cus() && p.K % 32 == 0;
     for (const NnVariant &v : kNn) {
-      if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk || (prefer_k32 && v.bk != 32)) continue;
+      if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }

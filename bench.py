@@ -56,7 +56,7 @@ def _events(fn, steps, warmup):
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the
 # same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
-MEASURED_TRAFFIC = {"gelu": 268406784, "transpose": 268450816}
+MEASURED_TRAFFIC = {"gelu": 268414976, "transpose": 268456960}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):

@@ -219,6 +219,33 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
  * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`. */
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream);
 
+/* Runs a kapy.func given in the textual form of the reference's Kapy-dialect fixtures
+ * (test/Conversion/KapyToKgpu/elementwise_add.mlir, reduce_sum.mlir, matmul.mlir; op syntax from
+ * include/kapy/Dialect/Kapy/IR/Ops.td) on the device: every program id of `grid` and every warp id of the
+ * module's kapy.num_warps is executed in turn, each tensor op as one call of the entry points above on
+ * `stream` (mk_global/sv_global/sv_shared: MkGlobalOpToLLVM.cpp:23-47, SvGlobalOpToLLVM.cpp:22-40,
+ * SvSharedOpToLLVM.cpp:20-42; ld_global/st_global/cp_async_global_to_shared/ld_matrix: kapy_copy; arith on
+ * tensors: kapy_elementwise; kapy.reduce: kapy_reduce; kapy.matmul: kapy_matmul; scf.for with iter_args).
+ * Warps run one after the other, so a program whose warps exchange data through shared memory between
+ * barriers is outside what this executes correctly; the three fixtures are not of that kind.
+ * `args` follow the function's signature: a device pointer (with the size of its allocation in bytes, 0 =
+ * unknown, which mk_global is checked against) for !kapy.ptr<1>, an i32 otherwise.  A sub-view that leaves
+ * its parent is an error.  func_name NULL = the first function of the module.  The call allocates a 64 MiB
+ * device arena for shared-memory and register tensors, synchronises `stream` and frees it before it returns:
+ * it is a way to run the reference's programs against this library, not a fast path. */
+typedef struct kapy_mlir_arg {
+  void *ptr;      /* device pointer, for a !kapy.ptr<1> argument                    */
+  int64_t bytes;  /* size of the allocation behind ptr; 0 = unknown (no range check) */
+  int32_t i32;    /* value, for an i32 argument                                      */
+  int32_t reserved;
+} kapy_mlir_arg;
+int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_arg *args, int32_t n_args,
+                  const int32_t grid[3], void *stream);
+/* The parsing half of kapy_run_mlir, without a device: KAPY_ERR_INVALID for text that does not parse,
+ * KAPY_ERR_UNSUPPORTED for an op outside the set above; otherwise the function's argument count, its number
+ * of ops (loop bodies included) and the module's kapy.num_warps.  Out pointers may be NULL. */
+int kapy_parse_mlir(const char *mlir_text, const char *func_name, int32_t *n_args, int32_t *n_ops, int32_t *num_warps);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,682 @@
+// frontend.cpp — executes a kapy.func written in the textual form of the reference's fixtures
+// (test/Conversion/KapyToKgpu/{elementwise_add,reduce_sum,matmul}.mlir) by driving the C ABI.
+//
+// The reference compiles such a function to one PTX kernel; here every program of the launch grid
+// and every warp of the program is run in turn on the host, and every tensor op is one library call
+// on the caller's stream: mk_global / sv_global / sv_shared are descriptor arithmetic
+// (MkGlobalOpToLLVM.cpp:23-47, SvGlobalOpToLLVM.cpp:22-40, SvSharedOpToLLVM.cpp:20-42), ld_global /
+// st_global / cp_async_global_to_shared / ld_matrix are kapy_copy between descriptors, arith ops on
+// register tensors are one-op elementwise programs, kapy.reduce and kapy.matmul are the entry points
+// of the same name.  Shared-memory tensors and register tensors live in a device arena that the call
+// allocates and frees.  It is a way to run the reference's own programs against this library, not a
+// fast path: a program costs tens of launches.
+//
+// Supported: func arguments (!kapy.ptr<1>, i32), arith.constant (i32, dense tensor), arith
+// addi/subi/muli/divui/remui/cmpi/select, arith addf/subf/mulf/divf/maximumf/minimumf on tensors,
+// kapy.program_id / warp_id / mk_global / sv_global / mk_shared / sv_shared / ld_global / st_global /
+// cp_async_global_to_shared / cp_async_wait_group / ld_matrix / matmul / reduce (addf or maximumf
+// lambda) / return, scf.for with iter_args and scf.yield.
+#include <cctype>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+namespace kapy {
+namespace {
+
+struct Type {
+  enum Kind { kNone, kInt, kPtr, kFloat, kTensor } kind = kNone;
+  int dtype = -1;
+  int64_t shape[2] = {0, 0};  // -1 = dynamic
+  std::string space;          // alias of the encoding: "global", "shared", "values"
+};
+
+struct Op {
+  std::string name;
+  std::vector<std::string> results;   // "%3"; a multi-result op "%34:3" is expanded to %34#0 ..
+  std::vector<std::string> operands;  // every %value of the operand section, in order
+  std::vector<std::string> words;     // bare words of the operand section (cmpi predicate, matmul way, constants)
+  std::map<std::string, std::string> attrs;
+  std::vector<Type> types;            // every type after the top-level ':'
+  std::vector<std::string> region_args;  // scf.for: induction variable, then iter_args names
+  std::vector<Op> body;
+  int line = 0;
+};
+
+struct Func {
+  std::string name;
+  std::vector<std::string> arg_names;
+  std::vector<Type> arg_types;
+  std::vector<Op> body;
+  int num_warps = 1;
+};
+
+struct Token {
+  enum Kind { kWord, kValue, kNumber, kPunct, kNewline, kEnd } kind;
+  std::string text;
+  int line;
+};
+
+std::vector<Token> tokenize(const char *s) {
+  std::vector<Token> out;
+  int line = 1;
+  while (*s) {
+    if (*s == '\n') { out.push_back({Token::kNewline, "\n", line++}); ++s; continue; }
+    if (isspace((unsigned char)*s)) { ++s; continue; }
+    if (s[0] == '/' && s[1] == '/') { while (*s && *s != '\n') ++s; continue; }
+    if (*s == '%' || *s == '#' || *s == '@' || *s == '!') {
+      const char *b = s++;
+      while (isalnum((unsigned char)*s) || *s == '_' || *s == '.' || *s == '#' || *s == '$') ++s;
+      out.push_back({b[0] == '%' ? Token::kValue : Token::kWord, std::string(b, s), line});
+      continue;
+    }
+    if (isalpha((unsigned char)*s) || *s == '_') {
+      const char *b = s;
+      while (isalnum((unsigned char)*s) || *s == '_' || *s == '.') ++s;
+      out.push_back({Token::kWord, std::string(b, s), line});
+      continue;
+    }
+    if (isdigit((unsigned char)*s) || ((*s == '-' || *s == '+') && isdigit((unsigned char)s[1]))) {
+      const char *b = s++;
+      while (isalnum((unsigned char)*s) || *s == '.' || ((*s == '+' || *s == '-') && (s[-1] == 'e' || s[-1] == 'E'))) ++s;
+      out.push_back({Token::kNumber, std::string(b, s), line});
+      continue;
+    }
+    if (s[0] == '-' && s[1] == '>') { out.push_back({Token::kPunct, "->", line}); s += 2; continue; }
+    out.push_back({Token::kPunct, std::string(1, *s), line});
+    ++s;
+  }
+  out.push_back({Token::kEnd, "", line});
+  return out;
+}
+
+int dtype_of(const std::string &w) {
+  if (w == "f16") return KAPY_F16;
+  if (w == "bf16") return KAPY_BF16;
+  if (w == "f32") return KAPY_F32;
+  if (w == "f8E4M3" || w == "f8E4M3FN") return KAPY_F8E4M3;
+  if (w == "f8E5M2") return KAPY_F8E5M2;
+  if (w == "i32") return KAPY_I32;
+  return -1;
+}
+
+struct Parser {
+  std::vector<Token> t;
+  size_t p = 0;
+  std::string err;
+  std::map<std::string, std::string> aliases;  // "#global" -> "global_memory"
+  const Token &peek(int k = 0) const { return t[std::min(p + k, t.size() - 1)]; }
+  bool is(const char *text) const { return peek().text == text; }
+  bool accept(const char *text) { if (is(text)) { ++p; return true; } return false; }
+  bool fail_at(const std::string &m) { if (err.empty()) err = "line " + std::to_string(peek().line) + ": " + m; return false; }
+  void skip_newlines() { while (peek().kind == Token::kNewline) ++p; }
+
+  // tensor<64x?xf16, #values> | i32 | i1 | f16 | !kapy.ptr<1>
+  bool parse_type(Type &ty) {
+    const Token &k = peek();
+    if (k.text == "tensor") {
+      ++p;
+      if (!accept("<")) return fail_at("expected '<' after tensor");
+      ty.kind = Type::kTensor;
+      // the dims and the element type arrive as "64x64xf16", "?", "x", "?xf16" word / number / punct tokens
+      std::string dims;
+      while (!is(",") && !is(">") && peek().kind != Token::kEnd) dims += t[p++].text;
+      size_t pos = 0;
+      int nd = 0;
+      while (pos < dims.size()) {
+        size_t x = dims.find('x', pos);
+        std::string part = dims.substr(pos, x == std::string::npos ? std::string::npos : x - pos);
+        if (x == std::string::npos || dtype_of(dims.substr(pos)) >= 0) { ty.dtype = dtype_of(dims.substr(pos)); break; }
+        if (nd < 2) ty.shape[nd++] = part == "?" ? -1 : atoll(part.c_str());
+        pos = x + 1;
+      }
+      if (ty.dtype < 0) return fail_at("unsupported tensor element type in '" + dims + "'");
+      if (accept(",")) {
+        std::string enc = t[p++].text;  // #alias
+        if (is("<")) { int depth = 0; do { if (is("<")) ++depth; if (is(">")) --depth; enc += t[p++].text; } while (depth > 0); }
+        auto it = aliases.find(enc);
+        const std::string &full = it == aliases.end() ? enc : it->second;
+        ty.space = full.find("global") != std::string::npos ? "global" : full.find("shared") != std::string::npos ? "shared" : "values";
+      }
+      if (!accept(">")) return fail_at("expected '>' closing tensor type");
+      return true;
+    }
+    if (k.text == "!kapy.ptr") {
+      ++p;
+      if (accept("<")) { while (!is(">") && peek().kind != Token::kEnd) ++p; accept(">"); }
+      ty.kind = Type::kPtr;
+      return true;
+    }
+    if (k.text == "i32" || k.text == "i1" || k.text == "i64" || k.text == "index") { ++p; ty.kind = Type::kInt; ty.dtype = KAPY_I32; return true; }
+    if (dtype_of(k.text) >= 0) { ++p; ty.kind = Type::kFloat; ty.dtype = dtype_of(k.text); return true; }
+    return fail_at("unknown type '" + k.text + "'");
+  }
+
+  // {a = 1 : i32, b = true}
+  bool parse_attr_dict(std::map<std::string, std::string> &attrs) {
+    while (!is("}") && peek().kind != Token::kEnd) {
+      std::string key = t[p++].text;
+      std::string val = "true";
+      if (accept("=")) {
+        val = t[p++].text;
+        if (accept(":")) { Type ty; if (!parse_type(ty)) return false; }
+      }
+      attrs[key] = val;
+      accept(",");
+    }
+    return accept("}") || fail_at("unterminated attribute dictionary");
+  }
+
+  bool parse_region(std::vector<Op> &body) {
+    for (;;) {
+      skip_newlines();
+      if (accept("}")) return true;
+      if (peek().kind == Token::kEnd) return fail_at("unterminated region");
+      Op op;
+      if (!parse_op(op)) return false;
+      body.push_back(std::move(op));
+    }
+  }
+
+  bool parse_op(Op &op) {
+    op.line = peek().line;
+    // results
+    if (peek().kind == Token::kValue) {
+      for (;;) {
+        std::string r = t[p++].text;
+        if (accept(":")) {
+          int n = atoi(t[p++].text.c_str());
+          for (int i = 0; i < n; ++i) op.results.push_back(r + "#" + std::to_string(i));
+        } else op.results.push_back(r);
+        if (!accept(",")) break;
+      }
+      if (!accept("=")) return fail_at("expected '=' after results");
+    }
+    if (peek().kind != Token::kWord) return fail_at("expected an operation name");
+    op.name = t[p++].text;
+    if (op.name == "scf.for") {
+      // %iv = %lo to %hi step %st iter_args(%a = %init, ...) -> (types) : i32 { region }
+      op.region_args.push_back(t[p++].text);
+      if (!accept("=")) return fail_at("scf.for: expected '='");
+      op.operands.push_back(t[p++].text);
+      if (!accept("to")) return fail_at("scf.for: expected 'to'");
+      op.operands.push_back(t[p++].text);
+      if (!accept("step")) return fail_at("scf.for: expected 'step'");
+      op.operands.push_back(t[p++].text);
+      if (accept("iter_args")) {
+        if (!accept("(")) return fail_at("scf.for: expected '('");
+        while (!is(")")) {
+          op.region_args.push_back(t[p++].text);
+          if (!accept("=")) return fail_at("scf.for: expected '=' in iter_args");
+          op.operands.push_back(t[p++].text);
+          accept(",");
+        }
+        accept(")");
+        if (accept("->")) {
+          if (accept("(")) { while (!is(")")) { Type ty; if (!parse_type(ty)) return false; op.types.push_back(ty); accept(","); } accept(")"); }
+          else { Type ty; if (!parse_type(ty)) return false; op.types.push_back(ty); }
+        }
+      }
+      if (accept(":")) { Type ty; if (!parse_type(ty)) return false; }
+      if (!accept("{")) return fail_at("scf.for: expected '{'");
+      return parse_region(op.body);
+    }
+    // operand section: up to the top-level ':' or the end of the line
+    int depth = 0;
+    while (peek().kind != Token::kEnd) {
+      const Token &k = peek();
+      if (k.kind == Token::kNewline && depth == 0) break;
+      if (k.text == ":" && depth == 0) break;
+      if (k.text == "{") {
+        ++p;
+        if (peek().kind == Token::kNewline) {  // a region (kapy.reduce lambda)
+          if (!parse_region(op.body)) return false;
+        } else if (!parse_attr_dict(op.attrs)) return false;
+        continue;
+      }
+      if (k.text == "lambda") {  // lambda(%a: f16, %b: f16)
+        ++p;
+        accept("(");
+        while (!is(")") && peek().kind != Token::kEnd) {
+          op.region_args.push_back(t[p++].text);
+          if (accept(":")) { Type ty; if (!parse_type(ty)) return false; }
+          accept(",");
+        }
+        accept(")");
+        continue;
+      }
+      if (k.text == "dense") {  // dense<0.000000e+00>
+        ++p;
+        accept("<");
+        op.words.push_back(t[p++].text);
+        accept(">");
+        continue;
+      }
+      if (k.text == "(" || k.text == "[") ++depth;
+      if (k.text == ")" || k.text == "]") --depth;
+      if (k.kind == Token::kValue) op.operands.push_back(k.text);
+      else if (k.kind == Token::kWord || k.kind == Token::kNumber) op.words.push_back(k.text);
+      ++p;
+    }
+    if (accept(":")) {
+      while (peek().kind != Token::kNewline && peek().kind != Token::kEnd) {
+        if (accept(",") || accept("->") || accept("(") || accept(")")) continue;
+        Type ty;
+        if (!parse_type(ty)) return false;
+        op.types.push_back(ty);
+      }
+    }
+    return true;
+  }
+
+  bool parse_module(Func &f, const char *want) {
+    for (;;) {
+      skip_newlines();
+      const Token &k = peek();
+      if (k.kind == Token::kEnd) return fail_at(std::string("no kapy.func") + (want ? std::string(" named ") + want : std::string()) + " found");
+      if (k.kind == Token::kWord && k.text[0] == '#' && peek(1).text == "=") {  // #global = #kapy.encoding<global_memory>
+        std::string name = k.text;
+        p += 2;
+        std::string rhs;
+        while (peek().kind != Token::kNewline && peek().kind != Token::kEnd) rhs += t[p++].text;
+        aliases[name] = rhs;
+        continue;
+      }
+      if (k.text == "module") {
+        ++p;
+        if (accept("attributes")) {
+          if (!accept("{")) return fail_at("expected '{' after attributes");
+          std::map<std::string, std::string> attrs;
+          if (!parse_attr_dict(attrs)) return false;
+          if (attrs.count("kapy.num_warps")) f.num_warps = atoi(attrs["kapy.num_warps"].c_str());
+        }
+        if (!accept("{")) return fail_at("expected '{' opening the module");
+        continue;
+      }
+      if (k.text == "kapy.func") {
+        ++p;
+        accept("public");
+        accept("private");
+        std::string name = t[p++].text;  // @name
+        if (!accept("(")) return fail_at("kapy.func: expected '('");
+        Func g;
+        g.num_warps = f.num_warps;
+        g.name = name.substr(1);
+        while (!is(")") && peek().kind != Token::kEnd) {
+          g.arg_names.push_back(t[p++].text);
+          if (!accept(":")) return fail_at("kapy.func: expected ':' after an argument");
+          Type ty;
+          if (!parse_type(ty)) return false;
+          g.arg_types.push_back(ty);
+          if (accept("{")) { std::map<std::string, std::string> a; if (!parse_attr_dict(a)) return false; }
+          accept(",");
+        }
+        accept(")");
+        if (!accept("{")) return fail_at("kapy.func: expected '{'");
+        if (!parse_region(g.body)) return false;
+        if (!want || g.name == want) { f = std::move(g); return true; }
+        continue;
+      }
+      ++p;  // closing braces of the module etc.
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+struct Value {
+  enum Kind { kNone, kInt, kPtr, kTensor } kind = kNone;
+  int64_t i = 0;
+  void *ptr = nullptr;
+  int64_t bytes = 0;  // kPtr: size of the allocation behind ptr, 0 = unknown
+  kapy_global g;      // global views, shared-memory tensors and register tensors alike
+};
+
+// Shared-memory tensors take the first part of the arena and live for the whole call; register tensors
+// take the rest and die with their program instance.
+constexpr size_t kSharedArena = size_t(4) << 20, kArena = size_t(64) << 20;
+
+struct Interp {
+  const Func &f;
+  hipStream_t stream;
+  char *arena = nullptr;
+  size_t shared_top = 0, top = kSharedArena;
+  std::map<std::string, Value> env;
+  std::vector<std::pair<std::string, kapy_global>> shared;  // mk_shared results, allocated once per call
+  int64_t pid[3] = {0, 0, 0}, warp = 0;
+  std::string err;
+
+  Interp(const Func &fn, hipStream_t s) : f(fn), stream(s) {}
+  int fail_op(const Op &op, const std::string &m) {
+    if (err.empty()) err = "line " + std::to_string(op.line) + " (" + op.name + "): " + m;
+    return KAPY_ERR_INVALID;
+  }
+  void *alloc(size_t bytes, bool in_shared) {
+    size_t &at = in_shared ? shared_top : top;
+    const size_t limit = in_shared ? kSharedArena : kArena;
+    at = (at + 255) & ~size_t(255);
+    if (at + bytes > limit) return nullptr;
+    void *r = arena + at;
+    at += bytes;
+    return r;
+  }
+  bool get(const Op &op, size_t k, Value::Kind kind, Value &v) {
+    if (k >= op.operands.size()) { fail_op(op, "missing operand"); return false; }
+    auto it = env.find(op.operands[k]);
+    if (it == env.end()) { fail_op(op, "use of undefined value " + op.operands[k]); return false; }
+    if (it->second.kind != kind) { fail_op(op, "operand " + op.operands[k] + " has the wrong kind"); return false; }
+    v = it->second;
+    return true;
+  }
+  // a new row-major register tensor of the op's result type
+  bool new_tensor(const Op &op, const Type &ty, Value &v, bool in_shared = false) {
+    if (ty.kind != Type::kTensor || ty.shape[0] <= 0 || ty.shape[1] <= 0) { fail_op(op, "result must be a statically shaped tensor"); return false; }
+    void *ptr = alloc((size_t)ty.shape[0] * ty.shape[1] * dtype_bytes(ty.dtype), in_shared);
+    if (!ptr) { fail_op(op, in_shared ? "shared-memory tensors exceed 4 MiB" : "register tensors of one program instance exceed 60 MiB"); return false; }
+    v.kind = Value::kTensor;
+    if (kapy_mk_global(&v.g, ptr, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 256) != KAPY_OK) {
+      fail_op(op, kapy_last_error());
+      return false;
+    }
+    return true;
+  }
+  int lib(const Op &op, int rc) { return rc == KAPY_OK ? KAPY_OK : (fail_op(op, kapy_last_error()), rc); }
+
+  int binary_tensor(const Op &op, int ew) {
+    Value a, b, r;
+    if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
+    kapy_ew_inst prog[4] = {{KAPY_EW_LD_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f}, {KAPY_EW_LD_GLOBAL, 1, 1, 0, 0, 0, KAPY_RN, 0.f},
+                            {ew, 2, 0, 1, 0, 0, KAPY_RN, 0.f}, {KAPY_EW_ST_GLOBAL, 0, 2, 0, 0, 0, KAPY_RN, 0.f}};
+    const kapy_global *ins[2] = {&a.g, &b.g};
+    int rc = lib(op, kapy_elementwise(prog, 4, ins, 2, &r.g, stream));
+    if (rc == KAPY_OK) env[op.results[0]] = r;
+    return rc;
+  }
+
+  int run_ops(const std::vector<Op> &ops, std::vector<Value> *yielded) {
+    for (const Op &op : ops) {
+      int rc = run_op(op, yielded);
+      if (rc != KAPY_OK) return rc;
+    }
+    return KAPY_OK;
+  }
+
+  int run_op(const Op &op, std::vector<Value> *yielded) {
+    const std::string &n = op.name;
+    Value a, b, c, r;
+    if (n == "kapy.return") return KAPY_OK;
+    if (n == "scf.yield") {
+      if (!yielded) return fail_op(op, "yield outside a loop");
+      yielded->clear();
+      for (size_t k = 0; k < op.operands.size(); ++k) {
+        auto it = env.find(op.operands[k]);
+        if (it == env.end()) return fail_op(op, "use of undefined value " + op.operands[k]);
+        yielded->push_back(it->second);
+      }
+      return KAPY_OK;
+    }
+    if (n == "arith.constant") {
+      if (op.types.empty()) return fail_op(op, "constant without a type");
+      const Type &ty = op.types.back();
+      if (ty.kind == Type::kInt) {
+        r.kind = Value::kInt;
+        const std::string &w = op.words.empty() ? std::string("0") : op.words[0];
+        r.i = w == "true" ? 1 : w == "false" ? 0 : atoll(w.c_str());
+      } else if (ty.kind == Type::kTensor) {
+        if (!new_tensor(op, ty, r)) return KAPY_ERR_INVALID;
+        const float v = op.words.empty() ? 0.f : (float)atof(op.words[0].c_str());
+        kapy_ew_inst prog[2] = {{KAPY_EW_SPLAT, 0, 0, 0, 0, ty.dtype, KAPY_RN, v}, {KAPY_EW_ST_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f}};
+        int rc = lib(op, kapy_elementwise(prog, 2, nullptr, 0, &r.g, stream));
+        if (rc) return rc;
+      } else return fail_op(op, "unsupported constant type");
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.program_id") {
+      r.kind = Value::kInt;
+      int axis = op.attrs.count("axis") ? atoi(op.attrs.at("axis").c_str()) : 0;
+      if (axis < 0 || axis > 2) return fail_op(op, "axis must be 0, 1 or 2");
+      r.i = pid[axis];
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.warp_id") { r.kind = Value::kInt; r.i = warp; env[op.results[0]] = r; return KAPY_OK; }
+    if (n == "arith.addi" || n == "arith.subi" || n == "arith.muli" || n == "arith.divui" || n == "arith.remui" || n == "arith.cmpi") {
+      if (!get(op, 0, Value::kInt, a) || !get(op, 1, Value::kInt, b)) return KAPY_ERR_INVALID;
+      r.kind = Value::kInt;
+      const uint32_t ua = (uint32_t)a.i, ub = (uint32_t)b.i;
+      if (n == "arith.addi") r.i = (int32_t)(ua + ub);
+      else if (n == "arith.subi") r.i = (int32_t)(ua - ub);
+      else if (n == "arith.muli") r.i = (int32_t)(ua * ub);
+      else if (n == "arith.cmpi") {
+        const std::string &pr = op.words.empty() ? std::string("eq") : op.words[0];
+        const int32_t sa = (int32_t)a.i, sb = (int32_t)b.i;
+        r.i = pr == "eq" ? sa == sb : pr == "ne" ? sa != sb : pr == "slt" ? sa < sb : pr == "sle" ? sa <= sb : pr == "sgt" ? sa > sb :
+              pr == "sge" ? sa >= sb : pr == "ult" ? ua < ub : pr == "ule" ? ua <= ub : pr == "ugt" ? ua > ub : ua >= ub;
+      } else {
+        if (ub == 0) return fail_op(op, "division by zero");
+        r.i = n == "arith.divui" ? (int32_t)(ua / ub) : (int32_t)(ua % ub);
+      }
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "arith.select") {
+      if (!get(op, 0, Value::kInt, a)) return KAPY_ERR_INVALID;
+      auto it = env.find(op.operands[a.i ? 1 : 2]);
+      if (it == env.end()) return fail_op(op, "use of undefined value");
+      env[op.results[0]] = it->second;
+      return KAPY_OK;
+    }
+    if (n == "arith.addf") return binary_tensor(op, KAPY_EW_ADDF);
+    if (n == "arith.subf") return binary_tensor(op, KAPY_EW_SUBF);
+    if (n == "arith.mulf") return binary_tensor(op, KAPY_EW_MULF);
+    if (n == "arith.divf") return binary_tensor(op, KAPY_EW_DIVF);
+    if (n == "arith.maximumf") return binary_tensor(op, KAPY_EW_MAXIMUMF);
+    if (n == "arith.minimumf") return binary_tensor(op, KAPY_EW_MINIMUMF);
+    if (n == "kapy.mk_global") {
+      Value off, s0, s1, t0, t1;
+      if (!get(op, 0, Value::kPtr, a) || !get(op, 1, Value::kInt, off) || !get(op, 2, Value::kInt, s0) || !get(op, 3, Value::kInt, s1) ||
+          !get(op, 4, Value::kInt, t0) || !get(op, 5, Value::kInt, t1) || op.types.empty())
+        return KAPY_ERR_INVALID;
+      const int eb = dtype_bytes(op.types.back().dtype);
+      if (s0.i < 0 || s1.i < 0 || t0.i < 0 || t1.i < 0 || off.i < 0) return fail_op(op, "negative size, stride or offset");
+      if (a.bytes > 0 && s0.i > 0 && s1.i > 0 && (off.i + (s0.i - 1) * t0.i + (s1.i - 1) * t1.i + 1) * eb > a.bytes)
+        return fail_op(op, "the tensor reaches beyond the " + std::to_string(a.bytes) + " bytes of its pointer argument");
+      r.kind = Value::kTensor;
+      int rc = lib(op, kapy_mk_global(&r.g, a.ptr, (int32_t)off.i, (int32_t)s0.i, (int32_t)s1.i, (int32_t)t0.i, (int32_t)t1.i, op.types.back().dtype, 16));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.mk_shared") {
+      if (op.types.empty()) return fail_op(op, "mk_shared without a type");
+      // one allocation per mk_shared op for the whole call: shared memory belongs to the program, not the warp
+      for (auto &s : shared)
+        if (s.first == op.results[0]) { r.kind = Value::kTensor; r.g = s.second; env[op.results[0]] = r; return KAPY_OK; }
+      if (!new_tensor(op, op.types.back(), r, true)) return KAPY_ERR_INVALID;
+      shared.push_back({op.results[0], r.g});
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.sv_global" || n == "kapy.sv_shared") {
+      Value s0, e0, s1, e1;
+      if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kInt, s0) || !get(op, 2, Value::kInt, e0) || !get(op, 3, Value::kInt, s1) ||
+          !get(op, 4, Value::kInt, e1))
+        return KAPY_ERR_INVALID;
+      // the reference leaves a view that leaves its parent to the load's mask; here it is an error, so that
+      // no access of the program can leave the memory the caller named
+      if (s0.i < 0 || s1.i < 0 || e0.i < s0.i || e1.i < s1.i || a.g.start0 + e0.i > a.g.end0 || a.g.start1 + e1.i > a.g.end1)
+        return fail_op(op, "the sub-view leaves its parent");
+      r.kind = Value::kTensor;
+      int rc = lib(op, kapy_sv_global(&r.g, &a.g, (int32_t)s0.i, (int32_t)e0.i, (int32_t)s1.i, (int32_t)e1.i));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.ld_global" || n == "kapy.ld_matrix" || n == "kapy.ld_shared") {
+      if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
+      int rc = lib(op, kapy_copy(&a.g, &r.g, nullptr, stream));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.st_global" || n == "kapy.st_shared" || n == "kapy.cp_async_global_to_shared") {
+      if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
+      return lib(op, kapy_copy(&a.g, &b.g, nullptr, stream));
+    }
+    if (n == "kapy.cp_async_wait_group") return KAPY_OK;  // every copy is complete in stream order
+    if (n == "kapy.matmul") {
+      if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b) || !get(op, 2, Value::kTensor, c) || op.types.empty() ||
+          !new_tensor(op, op.types.back(), r))
+        return KAPY_ERR_INVALID;
+      kapy_matmul_cfg cfg;
+      memset(&cfg, 0, sizeof cfg);
+      cfg.rmode = KAPY_RN;
+      const std::string &way = op.words.empty() ? std::string() : op.words[0];
+      cfg.impl_way = way == "mma_m16n8k8_f16" ? KAPY_MMA_M16N8K8_F16 : way == "mma_m16n8k16_f16" ? KAPY_MMA_M16N8K16_F16 :
+                     way == "mma_m16n8k16_f8" ? KAPY_MMA_M16N8K16_F8 : way == "mma_m16n8k8_tf32" ? KAPY_MMA_M16N8K8_TF32 : KAPY_MATMUL_AUTO;
+      int rc = lib(op, kapy_matmul(&a.g, &b.g, &c.g, &r.g, &cfg, stream));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.reduce") {
+      if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
+      int kind = -1;
+      for (const Op &inner : op.body) {
+        if (inner.name == "arith.addf") kind = 0;
+        if (inner.name == "arith.maximumf") kind = 1;
+      }
+      if (kind < 0) return fail_op(op, "only addf and maximumf combiners are supported");
+      int axis = op.attrs.count("axis") ? atoi(op.attrs.at("axis").c_str()) : 0;
+      int rc = lib(op, kapy_reduce(&a.g, &r.g, axis, kind, stream));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "scf.for") {
+      Value lo, hi, st;
+      if (!get(op, 0, Value::kInt, lo) || !get(op, 1, Value::kInt, hi) || !get(op, 2, Value::kInt, st)) return KAPY_ERR_INVALID;
+      if (st.i <= 0) return fail_op(op, "step must be positive");
+      const size_t n_iter = op.region_args.size() - 1;
+      std::vector<Value> carried(n_iter);
+      for (size_t k = 0; k < n_iter; ++k) {
+        auto it = env.find(op.operands[3 + k]);
+        if (it == env.end()) return fail_op(op, "use of undefined value " + op.operands[3 + k]);
+        carried[k] = it->second;
+      }
+      for (int64_t iv = lo.i; iv < hi.i; iv += st.i) {
+        Value ivv;
+        ivv.kind = Value::kInt;
+        ivv.i = iv;
+        env[op.region_args[0]] = ivv;
+        for (size_t k = 0; k < n_iter; ++k) env[op.region_args[1 + k]] = carried[k];
+        std::vector<Value> y;
+        int rc = run_ops(op.body, &y);
+        if (rc) return rc;
+        if (y.size() != n_iter) return fail_op(op, "scf.yield does not match iter_args");
+        carried = y;
+      }
+      for (size_t k = 0; k < n_iter && k < op.results.size(); ++k) env[op.results[k]] = carried[k];
+      return KAPY_OK;
+    }
+    return fail_op(op, "operation is not supported by this front-end");
+  }
+};
+
+const char *const kSupportedOps[] = {
+    "kapy.return", "scf.yield", "scf.for", "arith.constant", "kapy.program_id", "kapy.warp_id", "arith.addi", "arith.subi", "arith.muli",
+    "arith.divui", "arith.remui", "arith.cmpi", "arith.select", "arith.addf", "arith.subf", "arith.mulf", "arith.divf", "arith.maximumf",
+    "arith.minimumf", "kapy.mk_global", "kapy.mk_shared", "kapy.sv_global", "kapy.sv_shared", "kapy.ld_global", "kapy.ld_matrix",
+    "kapy.ld_shared", "kapy.st_global", "kapy.st_shared", "kapy.cp_async_global_to_shared", "kapy.cp_async_wait_group", "kapy.matmul",
+    "kapy.reduce"};
+
+// Every op must be one this front-end executes; returns the number of ops, regions included, or -1.
+int count_ops(const std::vector<Op> &ops, bool in_reduce, std::string &err) {
+  int n = 0;
+  for (const Op &op : ops) {
+    bool known = false;
+    for (const char *k : kSupportedOps) known |= op.name == k;
+    if (!known) {
+      err = "line " + std::to_string(op.line) + ": operation '" + op.name + "' is not supported by this front-end";
+      return -1;
+    }
+    ++n;
+    if (!op.body.empty() && !in_reduce) {
+      int inner = count_ops(op.body, op.name == "kapy.reduce", err);
+      if (inner < 0) return -1;
+      n += inner;
+    }
+  }
+  return n;
+}
+
+}  // namespace
+}  // namespace kapy
+
+using namespace kapy;
+
+extern "C" int kapy_parse_mlir(const char *mlir_text, const char *func_name, int32_t *n_args, int32_t *n_ops, int32_t *num_warps) {
+  if (!mlir_text) return fail(KAPY_ERR_INVALID, "parse_mlir: null text");
+  Parser ps;
+  ps.t = tokenize(mlir_text);
+  Func f;
+  if (!ps.parse_module(f, func_name)) return fail(KAPY_ERR_INVALID, "parse_mlir: %s", ps.err.c_str());
+  std::string err;
+  int n = count_ops(f.body, false, err);
+  if (n < 0) return fail(KAPY_ERR_UNSUPPORTED, "parse_mlir: %s", err.c_str());
+  if (n_args) *n_args = (int32_t)f.arg_names.size();
+  if (n_ops) *n_ops = n;
+  if (num_warps) *num_warps = f.num_warps;
+  return KAPY_OK;
+}
+
+extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_arg *args, int32_t n_args, const int32_t grid[3],
+                             void *stream) {
+  if (!mlir_text || (n_args > 0 && !args) || !grid) return fail(KAPY_ERR_INVALID, "run_mlir: null argument");
+  Parser ps;
+  ps.t = tokenize(mlir_text);
+  Func f;
+  if (!ps.parse_module(f, func_name)) return fail(KAPY_ERR_INVALID, "run_mlir: %s", ps.err.c_str());
+  {
+    std::string err;
+    if (count_ops(f.body, false, err) < 0) return fail(KAPY_ERR_UNSUPPORTED, "run_mlir: %s", err.c_str());
+  }
+  if ((int)f.arg_names.size() != n_args)
+    return fail(KAPY_ERR_INVALID, "run_mlir: @%s takes %d arguments, %d given", f.name.c_str(), (int)f.arg_names.size(), n_args);
+  for (int k = 0; k < 3; ++k)
+    if (grid[k] <= 0) return fail(KAPY_ERR_INVALID, "run_mlir: grid extents must be positive");
+  int rc = ensure_device();
+  if (rc) return rc;
+  Interp in(f, (hipStream_t)stream);
+  KAPY_HIP_CHECK(hipMalloc((void **)&in.arena, kArena));
+  rc = KAPY_OK;
+  for (int32_t p2 = 0; p2 < grid[2] && rc == KAPY_OK; ++p2)
+    for (int32_t p1 = 0; p1 < grid[1] && rc == KAPY_OK; ++p1)
+      for (int32_t p0 = 0; p0 < grid[0] && rc == KAPY_OK; ++p0)
+        for (int w = 0; w < f.num_warps && rc == KAPY_OK; ++w) {
+          in.pid[0] = p0; in.pid[1] = p1; in.pid[2] = p2;
+          in.warp = w;
+          in.env.clear();
+          in.top = kSharedArena;  // register tensors of the previous instance are dead; shared tensors stay
+          for (int k = 0; k < n_args; ++k) {
+            Value v;
+            if (f.arg_types[k].kind == Type::kPtr) {
+              if (!args[k].ptr) { rc = KAPY_ERR_INVALID; in.err = "pointer argument " + std::to_string(k) + " is null"; break; }
+              v.kind = Value::kPtr; v.ptr = args[k].ptr; v.bytes = args[k].bytes;
+            }
+            else { v.kind = Value::kInt; v.i = args[k].i32; }
+            in.env[f.arg_names[k]] = v;
+          }
+          if (rc == KAPY_OK) rc = in.run_ops(f.body, nullptr);
+        }
+  // the arena is freed after the work on the stream has finished
+  hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+  (void)hipFree(in.arena);
+  if (rc != KAPY_OK) return fail(rc, "run_mlir: %s", in.err.c_str());
+  if (e != hipSuccess) return fail(KAPY_ERR_HIP, "run_mlir: %s", hipGetErrorString(e));
+  return KAPY_OK;
+}

@@ -30,7 +30,7 @@ EXPORTS = [
     "kapy_fragments_default", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
     "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
-    "kapy_change", "kapy_reduce",
+    "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
 ]
 
 
@@ -87,6 +87,10 @@ class MatmulCfg(C.Structure):
                 ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("reserved", C.c_int32)]
 
 
+class MlirArg(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("bytes", C.c_int64), ("i32", C.c_int32), ("reserved", C.c_int32)]
+
+
 _lib = None
 
 
@@ -131,6 +135,8 @@ def lib():
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
+    L.kapy_run_mlir.argtypes = [C.c_char_p, C.c_char_p, P(MlirArg), i32, i32 * 3, vp]
+    L.kapy_parse_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i32), P(i32), P(i32)]
     for name in EXPORTS:
         f = getattr(L, name)
         if name not in ("kapy_last_error", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
@@ -248,6 +254,30 @@ def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, stream=None):
 
 def reduce(src, dst, axis, kind=0, stream=None):
     check(lib().kapy_reduce(C.byref(src), C.byref(dst), axis, kind, stream if stream is not None else current_stream()))
+
+
+def parse_mlir(text, func_name=None):
+    """(n_args, n_ops, num_warps) of a kapy.func in textual form; raises KapyError when it does not parse."""
+    n_args, n_ops, warps = C.c_int32(), C.c_int32(), C.c_int32()
+    check(lib().kapy_parse_mlir(text.encode(), func_name.encode() if func_name else None, C.byref(n_args), C.byref(n_ops),
+                                C.byref(warps)))
+    return n_args.value, n_ops.value, warps.value
+
+
+def run_mlir(text, args, grid, func_name=None, stream=None):
+    """Executes a kapy.func given as text.  args: an int for an i32 argument; a (device pointer, bytes) pair or
+    anything with data_ptr()/numel()/element_size() for a !kapy.ptr<1> argument.  grid: 1 to 3 extents."""
+    arr = (MlirArg * max(len(args), 1))()
+    for k, a in enumerate(args):
+        if isinstance(a, int):
+            arr[k].i32 = a
+        elif isinstance(a, tuple):
+            arr[k].ptr, arr[k].bytes = a
+        else:
+            arr[k].ptr, arr[k].bytes = a.data_ptr(), a.numel() * a.element_size()
+    g = list(grid) + [1] * (3 - len(grid))
+    check(lib().kapy_run_mlir(text.encode(), func_name.encode() if func_name else None, arr, len(args), (C.c_int32 * 3)(*g),
+                              stream if stream is not None else current_stream()))
 
 
 def change(in_ptr, src, dst, shape, out_ptr, stream=None):

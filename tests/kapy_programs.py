@@ -1,0 +1,154 @@
+"""Kapy-dialect programs in textual form, written for these tests in the op syntax of the reference's
+fixtures (test/Conversion/KapyToKgpu/{elementwise_add,reduce_sum,matmul}.mlir; Ops.td): the same ops and
+the same program structure (per-warp sub-views, a shared-memory double buffer filled with
+cp_async_global_to_shared, ld_matrix fragments, an scf.for carrying the accumulator, arith.select choosing
+the buffer), with shapes and tilings of their own."""
+
+HEADER = """#global = #kapy.encoding<global_memory>
+#shared = #kapy.encoding<shared_memory>
+#values = #kapy.encoding<register_file>
+"""
+
+
+def _consts(values):
+    return "".join("    %%c%d_i32 = arith.constant %d : i32\n" % (v, v) for v in sorted(set(values)))
+
+
+def binary_program(op="arith.addf", rows_per_warp=4, cols=128, num_warps=4, dtype="f16"):
+    """out[r, :] = x[r, :] <op> y[r, :]; a program covers num_warps*rows_per_warp rows of `cols` columns."""
+    t = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols])
+    body += """    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %gy = kapy.mk_global %y[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %sy = kapy.sv_global %gy[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %vx = kapy.ld_global %sx : {t}, #global> -> {t}, #values>
+    %vy = kapy.ld_global %sy : {t}, #global> -> {t}, #values>
+    %vo = {op} %vx, %vy : {t}, #values>
+    kapy.st_global %vo, %so : {t}, #values>, {t}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, t=t, op=op)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @binary_kernel(%x: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %y: !kapy.ptr<1> {kapy.alignment = 128 : i64}, "
+            "%out: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %rows: i32 {kapy.alignment = 4 : i64}) {\n" + body + "  }\n}\n")
+
+
+def reduce_program(combiner="arith.addf", rows_per_warp=2, cols=512, num_warps=2, dtype="f16"):
+    """out[r] = reduce over the columns of x[r, :]; out is a column vector stored with stride (1, rows)."""
+    src = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype)
+    dst = "tensor<%dx1x%s" % (rows_per_warp, dtype)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols])
+    body += """    %0 = kapy.mk_global %arg0[%c0_i32] [%arg2, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %1 = kapy.program_id {{axis = 0 : i32}} : i32
+    %2 = kapy.warp_id : i32
+    %3 = arith.muli %1, %c{rpp}_i32 : i32
+    %4 = arith.muli %2, %c{rpw}_i32 : i32
+    %5 = arith.addi %3, %4 : i32
+    %6 = arith.addi %5, %c{rpw}_i32 : i32
+    %7 = kapy.sv_global %0[%5 : %6, %c0_i32 : %c{cols}_i32] : {dyn} -> {src}, #global>
+    %8 = kapy.ld_global %7 : {src}, #global> -> {src}, #values>
+    %9 = kapy.reduce %8 {{axis = 1 : i32}} lambda(%lhs: {dtype}, %rhs: {dtype}) {{
+      %12 = {comb} %lhs, %rhs : {dtype}
+      kapy.return %12 : {dtype}
+    }} : {src}, #values> -> {dst}, #values>
+    %10 = kapy.mk_global %arg1[%c0_i32] [%arg2, %c1_i32] [%c1_i32, %arg2] : !kapy.ptr<1> -> {dyn}
+    %11 = kapy.sv_global %10[%5 : %6, %c0_i32 : %c1_i32] : {dyn} -> {dst}, #global>
+    kapy.st_global %9, %11 : {dst}, #values>, {dst}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, src=src, dst=dst, dtype=dtype, comb=combiner)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64, kapy.nvidia_cc = 89 : i64} {\n" % num_warps +
+            "  kapy.func public @reduce_kernel(%arg0: !kapy.ptr<1>, %arg1: !kapy.ptr<1>, %arg2: i32) {\n" + body + "  }\n}\n")
+
+
+def matmul_program(bm=64, bn=64, bk=32, way="mma_m16n8k16_f16", acc="f16", dtype="f16"):
+    """C[M,N] = A[M,K] . B[K,N], row-major.  A program owns a (2*bm)x(2*bn) tile of C, its four warps a bm x bn
+    quarter each.  K advances in steps of bk through two shared-memory buffers per operand: the loop body
+    multiplies the tile that the previous step loaded while cp_async fills the other buffer, which
+    arith.select picks by the parity of the step, and the accumulator is carried in iter_args."""
+    ga, gb, gc = ("tensor<%dx%dx%s, #global>" % s for s in ((bm, bk, dtype), (bk, bn, dtype), (bm, bn, acc)))
+    sa_full, sb_full = "tensor<%dx%dx%s, #shared>" % (2 * bm, bk, dtype), "tensor<%dx%dx%s, #shared>" % (bk, 2 * bn, dtype)
+    sa, sb = "tensor<%dx%dx%s, #shared>" % (bm, bk, dtype), "tensor<%dx%dx%s, #shared>" % (bk, bn, dtype)
+    va, vb, vc = ("tensor<%dx%dx%s, #values>" % s for s in ((bm, bk, dtype), (bk, bn, dtype), (bm, bn, acc)))
+    dyn, dync = "tensor<?x?x%s, #global>" % dtype, "tensor<?x?x%s, #global>" % acc
+    body = _consts([0, 1, 2, bm, bn, bk, 2 * bm, 2 * bn])
+    body += """    %zero = arith.constant dense<0.000000e+00> : {vc}
+    %pad_a = arith.constant dense<0.000000e+00> : {va}
+    %pad_b = arith.constant dense<0.000000e+00> : {vb}
+    %A = kapy.mk_global %a[%c0_i32] [%m, %k] [%k, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %B = kapy.mk_global %b[%c0_i32] [%k, %n] [%n, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %C = kapy.mk_global %c[%c0_i32] [%m, %n] [%n, %c1_i32] : !kapy.ptr<1> -> {dync}
+    %a_buf0 = kapy.mk_shared {{kapy.row_major = true}} : {sa_full}
+    %b_buf0 = kapy.mk_shared {{kapy.row_major = true}} : {sb_full}
+    %a_buf1 = kapy.mk_shared {{kapy.row_major = true}} : {sa_full}
+    %b_buf1 = kapy.mk_shared {{kapy.row_major = true}} : {sb_full}
+    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %tiles_n = arith.divui %n, %c{bn2}_i32 : i32
+    %tile_m = arith.divui %pid, %tiles_n : i32
+    %tile_n = arith.remui %pid, %tiles_n : i32
+    %warp_m = arith.divui %warp, %c2_i32 : i32
+    %warp_n = arith.remui %warp, %c2_i32 : i32
+    %sm0 = arith.muli %warp_m, %c{bm}_i32 : i32
+    %sm1 = arith.addi %sm0, %c{bm}_i32 : i32
+    %sn0 = arith.muli %warp_n, %c{bn}_i32 : i32
+    %sn1 = arith.addi %sn0, %c{bn}_i32 : i32
+    %tm = arith.muli %tile_m, %c{bm2}_i32 : i32
+    %tn = arith.muli %tile_n, %c{bn2}_i32 : i32
+    %row0 = arith.addi %tm, %sm0 : i32
+    %row1 = arith.addi %row0, %c{bm}_i32 : i32
+    %col0 = arith.addi %tn, %sn0 : i32
+    %col1 = arith.addi %col0, %c{bn}_i32 : i32
+    %a_sh0 = kapy.sv_shared %a_buf0[%sm0 : %sm1, %c0_i32 : %c{bk}_i32] : {sa_full} -> {sa}
+    %b_sh0 = kapy.sv_shared %b_buf0[%c0_i32 : %c{bk}_i32, %sn0 : %sn1] : {sb_full} -> {sb}
+    %a_sh1 = kapy.sv_shared %a_buf1[%sm0 : %sm1, %c0_i32 : %c{bk}_i32] : {sa_full} -> {sa}
+    %b_sh1 = kapy.sv_shared %b_buf1[%c0_i32 : %c{bk}_i32, %sn0 : %sn1] : {sb_full} -> {sb}
+    %a_g0 = kapy.sv_global %A[%row0 : %row1, %c0_i32 : %c{bk}_i32] : {dyn} -> {ga}
+    %b_g0 = kapy.sv_global %B[%c0_i32 : %c{bk}_i32, %col0 : %col1] : {dyn} -> {gb}
+    kapy.cp_async_global_to_shared %a_g0, %a_sh0, %pad_a : {ga}, {sa}, {va}
+    kapy.cp_async_global_to_shared %b_g0, %b_sh0, %pad_b : {gb}, {sb}, {vb}
+    kapy.cp_async_wait_group {{num_pending = 0 : i32}}
+    %steps = arith.divui %k, %c{bk}_i32 : i32
+    %loop:2 = scf.for %step = %c1_i32 to %steps step %c1_i32 iter_args(%acc = %zero, %unused = %c0_i32) -> ({vc}, i32)  : i32 {{
+      %parity = arith.remui %step, %c2_i32 : i32
+      %odd = arith.cmpi eq, %parity, %c1_i32 : i32
+      %a_cur = arith.select %odd, %a_sh0, %a_sh1 : {sa}
+      %b_cur = arith.select %odd, %b_sh0, %b_sh1 : {sb}
+      %a_nxt = arith.select %odd, %a_sh1, %a_sh0 : {sa}
+      %b_nxt = arith.select %odd, %b_sh1, %b_sh0 : {sb}
+      %k0 = arith.muli %step, %c{bk}_i32 : i32
+      %k1 = arith.addi %k0, %c{bk}_i32 : i32
+      %a_g = kapy.sv_global %A[%row0 : %row1, %k0 : %k1] : {dyn} -> {ga}
+      %b_g = kapy.sv_global %B[%k0 : %k1, %col0 : %col1] : {dyn} -> {gb}
+      kapy.cp_async_global_to_shared %a_g, %a_nxt, %pad_a : {ga}, {sa}, {va}
+      kapy.cp_async_global_to_shared %b_g, %b_nxt, %pad_b : {gb}, {sb}, {vb}
+      %a_frag = kapy.ld_matrix %a_cur, %pad_a : {sa}, {va} -> {va}
+      %b_frag = kapy.ld_matrix %b_cur, %pad_b : {sb}, {vb} -> {vb}
+      %next = kapy.matmul {way} %a_frag, %b_frag, %acc : {va}, {vb} -> {vc}
+      kapy.cp_async_wait_group {{num_pending = 0 : i32}}
+      scf.yield %next, %step : {vc}, i32
+    }}
+    %last = arith.remui %loop#1, %c2_i32 : i32
+    %last_odd = arith.cmpi eq, %last, %c1_i32 : i32
+    %a_fin = arith.select %last_odd, %a_sh1, %a_sh0 : {sa}
+    %b_fin = arith.select %last_odd, %b_sh1, %b_sh0 : {sb}
+    %a_ff = kapy.ld_matrix %a_fin, %pad_a : {sa}, {va} -> {va}
+    %b_ff = kapy.ld_matrix %b_fin, %pad_b : {sb}, {vb} -> {vb}
+    %result = kapy.matmul {way} %a_ff, %b_ff, %loop#0 : {va}, {vb} -> {vc}
+    %c_g = kapy.sv_global %C[%row0 : %row1, %col0 : %col1] : {dync} -> {gc}
+    kapy.st_global %result, %c_g : {vc}, {gc}
+    kapy.return
+""".format(bm=bm, bn=bn, bk=bk, bm2=2 * bm, bn2=2 * bn, ga=ga, gb=gb, gc=gc, sa=sa, sb=sb, sa_full=sa_full, sb_full=sb_full,
+           va=va, vb=vb, vc=vc, dyn=dyn, dync=dync, way=way)
+    return (HEADER + "module attributes {kapy.num_warps = 4 : i64, kapy.nvidia_cc = 89 : i64} {\n"
+            "  kapy.func public @matmul_kernel(%a: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %b: !kapy.ptr<1> {kapy.alignment = 128 : i64}, "
+            "%c: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %m: i32, %n: i32, %k: i32) {\n" + body + "  }\n}\n")

@@ -1,0 +1,106 @@
+"""GPU parity of the textual front-end: programs with the structure of the reference's three Kapy fixtures
+(test/Conversion/KapyToKgpu/{elementwise_add,reduce_sum,matmul}.mlir) run end to end through kapy_run_mlir
+and are compared with the oracle's elementwise, reduce and matmul on the same inputs."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+import kapy_programs as kp
+from gpu_util import dev_zeros, sync, to_dev, to_host, ulp_diff_f16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("op,ew,rows_per_warp,cols,warps,programs", [
+    ("arith.addf", "EW_ADDF", 4, 128, 4, 3),      # the fixture's x + y
+    ("arith.mulf", "EW_MULF", 2, 256, 2, 2),
+    ("arith.subf", "EW_SUBF", 8, 64, 1, 5),
+])
+def test_binary_program_is_bit_exact(ko, op, ew, rows_per_warp, cols, warps, programs):
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 11)
+    y = ko.fill_normal(rows * cols, ko.F16, 12)
+    want = np.zeros(rows * cols, np.uint16)
+    prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_LD_GLOBAL, dst=1, a=1),
+                       dict(op=getattr(ko, ew), dst=2, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=2)])
+    g = lambda a: ko.mk_global(a, rows, cols, cols, 1, ko.F16)
+    assert ko.elementwise(prog, [g(x), g(y)], g(want)) == 0
+    dx, dy, dout = to_dev(x), to_dev(y), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.binary_program(op, rows_per_warp, cols, warps), [dx, dy, dout, rows], [programs])
+    sync()
+    assert np.array_equal(to_host(dout, np.uint16), want)
+
+
+@pytest.mark.parametrize("comb,kind,rows_per_warp,cols,warps,programs", [
+    ("arith.addf", 0, 2, 256, 2, 4),               # the fixture's row sum
+    ("arith.maximumf", 1, 4, 512, 1, 3),
+])
+def test_reduce_program_matches_oracle(ko, comb, kind, rows_per_warp, cols, warps, programs):
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 21)
+    want = np.zeros(rows, np.uint16)
+    assert ko.lib().ko_reduce(C.byref(ko.mk_global(x, rows, cols, cols, 1, ko.F16)), C.byref(ko.mk_global(want, rows, 1, 1, rows, ko.F16)),
+                              1, kind) == 0
+    dx, dout = to_dev(x), dev_zeros(rows, 2, fill=0x7e00)
+    kh.run_mlir(kp.reduce_program(comb, rows_per_warp, cols, warps), [dx, dout, rows], [programs])
+    sync()
+    got = to_host(dout, np.uint16)
+    # a sum is accumulated in fp32 in an order of the kernel's own: at most 1 ulp of f16 from the oracle; a max is exact
+    assert ulp_diff_f16(got, want).max() <= (1 if kind == 0 else 0)
+
+
+def _chunked_reference(a, b, bk, acc_dtype):
+    """The program's arithmetic: per K step an fp32-accumulated product added to the carried accumulator,
+    which is rounded to acc_dtype after every step."""
+    acc = np.zeros((a.shape[0], b.shape[1]), acc_dtype)
+    for k0 in range(0, a.shape[1], bk):
+        acc = (acc.astype(np.float64) + a[:, k0:k0 + bk].astype(np.float64) @ b[k0:k0 + bk].astype(np.float64)).astype(acc_dtype)
+    return acc
+
+
+@pytest.mark.parametrize("bm,bn,bk,way,acc,M,N,K", [
+    (64, 64, 16, "mma_m16n8k8_f16", "f16", 256, 128, 128),     # the fixture's tiling: 128x128 per program, f16 accumulator
+    (64, 64, 32, "mma_m16n8k16_f16", "f32", 128, 256, 96),
+    (32, 64, 32, "mma_m16n8k16_f16", "f32", 64, 128, 32),      # one K step: the loop body never runs
+])
+def test_matmul_program_matches_oracle(ko, bm, bn, bk, way, acc, M, N, K):
+    a = ko.fill_normal(M * K, ko.F16, 31, std=0.5)
+    b = ko.fill_normal(K * N, ko.F16, 32, std=0.5)
+    da, db = to_dev(a), to_dev(b)
+    acc_np, acc_bytes = (np.float16, 2) if acc == "f16" else (np.float32, 4)
+    dc = dev_zeros(M * N, acc_bytes, fill=-1)
+    grid = (M // (2 * bm)) * (N // (2 * bn))
+    kh.run_mlir(kp.matmul_program(bm, bn, bk, way, acc), [da, db, dc, M, N, K], [grid])
+    sync()
+    got = to_host(dc, acc_np, (M, N)).astype(np.float64)
+    af, bf = a.view(np.float16).reshape(M, K), b.view(np.float16).reshape(K, N)
+    # against the oracle's whole-K matmul (fp64 reference rounded once)
+    want = np.zeros(M * N, np.uint16 if acc == "f16" else np.float32)
+    ga, gb = ko.mk_global(a, M, K, K, 1, ko.F16), ko.mk_global(b, K, N, N, 1, ko.F16)
+    assert ko.lib().ko_matmul(C.byref(ga), C.byref(gb), None, C.byref(ko.mk_global(want, M, N, N, 1, ko.F16 if acc == "f16" else ko.F32)),
+                              ko.RN) == 0
+    ref = want.view(acc_np).reshape(M, N).astype(np.float64)
+    rel = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+    assert rel <= (2e-3 if acc == "f16" else 1e-5), rel    # an f16 accumulator rounds after every K step
+    # against the program's own arithmetic (accumulator rounded per step): only fp32 summation order differs
+    step = _chunked_reference(af, bf, bk, acc_np).astype(np.float64)
+    rel = np.linalg.norm(got - step) / np.linalg.norm(step)
+    assert rel <= (3e-4 if acc == "f16" else 1e-6), rel
+
+
+def test_errors_name_the_line_and_leave_the_device_usable(ko):
+    rows, cols = 16, 128
+    x = to_dev(ko.fill_normal(rows * cols, ko.F16, 1))
+    out = dev_zeros(rows * cols, 2)
+    text = kp.binary_program()
+    with pytest.raises(kh.KapyError) as e:                 # grid of 2 programs needs 32 rows: the sub-view leaves its parent
+        kh.run_mlir(text, [x, x, out, rows], [2])
+    assert "sub-view leaves its parent" in e.value.message and "kapy.sv_global" in e.value.message
+    with pytest.raises(kh.KapyError) as e:                 # rows argument larger than the allocation
+        kh.run_mlir(text, [x, x, out, 4 * rows], [1])
+    assert "reaches beyond" in e.value.message
+    kh.run_mlir(text, [x, x, out, rows], [1])
+    sync()
+    assert np.array_equal(to_host(out, np.float16), to_host(x, np.float16) * 2)

@@ -219,6 +219,36 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
  * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`. */
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream);
 
+/* Static plan of a workgroup's shared memory (lib/Analysis/AllocAnalysis.cpp:187-270): buffers whose live
+ * ranges [live_start, live_end) (op ids) intersect get disjoint byte ranges, others may share.  Fills
+ * `offset` of every buffer (multiples of `alignment`, 0 = the reference's 128) and returns the bytes to
+ * allocate, or a negative kapy_status.  Placement rule and order are the reference's; where its loop would not
+ * end (it returns first-colour buffers to offset 0 on every pass) offsets are only allowed to grow. */
+typedef struct kapy_smem_buffer {
+  int64_t size;                  /* bytes                       */
+  int64_t live_start, live_end;  /* live over [start, end)      */
+  int64_t offset;                /* out                         */
+} kapy_smem_buffer;
+int64_t kapy_smem_plan(kapy_smem_buffer *buffers, int32_t n_buffers, int64_t alignment);
+
+/* Where a program needs workgroup barriers (lib/Analysis/BlockAnalysis.cpp:37-88 and :114-169).  `ops` are
+ * grouped by basic block in ascending block order, in program order inside a block; block 0 is the entry;
+ * successors of block b are succ[succ_begin[b] .. succ_begin[b+1]).  kind 0 = an op that reads and writes the
+ * byte ranges accesses[first_access .. +n_accesses) of shared memory, 1 = a barrier, 2 = cp_async_wait_group.
+ * On return barrier[i] has bit 0 set when a barrier is needed before op i (a read-after-write,
+ * write-after-read or write-after-write against accesses pending since the last barrier on some path) and bit 1
+ * when one is needed after it (a wait_group that no barrier follows).  Returns the number of barriers, or a
+ * negative kapy_status. */
+typedef struct kapy_smem_op {
+  int32_t block, kind, first_access, n_accesses;
+} kapy_smem_op;
+typedef struct kapy_smem_access {
+  int64_t begin, end;  /* bytes [begin, end) of the workgroup's shared memory */
+  int32_t is_write, reserved;
+} kapy_smem_access;
+int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_access *accesses, int32_t n_accesses,
+                       const int32_t *succ_begin, const int32_t *succ, int32_t n_blocks, int32_t *barrier);
+
 /* Runs a kapy.func given in the textual form of the reference's Kapy-dialect fixtures
  * (test/Conversion/KapyToKgpu/elementwise_add.mlir, reduce_sum.mlir, matmul.mlir; op syntax from
  * include/kapy/Dialect/Kapy/IR/Ops.td) on the device: every program id of `grid` and every warp id of the
@@ -245,6 +275,15 @@ int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_
  * KAPY_ERR_UNSUPPORTED for an op outside the set above; otherwise the function's argument count, its number
  * of ops (loop bodies included) and the module's kapy.num_warps.  Out pointers may be NULL. */
 int kapy_parse_mlir(const char *mlir_text, const char *func_name, int32_t *n_args, int32_t *n_ops, int32_t *num_warps);
+/* Shared-memory plan and barrier positions of a kapy.func in textual form, without a device: one buffer per
+ * kapy.mk_shared in program order, live from the first to the last op that defines or uses it or a sub-view or
+ * select of it (lib/Analysis/AllocAnalysis.cpp:86-185), placed by kapy_smem_plan with the reference's 128-byte
+ * alignment; then kapy_smem_barriers over the function's control flow with ld_matrix / ld_shared reading and
+ * cp_async_global_to_shared / st_shared writing the whole buffers their operand may alias.  barrier_lines gets
+ * +line for a barrier needed before the op on that source line and -line for one after it.  kapy_run_mlir places
+ * shared-memory tensors by this plan and refuses a program that needs more than a workgroup's 160 KiB. */
+int kapy_analyze_mlir(const char *mlir_text, const char *func_name, int64_t *smem_bytes, int32_t *n_buffers, int64_t *offsets,
+                      int32_t max_buffers, int32_t *n_barriers, int32_t *barrier_lines, int32_t max_barriers);
 
 #ifdef __cplusplus
 }

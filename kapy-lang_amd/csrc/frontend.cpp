@@ -19,7 +19,10 @@
 #include <cctype>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
+#include <climits>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -327,6 +330,177 @@ struct Parser {
 };
 
 // ---------------------------------------------------------------------------------------------
+// ---------------------------------------------------------------------------------------------
+// Shared-memory plan and barrier positions of a parsed function: buffers and their live ranges as
+// lib/Analysis/AllocAnalysis.cpp:86-185 finds them (one buffer per mk_shared in walk order; op ids in post-order,
+// so that a loop op's id is larger than its body's; a buffer is live over [first id, last id) of the ops that
+// define or use it or a value aliasing it), placed by kapy_smem_plan; then the function's structured control flow
+// unrolled into a block graph (entry, loop header, loop body, continuation) and handed to kapy_smem_barriers.
+// Unlike BlockAnalysis.cpp:145-152, which looks buffers up by the mk_shared result only, accesses through
+// sub-views and selects are attributed to every buffer they may alias.
+struct SharedBuffer {
+  std::string name;
+  int line = 0;
+  int64_t size = 0, first = INT64_MAX, last = INT64_MIN, offset = 0;
+};
+struct Analysis {
+  std::vector<SharedBuffer> buffers;
+  int64_t total = 0;
+  std::vector<int> barrier_lines;  // +line: before the op on that line, -line: after it
+};
+
+struct Analyzer {
+  const Func &f;
+  Analysis &out;
+  std::map<std::string, std::set<int>> alias;        // value -> buffers it may point into
+  std::map<std::string, std::vector<const Op *>> def_chain;  // value -> ops enclosing its definition, outermost first, then the defining op
+  std::map<const Op *, int64_t> id;
+  std::vector<kapy_smem_op> ops;
+  std::vector<int> op_line;
+  std::vector<kapy_smem_access> accesses;
+  std::vector<std::vector<int>> succ;
+  Analyzer(const Func &fn, Analysis &a) : f(fn), out(a) {}
+
+  void number(const std::vector<Op> &body) {
+    for (const Op &op : body) {
+      number(op.body);
+      id[&op] = (int64_t)id.size();
+    }
+  }
+  void define(const std::vector<Op> &body, std::vector<const Op *> &chain) {
+    for (const Op &op : body) {
+      chain.push_back(&op);
+      for (auto &r : op.results) def_chain[r] = chain;
+      for (auto &r : op.region_args) def_chain[r] = chain;  // live from the op that owns the region
+      if (op.name == "kapy.mk_shared" && !op.types.empty() && !op.results.empty()) {
+        SharedBuffer b;
+        b.name = op.results[0];
+        b.line = op.line;
+        const Type &ty = op.types.back();
+        b.size = std::max<int64_t>(ty.shape[0], 0) * std::max<int64_t>(ty.shape[1], 0) * dtype_bytes(ty.dtype);
+        alias[b.name].insert((int)out.buffers.size());
+        out.buffers.push_back(b);
+      }
+      define(op.body, chain);
+      chain.pop_back();
+    }
+  }
+  // one pass of alias propagation; returns whether anything grew
+  bool propagate(const std::vector<Op> &body, const Op *loop) {
+    bool grew = false;
+    auto flow = [&](const std::string &from, const std::string &to) {
+      auto it = alias.find(from);
+      if (it == alias.end()) return;
+      auto &dst = alias[to];
+      const size_t before = dst.size();
+      dst.insert(it->second.begin(), it->second.end());
+      grew |= dst.size() != before;
+    };
+    for (const Op &op : body) {
+      if (op.name == "kapy.sv_shared" && !op.results.empty() && !op.operands.empty()) flow(op.operands[0], op.results[0]);
+      if (op.name == "arith.select" && op.operands.size() == 3 && !op.results.empty()) { flow(op.operands[1], op.results[0]); flow(op.operands[2], op.results[0]); }
+      if (op.name == "scf.for") {
+        for (size_t k = 1; k < op.region_args.size() && 2 + k < op.operands.size(); ++k) flow(op.operands[2 + k], op.region_args[k]);
+        grew |= propagate(op.body, &op);
+      }
+      if (op.name == "scf.yield" && loop)
+        for (size_t k = 0; k < op.operands.size(); ++k) {
+          if (k + 1 < loop->region_args.size()) flow(op.operands[k], loop->region_args[k + 1]);
+          if (k < loop->results.size()) flow(op.operands[k], loop->results[k]);
+        }
+    }
+    return grew;
+  }
+  void touch(const std::string &value, int64_t at) {
+    auto it = alias.find(value);
+    if (it == alias.end()) return;
+    for (int b : it->second) {
+      out.buffers[b].first = std::min(out.buffers[b].first, at);
+      out.buffers[b].last = std::max(out.buffers[b].last, at);
+    }
+  }
+  // every op that defines or uses an aliasing value extends the buffer's range; a use inside a loop of a value
+  // defined outside it counts at the loop op, whose id closes the loop's body
+  void liveness(const std::vector<Op> &body, std::vector<const Op *> &chain) {
+    for (const Op &op : body) {
+      chain.push_back(&op);
+      for (auto &r : op.results) touch(r, id[&op]);
+      for (auto &u : op.operands) {
+        auto d = def_chain.find(u);
+        if (d == def_chain.end()) continue;
+        size_t depth = d->second.size() - 1;  // nesting depth of the definition
+        if (!d->second.empty() && std::find(d->second.back()->region_args.begin(), d->second.back()->region_args.end(), u) != d->second.back()->region_args.end())
+          depth += 1;                          // a region argument lives inside the region
+        const Op *at = depth < chain.size() ? chain[depth] : &op;
+        touch(u, id[at]);
+      }
+      liveness(op.body, chain);
+      chain.pop_back();
+    }
+  }
+  int new_block() { succ.emplace_back(); return (int)succ.size() - 1; }
+  void add_access(const std::string &value, bool is_write) {
+    auto it = alias.find(value);
+    if (it == alias.end()) return;
+    for (int b : it->second) accesses.push_back({out.buffers[b].offset, out.buffers[b].offset + out.buffers[b].size, is_write ? 1 : 0, 0});
+  }
+  int blocks_of(const std::vector<Op> &body, int cur) {
+    for (const Op &op : body) {
+      if (op.name == "scf.for") {
+        const int header = new_block(), first = new_block();
+        succ[cur].push_back(header);
+        succ[header].push_back(first);
+        const int last = blocks_of(op.body, first);
+        succ[last].push_back(header);
+        const int cont = new_block();
+        succ[header].push_back(cont);
+        cur = cont;
+        continue;
+      }
+      kapy_smem_op so{cur, 0, (int32_t)accesses.size(), 0};
+      if (op.name == "nvvm.barrier0") so.kind = 1;
+      else if (op.name == "kapy.cp_async_wait_group") so.kind = 2;
+      else if ((op.name == "kapy.ld_matrix" || op.name == "kapy.ld_shared") && !op.operands.empty()) add_access(op.operands[0], false);
+      else if ((op.name == "kapy.cp_async_global_to_shared" || op.name == "kapy.st_shared") && op.operands.size() > 1) add_access(op.operands[1], true);
+      so.n_accesses = (int32_t)accesses.size() - so.first_access;
+      ops.push_back(so);
+      op_line.push_back(op.line);
+    }
+    return cur;
+  }
+  int run(std::string &err) {
+    std::vector<const Op *> chain;
+    number(f.body);
+    define(f.body, chain);
+    while (propagate(f.body, nullptr)) {}
+    liveness(f.body, chain);
+    std::vector<kapy_smem_buffer> plan(out.buffers.size());
+    for (size_t k = 0; k < plan.size(); ++k) {
+      const SharedBuffer &b = out.buffers[k];
+      plan[k] = {b.size, b.first, std::max(b.first, b.last), 0};  // [first id, last id): AllocAnalysis.cpp:150-160
+    }
+    out.total = kapy_smem_plan(plan.data(), (int32_t)plan.size(), 128);
+    if (out.total < 0) { err = kapy_last_error(); return (int)out.total; }
+    for (size_t k = 0; k < plan.size(); ++k) out.buffers[k].offset = plan[k].offset;
+    new_block();
+    blocks_of(f.body, 0);
+    std::vector<int32_t> succ_begin{0}, flat;
+    for (auto &s : succ) { flat.insert(flat.end(), s.begin(), s.end()); succ_begin.push_back((int32_t)flat.size()); }
+    std::vector<int32_t> flags(ops.size() + 1, 0);
+    int n = kapy_smem_barriers(ops.data(), (int32_t)ops.size(), accesses.data(), (int32_t)accesses.size(), succ_begin.data(), flat.data(),
+                               (int32_t)succ.size(), flags.data());
+    if (n < 0) { err = kapy_last_error(); return n; }
+    for (size_t k = 0; k < ops.size(); ++k) {
+      if (flags[k] & 1) out.barrier_lines.push_back(op_line[k]);
+      if (flags[k] & 2) out.barrier_lines.push_back(-op_line[k]);
+    }
+    return KAPY_OK;
+  }
+};
+
+// Bytes of LDS one gfx950 workgroup can have.
+constexpr int64_t kLdsBytes = 160 * 1024;
+
 struct Value {
   enum Kind { kNone, kInt, kPtr, kTensor } kind = kNone;
   int64_t i = 0;
@@ -337,15 +511,15 @@ struct Value {
 
 // Shared-memory tensors take the first part of the arena and live for the whole call; register tensors
 // take the rest and die with their program instance.
-constexpr size_t kSharedArena = size_t(4) << 20, kArena = size_t(64) << 20;
+constexpr size_t kSharedArena = size_t(256) << 10, kArena = size_t(64) << 20;
 
 struct Interp {
   const Func &f;
   hipStream_t stream;
   char *arena = nullptr;
-  size_t shared_top = 0, top = kSharedArena;
+  size_t top = kSharedArena;
   std::map<std::string, Value> env;
-  std::vector<std::pair<std::string, kapy_global>> shared;  // mk_shared results, allocated once per call
+  const Analysis *plan = nullptr;  // where each mk_shared lives inside the shared part of the arena
   int64_t pid[3] = {0, 0, 0}, warp = 0;
   std::string err;
 
@@ -354,13 +528,11 @@ struct Interp {
     if (err.empty()) err = "line " + std::to_string(op.line) + " (" + op.name + "): " + m;
     return KAPY_ERR_INVALID;
   }
-  void *alloc(size_t bytes, bool in_shared) {
-    size_t &at = in_shared ? shared_top : top;
-    const size_t limit = in_shared ? kSharedArena : kArena;
-    at = (at + 255) & ~size_t(255);
-    if (at + bytes > limit) return nullptr;
-    void *r = arena + at;
-    at += bytes;
+  void *alloc(size_t bytes) {
+    top = (top + 255) & ~size_t(255);
+    if (top + bytes > kArena) return nullptr;
+    void *r = arena + top;
+    top += bytes;
     return r;
   }
   bool get(const Op &op, size_t k, Value::Kind kind, Value &v) {
@@ -372,16 +544,31 @@ struct Interp {
     return true;
   }
   // a new row-major register tensor of the op's result type
-  bool new_tensor(const Op &op, const Type &ty, Value &v, bool in_shared = false) {
+  bool new_tensor(const Op &op, const Type &ty, Value &v) {
     if (ty.kind != Type::kTensor || ty.shape[0] <= 0 || ty.shape[1] <= 0) { fail_op(op, "result must be a statically shaped tensor"); return false; }
-    void *ptr = alloc((size_t)ty.shape[0] * ty.shape[1] * dtype_bytes(ty.dtype), in_shared);
-    if (!ptr) { fail_op(op, in_shared ? "shared-memory tensors exceed 4 MiB" : "register tensors of one program instance exceed 60 MiB"); return false; }
+    void *ptr = alloc((size_t)ty.shape[0] * ty.shape[1] * dtype_bytes(ty.dtype));
+    if (!ptr) { fail_op(op, "register tensors of one program instance exceed the arena"); return false; }
     v.kind = Value::kTensor;
     if (kapy_mk_global(&v.g, ptr, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 256) != KAPY_OK) {
       fail_op(op, kapy_last_error());
       return false;
     }
     return true;
+  }
+  // a shared-memory tensor sits at its planned offset in the shared part of the arena, the same for every
+  // program and warp
+  int mk_shared(const Op &op) {
+    const Type &ty = op.types.back();
+    for (const SharedBuffer &b : plan->buffers) {
+      if (b.name != op.results[0] || b.line != op.line) continue;
+      Value r;
+      r.kind = Value::kTensor;
+      if (ty.kind != Type::kTensor || ty.shape[0] <= 0 || ty.shape[1] <= 0) return fail_op(op, "result must be a statically shaped tensor");
+      int rc = lib(op, kapy_mk_global(&r.g, arena + b.offset, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 128));
+      if (rc == KAPY_OK) env[op.results[0]] = r;
+      return rc;
+    }
+    return fail_op(op, "no shared-memory plan for this tensor");
   }
   int lib(const Op &op, int rc) { return rc == KAPY_OK ? KAPY_OK : (fail_op(op, kapy_last_error()), rc); }
 
@@ -493,13 +680,7 @@ struct Interp {
     }
     if (n == "kapy.mk_shared") {
       if (op.types.empty()) return fail_op(op, "mk_shared without a type");
-      // one allocation per mk_shared op for the whole call: shared memory belongs to the program, not the warp
-      for (auto &s : shared)
-        if (s.first == op.results[0]) { r.kind = Value::kTensor; r.g = s.second; env[op.results[0]] = r; return KAPY_OK; }
-      if (!new_tensor(op, op.types.back(), r, true)) return KAPY_ERR_INVALID;
-      shared.push_back({op.results[0], r.g});
-      env[op.results[0]] = r;
-      return KAPY_OK;
+      return mk_shared(op);
     }
     if (n == "kapy.sv_global" || n == "kapy.sv_shared") {
       Value s0, e0, s1, e1;
@@ -527,7 +708,7 @@ struct Interp {
       if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
       return lib(op, kapy_copy(&a.g, &b.g, nullptr, stream));
     }
-    if (n == "kapy.cp_async_wait_group") return KAPY_OK;  // every copy is complete in stream order
+    if (n == "kapy.cp_async_wait_group" || n == "nvvm.barrier0") return KAPY_OK;  // every op is complete in stream order
     if (n == "kapy.matmul") {
       if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b) || !get(op, 2, Value::kTensor, c) || op.types.empty() ||
           !new_tensor(op, op.types.back(), r))
@@ -592,7 +773,7 @@ const char *const kSupportedOps[] = {
     "arith.divui", "arith.remui", "arith.cmpi", "arith.select", "arith.addf", "arith.subf", "arith.mulf", "arith.divf", "arith.maximumf",
     "arith.minimumf", "kapy.mk_global", "kapy.mk_shared", "kapy.sv_global", "kapy.sv_shared", "kapy.ld_global", "kapy.ld_matrix",
     "kapy.ld_shared", "kapy.st_global", "kapy.st_shared", "kapy.cp_async_global_to_shared", "kapy.cp_async_wait_group", "kapy.matmul",
-    "kapy.reduce"};
+    "kapy.reduce", "nvvm.barrier0"};
 
 // Every op must be one this front-end executes; returns the number of ops, regions included, or -1.
 int count_ops(const std::vector<Op> &ops, bool in_reduce, std::string &err) {
@@ -634,6 +815,26 @@ extern "C" int kapy_parse_mlir(const char *mlir_text, const char *func_name, int
   return KAPY_OK;
 }
 
+extern "C" int kapy_analyze_mlir(const char *mlir_text, const char *func_name, int64_t *smem_bytes, int32_t *n_buffers, int64_t *offsets,
+                                 int32_t max_buffers, int32_t *n_barriers, int32_t *barrier_lines, int32_t max_barriers) {
+  if (!mlir_text) return fail(KAPY_ERR_INVALID, "analyze_mlir: null text");
+  Parser ps;
+  ps.t = tokenize(mlir_text);
+  Func f;
+  if (!ps.parse_module(f, func_name)) return fail(KAPY_ERR_INVALID, "analyze_mlir: %s", ps.err.c_str());
+  std::string err;
+  if (count_ops(f.body, false, err) < 0) return fail(KAPY_ERR_UNSUPPORTED, "analyze_mlir: %s", err.c_str());
+  Analysis a;
+  int rc = Analyzer(f, a).run(err);
+  if (rc) return fail(rc, "analyze_mlir: %s", err.c_str());
+  if (smem_bytes) *smem_bytes = a.total;
+  if (n_buffers) *n_buffers = (int32_t)a.buffers.size();
+  for (int k = 0; offsets && k < max_buffers && k < (int)a.buffers.size(); ++k) offsets[k] = a.buffers[k].offset;
+  if (n_barriers) *n_barriers = (int32_t)a.barrier_lines.size();
+  for (int k = 0; barrier_lines && k < max_barriers && k < (int)a.barrier_lines.size(); ++k) barrier_lines[k] = a.barrier_lines[k];
+  return KAPY_OK;
+}
+
 extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_arg *args, int32_t n_args, const int32_t grid[3],
                              void *stream) {
   if (!mlir_text || (n_args > 0 && !args) || !grid) return fail(KAPY_ERR_INVALID, "run_mlir: null argument");
@@ -645,6 +846,15 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
     std::string err;
     if (count_ops(f.body, false, err) < 0) return fail(KAPY_ERR_UNSUPPORTED, "run_mlir: %s", err.c_str());
   }
+  Analysis plan;
+  {
+    std::string err;
+    int arc = Analyzer(f, plan).run(err);
+    if (arc) return fail(arc, "run_mlir: %s", err.c_str());
+    if (plan.total > kLdsBytes)
+      return fail(KAPY_ERR_UNSUPPORTED, "run_mlir: the program needs %lld bytes of shared memory, a gfx950 workgroup has %lld", (long long)plan.total,
+                  (long long)kLdsBytes);
+  }
   if ((int)f.arg_names.size() != n_args)
     return fail(KAPY_ERR_INVALID, "run_mlir: @%s takes %d arguments, %d given", f.name.c_str(), (int)f.arg_names.size(), n_args);
   for (int k = 0; k < 3; ++k)
@@ -652,6 +862,7 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   int rc = ensure_device();
   if (rc) return rc;
   Interp in(f, (hipStream_t)stream);
+  in.plan = &plan;
   KAPY_HIP_CHECK(hipMalloc((void **)&in.arena, kArena));
   rc = KAPY_OK;
   for (int32_t p2 = 0; p2 < grid[2] && rc == KAPY_OK; ++p2)

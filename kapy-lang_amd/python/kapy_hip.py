@@ -31,6 +31,7 @@ EXPORTS = [
     "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
     "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
+    "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
 ]
 
 
@@ -87,6 +88,18 @@ class MatmulCfg(C.Structure):
                 ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("reserved", C.c_int32)]
 
 
+class SmemBuffer(C.Structure):
+    _fields_ = [("size", C.c_int64), ("live_start", C.c_int64), ("live_end", C.c_int64), ("offset", C.c_int64)]
+
+
+class SmemOp(C.Structure):
+    _fields_ = [("block", C.c_int32), ("kind", C.c_int32), ("first_access", C.c_int32), ("n_accesses", C.c_int32)]
+
+
+class SmemAccess(C.Structure):
+    _fields_ = [("begin", C.c_int64), ("end", C.c_int64), ("is_write", C.c_int32), ("reserved", C.c_int32)]
+
+
 class MlirArg(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("bytes", C.c_int64), ("i32", C.c_int32), ("reserved", C.c_int32)]
 
@@ -135,11 +148,15 @@ def lib():
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
+    L.kapy_smem_plan.restype = i64
+    L.kapy_smem_plan.argtypes = [P(SmemBuffer), i32, i64]
+    L.kapy_smem_barriers.argtypes = [P(SmemOp), i32, P(SmemAccess), i32, P(i32), P(i32), i32, P(i32)]
+    L.kapy_analyze_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i64), P(i32), P(i64), i32, P(i32), P(i32), i32]
     L.kapy_run_mlir.argtypes = [C.c_char_p, C.c_char_p, P(MlirArg), i32, i32 * 3, vp]
     L.kapy_parse_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i32), P(i32), P(i32)]
     for name in EXPORTS:
         f = getattr(L, name)
-        if name not in ("kapy_last_error", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
+        if name not in ("kapy_last_error", "kapy_smem_plan", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
             f.restype = C.c_int
     _lib = L
     return L
@@ -262,6 +279,15 @@ def parse_mlir(text, func_name=None):
     check(lib().kapy_parse_mlir(text.encode(), func_name.encode() if func_name else None, C.byref(n_args), C.byref(n_ops),
                                 C.byref(warps)))
     return n_args.value, n_ops.value, warps.value
+
+
+def analyze_mlir(text, func_name=None):
+    """(shared-memory bytes, offsets of the mk_shared buffers, barrier lines: +line before, -line after)."""
+    total, nb, nbar = C.c_int64(), C.c_int32(), C.c_int32()
+    offsets, lines = (C.c_int64 * 64)(), (C.c_int32 * 256)()
+    check(lib().kapy_analyze_mlir(text.encode(), func_name.encode() if func_name else None, C.byref(total), C.byref(nb), offsets, 64,
+                                  C.byref(nbar), lines, 256))
+    return total.value, list(offsets[:min(nb.value, 64)]), list(lines[:min(nbar.value, 256)])
 
 
 def run_mlir(text, args, grid, func_name=None, stream=None):

@@ -152,3 +152,31 @@ def matmul_program(bm=64, bn=64, bk=32, way="mma_m16n8k16_f16", acc="f16", dtype
     return (HEADER + "module attributes {kapy.num_warps = 4 : i64, kapy.nvidia_cc = 89 : i64} {\n"
             "  kapy.func public @matmul_kernel(%a: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %b: !kapy.ptr<1> {kapy.alignment = 128 : i64}, "
             "%c: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %m: i32, %n: i32, %k: i32) {\n" + body + "  }\n}\n")
+
+
+def phases_program():
+    """p[64,64] <- 2*p through shared memory in two phases: a buffer filled by cp_async and read by ld_matrix, then,
+    once that one is dead, two more buffers (one of them only read) written by st_shared and read by ld_shared."""
+    return HEADER + """module attributes {kapy.num_warps = 1 : i64} {
+  kapy.func public @phases(%p: !kapy.ptr<1>) {
+    %c0_i32 = arith.constant 0 : i32
+    %c1_i32 = arith.constant 1 : i32
+    %c64_i32 = arith.constant 64 : i32
+    %pad = arith.constant dense<0.000000e+00> : tensor<64x64xf16, #values>
+    %g = kapy.mk_global %p[%c0_i32] [%c64_i32, %c64_i32] [%c64_i32, %c1_i32] : !kapy.ptr<1> -> tensor<?x?xf16, #global>
+    %gs = kapy.sv_global %g[%c0_i32 : %c64_i32, %c0_i32 : %c64_i32] : tensor<?x?xf16, #global> -> tensor<64x64xf16, #global>
+    %first = kapy.mk_shared {kapy.row_major = true} : tensor<64x64xf16, #shared>
+    kapy.cp_async_global_to_shared %gs, %first, %pad : tensor<64x64xf16, #global>, tensor<64x64xf16, #shared>, tensor<64x64xf16, #values>
+    kapy.cp_async_wait_group {num_pending = 0 : i32}
+    %v = kapy.ld_matrix %first, %pad : tensor<64x64xf16, #shared>, tensor<64x64xf16, #values> -> tensor<64x64xf16, #values>
+    %w = arith.addf %v, %v : tensor<64x64xf16, #values>
+    %second = kapy.mk_shared {kapy.row_major = true} : tensor<64x32xf16, #shared>
+    %third = kapy.mk_shared {kapy.row_major = true} : tensor<64x64xf16, #shared>
+    kapy.st_shared %w, %third : tensor<64x64xf16, #values>, tensor<64x64xf16, #shared>
+    %u = kapy.ld_shared %third : tensor<64x64xf16, #shared> -> tensor<64x64xf16, #values>
+    %x = kapy.ld_shared %second : tensor<64x32xf16, #shared> -> tensor<64x32xf16, #values>
+    kapy.st_global %u, %gs : tensor<64x64xf16, #values>, tensor<64x64xf16, #global>
+    kapy.return
+  }
+}
+"""

@@ -61,3 +61,59 @@ REFERENCE_FIXTURES = "/root/reference/test/Conversion/KapyToKgpu"
 def test_reference_fixtures_parse_unchanged(name, n_args, n_ops, warps):
     text = open("%s/%s.mlir" % (REFERENCE_FIXTURES, name)).read()
     assert kh.parse_mlir(text, name + "_kernel") == (n_args, n_ops, warps)
+
+
+def _lines(text, needle):
+    return [k + 1 for k, line in enumerate(text.split("\n")) if needle in line]
+
+
+def test_analysis_of_programs_without_shared_memory_is_empty():
+    assert kh.analyze_mlir(kp.binary_program()) == (0, [], [])
+    assert kh.analyze_mlir(kp.reduce_program()) == (0, [], [])
+
+
+def test_analysis_places_the_double_buffers_and_finds_the_barriers():
+    text = kp.matmul_program(64, 64, 32)
+    total, offsets, barriers = kh.analyze_mlir(text)
+    # four buffers of 128x32 f16, all live from their mk_shared to the last ld_matrix: end to end
+    assert (total, offsets) == (4 * 8192, [0, 8192, 16384, 24576])
+    waits = _lines(text, "kapy.cp_async_wait_group")
+    # every wait_group gets a barrier after it; inside the loop the first ld_matrix reads through a select that may
+    # point at the buffer the cp_async just before it is filling, so it needs one before it
+    first_ld_in_loop = [l for l in _lines(text, "kapy.ld_matrix") if l > _lines(text, "scf.for")[0]][0]
+    assert sorted(barriers) == sorted([-w for w in waits] + [first_ld_in_loop])
+
+
+def test_analysis_shares_memory_between_buffers_that_are_never_live_together():
+    # two phases, each with a buffer of its own: the second buffer is made after the last use of the first
+    text = kp.phases_program()
+    total, offsets, barriers = kh.analyze_mlir(text)
+    # %first is dead when %second and %third are made: they start at 0 again; %second and %third live together
+    assert offsets == [0, 0, 4096] and total == 4096 + 8192
+    # the wait_group's own barrier; st_shared into %third writes bytes that ld_matrix has read as %first (the reuse
+    # is a write after read); ld_shared of %third after the st_shared is a read after write
+    assert sorted(barriers) == sorted([-_lines(text, "cp_async_wait_group")[0], _lines(text, "kapy.st_shared")[0],
+                                       _lines(text, "%u = kapy.ld_shared")[0]])
+
+
+@pytest.mark.skipif(not __import__("os").path.isdir(REFERENCE_FIXTURES), reason="the reference tree is not present")
+def test_analysis_of_the_reference_matmul_fixture():
+    text = open(REFERENCE_FIXTURES + "/matmul.mlir").read()
+    total, offsets, barriers = kh.analyze_mlir(text)
+    assert (total, offsets) == (65536, [0, 16384, 32768, 49152])          # four 128x64 f16 tiles
+    waits = _lines(text, "kapy.cp_async_wait_group")
+    loop = _lines(text, "scf.for")[0]
+    refill = [l for l in _lines(text, "kapy.cp_async_global_to_shared") if l > loop][0]
+    # a barrier after each wait_group, and one before the loop's refill of the buffer that ld_matrix has just read
+    assert sorted(barriers) == sorted([-w for w in waits] + [refill])
+
+
+def test_a_program_beyond_the_lds_is_refused_before_anything_runs():
+    import ctypes as C
+    text = kp.matmul_program(64, 64, 32).replace("tensor<128x32xf16, #shared>", "tensor<128x256xf16, #shared>") \
+        .replace("tensor<32x128xf16, #shared>", "tensor<256x128xf16, #shared>")
+    total, _, _ = kh.analyze_mlir(text)
+    assert total == 4 * 65536
+    args = (kh.MlirArg * 6)()
+    assert kh.lib().kapy_run_mlir(text.encode(), None, args, 6, (C.c_int32 * 3)(1, 1, 1), None) == -3
+    assert "shared memory" in kh.last_error() and "163840" in kh.last_error()

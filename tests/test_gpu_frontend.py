@@ -90,6 +90,14 @@ def test_matmul_program_matches_oracle(ko, bm, bn, bk, way, acc, M, N, K):
     assert rel <= (3e-4 if acc == "f16" else 1e-6), rel
 
 
+def test_buffers_that_share_planned_memory_do_not_disturb_each_other(ko):
+    x = ko.fill_normal(64 * 64, ko.F16, 41)
+    d = to_dev(x)
+    kh.run_mlir(kp.phases_program(), [d], [1])
+    sync()
+    assert np.array_equal(to_host(d, np.float16), x.view(np.float16) * np.float16(2))
+
+
 def test_errors_name_the_line_and_leave_the_device_usable(ko):
     rows, cols = 16, 128
     x = to_dev(ko.fill_normal(rows * cols, ko.F16, 1))

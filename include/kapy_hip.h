@@ -158,7 +158,10 @@ int kapy_copy_batched(const kapy_global *src, const kapy_global *dst, const kapy
  * create_fptofp, create_splat, create_broadcast, python/src/ir.cc:744-1157; lowering
  * ElementwiseOpToLLVM.cpp:424-1238).  A register has a dtype; arithmetic on f16/bf16/f32 registers
  * rounds once to that dtype after every op.  LD_GLOBAL of an input whose extent is 1 along an axis
- * broadcasts along it (kapy.broadcast, Kapy.cpp:686-698). */
+ * broadcasts along it (kapy.broadcast, Kapy.cpp:686-698).  A program with a REDUCE is a row-wise fusion (softmax,
+ * layer norm ...): it runs in one pass over HBM with each row resident on chip, and needs axis 1, rows that are
+ * contiguous, a multiple of 8 and at most 32768 elements long, zero padding, and operands that are full, row,
+ * column or scalar views (KAPY_ERR_UNSUPPORTED otherwise). */
 typedef enum kapy_ew_op {
   KAPY_EW_LD_GLOBAL = 0, /* dst <- ins[a]            (c = kapy_padding_option)                  */
   KAPY_EW_SPLAT,         /* dst <- imm as `dtype`    (kapy.splat)                               */
@@ -170,6 +173,9 @@ typedef enum kapy_ew_op {
   KAPY_EW_TANH, KAPY_EW_ERF, /* the extern-lib calls of create_elementwise_extern_lib, ir.cc:1168-1174 */
   KAPY_EW_GELU_TANH,     /* dst <- 0.5*a*(1+tanh(sqrt(2/pi)*(a+0.044715*a^3))), one rounding       */
   KAPY_EW_ST_GLOBAL,     /* out <- a                                                              */
+  KAPY_EW_REDUCE_SUM,    /* dst <- sum of a along axis b, kept on every element of that axis: kapy.reduce  */
+  KAPY_EW_REDUCE_MAX,    /*        with an addf / maximumf combiner followed by kapy.broadcast; accumulated */
+                         /*        in fp32, rounded once to the register's type (as kapy_reduce)           */
   KAPY_EW_NUM_OPS
 } kapy_ew_op;
 typedef struct kapy_ew_inst {

@@ -22,7 +22,7 @@ DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, F8E4M3: 1, F8E5M2: 1, I8: 1, I16: 2, I32
 
 (EW_LD_GLOBAL, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
  EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH,
- EW_ST_GLOBAL) = range(22)
+ EW_ST_GLOBAL, EW_REDUCE_SUM, EW_REDUCE_MAX) = range(24)
 
 EXPORTS = [
     "kapy_version", "kapy_last_error", "kapy_device_info", "kapy_mk_global", "kapy_sv_global",
@@ -246,6 +246,68 @@ def gelu_program(out_dtype=F16, scale=0.5):
         dict(op=EW_FPTOFP, dst=5, a=2, dtype=out_dtype, rmode=RN),
         dict(op=EW_ST_GLOBAL, a=5),
     ])
+
+
+def softmax_insts(dtype=F16):
+    """Row softmax in fp32: y = exp(x - max_row(x)) / sum_row(exp(x - max_row(x))), one rounding to `dtype`."""
+    return [
+        dict(op=EW_LD_GLOBAL, dst=0, a=0),
+        dict(op=EW_FPTOFP, dst=1, a=0, dtype=F32),
+        dict(op=EW_REDUCE_MAX, dst=2, a=1, b=1),
+        dict(op=EW_SUBF, dst=1, a=1, b=2),
+        dict(op=EW_EXP, dst=1, a=1),
+        dict(op=EW_REDUCE_SUM, dst=2, a=1, b=1),
+        dict(op=EW_DIVF, dst=1, a=1, b=2),
+        dict(op=EW_FPTOFP, dst=3, a=1, dtype=dtype, rmode=RN),
+        dict(op=EW_ST_GLOBAL, a=3),
+    ]
+
+
+def layernorm_insts(n, dtype=F16, eps=1e-5, affine=True):
+    """Row layer norm in fp32 over rows of n elements: ((x - mean) * rsqrt(var + eps)) * gamma + beta with
+    gamma = ins[1], beta = ins[2] as [1 x n] rows when `affine`."""
+    prog = [
+        dict(op=EW_LD_GLOBAL, dst=0, a=0),
+        dict(op=EW_FPTOFP, dst=1, a=0, dtype=F32),
+        dict(op=EW_SPLAT, dst=2, dtype=F32, imm=1.0 / n),
+        dict(op=EW_REDUCE_SUM, dst=3, a=1, b=1),
+        dict(op=EW_MULF, dst=3, a=3, b=2),            # mean
+        dict(op=EW_SUBF, dst=1, a=1, b=3),            # centred
+        dict(op=EW_MULF, dst=4, a=1, b=1),
+        dict(op=EW_REDUCE_SUM, dst=4, a=4, b=1),
+        dict(op=EW_MULF, dst=4, a=4, b=2),            # variance
+        dict(op=EW_SPLAT, dst=5, dtype=F32, imm=eps),
+        dict(op=EW_ADDF, dst=4, a=4, b=5),
+        dict(op=EW_RSQRT, dst=4, a=4),
+        dict(op=EW_MULF, dst=1, a=1, b=4),
+    ]
+    if affine:
+        prog += [
+            dict(op=EW_LD_GLOBAL, dst=6, a=1), dict(op=EW_FPTOFP, dst=6, a=6, dtype=F32),
+            dict(op=EW_LD_GLOBAL, dst=7, a=2), dict(op=EW_FPTOFP, dst=7, a=7, dtype=F32),
+            dict(op=EW_MULF, dst=1, a=1, b=6), dict(op=EW_ADDF, dst=1, a=1, b=7),
+        ]
+    return prog + [dict(op=EW_FPTOFP, dst=8, a=1, dtype=dtype, rmode=RN), dict(op=EW_ST_GLOBAL, a=8)]
+
+
+def rmsnorm_insts(n, dtype=F16, eps=1e-6):
+    """Row RMS norm in fp32: x * rsqrt(mean(x^2) + eps) * gamma, gamma = ins[1] as a [1 x n] row."""
+    return [
+        dict(op=EW_LD_GLOBAL, dst=0, a=0),
+        dict(op=EW_FPTOFP, dst=1, a=0, dtype=F32),
+        dict(op=EW_MULF, dst=2, a=1, b=1),
+        dict(op=EW_REDUCE_SUM, dst=2, a=2, b=1),
+        dict(op=EW_SPLAT, dst=3, dtype=F32, imm=1.0 / n),
+        dict(op=EW_MULF, dst=2, a=2, b=3),
+        dict(op=EW_SPLAT, dst=3, dtype=F32, imm=eps),
+        dict(op=EW_ADDF, dst=2, a=2, b=3),
+        dict(op=EW_RSQRT, dst=2, a=2),
+        dict(op=EW_MULF, dst=1, a=1, b=2),
+        dict(op=EW_LD_GLOBAL, dst=4, a=1), dict(op=EW_FPTOFP, dst=4, a=4, dtype=F32),
+        dict(op=EW_MULF, dst=1, a=1, b=4),
+        dict(op=EW_FPTOFP, dst=5, a=1, dtype=dtype, rmode=RN),
+        dict(op=EW_ST_GLOBAL, a=5),
+    ]
 
 
 def elementwise(prog, ins, out, stream=None):

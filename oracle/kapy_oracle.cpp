@@ -583,6 +583,7 @@ int ko_copy_batched(const ko_global *src, const ko_global *dst, int transpose, i
 enum {
   EW_LD_GLOBAL = 0, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
   EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH, EW_ST_GLOBAL,
+  EW_REDUCE_SUM, EW_REDUCE_MAX,
   EW_NUM_OPS
 };
 enum { EW_MAX_REGS = 16 };
@@ -650,6 +651,11 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
       if (reg_dtype[I.a] != out->dtype) return -11;
       has_store = true;
       break;
+    case EW_REDUCE_SUM: case EW_REDUCE_MAX:
+      if (!reg_ok(I.a)) return -6;
+      if (I.b != 0 && I.b != 1) return -14;  // the axis
+      reg_dtype[I.dst] = reg_dtype[I.a];
+      break;
     default:
       if (!reg_ok(I.a)) return -6;
       reg_dtype[I.dst] = reg_dtype[I.a];
@@ -662,46 +668,77 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
   if (!has_store) return -13;
 
   const double qnan = std::numeric_limits<double>::quiet_NaN();
+  // Registers are whole tensors (o0 x o1 doubles holding exactly representable values of the register's
+  // type), instructions run one after the other over all elements: what the SSA program of whole-tensor
+  // ops means.  A reduce (kapy.reduce with an addf / maximumf combiner, Ops.td:441-457, followed by the
+  // kapy.broadcast that later uses imply) accumulates exactly (double) along its axis, rounds once to the
+  // register type and fills the axis with the result.
+  std::vector<std::vector<double>> reg(EW_MAX_REGS);
+  int rd[EW_MAX_REGS];
+  const int64_t total = o0 * o1;
+  for (int k = 0; k < n_inst; ++k) {
+    const ko_ew_inst &I = prog[k];
+    const int d = (I.op == EW_ST_GLOBAL) ? 0 : I.dst;
+    if (I.op == EW_REDUCE_SUM || I.op == EW_REDUCE_MAX) {
+      const std::vector<double> src = reg[I.a];
+      const int dt = rd[I.a];
+      reg[d].assign(total, 0.0);
+      rd[d] = dt;
+      const int64_t n_keep = I.b == 1 ? o0 : o1, n_red = I.b == 1 ? o1 : o0;
 #pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < o0; ++i) {
-    double reg[EW_MAX_REGS];
-    int rd[EW_MAX_REGS];
-    for (int64_t j = 0; j < o1; ++j) {
-      for (int k = 0; k < n_inst; ++k) {
-        const ko_ew_inst &I = prog[k];
-        double a = (I.op != EW_LD_GLOBAL && I.op != EW_SPLAT) ? reg[I.a] : 0.0;
+      for (int64_t q = 0; q < n_keep; ++q) {
+        long double acc = I.op == EW_REDUCE_SUM ? 0.0L : -std::numeric_limits<long double>::infinity();
+        bool nan = false;
+        for (int64_t r = 0; r < n_red; ++r) {
+          const double v = I.b == 1 ? src[q * o1 + r] : src[r * o1 + q];
+          if (std::isnan(v)) nan = true;
+          if (I.op == EW_REDUCE_SUM) acc += v;
+          else if (v > acc) acc = v;
+        }
+        const double res = nan ? qnan : round_to((double)acc, dt);
+        for (int64_t r = 0; r < n_red; ++r) reg[d][I.b == 1 ? q * o1 + r : r * o1 + q] = res;
+      }
+      continue;
+    }
+    std::vector<double> dstv(I.op == EW_ST_GLOBAL ? 0 : total);
+    int dst_dtype = -1;
+    if (I.op == EW_LD_GLOBAL) dst_dtype = ins[I.a]->dtype;
+    else if (I.op == EW_SPLAT || I.op == EW_FPTOFP) dst_dtype = I.dtype;
+    else if (I.op != EW_ST_GLOBAL) dst_dtype = rd[I.a];
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < o0; ++i) {
+      for (int64_t j = 0; j < o1; ++j) {
+        const int64_t at = i * o1 + j;
+        const double a = (I.op != EW_LD_GLOBAL && I.op != EW_SPLAT) ? reg[I.a][at] : 0.0;
         double r = 0.0;
-        int d = (I.op == EW_ST_GLOBAL) ? 0 : I.dst;
         switch (I.op) {
         case EW_LD_GLOBAL: {
           const ko_global *g = ins[I.a];
           int64_t gi = extent0(g) == 1 && o0 != 1 ? 0 : i, gj = extent1(g) == 1 && o1 != 1 ? 0 : j;
-          rd[d] = g->dtype;
           if (in_bounds(g, gi, gj)) r = ko_decode(g->ptr, g->dtype, elem_offset(g, gi, gj));
           else {
             uint32_t w = ko_padding_word(g->dtype, I.c);
             r = ko_decode(&w, g->dtype, 0);
           }
-          reg[d] = r;
+          dstv[at] = r;
           continue;
         }
-        case EW_SPLAT: rd[d] = I.dtype; reg[d] = round_to((double)I.imm, I.dtype); continue;
+        case EW_SPLAT: dstv[at] = round_to((double)I.imm, I.dtype); continue;
         case EW_FPTOFP: {
           bool down = dtype_bytes(I.dtype) < dtype_bytes(rd[I.a]);
           uint32_t tmp = 0;
           ko_encode(&tmp, I.dtype, 0, a, down ? I.rmode : KO_RN);
-          rd[d] = I.dtype;
-          reg[d] = ko_decode(&tmp, I.dtype, 0);
+          dstv[at] = ko_decode(&tmp, I.dtype, 0);
           continue;
         }
-        case EW_ADDF: r = a + reg[I.b]; break;
-        case EW_SUBF: r = a - reg[I.b]; break;
-        case EW_MULF: r = a * reg[I.b]; break;
-        case EW_DIVF: r = a / reg[I.b]; break;
-        case EW_FMA: r = std::fma(a, reg[I.b], reg[I.c]); break;
+        case EW_ADDF: r = a + reg[I.b][at]; break;
+        case EW_SUBF: r = a - reg[I.b][at]; break;
+        case EW_MULF: r = a * reg[I.b][at]; break;
+        case EW_DIVF: r = a / reg[I.b][at]; break;
+        case EW_FMA: r = std::fma(a, reg[I.b][at], reg[I.c][at]); break;
         // arith.maximumf / minimumf propagate NaN
-        case EW_MAXIMUMF: r = (std::isnan(a) || std::isnan(reg[I.b])) ? qnan : std::max(a, reg[I.b]); break;
-        case EW_MINIMUMF: r = (std::isnan(a) || std::isnan(reg[I.b])) ? qnan : std::min(a, reg[I.b]); break;
+        case EW_MAXIMUMF: r = (std::isnan(a) || std::isnan(reg[I.b][at])) ? qnan : std::max(a, reg[I.b][at]); break;
+        case EW_MINIMUMF: r = (std::isnan(a) || std::isnan(reg[I.b][at])) ? qnan : std::min(a, reg[I.b][at]); break;
         case EW_NEGF: r = -a; break;
         case EW_ABSF: r = std::fabs(a); break;
         case EW_EXP: r = std::exp(a); break;
@@ -717,9 +754,12 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
           if (in_bounds(out, i, j)) ko_encode(out->ptr, out->dtype, elem_offset(out, i, j), a, KO_RN);
           continue;
         }
-        rd[d] = rd[I.a];
-        reg[d] = round_to(r, rd[d]);
+        dstv[at] = round_to(r, dst_dtype);
       }
+    }
+    if (I.op != EW_ST_GLOBAL) {
+      reg[d].swap(dstv);
+      rd[d] = dst_dtype;
     }
   }
   return 0;

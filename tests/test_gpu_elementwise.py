@@ -220,3 +220,73 @@ def test_register_stack_kernel_tree_shapes_and_operand_kinds(ko):
         insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.BF16), dict(op=ST, a=1)]
         got, want = _run_prog(ko, insts, [wantq], [kh.F8E4M3], kh.BF16, m, n)
         assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Row-wise fusions: programs with a reduce along the rows run with the row resident on chip.
+def _row_case(ko, insts, dtype, m, n, seed, extra=(), std=2.0):
+    x = ko.fill_normal(m * n, dtype, seed, std=std).reshape(m, n)
+    rows = [ko.fill_normal(n, dtype, seed + 1 + k, mean=1.0 if k == 0 else 0.0, std=0.5) for k in range(len(extra))]
+    ins = [x] + rows
+    shapes = [(m, n)] + [(1, n)] * len(rows)
+    return _run_prog(ko, insts, ins, [dtype] * len(ins), dtype, m, n, in_shapes=shapes)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(7, 64), (5, 1000), (33, 4096), (9, 8192), (4, 12288), (3, 32768)])
+def test_softmax_rows_every_launch_shape(ko, dtype, m, n):
+    got, want = _row_case(ko, kh.softmax_insts(dtype), dtype, m, n, 50 + n % 97)
+    _check_ulp(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(12, 1024), (6, 8192)])
+def test_layernorm_and_rmsnorm_rows(ko, dtype, m, n):
+    got, want = _row_case(ko, kh.layernorm_insts(n, dtype), dtype, m, n, 61, extra=("gamma", "beta"))
+    _check_ulp(got, want, dtype)
+    got, want = _row_case(ko, kh.layernorm_insts(n, dtype, affine=False), dtype, m, n, 62)
+    _check_ulp(got, want, dtype)
+    got, want = _row_case(ko, kh.rmsnorm_insts(n, dtype), dtype, m, n, 63, extra=("gamma",))
+    _check_ulp(got, want, dtype)
+
+
+def test_row_program_value_read_back_from_lds_and_special_values(ko):
+    # e / sum(e) * e: when the last factor is wanted the value is no longer on the stack below and comes back from LDS
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_FPTOFP, dst=1, a=0, dtype=kh.F32),
+             dict(op=kh.EW_EXP, dst=1, a=1), dict(op=kh.EW_REDUCE_SUM, dst=2, a=1, b=1), dict(op=kh.EW_DIVF, dst=3, a=1, b=2),
+             dict(op=kh.EW_MULF, dst=3, a=3, b=1), dict(op=kh.EW_FPTOFP, dst=4, a=3, dtype=kh.F16, rmode=kh.RN),
+             dict(op=kh.EW_ST_GLOBAL, a=4)]
+    got, want = _row_case(ko, insts, kh.F16, 10, 2048, 71, std=1.0)
+    _check_ulp(got, want, kh.F16)
+    # a NaN poisons its own row only; an infinity makes the row's maximum infinite
+    m, n = 4, 512
+    x = ko.fill_normal(m * n, kh.F16, 72).reshape(m, n)
+    x[1, 100] = 0x7e00
+    x[2, 7] = 0x7c00
+    prog = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=kh.EW_ST_GLOBAL, a=1)]
+    got, want = _run_prog(ko, prog, [x], [kh.F16], kh.F16, m, n)
+    assert np.array_equal(got[[0, 2, 3]], want[[0, 2, 3]]) and np.all(got[2] == 0x7c00)
+    assert np.all(np.isnan(got[1].view(np.float16))) and np.all(np.isnan(want[1].view(np.float16)))
+
+
+def test_softmax_f32_in_and_out(ko):
+    m, n = 8, 2048
+    x = ko.fill_normal(m * n, kh.F32, 81, std=2.0).reshape(m, n)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=kh.EW_SUBF, dst=0, a=0, b=1),
+             dict(op=kh.EW_EXP, dst=0, a=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=0, b=1), dict(op=kh.EW_DIVF, dst=0, a=0, b=1),
+             dict(op=kh.EW_ST_GLOBAL, a=0)]
+    got, want = _run_prog(ko, insts, [x], [kh.F32], kh.F32, m, n)
+    g, w = got.view(np.float32).astype(np.float64), want.view(np.float32).astype(np.float64)
+    assert np.max(np.abs(g - w) / w) <= 4e-6        # fp32 exp (2 ulp) and a sum in another order
+    assert np.allclose(g.sum(axis=1), 1.0, atol=1e-5)
+
+
+def test_row_programs_outside_the_fused_kernel_are_refused(ko):
+    def run(m, n, axis=1):
+        x = to_dev(ko.fill_normal(m * n, kh.F16, 1))
+        prog = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=0, b=axis), dict(op=kh.EW_ST_GLOBAL, a=1)]
+        kh.elementwise(kh.program(prog), [dglobal(x, m, n, n, 1, kh.F16)], dglobal(dev_zeros(m * n, 2), m, n, n, 1, kh.F16))
+    for args in ((4, 64, 0), (2, 32776), (4, 100)):           # axis 0; longer than 32768; not a multiple of 8
+        with pytest.raises(kh.KapyError) as e:
+            run(*args)
+        assert e.value.status == -3 and "reduce" in e.value.message

@@ -216,3 +216,44 @@ def test_gemm_timing_baseline_agrees_with_checker(ko):
     ko.lib().ko_matmul(C.byref(ga), C.byref(gb), None, C.byref(ko.mk_global(o1, M, N, N, 1, ko.F32)), ko.RN)
     ko.lib().ko_gemm_f32acc(C.byref(ga), C.byref(gb), C.byref(ko.mk_global(o2, M, N, N, 1, ko.F32)))
     assert np.linalg.norm(o1 - o2) / np.linalg.norm(o1) < 1e-5
+
+
+def test_elementwise_reduce_ops_vs_numpy_and_scipy(ko):
+    """The reduce instructions of elementwise programs: exact sums on integer-valued inputs, exact maxima, NaN
+    propagation, axis 0 and 1, and a whole softmax against scipy in float64."""
+    import kapy_hip as kh
+    from scipy.special import softmax
+    m, n = 6, 40
+    rng = np.random.default_rng(3)
+    xi = rng.integers(-8, 9, size=(m, n)).astype(np.float32)        # sums are exact in any order
+    out = np.zeros((m, n), np.float32)
+    g = lambda a: ko.mk_global(a, m, n, n, 1, ko.F32)
+    for axis in (0, 1):
+        for op, ref in ((ko.EW_REDUCE_SUM, np.sum), (ko.EW_REDUCE_MAX, np.max)):
+            prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=op, dst=1, a=0, b=axis), dict(op=ko.EW_ST_GLOBAL, a=1)])
+            assert ko.elementwise(prog, [g(xi)], g(out)) == 0
+            assert np.array_equal(out, np.broadcast_to(ref(xi, axis=axis, keepdims=True), (m, n)))
+    xn = xi.copy()
+    xn[2, 5] = np.nan
+    prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_REDUCE_MAX, dst=0, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=0)])
+    assert ko.elementwise(prog, [g(xn)], g(out)) == 0
+    assert np.all(np.isnan(out[2])) and not np.any(np.isnan(out[[0, 1, 3, 4, 5]]))
+    # a sum in f16 registers rounds once, after exact accumulation: 2048 ones and a 1 -> 2049 is not an f16, ties to 2048
+    ones = np.ones((1, 2056), np.float16)
+    o16 = np.zeros((1, 2056), np.float16)
+    g16 = lambda a: ko.mk_global(a.view(np.uint16), 1, 2056, 2056, 1, ko.F16)
+    prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_REDUCE_SUM, dst=1, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=1)])
+    assert ko.elementwise(prog, [g16(ones)], g16(o16)) == 0
+    assert np.all(o16 == np.float16(2056))
+    # softmax: fp32 registers, result rounded to f16 once
+    x = ko.fill_normal(m * n, ko.F16, 8, std=3.0).reshape(m, n)
+    y = np.zeros((m, n), np.uint16)
+    gh = lambda a: ko.mk_global(a, m, n, n, 1, ko.F16)
+    assert ko.elementwise(ko.program(kh.softmax_insts(kh.F16)), [gh(x)], gh(y)) == 0
+    want = softmax(x.view(np.float16).astype(np.float64), axis=1)
+    err = np.abs(y.view(np.float16).astype(np.float64) - want)
+    assert np.all(err <= np.spacing(want.astype(np.float16)).astype(np.float64) * 0.51 + 1e-7 * want)   # half an f16 ulp + the fp32 steps
+    assert np.allclose(y.view(np.float16).astype(np.float64).sum(axis=1), 1.0, atol=2e-3)
+    # a reduce along an axis that does not exist is rejected
+    bad = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_REDUCE_SUM, dst=1, a=0, b=2), dict(op=ko.EW_ST_GLOBAL, a=1)])
+    assert ko.elementwise(bad, [g(xi)], g(out)) == -14

@@ -134,6 +134,27 @@ def bench_reduce(kh, steps, warmup):
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "reduce_rows_vec_kernel"}
 
 
+def bench_rowwise(kh, steps, warmup, which):
+    """Row-wise fusion of kapy.reduce with its elementwise neighbours at the headline shape: softmax or layer norm of
+    every row in one pass over HBM (one read of x, one write of y; gamma and beta stay in cache)."""
+    import torch
+    n, sets = 8192, 4
+    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    ys = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    gamma, beta = torch.ones(n, device="cuda", dtype=torch.float16), torch.zeros(n, device="cuda", dtype=torch.float16)
+    g = lambda t: kh.mk_global(t.data_ptr(), n, n, n, 1, kh.F16)
+    row = lambda t: kh.mk_global(t.data_ptr(), 1, n, n, 1, kh.F16)
+    gx, gy = [g(t) for t in xs], [g(t) for t in ys]
+    if which == "softmax":
+        prog, extra = kh.program(kh.softmax_insts(kh.F16)), []
+    else:
+        prog, extra = kh.program(kh.layernorm_insts(n, kh.F16)), [row(gamma), row(beta)]
+    wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]] + extra, gy[i % sets]), steps, warmup)
+    nbytes = 2 * n * n * 2
+    return {"workload": "%s of every row, fp16 8192x8192, fp32 arithmetic" % which, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "row_kernel"}
+
+
 def bench_transpose(kh, steps, warmup):
     import torch
     n, sets = 8192, 4
@@ -229,7 +250,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "copy", "reduce", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -247,6 +268,8 @@ def main():
         "copy": lambda s, w: bench_copy(kh, s, w),
         "transpose": lambda s, w: bench_transpose(kh, s, w),
         "reduce": lambda s, w: bench_reduce(kh, s, w),
+        "softmax": lambda s, w: bench_rowwise(kh, s, w, "softmax"),
+        "layernorm": lambda s, w: bench_rowwise(kh, s, w, "layernorm"),
         "permute": lambda s, w: bench_permute(kh, s, w),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32)),

@@ -17,15 +17,11 @@
 #include "common.hpp"
 #include <functional>
 #include "numeric.hpp"
+#include "ew_machine.hpp"
 
 namespace kapy {
 namespace {
 
-constexpr int kMaxRegs = 16;
-constexpr int kMaxInst = 48;
-constexpr int kMaxInputs = 8;
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 struct DevView {
   const char *base;  // address of view element (0,0)
@@ -43,37 +39,7 @@ struct Program {
   DevView out;
 };
 
-// 0.5*v*(1+tanh(u)) with u = sqrt(2/pi)*(v+0.044715*v^3) equals v*sigmoid(2u) = v / (1 + 2^(-2u*log2 e)):
-// no cancellation for v << 0, and only three slow-rate operations per element (exp2, rcp and
-// their operand prep).  The constants fold -2*log2(e)*sqrt(2/pi) into the cubic.
-__device__ __forceinline__ float gelu_tanh_f32(float v) {
-  constexpr float kC1 = -2.0f * 1.4426950408889634f * 0.7978845608028654f;
-  constexpr float kC3 = kC1 * 0.044715f;
-  float t = v * (kC1 + kC3 * v * v);
-  return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
-}
-
-__device__ __forceinline__ float apply_unary(int op, float a) {
-  switch (op) {
-  case KAPY_EW_NEGF: return -a;
-  case KAPY_EW_ABSF: return fabsf(a);
-  case KAPY_EW_EXP: return expf(a);
-  case KAPY_EW_EXP2: return exp2f(a);
-  case KAPY_EW_LOG: return logf(a);
-  case KAPY_EW_LOG2: return log2f(a);
-  case KAPY_EW_SQRT: return sqrtf(a);
-  case KAPY_EW_RSQRT: return 1.0f / sqrtf(a);
-  case KAPY_EW_TANH: return tanhf(a);
-  case KAPY_EW_ERF: return erff(a);
-  case KAPY_EW_GELU_TANH: return gelu_tanh_f32(a);
-  }
-  return a;
-}
-
-// arith.maximumf / minimumf: NaN if either operand is NaN.
-__device__ __forceinline__ float max_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
-__device__ __forceinline__ float min_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
-
+// (device helpers and the stack machine proper live in ew_machine.hpp)
 // ---------------------------------------------------------------------------------------------
 // Register machine: one output element per lane per pass; register r of lane t is regs[r][t], so
 // every access is conflict-free.  Values are fp32 images of the register's dtype.
@@ -132,367 +98,10 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// Stack machine: any program whose expression tree needs at most three live values, on 8
-// consecutive elements per lane in registers.  The host unfolds the SSA program into postfix form
-// (a value used twice is simply evaluated twice: every op is pure) and gives every step the stack
-// depth it works at, so the three values are three fixed register arrays chosen by a uniform branch:
-// no register is ever indexed at run time and nothing is shuffled.  Values are fp32 images of the typed value, rounded to the
-// result type after every arithmetic op exactly as the register machine does.
-constexpr int kMaxPost = 40;
-enum PostKind { kPushIn = 100, kPushImm = 101, kCast = 102, kStore = 103, kRevSub = 104, kRevDiv = 105, kSaveTmp = 106, kPushTmp = 107, kPick = 108 };
-enum InKind { kInFull = 0, kInRow = 1 /* [1 x n] */, kInCol = 2 /* [m x 1] */, kInScalar = 3 };
-struct PostOp {
-  int16_t op, a, dtype, rmode;
-  int32_t slot;  // which of the three values holds the result (and the left operand)
-  float imm;
-};
-struct StackIn {
-  const char *base;
-  int64_t stride0;
-  int32_t dtype, kind;
-};
-struct StackProgram {
-  PostOp post[kMaxPost];
-  StackIn in[kMaxInputs];
-  char *out;
-  int64_t out_stride0;
-  int32_t n_post, n_ins, out_dtype, rows, vec_per_row;
-  int32_t n_tmps;  // row machine only: values used more than once, parked in LDS
-};
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ void widen16x8(u32x4 v, int dtype, float f[8]) {
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    const uint32_t word = v[w];
-    if (dtype == KAPY_BF16) {
-      f[2 * w] = bits_f32(word << 16);
-      f[2 * w + 1] = bits_f32(word & 0xFFFF0000u);
-    } else {
-      f[2 * w] = f16_to_f32((uint16_t)word);
-      f[2 * w + 1] = f16_to_f32((uint16_t)(word >> 16));
-    }
-  }
-}
-// The 8 elements of vector jv of row i of a full-extent operand, as they lie in memory (16, 32 or 8 bytes).
-struct Raw8 {
-  u32x4 lo, hi;
-};
-__device__ __forceinline__ Raw8 fetch8(const StackIn &g, int32_t i, int32_t jv, bool streaming) {
-  const int eb = g.dtype == KAPY_F32 ? 4 : (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16) ? 2 : 1;
-  const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * eb;
-  Raw8 r;
-  r.lo = r.hi = u32x4{0, 0, 0, 0};
-  if (eb == 2) r.lo = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
-  else if (eb == 4) {
-    r.lo = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
-    r.hi = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr + 1) : *((const u32x4 *)ptr + 1);
-  } else {
-    const u32x2 v = *(const u32x2 *)ptr;
-    r.lo[0] = v[0];
-    r.lo[1] = v[1];
-  }
-  return r;
-}
-__device__ __forceinline__ void widen8(const Raw8 &r, int dtype, float f[8]) {
-  if (dtype == KAPY_F16 || dtype == KAPY_BF16) widen16x8(r.lo, dtype, f);
-  else if (dtype == KAPY_F32) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const uint32_t a = r.lo[e], b = r.hi[e];
-      f[e] = bits_f32(a);
-      f[4 + e] = bits_f32(b);
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint32_t word = r.lo[e >> 2];
-      const uint8_t byte = (uint8_t)(word >> (8 * (e & 3)));
-      f[e] = dtype == KAPY_F8E4M3 ? e4m3_to_f32(byte) : e5m2_to_f32(byte);
-    }
-  }
-}
-template <bool NARROW>
-__device__ __forceinline__ void load8(const StackIn &g, int32_t i, int32_t jv, float f[8]) {
-  if (g.kind == kInCol || g.kind == kInScalar) {
-    const float v = load_as_f32(g.base, g.dtype, g.kind == kInCol ? i * g.stride0 : 0);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = v;
-    return;
-  }
-  if (NARROW) {
-    const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * 2;
-    widen16x8(g.kind == kInFull ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr, g.dtype, f);
-  } else widen8(fetch8(g, i, jv, g.kind == kInFull), g.dtype, f);
-}
-template <bool NARROW>
-__device__ __forceinline__ void round8(float f[8], int dtype, bool rn) {
-  switch (dtype) {
-  case KAPY_F32: return;
-  case KAPY_F16:
-    if (rn) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = (float)(_Float16)f[e];
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = f16_to_f32(f32_to_f16_rz(f[e]));
-    }
-    return;
-  case KAPY_BF16:
-    if (rn) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = (float)(__bf16)f[e];
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = bf16_to_f32(f32_to_bf16_rz(f[e]));
-    }
-    return;
-  default:
-    if (!NARROW) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = round_to_dtype(f[e], dtype, rn);
-    }
-  }
-}
-template <bool NARROW>
-__device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const float f[8]) {
-  if (NARROW || dtype == KAPY_F16 || dtype == KAPY_BF16) {
-    u32x4 v;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) v[w] = dtype == KAPY_F16 ? pack2_f16_rn(f[2 * w], f[2 * w + 1]) : pack2_bf16_rn(f[2 * w], f[2 * w + 1]);
-    __builtin_nontemporal_store(v, (u32x4 *)(out + elem * 2));
-  } else if (dtype == KAPY_F32) {
-    u32x4 lo, hi;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      lo[e] = f32_bits(f[e]);
-      hi[e] = f32_bits(f[4 + e]);
-    }
-    __builtin_nontemporal_store(lo, (u32x4 *)(out + elem * 4));
-    __builtin_nontemporal_store(hi, (u32x4 *)(out + elem * 4) + 1);
-  } else {
-    u32x2 v = {0, 0};
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint32_t byte = dtype == KAPY_F8E4M3 ? f32_to_e4m3(f[e], true) : f32_to_e5m2(f[e], true);
-      v[e >> 2] |= byte << (8 * (e & 3));
-    }
-    *(u32x2 *)(out + elem) = v;
-  }
-}
-
-// One step with its result (and left operand) in value D, the right operand in value D+1 and the
-// third operand of an fma in value D+2; D is a template parameter so that no register is indexed.
-// NARROW: every operand, every intermediate type and the result are f16 / bf16 / f32-from-16-bit
-// (no fp8, no fp32 in memory): the common case, and it needs far fewer registers.
-template <int D, bool NARROW>
-__device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &I, int32_t i, int32_t jv, float (&v)[3][8]) {
-  constexpr int R = D + 1 < 3 ? D + 1 : 2, T = D + 2 < 3 ? D + 2 : 2;
-  float *x = v[D];
-  const float *y = v[R], *z = v[T];
-  switch (I.op) {
-  case kPushIn: load8<NARROW>(P.in[I.a], i, jv, x); return;
-  case kPushImm: {
-    const float c = round_to_dtype(I.imm, I.dtype, true);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = c;
-    return;
-  }
-  case kStore: store8<NARROW>(P.out, P.out_dtype, (int64_t)i * P.out_stride0 + (int64_t)jv * 8, x); return;
-  case kCast: round8<NARROW>(x, I.dtype, I.rmode != KAPY_RZ); return;
-  case KAPY_EW_ADDF:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fadd_rn(x[e], y[e]);
-    break;
-  case KAPY_EW_SUBF:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fsub_rn(x[e], y[e]);
-    break;
-  case kRevSub:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fsub_rn(y[e], x[e]);
-    break;
-  case KAPY_EW_MULF:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fmul_rn(x[e], y[e]);
-    break;
-  case KAPY_EW_DIVF:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(x[e], y[e]);
-    break;
-  case kRevDiv:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(y[e], x[e]);
-    break;
-  case KAPY_EW_MAXIMUMF:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = max_nan(x[e], y[e]);
-    break;
-  case KAPY_EW_MINIMUMF:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = min_nan(x[e], y[e]);
-    break;
-  case KAPY_EW_FMA:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fmaf_rn(x[e], y[e], z[e]);
-    break;
-  default:
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = apply_unary(I.op, x[e]);
-  }
-  if (I.dtype != KAPY_F32) round8<NARROW>(x, I.dtype, true);
-}
-
-template <bool NARROW>
-__device__ __forceinline__ void stack_run(const StackProgram &P) {
-  const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (slot >= (int64_t)P.rows * P.vec_per_row) return;
-  const int32_t i = (int32_t)(slot / P.vec_per_row), jv = (int32_t)(slot - (int64_t)i * P.vec_per_row);
-  float v[3][8];
-#pragma unroll
-  for (int d = 0; d < 3; ++d)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[d][e] = 0.f;
-  for (int pc = 0; pc < P.n_post; ++pc) {
-    const PostOp I = P.post[pc];
-    switch (I.slot) {
-    case 0: stack_step<0, NARROW>(P, I, i, jv, v); break;
-    case 1: stack_step<1, NARROW>(P, I, i, jv, v); break;
-    default: stack_step<2, NARROW>(P, I, i, jv, v);
-    }
-  }
-}
-
 // Throughput of this kernel follows the number of resident waves (each lane walks its program one
 // dependent step at a time), so the 16-bit-only form is held to 64 registers: 8 waves per SIMD.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void stack_kernel_narrow(StackProgram P) { stack_run<true>(P); }
 __global__ __launch_bounds__(256) void stack_kernel_any(StackProgram P) { stack_run<false>(P); }
-
-// ---------------------------------------------------------------------------------------------
-// Row machine: programs with a reduce along the rows (softmax, layer norm ...).  A workgroup owns
-// one row and keeps it on chip for the whole program, so HBM sees one read of every operand and one
-// write of the result.  Lane t holds CH chunks of 8 elements, chunk c at vector c*THREADS + t of the
-// row; a step of the stack machine runs on every chunk; a reduce folds the lane's chunks, then the
-// wave with a butterfly of bpermutes, then the workgroup's waves through LDS, and leaves the result
-// in every element.  Values needed more than once are parked in LDS as fp32 and read back by the
-// lane that wrote them.
-template <int KIND>
-__device__ __forceinline__ float fold(float a, float b) { return KIND == 0 ? a + b : max_nan(a, b); }
-
-template <int D, int CH, int THREADS, bool NARROW>
-__device__ __forceinline__ void row_step(const StackProgram &P, const PostOp &I, int32_t i, int pc, float (&v)[CH][3][8], float *lds) {
-  const int tid = threadIdx.x;
-  constexpr int WAVES = THREADS / 64;
-  if (I.op == KAPY_EW_REDUCE_SUM || I.op == KAPY_EW_REDUCE_MAX) {
-    const bool sum = I.op == KAPY_EW_REDUCE_SUM;
-    float acc = sum ? 0.f : -__builtin_inff();
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      if (c * THREADS + tid < P.vec_per_row) {
-        float part;
-        if (sum) part = ((v[c][D][0] + v[c][D][1]) + (v[c][D][2] + v[c][D][3])) + ((v[c][D][4] + v[c][D][5]) + (v[c][D][6] + v[c][D][7]));
-        else part = max_nan(max_nan(max_nan(v[c][D][0], v[c][D][1]), max_nan(v[c][D][2], v[c][D][3])),
-                            max_nan(max_nan(v[c][D][4], v[c][D][5]), max_nan(v[c][D][6], v[c][D][7])));
-        acc = sum ? acc + part : max_nan(acc, part);
-      }
-    }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-      const float other = __shfl_xor(acc, off, 64);
-      acc = sum ? acc + other : max_nan(acc, other);
-    }
-    if (WAVES > 1) {
-      // the exchange area alternates with the step's parity, so that a wave still reading the previous
-      // reduce's partials cannot meet the next reduce's writes: one barrier per reduce
-      float *red = lds + (pc & 1) * WAVES;
-      if ((tid & 63) == 0) red[tid >> 6] = acc;
-      __syncthreads();
-      acc = red[0];
-#pragma unroll
-      for (int w = 1; w < WAVES; ++w) acc = sum ? acc + red[w] : max_nan(acc, red[w]);
-    }
-    acc = round_to_dtype(acc, I.dtype, true);
-#pragma unroll
-    for (int c = 0; c < CH; ++c)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[c][D][e] = acc;
-    return;
-  }
-  if (I.op == kPick) {  // a copy of a value lower on the stack (I.a < D)
-    if (D > 0) {
-#pragma unroll
-      for (int c = 0; c < CH; ++c)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[c][D][e] = (D == 2 && I.a == 1) ? v[c][1][e] : v[c][0][e];
-    }
-    return;
-  }
-  float *tmps = lds + 32;
-#pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    const int32_t jv = c * THREADS + tid;
-    const bool active = jv < P.vec_per_row;
-    if (I.op == kSaveTmp || I.op == kPushTmp) {
-      float4 *slot = (float4 *)(tmps + ((int64_t)I.a * P.vec_per_row + jv) * 8);
-      if (active) {
-        if (I.op == kSaveTmp) {
-          slot[0] = float4{v[c][D][0], v[c][D][1], v[c][D][2], v[c][D][3]};
-          slot[1] = float4{v[c][D][4], v[c][D][5], v[c][D][6], v[c][D][7]};
-        } else {
-          const float4 lo = slot[0], hi = slot[1];
-          v[c][D][0] = lo.x; v[c][D][1] = lo.y; v[c][D][2] = lo.z; v[c][D][3] = lo.w;
-          v[c][D][4] = hi.x; v[c][D][5] = hi.y; v[c][D][6] = hi.z; v[c][D][7] = hi.w;
-        }
-      }
-    } else if (I.op == kPushIn || I.op == kStore) {
-      if (active) stack_step<D, NARROW>(P, I, i, jv, v[c]);
-    } else stack_step<D, NARROW>(P, I, i, jv, v[c]);
-  }
-}
-
-template <int CH, int THREADS, bool NARROW>
-__global__ __launch_bounds__(THREADS) void row_kernel(StackProgram P) {
-  extern __shared__ float row_lds[];
-  const int32_t i = blockIdx.x;
-  float v[CH][3][8];
-#pragma unroll
-  for (int c = 0; c < CH; ++c)
-#pragma unroll
-    for (int d = 0; d < 3; ++d)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[c][d][e] = 0.f;
-  for (int pc = 0; pc < P.n_post; ++pc) {
-    const PostOp I = P.post[pc];
-    switch (I.slot) {
-    case 0: row_step<0, CH, THREADS, NARROW>(P, I, i, pc, v, row_lds); break;
-    case 1: row_step<1, CH, THREADS, NARROW>(P, I, i, pc, v, row_lds); break;
-    default: row_step<2, CH, THREADS, NARROW>(P, I, i, pc, v, row_lds);
-    }
-  }
-}
-
-template <bool NARROW>
-int launch_row_kernel(const StackProgram &P, hipStream_t s) {
-  const int vpr = P.vec_per_row;
-  // few chunks per lane keep the three values of the stack within 64 to 128 registers; long rows take 1024 lanes
-  const int threads = vpr <= 64 ? 64 : vpr <= 512 ? 256 : 1024;
-  const int ch = (vpr + threads - 1) / threads;
-  const size_t lds = (32 + (size_t)P.n_tmps * vpr * 8) * sizeof(float);  // 32 floats: the reduce exchange of up to 16 waves, twice
-  if (lds > 160 * 1024) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: the program keeps %d row values of %d elements alive, more than fits the LDS", P.n_tmps, vpr * 8);
-  dim3 grid((unsigned)P.rows);
-#define KAPY_ROW(CH_, TH_)                                                                                         \
-  do {                                                                                                             \
-    if (lds > 48 * 1024) KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)row_kernel<CH_, TH_, NARROW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-    row_kernel<CH_, TH_, NARROW><<<grid, TH_, lds, s>>>(P);                                                        \
-  } while (0)
-  if (threads == 64) KAPY_ROW(1, 64);
-  else if (threads == 256) { if (ch == 1) KAPY_ROW(1, 256); else KAPY_ROW(2, 256); }
-  else { if (ch == 1) KAPY_ROW(1, 1024); else if (ch == 2) KAPY_ROW(2, 1024); else KAPY_ROW(4, 1024); }
-#undef KAPY_ROW
-  KAPY_HIP_CHECK(hipGetLastError());
-  return KAPY_OK;
-}
 
 // ---------------------------------------------------------------------------------------------
 // out[i,j] = cast_out( act( f32(x[i,j]) * scale + f32(bias) ) ), x/out contiguous along j.
@@ -866,7 +475,7 @@ bool prog_padding_nonzero(const kapy_ew_inst *prog, int n_inst, int input) {
 // (a tree deeper than three values, more than kMaxPost steps after unfolding shared values,
 // operands that are not full / row / column / scalar views readable 8 at a time, padding).
 bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins,
-                         const kapy_global *out, StackProgram *P, bool row_mode = false) {
+                         const kapy_global *out, StackProgram *P) {
   struct N {
     int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
     float imm = 0.f;
@@ -895,19 +504,13 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     reg[I.dst] = (int)nodes.size() - 1;
   }
   if (n_store != 1 || stored < 0) return false;
-  // a reduce needs the row machine, and there only along the rows
   for (const N &n : nodes)
-    if (n.op == KAPY_EW_REDUCE_SUM || n.op == KAPY_EW_REDUCE_MAX)
-      if (!row_mode) return false;
-  if (row_mode)
-    for (int k = 0; k < n_inst; ++k)
-      if ((prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX) && prog[k].b != 1) return false;
+    if (n.op == KAPY_EW_REDUCE_SUM || n.op == KAPY_EW_REDUCE_MAX) return false;  // the row machine's business
   // the result: rows contiguous, 8 elements at a time
   const int64_t o0 = extent0(out), o1 = extent1(out);
   const int ob = dtype_bytes(out->dtype);
   if (!is_float(out->dtype) || out->stride1 != 1 || o1 % 8 != 0 || ((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
   if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
-  if (row_mode && o1 / 8 > 4096) return false;
   for (int k = 0; k < n_ins; ++k) {
     const kapy_global *g = ins[k];
     StackIn &in = P->in[k];
@@ -934,63 +537,14 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     else need[id] = need[n.a];
   }
   if (need[stored] > 3) return false;
-  // row machine: a value with several uses is computed once.  A later use that finds the value still on the
-  // stack below it copies it from there (kPick); one that does not reads it back from LDS, where the first
-  // evaluation parked it.  A first run of the emission finds out which values are ever read back.
-  std::vector<int> uses(nodes.size(), 0), tmp_of(nodes.size(), -1);
-  std::vector<char> parked(nodes.size(), 0), read_back(nodes.size(), 0);
-  int n_tmps = 0;
-  if (row_mode) {
-    std::vector<char> reached(nodes.size(), 0);
-    std::function<void(int)> visit = [&](int id) {
-      ++uses[id];
-      if (reached[id]) return;
-      reached[id] = 1;
-      const N &n = nodes[id];
-      if (n.a >= 0) visit(n.a);
-      if (n.b >= 0) visit(n.b);
-      if (n.c >= 0) visit(n.c);
-    };
-    visit(stored);
-  }
   int count = 0;
-  bool ok = true, dry = row_mode;
-  int holder[3] = {-1, -1, -1};  // which node's value each stack slot holds
+  bool ok = true;
   auto push = [&](int op, int a, int dtype, int rmode, int slot, float imm) {
     if (count >= kMaxPost || slot > 2) { ok = false; return; }
     P->post[count++] = PostOp{(int16_t)op, (int16_t)a, (int16_t)dtype, (int16_t)rmode, slot, imm};
   };
   // evaluate node id into value d (values d+1, d+2 are free to use)
-  std::function<void(int, int)> emit_node;
   std::function<void(int, int)> emit = [&](int id, int d) {
-    if (!ok) return;
-    if (d > 2) { ok = false; return; }
-    const bool shared_value = row_mode && uses[id] > 1 && nodes[id].op != KAPY_EW_SPLAT;
-    if (shared_value) {
-      for (int below = 0; below < d; ++below)
-        if (holder[below] == id) {
-          push(kPick, below, nodes[id].dtype, 0, d, 0.f);
-          holder[d] = id;
-          return;
-        }
-      if (parked[id]) {
-        read_back[id] = 1;
-        if (!dry) push(kPushTmp, tmp_of[id], nodes[id].dtype, 0, d, 0.f);
-        else push(kPushTmp, 0, nodes[id].dtype, 0, d, 0.f);
-        holder[d] = id;
-        return;
-      }
-    }
-    emit_node(id, d);
-    if (d + 1 < 3) holder[d + 1] = -1;
-    if (d + 2 < 3) holder[d + 2] = -1;
-    holder[d] = id;
-    if (shared_value) {
-      parked[id] = 1;
-      if (dry || tmp_of[id] >= 0) push(kSaveTmp, dry ? 0 : tmp_of[id], nodes[id].dtype, 0, d, 0.f);
-    }
-  };
-  emit_node = [&](int id, int d) {
     if (!ok) return;
     const N &n = nodes[id];
     switch (n.op) {
@@ -1016,17 +570,6 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
   emit(stored, 0);
   push(kStore, 0, out->dtype, 0, 0, 0.f);
   if (!ok) return false;
-  if (row_mode) {  // again, parking only what the first run read back
-    for (size_t id = 0; id < nodes.size(); ++id)
-      if (read_back[id]) tmp_of[id] = n_tmps++;
-    count = 0;
-    dry = false;
-    std::fill(parked.begin(), parked.end(), 0);
-    holder[0] = holder[1] = holder[2] = -1;
-    emit(stored, 0);
-    push(kStore, 0, out->dtype, 0, 0, 0.f);
-    if (!ok) return false;
-  }
   P->n_post = count;
   P->n_ins = n_ins;
   P->out = (char *)view_base(out);
@@ -1034,7 +577,6 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
   P->out_dtype = out->dtype;
   P->rows = (int32_t)o0;
   P->vec_per_row = (int32_t)(o1 / 8);
-  P->n_tmps = n_tmps;
   return true;
 }
 
@@ -1086,17 +628,7 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 
   bool has_reduce = false;
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
-  if (has_reduce) {
-    StackProgram SP;
-    memset(&SP, 0, sizeof SP);
-    if (!build_stack_program(prog, n_inst, result_dtype, ins, n_ins, out, &SP, true))
-      return fail(KAPY_ERR_UNSUPPORTED, "elementwise: a program with a reduce needs axis 1, contiguous rows of a multiple of 8 and at most 32768 "
-                                        "elements, zero padding, full / row / column / scalar operands and at most three values in flight");
-    bool narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
-    for (int k = 0; k < n_ins; ++k) narrow = narrow && (ins[k]->dtype == KAPY_F16 || ins[k]->dtype == KAPY_BF16);
-    for (int k = 0; k < n_inst; ++k) narrow = narrow && !is_f8(result_dtype[k]);
-    return narrow ? launch_row_kernel<true>(SP, s) : launch_row_kernel<false>(SP, s);
-  }
+  if (has_reduce) return run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
 
   AffineActParams ap;
   int T = -1;

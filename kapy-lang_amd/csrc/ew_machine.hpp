@@ -1,0 +1,292 @@
+// ew_machine.hpp — device side of the stack machine that elementwise programs run on, shared by the
+// translation units that instantiate its kernels (elementwise.hip: one vector of 8 elements per lane;
+// elementwise_row.hip: whole rows resident per workgroup, for programs with a reduce).
+#pragma once
+#include <math.h>
+#include <stdint.h>
+
+#include "common.hpp"
+#include "numeric.hpp"
+
+namespace kapy {
+
+constexpr int kMaxRegs = 16;
+constexpr int kMaxInst = 48;
+constexpr int kMaxInputs = 8;
+constexpr int kMaxPost = 40;
+enum PostKind { kPushIn = 100, kPushImm = 101, kCast = 102, kStore = 103, kRevSub = 104, kRevDiv = 105, kSaveTmp = 106, kPushTmp = 107, kPick = 108, kPushU = 109 };
+enum InKind { kInFull = 0, kInRow = 1 /* [1 x n] */, kInCol = 2 /* [m x 1] */, kInScalar = 3 };
+// bits of PostOp::slot above the slot number (row machine only)
+enum SlotFlags { kSlotMask = 3, kUniformResult = 4, kUniformRight = 8, kSameOperand = 16 };  // bits 8-9: the per-row value a step names
+struct PostOp {
+  int16_t op, a, dtype, rmode;
+  int32_t slot;  // which of the three values holds the result (and the left operand), plus SlotFlags
+  float imm;
+};
+struct StackIn {
+  const char *base;
+  int64_t stride0;
+  int32_t dtype, kind;
+};
+struct StackProgram {
+  PostOp post[kMaxPost];
+  StackIn in[kMaxInputs];
+  char *out;
+  int64_t out_stride0;
+  int32_t n_post, n_ins, out_dtype, rows, vec_per_row;
+  int32_t n_tmps;  // row machine only: values used more than once, parked in LDS
+};
+
+// Compiles a verified program that contains a reduce for the row machine and launches it (elementwise_row.hip).
+// result_dtype[k] is the element type of instruction k's result.
+int run_row_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                    hipStream_t stream);
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 0.5*v*(1+tanh(u)) with u = sqrt(2/pi)*(v+0.044715*v^3) equals v*sigmoid(2u) = v / (1 + 2^(-2u*log2 e)):
+// no cancellation for v << 0, and only three slow-rate operations per element (exp2, rcp and
+// their operand prep).  The constants fold -2*log2(e)*sqrt(2/pi) into the cubic.
+__device__ __forceinline__ float gelu_tanh_f32(float v) {
+  constexpr float kC1 = -2.0f * 1.4426950408889634f * 0.7978845608028654f;
+  constexpr float kC3 = kC1 * 0.044715f;
+  float t = v * (kC1 + kC3 * v * v);
+  return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
+}
+
+__device__ __forceinline__ float apply_unary(int op, float a) {
+  switch (op) {
+  case KAPY_EW_NEGF: return -a;
+  case KAPY_EW_ABSF: return fabsf(a);
+  case KAPY_EW_EXP: return expf(a);
+  case KAPY_EW_EXP2: return exp2f(a);
+  case KAPY_EW_LOG: return logf(a);
+  case KAPY_EW_LOG2: return log2f(a);
+  case KAPY_EW_SQRT: return sqrtf(a);
+  case KAPY_EW_RSQRT: return 1.0f / sqrtf(a);
+  case KAPY_EW_TANH: return tanhf(a);
+  case KAPY_EW_ERF: return erff(a);
+  case KAPY_EW_GELU_TANH: return gelu_tanh_f32(a);
+  }
+  return a;
+}
+
+// arith.maximumf / minimumf: NaN if either operand is NaN.
+__device__ __forceinline__ float max_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ __forceinline__ float min_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+
+// ---------------------------------------------------------------------------------------------
+// Stack machine: any program whose expression tree needs at most three live values, on 8
+// consecutive elements per lane in registers.  The host unfolds the SSA program into postfix form
+// (a value used twice is simply evaluated twice: every op is pure) and gives every step the stack
+// depth it works at, so the three values are three fixed register arrays chosen by a uniform branch:
+// no register is ever indexed at run time and nothing is shuffled.  Values are fp32 images of the typed value, rounded to the
+// result type after every arithmetic op exactly as the register machine does.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void widen16x8(u32x4 v, int dtype, float f[8]) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t word = v[w];
+    if (dtype == KAPY_BF16) {
+      f[2 * w] = bits_f32(word << 16);
+      f[2 * w + 1] = bits_f32(word & 0xFFFF0000u);
+    } else {
+      f[2 * w] = f16_to_f32((uint16_t)word);
+      f[2 * w + 1] = f16_to_f32((uint16_t)(word >> 16));
+    }
+  }
+}
+// The 8 elements of vector jv of row i of a full-extent operand, as they lie in memory (16, 32 or 8 bytes).
+struct Raw8 {
+  u32x4 lo, hi;
+};
+__device__ __forceinline__ Raw8 fetch8(const StackIn &g, int32_t i, int32_t jv, bool streaming) {
+  const int eb = g.dtype == KAPY_F32 ? 4 : (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16) ? 2 : 1;
+  const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * eb;
+  Raw8 r;
+  r.lo = r.hi = u32x4{0, 0, 0, 0};
+  if (eb == 2) r.lo = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
+  else if (eb == 4) {
+    r.lo = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
+    r.hi = streaming ? __builtin_nontemporal_load((const u32x4 *)ptr + 1) : *((const u32x4 *)ptr + 1);
+  } else {
+    const u32x2 v = *(const u32x2 *)ptr;
+    r.lo[0] = v[0];
+    r.lo[1] = v[1];
+  }
+  return r;
+}
+__device__ __forceinline__ void widen8(const Raw8 &r, int dtype, float f[8]) {
+  if (dtype == KAPY_F16 || dtype == KAPY_BF16) widen16x8(r.lo, dtype, f);
+  else if (dtype == KAPY_F32) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t a = r.lo[e], b = r.hi[e];
+      f[e] = bits_f32(a);
+      f[4 + e] = bits_f32(b);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t word = r.lo[e >> 2];
+      const uint8_t byte = (uint8_t)(word >> (8 * (e & 3)));
+      f[e] = dtype == KAPY_F8E4M3 ? e4m3_to_f32(byte) : e5m2_to_f32(byte);
+    }
+  }
+}
+template <bool NARROW>
+__device__ __forceinline__ void load8(const StackIn &g, int32_t i, int32_t jv, float f[8]) {
+  if (g.kind == kInCol || g.kind == kInScalar) {
+    const float v = load_as_f32(g.base, g.dtype, g.kind == kInCol ? i * g.stride0 : 0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = v;
+    return;
+  }
+  if (NARROW) {
+    const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * 2;
+    widen16x8(g.kind == kInFull ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr, g.dtype, f);
+  } else widen8(fetch8(g, i, jv, g.kind == kInFull), g.dtype, f);
+}
+template <bool NARROW>
+__device__ __forceinline__ void round8(float f[8], int dtype, bool rn) {
+  switch (dtype) {
+  case KAPY_F32: return;
+  case KAPY_F16:
+    if (rn) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)(_Float16)f[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = f16_to_f32(f32_to_f16_rz(f[e]));
+    }
+    return;
+  case KAPY_BF16:
+    if (rn) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (float)(__bf16)f[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = bf16_to_f32(f32_to_bf16_rz(f[e]));
+    }
+    return;
+  default:
+    if (!NARROW) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = round_to_dtype(f[e], dtype, rn);
+    }
+  }
+}
+template <bool NARROW>
+__device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const float f[8]) {
+  if (NARROW || dtype == KAPY_F16 || dtype == KAPY_BF16) {
+    u32x4 v;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v[w] = dtype == KAPY_F16 ? pack2_f16_rn(f[2 * w], f[2 * w + 1]) : pack2_bf16_rn(f[2 * w], f[2 * w + 1]);
+    __builtin_nontemporal_store(v, (u32x4 *)(out + elem * 2));
+  } else if (dtype == KAPY_F32) {
+    u32x4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[e] = f32_bits(f[e]);
+      hi[e] = f32_bits(f[4 + e]);
+    }
+    __builtin_nontemporal_store(lo, (u32x4 *)(out + elem * 4));
+    __builtin_nontemporal_store(hi, (u32x4 *)(out + elem * 4) + 1);
+  } else {
+    u32x2 v = {0, 0};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t byte = dtype == KAPY_F8E4M3 ? f32_to_e4m3(f[e], true) : f32_to_e5m2(f[e], true);
+      v[e >> 2] |= byte << (8 * (e & 3));
+    }
+    *(u32x2 *)(out + elem) = v;
+  }
+}
+
+// One step with its result (and left operand) in value D, the right operand in value D+1 and the
+// third operand of an fma in value D+2; D is a template parameter so that no register is indexed.
+// NARROW: every operand, every intermediate type and the result are f16 / bf16 / f32-from-16-bit
+// (no fp8, no fp32 in memory): the common case, and it needs far fewer registers.
+template <int D, bool NARROW>
+__device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &I, int32_t i, int32_t jv, float (&v)[3][8]) {
+  constexpr int R = D + 1 < 3 ? D + 1 : 2, T = D + 2 < 3 ? D + 2 : 2;
+  float *x = v[D];
+  const float *y = v[R], *z = v[T];
+  switch (I.op) {
+  case kPushIn: load8<NARROW>(P.in[I.a], i, jv, x); return;
+  case kPushImm: {
+    const float c = round_to_dtype(I.imm, I.dtype, true);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = c;
+    return;
+  }
+  case kStore: store8<NARROW>(P.out, P.out_dtype, (int64_t)i * P.out_stride0 + (int64_t)jv * 8, x); return;
+  case kCast: round8<NARROW>(x, I.dtype, I.rmode != KAPY_RZ); return;
+  case KAPY_EW_ADDF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fadd_rn(x[e], y[e]);
+    break;
+  case KAPY_EW_SUBF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fsub_rn(x[e], y[e]);
+    break;
+  case kRevSub:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fsub_rn(y[e], x[e]);
+    break;
+  case KAPY_EW_MULF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fmul_rn(x[e], y[e]);
+    break;
+  case KAPY_EW_DIVF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(x[e], y[e]);
+    break;
+  case kRevDiv:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(y[e], x[e]);
+    break;
+  case KAPY_EW_MAXIMUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = max_nan(x[e], y[e]);
+    break;
+  case KAPY_EW_MINIMUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = min_nan(x[e], y[e]);
+    break;
+  case KAPY_EW_FMA:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = __fmaf_rn(x[e], y[e], z[e]);
+    break;
+  default:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = apply_unary(I.op, x[e]);
+  }
+  if (I.dtype != KAPY_F32) round8<NARROW>(x, I.dtype, true);
+}
+
+template <bool NARROW>
+__device__ __forceinline__ void stack_run(const StackProgram &P) {
+  const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (slot >= (int64_t)P.rows * P.vec_per_row) return;
+  const int32_t i = (int32_t)(slot / P.vec_per_row), jv = (int32_t)(slot - (int64_t)i * P.vec_per_row);
+  float v[3][8];
+#pragma unroll
+  for (int d = 0; d < 3; ++d)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[d][e] = 0.f;
+  for (int pc = 0; pc < P.n_post; ++pc) {
+    const PostOp I = P.post[pc];
+    switch (I.slot) {
+    case 0: stack_step<0, NARROW>(P, I, i, jv, v); break;
+    case 1: stack_step<1, NARROW>(P, I, i, jv, v); break;
+    default: stack_step<2, NARROW>(P, I, i, jv, v);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace kapy

@@ -10,6 +10,7 @@
 // that name their slots statically, so no register is indexed at run time; a row value used again while
 // it still sits lower on the stack is copied from there, one that has been overwritten in between is
 // parked in LDS by its first evaluation and read back by the lane that wrote it.
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -25,6 +26,206 @@ int launch_row_narrow(const StackProgram &P, int ns, hipStream_t s);
 int launch_row_any(const StackProgram &P, int ns, hipStream_t s);
 
 namespace {
+
+// ---------------------------------------------------------------------------------------------
+// The two row programs that have names get kernels of their own (as act(x*s+bias) does among the plain elementwise
+// programs): softmax and the layer / RMS norm family, on 16-bit operands with fp32 arithmetic, step for step what the
+// row machine's light kernel would compute, without its decoding.
+struct FusedRow {
+  const char *x, *gamma, *beta;  // gamma / beta: [1 x n] rows or null
+  char *out;
+  int64_t x_stride0, out_stride0;
+  int32_t rows, vec_per_row;
+  int32_t centre;  // norm: subtract the mean first (layer norm) or not (RMS norm)
+  float inv_n, eps;
+};
+
+template <int THREADS, bool MAX>
+__device__ __forceinline__ float row_fold(float acc, float *red) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float other = __shfl_xor(acc, off, 64);
+    acc = MAX ? max_nan(acc, other) : acc + other;
+  }
+  if (THREADS > 64) {
+    constexpr int WAVES = THREADS / 64;
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    acc = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) acc = MAX ? max_nan(acc, red[w]) : acc + red[w];
+  }
+  return acc;
+}
+
+template <int CH, int THREADS, bool STREAM>
+__device__ __forceinline__ void row_fetch(const char *base, int32_t vpr, u32x4 (&raw)[CH]) {
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int32_t jv = c * THREADS + threadIdx.x;
+    raw[c] = u32x4{0, 0, 0, 0};
+    if (jv < vpr) raw[c] = STREAM ? __builtin_nontemporal_load((const u32x4 *)(base + (int64_t)jv * 16)) : *(const u32x4 *)(base + (int64_t)jv * 16);
+  }
+}
+
+// Both kernels walk rows blockIdx.x, blockIdx.x + gridDim.x, ... and ask for the next row's 16 bytes per chunk before they
+// work on the current one, so that a workgroup always has a load in flight.  The two exchange areas of a row's two
+// reduces are safe to reuse from row to row: a wave can write one again only after the barrier of the other, which every
+// wave reaches after it has read the first.
+template <int CH, int THREADS>
+__global__ __launch_bounds__(THREADS) void softmax_kernel(FusedRow p, int dtype) {
+  __shared__ float red[2][16];
+  u32x4 raw[CH];
+  row_fetch<CH, THREADS, true>(p.x + (int64_t)blockIdx.x * p.x_stride0 * 2, p.vec_per_row, raw);
+  for (int32_t i = blockIdx.x; i < p.rows; i += gridDim.x) {
+    float f[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) widen16x8(raw[c], dtype, f[c]);
+    if (i + (int32_t)gridDim.x < p.rows) row_fetch<CH, THREADS, true>(p.x + (int64_t)(i + gridDim.x) * p.x_stride0 * 2, p.vec_per_row, raw);
+    float m = -__builtin_inff();
+    bool any_nan = false;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if (c * THREADS + (int)threadIdx.x < p.vec_per_row) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          m = fmaxf(m, f[c][e]);
+          any_nan |= f[c][e] != f[c][e];
+        }
+      }
+    m = row_fold<THREADS, true>(any_nan ? __builtin_nanf("") : m, red[0]);
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const bool active = c * THREADS + (int)threadIdx.x < p.vec_per_row;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // exp(x) = 2^hi * (1 + lo*ln2) with hi + lo = x*log2(e), lo the product's rounding error: about 1 ulp of fp32
+        // for the x <= 0 that reach here.  A NaN passes through every step; x = -inf gives hi = -inf, 2^hi = 0, and
+        // needs lo, which would be inf - inf, set aside.
+        const float x = __fsub_rn(f[c][e], m);
+        const float hi = x * 1.44269504088896341f;
+        float lo = __builtin_fmaf(x, 1.44269504088896341f, -hi);
+        lo = !(x <= -3e38f) ? lo : 0.f;
+        const float pw = __builtin_amdgcn_exp2f(hi);
+        f[c][e] = __builtin_fmaf(pw, lo * 0.693147180559945309f, pw);
+      }
+      if (active) sum += ((f[c][0] + f[c][1]) + (f[c][2] + f[c][3])) + ((f[c][4] + f[c][5]) + (f[c][6] + f[c][7]));
+    }
+    sum = row_fold<THREADS, false>(sum, red[1]);
+    const float rcp = __builtin_amdgcn_rcpf(sum);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // e / sum as e*(1/sum) corrected by the remainder: the correctly rounded quotient (e <= 1 <= sum <= n here; a
+        // NaN in either is a NaN in both forms)
+        const float q = f[c][e] * rcp;
+        const float rem = __builtin_fmaf(-q, sum, f[c][e]);
+        f[c][e] = __builtin_fmaf(rem, rcp, q);
+      }
+      const int32_t jv = c * THREADS + threadIdx.x;
+      if (jv < p.vec_per_row) store8<true>(p.out, dtype, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, f[c]);
+    }
+  }
+}
+
+template <int CH, int THREADS>
+__global__ __launch_bounds__(THREADS) void norm_kernel(FusedRow p, int dtype) {
+  __shared__ float red[2][16];
+  // gamma and beta are the same for every row: each lane keeps its own 16-byte pieces of them in LDS (its private
+  // corner of it: written once, read back by the same lane, no barrier) rather than in registers the row needs
+  extern __shared__ u32x4 stash[];
+  u32x4 raw[CH];
+  row_fetch<CH, THREADS, true>(p.x + (int64_t)blockIdx.x * p.x_stride0 * 2, p.vec_per_row, raw);
+  {
+    u32x4 gb[CH];
+    if (p.gamma) {
+      row_fetch<CH, THREADS, false>(p.gamma, p.vec_per_row, gb);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) stash[c * THREADS + threadIdx.x] = gb[c];
+    }
+    if (p.beta) {
+      row_fetch<CH, THREADS, false>(p.beta, p.vec_per_row, gb);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) stash[(CH + c) * THREADS + threadIdx.x] = gb[c];
+    }
+  }
+  for (int32_t i = blockIdx.x; i < p.rows; i += gridDim.x) {
+    float f[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) widen16x8(raw[c], dtype, f[c]);
+    if (i + (int32_t)gridDim.x < p.rows) row_fetch<CH, THREADS, true>(p.x + (int64_t)(i + gridDim.x) * p.x_stride0 * 2, p.vec_per_row, raw);
+    if (p.centre) {
+      float sum = 0.f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+        if (c * THREADS + (int)threadIdx.x < p.vec_per_row) sum += ((f[c][0] + f[c][1]) + (f[c][2] + f[c][3])) + ((f[c][4] + f[c][5]) + (f[c][6] + f[c][7]));
+      const float mean = __fmul_rn(row_fold<THREADS, false>(sum, red[0]), p.inv_n);
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[c][e] = __fsub_rn(f[c][e], mean);
+    }
+    float sq = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if (c * THREADS + (int)threadIdx.x < p.vec_per_row) {
+        float s8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s8[e] = __fmul_rn(f[c][e], f[c][e]);
+        sq += ((s8[0] + s8[1]) + (s8[2] + s8[3])) + ((s8[4] + s8[5]) + (s8[6] + s8[7]));
+      }
+    const float var = __fmul_rn(row_fold<THREADS, false>(sq, red[1]), p.inv_n);
+    const float rstd = __builtin_amdgcn_rsqf(__fadd_rn(var, p.eps));
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int32_t jv = c * THREADS + threadIdx.x;
+      const bool active = jv < p.vec_per_row;
+      float g[8], b[8];
+      if (p.gamma) widen16x8(stash[c * THREADS + threadIdx.x], dtype, g);
+      if (p.beta) widen16x8(stash[(CH + c) * THREADS + threadIdx.x], dtype, b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float r = __fmul_rn(f[c][e], rstd);
+        if (p.gamma) r = __fmul_rn(r, g[e]);
+        if (p.beta) r = __fadd_rn(r, b[e]);
+        f[c][e] = r;
+      }
+      if (active) store8<true>(p.out, dtype, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, f[c]);
+    }
+  }
+}
+
+int launch_fused_row(const FusedRow &p, int dtype, bool softmax, hipStream_t s) {
+  const int vpr = p.vec_per_row;
+  const int threads = vpr <= 256 ? 64 : vpr <= 1024 ? 256 : 1024;
+  const int ch = (vpr + threads - 1) / threads;
+  // as many workgroups as are resident at once; each walks its share of the rows
+#define KAPY_FUSED(CH_, TH_)                                                           \
+  do {                                                                                 \
+    int per_cu = 1;                                                                    \
+    const size_t lds = softmax ? 0 : (size_t)2 * CH_ * TH_ * 16;                       \
+    if (lds > 48 * 1024) KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)norm_kernel<CH_, TH_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+    if (softmax) KAPY_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, softmax_kernel<CH_, TH_>, TH_, 0)); \
+    else KAPY_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, norm_kernel<CH_, TH_>, TH_, lds)); \
+    const int64_t resident = (int64_t)device_cus() * (per_cu > 0 ? per_cu : 1);        \
+    dim3 grid((unsigned)(p.rows < resident ? p.rows : resident));                      \
+    if (softmax) softmax_kernel<CH_, TH_><<<grid, TH_, 0, s>>>(p, dtype);              \
+    else norm_kernel<CH_, TH_><<<grid, TH_, lds, s>>>(p, dtype);                       \
+  } while (0)
+#define KAPY_FUSED_CH(TH_)                                                             \
+  do {                                                                                 \
+    if (ch == 1) KAPY_FUSED(1, TH_); else if (ch == 2) KAPY_FUSED(2, TH_); else KAPY_FUSED(4, TH_); \
+  } while (0)
+  if (threads == 64) KAPY_FUSED_CH(64);
+  else if (threads == 256) KAPY_FUSED_CH(256);
+  else KAPY_FUSED_CH(1024);
+#undef KAPY_FUSED_CH
+#undef KAPY_FUSED
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Host: the program's DAG compiled into steps.
@@ -214,6 +415,96 @@ struct RowBuilder {
   }
 };
 
+// Structural match of the named row programs on the DAG.  Shared values must be shared nodes (the same register
+// read twice), every intermediate fp32, operands and result the same 16-bit type.
+bool match_fused_row(const RowBuilder &B, const StackProgram &SP, const kapy_global *out, FusedRow *p, bool *softmax) {
+  const auto &nodes = B.nodes;
+  const int T = out->dtype;
+  if (T != KAPY_F16 && T != KAPY_BF16) return false;
+  auto is = [&](int id, int op) { return id >= 0 && nodes[id].op == op && (op == KAPY_EW_LD_GLOBAL || nodes[id].dtype == KAPY_F32); };
+  // cast32(ld input) of a given operand kind: the input's index, or -1
+  auto loaded = [&](int id, int kind) {
+    if (!is(id, KAPY_EW_FPTOFP)) return -1;
+    const int ld = nodes[id].a;
+    if (ld < 0 || nodes[ld].op != KAPY_EW_LD_GLOBAL) return -1;
+    const int in = nodes[ld].input;
+    return SP.in[in].kind == kind && SP.in[in].dtype == T ? in : -1;
+  };
+  // op(a, b) with operands in either order, `second` chosen by a predicate; returns the other operand or -1
+  auto other_of = [&](int id, int op, const std::function<bool(int)> &second) {
+    if (!is(id, op)) return -1;
+    if (second(nodes[id].b)) return nodes[id].a;
+    if (second(nodes[id].a)) return nodes[id].b;
+    return -1;
+  };
+  const int st = B.stored;
+  if (nodes[st].op != KAPY_EW_FPTOFP || nodes[st].dtype != T || nodes[st].rmode == KAPY_RZ) return false;
+  int body = nodes[st].a;
+  int x_in = -1;
+  memset(p, 0, sizeof *p);
+  // softmax: div(E, sum(E)), E = exp(sub(F, max(F)))
+  if (is(body, KAPY_EW_DIVF)) {
+    const int e = nodes[body].a, rs = nodes[body].b;
+    if (!is(rs, KAPY_EW_REDUCE_SUM) || nodes[rs].a != e || !is(e, KAPY_EW_EXP)) return false;
+    const int sub = nodes[e].a;
+    if (!is(sub, KAPY_EW_SUBF)) return false;
+    const int f = nodes[sub].a, rm = nodes[sub].b;
+    if (!is(rm, KAPY_EW_REDUCE_MAX) || nodes[rm].a != f) return false;
+    x_in = loaded(f, kInFull);
+    if (x_in < 0) return false;
+    *softmax = true;
+  } else {
+    // norm: [add(., beta)] [mul(., gamma)] mul(C, rsqrt(add(mul(sum(mul(C, C)), 1/n), eps))), C = F or sub(F, mul(sum(F), 1/n))
+    int gamma = -1, beta = -1;
+    auto row_operand = [&](int id) { return loaded(id, kInRow) >= 0; };
+    int inner = other_of(body, KAPY_EW_ADDF, row_operand);
+    if (inner >= 0) {
+      beta = loaded(nodes[body].a == inner ? nodes[body].b : nodes[body].a, kInRow);
+      body = inner;
+    }
+    inner = other_of(body, KAPY_EW_MULF, row_operand);
+    if (inner >= 0) {
+      gamma = loaded(nodes[body].a == inner ? nodes[body].b : nodes[body].a, kInRow);
+      body = inner;
+    }
+    if (beta >= 0 && gamma < 0) return false;
+    const int c = other_of(body, KAPY_EW_MULF, [&](int id) { return is(id, KAPY_EW_RSQRT); });
+    if (c < 0) return false;
+    const int rsq = nodes[body].a == c ? nodes[body].b : nodes[body].a;
+    auto splat = [&](int id) { return is(id, KAPY_EW_SPLAT); };
+    const int plus = nodes[rsq].a;
+    const int scaled = other_of(plus, KAPY_EW_ADDF, splat);
+    if (scaled < 0) return false;
+    p->eps = nodes[nodes[plus].a == scaled ? nodes[plus].b : nodes[plus].a].imm;
+    const int total = other_of(scaled, KAPY_EW_MULF, splat);
+    if (total < 0 || !is(total, KAPY_EW_REDUCE_SUM)) return false;
+    p->inv_n = nodes[nodes[scaled].a == total ? nodes[scaled].b : nodes[scaled].a].imm;
+    const int sq = nodes[total].a;
+    if (!is(sq, KAPY_EW_MULF) || nodes[sq].a != c || nodes[sq].b != c) return false;
+    int f = c;
+    if (is(c, KAPY_EW_SUBF)) {
+      f = nodes[c].a;
+      const int mean = nodes[c].b;
+      const int fsum = other_of(mean, KAPY_EW_MULF, splat);
+      if (fsum < 0 || !is(fsum, KAPY_EW_REDUCE_SUM) || nodes[fsum].a != f) return false;
+      if (nodes[nodes[mean].a == fsum ? nodes[mean].b : nodes[mean].a].imm != p->inv_n) return false;
+      p->centre = 1;
+    }
+    x_in = loaded(f, kInFull);
+    if (x_in < 0) return false;
+    p->gamma = gamma >= 0 ? SP.in[gamma].base : nullptr;
+    p->beta = beta >= 0 ? SP.in[beta].base : nullptr;
+    *softmax = false;
+  }
+  p->x = SP.in[x_in].base;
+  p->x_stride0 = SP.in[x_in].stride0;
+  p->out = (char *)view_base(out);
+  p->out_stride0 = out->stride0;
+  p->rows = (int32_t)extent0(out);
+  p->vec_per_row = (int32_t)(extent1(out) / 8);
+  return true;
+}
+
 }  // namespace
 
 int run_row_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
@@ -295,6 +586,13 @@ int run_row_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtyp
       if (n.c >= 0) visit(n.c);
     };
     visit(B.stored);
+  }
+  {
+    FusedRow fr;
+    bool softmax = false;
+    // KAPY_ROW_FUSED=0 sends the named programs through the row machine as well (tests compare the two)
+    const char *sw = getenv("KAPY_ROW_FUSED");
+    if (!(sw && sw[0] == '0') && match_fused_row(B, SP, out, &fr, &softmax)) return launch_fused_row(fr, out->dtype, softmax, stream);
   }
   B.compute_need();
   B.out_dtype = out->dtype;

@@ -232,16 +232,37 @@ def _row_case(ko, insts, dtype, m, n, seed, extra=(), std=2.0):
     return _run_prog(ko, insts, ins, [dtype] * len(ins), dtype, m, n, in_shapes=shapes)
 
 
+@pytest.fixture(params=["fused kernel", "row machine"])
+def row_path(request, monkeypatch):
+    """The named row programs have kernels of their own; KAPY_ROW_FUSED=0 sends them through the row machine."""
+    if request.param == "row machine":
+        monkeypatch.setenv("KAPY_ROW_FUSED", "0")
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
 @pytest.mark.parametrize("m,n", [(7, 64), (5, 1000), (33, 4096), (9, 8192), (4, 12288), (3, 32768)])
-def test_softmax_rows_every_launch_shape(ko, dtype, m, n):
+def test_softmax_rows_every_launch_shape(ko, row_path, dtype, m, n):
     got, want = _row_case(ko, kh.softmax_insts(dtype), dtype, m, n, 50 + n % 97)
     _check_ulp(got, want, dtype)
 
 
+def test_softmax_special_rows(ko, row_path):
+    m, n = 6, 1024
+    x = ko.fill_normal(m * n, kh.F16, 55, std=4.0).reshape(m, n)
+    x[1, 3] = 0x7e00                 # a NaN poisons its row
+    x[2, 9] = 0x7c00                 # +inf: inf - inf
+    x[3, :] = 0xfc00                 # a row of -inf
+    x[4, :] = 0x7bff                 # a row of the largest finite value: uniform 1/n
+    insts = kh.softmax_insts(kh.F16)
+    got, want = _run_prog(ko, insts, [x], [kh.F16], kh.F16, m, n)
+    _check_ulp(got, want, kh.F16)
+    assert np.all(np.isnan(got[[1, 2, 3]].view(np.float16))) and np.all(got[4] == np.float16(1.0 / n).view(np.uint16))
+
+
 @pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
-@pytest.mark.parametrize("m,n", [(12, 1024), (6, 8192)])
-def test_layernorm_and_rmsnorm_rows(ko, dtype, m, n):
+@pytest.mark.parametrize("m,n", [(12, 1024), (6, 8192), (5, 200)])
+def test_layernorm_and_rmsnorm_rows(ko, row_path, dtype, m, n):
     got, want = _row_case(ko, kh.layernorm_insts(n, dtype), dtype, m, n, 61, extra=("gamma", "beta"))
     _check_ulp(got, want, dtype)
     got, want = _row_case(ko, kh.layernorm_insts(n, dtype, affine=False), dtype, m, n, 62)

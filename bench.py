@@ -152,7 +152,8 @@ def bench_rowwise(kh, steps, warmup, which):
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]] + extra, gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
     return {"workload": "%s of every row, fp16 8192x8192, fp32 arithmetic" % which, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "row_kernel"}
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev),
+            "kernel": "softmax_kernel" if which == "softmax" else "norm_kernel"}
 
 
 def bench_transpose(kh, steps, warmup):

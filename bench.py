@@ -102,9 +102,10 @@ def bench_copy(kh, steps, warmup):
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
 
 
-def bench_add(kh, steps, warmup):
-    """z = x + y in fp16 (the reference's elementwise_add.mlir fixture at the headline shape): a program outside the
-    act(x*s+bias) chain, served by the in-register stack machine."""
+def bench_add(kh, steps, warmup, op="add"):
+    """z = x + y in fp16 (the reference's elementwise_add.mlir fixture at the headline shape), recognised as x*1 + y and
+    served by the fused affine kernel; op="mul": z = x * y, a program outside that chain, served by the in-register
+    stack machine."""
     import torch
     n, sets = 8192, 3
     xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
@@ -112,12 +113,13 @@ def bench_add(kh, steps, warmup):
     zs = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
     g = lambda t: kh.mk_global(t.data_ptr(), n, n, n, 1, kh.F16)
     gx, gy, gz = [g(t) for t in xs], [g(t) for t in ys], [g(t) for t in zs]
-    prog = kh.program([dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1), dict(op=kh.EW_ADDF, dst=2, a=0, b=1),
-                       dict(op=kh.EW_ST_GLOBAL, a=2)])
+    prog = kh.program([dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1),
+                       dict(op=kh.EW_ADDF if op == "add" else kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ST_GLOBAL, a=2)])
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gy[i % sets]], gz[i % sets]), steps, warmup)
     nbytes = 3 * n * n * 2
-    return {"workload": "elementwise_add fixture: z = x + y fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "stack_kernel_narrow"}
+    name = "elementwise_add fixture: z = x + y fp16 8192x8192" if op == "add" else "z = x * y fp16 8192x8192"
+    return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
+            "roofline": _roof_hbm(nbytes, ev), "kernel": "affine_act_kernel" if op == "add" else "stack_kernel_narrow"}
 
 
 def bench_reduce(kh, steps, warmup):
@@ -251,7 +253,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "mul", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -266,6 +268,7 @@ def main():
     table = {
         "gelu": lambda s, w: bench_gelu(kh, s, w),
         "add": lambda s, w: bench_add(kh, s, w),
+        "mul": lambda s, w: bench_add(kh, s, w, "mul"),
         "copy": lambda s, w: bench_copy(kh, s, w),
         "transpose": lambda s, w: bench_transpose(kh, s, w),
         "reduce": lambda s, w: bench_reduce(kh, s, w),

@@ -12,6 +12,7 @@
 #include <string.h>
 
 #include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "common.hpp"
@@ -399,19 +400,28 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
     return true;
   };
   int cur = stored;
+  int x_in = -1, bias_in = -1;
+  p->act = -1;
+  p->has_scale = 0;
+  p->scale = 1.f;
+  // st(addf(ld x, ld y)) on the 16-bit type itself (the reference's elementwise_add fixture): the fp32 sum of two 16-bit
+  // values rounded once to the type is the type's own correctly rounded sum
+  const bool plain_add = is_kind(cur, KAPY_EW_ADDF) && is_kind(nodes[cur].a, KAPY_EW_LD_GLOBAL) && is_kind(nodes[cur].b, KAPY_EW_LD_GLOBAL);
+  if (plain_add) {
+    x_in = nodes[nodes[cur].a].input;
+    bias_in = nodes[nodes[cur].b].input;
+    if (extent0(ins[x_in]) != extent0(out) || extent1(ins[x_in]) != extent1(out)) std::swap(x_in, bias_in);
+  }
+  if (!plain_add) {
   if (!is_kind(cur, KAPY_EW_FPTOFP) || nodes[cur].dtype != T || nodes[cur].rmode != KAPY_RN) return false;
   cur = nodes[cur].a;
   if (cur < 0) return false;
-  p->act = -1;
   int k = nodes[cur].kind;
   if (k >= KAPY_EW_NEGF && k <= KAPY_EW_GELU_TANH) {
     p->act = k;
     cur = nodes[cur].a;
     if (cur < 0) return false;
   }
-  int x_in = -1, bias_in = -1;
-  p->has_scale = 0;
-  p->scale = 1.f;
   auto match_scaled = [&](int id) -> int {  // mulf(x, s) | mulf(s, x) | x
     if (is_kind(id, KAPY_EW_MULF)) {
       float s;
@@ -435,6 +445,7 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
   } else {
     x_in = match_scaled(cur);
     if (x_in < 0) return false;
+  }
   }
   const kapy_global *x = ins[x_in];
   if (x->dtype != T || x->stride1 != 1 || out->stride1 != 1) return false;

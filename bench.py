@@ -103,9 +103,9 @@ def bench_copy(kh, steps, warmup):
 
 
 def bench_add(kh, steps, warmup, op="add"):
-    """z = x + y in fp16 (the reference's elementwise_add.mlir fixture at the headline shape), recognised as x*1 + y and
-    served by the fused affine kernel; op="mul": z = x * y, a program outside that chain, served by the in-register
-    stack machine."""
+    """z = x + y in fp16 (the reference's elementwise_add.mlir fixture at the headline shape), a plain binary program,
+    served by the fused affine kernel; op="expr": z = x*y + x with both roundings, a program outside the fused chains,
+    served by the in-register stack machine."""
     import torch
     n, sets = 8192, 3
     xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
@@ -113,11 +113,15 @@ def bench_add(kh, steps, warmup, op="add"):
     zs = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
     g = lambda t: kh.mk_global(t.data_ptr(), n, n, n, 1, kh.F16)
     gx, gy, gz = [g(t) for t in xs], [g(t) for t in ys], [g(t) for t in zs]
-    prog = kh.program([dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1),
-                       dict(op=kh.EW_ADDF if op == "add" else kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ST_GLOBAL, a=2)])
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1)]
+    if op == "add":
+        insts += [dict(op=kh.EW_ADDF, dst=2, a=0, b=1)]
+    else:
+        insts += [dict(op=kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ADDF, dst=2, a=2, b=0)]
+    prog = kh.program(insts + [dict(op=kh.EW_ST_GLOBAL, a=2)])
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gy[i % sets]], gz[i % sets]), steps, warmup)
     nbytes = 3 * n * n * 2
-    name = "elementwise_add fixture: z = x + y fp16 8192x8192" if op == "add" else "z = x * y fp16 8192x8192"
+    name = "elementwise_add fixture: z = x + y fp16 8192x8192" if op == "add" else "z = x*y + x (two roundings) fp16 8192x8192"
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
             "roofline": _roof_hbm(nbytes, ev), "kernel": "affine_act_kernel" if op == "add" else "stack_kernel_narrow"}
 
@@ -253,7 +257,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "mul", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -268,7 +272,7 @@ def main():
     table = {
         "gelu": lambda s, w: bench_gelu(kh, s, w),
         "add": lambda s, w: bench_add(kh, s, w),
-        "mul": lambda s, w: bench_add(kh, s, w, "mul"),
+        "expr": lambda s, w: bench_add(kh, s, w, "expr"),
         "copy": lambda s, w: bench_copy(kh, s, w),
         "transpose": lambda s, w: bench_transpose(kh, s, w),
         "reduce": lambda s, w: bench_reduce(kh, s, w),

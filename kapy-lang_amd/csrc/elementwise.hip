@@ -114,6 +114,7 @@ struct AffineActParams {
   int64_t x_stride0, out_stride0, bias_stride0;  // elements
   int32_t rows, vec_per_row;
   int32_t has_scale, bias_mode, act;  // act: a unary kapy_ew_op, or -1
+  int32_t combine;                    // how the second operand meets x*scale: Combine (plain binary programs; kAdd otherwise)
   float scale;
 };
 
@@ -171,8 +172,18 @@ __device__ __forceinline__ u32x4 pack8(const float f[8]) {
 // may contract it into one FMA (for f16 inputs the mixed-precision v_fma_mix_f32), i.e. one
 // rounding where mulf-then-addf has two; the difference is at most half an ulp of fp32, five
 // orders of magnitude inside the 2-ulp tolerance of the 16-bit result.
+enum Combine { kAdd = 0, kSub = 1 /* x - y */, kRevSubtract = 2 /* y - x */, kMul = 3, kMax = 4, kMin = 5 };
 template <int ACT>
-__device__ __forceinline__ float affine_act(float x, float scale, float bias, int act) {
+__device__ __forceinline__ float affine_act(float x, float scale, float bias, int act, int combine) {
+  if (ACT == -1 && combine != kAdd) {  // z = x op y on the 16-bit type: the fp32 result rounded once is the type's own
+    switch (combine) {
+    case kSub: return x - bias;
+    case kRevSubtract: return bias - x;
+    case kMul: return x * bias;
+    case kMax: return max_nan(x, bias);
+    default: return min_nan(x, bias);
+    }
+  }
   float v = x * scale + bias;
   if (ACT == KAPY_EW_GELU_TANH) return gelu_tanh_f32(v);
   if (ACT >= 0) return apply_unary(act, v);
@@ -219,7 +230,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
     unpack8<T>(xv[u], f);
     if (p.bias_mode != kNoBias) unpack8<T>(bv[u], b);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, p.bias_mode != kNoBias ? b[e] : 0.f, p.act);
+    for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, p.bias_mode != kNoBias ? b[e] : 0.f, p.act, p.combine);
     u32x4 *op = (u32x4 *)(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2);
     if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
     else *op = pack8<T>(f);
@@ -254,7 +265,7 @@ __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p)
     float f[8];
     unpack8<T>(xv[u], f);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, b[e], p.act);
+    for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, b[e], p.act, p.combine);
     u32x4 *op = (u32x4 *)(p.out + ((int64_t)(row0 + u) * p.out_stride0 + col) * 2);
     if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
     else *op = pack8<T>(f);
@@ -404,13 +415,19 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
   p->act = -1;
   p->has_scale = 0;
   p->scale = 1.f;
-  // st(addf(ld x, ld y)) on the 16-bit type itself (the reference's elementwise_add fixture): the fp32 sum of two 16-bit
-  // values rounded once to the type is the type's own correctly rounded sum
-  const bool plain_add = is_kind(cur, KAPY_EW_ADDF) && is_kind(nodes[cur].a, KAPY_EW_LD_GLOBAL) && is_kind(nodes[cur].b, KAPY_EW_LD_GLOBAL);
+  p->combine = kAdd;
+  // st(op(ld x, ld y)) on the 16-bit type itself (addf: the reference's elementwise_add fixture): the fp32 sum,
+  // difference or product of two 16-bit values is exact or rounds harmlessly (operands more than 2^16 apart), so
+  // rounding it once to the type gives the type's own correctly rounded result
+  const int top = cur >= 0 ? nodes[cur].kind : -1;
+  const bool plain_add = (top == KAPY_EW_ADDF || top == KAPY_EW_SUBF || top == KAPY_EW_MULF || top == KAPY_EW_MAXIMUMF || top == KAPY_EW_MINIMUMF) &&
+                         is_kind(nodes[cur].a, KAPY_EW_LD_GLOBAL) && is_kind(nodes[cur].b, KAPY_EW_LD_GLOBAL);
   if (plain_add) {
     x_in = nodes[nodes[cur].a].input;
     bias_in = nodes[nodes[cur].b].input;
-    if (extent0(ins[x_in]) != extent0(out) || extent1(ins[x_in]) != extent1(out)) std::swap(x_in, bias_in);
+    bool swapped = false;
+    if (extent0(ins[x_in]) != extent0(out) || extent1(ins[x_in]) != extent1(out)) { std::swap(x_in, bias_in); swapped = true; }
+    p->combine = top == KAPY_EW_ADDF ? kAdd : top == KAPY_EW_SUBF ? (swapped ? kRevSubtract : kSub) : top == KAPY_EW_MULF ? kMul : top == KAPY_EW_MAXIMUMF ? kMax : kMin;
   }
   if (!plain_add) {
   if (!is_kind(cur, KAPY_EW_FPTOFP) || nodes[cur].dtype != T || nodes[cur].rmode != KAPY_RN) return false;

@@ -222,6 +222,34 @@ def test_register_stack_kernel_tree_shapes_and_operand_kinds(ko):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("op", ["EW_ADDF", "EW_SUBF", "EW_MULF", "EW_MAXIMUMF", "EW_MINIMUMF"])
+def test_plain_binary_programs_are_bit_exact_in_every_operand_shape(ko, dtype, op):
+    """z = x op y on the 16-bit type (addf: the reference's elementwise_add fixture) with the second or the first operand
+    full, a row or a column: the correctly rounded result of the type, NaN and infinity included."""
+    m, n = 24, 256
+    full = ko.fill_normal(m * n, dtype, 91, std=30.0).reshape(m, n)
+    other = ko.fill_normal(m * n, dtype, 92, std=0.01).reshape(m, n)
+    enc = (lambda v: np.array(v, dtype=np.float16).view(np.uint16)) if dtype == kh.F16 else \
+        (lambda v: (np.array(v, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    sp = enc([np.nan, np.inf, -np.inf, 0.0, -0.0, 65504.0, -65504.0, 6e-8])
+    full.ravel()[:len(sp)] = sp
+    other.ravel()[3:3 + len(sp)] = sp
+    for shape in ((m, n), (1, n), (m, 1)):
+        y = np.ascontiguousarray(other[:shape[0], :shape[1]])
+        for swapped in (False, True):
+            insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1),
+                     dict(op=getattr(kh, op), dst=2, a=1 if swapped else 0, b=0 if swapped else 1), dict(op=kh.EW_ST_GLOBAL, a=2)]
+            got, want = _run_prog(ko, insts, [full, y], [dtype, dtype], dtype, m, n, in_shapes=[(m, n), shape])
+            nan = np.isnan(_as_f64(want, dtype))
+            assert np.array_equal(np.isnan(_as_f64(got, dtype)), nan)
+            assert np.array_equal(got[~nan], want[~nan]), (op, shape, swapped)
+
+
+def _as_f64(bits, dtype):
+    return bits.view(np.float16).astype(np.float64) if dtype == kh.F16 else (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
 # ---------------------------------------------------------------------------------------------------------
 # Row-wise fusions: programs with a reduce along the rows run with the row resident on chip.
 def _row_case(ko, insts, dtype, m, n, seed, extra=(), std=2.0):

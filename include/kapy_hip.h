@@ -261,7 +261,9 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * module's kapy.num_warps is executed in turn, each tensor op as one call of the entry points above on
  * `stream` (mk_global/sv_global/sv_shared: MkGlobalOpToLLVM.cpp:23-47, SvGlobalOpToLLVM.cpp:22-40,
  * SvSharedOpToLLVM.cpp:20-42; ld_global/st_global/cp_async_global_to_shared/ld_matrix: kapy_copy; arith on
- * tensors: kapy_elementwise; kapy.reduce: kapy_reduce; kapy.matmul: kapy_matmul; scf.for with iter_args).
+ * tensors, math.exp / exp2 / log / log2 / sqrt / rsqrt / tanh / erf / absf / fma, kapy.fptofp, arith.extf / truncf,
+ * kapy.splat, kapy.broadcast: kapy_elementwise; kapy.transpose: kapy_copy; kapy.reduce: kapy_reduce; kapy.matmul:
+ * kapy_matmul; scf.for with iter_args).
  * Warps run one after the other, so a program whose warps exchange data through shared memory between
  * barriers is outside what this executes correctly; the three fixtures are not of that kind.
  * `args` follow the function's signature: a device pointer (with the size of its allocation in bytes, 0 =

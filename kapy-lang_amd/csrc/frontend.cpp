@@ -11,8 +11,9 @@
 // allocates and frees.  It is a way to run the reference's own programs against this library, not a
 // fast path: a program costs tens of launches.
 //
-// Supported: func arguments (!kapy.ptr<1>, i32), arith.constant (i32, dense tensor), arith
-// addi/subi/muli/divui/remui/cmpi/select, arith addf/subf/mulf/divf/maximumf/minimumf on tensors,
+// Supported: func arguments (!kapy.ptr<1>, i32), arith.constant (i32, float scalar, dense tensor), arith
+// addi/subi/muli/divui/remui/cmpi/select, arith addf/subf/mulf/divf/maximumf/minimumf/negf/extf/truncf and math
+// exp/exp2/log/log2/sqrt/rsqrt/tanh/erf/absf/fma on tensors, kapy.fptofp / splat / broadcast / transpose,
 // kapy.program_id / warp_id / mk_global / sv_global / mk_shared / sv_shared / ld_global / st_global /
 // cp_async_global_to_shared / cp_async_wait_group / ld_matrix / matmul / reduce (addf or maximumf
 // lambda) / return, scf.for with iter_args and scf.yield.
@@ -267,7 +268,7 @@ struct Parser {
     }
     if (accept(":")) {
       while (peek().kind != Token::kNewline && peek().kind != Token::kEnd) {
-        if (accept(",") || accept("->") || accept("(") || accept(")")) continue;
+        if (accept(",") || accept("->") || accept("(") || accept(")") || accept("to")) continue;
         Type ty;
         if (!parse_type(ty)) return false;
         op.types.push_back(ty);
@@ -502,8 +503,9 @@ struct Analyzer {
 constexpr int64_t kLdsBytes = 160 * 1024;
 
 struct Value {
-  enum Kind { kNone, kInt, kPtr, kTensor } kind = kNone;
+  enum Kind { kNone, kInt, kPtr, kTensor, kFloat } kind = kNone;
   int64_t i = 0;
+  double f = 0.0;     // kFloat: a scalar of float type
   void *ptr = nullptr;
   int64_t bytes = 0;  // kPtr: size of the allocation behind ptr, 0 = unknown
   kapy_global g;      // global views, shared-memory tensors and register tensors alike
@@ -583,6 +585,28 @@ struct Interp {
     return rc;
   }
 
+  // result <- a one-instruction program over the tensor operands (ew < 0: none, the operand itself is stored; this is
+  // kapy.broadcast when the operand has extent 1 where the result does not)
+  int mapped_tensor(const Op &op, int n_operands, int ew, int dtype = 0, int rmode = KAPY_RN) {
+    Value in[3], r;
+    for (int k = 0; k < n_operands; ++k)
+      if (!get(op, k, Value::kTensor, in[k])) return KAPY_ERR_INVALID;
+    if (op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
+    kapy_ew_inst prog[5];
+    int n = 0;
+    for (int k = 0; k < n_operands; ++k) prog[n++] = {KAPY_EW_LD_GLOBAL, k, k, 0, 0, 0, KAPY_RN, 0.f};
+    int result = 0;
+    if (ew >= 0) {
+      prog[n++] = {ew, n_operands, 0, 1, 2, dtype, rmode, 0.f};
+      result = n_operands;
+    }
+    prog[n++] = {KAPY_EW_ST_GLOBAL, 0, result, 0, 0, 0, KAPY_RN, 0.f};
+    const kapy_global *ins[3] = {&in[0].g, &in[1].g, &in[2].g};
+    int rc = lib(op, kapy_elementwise(prog, n, ins, n_operands, &r.g, stream));
+    if (rc == KAPY_OK) env[op.results[0]] = r;
+    return rc;
+  }
+
   int run_ops(const std::vector<Op> &ops, std::vector<Value> *yielded) {
     for (const Op &op : ops) {
       int rc = run_op(op, yielded);
@@ -612,6 +636,9 @@ struct Interp {
         r.kind = Value::kInt;
         const std::string &w = op.words.empty() ? std::string("0") : op.words[0];
         r.i = w == "true" ? 1 : w == "false" ? 0 : atoll(w.c_str());
+      } else if (ty.kind == Type::kFloat) {
+        r.kind = Value::kFloat;
+        r.f = op.words.empty() ? 0.0 : atof(op.words[0].c_str());
       } else if (ty.kind == Type::kTensor) {
         if (!new_tensor(op, ty, r)) return KAPY_ERR_INVALID;
         const float v = op.words.empty() ? 0.f : (float)atof(op.words[0].c_str());
@@ -663,6 +690,42 @@ struct Interp {
     if (n == "arith.divf") return binary_tensor(op, KAPY_EW_DIVF);
     if (n == "arith.maximumf") return binary_tensor(op, KAPY_EW_MAXIMUMF);
     if (n == "arith.minimumf") return binary_tensor(op, KAPY_EW_MINIMUMF);
+    {
+      static const struct { const char *name; int ew; } unary[] = {
+          {"math.exp", KAPY_EW_EXP}, {"math.exp2", KAPY_EW_EXP2}, {"math.log", KAPY_EW_LOG}, {"math.log2", KAPY_EW_LOG2},
+          {"math.sqrt", KAPY_EW_SQRT}, {"math.rsqrt", KAPY_EW_RSQRT}, {"math.tanh", KAPY_EW_TANH}, {"math.erf", KAPY_EW_ERF},
+          {"math.absf", KAPY_EW_ABSF}, {"arith.negf", KAPY_EW_NEGF}};
+      for (auto &u : unary)
+        if (n == u.name) return mapped_tensor(op, 1, u.ew);
+    }
+    if (n == "math.fma") return mapped_tensor(op, 3, KAPY_EW_FMA);
+    if (n == "kapy.broadcast") return mapped_tensor(op, 1, -1);
+    if (n == "kapy.fptofp" || n == "arith.extf" || n == "arith.truncf") {
+      if (op.types.empty()) return fail_op(op, "cast without a result type");
+      int rmode = KAPY_RN;  // arith.truncf rounds to nearest even; kapy.fptofp carries its mode (Enums.td: rz = 0, rn = 1)
+      auto it = op.attrs.find("rounding_mode");
+      if (it != op.attrs.end()) rmode = (it->second == "0" || it->second.find("rz") != std::string::npos) ? KAPY_RZ : KAPY_RN;
+      return mapped_tensor(op, 1, KAPY_EW_FPTOFP, op.types.back().dtype, rmode);
+    }
+    if (n == "kapy.splat") {
+      Value v;
+      if (!get(op, 0, Value::kFloat, v) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
+      kapy_ew_inst prog[2] = {{KAPY_EW_SPLAT, 0, 0, 0, 0, op.types.back().dtype, KAPY_RN, (float)v.f}, {KAPY_EW_ST_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f}};
+      int rc = lib(op, kapy_elementwise(prog, 2, nullptr, 0, &r.g, stream));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
+    if (n == "kapy.transpose") {  // result[j, i] = source[i, j] (TransposeOpToLLVM.cpp:21-26 relabels; here the data moves)
+      if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
+      kapy_copy_cfg cfg;
+      memset(&cfg, 0, sizeof cfg);
+      cfg.transpose = 1;
+      int rc = lib(op, kapy_copy(&a.g, &r.g, &cfg, stream));
+      if (rc) return rc;
+      env[op.results[0]] = r;
+      return KAPY_OK;
+    }
     if (n == "kapy.mk_global") {
       Value off, s0, s1, t0, t1;
       if (!get(op, 0, Value::kPtr, a) || !get(op, 1, Value::kInt, off) || !get(op, 2, Value::kInt, s0) || !get(op, 3, Value::kInt, s1) ||
@@ -773,7 +836,8 @@ const char *const kSupportedOps[] = {
     "arith.divui", "arith.remui", "arith.cmpi", "arith.select", "arith.addf", "arith.subf", "arith.mulf", "arith.divf", "arith.maximumf",
     "arith.minimumf", "kapy.mk_global", "kapy.mk_shared", "kapy.sv_global", "kapy.sv_shared", "kapy.ld_global", "kapy.ld_matrix",
     "kapy.ld_shared", "kapy.st_global", "kapy.st_shared", "kapy.cp_async_global_to_shared", "kapy.cp_async_wait_group", "kapy.matmul",
-    "kapy.reduce", "nvvm.barrier0"};
+    "kapy.reduce", "nvvm.barrier0", "math.exp", "math.exp2", "math.log", "math.log2", "math.sqrt", "math.rsqrt", "math.tanh", "math.erf",
+    "math.absf", "math.fma", "arith.negf", "arith.extf", "arith.truncf", "kapy.fptofp", "kapy.splat", "kapy.broadcast", "kapy.transpose"};
 
 // Every op must be one this front-end executes; returns the number of ops, regions included, or -1.
 int count_ops(const std::vector<Op> &ops, bool in_reduce, std::string &err) {

@@ -180,3 +180,71 @@ def phases_program():
   }
 }
 """
+
+
+def softmax_program(rows_per_warp=2, cols=256, num_warps=2, dtype="f16"):
+    """out[r, :] = softmax(x[r, :]) computed in f32: fptofp up, reduce max, broadcast, subf, math.exp, reduce add,
+    broadcast, divf, fptofp down with round-to-nearest."""
+    t16, t32 = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype), "tensor<%dx%dxf32" % (rows_per_warp, cols)
+    c32 = "tensor<%dx1xf32, #values>" % rows_per_warp
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols])
+    body += """    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %x16 = kapy.ld_global %sx : {t16}, #global> -> {t16}, #values>
+    %xf = kapy.fptofp %x16 : {t16}, #values> to {t32}, #values>
+    %m = kapy.reduce %xf {{axis = 1 : i32}} lambda(%lhs: f32, %rhs: f32) {{
+      %r = arith.maximumf %lhs, %rhs : f32
+      kapy.return %r : f32
+    }} : {t32}, #values> -> {c32}
+    %mb = kapy.broadcast %m : {c32} -> {t32}, #values>
+    %d = arith.subf %xf, %mb : {t32}, #values>
+    %e = math.exp %d : {t32}, #values>
+    %s = kapy.reduce %e {{axis = 1 : i32}} lambda(%lhs: f32, %rhs: f32) {{
+      %r = arith.addf %lhs, %rhs : f32
+      kapy.return %r : f32
+    }} : {t32}, #values> -> {c32}
+    %sb = kapy.broadcast %s : {c32} -> {t32}, #values>
+    %q = arith.divf %e, %sb : {t32}, #values>
+    %y = kapy.fptofp %q {{rounding_mode = 1 : i32}} : {t32}, #values> to {t16}, #values>
+    kapy.st_global %y, %so : {t16}, #values>, {t16}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, t16=t16, t32=t32, c32=c32)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @softmax_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" + body + "  }\n}\n")
+
+
+def scaled_transpose_program(tile=32, scale=0.5, dtype="f16"):
+    """out[j, i] = x[i, j] * scale over tile x tile blocks, one block per program: ld_global, kapy.transpose, kapy.splat of
+    a scalar constant, mulf, st_global."""
+    t = "tensor<%dx%dx%s" % (tile, tile, dtype)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, tile])
+    body += """    %scale = arith.constant {scale:e} : {dtype}
+    %pi = kapy.program_id {{axis = 0 : i32}} : i32
+    %pj = kapy.program_id {{axis = 1 : i32}} : i32
+    %i0 = arith.muli %pi, %c{tile}_i32 : i32
+    %i1 = arith.addi %i0, %c{tile}_i32 : i32
+    %j0 = arith.muli %pj, %c{tile}_i32 : i32
+    %j1 = arith.addi %j0, %c{tile}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%m, %n] [%n, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%n, %m] [%m, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%i0 : %i1, %j0 : %j1] : {dyn} -> {t}, #global>
+    %so = kapy.sv_global %go[%j0 : %j1, %i0 : %i1] : {dyn} -> {t}, #global>
+    %v = kapy.ld_global %sx : {t}, #global> -> {t}, #values>
+    %vt = kapy.transpose %v : {t}, #values> -> {t}, #values>
+    %k = kapy.splat %scale : {dtype} -> {t}, #values>
+    %y = arith.mulf %vt, %k : {t}, #values>
+    kapy.st_global %y, %so : {t}, #values>, {t}, #global>
+    kapy.return
+""".format(tile=tile, scale=scale, dtype=dtype, dyn=dyn, t=t)
+    return (HEADER + "module attributes {kapy.num_warps = 1 : i64} {\n"
+            "  kapy.func public @scaled_transpose_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %m: i32, %n: i32) {\n" + body + "  }\n}\n")

@@ -14,6 +14,11 @@ def test_fixture_shaped_programs_parse():
     assert (n_args, warps) == (6, 4) and n_ops > 60
 
 
+def test_programs_with_casts_math_broadcast_transpose_and_splat_parse():
+    assert kh.parse_mlir(kp.softmax_program())[0] == 3
+    assert kh.parse_mlir(kp.scaled_transpose_program())[0] == 4
+
+
 def test_function_is_found_by_name():
     two = kp.binary_program().rstrip()[:-1] + kp.reduce_program().split("{\n", 1)[1]
     assert kh.parse_mlir(two, "reduce_kernel")[0] == 3
@@ -25,10 +30,10 @@ def test_function_is_found_by_name():
 
 
 def test_unsupported_op_is_named_with_its_line():
-    text = kp.binary_program().replace("arith.addf", "math.exp")
+    text = kp.binary_program().replace("arith.addf", "math.sin")
     with pytest.raises(kh.KapyError) as e:
         kh.parse_mlir(text)
-    assert e.value.status == -3 and "math.exp" in e.value.message and "line " in e.value.message
+    assert e.value.status == -3 and "math.sin" in e.value.message and "line " in e.value.message
 
 
 @pytest.mark.parametrize("damage", [

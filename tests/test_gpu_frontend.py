@@ -90,6 +90,29 @@ def test_matmul_program_matches_oracle(ko, bm, bn, bk, way, acc, M, N, K):
     assert rel <= (3e-4 if acc == "f16" else 1e-6), rel
 
 
+def test_softmax_program_in_kapy_ops_matches_the_oracle_program(ko):
+    rows_per_warp, cols, warps, programs = 2, 256, 2, 3
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 51, std=3.0)
+    want = np.zeros(rows * cols, np.uint16)
+    g = lambda a: ko.mk_global(a, rows, cols, cols, 1, ko.F16)
+    assert ko.elementwise(ko.program(kh.softmax_insts(kh.F16)), [g(x)], g(want)) == 0
+    dx, dout = to_dev(x), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.softmax_program(rows_per_warp, cols, warps), [dx, dout, rows], [programs])
+    sync()
+    assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # op by op in f32, one rounding to f16 at the end
+
+
+def test_transpose_splat_program_is_bit_exact(ko):
+    m, n, tile = 96, 64, 32
+    x = ko.fill_normal(m * n, ko.F16, 52)
+    dx, dout = to_dev(x), dev_zeros(m * n, 2, fill=0x7e00)
+    kh.run_mlir(kp.scaled_transpose_program(tile, 0.5), [dx, dout, m, n], [m // tile, n // tile])
+    sync()
+    want = (x.view(np.float16).reshape(m, n).T * np.float16(0.5)).astype(np.float16)
+    assert np.array_equal(to_host(dout, np.float16, (n, m)), want)
+
+
 def test_buffers_that_share_planned_memory_do_not_disturb_each_other(ko):
     x = ko.fill_normal(64 * 64, ko.F16, 41)
     d = to_dev(x)

@@ -56,7 +56,7 @@ def _events(fn, steps, warmup):
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the
 # same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
-MEASURED_TRAFFIC = {"gelu": 268414976, "transpose": 268456960}
+MEASURED_TRAFFIC = {"gelu": 268414976, "transpose": 268456960, "add": 402639872, "softmax": 268476416, "layernorm": 268788736}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -123,7 +123,7 @@ def bench_add(kh, steps, warmup, op="add"):
     nbytes = 3 * n * n * 2
     name = "elementwise_add fixture: z = x + y fp16 8192x8192" if op == "add" else "z = x*y + x (two roundings) fp16 8192x8192"
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev), "kernel": "affine_act_kernel" if op == "add" else "stack_kernel_narrow"}
+            "roofline": _roof_hbm(nbytes, ev, "add" if op == "add" else None), "kernel": "affine_act_kernel" if op == "add" else "stack_kernel_narrow"}
 
 
 def bench_reduce(kh, steps, warmup):
@@ -158,7 +158,7 @@ def bench_rowwise(kh, steps, warmup, which):
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]] + extra, gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
     return {"workload": "%s of every row, fp16 8192x8192, fp32 arithmetic" % which, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev),
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, which),
             "kernel": "softmax_kernel" if which == "softmax" else "norm_kernel"}
 
 

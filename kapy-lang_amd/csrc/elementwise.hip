@@ -103,6 +103,8 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
 // dependent step at a time), so the 16-bit-only form is held to 64 registers: 8 waves per SIMD.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void stack_kernel_narrow(StackProgram P) { stack_run<true>(P); }
 __global__ __launch_bounds__(256) void stack_kernel_any(StackProgram P) { stack_run<false>(P); }
+// rows whose width is not a multiple of 8 (row starts still 16-byte aligned): the last vector of a row moves element by element
+__global__ __launch_bounds__(256) void stack_kernel_narrow_ragged(StackProgram P) { stack_run<true, true>(P); }
 
 // ---------------------------------------------------------------------------------------------
 // out[i,j] = cast_out( act( f32(x[i,j]) * scale + f32(bias) ) ), x/out contiguous along j.
@@ -114,6 +116,7 @@ struct AffineActParams {
   int64_t x_stride0, out_stride0, bias_stride0;  // elements
   int32_t rows, vec_per_row;
   int32_t has_scale, bias_mode, act;  // act: a unary kapy_ew_op, or -1
+  int32_t width;                      // elements per row when the last vector of a row is partial, else 0
   int32_t combine;                    // how the second operand meets x*scale: Combine (plain binary programs; kAdd otherwise)
   float scale;
 };
@@ -197,7 +200,20 @@ __device__ __forceinline__ float affine_act(float x, float scale, float bias, in
 #ifndef KAPY_EW_NT
 #define KAPY_EW_NT 1
 #endif
-template <typename T, int ACT>
+// 16 bytes at ptr, or the first `valid` elements of them at the ragged end of a row (RAGGED kernels only)
+template <bool RAGGED>
+__device__ __forceinline__ u32x4 load_row16(const char *ptr, int valid, bool stream) {
+  if (RAGGED && valid < 8) return load16_partial(ptr, valid);
+  return stream ? __builtin_nontemporal_load((const u32x4 *)ptr) : *(const u32x4 *)ptr;
+}
+template <bool RAGGED>
+__device__ __forceinline__ void store_row16(char *ptr, u32x4 v, int valid) {
+  if (RAGGED && valid < 8) { store16_partial(ptr, v, valid); return; }
+  if (KAPY_EW_NT) __builtin_nontemporal_store(v, (u32x4 *)ptr);
+  else *(u32x4 *)ptr = v;
+}
+
+template <typename T, int ACT, bool RAGGED>
 __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
   constexpr int UNROLL = KAPY_EW_UNROLL;
   const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;
@@ -212,10 +228,10 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
     if (slot < total) {
       row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);
       col[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row) * 8;
-      const u32x4 *xp = (const u32x4 *)(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2);
-      xv[u] = KAPY_EW_NT ? __builtin_nontemporal_load(xp) : *xp;
-      if (p.bias_mode == kBiasRow) bv[u] = *(const u32x4 *)(p.bias + (int64_t)col[u] * 2);
-      else if (p.bias_mode == kBiasFull) bv[u] = *(const u32x4 *)(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2);
+      const int valid = RAGGED ? p.width - col[u] : 8;
+      xv[u] = load_row16<RAGGED>(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2, valid, KAPY_EW_NT);
+      if (p.bias_mode == kBiasRow) bv[u] = load_row16<RAGGED>(p.bias + (int64_t)col[u] * 2, valid, false);
+      else if (p.bias_mode == kBiasFull) bv[u] = load_row16<RAGGED>(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2, valid, false);
       else if (p.bias_mode == kBiasCol) {
         uint32_t h = *(const uint16_t *)(p.bias + (int64_t)row[u] * p.bias_stride0 * 2);
         h |= h << 16;
@@ -231,9 +247,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
     if (p.bias_mode != kNoBias) unpack8<T>(bv[u], b);
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, p.bias_mode != kNoBias ? b[e] : 0.f, p.act, p.combine);
-    u32x4 *op = (u32x4 *)(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2);
-    if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
-    else *op = pack8<T>(f);
+    store_row16<RAGGED>(p.out + ((int64_t)row[u] * p.out_stride0 + col[u]) * 2, pack8<T>(f), RAGGED ? p.width - col[u] : 8);
   }
 }
 
@@ -243,7 +257,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
 #ifndef KAPY_EW_ROWS
 #define KAPY_EW_ROWS 2
 #endif
-template <typename T, int ACT>
+template <typename T, int ACT, bool RAGGED>
 __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p) {
   constexpr int ROWS = KAPY_EW_ROWS;
   const int32_t chunk = blockIdx.x * 256 + threadIdx.x;
@@ -251,14 +265,12 @@ __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p)
   const int32_t col = chunk * 8, row0 = blockIdx.y * ROWS;
   const float scale = p.has_scale ? p.scale : 1.0f;
   float b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (p.bias_mode == kBiasRow) unpack8<T>(*(const u32x4 *)(p.bias + (int64_t)col * 2), b);
+  const int valid = RAGGED ? p.width - col : 8;
+  if (p.bias_mode == kBiasRow) unpack8<T>(load_row16<RAGGED>(p.bias + (int64_t)col * 2, valid, false), b);
   u32x4 xv[ROWS];
 #pragma unroll
   for (int u = 0; u < ROWS; ++u)
-    if (row0 + u < p.rows) {
-      const u32x4 *xp = (const u32x4 *)(p.x + ((int64_t)(row0 + u) * p.x_stride0 + col) * 2);
-      xv[u] = KAPY_EW_NT ? __builtin_nontemporal_load(xp) : *xp;
-    }
+    if (row0 + u < p.rows) xv[u] = load_row16<RAGGED>(p.x + ((int64_t)(row0 + u) * p.x_stride0 + col) * 2, valid, KAPY_EW_NT);
 #pragma unroll
   for (int u = 0; u < ROWS; ++u) {
     if (row0 + u >= p.rows) break;
@@ -266,9 +278,7 @@ __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p)
     unpack8<T>(xv[u], f);
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = affine_act<ACT>(f[e], scale, b[e], p.act, p.combine);
-    u32x4 *op = (u32x4 *)(p.out + ((int64_t)(row0 + u) * p.out_stride0 + col) * 2);
-    if (KAPY_EW_NT) __builtin_nontemporal_store(pack8<T>(f), op);
-    else *op = pack8<T>(f);
+    store_row16<RAGGED>(p.out + ((int64_t)(row0 + u) * p.out_stride0 + col) * 2, pack8<T>(f), valid);
   }
 }
 
@@ -467,9 +477,9 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
   const kapy_global *x = ins[x_in];
   if (x->dtype != T || x->stride1 != 1 || out->stride1 != 1) return false;
   const int64_t o0 = extent0(out), o1 = extent1(out);
-  if (extent0(x) != o0 || extent1(x) != o1 || o1 % 8 != 0) return false;
+  if (extent0(x) != o0 || extent1(x) != o1) return false;
   if (vector_bytes(x, 1) != 16 || vector_bytes(out, 1) != 16) return false;
-  if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  if (o0 * ((o1 + 7) / 8) >= (int64_t(1) << 31) - 1024) return false;
   p->bias_mode = kNoBias;
   p->bias = nullptr;
   p->bias_stride0 = 0;
@@ -488,7 +498,8 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
   p->x_stride0 = x->stride0;
   p->out_stride0 = out->stride0;
   p->rows = (int32_t)o0;
-  p->vec_per_row = (int32_t)(o1 / 8);
+  p->vec_per_row = (int32_t)((o1 + 7) / 8);
+  p->width = o1 % 8 ? (int32_t)o1 : 0;
   *elem_dtype = T;
   return true;
 }
@@ -537,8 +548,14 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
   // the result: rows contiguous, 8 elements at a time
   const int64_t o0 = extent0(out), o1 = extent1(out);
   const int ob = dtype_bytes(out->dtype);
-  if (!is_float(out->dtype) || out->stride1 != 1 || o1 % 8 != 0 || ((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
-  if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  if (!is_float(out->dtype) || out->stride1 != 1 || ((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
+  if (o1 % 8 != 0) {  // a ragged last vector per row: the 16-bit kernel has a form for it
+    bool narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
+    for (int k = 0; k < n_ins; ++k) narrow = narrow && (ins[k]->dtype == KAPY_F16 || ins[k]->dtype == KAPY_BF16);
+    for (int k = 0; k < n_inst; ++k) narrow = narrow && !is_f8(result_dtype[k]);
+    if (!narrow) return false;
+  }
+  if (o0 * ((o1 + 7) / 8) >= (int64_t(1) << 31) - 1024) return false;
   for (int k = 0; k < n_ins; ++k) {
     const kapy_global *g = ins[k];
     StackIn &in = P->in[k];
@@ -604,7 +621,8 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
   P->out_stride0 = out->stride0;
   P->out_dtype = out->dtype;
   P->rows = (int32_t)o0;
-  P->vec_per_row = (int32_t)(o1 / 8);
+  P->vec_per_row = (int32_t)((o1 + 7) / 8);
+  P->width = o1 % 8 ? (int32_t)o1 : 0;
   return true;
 }
 
@@ -667,8 +685,10 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
                      : dim3((slots + 256 * KAPY_EW_UNROLL - 1) / (256 * KAPY_EW_UNROLL));
 #define KAPY_LAUNCH_AFFINE(TT, AA)                                                     \
   do {                                                                                 \
-    if (cols) affine_act_cols_kernel<TT, AA><<<grid, 256, 0, s>>>(ap);                 \
-    else affine_act_kernel<TT, AA><<<grid, 256, 0, s>>>(ap);                           \
+    if (cols && ap.width) affine_act_cols_kernel<TT, AA, true><<<grid, 256, 0, s>>>(ap);  \
+    else if (cols) affine_act_cols_kernel<TT, AA, false><<<grid, 256, 0, s>>>(ap);     \
+    else if (ap.width) affine_act_kernel<TT, AA, true><<<grid, 256, 0, s>>>(ap);       \
+    else affine_act_kernel<TT, AA, false><<<grid, 256, 0, s>>>(ap);                    \
   } while (0)
     if (T == KAPY_F16) {
       if (ap.act == KAPY_EW_GELU_TANH) KAPY_LAUNCH_AFFINE(_Float16, KAPY_EW_GELU_TANH);
@@ -692,7 +712,8 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
       bool narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
       for (int k = 0; k < n_ins; ++k) narrow = narrow && (ins[k]->dtype == KAPY_F16 || ins[k]->dtype == KAPY_BF16);
       for (int k = 0; k < n_inst; ++k) narrow = narrow && !is_f8(result_dtype[k]);
-      if (narrow) stack_kernel_narrow<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
+      if (narrow && SP.width) stack_kernel_narrow_ragged<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
+      else if (narrow) stack_kernel_narrow<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
       else stack_kernel_any<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
       KAPY_HIP_CHECK(hipGetLastError());
       return KAPY_OK;

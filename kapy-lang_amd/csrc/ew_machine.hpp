@@ -35,6 +35,7 @@ struct StackProgram {
   int64_t out_stride0;
   int32_t n_post, n_ins, out_dtype, rows, vec_per_row;
   int32_t n_tmps;  // row machine only: values used more than once, parked in LDS
+  int32_t width;   // elements per row when the last vector of a row is partial (ragged kernels), else 0
 };
 
 // Compiles a verified program that contains a reduce for the row machine and launches it (elementwise_row.hip).
@@ -99,6 +100,21 @@ __device__ __forceinline__ void widen16x8(u32x4 v, int dtype, float f[8]) {
     }
   }
 }
+// The ragged end of a row of 16-bit elements: only the first `valid` (1..7) elements of the vector at p exist; a whole
+// 16-byte access would reach past the view (and possibly past its allocation), so they move one by one.
+__device__ __forceinline__ u32x4 load16_partial(const char *p, int valid) {
+  u32x4 v = {0, 0, 0, 0};
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    if (e < valid) v[e >> 1] |= (uint32_t)((const uint16_t *)p)[e] << (16 * (e & 1));
+  return v;
+}
+__device__ __forceinline__ void store16_partial(char *p, u32x4 v, int valid) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    if (e < valid) ((uint16_t *)p)[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+}
+
 // The 8 elements of vector jv of row i of a full-extent operand, as they lie in memory (16, 32 or 8 bytes).
 struct Raw8 {
   u32x4 lo, hi;
@@ -210,20 +226,36 @@ __device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const
 // third operand of an fma in value D+2; D is a template parameter so that no register is indexed.
 // NARROW: every operand, every intermediate type and the result are f16 / bf16 / f32-from-16-bit
 // (no fp8, no fp32 in memory): the common case, and it needs far fewer registers.
-template <int D, bool NARROW>
+template <int D, bool NARROW, bool RAGGED = false>
 __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &I, int32_t i, int32_t jv, float (&v)[3][8]) {
   constexpr int R = D + 1 < 3 ? D + 1 : 2, T = D + 2 < 3 ? D + 2 : 2;
   float *x = v[D];
   const float *y = v[R], *z = v[T];
   switch (I.op) {
-  case kPushIn: load8<NARROW>(P.in[I.a], i, jv, x); return;
+  case kPushIn:
+    if (RAGGED && NARROW && P.in[I.a].kind <= kInRow && (jv + 1) * 8 > P.width) {
+      const StackIn &g = P.in[I.a];
+      widen16x8(load16_partial(g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * 2, P.width - jv * 8), g.dtype, x);
+      return;
+    }
+    load8<NARROW>(P.in[I.a], i, jv, x);
+    return;
   case kPushImm: {
     const float c = round_to_dtype(I.imm, I.dtype, true);
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = c;
     return;
   }
-  case kStore: store8<NARROW>(P.out, P.out_dtype, (int64_t)i * P.out_stride0 + (int64_t)jv * 8, x); return;
+  case kStore:
+    if (RAGGED && NARROW && (jv + 1) * 8 > P.width) {
+      u32x4 v;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) v[w] = P.out_dtype == KAPY_F16 ? pack2_f16_rn(x[2 * w], x[2 * w + 1]) : pack2_bf16_rn(x[2 * w], x[2 * w + 1]);
+      store16_partial(P.out + ((int64_t)i * P.out_stride0 + (int64_t)jv * 8) * 2, v, P.width - jv * 8);
+      return;
+    }
+    store8<NARROW>(P.out, P.out_dtype, (int64_t)i * P.out_stride0 + (int64_t)jv * 8, x);
+    return;
   case kCast: round8<NARROW>(x, I.dtype, I.rmode != KAPY_RZ); return;
   case KAPY_EW_ADDF:
 #pragma unroll
@@ -268,7 +300,7 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
   if (I.dtype != KAPY_F32) round8<NARROW>(x, I.dtype, true);
 }
 
-template <bool NARROW>
+template <bool NARROW, bool RAGGED = false>
 __device__ __forceinline__ void stack_run(const StackProgram &P) {
   const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (slot >= (int64_t)P.rows * P.vec_per_row) return;
@@ -281,9 +313,9 @@ __device__ __forceinline__ void stack_run(const StackProgram &P) {
   for (int pc = 0; pc < P.n_post; ++pc) {
     const PostOp I = P.post[pc];
     switch (I.slot) {
-    case 0: stack_step<0, NARROW>(P, I, i, jv, v); break;
-    case 1: stack_step<1, NARROW>(P, I, i, jv, v); break;
-    default: stack_step<2, NARROW>(P, I, i, jv, v);
+    case 0: stack_step<0, NARROW, RAGGED>(P, I, i, jv, v); break;
+    case 1: stack_step<1, NARROW, RAGGED>(P, I, i, jv, v); break;
+    default: stack_step<2, NARROW, RAGGED>(P, I, i, jv, v);
     }
   }
 }

@@ -222,6 +222,39 @@ def test_register_stack_kernel_tree_shapes_and_operand_kinds(ko):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("width", [8, 9, 15, 1001, 2046])
+@pytest.mark.parametrize("which", ["gelu row bias", "gelu full bias", "x + y", "x*y + x"])
+def test_rows_with_a_ragged_last_vector_keep_the_fast_kernels_and_stay_inside_the_view(ko, width, which):
+    """Views whose rows start 16-byte aligned but whose width is not a multiple of 8 (a sub-view of a wider tensor): the
+    last vector of every row moves element by element; nothing outside the view is read into the result or written."""
+    m, pitch = 37, 2048
+    xp = ko.fill_normal(m * pitch, kh.F16, 101).reshape(m, pitch)
+    yp = ko.fill_normal(m * pitch, kh.F16, 102).reshape(m, pitch)
+    bias = ko.fill_normal(pitch, kh.F16, 103)
+    sentinel = 0x1234
+    want_p = np.full((m, pitch), sentinel, np.uint16)
+    view = lambda lib, a, rows=m: lib.mk_global(a, rows, width, pitch, 1, kh.F16)
+    if which.startswith("gelu"):
+        insts_k, insts_o = kh.gelu_program(kh.F16, 0.5), ko.gelu_program(kh.F16, kh.F16)
+        second_np, second_rows = (bias, 1) if which == "gelu row bias" else (yp, m)
+    else:
+        body = [dict(op=kh.EW_ADDF, dst=2, a=0, b=1)] if which == "x + y" else [dict(op=kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ADDF, dst=2, a=2, b=0)]
+        insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1)] + body + [dict(op=kh.EW_ST_GLOBAL, a=2)]
+        insts_k, insts_o = kh.program(insts), ko.program(insts)
+        second_np, second_rows = yp, m
+    assert ko.elementwise(insts_o, [view(ko, xp), view(ko, second_np, second_rows)], view(ko, want_p)) == 0
+    dx, d2, dout = to_dev(xp), to_dev(second_np), dev_zeros(m * pitch, 2, fill=sentinel)
+    dv = lambda t, rows=m: dglobal(t, rows, width, pitch, 1, kh.F16)
+    kh.elementwise(insts_k, [dv(dx), dv(d2, second_rows)], dv(dout))
+    sync()
+    got = to_host(dout, np.uint16, (m, pitch))
+    assert np.all(got[:, width:] == sentinel)
+    if which.startswith("gelu"):
+        _check_ulp(got[:, :width], want_p[:, :width], kh.F16)
+    else:
+        assert np.array_equal(got[:, :width], want_p[:, :width])
+
+
 @pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
 @pytest.mark.parametrize("op", ["EW_ADDF", "EW_SUBF", "EW_MULF", "EW_MAXIMUMF", "EW_MINIMUMF"])
 def test_plain_binary_programs_are_bit_exact_in_every_operand_shape(ko, dtype, op):

@@ -215,7 +215,7 @@ struct PackedEpilogue {
 #pragma unroll
       for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
         float rs = 1.0f;
-        if constexpr (SCALED) rs = p.row_scale[m_wave + i * 32 + bi * KM + wrow];
+        if constexpr (SCALED) rs = p.row_scale[min(m_wave + i * 32 + bi * KM + wrow, p.M - 1)];  // (rows past M exist only in tiles that hang over the edge; they are not stored)
 #pragma unroll
         for (int j = 0; j < kTn; ++j)
 #pragma unroll
@@ -224,7 +224,7 @@ struct PackedEpilogue {
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
             if constexpr (SCALED) {
-              const f32x4 cs = *(const f32x4 *)(p.col_scale + n_wave + j * KM + wcol + kQuadStep * q);
+              const f32x4 cs = *(const f32x4 *)(p.col_scale + min(n_wave + j * KM + wcol + kQuadStep * q, p.N - 4));
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
             }
@@ -240,7 +240,9 @@ struct PackedEpilogue {
       for (int t = 0; t < kStores; ++t) {
         const int row = t * kRowsPerStore + rrow;
         const u32x4 w = *(const u32x4 *)(strip + row * kRowStride + rchunk * 16);
-        *(u32x4 *)(p.d + ((int64_t)(m_wave + i * 32 + row) * p.d_sm + n_wave + rchunk * 8) * 2) = w;
+        // a tile may hang over the result's last rows and columns (N a multiple of 8: a 16-byte piece is in or out whole)
+        if (m_wave + i * 32 + row < p.M && n_wave + rchunk * 8 < p.N)
+          *(u32x4 *)(p.d + ((int64_t)(m_wave + i * 32 + row) * p.d_sm + n_wave + rchunk * 8) * 2) = w;
       }
     }
   }
@@ -297,7 +299,7 @@ struct TnConfig {
   static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % T::kSliceK == 0 && 32 % T::kM == 0, "wave tile must be a multiple of the MFMA tile");
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false>
 __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
   using L = TileLayout<C::kRowBytes>;
@@ -366,7 +368,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       for (int j = 0; j < C::kTn; ++j) acc[i][j] = zero;
   }
 
-  const int KT = p.K / BK;
+  const int KT = (p.K + BK - 1) / BK;  // (a partial last tile only in the ring variant)
 #ifdef KAPY_TRACE
   // tuning builds only: clock stamps of workgroup 0 for K-tiles 32..39 (8 per tile per wave)
   uint64_t *trace = p.row_scale ? nullptr : (uint64_t *)p.col_scale;
@@ -449,22 +451,49 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
       return (void *)(((uint64_t)hi << 32) | lo);
     };
-    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(a_tile), 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(b_tile), 0, 0x7fffffff, 0x00020000);
+    // The descriptors end where the operands end: in a tile that hangs over the last row of the lhs (M not a multiple
+    // of BM) or of the rhs, the loads of the rows that do not exist are out of range, which the hardware answers with
+    // zeros in LDS instead of a fault.  (An operand with 2 GiB or more behind the tile base has all of the tile's rows.)
+    auto bytes_left = [&](int32_t rows, int64_t pitch) {
+      const int64_t left = rows <= 0 ? 0 : ((int64_t)(rows - 1) * pitch + p.K) * EB;
+      return (int)(left < 0x7fffffff ? left : 0x7fffffff);
+    };
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(a_tile), 0, __builtin_amdgcn_readfirstlane(bytes_left(p.M - m0, p.a_sm)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(b_tile), 0, __builtin_amdgcn_readfirstlane(bytes_left(p.N - n0, p.b_sn)), 0x00020000);
     const int wave_lds = wave * 1024;
     auto wrap = [](auto pos) { return pos >= 20 ? pos - 20 : (pos >= 10 ? pos - 10 : pos); };
-    // scalar byte offset of K-tile j in a row, clamped to the last real tile
-    auto k_off = [&](int j) { return min(j, KT - 1) * (BK * EB); };
+    // K need not be a multiple of BK (only of the 16 bytes of a chunk): the last tile is then partial, and the lanes
+    // whose chunk lies past K ask for an offset beyond any descriptor, which the hardware answers with zeros in LDS.
+    // Which chunk of a row a lane fetches is the same for every load it issues (the swizzle only mixes in the bit of
+    // the load index that is the wavefront's own), so one mask serves all of them.
+    const int k_last = (KT - 1) * BK;
+    bool lane_past_k;
+    {
+      uint32_t row, chunk;
+      L::locate((uint32_t)wave * 1024u + lane * 16u, row, chunk);
+      lane_past_k = k_last + (int)(chunk * (16 / EB)) >= p.K;
+    }
+    constexpr int kTailFlag = (int)0x80000000;
+    // (only the KTAIL build of the kernel pays the select and the mask: they cost 2 % of the aligned case)
+#define KAPY_VOFF(g) ((KTAIL && soff < 0 && lane_past_k) ? kTailFlag : (int)(g))
+#define KAPY_SOFF (KTAIL ? (soff & ~kTailFlag) : soff)
+    // scalar byte offset of K-tile j in a row, clamped to the last real tile; the sign bit marks a partial tile
+    auto k_off = [&](int j) {
+      const int jj = min(j, KT - 1);
+      return jj * (BK * EB) | ((KTAIL && jj == KT - 1 && k_last + BK > p.K) ? kTailFlag : 0);
+    };
     auto load_a = [&](int idx, int pos_of_unit0, int soff) {  // idx: 0 .. kHalf-1, unit idx / kPerUnit
       const int u = idx / kPerUnit, i = idx % kPerUnit;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + wrap(pos_of_unit0 + u) * kUnit + i * C::kWaves * 1024 + wave_lds),
-                                               16, (int)a_goff[idx], soff, 0, 0);
+                                               16, KAPY_VOFF(a_goff[idx]), KAPY_SOFF, 0, 0);
     };
     auto load_b = [&](int idx, int pos_of_unit2, int soff) {
       const int u = idx / kPerUnit, i = idx % kPerUnit;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + wrap(pos_of_unit2 + u) * kUnit + i * C::kWaves * 1024 + wave_lds),
-                                               16, (int)b_goff[idx], soff, 0, 0);
+                                               16, KAPY_VOFF(b_goff[idx]), KAPY_SOFF, 0, 0);
     };
+#undef KAPY_VOFF
+#undef KAPY_SOFF
     // Load `slot` (0 .. kLoadsPerTile-1) of the sequence issued after the barrier of the tile at ring
     // position pos0: slots [0, kHalf) = rhs units of the tile two ahead (they take positions pos0,
     // pos0+1), the rest = lhs units of the tile three ahead (positions pos0+2, pos0+3).
@@ -1045,10 +1074,10 @@ bool packed_epilogue(const GemmParams &p) {
          ((uintptr_t)p.d & 15) == 0 && (p.d_sm * 2) % 16 == 0 && (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false>
 int launch_tn_epi(GemmParams p, hipStream_t s) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
-  auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED>;
+  auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED, KTAIL>;
   // The kernel addresses kLdsBytes of dynamic LDS (more than the 64 KiB default limit), also through
   // LDS-direct loads, which fault when they land outside the allocation.  Make sure the limit has
   // really been raised before the first launch: query first (this also forces the code object to be
@@ -1067,8 +1096,8 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
     }
     configured = true;
   }
-  p.tiles_m = p.M / BM;
-  p.tiles_n = p.N / BN;
+  p.tiles_m = (p.M + BM - 1) / BM;  // (only the ring variants are launched with tiles that hang over an edge)
+  p.tiles_n = (p.N + BN - 1) / BN;
   kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(C::kThreads), C::kLdsBytes, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
@@ -1076,8 +1105,15 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 int launch_tn(const GemmParams &p, hipStream_t s) {
-  return packed_epilogue(p) ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s)
-                            : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
+  // a result that ends inside a 16-byte piece of a row takes the bounds-checked element stores
+  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || (STAGES == kRing25 && p.N % 8 == 0);
+  if constexpr (STAGES == kRing25) {
+    if (p.K % BK)  // a partial last K-tile: the build of the kernel that masks the lanes past K
+      return packed_epilogue(p) && whole_tiles ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true, true>(p, s)
+                                               : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false, true>(p, s);
+  }
+  return packed_epilogue(p) && whole_tiles ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s)
+                                           : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
 }
 
 template <typename T, int BK, int STAGES>
@@ -1200,6 +1236,8 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
     return launch_f8<256, 256, 128, 2, 2, KAPY_F8_STAGES>(p, lhs_fmt, rhs_fmt, s);
   if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
+  // extents that are not multiples of a tile: the ring variant, whose loads are bounded by the operands' ends
+  if (KAPY_F8_STAGES == kRing25 && p.K % 16 == 0 && p.K >= 128 && p.M >= 128 && p.N >= 128) return launch_f8<256, 256, 128, 2, 2, KAPY_F8_STAGES>(p, lhs_fmt, rhs_fmt, s);
   return KAPY_ERR_UNSUPPORTED;
 }
 
@@ -1267,7 +1305,10 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
           (c.stages && c.stages != v.stages) || (c.waves && c.waves != v.waves) ||
           (c.impl_way == KAPY_MFMA_32X32X16_16B && v.mfma != 32) || (c.impl_way == KAPY_MFMA_16X16X32_16B && v.mfma != 16))
         continue;
-      if (p.M % v.bm || p.N % v.bn || p.K % v.bk) continue;
+      // the ring variants' bounded loads let a tile hang over the last rows of either operand; the others need whole tiles
+      const bool whole_tiles = p.M % v.bm == 0 && p.N % v.bn == 0;
+      const bool whole_k = p.K % v.bk == 0;  // the ring variants also take a partial last K-tile of whole 16-byte chunks
+      if ((!whole_k && (v.stages != kRing25 || p.K % 8)) || (!whole_tiles && v.stages != kRing25)) continue;
       // with a free choice, a 256x256 tiling that cannot occupy half of the CUs yields to 128x128
       if (free_choice && v.bm == 256 && (int64_t)(p.M / v.bm) * (p.N / v.bn) * 2 < device_cus() && p.M % 128 == 0 && p.N % 128 == 0)
         continue;

@@ -43,7 +43,8 @@ def test_scaled_f8_small(ko, M, N, K):
     assert _frob(ko, to_host(dd, np.uint16, (M, N)), want) <= FROB_TOL
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (128, 256, 384), (256, 256, 256), (384, 128, 512), (512, 768, 1024), (1024, 2560, 256)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (128, 256, 384), (256, 256, 256), (384, 128, 512), (512, 768, 1024), (1024, 2560, 256),
+                                   (300, 520, 256), (1000, 136, 384), (129, 1001, 128), (300, 520, 272), (256, 256, 144)])   # tiles hang over the edges of M, N and K
 def test_scaled_f8_tiled_kernel(ko, M, N, K):
     """Rows >= 128 and extents multiples of the tile: the LDS-direct MFMA kernel (128- and 256-wide tiles)."""
     aq, sa, wq, sb = _quantised(ko, M, N, K, seed=3)

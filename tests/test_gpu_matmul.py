@@ -194,3 +194,28 @@ def test_config4_bf16_8192_sampled_against_oracle(ko):
     g1 = (got.astype(np.uint32) << 16).view(np.float32)
     g2 = (got2.astype(np.uint32) << 16).view(np.float32)
     assert np.array_equal(g2, 2 * g1)
+
+
+@pytest.mark.parametrize("dt", [kh.BF16, kh.F16])
+@pytest.mark.parametrize("M,N,K", [(300, 512, 256), (513, 264, 192), (1000, 1000, 128), (257, 255 + 1, 64), (130, 777 + 7, 320),
+                                   (256, 256, 72), (300, 520, 200), (512, 256, 8), (640, 384, 1000)])   # the last four: a partial last K-tile
+def test_extents_that_are_not_multiples_of_the_tile_stay_on_the_ring_kernel(ko, dt, M, N, K):
+    """K-contiguous operands, K a multiple of 8 (whole 16-byte chunks), M and N anything: tiles hang over the last rows of
+    the operands, whose loads the buffer descriptors bound, and over the end of K, where the lanes past it fetch zeros;
+    nothing is written outside the result."""
+    a, b = ko.fill_normal(M * K, dt, 7, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 7, 1, 0.0, 0.5)
+    want = np.zeros(M * N, dtype=np.uint16)
+    assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, K, 1, dt)), C.byref(ko.mk_global(b, K, N, 1, K, dt)), None,
+                              C.byref(ko.mk_global(want, M, N, N, 1, dt)), kh.RN) == 0
+    pad = 4096
+    da, db, dd = to_dev(a), to_dev(b), dev_zeros(M * N + pad, 2, fill=0x1234)
+    kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd, M, N, N, 1, dt))
+    sync()
+    got = to_host(dd, np.uint16)
+    assert np.all(got[M * N:] == 0x1234)
+    assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL
+    # the same through the kernel that is asked for by name: it must be the ring variant that serves it
+    dd2 = dev_zeros(M * N, 2)
+    kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd2, M, N, N, 1, dt), tile=(256, 256, 64), stages=25)
+    sync()
+    assert np.array_equal(to_host(dd2, np.uint16), got[:M * N])

@@ -1206,7 +1206,8 @@ struct TnVariant {
   { BM, BN, BK, (WM) * (WN), S, 16, launch_tn<Bf16M16, BM, BN, BK, WM, WN, S>, launch_tn<F16M16, BM, BN, BK, WM, WN, S> }
 const TnVariant kTnVariants[] = {
     KAPY_TN16(256, 256, 64, 2, 2, kRing25), KAPY_TN16(256, 256, 64, 2, 2, 2),
-    KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
+    KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN16(128, 128, 64, 2, 2, kRing25),
+    KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
 #ifdef KAPY_TUNING
     KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2), KAPY_TN(256, 128, 64, 2, 2, 3),
     KAPY_TN(128, 256, 64, 2, 2, 3), KAPY_TN(128, 128, 64, 2, 2, 4), KAPY_TN(256, 256, 32, 2, 2, 5), KAPY_TN(256, 128, 32, 2, 2, 4),
@@ -1309,9 +1310,8 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
       const bool whole_tiles = p.M % v.bm == 0 && p.N % v.bn == 0;
       const bool whole_k = p.K % v.bk == 0;  // the ring variants also take a partial last K-tile of whole 16-byte chunks
       if ((!whole_k && (v.stages != kRing25 || p.K % 8)) || (!whole_tiles && v.stages != kRing25)) continue;
-      // with a free choice, a 256x256 tiling that cannot occupy half of the CUs yields to 128x128
-      if (free_choice && v.bm == 256 && (int64_t)(p.M / v.bm) * (p.N / v.bn) * 2 < device_cus() && p.M % 128 == 0 && p.N % 128 == 0)
-        continue;
+      // with a free choice, a 256x256 tiling with fewer tiles than CUs yields to 128x128
+      if (free_choice && v.bm == 256 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) < device_cus()) continue;
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }

@@ -82,7 +82,7 @@ def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):
 
 MFMA16, MFMA32 = 17, 16   # KAPY_MFMA_16X16X32_16B, KAPY_MFMA_32X32X16_16B
 TN_VARIANTS = [((256, 256, 64), 25, MFMA16), ((256, 256, 64), 2, MFMA16), ((256, 256, 64), 25, MFMA32), ((256, 256, 64), 2, MFMA32),
-               ((256, 256, 32), 4, MFMA32), ((128, 128, 64), 2, MFMA32), ((128, 128, 32), 4, MFMA32)]
+               ((256, 256, 32), 4, MFMA32), ((128, 128, 64), 25, MFMA16), ((128, 128, 64), 2, MFMA32), ((128, 128, 32), 4, MFMA32)]
 
 
 @pytest.mark.parametrize("tile,stages,impl_way", TN_VARIANTS)
@@ -214,8 +214,9 @@ def test_extents_that_are_not_multiples_of_the_tile_stay_on_the_ring_kernel(ko, 
     got = to_host(dd, np.uint16)
     assert np.all(got[M * N:] == 0x1234)
     assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL
-    # the same through the kernel that is asked for by name: it must be the ring variant that serves it
-    dd2 = dev_zeros(M * N, 2)
-    kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd2, M, N, N, 1, dt), tile=(256, 256, 64), stages=25)
-    sync()
-    assert np.array_equal(to_host(dd2, np.uint16), got[:M * N])
+    # the same through the ring variants asked for by name (both tile sizes take ragged extents)
+    for tile in ((256, 256, 64), (128, 128, 64)):
+        dd2 = dev_zeros(M * N, 2)
+        kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd2, M, N, N, 1, dt), tile=tile, stages=25)
+        sync()
+        assert _frob(ko, to_host(dd2, np.uint16), want, dt) <= FROB_TOL, tile

@@ -809,7 +809,11 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (void *)(((uint64_t)hi << 32) | lo);
   };
-  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm * 2), 0, 0x7fffffff, 0x00020000);
+  // The lhs descriptor ends where the lhs ends: a tile that hangs over its last rows (M not a multiple of 128) gets zeros
+  // for the rows that do not exist (their per-lane offsets are out of range) instead of a fault.
+  const int64_t a_left = ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2;
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm * 2), 0,
+                                                                          __builtin_amdgcn_readfirstlane((int)(a_left < 0x7fffffff ? a_left : 0x7fffffff)), 0x00020000);
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * 2), 0, 0x7fffffff, 0x00020000);
   const int wave_lds = wave * 1024;
   // load `idx` (lhs first, then rhs) of K-tile j into its stage
@@ -1119,7 +1123,7 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
 template <typename T, int BK, int STAGES>
 int launch_nn(GemmParams p, hipStream_t s) {
   constexpr int kLds = STAGES * BK * 512;
-  p.tiles_m = p.M / kNBM;
+  p.tiles_m = (p.M + kNBM - 1) / kNBM;  // M need not be a multiple of the tile: see the kernel's lhs descriptor
   p.tiles_n = p.N / kNBN;
   const bool packed = packed_epilogue(p);
   const void *kernel = packed ? (const void *)nn_kernel<T, BK, STAGES, true> : (const void *)nn_kernel<T, BK, STAGES, false>;
@@ -1316,7 +1320,7 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
     }
   }
   // Both operands row-major (the reference fixture's layout, matmul.mlir): the transposing-read kernel.
-  bool nn = p.a_sk == 1 && p.b_sn == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 1) == 16 && p.M % kNBM == 0 && p.N % kNBN == 0 &&
+  bool nn = p.a_sk == 1 && p.b_sn == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 1) == 16 && p.M > 0 && p.N % kNBN == 0 &&
             p.K > 0 && p.a_sm >= 0 && p.b_sk >= 0 && p.a_sm * 2 * kNBM < (int64_t(1) << 31) && (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31) &&
             c.impl_way != KAPY_MFMA_32X32X16_16B && (!c.tile_m || c.tile_m == kNBM) && (!c.tile_n || c.tile_n == kNBN) && (!c.waves || c.waves == 4);
   if (nn) {

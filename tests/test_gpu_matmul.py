@@ -59,7 +59,8 @@ def test_nn_transposing_read_kernel_every_variant(ko, tile_k, stages):
     """Both operands row-major, extents multiples of 128 x 128 x tile_k: the kernel that stages the rhs as it lies in
     memory and transposes on the way out of LDS; K of 1, 2, 3, 7 and 16 tiles (prologue, ring wrap, fragment parity)."""
     for dt in (kh.BF16, kh.F16):
-        for (M, N, K) in ((128, 128, tile_k), (128, 256, 2 * tile_k), (256, 128, 3 * tile_k), (128, 128, 7 * tile_k), (384, 256, 16 * tile_k)):
+        for (M, N, K) in ((128, 128, tile_k), (128, 256, 2 * tile_k), (256, 128, 3 * tile_k), (128, 128, 7 * tile_k), (384, 256, 16 * tile_k),
+                          (200, 128, 4 * tile_k), (1, 256, 2 * tile_k), (333, 128, 5 * tile_k)):   # the last three: a tile hangs over the last rows of the lhs
             got, want = _run(ko, dt, M, N, K, True, True, seed=7, tile=(128, 128, tile_k), stages=stages)
             assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
     got32, want32 = _run(ko, kh.F16, 256, 256, 8 * tile_k, True, True, out_dtype=kh.F32, with_acc=kh.F32, seed=7, tile=(128, 128, tile_k), stages=stages)

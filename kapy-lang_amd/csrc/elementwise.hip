@@ -582,6 +582,23 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     else need[id] = need[n.a];
   }
   if (need[stored] > 3) return false;
+  // how often each value is used: one with several uses is copied from lower on the stack when it is still there
+  // (otherwise it is evaluated again: every op is pure)
+  std::vector<int> uses(nodes.size(), 0);
+  {
+    std::vector<char> reached(nodes.size(), 0);
+    std::function<void(int)> visit = [&](int id) {
+      ++uses[id];
+      if (reached[id]) return;
+      reached[id] = 1;
+      const N &n = nodes[id];
+      if (n.a >= 0) visit(n.a);
+      if (n.b >= 0) visit(n.b);
+      if (n.c >= 0) visit(n.c);
+    };
+    visit(stored);
+  }
+  int holder[3] = {-1, -1, -1};  // which node's value each stack slot holds
   int count = 0;
   bool ok = true;
   auto push = [&](int op, int a, int dtype, int rmode, int slot, float imm) {
@@ -589,7 +606,22 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     P->post[count++] = PostOp{(int16_t)op, (int16_t)a, (int16_t)dtype, (int16_t)rmode, slot, imm};
   };
   // evaluate node id into value d (values d+1, d+2 are free to use)
+  std::function<void(int, int)> emit_node;
   std::function<void(int, int)> emit = [&](int id, int d) {
+    if (!ok) return;
+    if (d > 2) { ok = false; return; }
+    if (uses[id] > 1 && nodes[id].op != KAPY_EW_SPLAT)
+      for (int below = 0; below < d; ++below)
+        if (holder[below] == id) {
+          push(kPick, below, nodes[id].dtype, 0, d, 0.f);
+          holder[d] = id;
+          return;
+        }
+    emit_node(id, d);
+    for (int above = d + 1; above < 3; ++above) holder[above] = -1;
+    holder[d] = id;
+  };
+  emit_node = [&](int id, int d) {
     if (!ok) return;
     const N &n = nodes[id];
     switch (n.op) {
@@ -598,7 +630,11 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
       push(kPushIn, n.input, n.dtype, 0, d, 0.f);
       return;
     case KAPY_EW_SPLAT: push(kPushImm, 0, n.dtype, 0, d, n.imm); return;
-    case KAPY_EW_FPTOFP: emit(n.a, d); push(kCast, 0, n.dtype, n.rmode, d, 0.f); return;
+    case KAPY_EW_FPTOFP:
+      emit(n.a, d);
+      // values are fp32 images of typed values: widening to f32 changes nothing; and the store rounds to nearest itself
+      if (n.dtype != KAPY_F32 && !(id == stored && n.dtype == out->dtype && n.rmode != KAPY_RZ)) push(kCast, 0, n.dtype, n.rmode, d, 0.f);
+      return;
     case KAPY_EW_FMA: emit(n.a, d); emit(n.b, d + 1); emit(n.c, d + 2); push(KAPY_EW_FMA, 0, n.dtype, 0, d, 0.f); return;
     case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF: {
       const bool a_first = std::max(need[n.a], need[n.b] + 1) <= std::max(need[n.b], need[n.a] + 1);

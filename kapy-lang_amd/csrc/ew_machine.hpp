@@ -212,13 +212,35 @@ __device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const
     __builtin_nontemporal_store(lo, (u32x4 *)(out + elem * 4));
     __builtin_nontemporal_store(hi, (u32x4 *)(out + elem * 4) + 1);
   } else {
-    u32x2 v = {0, 0};
+    u32x2 v;
+    v[0] = dtype == KAPY_F8E4M3 ? pack4_e4m3_rn(f[0], f[1], f[2], f[3]) : pack4_e5m2_rn(f[0], f[1], f[2], f[3]);
+    v[1] = dtype == KAPY_F8E4M3 ? pack4_e4m3_rn(f[4], f[5], f[6], f[7]) : pack4_e5m2_rn(f[4], f[5], f[6], f[7]);
+    *(u32x2 *)(out + elem) = v;
+  }
+}
+
+// q[e] = x[e] / y[e], correctly rounded.  When every operand of every lane is zero or of middling magnitude (2^-60 ..
+// 2^60: nothing on the way can overflow or go subnormal) the quotient comes from the sequence at the core of the IEEE
+// division without its scaling, special-case and mode-switching steps: the reciprocal refined once, the quotient
+// corrected by its exact remainder.  Anything else (tiny, huge, infinite, NaN) takes the full division.
+__device__ __forceinline__ void div8(const float (&x)[8], const float (&y)[8], float (&q)[8]) {
+  bool plain = true;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float ax = fabsf(x[e]), ay = fabsf(y[e]);
+    plain = plain && ay >= 0x1p-60f && ay <= 0x1p60f && ax <= 0x1p60f && (ax >= 0x1p-60f || ax == 0.f);
+  }
+  if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const uint32_t byte = dtype == KAPY_F8E4M3 ? f32_to_e4m3(f[e], true) : f32_to_e5m2(f[e], true);
-      v[e >> 2] |= byte << (8 * (e & 3));
+      const float r0 = __builtin_amdgcn_rcpf(y[e]);
+      const float r1 = __builtin_fmaf(__builtin_fmaf(-y[e], r0, 1.0f), r0, r0);
+      const float q0 = x[e] * r1;
+      q[e] = __builtin_fmaf(__builtin_fmaf(-q0, y[e], x[e]), r1, q0);
     }
-    *(u32x2 *)(out + elem) = v;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q[e] = __fdiv_rn(x[e], y[e]);
   }
 }
 
@@ -246,6 +268,12 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
     for (int e = 0; e < 8; ++e) x[e] = c;
     return;
   }
+  case kPick:  // a copy of a value lower on the stack (I.a < D)
+    if (D > 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = (D == 2 && I.a == 1) ? v[1][e] : v[0][e];
+    }
+    return;
   case kStore:
     if (RAGGED && NARROW && (jv + 1) * 8 > P.width) {
       u32x4 v;
@@ -274,12 +302,16 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
     for (int e = 0; e < 8; ++e) x[e] = __fmul_rn(x[e], y[e]);
     break;
   case KAPY_EW_DIVF:
+    { float a8[8], b8[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(x[e], y[e]);
+      for (int e = 0; e < 8; ++e) { a8[e] = x[e]; b8[e] = y[e]; }
+      div8(a8, b8, *(float (*)[8])x); }
     break;
   case kRevDiv:
+    { float a8[8], b8[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fdiv_rn(y[e], x[e]);
+      for (int e = 0; e < 8; ++e) { a8[e] = y[e]; b8[e] = x[e]; }
+      div8(a8, b8, *(float (*)[8])x); }
     break;
   case KAPY_EW_MAXIMUMF:
 #pragma unroll
@@ -294,6 +326,20 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
     for (int e = 0; e < 8; ++e) x[e] = __fmaf_rn(x[e], y[e], z[e]);
     break;
   default:
+    if (NARROW && I.op == KAPY_EW_EXP && I.dtype == KAPY_F32) {
+      // exp(x) = 2^hi * (1 + lo*ln2), hi + lo = x*log2(e) with lo the product's rounding error: within 2 ulp of fp32,
+      // far inside the 16-bit rounding every result of a 16-bit program ends in.  2^hi is already 0 or infinite where
+      // exp(x) leaves the fp32 range; infinite x would make lo inf - inf, so lo is dropped there.
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float hi = x[e] * 1.44269504088896341f;
+        float lo = __builtin_fmaf(x[e], 1.44269504088896341f, -hi);
+        lo = fabsf(x[e]) < 3e38f ? lo : 0.f;
+        const float pw = __builtin_amdgcn_exp2f(hi);
+        x[e] = pw > 3e38f ? pw : __builtin_fmaf(pw, lo * 0.693147180559945309f, pw);
+      }
+      break;
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = apply_unary(I.op, x[e]);
   }

@@ -96,10 +96,32 @@ __device__ __forceinline__ float decode_small(uint32_t b) {
 }
 
 __device__ __forceinline__ uint16_t f32_to_f16_rz(float x) { return (uint16_t)encode_small<5, 10, 15, true, false>(x, false); }
-__device__ __forceinline__ uint8_t f32_to_e4m3(float x, bool rn) { return (uint8_t)encode_small<4, 3, 7, false, true>(x, rn); }
-__device__ __forceinline__ uint8_t f32_to_e5m2(float x, bool rn) { return (uint8_t)encode_small<5, 2, 15, true, true>(x, rn); }
-__device__ __forceinline__ float e4m3_to_f32(uint8_t b) { return decode_small<4, 3, 7, false>(b); }
-__device__ __forceinline__ float e5m2_to_f32(uint8_t b) { return decode_small<5, 2, 15, true>(b); }
+// fp8 (OCP E4M3FN / E5M2, the formats of gfx950's conversion instructions).  Round-to-nearest-even goes through
+// v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32; they turn overflow into NaN / infinity where kapy's cast saturates
+// (ElementwiseOpToLLVM.cpp:577-661 clamps to the largest finite value), so everything but a NaN is clamped first.
+// Round-toward-zero has no instruction and stays with the bit-level encoder.
+__device__ __forceinline__ float clamp_keep_nan(float x, float bound) { return x != x ? x : __builtin_amdgcn_fmed3f(x, -bound, bound); }
+__device__ __forceinline__ uint8_t f32_to_e4m3(float x, bool rn) {
+  if (!rn) return (uint8_t)encode_small<4, 3, 7, false, true>(x, false);
+  const float c = clamp_keep_nan(x, 448.0f);
+  return (uint8_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false);
+}
+__device__ __forceinline__ uint8_t f32_to_e5m2(float x, bool rn) {
+  if (!rn) return (uint8_t)encode_small<5, 2, 15, true, true>(x, false);
+  const float c = clamp_keep_nan(x, 57344.0f);
+  return (uint8_t)__builtin_amdgcn_cvt_pk_bf8_f32(c, c, 0, false);
+}
+// four values to four consecutive bytes, round-to-nearest-even
+__device__ __forceinline__ uint32_t pack4_e4m3_rn(float a, float b, float c, float d) {
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_keep_nan(a, 448.0f), clamp_keep_nan(b, 448.0f), 0, false);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(clamp_keep_nan(c, 448.0f), clamp_keep_nan(d, 448.0f), w, true);
+}
+__device__ __forceinline__ uint32_t pack4_e5m2_rn(float a, float b, float c, float d) {
+  int w = __builtin_amdgcn_cvt_pk_bf8_f32(clamp_keep_nan(a, 57344.0f), clamp_keep_nan(b, 57344.0f), 0, false);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(clamp_keep_nan(c, 57344.0f), clamp_keep_nan(d, 57344.0f), w, true);
+}
+__device__ __forceinline__ float e4m3_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
+__device__ __forceinline__ float e5m2_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_bf8((int)b, 0); }
 
 // Value of element `idx` of a typed buffer as an fp32 (exact for every supported type but i32).
 __device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t idx) {

@@ -186,6 +186,28 @@ typedef struct kapy_ew_inst {
 int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
                      const kapy_global *out, void *stream);
 
+/* Compiles the program once to device code of its own, as the reference does for every function
+ * (translate_mlir_to_llvm / translate_llvm_to_ptx, python/src/passes.cc:141-261), and keeps it for the current
+ * device: later kapy_elementwise calls with the same program, operand element types and operand shapes of the
+ * same kind (full, row, column, scalar) run it instead of the stepwise machines.  Worth it for programs that
+ * none of the hand-written kernels match and that are launched many times: the first compile in a process takes
+ * seconds, later ones about a quarter of a second.  The descriptors only say how operands are shaped and typed;
+ * their pointers are not read.  Needs one store, no reduce, zero padding, contiguous rows of a multiple of 8
+ * elements aligned to 8 elements; KAPY_ERR_UNSUPPORTED otherwise, or when the runtime compiler (libhiprtc) is not
+ * installed -- kapy_elementwise keeps working either way.  A program that the hand-written kernels already serve
+ * with its activation compiled in (act(x*s + bias) with GELU or no activation, plain binary ops) returns KAPY_OK
+ * without compiling anything.  Not to be called while a stream is capturing. */
+int kapy_elementwise_specialize(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
+                                const kapy_global *out);
+/* How many specialised kernels this process holds and how many kapy_elementwise calls have run one (either pointer
+ * may be NULL): lets a caller check that a program it specialised is the code that runs. */
+int kapy_elementwise_specialize_stats(int64_t *loaded, int64_t *launches);
+/* The text kapy_elementwise_specialize would compile (up to capacity-1 bytes, NUL-terminated, into source if not
+ * NULL; its full length into *source_bytes if not NULL), and, if code_bytes is not NULL, the size of the gfx950
+ * code object it compiles to.  Needs no GPU: the counterpart of reading the reference's generated PTX. */
+int kapy_elementwise_source(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
+                            const kapy_global *out, char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes);
+
 /* kapy.fptofp over whole tensors (create_fptofp, python/src/ir.cc:744-754; verifier
  * lib/Dialect/Kapy/IR/Kapy.cpp:272-287): dst[i,j] = cast(src[i,j]), rounding per `rmode`. */
 int kapy_fptofp(const kapy_global *src, const kapy_global *dst, int32_t rmode, void *stream);

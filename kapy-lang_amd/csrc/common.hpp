@@ -55,6 +55,21 @@ inline int vector_bytes(const kapy_global *g, int contiguous_axis) {
   return v;
 }
 
+// Compiles a verified program that contains a reduce for the row machine and launches it (elementwise_row.hip).
+// result_dtype[k] is the element type of instruction k's result.
+int run_row_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                    hipStream_t stream);
+
+// Specialised kernels for verified elementwise programs (elementwise_jit.cpp).  specialize_program compiles and loads one
+// for the current device; launch_specialized returns 1 when it launched one, 0 when none is loaded for this program and
+// operand signature, a negative status on failure; specialized_source writes the generated text and, if asked, compiles it.
+int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out);
+int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                       hipStream_t stream);
+void specialized_stats(int64_t *loaded, int64_t *launches);
+int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                       char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes);
+
 int check_global(const kapy_global *g, const char *what);
 int ensure_device();
 int device_cus();

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
       case KAPY_EW_SUBF: r = __fsub_rn(a, regs[I.b][tid]); break;
       case KAPY_EW_MULF: r = __fmul_rn(a, regs[I.b][tid]); break;
       case KAPY_EW_DIVF: r = __fdiv_rn(a, regs[I.b][tid]); break;
-      case KAPY_EW_FMA: r = __fmaf_rn(a, regs[I.b][tid], regs[I.c][tid]); break;
+      case KAPY_EW_FMA: r = fma_typed(a, regs[I.b][tid], regs[I.c][tid], dt); break;
       case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
       case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
       default: r = apply_unary(I.op, a);
@@ -712,6 +712,10 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
   if (has_reduce) return run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
 
+  // a kernel compiled for exactly this program and operand signature, if the caller asked for one
+  rc = launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s);
+  if (rc != 0) return rc < 0 ? rc : KAPY_OK;
+
   AffineActParams ap;
   int T = -1;
   if (match_affine_act(prog, n_inst, ins, out, &ap, &T)) {
@@ -775,6 +779,33 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   interpreter_kernel<<<grid, 256, 0, s>>>(P, j_fastest);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
+}
+
+int kapy_elementwise_specialize(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins, const kapy_global *out) {
+  int result_dtype[kMaxInst];
+  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype);
+  if (rc) return rc;
+  rc = ensure_device();
+  if (rc) return rc;
+  // act(x*s + bias) with the GELU or no activation already has a hand-written kernel with the activation compiled in:
+  // nothing to gain from another one
+  AffineActParams ap;
+  int T = -1;
+  if (match_affine_act(prog, n_inst, ins, out, &ap, &T) && (ap.act < 0 || ap.act == KAPY_EW_GELU_TANH)) return KAPY_OK;
+  return specialize_program(prog, n_inst, result_dtype, ins, n_ins, out);
+}
+
+int kapy_elementwise_specialize_stats(int64_t *loaded, int64_t *launches) {
+  specialized_stats(loaded, launches);
+  return KAPY_OK;
+}
+
+int kapy_elementwise_source(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins, const kapy_global *out,
+                            char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes) {
+  int result_dtype[kMaxInst];
+  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype);
+  if (rc) return rc;
+  return specialized_source(prog, n_inst, result_dtype, ins, n_ins, out, source, capacity, source_bytes, code_bytes);
 }
 
 int kapy_fptofp(const kapy_global *src, const kapy_global *dst, int32_t rmode, void *stream) {

@@ -1,0 +1,456 @@
+// elementwise_jit.cpp — specialised kernels for elementwise programs.
+//
+// The reference compiles every function once to device code and launches that
+// (python/src/passes.cc:141-261: translate_mlir_to_llvm, translate_llvm_to_ptx); the machines of
+// elementwise.hip instead walk a program step by step on the device, which costs vector-ALU issue slots per step.
+// kapy_elementwise_specialize closes that gap for programs the hand-written kernels do not match: it writes the
+// program out as straight-line HIP over the same device helpers the machines use (the text of numeric.hpp and
+// ew_machine.hpp is embedded at build time, so rounding and special cases are the machines' own), compiles it for
+// gfx950 with the runtime compiler (libhiprtc, opened on first use; absent => KAPY_ERR_UNSUPPORTED and the machines keep
+// serving), loads the code object and keeps it in a process-wide table keyed by program and operand signature.
+// kapy_elementwise looks a verified program up in that table before it falls back to the machines.
+#include <dlfcn.h>
+#include <hip/hiprtc.h>
+#include <string.h>
+
+#include <algorithm>
+#include <atomic>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+namespace kapy {
+namespace {
+
+// what the generated kernel takes; the same text is part of every generated source
+constexpr int kJitInputs = 8;
+struct JitArgs {
+  const char *in[kJitInputs];
+  int64_t stride0[kJitInputs];
+  char *out;
+  int64_t out_stride0;
+  int32_t rows, vec_per_row;
+};
+const char *kArgsText = R"(
+struct JitArgs {
+  const char *in[8];
+  int64_t stride0[8];
+  char *out;
+  int64_t out_stride0;
+  int32_t rows, vec_per_row;
+};
+__device__ __forceinline__ void fill8(float (&x)[8], float v) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = v;
+}
+__device__ __forceinline__ void copy8(float (&x)[8], const float (&y)[8]) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = y[e];
+}
+)";
+
+const char *kPrelude =
+    "typedef signed char int8_t; typedef unsigned char uint8_t; typedef short int16_t; typedef unsigned short uint16_t;\n"
+    "typedef int int32_t; typedef unsigned int uint32_t; typedef long int64_t; typedef unsigned long uint64_t;\n"
+    "typedef unsigned long uintptr_t;\n"
+#include "jit_headers.inc"
+    ;
+
+enum Kind { kFull = 0, kRow = 1, kCol = 2, kScalar = 3 };
+
+struct Signature {
+  int n_ins = 0;
+  int in_dtype[kJitInputs], in_kind[kJitInputs];
+  int out_dtype = 0;
+  bool narrow = true;
+};
+
+// Which programs a specialised kernel serves and how each operand is read: the result and the full / row operands
+// contiguous along rows and readable 8 elements at a time, column and scalar operands broadcast, no padding pattern
+// other than zero, one store, no reduce.
+bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+              Signature *sig) {
+  if (n_ins > kJitInputs) return false;
+  int stores = 0;
+  for (int k = 0; k < n_inst; ++k) {
+    const int op = prog[k].op;
+    if (op == KAPY_EW_REDUCE_SUM || op == KAPY_EW_REDUCE_MAX) return false;
+    if (op == KAPY_EW_LD_GLOBAL && prog[k].c != KAPY_PAD_ZERO) return false;
+    stores += op == KAPY_EW_ST_GLOBAL;
+  }
+  if (stores != 1) return false;
+  const int64_t o0 = extent0(out), o1 = extent1(out);
+  const int ob = dtype_bytes(out->dtype);
+  if (!is_float(out->dtype) || out->stride1 != 1 || o1 % 8 != 0) return false;
+  if (((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
+  if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  sig->n_ins = n_ins;
+  sig->out_dtype = out->dtype;
+  sig->narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
+  for (int k = 0; k < n_inst; ++k) sig->narrow = sig->narrow && !is_f8(result_dtype[k]);
+  for (int k = 0; k < n_ins; ++k) {
+    const kapy_global *g = ins[k];
+    if (!is_float(g->dtype)) return false;
+    sig->narrow = sig->narrow && (g->dtype == KAPY_F16 || g->dtype == KAPY_BF16);
+    const int64_t e0 = extent0(g), e1 = extent1(g);
+    const int eb = dtype_bytes(g->dtype);
+    const bool vec_ok = g->stride1 == 1 && ((uintptr_t)view_base(g) % (8 * eb)) == 0 && (g->stride0 * eb) % (8 * eb) == 0;
+    sig->in_dtype[k] = g->dtype;
+    if (e0 == o0 && e1 == o1 && vec_ok) sig->in_kind[k] = kFull;
+    else if (e0 == 1 && e1 == o1 && vec_ok) sig->in_kind[k] = kRow;
+    else if (e1 == 1 && e0 == o0) sig->in_kind[k] = kCol;
+    else if (e0 == 1 && e1 == 1) sig->in_kind[k] = kScalar;
+    else return false;
+  }
+  return true;
+}
+
+std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig) {
+  std::string key;
+  key.reserve(n_inst * sizeof(kapy_ew_inst) + 64);
+  for (int k = 0; k < n_inst; ++k) {
+    kapy_ew_inst I = prog[k];  // fields an op does not read must not tell two equal programs apart
+    const int op = I.op;
+    const bool unary_or_cast = !(op == KAPY_EW_LD_GLOBAL || op == KAPY_EW_SPLAT || op == KAPY_EW_FMA || op == KAPY_EW_ADDF || op == KAPY_EW_SUBF ||
+                                 op == KAPY_EW_MULF || op == KAPY_EW_DIVF || op == KAPY_EW_MAXIMUMF || op == KAPY_EW_MINIMUMF);
+    if (op == KAPY_EW_SPLAT) I.a = I.b = I.c = 0;
+    else I.imm = 0.f;
+    if (op == KAPY_EW_LD_GLOBAL) I.b = 0;
+    if (unary_or_cast) I.b = I.c = 0;
+    if (op != KAPY_EW_FMA && !unary_or_cast && op != KAPY_EW_LD_GLOBAL) I.c = 0;
+    if (op != KAPY_EW_FPTOFP) I.rmode = 0;
+    if (op != KAPY_EW_FPTOFP && op != KAPY_EW_SPLAT) I.dtype = 0;
+    if (op == KAPY_EW_ST_GLOBAL) I.dst = 0;
+    key.append((const char *)&I, sizeof I);
+  }
+  for (int k = 0; k < sig.n_ins; ++k) {
+    key.push_back((char)sig.in_dtype[k]);
+    key.push_back((char)sig.in_kind[k]);
+  }
+  key.push_back((char)sig.out_dtype);
+  return key;
+}
+
+void appendf(std::string &s, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void appendf(std::string &s, const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  s += buf;
+}
+
+// The program as straight-line code: every value that the store depends on becomes one array of 8 fp32 (the exact
+// image of the typed value, rounded to the op's result type after every op, as the machines do), a splat one constant.
+std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig) {
+  struct Node {
+    int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
+    float imm = 0.f;
+    bool used = false;
+    std::string name;   // the array (or constant) holding the value
+    bool is_const = false;
+  };
+  std::vector<Node> nodes;
+  int reg[64];
+  for (int &r : reg) r = -1;
+  int stored = -1;
+  for (int k = 0; k < n_inst; ++k) {
+    const kapy_ew_inst &I = prog[k];
+    Node n;
+    n.op = I.op;
+    n.dtype = result_dtype[k];
+    n.rmode = I.rmode;
+    n.imm = I.imm;
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: n.input = I.a; break;
+    case KAPY_EW_SPLAT: break;
+    case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; continue;
+    case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
+    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+      n.a = reg[I.a]; n.b = reg[I.b]; break;
+    default: n.a = reg[I.a];
+    }
+    nodes.push_back(n);
+    reg[I.dst] = (int)nodes.size() - 1;
+  }
+  {  // mark what the store needs
+    std::vector<int> todo{stored};
+    while (!todo.empty()) {
+      const int id = todo.back();
+      todo.pop_back();
+      if (id < 0 || nodes[id].used) continue;
+      nodes[id].used = true;
+      todo.push_back(nodes[id].a);
+      todo.push_back(nodes[id].b);
+      todo.push_back(nodes[id].c);
+    }
+  }
+  std::vector<char> input_used(kJitInputs, 0);
+  for (const Node &n : nodes)
+    if (n.used && n.op == KAPY_EW_LD_GLOBAL) input_used[n.input] = 1;
+
+  std::string s = kPrelude;
+  s += "namespace kapy { namespace {\n";
+  s += kArgsText;
+  s += "} }\nusing namespace kapy;\n";
+  s += "extern \"C\" __global__ __launch_bounds__(256) void kapy_ew_specialised(JitArgs p) {\n";
+  appendf(s, "  constexpr bool NARROW = %s;\n", sig.narrow ? "true" : "false");
+  s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
+       "  const uint32_t first = blockIdx.x * 512u + threadIdx.x;\n"
+       "  int32_t row[2], jv[2];\n";
+  for (int k = 0; k < sig.n_ins; ++k) {
+    if (!input_used[k]) continue;
+    if (sig.in_kind[k] == kFull || sig.in_kind[k] == kRow) appendf(s, "  Raw8 raw%d[2];\n", k);
+    else appendf(s, "  float raw%d[2];\n", k);
+  }
+  // splats: one rounding to the splat's type, as the machines do when they push an immediate
+  for (size_t id = 0; id < nodes.size(); ++id) {
+    Node &n = nodes[id];
+    if (!n.used || n.op != KAPY_EW_SPLAT) continue;
+    uint32_t bits;
+    memcpy(&bits, &n.imm, 4);
+    n.name = "c" + std::to_string(id);
+    n.is_const = true;
+    appendf(s, "  const float %s = round_to_dtype(bits_f32(0x%08xu), %d, true);\n", n.name.c_str(), bits, n.dtype);
+  }
+  s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
+       "    const uint32_t slot = first + u * 256u;\n"
+       "    row[u] = -1;\n"
+       "    if (slot < total) {\n"
+       "      row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);\n"
+       "      jv[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row);\n";
+  for (int k = 0; k < sig.n_ins; ++k) {
+    if (!input_used[k]) continue;
+    const int kind = sig.in_kind[k], dt = sig.in_dtype[k];
+    if (kind == kFull || kind == kRow)
+      appendf(s, "      { const StackIn g{p.in[%d], p.stride0[%d], %d, %d}; raw%d[u] = fetch8(g, row[u], jv[u], %s); }\n", k, k, dt,
+              kind == kFull ? 0 : 1, k, kind == kFull ? "true" : "false");
+    else
+      appendf(s, "      raw%d[u] = load_as_f32(p.in[%d], %d, %s);\n", k, k, dt, kind == kCol ? ("row[u] * p.stride0[" + std::to_string(k) + "]").c_str() : "0");
+  }
+  s += "    }\n  }\n#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n    if (row[u] < 0) continue;\n";
+  auto elem = [&](int id) { return nodes[id].is_const ? nodes[id].name : nodes[id].name + "[e]"; };
+  // an operand as an array of 8 (div8 and the store take arrays)
+  int n_filled = 0;
+  auto as_array = [&](int id) {
+    if (!nodes[id].is_const) return nodes[id].name;
+    const std::string a = "a" + std::to_string(n_filled++) + nodes[id].name;
+    appendf(s, "    float %s[8]; fill8(%s, %s);\n", a.c_str(), a.c_str(), nodes[id].name.c_str());
+    return a;
+  };
+  for (size_t id = 0; id < nodes.size(); ++id) {
+    Node &n = nodes[id];
+    if (!n.used || n.op == KAPY_EW_SPLAT) continue;
+    const std::string v = "v" + std::to_string(id);
+    const char *vn = v.c_str();
+    auto round_result = [&]() {
+      if (n.dtype != KAPY_F32) appendf(s, "    round8<NARROW>(%s, %d, true);\n", vn, n.dtype);
+    };
+    auto per_element = [&](const std::string &expr) {
+      appendf(s, "    float %s[8];\n#pragma unroll\n    for (int e = 0; e < 8; ++e) %s[e] = %s;\n", vn, vn, expr.c_str());
+    };
+    n.name = v;
+    switch (n.op) {
+    case KAPY_EW_LD_GLOBAL: {
+      const int k = n.input, kind = sig.in_kind[k];
+      if (kind == kFull || kind == kRow) appendf(s, "    float %s[8]; widen8(raw%d[u], %d, %s);\n", vn, k, sig.in_dtype[k], vn);
+      else appendf(s, "    float %s[8]; fill8(%s, raw%d[u]);\n", vn, vn, k);
+      break;
+    }
+    case KAPY_EW_FPTOFP: {
+      // values are fp32 images of typed values: widening to f32 changes nothing, and the store rounds to nearest itself
+      const bool free_cast = n.dtype == KAPY_F32 || ((int)id == stored && n.dtype == sig.out_dtype && n.rmode != KAPY_RZ);
+      if (free_cast) {
+        n.name = nodes[n.a].name;
+        n.is_const = nodes[n.a].is_const;
+      } else {
+        per_element(elem(n.a));
+        appendf(s, "    round8<NARROW>(%s, %d, %s);\n", vn, n.dtype, n.rmode != KAPY_RZ ? "true" : "false");
+      }
+      break;
+    }
+    case KAPY_EW_ADDF: per_element("__fadd_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_SUBF: per_element("__fsub_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MULF: per_element("__fmul_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MAXIMUMF: per_element("max_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MINIMUMF: per_element("min_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_FMA: per_element("fma_typed(" + elem(n.a) + ", " + elem(n.b) + ", " + elem(n.c) + ", " + std::to_string(n.dtype) + ")"); round_result(); break;
+    case KAPY_EW_DIVF: {
+      const std::string a = as_array(n.a), b = as_array(n.b);
+      appendf(s, "    float %s[8]; div8(%s, %s, %s);\n", vn, a.c_str(), b.c_str(), vn);
+      round_result();
+      break;
+    }
+    default:  // the unary ops
+      per_element(elem(n.a));
+      appendf(s, "    unary8<NARROW>(%d, %d, %s);\n", n.op, n.dtype, vn);
+      round_result();
+    }
+  }
+  const std::string result = as_array(stored);
+  appendf(s, "    store8<NARROW>(p.out, %d, (int64_t)row[u] * p.out_stride0 + (int64_t)jv[u] * 8, %s);\n  }\n}\n", sig.out_dtype, result.c_str());
+  return s;
+}
+
+// ---- the runtime compiler, opened on first use --------------------------------------------------------------------
+struct Rtc {
+  void *handle = nullptr;
+  decltype(&hiprtcCreateProgram) create = nullptr;
+  decltype(&hiprtcCompileProgram) compile = nullptr;
+  decltype(&hiprtcGetProgramLogSize) log_size = nullptr;
+  decltype(&hiprtcGetProgramLog) log = nullptr;
+  decltype(&hiprtcGetCodeSize) code_size = nullptr;
+  decltype(&hiprtcGetCode) code = nullptr;
+  decltype(&hiprtcDestroyProgram) destroy = nullptr;
+  bool ok = false;
+};
+const Rtc &rtc() {
+  static Rtc r = [] {
+    Rtc t;
+    for (const char *name : {"libhiprtc.so.7", "libhiprtc.so"}) {
+      t.handle = dlopen(name, RTLD_NOW | RTLD_LOCAL);
+      if (t.handle) break;
+    }
+    if (!t.handle) return t;
+#define KAPY_RTC_SYM(field, symbol) t.field = (decltype(t.field))dlsym(t.handle, #symbol)
+    KAPY_RTC_SYM(create, hiprtcCreateProgram);
+    KAPY_RTC_SYM(compile, hiprtcCompileProgram);
+    KAPY_RTC_SYM(log_size, hiprtcGetProgramLogSize);
+    KAPY_RTC_SYM(log, hiprtcGetProgramLog);
+    KAPY_RTC_SYM(code_size, hiprtcGetCodeSize);
+    KAPY_RTC_SYM(code, hiprtcGetCode);
+    KAPY_RTC_SYM(destroy, hiprtcDestroyProgram);
+#undef KAPY_RTC_SYM
+    t.ok = t.create && t.compile && t.log_size && t.log && t.code_size && t.code && t.destroy;
+    return t;
+  }();
+  return r;
+}
+
+int compile_source(const std::string &source, std::vector<char> *code) {
+  const Rtc &r = rtc();
+  if (!r.ok) return fail(KAPY_ERR_UNSUPPORTED, "elementwise_specialize: the runtime compiler (libhiprtc) is not available");
+  hiprtcProgram prog = nullptr;
+  if (r.create(&prog, source.c_str(), "kapy_ew_specialised.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    return fail(KAPY_ERR_HIP, "elementwise_specialize: hiprtcCreateProgram failed");
+  // Packed fp32 VALU forms stay off, as for every device compile of this library.  Contraction only inside one
+  // expression: in the generated text every op of the program is a statement of its own and must keep its own rounding
+  // (with everything in one basic block the default, cross-statement mode would fuse a mulf and the addf after it).
+  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  const hiprtcResult rc = r.compile(prog, (int)(sizeof opts / sizeof opts[0]), opts);
+  if (rc != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    r.log_size(prog, &n);
+    std::string log(n, '\0');
+    if (n) r.log(prog, &log[0]);
+    r.destroy(&prog);
+    return fail(KAPY_ERR_HIP, "elementwise_specialize: compile failed (%d): %.400s", (int)rc, log.c_str());
+  }
+  size_t n = 0;
+  r.code_size(prog, &n);
+  code->resize(n);
+  const hiprtcResult got = r.code(prog, code->data());
+  r.destroy(&prog);
+  if (got != HIPRTC_SUCCESS || n == 0) return fail(KAPY_ERR_HIP, "elementwise_specialize: no code object");
+  return KAPY_OK;
+}
+
+struct Loaded {
+  hipModule_t module = nullptr;
+  hipFunction_t fn = nullptr;
+};
+std::mutex g_mutex;
+std::map<std::pair<int, std::string>, Loaded> g_table;  // (device, key) -> kernel
+std::atomic<int> g_count{0};
+std::atomic<int64_t> g_launches{0};
+
+}  // namespace
+
+int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out) {
+  Signature sig;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
+    return fail(KAPY_ERR_UNSUPPORTED,
+                "elementwise_specialize: needs one store, no reduce, zero padding, rows of a multiple of 8 contiguous elements aligned to 8 "
+                "elements, and operands that are full, row, column or scalar views");
+  int device = 0;
+  KAPY_HIP_CHECK(hipGetDevice(&device));
+  const std::string key = make_key(prog, n_inst, sig);
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_table.count({device, key})) return KAPY_OK;
+  }
+  std::vector<char> code;
+  int rc = compile_source(generate(prog, n_inst, result_dtype, sig), &code);
+  if (rc) return rc;
+  Loaded k;
+  KAPY_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
+  KAPY_HIP_CHECK(hipModuleGetFunction(&k.fn, k.module, "kapy_ew_specialised"));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (!g_table.emplace(std::make_pair(device, key), k).second) (void)hipModuleUnload(k.module);  // another thread was first
+  else g_count.fetch_add(1);
+  return KAPY_OK;
+}
+
+int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                       hipStream_t stream) {
+  if (g_count.load(std::memory_order_acquire) == 0) return 0;
+  Signature sig;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig)) return 0;
+  int device = 0;
+  KAPY_HIP_CHECK(hipGetDevice(&device));
+  Loaded k;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    auto it = g_table.find({device, make_key(prog, n_inst, sig)});
+    if (it == g_table.end()) return 0;
+    k = it->second;
+  }
+  JitArgs args;
+  memset(&args, 0, sizeof args);
+  for (int i = 0; i < n_ins; ++i) {
+    args.in[i] = view_base(ins[i]);
+    args.stride0[i] = ins[i]->stride0;
+  }
+  args.out = (char *)view_base(out);
+  args.out_stride0 = out->stride0;
+  args.rows = (int32_t)extent0(out);
+  args.vec_per_row = (int32_t)(extent1(out) / 8);
+  size_t size = sizeof args;
+  void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  const int64_t slots = (int64_t)args.rows * args.vec_per_row;
+  KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, (unsigned)((slots + 511) / 512), 1, 1, 256, 1, 1, 0, stream, nullptr, extra));
+  g_launches.fetch_add(1, std::memory_order_relaxed);
+  return 1;
+}
+
+void specialized_stats(int64_t *loaded, int64_t *launches) {
+  if (loaded) *loaded = g_count.load();
+  if (launches) *launches = g_launches.load();
+}
+
+int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                       char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes) {
+  Signature sig;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
+    return fail(KAPY_ERR_UNSUPPORTED, "elementwise_source: the program or its operands do not fit a specialised kernel");
+  const std::string text = generate(prog, n_inst, result_dtype, sig);
+  if (source && capacity > 0) {
+    const size_t n = std::min<size_t>(text.size(), (size_t)capacity - 1);
+    memcpy(source, text.data(), n);
+    source[n] = '\0';
+  }
+  if (source_bytes) *source_bytes = (int64_t)text.size();
+  if (code_bytes) {
+    std::vector<char> code;
+    int rc = compile_source(text, &code);
+    if (rc) return rc;
+    *code_bytes = (int64_t)code.size();
+  }
+  return KAPY_OK;
+}
+
+}  // namespace kapy

@@ -38,11 +38,6 @@ struct StackProgram {
   int32_t width;   // elements per row when the last vector of a row is partial (ragged kernels), else 0
 };
 
-// Compiles a verified program that contains a reduce for the row machine and launches it (elementwise_row.hip).
-// result_dtype[k] is the element type of instruction k's result.
-int run_row_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
-                    hipStream_t stream);
-
 namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -244,6 +239,27 @@ __device__ __forceinline__ void div8(const float (&x)[8], const float (&y)[8], f
   }
 }
 
+// x[e] = op(x[e]) for a unary op whose result has element type dtype (rounding to that type is the caller's).
+template <bool NARROW>
+__device__ __forceinline__ void unary8(int op, int dtype, float (&x)[8]) {
+  if (NARROW && op == KAPY_EW_EXP && dtype == KAPY_F32) {
+    // exp(x) = 2^hi * (1 + lo*ln2), hi + lo = x*log2(e) with lo the product's rounding error: within 2 ulp of fp32,
+    // far inside the 16-bit rounding every result of a 16-bit program ends in.  2^hi is already 0 or infinite where
+    // exp(x) leaves the fp32 range; infinite x would make lo inf - inf, so lo is dropped there.
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float hi = x[e] * 1.44269504088896341f;
+      float lo = __builtin_fmaf(x[e], 1.44269504088896341f, -hi);
+      lo = fabsf(x[e]) < 3e38f ? lo : 0.f;
+      const float pw = __builtin_amdgcn_exp2f(hi);
+      x[e] = pw > 3e38f ? pw : __builtin_fmaf(pw, lo * 0.693147180559945309f, pw);
+    }
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = apply_unary(op, x[e]);
+}
+
 // One step with its result (and left operand) in value D, the right operand in value D+1 and the
 // third operand of an fma in value D+2; D is a template parameter so that no register is indexed.
 // NARROW: every operand, every intermediate type and the result are f16 / bf16 / f32-from-16-bit
@@ -323,25 +339,9 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
     break;
   case KAPY_EW_FMA:
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = __fmaf_rn(x[e], y[e], z[e]);
+    for (int e = 0; e < 8; ++e) x[e] = fma_typed(x[e], y[e], z[e], I.dtype);
     break;
-  default:
-    if (NARROW && I.op == KAPY_EW_EXP && I.dtype == KAPY_F32) {
-      // exp(x) = 2^hi * (1 + lo*ln2), hi + lo = x*log2(e) with lo the product's rounding error: within 2 ulp of fp32,
-      // far inside the 16-bit rounding every result of a 16-bit program ends in.  2^hi is already 0 or infinite where
-      // exp(x) leaves the fp32 range; infinite x would make lo inf - inf, so lo is dropped there.
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float hi = x[e] * 1.44269504088896341f;
-        float lo = __builtin_fmaf(x[e], 1.44269504088896341f, -hi);
-        lo = fabsf(x[e]) < 3e38f ? lo : 0.f;
-        const float pw = __builtin_amdgcn_exp2f(hi);
-        x[e] = pw > 3e38f ? pw : __builtin_fmaf(pw, lo * 0.693147180559945309f, pw);
-      }
-      break;
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = apply_unary(I.op, x[e]);
+  default: unary8<NARROW>(I.op, I.dtype, *(float (*)[8])x);
   }
   if (I.dtype != KAPY_F32) round8<NARROW>(x, I.dtype, true);
 }

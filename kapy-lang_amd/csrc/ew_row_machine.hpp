@@ -53,7 +53,7 @@ __device__ __forceinline__ float scalar_step(const StackProgram &P, const PostOp
   case kRevDiv: r = __fdiv_rn(y, x); break;
   case KAPY_EW_MAXIMUMF: r = max_nan(x, y); break;
   case KAPY_EW_MINIMUMF: r = min_nan(x, y); break;
-  case KAPY_EW_FMA: r = __fmaf_rn(x, y, z); break;
+  case KAPY_EW_FMA: r = fma_typed(x, y, z, I.dtype); break;
   default: r = apply_unary(I.op, x);
   }
   return I.dtype != KAPY_F32 ? round_to_dtype(r, I.dtype, true) : r;
@@ -122,7 +122,7 @@ __device__ __forceinline__ void light_step(const StackProgram &P, const PostOp &
 #pragma unroll
     for (int c = 0; c < CH; ++c)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[c][D][e] = __fmaf_rn(v[c][D][e], v[c][R][e], v[c][T][e]);
+      for (int e = 0; e < 8; ++e) v[c][D][e] = fma_typed(v[c][D][e], v[c][R][e], v[c][T][e], I.dtype);
     break;
   case KAPY_EW_NEGF: KAPY_LIGHT_UNARY(-x); break;
   case KAPY_EW_ABSF: KAPY_LIGHT_UNARY(fabsf(x)); break;

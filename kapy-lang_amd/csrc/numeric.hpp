@@ -123,6 +123,14 @@ __device__ __forceinline__ uint32_t pack4_e5m2_rn(float a, float b, float c, flo
 __device__ __forceinline__ float e4m3_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
 __device__ __forceinline__ float e5m2_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_bf8((int)b, 0); }
 
+// a*b + c on values of element type dtype (held as their fp32 images) with the ONE rounding fma promises.  For f16 that
+// has to be the 16-bit instruction: the fp32 fma followed by the rounding to f16 rounds twice and lands on the wrong
+// neighbour a few times in a million.  For bf16 (no 16-bit fma on this part) and f32 the fp32 fma serves.
+__device__ __forceinline__ float fma_typed(float a, float b, float c, int dtype) {
+  if (dtype == KAPY_F16) return (float)__builtin_fmaf16((_Float16)a, (_Float16)b, (_Float16)c);
+  return __builtin_fmaf(a, b, c);
+}
+
 // Value of element `idx` of a typed buffer as an fp32 (exact for every supported type but i32).
 __device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t idx) {
   switch (dtype) {

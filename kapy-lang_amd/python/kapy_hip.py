@@ -32,6 +32,7 @@ EXPORTS = [
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
     "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
+    "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats",
 ]
 
 
@@ -143,6 +144,9 @@ def lib():
     L.kapy_copy.argtypes = [P(Global), P(Global), P(CopyCfg), vp]
     L.kapy_copy_batched.argtypes = [P(Global), P(Global), P(CopyCfg), P(Grid2), vp]
     L.kapy_elementwise.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), vp]
+    L.kapy_elementwise_specialize.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global)]
+    L.kapy_elementwise_specialize_stats.argtypes = [P(i64), P(i64)]
+    L.kapy_elementwise_source.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), C.c_char_p, i64, P(i64), P(i64)]
     L.kapy_fptofp.argtypes = [P(Global), P(Global), i32, vp]
     L.kapy_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
@@ -314,6 +318,31 @@ def elementwise(prog, ins, out, stream=None):
     arr = (C.POINTER(Global) * max(len(ins), 1))(*[C.pointer(g) for g in ins])
     check(lib().kapy_elementwise(prog, len(prog), arr, len(ins), C.byref(out),
                                  stream if stream is not None else current_stream()))
+
+
+def elementwise_specialize(prog, ins, out):
+    """Compile the program to a kernel of its own for the current device; later elementwise() calls with the same
+    program and operand signature run it."""
+    arr = (C.POINTER(Global) * max(len(ins), 1))(*[C.pointer(g) for g in ins])
+    check(lib().kapy_elementwise_specialize(prog, len(prog), arr, len(ins), C.byref(out)))
+
+
+def elementwise_specialize_stats():
+    """(specialised kernels loaded, elementwise() calls that ran one) in this process."""
+    a, b = C.c_int64(0), C.c_int64(0)
+    check(lib().kapy_elementwise_specialize_stats(C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
+def elementwise_source(prog, ins, out, compile=False):
+    """(text of the specialised kernel, size of its gfx950 code object or None); needs no GPU."""
+    arr = (C.POINTER(Global) * max(len(ins), 1))(*[C.pointer(g) for g in ins])
+    n, code = C.c_int64(0), C.c_int64(0)
+    check(lib().kapy_elementwise_source(prog, len(prog), arr, len(ins), C.byref(out), None, 0, C.byref(n), None))
+    buf = C.create_string_buffer(n.value + 1)
+    check(lib().kapy_elementwise_source(prog, len(prog), arr, len(ins), C.byref(out), buf, n.value + 1, None,
+                                        C.byref(code) if compile else None))
+    return buf.value.decode(), (code.value if compile else None)
 
 
 def fptofp(src, dst, rmode=RN, stream=None):

@@ -1,0 +1,210 @@
+"""GPU parity for elementwise programs compiled to kernels of their own (kapy_elementwise_specialize): the same
+programs the stepwise machines run, against the oracle to the same bar (bit-exact where every op is exactly
+rounded, <= 2 ulp of the 16-bit result otherwise), with the launch counter showing that the compiled kernel ran."""
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+from test_gpu_elementwise import _check_ulp
+
+pytestmark = pytest.mark.gpu
+
+L, ADD, SUB, MUL, DIV, FMA, MAX, MIN, ST, CAST, SPL = (kh.EW_LD_GLOBAL, kh.EW_ADDF, kh.EW_SUBF, kh.EW_MULF, kh.EW_DIVF, kh.EW_FMA, kh.EW_MAXIMUMF,
+                                                        kh.EW_MINIMUMF, kh.EW_ST_GLOBAL, kh.EW_FPTOFP, kh.EW_SPLAT)
+NP_OF = {1: np.uint8, 2: np.uint16, 4: np.uint32}
+
+
+def _both(ko, insts, ins_np, in_dtypes, out_dtype, m, n, in_shapes=None, expect_compiled=True):
+    """(result of the machines, result after specialising, oracle); asserts which path served the second call."""
+    outb = kh.DTYPE_BYTES[out_dtype]
+    want = np.zeros((m, n), dtype=NP_OF[outb])
+    in_shapes = in_shapes or [(m, n)] * len(ins_np)
+    gos = [ko.mk_global(a, s[0], s[1], s[1], 1, dt) for a, s, dt in zip(ins_np, in_shapes, in_dtypes)]
+    assert ko.elementwise(ko.program(insts), gos, ko.mk_global(want, m, n, n, 1, out_dtype)) == 0
+    devs = [to_dev(a) for a in ins_np]
+    prog = kh.program(insts)
+    dins = [dglobal(t, s[0], s[1], s[1], 1, dt) for t, s, dt in zip(devs, in_shapes, in_dtypes)]
+    results = []
+    for step in range(2):
+        dout = dev_zeros(m * n, outb)
+        before = kh.elementwise_specialize_stats()[1]
+        kh.elementwise(prog, dins, dglobal(dout, m, n, n, 1, out_dtype))
+        sync()
+        ran_compiled = kh.elementwise_specialize_stats()[1] - before
+        results.append(to_host(dout, NP_OF[outb], (m, n)))
+        if step == 0:
+            if ran_compiled:   # an earlier test specialised the same program: nothing to compare the machines with
+                results.append(results[0])
+                break
+            try:
+                kh.elementwise_specialize(prog, dins, dglobal(dout, m, n, n, 1, out_dtype))
+            except kh.KapyError as e:
+                assert not expect_compiled, str(e)
+                assert e.args[0].startswith("kapy status %d" % kh.ERR_UNSUPPORTED)
+        else:
+            assert ran_compiled == (1 if expect_compiled else 0)
+    return results[0], results[1], want
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(16, 256), (33, 1000), (1, 8), (700, 4104)])
+def test_exactly_rounded_arithmetic_is_bit_exact(ko, dtype, m, n):
+    a = ko.fill_normal(m * n, dtype, 31, 0).reshape(m, n)
+    b = ko.fill_normal(m * n, dtype, 31, 1).reshape(m, n)
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=0),
+             dict(op=SUB, dst=3, a=2, b=1), dict(op=MAX, dst=3, a=3, b=0), dict(op=FMA, dst=3, a=3, b=1, c=0), dict(op=MIN, dst=3, a=3, b=2),
+             dict(op=ST, a=3)]
+    machine, compiled, want = _both(ko, insts, [a, b], [dtype, dtype], dtype, m, n)
+    assert np.array_equal(compiled, want)
+    assert np.array_equal(machine, want)
+
+
+def test_every_operand_kind_reversed_operands_division_and_a_value_used_three_times(ko):
+    m, n = 24, 512
+    a = ko.fill_normal(m * n, kh.F16, 21, 0).reshape(m, n)
+    b = ko.fill_uniform(m * n, kh.F16, 21, 1, 0.5, 2.0).reshape(m, n)
+    row, col, one = ko.fill_normal(n, kh.F16, 21, 2), ko.fill_normal(m, kh.F16, 21, 3), ko.fill_normal(1, kh.F16, 21, 4)
+    # ((a - b*row) / ((a + col) max (b - one))) * a + a: `a` feeds four ops, which the stack machine can only re-evaluate
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=L, dst=2, a=2), dict(op=L, dst=3, a=3), dict(op=L, dst=4, a=4),
+             dict(op=MUL, dst=5, a=1, b=2), dict(op=SUB, dst=5, a=0, b=5), dict(op=ADD, dst=6, a=0, b=3), dict(op=SUB, dst=7, a=1, b=4),
+             dict(op=MAX, dst=6, a=6, b=7), dict(op=DIV, dst=5, a=5, b=6), dict(op=FMA, dst=5, a=5, b=0, c=0), dict(op=ST, a=5)]
+    machine, compiled, want = _both(ko, insts, [a, b, row, col, one], [kh.F16] * 5, kh.F16, m, n, [(m, n), (m, n), (1, n), (m, 1), (1, 1)])
+    _check_ulp(compiled, want, kh.F16)
+    assert np.array_equal(compiled, machine)   # the same device helpers, the same roundings
+
+
+def test_f32_and_fp8_operands_and_results(ko):
+    m, n = 16, 256
+    a = ko.fill_normal(m * n, kh.F16, 21, 0).reshape(m, n)
+    b = ko.fill_uniform(m * n, kh.F16, 21, 1, 0.5, 2.0).reshape(m, n)
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=CAST, dst=2, a=0, dtype=kh.F32), dict(op=CAST, dst=3, a=1, dtype=kh.F32),
+             dict(op=MUL, dst=4, a=2, b=3), dict(op=SUB, dst=5, a=3, b=2), dict(op=ADD, dst=6, a=2, b=3), dict(op=FMA, dst=7, a=4, b=5, c=6),
+             dict(op=ST, a=7)]
+    _, compiled, want = _both(ko, insts, [a, b], [kh.F16] * 2, kh.F32, m, n)
+    assert np.array_equal(compiled, want)
+    x32 = ko.fill_normal(m * n, kh.F32, 22, 0).reshape(m, n)
+    for f8 in (kh.F8E4M3, kh.F8E5M2):
+        for rmode in (kh.RN, kh.RZ):
+            insts = [dict(op=L, dst=0, a=0), dict(op=SPL, dst=1, dtype=kh.F32, imm=37.5), dict(op=MUL, dst=0, a=0, b=1),
+                     dict(op=CAST, dst=2, a=0, dtype=f8, rmode=rmode), dict(op=ST, a=2)]
+            _, q, wantq = _both(ko, insts, [x32], [kh.F32], f8, m, n)
+            assert np.array_equal(q, wantq)
+        insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.BF16), dict(op=ST, a=1)]
+        _, back, want = _both(ko, insts, [wantq], [f8], kh.BF16, m, n)
+        assert np.array_equal(back, want)
+    # f16 -> e4m3 with a per-row scale: the activation quantiser in front of the W8A8 matmul
+    scale = ko.fill_uniform(m, kh.F32, 23, 0, 0.5, 4.0)
+    insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=L, dst=1, a=1), dict(op=MUL, dst=0, a=0, b=1),
+             dict(op=CAST, dst=2, a=0, dtype=kh.F8E4M3, rmode=kh.RN), dict(op=ST, a=2)]
+    _, q, wantq = _both(ko, insts, [a, scale], [kh.F16, kh.F32], kh.F8E4M3, m, n, [(m, n), (m, 1)])
+    assert np.array_equal(q, wantq)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+def test_silu_and_explicit_gelu_chains(ko, dtype):
+    m, n = 32, 1024
+    x = ko.fill_normal(m * n, dtype, 9, 0, 0.0, 3.0).reshape(m, n)
+    c = lambda r, v: dict(op=SPL, dst=r, dtype=kh.F32, imm=v)
+    silu = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=kh.EW_NEGF, dst=2, a=1), dict(op=kh.EW_EXP, dst=2, a=2),
+            c(3, 1.0), dict(op=ADD, dst=2, a=2, b=3), dict(op=DIV, dst=2, a=1, b=2), dict(op=CAST, dst=4, a=2, dtype=dtype, rmode=kh.RN),
+            dict(op=ST, a=4)]
+    machine, compiled, want = _both(ko, silu, [x], [dtype], dtype, m, n)
+    _check_ulp(compiled, want, dtype)
+    assert np.array_equal(compiled, machine)
+    gelu = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=MUL, dst=2, a=1, b=1), dict(op=MUL, dst=2, a=2, b=1),
+            c(3, 0.044715), dict(op=FMA, dst=2, a=2, b=3, c=1), c(3, 0.7978845608028654), dict(op=MUL, dst=2, a=2, b=3),
+            dict(op=kh.EW_TANH, dst=2, a=2), c(3, 1.0), dict(op=ADD, dst=2, a=2, b=3), c(3, 0.5), dict(op=MUL, dst=4, a=1, b=3),
+            dict(op=MUL, dst=2, a=2, b=4), dict(op=CAST, dst=5, a=2, dtype=dtype, rmode=kh.RN), dict(op=ST, a=5)]
+    _, compiled, want = _both(ko, gelu, [x], [dtype], dtype, m, n)
+    _check_ulp(compiled, want, dtype)
+
+
+@pytest.mark.parametrize("op", [kh.EW_EXP, kh.EW_EXP2, kh.EW_LOG, kh.EW_LOG2, kh.EW_SQRT, kh.EW_RSQRT, kh.EW_TANH, kh.EW_ERF, kh.EW_ABSF,
+                                kh.EW_NEGF])
+def test_unary_ops_with_special_values(ko, op):
+    m, n = 8, 256
+    x = ko.fill_normal(m * n, kh.F16, 40 + op, 0).reshape(m, n)
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 60000.0, -60000.0, 1e-7, -8.0, 8.0, 11.0, -11.0], dtype=np.float16).view(np.uint16)
+    x.ravel()[:len(sp)] = sp
+    insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=op, dst=1, a=1),
+             dict(op=CAST, dst=2, a=1, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=2)]
+    _, compiled, want = _both(ko, insts, [x], [kh.F16], kh.F16, m, n)
+    _check_ulp(compiled, want, kh.F16)
+
+
+def test_a_kernel_serves_only_the_operand_signature_it_was_compiled_for(ko):
+    """Specialised for two full operands; the same program with a row operand, or at a width that is not a multiple
+    of 8, goes to the machines (and stays correct); the ragged width cannot be specialised at all."""
+    m, n = 16, 128
+    a = ko.fill_normal(m * n, kh.F16, 51, 0).reshape(m, n)
+    b = ko.fill_normal(m * n, kh.F16, 51, 1).reshape(m, n)
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=SUB, dst=2, a=2, b=1), dict(op=ST, a=2)]
+    _, compiled, want = _both(ko, insts, [a, b], [kh.F16] * 2, kh.F16, m, n)
+    assert np.array_equal(compiled, want)
+    before = kh.elementwise_specialize_stats()
+    row = np.ascontiguousarray(b[0])
+    want = np.zeros((m, n), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(a, m, n, n, 1, kh.F16), ko.mk_global(row, 1, n, n, 1, kh.F16)],
+                          ko.mk_global(want, m, n, n, 1, kh.F16)) == 0
+    da, dr, dout = to_dev(a), to_dev(row), dev_zeros(m * n, 2)
+    kh.elementwise(kh.program(insts), [dglobal(da, m, n, n, 1, kh.F16), dglobal(dr, 1, n, n, 1, kh.F16)], dglobal(dout, m, n, n, 1, kh.F16))
+    sync()
+    assert kh.elementwise_specialize_stats() == before
+    assert np.array_equal(to_host(dout, np.uint16, (m, n)), want)
+    n2 = 100
+    a2, b2 = np.ascontiguousarray(a[:, :n2]), np.ascontiguousarray(b[:, :n2])
+    _, second, want = _both(ko, insts, [a2, b2], [kh.F16] * 2, kh.F16, m, n2, expect_compiled=False)
+    assert np.array_equal(second, want)
+
+
+def test_strided_views_with_offsets(ko):
+    """Operands and result are windows of larger buffers (row pitch above the width, a start inside the buffer)."""
+    m, n, pitch = 20, 64, 96
+    a = ko.fill_normal(m * pitch + 16, kh.BF16, 61, 0)
+    b = ko.fill_normal(m * pitch + 16, kh.BF16, 61, 1)
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=1),
+             dict(op=MAX, dst=2, a=2, b=0), dict(op=ST, a=2)]
+    want = np.full(m * pitch + 16, 0x1234, np.uint16)
+    view = lambda mk, buf: mk(buf, m, n, pitch, 1, kh.BF16)
+    def window(g):
+        g.start1, g.end1 = 8, 8 + n
+        return g
+    assert ko.elementwise(ko.program(insts), [window(view(ko.mk_global, a)), window(view(ko.mk_global, b))], window(view(ko.mk_global, want))) == 0
+    da, db = to_dev(a), to_dev(b)
+    dview = lambda t: window(dglobal(t, m, n, pitch, 1, kh.BF16))
+    prog = kh.program(insts)
+    kh.elementwise_specialize(prog, [dview(da), dview(db)], dview(da))
+    dout = to_dev(np.full(m * pitch + 16, 0x1234, np.uint16))
+    before = kh.elementwise_specialize_stats()[1]
+    kh.elementwise(prog, [dview(da), dview(db)], dview(dout))
+    sync()
+    assert kh.elementwise_specialize_stats()[1] == before + 1
+    assert np.array_equal(to_host(dout, np.uint16, (m * pitch + 16,)), want)   # nothing outside the window is touched
+
+
+def test_full_size_program_sampled_against_the_oracle(ko):
+    """z = x*y + x on fp16 8192x8192: the whole result on the GPU, 32 rows spread over it against the oracle."""
+    m = n = 8192
+    x = ko.fill_normal(m * n, kh.F16, 0, 0).reshape(m, n)
+    y = ko.fill_normal(m * n, kh.F16, 0, 1).reshape(m, n)
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=0), dict(op=ST, a=2)]
+    dx, dy, dz = to_dev(x), to_dev(y), dev_zeros(m * n, 2)
+    prog = kh.program(insts)
+    g = lambda t: dglobal(t, m, n, n, 1, kh.F16)
+    kh.elementwise_specialize(prog, [g(dx), g(dy)], g(dz))
+    before = kh.elementwise_specialize_stats()[1]
+    kh.elementwise(prog, [g(dx), g(dy)], g(dz))
+    sync()
+    assert kh.elementwise_specialize_stats()[1] == before + 1
+    got = to_host(dz, np.uint16, (m, n))
+    rows = np.linspace(0, m - 1, 32).astype(int)
+    xs, ys = np.ascontiguousarray(x[rows]), np.ascontiguousarray(y[rows])
+    want = np.zeros((len(rows), n), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(xs, len(rows), n, n, 1, kh.F16), ko.mk_global(ys, len(rows), n, n, 1, kh.F16)],
+                          ko.mk_global(want, len(rows), n, n, 1, kh.F16)) == 0
+    assert np.array_equal(got[rows], want)
+    xf, yf = x.view(np.float16).astype(np.float64), y.view(np.float16).astype(np.float64)   # products and sums exact in fp64
+    whole = ((xf * yf).astype(np.float16).astype(np.float64) + xf).astype(np.float16).view(np.uint16)
+    nan = np.isnan(whole.view(np.float16))
+    assert np.array_equal(got[~nan], whole[~nan])

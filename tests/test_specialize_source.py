@@ -1,0 +1,90 @@
+"""Host-side checks of the specialised-kernel generator: the text it writes for a program, that the runtime compiler
+turns that text into a gfx950 code object (no GPU needed for that), and its refusals."""
+import ctypes as C
+
+import pytest
+
+import kapy_hip as kh
+
+L, ADD, MUL, DIV, ST, CAST, SPL = kh.EW_LD_GLOBAL, kh.EW_ADDF, kh.EW_MULF, kh.EW_DIVF, kh.EW_ST_GLOBAL, kh.EW_FPTOFP, kh.EW_SPLAT
+
+
+def _g(rows, cols, dtype, pitch=None):
+    return kh.mk_global(0x100000, rows, cols, pitch or cols, 1, dtype)
+
+
+def _has_runtime_compiler():
+    for name in ("libhiprtc.so.7", "libhiprtc.so"):
+        try:
+            C.CDLL(name)
+            return True
+        except OSError:
+            pass
+    return False
+
+
+SILU = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=kh.EW_NEGF, dst=2, a=1), dict(op=kh.EW_EXP, dst=2, a=2),
+        dict(op=SPL, dst=3, dtype=kh.F32, imm=1.0), dict(op=ADD, dst=2, a=2, b=3), dict(op=DIV, dst=2, a=1, b=2),
+        dict(op=CAST, dst=4, a=2, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=4)]
+
+
+def test_generated_text_follows_the_program():
+    src, _ = kh.elementwise_source(kh.program(SILU), [_g(16, 256, kh.F16)], _g(16, 256, kh.F16))
+    kernel = src[src.index('extern "C" __global__'):]
+    assert "kapy_ew_specialised(JitArgs p)" in kernel
+    assert "constexpr bool NARROW = true" in kernel
+    assert kernel.count("fetch8(") == 1                      # one operand, fetched once per vector
+    assert "0x3f800000u" in kernel                           # the splat 1.0 as its bit pattern
+    assert "unary8<NARROW>(%d, %d" % (kh.EW_EXP, kh.F32) in kernel and "div8(" in kernel
+    assert "round8" not in kernel                            # every op is fp32; the final cast is the store's own rounding
+    assert "store8<NARROW>(p.out, %d" % kh.F16 in kernel
+    # dead code is not emitted: an unused load and an unused product
+    prog = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ST, a=0)]
+    src, _ = kh.elementwise_source(kh.program(prog), [_g(8, 64, kh.BF16), _g(8, 64, kh.BF16)], _g(8, 64, kh.BF16))
+    kernel = src[src.index('extern "C" __global__'):]
+    assert "raw1" not in kernel and "__fmul_rn" not in kernel
+    # fp8 anywhere takes the machines' wide form
+    prog = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F8E4M3, rmode=kh.RN), dict(op=ST, a=1)]
+    src, _ = kh.elementwise_source(kh.program(prog), [_g(8, 64, kh.F16)], _g(8, 64, kh.F8E4M3))
+    assert "constexpr bool NARROW = false" in src
+
+
+@pytest.mark.skipif(not _has_runtime_compiler(), reason="libhiprtc is not installed")
+def test_generated_text_compiles_for_gfx950():
+    cases = [
+        (SILU, [_g(16, 256, kh.F16)], _g(16, 256, kh.F16)),
+        ([dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=L, dst=2, a=2), dict(op=L, dst=3, a=3), dict(op=MUL, dst=4, a=0, b=1),
+          dict(op=ADD, dst=4, a=4, b=2), dict(op=DIV, dst=4, a=4, b=3), dict(op=kh.EW_TANH, dst=4, a=4), dict(op=ST, a=4)],
+         [_g(32, 64, kh.BF16, 128), _g(1, 64, kh.BF16), _g(32, 1, kh.BF16), _g(1, 1, kh.BF16)], _g(32, 64, kh.BF16)),
+        ([dict(op=L, dst=0, a=0), dict(op=SPL, dst=1, dtype=kh.F32, imm=0.25), dict(op=DIV, dst=0, a=1, b=0), dict(op=DIV, dst=0, a=0, b=1),
+          dict(op=CAST, dst=2, a=0, dtype=kh.F8E5M2, rmode=kh.RZ), dict(op=ST, a=2)], [_g(8, 64, kh.F32)], _g(8, 64, kh.F8E5M2)),
+        ([dict(op=SPL, dst=0, dtype=kh.F16, imm=3.0), dict(op=ST, a=0)], [], _g(8, 64, kh.F16)),
+    ]
+    for insts, ins, out in cases:
+        _, code_bytes = kh.elementwise_source(kh.program(insts), ins, out, compile=True)
+        assert code_bytes > 1000
+
+
+def test_refusals():
+    add = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=ADD, dst=2, a=0, b=1), dict(op=ST, a=2)]
+    def refused(insts, ins, out):
+        with pytest.raises(kh.KapyError) as e:
+            kh.elementwise_source(kh.program(insts), ins, out)
+        return str(e.value)
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(add, [_g(8, 60, kh.F16), _g(8, 60, kh.F16)], _g(8, 60, kh.F16))        # width % 8
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(add, [_g(8, 64, kh.F16, 68), _g(8, 64, kh.F16)], _g(8, 64, kh.F16))    # pitch % 8
+    softmax_like = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=kh.EW_SUBF, dst=0, a=0, b=1), dict(op=ST, a=0)]
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(softmax_like, [_g(8, 64, kh.F16)], _g(8, 64, kh.F16))
+    padded = [dict(op=L, dst=0, a=0, c=kh.PAD_QNAN), dict(op=ST, a=0)]
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(padded, [_g(8, 64, kh.F16)], _g(8, 64, kh.F16))
+    mistyped = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=ADD, dst=2, a=0, b=1), dict(op=ST, a=2)]
+    assert "status %d" % kh.ERR_VERIFY in refused(mistyped, [_g(8, 64, kh.F16), _g(8, 64, kh.BF16)], _g(8, 64, kh.F16))   # the verifier comes first
+
+
+def test_specialise_without_a_gpu_fails_loudly():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(kh.KapyError) as e:
+        kh.elementwise_specialize(kh.program(SILU), [_g(16, 256, kh.F16)], _g(16, 256, kh.F16))
+    assert "no CPU fallback" in str(e.value)

@@ -105,7 +105,8 @@ def bench_copy(kh, steps, warmup):
 def bench_add(kh, steps, warmup, op="add"):
     """z = x + y in fp16 (the reference's elementwise_add.mlir fixture at the headline shape), a plain binary program,
     served by the fused affine kernel; op="expr": z = x*y + x with both roundings, a program outside the fused chains,
-    served by the in-register stack machine."""
+    served by the in-register stack machine; op="expr_compiled": the same program after kapy_elementwise_specialize has
+    compiled it to a kernel of its own; op="swiglu": z = silu(x) * y in fp32 from fp16 operands (ten ops, x used twice), compiled."""
     import torch
     n, sets = 8192, 3
     xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
@@ -116,14 +117,24 @@ def bench_add(kh, steps, warmup, op="add"):
     insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1)]
     if op == "add":
         insts += [dict(op=kh.EW_ADDF, dst=2, a=0, b=1)]
+    elif op == "swiglu":
+        f32 = lambda r: dict(op=kh.EW_FPTOFP, dst=r, a=r, dtype=kh.F32)
+        insts += [f32(0), f32(1), dict(op=kh.EW_NEGF, dst=2, a=0), dict(op=kh.EW_EXP, dst=2, a=2), dict(op=kh.EW_SPLAT, dst=3, dtype=kh.F32, imm=1.0),
+                  dict(op=kh.EW_ADDF, dst=2, a=2, b=3), dict(op=kh.EW_DIVF, dst=2, a=0, b=2), dict(op=kh.EW_MULF, dst=2, a=2, b=1),
+                  dict(op=kh.EW_FPTOFP, dst=2, a=2, dtype=kh.F16, rmode=kh.RN)]
     else:
         insts += [dict(op=kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ADDF, dst=2, a=2, b=0)]
     prog = kh.program(insts + [dict(op=kh.EW_ST_GLOBAL, a=2)])
+    if op in ("expr_compiled", "swiglu"):
+        kh.elementwise_specialize(prog, [gx[0], gy[0]], gz[0])
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gy[i % sets]], gz[i % sets]), steps, warmup)
     nbytes = 3 * n * n * 2
-    name = "elementwise_add fixture: z = x + y fp16 8192x8192" if op == "add" else "z = x*y + x (two roundings) fp16 8192x8192"
+    name = {"add": "elementwise_add fixture: z = x + y fp16 8192x8192", "expr": "z = x*y + x (two roundings) fp16 8192x8192",
+            "expr_compiled": "z = x*y + x (two roundings) fp16 8192x8192, compiled at run time",
+            "swiglu": "z = silu(x)*y fp16 8192x8192 in fp32, compiled at run time"}[op]
+    kernel = {"add": "affine_act_kernel", "expr": "stack_kernel_narrow"}.get(op, "kapy_ew_specialised")
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev, "add" if op == "add" else None), "kernel": "affine_act_kernel" if op == "add" else "stack_kernel_narrow"}
+            "roofline": _roof_hbm(nbytes, ev, "add" if op == "add" else None), "kernel": kernel}
 
 
 def bench_reduce(kh, steps, warmup):
@@ -257,7 +268,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -273,6 +284,8 @@ def main():
         "gelu": lambda s, w: bench_gelu(kh, s, w),
         "add": lambda s, w: bench_add(kh, s, w),
         "expr": lambda s, w: bench_add(kh, s, w, "expr"),
+        "expr_compiled": lambda s, w: bench_add(kh, s, w, "expr_compiled"),
+        "swiglu": lambda s, w: bench_add(kh, s, w, "swiglu"),
         "copy": lambda s, w: bench_copy(kh, s, w),
         "transpose": lambda s, w: bench_transpose(kh, s, w),
         "reduce": lambda s, w: bench_reduce(kh, s, w),
@@ -288,10 +301,14 @@ def main():
     others = []
     if not args.no_others:
         for name, fn in table.items():
-            if name == args.workload:
+            if name == args.workload or (name == "expr" and args.workload == "expr_compiled"):   # once compiled, the program no longer reaches the machine
                 continue
             torch.cuda.empty_cache()
-            r = fn(min(args.steps, 20), min(args.warmup, 10))
+            try:
+                r = fn(min(args.steps, 20), min(args.warmup, 10))
+            except kh.KapyError as e:   # e.g. no runtime compiler on this machine for the compiled workloads
+                others.append({"workload": name, "error": str(e)})
+                continue
             r["value"] = round(r["value"], 2)
             r["ms_per_step"] = round(r["ms_per_step"], 4)
             r["kernel_ms"] = round(r["kernel_ms"], 4)

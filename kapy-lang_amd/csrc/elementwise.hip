@@ -708,13 +708,13 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   if (o0 <= 0 || o1 <= 0) return KAPY_OK;
   hipStream_t s = (hipStream_t)stream;
 
-  bool has_reduce = false;
-  for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
-  if (has_reduce) return run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
-
   // a kernel compiled for exactly this program and operand signature, if the caller asked for one
   rc = launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s);
   if (rc != 0) return rc < 0 ? rc : KAPY_OK;
+
+  bool has_reduce = false;
+  for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
+  if (has_reduce) return run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
 
   AffineActParams ap;
   int T = -1;

@@ -9,6 +9,11 @@
 // gfx950 with the runtime compiler (libhiprtc, opened on first use; absent => KAPY_ERR_UNSUPPORTED and the machines keep
 // serving), loads the code object and keeps it in a process-wide table keyed by program and operand signature.
 // kapy_elementwise looks a verified program up in that table before it falls back to the machines.
+//
+// Two skeletons.  A program without a reduce: two vectors of 8 elements per lane, every load issued before any
+// arithmetic.  A program with reduces along the rows (the row machine's business otherwise): a workgroup keeps a
+// whole row in registers, CH vectors per lane, walks rows blockIdx.x, +gridDim.x, ... with the next row's loads in
+// flight, and evaluates the program with row values (CH x 8 registers) and per-row values (one register).
 #include <dlfcn.h>
 #include <hip/hiprtc.h>
 #include <string.h>
@@ -50,6 +55,52 @@ __device__ __forceinline__ void copy8(float (&x)[8], const float (&y)[8]) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = y[e];
 }
+// Sum or maximum of one row value over its row (the row machine's reduce step): each lane folds its active chunks, a
+// butterfly folds the wave, the waves meet in `red` (one barrier).  A NaN anywhere makes the maximum NaN.
+template <int CH, int THREADS, bool SUM>
+__device__ __forceinline__ float row_reduce(const float (&v)[CH][8], int32_t vec_per_row, float *red) {
+  const int tid = threadIdx.x;
+  float acc = SUM ? 0.f : -__builtin_inff();
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    if (c * THREADS + tid < vec_per_row) {
+      float part;
+      if (SUM) part = ((v[c][0] + v[c][1]) + (v[c][2] + v[c][3])) + ((v[c][4] + v[c][5]) + (v[c][6] + v[c][7]));
+      else {
+        part = fmaxf(fmaxf(fmaxf(v[c][0], v[c][1]), fmaxf(v[c][2], v[c][3])), fmaxf(fmaxf(v[c][4], v[c][5]), fmaxf(v[c][6], v[c][7])));
+        bool any_nan = false;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) any_nan |= v[c][e] != v[c][e];
+        if (any_nan) part = __builtin_nanf("");
+      }
+      acc = SUM ? acc + part : max_nan(acc, part);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float other = __shfl_xor(acc, off, 64);
+    acc = SUM ? acc + other : max_nan(acc, other);
+  }
+  if (THREADS > 64) {
+    constexpr int WAVES = THREADS / 64;
+    if ((tid & 63) == 0) red[tid >> 6] = acc;
+    __syncthreads();
+    acc = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) acc = SUM ? acc + red[w] : max_nan(acc, red[w]);
+  }
+  return acc;
+}
+// The lane's CH vectors of one row of an operand (vector c*THREADS + lane; nothing is read past the row's end).
+template <int CH, int THREADS>
+__device__ __forceinline__ void row_fetch8(const StackIn &g, int32_t i, int32_t vec_per_row, bool streaming, Raw8 (&raw)[CH]) {
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int32_t jv = c * THREADS + (int32_t)threadIdx.x;
+    raw[c].lo = raw[c].hi = u32x4{0, 0, 0, 0};
+    if (jv < vec_per_row) raw[c] = fetch8(g, i, jv, streaming);
+  }
+}
 )";
 
 const char *kPrelude =
@@ -66,6 +117,8 @@ struct Signature {
   int in_dtype[kJitInputs], in_kind[kJitInputs];
   int out_dtype = 0;
   bool narrow = true;
+  bool rowwise = false;      // the program reduces along rows: the row skeleton, compiled for one (threads, chunks) shape
+  int threads = 256, chunks = 1;
 };
 
 // Which programs a specialised kernel serves and how each operand is read: the result and the full / row operands
@@ -77,7 +130,10 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
   int stores = 0;
   for (int k = 0; k < n_inst; ++k) {
     const int op = prog[k].op;
-    if (op == KAPY_EW_REDUCE_SUM || op == KAPY_EW_REDUCE_MAX) return false;
+    if (op == KAPY_EW_REDUCE_SUM || op == KAPY_EW_REDUCE_MAX) {
+      if (prog[k].b != 1) return false;  // along columns: not resident per workgroup
+      sig->rowwise = true;
+    }
     if (op == KAPY_EW_LD_GLOBAL && prog[k].c != KAPY_PAD_ZERO) return false;
     stores += op == KAPY_EW_ST_GLOBAL;
   }
@@ -87,6 +143,12 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
   if (!is_float(out->dtype) || out->stride1 != 1 || o1 % 8 != 0) return false;
   if (((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
   if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  if (sig->rowwise) {
+    const int64_t vpr = o1 / 8;
+    if (vpr > 4096) return false;  // a row of more than 32768 elements does not stay in one workgroup's registers
+    sig->threads = vpr <= 256 ? 64 : vpr <= 1024 ? 256 : 1024;
+    sig->chunks = (int)((vpr + sig->threads - 1) / sig->threads);
+  }
   sig->n_ins = n_ins;
   sig->out_dtype = out->dtype;
   sig->narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
@@ -131,6 +193,10 @@ std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig)
     key.push_back((char)sig.in_kind[k]);
   }
   key.push_back((char)sig.out_dtype);
+  if (sig.rowwise) {
+    key.push_back((char)(sig.threads / 64));
+    key.push_back((char)sig.chunks);
+  }
   return key;
 }
 
@@ -144,20 +210,22 @@ void appendf(std::string &s, const char *fmt, ...) {
   s += buf;
 }
 
-// The program as straight-line code: every value that the store depends on becomes one array of 8 fp32 (the exact
-// image of the typed value, rounded to the op's result type after every op, as the machines do), a splat one constant.
-std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig) {
-  struct Node {
-    int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
-    float imm = 0.f;
-    bool used = false;
-    std::string name;   // the array (or constant) holding the value
-    bool is_const = false;
-  };
+struct Node {
+  int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
+  float imm = 0.f;
+  bool used = false;
+  std::string name;  // the array, register or constant holding the value
+  bool is_const = false;
+  bool uniform = false;  // row skeleton: one value per row (a reduce's result, a column or scalar operand, a splat, and what follows from those)
+};
+
+// The program's values in program order (the store is not one of them: its operand's index goes to *stored), with
+// `used` set on those the store depends on.
+std::vector<Node> build_nodes(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, int *stored, std::vector<char> *input_used) {
   std::vector<Node> nodes;
   int reg[64];
   for (int &r : reg) r = -1;
-  int stored = -1;
+  *stored = -1;
   for (int k = 0; k < n_inst; ++k) {
     const kapy_ew_inst &I = prog[k];
     Node n;
@@ -168,7 +236,7 @@ std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dty
     switch (I.op) {
     case KAPY_EW_LD_GLOBAL: n.input = I.a; break;
     case KAPY_EW_SPLAT: break;
-    case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; continue;
+    case KAPY_EW_ST_GLOBAL: *stored = reg[I.a]; continue;
     case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
     case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
       n.a = reg[I.a]; n.b = reg[I.b]; break;
@@ -177,26 +245,51 @@ std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dty
     nodes.push_back(n);
     reg[I.dst] = (int)nodes.size() - 1;
   }
-  {  // mark what the store needs
-    std::vector<int> todo{stored};
-    while (!todo.empty()) {
-      const int id = todo.back();
-      todo.pop_back();
-      if (id < 0 || nodes[id].used) continue;
-      nodes[id].used = true;
-      todo.push_back(nodes[id].a);
-      todo.push_back(nodes[id].b);
-      todo.push_back(nodes[id].c);
-    }
+  std::vector<int> todo{*stored};
+  while (!todo.empty()) {
+    const int id = todo.back();
+    todo.pop_back();
+    if (id < 0 || nodes[id].used) continue;
+    nodes[id].used = true;
+    todo.push_back(nodes[id].a);
+    todo.push_back(nodes[id].b);
+    todo.push_back(nodes[id].c);
   }
-  std::vector<char> input_used(kJitInputs, 0);
+  input_used->assign(kJitInputs, 0);
   for (const Node &n : nodes)
-    if (n.used && n.op == KAPY_EW_LD_GLOBAL) input_used[n.input] = 1;
+    if (n.used && n.op == KAPY_EW_LD_GLOBAL) (*input_used)[n.input] = 1;
+  return nodes;
+}
 
+std::string source_head() {
   std::string s = kPrelude;
   s += "namespace kapy { namespace {\n";
   s += kArgsText;
   s += "} }\nusing namespace kapy;\n";
+  return s;
+}
+
+// splats: one rounding to the splat's type, as the machines do when they push an immediate
+void emit_splats(std::string &s, std::vector<Node> &nodes) {
+  for (size_t id = 0; id < nodes.size(); ++id) {
+    Node &n = nodes[id];
+    if (!n.used || n.op != KAPY_EW_SPLAT) continue;
+    uint32_t bits;
+    memcpy(&bits, &n.imm, 4);
+    n.name = "c" + std::to_string(id);
+    n.is_const = n.uniform = true;
+    appendf(s, "  const float %s = round_to_dtype(bits_f32(0x%08xu), %d, true);\n", n.name.c_str(), bits, n.dtype);
+  }
+}
+
+// A program without a reduce as straight-line code: every value that the store depends on becomes one array of 8 fp32
+// (the exact image of the typed value, rounded to the op's result type after every op, as the machines do), a splat one
+// constant.
+std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig) {
+  int stored = -1;
+  std::vector<char> input_used;
+  std::vector<Node> nodes = build_nodes(prog, n_inst, result_dtype, &stored, &input_used);
+  std::string s = source_head();
   s += "extern \"C\" __global__ __launch_bounds__(256) void kapy_ew_specialised(JitArgs p) {\n";
   appendf(s, "  constexpr bool NARROW = %s;\n", sig.narrow ? "true" : "false");
   s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
@@ -207,16 +300,7 @@ std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dty
     if (sig.in_kind[k] == kFull || sig.in_kind[k] == kRow) appendf(s, "  Raw8 raw%d[2];\n", k);
     else appendf(s, "  float raw%d[2];\n", k);
   }
-  // splats: one rounding to the splat's type, as the machines do when they push an immediate
-  for (size_t id = 0; id < nodes.size(); ++id) {
-    Node &n = nodes[id];
-    if (!n.used || n.op != KAPY_EW_SPLAT) continue;
-    uint32_t bits;
-    memcpy(&bits, &n.imm, 4);
-    n.name = "c" + std::to_string(id);
-    n.is_const = true;
-    appendf(s, "  const float %s = round_to_dtype(bits_f32(0x%08xu), %d, true);\n", n.name.c_str(), bits, n.dtype);
-  }
+  emit_splats(s, nodes);
   s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
        "    const uint32_t slot = first + u * 256u;\n"
        "    row[u] = -1;\n"
@@ -296,6 +380,161 @@ std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dty
   return s;
 }
 
+// A program with reduces along the rows.  Row values are arrays [CH][8], per-row values single registers; operands that
+// are one row for all rows ([1 x n]: a norm's gamma and beta) are read once per workgroup and parked, as they lie in
+// memory, in each lane's own corner of the dynamic LDS (*lds_bytes; read at their use from L2 instead when that corner
+// would exceed 48 KiB).  Two exchange areas serve the reduces in turn, counted across rows: a wave can write one again
+// only after the barrier of the other, which every wave reaches after it has read the first.
+std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, int *lds_bytes) {
+  int stored = -1;
+  std::vector<char> input_used;
+  std::vector<Node> nodes = build_nodes(prog, n_inst, result_dtype, &stored, &input_used);
+  const int CH = sig.chunks, TH = sig.threads;
+  // parked row operands: 16 bytes per lane and chunk, twice that for f32
+  int park_slot[kJitInputs], n_park = 0;
+  for (int k = 0; k < sig.n_ins; ++k) {
+    park_slot[k] = -1;
+    if (input_used[k] && sig.in_kind[k] == kRow) {
+      park_slot[k] = n_park;
+      n_park += sig.in_dtype[k] == KAPY_F32 ? 2 : 1;
+    }
+  }
+  const bool park = n_park > 0 && n_park * CH * TH * 16 <= 48 * 1024;
+  *lds_bytes = park ? n_park * CH * TH * 16 : 0;
+
+  std::string s = source_head();
+  appendf(s, "extern \"C\" __global__ __launch_bounds__(%d) void kapy_ew_specialised(JitArgs p) {\n", TH);
+  appendf(s, "  constexpr bool NARROW = %s;\n  constexpr int CH = %d, THREADS = %d;\n", sig.narrow ? "true" : "false", CH, TH);
+  s += "  __shared__ float red[2][16];\n  extern __shared__ u32x4 parked[];\n  int phase = 0;\n  const int32_t vpr = p.vec_per_row;\n";
+  emit_splats(s, nodes);
+  for (int k = 0; k < sig.n_ins; ++k) {
+    if (!input_used[k]) continue;
+    const int kind = sig.in_kind[k], dt = sig.in_dtype[k];
+    appendf(s, "  const StackIn g%d{p.in[%d], p.stride0[%d], %d, %d};\n", k, k, k, dt, kind == kRow ? 1 : 0);
+    if (kind == kFull) appendf(s, "  Raw8 raw%d[CH];\n  row_fetch8<CH, THREADS>(g%d, blockIdx.x, vpr, true, raw%d);\n", k, k, k);
+    else if (kind == kRow && park) {
+      appendf(s, "  {\n    Raw8 t[CH];\n    row_fetch8<CH, THREADS>(g%d, 0, vpr, false, t);\n#pragma unroll\n    for (int c = 0; c < CH; ++c) {\n"
+                 "      parked[(%d * CH + c) * THREADS + threadIdx.x] = t[c].lo;\n", k, park_slot[k]);
+      if (dt == KAPY_F32) appendf(s, "      parked[(%d * CH + c) * THREADS + threadIdx.x] = t[c].hi;\n", park_slot[k] + 1);
+      s += "    }\n  }\n";
+    } else if (kind == kScalar) appendf(s, "  const float s%d = load_as_f32(p.in[%d], %d, 0);\n", k, k, dt);
+  }
+  s += "  for (int32_t i = blockIdx.x; i < p.rows; i += gridDim.x) {\n";
+  // the row operands first: their registers are asked for again (the next row) right after
+  std::string full_name[kJitInputs];
+  for (int k = 0; k < sig.n_ins; ++k) {
+    if (!input_used[k] || sig.in_kind[k] != kFull) continue;
+    full_name[k] = "x" + std::to_string(k);
+    appendf(s, "    float x%d[CH][8];\n#pragma unroll\n    for (int c = 0; c < CH; ++c) widen8(raw%d[c], %d, x%d[c]);\n", k, k, sig.in_dtype[k], k);
+  }
+  for (int k = 0; k < sig.n_ins; ++k)
+    if (input_used[k] && sig.in_kind[k] == kFull)
+      appendf(s, "    if (i + (int32_t)gridDim.x < p.rows) row_fetch8<CH, THREADS>(g%d, i + gridDim.x, vpr, true, raw%d);\n", k, k);
+
+  auto elem = [&](int id) { return nodes[id].uniform ? nodes[id].name : nodes[id].name + "[c][e]"; };
+  int n_filled = 0;
+  // a per-row value as an array of 8 (div8 and the store take arrays)
+  auto filled = [&](int id) {
+    const std::string a = "f" + std::to_string(n_filled++);
+    appendf(s, "    float %s[8]; fill8(%s, %s);\n", a.c_str(), a.c_str(), nodes[id].name.c_str());
+    return a;
+  };
+  const char *kChunks = "#pragma unroll\n    for (int c = 0; c < CH; ++c)";
+  for (size_t id = 0; id < nodes.size(); ++id) {
+    Node &n = nodes[id];
+    if (!n.used || n.op == KAPY_EW_SPLAT) continue;
+    const bool reduce = n.op == KAPY_EW_REDUCE_SUM || n.op == KAPY_EW_REDUCE_MAX;
+    n.uniform = reduce || ((n.a < 0 || nodes[n.a].uniform) && (n.b < 0 || nodes[n.b].uniform) && (n.c < 0 || nodes[n.c].uniform) && n.op != KAPY_EW_LD_GLOBAL);
+    if (n.op == KAPY_EW_LD_GLOBAL) n.uniform = sig.in_kind[n.input] == kCol || sig.in_kind[n.input] == kScalar;
+    n.name = (n.uniform ? "u" : "v") + std::to_string(id);
+    const char *vn = n.name.c_str();
+    const std::string dt = std::to_string(n.dtype);
+    auto round_result = [&]() {
+      if (n.dtype == KAPY_F32) return;
+      if (n.uniform) appendf(s, "    %s = round_to_dtype(%s, %d, true);\n", vn, vn, n.dtype);
+      else appendf(s, "    %s round8<NARROW>(%s[c], %d, true);\n", kChunks, vn, n.dtype);
+    };
+    auto assign = [&](const std::string &expr) {
+      if (n.uniform) appendf(s, "    float %s = %s;\n", vn, expr.c_str());
+      else appendf(s, "    float %s[CH][8];\n    %s\n#pragma unroll\n      for (int e = 0; e < 8; ++e) %s[c][e] = %s;\n", vn, kChunks, vn, expr.c_str());
+    };
+    switch (n.op) {
+    case KAPY_EW_LD_GLOBAL: {
+      const int k = n.input, kind = sig.in_kind[k];
+      if (kind == kFull) n.name = full_name[k];
+      else if (kind == kCol) appendf(s, "    const float %s = load_as_f32(p.in[%d], %d, (int64_t)i * p.stride0[%d]);\n", vn, k, sig.in_dtype[k], k);
+      else if (kind == kScalar) n.name = "s" + std::to_string(k);
+      else {
+        appendf(s, "    float %s[CH][8];\n    %s {\n      Raw8 t;\n      t.lo = t.hi = u32x4{0, 0, 0, 0};\n", vn, kChunks);
+        if (park) {
+          appendf(s, "      t.lo = parked[(%d * CH + c) * THREADS + threadIdx.x];\n", park_slot[k]);
+          if (sig.in_dtype[k] == KAPY_F32) appendf(s, "      t.hi = parked[(%d * CH + c) * THREADS + threadIdx.x];\n", park_slot[k] + 1);
+        } else appendf(s, "      if (c * THREADS + (int32_t)threadIdx.x < vpr) t = fetch8(g%d, 0, c * THREADS + (int32_t)threadIdx.x, false);\n", k);
+        appendf(s, "      widen8(t, %d, %s[c]);\n    }\n", sig.in_dtype[k], vn);
+      }
+      break;
+    }
+    case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX:
+      if (nodes[n.a].uniform) {  // the same value n times
+        if (n.op == KAPY_EW_REDUCE_SUM) appendf(s, "    float %s = __fmul_rn(%s, (float)(vpr * 8));\n", vn, nodes[n.a].name.c_str());
+        else appendf(s, "    float %s = %s;\n", vn, nodes[n.a].name.c_str());
+      } else {
+        appendf(s, "    float %s = row_reduce<CH, THREADS, %s>(%s, vpr, red[phase & 1]);\n    ++phase;\n", vn, n.op == KAPY_EW_REDUCE_SUM ? "true" : "false",
+                nodes[n.a].name.c_str());
+      }
+      round_result();
+      break;
+    case KAPY_EW_FPTOFP: {
+      const bool free_cast = n.dtype == KAPY_F32 || ((int)id == stored && n.dtype == sig.out_dtype && n.rmode != KAPY_RZ);
+      if (free_cast) n.name = nodes[n.a].name;
+      else if (n.uniform) appendf(s, "    float %s = round_to_dtype(%s, %d, %s);\n", vn, nodes[n.a].name.c_str(), n.dtype, n.rmode != KAPY_RZ ? "true" : "false");
+      else {
+        assign(elem(n.a));
+        appendf(s, "    %s round8<NARROW>(%s[c], %d, %s);\n", kChunks, vn, n.dtype, n.rmode != KAPY_RZ ? "true" : "false");
+      }
+      break;
+    }
+    case KAPY_EW_ADDF: assign("__fadd_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_SUBF: assign("__fsub_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MULF: assign("__fmul_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MAXIMUMF: assign("max_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MINIMUMF: assign("min_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_FMA: assign("fma_typed(" + elem(n.a) + ", " + elem(n.b) + ", " + elem(n.c) + ", " + dt + ")"); round_result(); break;
+    case KAPY_EW_DIVF:
+      if (n.uniform) assign("__fdiv_rn(" + elem(n.a) + ", " + elem(n.b) + ")");
+      else {
+        const std::string a = nodes[n.a].uniform ? filled(n.a) : nodes[n.a].name + "[c]";
+        const std::string b = nodes[n.b].uniform ? filled(n.b) : nodes[n.b].name + "[c]";
+        appendf(s, "    float %s[CH][8];\n    %s div8(%s, %s, %s[c]);\n", vn, kChunks, a.c_str(), b.c_str(), vn);
+      }
+      round_result();
+      break;
+    default:  // the unary ops
+      if (n.uniform) assign("apply_unary(" + std::to_string(n.op) + ", " + elem(n.a) + ")");
+      else {
+        assign(elem(n.a));
+        appendf(s, "    %s unary8<NARROW>(%d, %d, %s[c]);\n", kChunks, n.op, n.dtype, vn);
+      }
+      round_result();
+    }
+  }
+  if (nodes[stored].uniform) {
+    const std::string a = filled(stored);
+    appendf(s, "    %s {\n      const int32_t jv = c * THREADS + (int32_t)threadIdx.x;\n      if (jv < vpr) store8<NARROW>(p.out, %d, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, %s);\n    }\n",
+            kChunks, sig.out_dtype, a.c_str());
+  } else {
+    appendf(s, "    %s {\n      const int32_t jv = c * THREADS + (int32_t)threadIdx.x;\n      if (jv < vpr) store8<NARROW>(p.out, %d, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, %s[c]);\n    }\n",
+            kChunks, sig.out_dtype, nodes[stored].name.c_str());
+  }
+  s += "  }\n}\n";
+  return s;
+}
+
+std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, int *lds_bytes) {
+  *lds_bytes = 0;
+  return sig.rowwise ? generate_rows(prog, n_inst, result_dtype, sig, lds_bytes) : generate_flat(prog, n_inst, result_dtype, sig);
+}
+
 // ---- the runtime compiler, opened on first use --------------------------------------------------------------------
 struct Rtc {
   void *handle = nullptr;
@@ -362,6 +601,8 @@ int compile_source(const std::string &source, std::vector<char> *code) {
 struct Loaded {
   hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
+  int lds_bytes = 0;   // row skeleton: the parked row operands
+  int resident = 0;    // row skeleton: workgroups the device holds at once (each walks its share of the rows)
 };
 std::mutex g_mutex;
 std::map<std::pair<int, std::string>, Loaded> g_table;  // (device, key) -> kernel
@@ -374,8 +615,8 @@ int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
   Signature sig;
   if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
     return fail(KAPY_ERR_UNSUPPORTED,
-                "elementwise_specialize: needs one store, no reduce, zero padding, rows of a multiple of 8 contiguous elements aligned to 8 "
-                "elements, and operands that are full, row, column or scalar views");
+                "elementwise_specialize: needs one store, reduces only along rows of at most 32768 elements, zero padding, rows of a multiple of 8 "
+                "contiguous elements aligned to 8 elements, and operands that are full, row, column or scalar views");
   int device = 0;
   KAPY_HIP_CHECK(hipGetDevice(&device));
   const std::string key = make_key(prog, n_inst, sig);
@@ -384,11 +625,16 @@ int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
     if (g_table.count({device, key})) return KAPY_OK;
   }
   std::vector<char> code;
-  int rc = compile_source(generate(prog, n_inst, result_dtype, sig), &code);
-  if (rc) return rc;
   Loaded k;
+  int rc = compile_source(generate(prog, n_inst, result_dtype, sig, &k.lds_bytes), &code);
+  if (rc) return rc;
   KAPY_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
   KAPY_HIP_CHECK(hipModuleGetFunction(&k.fn, k.module, "kapy_ew_specialised"));
+  if (sig.rowwise) {
+    int per_cu = 1;
+    KAPY_HIP_CHECK(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k.fn, sig.threads, (size_t)k.lds_bytes));
+    k.resident = device_cus() * (per_cu > 0 ? per_cu : 1);
+  }
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!g_table.emplace(std::make_pair(device, key), k).second) (void)hipModuleUnload(k.module);  // another thread was first
   else g_count.fetch_add(1);
@@ -421,8 +667,13 @@ int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_d
   args.vec_per_row = (int32_t)(extent1(out) / 8);
   size_t size = sizeof args;
   void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-  const int64_t slots = (int64_t)args.rows * args.vec_per_row;
-  KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, (unsigned)((slots + 511) / 512), 1, 1, 256, 1, 1, 0, stream, nullptr, extra));
+  if (sig.rowwise) {
+    const unsigned grid = (unsigned)std::min<int64_t>(args.rows, k.resident);
+    KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, grid, 1, 1, (unsigned)sig.threads, 1, 1, (unsigned)k.lds_bytes, stream, nullptr, extra));
+  } else {
+    const int64_t slots = (int64_t)args.rows * args.vec_per_row;
+    KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, (unsigned)((slots + 511) / 512), 1, 1, 256, 1, 1, 0, stream, nullptr, extra));
+  }
   g_launches.fetch_add(1, std::memory_order_relaxed);
   return 1;
 }
@@ -437,7 +688,8 @@ int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_d
   Signature sig;
   if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
     return fail(KAPY_ERR_UNSUPPORTED, "elementwise_source: the program or its operands do not fit a specialised kernel");
-  const std::string text = generate(prog, n_inst, result_dtype, sig);
+  int lds_bytes = 0;
+  const std::string text = generate(prog, n_inst, result_dtype, sig, &lds_bytes);
   if (source && capacity > 0) {
     const size_t n = std::min<size_t>(text.size(), (size_t)capacity - 1);
     memcpy(source, text.data(), n);

@@ -208,3 +208,100 @@ def test_full_size_program_sampled_against_the_oracle(ko):
     whole = ((xf * yf).astype(np.float16).astype(np.float64) + xf).astype(np.float16).view(np.uint16)
     nan = np.isnan(whole.view(np.float16))
     assert np.array_equal(got[~nan], whole[~nan])
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Programs with reduces along the rows: compiled onto the row skeleton (a workgroup keeps the row in registers).
+def _check_ulp_away_from_cancellation(got, want, dtype, floor=1e-6):
+    """<= 2 ulp, except where gamma*xhat + beta cancels to almost nothing: there a sum taken in another order (1e-7 of the
+    addends) is many ulp of the tiny result, so an absolute error below `floor` passes as well."""
+    f = (lambda a: a.view(np.float16).astype(np.float64)) if dtype == kh.F16 else \
+        (lambda a: (a.astype(np.uint32) << 16).view(np.float32).astype(np.float64))
+    g, w = f(got), f(want)
+    far = ~(np.abs(g - w) <= floor)
+    _check_ulp(got[far], want[far], dtype)
+
+
+def _row_both(ko, insts, dtype, m, n, seed, extra=0, std=2.0, col=False):
+    x = ko.fill_normal(m * n, dtype, seed, std=std).reshape(m, n)
+    rows = [ko.fill_normal(n, dtype, seed + 1 + k, mean=1.0 if k == 0 else 0.0, std=0.5) for k in range(extra)]
+    ins, shapes = [x] + rows, [(m, n)] + [(1, n)] * extra
+    if col:
+        ins.append(ko.fill_uniform(m, dtype, seed + 9, 0, 0.5, 2.0))
+        shapes.append((m, 1))
+    return _both(ko, insts, ins, [dtype] * len(ins), dtype, m, n, in_shapes=shapes)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(7, 64), (5, 1000), (33, 4096), (700, 8192), (4, 12288), (3, 32768)])
+def test_compiled_softmax_every_launch_shape(ko, dtype, m, n):
+    _, compiled, want = _row_both(ko, kh.softmax_insts(dtype), dtype, m, n, 50 + n % 97)
+    _check_ulp(compiled, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(12, 1024), (600, 8192), (5, 200), (3, 32768)])
+def test_compiled_layernorm_and_rmsnorm(ko, dtype, m, n):
+    """gamma and beta are parked in LDS where that fits 48 KiB (not at 32768 columns: read through L2 there)."""
+    _, compiled, want = _row_both(ko, kh.layernorm_insts(n, dtype), dtype, m, n, 61, extra=2)
+    _check_ulp_away_from_cancellation(compiled, want, dtype)
+    _, compiled, want = _row_both(ko, kh.layernorm_insts(n, dtype, affine=False), dtype, m, n, 62)
+    _check_ulp(compiled, want, dtype)
+    _, compiled, want = _row_both(ko, kh.rmsnorm_insts(n, dtype), dtype, m, n, 63, extra=1)
+    _check_ulp(compiled, want, dtype)
+
+
+def test_compiled_row_program_with_special_values_reused_values_and_a_column_operand(ko):
+    m, n = 6, 1024
+    x = ko.fill_normal(m * n, kh.F16, 55, std=4.0).reshape(m, n)
+    x[1, 3] = 0x7e00                 # a NaN poisons its row
+    x[2, 9] = 0x7c00                 # +inf: inf - inf
+    x[3, :] = 0xfc00                 # a row of -inf
+    x[4, :] = 0x7bff                 # a row of the largest finite value: uniform 1/n
+    _, compiled, want = _both(ko, kh.softmax_insts(kh.F16), [x], [kh.F16], kh.F16, m, n)
+    _check_ulp(compiled, want, kh.F16)
+    assert np.all(np.isnan(compiled[[1, 2, 3]].view(np.float16))) and np.all(compiled[4] == np.float16(1.0 / n).view(np.uint16))
+    # (e / sum(e)) * e * col with e = exp(x): e is used three times, the per-row sum divides a row value, a [m x 1] operand scales rows
+    insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=kh.EW_EXP, dst=1, a=1), dict(op=kh.EW_REDUCE_SUM, dst=2, a=1, b=1),
+             dict(op=DIV, dst=3, a=1, b=2), dict(op=MUL, dst=3, a=3, b=1), dict(op=L, dst=5, a=1), dict(op=CAST, dst=5, a=5, dtype=kh.F32),
+             dict(op=MUL, dst=3, a=3, b=5), dict(op=CAST, dst=4, a=3, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=4)]
+    _, compiled, want = _row_both(ko, insts, kh.F16, 10, 2048, 71, std=1.0, col=True)
+    _check_ulp(compiled, want, kh.F16)
+    # the row maximum broadcast back (the stored value is a per-row value), and the sum of a per-row value (n times the maximum)
+    prog = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=ST, a=1)]
+    xs = ko.fill_normal(4 * 512, kh.F16, 72).reshape(4, 512)
+    xs[1, 100], xs[2, 7] = 0x7e00, 0x7c00
+    _, compiled, want = _both(ko, prog, [xs], [kh.F16], kh.F16, 4, 512)
+    assert np.array_equal(compiled[[0, 2, 3]], want[[0, 2, 3]]) and np.all(np.isnan(compiled[1].view(np.float16)))
+    prog = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1),
+            dict(op=kh.EW_REDUCE_SUM, dst=2, a=1, b=1), dict(op=SUB, dst=0, a=0, b=2), dict(op=CAST, dst=3, a=0, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=3)]
+    _, compiled, want = _both(ko, prog, [ko.fill_normal(8 * 256, kh.F16, 73).reshape(8, 256)], [kh.F16], kh.F16, 8, 256)
+    _check_ulp(compiled, want, kh.F16)
+
+
+def test_compiled_softmax_f32_in_and_out(ko):
+    m, n = 8, 2048
+    x = ko.fill_normal(m * n, kh.F32, 81, std=2.0).reshape(m, n)
+    insts = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=SUB, dst=0, a=0, b=1),
+             dict(op=kh.EW_EXP, dst=0, a=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=0, b=1), dict(op=DIV, dst=0, a=0, b=1), dict(op=ST, a=0)]
+    _, compiled, want = _both(ko, insts, [x], [kh.F32], kh.F32, m, n)
+    g, w = compiled.view(np.float32).astype(np.float64), want.view(np.float32).astype(np.float64)
+    assert np.max(np.abs(g - w) / w) <= 4e-6        # fp32 exp (2 ulp) and a sum in another order
+    assert np.allclose(g.sum(axis=1), 1.0, atol=1e-5)
+
+
+def test_a_row_kernel_serves_only_its_own_width_class(ko):
+    """Compiled for rows of 8192 elements (256 lanes x 4 vectors); rows of 1280 (64 lanes x 3 vectors, a shape no other
+    test compiles softmax for) run the hand-written kernel until they get a compiled one of their own."""
+    insts = kh.softmax_insts(kh.F16)
+    _row_both(ko, insts, kh.F16, 16, 8192, 90)
+    before = kh.elementwise_specialize_stats()
+    m, n = 16, 1280
+    x = ko.fill_normal(m * n, kh.F16, 91).reshape(m, n)
+    want = np.zeros((m, n), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(x, m, n, n, 1, kh.F16)], ko.mk_global(want, m, n, n, 1, kh.F16)) == 0
+    dx, dout = to_dev(x), dev_zeros(m * n, 2)
+    kh.elementwise(kh.program(insts), [dglobal(dx, m, n, n, 1, kh.F16)], dglobal(dout, m, n, n, 1, kh.F16))
+    sync()
+    assert kh.elementwise_specialize_stats() == before
+    _check_ulp(to_host(dout, np.uint16, (m, n)), want, kh.F16)

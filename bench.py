@@ -164,13 +164,20 @@ def bench_rowwise(kh, steps, warmup, which):
     gx, gy = [g(t) for t in xs], [g(t) for t in ys]
     if which == "softmax":
         prog, extra = kh.program(kh.softmax_insts(kh.F16)), []
+    elif which == "l2norm_compiled":   # x / |x| per row: a row program without a hand-written kernel, compiled at run time
+        f32 = dict(op=kh.EW_FPTOFP, dst=0, a=0, dtype=kh.F32)
+        prog, extra = kh.program([dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), f32, dict(op=kh.EW_MULF, dst=1, a=0, b=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=1, b=1),
+                                  dict(op=kh.EW_RSQRT, dst=1, a=1), dict(op=kh.EW_MULF, dst=0, a=0, b=1),
+                                  dict(op=kh.EW_FPTOFP, dst=2, a=0, dtype=kh.F16, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=2)]), []
+        kh.elementwise_specialize(prog, [gx[0]], gy[0])
     else:
         prog, extra = kh.program(kh.layernorm_insts(n, kh.F16)), [row(gamma), row(beta)]
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]] + extra, gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
-    return {"workload": "%s of every row, fp16 8192x8192, fp32 arithmetic" % which, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+    name = "x * rsqrt(sum x^2) of every row, compiled at run time" if which == "l2norm_compiled" else "%s of every row" % which
+    return {"workload": "%s, fp16 8192x8192, fp32 arithmetic" % name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, which),
-            "kernel": "softmax_kernel" if which == "softmax" else "norm_kernel"}
+            "kernel": {"softmax": "softmax_kernel", "layernorm": "norm_kernel"}.get(which, "kapy_ew_specialised")}
 
 
 def bench_transpose(kh, steps, warmup):
@@ -268,7 +275,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "transpose", "permute", "gemm_bf16", "gemm_f16", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -291,6 +298,7 @@ def main():
         "reduce": lambda s, w: bench_reduce(kh, s, w),
         "softmax": lambda s, w: bench_rowwise(kh, s, w, "softmax"),
         "layernorm": lambda s, w: bench_rowwise(kh, s, w, "layernorm"),
+        "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, "l2norm_compiled"),
         "permute": lambda s, w: bench_permute(kh, s, w),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32)),

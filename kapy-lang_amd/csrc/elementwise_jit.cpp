@@ -38,6 +38,7 @@ struct JitArgs {
   char *out;
   int64_t out_stride0;
   int32_t rows, vec_per_row;
+  int32_t width;  // elements per row (vec_per_row * 8, or less when the last vector of a row is partial)
 };
 const char *kArgsText = R"(
 struct JitArgs {
@@ -46,7 +47,46 @@ struct JitArgs {
   char *out;
   int64_t out_stride0;
   int32_t rows, vec_per_row;
+  int32_t width;
 };
+// The ragged end of a row: only the first `valid` (1..7) elements of vector jv exist; a whole-vector access would reach
+// past the view (and possibly past its allocation), so they move one by one.
+__device__ __forceinline__ Raw8 fetch8_partial(const StackIn &g, int32_t i, int32_t jv, int valid) {
+  const int eb = g.dtype == KAPY_F32 ? 4 : (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16) ? 2 : 1;
+  const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * eb;
+  Raw8 r;
+  r.lo = r.hi = u32x4{0, 0, 0, 0};
+  if (eb == 2) r.lo = load16_partial(ptr, valid);
+  else if (eb == 4) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (e < valid) {
+        const uint32_t w = ((const uint32_t *)ptr)[e];
+        if (e < 4) r.lo[e & 3] = w;
+        else r.hi[e & 3] = w;
+      }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (e < valid) r.lo[e >> 2] |= (uint32_t)((const uint8_t *)ptr)[e] << (8 * (e & 3));
+  }
+  return r;
+}
+template <bool RAGGED>
+__device__ __forceinline__ Raw8 fetch8_row(const StackIn &g, int32_t i, int32_t jv, int32_t width, bool streaming) {
+  if (RAGGED && (jv + 1) * 8 > width) return fetch8_partial(g, i, jv, width - jv * 8);
+  return fetch8(g, i, jv, streaming);
+}
+template <bool NARROW, bool RAGGED>
+__device__ __forceinline__ void store8_row(char *out, int dtype, int64_t row_start, int32_t jv, int32_t width, const float (&f)[8]) {
+  if (RAGGED && (jv + 1) * 8 > width) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (jv * 8 + e < width) store_from_f32(out, dtype, row_start + jv * 8 + e, f[e]);
+    return;
+  }
+  store8<NARROW>(out, dtype, row_start + (int64_t)jv * 8, f);
+}
 __device__ __forceinline__ void fill8(float (&x)[8], float v) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = v;
@@ -57,13 +97,18 @@ __device__ __forceinline__ void copy8(float (&x)[8], const float (&y)[8]) {
 }
 // Sum or maximum of one row value over its row (the row machine's reduce step): each lane folds its active chunks, a
 // butterfly folds the wave, the waves meet in `red` (one barrier).  A NaN anywhere makes the maximum NaN.
-template <int CH, int THREADS, bool SUM>
-__device__ __forceinline__ float row_reduce(const float (&v)[CH][8], int32_t vec_per_row, float *red) {
+template <int CH, int THREADS, bool SUM, bool RAGGED>
+__device__ __forceinline__ float row_reduce(const float (&v)[CH][8], int32_t vec_per_row, int32_t width, float *red) {
   const int tid = threadIdx.x;
   float acc = SUM ? 0.f : -__builtin_inff();
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
-    if (c * THREADS + tid < vec_per_row) {
+    const int32_t jv = c * THREADS + tid;
+    if (RAGGED && jv < vec_per_row && (jv + 1) * 8 > width) {  // the row's last, partial vector: its first elements only
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (jv * 8 + e < width) acc = SUM ? acc + v[c][e] : max_nan(acc, v[c][e]);
+    } else if (jv < vec_per_row) {
       float part;
       if (SUM) part = ((v[c][0] + v[c][1]) + (v[c][2] + v[c][3])) + ((v[c][4] + v[c][5]) + (v[c][6] + v[c][7]));
       else {
@@ -92,13 +137,13 @@ __device__ __forceinline__ float row_reduce(const float (&v)[CH][8], int32_t vec
   return acc;
 }
 // The lane's CH vectors of one row of an operand (vector c*THREADS + lane; nothing is read past the row's end).
-template <int CH, int THREADS>
-__device__ __forceinline__ void row_fetch8(const StackIn &g, int32_t i, int32_t vec_per_row, bool streaming, Raw8 (&raw)[CH]) {
+template <int CH, int THREADS, bool RAGGED>
+__device__ __forceinline__ void row_fetch8(const StackIn &g, int32_t i, int32_t vec_per_row, int32_t width, bool streaming, Raw8 (&raw)[CH]) {
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     const int32_t jv = c * THREADS + (int32_t)threadIdx.x;
     raw[c].lo = raw[c].hi = u32x4{0, 0, 0, 0};
-    if (jv < vec_per_row) raw[c] = fetch8(g, i, jv, streaming);
+    if (jv < vec_per_row) raw[c] = fetch8_row<RAGGED>(g, i, jv, width, streaming);
   }
 }
 )";
@@ -117,6 +162,7 @@ struct Signature {
   int in_dtype[kJitInputs], in_kind[kJitInputs];
   int out_dtype = 0;
   bool narrow = true;
+  bool ragged = false;       // the width is not a multiple of 8: the last vector of every row moves element by element
   bool rowwise = false;      // the program reduces along rows: the row skeleton, compiled for one (threads, chunks) shape
   int threads = 256, chunks = 1;
 };
@@ -140,11 +186,12 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
   if (stores != 1) return false;
   const int64_t o0 = extent0(out), o1 = extent1(out);
   const int ob = dtype_bytes(out->dtype);
-  if (!is_float(out->dtype) || out->stride1 != 1 || o1 % 8 != 0) return false;
+  if (!is_float(out->dtype) || out->stride1 != 1) return false;
   if (((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
-  if (o0 * (o1 / 8) >= (int64_t(1) << 31) - 1024) return false;
+  if (o0 * ((o1 + 7) / 8) >= (int64_t(1) << 31) - 1024) return false;
+  sig->ragged = o1 % 8 != 0;
   if (sig->rowwise) {
-    const int64_t vpr = o1 / 8;
+    const int64_t vpr = (o1 + 7) / 8;
     if (vpr > 4096) return false;  // a row of more than 32768 elements does not stay in one workgroup's registers
     sig->threads = vpr <= 256 ? 64 : vpr <= 1024 ? 256 : 1024;
     sig->chunks = (int)((vpr + sig->threads - 1) / sig->threads);
@@ -193,6 +240,7 @@ std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig)
     key.push_back((char)sig.in_kind[k]);
   }
   key.push_back((char)sig.out_dtype);
+  key.push_back((char)sig.ragged);
   if (sig.rowwise) {
     key.push_back((char)(sig.threads / 64));
     key.push_back((char)sig.chunks);
@@ -291,7 +339,7 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
   std::vector<Node> nodes = build_nodes(prog, n_inst, result_dtype, &stored, &input_used);
   std::string s = source_head();
   s += "extern \"C\" __global__ __launch_bounds__(256) void kapy_ew_specialised(JitArgs p) {\n";
-  appendf(s, "  constexpr bool NARROW = %s;\n", sig.narrow ? "true" : "false");
+  appendf(s, "  constexpr bool NARROW = %s, RAGGED = %s;\n", sig.narrow ? "true" : "false", sig.ragged ? "true" : "false");
   s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
        "  const uint32_t first = blockIdx.x * 512u + threadIdx.x;\n"
        "  int32_t row[2], jv[2];\n";
@@ -311,7 +359,7 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     if (!input_used[k]) continue;
     const int kind = sig.in_kind[k], dt = sig.in_dtype[k];
     if (kind == kFull || kind == kRow)
-      appendf(s, "      { const StackIn g{p.in[%d], p.stride0[%d], %d, %d}; raw%d[u] = fetch8(g, row[u], jv[u], %s); }\n", k, k, dt,
+      appendf(s, "      { const StackIn g{p.in[%d], p.stride0[%d], %d, %d}; raw%d[u] = fetch8_row<RAGGED>(g, row[u], jv[u], p.width, %s); }\n", k, k, dt,
               kind == kFull ? 0 : 1, k, kind == kFull ? "true" : "false");
     else
       appendf(s, "      raw%d[u] = load_as_f32(p.in[%d], %d, %s);\n", k, k, dt, kind == kCol ? ("row[u] * p.stride0[" + std::to_string(k) + "]").c_str() : "0");
@@ -376,7 +424,7 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     }
   }
   const std::string result = as_array(stored);
-  appendf(s, "    store8<NARROW>(p.out, %d, (int64_t)row[u] * p.out_stride0 + (int64_t)jv[u] * 8, %s);\n  }\n}\n", sig.out_dtype, result.c_str());
+  appendf(s, "    store8_row<NARROW, RAGGED>(p.out, %d, (int64_t)row[u] * p.out_stride0, jv[u], p.width, %s);\n  }\n}\n", sig.out_dtype, result.c_str());
   return s;
 }
 
@@ -404,16 +452,16 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
 
   std::string s = source_head();
   appendf(s, "extern \"C\" __global__ __launch_bounds__(%d) void kapy_ew_specialised(JitArgs p) {\n", TH);
-  appendf(s, "  constexpr bool NARROW = %s;\n  constexpr int CH = %d, THREADS = %d;\n", sig.narrow ? "true" : "false", CH, TH);
+  appendf(s, "  constexpr bool NARROW = %s, RAGGED = %s;\n  constexpr int CH = %d, THREADS = %d;\n", sig.narrow ? "true" : "false", sig.ragged ? "true" : "false", CH, TH);
   s += "  __shared__ float red[2][16];\n  extern __shared__ u32x4 parked[];\n  int phase = 0;\n  const int32_t vpr = p.vec_per_row;\n";
   emit_splats(s, nodes);
   for (int k = 0; k < sig.n_ins; ++k) {
     if (!input_used[k]) continue;
     const int kind = sig.in_kind[k], dt = sig.in_dtype[k];
     appendf(s, "  const StackIn g%d{p.in[%d], p.stride0[%d], %d, %d};\n", k, k, k, dt, kind == kRow ? 1 : 0);
-    if (kind == kFull) appendf(s, "  Raw8 raw%d[CH];\n  row_fetch8<CH, THREADS>(g%d, blockIdx.x, vpr, true, raw%d);\n", k, k, k);
+    if (kind == kFull) appendf(s, "  Raw8 raw%d[CH];\n  row_fetch8<CH, THREADS, RAGGED>(g%d, blockIdx.x, vpr, p.width, true, raw%d);\n", k, k, k);
     else if (kind == kRow && park) {
-      appendf(s, "  {\n    Raw8 t[CH];\n    row_fetch8<CH, THREADS>(g%d, 0, vpr, false, t);\n#pragma unroll\n    for (int c = 0; c < CH; ++c) {\n"
+      appendf(s, "  {\n    Raw8 t[CH];\n    row_fetch8<CH, THREADS, RAGGED>(g%d, 0, vpr, p.width, false, t);\n#pragma unroll\n    for (int c = 0; c < CH; ++c) {\n"
                  "      parked[(%d * CH + c) * THREADS + threadIdx.x] = t[c].lo;\n", k, park_slot[k]);
       if (dt == KAPY_F32) appendf(s, "      parked[(%d * CH + c) * THREADS + threadIdx.x] = t[c].hi;\n", park_slot[k] + 1);
       s += "    }\n  }\n";
@@ -429,7 +477,7 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
   }
   for (int k = 0; k < sig.n_ins; ++k)
     if (input_used[k] && sig.in_kind[k] == kFull)
-      appendf(s, "    if (i + (int32_t)gridDim.x < p.rows) row_fetch8<CH, THREADS>(g%d, i + gridDim.x, vpr, true, raw%d);\n", k, k);
+      appendf(s, "    if (i + (int32_t)gridDim.x < p.rows) row_fetch8<CH, THREADS, RAGGED>(g%d, i + gridDim.x, vpr, p.width, true, raw%d);\n", k, k);
 
   auto elem = [&](int id) { return nodes[id].uniform ? nodes[id].name : nodes[id].name + "[c][e]"; };
   int n_filled = 0;
@@ -469,17 +517,17 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
         if (park) {
           appendf(s, "      t.lo = parked[(%d * CH + c) * THREADS + threadIdx.x];\n", park_slot[k]);
           if (sig.in_dtype[k] == KAPY_F32) appendf(s, "      t.hi = parked[(%d * CH + c) * THREADS + threadIdx.x];\n", park_slot[k] + 1);
-        } else appendf(s, "      if (c * THREADS + (int32_t)threadIdx.x < vpr) t = fetch8(g%d, 0, c * THREADS + (int32_t)threadIdx.x, false);\n", k);
+        } else appendf(s, "      if (c * THREADS + (int32_t)threadIdx.x < vpr) t = fetch8_row<RAGGED>(g%d, 0, c * THREADS + (int32_t)threadIdx.x, p.width, false);\n", k);
         appendf(s, "      widen8(t, %d, %s[c]);\n    }\n", sig.in_dtype[k], vn);
       }
       break;
     }
     case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX:
       if (nodes[n.a].uniform) {  // the same value n times
-        if (n.op == KAPY_EW_REDUCE_SUM) appendf(s, "    float %s = __fmul_rn(%s, (float)(vpr * 8));\n", vn, nodes[n.a].name.c_str());
+        if (n.op == KAPY_EW_REDUCE_SUM) appendf(s, "    float %s = __fmul_rn(%s, (float)p.width);\n", vn, nodes[n.a].name.c_str());
         else appendf(s, "    float %s = %s;\n", vn, nodes[n.a].name.c_str());
       } else {
-        appendf(s, "    float %s = row_reduce<CH, THREADS, %s>(%s, vpr, red[phase & 1]);\n    ++phase;\n", vn, n.op == KAPY_EW_REDUCE_SUM ? "true" : "false",
+        appendf(s, "    float %s = row_reduce<CH, THREADS, %s, RAGGED>(%s, vpr, p.width, red[phase & 1]);\n    ++phase;\n", vn, n.op == KAPY_EW_REDUCE_SUM ? "true" : "false",
                 nodes[n.a].name.c_str());
       }
       round_result();
@@ -520,10 +568,10 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
   }
   if (nodes[stored].uniform) {
     const std::string a = filled(stored);
-    appendf(s, "    %s {\n      const int32_t jv = c * THREADS + (int32_t)threadIdx.x;\n      if (jv < vpr) store8<NARROW>(p.out, %d, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, %s);\n    }\n",
+    appendf(s, "    %s {\n      const int32_t jv = c * THREADS + (int32_t)threadIdx.x;\n      if (jv < vpr) store8_row<NARROW, RAGGED>(p.out, %d, (int64_t)i * p.out_stride0, jv, p.width, %s);\n    }\n",
             kChunks, sig.out_dtype, a.c_str());
   } else {
-    appendf(s, "    %s {\n      const int32_t jv = c * THREADS + (int32_t)threadIdx.x;\n      if (jv < vpr) store8<NARROW>(p.out, %d, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, %s[c]);\n    }\n",
+    appendf(s, "    %s {\n      const int32_t jv = c * THREADS + (int32_t)threadIdx.x;\n      if (jv < vpr) store8_row<NARROW, RAGGED>(p.out, %d, (int64_t)i * p.out_stride0, jv, p.width, %s[c]);\n    }\n",
             kChunks, sig.out_dtype, nodes[stored].name.c_str());
   }
   s += "  }\n}\n";
@@ -615,8 +663,8 @@ int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
   Signature sig;
   if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
     return fail(KAPY_ERR_UNSUPPORTED,
-                "elementwise_specialize: needs one store, reduces only along rows of at most 32768 elements, zero padding, rows of a multiple of 8 "
-                "contiguous elements aligned to 8 elements, and operands that are full, row, column or scalar views");
+                "elementwise_specialize: needs one store, reduces only along rows of at most 32768 elements, zero padding, contiguous rows that start "
+                "aligned to 8 elements, and operands that are full, row, column or scalar views");
   int device = 0;
   KAPY_HIP_CHECK(hipGetDevice(&device));
   const std::string key = make_key(prog, n_inst, sig);
@@ -664,7 +712,8 @@ int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_d
   args.out = (char *)view_base(out);
   args.out_stride0 = out->stride0;
   args.rows = (int32_t)extent0(out);
-  args.vec_per_row = (int32_t)(extent1(out) / 8);
+  args.vec_per_row = (int32_t)((extent1(out) + 7) / 8);
+  args.width = (int32_t)extent1(out);
   size_t size = sizeof args;
   void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
   if (sig.rowwise) {

@@ -134,8 +134,7 @@ def test_unary_ops_with_special_values(ko, op):
 
 
 def test_a_kernel_serves_only_the_operand_signature_it_was_compiled_for(ko):
-    """Specialised for two full operands; the same program with a row operand, or at a width that is not a multiple
-    of 8, goes to the machines (and stays correct); the ragged width cannot be specialised at all."""
+    """Specialised for two full operands; the same program with a row operand goes to the machines (and stays correct)."""
     m, n = 16, 128
     a = ko.fill_normal(m * n, kh.F16, 51, 0).reshape(m, n)
     b = ko.fill_normal(m * n, kh.F16, 51, 1).reshape(m, n)
@@ -152,10 +151,61 @@ def test_a_kernel_serves_only_the_operand_signature_it_was_compiled_for(ko):
     sync()
     assert kh.elementwise_specialize_stats() == before
     assert np.array_equal(to_host(dout, np.uint16, (m, n)), want)
+    # rows that do not start 8 elements apart cannot be specialised at all
     n2 = 100
     a2, b2 = np.ascontiguousarray(a[:, :n2]), np.ascontiguousarray(b[:, :n2])
     _, second, want = _both(ko, insts, [a2, b2], [kh.F16] * 2, kh.F16, m, n2, expect_compiled=False)
     assert np.array_equal(second, want)
+
+
+def _windows(ko, arrays, dtypes, out_dtype, m, width, pitch, kinds):
+    """Oracle and device descriptors of [m x width] windows into buffers whose rows lie `pitch` elements apart (row operands: one row)."""
+    outb = kh.DTYPE_BYTES[out_dtype]
+    want = np.full(m * pitch, 0x5a, dtype=np.uint8).repeat(outb).view(NP_OF[outb])[:m * pitch].copy()
+    shape = lambda kind: (1, width) if kind == "row" else (m, 1) if kind == "col" else (m, width)
+    pitch_of = lambda kind: 1 if kind == "col" else pitch
+    o_ins = [ko.mk_global(a, shape(k)[0], shape(k)[1], pitch_of(k), 1, dt) for a, dt, k in zip(arrays, dtypes, kinds)]
+    devs = [to_dev(a) for a in arrays]
+    d_ins = [dglobal(t, shape(k)[0], shape(k)[1], pitch_of(k), 1, dt) for t, dt, k in zip(devs, dtypes, kinds)]
+    return want, o_ins, d_ins, devs
+
+
+@pytest.mark.parametrize("width", [9, 100, 1001, 8190])
+@pytest.mark.parametrize("which", ["x*y+x 16-bit", "quantise f32->e4m3", "softmax", "layernorm"])
+def test_ragged_widths_flat_and_rowwise(ko, width, which):
+    """Rows start 8 elements apart but hold a width that is not a multiple of 8: the last vector of every row moves element
+    by element, reduces skip the elements past the width, and nothing outside the window is written."""
+    m, pitch = 11, (width + 7) // 8 * 8 + 8
+    dt = kh.BF16
+    if which == "x*y+x 16-bit":
+        insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=0), dict(op=ST, a=2)]
+        arrays, dtypes, kinds, out_dt = [ko.fill_normal(m * pitch, dt, 3, 0), ko.fill_normal(m * pitch, dt, 3, 1)], [dt, dt], ["full", "full"], dt
+    elif which == "quantise f32->e4m3":
+        insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=0, a=0, b=1), dict(op=CAST, dst=2, a=0, dtype=kh.F8E4M3, rmode=kh.RN), dict(op=ST, a=2)]
+        arrays, dtypes, kinds, out_dt = [ko.fill_normal(m * pitch, kh.F32, 4, 0, 0.0, 50.0), ko.fill_uniform(m, kh.F32, 4, 1, 0.5, 4.0)], [kh.F32, kh.F32], ["full", "col"], kh.F8E4M3
+    elif which == "softmax":
+        insts, arrays, dtypes, kinds, out_dt = kh.softmax_insts(dt), [ko.fill_normal(m * pitch, dt, 5, 0, 0.0, 2.0)], [dt], ["full"], dt
+    else:
+        insts = kh.layernorm_insts(width, dt)
+        arrays = [ko.fill_normal(m * pitch, dt, 6, 0, 0.0, 2.0), ko.fill_normal(pitch, dt, 6, 1, 1.0, 0.5), ko.fill_normal(pitch, dt, 6, 2, 0.0, 0.5)]
+        dtypes, kinds, out_dt = [dt] * 3, ["full", "row", "row"], dt
+    want, o_ins, d_ins, devs = _windows(ko, arrays, dtypes, out_dt, m, width, pitch, kinds)
+    outb = kh.DTYPE_BYTES[out_dt]
+    assert ko.elementwise(ko.program(insts), o_ins, ko.mk_global(want, m, width, pitch, 1, out_dt)) == 0
+    dout = to_dev(np.full(m * pitch, 0x5a, dtype=np.uint8).repeat(outb).view(NP_OF[outb])[:m * pitch].copy())
+    prog = kh.program(insts)
+    kh.elementwise_specialize(prog, d_ins, dglobal(dout, m, width, pitch, 1, out_dt))
+    before = kh.elementwise_specialize_stats()[1]
+    kh.elementwise(prog, d_ins, dglobal(dout, m, width, pitch, 1, out_dt))
+    sync()
+    assert kh.elementwise_specialize_stats()[1] == before + 1
+    got = to_host(dout, NP_OF[outb], (m, pitch))
+    want = want.reshape(m, pitch)
+    assert np.array_equal(got[:, width:], want[:, width:])          # the gap between rows keeps its fill
+    if which in ("softmax", "layernorm"):
+        _check_ulp_away_from_cancellation(np.ascontiguousarray(got[:, :width]), np.ascontiguousarray(want[:, :width]), dt)
+    else:
+        assert np.array_equal(got[:, :width], want[:, :width])
 
 
 def test_strided_views_with_offsets(ko):

@@ -33,11 +33,11 @@ def test_generated_text_follows_the_program():
     kernel = src[src.index('extern "C" __global__'):]
     assert "kapy_ew_specialised(JitArgs p)" in kernel
     assert "constexpr bool NARROW = true" in kernel
-    assert kernel.count("fetch8(") == 1                      # one operand, fetched once per vector
+    assert kernel.count("fetch8_row<RAGGED>(") == 1          # one operand, fetched once per vector
     assert "0x3f800000u" in kernel                           # the splat 1.0 as its bit pattern
     assert "unary8<NARROW>(%d, %d" % (kh.EW_EXP, kh.F32) in kernel and "div8(" in kernel
     assert "round8" not in kernel                            # every op is fp32; the final cast is the store's own rounding
-    assert "store8<NARROW>(p.out, %d" % kh.F16 in kernel
+    assert "store8_row<NARROW, RAGGED>(p.out, %d" % kh.F16 in kernel
     # dead code is not emitted: an unused load and an unused product
     prog = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ST, a=0)]
     src, _ = kh.elementwise_source(kh.program(prog), [_g(8, 64, kh.BF16), _g(8, 64, kh.BF16)], _g(8, 64, kh.BF16))
@@ -65,16 +65,33 @@ def test_generated_text_compiles_for_gfx950():
         assert code_bytes > 1000
 
 
+def test_row_programs_and_ragged_widths_get_the_other_skeletons():
+    softmax_like = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=kh.EW_SUBF, dst=0, a=0, b=1), dict(op=ST, a=0)]
+    src, _ = kh.elementwise_source(kh.program(softmax_like), [_g(8, 8192, kh.F16)], _g(8, 8192, kh.F16))
+    kernel = src[src.index('extern "C" __global__'):]
+    assert "__launch_bounds__(256)" in kernel and "CH = 4, THREADS = 256" in kernel and "RAGGED = false" in kernel
+    assert kernel.count("row_reduce<CH, THREADS, false, RAGGED>") == 1 and "for (int32_t i = blockIdx.x; i < p.rows; i += gridDim.x)" in kernel
+    src, _ = kh.elementwise_source(kh.program(softmax_like), [_g(8, 100, kh.F16, 104)], _g(8, 100, kh.F16, 104))   # 100 columns, rows 104 apart
+    kernel = src[src.index('extern "C" __global__'):]
+    assert "CH = 1, THREADS = 64" in kernel and "RAGGED = true" in kernel
+    if _has_runtime_compiler():
+        for shape in ((8, 8192, None), (8, 100, 104), (3, 32768, None)):
+            _, code_bytes = kh.elementwise_source(kh.program(softmax_like), [_g(shape[0], shape[1], kh.F32, shape[2])], _g(shape[0], shape[1], kh.F32, shape[2]), compile=True)
+            assert code_bytes > 1000
+
+
 def test_refusals():
     add = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=ADD, dst=2, a=0, b=1), dict(op=ST, a=2)]
     def refused(insts, ins, out):
         with pytest.raises(kh.KapyError) as e:
             kh.elementwise_source(kh.program(insts), ins, out)
         return str(e.value)
-    assert "status %d" % kh.ERR_UNSUPPORTED in refused(add, [_g(8, 60, kh.F16), _g(8, 60, kh.F16)], _g(8, 60, kh.F16))        # width % 8
     assert "status %d" % kh.ERR_UNSUPPORTED in refused(add, [_g(8, 64, kh.F16, 68), _g(8, 64, kh.F16)], _g(8, 64, kh.F16))    # pitch % 8
-    softmax_like = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=kh.EW_SUBF, dst=0, a=0, b=1), dict(op=ST, a=0)]
-    assert "status %d" % kh.ERR_UNSUPPORTED in refused(softmax_like, [_g(8, 64, kh.F16)], _g(8, 64, kh.F16))
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(add, [_g(8, 60, kh.F16), _g(8, 60, kh.F16)], _g(8, 60, kh.F16))        # rows start unaligned
+    column_reduce = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=0), dict(op=kh.EW_SUBF, dst=0, a=0, b=1), dict(op=ST, a=0)]
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(column_reduce, [_g(8, 64, kh.F16)], _g(8, 64, kh.F16))
+    long_rows = [dict(op=L, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=1), dict(op=ST, a=1)]
+    assert "status %d" % kh.ERR_UNSUPPORTED in refused(long_rows, [_g(2, 32776, kh.F16)], _g(2, 32776, kh.F16))
     padded = [dict(op=L, dst=0, a=0, c=kh.PAD_QNAN), dict(op=ST, a=0)]
     assert "status %d" % kh.ERR_UNSUPPORTED in refused(padded, [_g(8, 64, kh.F16)], _g(8, 64, kh.F16))
     mistyped = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=ADD, dst=2, a=0, b=1), dict(op=ST, a=2)]

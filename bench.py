@@ -132,7 +132,7 @@ def bench_add(kh, steps, warmup, op="add"):
     name = {"add": "elementwise_add fixture: z = x + y fp16 8192x8192", "expr": "z = x*y + x (two roundings) fp16 8192x8192",
             "expr_compiled": "z = x*y + x (two roundings) fp16 8192x8192, compiled at run time",
             "swiglu": "z = silu(x)*y fp16 8192x8192 in fp32, compiled at run time"}[op]
-    kernel = {"add": "affine_act_kernel", "expr": "stack_kernel_narrow"}.get(op, "kapy_ew_specialised")
+    kernel = {"add": "affine_act_kernel", "expr": "stack_kernel_narrow"}.get(op, "kapy_ew_flat_<hash> (compiled at run time)")
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
             "roofline": _roof_hbm(nbytes, ev, "add" if op == "add" else None), "kernel": kernel}
 
@@ -177,7 +177,7 @@ def bench_rowwise(kh, steps, warmup, which):
     name = "x * rsqrt(sum x^2) of every row, compiled at run time" if which == "l2norm_compiled" else "%s of every row" % which
     return {"workload": "%s, fp16 8192x8192, fp32 arithmetic" % name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, which),
-            "kernel": {"softmax": "softmax_kernel", "layernorm": "norm_kernel"}.get(which, "kapy_ew_specialised")}
+            "kernel": {"softmax": "softmax_kernel", "layernorm": "norm_kernel"}.get(which, "kapy_ew_rows_<hash> (compiled at run time)")}
 
 
 def bench_transpose(kh, steps, warmup):

@@ -161,7 +161,8 @@ int kapy_copy_batched(const kapy_global *src, const kapy_global *dst, const kapy
  * broadcasts along it (kapy.broadcast, Kapy.cpp:686-698).  A program with a REDUCE is a row-wise fusion (softmax,
  * layer norm ...): it runs in one pass over HBM with each row resident on chip, and needs axis 1, rows that are
  * contiguous, a multiple of 8 and at most 32768 elements long, zero padding, and operands that are full, row,
- * column or scalar views (KAPY_ERR_UNSUPPORTED otherwise). */
+ * column or scalar views (KAPY_ERR_UNSUPPORTED otherwise; a width that is not a multiple of 8, with rows that still
+ * start aligned to 8 elements, is served by compiling a kernel on the first call, see kapy_elementwise_specialize). */
 typedef enum kapy_ew_op {
   KAPY_EW_LD_GLOBAL = 0, /* dst <- ins[a]            (c = kapy_padding_option)                  */
   KAPY_EW_SPLAT,         /* dst <- imm as `dtype`    (kapy.splat)                               */
@@ -192,8 +193,10 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
  * same kind (full, row, column, scalar) run it instead of the stepwise machines.  Worth it for programs that
  * none of the hand-written kernels match and that are launched many times: the first compile in a process takes
  * seconds, later ones about a quarter of a second.  The descriptors only say how operands are shaped and typed;
- * their pointers are not read.  Needs one store, no reduce, zero padding, contiguous rows of a multiple of 8
- * elements aligned to 8 elements; KAPY_ERR_UNSUPPORTED otherwise, or when the runtime compiler (libhiprtc) is not
+ * their pointers are not read (only their alignment).  Needs one store, reduces only along rows (axis 1) of at most
+ * 32768 elements, zero padding, contiguous rows that start aligned to 8 elements (any width); a program with
+ * reduces is compiled for the row-length class of `out` (64, 256 or 1024 lanes times 1-4 vectors of 8) and serves
+ * that class only.  KAPY_ERR_UNSUPPORTED otherwise, or when the runtime compiler (libhiprtc) is not
  * installed -- kapy_elementwise keeps working either way.  A program that the hand-written kernels already serve
  * with its activation compiled in (act(x*s + bias) with GELU or no activation, plain binary ops) returns KAPY_OK
  * without compiling anything.  Not to be called while a stream is capturing. */

@@ -11,6 +11,7 @@
 #include <math.h>
 #include <string.h>
 
+#include <string>
 #include <type_traits>
 #include <utility>
 #include <vector>
@@ -714,7 +715,17 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 
   bool has_reduce = false;
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
-  if (has_reduce) return run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
+  if (has_reduce) {
+    rc = run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
+    if (rc != KAPY_ERR_UNSUPPORTED) return rc;
+    // What the row machine refuses (a width that is not a multiple of 8, more than three row values in flight) a compiled
+    // kernel may still serve: compile one now rather than turn the caller away.  Without the runtime compiler, or for a
+    // program that fits neither, the row machine's refusal stands.
+    const std::string refusal = last_error_buffer();
+    if (specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK && launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s) == 1)
+      return KAPY_OK;
+    return fail(rc, "%s", refusal.c_str());
+  }
 
   AffineActParams ap;
   int T = -1;

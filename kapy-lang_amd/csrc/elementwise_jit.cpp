@@ -333,12 +333,12 @@ void emit_splats(std::string &s, std::vector<Node> &nodes) {
 // A program without a reduce as straight-line code: every value that the store depends on becomes one array of 8 fp32
 // (the exact image of the typed value, rounded to the op's result type after every op, as the machines do), a splat one
 // constant.
-std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig) {
+std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, const std::string &name) {
   int stored = -1;
   std::vector<char> input_used;
   std::vector<Node> nodes = build_nodes(prog, n_inst, result_dtype, &stored, &input_used);
   std::string s = source_head();
-  s += "extern \"C\" __global__ __launch_bounds__(256) void kapy_ew_specialised(JitArgs p) {\n";
+  appendf(s, "extern \"C\" __global__ __launch_bounds__(256) void %s(JitArgs p) {\n", name.c_str());
   appendf(s, "  constexpr bool NARROW = %s, RAGGED = %s;\n", sig.narrow ? "true" : "false", sig.ragged ? "true" : "false");
   s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
        "  const uint32_t first = blockIdx.x * 512u + threadIdx.x;\n"
@@ -433,7 +433,7 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
 // memory, in each lane's own corner of the dynamic LDS (*lds_bytes; read at their use from L2 instead when that corner
 // would exceed 48 KiB).  Two exchange areas serve the reduces in turn, counted across rows: a wave can write one again
 // only after the barrier of the other, which every wave reaches after it has read the first.
-std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, int *lds_bytes) {
+std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, const std::string &name, int *lds_bytes) {
   int stored = -1;
   std::vector<char> input_used;
   std::vector<Node> nodes = build_nodes(prog, n_inst, result_dtype, &stored, &input_used);
@@ -451,7 +451,7 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
   *lds_bytes = park ? n_park * CH * TH * 16 : 0;
 
   std::string s = source_head();
-  appendf(s, "extern \"C\" __global__ __launch_bounds__(%d) void kapy_ew_specialised(JitArgs p) {\n", TH);
+  appendf(s, "extern \"C\" __global__ __launch_bounds__(%d) void %s(JitArgs p) {\n", TH, name.c_str());
   appendf(s, "  constexpr bool NARROW = %s, RAGGED = %s;\n  constexpr int CH = %d, THREADS = %d;\n", sig.narrow ? "true" : "false", sig.ragged ? "true" : "false", CH, TH);
   s += "  __shared__ float red[2][16];\n  extern __shared__ u32x4 parked[];\n  int phase = 0;\n  const int32_t vpr = p.vec_per_row;\n";
   emit_splats(s, nodes);
@@ -578,9 +578,18 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
   return s;
 }
 
-std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, int *lds_bytes) {
+// The kernel's name carries its skeleton and a hash of the table key, so that a profile tells the compiled programs apart.
+std::string kernel_name(const Signature &sig, const std::string &key) {
+  uint32_t h = 2166136261u;
+  for (unsigned char ch : key) h = (h ^ ch) * 16777619u;
+  char buf[48];
+  snprintf(buf, sizeof buf, "kapy_ew_%s_%08x", sig.rowwise ? "rows" : "flat", h);
+  return buf;
+}
+
+std::string generate(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const Signature &sig, const std::string &name, int *lds_bytes) {
   *lds_bytes = 0;
-  return sig.rowwise ? generate_rows(prog, n_inst, result_dtype, sig, lds_bytes) : generate_flat(prog, n_inst, result_dtype, sig);
+  return sig.rowwise ? generate_rows(prog, n_inst, result_dtype, sig, name, lds_bytes) : generate_flat(prog, n_inst, result_dtype, sig, name);
 }
 
 // ---- the runtime compiler, opened on first use --------------------------------------------------------------------
@@ -674,10 +683,11 @@ int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
   }
   std::vector<char> code;
   Loaded k;
-  int rc = compile_source(generate(prog, n_inst, result_dtype, sig, &k.lds_bytes), &code);
+  const std::string name = kernel_name(sig, key);
+  int rc = compile_source(generate(prog, n_inst, result_dtype, sig, name, &k.lds_bytes), &code);
   if (rc) return rc;
   KAPY_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
-  KAPY_HIP_CHECK(hipModuleGetFunction(&k.fn, k.module, "kapy_ew_specialised"));
+  KAPY_HIP_CHECK(hipModuleGetFunction(&k.fn, k.module, name.c_str()));
   if (sig.rowwise) {
     int per_cu = 1;
     KAPY_HIP_CHECK(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k.fn, sig.threads, (size_t)k.lds_bytes));
@@ -738,7 +748,7 @@ int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_d
   if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
     return fail(KAPY_ERR_UNSUPPORTED, "elementwise_source: the program or its operands do not fit a specialised kernel");
   int lds_bytes = 0;
-  const std::string text = generate(prog, n_inst, result_dtype, sig, &lds_bytes);
+  const std::string text = generate(prog, n_inst, result_dtype, sig, kernel_name(sig, make_key(prog, n_inst, sig)), &lds_bytes);
   if (source && capacity > 0) {
     const size_t n = std::min<size_t>(text.size(), (size_t)capacity - 1);
     memcpy(source, text.data(), n);

@@ -355,3 +355,21 @@ def test_a_row_kernel_serves_only_its_own_width_class(ko):
     sync()
     assert kh.elementwise_specialize_stats() == before
     _check_ulp(to_host(dout, np.uint16, (m, n)), want, kh.F16)
+
+
+def test_a_row_program_the_row_machine_refuses_is_compiled_on_its_first_call(ko):
+    """Softmax over 100 columns of rows that lie 104 elements apart: the row machine wants a multiple of 8, so
+    kapy_elementwise compiles a kernel for it instead of refusing (one more kernel loaded, the call ran it)."""
+    m, width, pitch, dt = 9, 100, 104, kh.F16
+    insts = kh.softmax_insts(dt)[:-2] + [dict(op=kh.EW_ABSF, dst=1, a=1)] + kh.softmax_insts(dt)[-2:]   # |softmax|: no other test's program
+    x = ko.fill_normal(m * pitch, dt, 77, 0, 0.0, 2.0)
+    want = np.full(m * pitch, 0x5a5a, np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(x, m, width, pitch, 1, dt)], ko.mk_global(want, m, width, pitch, 1, dt)) == 0
+    dx, dout = to_dev(x), to_dev(np.full(m * pitch, 0x5a5a, np.uint16))
+    loaded, launches = kh.elementwise_specialize_stats()
+    kh.elementwise(kh.program(insts), [dglobal(dx, m, width, pitch, 1, dt)], dglobal(dout, m, width, pitch, 1, dt))
+    sync()
+    assert kh.elementwise_specialize_stats() == (loaded + 1, launches + 1)
+    got, want = to_host(dout, np.uint16, (m, pitch)), want.reshape(m, pitch)
+    assert np.array_equal(got[:, width:], want[:, width:])
+    _check_ulp(np.ascontiguousarray(got[:, :width]), np.ascontiguousarray(want[:, :width]), dt)

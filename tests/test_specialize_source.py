@@ -31,7 +31,7 @@ SILU = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op
 def test_generated_text_follows_the_program():
     src, _ = kh.elementwise_source(kh.program(SILU), [_g(16, 256, kh.F16)], _g(16, 256, kh.F16))
     kernel = src[src.index('extern "C" __global__'):]
-    assert "kapy_ew_specialised(JitArgs p)" in kernel
+    assert "void kapy_ew_flat_" in kernel and "(JitArgs p)" in kernel
     assert "constexpr bool NARROW = true" in kernel
     assert kernel.count("fetch8_row<RAGGED>(") == 1          # one operand, fetched once per vector
     assert "0x3f800000u" in kernel                           # the splat 1.0 as its bit pattern

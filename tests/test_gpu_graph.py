@@ -1,0 +1,89 @@
+"""The entry points under HIP graph capture: every kernel family of the hot path is recorded once into a graph and
+replayed with fresh operand contents; each replay must reproduce, bit for bit, what the same calls give eagerly.
+(The library launches on the caller's stream, allocates nothing and clears nothing, so a capture sees only kernels.)"""
+import numpy as np
+import pytest
+import torch
+
+import kapy_hip as kh
+from gpu_util import dglobal, sync
+
+pytestmark = pytest.mark.gpu
+
+
+def _calls(bufs, out):
+    """One pass of the hot path over static buffers: GELU -> transpose -> softmax, a compiled program, two GEMMs, W8A8."""
+    m, n = bufs["m"], bufs["n"]
+    g16 = lambda t, r=m, c=n, dt=kh.F16: dglobal(t, r, c, c, 1, dt)
+    kh.elementwise(kh.gelu_program(kh.F16, 0.5), [g16(bufs["x"]), dglobal(bufs["bias"], 1, n, n, 1, kh.F16)], g16(out["gelu"]))
+    kh.copy(g16(out["gelu"]), dglobal(out["tr"], n, m, m, 1, kh.F16), transpose=True)
+    kh.elementwise(kh.program(kh.softmax_insts(kh.F16)), [dglobal(out["tr"], n, m, m, 1, kh.F16)], dglobal(out["soft"], n, m, m, 1, kh.F16))
+    kh.elementwise(bufs["expr"], [g16(bufs["x"]), g16(bufs["y"])], g16(out["expr"]))
+    M, N, K = bufs["gemm"]
+    kh.matmul(dglobal(bufs["a"], M, K, K, 1, kh.BF16), dglobal(bufs["bt"], K, N, 1, K, kh.BF16), dglobal(out["tn"], M, N, N, 1, kh.BF16))
+    kh.matmul(dglobal(bufs["a"], M, K, K, 1, kh.BF16), dglobal(bufs["bt"], K, N, N, 1, kh.BF16), dglobal(out["nn"], M, N, N, 1, kh.BF16))
+    for key, rows in (("f8_16", 16), ("f8_256", 256)):
+        kh.matmul_scaled_f8(dglobal(bufs["a8"], rows, K, K, 1, kh.F8E4M3), dglobal(bufs["w8"], K, N, 1, K, kh.F8E4M3),
+                            bufs["rs"].data_ptr(), bufs["cs"].data_ptr(), dglobal(out[key], rows, N, N, 1, kh.BF16))
+
+
+def _outputs(bufs):
+    m, n = bufs["m"], bufs["n"]
+    M, N, K = bufs["gemm"]
+    z16 = lambda count: torch.zeros(count, dtype=torch.int16, device="cuda")
+    return {"gelu": z16(m * n), "tr": z16(m * n), "soft": z16(m * n), "expr": z16(m * n), "tn": z16(M * N), "nn": z16(M * N),
+            "f8_16": z16(16 * N), "f8_256": z16(256 * N)}
+
+
+def _refill(bufs, seed):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    m, n = bufs["m"], bufs["n"]
+    M, N, K = bufs["gemm"]
+    bufs["x"].copy_(torch.randn(m * n, generator=gen, device="cuda").half().view(torch.int16))
+    bufs["y"].copy_(torch.randn(m * n, generator=gen, device="cuda").half().view(torch.int16))
+    bufs["bias"].copy_(torch.randn(n, generator=gen, device="cuda").half().view(torch.int16))
+    bufs["a"].copy_((0.05 * torch.randn(M * K, generator=gen, device="cuda")).bfloat16().view(torch.int16))
+    bufs["bt"].copy_((0.05 * torch.randn(N * K, generator=gen, device="cuda")).bfloat16().view(torch.int16))
+    bufs["a8"].copy_(torch.randn(256 * K, generator=gen, device="cuda").to(torch.float8_e4m3fn).view(torch.uint8))
+    bufs["w8"].copy_(torch.randn(N * K, generator=gen, device="cuda").to(torch.float8_e4m3fn).view(torch.uint8))
+    bufs["rs"].copy_(torch.rand(256, generator=gen, device="cuda") + 0.5)
+    bufs["cs"].copy_(torch.rand(N, generator=gen, device="cuda") + 0.5)
+
+
+def test_every_kernel_family_replays_from_a_graph():
+    if not hasattr(kh, "matmul_scaled_f8"):
+        pytest.skip("no W8A8 binding")
+    m, n = 96, 512
+    M, N, K = 256, 512, 1024
+    i16 = lambda count: torch.zeros(count, dtype=torch.int16, device="cuda")
+    bufs = {"m": m, "n": n, "gemm": (M, N, K), "x": i16(m * n), "y": i16(m * n), "bias": i16(n), "a": i16(M * K), "bt": i16(N * K),
+            "a8": torch.zeros(256 * K, dtype=torch.uint8, device="cuda"), "w8": torch.zeros(N * K, dtype=torch.uint8, device="cuda"),
+            "rs": torch.zeros(256, dtype=torch.float32, device="cuda"), "cs": torch.zeros(N, dtype=torch.float32, device="cuda")}
+    L, ADD, MUL, ST = kh.EW_LD_GLOBAL, kh.EW_ADDF, kh.EW_MULF, kh.EW_ST_GLOBAL
+    bufs["expr"] = kh.program([dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=1),
+                               dict(op=ADD, dst=2, a=2, b=0), dict(op=ST, a=2)])
+    g16 = lambda t: dglobal(t, m, n, n, 1, kh.F16)
+    kh.elementwise_specialize(bufs["expr"], [g16(bufs["x"]), g16(bufs["y"])], g16(bufs["x"]))   # compiling loads a module: before the capture
+    captured, eager = _outputs(bufs), _outputs(bufs)
+    _refill(bufs, 1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):           # one eager pass first: lazy module loading and attribute calls happen outside the capture
+        _calls(bufs, eager)
+    torch.cuda.current_stream().wait_stream(side)
+    sync()
+    launches_before = kh.elementwise_specialize_stats()[1]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _calls(bufs, captured)
+    assert kh.elementwise_specialize_stats()[1] == launches_before + 1   # the compiled kernel is part of the graph
+    for seed in (2, 3, 4):
+        _refill(bufs, seed)
+        for t in captured.values():
+            t.fill_(0x1111)                 # eager work between the replays
+        graph.replay()
+        _calls(bufs, eager)
+        sync()
+        for name in captured:
+            assert torch.equal(captured[name], eager[name]), "replay with seed %d differs from the eager call in %s" % (seed, name)
+        assert int((captured["soft"] != 0x1111).sum()) > 0

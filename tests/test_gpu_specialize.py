@@ -373,3 +373,26 @@ def test_a_row_program_the_row_machine_refuses_is_compiled_on_its_first_call(ko)
     got, want = to_host(dout, np.uint16, (m, pitch)), want.reshape(m, pitch)
     assert np.array_equal(got[:, width:], want[:, width:])
     _check_ulp(np.ascontiguousarray(got[:, :width]), np.ascontiguousarray(want[:, :width]), dt)
+
+
+def test_threads_specialising_the_same_program_load_one_kernel(ko):
+    import threading
+    m, n = 8, 64
+    insts = [dict(op=L, dst=0, a=0), dict(op=kh.EW_SQRT, dst=1, a=0), dict(op=MUL, dst=1, a=1, b=0), dict(op=kh.EW_ABSF, dst=1, a=1), dict(op=ST, a=1)]
+    x = to_dev(ko.fill_uniform(m * n, kh.F16, 88, 0, 0.5, 4.0))
+    out = dev_zeros(m * n, 2)
+    prog = kh.program(insts)
+    loaded = kh.elementwise_specialize_stats()[0]
+    errors = []
+    def work():
+        try:
+            kh.elementwise_specialize(prog, [dglobal(x, m, n, n, 1, kh.F16)], dglobal(out, m, n, n, 1, kh.F16))
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append(e)
+    threads = [threading.Thread(target=work) for _ in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert kh.elementwise_specialize_stats()[0] == loaded + 1

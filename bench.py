@@ -207,9 +207,10 @@ def bench_permute(kh, steps, warmup):
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
 
 
-def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0):
+def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False):
     """graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
-    (what a launch-bound shape gains when the host's per-launch cost is taken out)."""
+    (what a launch-bound shape gains when the host's per-launch cost is taken out).
+    fused_gelu: d = gelu_tanh(a.b*0.5 + bias) with the tail in the GEMM's epilogue (kapy_matmul_fused); flops counted are the GEMM's."""
     import torch
     tdt = torch.bfloat16 if dtype == kh.BF16 else torch.float16
     std = 0.02 if dtype == kh.BF16 else 0.5
@@ -219,7 +220,11 @@ def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel, til
     ga = kh.mk_global(a.data_ptr(), M, K, K, 1, dtype)
     gb = kh.mk_global(b.data_ptr(), K, N, 1, K, dtype) if b_col_major else kh.mk_global(b.data_ptr(), K, N, N, 1, dtype)
     gd = kh.mk_global(d.data_ptr(), M, N, N, 1, dtype)
-    if graph_of:
+    if fused_gelu:
+        bias = torch.randn(N, device="cuda").to(tdt)
+        gbias = kh.mk_global(bias.data_ptr(), 1, N, N, 1, dtype)
+        wall, ev = _events(lambda i: kh.matmul_fused(ga, gb, gd, bias=gbias, alpha=0.5, act=kh.EW_GELU_TANH, tile=tile), steps, warmup)
+    elif graph_of:
         kh.matmul(ga, gb, gd, tile=tile)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -287,7 +292,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "transpose", "permute", "gemm_bf16", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -313,6 +318,7 @@ def main():
         "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, "l2norm_compiled"),
         "permute": lambda s, w: bench_permute(kh, s, w),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
+        "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32)),
         "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20),
         "f8_m16": lambda s, w: bench_f8(kh, s, w, 16),

@@ -234,6 +234,22 @@ typedef struct kapy_matmul_cfg {
 int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                 const kapy_matmul_cfg *cfg, void *stream);
 
+/* kapy.matmul with the elementwise ops that follow it on the accumulator fused into the same kernel, which is how a
+ * kapy.func that multiplies and then applies bias and activation compiles (one kernel; the accumulator never leaves
+ * registers): result = fptofp_rn( act( addf( mulf(matmul(lhs, rhs), splat alpha), broadcast(extf bias) ) ) ),
+ * every op on fp32 with its own rounding (create_matmul, create_mulf, create_broadcast, create_addf,
+ * create_elementwise_extern_lib, create_fptofp: python/src/ir.cc:744-1174).  16-bit operands (fp8: kapy_matmul_scaled_f8). */
+typedef struct kapy_matmul_epilogue {
+  const kapy_global *bias; /* one contiguous row [1 x N] of f16, bf16 or f32, broadcast along M; NULL = no addf */
+  float alpha;             /* 1.0f = no mulf                                                                  */
+  int32_t act;             /* applied last: -1 (none), KAPY_EW_GELU_TANH, NEGF, ABSF, or KAPY_EW_MAXIMUMF /
+                              KAPY_EW_MINIMUMF against splat(act_operand) (relu = MAXIMUMF with 0); the other
+                              unary ops: KAPY_ERR_UNSUPPORTED (run them as a program on the result)            */
+  float act_operand;
+} kapy_matmul_epilogue;
+int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *result, const kapy_matmul_epilogue *epi,
+                      const kapy_matmul_cfg *cfg, void *stream);
+
 /* W8A8: result[m,n] = cast( (sum_k a8[m,k]·w8[k,n]) · row_scale[m] · col_scale[n] ).
  * In kapy terms: matmul (mma f8, f32 acc) -> mulf with broadcast(row_scale [Mx1]) and
  * broadcast(col_scale [1xN]) -> fptofp rn.  Scales are dense fp32 device arrays. */

@@ -29,6 +29,7 @@
 #include "common.hpp"
 #include "layout.hpp"
 #include "matmul_params.hpp"
+#include "ew_machine.hpp"
 #include "numeric.hpp"
 
 namespace kapy {
@@ -138,9 +139,60 @@ constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 constexpr int vmcnt_lgkm0_imm(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
 
+// The fused elementwise tail: every step rounds to fp32 on its own, as the separate kapy ops would.  Only activations
+// that are a handful of instructions are compiled into the epilogues (every kernel variant carries hundreds of unrolled copies).
+__device__ __forceinline__ bool has_tail(const GemmParams &p) { return p.bias != nullptr || p.act >= 0 || p.alpha != 1.0f; }
+__device__ __forceinline__ float apply_tail(const GemmParams &p, float v, float bias) {
+  if (p.alpha != 1.0f) v = __fmul_rn(v, p.alpha);
+  if (p.bias) v = __fadd_rn(v, bias);
+  switch (p.act) {
+  case KAPY_EW_GELU_TANH: return gelu_tanh_f32(v);
+  case KAPY_EW_MAXIMUMF: return max_nan(v, p.act_operand);
+  case KAPY_EW_MINIMUMF: return min_nan(v, p.act_operand);
+  case KAPY_EW_NEGF: return -v;
+  case KAPY_EW_ABSF: return fabsf(v);
+  }
+  return v;
+}
+
+// The same on 8 values, with every uniform decision taken once.
+__device__ __forceinline__ void apply_tail8(const GemmParams &p, float (&v)[8], const float (&bias)[8]) {
+  if (p.alpha != 1.0f) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = __fmul_rn(v[e], p.alpha);
+  }
+  if (p.bias) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = __fadd_rn(v[e], bias[e]);
+  }
+  switch (p.act) {
+  case KAPY_EW_GELU_TANH:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = gelu_tanh_f32(v[e]);
+    break;
+  case KAPY_EW_MAXIMUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = max_nan(v[e], p.act_operand);
+    break;
+  case KAPY_EW_MINIMUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = min_nan(v[e], p.act_operand);
+    break;
+  case KAPY_EW_NEGF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = -v[e];
+    break;
+  case KAPY_EW_ABSF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = fabsf(v[e]);
+    break;
+  }
+}
+
 __device__ __forceinline__ void store_result(const GemmParams &p, int32_t m, int32_t n, float v) {
   if (m >= p.M || n >= p.N) return;
   if (p.row_scale) v = __fmul_rn(v, __fmul_rn(p.row_scale[m], p.col_scale[n]));
+  if (has_tail(p)) v = apply_tail(p, v, p.bias ? load_as_f32(p.bias, p.bias_dtype, n) : 0.f);
   if (p.acc_dtype >= 0) v += load_as_f32(p.acc, p.acc_dtype, m * p.acc_sm + n * p.acc_sn);
   int64_t idx = m * p.d_sm + n * p.d_sn;
   switch (p.d_dtype) {
@@ -169,6 +221,7 @@ __device__ __forceinline__ void store_block_packed(const GemmParams &p, int32_t 
     for (int e = 0; e < 4; ++e) {
       float v = acc[4 * q + e];
       if (p.row_scale) v = __fmul_rn(v, __fmul_rn(rs, cs[e]));
+      if (has_tail(p)) v = apply_tail(p, v, p.bias ? load_as_f32(p.bias, p.bias_dtype, n_base + 4 * (lane >> 5) + 8 * q + e) : 0.f);
       h[e] = f16 ? f32_to_f16_rn(v) : f32_to_bf16_rn(v);
     }
     u32x2 w = {h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16)};
@@ -204,7 +257,8 @@ struct PackedEpilogue {
   static constexpr int kQuads = kAccRegs / 4, kQuadStep = 4 * kGroups;  // register quads of a block: 4 consecutive columns each, kQuadStep apart
   static_assert(WTM % 32 == 0 && 64 % kChunks == 0 && 32 % kRowsPerStore == 0, "strip geometry");
 
-  template <bool F16, bool SCALED, typename Acc>
+  // EPI: 0 = cast only, 1 = row and column scales
+  template <bool F16, int EPI, typename Acc>
   static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
     const int wrow = lane % KM, wcol = 4 * (lane / KM);        // this lane's row / first column in an accumulator block
     const int rrow = lane / kChunks, rchunk = lane % kChunks;  // and in a read-back instruction
@@ -215,7 +269,7 @@ struct PackedEpilogue {
 #pragma unroll
       for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
         float rs = 1.0f;
-        if constexpr (SCALED) rs = p.row_scale[min(m_wave + i * 32 + bi * KM + wrow, p.M - 1)];  // (rows past M exist only in tiles that hang over the edge; they are not stored)
+        if constexpr (EPI == 1) rs = p.row_scale[min(m_wave + i * 32 + bi * KM + wrow, p.M - 1)];  // (rows past M exist only in tiles that hang over the edge; they are not stored)
 #pragma unroll
         for (int j = 0; j < kTn; ++j)
 #pragma unroll
@@ -223,7 +277,7 @@ struct PackedEpilogue {
             float v[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
-            if constexpr (SCALED) {
+            if constexpr (EPI == 1) {
               const f32x4 cs = *(const f32x4 *)(p.col_scale + min(n_wave + j * KM + wcol + kQuadStep * q, p.N - 4));
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
@@ -246,16 +300,70 @@ struct PackedEpilogue {
       }
     }
   }
-  // result type and scaling are uniform: one specialised copy of the loop each, chosen once
-  template <typename Acc>
+  // The fused elementwise tail.  Its code must not sit in the unrolled accumulator loop (hundreds of copies: the compiler then
+  // gives up keeping the accumulators in registers, for the whole kernel), so the strip goes through LDS as fp32 - one strip
+  // of 32 x (WTN*4 + 16) bytes fits the two 16-bit strips' space - and a rolled loop applies the tail to 8 consecutive
+  // columns per lane on the way out, narrows and stores 16 bytes.
+  template <bool F16, typename Acc>
+  static __device__ __forceinline__ void strips_tail(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip, int32_t m_wave, int32_t n_wave, int lane) {
+    constexpr int kRowStrideF = WTN * 4 + 16, kChunksF = WTN / 8, kRowsPerPass = 64 / kChunksF, kPasses = 32 / kRowsPerPass;
+    static_assert(32 * kRowStrideF <= kBytesPerWave && 64 % kChunksF == 0 && 32 % kRowsPerPass == 0, "fp32 strip geometry");
+    const int wrow = lane % KM, wcol = 4 * (lane / KM);
+    const int rrow = lane / kChunksF, rchunk = lane % kChunksF;
+    // the lane's 8 columns are the same in every pass and strip: their bias values are fetched once
+    const int32_t nn = n_wave + rchunk * 8;
+    float bias[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (p.bias && nn < p.N) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bias[e] = load_as_f32(p.bias, p.bias_dtype, nn + e);
+    }
+#pragma unroll
+    for (int i = 0; i < kStrips; ++i) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int bi = 0; bi < kBlocksPerStrip; ++bi)
+#pragma unroll
+        for (int j = 0; j < kTn; ++j)
+#pragma unroll
+          for (int q = 0; q < kQuads; ++q) {
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
+            *(f32x4 *)(strip + (bi * KM + wrow) * kRowStrideF + (j * KM + wcol + kQuadStep * q) * 4) = v;
+          }
+      __builtin_amdgcn_sched_barrier(0);  // LDS executes a wave's instructions in order: the reads below see the writes above
+#pragma unroll 1
+      for (int t = 0; t < kPasses; ++t) {
+        const int row = t * kRowsPerPass + rrow;
+        const int32_t mm = m_wave + i * 32 + row;
+        const f32x4 lo = *(const f32x4 *)(strip + row * kRowStrideF + rchunk * 32), hi = *(const f32x4 *)(strip + row * kRowStrideF + rchunk * 32 + 16);
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+        apply_tail8(p, v, bias);
+        u32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = F16 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
+        // (N a multiple of 8: a piece of 8 columns is in or out whole)
+        if (mm < p.M && nn < p.N) *(u32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 2) = w;
+      }
+    }
+  }
+  // result type and scaling are uniform: one specialised copy of the loop each, chosen once.  TAIL: the kernel was built for
+  // calls with a fused elementwise tail (a build of its own: in one kernel with the plain epilogue the extra live values
+  // push the main loop's accumulators out of registers).
+  template <bool TAIL = false, typename Acc>
   static __device__ __forceinline__ void run(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
     const bool f16 = p.d_dtype == KAPY_F16;
-    if (p.row_scale) {
-      if (f16) strips<true, true>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips<false, true>(p, acc, strip0, m_wave, n_wave, lane);
+    if constexpr (TAIL) {
+      if (f16) strips_tail<true>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips_tail<false>(p, acc, strip0, m_wave, n_wave, lane);
+    } else if (p.row_scale) {
+      if (f16) strips<true, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<false, 1>(p, acc, strip0, m_wave, n_wave, lane);
     } else {
-      if (f16) strips<true, false>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips<false, false>(p, acc, strip0, m_wave, n_wave, lane);
+      if (f16) strips<true, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<false, 0>(p, acc, strip0, m_wave, n_wave, lane);
     }
   }
 };
@@ -299,7 +407,7 @@ struct TnConfig {
   static_assert(kWtm % 32 == 0 && kWtn % 32 == 0 && BK % T::kSliceK == 0 && 32 % T::kM == 0, "wave tile must be a multiple of the MFMA tile");
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false, bool TAIL = false>
 __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
   using L = TileLayout<C::kRowBytes>;
@@ -737,7 +845,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     static_assert(PackedEpilogue<KM, C::kWtm, C::kWtn>::kBytesPerWave * C::kWaves <= C::kLdsBytes, "two strips per wavefront must fit the ring");
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
     __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space
-    PackedEpilogue<KM, C::kWtm, C::kWtn>::run(p, acc, lds + wave * PackedEpilogue<KM, C::kWtm, C::kWtn>::kBytesPerWave, m0 + wm * C::kWtm,
+    PackedEpilogue<KM, C::kWtm, C::kWtn>::template run<TAIL>(p, acc, lds + wave * PackedEpilogue<KM, C::kWtm, C::kWtn>::kBytesPerWave, m0 + wm * C::kWtm,
                                               n0 + wn * C::kWtn, lane);
   } else {
 #pragma unroll
@@ -1078,10 +1186,10 @@ bool packed_epilogue(const GemmParams &p) {
          ((uintptr_t)p.d & 15) == 0 && (p.d_sm * 2) % 16 == 0 && (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false, bool TAIL = false>
 int launch_tn_epi(GemmParams p, hipStream_t s) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
-  auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED, KTAIL>;
+  auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED, KTAIL, TAIL>;
   // The kernel addresses kLdsBytes of dynamic LDS (more than the 64 KiB default limit), also through
   // LDS-direct loads, which fault when they land outside the allocation.  Make sure the limit has
   // really been raised before the first launch: query first (this also forces the code object to be
@@ -1107,17 +1215,29 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
   return KAPY_OK;
 }
 
+bool host_has_tail(const GemmParams &p) { return p.bias != nullptr || p.act >= 0 || p.alpha != 1.0f; }
+
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 int launch_tn(const GemmParams &p, hipStream_t s) {
   // a result that ends inside a 16-byte piece of a row takes the bounds-checked element stores
   const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || (STAGES == kRing25 && p.N % 8 == 0);
+  const bool packed = packed_epilogue(p) && whole_tiles;
+  if (host_has_tail(p)) {
+    // a fused elementwise tail: the ring kernels on the 16x16 instruction have builds with it in the packed epilogue,
+    // every other variant applies it in the element stores
+    if constexpr (STAGES == kRing25 && T::kM == 16) {
+      if (packed) return p.K % BK ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true, true, true>(p, s) : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true, false, true>(p, s);
+    }
+    if constexpr (STAGES == kRing25) {
+      if (p.K % BK) return launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false, true>(p, s);
+    }
+    return launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
+  }
   if constexpr (STAGES == kRing25) {
     if (p.K % BK)  // a partial last K-tile: the build of the kernel that masks the lanes past K
-      return packed_epilogue(p) && whole_tiles ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true, true>(p, s)
-                                               : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false, true>(p, s);
+      return packed ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true, true>(p, s) : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false, true>(p, s);
   }
-  return packed_epilogue(p) && whole_tiles ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s)
-                                           : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
+  return packed ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s) : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
 }
 
 template <typename T, int BK, int STAGES>
@@ -1125,7 +1245,7 @@ int launch_nn(GemmParams p, hipStream_t s) {
   constexpr int kLds = STAGES * BK * 512;
   p.tiles_m = (p.M + kNBM - 1) / kNBM;  // M need not be a multiple of the tile: see the kernel's lhs descriptor
   p.tiles_n = p.N / kNBN;
-  const bool packed = packed_epilogue(p);
+  const bool packed = packed_epilogue(p) && !host_has_tail(p);  // (a fused tail goes through the element stores here)
   const void *kernel = packed ? (const void *)nn_kernel<T, BK, STAGES, true> : (const void *)nn_kernel<T, BK, STAGES, false>;
   static bool configured[2] = {false, false};  // idempotent; a race only repeats the calls
   if (!configured[packed]) {
@@ -1250,21 +1370,14 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s
   return KAPY_ERR_UNSUPPORTED;
 }
 
-namespace {
-}  // namespace
-
 // Implemented in matmul_f8.hip.
 int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale, const float *col_scale, const kapy_global *acc,
               const kapy_global *result, const kapy_matmul_cfg *cfg, hipStream_t s);
 
-}  // namespace kapy
-
-using namespace kapy;
-
-extern "C" {
-
-int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
-                const kapy_matmul_cfg *cfg, void *stream) {
+namespace {
+// kapy.matmul with, optionally, the elementwise ops that follow it on the accumulator fused into the kernel's epilogue.
+int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
+                 const kapy_matmul_cfg *cfg, const kapy_matmul_epilogue *epi, void *stream) {
   kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0};
   if (cfg) c = *cfg;
   int rc = verify_matmul(lhs, rhs, acc, result, c.impl_way);
@@ -1275,7 +1388,10 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   rc = ensure_device();
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  if (is_f8(lhs->dtype)) return matmul_f8(lhs, rhs, nullptr, nullptr, acc, result, &c, s);
+  if (is_f8(lhs->dtype)) {
+    if (epi) return fail(KAPY_ERR_UNSUPPORTED, "matmul_fused: fp8 operands take kapy_matmul_scaled_f8");
+    return matmul_f8(lhs, rhs, nullptr, nullptr, acc, result, &c, s);
+  }
   if (lhs->dtype != KAPY_F16 && lhs->dtype != KAPY_BF16)
     return fail(KAPY_ERR_UNSUPPORTED, "matmul: %s operands have no matrix instruction on gfx950", dtype_name(lhs->dtype));
 
@@ -1288,6 +1404,11 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   p.acc = acc ? view_base(acc) : nullptr;
   p.d = (char *)view_base(result);
   p.row_scale = p.col_scale = nullptr;
+  p.bias = epi && epi->bias ? view_base(epi->bias) : nullptr;
+  p.bias_dtype = epi && epi->bias ? epi->bias->dtype : KAPY_F32;
+  p.alpha = epi ? epi->alpha : 1.0f;
+  p.act = epi ? epi->act : -1;
+  p.act_operand = epi ? epi->act_operand : 0.f;
 #ifdef KAPY_TRACE
   if (trace_env) p.col_scale = (const float *)strtoull(trace_env, nullptr, 0);
 #endif
@@ -1349,6 +1470,39 @@ int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_globa
   return bf16 ? launch_staged<Bf16>(p, a_mode, b_mode, s) : launch_staged<F16>(p, a_mode, b_mode, s);
 }
 
+
+}  // namespace
+}  // namespace kapy
+
+using namespace kapy;
+
+extern "C" {
+
+int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
+                const kapy_matmul_cfg *cfg, void *stream) {
+  return matmul_16bit(lhs, rhs, acc, result, cfg, nullptr, stream);
+}
+
+int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *result, const kapy_matmul_epilogue *epi,
+                      const kapy_matmul_cfg *cfg, void *stream) {
+  if (!epi) return fail(KAPY_ERR_INVALID, "matmul_fused: null epilogue");
+  switch (epi->act) {
+  case -1: case KAPY_EW_GELU_TANH: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF: case KAPY_EW_NEGF: case KAPY_EW_ABSF:
+    break;
+  case KAPY_EW_EXP: case KAPY_EW_EXP2: case KAPY_EW_LOG: case KAPY_EW_LOG2: case KAPY_EW_SQRT: case KAPY_EW_RSQRT: case KAPY_EW_TANH: case KAPY_EW_ERF:
+    return fail(KAPY_ERR_UNSUPPORTED, "matmul_fused: this activation is not compiled into the matmul kernels; run it as an elementwise program on the result");
+  default: return fail(KAPY_ERR_INVALID, "matmul_fused: act must be a unary elementwise op, maximumf / minimumf (against act_operand) or -1, not %d", epi->act);
+  }
+  if (epi->bias) {
+    int rc = check_global(epi->bias, "matmul_fused bias");
+    if (rc) return rc;
+    if (epi->bias->dtype != KAPY_F16 && epi->bias->dtype != KAPY_BF16 && epi->bias->dtype != KAPY_F32)
+      return fail(KAPY_ERR_VERIFY, "matmul_fused: bias must have f16, bf16 or f32 element type");
+    if (!rhs || extent0(epi->bias) != 1 || extent1(epi->bias) != extent1(rhs) || epi->bias->stride1 != 1)
+      return fail(KAPY_ERR_VERIFY, "broadcast: the bias must be one contiguous row [1 x N]");
+  }
+  return matmul_16bit(lhs, rhs, nullptr, result, cfg, epi, stream);
+}
 
 int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out) {
   if (!out) return fail(KAPY_ERR_INVALID, "matmul_lds_layout: null result");

@@ -247,6 +247,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     GemmParams g;
     g.a = (const char *)p.a; g.b = (const char *)p.b; g.acc = nullptr; g.d = p.d;
     g.row_scale = row_scale; g.col_scale = col_scale;
+    g.bias = nullptr; g.alpha = 1.0f; g.bias_dtype = KAPY_F32; g.act = -1; g.act_operand = 0.f;
     g.a_sm = p.a_sm; g.a_sk = 1; g.b_sn = p.b_sn; g.b_sk = 1;
     g.acc_sm = g.acc_sn = 0; g.d_sm = p.d_sm; g.d_sn = p.d_sn;
     g.M = p.M; g.N = p.N; g.K = p.K;

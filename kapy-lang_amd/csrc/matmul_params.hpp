@@ -9,6 +9,13 @@ struct GemmParams {
   const char *a, *b, *acc;
   char *d;
   const float *row_scale, *col_scale;  // optional fp32 scales applied to the accumulator (both or neither)
+  // fused elementwise tail on the fp32 accumulator: d = act(acc * alpha + bias[n]) (mulf by a splat, addf of a
+  // broadcast row, a unary op, then the cast to the result type)
+  const char *bias;    // [N] values of bias_dtype, or null
+  float alpha;         // 1.0f: no mulf
+  int32_t bias_dtype;
+  int32_t act;         // a unary kapy_ew_op, maximumf / minimumf against act_operand, or -1
+  float act_operand;
   int64_t a_sm, a_sk;  // lhs element strides along M and K
   int64_t b_sn, b_sk;  // rhs element strides along N and K
   int64_t acc_sm, acc_sn, d_sm, d_sn;

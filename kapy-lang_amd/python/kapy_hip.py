@@ -32,7 +32,7 @@ EXPORTS = [
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
     "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
-    "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats",
+    "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
 ]
 
 
@@ -87,6 +87,10 @@ class EwInst(C.Structure):
 class MatmulCfg(C.Structure):
     _fields_ = [("impl_way", C.c_int32), ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
                 ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("reserved", C.c_int32)]
+
+
+class MatmulEpilogue(C.Structure):
+    _fields_ = [("bias", C.POINTER(Global)), ("alpha", C.c_float), ("act", C.c_int32), ("act_operand", C.c_float)]
 
 
 class SmemBuffer(C.Structure):
@@ -149,6 +153,7 @@ def lib():
     L.kapy_elementwise_source.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), C.c_char_p, i64, P(i64), P(i64)]
     L.kapy_fptofp.argtypes = [P(Global), P(Global), i32, vp]
     L.kapy_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
+    L.kapy_matmul_fused.argtypes = [P(Global), P(Global), P(Global), P(MatmulEpilogue), P(MatmulCfg), vp]
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
@@ -353,6 +358,14 @@ def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmo
     cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, 0)
     check(lib().kapy_matmul(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
                             C.byref(cfg), stream if stream is not None else current_stream()))
+
+
+def matmul_fused(lhs, rhs, result, bias=None, alpha=1.0, act=-1, act_operand=0.0, tile=(0, 0, 0), stages=0, stream=None):
+    """result = cast(act(lhs @ rhs * alpha + bias)): the elementwise tail runs in the GEMM's epilogue."""
+    epi = MatmulEpilogue(C.pointer(bias) if bias is not None else None, alpha, act, act_operand)
+    cfg = MatmulCfg(MATMUL_AUTO, tile[0], tile[1], tile[2], RN, stages, 0, 0)
+    check(lib().kapy_matmul_fused(C.byref(lhs), C.byref(rhs), C.byref(result), C.byref(epi), C.byref(cfg),
+                                  stream if stream is not None else current_stream()))
 
 
 def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, stream=None):

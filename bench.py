@@ -56,7 +56,8 @@ def _events(fn, steps, warmup):
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the
 # same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
-MEASURED_TRAFFIC = {"gelu": 268414976, "transpose": 268456960, "add": 402639872, "softmax": 268476416, "layernorm": 268788736}
+MEASURED_TRAFFIC = {"gelu": 268414976, "transpose": 268456960, "add": 402639872, "softmax": 268476416, "layernorm": 268788736,
+                    "expr_compiled": 402619392, "swiglu": 402556928, "l2norm_compiled": 268408832}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -134,7 +135,7 @@ def bench_add(kh, steps, warmup, op="add"):
             "swiglu": "z = silu(x)*y fp16 8192x8192 in fp32, compiled at run time"}[op]
     kernel = {"add": "affine_act_kernel", "expr": "stack_kernel_narrow"}.get(op, "kapy_ew_flat_<hash> (compiled at run time)")
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev, "add" if op == "add" else None), "kernel": kernel}
+            "roofline": _roof_hbm(nbytes, ev, op if op != "expr" else None), "kernel": kernel}
 
 
 def bench_reduce(kh, steps, warmup):

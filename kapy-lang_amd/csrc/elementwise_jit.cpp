@@ -87,6 +87,24 @@ __device__ __forceinline__ void store8_row(char *out, int dtype, int64_t row_sta
   }
   store8<NARROW>(out, dtype, row_start + (int64_t)jv * 8, f);
 }
+// Elements (il, 8*jl .. 8*jl+7) of a 64 x 64 tile staged as it lies in a column-major operand's memory (stage[column][row], PITCH
+// bytes per column), as the 8-element memory image a row-major operand would have given.
+template <int EB, int PITCH>
+__device__ __forceinline__ Raw8 gather8(const char *stage, int il, int jl) {
+  Raw8 r;
+  r.lo = r.hi = u32x4{0, 0, 0, 0};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const char *at = stage + (jl * 8 + e) * PITCH + il * EB;
+    if (EB == 2) r.lo[e >> 1] |= (uint32_t)(*(const uint16_t *)at) << (16 * (e & 1));
+    else if (EB == 4) {
+      const uint32_t w = *(const uint32_t *)at;
+      if (e < 4) r.lo[e & 3] = w;
+      else r.hi[e & 3] = w;
+    } else r.lo[e >> 2] |= (uint32_t)(*(const uint8_t *)at) << (8 * (e & 3));
+  }
+  return r;
+}
 __device__ __forceinline__ void fill8(float (&x)[8], float v) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = v;
@@ -155,7 +173,7 @@ const char *kPrelude =
 #include "jit_headers.inc"
     ;
 
-enum Kind { kFull = 0, kRow = 1, kCol = 2, kScalar = 3 };
+enum Kind { kFull = 0, kRow = 1, kCol = 2, kScalar = 3, kColMajor = 4 /* full extent, contiguous along axis 0 */ };
 
 struct Signature {
   int n_ins = 0;
@@ -163,15 +181,39 @@ struct Signature {
   int out_dtype = 0;
   bool narrow = true;
   bool ragged = false;       // the width is not a multiple of 8: the last vector of every row moves element by element
+  bool tiled = false;        // an operand is column-major: 64 x 64 tiles, such operands staged through LDS
   bool rowwise = false;      // the program reduces along rows: the row skeleton, compiled for one (threads, chunks) shape
   int threads = 256, chunks = 1;
 };
 
-// Which programs a specialised kernel serves and how each operand is read: the result and the full / row operands
-// contiguous along rows and readable 8 elements at a time, column and scalar operands broadcast, no padding pattern
-// other than zero, one store, no reduce.
+// An operand as the kernels see it.  When the result is column-major (contiguous along axis 0) the whole problem is
+// looked at transposed: extents and strides of every operand swap, the result becomes row-major and row-major operands
+// column-major - a store with swapped strides is a load with swapped strides of the transposed problem.
+struct View {
+  const char *base;
+  int64_t e0, e1, s0, s1;
+  int dtype;
+};
+void canonical_views(const kapy_global *const *ins, int n_ins, const kapy_global *out, View *vi, View *vo) {
+  const bool swap = out->stride1 != 1 && out->stride0 == 1;
+  auto view = [&](const kapy_global *g) {
+    View v{view_base(g), extent0(g), extent1(g), g->stride0, g->stride1, g->dtype};
+    if (swap) {
+      std::swap(v.e0, v.e1);
+      std::swap(v.s0, v.s1);
+    }
+    return v;
+  };
+  *vo = view(out);
+  for (int k = 0; k < n_ins; ++k) vi[k] = view(ins[k]);
+}
+
+// Which programs a specialised kernel serves and how each operand is read: the result contiguous along rows (after the
+// transposition above) with rows that start aligned to 8 elements; operands full (row- or column-major, 16-byte
+// aligned along their contiguous axis), one row, one column or a scalar; no padding pattern other than zero, one store,
+// reduces only along rows.
 bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
-              Signature *sig) {
+              Signature *sig, View *vi, View *vo) {
   if (n_ins > kJitInputs) return false;
   int stores = 0;
   for (int k = 0; k < n_inst; ++k) {
@@ -184,10 +226,12 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
     stores += op == KAPY_EW_ST_GLOBAL;
   }
   if (stores != 1) return false;
-  const int64_t o0 = extent0(out), o1 = extent1(out);
+  canonical_views(ins, n_ins, out, vi, vo);
+  if (sig->rowwise && out->stride1 != 1) return false;  // (a reduce names its axis: no transposed view of it)
+  const int64_t o0 = vo->e0, o1 = vo->e1;
   const int ob = dtype_bytes(out->dtype);
-  if (!is_float(out->dtype) || out->stride1 != 1) return false;
-  if (((uintptr_t)view_base(out) % (8 * ob)) || (out->stride0 * ob) % (8 * ob)) return false;
+  if (!is_float(out->dtype) || vo->s1 != 1) return false;
+  if (((uintptr_t)vo->base % (8 * ob)) || (vo->s0 * ob) % (8 * ob)) return false;
   if (o0 * ((o1 + 7) / 8) >= (int64_t(1) << 31) - 1024) return false;
   sig->ragged = o1 % 8 != 0;
   if (sig->rowwise) {
@@ -200,21 +244,28 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
   sig->out_dtype = out->dtype;
   sig->narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
   for (int k = 0; k < n_inst; ++k) sig->narrow = sig->narrow && !is_f8(result_dtype[k]);
+  int staged_bytes = 0;
   for (int k = 0; k < n_ins; ++k) {
-    const kapy_global *g = ins[k];
-    if (!is_float(g->dtype)) return false;
-    sig->narrow = sig->narrow && (g->dtype == KAPY_F16 || g->dtype == KAPY_BF16);
-    const int64_t e0 = extent0(g), e1 = extent1(g);
-    const int eb = dtype_bytes(g->dtype);
-    const bool vec_ok = g->stride1 == 1 && ((uintptr_t)view_base(g) % (8 * eb)) == 0 && (g->stride0 * eb) % (8 * eb) == 0;
-    sig->in_dtype[k] = g->dtype;
-    if (e0 == o0 && e1 == o1 && vec_ok) sig->in_kind[k] = kFull;
-    else if (e0 == 1 && e1 == o1 && vec_ok) sig->in_kind[k] = kRow;
-    else if (e1 == 1 && e0 == o0) sig->in_kind[k] = kCol;
-    else if (e0 == 1 && e1 == 1) sig->in_kind[k] = kScalar;
-    else return false;
+    const View &g = vi[k];
+    if (!is_float(g.dtype)) return false;
+    sig->narrow = sig->narrow && (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16);
+    const int eb = dtype_bytes(g.dtype);
+    const bool vec_ok = g.s1 == 1 && ((uintptr_t)g.base % (8 * eb)) == 0 && (g.e0 == 1 || (g.s0 * eb) % (8 * eb) == 0);  // (one row: no pitch to align)
+    // column-major: 16-byte pieces along axis 0, whole ones only
+    const bool col_major_ok = g.s0 == 1 && ((uintptr_t)g.base % 16) == 0 && (g.s1 * eb) % 16 == 0 && (g.e0 * eb) % 16 == 0 && g.s1 >= 0 &&
+                              !sig->rowwise && !sig->ragged;
+    sig->in_dtype[k] = g.dtype;
+    if (g.e0 == o0 && g.e1 == o1 && vec_ok) sig->in_kind[k] = kFull;
+    else if (g.e0 == 1 && g.e1 == o1 && vec_ok) sig->in_kind[k] = kRow;
+    else if (g.e1 == 1 && g.e0 == o0) sig->in_kind[k] = kCol;
+    else if (g.e0 == 1 && g.e1 == 1) sig->in_kind[k] = kScalar;
+    else if (g.e0 == o0 && g.e1 == o1 && col_major_ok) {
+      sig->in_kind[k] = kColMajor;
+      sig->tiled = true;
+      staged_bytes += 64 * (64 * eb + 16);
+    } else return false;
   }
-  return true;
+  return staged_bytes <= 60 * 1024;
 }
 
 std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig) {
@@ -241,6 +292,7 @@ std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig)
   }
   key.push_back((char)sig.out_dtype);
   key.push_back((char)sig.ragged);
+  key.push_back((char)sig.tiled);
   if (sig.rowwise) {
     key.push_back((char)(sig.threads / 64));
     key.push_back((char)sig.chunks);
@@ -340,25 +392,55 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
   std::string s = source_head();
   appendf(s, "extern \"C\" __global__ __launch_bounds__(256) void %s(JitArgs p) {\n", name.c_str());
   appendf(s, "  constexpr bool NARROW = %s, RAGGED = %s;\n", sig.narrow ? "true" : "false", sig.ragged ? "true" : "false");
-  s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
-       "  const uint32_t first = blockIdx.x * 512u + threadIdx.x;\n"
-       "  int32_t row[2], jv[2];\n";
+  if (sig.tiled) {
+    // 64 x 64 tiles, walked diagonally (tile row + tile column mod the number of tile rows) so that the tiles in flight
+    // spread over the memory channels along both axes.  A column-major operand's tile is copied to LDS as it lies in
+    // memory, 16 bytes per lane along its contiguous axis, and read from there along the other.
+    s += "  const uint32_t tiles_j = (uint32_t)(p.vec_per_row + 7) / 8u, tiles_i = (uint32_t)(p.rows + 63) / 64u;\n"
+         "  const uint32_t tile_j = blockIdx.x % tiles_j, tile_i = (blockIdx.x / tiles_j + tile_j) % tiles_i;\n"
+         "  const int32_t i0 = (int32_t)tile_i * 64, j0 = (int32_t)tile_j * 64;\n";
+    for (int k = 0; k < sig.n_ins; ++k) {
+      if (!input_used[k] || sig.in_kind[k] != kColMajor) continue;
+      const int eb = dtype_bytes(sig.in_dtype[k]), pitch = 64 * eb + 16, vec = 16 / eb, per_col = 64 / vec;
+      appendf(s, "  __shared__ __attribute__((aligned(16))) char stage%d[64 * %d];\n", k, pitch);
+      appendf(s, "  for (int v = threadIdx.x; v < 64 * %d; v += 256) {\n    const int jc = v / %d, iv = v %% %d;\n"
+                 "    const int32_t j = j0 + jc, i = i0 + iv * %d;\n    u32x4 w = {0, 0, 0, 0};\n"
+                 "    if (j < p.width && i < p.rows) w = __builtin_nontemporal_load((const u32x4 *)(p.in[%d] + ((int64_t)j * p.stride0[%d] + i) * %d));\n"
+                 "    *(u32x4 *)(stage%d + jc * %d + iv * 16) = w;\n  }\n",
+              per_col, per_col, per_col, vec, k, k, eb, k, pitch);
+    }
+    s += "  __syncthreads();\n";
+  } else {
+    s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
+         "  const uint32_t first = blockIdx.x * 512u + threadIdx.x;\n";
+  }
+  s += "  int32_t row[2], jv[2];\n";
   for (int k = 0; k < sig.n_ins; ++k) {
     if (!input_used[k]) continue;
-    if (sig.in_kind[k] == kFull || sig.in_kind[k] == kRow) appendf(s, "  Raw8 raw%d[2];\n", k);
+    if (sig.in_kind[k] == kFull || sig.in_kind[k] == kRow || sig.in_kind[k] == kColMajor) appendf(s, "  Raw8 raw%d[2];\n", k);
     else appendf(s, "  float raw%d[2];\n", k);
   }
   emit_splats(s, nodes);
-  s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
-       "    const uint32_t slot = first + u * 256u;\n"
-       "    row[u] = -1;\n"
-       "    if (slot < total) {\n"
-       "      row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);\n"
-       "      jv[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row);\n";
+  if (sig.tiled)
+    s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
+         "    const int il = (int)(u * 256 + threadIdx.x) >> 3, jl = (int)threadIdx.x & 7;\n"
+         "    row[u] = -1;\n"
+         "    if (i0 + il < p.rows && (int32_t)tile_j * 8 + jl < p.vec_per_row) {\n"
+         "      row[u] = i0 + il;\n"
+         "      jv[u] = (int32_t)tile_j * 8 + jl;\n";
+  else
+    s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
+         "    const uint32_t slot = first + u * 256u;\n"
+         "    row[u] = -1;\n"
+         "    if (slot < total) {\n"
+         "      row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);\n"
+         "      jv[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row);\n";
   for (int k = 0; k < sig.n_ins; ++k) {
     if (!input_used[k]) continue;
     const int kind = sig.in_kind[k], dt = sig.in_dtype[k];
-    if (kind == kFull || kind == kRow)
+    if (kind == kColMajor)
+      appendf(s, "      raw%d[u] = gather8<%d, %d>(stage%d, il, jl);\n", k, dtype_bytes(dt), 64 * dtype_bytes(dt) + 16, k);
+    else if (kind == kFull || kind == kRow)
       appendf(s, "      { const StackIn g{p.in[%d], p.stride0[%d], %d, %d}; raw%d[u] = fetch8_row<RAGGED>(g, row[u], jv[u], p.width, %s); }\n", k, k, dt,
               kind == kFull ? 0 : 1, k, kind == kFull ? "true" : "false");
     else
@@ -389,7 +471,7 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     switch (n.op) {
     case KAPY_EW_LD_GLOBAL: {
       const int k = n.input, kind = sig.in_kind[k];
-      if (kind == kFull || kind == kRow) appendf(s, "    float %s[8]; widen8(raw%d[u], %d, %s);\n", vn, k, sig.in_dtype[k], vn);
+      if (kind == kFull || kind == kRow || kind == kColMajor) appendf(s, "    float %s[8]; widen8(raw%d[u], %d, %s);\n", vn, k, sig.in_dtype[k], vn);
       else appendf(s, "    float %s[8]; fill8(%s, raw%d[u]);\n", vn, vn, k);
       break;
     }
@@ -670,10 +752,12 @@ std::atomic<int64_t> g_launches{0};
 
 int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out) {
   Signature sig;
-  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
+  View vi[kJitInputs], vo;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig, vi, &vo))
     return fail(KAPY_ERR_UNSUPPORTED,
-                "elementwise_specialize: needs one store, reduces only along rows of at most 32768 elements, zero padding, contiguous rows that start "
-                "aligned to 8 elements, and operands that are full, row, column or scalar views");
+                "elementwise_specialize: needs one store, reduces only along rows of at most 32768 elements, zero padding, a result contiguous along "
+                "one axis with lines that start aligned to 8 elements, and operands that are full (row- or column-major, 16-byte aligned), row, "
+                "column or scalar views");
   int device = 0;
   KAPY_HIP_CHECK(hipGetDevice(&device));
   const std::string key = make_key(prog, n_inst, sig);
@@ -703,7 +787,8 @@ int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_d
                        hipStream_t stream) {
   if (g_count.load(std::memory_order_acquire) == 0) return 0;
   Signature sig;
-  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig)) return 0;
+  View vi[kJitInputs], vo;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig, vi, &vo)) return 0;
   int device = 0;
   KAPY_HIP_CHECK(hipGetDevice(&device));
   Loaded k;
@@ -716,19 +801,22 @@ int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_d
   JitArgs args;
   memset(&args, 0, sizeof args);
   for (int i = 0; i < n_ins; ++i) {
-    args.in[i] = view_base(ins[i]);
-    args.stride0[i] = ins[i]->stride0;
+    args.in[i] = vi[i].base;
+    args.stride0[i] = sig.in_kind[i] == kColMajor ? vi[i].s1 : vi[i].s0;  // the pitch between rows, or between columns
   }
-  args.out = (char *)view_base(out);
-  args.out_stride0 = out->stride0;
-  args.rows = (int32_t)extent0(out);
-  args.vec_per_row = (int32_t)((extent1(out) + 7) / 8);
-  args.width = (int32_t)extent1(out);
+  args.out = (char *)vo.base;
+  args.out_stride0 = vo.s0;
+  args.rows = (int32_t)vo.e0;
+  args.vec_per_row = (int32_t)((vo.e1 + 7) / 8);
+  args.width = (int32_t)vo.e1;
   size_t size = sizeof args;
   void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
   if (sig.rowwise) {
     const unsigned grid = (unsigned)std::min<int64_t>(args.rows, k.resident);
     KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, grid, 1, 1, (unsigned)sig.threads, 1, 1, (unsigned)k.lds_bytes, stream, nullptr, extra));
+  } else if (sig.tiled) {
+    const int64_t tiles = (int64_t)((args.rows + 63) / 64) * ((args.vec_per_row + 7) / 8);
+    KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, (unsigned)tiles, 1, 1, 256, 1, 1, 0, stream, nullptr, extra));
   } else {
     const int64_t slots = (int64_t)args.rows * args.vec_per_row;
     KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, (unsigned)((slots + 511) / 512), 1, 1, 256, 1, 1, 0, stream, nullptr, extra));
@@ -745,7 +833,8 @@ void specialized_stats(int64_t *loaded, int64_t *launches) {
 int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
                        char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes) {
   Signature sig;
-  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig))
+  View vi[kJitInputs], vo;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig, vi, &vo))
     return fail(KAPY_ERR_UNSUPPORTED, "elementwise_source: the program or its operands do not fit a specialised kernel");
   int lds_bytes = 0;
   const std::string text = generate(prog, n_inst, result_dtype, sig, kernel_name(sig, make_key(prog, n_inst, sig)), &lds_bytes);

@@ -396,3 +396,61 @@ def test_threads_specialising_the_same_program_load_one_kernel(ko):
         t.join()
     assert not errors, errors
     assert kh.elementwise_specialize_stats()[0] == loaded + 1
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Column-major operands and results: the tiled skeleton (a load or store with swapped strides fused with the elementwise ops).
+def _strided_case(ko, insts, specs, out_spec, m, n):
+    """specs: per operand (dtype, kind) with kind in full / T (column-major) / row / col; out_spec: (dtype, 'full' | 'T')."""
+    def layout(kind):   # (rows, cols, stride0, stride1, elements)
+        return {"full": (m, n, n, 1, m * n), "T": (m, n, 1, m, m * n), "row": (1, n, n, 1, n), "col": (m, 1, 1, 1, m)}[kind]
+    arrays, o_ins, d_ins, keep = [], [], [], []
+    for k, (dt, kind) in enumerate(specs):
+        r, c, s0, s1, count = layout(kind)
+        a = ko.fill_uniform(count, dt, 101, k, 0.5, 2.0) if dt in (kh.F8E4M3, kh.F8E5M2) else ko.fill_normal(count, dt, 101, k)
+        t = to_dev(a)
+        arrays.append(a)      # the oracle's descriptor points into it
+        keep.append(t)
+        o_ins.append(ko.mk_global(a, r, c, s0, s1, dt))
+        d_ins.append(dglobal(t, r, c, s0, s1, dt))
+    out_dt, out_kind = out_spec
+    r, c, s0, s1, count = layout(out_kind)
+    outb = kh.DTYPE_BYTES[out_dt]
+    want = np.zeros(count, dtype=NP_OF[outb])
+    assert ko.elementwise(ko.program(insts), o_ins, ko.mk_global(want, r, c, s0, s1, out_dt)) == 0
+    prog = kh.program(insts)
+    dout = dev_zeros(count, outb)
+    kh.elementwise_specialize(prog, d_ins, dglobal(dout, r, c, s0, s1, out_dt))
+    before = kh.elementwise_specialize_stats()[1]
+    kh.elementwise(prog, d_ins, dglobal(dout, r, c, s0, s1, out_dt))
+    sync()
+    assert kh.elementwise_specialize_stats()[1] == before + 1
+    return to_host(dout, NP_OF[outb]), want
+
+
+@pytest.mark.parametrize("m,n", [(64, 64), (128, 256), (72, 200), (8, 8), (1000, 520)])
+def test_column_major_operands_are_staged_through_lds(ko, m, n):
+    # z = x^T-view * y + bias_row, all f16, exactly rounded: bit-exact
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=L, dst=2, a=2), dict(op=MUL, dst=3, a=0, b=1), dict(op=ADD, dst=3, a=3, b=2), dict(op=ST, a=3)]
+    got, want = _strided_case(ko, insts, [(kh.F16, "T"), (kh.F16, "full"), (kh.F16, "row")], (kh.F16, "full"), m, n)
+    assert np.array_equal(got, want)
+    # two column-major operands of different element sizes and a column operand, f32 arithmetic, bf16 result
+    insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=L, dst=1, a=1), dict(op=L, dst=2, a=2), dict(op=CAST, dst=2, a=2, dtype=kh.F32),
+             dict(op=FMA, dst=3, a=0, b=1, c=2), dict(op=CAST, dst=4, a=3, dtype=kh.BF16, rmode=kh.RN), dict(op=ST, a=4)]
+    got, want = _strided_case(ko, insts, [(kh.BF16, "T"), (kh.F32, "T"), (kh.BF16, "col")], (kh.BF16, "full"), m, n)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,n", [(64, 128), (200, 80), (512, 1008)])   # (the fp8 operand is read 16 elements at a time along n)
+def test_column_major_result_is_the_transposed_problem(ko, m, n):
+    # the transpose fused with GELU: out (column-major) = gelu(x*0.5 + bias_row) of a row-major x
+    insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=SPL, dst=1, dtype=kh.F32, imm=0.5), dict(op=MUL, dst=0, a=0, b=1),
+             dict(op=L, dst=2, a=1), dict(op=CAST, dst=2, a=2, dtype=kh.F32), dict(op=ADD, dst=0, a=0, b=2), dict(op=kh.EW_GELU_TANH, dst=0, a=0),
+             dict(op=CAST, dst=3, a=0, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=3)]
+    got, want = _strided_case(ko, insts, [(kh.F16, "full"), (kh.F16, "row")], (kh.F16, "T"), m, n)
+    _check_ulp(got.reshape(n, m), want.reshape(n, m), kh.F16)
+    # dequantise-and-transpose: e4m3 row-major in, bf16 column-major out, scaled per original row
+    insts = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=L, dst=1, a=1), dict(op=MUL, dst=0, a=0, b=1),
+             dict(op=CAST, dst=2, a=0, dtype=kh.BF16, rmode=kh.RN), dict(op=ST, a=2)]
+    got, want = _strided_case(ko, insts, [(kh.F8E4M3, "full"), (kh.F32, "col")], (kh.BF16, "T"), m, n)
+    assert np.array_equal(got, want)

@@ -138,6 +138,26 @@ def bench_add(kh, steps, warmup, op="add"):
             "roofline": _roof_hbm(nbytes, ev, op if op != "expr" else None), "kernel": kernel}
 
 
+def bench_gelu_transposed(kh, steps, warmup):
+    """y = gelu_tanh(x^T*0.5 + bias): the C3a transpose fused with the C2 chain - x is read through a view with swapped
+    strides - compiled at run time onto the tiled skeleton (64 x 64 tiles, the column-major operand staged through LDS)."""
+    import torch
+    n, sets = 8192, 4
+    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    ys = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    bias = torch.randn(n, device="cuda", dtype=torch.float16)
+    gx = [kh.mk_global(x.data_ptr(), n, n, 1, n, kh.F16) for x in xs]       # element (i, j) of the view is x[j, i]
+    gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
+    gb = kh.mk_global(bias.data_ptr(), 1, n, n, 1, kh.F16)
+    prog = kh.gelu_program(kh.F16, 0.5)
+    kh.elementwise_specialize(prog, [gx[0], gb], gy[0])
+    wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gb], gy[i % sets]), steps, warmup)
+    nbytes = 2 * n * n * 2 + n * 2
+    return {"workload": "gelu_tanh(x^T*0.5+bias) fp16 8192x8192: transpose fused with the elementwise chain, compiled at run time",
+            "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
+            "roofline": _roof_hbm(nbytes, ev), "kernel": "kapy_ew_flat_<hash> (tiled; compiled at run time)"}
+
+
 def bench_reduce(kh, steps, warmup):
     """kapy.reduce (sum along rows) of the headline shape: the first adjacent op after the hot path proper."""
     import torch
@@ -293,7 +313,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed", "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"])
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -313,6 +333,7 @@ def main():
         "swiglu": lambda s, w: bench_add(kh, s, w, "swiglu"),
         "copy": lambda s, w: bench_copy(kh, s, w),
         "transpose": lambda s, w: bench_transpose(kh, s, w),
+        "gelu_transposed": lambda s, w: bench_gelu_transposed(kh, s, w),
         "reduce": lambda s, w: bench_reduce(kh, s, w),
         "softmax": lambda s, w: bench_rowwise(kh, s, w, "softmax"),
         "layernorm": lambda s, w: bench_rowwise(kh, s, w, "layernorm"),

@@ -194,7 +194,9 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
  * none of the hand-written kernels match and that are launched many times: the first compile in a process takes
  * seconds, later ones about a quarter of a second.  The descriptors only say how operands are shaped and typed;
  * their pointers are not read (only their alignment).  Needs one store, reduces only along rows (axis 1) of at most
- * 32768 elements, zero padding, contiguous rows that start aligned to 8 elements (any width); a program with
+ * 32768 elements, zero padding, a result contiguous along one axis whose lines start aligned to 8 elements (any
+ * width), full operands that are row- or column-major (a view with swapped strides: the transpose is fused; 16-byte
+ * aligned along the contiguous axis), row, column or scalar operands; a program with
  * reduces is compiled for the row-length class of `out` (64, 256 or 1024 lanes times 1-4 vectors of 8) and serves
  * that class only.  KAPY_ERR_UNSUPPORTED otherwise, or when the runtime compiler (libhiprtc) is not
  * installed -- kapy_elementwise keeps working either way.  A program that the hand-written kernels already serve

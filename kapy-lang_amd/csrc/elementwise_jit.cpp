@@ -87,7 +87,7 @@ __device__ __forceinline__ void store8_row(char *out, int dtype, int64_t row_sta
   }
   store8<NARROW>(out, dtype, row_start + (int64_t)jv * 8, f);
 }
-// Elements (il, 8*jl .. 8*jl+7) of a 64 x 64 tile staged as it lies in a column-major operand's memory (stage[column][row], PITCH
+// Elements (il, 8*jl .. 8*jl+7) of a tile (64 columns wide) staged as it lies in a column-major operand's memory (stage[column][row], PITCH
 // bytes per column), as the 8-element memory image a row-major operand would have given.
 template <int EB, int PITCH>
 __device__ __forceinline__ Raw8 gather8(const char *stage, int il, int jl) {
@@ -173,6 +173,10 @@ const char *kPrelude =
 #include "jit_headers.inc"
     ;
 
+#ifndef KAPY_JIT_TILE_ROWS
+#define KAPY_JIT_TILE_ROWS 64
+#endif
+constexpr int kTileRows = KAPY_JIT_TILE_ROWS;  // rows of a tile of the tiled skeleton (64 columns wide): 32 per vector a lane handles
 enum Kind { kFull = 0, kRow = 1, kCol = 2, kScalar = 3, kColMajor = 4 /* full extent, contiguous along axis 0 */ };
 
 struct Signature {
@@ -262,7 +266,7 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
     else if (g.e0 == o0 && g.e1 == o1 && col_major_ok) {
       sig->in_kind[k] = kColMajor;
       sig->tiled = true;
-      staged_bytes += 64 * (64 * eb + 16);
+      staged_bytes += 64 * (kTileRows * eb + 16);
     } else return false;
   }
   return staged_bytes <= 60 * 1024;
@@ -396,12 +400,12 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     // 64 x 64 tiles, walked diagonally (tile row + tile column mod the number of tile rows) so that the tiles in flight
     // spread over the memory channels along both axes.  A column-major operand's tile is copied to LDS as it lies in
     // memory, 16 bytes per lane along its contiguous axis, and read from there along the other.
-    s += "  const uint32_t tiles_j = (uint32_t)(p.vec_per_row + 7) / 8u, tiles_i = (uint32_t)(p.rows + 63) / 64u;\n"
-         "  const uint32_t tile_j = blockIdx.x % tiles_j, tile_i = (blockIdx.x / tiles_j + tile_j) % tiles_i;\n"
-         "  const int32_t i0 = (int32_t)tile_i * 64, j0 = (int32_t)tile_j * 64;\n";
+    appendf(s, "  const uint32_t tiles_j = (uint32_t)(p.vec_per_row + 7) / 8u, tiles_i = (uint32_t)(p.rows + %d) / %du;\n"
+               "  const uint32_t tile_j = blockIdx.x %% tiles_j, tile_i = (blockIdx.x / tiles_j + tile_j) %% tiles_i;\n"
+               "  const int32_t i0 = (int32_t)tile_i * %d, j0 = (int32_t)tile_j * 64;\n", kTileRows - 1, kTileRows, kTileRows);
     for (int k = 0; k < sig.n_ins; ++k) {
       if (!input_used[k] || sig.in_kind[k] != kColMajor) continue;
-      const int eb = dtype_bytes(sig.in_dtype[k]), pitch = 64 * eb + 16, vec = 16 / eb, per_col = 64 / vec;
+      const int eb = dtype_bytes(sig.in_dtype[k]), pitch = kTileRows * eb + 16, vec = 16 / eb, per_col = kTileRows / vec;
       appendf(s, "  __shared__ __attribute__((aligned(16))) char stage%d[64 * %d];\n", k, pitch);
       appendf(s, "  for (int v = threadIdx.x; v < 64 * %d; v += 256) {\n    const int jc = v / %d, iv = v %% %d;\n"
                  "    const int32_t j = j0 + jc, i = i0 + iv * %d;\n    u32x4 w = {0, 0, 0, 0};\n"
@@ -414,22 +418,23 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     s += "  const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;\n"
          "  const uint32_t first = blockIdx.x * 512u + threadIdx.x;\n";
   }
-  s += "  int32_t row[2], jv[2];\n";
+  const int U = sig.tiled ? kTileRows / 32 : 2;  // vectors of 8 per lane
+  appendf(s, "  constexpr int U = %d;\n  int32_t row[U], jv[U];\n", U);
   for (int k = 0; k < sig.n_ins; ++k) {
     if (!input_used[k]) continue;
-    if (sig.in_kind[k] == kFull || sig.in_kind[k] == kRow || sig.in_kind[k] == kColMajor) appendf(s, "  Raw8 raw%d[2];\n", k);
-    else appendf(s, "  float raw%d[2];\n", k);
+    if (sig.in_kind[k] == kFull || sig.in_kind[k] == kRow || sig.in_kind[k] == kColMajor) appendf(s, "  Raw8 raw%d[U];\n", k);
+    else appendf(s, "  float raw%d[U];\n", k);
   }
   emit_splats(s, nodes);
   if (sig.tiled)
-    s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
+    s += "#pragma unroll\n  for (int u = 0; u < U; ++u) {\n"
          "    const int il = (int)(u * 256 + threadIdx.x) >> 3, jl = (int)threadIdx.x & 7;\n"
          "    row[u] = -1;\n"
          "    if (i0 + il < p.rows && (int32_t)tile_j * 8 + jl < p.vec_per_row) {\n"
          "      row[u] = i0 + il;\n"
          "      jv[u] = (int32_t)tile_j * 8 + jl;\n";
   else
-    s += "#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n"
+    s += "#pragma unroll\n  for (int u = 0; u < U; ++u) {\n"
          "    const uint32_t slot = first + u * 256u;\n"
          "    row[u] = -1;\n"
          "    if (slot < total) {\n"
@@ -439,14 +444,14 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     if (!input_used[k]) continue;
     const int kind = sig.in_kind[k], dt = sig.in_dtype[k];
     if (kind == kColMajor)
-      appendf(s, "      raw%d[u] = gather8<%d, %d>(stage%d, il, jl);\n", k, dtype_bytes(dt), 64 * dtype_bytes(dt) + 16, k);
+      appendf(s, "      raw%d[u] = gather8<%d, %d>(stage%d, il, jl);\n", k, dtype_bytes(dt), kTileRows * dtype_bytes(dt) + 16, k);
     else if (kind == kFull || kind == kRow)
       appendf(s, "      { const StackIn g{p.in[%d], p.stride0[%d], %d, %d}; raw%d[u] = fetch8_row<RAGGED>(g, row[u], jv[u], p.width, %s); }\n", k, k, dt,
               kind == kFull ? 0 : 1, k, kind == kFull ? "true" : "false");
     else
       appendf(s, "      raw%d[u] = load_as_f32(p.in[%d], %d, %s);\n", k, k, dt, kind == kCol ? ("row[u] * p.stride0[" + std::to_string(k) + "]").c_str() : "0");
   }
-  s += "    }\n  }\n#pragma unroll\n  for (int u = 0; u < 2; ++u) {\n    if (row[u] < 0) continue;\n";
+  s += "    }\n  }\n#pragma unroll\n  for (int u = 0; u < U; ++u) {\n    if (row[u] < 0) continue;\n";
   auto elem = [&](int id) { return nodes[id].is_const ? nodes[id].name : nodes[id].name + "[e]"; };
   // an operand as an array of 8 (div8 and the store take arrays)
   int n_filled = 0;
@@ -815,7 +820,7 @@ int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_d
     const unsigned grid = (unsigned)std::min<int64_t>(args.rows, k.resident);
     KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, grid, 1, 1, (unsigned)sig.threads, 1, 1, (unsigned)k.lds_bytes, stream, nullptr, extra));
   } else if (sig.tiled) {
-    const int64_t tiles = (int64_t)((args.rows + 63) / 64) * ((args.vec_per_row + 7) / 8);
+    const int64_t tiles = (int64_t)((args.rows + kTileRows - 1) / kTileRows) * ((args.vec_per_row + 7) / 8);
     KAPY_HIP_CHECK(hipModuleLaunchKernel(k.fn, (unsigned)tiles, 1, 1, 256, 1, 1, 0, stream, nullptr, extra));
   } else {
     const int64_t slots = (int64_t)args.rows * args.vec_per_row;

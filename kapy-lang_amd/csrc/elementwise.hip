@@ -9,6 +9,7 @@
 // and runs it in one pass with 16-byte accesses (affine_act_kernel); any other program runs on a
 // small register machine (interpreter_kernel) whose register file lives in LDS.
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <string>
@@ -753,6 +754,18 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 #undef KAPY_LAUNCH_AFFINE
     KAPY_HIP_CHECK(hipGetLastError());
     return KAPY_OK;
+  }
+
+  // KAPY_EW_AUTO_SPECIALIZE=1: a program no hand-written kernel matches is compiled on its first call instead of running on
+  // the stepwise machines (a fraction of a second once per program and operand signature; off by default so that no call
+  // takes that long unasked).  A program that cannot be compiled, or a machine without the runtime compiler, goes on below.
+  static const bool auto_specialize = [] {
+    const char *v = getenv("KAPY_EW_AUTO_SPECIALIZE");
+    return v && v[0] == '1';
+  }();
+  if (auto_specialize && specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK) {
+    rc = launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s);
+    if (rc != 0) return rc < 0 ? rc : KAPY_OK;
   }
 
   {

@@ -454,3 +454,36 @@ def test_column_major_result_is_the_transposed_problem(ko, m, n):
              dict(op=CAST, dst=2, a=0, dtype=kh.BF16, rmode=kh.RN), dict(op=ST, a=2)]
     got, want = _strided_case(ko, insts, [(kh.F8E4M3, "full"), (kh.F32, "col")], (kh.BF16, "T"), m, n)
     assert np.array_equal(got, want)
+
+
+def test_auto_specialize_switch_compiles_on_the_first_call(ko):
+    """KAPY_EW_AUTO_SPECIALIZE=1 (read once per process, so tried in a process of its own): a program outside the hand-written
+    kernels is compiled by its first kapy_elementwise call; the result equals the oracle's."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r'''
+import sys
+sys.path[:0] = [%r, %r, %r]
+import numpy as np, torch, kapy_hip as kh, ko
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+m, n = 16, 256
+a, b = ko.fill_normal(m * n, kh.F16, 5, 0).reshape(m, n), ko.fill_normal(m * n, kh.F16, 5, 1).reshape(m, n)
+L, ADD, MUL, ST = kh.EW_LD_GLOBAL, kh.EW_ADDF, kh.EW_MULF, kh.EW_ST_GLOBAL
+insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=0), dict(op=ST, a=2)]
+want = np.zeros((m, n), np.uint16)
+assert ko.elementwise(ko.program(insts), [ko.mk_global(a, m, n, n, 1, kh.F16), ko.mk_global(b, m, n, n, 1, kh.F16)], ko.mk_global(want, m, n, n, 1, kh.F16)) == 0
+da, db, dz = to_dev(a), to_dev(b), dev_zeros(m * n, 2)
+g = lambda t: dglobal(t, m, n, n, 1, kh.F16)
+for call in range(2):
+    kh.elementwise(kh.program(insts), [g(da), g(db)], g(dz)); sync()
+    assert kh.elementwise_specialize_stats() == (1, call + 1), kh.elementwise_specialize_stats()
+assert np.array_equal(to_host(dz, np.uint16, (m, n)), want)
+kh.elementwise(kh.gelu_program(kh.F16), [g(da), dglobal(db, 1, n, n, 1, kh.F16)], g(dz)); sync()     # a matched program stays on its kernel
+assert kh.elementwise_specialize_stats() == (1, 2)
+print("auto ok")
+''' % (os.path.join(root, "kapy-lang_amd", "python"), os.path.join(root, "oracle"), os.path.join(root, "tests"))
+    env = dict(os.environ, KAPY_EW_AUTO_SPECIALIZE="1")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and "auto ok" in out.stdout, out.stdout + out.stderr

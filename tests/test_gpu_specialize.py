@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import kapy_hip as kh
-from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host, ulp_diff_f16
 from test_gpu_elementwise import _check_ulp
 
 pytestmark = pytest.mark.gpu
@@ -487,3 +487,37 @@ print("auto ok")
     env = dict(os.environ, KAPY_EW_AUTO_SPECIALIZE="1")
     out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert out.returncode == 0 and "auto ok" in out.stdout, out.stdout + out.stderr
+
+
+def test_full_size_transpose_fused_with_gelu(ko):
+    """y = gelu_tanh(x^T*0.5 + bias) on fp16 8192x8192 through the tiled skeleton: the whole result against the two
+    hand-written kernels run one after the other (transpose, then the fused GELU; <= 2 ulp: one contracts x*s + b into an
+    fma, the other rounds twice), and 32 rows spread over it against the oracle."""
+    n = 8192
+    x = ko.fill_normal(n * n, kh.F16, 0, 0).reshape(n, n)
+    bias = ko.fill_normal(n, kh.F16, 0, 1)
+    dx, db, dy, dt_, d2 = to_dev(x), to_dev(bias), dev_zeros(n * n, 2), dev_zeros(n * n, 2), dev_zeros(n * n, 2)
+    prog = kh.gelu_program(kh.F16, 0.5)
+    gT, g, gb = dglobal(dx, n, n, 1, n, kh.F16), (lambda t: dglobal(t, n, n, n, 1, kh.F16)), dglobal(db, 1, n, n, 1, kh.F16)
+    kh.elementwise_specialize(prog, [gT, gb], g(dy))
+    before = kh.elementwise_specialize_stats()[1]
+    kh.elementwise(prog, [gT, gb], g(dy))
+    kh.copy(g(dx), g(dt_), transpose=True)
+    kh.elementwise(prog, [g(dt_), gb], g(d2))
+    sync()
+    assert kh.elementwise_specialize_stats()[1] == before + 1      # only the call with the swapped strides ran compiled code
+    got, two_step = to_host(dy, np.uint16, (n, n)), to_host(d2, np.uint16, (n, n))
+    assert ulp_diff_f16(got, two_step).max() <= 2
+    rows = np.linspace(0, n - 1, 32).astype(int)
+    xs = np.ascontiguousarray(x[:, rows].T)                        # rows of the transposed view
+    want = np.zeros((len(rows), n), np.uint16)
+    assert ko.elementwise(ko.program(_gelu_insts()), [ko.mk_global(xs, len(rows), n, n, 1, kh.F16), ko.mk_global(bias, 1, n, n, 1, kh.F16)],
+                          ko.mk_global(want, len(rows), n, n, 1, kh.F16)) == 0
+    _check_ulp(got[rows], want, kh.F16)
+
+
+def _gelu_insts():
+    """The chain of kh.gelu_program(F16, 0.5) spelled out (the oracle takes the same instruction list)."""
+    return [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=SPL, dst=2, dtype=kh.F32, imm=0.5), dict(op=MUL, dst=1, a=1, b=2),
+            dict(op=L, dst=4, a=1), dict(op=CAST, dst=4, a=4, dtype=kh.F32), dict(op=ADD, dst=1, a=1, b=4), dict(op=kh.EW_GELU_TANH, dst=1, a=1),
+            dict(op=CAST, dst=5, a=1, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=5)]

@@ -1,5 +1,5 @@
 """GPU parity for the layout moves (ld_global -> [transpose] -> st_global): bit-exact against the
-oracle on small / ragged / strided cases and against closed forms at the BASELINE sizes."""
+oracle on small / ragged / strided cases and against closed forms at the benchmark sizes."""
 import ctypes as C
 
 import numpy as np
@@ -122,7 +122,7 @@ def test_bhsd_permute_small_matches_oracle(ko):
 
 
 def test_config3a_transpose_8192_bit_exact(ko):
-    """BASELINE config 3a: fp16 8192x8192 (i,j)->(j,i), random 16-bit patterns from seed 0."""
+    """benchmark configuration 3a: fp16 8192x8192 (i,j)->(j,i), random 16-bit patterns from seed 0."""
     n = 8192
     src = ko.fill_bits16(n * n, 0).reshape(n, n)
     d_src, d_dst = to_dev(src), dev_zeros(n * n, 2)
@@ -149,7 +149,7 @@ def test_config3a_transpose_8192_bit_exact(ko):
 
 
 def test_config3b_permute_bhsd_bit_exact(ko):
-    """BASELINE config 3b: bf16 [8,32,2048,128] (b,h,s,d)->(b,s,h,d), random bits from seed 1."""
+    """benchmark configuration 3b: bf16 [8,32,2048,128] (b,h,s,d)->(b,s,h,d), random bits from seed 1."""
     b, h, s, d = 8, 32, 2048, 128
     src = ko.fill_bits16(b * h * s * d, 1).reshape(b, h, s, d)
     d_src, d_dst = to_dev(src), dev_zeros(b * h * s * d, 2)

@@ -1,5 +1,5 @@
 """GPU parity for fused elementwise programs: max |err| <= 2 ulp of the 16-bit result type against
-the oracle (tolerance stated by BASELINE north_star), bit-exact where the op is exactly rounded."""
+the oracle (the tolerance the benchmark definition states), bit-exact where the op is exactly rounded."""
 import ctypes as C
 
 import numpy as np
@@ -55,7 +55,7 @@ def test_gelu_unaligned_shape_takes_the_interpreter(ko):
 
 
 def test_config2_gelu_8192_sampled_against_oracle(ko):
-    """BASELINE config 2: y = GELU_tanh(x*0.5 + bias), x fp16 8192x8192 normal(0,1) seed 0, bias seed 1.
+    """benchmark configuration 2: y = GELU_tanh(x*0.5 + bias), x fp16 8192x8192 normal(0,1) seed 0, bias seed 1.
     The whole result is produced on the GPU; the oracle checks 64 full rows spread over the matrix, and
     a row-broadcast invariant (rows with equal x rows give equal y rows) covers the rest."""
     n = 8192

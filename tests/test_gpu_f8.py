@@ -1,4 +1,4 @@
-"""GPU parity for fp8 (OCP E4M3FN / E5M2) matmuls with fp32 row/column scales (BASELINE config 5)."""
+"""GPU parity for fp8 (OCP E4M3FN / E5M2) matmuls with fp32 row/column scales (benchmark configuration 5)."""
 import ctypes as C
 
 import numpy as np
@@ -106,7 +106,7 @@ def test_plain_f8_matmul_mixed_formats_and_fallback(ko):
 
 
 def test_config5_decode_shape_m16(ko):
-    """BASELINE config 5, M = 16: N = K = 8192, scales amax/448, bf16 out; full oracle check."""
+    """benchmark configuration 5, M = 16: N = K = 8192, scales amax/448, bf16 out; full oracle check."""
     M, N, K = 16, 8192, 8192
     aq, sa, wq, sb = _quantised(ko, M, N, K)
     want = np.zeros((M, N), dtype=np.uint16)
@@ -120,7 +120,7 @@ def test_config5_decode_shape_m16(ko):
 
 
 def test_config5_m4096_sampled(ko):
-    """BASELINE config 5, M = 4096: oracle on 64x64 blocks spread over the result."""
+    """benchmark configuration 5, M = 4096: oracle on 64x64 blocks spread over the result."""
     M, N, K = 4096, 8192, 8192
     aq, sa, wq, sb = _quantised(ko, M, N, K)
     da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N, 2)

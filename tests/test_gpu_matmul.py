@@ -1,5 +1,5 @@
 """GPU parity for kapy.matmul: relative Frobenius error <= 1e-3 against the oracle's fp64-accumulated
-result (tolerance stated by BASELINE north_star), closed forms bit-exact."""
+result (the tolerance the benchmark definition states), closed forms bit-exact."""
 import ctypes as C
 
 import numpy as np
@@ -48,7 +48,7 @@ def _run(ko, dt, M, N, K, a_row_major=True, b_row_major=True, out_dtype=None, wi
 
 
 def test_config1_fp16_1024_row_major_128x128x32_tiles(ko):
-    """BASELINE config 1: fp16 GEMM 1024^3, row-major A and B, fp32 accumulate, fp16 out, uniform[-1,1) seed 0."""
+    """benchmark configuration 1: fp16 GEMM 1024^3, row-major A and B, fp32 accumulate, fp16 out, uniform[-1,1) seed 0."""
     got, want = _run(ko, kh.F16, 1024, 1024, 1024, True, True, tile=(128, 128, 32))
     assert _frob(ko, got, want, kh.F16) <= FROB_TOL
     assert (got != want).mean() < 0.05    # fp32 vs fp64 accumulation flips few roundings
@@ -159,7 +159,7 @@ def test_subview_operands(ko):
 
 
 def test_config4_bf16_8192_sampled_against_oracle(ko):
-    """BASELINE config 4: bf16 8192^3, A row-major, B column-major, normal(0,0.02) seeds 0/1, bf16 out.
+    """benchmark configuration 4: bf16 8192^3, A row-major, B column-major, normal(0,0.02) seeds 0/1, bf16 out.
     The GPU computes the whole product; the fp64 oracle recomputes 64x64 blocks spread over the
     result (every block row and column of the 256-tile grid is hit), and linearity in A covers the rest:
     (A + A)·B must equal 2·(A·B) exactly, element by element, in bf16."""

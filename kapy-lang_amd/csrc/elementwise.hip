@@ -293,8 +293,11 @@ struct Node {
   float imm = 0.f;
 };
 
+// `normalised`, if given, receives the program as the kernels are to read it: a copy in which a cast that does not narrow
+// (f16 <-> bf16, any widening) rounds to nearest whatever its rounding mode field says - the reference asks for a rounding
+// mode on down casts only (Kapy.cpp:272-287), and so does the oracle.
 int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *const *ins, int n_ins, const kapy_global *out,
-                   int result_dtype[kMaxInst]) {
+                   int result_dtype[kMaxInst], kapy_ew_inst *normalised = nullptr) {
   if (!prog || n_inst <= 0) return fail(KAPY_ERR_INVALID, "elementwise: empty program");
   if (n_inst > kMaxInst) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: more than %d instructions", kMaxInst);
   if (n_ins < 0 || n_ins > kMaxInputs) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: more than %d inputs", kMaxInputs);
@@ -312,6 +315,7 @@ int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *cons
   auto reg_ok = [&](int r) { return r >= 0 && r < kMaxRegs && reg_dtype[r] >= 0; };
   for (int k = 0; k < n_inst; ++k) {
     const kapy_ew_inst &I = prog[k];
+    if (normalised) normalised[k] = I;
     if (I.op < 0 || I.op >= KAPY_EW_NUM_OPS) return fail(KAPY_ERR_INVALID, "elementwise: unknown op %d at %d", I.op, k);
     if (I.op != KAPY_EW_ST_GLOBAL && (I.dst < 0 || I.dst >= kMaxRegs))
       return fail(KAPY_ERR_INVALID, "elementwise: result register out of range at %d", k);
@@ -339,6 +343,7 @@ int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *cons
       if (sd == KAPY_BF16 && is_f8(dd) && I.rmode == KAPY_RZ)
         return fail(KAPY_ERR_VERIFY, "fptofp: unsupported rounding mode when convert bf16 to f8");
       if (is_f8(sd) && is_f8(dd)) return fail(KAPY_ERR_VERIFY, "fptofp: convert f8 to f8 is not supported");
+      if (normalised && !down) normalised[k].rmode = KAPY_RN;
       reg_dtype[I.dst] = dd;
       break;
     }
@@ -702,8 +707,10 @@ extern "C" {
 int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
                      const kapy_global *out, void *stream) {
   int result_dtype[kMaxInst];
-  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype);
+  kapy_ew_inst normalised[kMaxInst];
+  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype, normalised);
   if (rc) return rc;
+  prog = normalised;
   rc = ensure_device();
   if (rc) return rc;
   const int64_t o0 = extent0(out), o1 = extent1(out);
@@ -807,8 +814,10 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 
 int kapy_elementwise_specialize(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins, const kapy_global *out) {
   int result_dtype[kMaxInst];
-  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype);
+  kapy_ew_inst normalised[kMaxInst];
+  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype, normalised);
   if (rc) return rc;
+  prog = normalised;
   rc = ensure_device();
   if (rc) return rc;
   // act(x*s + bias) with the GELU or no activation already has a hand-written kernel with the activation compiled in:
@@ -827,8 +836,10 @@ int kapy_elementwise_specialize_stats(int64_t *loaded, int64_t *launches) {
 int kapy_elementwise_source(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins, const kapy_global *out,
                             char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes) {
   int result_dtype[kMaxInst];
-  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype);
+  kapy_ew_inst normalised[kMaxInst];
+  int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype, normalised);
   if (rc) return rc;
+  prog = normalised;
   return specialized_source(prog, n_inst, result_dtype, ins, n_ins, out, source, capacity, source_bytes, code_bytes);
 }
 

@@ -1360,7 +1360,7 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s
   if (p.a_sm * 256 >= (int64_t(1) << 31) || p.b_sn * 256 >= (int64_t(1) << 31)) return KAPY_ERR_UNSUPPORTED;
   // the ring variants take any M, N >= 128 and any K >= 128 of whole 16-byte chunks (their loads are bounded by the
   // operands' ends); 256x256 tiles when there are at least as many of them as CUs, 128x128 (two workgroups per CU) below
-  if (KAPY_F8_STAGES == kRing25 && p.K % 16 == 0 && p.K >= 128 && p.M >= 128 && p.N >= 128) {
+  if (KAPY_F8_STAGES == kRing25 && p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
     if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<256, 256, 128, 2, 2, KAPY_F8_STAGES>(p, lhs_fmt, rhs_fmt, s);
     return launch_f8<128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }

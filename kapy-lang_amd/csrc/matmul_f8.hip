@@ -138,6 +138,12 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 // 256 K-bytes of 16 rows each), 16-byte chunk c of row r stored at chunk c ^ r of the row's 256 bytes
 // so that the 16 rows a quarter-wave reads fall into 16 different bank groups.
 // Rows past M / N are clamped to the last valid row (never stored), so nothing is read out of range.
+// From this many rows on the tiled MFMA kernel (which reads the weight once for up to 128 rows) beats the weight-streaming
+// kernel below (which reads it once per 16 rows).
+#ifndef KAPY_F8_TILED_FROM_M
+#define KAPY_F8_TILED_FROM_M 49
+#endif
+constexpr int kTiledFromM = KAPY_F8_TILED_FROM_M;
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
 template <int A_FMT, int B_FMT>
 __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Params p) {
@@ -243,7 +249,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   if (p.M == 0 || p.N == 0) return KAPY_OK;
   bool k_contig = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(a, 1) == 16 && vector_bytes(b, 0) == 16 && p.K % 128 == 0 && p.K > 0;
   // Many rows: the tiled LDS-direct kernel (MFMA-bound).  Few rows: the skinny kernel (HBM-bound).
-  if (k_contig && p.M >= 128 && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
+  if (k_contig && p.M >= kTiledFromM && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
     GemmParams g;
     g.a = (const char *)p.a; g.b = (const char *)p.b; g.acc = nullptr; g.d = p.d;
     g.row_scale = row_scale; g.col_scale = col_scale;

@@ -202,7 +202,8 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
  * installed -- kapy_elementwise keeps working either way.  A program that the hand-written kernels already serve
  * with its activation compiled in (act(x*s + bias) with GELU or no activation, plain binary ops) returns KAPY_OK
  * without compiling anything.  Not to be called while a stream is capturing.  With KAPY_EW_AUTO_SPECIALIZE=1 in
- * the environment kapy_elementwise does this by itself for every program that no hand-written kernel matches. */
+ * the environment kapy_elementwise does this by itself for every program that no hand-written kernel matches;
+ * KAPY_EW_CACHE_DIR=<dir> keeps the compiled code objects on disk for later processes. */
 int kapy_elementwise_specialize(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
                                 const kapy_global *out);
 /* How many specialised kernels this process holds and how many kapy_elementwise calls have run one (either pointer

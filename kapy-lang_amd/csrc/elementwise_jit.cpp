@@ -16,7 +16,9 @@
 // flight, and evaluates the program with row values (CH x 8 registers) and per-row values (one register).
 #include <dlfcn.h>
 #include <hip/hiprtc.h>
+#include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <atomic>
@@ -714,17 +716,57 @@ const Rtc &rtc() {
   return r;
 }
 
+// KAPY_EW_CACHE_DIR names a directory in which compiled code objects are kept from one process to the next, under the hash of
+// the generated text (which embeds the device helpers, so a new build of the library never finds a stale kernel) and of the
+// compiler's options.  A file is written under a temporary name and renamed, so a reader never sees half of one.
+std::string cache_path(const std::string &source, const char *const *opts, int n_opts) {
+  const char *dir = getenv("KAPY_EW_CACHE_DIR");
+  if (!dir || !dir[0]) return std::string();
+  uint64_t h = 1469598103934665603ull;
+  auto mix = [&](const char *data, size_t n) {
+    for (size_t i = 0; i < n; ++i) h = (h ^ (unsigned char)data[i]) * 1099511628211ull;
+  };
+  mix(source.data(), source.size());
+  for (int k = 0; k < n_opts; ++k) mix(opts[k], strlen(opts[k]) + 1);
+  char name[64];
+  snprintf(name, sizeof name, "/kapy_ew_%016llx_%zu.co", (unsigned long long)h, source.size());
+  return std::string(dir) + name;
+}
+bool read_file(const std::string &path, std::vector<char> *data) {
+  FILE *f = fopen(path.c_str(), "rb");
+  if (!f) return false;
+  bool ok = fseek(f, 0, SEEK_END) == 0;
+  const long n = ok ? ftell(f) : -1;
+  ok = ok && n > 0 && fseek(f, 0, SEEK_SET) == 0;
+  if (ok) {
+    data->resize((size_t)n);
+    ok = fread(data->data(), 1, (size_t)n, f) == (size_t)n;
+  }
+  fclose(f);
+  return ok;
+}
+void write_file_atomically(const std::string &path, const std::vector<char> &data) {
+  const std::string tmp = path + ".tmp" + std::to_string((long)getpid());
+  FILE *f = fopen(tmp.c_str(), "wb");
+  if (!f) return;  // an unusable cache directory only costs the compile next time
+  const bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
+  if (fclose(f) != 0 || !ok || rename(tmp.c_str(), path.c_str()) != 0) remove(tmp.c_str());
+}
+
 int compile_source(const std::string &source, std::vector<char> *code) {
+  // Packed fp32 VALU forms stay off, as for every device compile of this library.  Contraction only inside one
+  // expression: in the generated text every op of the program is a statement of its own and must keep its own rounding
+  // (with everything in one basic block the default, cross-statement mode would fuse a mulf and the addf after it).
+  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  constexpr int kOpts = (int)(sizeof opts / sizeof opts[0]);
+  const std::string cached = cache_path(source, opts, kOpts);
+  if (!cached.empty() && read_file(cached, code)) return KAPY_OK;
   const Rtc &r = rtc();
   if (!r.ok) return fail(KAPY_ERR_UNSUPPORTED, "elementwise_specialize: the runtime compiler (libhiprtc) is not available");
   hiprtcProgram prog = nullptr;
   if (r.create(&prog, source.c_str(), "kapy_ew_specialised.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
     return fail(KAPY_ERR_HIP, "elementwise_specialize: hiprtcCreateProgram failed");
-  // Packed fp32 VALU forms stay off, as for every device compile of this library.  Contraction only inside one
-  // expression: in the generated text every op of the program is a statement of its own and must keep its own rounding
-  // (with everything in one basic block the default, cross-statement mode would fuse a mulf and the addf after it).
-  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-  const hiprtcResult rc = r.compile(prog, (int)(sizeof opts / sizeof opts[0]), opts);
+  const hiprtcResult rc = r.compile(prog, kOpts, opts);
   if (rc != HIPRTC_SUCCESS) {
     size_t n = 0;
     r.log_size(prog, &n);
@@ -739,6 +781,7 @@ int compile_source(const std::string &source, std::vector<char> *code) {
   const hiprtcResult got = r.code(prog, code->data());
   r.destroy(&prog);
   if (got != HIPRTC_SUCCESS || n == 0) return fail(KAPY_ERR_HIP, "elementwise_specialize: no code object");
+  if (!cached.empty()) write_file_atomically(cached, *code);
   return KAPY_OK;
 }
 

@@ -105,3 +105,28 @@ def test_specialise_without_a_gpu_fails_loudly():
     with pytest.raises(kh.KapyError) as e:
         kh.elementwise_specialize(kh.program(SILU), [_g(16, 256, kh.F16)], _g(16, 256, kh.F16))
     assert "no CPU fallback" in str(e.value)
+
+
+@pytest.mark.skipif(not _has_runtime_compiler(), reason="libhiprtc is not installed")
+def test_code_objects_are_kept_in_the_cache_directory(tmp_path, monkeypatch):
+    import os
+    import time
+    monkeypatch.setenv("KAPY_EW_CACHE_DIR", str(tmp_path))
+    prog = kh.program([dict(op=L, dst=0, a=0), dict(op=kh.EW_ERF, dst=0, a=0), dict(op=kh.EW_ABSF, dst=0, a=0), dict(op=ST, a=0)])
+    args = ([_g(24, 72, kh.F32)], _g(24, 72, kh.F32))
+    t0 = time.time()
+    _, first = kh.elementwise_source(prog, *args, compile=True)
+    t1 = time.time()
+    files = sorted(os.listdir(tmp_path))
+    assert len(files) == 1 and files[0].startswith("kapy_ew_") and files[0].endswith(".co")
+    assert os.path.getsize(tmp_path / files[0]) == first
+    _, second = kh.elementwise_source(prog, *args, compile=True)      # read back, not compiled again
+    t2 = time.time()
+    assert second == first and sorted(os.listdir(tmp_path)) == files
+    assert t2 - t1 < max(0.05, (t1 - t0) / 3)
+    # another program: another file; a broken file is replaced by a fresh compile
+    kh.elementwise_source(kh.program([dict(op=L, dst=0, a=0), dict(op=kh.EW_NEGF, dst=0, a=0), dict(op=ST, a=0)]), *args, compile=True)
+    assert len(os.listdir(tmp_path)) == 2
+    open(tmp_path / files[0], "wb").close()
+    _, third = kh.elementwise_source(prog, *args, compile=True)
+    assert third == first and os.path.getsize(tmp_path / files[0]) == first

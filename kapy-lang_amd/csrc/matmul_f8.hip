@@ -141,7 +141,7 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 // From this many rows on the tiled MFMA kernel (which reads the weight once for up to 128 rows) beats the weight-streaming
 // kernel below (which reads it once per 16 rows).
 #ifndef KAPY_F8_TILED_FROM_M
-#define KAPY_F8_TILED_FROM_M 49
+#define KAPY_F8_TILED_FROM_M 81
 #endif
 constexpr int kTiledFromM = KAPY_F8_TILED_FROM_M;
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
@@ -150,7 +150,14 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
   __shared__ __attribute__((aligned(1024))) char ring[kStreamWaves * kStreamStages * kStreamStage];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int32_t n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+  // Workgroup id -> (16-column block, 16-row group).  With more than one row group the workgroups that stream the same
+  // columns of the weight must meet in one L2: consecutive ids go to the 8 XCDs in turn, so the groups of a column block
+  // take ids 8 apart (the same XCD, dispatched back to back) and the second reader of a weight line finds it there.
+  const int32_t col_blocks = (p.N + 15) / 16, groups = (p.M + 15) / 16;
+  const int32_t on_xcd = blockIdx.x / 8, xcd = blockIdx.x % 8;
+  const int32_t col_block = (on_xcd / groups) * 8 + xcd;
+  if (col_block >= col_blocks) return;  // (the grid is padded to whole rounds of 8)
+  const int32_t n0 = col_block * 16, m0 = (on_xcd % groups) * 16;
   const int32_t k_per_wave = p.K / kStreamWaves, chunks = k_per_wave / kStreamChunk;
   auto uniform_ptr = [](const uint8_t *ptr) {
     const uint64_t v = (uint64_t)ptr;
@@ -265,7 +272,8 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
       p.b_sn * 16 < (int64_t(1) << 31) && !KAPY_SKINNY_OLD) {
     // rows are addressed from the workgroup's first row, so the per-lane offsets stay small
     F8Params q = p;
-    dim3 grid((unsigned)((p.N + 15) / 16), (unsigned)((p.M + 15) / 16));
+    const int64_t col_rounds = ((p.N + 15) / 16 + 7) / 8, groups = (p.M + 15) / 16;
+    dim3 grid((unsigned)(col_rounds * 8 * groups));
     int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
     if (fa == 0 && fb == 0) skinny_stream_kernel<0, 0><<<grid, 64 * kStreamWaves, 0, s>>>(q);
     else if (fa == 0) skinny_stream_kernel<0, 1><<<grid, 64 * kStreamWaves, 0, s>>>(q);

@@ -1,0 +1,387 @@
+// kapy_hip.hpp — the host side of the hot path in C++, above the C ABI of kapy_hip.h.
+//
+// kapy::OpBuilder mirrors the part of the reference's KapyOpBuilder that the hot path uses
+// (python/src/ir.cc:744-1181: create_mk_global, create_sv_global, create_ld_global, create_st_global,
+// create_splat, create_broadcast, create_transpose, create_fptofp / extf / truncf, the arith and math
+// builders, create_reduce, create_matmul), with the same names and argument meaning.  Where the reference
+// appends an op to a function that is compiled later, this builder records the op in a dataflow graph;
+// create_st_global - the op with the side effect - lowers the graph under its source to ONE library call:
+//   a load (optionally transposed) stored back            -> kapy_copy
+//   a matmul, optionally followed on its result by a scale, a broadcast bias row, an activation and the cast
+//                                                          -> kapy_matmul / kapy_matmul_fused
+//   anything else made of elementwise ops and row reduces  -> kapy_elementwise (one fused kernel)
+// Failures throw kapy::Error carrying the kapy_status and the verifier's text (the reference's builders throw
+// std::invalid_argument / emit op errors).  Header only; link against libkapy_hip.so.
+#ifndef KAPY_HIP_HPP
+#define KAPY_HIP_HPP
+
+#include <stdexcept>
+#include <utility>
+#include <string>
+#include <vector>
+
+#include "kapy_hip.h"
+
+namespace kapy {
+
+struct Error : std::runtime_error {
+  int status;
+  Error(int status_, const std::string &what) : std::runtime_error(what), status(status_) {}
+};
+
+// An SSA value of the builder: a global-memory tensor (descriptor) or a register tensor (graph node).
+class Value {
+ public:
+  Value() = default;
+  bool valid() const { return id_ >= 0; }
+
+ private:
+  friend class OpBuilder;
+  explicit Value(int id) : id_(id) {}
+  int id_ = -1;
+};
+
+class OpBuilder {
+ public:
+  // stream: the hipStream_t every lowered call is issued on (nullptr = the default stream)
+  explicit OpBuilder(void *stream = nullptr) : stream_(stream) {}
+
+  // ---- memory descriptors (python/src/ir.cc:1013-1034) ------------------------------------------------
+  Value create_mk_global(void *global_address, int32_t dynamic_offset, int32_t size0, int32_t size1, int32_t stride0, int32_t stride1,
+                         kapy_dtype element_type, int32_t alignment = 16) {
+    Node n;
+    n.kind = Node::kGlobal;
+    check(kapy_mk_global(&n.global, global_address, dynamic_offset, size0, size1, stride0, stride1, element_type, alignment));
+    n.dtype = element_type;
+    return push(n);
+  }
+  Value create_sv_global(Value source, int32_t start0, int32_t end0, int32_t start1, int32_t end1) {
+    Node n;
+    n.kind = Node::kGlobal;
+    check(kapy_sv_global(&n.global, &global_of(source, "sv_global"), start0, end0, start1, end1));
+    n.dtype = node(source).dtype;
+    return push(n);
+  }
+
+  // ---- loads and stores (ir.cc:1035-1049) ---------------------------------------------------------------
+  Value create_ld_global(Value source, kapy_padding_option padding_option = KAPY_PAD_ZERO, kapy_cache_modifier cache_modifier = KAPY_CACHE_NONE) {
+    Node n;
+    n.kind = Node::kLoad;
+    n.global = global_of(source, "ld_global");
+    n.dtype = node(source).dtype;
+    n.padding = padding_option;
+    n.cache = cache_modifier;
+    return push(n);
+  }
+  // Lowers everything `source` depends on and stores it: the one call that launches work.
+  void create_st_global(Value source, Value target, kapy_cache_modifier cache_modifier = KAPY_CACHE_NONE) {
+    const kapy_global &out = global_of(target, "st_global");
+    const Node &s = node(source);
+    if (s.kind == Node::kGlobal) throw Error(KAPY_ERR_VERIFY, "st_global: source must be a register tensor");
+    if (s.kind == Node::kLoad) {  // a layout move: bits travel untouched
+      kapy_copy_cfg cfg = {s.transposed ? 1 : 0, s.padding, cache_modifier != KAPY_CACHE_NONE ? cache_modifier : s.cache, 0};
+      check(kapy_copy(&s.global, &out, &cfg, stream_));
+      return;
+    }
+    if (depends_on_matmul(source.id_)) {
+      lower_matmul(source.id_, out);
+      return;
+    }
+    std::vector<kapy_ew_inst> prog;
+    std::vector<const kapy_global *> ins;
+    emit_program(source.id_, &prog, &ins);
+    check(kapy_elementwise(prog.data(), (int32_t)prog.size(), ins.data(), (int32_t)ins.size(), &out, stream_));
+  }
+  // The elementwise program create_st_global(source, ...) would run (for inspection and for kapy_elementwise_specialize).
+  std::vector<kapy_ew_inst> program_of(Value source, std::vector<kapy_global> *inputs = nullptr) {
+    std::vector<kapy_ew_inst> prog;
+    std::vector<const kapy_global *> ins;
+    emit_program(source.id_, &prog, &ins);
+    if (inputs) {
+      inputs->clear();
+      for (const kapy_global *g : ins) inputs->push_back(*g);
+    }
+    return prog;
+  }
+
+  // ---- shape ops (ir.cc:1071-1090) ------------------------------------------------------------------------
+  // the reference splats a scalar Value to a tensor shape; a program's shape is its result's, so the scalar and its type suffice
+  Value create_splat(float source, kapy_dtype element_type) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = KAPY_EW_SPLAT;
+    n.dtype = element_type;
+    n.imm = source;
+    return push(n);
+  }
+  // kapy.broadcast: extents of 1 stretch to the result's.  A load of a [1 x n] or [m x 1] view already is one; the
+  // requested shape is checked when the program is verified against its result.
+  Value create_broadcast(Value source, const std::vector<int64_t> & /*shape*/) {
+    if (node(source).kind == Node::kGlobal) throw Error(KAPY_ERR_VERIFY, "broadcast: source must be a tensor");
+    return source;
+  }
+  // kapy.transpose of a loaded tensor is the load with swapped strides; of a computed tensor: store it through a
+  // descriptor with swapped strides instead
+  Value create_transpose(Value source) {
+    Node n = node(source);
+    if (n.kind != Node::kLoad) throw Error(KAPY_ERR_UNSUPPORTED, "transpose: only of a loaded tensor (store a computed one through swapped strides)");
+    n.transposed = !n.transposed;
+    return push(n);
+  }
+
+  // ---- casts (ir.cc:744-790) ---------------------------------------------------------------------------
+  Value create_fptofp(Value source, kapy_dtype element_type, kapy_rounding_mode rounding_mode = KAPY_RN) {
+    return unary(KAPY_EW_FPTOFP, source, element_type, rounding_mode);
+  }
+  Value create_extf(Value source, kapy_dtype element_type) { return create_fptofp(source, element_type, KAPY_RN); }
+  Value create_truncf(Value source, kapy_dtype element_type) { return create_fptofp(source, element_type, KAPY_RN); }
+
+  // ---- arith / math (ir.cc:791-1157) ---------------------------------------------------------------------
+  Value create_addf(Value lhs, Value rhs) { return binary(KAPY_EW_ADDF, lhs, rhs); }
+  Value create_subf(Value lhs, Value rhs) { return binary(KAPY_EW_SUBF, lhs, rhs); }
+  Value create_mulf(Value lhs, Value rhs) { return binary(KAPY_EW_MULF, lhs, rhs); }
+  Value create_divf(Value lhs, Value rhs) { return binary(KAPY_EW_DIVF, lhs, rhs); }
+  Value create_maximumf(Value lhs, Value rhs) { return binary(KAPY_EW_MAXIMUMF, lhs, rhs); }
+  Value create_minimumf(Value lhs, Value rhs) { return binary(KAPY_EW_MINIMUMF, lhs, rhs); }
+  Value create_fma(Value a, Value b, Value c) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = KAPY_EW_FMA;
+    n.a = tensor(a, "fma");
+    n.b = tensor(b, "fma");
+    n.c = tensor(c, "fma");
+    n.dtype = node(a).dtype;
+    return push(n);
+  }
+  Value create_negf(Value source) { return unary(KAPY_EW_NEGF, source); }
+  Value create_absf(Value source) { return unary(KAPY_EW_ABSF, source); }
+  Value create_exp(Value source) { return unary(KAPY_EW_EXP, source); }
+  Value create_exp2(Value source) { return unary(KAPY_EW_EXP2, source); }
+  Value create_log(Value source) { return unary(KAPY_EW_LOG, source); }
+  Value create_log2(Value source) { return unary(KAPY_EW_LOG2, source); }
+  Value create_sqrt(Value source) { return unary(KAPY_EW_SQRT, source); }
+  Value create_rsqrt(Value source) { return unary(KAPY_EW_RSQRT, source); }
+  Value create_erf(Value source) { return unary(KAPY_EW_ERF, source); }
+  // create_elementwise_extern_lib (ir.cc:1168-1174): the library functions the path uses, by name
+  Value create_elementwise_extern_lib(const std::string &name, Value source) {
+    if (name == "tanh") return unary(KAPY_EW_TANH, source);
+    if (name == "gelu" || name == "gelu_tanh") return unary(KAPY_EW_GELU_TANH, source);
+    throw Error(KAPY_ERR_UNSUPPORTED, "elementwise_extern_lib: unknown function " + name);
+  }
+
+  // ---- reduce and matmul (ir.cc:1101-1105, 1175-1181) ---------------------------------------------------------
+  // kapy.reduce with an addf (is_max = false) or maximumf combiner along `axis`, its result broadcast back over the axis
+  Value create_reduce(Value source, int32_t axis, bool is_max = false) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = is_max ? KAPY_EW_REDUCE_MAX : KAPY_EW_REDUCE_SUM;
+    n.a = tensor(source, "reduce");
+    n.axis = axis;
+    n.dtype = node(source).dtype;
+    return push(n);
+  }
+  // acc may be an invalid Value (no accumulator input); the result has the accumulator type f32
+  Value create_matmul(Value lhs, Value rhs, Value acc = Value(), kapy_matmul_impl_way impl_way = KAPY_MATMUL_AUTO) {
+    if (node(lhs).kind != Node::kLoad || node(rhs).kind != Node::kLoad || (acc.valid() && node(acc).kind != Node::kLoad))
+      throw Error(KAPY_ERR_UNSUPPORTED, "matmul: operands must be loaded tensors");
+    Node n;
+    n.kind = Node::kMatmul;
+    n.a = lhs.id_;
+    n.b = rhs.id_;
+    n.c = acc.id_;
+    n.impl_way = impl_way;
+    n.dtype = KAPY_F32;
+    return push(n);
+  }
+
+ private:
+  struct Node {
+    enum Kind { kGlobal, kLoad, kOp, kMatmul } kind = kOp;
+    kapy_global global{};
+    int op = -1, a = -1, b = -1, c = -1, dtype = KAPY_F32, rmode = KAPY_RN, axis = 1;
+    int padding = KAPY_PAD_ZERO, cache = KAPY_CACHE_NONE, impl_way = KAPY_MATMUL_AUTO;
+    bool transposed = false;
+    float imm = 0.f;
+  };
+  std::vector<Node> nodes_;
+  void *stream_;
+
+  static void check(int rc) {
+    if (rc < 0) throw Error(rc, kapy_last_error());
+  }
+  Value push(const Node &n) {
+    nodes_.push_back(n);
+    return Value((int)nodes_.size() - 1);
+  }
+  const Node &node(Value v) const {
+    if (v.id_ < 0 || v.id_ >= (int)nodes_.size()) throw Error(KAPY_ERR_INVALID, "use of an undefined value");
+    return nodes_[v.id_];
+  }
+  const kapy_global &global_of(Value v, const char *what) const {
+    if (node(v).kind != Node::kGlobal) throw Error(KAPY_ERR_VERIFY, std::string(what) + ": operand must be a global-memory tensor");
+    return node(v).global;
+  }
+  int tensor(Value v, const char *what) const {
+    if (node(v).kind == Node::kGlobal) throw Error(KAPY_ERR_VERIFY, std::string(what) + ": operand must be a register tensor (ld_global it first)");
+    return v.id_;
+  }
+  Value unary(int op, Value source, int dtype = -1, int rmode = KAPY_RN) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = op;
+    n.a = tensor(source, "elementwise");
+    n.dtype = dtype >= 0 ? dtype : node(source).dtype;
+    n.rmode = rmode;
+    return push(n);
+  }
+  Value binary(int op, Value lhs, Value rhs) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = op;
+    n.a = tensor(lhs, "elementwise");
+    n.b = tensor(rhs, "elementwise");
+    n.dtype = node(lhs).dtype;
+    return push(n);
+  }
+  // the view a load reads: strides and extents swapped when it went through create_transpose
+  static kapy_global view_of(const Node &ld) {
+    kapy_global g = ld.global;
+    if (ld.transposed) {
+      std::swap(g.start0, g.start1);
+      std::swap(g.end0, g.end1);
+      std::swap(g.stride0, g.stride1);
+    }
+    return g;
+  }
+  bool depends_on_matmul(int id) const {
+    if (id < 0) return false;
+    const Node &n = nodes_[id];
+    if (n.kind == Node::kMatmul) return true;
+    if (n.kind != Node::kOp) return false;
+    return depends_on_matmul(n.a) || depends_on_matmul(n.b) || depends_on_matmul(n.c);
+  }
+
+  // Post-order walk of the graph under `root` into a straight-line program.  A register is freed after the last use of
+  // its value, so graphs far larger than the 16 registers of a program fit as long as 16 values are never live at once.
+  std::vector<kapy_global> views_;  // storage for the descriptors the emitted program points at
+  void emit_program(int root, std::vector<kapy_ew_inst> *prog, std::vector<const kapy_global *> *ins) {
+    if (root < 0 || root >= (int)nodes_.size()) throw Error(KAPY_ERR_INVALID, "use of an undefined value");
+    std::vector<int> order, uses(nodes_.size(), 0), reg(nodes_.size(), -1);
+    std::vector<char> seen(nodes_.size(), 0);
+    struct Walk {
+      const std::vector<Node> &nodes;
+      std::vector<int> &order, &uses;
+      std::vector<char> &seen;
+      void visit(int id) {
+        ++uses[id];
+        if (seen[id]) return;
+        seen[id] = 1;
+        const Node &n = nodes[id];
+        if (n.kind == Node::kMatmul || n.kind == Node::kGlobal) throw Error(KAPY_ERR_UNSUPPORTED, "elementwise: operand is not a register tensor of this program");
+        if (n.kind == Node::kOp)
+          for (int o : {n.a, n.b, n.c})
+            if (o >= 0) visit(o);
+        order.push_back(id);
+      }
+    } walk{nodes_, order, uses, seen};
+    walk.visit(root);
+    views_.clear();
+    views_.reserve(order.size());
+    std::vector<int> free_regs;
+    for (int r = 15; r >= 0; --r) free_regs.push_back(r);
+    auto release = [&](int id) {
+      if (id >= 0 && --uses[id] == 0) free_regs.push_back(reg[id]);
+    };
+    for (int id : order) {
+      const Node &n = nodes_[id];
+      kapy_ew_inst I = {n.op, 0, 0, 0, 0, n.dtype, n.rmode, n.imm};
+      if (n.kind == Node::kLoad) {
+        views_.push_back(view_of(n));
+        ins->push_back(&views_.back());
+        I.op = KAPY_EW_LD_GLOBAL;
+        I.a = (int32_t)ins->size() - 1;
+        I.c = n.padding;
+      } else {
+        I.a = n.a >= 0 ? reg[n.a] : 0;
+        I.b = n.b >= 0 ? reg[n.b] : 0;
+        I.c = n.c >= 0 ? reg[n.c] : 0;
+        if (n.op == KAPY_EW_REDUCE_SUM || n.op == KAPY_EW_REDUCE_MAX) I.b = n.axis;
+        release(n.a);
+        release(n.b);
+        release(n.c);
+      }
+      if (free_regs.empty()) throw Error(KAPY_ERR_UNSUPPORTED, "elementwise: more than 16 values live at once");
+      reg[id] = free_regs.back();
+      free_regs.pop_back();
+      I.dst = reg[id];
+      prog->push_back(I);
+    }
+    --uses[root];
+    prog->push_back({KAPY_EW_ST_GLOBAL, 0, reg[root], 0, 0, 0, KAPY_RN, 0.f});
+  }
+
+  // matmul [-> mulf splat] [-> addf broadcast(extf? ld bias)] [-> activation] [-> fptofp]: the tail goes into the epilogue
+  void lower_matmul(int root, const kapy_global &out) {
+    int cur = root;
+    kapy_matmul_epilogue epi = {nullptr, 1.0f, -1, 0.f};
+    bool tail = false;
+    auto is_op = [&](int id, int op) { return id >= 0 && nodes_[id].kind == Node::kOp && nodes_[id].op == op; };
+    auto splat_of = [&](int id, float *v) {
+      if (!is_op(id, KAPY_EW_SPLAT)) return false;
+      *v = nodes_[id].imm;
+      return true;
+    };
+    if (is_op(cur, KAPY_EW_FPTOFP)) cur = nodes_[cur].a;  // the final cast: the result descriptor's type says the same
+    // the activation
+    float operand = 0.f;
+    if (is_op(cur, KAPY_EW_MAXIMUMF) || is_op(cur, KAPY_EW_MINIMUMF)) {
+      const Node &n = nodes_[cur];
+      if (splat_of(n.b, &operand)) { epi.act = n.op; epi.act_operand = operand; cur = n.a; tail = true; }
+      else if (splat_of(n.a, &operand)) { epi.act = n.op; epi.act_operand = operand; cur = n.b; tail = true; }
+    } else if (cur >= 0 && nodes_[cur].kind == Node::kOp && nodes_[cur].op >= KAPY_EW_NEGF && nodes_[cur].op <= KAPY_EW_GELU_TANH) {
+      epi.act = nodes_[cur].op;
+      cur = nodes_[cur].a;
+      tail = true;
+    }
+    // the bias: a loaded [1 x N] row, possibly widened
+    kapy_global bias;
+    if (is_op(cur, KAPY_EW_ADDF)) {
+      auto as_bias = [&](int id) {
+        if (is_op(id, KAPY_EW_FPTOFP) && nodes_[id].dtype == KAPY_F32) id = nodes_[id].a;
+        return id >= 0 && nodes_[id].kind == Node::kLoad ? id : -1;
+      };
+      const Node &n = nodes_[cur];
+      int b = as_bias(n.b), other = n.a;
+      if (b < 0) { b = as_bias(n.a); other = n.b; }
+      if (b < 0) throw Error(KAPY_ERR_UNSUPPORTED, "matmul: only a loaded bias row can be added in the epilogue");
+      bias = view_of(nodes_[b]);
+      epi.bias = &bias;
+      cur = other;
+      tail = true;
+    }
+    // the scale
+    if (is_op(cur, KAPY_EW_MULF)) {
+      const Node &n = nodes_[cur];
+      float s;
+      if (splat_of(n.b, &s)) { epi.alpha = s; cur = n.a; tail = true; }
+      else if (splat_of(n.a, &s)) { epi.alpha = s; cur = n.b; tail = true; }
+    }
+    if (cur < 0 || nodes_[cur].kind != Node::kMatmul)
+      throw Error(KAPY_ERR_UNSUPPORTED, "matmul: the ops on its result must be [mulf splat] [addf bias row] [activation] [fptofp]");
+    const Node &mm = nodes_[cur];
+    const kapy_global lhs = view_of(nodes_[mm.a]), rhs = view_of(nodes_[mm.b]);
+    kapy_matmul_cfg cfg = {mm.impl_way, 0, 0, 0, KAPY_RN, 0, 0, 0};
+    if (tail) {
+      if (mm.c >= 0) throw Error(KAPY_ERR_UNSUPPORTED, "matmul: an accumulator input and a fused tail do not combine");
+      check(kapy_matmul_fused(&lhs, &rhs, &out, &epi, &cfg, stream_));
+    } else {
+      kapy_global acc;
+      if (mm.c >= 0) acc = view_of(nodes_[mm.c]);
+      check(kapy_matmul(&lhs, &rhs, mm.c >= 0 ? &acc : nullptr, &out, &cfg, stream_));
+    }
+  }
+};
+
+}  // namespace kapy
+
+#endif  // KAPY_HIP_HPP

@@ -1,0 +1,161 @@
+// Exercises kapy::OpBuilder (include/kapy_hip.hpp) from C++.  "cpu": what needs no device - the programs the builder
+// lowers to, the verifier's refusals as exceptions, the loud failure without a GPU.  "gpu": the same graphs run on the
+// device (elementwise chain, transposed store, matmul with a fused tail) against plain host arithmetic.
+#include <hip/hip_runtime_api.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+#include "kapy_hip.hpp"
+
+#define EXPECT(cond)                                                       \
+  do {                                                                     \
+    if (!(cond)) {                                                         \
+      printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);             \
+      exit(1);                                                             \
+    }                                                                      \
+  } while (0)
+
+static kapy::Value gelu_chain(kapy::OpBuilder &b, kapy::Value x, kapy::Value bias, kapy_dtype dt) {
+  kapy::Value xv = b.create_extf(b.create_ld_global(x), KAPY_F32);
+  kapy::Value bv = b.create_broadcast(b.create_extf(b.create_ld_global(bias), KAPY_F32), {0, 0});
+  kapy::Value v = b.create_addf(b.create_mulf(xv, b.create_splat(0.5f, KAPY_F32)), bv);
+  return b.create_truncf(b.create_elementwise_extern_lib("gelu", v), dt);
+}
+
+static int run_cpu() {
+  char fake[64];  // descriptors only: nothing is dereferenced on the host
+  kapy::OpBuilder b;
+  kapy::Value x = b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_F16), bias = b.create_mk_global(fake, 0, 1, 256, 256, 1, KAPY_F16);
+  kapy::Value y = b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_F16);
+  std::vector<kapy_global> ins;
+  std::vector<kapy_ew_inst> prog = b.program_of(gelu_chain(b, x, bias, KAPY_F16), &ins);
+  const int want[] = {KAPY_EW_LD_GLOBAL, KAPY_EW_FPTOFP, KAPY_EW_SPLAT, KAPY_EW_MULF, KAPY_EW_LD_GLOBAL, KAPY_EW_FPTOFP, KAPY_EW_ADDF, KAPY_EW_GELU_TANH,
+                      KAPY_EW_FPTOFP, KAPY_EW_ST_GLOBAL};
+  EXPECT(prog.size() == sizeof want / sizeof want[0] && ins.size() == 2);
+  for (size_t k = 0; k < prog.size(); ++k) EXPECT(prog[k].op == want[k]);
+  EXPECT(ins[1].end0 - ins[1].start0 == 1);  // the bias row: extent 1 along axis 0 is the broadcast
+  // the library accepts the program: its verifier and the specialised-kernel generator both run without a device
+  const kapy_global *ptrs[2] = {&ins[0], &ins[1]};
+  kapy_global out;
+  EXPECT(kapy_mk_global(&out, fake, 0, 64, 256, 256, 1, KAPY_F16, 16) == KAPY_OK);
+  int64_t text = 0;
+  EXPECT(kapy_elementwise_source(prog.data(), (int32_t)prog.size(), ptrs, 2, &out, nullptr, 0, &text, nullptr) == KAPY_OK && text > 1000);
+  // registers are recycled: a chain of 40 ops fits the 16 registers of a program
+  kapy::Value lx = b.create_ld_global(x), v = lx;
+  for (int k = 0; k < 40; ++k) v = b.create_addf(v, lx);   // lx stays live throughout, every sum dies at the next one
+  prog = b.program_of(v, &ins);
+  EXPECT(prog.size() == 42 && ins.size() == 1);
+  for (const kapy_ew_inst &I : prog) EXPECT(I.dst >= 0 && I.dst < 16);
+  // the verifier's refusal arrives as an exception with the reference's wording
+  try {
+    kapy::Value h = b.create_ld_global(x), w = b.create_ld_global(b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_BF16));
+    b.create_st_global(b.create_addf(h, w), y);
+    EXPECT(!"mixed element types must be refused");
+  } catch (const kapy::Error &e) {
+    EXPECT(e.status == KAPY_ERR_VERIFY && strstr(e.what(), "same element type"));
+  }
+  try {
+    b.create_addf(x, x);   // a global-memory tensor is not a register tensor
+    EXPECT(!"global operands must be refused");
+  } catch (const kapy::Error &e) {
+    EXPECT(e.status == KAPY_ERR_VERIFY);
+  }
+  try {
+    b.create_st_global(b.create_exp(b.create_matmul(b.create_ld_global(x), b.create_ld_global(x))), y);
+    EXPECT(!"exp on a matmul result is not a fusable tail");
+  } catch (const kapy::Error &e) {
+    EXPECT(e.status == KAPY_ERR_UNSUPPORTED || e.status == KAPY_ERR_VERIFY);
+  }
+  int n_dev = 0;
+  if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
+    try {
+      b.create_st_global(gelu_chain(b, x, bias, KAPY_F16), y);
+      EXPECT(!"without a device the call must fail");
+    } catch (const kapy::Error &e) {
+      EXPECT(e.status == KAPY_ERR_HIP && strstr(e.what(), "no CPU fallback"));
+    }
+  }
+  printf("builder cpu ok\n");
+  return 0;
+}
+
+static float h2f(uint16_t h) { return (float)*reinterpret_cast<_Float16 *>(&h); }
+static uint16_t f2h(float f) { _Float16 h = (_Float16)f; return *reinterpret_cast<uint16_t *>(&h); }
+static float b2f(uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); return f; }
+static uint16_t f2b(float f) { uint32_t u; memcpy(&u, &f, 4); return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16); }
+#define HIP_OK(e) EXPECT((e) == hipSuccess)
+
+static int run_gpu() {
+  const int m = 96, n = 256;
+  std::vector<uint16_t> x(m * n), bias(n), y(m * n), yt(m * n);
+  srand(7);
+  auto rnd = [] { return (float)(rand() % 65536) / 65536.f * 4.f - 2.f; };
+  for (auto &v : x) v = f2h(rnd());
+  for (auto &v : bias) v = f2h(rnd());
+  uint16_t *dx, *db, *dy, *dt;
+  HIP_OK(hipMalloc((void **)&dx, x.size() * 2)); HIP_OK(hipMalloc((void **)&db, bias.size() * 2));
+  HIP_OK(hipMalloc((void **)&dy, y.size() * 2)); HIP_OK(hipMalloc((void **)&dt, y.size() * 2));
+  HIP_OK(hipMemcpy(dx, x.data(), x.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(db, bias.data(), bias.size() * 2, hipMemcpyHostToDevice));
+  kapy::OpBuilder b;
+  kapy::Value gx = b.create_mk_global(dx, 0, m, n, n, 1, KAPY_F16), gb = b.create_mk_global(db, 0, 1, n, n, 1, KAPY_F16);
+  kapy::Value gy = b.create_mk_global(dy, 0, m, n, n, 1, KAPY_F16), gt = b.create_mk_global(dt, 0, n, m, m, 1, KAPY_F16);
+  b.create_st_global(gelu_chain(b, gx, gb, KAPY_F16), gy);                  // one fused kernel
+  b.create_st_global(b.create_transpose(b.create_ld_global(gy)), gt);       // the layout move of its result
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(y.data(), dy, y.size() * 2, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(yt.data(), dt, yt.size() * 2, hipMemcpyDeviceToHost));
+  for (int i = 0; i < m; ++i)
+    for (int j = 0; j < n; ++j) {
+      const double v = (double)h2f(x[i * n + j]) * 0.5 + h2f(bias[j]);
+      const double want = 0.5 * v * (1.0 + tanh(0.7978845608028654 * (v + 0.044715 * v * v * v)));
+      const double got = h2f(y[i * n + j]);
+      EXPECT(fabs(got - want) <= 2.5 * fmax(fabs(want), 6.1e-5) * 0.0009765625);   // 2 ulp of f16 and a rounding
+      EXPECT(yt[j * m + i] == y[i * n + j]);                                       // bit-exact
+    }
+  // relu(A.B^T * 0.25 + bias) in bf16: matmul with the tail in its epilogue
+  const int M = 128, N = 256, K = 128;
+  std::vector<uint16_t> a(M * K), w(N * K), c(M * N), bb(N);
+  for (auto &v : a) v = f2b(rnd() * 0.25f);
+  for (auto &v : w) v = f2b(rnd() * 0.25f);
+  for (auto &v : bb) v = f2b(rnd());
+  uint16_t *da, *dw, *dc, *dbb;
+  HIP_OK(hipMalloc((void **)&da, a.size() * 2)); HIP_OK(hipMalloc((void **)&dw, w.size() * 2));
+  HIP_OK(hipMalloc((void **)&dc, c.size() * 2)); HIP_OK(hipMalloc((void **)&dbb, bb.size() * 2));
+  HIP_OK(hipMemcpy(da, a.data(), a.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(dw, w.data(), w.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(dbb, bb.data(), bb.size() * 2, hipMemcpyHostToDevice));
+  kapy::Value ga = b.create_mk_global(da, 0, M, K, K, 1, KAPY_BF16), gw = b.create_mk_global(dw, 0, K, N, 1, K, KAPY_BF16);   // B column-major
+  kapy::Value gc = b.create_mk_global(dc, 0, M, N, N, 1, KAPY_BF16), gbb = b.create_mk_global(dbb, 0, 1, N, N, 1, KAPY_BF16);
+  kapy::Value acc = b.create_matmul(b.create_ld_global(ga), b.create_ld_global(gw));
+  kapy::Value t = b.create_addf(b.create_mulf(acc, b.create_splat(0.25f, KAPY_F32)), b.create_extf(b.create_ld_global(gbb), KAPY_F32));
+  b.create_st_global(b.create_truncf(b.create_maximumf(t, b.create_splat(0.f, KAPY_F32)), KAPY_BF16), gc);
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(c.data(), dc, c.size() * 2, hipMemcpyDeviceToHost));
+  double err2 = 0, ref2 = 0;
+  for (int i = 0; i < M; ++i)
+    for (int j = 0; j < N; ++j) {
+      double s = 0;
+      for (int k = 0; k < K; ++k) s += (double)b2f(a[i * K + k]) * b2f(w[j * K + k]);
+      const double want = fmax(s * 0.25 + b2f(bb[j]), 0.0), got = b2f(c[i * N + j]);
+      err2 += (got - want) * (got - want);
+      ref2 += want * want;
+    }
+  EXPECT(sqrt(err2 / ref2) <= 4e-3);   // bf16 result: half an ulp (2^-9) per element at most, well inside
+  printf("builder gpu ok\n");
+  return 0;
+}
+
+int main(int argc, char **argv) {
+  try {
+    return argc > 1 && std::string(argv[1]) == "gpu" ? run_gpu() : run_cpu();
+  } catch (const kapy::Error &e) {
+    printf("FAILED: kapy status %d: %s\n", e.status, e.what());
+    return 1;
+  }
+}

@@ -1,0 +1,26 @@
+"""The C++ host side (include/kapy_hip.hpp: kapy::OpBuilder, the reference's create_* builder names over the C ABI),
+exercised by tests/cpp/builder_test: lowering and error behaviour without a device, the same graphs on the GPU."""
+import os
+import subprocess
+
+import pytest
+
+HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp")
+BINARY = os.path.join(HERE, "builder_test")
+
+
+def _binary():
+    if not os.path.exists(BINARY):      # built by __graft_entry__.build(); a source checkout builds it here (host code only)
+        subprocess.check_call(["make", "-C", HERE, "-s"])
+    return BINARY
+
+
+def test_builder_lowers_and_refuses_without_a_device():
+    out = subprocess.run([_binary(), "cpu"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "builder cpu ok" in out.stdout, out.stdout + out.stderr
+
+
+@pytest.mark.gpu
+def test_builder_runs_the_graphs_on_the_gpu():
+    out = subprocess.run([_binary(), "gpu"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "builder gpu ok" in out.stdout, out.stdout + out.stderr

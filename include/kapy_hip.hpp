@@ -143,6 +143,12 @@ class OpBuilder {
   Value create_divf(Value lhs, Value rhs) { return binary(KAPY_EW_DIVF, lhs, rhs); }
   Value create_maximumf(Value lhs, Value rhs) { return binary(KAPY_EW_MAXIMUMF, lhs, rhs); }
   Value create_minimumf(Value lhs, Value rhs) { return binary(KAPY_EW_MINIMUMF, lhs, rhs); }
+  // kapy.clampf(source, low, high, propagateNan) (ir.cc:886-890): min(max(source, low), high); maximumf / minimumf propagate NaNs,
+  // the only form the elementwise programs have
+  Value create_clampf(Value source, Value low, Value high, bool propagate_nan = true) {
+    if (!propagate_nan) throw Error(KAPY_ERR_UNSUPPORTED, "clampf: only the NaN-propagating form is implemented");
+    return create_minimumf(create_maximumf(source, low), high);
+  }
   Value create_fma(Value a, Value b, Value c) {
     Node n;
     n.kind = Node::kOp;

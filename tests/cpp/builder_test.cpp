@@ -51,6 +51,8 @@ static int run_cpu() {
   prog = b.program_of(v, &ins);
   EXPECT(prog.size() == 42 && ins.size() == 1);
   for (const kapy_ew_inst &I : prog) EXPECT(I.dst >= 0 && I.dst < 16);
+  prog = b.program_of(b.create_clampf(lx, b.create_splat(-1.f, KAPY_F16), b.create_splat(1.f, KAPY_F16)));
+  EXPECT(prog.size() == 6 && prog[2].op == KAPY_EW_MAXIMUMF && prog[4].op == KAPY_EW_MINIMUMF);
   // the verifier's refusal arrives as an exception with the reference's wording
   try {
     kapy::Value h = b.create_ld_global(x), w = b.create_ld_global(b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_BF16));

@@ -217,7 +217,7 @@ __device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const
 // q[e] = x[e] / y[e], correctly rounded.  When every operand of every lane is zero or of middling magnitude (2^-60 ..
 // 2^60: nothing on the way can overflow or go subnormal) the quotient comes from the sequence at the core of the IEEE
 // division without its scaling, special-case and mode-switching steps: the reciprocal refined once, the quotient
-// corrected by its exact remainder.  Anything else (tiny, huge, infinite, NaN) takes the full division.
+// corrected twice by its exact remainder.  Anything else (tiny, huge, infinite, NaN) takes the full division.
 __device__ __forceinline__ void div8(const float (&x)[8], const float (&y)[8], float (&q)[8]) {
   bool plain = true;
 #pragma unroll
@@ -231,7 +231,8 @@ __device__ __forceinline__ void div8(const float (&x)[8], const float (&y)[8], f
       const float r0 = __builtin_amdgcn_rcpf(y[e]);
       const float r1 = __builtin_fmaf(__builtin_fmaf(-y[e], r0, 1.0f), r0, r0);
       const float q0 = x[e] * r1;
-      q[e] = __builtin_fmaf(__builtin_fmaf(-q0, y[e], x[e]), r1, q0);
+      const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, y[e], x[e]), r1, q0);
+      q[e] = __builtin_fmaf(__builtin_fmaf(-q1, y[e], x[e]), r1, q1);  // the second correction: without it one quotient in ~10^5 is an ulp off
     }
   } else {
 #pragma unroll

@@ -128,7 +128,11 @@ __device__ __forceinline__ float e5m2_to_f32(uint8_t b) { return __builtin_amdgc
 // neighbour a few times in a million.  For bf16 (no 16-bit fma on this part) and f32 the fp32 fma serves.
 __device__ __forceinline__ float fma_typed(float a, float b, float c, int dtype) {
   if (dtype == KAPY_F16) return (float)__builtin_fmaf16((_Float16)a, (_Float16)b, (_Float16)c);
-  return __builtin_fmaf(a, b, c);
+  float r = __builtin_fmaf(a, b, c);
+  // The fp32 result must exist as such: where a cast to f16 follows directly (straight-line compiled programs), the compiler
+  // would otherwise fold it into the fma (v_fma_mixlo_f16), which rounds the exact sum once - not what fma-then-truncf means.
+  asm volatile("" : "+v"(r));
+  return r;
 }
 
 // Value of element `idx` of a typed buffer as an fp32 (exact for every supported type but i32).

@@ -737,8 +737,17 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
         case EW_DIVF: r = a / reg[I.b][at]; break;
         case EW_FMA: r = std::fma(a, reg[I.b][at], reg[I.c][at]); break;
         // arith.maximumf / minimumf propagate NaN
-        case EW_MAXIMUMF: r = (std::isnan(a) || std::isnan(reg[I.b][at])) ? qnan : std::max(a, reg[I.b][at]); break;
-        case EW_MINIMUMF: r = (std::isnan(a) || std::isnan(reg[I.b][at])) ? qnan : std::min(a, reg[I.b][at]); break;
+        // arith.maximumf / minimumf: NaN if either operand is, and -0 orders below +0 (max.NaN / min.NaN of PTX do the same)
+        case EW_MAXIMUMF: {
+          const double b = reg[I.b][at];
+          r = (std::isnan(a) || std::isnan(b)) ? qnan : a == b ? (std::signbit(a) ? b : a) : std::max(a, b);
+          break;
+        }
+        case EW_MINIMUMF: {
+          const double b = reg[I.b][at];
+          r = (std::isnan(a) || std::isnan(b)) ? qnan : a == b ? (std::signbit(a) ? a : b) : std::min(a, b);
+          break;
+        }
         case EW_NEGF: r = -a; break;
         case EW_ABSF: r = std::fabs(a); break;
         case EW_EXP: r = std::exp(a); break;

@@ -72,7 +72,7 @@ def _same(got, want, dtype):
     return np.array_equal(is_nan(got), nan) and np.array_equal(got[~nan], want[~nan])
 
 
-@pytest.mark.parametrize("seed", range(60))
+@pytest.mark.parametrize("seed", list(range(100)) + [212])      # (98 and 212 once differed: min(+0, -0) in the oracle, an fma folded into the cast after it)
 def test_random_exact_program(ko, seed):
     rng = np.random.RandomState(1000 + seed)
     m, n, insts, kinds, in_dtypes, out_dtype, out_kind = _random_case(rng)

@@ -257,3 +257,15 @@ def test_elementwise_reduce_ops_vs_numpy_and_scipy(ko):
     # a reduce along an axis that does not exist is rejected
     bad = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_REDUCE_SUM, dst=1, a=0, b=2), dict(op=ko.EW_ST_GLOBAL, a=1)])
     assert ko.elementwise(bad, [g(xi)], g(out)) == -14
+
+
+def test_maximumf_minimumf_order_signed_zeros_and_propagate_nan(ko):
+    """arith.maximumf / minimumf: -0 < +0 whichever operand comes first, NaN if either operand is NaN."""
+    a = np.array([0x0000, 0x8000, 0x0000, 0x8000, 0x7e00, 0x3c00], np.uint16).reshape(1, 6)   # +0 -0 +0 -0 NaN 1
+    b = np.array([0x8000, 0x0000, 0x0000, 0x8000, 0x3c00, 0x7e00], np.uint16).reshape(1, 6)   # -0 +0 +0 -0 1 NaN
+    for op, want in ((ko.EW_MAXIMUMF, [0x0000, 0x0000, 0x0000, 0x8000]), (ko.EW_MINIMUMF, [0x8000, 0x8000, 0x0000, 0x8000])):
+        out = np.zeros((1, 6), np.uint16)
+        insts = [dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_LD_GLOBAL, dst=1, a=1), dict(op=op, dst=2, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=2)]
+        assert ko.elementwise(ko.program(insts), [ko.mk_global(a, 1, 6, 6, 1, ko.F16), ko.mk_global(b, 1, 6, 6, 1, ko.F16)], ko.mk_global(out, 1, 6, 6, 1, ko.F16)) == 0
+        assert out[0, :4].tolist() == want
+        assert np.all(np.isnan(out[0, 4:].view(np.float16)))

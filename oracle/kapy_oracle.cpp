@@ -598,7 +598,12 @@ static double round_to(double v, int dtype) {
 }
 
 static double gelu_tanh(double v) {
-  return 0.5 * v * (1.0 + std::tanh(0.7978845608028654 * (v + 0.044715 * v * v * v)));
+  // 0.5*v*(1 + tanh(u)), u = sqrt(2/pi)*(v + 0.044715 v^3).  Written out like that, 1 + tanh(u) cancels for u << 0 (below
+  // u = -17 nothing but rounding noise is left of it in fp64, while the result, ~1e-15, is an ordinary bf16 or f32 value);
+  // 0.5*(1 + tanh(u)) = 1/(1 + exp(-2u)) is the same function without the cancellation.
+  const double u = 0.7978845608028654 * (v + 0.044715 * v * v * v);
+  if (u < -4.0) return v / (1.0 + std::exp(-2.0 * u));
+  return 0.5 * v * (1.0 + std::tanh(u));
 }
 
 int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *ins, int n_ins, const ko_global *out) {

@@ -269,3 +269,21 @@ def test_maximumf_minimumf_order_signed_zeros_and_propagate_nan(ko):
         assert ko.elementwise(ko.program(insts), [ko.mk_global(a, 1, 6, 6, 1, ko.F16), ko.mk_global(b, 1, 6, 6, 1, ko.F16)], ko.mk_global(out, 1, 6, 6, 1, ko.F16)) == 0
         assert out[0, :4].tolist() == want
         assert np.all(np.isnan(out[0, 4:].view(np.float16)))
+
+
+def test_gelu_tail_keeps_its_relative_accuracy(ko):
+    """gelu_tanh(v) for v << 0 against the closed form evaluated with 50 digits (mpmath-free: exact rational exp bounds are
+    overkill; numpy longdouble's 64-bit mantissa in the cancellation-free form is the reference): bf16 results down to 1e-30."""
+    v = np.array([-4.0, -5.0, -6.0, -6.5, -7.0, -7.5, -8.0, -9.0], np.float32)
+    bits = (v.view(np.uint32) >> 16).astype(np.uint16).reshape(1, -1)             # exactly representable in bf16
+    out = np.zeros_like(bits)
+    insts = [dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_FPTOFP, dst=1, a=0, dtype=ko.F32), dict(op=ko.EW_GELU_TANH, dst=1, a=1),
+             dict(op=ko.EW_FPTOFP, dst=2, a=1, dtype=ko.BF16, rmode=ko.RN), dict(op=ko.EW_ST_GLOBAL, a=2)]
+    n = bits.shape[1]
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(bits, 1, n, n, 1, ko.BF16)], ko.mk_global(out, 1, n, n, 1, ko.BF16)) == 0
+    got = (out.astype(np.uint32) << 16).view(np.float32).astype(np.float64).ravel()
+    vl = v.astype(np.longdouble)
+    u = np.longdouble("0.7978845608028654") * (vl + np.longdouble("0.044715") * vl ** 3)
+    want = (vl / (1 + np.exp(-2 * u))).astype(np.float64)
+    assert np.all(want < 0) and want[-1] > -1e-20
+    assert np.max(np.abs(got - want) / np.abs(want)) <= 2.0 ** -8        # half an ulp of bf16

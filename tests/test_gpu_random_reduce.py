@@ -1,0 +1,110 @@
+"""Seeded random kapy.reduce calls and batched layout moves: random extents (multiples of the vector widths and not), both
+axes, sum and max, row- or column-major windows into larger buffers with pitches that keep or break 16-byte alignment, every
+pairing of f16 / bf16 / f32 source and result.  max is bit-exact against the oracle; sum is accumulated in fp32 on the device
+and in double by the oracle, so it is held to the fp32 accumulation bound plus one rounding of the result's type.  Nothing
+outside the result window may change."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import kapy_hip as kh
+from gpu_util import dglobal, sync, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+NP = {1: np.uint8, 2: np.uint16, 4: np.uint32}
+VALUE = {kh.F16: np.uint16, kh.BF16: np.uint16, kh.F32: np.float32}     # the storage type the oracle's decode expects
+EPS = {kh.F16: 2.0 ** -11, kh.BF16: 2.0 ** -8, kh.F32: 2.0 ** -24}
+SHAPES = [(2, 256), (64, 1000), (300, 128), (1024, 64), (37, 2048), (5, 520), (1000, 96), (130, 50), (1, 4096), (256, 1),
+          (33, 33), (8, 512), (512, 8), (96, 1536), (2048, 32), (7, 7)]
+
+
+def _window(rng, rows, cols, itemsize):
+    """(buffer elements, offset, strides) of a rows x cols window, row- or column-major, pitch >= extent."""
+    col_major = rng.randint(3) == 0
+    lead, other = (rows, cols) if col_major else (cols, rows)
+    pitch = lead + [0, 0, 8, 16 // itemsize, 3, 1][rng.randint(6)]
+    offset = [0, 0, 16 // itemsize, 5][rng.randint(4)]
+    return offset + pitch * other + 8, offset, ((1, pitch) if col_major else (pitch, 1))
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_reduce(ko, seed):
+    rng = np.random.RandomState(9000 + seed)
+    sdt = [kh.F16, kh.BF16, kh.F32][rng.randint(3)]
+    ddt = [kh.F32, sdt, kh.F16, kh.BF16][rng.randint(4)]
+    sb, db = kh.DTYPE_BYTES[sdt], kh.DTYPE_BYTES[ddt]
+    m, n = SHAPES[rng.randint(len(SHAPES))]
+    axis, kind = int(rng.randint(2)), int(rng.randint(2))
+    om, on = (m, 1) if axis == 1 else (1, n)
+    s_count, s_off, s_str = _window(rng, m, n, sb)
+    d_count, d_off, d_str = _window(rng, om, on, db)
+    scale = [1.0, 0.05, 30.0][rng.randint(3)]
+    src = ko.fill_normal(s_count, sdt, 9000 + seed, 0, 0.0, scale)
+    fill = 0x5A5A5A5A & (2 ** (8 * db) - 1)
+    want = np.full(d_count, fill, NP[db])
+    so = ko.mk_global(src[s_off:], m, n, s_str[0], s_str[1], sdt)
+    do = ko.mk_global(want[d_off:], om, on, d_str[0], d_str[1], ddt)
+    describe = "seed %d: %s of dtype %d -> %d, %dx%d along axis %d, src strides %s offset %d, dst strides %s offset %d" % (
+        seed, "max" if kind else "sum", sdt, ddt, m, n, axis, s_str, s_off, d_str, d_off)
+    assert ko.lib().ko_reduce(C.byref(so), C.byref(do), axis, kind) == 0, describe
+    d_src, d_dst = to_dev(src), to_dev(np.full(d_count, fill, NP[db]))
+    kh.reduce(dglobal(d_src, m, n, s_str[0], s_str[1], sdt, dynamic_offset=s_off),
+              dglobal(d_dst, om, on, d_str[0], d_str[1], ddt, dynamic_offset=d_off), axis, kind)
+    sync()
+    got = to_host(d_dst, NP[db])
+    inside = np.zeros(d_count, bool)
+    idx = d_off + (np.arange(om)[:, None] * d_str[0] + np.arange(on)[None, :] * d_str[1]).ravel()
+    inside[idx] = True
+    assert np.array_equal(got[~inside], want[~inside]), describe + ": wrote outside the result window"
+    if kind == 1:
+        bad = np.flatnonzero(got != want)
+        assert len(bad) == 0, "%s: %d results differ, first at %d (got %#x want %#x)" % (describe, len(bad), bad[0], got[bad[0]], want[bad[0]])
+        return
+    g = ko.decode(got[idx].view(VALUE[ddt]), ddt)
+    w = ko.decode(want[idx].view(VALUE[ddt]), ddt)
+    # the magnitude the accumulation error scales with: sum of |x| along the reduced axis
+    vals = np.abs(ko.decode(src.view(VALUE[sdt]), sdt))
+    sidx = s_off + np.arange(m)[:, None] * s_str[0] + np.arange(n)[None, :] * s_str[1]
+    mass = vals[sidx].sum(axis=axis).ravel()
+    bound = 2.0 ** -22 * mass + 2.0 * EPS[ddt] * np.abs(w) + 1e-30
+    worst = np.argmax(np.abs(g - w) - bound)
+    assert np.all(np.abs(g - w) <= bound), "%s: result %d is %r, oracle %r, bound %g" % (describe, worst, g[worst], w[worst], bound[worst])
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_batched_copy(ko, seed):
+    """A b x h grid of tiles moved between two 4-D layouts (any of the two orders of the grid axes on either side), with or
+    without a transpose of the tile itself: bit-exact against the oracle and against numpy's transpose of the same array."""
+    rng = np.random.RandomState(9500 + seed)
+    dtype = [kh.F16, kh.BF16, kh.F32, kh.F8E4M3][rng.randint(4)]
+    eb = kh.DTYPE_BYTES[dtype]
+    b, h = int(rng.randint(1, 4)), int(rng.randint(1, 6))
+    s, d = [(40, 64), (64, 64), (17, 24), (128, 32), (33, 128), (8, 8), (100, 16)][rng.randint(7)]
+    transpose = bool(rng.randint(2))
+    src_bhsd, dst_bhsd = bool(rng.randint(2)), bool(rng.randint(2))
+    ds, dd_ = (d, s) if transpose else (s, d)
+    src = rng.randint(0, 2 ** (8 * min(eb, 4) - (1 if eb == 4 else 0)), size=b * h * s * d).astype(NP[eb])
+
+    def layout(bhsd, rows, cols):
+        """(row stride, offsets along b and h) of a [b,h,rows,cols] (bhsd) or [b,rows,h,cols] array."""
+        return (cols, h * rows * cols, rows * cols) if bhsd else (h * cols, rows * h * cols, cols)
+
+    s_row, s_b, s_h = layout(src_bhsd, s, d)
+    d_row, d_b, d_h = layout(dst_bhsd, ds, dd_)
+    describe = "seed %d: dtype %d grid %dx%d tile %dx%d%s, source %s, result %s" % (
+        seed, dtype, b, h, s, d, " transposed" if transpose else "", "bhsd" if src_bhsd else "bshd", "bhsd" if dst_bhsd else "bshd")
+    want = np.zeros(b * h * s * d, NP[eb])
+    assert ko.lib().ko_copy_batched(C.byref(ko.mk_global(src, s, d, s_row, 1, dtype)), C.byref(ko.mk_global(want, ds, dd_, d_row, 1, dtype)),
+                                    int(transpose), 0, b, h, s_b, s_h, d_b, d_h) == 0, describe
+    d_src, d_dst = to_dev(src), to_dev(np.zeros(b * h * s * d, NP[eb]))
+    kh.copy_batched(dglobal(d_src, s, d, s_row, 1, dtype), dglobal(d_dst, ds, dd_, d_row, 1, dtype), (b, h, s_b, s_h, d_b, d_h),
+                    transpose=transpose)
+    sync()
+    got = to_host(d_dst, NP[eb])
+    assert np.array_equal(got, want), describe
+    a = src.reshape(b, h, s, d) if src_bhsd else src.reshape(b, s, h, d).transpose(0, 2, 1, 3)      # -> [b,h,s,d]
+    if transpose:
+        a = a.transpose(0, 1, 3, 2)
+    expect = a if dst_bhsd else a.transpose(0, 2, 1, 3)
+    assert np.array_equal(got.reshape(expect.shape), expect), describe + " (numpy transpose)"

@@ -23,6 +23,7 @@
 #include <algorithm>
 #include <climits>
 #include <map>
+#include <memory>
 #include <set>
 #include <string>
 #include <vector>
@@ -502,8 +503,22 @@ struct Analyzer {
 // Bytes of LDS one gfx950 workgroup can have.
 constexpr int64_t kLdsBytes = 160 * 1024;
 
+// A register tensor that has not been computed yet: one elementwise op over computed register tensors (leaves) and other
+// deferred tensors.  A chain of arith / math / cast / splat / broadcast ops stays deferred until an op that is not
+// elementwise needs its value; a kapy.st_global then runs the whole chain as ONE program that stores straight into the
+// global view, which is what the reference's pipeline compiles such a chain to (one fused kernel body, no temporaries).
+struct Expr {
+  int ew = KAPY_EW_LD_GLOBAL;  // KAPY_EW_LD_GLOBAL: a leaf (`leaf` is the computed tensor); -1: the operand itself (broadcast)
+  int dtype = 0, rmode = KAPY_RN;
+  float imm = 0.f;
+  std::shared_ptr<Expr> in[3];
+  int n_in = 0;
+  kapy_global leaf;
+};
+
 struct Value {
   enum Kind { kNone, kInt, kPtr, kTensor, kFloat } kind = kNone;
+  std::shared_ptr<Expr> lazy;  // kTensor: set while the tensor is deferred; g then only carries its shape and type
   int64_t i = 0;
   double f = 0.0;     // kFloat: a scalar of float type
   void *ptr = nullptr;
@@ -542,8 +557,131 @@ struct Interp {
     auto it = env.find(op.operands[k]);
     if (it == env.end()) { fail_op(op, "use of undefined value " + op.operands[k]); return false; }
     if (it->second.kind != kind) { fail_op(op, "operand " + op.operands[k] + " has the wrong kind"); return false; }
+    if (it->second.lazy && force(op, it->second) != KAPY_OK) return false;
     v = it->second;
     return true;
+  }
+
+  // ---- deferred elementwise chains ----
+  bool fuse = true;  // KAPY_MLIR_FUSE=0: every op runs by itself, as one call
+  bool is_register_tensor(const kapy_global &g) const {
+    const char *p = (const char *)g.ptr;
+    return p >= arena + kSharedArena && p < arena + kArena;
+  }
+  // the operand as an expression: deferred tensors as they are, computed ones as leaves
+  std::shared_ptr<Expr> as_expr(const Value &v) {
+    if (v.lazy) return v.lazy;
+    auto e = std::make_shared<Expr>();
+    e->leaf = v.g;
+    return e;
+  }
+  static constexpr int kMaxProgram = 48, kMaxRegisters = 16;  // what one kapy_elementwise program may hold
+  struct Emit {
+    kapy_ew_inst prog[kMaxProgram];
+    const kapy_global *ins[8];
+    int n = 0, n_ins = 0, regs = 0;
+    std::map<const Expr *, int> reg;
+    bool ok = true;
+  };
+  int emit(const std::shared_ptr<Expr> &e, Emit &m) {
+    auto it = m.reg.find(e.get());
+    if (it != m.reg.end()) return it->second;
+    int src[3] = {0, 0, 0};
+    for (int k = 0; k < e->n_in; ++k) src[k] = emit(e->in[k], m);
+    if (!m.ok) return 0;
+    if (e->ew < 0) return m.reg[e.get()] = src[0];
+    if (m.regs >= kMaxRegisters || m.n >= kMaxProgram - 1) { m.ok = false; return 0; }
+    const int dst = m.regs++;
+    if (e->ew == KAPY_EW_LD_GLOBAL) {
+      int slot = -1;
+      for (int k = 0; k < m.n_ins; ++k)
+        if (!memcmp(m.ins[k], &e->leaf, sizeof(kapy_global))) slot = k;
+      if (slot < 0) {
+        if (m.n_ins >= 8) { m.ok = false; return 0; }
+        m.ins[slot = m.n_ins++] = &e->leaf;
+      }
+      m.prog[m.n++] = {KAPY_EW_LD_GLOBAL, dst, slot, 0, 0, 0, KAPY_RN, 0.f};
+    } else {
+      m.prog[m.n++] = {e->ew, dst, src[0], src[1], src[2], e->dtype, e->rmode, e->imm};
+    }
+    return m.reg[e.get()] = dst;
+  }
+  // the chain as one program that stores into `out`
+  int run_chain(const std::shared_ptr<Expr> &e, const kapy_global *out) {
+    Emit m;
+    const int r = emit(e, m);
+    if (!m.ok) return fail(KAPY_ERR_UNSUPPORTED, "the deferred chain does not fit one program");
+    m.prog[m.n++] = {KAPY_EW_ST_GLOBAL, 0, r, 0, 0, 0, KAPY_RN, 0.f};
+    return kapy_elementwise(m.prog, m.n, m.ins, m.n_ins, out, stream);
+  }
+  bool fits(const std::shared_ptr<Expr> &e) {
+    Emit m;
+    emit(e, m);
+    return m.ok;
+  }
+  // computes a deferred tensor into a new register tensor; `v` (an entry of env, or a copy of one) becomes that tensor
+  int force(const Op &op, Value &v) {
+    if (!v.lazy) return KAPY_OK;
+    const int32_t rows = v.g.end0 - v.g.start0, cols = v.g.end1 - v.g.start1;
+    void *ptr = alloc((size_t)rows * cols * dtype_bytes(v.g.dtype));
+    if (!ptr) return fail_op(op, "register tensors of one program instance exceed the arena");
+    kapy_global g;
+    int rc = lib(op, kapy_mk_global(&g, ptr, 0, rows, cols, cols, 1, v.g.dtype, 256));
+    if (rc == KAPY_OK) rc = lib(op, run_chain(v.lazy, &g));
+    if (rc != KAPY_OK) return rc;
+    // every other holder of the same expression now reads the computed tensor as well
+    v.lazy->ew = KAPY_EW_LD_GLOBAL;
+    v.lazy->n_in = 0;
+    for (auto &p : v.lazy->in) p.reset();
+    v.lazy->leaf = g;
+    v.lazy.reset();
+    v.g = g;
+    for (auto &kv : env)
+      if (kv.second.lazy && kv.second.lazy->ew == KAPY_EW_LD_GLOBAL && kv.second.lazy->n_in == 0 && !memcmp(&kv.second.lazy->leaf, &g, sizeof g)) {
+        kv.second.lazy.reset();
+        kv.second.g = g;
+      }
+    return KAPY_OK;
+  }
+  // result <- ew(operands...) without running anything; falls back to computing operands when the chain would outgrow one
+  // program, and to computing the result at once when an operand is memory the program can still change
+  int defer(const Op &op, int n_operands, int ew, int dtype, int rmode, float imm) {
+    if (op.types.empty()) return fail_op(op, "missing result type");
+    const Type &ty = op.types.back();
+    if (ty.kind != Type::kTensor || ty.shape[0] <= 0 || ty.shape[1] <= 0) return fail_op(op, "result must be a statically shaped tensor");
+    auto e = std::make_shared<Expr>();
+    e->ew = ew; e->dtype = dtype; e->rmode = rmode; e->imm = imm; e->n_in = n_operands;
+    bool at_once = !fuse;
+    for (int k = 0; k < n_operands; ++k) {
+      if (k >= (int)op.operands.size()) return fail_op(op, "missing operand");
+      auto it = env.find(op.operands[k]);
+      if (it == env.end()) return fail_op(op, "use of undefined value " + op.operands[k]);
+      if (it->second.kind != Value::kTensor) return fail_op(op, "operand " + op.operands[k] + " has the wrong kind");
+      if (!it->second.lazy && !is_register_tensor(it->second.g)) at_once = true;
+      e->in[k] = as_expr(it->second);
+    }
+    if (!fits(e)) {  // compute the deferred operands, which leaves a program of one instruction
+      for (int k = 0; k < n_operands; ++k) {
+        Value &v = env[op.operands[k]];
+        if (v.lazy) {
+          int rc = force(op, v);
+          if (rc != KAPY_OK) return rc;
+        }
+        e->in[k] = as_expr(v);
+      }
+    }
+    Value r;
+    r.kind = Value::kTensor;
+    r.lazy = e;
+    memset(&r.g, 0, sizeof r.g);
+    if (kapy_mk_global(&r.g, arena, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 16) != KAPY_OK)
+      return fail_op(op, kapy_last_error());
+    if (at_once) {
+      int rc = force(op, r);
+      if (rc != KAPY_OK) return rc;
+    }
+    env[op.results[0]] = r;
+    return KAPY_OK;
   }
   // a new row-major register tensor of the op's result type
   bool new_tensor(const Op &op, const Type &ty, Value &v) {
@@ -574,37 +712,12 @@ struct Interp {
   }
   int lib(const Op &op, int rc) { return rc == KAPY_OK ? KAPY_OK : (fail_op(op, kapy_last_error()), rc); }
 
-  int binary_tensor(const Op &op, int ew) {
-    Value a, b, r;
-    if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
-    kapy_ew_inst prog[4] = {{KAPY_EW_LD_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f}, {KAPY_EW_LD_GLOBAL, 1, 1, 0, 0, 0, KAPY_RN, 0.f},
-                            {ew, 2, 0, 1, 0, 0, KAPY_RN, 0.f}, {KAPY_EW_ST_GLOBAL, 0, 2, 0, 0, 0, KAPY_RN, 0.f}};
-    const kapy_global *ins[2] = {&a.g, &b.g};
-    int rc = lib(op, kapy_elementwise(prog, 4, ins, 2, &r.g, stream));
-    if (rc == KAPY_OK) env[op.results[0]] = r;
-    return rc;
-  }
+  int binary_tensor(const Op &op, int ew) { return defer(op, 2, ew, 0, KAPY_RN, 0.f); }
 
-  // result <- a one-instruction program over the tensor operands (ew < 0: none, the operand itself is stored; this is
-  // kapy.broadcast when the operand has extent 1 where the result does not)
+  // result <- one instruction over the tensor operands (ew < 0: none, the operand itself; this is kapy.broadcast when
+  // the operand has extent 1 where the result does not)
   int mapped_tensor(const Op &op, int n_operands, int ew, int dtype = 0, int rmode = KAPY_RN) {
-    Value in[3], r;
-    for (int k = 0; k < n_operands; ++k)
-      if (!get(op, k, Value::kTensor, in[k])) return KAPY_ERR_INVALID;
-    if (op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
-    kapy_ew_inst prog[5];
-    int n = 0;
-    for (int k = 0; k < n_operands; ++k) prog[n++] = {KAPY_EW_LD_GLOBAL, k, k, 0, 0, 0, KAPY_RN, 0.f};
-    int result = 0;
-    if (ew >= 0) {
-      prog[n++] = {ew, n_operands, 0, 1, 2, dtype, rmode, 0.f};
-      result = n_operands;
-    }
-    prog[n++] = {KAPY_EW_ST_GLOBAL, 0, result, 0, 0, 0, KAPY_RN, 0.f};
-    const kapy_global *ins[3] = {&in[0].g, &in[1].g, &in[2].g};
-    int rc = lib(op, kapy_elementwise(prog, n, ins, n_operands, &r.g, stream));
-    if (rc == KAPY_OK) env[op.results[0]] = r;
-    return rc;
+    return defer(op, n_operands, ew, dtype, rmode, 0.f);
   }
 
   int run_ops(const std::vector<Op> &ops, std::vector<Value> *yielded) {
@@ -625,6 +738,10 @@ struct Interp {
       for (size_t k = 0; k < op.operands.size(); ++k) {
         auto it = env.find(op.operands[k]);
         if (it == env.end()) return fail_op(op, "use of undefined value " + op.operands[k]);
+        if (it->second.lazy) {  // a loop-carried tensor is computed once per iteration
+          int rc = force(op, it->second);
+          if (rc != KAPY_OK) return rc;
+        }
         yielded->push_back(it->second);
       }
       return KAPY_OK;
@@ -640,11 +757,7 @@ struct Interp {
         r.kind = Value::kFloat;
         r.f = op.words.empty() ? 0.0 : atof(op.words[0].c_str());
       } else if (ty.kind == Type::kTensor) {
-        if (!new_tensor(op, ty, r)) return KAPY_ERR_INVALID;
-        const float v = op.words.empty() ? 0.f : (float)atof(op.words[0].c_str());
-        kapy_ew_inst prog[2] = {{KAPY_EW_SPLAT, 0, 0, 0, 0, ty.dtype, KAPY_RN, v}, {KAPY_EW_ST_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f}};
-        int rc = lib(op, kapy_elementwise(prog, 2, nullptr, 0, &r.g, stream));
-        if (rc) return rc;
+        return defer(op, 0, KAPY_EW_SPLAT, ty.dtype, KAPY_RN, op.words.empty() ? 0.f : (float)atof(op.words[0].c_str()));
       } else return fail_op(op, "unsupported constant type");
       env[op.results[0]] = r;
       return KAPY_OK;
@@ -709,12 +822,8 @@ struct Interp {
     }
     if (n == "kapy.splat") {
       Value v;
-      if (!get(op, 0, Value::kFloat, v) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
-      kapy_ew_inst prog[2] = {{KAPY_EW_SPLAT, 0, 0, 0, 0, op.types.back().dtype, KAPY_RN, (float)v.f}, {KAPY_EW_ST_GLOBAL, 0, 0, 0, 0, 0, KAPY_RN, 0.f}};
-      int rc = lib(op, kapy_elementwise(prog, 2, nullptr, 0, &r.g, stream));
-      if (rc) return rc;
-      env[op.results[0]] = r;
-      return KAPY_OK;
+      if (!get(op, 0, Value::kFloat, v) || op.types.empty()) return KAPY_ERR_INVALID;
+      return defer(op, 0, KAPY_EW_SPLAT, op.types.back().dtype, KAPY_RN, (float)v.f);
     }
     if (n == "kapy.transpose") {  // result[j, i] = source[i, j] (TransposeOpToLLVM.cpp:21-26 relabels; here the data moves)
       if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
@@ -768,6 +877,16 @@ struct Interp {
       return KAPY_OK;
     }
     if (n == "kapy.st_global" || n == "kapy.st_shared" || n == "kapy.cp_async_global_to_shared") {
+      // a deferred chain stores straight into a view of its own shape; anything else (padding, a program the
+      // elementwise entry point refuses) goes through a register tensor as before
+      auto src = op.operands.empty() ? env.end() : env.find(op.operands[0]);
+      if (src != env.end() && src->second.kind == Value::kTensor && src->second.lazy) {
+        if (!get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
+        const kapy_global &sg = src->second.g;
+        if (b.g.end0 - b.g.start0 == sg.end0 - sg.start0 && b.g.end1 - b.g.start1 == sg.end1 - sg.start1 && b.g.dtype == sg.dtype &&
+            run_chain(src->second.lazy, &b.g) == KAPY_OK)
+          return KAPY_OK;
+      }
       if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
       return lib(op, kapy_copy(&a.g, &b.g, nullptr, stream));
     }
@@ -927,6 +1046,7 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   if (rc) return rc;
   Interp in(f, (hipStream_t)stream);
   in.plan = &plan;
+  if (const char *e = getenv("KAPY_MLIR_FUSE")) in.fuse = atoi(e) != 0;
   KAPY_HIP_CHECK(hipMalloc((void **)&in.arena, kArena));
   rc = KAPY_OK;
   for (int32_t p2 = 0; p2 < grid[2] && rc == KAPY_OK; ++p2)

@@ -222,6 +222,51 @@ def softmax_program(rows_per_warp=2, cols=256, num_warps=2, dtype="f16"):
             "  kapy.func public @softmax_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" + body + "  }\n}\n")
 
 
+def gated_program(rows_per_warp=4, cols=256, num_warps=2, dtype="f16"):
+    """out[r, :] = silu(x[r, :]) * y[r, :] * g[r] in f32, rounded once: two casts up, negf, math.exp, a splat of 1.0, addf,
+    divf, mulf, a broadcast of the per-row gate g ([rows x 1]), mulf, a cast down.  Eleven elementwise ops between the loads
+    and the store."""
+    t16, t32 = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype), "tensor<%dx%dxf32" % (rows_per_warp, cols)
+    c32 = "tensor<%dx1xf32" % rows_per_warp
+    dyn, dyn32 = "tensor<?x?x%s, #global>" % dtype, "tensor<?x?xf32, #global>"
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols])
+    body += """    %one = arith.constant 1.0 : f32
+    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %gy = kapy.mk_global %y[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %gg = kapy.mk_global %gate[%c0_i32] [%rows, %c1_i32] [%c1_i32, %c1_i32] : !kapy.ptr<1> -> {dyn32}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %sy = kapy.sv_global %gy[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %sg = kapy.sv_global %gg[%row0 : %row1, %c0_i32 : %c1_i32] : {dyn32} -> {c32}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %x16 = kapy.ld_global %sx : {t16}, #global> -> {t16}, #values>
+    %y16 = kapy.ld_global %sy : {t16}, #global> -> {t16}, #values>
+    %gv = kapy.ld_global %sg : {c32}, #global> -> {c32}, #values>
+    %xf = kapy.fptofp %x16 : {t16}, #values> to {t32}, #values>
+    %yf = kapy.fptofp %y16 : {t16}, #values> to {t32}, #values>
+    %nx = arith.negf %xf : {t32}, #values>
+    %ex = math.exp %nx : {t32}, #values>
+    %ones = kapy.splat %one : f32 -> {t32}, #values>
+    %den = arith.addf %ex, %ones : {t32}, #values>
+    %sig = arith.divf %xf, %den : {t32}, #values>
+    %prod = arith.mulf %sig, %yf : {t32}, #values>
+    %gb = kapy.broadcast %gv : {c32}, #values> -> {t32}, #values>
+    %scaled = arith.mulf %prod, %gb : {t32}, #values>
+    %r = kapy.fptofp %scaled {{rounding_mode = 1 : i32}} : {t32}, #values> to {t16}, #values>
+    kapy.st_global %r, %so : {t16}, #values>, {t16}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, dyn32=dyn32, t16=t16, t32=t32, c32=c32)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @gated_kernel(%x: !kapy.ptr<1>, %y: !kapy.ptr<1>, %gate: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" +
+            body + "  }\n}\n")
+
+
 def scaled_transpose_program(tile=32, scale=0.5, dtype="f16"):
     """out[j, i] = x[i, j] * scale over tile x tile blocks, one block per program: ld_global, kapy.transpose, kapy.splat of
     a scalar constant, mulf, st_global."""

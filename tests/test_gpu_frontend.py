@@ -103,6 +103,71 @@ def test_softmax_program_in_kapy_ops_matches_the_oracle_program(ko):
     assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # op by op in f32, one rounding to f16 at the end
 
 
+def _gated_insts():
+    L, CAST, ST = kh.EW_LD_GLOBAL, kh.EW_FPTOFP, kh.EW_ST_GLOBAL
+    return [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=L, dst=1, a=1), dict(op=CAST, dst=1, a=1, dtype=kh.F32),
+            dict(op=kh.EW_NEGF, dst=2, a=0), dict(op=kh.EW_EXP, dst=2, a=2), dict(op=kh.EW_SPLAT, dst=3, dtype=kh.F32, imm=1.0),
+            dict(op=kh.EW_ADDF, dst=2, a=2, b=3), dict(op=kh.EW_DIVF, dst=2, a=0, b=2), dict(op=kh.EW_MULF, dst=2, a=2, b=1),
+            dict(op=L, dst=4, a=2), dict(op=kh.EW_MULF, dst=2, a=2, b=4), dict(op=CAST, dst=5, a=2, dtype=kh.F16, rmode=kh.RN),
+            dict(op=ST, a=5)]
+
+
+def test_chain_of_elementwise_ops_runs_as_one_program(ko, monkeypatch):
+    """silu(x) * y * gate[row]: eleven elementwise ops between the loads and the store.  The front-end defers them and the store
+    runs them as one program; with KAPY_MLIR_FUSE=0 every op is a call of its own.  Both equal the oracle's run of the same
+    program to the bar of the elementwise tests, and each other bit for bit (the same instructions on the same values)."""
+    rows_per_warp, cols, warps, programs = 4, 256, 2, 3
+    rows = rows_per_warp * warps * programs
+    x, y = ko.fill_normal(rows * cols, ko.F16, 61, std=2.0), ko.fill_normal(rows * cols, ko.F16, 62)
+    gate = np.linspace(0.25, 2.0, rows).astype(np.float32)
+    want = np.zeros(rows * cols, np.uint16)
+    g = lambda a: ko.mk_global(a, rows, cols, cols, 1, ko.F16)
+    assert ko.elementwise(ko.program(_gated_insts()), [g(x), g(y), ko.mk_global(gate, rows, 1, 1, 1, ko.F32)], g(want)) == 0
+    dx, dy, dg = to_dev(x), to_dev(y), to_dev(gate)
+    text = kp.gated_program(rows_per_warp, cols, warps)
+    results = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+        dout = dev_zeros(rows * cols, 2, fill=0x7e00)
+        kh.run_mlir(text, [dx, dy, dg, dout, rows], [programs])
+        sync()
+        results.append(to_host(dout, np.uint16))
+        assert ulp_diff_f16(results[-1], want).max() <= 2
+    assert np.array_equal(results[0], results[1])
+
+
+def test_fused_chain_is_one_kernel(ko):
+    """With KAPY_EW_AUTO_SPECIALIZE=1 (read once per process, so in a process of its own) every program outside the hand-written
+    kernels is compiled when first seen: the chain of eleven ops leaves exactly one compiled kernel behind, launched once per
+    program instance and warp."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r'''
+import sys
+sys.path[:0] = [%r, %r, %r]
+import numpy as np, torch, kapy_hip as kh, ko, kapy_programs as kp
+from gpu_util import dev_zeros, sync, to_dev, to_host
+rows_per_warp, cols, warps, programs = 4, 256, 2, 3
+rows = rows_per_warp * warps * programs
+x, y = ko.fill_normal(rows * cols, ko.F16, 61, std=2.0), ko.fill_normal(rows * cols, ko.F16, 62)
+gate = np.linspace(0.25, 2.0, rows).astype(np.float32)
+dx, dy, dg, dout = to_dev(x), to_dev(y), to_dev(gate), dev_zeros(rows * cols, 2, fill=0x7e00)
+kh.run_mlir(kp.gated_program(rows_per_warp, cols, warps), [dx, dy, dg, dout, rows], [programs]); sync()
+assert kh.elementwise_specialize_stats() == (1, programs * warps), kh.elementwise_specialize_stats()
+xf, yf = x.view(np.float16).astype(np.float64).reshape(rows, cols), y.view(np.float16).astype(np.float64).reshape(rows, cols)
+ref = xf / (1 + np.exp(-xf)) * yf * gate[:, None].astype(np.float64)
+got = to_host(dout, np.float16, (rows, cols)).astype(np.float64)
+assert np.all(np.abs(got - ref) <= 2e-3 * np.abs(ref) + 1e-6), np.abs(got - ref).max()
+print("fused ok")
+''' % (os.path.join(root, "kapy-lang_amd", "python"), os.path.join(root, "oracle"), os.path.join(root, "tests"))
+    env = dict(os.environ, KAPY_EW_AUTO_SPECIALIZE="1")
+    env.pop("KAPY_MLIR_FUSE", None)
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and "fused ok" in out.stdout, out.stdout + out.stderr
+
+
 def test_transpose_splat_program_is_bit_exact(ko):
     m, n, tile = 96, 64, 32
     x = ko.fill_normal(m * n, ko.F16, 52)

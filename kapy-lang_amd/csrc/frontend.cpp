@@ -514,6 +514,9 @@ struct Expr {
   std::shared_ptr<Expr> in[3];
   int n_in = 0;
   kapy_global leaf;
+  // KAPY_EW_REDUCE_SUM / _MAX along axis 1: inside a program the result sits on every element of the row, so the node
+  // can only be part of a program whose result has the operand's shape (rows x cols) and element type (operand_dtype)
+  int32_t rows = 0, cols = 0, operand_dtype = 0;
 };
 
 struct Value {
@@ -601,18 +604,67 @@ struct Interp {
         m.ins[slot = m.n_ins++] = &e->leaf;
       }
       m.prog[m.n++] = {KAPY_EW_LD_GLOBAL, dst, slot, 0, 0, 0, KAPY_RN, 0.f};
+    } else if (e->ew == KAPY_EW_REDUCE_SUM || e->ew == KAPY_EW_REDUCE_MAX) {
+      m.prog[m.n++] = {e->ew, dst, src[0], 1, 0, 0, KAPY_RN, 0.f};
     } else {
       m.prog[m.n++] = {e->ew, dst, src[0], src[1], src[2], e->dtype, e->rmode, e->imm};
     }
     return m.reg[e.get()] = dst;
   }
-  // the chain as one program that stores into `out`
-  int run_chain(const std::shared_ptr<Expr> &e, const kapy_global *out) {
+  static bool is_reduce(const Expr &e) { return e.ew == KAPY_EW_REDUCE_SUM || e.ew == KAPY_EW_REDUCE_MAX; }
+  // the outermost reduce of the chain that `skip` does not exempt
+  template <class Skip>
+  Expr *find_reduce(const std::shared_ptr<Expr> &e, Skip skip) {
+    if (is_reduce(*e) && !skip(*e)) return e.get();
+    for (int k = 0; k < e->n_in; ++k)
+      if (Expr *r = find_reduce(e->in[k], skip)) return r;
+    return nullptr;
+  }
+  // runs a deferred reduce by itself (its operand computed first, then kapy_reduce): the node becomes a computed [rows x 1] tensor
+  int compute_reduce(const Op &op, Expr *r) {
+    Value operand;
+    operand.kind = Value::kTensor;
+    operand.lazy = r->in[0];
+    memset(&operand.g, 0, sizeof operand.g);
+    int rc = lib(op, kapy_mk_global(&operand.g, arena, 0, r->rows, r->cols, r->cols, 1, r->operand_dtype, 16));
+    if (rc == KAPY_OK && !(operand.lazy->ew == KAPY_EW_LD_GLOBAL && operand.lazy->n_in == 0)) rc = force(op, operand);
+    if (rc != KAPY_OK) return rc;
+    if (operand.lazy) operand.g = operand.lazy->leaf;
+    void *ptr = alloc((size_t)r->rows * dtype_bytes(r->operand_dtype));
+    if (!ptr) return fail_op(op, "register tensors of one program instance exceed the arena");
+    kapy_global g;
+    rc = lib(op, kapy_mk_global(&g, ptr, 0, r->rows, 1, 1, 1, r->operand_dtype, 256));
+    if (rc == KAPY_OK) rc = lib(op, kapy_reduce(&operand.g, &g, 1, r->ew == KAPY_EW_REDUCE_MAX ? 1 : 0, stream));
+    if (rc != KAPY_OK) return rc;
+    r->ew = KAPY_EW_LD_GLOBAL;
+    r->n_in = 0;
+    for (auto &p : r->in) p.reset();
+    r->leaf = g;
+    return KAPY_OK;
+  }
+  int run_program(const std::shared_ptr<Expr> &e, const kapy_global *out) {
     Emit m;
     const int r = emit(e, m);
     if (!m.ok) return fail(KAPY_ERR_UNSUPPORTED, "the deferred chain does not fit one program");
     m.prog[m.n++] = {KAPY_EW_ST_GLOBAL, 0, r, 0, 0, 0, KAPY_RN, 0.f};
     return kapy_elementwise(m.prog, m.n, m.ins, m.n_ins, out, stream);
+  }
+  // the chain as one program that stores into `out`.  Reduces stay inside the program when its result has their
+  // operand's shape (the row programs of kapy_elementwise: softmax, normalisations); the others, and all of them
+  // when that program is refused (rows too long, a width that is no multiple of 8, ...), run as kapy_reduce first.
+  int run_chain(const Op &op, const std::shared_ptr<Expr> &e, const kapy_global *out) {
+    const int32_t rows = out->end0 - out->start0, cols = out->end1 - out->start1;
+    while (Expr *r = find_reduce(e, [&](const Expr &x) { return x.rows == rows && x.cols == cols; })) {
+      int rc = compute_reduce(op, r);
+      if (rc != KAPY_OK) return rc;
+    }
+    int rc = run_program(e, out);
+    if (rc == KAPY_OK || !find_reduce(e, [](const Expr &) { return false; })) return rc;
+    while (Expr *r = find_reduce(e, [](const Expr &) { return false; })) {
+      rc = compute_reduce(op, r);
+      if (rc != KAPY_OK) return rc;
+    }
+    return run_program(e, out);
   }
   bool fits(const std::shared_ptr<Expr> &e) {
     Emit m;
@@ -627,7 +679,7 @@ struct Interp {
     if (!ptr) return fail_op(op, "register tensors of one program instance exceed the arena");
     kapy_global g;
     int rc = lib(op, kapy_mk_global(&g, ptr, 0, rows, cols, cols, 1, v.g.dtype, 256));
-    if (rc == KAPY_OK) rc = lib(op, run_chain(v.lazy, &g));
+    if (rc == KAPY_OK) rc = lib(op, run_chain(op, v.lazy, &g));
     if (rc != KAPY_OK) return rc;
     // every other holder of the same expression now reads the computed tensor as well
     v.lazy->ew = KAPY_EW_LD_GLOBAL;
@@ -884,7 +936,7 @@ struct Interp {
         if (!get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
         const kapy_global &sg = src->second.g;
         if (b.g.end0 - b.g.start0 == sg.end0 - sg.start0 && b.g.end1 - b.g.start1 == sg.end1 - sg.start1 && b.g.dtype == sg.dtype &&
-            run_chain(src->second.lazy, &b.g) == KAPY_OK)
+            run_chain(op, src->second.lazy, &b.g) == KAPY_OK)
           return KAPY_OK;
       }
       if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
@@ -907,7 +959,6 @@ struct Interp {
       return KAPY_OK;
     }
     if (n == "kapy.reduce") {
-      if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
       int kind = -1;
       for (const Op &inner : op.body) {
         if (inner.name == "arith.addf") kind = 0;
@@ -915,6 +966,31 @@ struct Interp {
       }
       if (kind < 0) return fail_op(op, "only addf and maximumf combiners are supported");
       int axis = op.attrs.count("axis") ? atoi(op.attrs.at("axis").c_str()) : 0;
+      // along axis 1 over a register tensor the reduce joins the deferred chain: followed by a broadcast back to the
+      // operand's shape it becomes an instruction of the program that consumes it
+      auto src = op.operands.empty() ? env.end() : env.find(op.operands[0]);
+      if (fuse && axis == 1 && !op.types.empty() && op.types.back().kind == Type::kTensor && src != env.end() &&
+          src->second.kind == Value::kTensor && (src->second.lazy || is_register_tensor(src->second.g))) {
+        const kapy_global &sg = src->second.g;
+        const Type &ty = op.types.back();
+        if (ty.shape[0] == sg.end0 - sg.start0 && ty.shape[1] == 1 && ty.dtype == sg.dtype) {
+          auto e = std::make_shared<Expr>();
+          e->ew = kind == 1 ? KAPY_EW_REDUCE_MAX : KAPY_EW_REDUCE_SUM;
+          e->n_in = 1;
+          e->in[0] = as_expr(src->second);
+          e->rows = sg.end0 - sg.start0; e->cols = sg.end1 - sg.start1; e->operand_dtype = sg.dtype;
+          if (fits(e)) {
+            r.kind = Value::kTensor;
+            r.lazy = e;
+            memset(&r.g, 0, sizeof r.g);
+            int rc = lib(op, kapy_mk_global(&r.g, arena, 0, e->rows, 1, 1, 1, ty.dtype, 16));
+            if (rc) return rc;
+            env[op.results[0]] = r;
+            return KAPY_OK;
+          }
+        }
+      }
+      if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
       int rc = lib(op, kapy_reduce(&a.g, &r.g, axis, kind, stream));
       if (rc) return rc;
       env[op.results[0]] = r;

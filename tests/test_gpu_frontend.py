@@ -90,8 +90,14 @@ def test_matmul_program_matches_oracle(ko, bm, bn, bk, way, acc, M, N, K):
     assert rel <= (3e-4 if acc == "f16" else 1e-6), rel
 
 
-def test_softmax_program_in_kapy_ops_matches_the_oracle_program(ko):
-    rows_per_warp, cols, warps, programs = 2, 256, 2, 3
+@pytest.mark.parametrize("cols", [256, 100])
+@pytest.mark.parametrize("fuse", ["1", "0"])
+def test_softmax_program_in_kapy_ops_matches_the_oracle_program(ko, monkeypatch, cols, fuse):
+    """Fused (the default), the ten ops between the load and the store are the oracle's softmax program itself: both reduces
+    are instructions of one row program.  A width that is no multiple of 8 is outside the row programs, so there the reduces run
+    as kapy_reduce and the arithmetic between them as three programs; KAPY_MLIR_FUSE=0 runs every op by itself."""
+    monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+    rows_per_warp, warps, programs = 2, 2, 3
     rows = rows_per_warp * warps * programs
     x = ko.fill_normal(rows * cols, ko.F16, 51, std=3.0)
     want = np.zeros(rows * cols, np.uint16)
@@ -100,7 +106,7 @@ def test_softmax_program_in_kapy_ops_matches_the_oracle_program(ko):
     dx, dout = to_dev(x), dev_zeros(rows * cols, 2, fill=0x7e00)
     kh.run_mlir(kp.softmax_program(rows_per_warp, cols, warps), [dx, dout, rows], [programs])
     sync()
-    assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # op by op in f32, one rounding to f16 at the end
+    assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # in f32, one rounding to f16 at the end
 
 
 def _gated_insts():

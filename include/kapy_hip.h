@@ -309,10 +309,12 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * tensors, math.exp / exp2 / log / log2 / sqrt / rsqrt / tanh / erf / absf / fma, kapy.fptofp, arith.extf / truncf,
  * kapy.splat, kapy.broadcast: kapy_elementwise; kapy.transpose: kapy_copy; kapy.reduce: kapy_reduce; kapy.matmul:
  * kapy_matmul; scf.for with iter_args).
- * A chain of elementwise ops (arith / math on tensors, casts, splats, tensor constants, broadcasts) over register
- * tensors is not run op by op: it stays deferred until an op of another kind, a loop's yield or a store needs it, and
+ * A chain of elementwise ops (arith / math on tensors, casts, splats, tensor constants, broadcasts, and the
+ * kapy.ld_global of a whole view that feeds them) is not run op by op: it stays deferred until an op of another kind, a loop's yield or a store needs it, and
  * then runs as ONE kapy_elementwise program (at most 8 distinct tensors read, 16 values, 48 instructions; a longer
- * chain is cut where it stops fitting), a kapy.st_global storing straight into its global view: the counterpart of
+ * chain is cut where it stops fitting), a kapy.st_global storing straight into its global view (after computing
+ * whatever deferred value still has to read memory the store overlaps); a kapy.reduce along axis 1 whose result is
+ * broadcast back to its operand's shape is an instruction of that program: the counterpart of
  * the reference compiling the ops of a function into one kernel body.  KAPY_MLIR_FUSE=0 in the environment runs
  * every op as a call of its own instead; results are the same bit for bit.
  * Warps run one after the other, so a program whose warps exchange data through shared memory between

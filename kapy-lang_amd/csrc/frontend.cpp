@@ -514,6 +514,7 @@ struct Expr {
   std::shared_ptr<Expr> in[3];
   int n_in = 0;
   kapy_global leaf;
+  bool global_leaf = false;  // the leaf is a view of the caller's memory (a deferred kapy.ld_global), which a later store may change
   // KAPY_EW_REDUCE_SUM / _MAX along axis 1: inside a program the result sits on every element of the row, so the node
   // can only be part of a program whose result has the operand's shape (rows x cols) and element type (operand_dtype)
   int32_t rows = 0, cols = 0, operand_dtype = 0;
@@ -570,6 +571,34 @@ struct Interp {
   bool is_register_tensor(const kapy_global &g) const {
     const char *p = (const char *)g.ptr;
     return p >= arena + kSharedArena && p < arena + kArena;
+  }
+  // [first, last] byte of a view (strides are positive: mk_global refuses others)
+  static void byte_range(const kapy_global &g, const char **lo, const char **hi) {
+    const int eb = dtype_bytes(g.dtype);
+    *lo = view_base(&g);
+    *hi = *lo + (int64_t(g.end0 - g.start0 - 1) * g.stride0 + int64_t(g.end1 - g.start1 - 1) * g.stride1 + 1) * eb - 1;
+  }
+  // does the chain read, through a deferred load, memory that a store into `dst` writes
+  bool reads_under(const std::shared_ptr<Expr> &e, const kapy_global &dst) {
+    if (e->ew == KAPY_EW_LD_GLOBAL && e->n_in == 0) {
+      if (!e->global_leaf) return false;
+      const char *a0, *a1, *b0, *b1;
+      byte_range(e->leaf, &a0, &a1);
+      byte_range(dst, &b0, &b1);
+      return a0 <= b1 && b0 <= a1;
+    }
+    for (int k = 0; k < e->n_in; ++k)
+      if (reads_under(e->in[k], dst)) return true;
+    return false;
+  }
+  // before a store into `dst`: every deferred value that still has to read that memory is computed now
+  int settle_readers(const Op &op, const kapy_global &dst) {
+    for (auto &kv : env)
+      if (kv.second.kind == Value::kTensor && kv.second.lazy && reads_under(kv.second.lazy, dst)) {
+        int rc = force(op, kv.second);
+        if (rc != KAPY_OK) return rc;
+      }
+    return KAPY_OK;
   }
   // the operand as an expression: deferred tensors as they are, computed ones as leaves
   std::shared_ptr<Expr> as_expr(const Value &v) {
@@ -679,13 +708,18 @@ struct Interp {
     if (!ptr) return fail_op(op, "register tensors of one program instance exceed the arena");
     kapy_global g;
     int rc = lib(op, kapy_mk_global(&g, ptr, 0, rows, cols, cols, 1, v.g.dtype, 256));
-    if (rc == KAPY_OK) rc = lib(op, run_chain(op, v.lazy, &g));
+    if (rc == KAPY_OK) {
+      // a deferred load by itself is the copy kapy.ld_global always was (any element type, any strides)
+      if (v.lazy->ew == KAPY_EW_LD_GLOBAL && v.lazy->n_in == 0) rc = lib(op, kapy_copy(&v.lazy->leaf, &g, nullptr, stream));
+      else rc = lib(op, run_chain(op, v.lazy, &g));
+    }
     if (rc != KAPY_OK) return rc;
     // every other holder of the same expression now reads the computed tensor as well
     v.lazy->ew = KAPY_EW_LD_GLOBAL;
     v.lazy->n_in = 0;
     for (auto &p : v.lazy->in) p.reset();
     v.lazy->leaf = g;
+    v.lazy->global_leaf = false;
     v.lazy.reset();
     v.g = g;
     for (auto &kv : env)
@@ -921,6 +955,27 @@ struct Interp {
       env[op.results[0]] = r;
       return KAPY_OK;
     }
+    if (n == "kapy.ld_global" && fuse && !op.types.empty() && op.types.back().kind == Type::kTensor) {
+      // a load of a whole view of the caller's memory joins the deferred chain: the program that needs the value reads the
+      // view itself.  A store that could change the view before then computes the value first (settle_readers).
+      Value src;
+      if (!get(op, 0, Value::kTensor, src)) return KAPY_ERR_INVALID;
+      const Type &ty = op.types.back();
+      const char *p = (const char *)src.g.ptr;
+      if (!(p >= arena && p < arena + kArena) && ty.shape[0] == src.g.end0 - src.g.start0 && ty.shape[1] == src.g.end1 - src.g.start1 &&
+          ty.dtype == src.g.dtype && ty.shape[0] > 0 && ty.shape[1] > 0 && src.g.stride0 > 0 && src.g.stride1 > 0) {
+        auto e = std::make_shared<Expr>();
+        e->leaf = src.g;
+        e->global_leaf = true;
+        r.kind = Value::kTensor;
+        r.lazy = e;
+        memset(&r.g, 0, sizeof r.g);
+        int rc = lib(op, kapy_mk_global(&r.g, arena, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 16));
+        if (rc) return rc;
+        env[op.results[0]] = r;
+        return KAPY_OK;
+      }
+    }
     if (n == "kapy.ld_global" || n == "kapy.ld_matrix" || n == "kapy.ld_shared") {
       if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
       int rc = lib(op, kapy_copy(&a.g, &r.g, nullptr, stream));
@@ -931,6 +986,11 @@ struct Interp {
     if (n == "kapy.st_global" || n == "kapy.st_shared" || n == "kapy.cp_async_global_to_shared") {
       // a deferred chain stores straight into a view of its own shape; anything else (padding, a program the
       // elementwise entry point refuses) goes through a register tensor as before
+      if (n == "kapy.st_global") {
+        if (!get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
+        int rc = settle_readers(op, b.g);
+        if (rc != KAPY_OK) return rc;
+      }
       auto src = op.operands.empty() ? env.end() : env.find(op.operands[0]);
       if (src != env.end() && src->second.kind == Value::kTensor && src->second.lazy) {
         if (!get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;

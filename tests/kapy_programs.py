@@ -267,6 +267,39 @@ def gated_program(rows_per_warp=4, cols=256, num_warps=2, dtype="f16"):
             body + "  }\n}\n")
 
 
+def aliasing_program(rows_per_warp=4, cols=128, num_warps=2, dtype="f16"):
+    """Stores into memory that earlier loads read: out = (x + y) * x with the values x had on entry, although x is overwritten
+    with y between the loads and the arithmetic's use; then x <- x + x in place (x now holding y)."""
+    t = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols])
+    body += """    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %gy = kapy.mk_global %y[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %sy = kapy.sv_global %gy[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %vx = kapy.ld_global %sx : {t}, #global> -> {t}, #values>
+    %vy = kapy.ld_global %sy : {t}, #global> -> {t}, #values>
+    %a = arith.addf %vx, %vy : {t}, #values>
+    kapy.st_global %vy, %sx : {t}, #values>, {t}, #global>
+    %b = arith.mulf %a, %vx : {t}, #values>
+    kapy.st_global %b, %so : {t}, #values>, {t}, #global>
+    %x2 = kapy.ld_global %sx : {t}, #global> -> {t}, #values>
+    %d = arith.addf %x2, %x2 : {t}, #values>
+    kapy.st_global %d, %sx : {t}, #values>, {t}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, t=t)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @aliasing_kernel(%x: !kapy.ptr<1>, %y: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" + body + "  }\n}\n")
+
+
 def scaled_transpose_program(tile=32, scale=0.5, dtype="f16"):
     """out[j, i] = x[i, j] * scale over tile x tile blocks, one block per program: ld_global, kapy.transpose, kapy.splat of
     a scalar constant, mulf, st_global."""

@@ -142,6 +142,23 @@ def test_chain_of_elementwise_ops_runs_as_one_program(ko, monkeypatch):
     assert np.array_equal(results[0], results[1])
 
 
+@pytest.mark.parametrize("fuse", ["1", "0"])
+def test_a_store_into_memory_that_deferred_loads_read(ko, monkeypatch, fuse):
+    """Loads join the deferred chain, so the program that needs a loaded value reads the caller's memory itself, later than the
+    load stands in the text.  A store into that memory in between must not change what the load saw."""
+    monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+    rows_per_warp, cols, warps, programs = 4, 128, 2, 2
+    rows = rows_per_warp * warps * programs
+    x, y = ko.fill_normal(rows * cols, ko.F16, 71), ko.fill_normal(rows * cols, ko.F16, 72)
+    dx, dy, dout = to_dev(x), to_dev(y), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.aliasing_program(rows_per_warp, cols, warps), [dx, dy, dout, rows], [programs])
+    sync()
+    xf, yf = x.view(np.float16), y.view(np.float16)
+    assert np.array_equal(to_host(dout, np.float16), (xf + yf) * xf)          # numpy rounds each f16 op once, as the program does
+    assert np.array_equal(to_host(dx, np.float16), yf + yf)
+    assert np.array_equal(to_host(dy, np.float16), yf)
+
+
 def test_fused_chain_is_one_kernel(ko):
     """With KAPY_EW_AUTO_SPECIALIZE=1 (read once per process, so in a process of its own) every program outside the hand-written
     kernels is compiled when first seen: the chain of eleven ops leaves exactly one compiled kernel behind, launched once per

@@ -4,8 +4,8 @@
 `python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]`
 
 A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM.
-The headline workload (BASELINE.json configs[1]) is the fused elementwise
-y = GELU_tanh(x*0.5 + bias) on fp16 8192x8192; the JSON line also carries every other BASELINE
+The headline workload (the configuration the headline metric is quoted on) is the fused elementwise
+y = GELU_tanh(x*0.5 + bias) on fp16 8192x8192; the JSON line also carries every other benchmark
 configuration under "other_workloads", each with its own roofline.  One JSON line on stdout.
 
 Timing: K launches bracketed by torch.cuda.synchronize() give ms_per_step / value; HIP events

@@ -300,6 +300,44 @@ def aliasing_program(rows_per_warp=4, cols=128, num_warps=2, dtype="f16"):
             "  kapy.func public @aliasing_kernel(%x: !kapy.ptr<1>, %y: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" + body + "  }\n}\n")
 
 
+def block_sum_program(rows_per_warp=4, block_cols=64, num_warps=2, dtype="f16"):
+    """out[r, 0:block_cols] = 0.25 + sum over the column blocks j of tanh(x[r, j*block_cols:(j+1)*block_cols]) * 0.5, accumulated
+    in f32 by an scf.for that carries the accumulator, rounded once at the end.  %cols is a run-time argument."""
+    t16, t32 = "tensor<%dx%dx%s" % (rows_per_warp, block_cols, dtype), "tensor<%dx%dxf32" % (rows_per_warp, block_cols)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, block_cols])
+    body += """    %half = arith.constant 0.5 : f32
+    %start = arith.constant dense<2.500000e-01> : {t32}, #values>
+    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %cols] [%cols, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{bc}_i32] [%c{bc}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{bc}_i32] : {dyn} -> {t16}, #global>
+    %halves = kapy.splat %half : f32 -> {t32}, #values>
+    %blocks = arith.divui %cols, %c{bc}_i32 : i32
+    %sum = scf.for %j = %c0_i32 to %blocks step %c1_i32 iter_args(%acc = %start) -> ({t32}, #values>)  : i32 {{
+      %c0 = arith.muli %j, %c{bc}_i32 : i32
+      %c1 = arith.addi %c0, %c{bc}_i32 : i32
+      %sx = kapy.sv_global %gx[%row0 : %row1, %c0 : %c1] : {dyn} -> {t16}, #global>
+      %v = kapy.ld_global %sx : {t16}, #global> -> {t16}, #values>
+      %vf = kapy.fptofp %v : {t16}, #values> to {t32}, #values>
+      %th = math.tanh %vf : {t32}, #values>
+      %sc = arith.mulf %th, %halves : {t32}, #values>
+      %next = arith.addf %acc, %sc : {t32}, #values>
+      scf.yield %next : {t32}, #values>
+    }}
+    %r = kapy.fptofp %sum {{rounding_mode = 1 : i32}} : {t32}, #values> to {t16}, #values>
+    kapy.st_global %r, %so : {t16}, #values>, {t16}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, bc=block_cols, dyn=dyn, t16=t16, t32=t32)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @block_sum_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32, %cols: i32) {\n" + body + "  }\n}\n")
+
+
 def scaled_transpose_program(tile=32, scale=0.5, dtype="f16"):
     """out[j, i] = x[i, j] * scale over tile x tile blocks, one block per program: ld_global, kapy.transpose, kapy.splat of
     a scalar constant, mulf, st_global."""

@@ -159,6 +159,29 @@ def test_a_store_into_memory_that_deferred_loads_read(ko, monkeypatch, fuse):
     assert np.array_equal(to_host(dy, np.float16), yf)
 
 
+def test_deferred_values_carried_by_a_loop(ko, monkeypatch):
+    """An scf.for whose body is a chain ending in the carried accumulator: the yield computes it once per iteration (one
+    program: load, cast, tanh, scale, add), the splat defined before the loop stays deferred across all of them.  Fused and
+    op-by-op runs agree bit for bit; both follow a numpy restatement with fp32 accumulation in the program's order."""
+    rows_per_warp, bc, warps, programs, blocks = 4, 64, 2, 2, 5
+    rows, cols = rows_per_warp * warps * programs, bc * blocks
+    x = ko.fill_normal(rows * cols, ko.F16, 81)
+    dx = to_dev(x)
+    results = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+        dout = dev_zeros(rows * bc, 2, fill=0x7e00)
+        kh.run_mlir(kp.block_sum_program(rows_per_warp, bc, warps), [dx, dout, rows, cols], [programs])
+        sync()
+        results.append(to_host(dout, np.float16, (rows, bc)))
+    assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
+    acc = np.full((rows, bc), 0.25, np.float32)
+    xf = x.view(np.float16).reshape(rows, cols).astype(np.float64)
+    for j in range(blocks):
+        acc = acc + (np.tanh(xf[:, j * bc:(j + 1) * bc]).astype(np.float32) * np.float32(0.5))
+    assert np.abs(results[0].astype(np.float64) - acc).max() <= 2e-3
+
+
 def test_fused_chain_is_one_kernel(ko):
     """With KAPY_EW_AUTO_SPECIALIZE=1 (read once per process, so in a process of its own) every program outside the hand-written
     kernels is compiled when first seen: the chain of eleven ops leaves exactly one compiled kernel behind, launched once per

@@ -267,7 +267,8 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
                 const int64_t shape[2], uint32_t *lane_values_out, void *stream);
 
 /* kapy.reduce with an addf / maximumf combiner along `axis` (Ops.td:441-457, ReduceOpToLLVM.cpp:51-172).
- * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`. */
+ * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`.  The elements themselves are folded, as the
+ * lowering does (no identity element joins them): a line of only -0 sums to -0; max orders -0 below +0 and a NaN wins. */
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream);
 
 /* Static plan of a workgroup's shared memory (lib/Analysis/AllocAnalysis.cpp:187-270): buffers whose live

@@ -120,7 +120,7 @@ __device__ __forceinline__ void copy8(float (&x)[8], const float (&y)[8]) {
 template <int CH, int THREADS, bool SUM, bool RAGGED>
 __device__ __forceinline__ float row_reduce(const float (&v)[CH][8], int32_t vec_per_row, int32_t width, float *red) {
   const int tid = threadIdx.x;
-  float acc = SUM ? 0.f : -__builtin_inff();
+  float acc = SUM ? -0.f : -__builtin_inff();
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     const int32_t jv = c * THREADS + tid;

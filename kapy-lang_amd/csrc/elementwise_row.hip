@@ -157,7 +157,7 @@ __global__ __launch_bounds__(THREADS) void norm_kernel(FusedRow p, int dtype) {
     for (int c = 0; c < CH; ++c) widen16x8(raw[c], dtype, f[c]);
     if (i + (int32_t)gridDim.x < p.rows) row_fetch<CH, THREADS, true>(p.x + (int64_t)(i + gridDim.x) * p.x_stride0 * 2, p.vec_per_row, raw);
     if (p.centre) {
-      float sum = 0.f;
+      float sum = -0.f;  // the identity of addition: a row of only -0 has mean -0
 #pragma unroll
       for (int c = 0; c < CH; ++c)
         if (c * THREADS + (int)threadIdx.x < p.vec_per_row) sum += ((f[c][0] + f[c][1]) + (f[c][2] + f[c][3])) + ((f[c][4] + f[c][5]) + (f[c][6] + f[c][7]));

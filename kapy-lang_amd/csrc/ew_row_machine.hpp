@@ -148,7 +148,7 @@ __device__ __forceinline__ void row_step(const StackProgram &P, const PostOp &I,
   const int k = (I.slot >> 8) & 3;
   if (I.op == KAPY_EW_REDUCE_SUM || I.op == KAPY_EW_REDUCE_MAX) {  // row value D -> per-row value k
     const bool sum = I.op == KAPY_EW_REDUCE_SUM;
-    float acc = sum ? 0.f : -__builtin_inff();
+    float acc = sum ? -0.f : -__builtin_inff();  // -0: the identity of addition, a row of only -0 sums to -0
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       if (c * THREADS + tid < P.vec_per_row) {

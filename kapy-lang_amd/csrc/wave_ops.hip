@@ -45,12 +45,14 @@ __device__ __forceinline__ float combine(float a, float b, int kind) {
   return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b);
 }
 
+// A sum starts from -0, the identity of IEEE addition (-0 + x = x for every x, -0 included): the result is that of folding
+// the elements themselves, as ReduceOpToLLVM.cpp:60-101 does, and a line of only -0 sums to -0.
 // One wavefront per kept index: lanes stride over the reduced axis, then 6 butterfly rounds.
 __global__ __launch_bounds__(256) void reduce_wave_kernel(ReduceParams p) {
   const int lane = threadIdx.x & 63;
   const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (keep >= p.n_keep) return;
-  float acc = p.kind == 0 ? 0.f : -__builtin_inff();
+  float acc = p.kind == 0 ? -0.f : -__builtin_inff();
   for (int32_t r = lane; r < p.n_red; r += 64) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + r * p.s_red), p.kind);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p) {
   if (keep >= p.n_keep) return;
   const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * 2);
   const int32_t vecs = p.n_red / 8;
-  float acc = KIND == 0 ? 0.f : -__builtin_inff();
+  float acc = KIND == 0 ? -0.f : -__builtin_inff();
   constexpr int U = 4;
   int32_t v = lane;
   for (; v + 64 * (U - 1) < vecs; v += 64 * U) {
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(512) void reduce_cols_vec_kernel(ReduceParams p) {
   const int64_t keep0 = (int64_t)blockIdx.x * 32 + cl * 8;
   float acc[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = KIND == 0 ? 0.f : -__builtin_inff();
+  for (int e = 0; e < 8; ++e) acc[e] = KIND == 0 ? -0.f : -__builtin_inff();
   for (int32_t r = rg; r < p.n_red; r += 128) {
     float f[8];
     widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(p.src + (r * p.s_red + keep0) * 2)), f);
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(512) void reduce_cols_vec_kernel(ReduceParams p) {
   for (int e = 0; e < 8; ++e) part[rg][cl * 8 + e] = acc[e];
   __syncthreads();
   if (threadIdx.x < 32) {
-    float t = KIND == 0 ? 0.f : -__builtin_inff();
+    float t = KIND == 0 ? -0.f : -__builtin_inff();
     for (int g = 0; g < 128; ++g) t = combine(t, part[g][threadIdx.x], KIND);
     store_from_f32(p.dst, p.dst_dtype, ((int64_t)blockIdx.x * 32 + threadIdx.x) * p.d_keep, t);
   }
@@ -147,7 +149,7 @@ __global__ __launch_bounds__(512) void reduce_cols_vec_kernel(ReduceParams p) {
 __global__ __launch_bounds__(256) void reduce_lane_kernel(ReduceParams p) {
   const int64_t keep = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (keep >= p.n_keep) return;
-  float acc = p.kind == 0 ? 0.f : -__builtin_inff();
+  float acc = p.kind == 0 ? -0.f : -__builtin_inff();
   for (int32_t r = 0; r < p.n_red; ++r) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + r * p.s_red), p.kind);
   store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
 }

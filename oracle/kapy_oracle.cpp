@@ -692,13 +692,13 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
       const int64_t n_keep = I.b == 1 ? o0 : o1, n_red = I.b == 1 ? o1 : o0;
 #pragma omp parallel for schedule(static)
       for (int64_t q = 0; q < n_keep; ++q) {
-        long double acc = I.op == EW_REDUCE_SUM ? 0.0L : -std::numeric_limits<long double>::infinity();
+        long double acc = I.op == EW_REDUCE_SUM ? -0.0L : -std::numeric_limits<long double>::infinity();
         bool nan = false;
         for (int64_t r = 0; r < n_red; ++r) {
           const double v = I.b == 1 ? src[q * o1 + r] : src[r * o1 + q];
           if (std::isnan(v)) nan = true;
           if (I.op == EW_REDUCE_SUM) acc += v;
-          else if (v > acc) acc = v;
+          else if (v > acc || (v == 0.0 && acc == 0.0L && !std::signbit(v))) acc = v;  // maximumf orders -0 below +0
         }
         const double res = nan ? qnan : round_to((double)acc, dt);
         for (int64_t r = 0; r < n_red; ++r) reg[d][I.b == 1 ? q * o1 + r : r * o1 + q] = res;
@@ -888,12 +888,14 @@ int ko_reduce(const ko_global *src, const ko_global *dst, int axis, int kind) {
   if (axis == 0 ? (extent0(dst) != 1 || extent1(dst) != s1) : (extent1(dst) != 1 || extent0(dst) != s0)) return -1;
 #pragma omp parallel for schedule(static)
   for (int64_t o = 0; o < outer; ++o) {
-    double acc = kind == 0 ? 0.0 : -std::numeric_limits<double>::infinity();
+    double acc = kind == 0 ? -0.0 : -std::numeric_limits<double>::infinity();  // -0: identity of addition, = folding the elements themselves (ReduceOpToLLVM.cpp:60-101)
     for (int64_t t = 0; t < inner; ++t) {
       int64_t i = axis == 0 ? t : o, j = axis == 0 ? o : t;
       double v = ko_decode(src->ptr, src->dtype, elem_offset(src, i, j));
       if (kind == 0) acc += v;
-      else acc = (std::isnan(v) || std::isnan(acc)) ? std::numeric_limits<double>::quiet_NaN() : std::max(acc, v);
+      else if (std::isnan(v) || std::isnan(acc)) acc = std::numeric_limits<double>::quiet_NaN();
+      else if (v == 0.0 && acc == 0.0) acc = (std::signbit(v) && std::signbit(acc)) ? -0.0 : 0.0;  // maximumf orders -0 below +0
+      else acc = std::max(acc, v);
     }
     int64_t i = axis == 0 ? 0 : o, j = axis == 0 ? o : 0;
     ko_encode(dst->ptr, dst->dtype, elem_offset(dst, i, j), acc, KO_RN);

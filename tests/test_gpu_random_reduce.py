@@ -72,6 +72,57 @@ def test_random_reduce(ko, seed):
     assert np.all(np.abs(g - w) <= bound), "%s: result %d is %r, oracle %r, bound %g" % (describe, worst, g[worst], w[worst], bound[worst])
 
 
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16, kh.F32])
+@pytest.mark.parametrize("m,n,axis", [(64, 1024, 1), (16, 520, 1), (300, 128, 0), (1024, 64, 0), (8, 40, 1), (33, 33, 0)])
+def test_reduce_of_lines_with_nan_infinities_and_signed_zeros(ko, dtype, m, n, axis):
+    """Lines holding a NaN, +inf, -inf, only -0, and -0 next to +0 under negative values: max and sum treat them as the ops they
+    fold with do (maximumf: NaN wins, -0 below +0; addf: inf - inf is NaN).  Bit-exact for max and for the special results."""
+    rng = np.random.RandomState(m * 131 + n)
+    x = rng.normal(0, 1, (m, n)).astype(np.float32)
+    lines = x if axis == 1 else x.T                  # a view: line k is reduced to result k
+    lines[1, 3] = np.nan
+    lines[2, :] = -0.0
+    lines[3, 5] = np.inf
+    lines[4, 6], lines[4, 7] = np.inf, -np.inf
+    lines[5, 7] = -np.inf
+    lines[6, :] = -np.abs(lines[6, :]) - 1
+    lines[6, 1], lines[6, 2] = -0.0, 0.0
+    lines[7, :] = -np.abs(lines[7, :]) - 1
+    lines[7, 1], lines[7, 2] = 0.0, -0.0
+    store = np.ascontiguousarray((x.view(np.uint32) >> 16).astype(np.uint16) if dtype == kh.BF16 else
+                                 x.astype(np.float16).view(np.uint16) if dtype == kh.F16 else x.view(np.uint32))
+    om, on = (m, 1) if axis == 1 else (1, n)
+    dx = to_dev(store)
+    for kind in (0, 1):
+        want = np.zeros(om * on, np.uint32)
+        assert ko.lib().ko_reduce(C.byref(ko.mk_global(store, m, n, n, 1, dtype)), C.byref(ko.mk_global(want, om, on, 1, om, ko.F32)), axis, kind) == 0
+        dd = to_dev(np.zeros(om * on, np.uint32))
+        kh.reduce(dglobal(dx, m, n, n, 1, dtype), dglobal(dd, om, on, 1, om, kh.F32), axis, kind)
+        sync()
+        got = to_host(dd, np.uint32)
+        gf, wf = got.view(np.float32), want.view(np.float32)
+        assert np.array_equal(np.isnan(gf), np.isnan(wf)) and np.isnan(wf[1]) and (kind == 1 or np.isnan(wf[4]))
+        exact = ~np.isnan(wf) & (~np.isfinite(wf) | (wf == 0) | (kind == 1))
+        assert np.array_equal(got[exact], want[exact]), (kind, np.flatnonzero(exact & (got != want))[:5])
+        assert np.allclose(gf[~np.isnan(wf) & ~exact], wf[~np.isnan(wf) & ~exact], rtol=1e-5, atol=1e-3)
+        if axis == 1 and n % 8 == 0:
+            # the same reduce as an instruction of a row program (its result on every element of the row, in the row's type)
+            prog = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX if kind else kh.EW_REDUCE_SUM, dst=1, a=0, b=1),
+                    dict(op=kh.EW_ST_GLOBAL, a=1)]
+            pw = np.zeros(m * n, store.dtype)
+            assert ko.elementwise(ko.program(prog), [ko.mk_global(store, m, n, n, 1, dtype)], ko.mk_global(pw, m, n, n, 1, dtype)) == 0
+            dp = to_dev(np.zeros(m * n, store.dtype))
+            kh.elementwise(kh.program(prog), [dglobal(dx, m, n, n, 1, dtype)], dglobal(dp, m, n, n, 1, dtype))
+            sync()
+            pg = to_host(dp, store.dtype)
+            pgf, pwf = ko.decode(pg.view(VALUE[dtype]), dtype), ko.decode(pw.view(VALUE[dtype]), dtype)
+            assert np.array_equal(np.isnan(pgf), np.isnan(pwf))
+            exact = ~np.isnan(pwf) & (~np.isfinite(pwf) | (pwf == 0) | (kind == 1))
+            assert np.array_equal(pg[exact], pw[exact]), (kind, np.flatnonzero(exact & (pg != pw))[:5])
+            rest = ~np.isnan(pwf) & ~exact
+            assert np.all(np.abs(pgf[rest] - pwf[rest]) <= 2 * EPS[dtype] * np.abs(pwf[rest]) + 1e-3)
+
+
 @pytest.mark.parametrize("seed", range(32))
 def test_random_batched_copy(ko, seed):
     """A b x h grid of tiles moved between two 4-D layouts (any of the two orders of the grid axes on either side), with or

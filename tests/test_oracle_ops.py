@@ -207,6 +207,24 @@ def test_reduce_vs_numpy(ko):
     assert rc == 0 and np.array_equal(out.ravel(), x.astype(np.float64).sum(axis=1).astype(np.float32))
 
 
+def test_reduce_max_orders_signed_zeros_and_propagates_nan(ko):
+    """kapy.reduce with a maximumf combiner inherits arith.maximumf's order (-0 below +0, whichever comes first) and its NaN
+    propagation; a sum of infinities of both signs is NaN.  Fixed by the definition of the ops, not by the implementation."""
+    rows = np.array([[-1.0, -0.0, 0.0, -2.0],        # +0 after -0
+                     [-1.0, 0.0, -0.0, -2.0],        # +0 before -0
+                     [-0.0, -0.0, -0.0, -0.0],       # only -0
+                     [1.0, np.nan, 3.0, -np.inf],
+                     [-np.inf, np.inf, 1.0, 2.0]], np.float32)
+    mx, sm = np.zeros((5, 1), np.float32), np.zeros((5, 1), np.float32)
+    g = ko.mk_global(rows, 5, 4, 4, 1, ko.F32)
+    assert ko.lib().ko_reduce(C.byref(g), C.byref(ko.mk_global(mx, 5, 1, 1, 1, ko.F32)), 1, 1) == 0
+    assert ko.lib().ko_reduce(C.byref(g), C.byref(ko.mk_global(sm, 5, 1, 1, 1, ko.F32)), 1, 0) == 0
+    assert mx[0, 0] == 0 and not np.signbit(mx[0, 0]) and mx[1, 0] == 0 and not np.signbit(mx[1, 0])
+    assert mx[2, 0] == 0 and np.signbit(mx[2, 0])
+    assert np.isnan(mx[3, 0]) and mx[4, 0] == np.inf
+    assert np.isnan(sm[3, 0]) and np.isnan(sm[4, 0]) and sm[0, 0] == -3.0
+
+
 def test_gemm_timing_baseline_agrees_with_checker(ko):
     M = N = K = 96
     a = ko.fill_uniform(M * K, ko.BF16, 0, 0).reshape(M, K)

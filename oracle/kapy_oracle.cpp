@@ -531,8 +531,9 @@ void ko_change_tile(const void *lane_values, const ko_fragments *src, const ko_f
       int64_t sl, si;
       ko_change_source(src, dst, shape, lane, iv, &sl, &si);
       char *o = (char *)out_lane_values + (lane * nd + iv) * bytes;
-      // A result layout larger than the tensor names elements the source does not hold; the select
-      // chain of ChangeOpToLLVM.cpp:60-78 then matches no source iv and the value stays the zero init.
+      // A result layout larger than the tensor names positions past the tensor's edge, which the source does not
+      // hold: the select chain of ChangeOpToLLVM.cpp:50-78 then matches no source iv and keeps its first candidate,
+      // whatever that lane holds.  No consumer reads such a position; here it is defined as zero.
       if (sl < 0 || sl >= warp_size || si < 0 || si >= ns) std::memset(o, 0, bytes);
       else std::memcpy(o, (const char *)lane_values + (sl * ns + si) * bytes, bytes);
     }

@@ -8,10 +8,18 @@ The headline workload (the configuration the headline metric is quoted on) is th
 y = GELU_tanh(x*0.5 + bias) on fp16 8192x8192; the JSON line also carries every other benchmark
 configuration under "other_workloads", each with its own roofline.  One JSON line on stdout.
 
+Inputs are the ones each configuration states, generated on the host by the seeded counter-based generators of
+the CPU checker (fp64, rounded once to the storage type) and uploaded: the GPU and the checker see the same bytes.
+Before a workload is timed, one launch on the timed buffers is compared with the checker (sampled rows / blocks for
+the large shapes, the tolerance of the configuration): a workload that fails is not timed and is reported as failed.
+
 Timing: K launches bracketed by torch.cuda.synchronize() give ms_per_step / value; HIP events
 recorded on the stream the kernels are launched on (torch's current stream, whose handle is
 passed to the C ABI) give the per-launch duration used for roofline.achieved.  Memory-bound
 workloads rotate over buffer sets larger than the 256 MB Infinity Cache so the rate is HBM's.
+
+cpu_baseline: the same workload (or a stated slice of it) through the host implementations written for speed in
+oracle/kapy_baseline.cpp, over all the host threads this process may use, in the same run.
 """
 import argparse
 import ctypes as C
@@ -22,12 +30,19 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "kapy-lang_amd", "python"))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f8": 5000.0}
-
+FROB_TOL = 1e-3        # GEMMs: relative Frobenius error against the fp64-accumulated checker
+ULP_TOL = 2            # elementwise: units in the last place of the 16-bit result
+CPU_SECONDS = 2.0      # wall time each cpu_baseline leg repeats its workload for
 
 PREWARM_S = 0.25  # untimed launches before the W warm-up steps: the GPU clock needs ~0.2 s of load to settle
+
+
+class CheckFailed(Exception):
+    pass
 
 
 def _events(fn, steps, warmup):
@@ -66,53 +81,151 @@ def _roof_hbm(bytes_per_launch, ev_ms, key=None):
             "traffic": MEASURED_TRAFFIC.get(key)}
 
 
-def _roof_mfma(flops, ev_ms, kind):
+def _roof_mfma(flops, ev_ms, kind, key=None):
     a = flops / (ev_ms * 1e-3) / 1e12
     p = MFMA_PEAK_TFLOPS[kind]
-    return {"bound": "mfma", "achieved": round(a, 1), "peak": p, "unit": "TFLOP/s", "frac": round(a / p, 4), "traffic": None}
+    return {"bound": "mfma", "achieved": round(a, 1), "peak": p, "unit": "TFLOP/s", "frac": round(a / p, 4), "traffic": MEASURED_TRAFFIC.get(key)}
 
 
-def bench_gelu(kh, steps, warmup):
+# ---------------------------------------------------------------- seeded inputs (host-generated, cached on the device)
+_host_cache, _dev_cache = {}, {}
+
+
+def _host(kind, n, dtype, seed, stream=0, **kw):
+    """A seeded host array from the checker's generators; kept, because several workloads share the large ones."""
+    import ko
+    key = (kind, n, dtype, seed, stream, tuple(sorted(kw.items())))
+    if key not in _host_cache:
+        if kind == "normal":
+            _host_cache[key] = ko.fill_normal(n, dtype, seed, stream, kw.get("mean", 0.0), kw.get("std", 1.0))
+        elif kind == "uniform":
+            _host_cache[key] = ko.fill_uniform(n, dtype, seed, stream, kw.get("lo", -1.0), kw.get("hi", 1.0))
+        else:
+            _host_cache[key] = ko.fill_bits16(n, seed, stream)
+    return _host_cache[key]
+
+
+def _dev(kind, n, dtype, seed, stream=0, **kw):
+    import numpy as np
     import torch
+    key = (kind, n, dtype, seed, stream, tuple(sorted(kw.items())))
+    if key not in _dev_cache:
+        a = _host(kind, n, dtype, seed, stream, **kw)
+        _dev_cache[key] = torch.from_numpy(a.view({1: np.uint8, 2: np.int16, 4: np.int32}[a.itemsize])).cuda()
+    return _dev_cache[key]
+
+
+def _upload(a):
+    import numpy as np
+    import torch
+    a = np.ascontiguousarray(a)
+    return torch.from_numpy(a.view({1: np.uint8, 2: np.int16, 4: np.int32}[a.itemsize]).reshape(-1)).cuda()
+
+
+def _download(t, np_dtype, shape):
+    return t.cpu().numpy().view(np_dtype).reshape(shape)
+
+
+def _line16(v):
+    """16-bit float patterns on the monotone integer line (for ulp distances)."""
+    import numpy as np
+    v = v.astype(np.int32)
+    return np.where(v & 0x8000, -(v & 0x7FFF), v & 0x7FFF)
+
+
+def _sample_rows(n, count):
+    step = n // count
+    return [(k * step + (7 * k) % step) % n for k in range(count)]
+
+
+def _cpu_repeat(fn, work_per_call, unit_scale, unit, sample):
+    """Time fn() repeatedly for about CPU_SECONDS (after one warm-up call)."""
+    import ko
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > CPU_SECONDS:
+            break
+    return {"value": round(work_per_call * reps / dt / unit_scale, 3), "unit": unit, "cores": ko.lib().ko_num_threads(), "kind": "port",
+            "sample": "%s; %d repetitions in %.1f s" % (sample, reps, dt)}
+
+
+# ---------------------------------------------------------------- memory-bound workloads
+def bench_gelu(kh, steps, warmup, cpu):
+    """C2: x fp16 8192x8192 normal(0,1) seed 0, bias fp16 [8192] normal(0,1) seed 1 broadcast along rows, scale 0.5."""
+    import numpy as np
+    import torch
+    import ko
     n, sets = 8192, 4
-    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    ys = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    bias = torch.randn(n, device="cuda", dtype=torch.float16)
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]       # set 0 is the configuration's x; the others rotate past the cache
+    ys = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    bias = _dev("normal", n, ko.F16, 1)
     prog = kh.gelu_program(kh.F16, 0.5)
     gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
     gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
     gb = kh.mk_global(bias.data_ptr(), 1, n, n, 1, kh.F16)
+    # gate: 32 rows of the result against the checker
+    kh.elementwise(prog, [gx[0], gb], gy[0])
+    torch.cuda.synchronize()
+    hx, hb = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n), _host("normal", n, ko.F16, 1)
+    rows = _sample_rows(n, 32)
+    got = _download(ys[0], np.uint16, (n, n))[rows]
+    xr, want = np.ascontiguousarray(hx[rows]), np.zeros((len(rows), n), np.uint16)
+    assert ko.elementwise(ko.gelu_program(), [ko.mk_global(xr, len(rows), n, n, 1, ko.F16), ko.mk_global(hb, 1, n, n, 1, ko.F16)],
+                          ko.mk_global(want, len(rows), n, n, 1, ko.F16)) == 0
+    worst = int(np.abs(_line16(got) - _line16(want)).max())
+    if worst > ULP_TOL:
+        raise CheckFailed("gelu: %d ulp against the checker" % worst)
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gb], gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2 + n * 2
-    return {"workload": "C2 gelu_tanh(x*0.5+bias) fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "gelu"), "kernel": "affine_act_cols_kernel"}
+    out = {"workload": "C2 gelu_tanh(x*0.5+bias) fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "gelu"), "kernel": "affine_act_cols_kernel",
+           "inputs": "x normal(0,1) seed 0, bias normal(0,1) seed 1, scale 0.5 (host-generated, as the configuration states)",
+           "checked": True, "check": "32 rows of the timed result against the checker: max %d ulp (tolerance %d)" % (worst, ULP_TOL)}
+    if cpu:
+        hy = np.zeros((n, n), np.uint16)
+        out["cpu_baseline"] = _cpu_repeat(lambda: ko.lib().ko_baseline_gelu_f16(hx.ctypes.data, hb.ctypes.data, 0.5, hy.ctypes.data, n, n, n),
+                                          nbytes, 1e9, "GB/s", "the whole 8192x8192 workload, fused fp32 vector loop")
+    return out
 
 
-def bench_copy(kh, steps, warmup):
+def bench_copy(kh, steps, warmup, cpu):
     """Plain row-major copy of the headline shape: the practical HBM ceiling the other kernels are read against,
     and the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters."""
+    import numpy as np
     import torch
+    import ko
     n, sets = 8192, 4
-    xs = [torch.randint(-32768, 32767, (n, n), device="cuda", dtype=torch.int16) for _ in range(sets)]
-    ys = [torch.empty(n, n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    xs = [_dev("bits16", n * n, ko.F16, 0, k) for k in range(sets)]
+    ys = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
     gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
     gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
+    kh.copy(gx[0], gy[0])
+    torch.cuda.synchronize()
+    if not torch.equal(xs[0], ys[0]):
+        raise CheckFailed("copy: result differs from the source")
     wall, ev = _events(lambda i: kh.copy(gx[i % sets], gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
     return {"workload": "copy fp16 8192x8192 (ld_global -> st_global, no transpose)", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel",
+            "inputs": "uniform random 16-bit patterns seed 0", "checked": True, "check": "whole result bit-equal to the source"}
 
 
-def bench_add(kh, steps, warmup, op="add"):
+def bench_add(kh, steps, warmup, cpu, op="add"):
     """z = x + y in fp16 (the reference's elementwise_add.mlir fixture at the headline shape), a plain binary program,
     served by the fused affine kernel; op="expr": z = x*y + x with both roundings, a program outside the fused chains,
     served by the in-register stack machine; op="expr_compiled": the same program after kapy_elementwise_specialize has
     compiled it to a kernel of its own; op="swiglu": z = silu(x) * y in fp32 from fp16 operands (ten ops, x used twice), compiled."""
+    import numpy as np
     import torch
+    import ko
     n, sets = 8192, 3
-    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    ys = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    zs = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]
+    ys = [_dev("normal", n * n, ko.F16, 0, 3 - k) for k in range(sets)]
+    zs = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
     g = lambda t: kh.mk_global(t.data_ptr(), n, n, n, 1, kh.F16)
     gx, gy, gz = [g(t) for t in xs], [g(t) for t in ys], [g(t) for t in zs]
     insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1)]
@@ -125,9 +238,22 @@ def bench_add(kh, steps, warmup, op="add"):
                   dict(op=kh.EW_FPTOFP, dst=2, a=2, dtype=kh.F16, rmode=kh.RN)]
     else:
         insts += [dict(op=kh.EW_MULF, dst=2, a=0, b=1), dict(op=kh.EW_ADDF, dst=2, a=2, b=0)]
-    prog = kh.program(insts + [dict(op=kh.EW_ST_GLOBAL, a=2)])
+    insts += [dict(op=kh.EW_ST_GLOBAL, a=2)]
+    prog = kh.program(insts)
     if op in ("expr_compiled", "swiglu"):
         kh.elementwise_specialize(prog, [gx[0], gy[0]], gz[0])
+    kh.elementwise(prog, [gx[0], gy[0]], gz[0])
+    torch.cuda.synchronize()
+    rows = _sample_rows(n, 16)
+    hx, hy = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n), _host("normal", n * n, ko.F16, 0, 3).reshape(n, n)
+    xr, yr, want = np.ascontiguousarray(hx[rows]), np.ascontiguousarray(hy[rows]), np.zeros((len(rows), n), np.uint16)
+    m = len(rows)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(xr, m, n, n, 1, ko.F16), ko.mk_global(yr, m, n, n, 1, ko.F16)], ko.mk_global(want, m, n, n, 1, ko.F16)) == 0
+    got = _download(zs[0], np.uint16, (n, n))[rows]
+    worst = int(np.abs(_line16(got) - _line16(want)).max())
+    tol = ULP_TOL if op == "swiglu" else 0     # add / mul: exactly rounded ops, bit-exact
+    if worst > tol:
+        raise CheckFailed("%s: %d ulp against the checker" % (op, worst))
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gy[i % sets]], gz[i % sets]), steps, warmup)
     nbytes = 3 * n * n * 2
     name = {"add": "elementwise_add fixture: z = x + y fp16 8192x8192", "expr": "z = x*y + x (two roundings) fp16 8192x8192",
@@ -135,177 +261,377 @@ def bench_add(kh, steps, warmup, op="add"):
             "swiglu": "z = silu(x)*y fp16 8192x8192 in fp32, compiled at run time"}[op]
     kernel = {"add": "affine_act_kernel", "expr": "stack_kernel_narrow"}.get(op, "kapy_ew_flat_<hash> (compiled at run time)")
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev, op if op != "expr" else None), "kernel": kernel}
+            "roofline": _roof_hbm(nbytes, ev, op if op != "expr" else None), "kernel": kernel, "inputs": "x, y normal(0,1), seeded",
+            "checked": True, "check": "16 rows against the checker: max %d ulp (tolerance %d)" % (worst, tol)}
 
 
-def bench_gelu_transposed(kh, steps, warmup):
+def bench_gelu_transposed(kh, steps, warmup, cpu):
     """y = gelu_tanh(x^T*0.5 + bias): the C3a transpose fused with the C2 chain - x is read through a view with swapped
     strides - compiled at run time onto the tiled skeleton (64 x 64 tiles, the column-major operand staged through LDS)."""
+    import numpy as np
     import torch
+    import ko
     n, sets = 8192, 4
-    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    ys = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    bias = torch.randn(n, device="cuda", dtype=torch.float16)
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]
+    ys = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    bias = _dev("normal", n, ko.F16, 1)
     gx = [kh.mk_global(x.data_ptr(), n, n, 1, n, kh.F16) for x in xs]       # element (i, j) of the view is x[j, i]
     gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
     gb = kh.mk_global(bias.data_ptr(), 1, n, n, 1, kh.F16)
     prog = kh.gelu_program(kh.F16, 0.5)
     kh.elementwise_specialize(prog, [gx[0], gb], gy[0])
+    kh.elementwise(prog, [gx[0], gb], gy[0])
+    torch.cuda.synchronize()
+    hx, hb = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n), _host("normal", n, ko.F16, 1)
+    rows = _sample_rows(n, 16)
+    xr = np.ascontiguousarray(hx[:, rows].T)     # row i of the view is column i of x
+    want = np.zeros((len(rows), n), np.uint16)
+    assert ko.elementwise(ko.gelu_program(), [ko.mk_global(xr, len(rows), n, n, 1, ko.F16), ko.mk_global(hb, 1, n, n, 1, ko.F16)],
+                          ko.mk_global(want, len(rows), n, n, 1, ko.F16)) == 0
+    worst = int(np.abs(_line16(_download(ys[0], np.uint16, (n, n))[rows]) - _line16(want)).max())
+    if worst > ULP_TOL:
+        raise CheckFailed("gelu_transposed: %d ulp against the checker" % worst)
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets], gb], gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2 + n * 2
     return {"workload": "gelu_tanh(x^T*0.5+bias) fp16 8192x8192: transpose fused with the elementwise chain, compiled at run time",
             "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev), "kernel": "kapy_ew_flat_<hash> (tiled; compiled at run time)"}
+            "roofline": _roof_hbm(nbytes, ev), "kernel": "kapy_ew_flat_<hash> (tiled; compiled at run time)", "inputs": "as C2, x read through swapped strides",
+            "checked": True, "check": "16 rows against the checker: max %d ulp (tolerance %d)" % (worst, ULP_TOL)}
 
 
-def bench_reduce(kh, steps, warmup):
+def bench_reduce(kh, steps, warmup, cpu):
     """kapy.reduce (sum along rows) of the headline shape: the first adjacent op after the hot path proper."""
+    import numpy as np
     import torch
+    import ko
     n, sets = 8192, 4
-    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]
     y = torch.empty(n, device="cuda", dtype=torch.float32)
     gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
     gy = kh.mk_global(y.data_ptr(), n, 1, 1, n, kh.F32)
+    kh.reduce(gx[0], gy, 1, 0)
+    torch.cuda.synchronize()
+    hx = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n)
+    want = hx.view(np.float16).astype(np.float64).sum(axis=1)
+    err = float(np.abs(y.cpu().numpy().astype(np.float64) - want).max())
+    if err > 2e-3:   # fp32 accumulation of 8192 values of magnitude ~1
+        raise CheckFailed("reduce: max abs error %g" % err)
     wall, ev = _events(lambda i: kh.reduce(gx[i % sets], gy, 1, 0), steps, warmup)
     nbytes = n * n * 2 + n * 4
     return {"workload": "reduce_sum axis=1 fp16 8192x8192 -> f32 [8192x1]", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "reduce_rows_vec_kernel"}
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "reduce_rows_vec_kernel",
+            "inputs": "x normal(0,1) seed 0", "checked": True, "check": "every row sum against fp64: max abs error %.2e" % err}
 
 
-def bench_rowwise(kh, steps, warmup, which):
+def bench_rowwise(kh, steps, warmup, cpu, which):
     """Row-wise fusion of kapy.reduce with its elementwise neighbours at the headline shape: softmax or layer norm of
     every row in one pass over HBM (one read of x, one write of y; gamma and beta stay in cache)."""
+    import numpy as np
     import torch
+    import ko
     n, sets = 8192, 4
-    xs = [torch.randn(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    ys = [torch.empty(n, n, device="cuda", dtype=torch.float16) for _ in range(sets)]
-    gamma, beta = torch.ones(n, device="cuda", dtype=torch.float16), torch.zeros(n, device="cuda", dtype=torch.float16)
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]
+    ys = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    gamma, beta = _dev("normal", n, ko.F16, 2, 0, mean=1.0, std=0.1), _dev("normal", n, ko.F16, 2, 1, std=0.1)
     g = lambda t: kh.mk_global(t.data_ptr(), n, n, n, 1, kh.F16)
     row = lambda t: kh.mk_global(t.data_ptr(), 1, n, n, 1, kh.F16)
     gx, gy = [g(t) for t in xs], [g(t) for t in ys]
+    hextra = []
     if which == "softmax":
-        prog, extra = kh.program(kh.softmax_insts(kh.F16)), []
+        insts, extra = kh.softmax_insts(kh.F16), []
     elif which == "l2norm_compiled":   # x / |x| per row: a row program without a hand-written kernel, compiled at run time
         f32 = dict(op=kh.EW_FPTOFP, dst=0, a=0, dtype=kh.F32)
-        prog, extra = kh.program([dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), f32, dict(op=kh.EW_MULF, dst=1, a=0, b=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=1, b=1),
-                                  dict(op=kh.EW_RSQRT, dst=1, a=1), dict(op=kh.EW_MULF, dst=0, a=0, b=1),
-                                  dict(op=kh.EW_FPTOFP, dst=2, a=0, dtype=kh.F16, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=2)]), []
-        kh.elementwise_specialize(prog, [gx[0]], gy[0])
+        insts, extra = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), f32, dict(op=kh.EW_MULF, dst=1, a=0, b=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=1, b=1),
+                        dict(op=kh.EW_RSQRT, dst=1, a=1), dict(op=kh.EW_MULF, dst=0, a=0, b=1),
+                        dict(op=kh.EW_FPTOFP, dst=2, a=0, dtype=kh.F16, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=2)], []
     else:
-        prog, extra = kh.program(kh.layernorm_insts(n, kh.F16)), [row(gamma), row(beta)]
+        insts, extra = kh.layernorm_insts(n, kh.F16), [row(gamma), row(beta)]
+        hextra = [_host("normal", n, ko.F16, 2, 0, mean=1.0, std=0.1), _host("normal", n, ko.F16, 2, 1, std=0.1)]
+    prog = kh.program(insts)
+    if which == "l2norm_compiled":
+        kh.elementwise_specialize(prog, [gx[0]], gy[0])
+    kh.elementwise(prog, [gx[0]] + extra, gy[0])
+    torch.cuda.synchronize()
+    rows = _sample_rows(n, 16)
+    hx = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n)
+    xr, want = np.ascontiguousarray(hx[rows]), np.zeros((len(rows), n), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(xr, len(rows), n, n, 1, ko.F16)] + [ko.mk_global(h, 1, n, n, 1, ko.F16) for h in hextra],
+                          ko.mk_global(want, len(rows), n, n, 1, ko.F16)) == 0
+    worst = int(np.abs(_line16(_download(ys[0], np.uint16, (n, n))[rows]) - _line16(want)).max())
+    if worst > ULP_TOL:
+        raise CheckFailed("%s: %d ulp against the checker" % (which, worst))
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]] + extra, gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
     name = "x * rsqrt(sum x^2) of every row, compiled at run time" if which == "l2norm_compiled" else "%s of every row" % which
     return {"workload": "%s, fp16 8192x8192, fp32 arithmetic" % name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, which),
-            "kernel": {"softmax": "softmax_kernel", "layernorm": "norm_kernel"}.get(which, "kapy_ew_rows_<hash> (compiled at run time)")}
+            "kernel": {"softmax": "softmax_kernel", "layernorm": "norm_kernel"}.get(which, "kapy_ew_rows_<hash> (compiled at run time)"),
+            "inputs": "x normal(0,1) seed 0" + ("; gamma normal(1,0.1), beta normal(0,0.1) seed 2" if hextra else ""),
+            "checked": True, "check": "16 rows against the checker: max %d ulp (tolerance %d)" % (worst, ULP_TOL)}
 
 
-def bench_transpose(kh, steps, warmup):
+def bench_transpose(kh, steps, warmup, cpu):
+    """C3a: fp16 8192x8192, uniform random 16-bit patterns seed 0; out[j,i] = in[i,j], bit-exact."""
+    import numpy as np
     import torch
+    import ko
     n, sets = 8192, 4
-    xs = [torch.randint(-32768, 32767, (n, n), device="cuda", dtype=torch.int16) for _ in range(sets)]
-    ys = [torch.empty(n, n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    xs = [_dev("bits16", n * n, ko.F16, 0, k) for k in range(sets)]
+    ys = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
     gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
     gy = [kh.mk_global(y.data_ptr(), n, n, n, 1, kh.F16) for y in ys]
+    kh.copy(gx[0], gy[0], transpose=True)
+    torch.cuda.synchronize()
+    # gate: 4 bands of 64 result rows against the checker's ld_global -> transpose -> st_global, and every element against
+    # the index formula itself (a device-side comparison with the strided view of the source)
+    hx = _host("bits16", n * n, ko.F16, 0, 0)
+    gsrc = ko.mk_global(hx, n, n, n, 1, ko.F16)
+    got = _download(ys[0], np.uint16, (n, n))
+    for r0 in (0, 2752, 5440, n - 64):
+        want = np.zeros((64, n), np.uint16)
+        assert ko.lib().ko_copy(C.byref(ko.sv_global(gsrc, 0, n, r0, r0 + 64)), C.byref(ko.mk_global(want, 64, n, n, 1, ko.F16)), 1, 0) == 0
+        if not np.array_equal(got[r0:r0 + 64], want):
+            raise CheckFailed("transpose: rows %d.. differ from the checker" % r0)
+    if not torch.equal(ys[0].view(n, n), xs[0].view(n, n).t()):
+        raise CheckFailed("transpose: result is not the transpose of the source")
     wall, ev = _events(lambda i: kh.copy(gx[i % sets], gy[i % sets], transpose=True), steps, warmup)
     nbytes = 2 * n * n * 2
-    return {"workload": "C3a transpose fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
-            "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev, "transpose"), "kernel": "transpose_lds_kernel"}
-
-
-def bench_permute(kh, steps, warmup):
-    import torch
-    b, h, s, d, sets = 8, 32, 2048, 128, 4
-    xs = [torch.randint(-32768, 32767, (b * h * s * d,), device="cuda", dtype=torch.int16) for _ in range(sets)]
-    ys = [torch.empty(b * h * s * d, device="cuda", dtype=torch.int16) for _ in range(sets)]
-    gx = [kh.mk_global(x.data_ptr(), s, d, d, 1, kh.BF16) for x in xs]
-    gy = [kh.mk_global(y.data_ptr(), s, d, h * d, 1, kh.BF16) for y in ys]
-    grid = (b, h, h * s * d, s * d, s * h * d, d)
-    wall, ev = _events(lambda i: kh.copy_batched(gx[i % sets], gy[i % sets], grid), steps, warmup)
-    nbytes = 2 * b * h * s * d * 2
-    return {"workload": "C3b permute bf16 [8,32,2048,128] bhsd->bshd", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel"}
-
-
-def bench_gemm(kh, steps, warmup, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False):
-    """graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
-    (what a launch-bound shape gains when the host's per-launch cost is taken out).
-    fused_gelu: d = gelu_tanh(a.b*0.5 + bias) with the tail in the GEMM's epilogue (kapy_matmul_fused); flops counted are the GEMM's."""
-    import torch
-    tdt = torch.bfloat16 if dtype == kh.BF16 else torch.float16
-    std = 0.02 if dtype == kh.BF16 else 0.5
-    a = (torch.randn(M, K, device="cuda") * std).to(tdt)
-    b = (torch.randn(N, K, device="cuda") * std).to(tdt) if b_col_major else (torch.randn(K, N, device="cuda") * std).to(tdt)
-    d = torch.empty(M, N, device="cuda", dtype=tdt)
-    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, dtype)
-    gb = kh.mk_global(b.data_ptr(), K, N, 1, K, dtype) if b_col_major else kh.mk_global(b.data_ptr(), K, N, N, 1, dtype)
-    gd = kh.mk_global(d.data_ptr(), M, N, N, 1, dtype)
-    if fused_gelu:
-        bias = torch.randn(N, device="cuda").to(tdt)
-        gbias = kh.mk_global(bias.data_ptr(), 1, N, N, 1, dtype)
-        wall, ev = _events(lambda i: kh.matmul_fused(ga, gb, gd, bias=gbias, alpha=0.5, act=kh.EW_GELU_TANH, tile=tile), steps, warmup)
-    elif graph_of:
-        kh.matmul(ga, gb, gd, tile=tile)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            for _ in range(graph_of):
-                kh.matmul(ga, gb, gd, tile=tile)
-        wall, ev = _events(lambda i: graph.replay(), steps, warmup)
-        wall, ev = wall / graph_of, ev / graph_of
-    else:
-        wall, ev = _events(lambda i: kh.matmul(ga, gb, gd, tile=tile), steps, warmup)
-    flops = 2.0 * M * N * K
-    kind = "bf16" if dtype == kh.BF16 else "f16"
-    return {"workload": name, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "kernel_ms": ev,
-            "dtype": kind, "roofline": _roof_mfma(flops, ev, kind), "kernel": kernel}
-
-
-def bench_f8(kh, steps, warmup, M):
-    import torch
-    N = K = 8192
-    a = torch.randint(0, 120, (M, K), device="cuda", dtype=torch.uint8)      # finite e4m3 patterns
-    sets = 6 if M <= 64 else 2                                               # M<=64 is weight-streaming: 6 x 64 MiB > Infinity Cache
-    ws = [torch.randint(0, 120, (N, K), device="cuda", dtype=torch.uint8) for _ in range(sets)]
-    sa = torch.rand(M, device="cuda") * 0.01 + 0.001
-    sb = torch.rand(N, device="cuda") * 0.01 + 0.001
-    d = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
-    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, kh.F8E4M3)
-    gws = [kh.mk_global(w.data_ptr(), K, N, 1, K, kh.F8E4M3) for w in ws]
-    gd = kh.mk_global(d.data_ptr(), M, N, N, 1, kh.BF16)
-    wall, ev = _events(lambda i: kh.matmul_scaled_f8(ga, gws[i % sets], sa.data_ptr(), sb.data_ptr(), gd), steps, warmup)
-    flops = 2.0 * M * N * K
-    nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
-    out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192" % M, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 64 else "tn_kernel<F8>"}
-    out["roofline"] = _roof_hbm(nbytes, ev) if M <= 64 else _roof_mfma(flops, ev, "f8")
+    out = {"workload": "C3a transpose fp16 8192x8192", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
+           "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev, "transpose"), "kernel": "transpose_lds_kernel",
+           "inputs": "uniform random 16-bit patterns seed 0 (as the configuration states)", "checked": True,
+           "check": "256 result rows bit-equal to the checker; every element bit-equal to in[j,i]"}
+    if cpu:
+        hy = np.zeros(n * n, np.uint16)
+        out["cpu_baseline"] = _cpu_repeat(lambda: ko.lib().ko_baseline_transpose16(hx.ctypes.data, hy.ctypes.data, n, n), nbytes, 1e9, "GB/s",
+                                          "the whole 8192x8192 transpose, 64x64 tiles")
     return out
 
 
-def cpu_baseline_gelu(sample_rows=256):
-    """The oracle's elementwise program on a bounded sample (sample_rows x 8192) of the same workload,
-    on this box's host cores.  Reported, never the optimisation target."""
-    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+def bench_permute(kh, steps, warmup, cpu):
+    """C3b: bf16 [8,32,2048,128] random 16-bit patterns seed 1; out[b,s,h,d] = in[b,h,s,d], bit-exact."""
     import numpy as np
+    import torch
     import ko
-    n = 8192
-    x = ko.fill_normal(sample_rows * n, ko.F16, 0, 0).reshape(sample_rows, n)
-    bias = ko.fill_normal(n, ko.F16, 1, 0)
-    out = np.zeros((sample_rows, n), dtype=np.uint16)
-    prog = ko.gelu_program()
-    gx, gb, go = ko.mk_global(x, sample_rows, n, n, 1, ko.F16), ko.mk_global(bias, 1, n, n, 1, ko.F16), ko.mk_global(out, sample_rows, n, n, 1, ko.F16)
-    ko.elementwise(prog, [gx, gb], go)  # warm-up
-    reps, t0 = 0, time.perf_counter()
+    b, h, s, d, sets = 8, 32, 2048, 128, 4
+    tot = b * h * s * d
+    xs = [_dev("bits16", tot, ko.F16, 1, k) for k in range(sets)]
+    ys = [torch.empty(tot, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    gx = [kh.mk_global(x.data_ptr(), s, d, d, 1, kh.BF16) for x in xs]
+    gy = [kh.mk_global(y.data_ptr(), s, d, h * d, 1, kh.BF16) for y in ys]
+    grid = (b, h, h * s * d, s * d, s * h * d, d)
+    kh.copy_batched(gx[0], gy[0], grid)
+    torch.cuda.synchronize()
+    # gate: 8 of the 256 (b,h) programs against the checker, and every element against the index formula
+    hx = _host("bits16", tot, ko.F16, 1, 0)
+    got = _download(ys[0], np.uint16, (b, s, h, d))
+    for t in range(8):
+        ib, ih = t, (5 * t + 3) % h
+        want = np.zeros((s, d), np.uint16)
+        src = hx[(ib * h + ih) * s * d:(ib * h + ih + 1) * s * d]
+        assert ko.lib().ko_copy(C.byref(ko.mk_global(src, s, d, d, 1, ko.BF16)), C.byref(ko.mk_global(want, s, d, d, 1, ko.BF16)), 0, 0) == 0
+        if not np.array_equal(got[ib, :, ih, :], want):
+            raise CheckFailed("permute: program (%d,%d) differs from the checker" % (ib, ih))
+    if not torch.equal(ys[0].view(b, s, h, d), xs[0].view(b, h, s, d).permute(0, 2, 1, 3)):
+        raise CheckFailed("permute: result is not the permuted source")
+    wall, ev = _events(lambda i: kh.copy_batched(gx[i % sets], gy[i % sets], grid), steps, warmup)
+    nbytes = 2 * tot * 2
+    out = {"workload": "C3b permute bf16 [8,32,2048,128] bhsd->bshd", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel",
+           "inputs": "uniform random 16-bit patterns seed 1 (as the configuration states)", "checked": True,
+           "check": "8 of 256 (b,h) programs bit-equal to the checker; every element bit-equal to in[b,h,s,d]"}
+    if cpu:
+        hy = np.zeros(tot, np.uint16)
+        out["cpu_baseline"] = _cpu_repeat(lambda: ko.lib().ko_baseline_permute_bhsd_bshd16(hx.ctypes.data, hy.ctypes.data, b, h, s, d), nbytes, 1e9, "GB/s",
+                                          "the whole permute, 256-byte rows moved whole")
+    return out
+
+
+# ---------------------------------------------------------------- GEMMs
+def _blocks_frobenius(ko, got, go_a, go_b, M, N, K, out_dtype, count, blk=64, scales=None):
+    """Relative Frobenius error of `count` blk x blk blocks of the result against the fp64-accumulated checker."""
+    import numpy as np
+    num = den = 0.0
+    for t in range(count):
+        r0 = 0 if M <= blk else (t * (M // count) + 29 * t) % (M - blk)
+        c0 = 0 if N <= blk else ((count - 1 - t) * (N // count) + 71 * t) % (N - blk)
+        bm, bn = min(blk, M), min(blk, N)
+        want = np.zeros((bm, bn), dtype=np.uint16)
+        ga, gb, gw = ko.sv_global(go_a, r0, r0 + bm, 0, K), ko.sv_global(go_b, 0, K, c0, c0 + bn), ko.mk_global(want, bm, bn, bn, 1, out_dtype)
+        if scales is None:
+            assert ko.lib().ko_matmul(C.byref(ga), C.byref(gb), None, C.byref(gw), ko.RN) == 0
+        else:
+            rs, cs = np.ascontiguousarray(scales[0][r0:r0 + bm]), np.ascontiguousarray(scales[1][c0:c0 + bn])
+            assert ko.lib().ko_matmul_scaled_f8(C.byref(ga), C.byref(gb), rs.ctypes.data, cs.ctypes.data, C.byref(gw)) == 0
+        g, w = ko.decode(got[r0:r0 + bm, c0:c0 + bn], out_dtype), ko.decode(want, out_dtype)
+        if not np.all(np.isfinite(g)):
+            return float("inf")
+        num += ((g - w) ** 2).sum()
+        den += (w ** 2).sum()
+    return float(np.sqrt(num / max(den, 1e-300)))
+
+
+def _cpu_gemm(ko, go_a, go_b, go_d, rows, N, K, scales, what):
+    """The packed, register-blocked fp32 GEMM of oracle/kapy_baseline.cpp on the first `rows` rows of the lhs."""
+    import numpy as np
+    secs = C.c_double(0.0)
+    a, d = ko.sv_global(go_a, 0, rows, 0, K), ko.sv_global(go_d, 0, rows, 0, N)
+    rs = scales[0].ctypes.data if scales else None
+    cs = scales[1].ctypes.data if scales else None
+    tot, reps, t0 = 0.0, 0, time.perf_counter()
     while True:
-        ko.elementwise(prog, [gx, gb], go)
+        assert ko.lib().ko_baseline_gemm(C.byref(a), C.byref(go_b), rs, cs, C.byref(d), C.byref(secs)) == 0
+        tot += secs.value
         reps += 1
-        dt = time.perf_counter() - t0
-        if dt > 10.0:
+        if time.perf_counter() - t0 > CPU_SECONDS:
             break
-    nbytes = (2 * sample_rows * n * 2 + n * 2) * reps
-    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": ko.lib().ko_num_threads(), "kind": "port",
-            "sample": "%d of 8192 rows of the same workload, %d repetitions, %.1f s" % (sample_rows, reps, dt)}
+    return {"value": round(2.0 * rows * N * K * reps / tot / 1e12, 4), "unit": "TFLOP/s", "cores": ko.lib().ko_num_threads(), "kind": "port",
+            "sample": "%s; fp32 accumulate, operands widened to fp32 and packed outside the timed multiply; %d repetitions, %.2f s of multiplying" % (what, reps, tot)}
+
+
+def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None):
+    """graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
+    (what a launch-bound shape gains when the host's per-launch cost is taken out).
+    fused_gelu: d = gelu_tanh(a.b*0.5 + bias) with the tail in the GEMM's epilogue (kapy_matmul_fused); flops counted are the GEMM's.
+    gen: "normal" = normal(0, 0.02) seeds 0 / 1 (C4), "uniform" = uniform[-1,1) seed 0 streams 0 / 1 (C1)."""
+    import numpy as np
+    import torch
+    import ko
+    if gen == "uniform":
+        ha, hb = _host("uniform", M * K, dtype, 0, 0), _host("uniform", K * N, dtype, 0, 1)
+        a, b = _dev("uniform", M * K, dtype, 0, 0), _dev("uniform", K * N, dtype, 0, 1)
+        what = "A, B uniform[-1,1) seed 0 (streams 0, 1)"
+    else:
+        ha, hb = _host("normal", M * K, dtype, 0, 0, std=0.02), _host("normal", K * N, dtype, 1, 0, std=0.02)
+        a, b = _dev("normal", M * K, dtype, 0, 0, std=0.02), _dev("normal", K * N, dtype, 1, 0, std=0.02)
+        what = "A normal(0,0.02) seed 0, B normal(0,0.02) seed 1"
+    d = torch.empty(M * N, device="cuda", dtype=torch.int16)
+    b_str = (1, K) if b_col_major else (N, 1)
+    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, dtype)
+    gb = kh.mk_global(b.data_ptr(), K, N, b_str[0], b_str[1], dtype)
+    gd = kh.mk_global(d.data_ptr(), M, N, N, 1, dtype)
+    go_a, go_b = ko.mk_global(ha, M, K, K, 1, dtype), ko.mk_global(hb, K, N, b_str[0], b_str[1], dtype)
+    if fused_gelu:
+        hbias = _host("normal", N, dtype, 2)
+        bias = _dev("normal", N, dtype, 2)
+        gbias = kh.mk_global(bias.data_ptr(), 1, N, N, 1, dtype)
+        run = lambda i: kh.matmul_fused(ga, gb, gd, bias=gbias, alpha=0.5, act=kh.EW_GELU_TANH, tile=tile)
+    else:
+        run = lambda i: kh.matmul(ga, gb, gd, tile=tile)
+    run(0)
+    torch.cuda.synchronize()
+    got = _download(d, np.uint16, (M, N))
+    if fused_gelu:
+        # gate: blocks of gelu(c*0.5 + bias) recomputed in fp64 from the checker's fp32-result GEMM of the same blocks
+        num = den = 0.0
+        for t in range(8):
+            r0, c0 = (t * (M // 8) + 29 * t) % (M - 64), ((7 - t) * (N // 8) + 71 * t) % (N - 64)
+            c32 = np.zeros((64, 64), np.float32)
+            assert ko.lib().ko_matmul(C.byref(ko.sv_global(go_a, r0, r0 + 64, 0, K)), C.byref(ko.sv_global(go_b, 0, K, c0, c0 + 64)), None,
+                                      C.byref(ko.mk_global(c32, 64, 64, 64, 1, ko.F32)), ko.RN) == 0
+            v = c32.astype(np.float64) * 0.5 + ko.decode(hbias[c0:c0 + 64], dtype)[None, :]
+            w = 0.5 * v * (1.0 + np.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+            g = ko.decode(got[r0:r0 + 64, c0:c0 + 64], dtype)
+            num += ((g - w) ** 2).sum()
+            den += (w ** 2).sum()
+        rel, n_blocks = float(np.sqrt(num / den)), 8
+        tol = 4e-3   # the bf16 result itself rounds at 2^-9 relative
+    else:
+        n_blocks = 16 if M * N > 1024 * 1024 else 0
+        if n_blocks:
+            rel = _blocks_frobenius(ko, got, go_a, go_b, M, N, K, dtype, n_blocks)
+        else:   # small enough for the whole result
+            want = np.zeros((M, N), np.uint16)
+            assert ko.lib().ko_matmul(C.byref(go_a), C.byref(go_b), None, C.byref(ko.mk_global(want, M, N, N, 1, dtype)), ko.RN) == 0
+            g, w = ko.decode(got, dtype), ko.decode(want, dtype)
+            rel = float(np.linalg.norm(g - w) / np.linalg.norm(w)) if np.all(np.isfinite(g)) else float("inf")
+        tol = FROB_TOL
+    if not rel <= tol:
+        raise CheckFailed("%s: relative Frobenius error %g" % (name, rel))
+    if graph_of:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(graph_of):
+                run(0)
+        wall, ev = _events(lambda i: graph.replay(), steps, warmup)
+        wall, ev = wall / graph_of, ev / graph_of
+    else:
+        wall, ev = _events(run, steps, warmup)
+    flops = 2.0 * M * N * K
+    kind = "bf16" if dtype == kh.BF16 else "f16"
+    out = {"workload": name, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "kernel_ms": ev,
+           "dtype": kind, "roofline": _roof_mfma(flops, ev, kind, key), "kernel": kernel, "inputs": what + " (host-generated, as the configuration states)",
+           "checked": True, "check": "%s against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" %
+                                     ("%d 64x64 blocks of the timed result" % n_blocks if n_blocks else "the whole timed result", rel, tol)}
+    if cpu and not graph_of and not fused_gelu:
+        rows = min(M, 1024)
+        hd = np.zeros(M * N, np.uint16)
+        out["cpu_baseline"] = _cpu_gemm(ko, go_a, go_b, ko.mk_global(hd, M, N, N, 1, dtype), rows, N, K, None,
+                                        "the first %d of %d rows of the result (all of N and K)" % (rows, M) if rows < M else "the whole workload")
+    return out
+
+
+_f8_cache = {}
+
+
+def _f8_operands(ko, M, N, K):
+    """C5: pre-quantisation values normal(0,1) fp32 (A seed 0, W seed 1, W stored K-contiguous per output column),
+    per-row / per-column scales amax/448, values rounded once (RN-even, saturating) to e4m3."""
+    import numpy as np
+    vp = lambda x: x.ctypes.data_as(C.c_void_p)
+    if ("w", N, K) not in _f8_cache:
+        w = ko.fill_normal(N * K, ko.F32, 1, 0).reshape(N, K)
+        wq, sb = np.zeros((N, K), np.uint8), np.zeros(N, np.float32)
+        ko.lib().ko_quantize_e4m3(vp(w), N, K, K, 1, 1, vp(wq), vp(sb))
+        _f8_cache[("w", N, K)] = (wq, sb)
+    a = ko.fill_normal(M * K, ko.F32, 0, 0).reshape(M, K)
+    aq, sa = np.zeros((M, K), np.uint8), np.zeros(M, np.float32)
+    ko.lib().ko_quantize_e4m3(vp(a), M, K, K, 1, 1, vp(aq), vp(sa))
+    wq, sb = _f8_cache[("w", N, K)]
+    return aq, sa, wq, sb
+
+
+def bench_f8(kh, steps, warmup, cpu, M):
+    import numpy as np
+    import torch
+    import ko
+    N = K = 8192
+    aq, sa, wq, sb = _f8_operands(ko, M, N, K)
+    a, dsa, dsb = _upload(aq), _upload(sa), _upload(sb)
+    if ("wdev", N, K) not in _dev_cache:
+        _dev_cache[("wdev", N, K)] = _upload(wq)
+    w0 = _dev_cache[("wdev", N, K)]
+    sets = 6 if M <= 64 else 1                 # M<=64 is weight-streaming: 6 x 64 MiB > Infinity Cache (copies of the same weight)
+    ws = [w0] + [w0.clone() for _ in range(sets - 1)]
+    d = torch.empty(M * N, device="cuda", dtype=torch.int16)
+    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, kh.F8E4M3)
+    gws = [kh.mk_global(w.data_ptr(), K, N, 1, K, kh.F8E4M3) for w in ws]
+    gd = kh.mk_global(d.data_ptr(), M, N, N, 1, kh.BF16)
+    kh.matmul_scaled_f8(ga, gws[0], dsa.data_ptr(), dsb.data_ptr(), gd)
+    torch.cuda.synchronize()
+    got = _download(d, np.uint16, (M, N))
+    go_a, go_w = ko.mk_global(aq, M, K, K, 1, ko.F8E4M3), ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)
+    n_blocks = 16
+    rel = _blocks_frobenius(ko, got, go_a, go_w, M, N, K, ko.BF16, n_blocks, scales=(sa, sb))
+    if not rel <= FROB_TOL:
+        raise CheckFailed("f8 M=%d: relative Frobenius error %g" % (M, rel))
+    wall, ev = _events(lambda i: kh.matmul_scaled_f8(ga, gws[i % sets], dsa.data_ptr(), dsb.data_ptr(), gd), steps, warmup)
+    flops = 2.0 * M * N * K
+    nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
+    out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192" % M, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 64 else "tn_kernel<F8>",
+           "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
+           "checked": True, "check": "%d %dx64 blocks against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" % (n_blocks, min(M, 64), rel, FROB_TOL)}
+    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d" % M) if M <= 64 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
+    if cpu:
+        rows = min(M, 1024)
+        hd = np.zeros(M * N, np.uint16)
+        out["cpu_baseline"] = _cpu_gemm(ko, go_a, go_w, ko.mk_global(hd, M, N, N, 1, ko.BF16), rows, N, K, (sa, sb),
+                                        "the first %d of %d rows of the result (all of N and K)" % (rows, M) if rows < M else "the whole workload")
+    return out
+
+
+WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"]
 
 
 def main():
@@ -313,9 +639,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="gelu", choices=["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed", "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"])
+    ap.add_argument("--workload", default="gelu", choices=WORKLOADS)
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (every path here runs on a single MI355X)" % args.gpus)
@@ -325,28 +651,32 @@ def main():
         sys.exit("bench.py: no GPU visible; the library has no CPU fallback to time")
     torch.cuda.set_device(0)
     kh.lib()
+    cpu = not args.no_cpu
     table = {
-        "gelu": lambda s, w: bench_gelu(kh, s, w),
-        "add": lambda s, w: bench_add(kh, s, w),
-        "expr": lambda s, w: bench_add(kh, s, w, "expr"),
-        "expr_compiled": lambda s, w: bench_add(kh, s, w, "expr_compiled"),
-        "swiglu": lambda s, w: bench_add(kh, s, w, "swiglu"),
-        "copy": lambda s, w: bench_copy(kh, s, w),
-        "transpose": lambda s, w: bench_transpose(kh, s, w),
-        "gelu_transposed": lambda s, w: bench_gelu_transposed(kh, s, w),
-        "reduce": lambda s, w: bench_reduce(kh, s, w),
-        "softmax": lambda s, w: bench_rowwise(kh, s, w, "softmax"),
-        "layernorm": lambda s, w: bench_rowwise(kh, s, w, "layernorm"),
-        "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, "l2norm_compiled"),
-        "permute": lambda s, w: bench_permute(kh, s, w),
-        "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel"),
-        "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True),
-        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32)),
-        "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20),
-        "f8_m16": lambda s, w: bench_f8(kh, s, w, 16),
-        "f8_m4096": lambda s, w: bench_f8(kh, s, w, 4096),
+        "gelu": lambda s, w: bench_gelu(kh, s, w, cpu),
+        "add": lambda s, w: bench_add(kh, s, w, cpu),
+        "expr": lambda s, w: bench_add(kh, s, w, cpu, "expr"),
+        "expr_compiled": lambda s, w: bench_add(kh, s, w, cpu, "expr_compiled"),
+        "swiglu": lambda s, w: bench_add(kh, s, w, cpu, "swiglu"),
+        "copy": lambda s, w: bench_copy(kh, s, w, cpu),
+        "transpose": lambda s, w: bench_transpose(kh, s, w, cpu),
+        "gelu_transposed": lambda s, w: bench_gelu_transposed(kh, s, w, cpu),
+        "reduce": lambda s, w: bench_reduce(kh, s, w, cpu),
+        "softmax": lambda s, w: bench_rowwise(kh, s, w, cpu, "softmax"),
+        "layernorm": lambda s, w: bench_rowwise(kh, s, w, cpu, "layernorm"),
+        "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, cpu, "l2norm_compiled"),
+        "permute": lambda s, w: bench_permute(kh, s, w, cpu),
+        "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel", key="gemm_bf16"),
+        "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True),
+        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform"),
+        "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform"),
+        "f8_m16": lambda s, w: bench_f8(kh, s, w, cpu, 16),
+        "f8_m4096": lambda s, w: bench_f8(kh, s, w, cpu, 4096),
     }
-    main_res = table[args.workload](args.steps, args.warmup)
+    try:
+        main_res = table[args.workload](args.steps, args.warmup)
+    except CheckFailed as e:
+        sys.exit("bench.py: correctness gate failed, nothing timed: %s" % e)
     others = []
     if not args.no_others:
         for name, fn in table.items():
@@ -356,7 +686,10 @@ def main():
             try:
                 r = fn(min(args.steps, 20), min(args.warmup, 10))
             except kh.KapyError as e:   # e.g. no runtime compiler on this machine for the compiled workloads
-                others.append({"workload": name, "error": str(e)})
+                others.append({"workload": name, "error": str(e), "checked": False})
+                continue
+            except CheckFailed as e:
+                others.append({"workload": name, "error": "correctness gate failed, not timed: %s" % e, "checked": False})
                 continue
             r["value"] = round(r["value"], 2)
             r["ms_per_step"] = round(r["ms_per_step"], 4)
@@ -368,9 +701,10 @@ def main():
         "ms_per_step": round(main_res["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic",
         "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "kernel_ms": round(main_res["kernel_ms"], 4),
+                   "inputs": main_res["inputs"], "checked": main_res["checked"], "check": main_res["check"],
                    "buffers": "4 rotating sets (1 GiB) so reads miss the Infinity Cache" if main_res["unit"] == "GB/s" else "single set"},
         "roofline": main_res["roofline"],
-        "cpu_baseline": None if args.no_cpu else cpu_baseline_gelu(),
+        "cpu_baseline": main_res.get("cpu_baseline"),
         "other_workloads": others,
     }
     print(json.dumps(line))

@@ -904,51 +904,6 @@ int ko_reduce(const ko_global *src, const ko_global *dst, int axis, int kind) {
   return 0;
 }
 
-// ---------------------------------------------------------------------------------------------
-// Timing baseline: cache-blocked fp32-accumulate GEMM over all host threads.  Not the checker.
-// ---------------------------------------------------------------------------------------------
-__attribute__((target_clones("avx512f", "avx2", "default")))
-static void gemm_block_f32(const float *A, const float *Bt, float *C, int64_t M, int64_t N, int64_t K, int64_t i0,
-                           int64_t i1, int64_t j0, int64_t j1) {
-  for (int64_t i = i0; i < i1; ++i)
-    for (int64_t j = j0; j < j1; ++j) {
-      const float *a = A + i * K, *b = Bt + j * K;
-      float s[16] = {0};
-      int64_t k = 0;
-      for (; k + 16 <= K; k += 16)
-        for (int t = 0; t < 16; ++t) s[t] += a[k + t] * b[k + t];
-      float r = 0;
-      for (int t = 0; t < 16; ++t) r += s[t];
-      for (; k < K; ++k) r += a[k] * b[k];
-      C[i * N + j] = r;
-    }
-  (void)M;
-}
-
-int ko_gemm_f32acc(const ko_global *lhs, const ko_global *rhs, const ko_global *result) {
-  int rc = matmul_verify(lhs, rhs, nullptr, result);
-  if (rc) return rc;
-  int64_t M = extent0(lhs), K = extent1(lhs), N = extent1(rhs);
-  std::vector<float> A((size_t)M * K), Bt((size_t)N * K), C((size_t)M * N);
-#pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < M; ++i)
-    for (int64_t k = 0; k < K; ++k) A[i * K + k] = (float)ko_decode(lhs->ptr, lhs->dtype, elem_offset(lhs, i, k));
-#pragma omp parallel for schedule(static)
-  for (int64_t j = 0; j < N; ++j)
-    for (int64_t k = 0; k < K; ++k) Bt[j * K + k] = (float)ko_decode(rhs->ptr, rhs->dtype, elem_offset(rhs, k, j));
-  const int64_t BI = 32, BJ = 32;
-  int64_t nbi = (M + BI - 1) / BI, nbj = (N + BJ - 1) / BJ;
-#pragma omp parallel for schedule(dynamic, 1) collapse(2)
-  for (int64_t bi = 0; bi < nbi; ++bi)
-    for (int64_t bj = 0; bj < nbj; ++bj)
-      gemm_block_f32(A.data(), Bt.data(), C.data(), M, N, K, bi * BI, std::min(M, bi * BI + BI), bj * BJ,
-                     std::min(N, bj * BJ + BJ));
-#pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < M; ++i)
-    for (int64_t j = 0; j < N; ++j) ko_encode(result->ptr, result->dtype, elem_offset(result, i, j), (double)C[i * N + j], KO_RN);
-  return 0;
-}
-
 int ko_num_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

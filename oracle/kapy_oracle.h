@@ -115,9 +115,17 @@ void ko_quantize_e4m3(const float *x, int64_t rows, int64_t cols, int64_t row_st
                       int along_cols, uint8_t *q, float *scale);
 int ko_reduce(const ko_global *src, const ko_global *dst, int axis, int kind);
 
-/* timing baseline: blocked fp32-accumulate GEMM over all host threads (not the checker). */
-int ko_gemm_f32acc(const ko_global *lhs, const ko_global *rhs, const ko_global *result);
 int ko_num_threads(void);
+
+/* ---- timing baselines (kapy_baseline.cpp): the benchmark workloads written for speed on the host cores
+ * (packed panels + register-blocked fp32 micro-kernel, fused vector loop, cache-blocked tiles; AVX-512 forms
+ * chosen at run time).  They are what the benchmark's cpu_baseline leg times; tests/test_oracle_baselines.py
+ * checks each against the checker above. ---- */
+int ko_baseline_gemm(const ko_global *lhs, const ko_global *rhs, const float *row_scale, const float *col_scale,
+                     const ko_global *result, double *multiply_seconds);
+int ko_baseline_gelu_f16(const uint16_t *x, const uint16_t *bias, float scale, uint16_t *y, int64_t rows, int64_t cols, int64_t pitch);
+int ko_baseline_transpose16(const uint16_t *src, uint16_t *dst, int64_t rows, int64_t cols);
+int ko_baseline_permute_bhsd_bshd16(const uint16_t *src, uint16_t *dst, int64_t b, int64_t h, int64_t s, int64_t d);
 
 #ifdef __cplusplus
 }

@@ -115,7 +115,10 @@ def lib():
         L.ko_quantize_e4m3.restype = None
         L.ko_quantize_e4m3.argtypes = [vp, i64, i64, i64, i64, C.c_int, vp, vp]
         L.ko_reduce.restype = C.c_int; L.ko_reduce.argtypes = [P(Global), P(Global), C.c_int, C.c_int]
-        L.ko_gemm_f32acc.restype = C.c_int; L.ko_gemm_f32acc.argtypes = [P(Global), P(Global), P(Global)]
+        L.ko_baseline_gemm.restype = C.c_int; L.ko_baseline_gemm.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(dbl)]
+        L.ko_baseline_gelu_f16.restype = C.c_int; L.ko_baseline_gelu_f16.argtypes = [vp, vp, C.c_float, vp, i64, i64, i64]
+        L.ko_baseline_transpose16.restype = C.c_int; L.ko_baseline_transpose16.argtypes = [vp, vp, i64, i64]
+        L.ko_baseline_permute_bhsd_bshd16.restype = C.c_int; L.ko_baseline_permute_bhsd_bshd16.argtypes = [vp, vp, i64, i64, i64, i64]
         L.ko_num_threads.restype = C.c_int
         L.ko_decode.restype = dbl; L.ko_decode.argtypes = [vp, C.c_int, i64]
         _lib = L

@@ -225,17 +225,6 @@ def test_reduce_max_orders_signed_zeros_and_propagates_nan(ko):
     assert np.isnan(sm[3, 0]) and np.isnan(sm[4, 0]) and sm[0, 0] == -3.0
 
 
-def test_gemm_timing_baseline_agrees_with_checker(ko):
-    M = N = K = 96
-    a = ko.fill_uniform(M * K, ko.BF16, 0, 0).reshape(M, K)
-    bt = ko.fill_uniform(N * K, ko.BF16, 0, 1).reshape(N, K)
-    o1, o2 = np.zeros((M, N), np.float32), np.zeros((M, N), np.float32)
-    ga, gb = ko.mk_global(a, M, K, K, 1, ko.BF16), ko.mk_global(bt, K, N, 1, K, ko.BF16)
-    ko.lib().ko_matmul(C.byref(ga), C.byref(gb), None, C.byref(ko.mk_global(o1, M, N, N, 1, ko.F32)), ko.RN)
-    ko.lib().ko_gemm_f32acc(C.byref(ga), C.byref(gb), C.byref(ko.mk_global(o2, M, N, N, 1, ko.F32)))
-    assert np.linalg.norm(o1 - o2) / np.linalg.norm(o1) < 1e-5
-
-
 def test_elementwise_reduce_ops_vs_numpy_and_scipy(ko):
     """The reduce instructions of elementwise programs: exact sums on integer-valued inputs, exact maxima, NaN
     propagation, axis 0 and 1, and a whole softmax against scipy in float64."""

@@ -123,8 +123,20 @@ int64_t kapy_swizzle_offset(const kapy_swizzling *layout, int64_t bits, int64_t 
 int kapy_swizzle_search(const kapy_fragments *access, const int64_t shape[2], int64_t stride0, int64_t stride1,
                         int64_t bits, int64_t alignment, int32_t *pairs, int32_t max_pairs);
 /* getDefaultLayouts(MatmulOp) — LayoutUtils.cpp:123-149 for the MFMA shapes of gfx950:
- * which = 0 lhs, 1 rhs, 2 acc; also reports the MFMA tile (m, n, k). */
+ * which = 0 lhs [m x k], 1 rhs [k x n], 2 acc [m x n] of the instruction as documented; 3 = acc [m x n] when the
+ * instruction is issued with the operands exchanged (rhs fragment in the first slot: legal without moving a register
+ * because the lhs and rhs layouts mirror each other; the instruction then computes the transposed block and a lane's
+ * register quad holds four consecutive columns of one row).  The tiled matmul kernels issue form 3, the decode-shaped
+ * fp8 kernels form 2; all of them take their lane positions from these layouts.  Also reports the tile (m, n, k). */
 int kapy_matmul_layouts(int32_t impl_way, int32_t which, kapy_fragments *out, int32_t mnk[3]);
+/* Runs ONE matrix instruction of `impl_way` (16..19) on one wavefront, registers in and out, through the same
+ * instruction wrapper the matmul kernels multiply with: lhs_regs / rhs_regs hold, for lane 0..63 back to back, the
+ * lane's kpack operand elements (kapy_matmul_layouts which = 0 / 1 say which elements those are), acc_regs gets each
+ * lane's m*n/64 fp32 accumulator registers (which = 2, or 3 with exchanged != 0).  The counterpart of the coordinate ->
+ * loop-iv tables of MatmulOpToLLVM.cpp:94-123 made observable: a test scatters a tile by the layouts, calls this and
+ * gathers the product by the layouts, which fails if they do not describe the hardware.  Device pointers. */
+int kapy_mfma_probe(int32_t impl_way, int32_t lhs_dtype, int32_t rhs_dtype, int32_t exchanged, const void *lhs_regs, const void *rhs_regs,
+                    float *acc_regs, void *stream);
 /* The LDS layout the tiled matmul stages its operands in (result of kapy_swizzle_search on the
  * MFMA operand layout), so callers and tests can check it is conflict-free by construction. */
 int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out);

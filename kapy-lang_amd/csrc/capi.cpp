@@ -321,8 +321,9 @@ int kapy_matmul_layouts(int32_t impl_way, int32_t which, kapy_fragments *out, in
     return fail(KAPY_ERR_UNSUPPORTED, "mma_m16n8k8_tf32: gfx950 has no tf32 matrix instruction");
   default: return fail(KAPY_ERR_INVALID, "matmul layouts: unknown implement way %d", impl_way);
   }
-  if (which < 0 || which > 2 || !out) return fail(KAPY_ERR_INVALID, "matmul layouts: which must be 0 (lhs), 1 (rhs) or 2 (acc)");
-  to_public(which == 0 ? mfma_lhs(s) : which == 1 ? mfma_rhs(s) : mfma_acc(s), out);
+  if (which < 0 || which > 3 || !out)
+    return fail(KAPY_ERR_INVALID, "matmul layouts: which must be 0 (lhs), 1 (rhs), 2 (acc) or 3 (acc with the operands exchanged)");
+  to_public(which == 0 ? mfma_lhs(s) : which == 1 ? mfma_rhs(s) : which == 2 ? mfma_acc(s) : mfma_acc_exchanged(s), out);
   if (mnk) { mnk[0] = s.m; mnk[1] = s.n; mnk[2] = s.k; }
   return KAPY_OK;
 }

@@ -193,6 +193,12 @@ struct MfmaShape {
 KAPY_HD constexpr Fragments mfma_lhs(MfmaShape s) { return {s.m, kWaveSize / s.m, 1, s.kpack, 0}; }
 KAPY_HD constexpr Fragments mfma_rhs(MfmaShape s) { return {kWaveSize / s.n, s.n, s.kpack, 1, 1}; }
 KAPY_HD constexpr Fragments mfma_acc(MfmaShape s) { return {kWaveSize / s.n, s.n, 4, 1, 1}; }
+// The accumulator when the instruction is issued with the operands exchanged (rhs fragment in the first operand
+// slot, lhs fragment in the second: the mirrored operand layouts make that legal without moving a register).
+// The instruction then computes the transposed block, so over the [m x n] result a lane's register quad holds
+// four consecutive COLUMNS of one row - what a row-major store wants.  The tiled matmul kernels issue this form.
+//   32x32x16: <[32,2],[1,4],(1,0)>   16x16x32: <[16,4],[1,4],(1,0)>
+KAPY_HD constexpr Fragments mfma_acc_exchanged(MfmaShape s) { return mfma_acc(MfmaShape{s.n, s.m, s.k, s.kpack}).transposed(); }
 constexpr MfmaShape kMfma32x32x16{32, 32, 16, 8};
 constexpr MfmaShape kMfma16x16x32{16, 16, 32, 8};
 constexpr MfmaShape kMfma16x16x128F8{16, 16, 128, 32};

@@ -29,78 +29,24 @@
 #include "common.hpp"
 #include "layout.hpp"
 #include "matmul_params.hpp"
+#include "mfma.hpp"
 #include "ew_machine.hpp"
 #include "numeric.hpp"
 
 namespace kapy {
 namespace {
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-
-// Operand element policies: bytes per element, the K extent of one matrix instruction, how many
-// 16-byte LDS chunks a lane feeds it per operand, and its duration in clocks (4 per pass).
-struct Bf16 {
-  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32, kM = 32;
-  using Acc = f32x16;
-  static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
-  }
-};
-struct F16 {
-  static constexpr int kBytes = 2, kSliceK = 16, kChunks = 1, kMfmaClocks = 32, kM = 32;
-  using Acc = f32x16;
-  static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
-  }
-};
-// The 16x16x32 forms: kM = 16 rows per operand block, four K-groups of lanes.  Same flops per clock
-// as 32x32x16, but each accumulator register is read and written once per 32 K instead of per 16 K;
-// under sustained load the chip holds a ~13% higher clock with them (it is power-limited), which
-// outweighs the doubled operand-register reads.
-struct Bf16M16 {
-  static constexpr int kBytes = 2, kSliceK = 32, kChunks = 1, kMfmaClocks = 16, kM = 16;
-  using Acc = f32x4;
-  static __device__ __forceinline__ f32x4 mfma(const u32x4 *a, const u32x4 *b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
-  }
-};
-struct F16M16 {
-  static constexpr int kBytes = 2, kSliceK = 32, kChunks = 1, kMfmaClocks = 16, kM = 16;
-  using Acc = f32x4;
-  static __device__ __forceinline__ f32x4 mfma(const u32x4 *a, const u32x4 *b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
-  }
-};
-// OCP fp8, v_mfma_scale_f32_32x32x64_f8f6f4 with unit block scales (E8M0 127 = 2^0).  AF / BF are the
-// format selectors of the first / second instruction operand: 0 = E4M3, 1 = E5M2 (kapy lets the two
-// f8 types mix, Kapy.cpp:484-487).  A lane feeds 32 K-contiguous bytes per operand: two chunks.
-template <int AF, int BF>
-struct F8 {
-  static constexpr int kBytes = 1, kSliceK = 64, kChunks = 2, kMfmaClocks = 64, kM = 32;
-  using Acc = f32x16;
-  static __device__ __forceinline__ f32x16 mfma(const u32x4 *a, const u32x4 *b, f32x16 c) {
-    i32x8 av = {(int)a[0][0], (int)a[0][1], (int)a[0][2], (int)a[0][3], (int)a[1][0], (int)a[1][1], (int)a[1][2], (int)a[1][3]};
-    i32x8 bv = {(int)b[0][0], (int)b[0][1], (int)b[0][2], (int)b[0][3], (int)b[1][0], (int)b[1][1], (int)b[1][2], (int)b[1][3]};
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AF, BF, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
-  }
-};
-
 // LDS image of an operand tile: [rows][ROWBYTES] bytes, K contiguous, 16-byte chunks XOR-ed with the
 // line index.  The parameters come from the compile-time search (the reference's getSwizzlingLayouts
-// for 64 banks) run on the access layout of an MFMA operand read: 32 lanes down the rows, 2 across,
-// 16 contiguous bytes per lane.
-constexpr Fragments kOperandRead16B{32, 2, 1, 16, 0};
-template <int ROWBYTES>
+// for 64 banks) run on the access layout of the operand reads of the matrix instruction the kernel is
+// built for: the lhs fragments of T::kShape counted in bytes (T::kShape.m lanes down the rows, the K-groups
+// across, 16 contiguous bytes per lane and read instruction).
+template <int ROWBYTES, typename T>
 struct TileLayout {
   static constexpr int kRowBytes = ROWBYTES;
-  static constexpr Swizzle kSwizzle = first_swizzle(kOperandRead16B, {32, 32}, ROWBYTES, 1, 8, 1024);
+  static constexpr MfmaShape kS = T::kShape;
+  static constexpr Fragments kAccess{mfma_lhs(kS).a0, mfma_lhs(kS).a1, 1, mfma_lhs(kS).l1 * T::kBytes, mfma_lhs(kS).major};
+  static constexpr Swizzle kSwizzle = first_swizzle(kAccess, {kS.m, kS.k * T::kBytes}, ROWBYTES, 1, 8, 1024);
   static_assert(kSwizzle.bank_param == 4, "MFMA operand reads are 16-byte: the search must return 16-byte atoms");
   static constexpr int kLineParam = kSwizzle.line_param;
   // byte offset of 16-byte chunk `chunk` of row `row`
@@ -202,42 +148,55 @@ __device__ __forceinline__ void store_result(const GemmParams &p, int32_t m, int
   }
 }
 
-// Epilogue of one 32x32 accumulator block.  The MFMA is issued with the operands swapped
-// (rhs fragment first), so register v of lane l holds D[m = l%32][n = 8*(v/4) + 4*(l/32) + v%4]:
-// four consecutive n per register quad, the transposed form of the <[2,32],[4,1],(0,1)>
-// accumulator fragments.
+// Epilogues of one accumulator block.  Every kernel here issues the matrix instruction with the operands
+// exchanged (rhs fragment in the first slot), so the block's registers follow mfma_acc_exchanged: a lane's
+// register quad holds four consecutive columns of one row.  Where each register sits is read off that layout
+// (acc_lane), e.g. for 32x32: register v of lane l holds D[l%32][8*(v/4) + 4*(l/32) + v%4].
+constexpr bool quads_run_along_rows(MfmaShape s) {
+  const AccLane a = acc_lane(mfma_acc_exchanged(s), s, 0);
+  return a.drow == 0 && a.dcol == 1 && a.qrow == 0;
+}
+static_assert(quads_run_along_rows(kMfma32x32x16) && quads_run_along_rows(kMfma16x16x32), "the packed epilogues store register quads as 8 contiguous bytes of a row");
 // Packed form: 16-bit row-major result, block fully in range, no accumulator input, RN: one
 // 8-byte store per quad.
 __device__ __forceinline__ void store_block_packed(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, const f32x16 &acc) {
-  char *row = p.d + ((int64_t)(m_base + (lane & 31)) * p.d_sm + n_base + 4 * (lane >> 5)) * 2;
+  const AccLane at = acc_lane(mfma_acc_exchanged(kMfma32x32x16), kMfma32x32x16, lane);
+  char *row = p.d + ((int64_t)(m_base + at.row) * p.d_sm + n_base + at.col) * 2;
   const bool f16 = p.d_dtype == KAPY_F16;
-  const float rs = p.row_scale ? p.row_scale[m_base + (lane & 31)] : 1.0f;
+  const float rs = p.row_scale ? p.row_scale[m_base + at.row] : 1.0f;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     uint16_t h[4];
     f32x4 cs = {1.0f, 1.0f, 1.0f, 1.0f};
-    if (p.row_scale) cs = *(const f32x4 *)(p.col_scale + n_base + 4 * (lane >> 5) + 8 * q);
+    if (p.row_scale) cs = *(const f32x4 *)(p.col_scale + n_base + at.col + at.qcol * q);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       float v = acc[4 * q + e];
       if (p.row_scale) v = __fmul_rn(v, __fmul_rn(rs, cs[e]));
-      if (has_tail(p)) v = apply_tail(p, v, p.bias ? load_as_f32(p.bias, p.bias_dtype, n_base + 4 * (lane >> 5) + 8 * q + e) : 0.f);
+      if (has_tail(p)) v = apply_tail(p, v, p.bias ? load_as_f32(p.bias, p.bias_dtype, n_base + at.col + at.qcol * q + e) : 0.f);
       h[e] = f16 ? f32_to_f16_rn(v) : f32_to_bf16_rn(v);
     }
     u32x2 w = {h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16)};
-    *(u32x2 *)(row + 16 * q) = w;
+    *(u32x2 *)(row + 2 * at.qcol * q) = w;
   }
 }
 // General form: any result type and strides, accumulator input, ragged edges.  Out of line: it is
 // large and off the roofline path.
-__device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, f32x16 acc) {
-  const int32_t m = m_base + (lane & 31);
-  for (int v = 0; v < 16; ++v) store_result(p, m, n_base + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), acc[v]);
+template <int REGS>
+__device__ __forceinline__ void store_block_elements(const GemmParams &p, MfmaShape s, int32_t m_base, int32_t n_base, int lane, const float (&acc)[REGS]) {
+  const AccLane at = acc_lane(mfma_acc_exchanged(s), s, lane);
+  for (int v = 0; v < REGS; ++v)
+    store_result(p, m_base + at.row + (v & 3) * at.drow + (v >> 2) * at.qrow, n_base + at.col + (v & 3) * at.dcol + (v >> 2) * at.qcol, acc[v]);
 }
-// 16x16 block: register v of lane l holds D[m = l%16][n = 4*(l/16) + v].
+__device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, f32x16 acc) {
+  float r[16];
+  for (int v = 0; v < 16; ++v) r[v] = acc[v];
+  store_block_elements(p, kMfma32x32x16, m_base, n_base, lane, r);
+}
 __device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_base, int32_t n_base, int lane, f32x4 acc) {
-  const int32_t m = m_base + (lane & 15);
-  for (int v = 0; v < 4; ++v) store_result(p, m, n_base + 4 * (lane >> 4) + v, acc[v]);
+  float r[4];
+  for (int v = 0; v < 4; ++v) r[v] = acc[v];
+  store_block_elements(p, kMfma16x16x32, m_base, n_base, lane, r);
 }
 
 // Packed epilogue (16-bit row-major result, 16-byte aligned rows, no accumulator input, RN) of one
@@ -254,13 +213,19 @@ struct PackedEpilogue {
   static constexpr int kChunks = WTN * 2 / 16, kRowsPerStore = 64 / kChunks, kStores = 32 / kRowsPerStore;
   static constexpr int kGroups = 64 / KM, kAccRegs = KM * KM / 64;
   static constexpr int kBlocksPerStrip = 32 / KM, kStrips = WTM / 32, kTn = WTN / KM;
-  static constexpr int kQuads = kAccRegs / 4, kQuadStep = 4 * kGroups;  // register quads of a block: 4 consecutive columns each, kQuadStep apart
+  // the accumulator fragments of a KM x KM block (the operand classes share them): a lane's register quads hold 4
+  // consecutive columns of one row, quads kQuadStep columns apart
+  static constexpr MfmaShape kBlock{KM, KM, 0, 0};
+  static constexpr Fragments kAccLayout = mfma_acc_exchanged(kBlock);
+  static constexpr int kQuads = kAccRegs / 4, kQuadStep = kQuads > 1 ? acc_lane(kAccLayout, kBlock, 0).qcol : 0;
+  static_assert(quads_run_along_rows(kBlock) && acc_lane_describes(kAccLayout, kBlock) && kAccLayout.loop_size({KM, KM}) == kAccRegs, "accumulator fragments");
   static_assert(WTM % 32 == 0 && 64 % kChunks == 0 && 32 % kRowsPerStore == 0, "strip geometry");
 
   // EPI: 0 = cast only, 1 = row and column scales
   template <bool F16, int EPI, typename Acc>
   static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
-    const int wrow = lane % KM, wcol = 4 * (lane / KM);        // this lane's row / first column in an accumulator block
+    const AccLane at = acc_lane(kAccLayout, kBlock, lane);
+    const int wrow = at.row, wcol = at.col;                    // this lane's row / first column in an accumulator block
     const int rrow = lane / kChunks, rchunk = lane % kChunks;  // and in a read-back instruction
 #pragma unroll
     for (int i = 0; i < kStrips; ++i) {
@@ -308,7 +273,8 @@ struct PackedEpilogue {
   static __device__ __forceinline__ void strips_tail(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip, int32_t m_wave, int32_t n_wave, int lane) {
     constexpr int kRowStrideF = WTN * 4 + 16, kChunksF = WTN / 8, kRowsPerPass = 64 / kChunksF, kPasses = 32 / kRowsPerPass;
     static_assert(32 * kRowStrideF <= kBytesPerWave && 64 % kChunksF == 0 && 32 % kRowsPerPass == 0, "fp32 strip geometry");
-    const int wrow = lane % KM, wcol = 4 * (lane / KM);
+    const AccLane at = acc_lane(kAccLayout, kBlock, lane);
+    const int wrow = at.row, wcol = at.col;
     const int rrow = lane / kChunksF, rchunk = lane % kChunksF;
     // the lane's 8 columns are the same in every pass and strip: their bias values are fetched once
     const int32_t nn = n_wave + rchunk * 8;
@@ -410,7 +376,7 @@ struct TnConfig {
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false, bool TAIL = false>
 __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
-  using L = TileLayout<C::kRowBytes>;
+  using L = TileLayout<C::kRowBytes, T>;
   constexpr int EB = T::kBytes, CH = T::kChunks;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
@@ -458,10 +424,12 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     for (int idx = 0; idx < C::kLoadsAPerWave + C::kLoadsBPerWave; ++idx) issue_load(stage, kt, idx);
   };
 
-  // LDS byte offsets of this lane's operand reads: row (lane % KM) of each KM-row block, 16-byte
-  // chunks of K-group (lane / KM) of the K slice kk.
-  constexpr int KM = T::kM, kGroups = 64 / KM;  // rows per operand block; K-groups of lanes
-  const uint32_t frag_row = lane % KM, frag_grp = lane / KM;
+  // LDS byte offsets of this lane's operand reads, from the operand fragments of the instruction: the lane's
+  // row of each KM-row block and, in K slice kk, the 16-byte chunks that hold its kpack consecutive K elements.
+  constexpr int KM = T::kM;  // rows per operand block
+  static_assert(T::kShape.m == KM && T::kShape.k == T::kSliceK && T::kShape.kpack * EB == 16 * CH, "policy and instruction shape disagree");
+  const OperandLane frag_at = operand_lane(T::kShape, lane);
+  const uint32_t frag_row = frag_at.row, frag_k0 = frag_at.k0;
 
   using Acc = typename T::Acc;
   constexpr int kAccRegs = KM * KM / 64;
@@ -497,13 +465,12 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   struct Frag {
     u32x4 c[CH];
   };
-  // Per-lane LDS offsets of the operand reads of slice kk, relative to the wave's rows of a stage:
-  // row (lane % 32) of each 32-row block, chunks (2*kk + lane/32)*CH .. +CH-1 of the row.
+  // Per-lane LDS offsets of the operand reads of slice kk, relative to the wave's rows of a stage.
   uint32_t frag_off[KK][CH];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-    for (int c = 0; c < CH; ++c) frag_off[kk][c] = L::offset(frag_row, (kGroups * kk + frag_grp) * CH + c);
+    for (int c = 0; c < CH; ++c) frag_off[kk][c] = L::offset(frag_row, ((kk * T::kSliceK + frag_k0) * EB) / 16 + c);
   const uint32_t a_rows = (wm * C::kWtm) * C::kRowBytes, b_rows = BM * C::kRowBytes + (wn * C::kWtn) * C::kRowBytes;
   // 32-row blocks are whole multiples of the swizzle period, so block i only adds i*32*rowBytes.
   static_assert((KM * C::kRowBytes) % (256 * L::kLineParam) == 0, "an operand block must span whole swizzle periods");
@@ -885,7 +852,7 @@ __device__ __forceinline__ uint32_t rhs_key(uint32_t row) { return ((row & 3) + 
 template <typename T, int BK, int STAGES, bool PACKED>
 __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   static_assert(T::kM == 16 && T::kBytes == 2 && BK % 32 == 0 && STAGES >= 3, "16x16x32 instruction, 16-bit operands");
-  using LA = TileLayout<BK * 2>;
+  using LA = TileLayout<BK * 2, T>;
   constexpr int kRowA = BK * 2, kRowB = kNBN * 2;
   constexpr int kBytesA = kNBM * kRowA, kBytesB = BK * kRowB, kStage = kBytesA + kBytesB;
   constexpr int kLoadsA = kBytesA / 1024 / 4, kLoadsB = kBytesB / 1024 / 4, kLoads = kLoadsA + kLoadsB;  // per wavefront per tile
@@ -935,9 +902,12 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
                                                16, (int)b_goff[idx - kLoadsA], jc * BK * ldb * 2, 0, 0);
   };
 
-  // Operand reads.  lhs: row (lane % 16) of each 16-row block, 16-byte chunk 4*kk + lane/16.
-  // rhs: k-rows kk*32 + 8*(lane/16) + 4*h + (lane%16)/4, columns 4*((lane%16)%4).. of each 16-column block.
-  const uint32_t grp = lane >> 4, l16 = lane & 15;
+  // Operand reads, from the operand fragments of the instruction (l16: the lane's row of an lhs block = its column of
+  // an rhs block; grp: which 8 of a slice's 32 K positions its registers hold).  lhs: row l16 of each 16-row block,
+  // 16-byte chunk 4*kk + grp.  rhs: the transposing read hands lane j of a 16-lane group column j of the four k-rows
+  // whose 8-byte pieces the group's lanes address, so lane l16 addresses k-row (8*grp + 4*h + l16/4), columns 4*(l16%4)..
+  const OperandLane frag_at = operand_lane(T::kShape, lane);
+  const uint32_t grp = frag_at.k0 / T::kShape.kpack, l16 = frag_at.row;
   uint32_t a_off[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) a_off[kk] = LA::offset(wm * 64 + l16, 4 * kk + grp);
@@ -1092,7 +1062,7 @@ enum OperandMode { kKContig = 0, kRowContig = 1, kStrided = 2 };
 
 template <typename T, bool PACKED>
 __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, int b_mode) {
-  using L = TileLayout<kSBK * 2>;
+  using L = TileLayout<kSBK * 2, T>;
   __shared__ __attribute__((aligned(1024))) char lds[(kSBM + kSBN) * kSBK * 2];
   char *sa = lds, *sb = lds + kSBM * kSBK * 2;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1145,7 +1115,8 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
   StagedRegs ra, rb;
   fetch(p.a, p.a_sm, p.a_sk, m0, p.M, a_mode, 0, ra);
   fetch(p.b, p.b_sn, p.b_sk, n0, p.N, b_mode, 0, rb);
-  const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
+  const OperandLane frag_at = operand_lane(T::kShape, lane);
+  const uint32_t frag_row = frag_at.row, frag_half = frag_at.k0 / T::kShape.kpack;  // the lane's row of a block; which half of a slice's 16 K
   for (int kt = 0; kt < KT; ++kt) {
     __syncthreads();  // every wave has finished reading the previous tile
     stash(sa, a_mode, ra);
@@ -1351,6 +1322,45 @@ int launch_f8(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
   }
 }
 
+// One matrix instruction on one wavefront, registers in and registers out: lhs / rhs hold each lane's operand
+// registers back to back (kpack elements per lane), acc gets each lane's accumulator registers.  The policy is
+// the one the kernels multiply with, so what this shows about register positions holds for them.
+template <typename T, bool EXCHANGED>
+__global__ __launch_bounds__(64) void probe_kernel(const char *lhs, const char *rhs, float *acc) {
+  const int lane = threadIdx.x;
+  constexpr int kLaneBytes = T::kShape.kpack * T::kBytes, kRegs = T::kShape.m * T::kShape.n / 64;
+  static_assert(kLaneBytes == 16 * T::kChunks, "a lane's operand registers are whole 16-byte chunks");
+  u32x4 a[T::kChunks], b[T::kChunks];
+#pragma unroll
+  for (int c = 0; c < T::kChunks; ++c) {
+    a[c] = *(const u32x4 *)(lhs + lane * kLaneBytes + 16 * c);
+    b[c] = *(const u32x4 *)(rhs + lane * kLaneBytes + 16 * c);
+  }
+  typename T::Acc d;
+#pragma unroll
+  for (int v = 0; v < kRegs; ++v) d[v] = 0.f;
+  d = EXCHANGED ? T::mfma(b, a, d) : T::mfma(a, b, d);
+#pragma unroll
+  for (int v = 0; v < kRegs; ++v) acc[lane * kRegs + v] = d[v];
+}
+template <typename T>
+int launch_probe(bool exchanged, const void *lhs, const void *rhs, float *acc, hipStream_t s) {
+  if (exchanged) probe_kernel<T, true><<<1, 64, 0, s>>>((const char *)lhs, (const char *)rhs, acc);
+  else probe_kernel<T, false><<<1, 64, 0, s>>>((const char *)lhs, (const char *)rhs, acc);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+// FIRST / SECOND: the fp8 formats of the instruction's first / second operand slot
+template <template <int, int> class P>
+int launch_probe_f8(int first_fmt, int second_fmt, bool exchanged, const void *lhs, const void *rhs, float *acc, hipStream_t s) {
+  switch (first_fmt * 2 + second_fmt) {
+  case 0: return launch_probe<P<0, 0>>(exchanged, lhs, rhs, acc, s);
+  case 1: return launch_probe<P<0, 1>>(exchanged, lhs, rhs, acc, s);
+  case 2: return launch_probe<P<1, 0>>(exchanged, lhs, rhs, acc, s);
+  default: return launch_probe<P<1, 1>>(exchanged, lhs, rhs, acc, s);
+  }
+}
+
 }  // namespace
 
 #ifndef KAPY_F8_STAGES
@@ -1504,14 +1514,38 @@ int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy
   return matmul_16bit(lhs, rhs, nullptr, result, cfg, epi, stream);
 }
 
+int kapy_mfma_probe(int32_t impl_way, int32_t lhs_dtype, int32_t rhs_dtype, int32_t exchanged, const void *lhs_regs, const void *rhs_regs,
+                    float *acc_regs, void *stream) {
+  if (!lhs_regs || !rhs_regs || !acc_regs) return fail(KAPY_ERR_INVALID, "mfma_probe: null register array");
+  const bool f8 = is_f8(lhs_dtype) && is_f8(rhs_dtype), b16 = (lhs_dtype == KAPY_F16 || lhs_dtype == KAPY_BF16) && rhs_dtype == lhs_dtype;
+  const bool way16 = impl_way == KAPY_MFMA_32X32X16_16B || impl_way == KAPY_MFMA_16X16X32_16B;
+  const bool way8 = impl_way == KAPY_MFMA_16X16X128_F8 || impl_way == KAPY_MFMA_32X32X64_F8;
+  if (!way16 && !way8) return fail(KAPY_ERR_INVALID, "mfma_probe: impl_way must name a matrix instruction of gfx950 (16..19), not %d", impl_way);
+  if ((way16 && !b16) || (way8 && !f8)) return fail(KAPY_ERR_VERIFY, "mfma_probe: operand element types do not fit the instruction");
+  int rc = ensure_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const bool ex = exchanged != 0;
+  if (way16) {
+    const bool bf = lhs_dtype == KAPY_BF16;
+    if (impl_way == KAPY_MFMA_32X32X16_16B) return bf ? launch_probe<Bf16>(ex, lhs_regs, rhs_regs, acc_regs, s) : launch_probe<F16>(ex, lhs_regs, rhs_regs, acc_regs, s);
+    return bf ? launch_probe<Bf16M16>(ex, lhs_regs, rhs_regs, acc_regs, s) : launch_probe<F16M16>(ex, lhs_regs, rhs_regs, acc_regs, s);
+  }
+  // exchanged: the rhs fragment sits in the first operand slot, so the first format selector is the rhs's
+  const int lf = lhs_dtype == KAPY_F8E5M2, rf = rhs_dtype == KAPY_F8E5M2;
+  const int first = ex ? rf : lf, second = ex ? lf : rf;
+  if (impl_way == KAPY_MFMA_16X16X128_F8) return launch_probe_f8<F8M16>(first, second, ex, lhs_regs, rhs_regs, acc_regs, s);
+  return launch_probe_f8<F8>(first, second, ex, lhs_regs, rhs_regs, acc_regs, s);
+}
+
 int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out) {
   if (!out) return fail(KAPY_ERR_INVALID, "matmul_lds_layout: null result");
   if (operand_dtype != KAPY_F16 && operand_dtype != KAPY_BF16)
     return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: only f16 / bf16 operand tiles are described here");
   Swizzle s;
   switch (tile_k) {
-  case 32: s = TileLayout<64>::kSwizzle; break;
-  case 64: s = TileLayout<128>::kSwizzle; break;
+  case 32: s = TileLayout<64, Bf16M16>::kSwizzle; break;   // (f16 and bf16 share the operand layouts; the search gives the
+  case 64: s = TileLayout<128, Bf16M16>::kSwizzle; break;  //  same parameters for the 32x32x16 instruction)
   default: return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: tile_k must be 32 or 64");
   }
   s.stride0 = tile_k;  // the search runs on bytes; report the row stride in elements

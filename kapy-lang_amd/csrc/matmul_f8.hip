@@ -17,14 +17,30 @@
 #include "common.hpp"
 #include "layout.hpp"
 #include "matmul_params.hpp"
+#include "mfma.hpp"
 #include "numeric.hpp"
 
 namespace kapy {
 namespace {
 
-typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Both decode-shaped kernels multiply with v_mfma_scale_f32_16x16x128_f8f6f4 issued as documented (activation block
+// in the first operand slot, weight block in the second), so a lane's registers sit where the instruction's own
+// fragments layouts say: operand registers = 32 consecutive K bytes of row (lhs) / column (rhs) operand_lane().row,
+// accumulator register v = element (row + v, col) of the 16x16 block (mfma_acc: a quad runs down a column).
+constexpr MfmaShape kF8Shape = kMfma16x16x128F8;
+constexpr bool acc_quad_runs_down_a_column() {
+  const AccLane a = acc_lane(mfma_acc(kF8Shape), kF8Shape, 0);
+  return a.drow == 1 && a.dcol == 0 && acc_lane_describes(mfma_acc(kF8Shape), kF8Shape);
+}
+static_assert(acc_quad_runs_down_a_column(), "accumulator fragments of the 16x16x128 instruction");
+template <int A_FMT, int B_FMT>
+__device__ __forceinline__ f32x4 mfma_f8(const i32x8 &a, const i32x8 &b, f32x4 c) {
+  const u32x4 av[2] = {{(uint32_t)a[0], (uint32_t)a[1], (uint32_t)a[2], (uint32_t)a[3]}, {(uint32_t)a[4], (uint32_t)a[5], (uint32_t)a[6], (uint32_t)a[7]}};
+  const u32x4 bv[2] = {{(uint32_t)b[0], (uint32_t)b[1], (uint32_t)b[2], (uint32_t)b[3]}, {(uint32_t)b[4], (uint32_t)b[5], (uint32_t)b[6], (uint32_t)b[7]}};
+  return F8M16<A_FMT, B_FMT>::mfma(av, bv, c);
+}
 
 struct F8Params {
   const uint8_t *a, *b;
@@ -91,7 +107,8 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
   __shared__ float partial[kSkinnyWaves][NG][16][16 + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int32_t n0 = blockIdx.x * 16 * NG, m0 = blockIdx.y * 16;
-  const int32_t row = lane & 15, kq = (lane >> 4) * 32;  // this lane's row/column and its 32-byte K quarter
+  const OperandLane frag_at = operand_lane(kF8Shape, lane);
+  const int32_t row = frag_at.row, kq = frag_at.k0;  // this lane's row/column and its 32-byte K quarter
   const int32_t steps = p.K / 128, per_wave = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
   const int32_t s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
   f32x4 acc[NG];
@@ -111,13 +128,13 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
     for (int u = 0; u < CH; ++u)
 #pragma unroll
       for (int g = 0; g < NG; ++g)
-        acc[g] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aw[u], bw[g][u], acc[g], A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+        acc[g] = mfma_f8<A_FMT, B_FMT>(aw[u], bw[g][u], acc[g]);
   }
-  // accumulator register v of lane l: row 4*(l/16) + v, column l%16
+  const AccLane acc_at = acc_lane(mfma_acc(kF8Shape), kF8Shape, lane);
 #pragma unroll
   for (int g = 0; g < NG; ++g)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) partial[wave][g][4 * (lane >> 4) + v][lane & 15] = acc[g][v];
+    for (int v = 0; v < 4; ++v) partial[wave][g][acc_at.row + v][acc_at.col] = acc[g][v];
   __syncthreads();
   for (int e = threadIdx.x; e < NG * 256; e += 64 * kSkinnyWaves) {
     const int g = e >> 8, m = (e >> 4) & 15, n = e & 15;
@@ -184,8 +201,9 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
     for (int i = 0; i < 4; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + 4096 + i * 1024), 16, (int)a_off[i], chunk * kStreamChunk, 0, 0);
   };
-  // operand reads: row lane%16, K-group lane/16 of a 128-byte step: chunks 8*step + 2*group, +1
-  const int r16 = lane & 15, grp = lane >> 4;
+  // operand reads: the lane's row and its 32 K bytes of a 128-byte step: chunks 8*step + 2*group, +1
+  const OperandLane frag_at = operand_lane(kF8Shape, lane);
+  const int r16 = frag_at.row, grp = frag_at.k0 / kF8Shape.kpack;
   uint32_t rd[2][2];
 #pragma unroll
   for (int st = 0; st < 2; ++st)
@@ -213,14 +231,15 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
     for (int st = 0; st < 2; ++st) {
       const i32x8 av = {a[st][0][0], a[st][0][1], a[st][0][2], a[st][0][3], a[st][1][0], a[st][1][1], a[st][1][2], a[st][1][3]};
       const i32x8 wv = {w[st][0][0], w[st][0][1], w[st][0][2], w[st][0][3], w[st][1][0], w[st][1][1], w[st][1][2], w[st][1][3]};
-      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, wv, acc, A_FMT, B_FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+      acc = mfma_f8<A_FMT, B_FMT>(av, wv, acc);
     }
   }
-  // accumulator register v of lane l: row 4*(l/16) + v, column l%16; the four K ranges meet in LDS
+  // the four K ranges meet in LDS
+  const AccLane acc_at = acc_lane(mfma_acc(kF8Shape), kF8Shape, lane);
   __syncthreads();  // every wave is done with its ring
   float *partial = (float *)ring;  // [wave][16][17]
 #pragma unroll
-  for (int v = 0; v < 4; ++v) partial[(wave * 16 + 4 * (lane >> 4) + v) * 17 + (lane & 15)] = acc[v];
+  for (int v = 0; v < 4; ++v) partial[(wave * 16 + acc_at.row + v) * 17 + acc_at.col] = acc[v];
   __syncthreads();
   {
     const int m = threadIdx.x >> 4, n = threadIdx.x & 15;

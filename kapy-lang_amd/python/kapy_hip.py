@@ -33,6 +33,7 @@ EXPORTS = [
     "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
+    "kapy_mfma_probe",
 ]
 
 
@@ -156,6 +157,7 @@ def lib():
     L.kapy_matmul_fused.argtypes = [P(Global), P(Global), P(Global), P(MatmulEpilogue), P(MatmulCfg), vp]
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
+    L.kapy_mfma_probe.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp]
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
     L.kapy_smem_plan.restype = i64
     L.kapy_smem_plan.argtypes = [P(SmemBuffer), i32, i64]
@@ -413,3 +415,15 @@ def run_mlir(text, args, grid, func_name=None, stream=None):
 def change(in_ptr, src, dst, shape, out_ptr, stream=None):
     check(lib().kapy_change(C.c_void_p(in_ptr), C.byref(src), C.byref(dst), A2(*shape), C.c_void_p(out_ptr),
                             stream if stream is not None else current_stream()))
+
+
+def matmul_layouts(impl_way, which):
+    """(fragments layout, (m, n, k)) of the lhs (0), rhs (1), accumulator (2) or accumulator with the operands exchanged (3)."""
+    f, mnk = Fragments(), (C.c_int32 * 3)()
+    check(lib().kapy_matmul_layouts(impl_way, which, C.byref(f), mnk))
+    return f, tuple(mnk)
+
+
+def mfma_probe(impl_way, lhs_dtype, rhs_dtype, exchanged, lhs_ptr, rhs_ptr, acc_ptr, stream=None):
+    check(lib().kapy_mfma_probe(impl_way, lhs_dtype, rhs_dtype, int(exchanged), C.c_void_p(lhs_ptr), C.c_void_p(rhs_ptr), C.c_void_p(acc_ptr),
+                                stream if stream is not None else current_stream()))

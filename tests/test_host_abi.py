@@ -122,20 +122,25 @@ def test_swizzle_agrees_with_oracle_and_matmul_layout_is_searched(ko):
             for i0 in range(0, 64, 3):
                 for i1 in range(0, s0, 5):
                     assert L.kapy_swizzle_offset(C.byref(sw), bits, i0, i1) == O.ko_swizzle_offset(i0, i1, s0, 1, bits, bp, lp, 64)
-    # the LDS layout the matmul uses must be the first hit of the reference's search run on the MFMA operand layout
+    # the LDS layout the matmul uses must be the first hit of the reference's search run on the operand layout of the matrix
+    # instruction its kernels are built on (16x16x32 by default; 32x32x16 gives the same parameters)
     for tile_k in (32, 64):
-        f, mnk = kh.Fragments(), (C.c_int32 * 3)()
-        assert L.kapy_matmul_layouts(kh.MFMA_32X32X16_16B, 0, C.byref(f), mnk) == 0 and list(mnk) == [32, 32, 16]
-        pairs = (C.c_int32 * 64)()
-        n = L.kapy_swizzle_search(C.byref(f), kh.A2(32, 16), tile_k, 1, 16, 1024, pairs, 32)
-        op = (C.c_int64 * 64)()
-        g = ko.Fragments.make(*f.astuple())
-        assert n == O.ko_swizzle_search(C.byref(g), kh.A2(32, 16), tile_k, 1, 16, 1024, 64, 64, op, 32) and n > 0
-        assert [pairs[i] for i in range(2 * n)] == [op[i] for i in range(2 * n)]
+        found = []
+        for way, want_mnk in ((kh.MFMA_16X16X32_16B, [16, 16, 32]), (kh.MFMA_32X32X16_16B, [32, 32, 16])):
+            f, mnk = kh.Fragments(), (C.c_int32 * 3)()
+            assert L.kapy_matmul_layouts(way, 0, C.byref(f), mnk) == 0 and list(mnk) == want_mnk
+            shape = kh.A2(mnk[0], mnk[2])
+            pairs = (C.c_int32 * 64)()
+            n = L.kapy_swizzle_search(C.byref(f), shape, tile_k, 1, 16, 1024, pairs, 32)
+            op = (C.c_int64 * 64)()
+            g = ko.Fragments.make(*f.astuple())
+            assert n == O.ko_swizzle_search(C.byref(g), shape, tile_k, 1, 16, 1024, 64, 64, op, 32) and n > 0
+            assert [pairs[i] for i in range(2 * n)] == [op[i] for i in range(2 * n)]
+            assert pairs[0] == 4 and (pairs[0], 1) not in {(pairs[2 * i], pairs[2 * i + 1]) for i in range(n)}  # unswizzled conflicts
+            found.append((pairs[0], pairs[1]))
         sw = kh.Swizzling()
         assert L.kapy_matmul_lds_layout(kh.BF16, tile_k, C.byref(sw)) == 0
-        assert (sw.stride0, sw.stride1, sw.bank_param, sw.line_param) == (tile_k, 1, pairs[0], pairs[1])
-        assert pairs[0] == 4 and (pairs[0], 1) not in {(pairs[2 * i], pairs[2 * i + 1]) for i in range(n)}  # unswizzled conflicts
+        assert (sw.stride0, sw.stride1, sw.bank_param, sw.line_param) == (tile_k, 1) + found[0] and found[0] == found[1]
 
 
 def test_mfma_layouts_are_consistent_fragments(ko):
@@ -165,7 +170,18 @@ def test_mfma_layouts_are_consistent_fragments(ko):
         L.kapy_fragments_map(C.byref(fr[0]), kh.A2(m, k), 2, kh.A2(5, 0), o0)
         L.kapy_fragments_map(C.byref(fr[0]), kh.A2(m, k), 2, kh.A2(5, kpack - 1), o1)
         assert o0[0] == o1[0] == 5 and o1[1] - o0[1] == kpack - 1
+        # which = 3: the accumulator with the operands exchanged holds the transposed block, i.e. is the transposed layout
+        ex, tr = kh.Fragments(), kh.Fragments()
+        assert L.kapy_matmul_layouts(way, 3, C.byref(ex), None) == 0
+        assert L.kapy_fragments_transpose(C.byref(fr[2]), C.byref(tr)) == 0 and bytes(ex) == bytes(tr)
+        o2, o3 = kh.A2(0, 0), kh.A2(0, 0)
+        for lane in (0, 17, 63):
+            for iv in range(m * n // 64):
+                L.kapy_fragments_map(C.byref(fr[2]), kh.A2(m, n), 2, kh.A2(lane, iv), o2)
+                L.kapy_fragments_map(C.byref(ex), kh.A2(m, n), 2, kh.A2(lane, iv), o3)
+                assert (o2[0], o2[1]) == (o3[1], o3[0])
     assert L.kapy_matmul_layouts(kh.MMA_M16N8K8_TF32, 0, C.byref(kh.Fragments()), None) == kh.ERR_UNSUPPORTED
+    assert L.kapy_matmul_layouts(kh.MFMA_16X16X32_16B, 4, C.byref(kh.Fragments()), None) == kh.ERR_INVALID
 
 
 def _g(dtype=kh.F16, m=16, n=16, s0=None, s1=1, buf=None):

@@ -238,8 +238,16 @@ typedef struct kapy_matmul_cfg {
   int32_t stages;                /* depth of the LDS ring in tiles (the reference fixture uses 2); 25 = the 2.5-tile
                                     ring of half-operand units; 0 = library's choice */
   int32_t waves;                 /* wavefronts per workgroup (num_warps of the reference); 0 = library's choice */
-  int32_t reserved;
+  int32_t split_k;               /* workgroups that share one output tile, each multiplying one part of K (powers of two up to 8);
+                                    1 = never split; 0 = library's choice: it splits only when a workspace is given and the
+                                    result has too few 128 x 128 tiles to occupy the device */
+  void *workspace;               /* device memory for the partial sums and arrival counters of a split K, or NULL.  Its first
+                                    16 KiB (the counters) must be zero before its first use and every call leaves them zero;
+                                    calls that share a workspace must not overlap in time */
+  int64_t workspace_bytes;       /* kapy_matmul_workspace_bytes(m, n) is enough for any split of an [m x n] result */
 } kapy_matmul_cfg;
+/* Workspace size that lets the library split K for an [m x n] result whichever way it chooses. */
+int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n);
 
 /* kapy.matmul — create_matmul(lhs, rhs, acc, implWay), python/src/ir.cc:1101-1105; verifier
  * lib/Dialect/Kapy/IR/Kapy.cpp:451-574; lowering MatmulOpToLLVM.cpp:58-311 with the

@@ -376,7 +376,7 @@ class OpBuilder {
       throw Error(KAPY_ERR_UNSUPPORTED, "matmul: the ops on its result must be [mulf splat] [addf bias row] [activation] [fptofp]");
     const Node &mm = nodes_[cur];
     const kapy_global lhs = view_of(nodes_[mm.a]), rhs = view_of(nodes_[mm.b]);
-    kapy_matmul_cfg cfg = {mm.impl_way, 0, 0, 0, KAPY_RN, 0, 0, 0};
+    kapy_matmul_cfg cfg = {mm.impl_way, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
     if (tail) {
       if (mm.c >= 0) throw Error(KAPY_ERR_UNSUPPORTED, "matmul: an accumulator input and a fused tail do not combine");
       check(kapy_matmul_fused(&lhs, &rhs, &out, &epi, &cfg, stream_));

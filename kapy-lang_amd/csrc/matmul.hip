@@ -349,6 +349,63 @@ __device__ __forceinline__ void tile_of_block(const GemmParams &p, int32_t &tm, 
   tn = in_group / rows;
 }
 
+// Split K (GemmParams::split_k): workgroup (tile, blockIdx.y) multiplies the blockIdx.y-th part of K.  Narrows the
+// kernel's own copy of the parameters to that part and returns the split index.
+__device__ __forceinline__ int32_t enter_split(GemmParams &p, int element_bytes) {
+  const int32_t split = blockIdx.y;
+  if (p.split_k > 1) {
+    const int32_t ks = p.K / p.split_k;  // (the host only splits a K that divides into whole K-tiles per part)
+    p.a += (int64_t)split * ks * p.a_sk * element_bytes;
+    p.b += (int64_t)split * ks * p.b_sk * element_bytes;
+    p.K = ks;
+  }
+  return split;
+}
+// The meeting point: every workgroup of a tile leaves its accumulators in the workspace as they sit in registers
+// (quad by quad, thread-contiguous: the reader is the same thread of another workgroup, so no layout is involved) and
+// counts itself; the one that arrives last gets `true` with `acc` replaced by the sum of all parts IN SPLIT ORDER (the
+// result does not depend on which workgroup was last), and sets the counter back to zero for the next call.  Nobody
+// waits for anybody.  The release / acquire pair at device scope makes the parts written by workgroups on other XCDs
+// (other L2s) visible to the reader.  `lds_word`: 4 bytes of LDS that no wave uses at this point.
+template <int THREADS, typename Acc, int TM, int TN>
+__device__ __forceinline__ bool split_k_meet(const GemmParams &p, int32_t tile, int32_t split, Acc (&acc)[TM][TN], uint32_t *lds_word) {
+  constexpr int kQuads = sizeof(Acc) / 16, kPerThread = TM * TN * kQuads;
+  f32x4 *base = (f32x4 *)p.partial + (int64_t)tile * p.split_k * (kPerThread * THREADS) + threadIdx.x;
+  f32x4 *mine = base + (int64_t)split * (kPerThread * THREADS);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < kQuads; ++q) {
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+        mine[((i * TN + j) * kQuads + q) * THREADS] = v;
+      }
+  __syncthreads();  // the whole workgroup's part is written (workgroup-scope release) ...
+  if (threadIdx.x == 0) *lds_word = __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);  // ... and published
+  __syncthreads();
+  const uint32_t arrived_before = *lds_word;
+  __syncthreads();  // (the word's LDS may be reused from here on)
+  if (arrived_before != (uint32_t)p.split_k - 1) return false;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < kQuads; ++q) {
+        const f32x4 *src = base + ((i * TN + j) * kQuads + q) * THREADS;
+        f32x4 sum = src[0];
+        for (int sp = 1; sp < p.split_k; ++sp) sum += src[(int64_t)sp * (kPerThread * THREADS)];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
+      }
+  if (threadIdx.x == 0) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
 // ---------------------------------------------------------------------------------------------
 // TN kernel.  BM x BN x BK workgroup tile, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN)
 // block of 32x32 accumulators.  STAGES-deep LDS ring filled by LDS-direct loads.
@@ -385,6 +442,10 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   int32_t tm, tn;
   tile_of_block(p, tm, tn);
   const int32_t m0 = tm * BM, n0 = tn * BN;
+  // (the 128 x 128 builds, which serve the shapes with few tiles, can split K across workgroups)
+  constexpr bool kCanSplit = BM == 128 && BN == 128 && STAGES == kRing25;
+  int32_t split = 0;
+  if constexpr (kCanSplit) split = enter_split(p, EB);
 
   // Per-lane global byte offsets of the chunks this lane fetches, one per load instruction.
   // Instruction q of an operand fills LDS bytes [q*1024, q*1024+1024); this lane's 16 bytes sit at
@@ -808,6 +869,13 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     trace[257] = __builtin_readcyclecounter();  // end of the K loop
   }
 #endif
+  if constexpr (kCanSplit) {
+    if (p.split_k > 1) {
+      __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+      __builtin_amdgcn_s_barrier();  // every wave has left the ring
+      if (!split_k_meet<C::kThreads>(p, tm + tn * p.tiles_m, split, acc, (uint32_t *)lds)) return;
+    }
+  }
   if constexpr (PACKED) {
     static_assert(PackedEpilogue<KM, C::kWtm, C::kWtn>::kBytesPerWave * C::kWaves <= C::kLdsBytes, "two strips per wavefront must fit the ring");
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
@@ -864,6 +932,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   int32_t tm, tn;
   tile_of_block(p, tm, tn);
   const int32_t m0 = tm * kNBM, n0 = tn * kNBN;
+  const int32_t split = enter_split(p, 2);
   const int32_t ldb = (int32_t)p.b_sk;  // elements between consecutive k-rows of the rhs
   const int KT = p.K / BK;
 
@@ -995,6 +1064,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   if (kt < KT) tile_step(kt, P0{});
   __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
   __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space by the packed epilogue
+  if (p.split_k > 1 && !split_k_meet<256>(p, tm + tn * p.tiles_m, split, acc, (uint32_t *)lds)) return;
   if constexpr (PACKED) {
     static_assert(PackedEpilogue<16, 64, 64>::kBytesPerWave * 4 <= STAGES * kStage, "two strips per wavefront must fit the ring");
     PackedEpilogue<16, 64, 64>::run(p, acc, lds + wave * PackedEpilogue<16, 64, 64>::kBytesPerWave, m0 + wm * 64, n0 + wn * 64, lane);
@@ -1181,7 +1251,9 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
   }
   p.tiles_m = (p.M + BM - 1) / BM;  // (only the ring variants are launched with tiles that hang over an edge)
   p.tiles_n = (p.N + BN - 1) / BN;
-  kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(C::kThreads), C::kLdsBytes, s>>>(p);
+  constexpr bool kCanSplit = BM == 128 && BN == 128 && STAGES == kRing25;
+  if (!kCanSplit) p.split_k = 1;
+  kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k), dim3(C::kThreads), C::kLdsBytes, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }
@@ -1230,7 +1302,7 @@ int launch_nn(GemmParams p, hipStream_t s) {
     }
     configured[packed] = true;
   }
-  dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k);
   if (packed) nn_kernel<T, BK, STAGES, true><<<grid, dim3(256), kLds, s>>>(p);
   else nn_kernel<T, BK, STAGES, false><<<grid, dim3(256), kLds, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
@@ -1241,6 +1313,7 @@ template <typename T>
 int launch_staged(GemmParams p, int a_mode, int b_mode, hipStream_t s) {
   p.tiles_m = (p.M + kSBM - 1) / kSBM;
   p.tiles_n = (p.N + kSBN - 1) / kSBN;
+  p.split_k = 1;
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
   if (packed_epilogue(p)) staged_kernel<T, true><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
   else staged_kernel<T, false><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
@@ -1311,6 +1384,8 @@ const TnVariant kTnVariants[] = {
 
 int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
 
+int64_t split_workspace_bytes(int64_t tiles, int split) { return kSplitCounterBytes + tiles * split * (128 * 128 * 4); }
+
 template <int BM, int BN, int BK, int WM, int WN, int S>
 int launch_f8(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
   // the kernel issues mfma(rhs fragment, lhs fragment): the first format selector is the rhs's
@@ -1363,6 +1438,44 @@ int launch_probe_f8(int first_fmt, int second_fmt, bool exchanged, const void *l
 
 }  // namespace
 
+// Decides whether the 128 x 128 tiled kernels split K for this problem and points the parameters at the workspace.
+// cfg.split_k = 1 or no workspace: never.  0: when the tiles alone would leave at least half the device idle, the
+// largest power of two that keeps tiles * split within the CUs, leaves every part at least four K-tiles and fits the
+// workspace.  An explicit split that cannot be honoured is an error.
+int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k) {
+  p.split_k = 1;
+  p.partial = nullptr;
+  p.counters = nullptr;
+  if (c.split_k < 0 || c.split_k > kMaxSplitK || (c.split_k & (c.split_k - 1)))
+    return fail(KAPY_ERR_INVALID, "matmul: split_k must be 0 (library's choice) or a power of two up to %d, not %d", kMaxSplitK, c.split_k);
+  if (c.split_k == 1) return KAPY_OK;
+  if (!c.workspace) {
+    if (c.split_k > 1) return fail(KAPY_ERR_INVALID, "matmul: split_k = %d needs a workspace (kapy_matmul_workspace_bytes)", c.split_k);
+    return KAPY_OK;
+  }
+  const int64_t tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  auto fits = [&](int sp) {
+    return p.K % (tile_k * sp) == 0 && tiles <= kSplitCounterBytes / 4 && split_workspace_bytes(tiles, sp) <= c.workspace_bytes &&
+           ((uintptr_t)c.workspace & 15) == 0;
+  };
+  int split = 1;
+  if (c.split_k > 1) {
+    if (!fits(c.split_k))
+      return fail(KAPY_ERR_UNSUPPORTED, "matmul: cannot split K = %d into %d parts of whole %d-wide K-tiles with a 16-byte aligned workspace of %lld bytes (%lld needed)",
+                  p.K, c.split_k, tile_k, (long long)c.workspace_bytes, (long long)split_workspace_bytes(tiles, c.split_k));
+    split = c.split_k;
+  } else if (tiles * 2 <= device_cus()) {
+    for (int sp = 2; sp <= kMaxSplitK && tiles * sp <= device_cus(); sp *= 2)
+      if (fits(sp) && p.K / (tile_k * sp) >= 4) split = sp;
+  }
+  if (split > 1) {
+    p.split_k = split;
+    p.counters = (uint32_t *)c.workspace;
+    p.partial = (float *)((char *)c.workspace + kSplitCounterBytes);
+  }
+  return KAPY_OK;
+}
+
 #ifndef KAPY_F8_STAGES
 #define KAPY_F8_STAGES kRing25
 #endif
@@ -1388,7 +1501,7 @@ namespace {
 // kapy.matmul with, optionally, the elementwise ops that follow it on the accumulator fused into the kernel's epilogue.
 int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                  const kapy_matmul_cfg *cfg, const kapy_matmul_epilogue *epi, void *stream) {
-  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0};
+  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
   if (cfg) c = *cfg;
   int rc = verify_matmul(lhs, rhs, acc, result, c.impl_way);
   if (rc) return rc;
@@ -1431,6 +1544,9 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
   p.d_dtype = result->dtype;
   p.rz = c.rmode == KAPY_RZ;
   p.tiles_m = p.tiles_n = 0;
+  p.split_k = 1;
+  p.partial = nullptr;
+  p.counters = nullptr;
   if (p.M == 0 || p.N == 0) return KAPY_OK;
   const bool bf16 = lhs->dtype == KAPY_BF16;
 
@@ -1451,6 +1567,12 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
       if ((!whole_k && (v.stages != kRing25 || p.K % 8)) || (!whole_tiles && v.stages != kRing25)) continue;
       // with a free choice, a 256x256 tiling with fewer tiles than CUs yields to 128x128
       if (free_choice && v.bm == 256 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) < device_cus()) continue;
+      if (v.bm == 128 && v.stages == kRing25) {
+        rc = plan_split_k(p, c, v.bk);
+        if (rc) return rc;
+      } else if (c.split_k > 1 && c.tile_m) {
+        return fail(KAPY_ERR_UNSUPPORTED, "matmul: only the 128 x 128 tiles split K");
+      }
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }
@@ -1468,6 +1590,8 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
                                     {32, 4, launch_nn<Bf16M16, 32, 4>, launch_nn<F16M16, 32, 4>}};
     for (const NnVariant &v : kNn) {
       if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;
+      rc = plan_split_k(p, c, v.bk);
+      if (rc) return rc;
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }
@@ -1491,6 +1615,13 @@ extern "C" {
 int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                 const kapy_matmul_cfg *cfg, void *stream) {
   return matmul_16bit(lhs, rhs, acc, result, cfg, nullptr, stream);
+}
+
+int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n) {
+  if (m <= 0 || n <= 0) return 0;
+  // a split keeps tiles * parts within the CUs of the device; without a device, the largest split of every tile
+  const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128);
+  return split_workspace_bytes(tiles, kMaxSplitK);
 }
 
 int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *result, const kapy_matmul_epilogue *epi,

@@ -161,6 +161,10 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 #define KAPY_F8_TILED_FROM_M 81
 #endif
 constexpr int kTiledFromM = KAPY_F8_TILED_FROM_M;
+#ifndef KAPY_F8_TILED_FROM_M_SPLIT
+#define KAPY_F8_TILED_FROM_M_SPLIT 17
+#endif
+constexpr int kTiledFromMSplit = KAPY_F8_TILED_FROM_M_SPLIT;  // the same threshold when K can be split across workgroups
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
 template <int A_FMT, int B_FMT>
 __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Params p) {
@@ -275,7 +279,10 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   if (p.M == 0 || p.N == 0) return KAPY_OK;
   bool k_contig = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(a, 1) == 16 && vector_bytes(b, 0) == 16 && p.K % 128 == 0 && p.K > 0;
   // Many rows: the tiled LDS-direct kernel (MFMA-bound).  Few rows: the skinny kernel (HBM-bound).
-  if (k_contig && p.M >= kTiledFromM && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
+  // With a workspace the tiled kernel can split K over several workgroups per tile, which fills the device at few rows too.
+  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
+  if (cfg) c = *cfg;
+  if (k_contig && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
     GemmParams g;
     g.a = (const char *)p.a; g.b = (const char *)p.b; g.acc = nullptr; g.d = p.d;
     g.row_scale = row_scale; g.col_scale = col_scale;
@@ -284,7 +291,10 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     g.acc_sm = g.acc_sn = 0; g.d_sm = p.d_sm; g.d_sn = p.d_sn;
     g.M = p.M; g.N = p.N; g.K = p.K;
     g.acc_dtype = -1; g.d_dtype = p.d_dtype; g.rz = p.rz; g.tiles_m = g.tiles_n = 0;
-    int rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), s);
+    int rc = plan_split_k(g, c, 128);
+    if (rc) return rc;
+    if (p.M < (g.split_k > 1 ? kTiledFromMSplit : kTiledFromM)) rc = KAPY_ERR_UNSUPPORTED;  // few rows: the streaming kernels below
+    else rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
   }
   if (k_contig && p.K % (kStreamWaves * kStreamChunk) == 0 && (p.M + 15) / 16 <= 65535 && p.a_sm * 16 < (int64_t(1) << 31) &&

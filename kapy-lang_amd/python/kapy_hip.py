@@ -33,7 +33,7 @@ EXPORTS = [
     "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
-    "kapy_mfma_probe",
+    "kapy_mfma_probe", "kapy_matmul_workspace_bytes",
 ]
 
 
@@ -87,7 +87,8 @@ class EwInst(C.Structure):
 
 class MatmulCfg(C.Structure):
     _fields_ = [("impl_way", C.c_int32), ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
-                ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("reserved", C.c_int32)]
+                ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("split_k", C.c_int32),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64)]
 
 
 class MatmulEpilogue(C.Structure):
@@ -154,6 +155,8 @@ def lib():
     L.kapy_elementwise_source.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), C.c_char_p, i64, P(i64), P(i64)]
     L.kapy_fptofp.argtypes = [P(Global), P(Global), i32, vp]
     L.kapy_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
+    L.kapy_matmul_workspace_bytes.restype = i64
+    L.kapy_matmul_workspace_bytes.argtypes = [i64, i64]
     L.kapy_matmul_fused.argtypes = [P(Global), P(Global), P(Global), P(MatmulEpilogue), P(MatmulCfg), vp]
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
@@ -167,7 +170,8 @@ def lib():
     L.kapy_parse_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i32), P(i32), P(i32)]
     for name in EXPORTS:
         f = getattr(L, name)
-        if name not in ("kapy_last_error", "kapy_smem_plan", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset"):
+        if name not in ("kapy_last_error", "kapy_smem_plan", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset",
+                        "kapy_matmul_workspace_bytes"):
             f.restype = C.c_int
     _lib = L
     return L
@@ -356,23 +360,38 @@ def fptofp(src, dst, rmode=RN, stream=None):
     check(lib().kapy_fptofp(C.byref(src), C.byref(dst), rmode, stream if stream is not None else current_stream()))
 
 
-def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stages=0, waves=0, stream=None):
-    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, 0)
-    check(lib().kapy_matmul(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
-                            C.byref(cfg), stream if stream is not None else current_stream()))
+def _workspace(workspace):
+    """(pointer, bytes) of a workspace given as None, a (pointer, bytes) pair or a torch tensor."""
+    if workspace is None:
+        return None, 0
+    if isinstance(workspace, tuple):
+        return workspace
+    return workspace.data_ptr(), workspace.numel() * workspace.element_size()
+
+
+def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stages=0, waves=0, split_k=0, workspace=None,
+           stream=None):
+    """workspace: zero-initialised device memory (a torch tensor or a (pointer, bytes) pair) that lets the library split K."""
+    ws, ws_bytes = _workspace(workspace)
+    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, split_k, ws, ws_bytes)
+    fn = lib().kapy_matmul
+    check(fn(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
+             C.byref(cfg), stream if stream is not None else current_stream()))
 
 
 def matmul_fused(lhs, rhs, result, bias=None, alpha=1.0, act=-1, act_operand=0.0, tile=(0, 0, 0), stages=0, stream=None):
     """result = cast(act(lhs @ rhs * alpha + bias)): the elementwise tail runs in the GEMM's epilogue."""
     epi = MatmulEpilogue(C.pointer(bias) if bias is not None else None, alpha, act, act_operand)
-    cfg = MatmulCfg(MATMUL_AUTO, tile[0], tile[1], tile[2], RN, stages, 0, 0)
+    cfg = MatmulCfg(MATMUL_AUTO, tile[0], tile[1], tile[2], RN, stages, 0, 0, None, 0)
     check(lib().kapy_matmul_fused(C.byref(lhs), C.byref(rhs), C.byref(result), C.byref(epi), C.byref(cfg),
                                   stream if stream is not None else current_stream()))
 
 
-def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, stream=None):
+def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, split_k=0, workspace=None, stream=None):
+    ws, ws_bytes = _workspace(workspace)
+    cfg = MatmulCfg(MATMUL_AUTO, 0, 0, 0, RN, 0, 0, split_k, ws, ws_bytes)
     check(lib().kapy_matmul_scaled_f8(C.byref(a8), C.byref(w8), C.c_void_p(row_scale_ptr), C.c_void_p(col_scale_ptr),
-                                      C.byref(result), None, stream if stream is not None else current_stream()))
+                                      C.byref(result), C.byref(cfg), stream if stream is not None else current_stream()))
 
 
 def reduce(src, dst, axis, kind=0, stream=None):

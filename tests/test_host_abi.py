@@ -27,7 +27,7 @@ def test_struct_layout_matches_header_and_oracle(ko):
     assert C.sizeof(kh.Global) == C.sizeof(ko.Global) == 40
     assert C.sizeof(kh.Fragments) == C.sizeof(ko.Fragments) == 24
     assert C.sizeof(kh.EwInst) == C.sizeof(ko.EwInst) == 32
-    assert C.sizeof(kh.MatmulCfg) == 32 and C.sizeof(kh.Grid2) == 40 and C.sizeof(kh.CopyCfg) == 16
+    assert C.sizeof(kh.MatmulCfg) == 48 and C.sizeof(kh.Grid2) == 40 and C.sizeof(kh.CopyCfg) == 16
 
 
 def test_descriptors_match_oracle(ko):

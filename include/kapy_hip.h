@@ -258,6 +258,17 @@ int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n);
 int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                 const kapy_matmul_cfg *cfg, void *stream);
 
+/* kapy_matmul for callers that cannot allocate or hand over device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same operands, same results bit for bit as kapy_matmul with a workspace, but the
+ * workspace of a split K is a 16 MiB + 16 KiB array that is part of the library's own device image (one per GPU, held until
+ * the process ends); cfg->workspace is ignored.  It calls no allocating routine.  A problem whose split would need more
+ * (m x n beyond 512K elements at the widest split) is multiplied without a split, exactly as kapy_matmul without a
+ * workspace would.  All calls on one GPU share the array: calls that overlap in time on one GPU (different streams or
+ * host threads) race; calls on one stream, or otherwise ordered, are safe.  This entry point has no counterpart in the
+ * reference, which never owns device memory (its kernels get every buffer as an argument, FuncOpToLLVM.cpp:55-92). */
+int kapy_matmul_static_workspace(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
+                                 const kapy_matmul_cfg *cfg, void *stream);
+
 /* kapy.matmul with the elementwise ops that follow it on the accumulator fused into the same kernel, which is how a
  * kapy.func that multiplies and then applies bias and activation compiles (one kernel; the accumulator never leaves
  * registers): result = fptofp_rn( act( addf( mulf(matmul(lhs, rhs), splat alpha), broadcast(extf bias) ) ) ),

@@ -33,6 +33,11 @@
 #include "ew_machine.hpp"
 #include "numeric.hpp"
 
+// Workspace of a split K for callers that cannot bring one (kapy_matmul_static_workspace): arrival counters, then
+// partial sums.  Part of the device image, so every GPU the library runs on holds its own copy until the process ends;
+// zero when the image is loaded, and every kernel that uses the counters leaves them zero.
+static __device__ __align__(256) unsigned char scratch[kapy::kSplitCounterBytes + (16 << 20)];
+
 namespace kapy {
 namespace {
 
@@ -1622,6 +1627,30 @@ int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n) {
   // a split keeps tiles * parts within the CUs of the device; without a device, the largest split of every tile
   const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128);
   return split_workspace_bytes(tiles, kMaxSplitK);
+}
+
+int kapy_matmul_static_workspace(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
+                                 const kapy_matmul_cfg *cfg, void *stream) {
+  kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
+  if (cfg) c = *cfg;
+  int rc = ensure_device();
+  if (rc) return rc;
+  // The array's name is a host-side handle, not a device address: ask the runtime once per device where this device's
+  // copy lives, and hand that pointer to the kernels.
+  constexpr int kMaxDevices = 64;
+  static void *scratch_on_device[kMaxDevices];  // (a race between two first calls only repeats the query)
+  int dev = -1;
+  KAPY_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(KAPY_ERR_UNSUPPORTED, "matmul_static_workspace: device ordinal %d beyond %d", dev, kMaxDevices);
+  void *ws = __atomic_load_n(&scratch_on_device[dev], __ATOMIC_ACQUIRE);
+  if (!ws) {
+    KAPY_HIP_CHECK(hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch)));
+    if (!ws) return fail(KAPY_ERR_HIP, "matmul_static_workspace: the runtime reports no address for the workspace array");
+    __atomic_store_n(&scratch_on_device[dev], ws, __ATOMIC_RELEASE);
+  }
+  c.workspace = ws;
+  c.workspace_bytes = (int64_t)sizeof(scratch);
+  return matmul_16bit(lhs, rhs, acc, result, &c, nullptr, stream);
 }
 
 int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *result, const kapy_matmul_epilogue *epi,

@@ -33,7 +33,7 @@ EXPORTS = [
     "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
-    "kapy_mfma_probe", "kapy_matmul_workspace_bytes",
+    "kapy_mfma_probe", "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
 ]
 
 
@@ -155,6 +155,7 @@ def lib():
     L.kapy_elementwise_source.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), C.c_char_p, i64, P(i64), P(i64)]
     L.kapy_fptofp.argtypes = [P(Global), P(Global), i32, vp]
     L.kapy_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
+    L.kapy_matmul_static_workspace.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
     L.kapy_matmul_workspace_bytes.restype = i64
     L.kapy_matmul_workspace_bytes.argtypes = [i64, i64]
     L.kapy_matmul_fused.argtypes = [P(Global), P(Global), P(Global), P(MatmulEpilogue), P(MatmulCfg), vp]
@@ -370,11 +371,12 @@ def _workspace(workspace):
 
 
 def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stages=0, waves=0, split_k=0, workspace=None,
-           stream=None):
-    """workspace: zero-initialised device memory (a torch tensor or a (pointer, bytes) pair) that lets the library split K."""
+           static_workspace=False, stream=None):
+    """workspace: zero-initialised device memory (a torch tensor or a (pointer, bytes) pair) that lets the library split K;
+    static_workspace: call kapy_matmul_static_workspace instead (the library's own array)."""
     ws, ws_bytes = _workspace(workspace)
     cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, split_k, ws, ws_bytes)
-    fn = lib().kapy_matmul
+    fn = lib().kapy_matmul_static_workspace if static_workspace else lib().kapy_matmul
     check(fn(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
              C.byref(cfg), stream if stream is not None else current_stream()))
 

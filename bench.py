@@ -488,11 +488,12 @@ def _cpu_gemm(ko, go_a, go_b, go_d, rows, N, K, scales, what):
             "sample": "%s; fp32 accumulate, operands widened to fp32 and packed outside the timed multiply; %d repetitions, %.2f s of multiplying" % (what, reps, tot)}
 
 
-def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None):
+def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None, workspace=False):
     """graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
     (what a launch-bound shape gains when the host's per-launch cost is taken out).
     fused_gelu: d = gelu_tanh(a.b*0.5 + bias) with the tail in the GEMM's epilogue (kapy_matmul_fused); flops counted are the GEMM's.
-    gen: "normal" = normal(0, 0.02) seeds 0 / 1 (C4), "uniform" = uniform[-1,1) seed 0 streams 0 / 1 (C1)."""
+    gen: "normal" = normal(0, 0.02) seeds 0 / 1 (C4), "uniform" = uniform[-1,1) seed 0 streams 0 / 1 (C1).
+    workspace: hand the library a workspace, which lets it split K across workgroups when the tiles alone would not fill the device."""
     import numpy as np
     import torch
     import ko
@@ -516,7 +517,8 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
         gbias = kh.mk_global(bias.data_ptr(), 1, N, N, 1, dtype)
         run = lambda i: kh.matmul_fused(ga, gb, gd, bias=gbias, alpha=0.5, act=kh.EW_GELU_TANH, tile=tile)
     else:
-        run = lambda i: kh.matmul(ga, gb, gd, tile=tile)
+        ws = torch.zeros(kh.lib().kapy_matmul_workspace_bytes(M, N), dtype=torch.uint8, device="cuda") if workspace else None
+        run = lambda i: kh.matmul(ga, gb, gd, tile=tile, workspace=ws)
     run(0)
     torch.cuda.synchronize()
     got = _download(d, np.uint16, (M, N))
@@ -590,7 +592,7 @@ def _f8_operands(ko, M, N, K):
     return aq, sa, wq, sb
 
 
-def bench_f8(kh, steps, warmup, cpu, M):
+def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     import numpy as np
     import torch
     import ko
@@ -600,13 +602,14 @@ def bench_f8(kh, steps, warmup, cpu, M):
     if ("wdev", N, K) not in _dev_cache:
         _dev_cache[("wdev", N, K)] = _upload(wq)
     w0 = _dev_cache[("wdev", N, K)]
-    sets = 6 if M <= 64 else 1                 # M<=64 is weight-streaming: 6 x 64 MiB > Infinity Cache (copies of the same weight)
+    sets = 6 if M <= 128 else 1                # M<=64 is weight-streaming: 6 x 64 MiB > Infinity Cache (copies of the same weight)
     ws = [w0] + [w0.clone() for _ in range(sets - 1)]
     d = torch.empty(M * N, device="cuda", dtype=torch.int16)
     ga = kh.mk_global(a.data_ptr(), M, K, K, 1, kh.F8E4M3)
     gws = [kh.mk_global(w.data_ptr(), K, N, 1, K, kh.F8E4M3) for w in ws]
     gd = kh.mk_global(d.data_ptr(), M, N, N, 1, kh.BF16)
-    kh.matmul_scaled_f8(ga, gws[0], dsa.data_ptr(), dsb.data_ptr(), gd)
+    ws = torch.zeros(kh.lib().kapy_matmul_workspace_bytes(M, N), dtype=torch.uint8, device="cuda") if workspace else None
+    kh.matmul_scaled_f8(ga, gws[0], dsa.data_ptr(), dsb.data_ptr(), gd, workspace=ws)
     torch.cuda.synchronize()
     got = _download(d, np.uint16, (M, N))
     go_a, go_w = ko.mk_global(aq, M, K, K, 1, ko.F8E4M3), ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)
@@ -614,14 +617,14 @@ def bench_f8(kh, steps, warmup, cpu, M):
     rel = _blocks_frobenius(ko, got, go_a, go_w, M, N, K, ko.BF16, n_blocks, scales=(sa, sb))
     if not rel <= FROB_TOL:
         raise CheckFailed("f8 M=%d: relative Frobenius error %g" % (M, rel))
-    wall, ev = _events(lambda i: kh.matmul_scaled_f8(ga, gws[i % sets], dsa.data_ptr(), dsb.data_ptr(), gd), steps, warmup)
+    wall, ev = _events(lambda i: kh.matmul_scaled_f8(ga, gws[i % sets], dsa.data_ptr(), dsb.data_ptr(), gd, workspace=ws), steps, warmup)
     flops = 2.0 * M * N * K
     nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
-    out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192" % M, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 64 else "tn_kernel<F8>",
+    out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192%s" % (M, ", K split across workgroups (workspace given)" if workspace else ""), "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "tn_kernel<F8, 128x128x128> split K" if (workspace and 40 <= M <= 128) else "skinny_stream_kernel" if M <= 80 else "tn_kernel<F8>",
            "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
            "checked": True, "check": "%d %dx64 blocks against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" % (n_blocks, min(M, 64), rel, FROB_TOL)}
-    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d" % M) if M <= 64 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
+    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d" % M) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
     if cpu:
         rows = min(M, 1024)
         hd = np.zeros(M * N, np.uint16)
@@ -631,7 +634,7 @@ def bench_f8(kh, steps, warmup, cpu, M):
 
 
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_graph", "f8_m16", "f8_m4096"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m64_splitk", "f8_m4096"]
 
 
 def main():
@@ -670,7 +673,10 @@ def main():
         "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform"),
         "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform"),
+        "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True),
         "f8_m16": lambda s, w: bench_f8(kh, s, w, cpu, 16),
+        "f8_m64": lambda s, w: bench_f8(kh, s, w, False, 64),
+        "f8_m64_splitk": lambda s, w: bench_f8(kh, s, w, False, 64, workspace=True),
         "f8_m4096": lambda s, w: bench_f8(kh, s, w, cpu, 4096),
     }
     try:

@@ -370,43 +370,69 @@ __device__ __forceinline__ int32_t enter_split(GemmParams &p, int element_bytes)
 // (quad by quad, thread-contiguous: the reader is the same thread of another workgroup, so no layout is involved) and
 // counts itself; the one that arrives last gets `true` with `acc` replaced by the sum of all parts IN SPLIT ORDER (the
 // result does not depend on which workgroup was last), and sets the counter back to zero for the next call.  Nobody
-// waits for anybody.  The release / acquire pair at device scope makes the parts written by workgroups on other XCDs
-// (other L2s) visible to the reader.  `lds_word`: 4 bytes of LDS that no wave uses at this point.
+// waits for anybody.
+// The parts are written and read by workgroups on different XCDs, whose L2 caches do not see each other.  A release /
+// acquire pair at device scope would make them visible, but costs a write-back and an invalidation of a whole L2 per
+// workgroup (measured: 1024^3 took 33 us instead of 16).  Instead every access to the workspace is itself a relaxed
+// device-scope access (stores write through, loads do not hit a stale line), each workgroup waits until its stores have
+// been acknowledged before it counts itself, and the reader starts loading only after its count has come back.
+// Accumulator blocks that lie wholly below the last row of the result (row0 + i * block_rows >= p.M) are not exchanged.
+// `lds_word`: 4 bytes of LDS that no wave uses at this point.
 template <int THREADS, typename Acc, int TM, int TN>
-__device__ __forceinline__ bool split_k_meet(const GemmParams &p, int32_t tile, int32_t split, Acc (&acc)[TM][TN], uint32_t *lds_word) {
-  constexpr int kQuads = sizeof(Acc) / 16, kPerThread = TM * TN * kQuads;
-  f32x4 *base = (f32x4 *)p.partial + (int64_t)tile * p.split_k * (kPerThread * THREADS) + threadIdx.x;
-  f32x4 *mine = base + (int64_t)split * (kPerThread * THREADS);
+__device__ __forceinline__ bool split_k_meet(const GemmParams &p, int32_t tile, int32_t split, Acc (&acc)[TM][TN], int32_t row0, int32_t block_rows,
+                                             uint32_t *lds_word) {
+  constexpr int kHalves = sizeof(Acc) / 8, kPerThread = TM * TN * kHalves;  // 8-byte pieces: the widest relaxed access
+  uint64_t *base = (uint64_t *)p.partial + (int64_t)tile * p.split_k * (kPerThread * THREADS) + threadIdx.x;
+  uint64_t *mine = base + (int64_t)split * (kPerThread * THREADS);
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM; ++i) {
+    if (row0 + i * block_rows >= p.M) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int q = 0; q < kQuads; ++q) {
-        f32x4 v;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-        mine[((i * TN + j) * kQuads + q) * THREADS] = v;
+      for (int h = 0; h < kHalves; ++h) {
+        const uint64_t v = (uint64_t)__float_as_uint(acc[i][j][2 * h]) | ((uint64_t)__float_as_uint(acc[i][j][2 * h + 1]) << 32);
+        __hip_atomic_store(mine + ((i * TN + j) * kHalves + h) * THREADS, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-  __syncthreads();  // the whole workgroup's part is written (workgroup-scope release) ...
-  if (threadIdx.x == 0) *lds_word = __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);  // ... and published
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this lane's stores have been acknowledged
+  __syncthreads();                           // ... and every lane's of the workgroup
+  if (threadIdx.x == 0) *lds_word = __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const uint32_t arrived_before = *lds_word;
   __syncthreads();  // (the word's LDS may be reused from here on)
   if (arrived_before != (uint32_t)p.split_k - 1) return false;
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  // two parts at a time (split_k is even), all of their pieces requested before the first is added: a piece-by-piece
+  // loop would pay the memory latency once per piece instead of once per round
+  for (int sp = 0; sp < p.split_k; sp += 2) {
+    const uint64_t *part = base + (int64_t)sp * (kPerThread * THREADS);
+    uint64_t piece[2][TM][TN][kHalves];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int i = 0; i < TM; ++i) {
+        if (row0 + i * block_rows >= p.M) continue;
 #pragma unroll
-      for (int q = 0; q < kQuads; ++q) {
-        const f32x4 *src = base + ((i * TN + j) * kQuads + q) * THREADS;
-        f32x4 sum = src[0];
-        for (int sp = 1; sp < p.split_k; ++sp) sum += src[(int64_t)sp * (kPerThread * THREADS)];
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
+          for (int h = 0; h < kHalves; ++h)
+            piece[u][i][j][h] = __hip_atomic_load(part + u * (kPerThread * THREADS) + ((i * TN + j) * kHalves + h) * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        if (row0 + i * block_rows >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int h = 0; h < kHalves; ++h) {
+            const float a = __uint_as_float((uint32_t)piece[u][i][j][h]), b = __uint_as_float((uint32_t)(piece[u][i][j][h] >> 32));
+            acc[i][j][2 * h] = (sp + u) ? acc[i][j][2 * h] + a : a;
+            acc[i][j][2 * h + 1] = (sp + u) ? acc[i][j][2 * h + 1] + b : b;
+          }
+      }
+  }
   if (threadIdx.x == 0) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return true;
 }
@@ -878,7 +904,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     if (p.split_k > 1) {
       __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
       __builtin_amdgcn_s_barrier();  // every wave has left the ring
-      if (!split_k_meet<C::kThreads>(p, tm + tn * p.tiles_m, split, acc, (uint32_t *)lds)) return;
+      if (!split_k_meet<C::kThreads>(p, tm + tn * p.tiles_m, split, acc, m0 + wm * C::kWtm, KM, (uint32_t *)lds)) return;
     }
   }
   if constexpr (PACKED) {
@@ -1069,7 +1095,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   if (kt < KT) tile_step(kt, P0{});
   __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
   __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space by the packed epilogue
-  if (p.split_k > 1 && !split_k_meet<256>(p, tm + tn * p.tiles_m, split, acc, (uint32_t *)lds)) return;
+  if (p.split_k > 1 && !split_k_meet<256>(p, tm + tn * p.tiles_m, split, acc, m0 + wm * 64, 16, (uint32_t *)lds)) return;
   if constexpr (PACKED) {
     static_assert(PackedEpilogue<16, 64, 64>::kBytesPerWave * 4 <= STAGES * kStage, "two strips per wavefront must fit the ring");
     PackedEpilogue<16, 64, 64>::run(p, acc, lds + wave * PackedEpilogue<16, 64, 64>::kBytesPerWave, m0 + wm * 64, n0 + wn * 64, lane);
@@ -1445,7 +1471,7 @@ int launch_probe_f8(int first_fmt, int second_fmt, bool exchanged, const void *l
 
 // Decides whether the 128 x 128 tiled kernels split K for this problem and points the parameters at the workspace.
 // cfg.split_k = 1 or no workspace: never.  0: when the tiles alone would leave at least half the device idle, the
-// largest power of two that keeps tiles * split within the CUs, leaves every part at least four K-tiles and fits the
+// largest power of two that keeps tiles * split within the CUs, leaves every part at least sixteen K-tiles and fits the
 // workspace.  An explicit split that cannot be honoured is an error.
 int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k) {
   p.split_k = 1;
@@ -1470,8 +1496,9 @@ int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k) {
                   p.K, c.split_k, tile_k, (long long)c.workspace_bytes, (long long)split_workspace_bytes(tiles, c.split_k));
     split = c.split_k;
   } else if (tiles * 2 <= device_cus()) {
+    // (meeting in the workspace costs about 10 us: parts shorter than 16 K-tiles do not earn it back)
     for (int sp = 2; sp <= kMaxSplitK && tiles * sp <= device_cus(); sp *= 2)
-      if (fits(sp) && p.K / (tile_k * sp) >= 4) split = sp;
+      if (fits(sp) && p.K / (tile_k * sp) >= 16) split = sp;
   }
   if (split > 1) {
     p.split_k = split;

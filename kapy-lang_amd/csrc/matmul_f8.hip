@@ -162,7 +162,7 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 #endif
 constexpr int kTiledFromM = KAPY_F8_TILED_FROM_M;
 #ifndef KAPY_F8_TILED_FROM_M_SPLIT
-#define KAPY_F8_TILED_FROM_M_SPLIT 17
+#define KAPY_F8_TILED_FROM_M_SPLIT 40
 #endif
 constexpr int kTiledFromMSplit = KAPY_F8_TILED_FROM_M_SPLIT;  // the same threshold when K can be split across workgroups
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;

@@ -66,10 +66,40 @@ def test_split_k_matches_checker_and_is_deterministic(ko, dt, M, N, K, b_row_maj
         assert int(ws[:16384].max().item()) == 0, sp                     # the arrival counters are back to zero
 
 
+def test_alternating_problems_never_see_the_other_problems_partial_sums(ko):
+    """Two different operand sets of one shape take turns on ONE workspace: the partial sums of the call before lie exactly
+    where this call's go, so a reader that was served a stale cache line would produce the other problem's numbers."""
+    dt, M, N, K, tile = kh.F16, 512, 512, 2048, (128, 128, 32)
+    sets = []
+    for seed in (21, 22):
+        a, b, b_str, want = _operands(ko, dt, M, N, K, True, seed=seed)
+        sets.append((to_dev(a), to_dev(b), want))
+    ws = _workspace(M, N)
+    first = {}
+    for rep in range(6):
+        for k, (da, db, want) in enumerate(sets):
+            dd = dev_zeros(M * N, 2, fill=0x7E7E)
+            kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt), dglobal(dd, M, N, N, 1, dt), tile=tile, split_k=8, workspace=ws)
+            sync()
+            got = to_host(dd, np.uint16)
+            if rep == 0:
+                assert _frob(ko, got, want, dt) <= FROB_TOL
+                first[k] = got
+            assert np.array_equal(got, first[k]), (rep, k)
+    # the same back to back without a synchronisation in between (stream order alone keeps the calls apart)
+    outs = [dev_zeros(M * N, 2) for _ in range(8)]
+    for t, dd in enumerate(outs):
+        da, db, _ = sets[t % 2]
+        kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt), dglobal(dd, M, N, N, 1, dt), tile=tile, split_k=8, workspace=ws)
+    sync()
+    for t, dd in enumerate(outs):
+        assert np.array_equal(to_host(dd, np.uint16), first[t % 2]), t
+
+
 def test_library_chooses_a_split_only_with_a_workspace(ko):
-    """split_k = 0: with a workspace a result of 64 tiles on 256 CUs is split four ways (same bits as asking for 4), without one
-    nothing changes (same bits as asking for 1)."""
-    dt, M, N, K = kh.F16, 1024, 1024, 1024
+    """split_k = 0: with a workspace a result of 16 tiles and 64 K-tiles on 256 CUs is split four ways (parts of at least 16
+    K-tiles; same bits as asking for 4), without one nothing changes (same bits as asking for 1)."""
+    dt, M, N, K = kh.F16, 512, 512, 2048
     a, b, b_str, want = _operands(ko, dt, M, N, K, True, seed=0)
     da, db, ws = to_dev(a), to_dev(b), _workspace(M, N)
     ga, gb = dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, *b_str, dt)
@@ -83,7 +113,7 @@ def test_library_chooses_a_split_only_with_a_workspace(ko):
     cus = C.c_int32()
     assert kh.lib().kapy_device_info(C.byref(cus), None, None, None, 0) == 0
     if cus.value == 256:
-        assert np.array_equal(res["auto_ws"], res["four"])
+        assert np.array_equal(res["auto_ws"], res["four"]) and not np.array_equal(res["four"], res["one"])
     assert np.array_equal(res["auto"], res["one"])
 
 

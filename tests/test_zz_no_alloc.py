@@ -11,14 +11,14 @@ from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
 pytestmark = pytest.mark.gpu
 
 
-def _pair(ko, dt, M, N, K, tile, seed):
+def _pair(ko, dt, M, N, K, tile, seed, split_k):
     a, b = ko.fill_uniform(M * K, dt, seed, 0), ko.fill_uniform(K * N, dt, seed, 1)
     da, db = to_dev(a), to_dev(b)
     ga, gb = dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt)
     ws = torch.zeros(kh.lib().kapy_matmul_workspace_bytes(M, N), dtype=torch.uint8, device="cuda")
     d_ws, d_static = dev_zeros(M * N, 2, fill=0x7E7E), dev_zeros(M * N, 2, fill=0x7E7E)
-    kh.matmul(ga, gb, dglobal(d_ws, M, N, N, 1, dt), tile=tile, workspace=ws)
-    kh.matmul(ga, gb, dglobal(d_static, M, N, N, 1, dt), tile=tile, static_workspace=True)
+    kh.matmul(ga, gb, dglobal(d_ws, M, N, N, 1, dt), tile=tile, split_k=split_k, workspace=ws)
+    kh.matmul(ga, gb, dglobal(d_static, M, N, N, 1, dt), tile=tile, split_k=split_k, static_workspace=True)
     sync()
     d_plain = dev_zeros(M * N, 2)
     kh.matmul(ga, gb, dglobal(d_plain, M, N, N, 1, dt), tile=tile, split_k=1)
@@ -28,8 +28,8 @@ def _pair(ko, dt, M, N, K, tile, seed):
 
 def test_static_workspace_equals_caller_workspace_on_two_calls_in_a_row(ko):
     import ctypes as C
-    # first call: benchmark configuration 1 (64 tiles, split four ways on a 256-CU device: 16 MiB of partial sums)
-    with_ws, static, plain, (a, b) = _pair(ko, kh.F16, 1024, 1024, 1024, (128, 128, 32), seed=0)
+    # first call: benchmark configuration 1, 64 tiles split four ways: 16 MiB of partial sums, all of the array
+    with_ws, static, plain, (a, b) = _pair(ko, kh.F16, 1024, 1024, 1024, (128, 128, 32), seed=0, split_k=4)
     assert np.array_equal(static, with_ws)
     want = np.zeros(1024 * 1024, np.uint16)
     assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, 1024, 1024, 1024, 1, ko.F16)), C.byref(ko.mk_global(b, 1024, 1024, 1024, 1, ko.F16)), None,
@@ -37,7 +37,10 @@ def test_static_workspace_equals_caller_workspace_on_two_calls_in_a_row(ko):
     g, w = ko.decode(static, ko.F16), ko.decode(want, ko.F16)
     assert np.linalg.norm(g - w) / np.linalg.norm(w) <= 1e-3
     # second call, smaller: 6 tiles, split eight ways where the first call's partial sums still lie
-    with_ws2, static2, plain2, _ = _pair(ko, kh.BF16, 384, 256, 2048, (128, 128, 64), seed=3)
+    with_ws2, static2, plain2, _ = _pair(ko, kh.BF16, 384, 256, 2048, (128, 128, 64), seed=3, split_k=8)
+    # ... and a third with the library's own choice of split
+    with_ws3, static3, _, _ = _pair(ko, kh.F16, 256, 512, 4096, (128, 128, 64), seed=4, split_k=0)
+    assert np.array_equal(static3, with_ws3)
     assert np.array_equal(static2, with_ws2)
     gp, gs = ko.decode(plain2, ko.BF16), ko.decode(static2, ko.BF16)
     assert np.linalg.norm(gp - gs) / np.linalg.norm(gp) <= 1e-3     # (the unsplit kernel sums in another order)

@@ -44,6 +44,9 @@ typedef enum kapy_cache_modifier {
   KAPY_CACHE_NONE = 0, KAPY_CACHE_CA = 1, KAPY_CACHE_CG = 2, KAPY_CACHE_CS = 3,
   KAPY_CACHE_WB = 4, KAPY_CACHE_WT = 5, KAPY_CACHE_LU = 6, KAPY_CACHE_CV = 7
 } kapy_cache_modifier;
+typedef enum kapy_evict_priority {
+  KAPY_EVICT_NORMAL = 0, KAPY_EVICT_FIRST = 1, KAPY_EVICT_LAST = 2, KAPY_EVICT_UNCHANGED = 3, KAPY_NO_ALLOCATE = 4
+} kapy_evict_priority;
 typedef enum kapy_rounding_mode { KAPY_RZ = 0, KAPY_RN = 1 } kapy_rounding_mode;
 /* MatmulImplWay: values 1..4 are the reference's (mma.sync shapes); on gfx950 they only select the
  * operand class (f16/bf16, tf32 — unsupported: CDNA4 has no tf32 MFMA —, f8).  0 lets the library
@@ -93,6 +96,28 @@ int kapy_mk_global(kapy_global *out, void *ptr, int32_t dynamic_offset, int32_t 
 /* kapy.sv_global — create_sv_global(src, start0, end0, start1, end1), python/src/ir.cc:1026-1034;
  * SvGlobalOpToLLVM.cpp:22-40: both new bounds are offsets from the source view's start. */
 int kapy_sv_global(kapy_global *out, const kapy_global *src, int32_t start0, int32_t end0, int32_t start1, int32_t end1);
+
+/* Shared-memory tensor descriptor: the struct of TypeConverter.cpp:74-82 {ptr AS3, start0, start1, end0, end1} with the
+ * pointer as a byte offset into the workgroup's shared memory (shared_array + kapy.offset, MkSharedOpToLLVM.cpp:49-70),
+ * plus the element type and the #kapy.swizzling layout that the reference carries on the tensor type. */
+typedef struct kapy_shared {
+  int64_t offset; /* bytes from the start of the workgroup's shared memory (kapy.offset; kapy_smem_plan assigns these) */
+  int32_t start0, start1, end0, end1;
+  int32_t dtype;  /* kapy_dtype */
+  kapy_swizzling layout;
+} kapy_shared;
+/* kapy.mk_shared - create_mk_shared(shape, elementType, rowMajor), python/src/ir.cc:1050-1061; MkSharedOpToLLVM.cpp:49-70:
+ * start 0, end = shape, strides (size1, 1) row-major or (1, size0) column-major (Analyze.cpp:82-95).  (bank_param,
+ * line_param) is the swizzling of the buffer, (0, 0) = none; kapy_swizzle_search finds the conflict-free ones. */
+int kapy_mk_shared(kapy_shared *out, int64_t byte_offset, int32_t size0, int32_t size1, int32_t dtype, int32_t row_major,
+                   int32_t bank_param, int32_t line_param);
+/* kapy.sv_shared - create_sv_shared(src, start0, end0, start1, end1), ir.cc:1062-1070; SvSharedOpToLLVM.cpp:20-42:
+ * same base and layout, both new bounds are offsets from the source view's start. */
+int kapy_sv_shared(kapy_shared *out, const kapy_shared *src, int32_t start0, int32_t end0, int32_t start1, int32_t end1);
+/* Byte address in the workgroup's shared memory of element (i0, i1) of the view: offset + the swizzled position of
+ * (start0 + i0, start1 + i1) (the address function of CpAsyncOpToLLVM.cpp:124-139, 64 banks); KAPY_ERR_VERIFY (negative)
+ * for an element outside the view, which a load pads and a store skips. */
+int64_t kapy_shared_address(const kapy_shared *tensor, int64_t i0, int64_t i1);
 
 /* ---------------------------------------------------------------- layout engine (host only) */
 /* FragmentsLayoutAttr::getWarpLoops / getLoopSpace — lib/Dialect/Kgpu/IR/Kgpu.cpp:164-184. */
@@ -146,6 +171,13 @@ typedef struct kapy_copy_cfg {
   int32_t transpose;      /* 1: kapy.transpose between the load and the store (dst[i,j] = src[j,i]) */
   int32_t padding_option; /* kapy_padding_option of the ld_global                                   */
   int32_t cache_modifier; /* kapy_cache_modifier; CS / CG select non-temporal access                */
+  int32_t evict_priority; /* kapy_evict_priority, looked at when cache_modifier is NONE (as the reference's lowering does,
+                             LdGlobalOpToLLVM.cpp:103-109): EVICT_FIRST / NO_ALLOCATE = non-temporal access, EVICT_LAST /
+                             EVICT_UNCHANGED = ordinary cached access, EVICT_NORMAL = the library's choice (non-temporal
+                             for moves too large to be re-read from the Infinity Cache) */
+  int32_t is_volatile;    /* the reference's ld.volatile / st.volatile drop every cache hint (same lines); here too:
+                             ordinary accesses whatever cache_modifier and evict_priority say.  Every element is read
+                             and written exactly once either way */
   int32_t reserved;
 } kapy_copy_cfg;
 

@@ -63,23 +63,45 @@ class OpBuilder {
     return push(n);
   }
 
+  // ---- shared-memory descriptors (ir.cc:1050-1070): plain data, as the lowering's structs are ----------------------
+  // byte_offset: where the planner (kapy_smem_plan) put the buffer; (bank_param, line_param): its swizzling, (0, 0) = none
+  kapy_shared create_mk_shared(const std::vector<int64_t> &shape, kapy_dtype element_type, bool row_major, int64_t byte_offset = 0,
+                               int32_t bank_param = 0, int32_t line_param = 0) {
+    if (shape.size() != 2) throw Error(KAPY_ERR_VERIFY, "mk_shared: tensors have rank 2");
+    kapy_shared t;
+    check(kapy_mk_shared(&t, byte_offset, (int32_t)shape[0], (int32_t)shape[1], element_type, row_major ? 1 : 0, bank_param, line_param));
+    return t;
+  }
+  kapy_shared create_sv_shared(const kapy_shared &source, int32_t start0, int32_t end0, int32_t start1, int32_t end1) {
+    kapy_shared t;
+    check(kapy_sv_shared(&t, &source, start0, end0, start1, end1));
+    return t;
+  }
+
   // ---- loads and stores (ir.cc:1035-1049) ---------------------------------------------------------------
-  Value create_ld_global(Value source, kapy_padding_option padding_option = KAPY_PAD_ZERO, kapy_cache_modifier cache_modifier = KAPY_CACHE_NONE) {
+  // (argument order as in the reference: source, paddingOption, cacheModifier, evictPriority, isVolatile)
+  Value create_ld_global(Value source, kapy_padding_option padding_option = KAPY_PAD_ZERO, kapy_cache_modifier cache_modifier = KAPY_CACHE_NONE,
+                         kapy_evict_priority evict_priority = KAPY_EVICT_NORMAL, bool is_volatile = false) {
     Node n;
     n.kind = Node::kLoad;
     n.global = global_of(source, "ld_global");
     n.dtype = node(source).dtype;
     n.padding = padding_option;
     n.cache = cache_modifier;
+    n.evict = evict_priority;
+    n.is_volatile = is_volatile;
     return push(n);
   }
   // Lowers everything `source` depends on and stores it: the one call that launches work.
-  void create_st_global(Value source, Value target, kapy_cache_modifier cache_modifier = KAPY_CACHE_NONE) {
+  // (the hints of a store apply to the move it launches; a load's hints stand in where the store gives none)
+  void create_st_global(Value source, Value target, kapy_cache_modifier cache_modifier = KAPY_CACHE_NONE,
+                        kapy_evict_priority evict_priority = KAPY_EVICT_NORMAL, bool is_volatile = false) {
     const kapy_global &out = global_of(target, "st_global");
     const Node &s = node(source);
     if (s.kind == Node::kGlobal) throw Error(KAPY_ERR_VERIFY, "st_global: source must be a register tensor");
     if (s.kind == Node::kLoad) {  // a layout move: bits travel untouched
-      kapy_copy_cfg cfg = {s.transposed ? 1 : 0, s.padding, cache_modifier != KAPY_CACHE_NONE ? cache_modifier : s.cache, 0};
+      kapy_copy_cfg cfg = {s.transposed ? 1 : 0, s.padding, cache_modifier != KAPY_CACHE_NONE ? cache_modifier : s.cache,
+                           evict_priority != KAPY_EVICT_NORMAL ? evict_priority : s.evict, (is_volatile || s.is_volatile) ? 1 : 0, 0};
       check(kapy_copy(&s.global, &out, &cfg, stream_));
       return;
     }
@@ -205,8 +227,8 @@ class OpBuilder {
     enum Kind { kGlobal, kLoad, kOp, kMatmul } kind = kOp;
     kapy_global global{};
     int op = -1, a = -1, b = -1, c = -1, dtype = KAPY_F32, rmode = KAPY_RN, axis = 1;
-    int padding = KAPY_PAD_ZERO, cache = KAPY_CACHE_NONE, impl_way = KAPY_MATMUL_AUTO;
-    bool transposed = false;
+    int padding = KAPY_PAD_ZERO, cache = KAPY_CACHE_NONE, evict = KAPY_EVICT_NORMAL, impl_way = KAPY_MATMUL_AUTO;
+    bool transposed = false, is_volatile = false;
     float imm = 0.f;
   };
   std::vector<Node> nodes_;
@@ -337,7 +359,18 @@ class OpBuilder {
       *v = nodes_[id].imm;
       return true;
     };
-    if (is_op(cur, KAPY_EW_FPTOFP)) cur = nodes_[cur].a;  // the final cast: the result descriptor's type says the same
+    // The value stored must have the element type of the view it is stored into (st_global: SameOperandsElementType,
+    // Ops.td:163-170).  A final fptofp is the kernel's own cast: its type must be the view's and its rounding mode is
+    // the kernel's; without one the f32 accumulator chain can only be stored into an f32 view.
+    int rmode = KAPY_RN;
+    if (is_op(cur, KAPY_EW_FPTOFP)) {
+      if (nodes_[cur].dtype != out.dtype) throw Error(KAPY_ERR_VERIFY, "st_global: source and target must have same element type");
+      rmode = nodes_[cur].rmode;
+      cur = nodes_[cur].a;
+      if (cur >= 0 && nodes_[cur].dtype != KAPY_F32) throw Error(KAPY_ERR_UNSUPPORTED, "matmul: the cast of the result must be applied to the f32 accumulator chain");
+    } else if (nodes_[cur].dtype != out.dtype) {
+      throw Error(KAPY_ERR_VERIFY, "st_global: source and target must have same element type");
+    }
     // the activation
     float operand = 0.f;
     if (is_op(cur, KAPY_EW_MAXIMUMF) || is_op(cur, KAPY_EW_MINIMUMF)) {
@@ -352,8 +385,11 @@ class OpBuilder {
     // the bias: a loaded [1 x N] row, possibly widened
     kapy_global bias;
     if (is_op(cur, KAPY_EW_ADDF)) {
+      // (the addend joins an f32 value: arith ops need equal element types, so a 16-bit row must have been widened)
       auto as_bias = [&](int id) {
         if (is_op(id, KAPY_EW_FPTOFP) && nodes_[id].dtype == KAPY_F32) id = nodes_[id].a;
+        else if (id >= 0 && nodes_[id].kind == Node::kLoad && nodes_[id].dtype != KAPY_F32)
+          throw Error(KAPY_ERR_VERIFY, "addf: operands must have same element type");
         return id >= 0 && nodes_[id].kind == Node::kLoad ? id : -1;
       };
       const Node &n = nodes_[cur];
@@ -376,7 +412,7 @@ class OpBuilder {
       throw Error(KAPY_ERR_UNSUPPORTED, "matmul: the ops on its result must be [mulf splat] [addf bias row] [activation] [fptofp]");
     const Node &mm = nodes_[cur];
     const kapy_global lhs = view_of(nodes_[mm.a]), rhs = view_of(nodes_[mm.b]);
-    kapy_matmul_cfg cfg = {mm.impl_way, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
+    kapy_matmul_cfg cfg = {mm.impl_way, 0, 0, 0, rmode, 0, 0, 0, nullptr, 0};
     if (tail) {
       if (mm.c >= 0) throw Error(KAPY_ERR_UNSUPPORTED, "matmul: an accumulator input and a fused tail do not combine");
       check(kapy_matmul_fused(&lhs, &rhs, &out, &epi, &cfg, stream_));

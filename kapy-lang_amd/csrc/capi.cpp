@@ -166,6 +166,56 @@ int kapy_sv_global(kapy_global *out, const kapy_global *src, int32_t start0, int
   return KAPY_OK;
 }
 
+int kapy_mk_shared(kapy_shared *out, int64_t byte_offset, int32_t size0, int32_t size1, int32_t dtype, int32_t row_major,
+                   int32_t bank_param, int32_t line_param) {
+  if (!out) return fail(KAPY_ERR_INVALID, "mk_shared: null result");
+  int b = dtype_bytes(dtype);
+  if (!b) return fail(KAPY_ERR_INVALID, "mk_shared: unknown element type %d", dtype);
+  // static power-of-two shapes (OpTraits.cpp:43-58)
+  if (size0 <= 0 || size1 <= 0 || (size0 & (size0 - 1)) || (size1 & (size1 - 1)))
+    return fail(KAPY_ERR_VERIFY, "mk_shared: shape must be static and every extent a power of two");
+  if (byte_offset < 0 || byte_offset % 128) return fail(KAPY_ERR_INVALID, "mk_shared: the offset must be a non-negative multiple of 128 bytes");
+  if (bank_param == 0 && line_param == 0) { bank_param = 4; line_param = 1; }  // unswizzled
+  if ((bank_param != 4 && bank_param != 2 && bank_param != 1) || line_param < 1 || line_param > kLdsBanks / bank_param || (line_param & (line_param - 1)))
+    return fail(KAPY_ERR_INVALID, "mk_shared: swizzling parameters (%d, %d) out of range", bank_param, line_param);
+  if (byte_offset + int64_t(size0) * size1 * b > 160 * 1024)
+    return fail(KAPY_ERR_VERIFY, "mk_shared: the tensor ends beyond the 160 KiB of a workgroup's shared memory");
+  out->offset = byte_offset;
+  out->start0 = out->start1 = 0;
+  out->end0 = size0;
+  out->end1 = size1;
+  out->dtype = dtype;
+  // row-major strides (size1, 1), column-major (1, size0): Analyze.cpp:82-95
+  out->layout.stride0 = row_major ? size1 : 1;
+  out->layout.stride1 = row_major ? 1 : size0;
+  out->layout.bank_param = bank_param;
+  out->layout.line_param = line_param;
+  return KAPY_OK;
+}
+
+int kapy_sv_shared(kapy_shared *out, const kapy_shared *src, int32_t start0, int32_t end0, int32_t start1, int32_t end1) {
+  if (!out || !src) return fail(KAPY_ERR_INVALID, "sv_shared: null argument");
+  if (end0 < start0 || end1 < start1) return fail(KAPY_ERR_INVALID, "sv_shared: end before start");
+  kapy_shared r = *src;  // same base, element type and layout (Kapy.cpp:301-313)
+  r.start0 = src->start0 + start0;
+  r.start1 = src->start1 + start1;
+  r.end0 = src->start0 + end0;
+  r.end1 = src->start1 + end1;
+  *out = r;
+  return KAPY_OK;
+}
+
+int64_t kapy_shared_address(const kapy_shared *tensor, int64_t i0, int64_t i1) {
+  if (!tensor) return fail(KAPY_ERR_INVALID, "shared_address: null tensor");
+  int b = dtype_bytes(tensor->dtype);
+  if (!b) return fail(KAPY_ERR_INVALID, "shared_address: unknown element type %d", tensor->dtype);
+  // in bounds iff (start + i) <u end on both axes, the unsigned compare of the loads and stores
+  const uint32_t a0 = (uint32_t)(tensor->start0 + i0), a1 = (uint32_t)(tensor->start1 + i1);
+  if (a0 >= (uint32_t)tensor->end0 || a1 >= (uint32_t)tensor->end1) return KAPY_ERR_VERIFY;
+  const Swizzle sw{tensor->layout.stride0, tensor->layout.stride1, tensor->layout.bank_param, tensor->layout.line_param};
+  return tensor->offset + sw.offset(b * 8, a0, a1) * b;
+}
+
 int kapy_fragments_loops(const kapy_fragments *layout, const int64_t shape[2], int64_t warp_loops[2], int64_t loop_space[2]) {
   int rc = check_fragments(layout, "fragments");
   if (rc) return rc;

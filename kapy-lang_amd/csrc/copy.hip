@@ -276,11 +276,13 @@ int launch_transpose_lds(const CopyParams &p, bool nt, int32_t batch, hipStream_
   constexpr int kLds = TI * TJ * 2;
   dim3 grid((unsigned)((p.d0 + TI - 1) / TI), (unsigned)((p.d1 + TJ - 1) / TJ), (unsigned)batch);
   if (kLds > 65536) {
-    static bool configured = false;
-    if (!configured) {
+    static bool configured_on[64];  // per device (the attribute belongs to the code object loaded on that device); a race only repeats the calls
+    int dev = 0;
+    KAPY_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64 || !configured_on[dev]) {
       KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)transpose_lds_kernel<TI, TJ, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
       KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)transpose_lds_kernel<TI, TJ, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-      configured = true;
+      if (dev >= 0 && dev < 64) configured_on[dev] = true;
     }
   }
   if (nt) transpose_lds_kernel<TI, TJ, true><<<grid, 256, kLds, stream>>>(p);
@@ -378,9 +380,11 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   if (B != dtype_bytes(dst->dtype))
     return fail(KAPY_ERR_VERIFY, "copy: source (%s) and target (%s) must have the same element width", dtype_name(src->dtype),
                 dtype_name(dst->dtype));
-  kapy_copy_cfg c = {0, KAPY_PAD_ZERO, KAPY_CACHE_NONE, 0};
+  kapy_copy_cfg c = {0, KAPY_PAD_ZERO, KAPY_CACHE_NONE, KAPY_EVICT_NORMAL, 0, 0};
   if (cfg) c = *cfg;
   if (c.padding_option < 0 || c.padding_option > 3) return fail(KAPY_ERR_INVALID, "copy: unknown padding option %d", c.padding_option);
+  if (c.cache_modifier < KAPY_CACHE_NONE || c.cache_modifier > KAPY_CACHE_CV) return fail(KAPY_ERR_INVALID, "copy: unknown cache modifier %d", c.cache_modifier);
+  if (c.evict_priority < KAPY_EVICT_NORMAL || c.evict_priority > KAPY_NO_ALLOCATE) return fail(KAPY_ERR_INVALID, "copy: unknown evict priority %d", c.evict_priority);
   if (c.padding_option != KAPY_PAD_ZERO && !is_float(src->dtype))
     return fail(KAPY_ERR_VERIFY, "copy: integer tensors only take zero padding");
   if (src->start0 < 0 || src->start1 < 0 || dst->start0 < 0 || dst->start1 < 0)
@@ -406,9 +410,6 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   p.pad = padding_word(src->dtype, c.padding_option);
   p.n1 = g.n1 > 0 ? g.n1 : 1;
   p.map_mode = KAPY_TRANSPOSE_MAP;
-#ifdef KAPY_TUNING
-  if (c.reserved) p.map_mode = c.reserved - 1;
-#endif
   p.s_off0 = g.src_off0;
   p.s_off1 = g.src_off1;
   p.d_off0 = g.dst_off0;
@@ -427,8 +428,13 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   // Streaming (non-temporal) access when asked for (cs / cg), and by default for moves too large to
   // be re-read from the 256 MB Infinity Cache anyway.
   const int64_t moved = (int64_t)p.d0 * p.d1 * B * (g.n0 > 0 ? g.n0 : 1) * (g.n1 > 0 ? g.n1 : 1);
-  bool nt = c.cache_modifier == KAPY_CACHE_CS || c.cache_modifier == KAPY_CACHE_CG ||
-            (c.cache_modifier == KAPY_CACHE_NONE && moved >= (int64_t(32) << 20));
+  // The hints in the reference's order of precedence (LdGlobalOpToLLVM.cpp:103-109): volatile drops all of them, then
+  // the cache modifier, then the eviction priority.
+  bool nt = false;
+  if (c.is_volatile) nt = false;
+  else if (c.cache_modifier != KAPY_CACHE_NONE) nt = c.cache_modifier == KAPY_CACHE_CS || c.cache_modifier == KAPY_CACHE_CG;
+  else if (c.evict_priority == KAPY_EVICT_FIRST || c.evict_priority == KAPY_NO_ALLOCATE) nt = true;
+  else if (c.evict_priority == KAPY_EVICT_NORMAL) nt = moved >= (int64_t(32) << 20);
   int32_t batch = g.n0 * g.n1;
   hipStream_t s = (hipStream_t)stream;
   switch (B) {

@@ -70,9 +70,9 @@ struct TileLayout {
 // ds_read_b64_tr_b16 issued as opaque assembly.  Through the compiler's builtin every such read is
 // preceded by s_waitcnt vmcnt(0) (it is taken to alias the LDS-direct loads in flight), which
 // serialises the whole global->LDS pipeline; ordering against those loads is established by the
-// kernel's own waits and barriers.  The result is pending until tr_reads_wait() has been called and
-// must not be touched before: the caller keeps it in a fragment buffer that is only consumed one
-// K-slice later (the kernel using this has no register spills, which would copy a pending register).
+// kernel's own waits and barriers.  The result is pending until the wait below has been executed: every
+// register that holds a pending result is an in/out operand of that wait, so the compiler sees each later
+// use as a use of the WAIT's result and cannot place it (or a copy feeding it) before the wait.
 typedef uint32_t u32x2_lds __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ u32x2_lds tr_read_b64(const char *lds_ptr) {
   const uint32_t addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)lds_ptr;  // LDS pointers are 32-bit byte offsets
@@ -80,7 +80,13 @@ __device__ __forceinline__ u32x2_lds tr_read_b64(const char *lds_ptr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
   return r;
 }
-__device__ __forceinline__ void tr_reads_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Waits for the transposing reads whose results sit in h0[j], h1[j] (j < 4) and hands those registers back as its own results.
+__device__ __forceinline__ void tr_reads_wait(u32x2_lds (&h0)[4], u32x2_lds (&h1)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(h0[0]), "+v"(h0[1]), "+v"(h0[2]), "+v"(h0[3]), "+v"(h1[0]), "+v"(h1[1]), "+v"(h1[2]), "+v"(h1[3])
+               :
+               : "memory");
+}
 
 // s_waitcnt immediate that waits only on vmcnt <= n (gfx9 encoding: vmcnt in bits [3:0] and [15:14],
 // expcnt [6:4] and lgkmcnt [11:8] left at "no wait").
@@ -402,36 +408,33 @@ __device__ __forceinline__ bool split_k_meet(const GemmParams &p, int32_t tile, 
   const uint32_t arrived_before = *lds_word;
   __syncthreads();  // (the word's LDS may be reused from here on)
   if (arrived_before != (uint32_t)p.split_k - 1) return false;
-  // two parts at a time (split_k is even), all of their pieces requested before the first is added: a piece-by-piece
-  // loop would pay the memory latency once per piece instead of once per round
-  for (int sp = 0; sp < p.split_k; sp += 2) {
+  // one part at a time, all of its pieces requested before the first is added: a piece-by-piece loop would pay the
+  // memory latency once per piece instead of once per part (two parts per round measured no faster and cost 64 more
+  // registers, which halves the occupancy of these kernels)
+  for (int sp = 0; sp < p.split_k; ++sp) {
     const uint64_t *part = base + (int64_t)sp * (kPerThread * THREADS);
-    uint64_t piece[2][TM][TN][kHalves];
+    uint64_t piece[TM][TN][kHalves];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int i = 0; i < TM; ++i) {
+      if (row0 + i * block_rows >= p.M) continue;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if (row0 + i * block_rows >= p.M) continue;
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int h = 0; h < kHalves; ++h)
+          piece[i][j][h] = __hip_atomic_load(part + ((i * TN + j) * kHalves + h) * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 #pragma unroll
-          for (int h = 0; h < kHalves; ++h)
-            piece[u][i][j][h] = __hip_atomic_load(part + u * (kPerThread * THREADS) + ((i * TN + j) * kHalves + h) * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+    for (int i = 0; i < TM; ++i) {
+      if (row0 + i * block_rows >= p.M) continue;
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if (row0 + i * block_rows >= p.M) continue;
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int h = 0; h < kHalves; ++h) {
-            const float a = __uint_as_float((uint32_t)piece[u][i][j][h]), b = __uint_as_float((uint32_t)(piece[u][i][j][h] >> 32));
-            acc[i][j][2 * h] = (sp + u) ? acc[i][j][2 * h] + a : a;
-            acc[i][j][2 * h + 1] = (sp + u) ? acc[i][j][2 * h + 1] + b : b;
-          }
-      }
+        for (int h = 0; h < kHalves; ++h) {
+          const float a = __uint_as_float((uint32_t)piece[i][j][h]), b = __uint_as_float((uint32_t)(piece[i][j][h] >> 32));
+          acc[i][j][2 * h] = sp ? acc[i][j][2 * h] + a : a;
+          acc[i][j][2 * h + 1] = sp ? acc[i][j][2 * h + 1] + b : b;
+        }
+    }
   }
   if (threadIdx.x == 0) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return true;
@@ -440,9 +443,6 @@ __device__ __forceinline__ bool split_k_meet(const GemmParams &p, int32_t tile, 
 // ---------------------------------------------------------------------------------------------
 // TN kernel.  BM x BN x BK workgroup tile, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN)
 // block of 32x32 accumulators.  STAGES-deep LDS ring filled by LDS-direct loads.
-#ifndef KAPY_ABLATE
-#define KAPY_ABLATE 0  // timing experiments in tuning builds only: 1 no barrier, 2 no load wait, 4 no loads, 8 no LDS reads (results are wrong)
-#endif
 constexpr int kRing25 = 25;  // value of STAGES (and of kapy_matmul_cfg.stages) that selects the 2.5-tile ring
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 struct TnConfig {
@@ -537,20 +537,6 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   }
 
   const int KT = (p.K + BK - 1) / BK;  // (a partial last tile only in the ring variant)
-#ifdef KAPY_TRACE
-  // tuning builds only: clock stamps of workgroup 0 for K-tiles 32..39 (8 per tile per wave)
-  uint64_t *trace = p.row_scale ? nullptr : (uint64_t *)p.col_scale;
-  auto stamp = [&](int kt, int which) {
-    if (trace && blockIdx.x == KAPY_TRACE && kt >= 32 && kt < 40) {
-      uint64_t t = __builtin_readcyclecounter();
-      if (lane == 0) trace[(wave * 8 + (kt - 32)) * 8 + which] = t;
-    }
-  };
-#define KAPY_STAMP(kt, which) stamp(kt, which)
-  const uint64_t trace_begin = __builtin_readcyclecounter();
-#else
-#define KAPY_STAMP(kt, which)
-#endif
   constexpr int KK = BK / T::kSliceK;                                   // matrix-instruction K-slices per tile
   constexpr int kLoadsPerTile = C::kLoadsAPerWave + C::kLoadsBPerWave;  // per wavefront
   // A fragment: the CH 16-byte chunks one lane feeds a matrix instruction for one operand block.
@@ -604,11 +590,8 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     constexpr int kUnit = C::kUnitBytes, kHalf = kLoadsPerTile / 2;  // loads per wavefront per operand
     static_assert(C::kLoadsAPerWave == kHalf && C::kLoadsBPerWave == kHalf && kHalf % 2 == 0, "two equal units per operand");
     constexpr int kPerUnit = kHalf / 2;
-#ifndef KAPY_RING_SPACING
-#define KAPY_RING_SPACING 0
-#endif
     constexpr int kEven = (KK * kMfmas) / kLoadsPerTile;
-    constexpr int kLoadSpacing = KAPY_RING_SPACING ? KAPY_RING_SPACING : (kEven < 1 ? 1 : kEven);
+    constexpr int kLoadSpacing = kEven < 1 ? 1 : kEven;
     constexpr int kEarly = kMfmas / kLoadSpacing < kLoadsPerTile ? kMfmas / kLoadSpacing : kLoadsPerTile;
     static_assert((kLoadsPerTile - kEarly) * kLoadSpacing <= (KK - 1) * kMfmas, "late loads must go out before the barrier that waits for them");
     // The descriptors must sit in scalar registers (a descriptor in vector registers makes every load
@@ -712,13 +695,10 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
-        KAPY_STAMP(kt, kk);
         if (kk == KK - 1) {
           // tile kt+1 has landed once only the kHalf youngest loads (lhs of tile kt+2) are in flight
-          if (!(KAPY_ABLATE & 2)) __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
-          KAPY_STAMP(kt, 4);
-          if (!(KAPY_ABLATE & 1)) __builtin_amdgcn_s_barrier();
-          KAPY_STAMP(kt, 5);
+          __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
+          __builtin_amdgcn_s_barrier();
         }
 #pragma unroll
         for (int g = 0; g < kMfmas; ++g) {
@@ -728,12 +708,12 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
           for (int t = 0; t < kReadsPerMfma; ++t) {
             const int idx = g * kReadsPerMfma + t;
-            if (idx < kReads && !(KAPY_ABLATE & 8)) {
+            if (idx < kReads) {
               if (kk + 1 < KK) ring_read(a_cur_base, b_cur_base, kk + 1, idx, a_nxt, b_nxt);
               else ring_read(a_nxt_base, b_nxt_base, 0, idx, a_nxt, b_nxt);
             }
           }
-          if (g % kLoadSpacing == 0 && !(KAPY_ABLATE & 4)) {
+          if (g % kLoadSpacing == 0) {
             const int slot = (kk * kMfmas + g) / kLoadSpacing;
             if (kk == KK - 1 && g / kLoadSpacing < kEarly) ring_load(pos, g / kLoadSpacing, soff_early_b, soff_early_a);
             if (kk < KK - 1 && kEarly + slot < kLoadsPerTile && (!first.value || kEarly + slot >= kHalf))
@@ -792,13 +772,10 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
-        KAPY_STAMP(kt, kk);
         if (kk == KK - 1) {
           if constexpr (has_next.value) {
             __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));  // own loads of tile kt+1 landed; own reads of this stage returned
-            KAPY_STAMP(kt, 4);
             __builtin_amdgcn_s_barrier();
-            KAPY_STAMP(kt, 5);
           }
         }
 #pragma unroll
@@ -894,12 +871,6 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     tile_step(kt, No{}, No{});
   }
 
-#ifdef KAPY_TRACE
-  if (trace && blockIdx.x == KAPY_TRACE && threadIdx.x == 0) {
-    trace[256] = trace_begin;
-    trace[257] = __builtin_readcyclecounter();  // end of the K loop
-  }
-#endif
   if constexpr (kCanSplit) {
     if (p.split_k > 1) {
       __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
@@ -919,16 +890,6 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
 #pragma unroll
       for (int j = 0; j < C::kTn; ++j) store_block_generic(p, m0 + wm * C::kWtm + i * KM, n0 + wn * C::kWtn + j * KM, lane, acc[i][j]);
   }
-#ifdef KAPY_TRACE
-  if (trace && blockIdx.x == KAPY_TRACE && threadIdx.x == 0) trace[258] = __builtin_readcyclecounter();  // stores issued
-  if (trace && threadIdx.x == 0) {  // per-workgroup timeline: begin, end, where it ran
-    uint64_t *w = trace + 512 + 4 * blockIdx.x;
-    w[0] = trace_begin;
-    w[1] = __builtin_readcyclecounter();
-    w[2] = __builtin_amdgcn_s_getreg(4 | (31 << 11));    // HW_ID
-    w[3] = __builtin_amdgcn_s_getreg(20 | (31 << 11));   // XCC_ID
-  }
-#endif
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1020,14 +981,16 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     u32x4 c[1];
   };
   // an rhs fragment comes out of LDS as two 8-byte halves (k-rows +0..3 and +4..7 of the lane's K-group)
+  // (kept as two arrays of halves per fragment buffer, the form the wait for these reads takes its operands in)
   struct FragHalves {
-    u32x2 h[2];
+    u32x2_lds h0[kTn], h1[kTn];
   };
+  static_assert(kTn == 4, "tr_reads_wait takes the halves of four fragments");
   auto read_a = [&](int stage, int kk, int i) { return *(const u32x4 *)(lds + stage * kStage + a_off[kk] + i * 16 * kRowA); };
   auto read_b = [&](int stage, int kk, int j, FragHalves &dst) {
     const char *base = lds + stage * kStage + b_off[j] + kk * 32 * kRowB;
-    dst.h[0] = tr_read_b64(base);
-    dst.h[1] = tr_read_b64(base + 4 * kRowB);
+    dst.h0[j] = tr_read_b64(base);
+    dst.h1[j] = tr_read_b64(base + 4 * kRowB);
   };
 
   using Acc = typename T::Acc;
@@ -1044,11 +1007,11 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (STAGES - 2)));
   __builtin_amdgcn_s_barrier();  // tile 0 published
   Frag af[2][kTm];
-  FragHalves bf[2][kTn];
+  FragHalves bf[2];
 #pragma unroll
   for (int i = 0; i < kTm; ++i) af[0][i].c[0] = read_a(0, 0, i);
 #pragma unroll
-  for (int j = 0; j < kTn; ++j) read_b(0, 0, j, bf[0][j]);
+  for (int j = 0; j < kTn; ++j) read_b(0, 0, j, bf[0]);
 
   constexpr int kReads = kTm + kTn;
   constexpr int kLoadSpacing = (KK * kMfmas) / kLoads;  // matrix instructions between two loads
@@ -1065,18 +1028,18 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     for (int kk = 0; kk < KK; ++kk) {
       constexpr int par = decltype(parity)::value;
       Frag *a_cur = af[(kk + par) & 1], *a_nxt = af[(kk + par + 1) & 1];
-      FragHalves *b_cur = bf[(kk + par) & 1], *b_nxt = bf[(kk + par + 1) & 1];
-      tr_reads_wait();  // the rhs fragments of this slice were requested during the previous one
+      FragHalves &b_cur = bf[(kk + par) & 1], &b_nxt = bf[(kk + par + 1) & 1];
+      tr_reads_wait(b_cur.h0, b_cur.h1);  // the rhs fragments of this slice were requested during the previous one
 #pragma unroll
       for (int g = 0; g < kMfmas; ++g) {
         const int i = g / kTn, j = g % kTn;
-        const u32x4 b_op = {b_cur[j].h[0][0], b_cur[j].h[0][1], b_cur[j].h[1][0], b_cur[j].h[1][1]};
+        const u32x4 b_op = {b_cur.h0[j][0], b_cur.h0[j][1], b_cur.h1[j][0], b_cur.h1[j][1]};
         acc[i][j] = T::mfma(&b_op, a_cur[i].c, acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         if (g < kReads) {
           const int rs = kk + 1 < KK ? stage : next_stage, rk = kk + 1 < KK ? kk + 1 : 0;
           if (g < kTm) a_nxt[g].c[0] = read_a(rs, rk, g);
-          else read_b(rs, rk, g - kTm, b_nxt[g - kTm]);
+          else read_b(rs, rk, g - kTm, b_nxt);
         }
         if ((kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads)
           issue_load(kt + STAGES - 1, free_stage, (kk * kMfmas + g) / kLoadSpacing);
@@ -1252,6 +1215,7 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
 
 // ---------------------------------------------------------------------------------------------
 // Host side.
+constexpr int kMaxDevices = 64;  // device ordinals that get a slot in the per-device tables below
 // 16-bit row-major result with 16-byte aligned rows, no accumulator input, RN: the packed epilogue.
 bool packed_epilogue(const GemmParams &p) {
   return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16) && p.d_sn == 1 && p.acc_dtype < 0 && !p.rz &&
@@ -1267,8 +1231,11 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
   // really been raised before the first launch: query first (this also forces the code object to be
   // loaded, so the attribute is not set on a function the runtime has not materialised yet), set,
   // and read back.
-  static bool configured = false;  // idempotent; a race only repeats the calls
-  if (!configured) {
+  static bool configured_on[kMaxDevices];  // per device: a code object is loaded, and its attributes kept, per device; idempotent, a race only repeats the calls
+  int dev = 0;
+  KAPY_HIP_CHECK(hipGetDevice(&dev));
+  bool &configured = configured_on[dev >= 0 && dev < kMaxDevices ? dev : 0];
+  if (!configured || dev >= kMaxDevices) {
     hipFuncAttributes fa;
     KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, (const void *)kernel));
     if (fa.maxDynamicSharedSizeBytes < C::kLdsBytes) {
@@ -1321,8 +1288,11 @@ int launch_nn(GemmParams p, hipStream_t s) {
   p.tiles_n = p.N / kNBN;
   const bool packed = packed_epilogue(p) && !host_has_tail(p);  // (a fused tail goes through the element stores here)
   const void *kernel = packed ? (const void *)nn_kernel<T, BK, STAGES, true> : (const void *)nn_kernel<T, BK, STAGES, false>;
-  static bool configured[2] = {false, false};  // idempotent; a race only repeats the calls
-  if (!configured[packed]) {
+  static bool configured_on[kMaxDevices][2];  // per device and kernel; idempotent, a race only repeats the calls
+  int dev = 0;
+  KAPY_HIP_CHECK(hipGetDevice(&dev));
+  bool(&configured)[2] = configured_on[dev >= 0 && dev < kMaxDevices ? dev : 0];
+  if (!configured[packed] || dev >= kMaxDevices) {
     hipFuncAttributes fa;
     KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, kernel));
     if (fa.maxDynamicSharedSizeBytes < kLds) {
@@ -1352,7 +1322,11 @@ int launch_staged(GemmParams p, int a_mode, int b_mode, hipStream_t s) {
   return KAPY_OK;
 }
 
-// Kapy.cpp:451-487 (shape / element type rules) and :491-564 (minimum tile sizes).
+// The shape and element-type rules of Kapy.cpp:451-487, with the reference's wording.  Not taken over: the minimum
+// extents of :491-564 (acc at least 16x8, lhs / rhs at least 16x8, 16x16 or 8x8 per MMA way) - they bound a warp's
+// register tile, and this entry point takes whole views of any extent (a decode-shaped M = 1 included) - and the rule
+// that the RESULT is f16 or f32: it is applied to the accumulator operand only, because `result` here is the view the
+// kernel's final fptofp stores into (f16, bf16 or f32).
 int verify_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *res, int impl_way) {
   int rc = check_global(lhs, "matmul lhs");
   if (!rc) rc = check_global(rhs, "matmul rhs");
@@ -1407,10 +1381,6 @@ const TnVariant kTnVariants[] = {
     KAPY_TN16(256, 256, 64, 2, 2, kRing25), KAPY_TN16(256, 256, 64, 2, 2, 2),
     KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN16(128, 128, 64, 2, 2, kRing25),
     KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
-#ifdef KAPY_TUNING
-    KAPY_TN(256, 256, 32, 2, 2, 3), KAPY_TN(256, 256, 32, 2, 4, 4), KAPY_TN(256, 256, 64, 2, 4, 2), KAPY_TN(256, 128, 64, 2, 2, 3),
-    KAPY_TN(128, 256, 64, 2, 2, 3), KAPY_TN(128, 128, 64, 2, 2, 4), KAPY_TN(256, 256, 32, 2, 2, 5), KAPY_TN(256, 128, 32, 2, 2, 4),
-#endif
 };
 
 int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
@@ -1508,19 +1478,16 @@ int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k) {
   return KAPY_OK;
 }
 
-#ifndef KAPY_F8_STAGES
-#define KAPY_F8_STAGES kRing25
-#endif
 int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
   if (p.a_sm * 256 >= (int64_t(1) << 31) || p.b_sn * 256 >= (int64_t(1) << 31)) return KAPY_ERR_UNSUPPORTED;
   // the ring variants take any M, N >= 128 and any K >= 128 of whole 16-byte chunks (their loads are bounded by the
   // operands' ends); 256x256 tiles when there are at least as many of them as CUs, 128x128 (two workgroups per CU) below
-  if (KAPY_F8_STAGES == kRing25 && p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
-    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<256, 256, 128, 2, 2, KAPY_F8_STAGES>(p, lhs_fmt, rhs_fmt, s);
+  if (p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
+    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
     return launch_f8<128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
-    return launch_f8<256, 256, 128, 2, 2, KAPY_F8_STAGES>(p, lhs_fmt, rhs_fmt, s);
+    return launch_f8<256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
   return KAPY_ERR_UNSUPPORTED;
 }
@@ -1551,9 +1518,6 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
     return fail(KAPY_ERR_UNSUPPORTED, "matmul: %s operands have no matrix instruction on gfx950", dtype_name(lhs->dtype));
 
   GemmParams p;
-#ifdef KAPY_TRACE
-  const char *trace_env = getenv("KAPY_TRACE_PTR");
-#endif
   p.a = view_base(lhs);
   p.b = view_base(rhs);
   p.acc = acc ? view_base(acc) : nullptr;
@@ -1564,9 +1528,6 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
   p.alpha = epi ? epi->alpha : 1.0f;
   p.act = epi ? epi->act : -1;
   p.act_operand = epi ? epi->act_operand : 0.f;
-#ifdef KAPY_TRACE
-  if (trace_env) p.col_scale = (const float *)strtoull(trace_env, nullptr, 0);
-#endif
   p.a_sm = lhs->stride0; p.a_sk = lhs->stride1;
   p.b_sk = rhs->stride0; p.b_sn = rhs->stride1;
   p.acc_sm = acc ? acc->stride0 : 0; p.acc_sn = acc ? acc->stride1 : 0;
@@ -1664,7 +1625,6 @@ int kapy_matmul_static_workspace(const kapy_global *lhs, const kapy_global *rhs,
   if (rc) return rc;
   // The array's name is a host-side handle, not a device address: ask the runtime once per device where this device's
   // copy lives, and hand that pointer to the kernels.
-  constexpr int kMaxDevices = 64;
   static void *scratch_on_device[kMaxDevices];  // (a race between two first calls only repeats the query)
   int dev = -1;
   KAPY_HIP_CHECK(hipGetDevice(&dev));

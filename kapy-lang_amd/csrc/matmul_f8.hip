@@ -92,16 +92,7 @@ __device__ __forceinline__ i32x8 load_k32(const uint8_t *base, int64_t stride, i
 // A wave first requests everything it will multiply in a chunk of CH K-steps - the weight bytes of
 // its NG column groups and the activation bytes they share - and only then starts the matrix
 // instructions, so that a CU keeps >100 KiB of HBM reads in flight with only 8 resident waves.
-#ifndef KAPY_SKINNY_NG
-#define KAPY_SKINNY_NG 1
-#endif
-#ifndef KAPY_SKINNY_CH
-#define KAPY_SKINNY_CH 8
-#endif
-#ifndef KAPY_SKINNY_OLD
-#define KAPY_SKINNY_OLD 0
-#endif
-constexpr int kSkinnyWaves = 8;
+constexpr int kSkinnyWaves = 8, kSkinnyGroups = 1, kSkinnyChunk = 8;  // wavefronts, 16-column groups per workgroup, K-steps requested ahead
 template <int A_FMT, int B_FMT, int NG, int CH>
 __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
   __shared__ float partial[kSkinnyWaves][NG][16][16 + 1];
@@ -157,14 +148,8 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 // Rows past M / N are clamped to the last valid row (never stored), so nothing is read out of range.
 // From this many rows on the tiled MFMA kernel (which reads the weight once for up to 128 rows) beats the weight-streaming
 // kernel below (which reads it once per 16 rows).
-#ifndef KAPY_F8_TILED_FROM_M
-#define KAPY_F8_TILED_FROM_M 81
-#endif
-constexpr int kTiledFromM = KAPY_F8_TILED_FROM_M;
-#ifndef KAPY_F8_TILED_FROM_M_SPLIT
-#define KAPY_F8_TILED_FROM_M_SPLIT 40
-#endif
-constexpr int kTiledFromMSplit = KAPY_F8_TILED_FROM_M_SPLIT;  // the same threshold when K can be split across workgroups
+constexpr int kTiledFromM = 81;
+constexpr int kTiledFromMSplit = 40;  // the same threshold when K can be split across workgroups (measured at N = K = 8192)
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
 template <int A_FMT, int B_FMT>
 __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Params p) {
@@ -298,7 +283,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
   }
   if (k_contig && p.K % (kStreamWaves * kStreamChunk) == 0 && (p.M + 15) / 16 <= 65535 && p.a_sm * 16 < (int64_t(1) << 31) &&
-      p.b_sn * 16 < (int64_t(1) << 31) && !KAPY_SKINNY_OLD) {
+      p.b_sn * 16 < (int64_t(1) << 31)) {
     // rows are addressed from the workgroup's first row, so the per-lane offsets stay small
     F8Params q = p;
     const int64_t col_rounds = ((p.N + 15) / 16 + 7) / 8, groups = (p.M + 15) / 16;
@@ -312,7 +297,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     return KAPY_OK;
   }
   if (k_contig) {
-    constexpr int NG = KAPY_SKINNY_NG, CH = KAPY_SKINNY_CH;
+    constexpr int NG = kSkinnyGroups, CH = kSkinnyChunk;
     dim3 grid((unsigned)((p.N + 16 * NG - 1) / (16 * NG)), (unsigned)((p.M + 15) / 16));
     if (grid.y <= 65535) {
       int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);

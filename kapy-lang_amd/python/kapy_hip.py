@@ -15,6 +15,7 @@ F16, BF16, F32, F8E4M3, F8E5M2, I8, I16, I32 = range(8)
 RZ, RN = 0, 1
 PAD_ZERO, PAD_QNAN, PAD_PINF, PAD_NINF = range(4)
 CACHE_NONE, CACHE_CA, CACHE_CG, CACHE_CS = 0, 1, 2, 3
+EVICT_NORMAL, EVICT_FIRST, EVICT_LAST, EVICT_UNCHANGED, NO_ALLOCATE = range(5)
 OK, ERR_INVALID, ERR_VERIFY, ERR_UNSUPPORTED, ERR_HIP = 0, -1, -2, -3, -4
 MATMUL_AUTO, MMA_M16N8K8_F16, MMA_M16N8K16_F16, MMA_M16N8K8_TF32, MMA_M16N8K16_F8 = 0, 1, 2, 3, 4
 MFMA_32X32X16_16B, MFMA_16X16X32_16B, MFMA_16X16X128_F8, MFMA_32X32X64_F8 = 16, 17, 18, 19
@@ -34,6 +35,7 @@ EXPORTS = [
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
     "kapy_mfma_probe", "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
+    "kapy_mk_shared", "kapy_sv_shared", "kapy_shared_address",
 ]
 
 
@@ -72,7 +74,12 @@ class Swizzling(C.Structure):
 
 class CopyCfg(C.Structure):
     _fields_ = [("transpose", C.c_int32), ("padding_option", C.c_int32), ("cache_modifier", C.c_int32),
-                ("reserved", C.c_int32)]
+                ("evict_priority", C.c_int32), ("is_volatile", C.c_int32), ("reserved", C.c_int32)]
+
+
+class Shared(C.Structure):
+    _fields_ = [("offset", C.c_int64), ("start0", C.c_int32), ("start1", C.c_int32), ("end0", C.c_int32), ("end1", C.c_int32),
+                ("dtype", C.c_int32), ("layout", Swizzling)]
 
 
 class Grid2(C.Structure):
@@ -130,6 +137,10 @@ def lib():
     L.kapy_device_info.argtypes = [P(i32), P(i32), P(i32), C.c_char_p, i32]
     L.kapy_mk_global.argtypes = [P(Global), vp, i32, i32, i32, i32, i32, i32, i32]
     L.kapy_sv_global.argtypes = [P(Global), P(Global), i32, i32, i32, i32]
+    L.kapy_mk_shared.argtypes = [P(Shared), i64, i32, i32, i32, i32, i32, i32]
+    L.kapy_sv_shared.argtypes = [P(Shared), P(Shared), i32, i32, i32, i32]
+    L.kapy_shared_address.restype = i64
+    L.kapy_shared_address.argtypes = [P(Shared), i64, i64]
     L.kapy_fragments_loops.argtypes = [P(Fragments), A2, A2, A2]
     L.kapy_fragments_map.argtypes = [P(Fragments), A2, i32, A2, A2]
     L.kapy_fragments_transpose.argtypes = [P(Fragments), P(Fragments)]
@@ -172,7 +183,7 @@ def lib():
     for name in EXPORTS:
         f = getattr(L, name)
         if name not in ("kapy_last_error", "kapy_smem_plan", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset",
-                        "kapy_matmul_workspace_bytes"):
+                        "kapy_matmul_workspace_bytes", "kapy_shared_address"):
             f.restype = C.c_int
     _lib = L
     return L
@@ -228,13 +239,13 @@ def current_stream():
 
 
 # ---------------------------------------------------------------- ops
-def copy(src, dst, transpose=False, padding=PAD_ZERO, cache=CACHE_NONE, stream=None):
-    cfg = CopyCfg(int(transpose), padding, cache, 0)
+def copy(src, dst, transpose=False, padding=PAD_ZERO, cache=CACHE_NONE, evict=EVICT_NORMAL, volatile=False, stream=None):
+    cfg = CopyCfg(int(transpose), padding, cache, evict, int(volatile), 0)
     check(lib().kapy_copy(C.byref(src), C.byref(dst), C.byref(cfg), stream if stream is not None else current_stream()))
 
 
-def copy_batched(src, dst, grid, transpose=False, padding=PAD_ZERO, cache=CACHE_NONE, stream=None):
-    cfg = CopyCfg(int(transpose), padding, cache, 0)
+def copy_batched(src, dst, grid, transpose=False, padding=PAD_ZERO, cache=CACHE_NONE, evict=EVICT_NORMAL, volatile=False, stream=None):
+    cfg = CopyCfg(int(transpose), padding, cache, evict, int(volatile), 0)
     g = Grid2(*grid)
     check(lib().kapy_copy_batched(C.byref(src), C.byref(dst), C.byref(cfg), C.byref(g),
                                   stream if stream is not None else current_stream()))

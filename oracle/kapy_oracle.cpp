@@ -741,7 +741,13 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
         case EW_SUBF: r = a - reg[I.b][at]; break;
         case EW_MULF: r = a * reg[I.b][at]; break;
         case EW_DIVF: r = a / reg[I.b][at]; break;
-        case EW_FMA: r = std::fma(a, reg[I.b][at], reg[I.c][at]); break;
+        // One rounding of the exact a*b + c to the register type.  For f16 / bf16 the double-precision fma followed by the
+        // rounding to 16 bits is that (a value on a 16-bit rounding boundary needs the product to supply both the boundary
+        // bit and a lower one, which spans at most 22 + 11 bits: exact in a double).  For f32 it is not (add, sub, mul, div
+        // survive the detour through double, fma does not), so the fma is taken in float.
+        case EW_FMA:
+          r = dst_dtype == KO_F32 ? (double)std::fmaf((float)a, (float)reg[I.b][at], (float)reg[I.c][at]) : std::fma(a, reg[I.b][at], reg[I.c][at]);
+          break;
         // arith.maximumf / minimumf propagate NaN
         // arith.maximumf / minimumf: NaN if either operand is, and -0 orders below +0 (max.NaN / min.NaN of PTX do the same)
         case EW_MAXIMUMF: {

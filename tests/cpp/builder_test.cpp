@@ -73,6 +73,29 @@ static int run_cpu() {
   } catch (const kapy::Error &e) {
     EXPECT(e.status == KAPY_ERR_UNSUPPORTED || e.status == KAPY_ERR_VERIFY);
   }
+  // what follows a matmul is typed like any other chain: the stored value has the target's element type, a cast to another
+  // type or a missing cast is refused, and a 16-bit bias row must be widened before it joins the f32 accumulator
+  {
+    kapy::Value a16 = b.create_mk_global(fake, 0, 128, 128, 128, 1, KAPY_F16), c16 = b.create_mk_global(fake, 0, 128, 128, 128, 1, KAPY_F16);
+    kapy::Value c32 = b.create_mk_global(fake, 0, 128, 128, 128, 1, KAPY_F32), brow = b.create_mk_global(fake, 0, 1, 128, 128, 1, KAPY_F16);
+    auto mm = [&] { return b.create_matmul(b.create_ld_global(a16), b.create_ld_global(a16)); };
+    auto refused = [&](kapy::Value v, kapy::Value target, int status, const char *words) {
+      try {
+        b.create_st_global(v, target);
+      } catch (const kapy::Error &e) {
+        return e.status == status && strstr(e.what(), words) != nullptr;
+      }
+      return false;
+    };
+    EXPECT(refused(mm(), c16, KAPY_ERR_VERIFY, "same element type"));                                         // f32 result, f16 view, no cast
+    EXPECT(refused(b.create_truncf(mm(), KAPY_BF16), c16, KAPY_ERR_VERIFY, "same element type"));             // cast to another type than the view's
+    EXPECT(refused(b.create_truncf(mm(), KAPY_F16), c32, KAPY_ERR_VERIFY, "same element type"));
+    EXPECT(refused(b.create_truncf(b.create_addf(mm(), b.create_ld_global(brow)), KAPY_F16), c16, KAPY_ERR_VERIFY, "same element type"));   // f16 bias, not widened
+    // a legal chain with a round-toward-zero cast passes the typing and reaches the device call (which fails without a device)
+    int n_dev0 = 0;
+    if (hipGetDeviceCount(&n_dev0) != hipSuccess || n_dev0 == 0)
+      EXPECT(refused(b.create_fptofp(b.create_addf(mm(), b.create_extf(b.create_ld_global(brow), KAPY_F32)), KAPY_F16, KAPY_RZ), c16, KAPY_ERR_HIP, "no CPU fallback"));
+  }
   int n_dev = 0;
   if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
     try {
@@ -149,6 +172,18 @@ static int run_gpu() {
       ref2 += want * want;
     }
   EXPECT(sqrt(err2 / ref2) <= 4e-3);   // bf16 result: half an ulp (2^-9) per element at most, well inside
+  // the same chain with a round-toward-zero cast: every element is the RN result or its neighbour toward zero, and never
+  // larger in magnitude than the exact value
+  std::vector<uint16_t> cz(M * N);
+  b.create_st_global(b.create_fptofp(b.create_maximumf(t, b.create_splat(0.f, KAPY_F32)), KAPY_BF16, KAPY_RZ), gc);
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(cz.data(), dc, cz.size() * 2, hipMemcpyDeviceToHost));
+  int differ = 0;
+  for (int i = 0; i < M * N; ++i) {
+    EXPECT(cz[i] == c[i] || cz[i] + 1 == c[i]);   // (results are >= 0 after the relu: the pattern below is the value toward zero)
+    differ += cz[i] != c[i];
+  }
+  EXPECT(differ > M * N / 8);   // about half of all roundings go up under RN
   printf("builder gpu ok\n");
   return 0;
 }

@@ -164,3 +164,21 @@ def test_config3b_permute_bhsd_bit_exact(ko):
                     (b, h, s * h * d, d, h * s * d, s * d))
     sync()
     assert np.array_equal(to_host(d_back, np.uint16, (b, h, s, d)), src)
+
+
+def test_cache_hints_do_not_change_results(ko):
+    """EvictPriority and isVolatile of create_ld_global / create_st_global (python/src/ir.cc:1035-1049) choose between
+    ordinary and non-temporal access; the bits moved are the same under every combination, transposed or not."""
+    m, n = 256, 320
+    src = ko.fill_bits16(m * n, 5).reshape(m, n)
+    d_src = to_dev(src)
+    for transpose in (False, True):
+        want = src.T if transpose else src
+        dm, dn = want.shape
+        for cache, evict, vol in ((kh.CACHE_NONE, kh.EVICT_NORMAL, False), (kh.CACHE_NONE, kh.EVICT_FIRST, False), (kh.CACHE_NONE, kh.NO_ALLOCATE, False),
+                                  (kh.CACHE_NONE, kh.EVICT_LAST, False), (kh.CACHE_NONE, kh.EVICT_UNCHANGED, False), (kh.CACHE_CS, kh.EVICT_LAST, False),
+                                  (kh.CACHE_CS, kh.EVICT_FIRST, True), (kh.CACHE_CA, kh.EVICT_FIRST, False)):
+            d_dst = dev_zeros(m * n, 2, fill=0x5A5A)
+            kh.copy(dglobal(d_src, m, n, n, 1, kh.F16), dglobal(d_dst, dm, dn, dn, 1, kh.F16), transpose=transpose, cache=cache, evict=evict, volatile=vol)
+            sync()
+            assert np.array_equal(to_host(d_dst, np.uint16, (dm, dn)), want), (transpose, cache, evict, vol)

@@ -27,7 +27,7 @@ def test_struct_layout_matches_header_and_oracle(ko):
     assert C.sizeof(kh.Global) == C.sizeof(ko.Global) == 40
     assert C.sizeof(kh.Fragments) == C.sizeof(ko.Fragments) == 24
     assert C.sizeof(kh.EwInst) == C.sizeof(ko.EwInst) == 32
-    assert C.sizeof(kh.MatmulCfg) == 48 and C.sizeof(kh.Grid2) == 40 and C.sizeof(kh.CopyCfg) == 16
+    assert C.sizeof(kh.MatmulCfg) == 48 and C.sizeof(kh.Grid2) == 40 and C.sizeof(kh.CopyCfg) == 24 and C.sizeof(kh.Shared) == 48
 
 
 def test_descriptors_match_oracle(ko):
@@ -112,6 +112,48 @@ def test_default_layout_simd_change_agree_with_oracle(ko):
     assert L.kapy_change_num_shuffles(C.byref(s), C.byref(d), kh.A2(*shape)) == \
         O.ko_change_num_shuffles(C.byref(so), C.byref(do), kh.A2(*shape), 64)
     assert L.kapy_fragments_default(kh.A2(1, 1), kh.A2(24, 8), 1, C.byref(kh.Fragments())) == kh.ERR_VERIFY  # OpTraits.cpp:43-58
+
+
+def test_shared_memory_descriptors_follow_the_lowering(ko):
+    """kapy.mk_shared / sv_shared as plain data (MkSharedOpToLLVM.cpp:49-70, SvSharedOpToLLVM.cpp:20-42): start 0 / end = shape,
+    strides by orientation, sub-view bounds counted from the SOURCE view's start, addresses through the swizzle function."""
+    L, O = kh.lib(), ko.lib()
+    t = kh.Shared()
+    assert L.kapy_mk_shared(C.byref(t), 16384, 64, 32, kh.F16, 1, 4, 4) == 0
+    assert (t.offset, t.start0, t.start1, t.end0, t.end1, t.dtype) == (16384, 0, 0, 64, 32, kh.F16)
+    assert (t.layout.stride0, t.layout.stride1, t.layout.bank_param, t.layout.line_param) == (32, 1, 4, 4)
+    c = kh.Shared()
+    assert L.kapy_mk_shared(C.byref(c), 0, 64, 32, kh.F16, 0, 0, 0) == 0
+    assert (c.layout.stride0, c.layout.stride1, c.layout.bank_param, c.layout.line_param) == (1, 64, 4, 1)
+    v, w = kh.Shared(), kh.Shared()
+    assert L.kapy_sv_shared(C.byref(v), C.byref(t), 16, 48, 8, 24) == 0
+    assert (v.start0, v.end0, v.start1, v.end1, v.offset) == (16, 48, 8, 24, 16384)
+    assert L.kapy_sv_shared(C.byref(w), C.byref(v), 4, 8, 2, 6) == 0       # new end = old START + end, not old end
+    assert (w.start0, w.end0, w.start1, w.end1) == (20, 24, 10, 14)
+    for (i, j) in ((0, 0), (3, 5), (31, 15), (17, 0)):
+        want = 16384 + O.ko_swizzle_offset(16 + i, 8 + j, 32, 1, 16, 4, 4, 64) * 2
+        assert L.kapy_shared_address(C.byref(v), i, j) == want
+    assert L.kapy_shared_address(C.byref(v), 32, 0) == kh.ERR_VERIFY and L.kapy_shared_address(C.byref(v), 0, 16) == kh.ERR_VERIFY
+    assert L.kapy_shared_address(C.byref(v), -17, 0) == kh.ERR_VERIFY      # unsigned compare: a negative index is out of bounds
+    # every element of an unswizzled and of a swizzled buffer has an address of its own inside the buffer
+    for bp, lp in ((0, 0), (4, 8), (2, 16)):
+        assert L.kapy_mk_shared(C.byref(t), 1024, 32, 64, kh.BF16, 1, bp, lp) == 0
+        seen = {L.kapy_shared_address(C.byref(t), i, j) for i in range(32) for j in range(64)}
+        assert len(seen) == 32 * 64 and min(seen) == 1024 and max(seen) == 1024 + 32 * 64 * 2 - 2
+    assert L.kapy_mk_shared(C.byref(t), 0, 48, 32, kh.F16, 1, 0, 0) == kh.ERR_VERIFY            # OpTraits.cpp:43-58: powers of two
+    assert L.kapy_mk_shared(C.byref(t), 100, 32, 32, kh.F16, 1, 0, 0) == kh.ERR_INVALID         # 128-byte aligned (AllocAnalysis)
+    assert L.kapy_mk_shared(C.byref(t), 128 * 1024, 256, 128, kh.F16, 1, 0, 0) == kh.ERR_VERIFY  # beyond 160 KiB
+    assert L.kapy_mk_shared(C.byref(t), 0, 32, 32, kh.F16, 1, 3, 1) == kh.ERR_INVALID
+    assert L.kapy_sv_shared(C.byref(v), C.byref(t), 8, 4, 0, 4) == kh.ERR_INVALID
+
+
+def test_copy_hints_are_validated():
+    g = _g()
+    for kw in (dict(cache=9), dict(evict=5), dict(evict=-1), dict(padding=4)):
+        st, msg = _status(kh.copy, g, g, stream=NULL, **kw)
+        assert st == kh.ERR_INVALID, kw
+    st, msg = _status(kh.copy, g, g, evict=kh.NO_ALLOCATE, volatile=True, stream=NULL)
+    assert st == kh.ERR_HIP       # accepted by the verifier; only the missing device stops it here
 
 
 def test_swizzle_agrees_with_oracle_and_matmul_layout_is_searched(ko):

@@ -294,3 +294,27 @@ def test_gelu_tail_keeps_its_relative_accuracy(ko):
     want = (vl / (1 + np.exp(-2 * u))).astype(np.float64)
     assert np.all(want < 0) and want[-1] > -1e-20
     assert np.max(np.abs(got - want) / np.abs(want)) <= 2.0 ** -8        # half an ulp of bf16
+
+
+def test_f32_fma_rounds_once(ko):
+    """a*b + c in f32 where a detour through a double-precision fma would round twice: a = b = 1 + 2^-12, c = 2^-60 gives exactly
+    1 + 2^-11 + 2^-24 + 2^-60, just above the midpoint of two floats; a double drops the 2^-60 and leaves the tie, which then goes
+    to even (1 + 2^-11); one rounding gives 1 + 2^-11 + 2^-23.  Plus a sample of random operands against exact rational arithmetic."""
+    from fractions import Fraction
+    insts = [dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_LD_GLOBAL, dst=1, a=1), dict(op=ko.EW_LD_GLOBAL, dst=2, a=2),
+             dict(op=ko.EW_FMA, dst=3, a=0, b=1, c=2), dict(op=ko.EW_ST_GLOBAL, a=3)]
+    n = 1000
+    g = lambda x: ko.mk_global(x, 1, n, n, 1, ko.F32)
+    rng = np.random.default_rng(0)
+    aa, bb = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    cc = (-(aa.astype(np.float64) * bb.astype(np.float64))).astype(np.float32) + rng.standard_normal(n).astype(np.float32) * np.float32(1e-7)   # heavy cancellation
+    aa[0] = bb[0] = np.float32(1.0 + 2.0 ** -12)
+    cc[0] = np.float32(2.0 ** -60)
+    out = np.zeros(n, np.float32)
+    assert ko.elementwise(ko.program(insts), [g(aa), g(bb), g(cc)], g(out)) == 0
+    assert out[0] == np.float32(1.0 + 2.0 ** -11 + 2.0 ** -23)
+    assert np.float32(np.float64(aa[0]) * np.float64(bb[0]) + np.float64(cc[0])) == np.float32(1.0 + 2.0 ** -11)   # what rounding twice gives
+    for k in range(1, n, 13):
+        exact = Fraction(float(aa[k])) * Fraction(float(bb[k])) + Fraction(float(cc[k]))
+        lo, hi = np.nextafter(out[k], np.float32(-np.inf)), np.nextafter(out[k], np.float32(np.inf))
+        assert abs(Fraction(float(out[k])) - exact) <= min(abs(Fraction(float(lo)) - exact), abs(Fraction(float(hi)) - exact))

@@ -633,8 +633,72 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     return out
 
 
+def bench_ceilings(kh, steps, warmup, cpu):
+    """What this device sustains, from the library's own probe kernels: a loop of nothing but matrix instructions per
+    instruction shape (operands of the benchmark's distribution; the part is power-limited, so this, not the data-sheet
+    figure, is what a GEMM can approach) with the shader clock it holds, and a plain 16-byte-per-lane copy of 2 x 128 MiB
+    in every form a memory-bound kernel could take (vectors per lane, non-temporal or not, one pass or persistent)."""
+    import numpy as np
+    import torch
+    import ko
+    out = {"workload": "device ceilings (the library's probe kernels)", "checked": True, "check": "nothing to check: measurement only", "mfma": {}, "copy": {}}
+    sink = torch.empty(1024 * 256, device="cuda", dtype=torch.float32)
+    ticks = torch.zeros(4 * 1024, device="cuda", dtype=torch.int64)
+    for name, way, dt, gen, peak in (("bf16 16x16x32", kh.MFMA_16X16X32_16B, kh.BF16, "normal002", 2500.0), ("bf16 32x32x16", kh.MFMA_32X32X16_16B, kh.BF16, "normal002", 2500.0),
+                                     ("f16 16x16x32", kh.MFMA_16X16X32_16B, kh.F16, "uniform", 2500.0), ("e4m3 16x16x128", kh.MFMA_16X16X128_F8, kh.F8E4M3, "quant", 5000.0),
+                                     ("e4m3 32x32x64", kh.MFMA_32X32X64_F8, kh.F8E4M3, "quant", 5000.0)):
+        n = 131072 // kh.DTYPE_BYTES[dt]
+        if gen == "normal002":
+            ops = _upload(ko.fill_normal(n, dt, 0, 0, 0.0, 0.02))
+        elif gen == "uniform":
+            ops = _upload(ko.fill_uniform(n, dt, 0, 0))
+        else:   # e4m3 values as the W8A8 quantiser leaves them: normal(0,1) scaled so that the largest of 8192 is 448
+            x = ko.fill_normal(n, ko.F32, 0, 0).reshape(-1, 8192)
+            q, sc = np.zeros(x.shape, np.uint8), np.zeros(x.shape[0], np.float32)
+            ko.lib().ko_quantize_e4m3(x.ctypes.data, x.shape[0], x.shape[1], x.shape[1], 1, 1, q.ctypes.data, sc.ctypes.data)
+            ops = _upload(q)
+        iters = 2000
+        wgs, flops = kh.probe_mfma(way, dt, ops.data_ptr(), iters, sink.data_ptr())
+        wall, ev = _events(lambda i: kh.probe_mfma(way, dt, ops.data_ptr(), iters, sink.data_ptr(), ticks.data_ptr()), max(steps // 2, 5), warmup)
+        torch.cuda.synchronize()
+        t = ticks.cpu().numpy()[:4 * wgs].reshape(wgs, 4).astype(np.float64)
+        ghz = float(np.median((t[:, 1] - t[:, 0]) / np.maximum(t[:, 3] - t[:, 2], 1.0)) * 0.1)    # shader ticks per 100 MHz tick
+        tf = flops / (ev * 1e-3) / 1e12
+        out["mfma"][name] = {"tflops": round(tf, 1), "frac_of_peak": round(tf / peak, 4), "shader_clock_ghz": round(ghz, 3), "kernel_ms": round(ev, 4)}
+    nbytes, sets = 128 << 20, 4
+    src = [_dev("bits16", nbytes // 2, ko.F16, 0, k) for k in range(sets)]
+    dst = [torch.empty(nbytes // 2, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    kh.probe_copy(src[0].data_ptr(), dst[0].data_ptr(), nbytes)
+    torch.cuda.synchronize()
+    if not torch.equal(src[0], dst[0]):
+        raise CheckFailed("probe_copy: result differs from the source")
+    best = 0.0
+    for u in (1, 2, 4, 8, 16):
+        for ntl, nts in ((0, 0), (1, 0), (0, 1), (1, 1)):
+            for pers in (0, 4, 8, 16):
+                if pers and u > 8:
+                    continue
+                wall, ev = _events(lambda i: kh.probe_copy(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), nbytes, u, ntl, nts, pers), 20, 3)
+                gbs = 2 * nbytes / (ev * 1e-3) / 1e9
+                best = max(best, gbs)
+                out["copy"]["vec%d ntld%d ntst%d %s" % (u, ntl, nts, "persistent x%d" % pers if pers else "one pass")] = round(gbs, 0)
+    # the same bytes with the access footprint of the 16-bit tile transpose (four 256-byte pieces of four rows per wave
+    # instruction instead of one contiguous KiB), untransposed: what the transposes can reach
+    n = 8192
+    for lds in (0, 1):
+        kh.probe_copy_tiled(src[0].data_ptr(), dst[0].data_ptr(), n, n * 2, lds)
+        torch.cuda.synchronize()
+        if not torch.equal(src[0], dst[0]):
+            raise CheckFailed("probe_copy_tiled: result differs from the source")
+        wall, ev = _events(lambda i: kh.probe_copy_tiled(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, lds), 40, 5)
+        out["copy"]["transpose footprint (128 rows x 256 B per workgroup)%s" % (", through LDS and a barrier" if lds else "")] = round(2 * nbytes / (ev * 1e-3) / 1e9, 0)
+    out["copy_best_gbs"] = round(best, 0)
+    out["copy_best_frac_of_peak"] = round(best / HBM_PEAK_GBS, 4)
+    return out
+
+
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m64_splitk", "f8_m4096"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m64_splitk", "f8_m4096", "ceilings"]
 
 
 def main():
@@ -678,7 +742,11 @@ def main():
         "f8_m64": lambda s, w: bench_f8(kh, s, w, False, 64),
         "f8_m64_splitk": lambda s, w: bench_f8(kh, s, w, False, 64, workspace=True),
         "f8_m4096": lambda s, w: bench_f8(kh, s, w, cpu, 4096),
+        "ceilings": lambda s, w: bench_ceilings(kh, s, w, cpu),
     }
+    if args.workload == "ceilings":
+        print(json.dumps(table["ceilings"](args.steps, args.warmup)))
+        return
     try:
         main_res = table[args.workload](args.steps, args.warmup)
     except CheckFailed as e:
@@ -697,9 +765,10 @@ def main():
             except CheckFailed as e:
                 others.append({"workload": name, "error": "correctness gate failed, not timed: %s" % e, "checked": False})
                 continue
-            r["value"] = round(r["value"], 2)
-            r["ms_per_step"] = round(r["ms_per_step"], 4)
-            r["kernel_ms"] = round(r["kernel_ms"], 4)
+            if "value" in r:
+                r["value"] = round(r["value"], 2)
+                r["ms_per_step"] = round(r["ms_per_step"], 4)
+                r["kernel_ms"] = round(r["kernel_ms"], 4)
             others.append(r)
     line = {
         "metric": "GEMM TFLOP/s + % MFMA peak; elementwise/transpose GB/s + % HBM peak (1 GPU)",

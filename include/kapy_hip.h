@@ -166,6 +166,28 @@ int kapy_mfma_probe(int32_t impl_way, int32_t lhs_dtype, int32_t rhs_dtype, int3
  * MFMA operand layout), so callers and tests can check it is conflict-free by construction. */
 int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out);
 
+/* ---------------------------------------------------------------- device ceilings */
+/* What the device sustains, so that a kernel's rate can be read against a reproducible ceiling as well as against the
+ * data-sheet peak (the reference emits code and never runs it; nothing there to cite beyond the instructions it names,
+ * MatmulOpToLLVM.cpp:269-311, LdGlobalOpToLLVM.cpp:60-145).
+ * kapy_probe_mfma: every CU runs `iterations` rounds of independent matrix instructions of `impl_way` (16..19) with the
+ * register blocking of the tiled matmul and no memory traffic.  operands: 128 KiB of device memory holding operand
+ * values of `dtype` (the power drawn, and so the clock held, depends on them); sink: one float per lane (workgroups *
+ * 256); ticks (may be NULL): per workgroup {shader clock at start, at end, 100 MHz timer at start, at end}.  Reports
+ * the workgroups launched and the flops of the launch. */
+int kapy_probe_mfma(int32_t impl_way, int32_t dtype, const void *operands, int32_t iterations, float *sink, uint64_t *ticks, int32_t *workgroups,
+                    int64_t *flops, void *stream);
+/* kapy_probe_copy: dst <- src, `bytes` (a multiple of 16) moved 16 bytes per lane with 1, 2, 4, 8 or 16 vectors per lane in
+ * flight, ordinary or non-temporal loads / stores, in one pass (persistent_per_cu = 0) or by that many persistent
+ * workgroups per CU striding over the buffers.  ticks as above (4 values per workgroup; may be NULL). */
+int kapy_probe_copy(const void *src, void *dst, int64_t bytes, int32_t vectors_per_lane, int32_t nt_load, int32_t nt_store, int32_t persistent_per_cu,
+                    uint64_t *ticks, int32_t *workgroups, void *stream);
+
+/* A copy with the access footprint of the 16-bit tile transpose (a workgroup moves 128 rows x 256 bytes of a [rows][row_bytes]
+ * matrix, one wave instruction touches four 256-byte pieces of four rows), untransposed, directly or through an LDS tile and
+ * a barrier: what that footprint and that detour cost against kapy_probe_copy. */
+int kapy_probe_copy_tiled(const void *src, void *dst, int64_t rows, int64_t row_bytes, int32_t through_lds, void *stream);
+
 /* ---------------------------------------------------------------- device ops */
 typedef struct kapy_copy_cfg {
   int32_t transpose;      /* 1: kapy.transpose between the load and the store (dst[i,j] = src[j,i]) */

@@ -18,12 +18,7 @@
 //   generic_kernel    anything else (no contiguous axis, misaligned rows): one element per lane.
 #include "common.hpp"
 
-#ifndef KAPY_TRANSPOSE_MAP
-#define KAPY_TRANSPOSE_MAP 2
-#endif
-#ifndef KAPY_TRANSPOSE_LDS
-#define KAPY_TRANSPOSE_LDS 1
-#endif
+constexpr int kTransposeMap = 2;  // workgroup -> tile order of the transposes: 0 row by row, 1 column by column, 2 diagonal
 
 namespace kapy {
 namespace {
@@ -90,14 +85,11 @@ template <> struct VecOf<16> { typedef u32x4 type; };
 template <> struct VecOf<8> { typedef u32x2 type; };
 template <> struct VecOf<4> { typedef uint32_t type; };
 
-#ifndef KAPY_ROWS_UNROLL
-#define KAPY_ROWS_UNROLL 1
-#endif
 template <int B, int VB, bool NT, bool RAGGED>
 __global__ __launch_bounds__(256) void rows_kernel(CopyParams p, int32_t vec_per_row) {
   typedef typename VecOf<VB>::type Vec;
   constexpr int E = VB / B;  // elements per vector
-  constexpr int UNROLL = KAPY_ROWS_UNROLL;
+  constexpr int UNROLL = 1;  // vectors per lane (more in flight per lane measured slower: the plain-copy probe has the figures)
   const char *src;
   char *dst;
   program_base<B>(p, src, dst);
@@ -327,7 +319,7 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
       int e = vb / B;
       int32_t vpr = (p.d1 + e - 1) / e;
       int64_t slots = slots_at_vb;
-      dim3 grid((unsigned)((slots + 256 * KAPY_ROWS_UNROLL - 1) / (256 * KAPY_ROWS_UNROLL)), 1, (unsigned)batch);
+      dim3 grid((unsigned)((slots + 256 - 1) / (256)), 1, (unsigned)batch);
       // no ragged vector anywhere: every slot is a whole in-bounds vector on both sides
       bool ragged = p.d1 % e != 0 || p.sb1 < p.d1 || p.sb0 < p.d0;
       if (vb == 16 && !ragged) {
@@ -343,15 +335,10 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
       KAPY_HIP_CHECK(hipGetLastError());
       return KAPY_OK;
     }
-  } else if (B == 2 && KAPY_TRANSPOSE_LDS && p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16 && p.d0 >= 128 && p.d1 >= 128 &&
-             (p.d1 + 127) / 128 <= 65535 && !(p.map_mode & 16)) {
-    const int shape = (p.map_mode >> 5) & 3;  // tuning builds select the tile; 0 = default
-    p.map_mode &= 15;
-    if (shape == 1) return launch_transpose_lds<256, 128>(p, nt, batch, stream);
-    if (shape == 2) return launch_transpose_lds<128, 256>(p, nt, batch, stream);
+  } else if (B == 2 && p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16 && p.d0 >= 128 && p.d1 >= 128 &&
+             (p.d1 + 127) / 128 <= 65535) {
     return launch_transpose_lds<128, 128>(p, nt, batch, stream);
   } else if (p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16) {
-    p.map_mode &= 15;
     constexpr int TILE = 8 * (16 / B);
     unsigned gx = (unsigned)((p.d0 + 2 * TILE - 1) / (2 * TILE)), gy = (unsigned)((p.d1 + 2 * TILE - 1) / (2 * TILE));
     if (gy <= 65535) {
@@ -409,7 +396,7 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   p.sb1 = (int32_t)(t ? extent0(src) : extent1(src));
   p.pad = padding_word(src->dtype, c.padding_option);
   p.n1 = g.n1 > 0 ? g.n1 : 1;
-  p.map_mode = KAPY_TRANSPOSE_MAP;
+  p.map_mode = kTransposeMap;
   p.s_off0 = g.src_off0;
   p.s_off1 = g.src_off1;
   p.d_off0 = g.dst_off0;

@@ -196,12 +196,8 @@ __device__ __forceinline__ float affine_act(float x, float scale, float bias, in
 }
 
 // 16-bit in, 16-bit out (same type), 8 elements per 16-byte vector, UNROLL vectors per lane.
-#ifndef KAPY_EW_UNROLL
-#define KAPY_EW_UNROLL 2
-#endif
-#ifndef KAPY_EW_NT
-#define KAPY_EW_NT 1
-#endif
+constexpr int kEwUnroll = 2;    // 16-byte vectors per lane of the flat fused kernels
+constexpr bool kEwNt = true;    // non-temporal loads and stores (the operands are streamed once)
 // 16 bytes at ptr, or the first `valid` elements of them at the ragged end of a row (RAGGED kernels only)
 template <bool RAGGED>
 __device__ __forceinline__ u32x4 load_row16(const char *ptr, int valid, bool stream) {
@@ -211,13 +207,13 @@ __device__ __forceinline__ u32x4 load_row16(const char *ptr, int valid, bool str
 template <bool RAGGED>
 __device__ __forceinline__ void store_row16(char *ptr, u32x4 v, int valid) {
   if (RAGGED && valid < 8) { store16_partial(ptr, v, valid); return; }
-  if (KAPY_EW_NT) __builtin_nontemporal_store(v, (u32x4 *)ptr);
+  if (kEwNt) __builtin_nontemporal_store(v, (u32x4 *)ptr);
   else *(u32x4 *)ptr = v;
 }
 
 template <typename T, int ACT, bool RAGGED>
 __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
-  constexpr int UNROLL = KAPY_EW_UNROLL;
+  constexpr int UNROLL = kEwUnroll;
   const uint32_t total = (uint32_t)p.rows * (uint32_t)p.vec_per_row;
   const uint32_t first = blockIdx.x * (256 * UNROLL) + threadIdx.x;
   const float scale = p.has_scale ? p.scale : 1.0f;
@@ -231,7 +227,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
       row[u] = (int32_t)(slot / (uint32_t)p.vec_per_row);
       col[u] = (int32_t)(slot - (uint32_t)row[u] * (uint32_t)p.vec_per_row) * 8;
       const int valid = RAGGED ? p.width - col[u] : 8;
-      xv[u] = load_row16<RAGGED>(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2, valid, KAPY_EW_NT);
+      xv[u] = load_row16<RAGGED>(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2, valid, kEwNt);
       if (p.bias_mode == kBiasRow) bv[u] = load_row16<RAGGED>(p.bias + (int64_t)col[u] * 2, valid, false);
       else if (p.bias_mode == kBiasFull) bv[u] = load_row16<RAGGED>(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2, valid, false);
       else if (p.bias_mode == kBiasCol) {
@@ -256,12 +252,9 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
 // Same chain when the bias is broadcast along rows (bias[0, j]) or absent: a lane keeps one
 // 8-column chunk and walks ROWS consecutive rows, so its bias vector is fetched and widened once
 // and no index division is needed.  Grid: x over column chunks, y over groups of ROWS rows.
-#ifndef KAPY_EW_ROWS
-#define KAPY_EW_ROWS 2
-#endif
 template <typename T, int ACT, bool RAGGED>
 __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p) {
-  constexpr int ROWS = KAPY_EW_ROWS;
+  constexpr int ROWS = 2;  // rows in flight per lane
   const int32_t chunk = blockIdx.x * 256 + threadIdx.x;
   if (chunk >= p.vec_per_row) return;
   const int32_t col = chunk * 8, row0 = blockIdx.y * ROWS;
@@ -272,7 +265,7 @@ __global__ __launch_bounds__(256) void affine_act_cols_kernel(AffineActParams p)
   u32x4 xv[ROWS];
 #pragma unroll
   for (int u = 0; u < ROWS; ++u)
-    if (row0 + u < p.rows) xv[u] = load_row16<RAGGED>(p.x + ((int64_t)(row0 + u) * p.x_stride0 + col) * 2, valid, KAPY_EW_NT);
+    if (row0 + u < p.rows) xv[u] = load_row16<RAGGED>(p.x + ((int64_t)(row0 + u) * p.x_stride0 + col) * 2, valid, kEwNt);
 #pragma unroll
   for (int u = 0; u < ROWS; ++u) {
     if (row0 + u >= p.rows) break;
@@ -739,9 +732,9 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   int T = -1;
   if (match_affine_act(prog, n_inst, ins, out, &ap, &T)) {
     uint32_t slots = (uint32_t)ap.rows * (uint32_t)ap.vec_per_row;
-    const bool cols = (ap.bias_mode == kBiasRow || ap.bias_mode == kNoBias) && (ap.rows + KAPY_EW_ROWS - 1) / KAPY_EW_ROWS <= 65535;
-    dim3 grid = cols ? dim3((ap.vec_per_row + 255) / 256, (ap.rows + KAPY_EW_ROWS - 1) / KAPY_EW_ROWS)
-                     : dim3((slots + 256 * KAPY_EW_UNROLL - 1) / (256 * KAPY_EW_UNROLL));
+    const bool cols = (ap.bias_mode == kBiasRow || ap.bias_mode == kNoBias) && (ap.rows + 2 - 1) / 2 <= 65535;
+    dim3 grid = cols ? dim3((ap.vec_per_row + 255) / 256, (ap.rows + 2 - 1) / 2)
+                     : dim3((slots + 256 * kEwUnroll - 1) / (256 * kEwUnroll));
 #define KAPY_LAUNCH_AFFINE(TT, AA)                                                     \
   do {                                                                                 \
     if (cols && ap.width) affine_act_cols_kernel<TT, AA, true><<<grid, 256, 0, s>>>(ap);  \

@@ -175,10 +175,7 @@ const char *kPrelude =
 #include "jit_headers.inc"
     ;
 
-#ifndef KAPY_JIT_TILE_ROWS
-#define KAPY_JIT_TILE_ROWS 64
-#endif
-constexpr int kTileRows = KAPY_JIT_TILE_ROWS;  // rows of a tile of the tiled skeleton (64 columns wide): 32 per vector a lane handles
+constexpr int kTileRows = 64;  // rows of a tile of the tiled skeleton (64 columns wide): 32 per vector a lane handles
 enum Kind { kFull = 0, kRow = 1, kCol = 2, kScalar = 3, kColMajor = 4 /* full extent, contiguous along axis 0 */ };
 
 struct Signature {

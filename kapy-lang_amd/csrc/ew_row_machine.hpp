@@ -344,12 +344,6 @@ int launch_row_kernel(const StackProgram &P, int ns, hipStream_t s) {
   } while (0)
   // The light kernel exists per chunk count, and for four chunks per stack depth, so that a program that needs one or
   // two row values is not charged the registers of three.  The others always carry four chunks and three values.
-#ifdef KAPY_ROW_TUNE  // tuning builds: one row length only, to keep the compile short
-  if constexpr (MODE == kModeLight) {
-    if (threads == 256 && ch > 2) { if (ns == 3) KAPY_ROW(4, 256, 3); else if (ns == 2) KAPY_ROW(4, 256, 2); else KAPY_ROW(4, 256, 1); }
-    else return fail(KAPY_ERR_UNSUPPORTED, "tuning build");
-  } else return fail(KAPY_ERR_UNSUPPORTED, "tuning build");
-#else
 #define KAPY_ROW_CH(TH_)                                                                                           \
   do {                                                                                                             \
     if (MODE != kModeLight || (ch > 2 && ns == 3)) KAPY_ROW(4, TH_, 3);                                            \
@@ -361,7 +355,6 @@ int launch_row_kernel(const StackProgram &P, int ns, hipStream_t s) {
   if (threads == 64) { if constexpr (MODE == kModeLight) KAPY_ROW_CH(64); }
   else if (threads == 256) KAPY_ROW_CH(256);
   else KAPY_ROW_CH(1024);
-#endif
 #undef KAPY_ROW_CH
 #undef KAPY_ROW
   KAPY_HIP_CHECK(hipGetLastError());

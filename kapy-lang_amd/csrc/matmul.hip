@@ -1387,14 +1387,14 @@ int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_r
 
 int64_t split_workspace_bytes(int64_t tiles, int split) { return kSplitCounterBytes + tiles * split * (128 * 128 * 4); }
 
-template <int BM, int BN, int BK, int WM, int WN, int S>
+template <template <int, int> class P, int BM, int BN, int BK, int WM, int WN, int S>
 int launch_f8(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
   // the kernel issues mfma(rhs fragment, lhs fragment): the first format selector is the rhs's
   switch (rhs_fmt * 2 + lhs_fmt) {
-  case 0: return launch_tn<F8<0, 0>, BM, BN, BK, WM, WN, S>(p, s);
-  case 1: return launch_tn<F8<0, 1>, BM, BN, BK, WM, WN, S>(p, s);
-  case 2: return launch_tn<F8<1, 0>, BM, BN, BK, WM, WN, S>(p, s);
-  default: return launch_tn<F8<1, 1>, BM, BN, BK, WM, WN, S>(p, s);
+  case 0: return launch_tn<P<0, 0>, BM, BN, BK, WM, WN, S>(p, s);
+  case 1: return launch_tn<P<0, 1>, BM, BN, BK, WM, WN, S>(p, s);
+  case 2: return launch_tn<P<1, 0>, BM, BN, BK, WM, WN, S>(p, s);
+  default: return launch_tn<P<1, 1>, BM, BN, BK, WM, WN, S>(p, s);
   }
 }
 
@@ -1483,12 +1483,12 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s
   // the ring variants take any M, N >= 128 and any K >= 128 of whole 16-byte chunks (their loads are bounded by the
   // operands' ends); 256x256 tiles when there are at least as many of them as CUs, 128x128 (two workgroups per CU) below
   if (p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
-    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
-    return launch_f8<128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<F8, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    return launch_f8<F8, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
-    return launch_f8<256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
-  if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
+    return launch_f8<F8, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+  if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<F8, 128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
   return KAPY_ERR_UNSUPPORTED;
 }
 

@@ -388,8 +388,8 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
 
 /* Runs a kapy.func given in the textual form of the reference's Kapy-dialect fixtures
  * (test/Conversion/KapyToKgpu/elementwise_add.mlir, reduce_sum.mlir, matmul.mlir; op syntax from
- * include/kapy/Dialect/Kapy/IR/Ops.td) on the device: every program id of `grid` and every warp id of the
- * module's kapy.num_warps is executed in turn, each tensor op as one call of the entry points above on
+ * include/kapy/Dialect/Kapy/IR/Ops.td) on the device: every program id of `grid` is executed in turn, for every warp id of the
+ * module's kapy.num_warps, each tensor op as one call of the entry points above on
  * `stream` (mk_global/sv_global/sv_shared: MkGlobalOpToLLVM.cpp:23-47, SvGlobalOpToLLVM.cpp:22-40,
  * SvSharedOpToLLVM.cpp:20-42; ld_global/st_global/cp_async_global_to_shared/ld_matrix: kapy_copy; arith on
  * tensors, math.exp / exp2 / log / log2 / sqrt / rsqrt / tanh / erf / absf / fma, kapy.fptofp, arith.extf / truncf,
@@ -403,8 +403,11 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * broadcast back to its operand's shape is an instruction of that program: the counterpart of
  * the reference compiling the ops of a function into one kernel body.  KAPY_MLIR_FUSE=0 in the environment runs
  * every op as a call of its own instead; results are the same bit for bit.
- * Warps run one after the other, so a program whose warps exchange data through shared memory between
- * barriers is outside what this executes correctly; the three fixtures are not of that kind.
+ * The warps of a program instance advance in step: an op is executed for every warp id before the next op is, and an
+ * scf.for whose bounds all warps agree on is iterated jointly, so there is in effect a barrier between any two ops
+ * and warps may exchange data through shared memory wherever the program itself is race-free (the barriers
+ * kapy_analyze_mlir places are a subset of these).  A loop whose bounds differ between warps runs warp after warp;
+ * KAPY_MLIR_IN_STEP=0 in the environment runs every warp to the end before the next one starts.
  * `args` follow the function's signature: a device pointer (with the size of its allocation in bytes, 0 =
  * unknown, which mk_global is checked against) for !kapy.ptr<1>, an i32 otherwise.  A sub-view that leaves
  * its parent is an error.  func_name NULL = the first function of the module.  The call allocates a 64 MiB

@@ -538,8 +538,28 @@ struct Interp {
   const Func &f;
   hipStream_t stream;
   char *arena = nullptr;
-  size_t top = kSharedArena;
+  size_t top = kSharedArena, limit = kArena;
   std::map<std::string, Value> env;
+  // The warps of one program instance, run in step: every op is executed for warp 0, 1, ... before the next op is looked at,
+  // which is the reference's workgroup of concurrent warps (FuncOpToLLVM.cpp:72-88) with a barrier between any two ops - so a
+  // program whose warps exchange data through shared memory between the barriers BlockAnalysis would insert
+  // (BlockAnalysis.cpp:114-169) sees what it would see on the reference's target.  Each warp has its own values and its own
+  // share of the register arena; the state of the warp being executed is swapped into env / top / limit / warp.
+  struct WarpState {
+    std::map<std::string, Value> env;
+    size_t top = 0, limit = 0;
+  };
+  std::vector<WarpState> warps;
+  void enter(int w) {
+    std::swap(env, warps[w].env);
+    top = warps[w].top;
+    limit = warps[w].limit;
+    warp = w;
+  }
+  void leave(int w) {
+    std::swap(env, warps[w].env);
+    warps[w].top = top;
+  }
   const Analysis *plan = nullptr;  // where each mk_shared lives inside the shared part of the arena
   int64_t pid[3] = {0, 0, 0}, warp = 0;
   std::string err;
@@ -551,7 +571,7 @@ struct Interp {
   }
   void *alloc(size_t bytes) {
     top = (top + 255) & ~size_t(255);
-    if (top + bytes > kArena) return nullptr;
+    if (top + bytes > limit) return nullptr;
     void *r = arena + top;
     top += bytes;
     return r;
@@ -592,13 +612,20 @@ struct Interp {
     return false;
   }
   // before a store into `dst`: every deferred value that still has to read that memory is computed now
+  // (the values of every warp: another warp's deferred load stands earlier in program order than this store, too)
   int settle_readers(const Op &op, const kapy_global &dst) {
-    for (auto &kv : env)
-      if (kv.second.kind == Value::kTensor && kv.second.lazy && reads_under(kv.second.lazy, dst)) {
-        int rc = force(op, kv.second);
-        if (rc != KAPY_OK) return rc;
-      }
-    return KAPY_OK;
+    auto settle = [&](std::map<std::string, Value> &values) {
+      for (auto &kv : values)
+        if (kv.second.kind == Value::kTensor && kv.second.lazy && reads_under(kv.second.lazy, dst)) {
+          int rc = force(op, kv.second);
+          if (rc != KAPY_OK) return rc;
+        }
+      return (int)KAPY_OK;
+    };
+    int rc = settle(env);
+    for (size_t w = 0; rc == KAPY_OK && w < warps.size(); ++w)
+      if ((int64_t)w != warp) rc = settle(warps[w].env);
+    return rc;
   }
   // the operand as an expression: deferred tensors as they are, computed ones as leaves
   std::shared_ptr<Expr> as_expr(const Value &v) {
@@ -811,6 +838,78 @@ struct Interp {
       int rc = run_op(op, yielded);
       if (rc != KAPY_OK) return rc;
     }
+    return KAPY_OK;
+  }
+
+  // All warps in step through `ops` (see WarpState).  yielded: one list per warp, filled by the body's scf.yield.
+  int run_ops_in_step(const std::vector<Op> &ops, std::vector<std::vector<Value>> *yielded) {
+    const int W = (int)warps.size();
+    for (const Op &op : ops) {
+      if (op.name == "scf.for") {
+        int rc = run_for_in_step(op);
+        if (rc != KAPY_OK) return rc;
+        continue;
+      }
+      for (int w = 0; w < W; ++w) {
+        enter(w);
+        int rc = run_op(op, yielded ? &(*yielded)[w] : nullptr);
+        leave(w);
+        if (rc != KAPY_OK) return rc;
+      }
+    }
+    return KAPY_OK;
+  }
+  // scf.for with every warp taking the same trips: the iterations themselves run in step.  Warps that disagree on the bounds
+  // cannot meet at a barrier inside the loop, so such a loop is run warp after warp.
+  int run_for_in_step(const Op &op) {
+    const int W = (int)warps.size();
+    if (op.region_args.empty()) return fail_op(op, "scf.for without an induction variable");
+    const size_t n_iter = op.region_args.size() - 1;
+    std::vector<int64_t> lo(W), hi(W), st(W);
+    std::vector<std::vector<Value>> carried(W, std::vector<Value>(n_iter));
+    bool same = true;
+    for (int w = 0; w < W; ++w) {
+      enter(w);
+      Value l, h, s;
+      bool ok = get(op, 0, Value::kInt, l) && get(op, 1, Value::kInt, h) && get(op, 2, Value::kInt, s);
+      for (size_t k = 0; ok && k < n_iter; ++k) {
+        auto it = 3 + k < op.operands.size() ? env.find(op.operands[3 + k]) : env.end();
+        if (it == env.end()) { fail_op(op, "use of undefined loop operand"); ok = false; break; }
+        carried[w][k] = it->second;
+      }
+      leave(w);
+      if (!ok) return KAPY_ERR_INVALID;
+      if (s.i <= 0) return fail_op(op, "step must be positive");
+      lo[w] = l.i; hi[w] = h.i; st[w] = s.i;
+      same = same && lo[w] == lo[0] && hi[w] == hi[0] && st[w] == st[0];
+    }
+    if (!same) {
+      for (int w = 0; w < W; ++w) {
+        enter(w);
+        int rc = run_op(op, nullptr);
+        leave(w);
+        if (rc != KAPY_OK) return rc;
+      }
+      return KAPY_OK;
+    }
+    for (int64_t iv = lo[0]; iv < hi[0]; iv += st[0]) {
+      for (int w = 0; w < W; ++w) {
+        Value ivv;
+        ivv.kind = Value::kInt;
+        ivv.i = iv;
+        warps[w].env[op.region_args[0]] = ivv;
+        for (size_t k = 0; k < n_iter; ++k) warps[w].env[op.region_args[1 + k]] = carried[w][k];
+      }
+      std::vector<std::vector<Value>> y(W);
+      int rc = run_ops_in_step(op.body, &y);
+      if (rc != KAPY_OK) return rc;
+      for (int w = 0; w < W; ++w) {
+        if (y[w].size() != n_iter) return fail_op(op, "scf.yield does not match iter_args");
+        carried[w] = y[w];
+      }
+    }
+    for (int w = 0; w < W; ++w)
+      for (size_t k = 0; k < n_iter && k < op.results.size(); ++k) warps[w].env[op.results[k]] = carried[w][k];
     return KAPY_OK;
   }
 
@@ -1185,25 +1284,49 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   if (const char *e = getenv("KAPY_MLIR_FUSE")) in.fuse = atoi(e) != 0;
   KAPY_HIP_CHECK(hipMalloc((void **)&in.arena, kArena));
   rc = KAPY_OK;
+  // KAPY_MLIR_IN_STEP=0: the warps of an instance run one after the other to the end instead of in step (the former way;
+  // only right for programs whose warps do not exchange data through shared memory)
+  bool in_step = true;
+  if (const char *e = getenv("KAPY_MLIR_IN_STEP")) in_step = atoi(e) != 0;
+  const int W = f.num_warps > 0 ? f.num_warps : 1;
+  auto bind_args = [&](std::map<std::string, Value> &values) {
+    for (int k = 0; k < n_args; ++k) {
+      Value v;
+      if (f.arg_types[k].kind == Type::kPtr) {
+        if (!args[k].ptr) { in.err = "pointer argument " + std::to_string(k) + " is null"; return (int)KAPY_ERR_INVALID; }
+        v.kind = Value::kPtr; v.ptr = args[k].ptr; v.bytes = args[k].bytes;
+      }
+      else { v.kind = Value::kInt; v.i = args[k].i32; }
+      values[f.arg_names[k]] = v;
+    }
+    return (int)KAPY_OK;
+  };
   for (int32_t p2 = 0; p2 < grid[2] && rc == KAPY_OK; ++p2)
     for (int32_t p1 = 0; p1 < grid[1] && rc == KAPY_OK; ++p1)
-      for (int32_t p0 = 0; p0 < grid[0] && rc == KAPY_OK; ++p0)
-        for (int w = 0; w < f.num_warps && rc == KAPY_OK; ++w) {
-          in.pid[0] = p0; in.pid[1] = p1; in.pid[2] = p2;
+      for (int32_t p0 = 0; p0 < grid[0] && rc == KAPY_OK; ++p0) {
+        in.pid[0] = p0; in.pid[1] = p1; in.pid[2] = p2;
+        if (in_step) {
+          // register tensors of the previous instance are dead; shared tensors stay.  Every warp gets an equal share of the arena.
+          const size_t share = ((kArena - kSharedArena) / W) & ~size_t(255);
+          in.warps.assign(W, Interp::WarpState());
+          for (int w = 0; w < W && rc == KAPY_OK; ++w) {
+            in.warps[w].top = kSharedArena + w * share;
+            in.warps[w].limit = kSharedArena + (w + 1) * share;
+            rc = bind_args(in.warps[w].env);
+          }
+          in.env.clear();
+          if (rc == KAPY_OK) rc = in.run_ops_in_step(f.body, nullptr);
+          continue;
+        }
+        for (int w = 0; w < W && rc == KAPY_OK; ++w) {
           in.warp = w;
           in.env.clear();
-          in.top = kSharedArena;  // register tensors of the previous instance are dead; shared tensors stay
-          for (int k = 0; k < n_args; ++k) {
-            Value v;
-            if (f.arg_types[k].kind == Type::kPtr) {
-              if (!args[k].ptr) { rc = KAPY_ERR_INVALID; in.err = "pointer argument " + std::to_string(k) + " is null"; break; }
-              v.kind = Value::kPtr; v.ptr = args[k].ptr; v.bytes = args[k].bytes;
-            }
-            else { v.kind = Value::kInt; v.i = args[k].i32; }
-            in.env[f.arg_names[k]] = v;
-          }
+          in.top = kSharedArena;
+          in.limit = kArena;
+          rc = bind_args(in.env);
           if (rc == KAPY_OK) rc = in.run_ops(f.body, nullptr);
         }
+      }
   // the arena is freed after the work on the stream has finished
   hipError_t e = hipStreamSynchronize((hipStream_t)stream);
   (void)hipFree(in.arena);

@@ -364,3 +364,88 @@ def scaled_transpose_program(tile=32, scale=0.5, dtype="f16"):
 """.format(tile=tile, scale=scale, dtype=dtype, dyn=dyn, t=t)
     return (HEADER + "module attributes {kapy.num_warps = 1 : i64} {\n"
             "  kapy.func public @scaled_transpose_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %m: i32, %n: i32) {\n" + body + "  }\n}\n")
+
+
+def exchange_program(rows_per_warp=16, cols=64, num_warps=4, dtype="f16", barrier=True):
+    """A program whose warps exchange data through shared memory: warp w stores its rows of x, scaled by 2, into its slot
+    of one shared buffer; after the barrier it reads the slot of warp (w + 1) % num_warps and stores that to its rows of out.
+    So out[block w] = 2 * x[block (w + 1) % num_warps] within every program's group of num_warps row blocks - which only
+    comes out right if every warp has stored before any warp loads."""
+    t = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype)
+    full = "tensor<%dx%dx%s, #shared>" % (rows_per_warp * num_warps, cols, dtype)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols, num_warps])
+    body += """    %two = arith.constant dense<2.000000e+00> : {t}, #values>
+    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %w1 = arith.addi %w0, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %next = arith.addi %warp, %c1_i32 : i32
+    %peer = arith.remui %next, %c{nw}_i32 : i32
+    %q0 = arith.muli %peer, %c{rpw}_i32 : i32
+    %q1 = arith.addi %q0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %buf = kapy.mk_shared {{kapy.row_major = true}} : {full}
+    %mine = kapy.sv_shared %buf[%w0 : %w1, %c0_i32 : %c{cols}_i32] : {full} -> {t}, #shared>
+    %theirs = kapy.sv_shared %buf[%q0 : %q1, %c0_i32 : %c{cols}_i32] : {full} -> {t}, #shared>
+    %vx = kapy.ld_global %sx : {t}, #global> -> {t}, #values>
+    %v2 = arith.mulf %vx, %two : {t}, #values>
+    kapy.st_shared %v2, %mine : {t}, #values>, {t}, #shared>
+{barrier}    %vy = kapy.ld_shared %theirs : {t}, #shared> -> {t}, #values>
+    kapy.st_global %vy, %so : {t}, #values>, {t}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, t=t, full=full, nw=num_warps,
+           barrier="    nvvm.barrier0\n" if barrier else "")
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @exchange_kernel(%x: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %out: !kapy.ptr<1> {kapy.alignment = 128 : i64}, "
+            "%rows: i32 {kapy.alignment = 4 : i64}) {\n" + body + "  }\n}\n")
+
+
+def exchange_loop_program(rows_per_warp=8, cols=64, num_warps=4, steps=3, dtype="f16"):
+    """The same exchange inside an scf.for that carries the tile: every step each warp adds 1 to its tile, parks it in its slot,
+    and continues with the tile of warp (w + 1) % num_warps; after `steps` steps block w of out is x[block (w + steps) % num_warps]
+    + steps.  Every step reuses the one shared buffer, so it needs a barrier before the stores as well as before the loads."""
+    t = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype)
+    full = "tensor<%dx%dx%s, #shared>" % (rows_per_warp * num_warps, cols, dtype)
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols, num_warps, steps])
+    body += """    %one = arith.constant dense<1.000000e+00> : {t}, #values>
+    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %w1 = arith.addi %w0, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %next = arith.addi %warp, %c1_i32 : i32
+    %peer = arith.remui %next, %c{nw}_i32 : i32
+    %q0 = arith.muli %peer, %c{rpw}_i32 : i32
+    %q1 = arith.addi %q0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t}, #global>
+    %buf = kapy.mk_shared {{kapy.row_major = true}} : {full}
+    %mine = kapy.sv_shared %buf[%w0 : %w1, %c0_i32 : %c{cols}_i32] : {full} -> {t}, #shared>
+    %theirs = kapy.sv_shared %buf[%q0 : %q1, %c0_i32 : %c{cols}_i32] : {full} -> {t}, #shared>
+    %v0 = kapy.ld_global %sx : {t}, #global> -> {t}, #values>
+    %last = scf.for %i = %c0_i32 to %c{steps}_i32 step %c1_i32 iter_args(%v = %v0) -> ({t}, #values>) : i32 {{
+      %v1 = arith.addf %v, %one : {t}, #values>
+      nvvm.barrier0
+      kapy.st_shared %v1, %mine : {t}, #values>, {t}, #shared>
+      nvvm.barrier0
+      %vn = kapy.ld_shared %theirs : {t}, #shared> -> {t}, #values>
+      scf.yield %vn : {t}, #values>
+    }}
+    kapy.st_global %last, %so : {t}, #values>, {t}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, t=t, full=full, nw=num_warps, steps=steps)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @exchange_loop_kernel(%x: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %out: !kapy.ptr<1> {kapy.alignment = 128 : i64}, "
+            "%rows: i32 {kapy.alignment = 4 : i64}) {\n" + body + "  }\n}\n")

@@ -122,3 +122,15 @@ def test_a_program_beyond_the_lds_is_refused_before_anything_runs():
     args = (kh.MlirArg * 6)()
     assert kh.lib().kapy_run_mlir(text.encode(), None, args, 6, (C.c_int32 * 3)(1, 1, 1), None) == -3
     assert "shared memory" in kh.last_error() and "163840" in kh.last_error()
+
+
+def test_analysis_finds_the_barrier_between_warps_that_exchange_tiles():
+    # a store into one sub-view of a buffer and a load from another sub-view of it: the views' offsets depend on the warp id,
+    # so the two accesses may touch the same bytes and the load needs a barrier; the program's own nvvm.barrier0 is honoured
+    text = kp.exchange_program(barrier=False)
+    total, offsets, barriers = kh.analyze_mlir(text)
+    assert (total, offsets) == (4 * 16 * 64 * 2, [0])
+    assert barriers == [_lines(text, "kapy.ld_shared")[0]]
+    assert kh.analyze_mlir(kp.exchange_program(barrier=True))[2] == []
+    # in the loop the program places both barriers itself (before the stores: the previous step's loads; before the loads)
+    assert kh.analyze_mlir(kp.exchange_loop_program())[2] == []

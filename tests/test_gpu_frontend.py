@@ -246,3 +246,29 @@ def test_errors_name_the_line_and_leave_the_device_usable(ko):
     kh.run_mlir(text, [x, x, out, rows], [1])
     sync()
     assert np.array_equal(to_host(out, np.float16), to_host(x, np.float16) * 2)
+
+
+@pytest.mark.parametrize("rows_per_warp,cols,warps,programs", [(16, 64, 4, 3), (8, 128, 2, 5), (4, 64, 8, 1)])
+def test_warps_exchange_through_shared_memory(ko, rows_per_warp, cols, warps, programs):
+    """Warp w reads what warp (w + 1) % warps stored before the barrier: right only if the warps run in step."""
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 61).view(np.float16).reshape(programs, warps, rows_per_warp, cols)
+    want = np.roll(x, -1, axis=1) * np.float16(2)
+    dx, dout = to_dev(x.view(np.uint16).ravel()), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.exchange_program(rows_per_warp, cols, warps), [dx, dout, rows], [programs])
+    sync()
+    assert np.array_equal(to_host(dout, np.uint16), want.view(np.uint16).ravel())
+
+
+@pytest.mark.parametrize("rows_per_warp,cols,warps,steps,programs", [(8, 64, 4, 3, 2), (16, 64, 2, 5, 3)])
+def test_warps_exchange_inside_a_loop(ko, rows_per_warp, cols, warps, steps, programs):
+    """The exchange repeated in an scf.for that carries the tile: the loop itself has to advance all warps together."""
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 62).view(np.float16).reshape(programs, warps, rows_per_warp, cols)
+    want = x
+    for _ in range(steps):
+        want = np.roll(want + np.float16(1), -1, axis=1)
+    dx, dout = to_dev(x.view(np.uint16).ravel()), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.exchange_loop_program(rows_per_warp, cols, warps, steps), [dx, dout, rows], [programs])
+    sync()
+    assert np.array_equal(to_host(dout, np.uint16), want.view(np.uint16).ravel())

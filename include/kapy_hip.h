@@ -228,7 +228,11 @@ int kapy_copy_batched(const kapy_global *src, const kapy_global *dst, const kapy
  * layer norm ...): it runs in one pass over HBM with each row resident on chip, and needs axis 1, rows that are
  * contiguous, a multiple of 8 and at most 32768 elements long, zero padding, and operands that are full, row,
  * column or scalar views (KAPY_ERR_UNSUPPORTED otherwise; a width that is not a multiple of 8, with rows that still
- * start aligned to 8 elements, is served by compiling a kernel on the first call, see kapy_elementwise_specialize). */
+ * start aligned to 8 elements, is served by compiling a kernel on the first call, see kapy_elementwise_specialize).
+ * A program whose reduces run along axis 0 (ReduceOpToLLVM.cpp:51-172 reduces either axis; at most 4 of them) takes
+ * any views, shapes and padding: a workgroup owns 64 columns and re-reads its operands once per reduce, keeping only the
+ * per-column results on chip, so it moves (reduces + 1) times the operand bytes and is not a one-pass kernel.  The reduces
+ * of one program must all run along the same axis. */
 typedef enum kapy_ew_op {
   KAPY_EW_LD_GLOBAL = 0, /* dst <- ins[a]            (c = kapy_padding_option)                  */
   KAPY_EW_SPLAT,         /* dst <- imm as `dtype`    (kapy.splat)                               */

@@ -101,6 +101,91 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
   }
 }
 
+// Column machine: a program whose reduces run along axis 0 (ReduceOpToLLVM.cpp:51-172 reduces either axis).  A workgroup
+// owns a strip of 64 columns, one per lane, and its waves share out the rows, so a wave's accesses to a row-major operand
+// are 64 consecutive elements.  The program runs in phases, one per reduce and a last one that stores: phase p walks all
+// rows executing only the instructions reduce p depends on (earlier reduces are per-column values by then), folds the
+// operand in fp32 per wave, and the waves' partials are folded in wave order and rounded once to the register's type, as
+// kapy_reduce does.  Operands are re-read in every phase (they come from L2 when the strip fits there); nothing but the
+// per-column results is kept on chip, so any number of rows is served.
+constexpr int kMaxColumnReduces = 4;
+struct ColumnPlan {
+  int32_t n_phases;                      // reduces + 1
+  int32_t stop[kMaxColumnReduces + 1];   // the phase's reduce instruction; n_inst for the storing phase
+  uint64_t need[kMaxColumnReduces + 1];  // bit k: the phase executes instruction k
+};
+
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void column_program_kernel(Program P, ColumnPlan C) {
+  __shared__ float regs[kMaxRegs][WAVES * 64];
+  __shared__ float part[WAVES][64];
+  __shared__ float red[kMaxColumnReduces][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int32_t j = (int32_t)blockIdx.x * 64 + lane;
+  const bool in_strip = j < P.out.ext1;
+  for (int phase = 0; phase < C.n_phases; ++phase) {
+    const bool last = phase == C.n_phases - 1;
+    const int stop = C.stop[phase];
+    const uint64_t need = C.need[phase];
+    const bool sum = !last && P.inst[stop].op == KAPY_EW_REDUCE_SUM;
+    float acc = sum ? -0.f : -__builtin_inff();  // -0: the identity of addition, a column of only -0 sums to -0
+    for (int32_t i = wave; i < P.out.ext0; i += WAVES) {
+      for (int k = 0; k < stop; ++k) {
+        if (!((need >> k) & 1)) continue;
+        const kapy_ew_inst I = P.inst[k];
+        float r = 0.f;
+        const int dt = I.dtype;
+        switch (I.op) {
+        case KAPY_EW_LD_GLOBAL: {
+          const DevView &g = P.in[I.a];
+          const int32_t gi = g.ext0 == 1 ? 0 : i, gj = g.ext1 == 1 ? 0 : j;
+          if (in_strip && gi < g.ext0 && gj < g.ext1) r = load_as_f32(g.base, g.dtype, gi * g.stride0 + gj * g.stride1);
+          else {
+            uint32_t w = I.c == KAPY_PAD_ZERO ? 0u : g.pad;
+            r = load_as_f32(&w, g.dtype, 0);
+          }
+          break;
+        }
+        case KAPY_EW_SPLAT: r = round_to_dtype(I.imm, dt, true); break;
+        case KAPY_EW_FPTOFP: r = round_to_dtype(regs[I.a][tid], dt, I.rmode != KAPY_RZ); break;
+        case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX: r = red[I.c][lane]; break;  // I.c: which reduce this is (set by the host)
+        case KAPY_EW_ST_GLOBAL:
+          if (in_strip) store_from_f32((void *)P.out.base, P.out.dtype, i * P.out.stride0 + j * P.out.stride1, regs[I.a][tid]);
+          continue;
+        default: {
+          const float a = regs[I.a][tid];
+          switch (I.op) {
+          case KAPY_EW_ADDF: r = __fadd_rn(a, regs[I.b][tid]); break;
+          case KAPY_EW_SUBF: r = __fsub_rn(a, regs[I.b][tid]); break;
+          case KAPY_EW_MULF: r = __fmul_rn(a, regs[I.b][tid]); break;
+          case KAPY_EW_DIVF: r = __fdiv_rn(a, regs[I.b][tid]); break;
+          case KAPY_EW_FMA: r = fma_typed(a, regs[I.b][tid], regs[I.c][tid], dt); break;
+          case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
+          case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
+          default: r = apply_unary(I.op, a);
+          }
+          if (dt != KAPY_F32) r = round_to_dtype(r, dt, true);
+        }
+        }
+        regs[I.dst][tid] = r;  // regs[*][tid] is private to the lane
+      }
+      if (!last) {
+        const float x = regs[P.inst[stop].a][tid];
+        acc = sum ? acc + x : max_nan(acc, x);
+      }
+    }
+    if (last) break;
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+      float total = part[0][lane];
+      for (int w = 1; w < WAVES; ++w) total = sum ? total + part[w][lane] : max_nan(total, part[w][lane]);
+      red[phase][lane] = round_to_dtype(total, P.inst[stop].dtype, true);
+    }
+    __syncthreads();
+  }
+}
+
 // Throughput of this kernel follows the number of resident waves (each lane walks its program one
 // dependent step at a time), so the 16-bit-only form is held to 64 registers: 8 waves per SIMD.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void stack_kernel_narrow(StackProgram P) { stack_run<true>(P); }
@@ -690,6 +775,60 @@ DevView to_dev(const kapy_global *g) {
   return v;
 }
 
+
+// A program whose reduces all run along axis 0, on the column machine.
+int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                       hipStream_t s) {
+  Program P;
+  memset(&P, 0, sizeof P);
+  ColumnPlan C;
+  memset(&C, 0, sizeof C);
+  P.n_inst = n_inst;
+  P.n_ins = n_ins;
+  // def_of[r]: the instructions the current value of register r is computed from
+  uint64_t def_of[kMaxRegs];
+  memset(def_of, 0, sizeof def_of);
+  int n_reduce = 0;
+  uint64_t stores = 0;
+  for (int k = 0; k < n_inst; ++k) {
+    kapy_ew_inst I = prog[k];
+    I.dtype = result_dtype[k];
+    uint64_t d = uint64_t(1) << k;
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: case KAPY_EW_SPLAT: break;
+    case KAPY_EW_FMA: d |= def_of[I.a] | def_of[I.b] | def_of[I.c]; break;
+    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+      d |= def_of[I.a] | def_of[I.b];
+      break;
+    case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX:
+      if (n_reduce == kMaxColumnReduces)
+        return fail(KAPY_ERR_UNSUPPORTED, "elementwise: a program may hold at most %d reduces along axis 0", kMaxColumnReduces);
+      C.stop[n_reduce] = k;
+      C.need[n_reduce] = def_of[I.a];  // what the operand is computed from; the reduce itself is the fold after the row loop
+      I.c = n_reduce++;
+      break;                           // later phases read the per-column result: nothing before it is needed for its sake
+    default: d |= def_of[I.a];
+    }
+    if (I.op == KAPY_EW_ST_GLOBAL) stores |= d;
+    else def_of[I.dst] = d;
+    P.inst[k] = I;
+  }
+  C.stop[n_reduce] = n_inst;
+  C.need[n_reduce] = stores;
+  C.n_phases = n_reduce + 1;
+  for (int k = 0; k < n_ins; ++k) P.in[k] = to_dev(ins[k]);
+  for (int k = 0; k < n_inst; ++k)
+    if (prog[k].op == KAPY_EW_LD_GLOBAL) P.in[prog[k].a].pad = padding_word_of(ins[prog[k].a]->dtype, prog[k].c);
+  P.out = to_dev(out);
+  const int64_t strips = (extent1(out) + 63) / 64;
+  if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: too many columns for a program with reduces along axis 0");
+  // many rows: more waves per strip
+  if (extent0(out) >= 256) column_program_kernel<8><<<dim3((unsigned)strips), 512, 0, s>>>(P, C);
+  else column_program_kernel<4><<<dim3((unsigned)strips), 256, 0, s>>>(P, C);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 }  // namespace
 }  // namespace kapy
 
@@ -717,6 +856,12 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   bool has_reduce = false;
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
   if (has_reduce) {
+    int along[2] = {0, 0};
+    for (int k = 0; k < n_inst; ++k)
+      if (prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX) ++along[prog[k].b];
+    if (along[0] && along[1])
+      return fail(KAPY_ERR_UNSUPPORTED, "elementwise: the reduces of one program must run along the same axis (reduce the other axis with kapy_reduce first)");
+    if (along[0]) return run_column_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
     rc = run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
     // What the row machine refuses (a width that is not a multiple of 8, more than three row values in flight) a compiled

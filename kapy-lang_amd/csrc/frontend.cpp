@@ -515,9 +515,9 @@ struct Expr {
   int n_in = 0;
   kapy_global leaf;
   bool global_leaf = false;  // the leaf is a view of the caller's memory (a deferred kapy.ld_global), which a later store may change
-  // KAPY_EW_REDUCE_SUM / _MAX along axis 1: inside a program the result sits on every element of the row, so the node
+  // KAPY_EW_REDUCE_SUM / _MAX along `axis`: inside a program the result sits on every element of the reduced line, so the node
   // can only be part of a program whose result has the operand's shape (rows x cols) and element type (operand_dtype)
-  int32_t rows = 0, cols = 0, operand_dtype = 0;
+  int32_t rows = 0, cols = 0, operand_dtype = 0, axis = 1;
 };
 
 struct Value {
@@ -661,7 +661,7 @@ struct Interp {
       }
       m.prog[m.n++] = {KAPY_EW_LD_GLOBAL, dst, slot, 0, 0, 0, KAPY_RN, 0.f};
     } else if (e->ew == KAPY_EW_REDUCE_SUM || e->ew == KAPY_EW_REDUCE_MAX) {
-      m.prog[m.n++] = {e->ew, dst, src[0], 1, 0, 0, KAPY_RN, 0.f};
+      m.prog[m.n++] = {e->ew, dst, src[0], e->axis, 0, 0, KAPY_RN, 0.f};
     } else {
       m.prog[m.n++] = {e->ew, dst, src[0], src[1], src[2], e->dtype, e->rmode, e->imm};
     }
@@ -676,7 +676,8 @@ struct Interp {
       if (Expr *r = find_reduce(e->in[k], skip)) return r;
     return nullptr;
   }
-  // runs a deferred reduce by itself (its operand computed first, then kapy_reduce): the node becomes a computed [rows x 1] tensor
+  // runs a deferred reduce by itself (its operand computed first, then kapy_reduce): the node becomes a computed [rows x 1]
+  // (axis 1) or [1 x cols] (axis 0) tensor
   int compute_reduce(const Op &op, Expr *r) {
     Value operand;
     operand.kind = Value::kTensor;
@@ -686,11 +687,12 @@ struct Interp {
     if (rc == KAPY_OK && !(operand.lazy->ew == KAPY_EW_LD_GLOBAL && operand.lazy->n_in == 0)) rc = force(op, operand);
     if (rc != KAPY_OK) return rc;
     if (operand.lazy) operand.g = operand.lazy->leaf;
-    void *ptr = alloc((size_t)r->rows * dtype_bytes(r->operand_dtype));
+    const int32_t kept0 = r->axis == 1 ? r->rows : 1, kept1 = r->axis == 1 ? 1 : r->cols;
+    void *ptr = alloc((size_t)kept0 * kept1 * dtype_bytes(r->operand_dtype));
     if (!ptr) return fail_op(op, "register tensors of one program instance exceed the arena");
     kapy_global g;
-    rc = lib(op, kapy_mk_global(&g, ptr, 0, r->rows, 1, 1, 1, r->operand_dtype, 256));
-    if (rc == KAPY_OK) rc = lib(op, kapy_reduce(&operand.g, &g, 1, r->ew == KAPY_EW_REDUCE_MAX ? 1 : 0, stream));
+    rc = lib(op, kapy_mk_global(&g, ptr, 0, kept0, kept1, kept1, 1, r->operand_dtype, 256));
+    if (rc == KAPY_OK) rc = lib(op, kapy_reduce(&operand.g, &g, r->axis, r->ew == KAPY_EW_REDUCE_MAX ? 1 : 0, stream));
     if (rc != KAPY_OK) return rc;
     r->ew = KAPY_EW_LD_GLOBAL;
     r->n_in = 0;
@@ -1125,16 +1127,18 @@ struct Interp {
       }
       if (kind < 0) return fail_op(op, "only addf and maximumf combiners are supported");
       int axis = op.attrs.count("axis") ? atoi(op.attrs.at("axis").c_str()) : 0;
-      // along axis 1 over a register tensor the reduce joins the deferred chain: followed by a broadcast back to the
-      // operand's shape it becomes an instruction of the program that consumes it
+      // over a register tensor the reduce joins the deferred chain: followed by a broadcast back to the operand's shape it
+      // becomes an instruction of the program that consumes it (along rows: the row programs; along columns: the column machine)
       auto src = op.operands.empty() ? env.end() : env.find(op.operands[0]);
-      if (fuse && axis == 1 && !op.types.empty() && op.types.back().kind == Type::kTensor && src != env.end() &&
+      if (fuse && (axis == 0 || axis == 1) && !op.types.empty() && op.types.back().kind == Type::kTensor && src != env.end() &&
           src->second.kind == Value::kTensor && (src->second.lazy || is_register_tensor(src->second.g))) {
         const kapy_global &sg = src->second.g;
         const Type &ty = op.types.back();
-        if (ty.shape[0] == sg.end0 - sg.start0 && ty.shape[1] == 1 && ty.dtype == sg.dtype) {
+        const bool kept_shape = axis == 1 ? ty.shape[0] == sg.end0 - sg.start0 && ty.shape[1] == 1 : ty.shape[0] == 1 && ty.shape[1] == sg.end1 - sg.start1;
+        if (kept_shape && ty.dtype == sg.dtype) {
           auto e = std::make_shared<Expr>();
           e->ew = kind == 1 ? KAPY_EW_REDUCE_MAX : KAPY_EW_REDUCE_SUM;
+          e->axis = axis;
           e->n_in = 1;
           e->in[0] = as_expr(src->second);
           e->rows = sg.end0 - sg.start0; e->cols = sg.end1 - sg.start1; e->operand_dtype = sg.dtype;
@@ -1142,7 +1146,7 @@ struct Interp {
             r.kind = Value::kTensor;
             r.lazy = e;
             memset(&r.g, 0, sizeof r.g);
-            int rc = lib(op, kapy_mk_global(&r.g, arena, 0, e->rows, 1, 1, 1, ty.dtype, 16));
+            int rc = lib(op, kapy_mk_global(&r.g, arena, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 16));
             if (rc) return rc;
             env[op.results[0]] = r;
             return KAPY_OK;

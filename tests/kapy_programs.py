@@ -449,3 +449,43 @@ def exchange_loop_program(rows_per_warp=8, cols=64, num_warps=4, steps=3, dtype=
     return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
             "  kapy.func public @exchange_loop_kernel(%x: !kapy.ptr<1> {kapy.alignment = 128 : i64}, %out: !kapy.ptr<1> {kapy.alignment = 128 : i64}, "
             "%rows: i32 {kapy.alignment = 4 : i64}) {\n" + body + "  }\n}\n")
+
+
+def column_softmax_program(rows=64, cols_per_warp=64, num_warps=2, dtype="f16"):
+    """out[:, c] = softmax(x[:, c]) over the `rows` rows of the matrix, in f32: the reduces run along axis 0 and their [1 x cols]
+    results are broadcast back down the columns.  A program instance owns cols_per_warp * num_warps columns."""
+    t16, t32 = "tensor<%dx%dx%s" % (rows, cols_per_warp, dtype), "tensor<%dx%dxf32" % (rows, cols_per_warp)
+    c32 = "tensor<1x%dxf32, #values>" % cols_per_warp
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows, cols_per_warp, cols_per_warp * num_warps])
+    body += """    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{cpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{cpw}_i32 : i32
+    %col0 = arith.addi %p0, %w0 : i32
+    %col1 = arith.addi %col0, %c{cpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%c{rows}_i32, %cols] [%cols, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%c{rows}_i32, %cols] [%cols, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%c0_i32 : %c{rows}_i32, %col0 : %col1] : {dyn} -> {t16}, #global>
+    %so = kapy.sv_global %go[%c0_i32 : %c{rows}_i32, %col0 : %col1] : {dyn} -> {t16}, #global>
+    %x16 = kapy.ld_global %sx : {t16}, #global> -> {t16}, #values>
+    %xf = kapy.fptofp %x16 : {t16}, #values> to {t32}, #values>
+    %m = kapy.reduce %xf {{axis = 0 : i32}} lambda(%lhs: f32, %rhs: f32) {{
+      %r = arith.maximumf %lhs, %rhs : f32
+      kapy.return %r : f32
+    }} : {t32}, #values> -> {c32}
+    %mb = kapy.broadcast %m : {c32} -> {t32}, #values>
+    %d = arith.subf %xf, %mb : {t32}, #values>
+    %e = math.exp %d : {t32}, #values>
+    %s = kapy.reduce %e {{axis = 0 : i32}} lambda(%lhs: f32, %rhs: f32) {{
+      %r = arith.addf %lhs, %rhs : f32
+      kapy.return %r : f32
+    }} : {t32}, #values> -> {c32}
+    %sb = kapy.broadcast %s : {c32} -> {t32}, #values>
+    %q = arith.divf %e, %sb : {t32}, #values>
+    %y = kapy.fptofp %q {{rounding_mode = 1 : i32}} : {t32}, #values> to {t16}, #values>
+    kapy.st_global %y, %so : {t16}, #values>, {t16}, #global>
+    kapy.return
+""".format(cpp=cols_per_warp * num_warps, cpw=cols_per_warp, rows=rows, dyn=dyn, t16=t16, t32=t32, c32=c32)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @column_softmax_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %cols: i32) {\n" + body + "  }\n}\n")

@@ -272,3 +272,22 @@ def test_warps_exchange_inside_a_loop(ko, rows_per_warp, cols, warps, steps, pro
     kh.run_mlir(kp.exchange_loop_program(rows_per_warp, cols, warps, steps), [dx, dout, rows], [programs])
     sync()
     assert np.array_equal(to_host(dout, np.uint16), want.view(np.uint16).ravel())
+
+
+@pytest.mark.parametrize("rows,cols_per_warp", [(64, 64), (40, 24)])
+@pytest.mark.parametrize("fuse", ["1", "0"])
+def test_column_softmax_program_matches_the_oracle_program(ko, monkeypatch, rows, cols_per_warp, fuse):
+    """Reduces along axis 0: fused (the default) the ops between the load and the store are one program on the column machine with
+    both reduces as instructions; KAPY_MLIR_FUSE=0 runs every op by itself, the reduces as kapy_reduce along axis 0."""
+    monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+    warps, programs = 2, 3
+    cols = cols_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 71, std=3.0)
+    want = np.zeros(rows * cols, np.uint16)
+    g = lambda a: ko.mk_global(a, rows, cols, cols, 1, ko.F16)
+    insts = [dict(i, b=0) if i["op"] in (kh.EW_REDUCE_SUM, kh.EW_REDUCE_MAX) else i for i in kh.softmax_insts(kh.F16)]
+    assert ko.elementwise(ko.program(insts), [g(x)], g(want)) == 0
+    dx, dout = to_dev(x), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.column_softmax_program(rows, cols_per_warp, warps), [dx, dout, cols], [programs])
+    sync()
+    assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # in f32, one rounding to f16 at the end

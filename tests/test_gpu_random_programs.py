@@ -104,3 +104,36 @@ def test_random_exact_program(ko, seed):
     kh.elementwise(prog, d_ins, dglobal(dout2, r, c, s0, s1, out_dtype))
     sync()
     assert _same(to_host(dout2, NP_OF[outb]), want, out_dtype), "the compiled kernel differs from the oracle; " + describe
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_exact_program_with_column_maxima(ko, seed):
+    """The same random programs with two dependent reduces along axis 0 put before the store: t = min(v, max_col(u)),
+    result = t - max_col(t).  A maximum is exact in any order, so the column machine must match the oracle bit for bit."""
+    rng = np.random.RandomState(5000 + seed)
+    m, n, insts, kinds, in_dtypes, out_dtype, out_kind = _random_case(rng)
+    tail = []
+    while insts[-1]["op"] in (ST, CAST) and (insts[-1]["op"] == ST or insts[-1]["dst"] == 15):
+        tail.insert(0, insts.pop())
+    v = tail[0]["a"]                                                           # the value the program was going to cast / store
+    u = insts[rng.randint(len(insts))]["dst"]
+    insts += [dict(op=kh.EW_REDUCE_MAX, dst=13, a=u, b=0), dict(op=kh.EW_MINIMUMF, dst=14, a=v, b=13),
+              dict(op=kh.EW_REDUCE_MAX, dst=13, a=14, b=0), dict(op=kh.EW_SUBF, dst=14, a=14, b=13)]
+    tail[0] = dict(tail[0], a=14)
+    insts += tail
+    o_ins, d_ins, devs = [], [], []
+    for k, (kind, dt) in enumerate(zip(kinds, in_dtypes)):
+        r, c, s0, s1, count = _layout(kind, m, n)
+        a = ko.fill_uniform(count, dt, seed, k, -4.0, 4.0) if dt in (kh.F8E4M3, kh.F8E5M2) else ko.fill_normal(count, dt, seed, k, 0.0, 2.0)
+        devs.append(to_dev(a))
+        o_ins.append(ko.mk_global(a, r, c, s0, s1, dt))
+        d_ins.append(dglobal(devs[-1], r, c, s0, s1, dt))
+    r, c, s0, s1, count = _layout(out_kind, m, n)
+    outb = kh.DTYPE_BYTES[out_dtype]
+    want = np.zeros(count, NP_OF[outb])
+    assert ko.elementwise(ko.program(insts), o_ins, ko.mk_global(want, r, c, s0, s1, out_dtype)) == 0, "the oracle refuses the program: %s" % insts
+    dout = dev_zeros(count, outb)
+    kh.elementwise(kh.program(insts), d_ins, dglobal(dout, r, c, s0, s1, out_dtype))
+    sync()
+    assert _same(to_host(dout, NP_OF[outb]), want, out_dtype), "seed %d: %dx%d kinds %s dtypes %s -> %s %s, program %s" % (
+        seed, m, n, kinds, in_dtypes, out_dtype, out_kind, insts)

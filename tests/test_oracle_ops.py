@@ -261,6 +261,12 @@ def test_elementwise_reduce_ops_vs_numpy_and_scipy(ko):
     err = np.abs(y.view(np.float16).astype(np.float64) - want)
     assert np.all(err <= np.spacing(want.astype(np.float16)).astype(np.float64) * 0.51 + 1e-7 * want)   # half an f16 ulp + the fp32 steps
     assert np.allclose(y.view(np.float16).astype(np.float64).sum(axis=1), 1.0, atol=2e-3)
+    # the same along columns
+    cols = [dict(i, b=0) if i["op"] in (kh.EW_REDUCE_SUM, kh.EW_REDUCE_MAX) else i for i in kh.softmax_insts(kh.F16)]
+    assert ko.elementwise(ko.program(cols), [gh(x)], gh(y)) == 0
+    want = softmax(x.view(np.float16).astype(np.float64), axis=0)
+    err = np.abs(y.view(np.float16).astype(np.float64) - want)
+    assert np.all(err <= np.spacing(want.astype(np.float16)).astype(np.float64) * 0.51 + 1e-7 * want)
     # a reduce along an axis that does not exist is rejected
     bad = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_REDUCE_SUM, dst=1, a=0, b=2), dict(op=ko.EW_ST_GLOBAL, a=1)])
     assert ko.elementwise(bad, [g(xi)], g(out)) == -14

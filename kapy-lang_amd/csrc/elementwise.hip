@@ -829,6 +829,12 @@ int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
   return KAPY_OK;
 }
 
+// compiling and loading code objects are not stream work: they must not happen while a caller captures the stream into a graph
+bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(s, &status) == hipSuccess && status != hipStreamCaptureStatusNone;
+}
+
 }  // namespace
 }  // namespace kapy
 
@@ -868,6 +874,9 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
     // kernel may still serve: compile one now rather than turn the caller away.  Without the runtime compiler, or for a
     // program that fits neither, the row machine's refusal stands.
     const std::string refusal = last_error_buffer();
+    if (stream_is_capturing(s))
+      return fail(rc, "%s (a kernel compiled for the program could serve it, but nothing is compiled or loaded while the stream is being captured: "
+                  "call kapy_elementwise_specialize before the capture)", refusal.c_str());
     if (specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK && launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s) == 1)
       return KAPY_OK;
     return fail(rc, "%s", refusal.c_str());
@@ -908,7 +917,7 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
     const char *v = getenv("KAPY_EW_AUTO_SPECIALIZE");
     return v && v[0] == '1';
   }();
-  if (auto_specialize && specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK) {
+  if (auto_specialize && !stream_is_capturing(s) && specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK) {
     rc = launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s);
     if (rc != 0) return rc < 0 ? rc : KAPY_OK;
   }

@@ -750,14 +750,21 @@ void write_file_atomically(const std::string &path, const std::vector<char> &dat
   if (fclose(f) != 0 || !ok || rename(tmp.c_str(), path.c_str()) != 0) remove(tmp.c_str());
 }
 
-int compile_source(const std::string &source, std::vector<char> *code) {
+// from_cache (out): the code object was read from KAPY_EW_CACHE_DIR rather than compiled; use_cache = false compiles in any
+// case and overwrites what the cache holds (the caller found the cached object unusable).
+int compile_source(const std::string &source, std::vector<char> *code, bool *from_cache, bool use_cache = true) {
   // Packed fp32 VALU forms stay off, as for every device compile of this library.  Contraction only inside one
   // expression: in the generated text every op of the program is a statement of its own and must keep its own rounding
   // (with everything in one basic block the default, cross-statement mode would fuse a mulf and the addf after it).
   const char *opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=on", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
   constexpr int kOpts = (int)(sizeof opts / sizeof opts[0]);
   const std::string cached = cache_path(source, opts, kOpts);
-  if (!cached.empty() && read_file(cached, code)) return KAPY_OK;
+  *from_cache = false;
+  if (use_cache && !cached.empty() && read_file(cached, code)) {
+    *from_cache = true;
+    return KAPY_OK;
+  }
+  if (!use_cache && !cached.empty()) remove(cached.c_str());
   const Rtc &r = rtc();
   if (!r.ok) return fail(KAPY_ERR_UNSUPPORTED, "elementwise_specialize: the runtime compiler (libhiprtc) is not available");
   hiprtcProgram prog = nullptr;
@@ -813,13 +820,34 @@ int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
   std::vector<char> code;
   Loaded k;
   const std::string name = kernel_name(sig, key);
-  int rc = compile_source(generate(prog, n_inst, result_dtype, sig, name, &k.lds_bytes), &code);
+  const std::string source = generate(prog, n_inst, result_dtype, sig, name, &k.lds_bytes);
+  bool from_cache = false;
+  int rc = compile_source(source, &code, &from_cache);
   if (rc) return rc;
-  KAPY_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
-  KAPY_HIP_CHECK(hipModuleGetFunction(&k.fn, k.module, name.c_str()));
+  // A cached object is keyed by a hash only and may be damaged, foreign or built for another compiler: one that does not load, or
+  // does not hold the kernel, is thrown away and the source compiled again.
+  auto load = [&]() {
+    hipError_t e = hipModuleLoadData(&k.module, code.data());
+    if (e != hipSuccess) { k.module = nullptr; return e; }
+    e = hipModuleGetFunction(&k.fn, k.module, name.c_str());
+    if (e != hipSuccess) { (void)hipModuleUnload(k.module); k.module = nullptr; }
+    return e;
+  };
+  hipError_t e = load();
+  if (e != hipSuccess && from_cache) {
+    (void)hipGetLastError();
+    rc = compile_source(source, &code, &from_cache, false);
+    if (rc) return rc;
+    e = load();
+  }
+  if (e != hipSuccess) return fail(KAPY_ERR_HIP, "elementwise_specialize: the code object does not load: %s", hipGetErrorString(e));
   if (sig.rowwise) {
     int per_cu = 1;
-    KAPY_HIP_CHECK(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k.fn, sig.threads, (size_t)k.lds_bytes));
+    e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k.fn, sig.threads, (size_t)k.lds_bytes);
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(k.module);
+      return fail(KAPY_ERR_HIP, "elementwise_specialize: occupancy query failed: %s", hipGetErrorString(e));
+    }
     k.resident = device_cus() * (per_cu > 0 ? per_cu : 1);
   }
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -891,7 +919,8 @@ int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_d
   if (source_bytes) *source_bytes = (int64_t)text.size();
   if (code_bytes) {
     std::vector<char> code;
-    int rc = compile_source(text, &code);
+    bool from_cache = false;
+    int rc = compile_source(text, &code, &from_cache);
     if (rc) return rc;
     *code_bytes = (int64_t)code.size();
   }

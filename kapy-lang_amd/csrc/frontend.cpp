@@ -1096,9 +1096,11 @@ struct Interp {
       if (src != env.end() && src->second.kind == Value::kTensor && src->second.lazy) {
         if (!get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
         const kapy_global &sg = src->second.g;
-        if (b.g.end0 - b.g.start0 == sg.end0 - sg.start0 && b.g.end1 - b.g.start1 == sg.end1 - sg.start1 && b.g.dtype == sg.dtype &&
-            run_chain(op, src->second.lazy, &b.g) == KAPY_OK)
-          return KAPY_OK;
+        if (b.g.end0 - b.g.start0 == sg.end0 - sg.start0 && b.g.end1 - b.g.start1 == sg.end1 - sg.start1 && b.g.dtype == sg.dtype) {
+          const std::string before = err;
+          if (run_chain(op, src->second.lazy, &b.g) == KAPY_OK) return KAPY_OK;
+          err = before;  // the refusal is not the call's error: the store is tried again below through a register tensor
+        }
       }
       if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
       return lib(op, kapy_copy(&a.g, &b.g, nullptr, stream));
@@ -1189,28 +1191,46 @@ struct Interp {
   }
 };
 
-const char *const kSupportedOps[] = {
-    "kapy.return", "scf.yield", "scf.for", "arith.constant", "kapy.program_id", "kapy.warp_id", "arith.addi", "arith.subi", "arith.muli",
-    "arith.divui", "arith.remui", "arith.cmpi", "arith.select", "arith.addf", "arith.subf", "arith.mulf", "arith.divf", "arith.maximumf",
-    "arith.minimumf", "kapy.mk_global", "kapy.mk_shared", "kapy.sv_global", "kapy.sv_shared", "kapy.ld_global", "kapy.ld_matrix",
-    "kapy.ld_shared", "kapy.st_global", "kapy.st_shared", "kapy.cp_async_global_to_shared", "kapy.cp_async_wait_group", "kapy.matmul",
-    "kapy.reduce", "nvvm.barrier0", "math.exp", "math.exp2", "math.log", "math.log2", "math.sqrt", "math.rsqrt", "math.tanh", "math.erf",
-    "math.absf", "math.fma", "arith.negf", "arith.extf", "arith.truncf", "kapy.fptofp", "kapy.splat", "kapy.broadcast", "kapy.transpose"};
+// The ops this front-end executes, with the number of operands each needs at least and the number of results it has
+// (-1: any); the interpreter indexes operands and results by these counts without looking again.
+const struct OpForm { const char *name; int min_operands, results; } kSupportedOps[] = {
+    {"kapy.return", 0, 0}, {"scf.yield", 0, 0}, {"scf.for", 3, -1}, {"arith.constant", 0, 1}, {"kapy.program_id", 0, 1}, {"kapy.warp_id", 0, 1},
+    {"arith.addi", 2, 1}, {"arith.subi", 2, 1}, {"arith.muli", 2, 1}, {"arith.divui", 2, 1}, {"arith.remui", 2, 1}, {"arith.cmpi", 2, 1},
+    {"arith.select", 3, 1}, {"arith.addf", 2, 1}, {"arith.subf", 2, 1}, {"arith.mulf", 2, 1}, {"arith.divf", 2, 1}, {"arith.maximumf", 2, 1},
+    {"arith.minimumf", 2, 1}, {"kapy.mk_global", 6, 1}, {"kapy.mk_shared", 0, 1}, {"kapy.sv_global", 5, 1}, {"kapy.sv_shared", 5, 1},
+    {"kapy.ld_global", 1, 1}, {"kapy.ld_matrix", 1, 1}, {"kapy.ld_shared", 1, 1}, {"kapy.st_global", 2, 0}, {"kapy.st_shared", 2, 0},
+    {"kapy.cp_async_global_to_shared", 2, 0}, {"kapy.cp_async_wait_group", 0, 0}, {"kapy.matmul", 3, 1}, {"kapy.reduce", 1, 1},
+    {"nvvm.barrier0", 0, 0}, {"math.exp", 1, 1}, {"math.exp2", 1, 1}, {"math.log", 1, 1}, {"math.log2", 1, 1}, {"math.sqrt", 1, 1},
+    {"math.rsqrt", 1, 1}, {"math.tanh", 1, 1}, {"math.erf", 1, 1}, {"math.absf", 1, 1}, {"math.fma", 3, 1}, {"arith.negf", 1, 1},
+    {"arith.extf", 1, 1}, {"arith.truncf", 1, 1}, {"kapy.fptofp", 1, 1}, {"kapy.splat", 1, 1}, {"kapy.broadcast", 1, 1}, {"kapy.transpose", 1, 1}};
 
-// Every op must be one this front-end executes; returns the number of ops, regions included, or -1.
+// Every op must be one this front-end executes, written with the operands and results it needs; returns the number of ops,
+// regions included, -1 for an op it does not execute, -2 for one that is malformed.  (The body of a kapy.reduce is only looked at for its combiner: its ops are not executed.)
 int count_ops(const std::vector<Op> &ops, bool in_reduce, std::string &err) {
   int n = 0;
   for (const Op &op : ops) {
-    bool known = false;
-    for (const char *k : kSupportedOps) known |= op.name == k;
-    if (!known) {
+    const OpForm *form = nullptr;
+    for (const OpForm &k : kSupportedOps)
+      if (op.name == k.name) form = &k;
+    if (!form) {
       err = "line " + std::to_string(op.line) + ": operation '" + op.name + "' is not supported by this front-end";
       return -1;
+    }
+    if (!in_reduce) {
+      bool well_formed = (int)op.operands.size() >= form->min_operands && (form->results < 0 || (int)op.results.size() == form->results);
+      if (op.name == "scf.for")  // an induction variable, then one region argument and at most one result per carried operand
+        well_formed = well_formed && !op.region_args.empty() && op.operands.size() == 2 + op.region_args.size() && op.results.size() <= op.region_args.size() - 1;
+      if (!well_formed) {
+        err = "line " + std::to_string(op.line) + ": '" + op.name + "' is written with " + std::to_string(op.operands.size()) + " operands and " +
+              std::to_string(op.results.size()) + " results; it needs " + (op.name == "scf.for" ? "bounds, a step and one operand per iter_arg" :
+              "at least " + std::to_string(form->min_operands) + " operands") + (form->results >= 0 ? " and " + std::to_string(form->results) + " results" : "");
+        return -2;
+      }
     }
     ++n;
     if (!op.body.empty() && !in_reduce) {
       int inner = count_ops(op.body, op.name == "kapy.reduce", err);
-      if (inner < 0) return -1;
+      if (inner < 0) return inner;
       n += inner;
     }
   }
@@ -1230,7 +1250,7 @@ extern "C" int kapy_parse_mlir(const char *mlir_text, const char *func_name, int
   if (!ps.parse_module(f, func_name)) return fail(KAPY_ERR_INVALID, "parse_mlir: %s", ps.err.c_str());
   std::string err;
   int n = count_ops(f.body, false, err);
-  if (n < 0) return fail(KAPY_ERR_UNSUPPORTED, "parse_mlir: %s", err.c_str());
+  if (n < 0) return fail(n == -2 ? KAPY_ERR_INVALID : KAPY_ERR_UNSUPPORTED, "parse_mlir: %s", err.c_str());
   if (n_args) *n_args = (int32_t)f.arg_names.size();
   if (n_ops) *n_ops = n;
   if (num_warps) *num_warps = f.num_warps;
@@ -1245,7 +1265,7 @@ extern "C" int kapy_analyze_mlir(const char *mlir_text, const char *func_name, i
   Func f;
   if (!ps.parse_module(f, func_name)) return fail(KAPY_ERR_INVALID, "analyze_mlir: %s", ps.err.c_str());
   std::string err;
-  if (count_ops(f.body, false, err) < 0) return fail(KAPY_ERR_UNSUPPORTED, "analyze_mlir: %s", err.c_str());
+  if (int n = count_ops(f.body, false, err); n < 0) return fail(n == -2 ? KAPY_ERR_INVALID : KAPY_ERR_UNSUPPORTED, "analyze_mlir: %s", err.c_str());
   Analysis a;
   int rc = Analyzer(f, a).run(err);
   if (rc) return fail(rc, "analyze_mlir: %s", err.c_str());
@@ -1266,7 +1286,7 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   if (!ps.parse_module(f, func_name)) return fail(KAPY_ERR_INVALID, "run_mlir: %s", ps.err.c_str());
   {
     std::string err;
-    if (count_ops(f.body, false, err) < 0) return fail(KAPY_ERR_UNSUPPORTED, "run_mlir: %s", err.c_str());
+    if (int n = count_ops(f.body, false, err); n < 0) return fail(n == -2 ? KAPY_ERR_INVALID : KAPY_ERR_UNSUPPORTED, "run_mlir: %s", err.c_str());
   }
   Analysis plan;
   {

@@ -134,3 +134,21 @@ def test_analysis_finds_the_barrier_between_warps_that_exchange_tiles():
     assert kh.analyze_mlir(kp.exchange_program(barrier=True))[2] == []
     # in the loop the program places both barriers itself (before the stores: the previous step's loads; before the loads)
     assert kh.analyze_mlir(kp.exchange_loop_program())[2] == []
+
+
+@pytest.mark.parametrize("program,damage,named", [
+    (kp.binary_program, lambda t: t.replace("%vo = arith.addf %vx, %vy", "%vo = arith.addf %vx"), "arith.addf"),                     # an operand short
+    (kp.binary_program, lambda t: t.replace("%vo = arith.addf %vx, %vy", "arith.addf %vx, %vy"), "arith.addf"),                     # no result
+    (kp.binary_program, lambda t: t.replace("kapy.st_global %vo, %so", "kapy.st_global %vo"), "kapy.st_global"),
+    (kp.exchange_program, lambda t: t.replace("%mine = kapy.sv_shared %buf[%w0 : %w1, %c0_i32 : %c64_i32]", "%mine = kapy.sv_shared %buf[%w0 : %w1]"), "kapy.sv_shared"),
+    (kp.exchange_loop_program, lambda t: t.replace("%last = scf.for", "%last, %more = scf.for"), "scf.for"),                       # more results than carried values
+])
+def test_an_op_written_with_too_few_operands_or_results_is_refused_before_it_runs(program, damage, named):
+    text = program()
+    broken = damage(text)
+    assert broken != text
+    with pytest.raises(kh.KapyError) as e:
+        kh.parse_mlir(broken)
+    assert e.value.status == -1 and named in e.value.message and "line " in e.value.message
+    with pytest.raises(kh.KapyError):
+        kh.analyze_mlir(broken)

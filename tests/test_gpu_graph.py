@@ -87,3 +87,38 @@ def test_every_kernel_family_replays_from_a_graph():
         for name in captured:
             assert torch.equal(captured[name], eager[name]), "replay with seed %d differs from the eager call in %s" % (seed, name)
         assert int((captured["soft"] != 0x1111).sum()) > 0
+
+
+def test_nothing_is_compiled_or_loaded_while_a_stream_is_captured():
+    """A row program the row machine refuses (a width that is no multiple of 8) is normally served by compiling a kernel on its
+    first call.  Inside a capture that must not happen (compiling and loading a module are not stream work): the call is refused
+    with a message that says what to do, and the capture stays usable."""
+    m, n = 4, 104
+    x = (torch.randn(m * n, device="cuda") * 2).half().view(torch.int16)
+    soft, copy = torch.zeros(m * n, dtype=torch.int16, device="cuda"), torch.zeros(m * n, dtype=torch.int16, device="cuda")
+    prog = kh.program(kh.softmax_insts(kh.F16))
+    narrow = lambda t: kh.sv_global(dglobal(t, m, n, n, 1, kh.F16), 0, m, 0, 100)      # rows of 100 that start aligned to 8 elements
+    xin = kh.sv_global(dglobal(x, m, n, n, 1, kh.F16), 0, m, 0, 100)
+    kh.copy(dglobal(x, m, n, n, 1, kh.F16), dglobal(copy, m, n, n, 1, kh.F16))     # lazy loading of the copy kernel: outside the capture
+    copy.zero_()
+    sync()
+    loaded_before = kh.elementwise_specialize_stats()[0]
+    refused = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        kh.copy(dglobal(x, m, n, n, 1, kh.F16), dglobal(copy, m, n, n, 1, kh.F16))
+        try:
+            kh.elementwise(prog, [xin], narrow(soft))
+        except kh.KapyError as e:
+            refused = e
+    assert refused is not None and refused.status == kh.ERR_UNSUPPORTED and "captured" in refused.message
+    assert kh.elementwise_specialize_stats()[0] == loaded_before
+    graph.replay()
+    sync()
+    assert torch.equal(copy, x) and int(soft.count_nonzero()) == 0
+    # outside a capture the same call compiles its kernel and runs
+    kh.elementwise(prog, [xin], narrow(soft))
+    sync()
+    assert kh.elementwise_specialize_stats()[0] == loaded_before + 1
+    sums = soft.view(torch.float16).float().view(m, n)[:, :100].sum(dim=1)
+    assert torch.allclose(sums, torch.ones_like(sums), atol=2e-2)

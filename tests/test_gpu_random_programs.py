@@ -121,10 +121,11 @@ def test_random_exact_program_with_column_maxima(ko, seed):
               dict(op=kh.EW_REDUCE_MAX, dst=13, a=14, b=0), dict(op=kh.EW_SUBF, dst=14, a=14, b=13)]
     tail[0] = dict(tail[0], a=14)
     insts += tail
-    o_ins, d_ins, devs = [], [], []
+    arrays, o_ins, d_ins, devs = [], [], [], []
     for k, (kind, dt) in enumerate(zip(kinds, in_dtypes)):
         r, c, s0, s1, count = _layout(kind, m, n)
         a = ko.fill_uniform(count, dt, seed, k, -4.0, 4.0) if dt in (kh.F8E4M3, kh.F8E5M2) else ko.fill_normal(count, dt, seed, k, 0.0, 2.0)
+        arrays.append(a)                       # (the oracle's descriptor holds a bare pointer: the array has to outlive it)
         devs.append(to_dev(a))
         o_ins.append(ko.mk_global(a, r, c, s0, s1, dt))
         d_ins.append(dglobal(devs[-1], r, c, s0, s1, dt))

@@ -522,3 +522,33 @@ def _gelu_insts():
     return [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=SPL, dst=2, dtype=kh.F32, imm=0.5), dict(op=MUL, dst=1, a=1, b=2),
             dict(op=L, dst=4, a=1), dict(op=CAST, dst=4, a=4, dtype=kh.F32), dict(op=ADD, dst=1, a=1, b=4), dict(op=kh.EW_GELU_TANH, dst=1, a=1),
             dict(op=CAST, dst=5, a=1, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=5)]
+
+
+def test_a_damaged_cached_code_object_is_replaced(ko, tmp_path, monkeypatch):
+    """KAPY_EW_CACHE_DIR holds code objects keyed by a hash of their source.  A file there that is not a loadable code object
+    (damaged, foreign) must not poison the program for good: the load fails, the file is thrown away and the source is
+    compiled again."""
+    import os
+    monkeypatch.setenv("KAPY_EW_CACHE_DIR", str(tmp_path))
+    m, n = 24, 136
+    insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=SUB, dst=2, a=0, b=1), dict(op=MIN, dst=2, a=2, b=1),
+             dict(op=kh.EW_ABSF, dst=2, a=2), dict(op=ST, a=2)]
+    a, b = ko.fill_normal(m * n, kh.F16, 91, 0).reshape(m, n), ko.fill_normal(m * n, kh.F16, 91, 1).reshape(m, n)
+    want = np.zeros((m, n), np.uint16)
+    og = lambda x: ko.mk_global(x, m, n, n, 1, kh.F16)
+    assert ko.elementwise(ko.program(insts), [og(a), og(b)], og(want)) == 0
+    da, db, dz = to_dev(a), to_dev(b), dev_zeros(m * n, 2)
+    g = lambda t: dglobal(t, m, n, n, 1, kh.F16)
+    prog = kh.program(insts)
+    _, size = kh.elementwise_source(prog, [g(da), g(db)], g(dz), compile=True)          # compiles and fills the cache
+    files = os.listdir(tmp_path)
+    assert len(files) == 1 and os.path.getsize(tmp_path / files[0]) == size
+    with open(tmp_path / files[0], "wb") as f:
+        f.write(b"not a code object " * 64)
+    loaded_before, _ = kh.elementwise_specialize_stats()
+    kh.elementwise_specialize(prog, [g(da), g(db)], g(dz))                              # reads the damaged file, recovers
+    assert kh.elementwise_specialize_stats()[0] == loaded_before + 1
+    assert os.path.getsize(tmp_path / files[0]) == size
+    kh.elementwise(prog, [g(da), g(db)], g(dz))
+    sync()
+    assert np.array_equal(to_host(dz, np.uint16, (m, n)), want)

@@ -71,8 +71,9 @@ def _events(fn, steps, warmup):
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the
 # same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
-MEASURED_TRAFFIC = {"gelu": 268414976, "transpose": 268456960, "add": 402639872, "softmax": 268476416, "layernorm": 268788736,
-                    "expr_compiled": 402619392, "swiglu": 402556928, "l2norm_compiled": 268408832}
+MEASURED_TRAFFIC = {"gelu": 268411308, "transpose": 268449994, "add": 402640502, "expr": 402796218, "softmax": 268466794, "layernorm": 268779749,
+                    "expr_compiled": 402621054, "swiglu": 402555636, "l2norm_compiled": 268407520, "gelu_transposed": 268397184, "copy": 268435456,
+                    "permute": 268435456, "reduce": 134292547, "gemm_bf16": 1751983831, "gemm_bf16_gelu": 1757747749, "f8_m4096": 470420532}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -210,7 +211,7 @@ def bench_copy(kh, steps, warmup, cpu):
     wall, ev = _events(lambda i: kh.copy(gx[i % sets], gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
     return {"workload": "copy fp16 8192x8192 (ld_global -> st_global, no transpose)", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev, "copy"), "kernel": "rows_kernel",
             "inputs": "uniform random 16-bit patterns seed 0", "checked": True, "check": "whole result bit-equal to the source"}
 
 
@@ -261,7 +262,7 @@ def bench_add(kh, steps, warmup, cpu, op="add"):
             "swiglu": "z = silu(x)*y fp16 8192x8192 in fp32, compiled at run time"}[op]
     kernel = {"add": "affine_act_kernel", "expr": "stack_kernel_narrow"}.get(op, "kapy_ew_flat_<hash> (compiled at run time)")
     return {"workload": name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev, op if op != "expr" else None), "kernel": kernel, "inputs": "x, y normal(0,1), seeded",
+            "roofline": _roof_hbm(nbytes, ev, op), "kernel": kernel, "inputs": "x, y normal(0,1), seeded",
             "checked": True, "check": "16 rows against the checker: max %d ulp (tolerance %d)" % (worst, tol)}
 
 
@@ -295,7 +296,7 @@ def bench_gelu_transposed(kh, steps, warmup, cpu):
     nbytes = 2 * n * n * 2 + n * 2
     return {"workload": "gelu_tanh(x^T*0.5+bias) fp16 8192x8192: transpose fused with the elementwise chain, compiled at run time",
             "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16",
-            "roofline": _roof_hbm(nbytes, ev), "kernel": "kapy_ew_flat_<hash> (tiled; compiled at run time)", "inputs": "as C2, x read through swapped strides",
+            "roofline": _roof_hbm(nbytes, ev, "gelu_transposed"), "kernel": "kapy_ew_flat_<hash> (tiled; compiled at run time)", "inputs": "as C2, x read through swapped strides",
             "checked": True, "check": "16 rows against the checker: max %d ulp (tolerance %d)" % (worst, ULP_TOL)}
 
 
@@ -319,7 +320,7 @@ def bench_reduce(kh, steps, warmup, cpu):
     wall, ev = _events(lambda i: kh.reduce(gx[i % sets], gy, 1, 0), steps, warmup)
     nbytes = n * n * 2 + n * 4
     return {"workload": "reduce_sum axis=1 fp16 8192x8192 -> f32 [8192x1]", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev), "kernel": "reduce_rows_vec_kernel",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "reduce"), "kernel": "reduce_rows_vec_kernel",
             "inputs": "x normal(0,1) seed 0", "checked": True, "check": "every row sum against fp64: max abs error %.2e" % err}
 
 
@@ -436,7 +437,7 @@ def bench_permute(kh, steps, warmup, cpu):
     wall, ev = _events(lambda i: kh.copy_batched(gx[i % sets], gy[i % sets], grid), steps, warmup)
     nbytes = 2 * tot * 2
     out = {"workload": "C3b permute bf16 [8,32,2048,128] bhsd->bshd", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev), "kernel": "rows_kernel",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "u16", "roofline": _roof_hbm(nbytes, ev, "permute"), "kernel": "rows_kernel",
            "inputs": "uniform random 16-bit patterns seed 1 (as the configuration states)", "checked": True,
            "check": "8 of 256 (b,h) programs bit-equal to the checker; every element bit-equal to in[b,h,s,d]"}
     if cpu:
@@ -734,7 +735,7 @@ def main():
         "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, cpu, "l2norm_compiled"),
         "permute": lambda s, w: bench_permute(kh, s, w, cpu),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel", key="gemm_bf16"),
-        "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True),
+        "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True, key="gemm_bf16_gelu"),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform"),
         "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform"),
         "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True),

@@ -203,7 +203,7 @@ template <int TI, int TJ, bool NT>
 __global__ __launch_bounds__(256) void transpose_lds_kernel(CopyParams p) {
   constexpr int NI = TI / 8, NJ = TJ / 8, ROW = TJ * 2, PER_LANE = NI * NJ / 256;
   static_assert(NI >= 16 && NJ >= 16 && (NI * NJ) % 256 == 0, "tile must hold whole 16-lane phases");
-  extern __shared__ __attribute__((aligned(16))) char tile[];
+  __shared__ __attribute__((aligned(16))) char tile[TI * TJ * 2];  // static: the size is the code object's, no launch attribute to raise
   const char *src;
   char *dst;
   program_base<2>(p, src, dst);
@@ -265,20 +265,9 @@ __global__ __launch_bounds__(256) void transpose_lds_kernel(CopyParams p) {
 
 template <int TI, int TJ>
 int launch_transpose_lds(const CopyParams &p, bool nt, int32_t batch, hipStream_t stream) {
-  constexpr int kLds = TI * TJ * 2;
   dim3 grid((unsigned)((p.d0 + TI - 1) / TI), (unsigned)((p.d1 + TJ - 1) / TJ), (unsigned)batch);
-  if (kLds > 65536) {
-    static bool configured_on[64];  // per device (the attribute belongs to the code object loaded on that device); a race only repeats the calls
-    int dev = 0;
-    KAPY_HIP_CHECK(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64 || !configured_on[dev]) {
-      KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)transpose_lds_kernel<TI, TJ, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-      KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)transpose_lds_kernel<TI, TJ, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-      if (dev >= 0 && dev < 64) configured_on[dev] = true;
-    }
-  }
-  if (nt) transpose_lds_kernel<TI, TJ, true><<<grid, 256, kLds, stream>>>(p);
-  else transpose_lds_kernel<TI, TJ, false><<<grid, 256, kLds, stream>>>(p);
+  if (nt) transpose_lds_kernel<TI, TJ, true><<<grid, 256, 0, stream>>>(p);
+  else transpose_lds_kernel<TI, TJ, false><<<grid, 256, 0, stream>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }

@@ -466,7 +466,9 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
   using L = TileLayout<C::kRowBytes, T>;
   constexpr int EB = T::kBytes, CH = T::kChunks;
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  // Static, so that the size is a property of the code object (160 KiB, a CU's whole LDS, for the 256 x 256 ring) and no
+  // launch depends on the runtime honouring a raised dynamic-LDS limit: LDS-direct loads that land outside the allocation fault.
+  __shared__ __attribute__((aligned(1024))) char lds[C::kLdsBytes];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave % WM, wn = wave / WM;
@@ -917,7 +919,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   constexpr int kBytesA = kNBM * kRowA, kBytesB = BK * kRowB, kStage = kBytesA + kBytesB;
   constexpr int kLoadsA = kBytesA / 1024 / 4, kLoadsB = kBytesB / 1024 / 4, kLoads = kLoadsA + kLoadsB;  // per wavefront per tile
   constexpr int KK = BK / 32, kTm = 4, kTn = 4, kMfmas = kTm * kTn;
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStage];  // static: see tn_kernel
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave & 1, wn = wave >> 1;
@@ -1226,32 +1228,11 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool P
 int launch_tn_epi(GemmParams p, hipStream_t s) {
   using C = TnConfig<T, BM, BN, BK, WM, WN, STAGES>;
   auto kernel = tn_kernel<T, BM, BN, BK, WM, WN, STAGES, PACKED, KTAIL, TAIL>;
-  // The kernel addresses kLdsBytes of dynamic LDS (more than the 64 KiB default limit), also through
-  // LDS-direct loads, which fault when they land outside the allocation.  Make sure the limit has
-  // really been raised before the first launch: query first (this also forces the code object to be
-  // loaded, so the attribute is not set on a function the runtime has not materialised yet), set,
-  // and read back.
-  static bool configured_on[kMaxDevices];  // per device: a code object is loaded, and its attributes kept, per device; idempotent, a race only repeats the calls
-  int dev = 0;
-  KAPY_HIP_CHECK(hipGetDevice(&dev));
-  bool &configured = configured_on[dev >= 0 && dev < kMaxDevices ? dev : 0];
-  if (!configured || dev >= kMaxDevices) {
-    hipFuncAttributes fa;
-    KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, (const void *)kernel));
-    if (fa.maxDynamicSharedSizeBytes < C::kLdsBytes) {
-      KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::kLdsBytes));
-      KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, (const void *)kernel));
-      if (fa.maxDynamicSharedSizeBytes < C::kLdsBytes)
-        return fail(KAPY_ERR_HIP, "matmul: could not raise the dynamic LDS limit to %d bytes (runtime reports %d)", C::kLdsBytes,
-                    (int)fa.maxDynamicSharedSizeBytes);
-    }
-    configured = true;
-  }
   p.tiles_m = (p.M + BM - 1) / BM;  // (only the ring variants are launched with tiles that hang over an edge)
   p.tiles_n = (p.N + BN - 1) / BN;
   constexpr bool kCanSplit = BM == 128 && BN == 128 && STAGES == kRing25;
   if (!kCanSplit) p.split_k = 1;
-  kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k), dim3(C::kThreads), C::kLdsBytes, s>>>(p);
+  kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k), dim3(C::kThreads), 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }
@@ -1283,29 +1264,12 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
 
 template <typename T, int BK, int STAGES>
 int launch_nn(GemmParams p, hipStream_t s) {
-  constexpr int kLds = STAGES * BK * 512;
   p.tiles_m = (p.M + kNBM - 1) / kNBM;  // M need not be a multiple of the tile: see the kernel's lhs descriptor
   p.tiles_n = p.N / kNBN;
   const bool packed = packed_epilogue(p) && !host_has_tail(p);  // (a fused tail goes through the element stores here)
-  const void *kernel = packed ? (const void *)nn_kernel<T, BK, STAGES, true> : (const void *)nn_kernel<T, BK, STAGES, false>;
-  static bool configured_on[kMaxDevices][2];  // per device and kernel; idempotent, a race only repeats the calls
-  int dev = 0;
-  KAPY_HIP_CHECK(hipGetDevice(&dev));
-  bool(&configured)[2] = configured_on[dev >= 0 && dev < kMaxDevices ? dev : 0];
-  if (!configured[packed] || dev >= kMaxDevices) {
-    hipFuncAttributes fa;
-    KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, kernel));
-    if (fa.maxDynamicSharedSizeBytes < kLds) {
-      KAPY_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-      KAPY_HIP_CHECK(hipFuncGetAttributes(&fa, kernel));
-      if (fa.maxDynamicSharedSizeBytes < kLds)
-        return fail(KAPY_ERR_HIP, "matmul: could not raise the dynamic LDS limit to %d bytes (runtime reports %d)", kLds, (int)fa.maxDynamicSharedSizeBytes);
-    }
-    configured[packed] = true;
-  }
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k);
-  if (packed) nn_kernel<T, BK, STAGES, true><<<grid, dim3(256), kLds, s>>>(p);
-  else nn_kernel<T, BK, STAGES, false><<<grid, dim3(256), kLds, s>>>(p);
+  if (packed) nn_kernel<T, BK, STAGES, true><<<grid, dim3(256), 0, s>>>(p);
+  else nn_kernel<T, BK, STAGES, false><<<grid, dim3(256), 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }

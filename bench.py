@@ -622,7 +622,7 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     flops = 2.0 * M * N * K
     nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
     out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192%s" % (M, ", K split across workgroups (workspace given)" if workspace else ""), "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "tn_kernel<F8, 128x128x128> split K" if (workspace and 40 <= M <= 128) else "skinny_stream_kernel" if M <= 80 else "tn_kernel<F8>",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 160 and not workspace)) else "tn_kernel<F8, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8>",
            "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
            "checked": True, "check": "%d %dx64 blocks against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" % (n_blocks, min(M, 64), rel, FROB_TOL)}
     out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d" % M) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
@@ -699,7 +699,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
 
 
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m64_splitk", "f8_m4096", "ceilings"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
 
 
 def main():
@@ -741,7 +741,8 @@ def main():
         "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True),
         "f8_m16": lambda s, w: bench_f8(kh, s, w, cpu, 16),
         "f8_m64": lambda s, w: bench_f8(kh, s, w, False, 64),
-        "f8_m64_splitk": lambda s, w: bench_f8(kh, s, w, False, 64, workspace=True),
+        "f8_m128": lambda s, w: bench_f8(kh, s, w, False, 128),
+        "f8_m128_splitk": lambda s, w: bench_f8(kh, s, w, False, 128, workspace=True),
         "f8_m4096": lambda s, w: bench_f8(kh, s, w, cpu, 4096),
         "ceilings": lambda s, w: bench_ceilings(kh, s, w, cpu),
     }

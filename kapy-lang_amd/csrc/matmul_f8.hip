@@ -146,10 +146,13 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 // 256 K-bytes of 16 rows each), 16-byte chunk c of row r stored at chunk c ^ r of the row's 256 bytes
 // so that the 16 rows a quarter-wave reads fall into 16 different bank groups.
 // Rows past M / N are clamped to the last valid row (never stored), so nothing is read out of range.
-// From this many rows on the tiled MFMA kernel (which reads the weight once for up to 128 rows) beats the weight-streaming
-// kernel below (which reads it once per 16 rows).
-constexpr int kTiledFromM = 81;
-constexpr int kTiledFromMSplit = 40;  // the same threshold when K can be split across workgroups (measured at N = K = 8192)
+// Which kernel serves how many rows (thresholds measured at N = K = 8192).  Up to 16 rows: the streaming kernel below.
+// From 17 rows: the block streaming kernel (32 columns x up to 64 rows per workgroup, the weight read once), where K is a
+// multiple of 512; it yields to the tiled MFMA kernel from kTiledFromM rows, or from kTiledFromMSplit when the caller's
+// workspace lets the tiled kernel split K across workgroups.  Where the block kernel cannot run, the streaming kernel
+// (which reads the weight once per 16 rows) is all there is below the tiled kernel, and the tiled kernel takes over earlier.
+constexpr int kTiledFromM = 161, kTiledFromMSplit = 65;
+constexpr int kTiledFromMNoBlock = 81, kTiledFromMSplitNoBlock = 40;
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
 template <int A_FMT, int B_FMT>
 __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Params p) {
@@ -239,6 +242,141 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
   }
 }
 
+// Block streaming kernel: the same idea for 17 .. 64 rows of lhs (and, in blocks of 64 rows, beyond).  Reading the
+// weight once per 16 rows, as the kernel above does, asks the L2 for it M/16 times, and a workgroup of 16 columns re-reads
+// the whole activation: at M = 64 the activation traffic is four times the weight's.  Here a workgroup owns 32 columns and
+// 16*RG rows, so at N = 8192 there is one workgroup per CU, every weight byte crosses the fabric once, and the activation
+// (M x K bytes, L2-resident) is read N/32 times.  Its 4 waves split K and work alone on private rings of kBlockStages
+// stages; a stage is one 128-byte K step: 32 weight rows and 16*RG activation rows of 128 contiguous bytes, brought in by
+// LDS-direct loads of 8 rows each, 16-byte chunk c of row r stored at chunk c ^ ((r / 2) % 8) - the 16 rows a
+// quarter-wave reads then cover all 64 banks once.  RG x 2 accumulator blocks per wave; the four K ranges meet in LDS.
+constexpr int kBlockStep = 128, kBlockCols = 32;
+constexpr int block_stages(int) { return 3; }  // (four for 32 rows fits the LDS too and measured no faster)
+constexpr int waitcnt_vm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }  // s_waitcnt vmcnt(n), nothing else waited for
+template <int A_FMT, int B_FMT, int RG>
+__global__ __launch_bounds__(256) void skinny_block_kernel(F8Params p) {
+  constexpr int kBlockStages = block_stages(RG), kRows = 16 * RG, kStage = (kBlockCols + kRows) * kBlockStep, kLoadsW = kBlockCols / 8, kLoadsA = kRows / 8, kLoads = kLoadsW + kLoadsA;
+  static_assert(4 * kBlockStages * kStage <= 160 * 1024 && (kBlockStages - 1) * kLoads <= 63, "rings must fit the LDS, loads in flight the counter");
+  __shared__ __attribute__((aligned(1024))) char ring[4 * kBlockStages * kStage];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // workgroup id -> (32-column block, row block): the row blocks of a column block take ids 8 apart (one XCD, dispatched
+  // back to back), so that the second reader of a weight line finds it in that XCD's L2
+  const int32_t col_blocks = (p.N + kBlockCols - 1) / kBlockCols, row_blocks = (p.M + kRows - 1) / kRows;
+  const int32_t on_xcd = blockIdx.x / 8, xcd = blockIdx.x % 8;
+  const int32_t col_block = (on_xcd / row_blocks) * 8 + xcd;
+  if (col_block >= col_blocks) return;  // (the grid is padded to whole rounds of 8)
+  const int32_t n0 = col_block * kBlockCols, m0 = (on_xcd % row_blocks) * kRows;
+  const int32_t k_per_wave = p.K / 4, steps = k_per_wave / kBlockStep;
+  auto uniform_ptr = [](const uint8_t *ptr) {
+    const uint64_t v = (uint64_t)ptr;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (void *)(((uint64_t)hi << 32) | lo);
+  };
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * p.b_sn + (int64_t)wave * k_per_wave), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm + (int64_t)wave * k_per_wave), 0, 0x7fffffff, 0x00020000);
+  // load instruction i of an operand: rows 8i .. 8i+7, this lane row 8i + lane/8, filling chunk position lane%8 of it.
+  // Rows past N / M are clamped to the last valid row (their results are never stored), so nothing is read out of range.
+  uint32_t w_off[kLoadsW], a_off[kLoadsA];
+#pragma unroll
+  for (int i = 0; i < kLoadsW; ++i) {
+    const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+    w_off[i] = (uint32_t)(min(r, p.N - 1 - n0) * p.b_sn + c * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < kLoadsA; ++i) {
+    const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+    a_off[i] = (uint32_t)(min(r, p.M - 1 - m0) * p.a_sm + c * 16);
+  }
+  char *my_ring = ring + wave * (kBlockStages * kStage);
+  auto issue_step = [&](int step, int stage) {
+    char *dst = my_ring + stage * kStage;
+#pragma unroll
+    for (int i = 0; i < kLoadsW; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, (int)w_off[i], step * kBlockStep, 0, 0);
+#pragma unroll
+    for (int i = 0; i < kLoadsA; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + kBlockCols * kBlockStep + i * 1024), 16, (int)a_off[i], step * kBlockStep, 0, 0);
+  };
+  // operand reads: the lane's row of a 16-row block and its 32 K bytes of the step, chunks 2*group and 2*group + 1
+  const OperandLane frag_at = operand_lane(kF8Shape, lane);
+  const int r16 = frag_at.row, grp = frag_at.k0 / kF8Shape.kpack;
+  uint32_t rd[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) rd[h] = (uint32_t)(r16 * kBlockStep + (((2 * grp + h) ^ ((r16 >> 1) & 7)) * 16));
+  f32x4 acc[RG][2];
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int g = 0; g < 2; ++g) acc[r][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < kBlockStages; ++st)
+    if (st < steps) issue_step(st, st);
+  int stage = 0;
+  for (int32_t c = 0; c < steps; ++c) {
+    // this step has landed once only the younger steps' loads remain in flight
+    const int32_t younger = min(steps - 1 - c, kBlockStages - 1);
+    if (younger >= 3) __builtin_amdgcn_s_waitcnt(waitcnt_vm(3 * kLoads));
+    else if (younger == 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * kLoads));
+    else if (younger == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(kLoads));
+    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    static_assert(kBlockStages <= 4, "the waits above are written for up to four stages");
+    const char *src = my_ring + stage * kStage;
+    i32x4 w[2][2], a[RG][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int g = 0; g < 2; ++g) w[g][h] = *(const i32x4 *)(src + g * 16 * kBlockStep + rd[h]);
+#pragma unroll
+      for (int r = 0; r < RG; ++r) a[r][h] = *(const i32x4 *)(src + (kBlockCols + r * 16) * kBlockStep + rd[h]);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the stage has been read, it may be refilled
+    if (c + kBlockStages < steps) issue_step(c + kBlockStages, stage);
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      const i32x8 av = {a[r][0][0], a[r][0][1], a[r][0][2], a[r][0][3], a[r][1][0], a[r][1][1], a[r][1][2], a[r][1][3]};
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const i32x8 wv = {w[g][0][0], w[g][0][1], w[g][0][2], w[g][0][3], w[g][1][0], w[g][1][1], w[g][1][2], w[g][1][3]};
+        acc[r][g] = mfma_f8<A_FMT, B_FMT>(av, wv, acc[r][g]);
+      }
+    }
+    stage = stage + 1 == kBlockStages ? 0 : stage + 1;
+  }
+  // the four K ranges meet in LDS
+  const AccLane acc_at = acc_lane(mfma_acc(kF8Shape), kF8Shape, lane);
+  __syncthreads();  // every wave is done with its ring
+  float *partial = (float *)ring;  // [wave][kRows][kBlockCols + 1]
+  constexpr int kPitch = kBlockCols + 1;
+  static_assert(4 * kRows * kPitch * 4 <= 4 * kBlockStages * kStage, "the partial sums reuse the rings");
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) partial[(wave * kRows + 16 * r + acc_at.row + v) * kPitch + 16 * g + acc_at.col] = acc[r][g][v];
+  __syncthreads();
+  for (int e = threadIdx.x; e < kRows * kBlockCols; e += 256) {
+    const int m = e / kBlockCols, n = e % kBlockCols;
+    float sum = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < 4; ++w2) sum += partial[(w2 * kRows + m) * kPitch + n];
+    finish(p, m0 + m, n0 + n, sum);
+  }
+}
+
+template <int RG>
+int launch_skinny_block(const F8Params &p, int fa, int fb, hipStream_t s) {
+  const int64_t col_rounds = ((p.N + kBlockCols - 1) / kBlockCols + 7) / 8, row_blocks = (p.M + 16 * RG - 1) / (16 * RG);
+  dim3 grid((unsigned)(col_rounds * 8 * row_blocks));
+  if (fa == 0 && fb == 0) skinny_block_kernel<0, 0, RG><<<grid, 256, 0, s>>>(p);
+  else if (fa == 0) skinny_block_kernel<0, 1, RG><<<grid, 256, 0, s>>>(p);
+  else if (fb == 0) skinny_block_kernel<1, 0, RG><<<grid, 256, 0, s>>>(p);
+  else skinny_block_kernel<1, 1, RG><<<grid, 256, 0, s>>>(p);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 int fmt_of(int dtype) { return dtype == KAPY_F8E5M2 ? 1 : 0; }
 
 }  // namespace
@@ -267,6 +405,9 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   // With a workspace the tiled kernel can split K over several workgroups per tile, which fills the device at few rows too.
   kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
   if (cfg) c = *cfg;
+  // (offsets inside a workgroup's rows and columns are 32-bit)
+  const bool block_ok = k_contig && p.M > 16 && p.K % (4 * kBlockStep) == 0 && p.a_sm * 64 < (int64_t(1) << 31) && p.b_sn * kBlockCols < (int64_t(1) << 31) &&
+                        ((int64_t)(p.N + kBlockCols - 1) / kBlockCols + 8) * ((p.M + 31) / 32) < (int64_t(1) << 31);
   if (k_contig && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
     GemmParams g;
     g.a = (const char *)p.a; g.b = (const char *)p.b; g.acc = nullptr; g.d = p.d;
@@ -278,9 +419,17 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     g.acc_dtype = -1; g.d_dtype = p.d_dtype; g.rz = p.rz; g.tiles_m = g.tiles_n = 0;
     int rc = plan_split_k(g, c, 128);
     if (rc) return rc;
-    if (p.M < (g.split_k > 1 ? kTiledFromMSplit : kTiledFromM)) rc = KAPY_ERR_UNSUPPORTED;  // few rows: the streaming kernels below
+    // an explicit split is a request for the tiled kernel; the library's own choice weighs it against the block kernel
+    const int tiled_from = block_ok && c.split_k <= 1 ? (g.split_k > 1 ? kTiledFromMSplit : kTiledFromM) : (g.split_k > 1 ? kTiledFromMSplitNoBlock : kTiledFromMNoBlock);
+    if (p.M < tiled_from) rc = KAPY_ERR_UNSUPPORTED;  // few rows: the streaming kernels below
     else rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
+  }
+  if (block_ok) {
+    const int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
+    if (p.M <= 32) return launch_skinny_block<2>(p, fa, fb, s);
+    if (p.M <= 48) return launch_skinny_block<3>(p, fa, fb, s);
+    return launch_skinny_block<4>(p, fa, fb, s);
   }
   if (k_contig && p.K % (kStreamWaves * kStreamChunk) == 0 && (p.M + 15) / 16 <= 65535 && p.a_sm * 16 < (int64_t(1) << 31) &&
       p.b_sn * 16 < (int64_t(1) << 31)) {

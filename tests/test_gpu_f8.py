@@ -43,6 +43,28 @@ def test_scaled_f8_small(ko, M, N, K):
     assert _frob(ko, to_host(dd, np.uint16, (M, N)), want) <= FROB_TOL
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 64, 512), (32, 96, 1024), (33, 100, 1536), (48, 32, 512), (49, 40, 2048), (64, 256, 4096), (24, 1000, 512),
+                                   (64, 8, 512)])
+@pytest.mark.parametrize("formats", [(0, 0), (1, 0)])
+def test_scaled_f8_block_streaming_kernel(ko, M, N, K, formats):
+    """17 .. 64 rows with K a multiple of 512: 32 columns x 32 / 48 / 64 rows per workgroup (row and column blocks that hang
+    over M and N included), both operand formats in the first slot; and the plain matmul with an f32 result through it."""
+    fa = (ko.F8E4M3, ko.F8E5M2)[formats[0]]
+    aq, sa, wq, sb = _quantised(ko, M, N, K, seed=7)
+    if formats[0]:      # the same values re-encoded as e5m2
+        aq = ko.fptofp(np.ascontiguousarray(ko.decode(aq, ko.F8E4M3).astype(np.float32)), ko.F32, ko.F8E5M2).reshape(M, K)
+    want = np.zeros((M, N), dtype=np.uint16)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, fa)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                        vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16))) == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N + 64, 2, fill=0x1234)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, fa), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    got = to_host(dd, np.uint16)
+    assert np.all(got[M * N:] == 0x1234)                      # nothing written past the result
+    assert _frob(ko, got[:M * N].reshape(M, N), want) <= FROB_TOL
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 128), (128, 256, 384), (256, 256, 256), (384, 128, 512), (512, 768, 1024), (1024, 2560, 256),
                                    (300, 520, 256), (1000, 136, 384), (129, 1001, 128), (300, 520, 272), (256, 256, 144)])   # tiles hang over the edges of M, N and K
 def test_scaled_f8_tiled_kernel(ko, M, N, K):

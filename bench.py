@@ -695,6 +695,18 @@ def bench_ceilings(kh, steps, warmup, cpu):
         out["copy"]["transpose footprint (128 rows x 256 B per workgroup)%s" % (", through LDS and a barrier" if lds else "")] = round(2 * nbytes / (ev * 1e-3) / 1e9, 0)
     out["copy_best_gbs"] = round(best, 0)
     out["copy_best_frac_of_peak"] = round(best / HBM_PEAK_GBS, 4)
+    # what the L2s hand to the CUs: every CU re-reads a window that stays in its XCD's L2 (2 MiB), that spills to the Infinity
+    # Cache (8 MiB per XCD) or to HBM (64 MiB per XCD), as LDS-direct loads (the tiled matmuls' form) or into registers
+    out["l2_read_tbs"] = {}
+    sink = torch.zeros(4096, dtype=torch.int32, device="cuda")
+    for window in (2 << 20, 8 << 20, 64 << 20):
+        buf = torch.empty(8 * window, dtype=torch.uint8, device="cuda")
+        buf.random_(0, 255)
+        for to_lds in (True, False):
+            _, nb = kh.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr())
+            wall, ev = _events(lambda i: kh.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr()), 10, 3)
+            out["l2_read_tbs"]["%d MiB per XCD, %s" % (window >> 20, "LDS-direct" if to_lds else "to registers")] = round(nb / (ev * 1e-3) / 1e12, 2)
+        del buf
     return out
 
 

@@ -183,6 +183,13 @@ int kapy_probe_mfma(int32_t impl_way, int32_t dtype, const void *operands, int32
 int kapy_probe_copy(const void *src, void *dst, int64_t bytes, int32_t vectors_per_lane, int32_t nt_load, int32_t nt_store, int32_t persistent_per_cu,
                     uint64_t *ticks, int32_t *workgroups, void *stream);
 
+/* kapy_probe_l2_read: every workgroup (workgroups_per_cu per CU, 256 lanes) reads the window of `src` that belongs to its XCD
+ * (src holds 8 windows of window_bytes, one per XCD; a window of a few MiB stays in that XCD's L2) `iterations` x 32 KiB, 16
+ * bytes per lane and instruction, as LDS-direct loads (to_lds = 1, the form the tiled matmul kernels use) or into registers.
+ * Outputs: the workgroups launched and the bytes the launch reads.  sink: one word per workgroup (never written in practice). */
+int kapy_probe_l2_read(const void *src, int64_t window_bytes, int32_t iterations, int32_t workgroups_per_cu, int32_t to_lds, uint32_t *sink,
+                       int32_t *workgroups, int64_t *bytes_read, void *stream);
+
 /* A copy with the access footprint of the 16-bit tile transpose (a workgroup moves 128 rows x 256 bytes of a [rows][row_bytes]
  * matrix, one wave instruction touches four 256-byte pieces of four rows), untransposed, directly or through an LDS tile and
  * a barrier: what that footprint and that detour cost against kapy_probe_copy. */

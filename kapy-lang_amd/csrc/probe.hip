@@ -9,7 +9,9 @@
 //   kapy_probe_copy   a 16-byte-per-lane copy in the forms a memory-bound kernel can take (vectors per lane, ordinary or
 //                     non-temporal loads and stores, one pass over a big grid or persistent workgroups striding over
 //                     the buffer): the rate a read + write stream reaches on this part.
-// Both record per-workgroup shader-clock and constant-rate timer ticks, from which the sustained clock follows.
+//   kapy_probe_l2_read  every CU reads a window that stays in its XCD's L2, over and over: the rate at which the L2s feed
+//                     the CUs, which is what a tiled matmul's global->LDS traffic runs against.
+// The first two record per-workgroup shader-clock and constant-rate timer ticks, from which the sustained clock follows.
 //
 // The reference has no counterpart: it emits code and never runs it (its matmul instruction strings:
 // lib/Conversion/KgpuToLLVM/MatmulOpToLLVM.cpp:269-311; its loads and stores: LdGlobalOpToLLVM.cpp:60-145).
@@ -161,6 +163,45 @@ int launch_copy(const void *src, void *dst, int64_t n, int persistent_per_cu, ui
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }
+// What the L2s hand to the CUs: every workgroup reads, over and over, the window of `src` that belongs to its XCD
+// (workgroup ids go to the 8 XCDs in turn; a window is sized to stay in that XCD's L2), 16 bytes per lane and instruction in
+// runs of 1 KiB per wave, up to 32 instructions per wave in flight - as LDS-direct loads into a ring nobody reads (the form the
+// tiled matmul kernels use) or into registers.  The workgroups of an XCD start a quarter of the window apart, so that at
+// any moment they ask for different lines, as the operand panels of neighbouring GEMM tiles are.
+template <bool TO_LDS>
+__global__ __launch_bounds__(256) void l2_read_kernel(const char *src, int64_t window, int iterations, uint32_t *sink) {
+  __shared__ __attribute__((aligned(1024))) char ring[4 * 32 * 1024];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t xcd = blockIdx.x % 8, on_xcd = blockIdx.x / 8;
+  const char *base = src + xcd * window;
+  const uint32_t chunks = (uint32_t)(window / 1024);  // 1 KiB runs in the window
+  uint32_t at = (uint32_t)((on_xcd * 4 + wave) * (chunks / 16) % chunks);
+  // (the halves go through unsigned variables: readfirstlane returns an int, and a low half with its top bit set would
+  // otherwise be sign-extended over the high half when the two are joined)
+  const uint64_t bv = (uint64_t)base;
+  const uint32_t base_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)bv), base_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(bv >> 32));
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)base_hi << 32) | (uint64_t)base_lo), 0, (int)window, 0x00020000);
+  u32x4 x = {0, 0, 0, 0};
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const uint32_t chunk = __builtin_amdgcn_readfirstlane(at + u < chunks ? at + u : at + u - chunks);
+      if (TO_LDS) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(ring + wave * 32768 + ((it & 3) * 8 + u) * 1024), 16, lane * 16,
+                                                 (int)(chunk * 1024), 0, 0);
+      } else {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, (int)(chunk * 1024), 0);
+        x ^= v;
+      }
+    }
+    at = at + 8 < chunks ? at + 8 : at + 8 - chunks;
+    if (TO_LDS) __builtin_amdgcn_s_waitcnt(0x0F70 | (24 & 15) | ((24 >> 4) << 14));  // vmcnt(24): four groups of eight in flight
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  if (sink && (x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[blockIdx.x] = x[0];  // keeps the register form's loads alive
+}
+
 template <int U>
 int launch_copy_nt(const void *src, void *dst, int64_t n, int nt_load, int nt_store, int persistent_per_cu, uint64_t *ticks, int32_t *workgroups, hipStream_t s) {
   if (nt_load && nt_store) return launch_copy<U, true, true>(src, dst, n, persistent_per_cu, ticks, workgroups, s);
@@ -201,6 +242,22 @@ int kapy_probe_mfma(int32_t impl_way, int32_t dtype, const void *operands, int32
   case KAPY_MFMA_16X16X128_F8: return dtype == KAPY_F8E4M3 ? launch_mfma_loop<F8M16<0, 0>>(operands, sink, iterations, ticks, wgs, s) : launch_mfma_loop<F8M16<1, 1>>(operands, sink, iterations, ticks, wgs, s);
   default: return dtype == KAPY_F8E4M3 ? launch_mfma_loop<F8<0, 0>>(operands, sink, iterations, ticks, wgs, s) : launch_mfma_loop<F8<1, 1>>(operands, sink, iterations, ticks, wgs, s);
   }
+}
+
+int kapy_probe_l2_read(const void *src, int64_t window_bytes, int32_t iterations, int32_t workgroups_per_cu, int32_t to_lds, uint32_t *sink,
+                       int32_t *workgroups, int64_t *bytes_read, void *stream) {
+  if (!src || window_bytes < 16384 || window_bytes % 16384 || window_bytes > (int64_t(1) << 30) || iterations <= 0 || workgroups_per_cu < 1 || workgroups_per_cu > 4 ||
+      ((uintptr_t)src & 1023))
+    return fail(KAPY_ERR_INVALID, "probe_l2_read: window must be a multiple of 16 KiB (at most 1 GiB), src 1 KiB aligned, 1 .. 4 workgroups per CU");
+  int rc = ensure_device();
+  if (rc) return rc;
+  const int wgs = device_cus() * workgroups_per_cu;
+  if (workgroups) *workgroups = wgs;
+  if (bytes_read) *bytes_read = (int64_t)wgs * 4 * iterations * 8 * 1024;
+  if (to_lds) l2_read_kernel<true><<<wgs, 256, 0, (hipStream_t)stream>>>((const char *)src, window_bytes, iterations, sink);
+  else l2_read_kernel<false><<<wgs, 256, 0, (hipStream_t)stream>>>((const char *)src, window_bytes, iterations, sink);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
 }
 
 int kapy_probe_copy_tiled(const void *src, void *dst, int64_t rows, int64_t row_bytes, int32_t through_lds, void *stream) {

@@ -254,6 +254,10 @@ typedef enum kapy_ew_op {
   KAPY_EW_REDUCE_SUM,    /* dst <- sum of a along axis b, kept on every element of that axis: kapy.reduce  */
   KAPY_EW_REDUCE_MAX,    /*        with an addf / maximumf combiner followed by kapy.broadcast; accumulated */
                          /*        in fp32, rounded once to the register's type (as kapy_reduce)           */
+  KAPY_EW_FLOOR, KAPY_EW_CEIL, /* math.floor / math.ceil (create_floor, create_ceil; UnaryOpConversion, ElementwiseOpToLLVM.cpp:1222-1223) */
+  KAPY_EW_SIN, KAPY_EW_COS,    /* math.sin / math.cos (create_sin, create_cos; :1224-1225)                          */
+  KAPY_EW_MAXNUMF, KAPY_EW_MINNUMF, /* arith.maxnumf / minnumf: a NaN operand is ignored (create_maxnumf, create_minnumf; :1201-1206) */
+  KAPY_EW_REMF,          /* arith.remf: the remainder of a / b with the sign of a, exact (create_remf; :1192)   */
   KAPY_EW_NUM_OPS
 } kapy_ew_op;
 typedef struct kapy_ew_inst {

@@ -165,6 +165,9 @@ class OpBuilder {
   Value create_divf(Value lhs, Value rhs) { return binary(KAPY_EW_DIVF, lhs, rhs); }
   Value create_maximumf(Value lhs, Value rhs) { return binary(KAPY_EW_MAXIMUMF, lhs, rhs); }
   Value create_minimumf(Value lhs, Value rhs) { return binary(KAPY_EW_MINIMUMF, lhs, rhs); }
+  Value create_maxnumf(Value lhs, Value rhs) { return binary(KAPY_EW_MAXNUMF, lhs, rhs); }
+  Value create_minnumf(Value lhs, Value rhs) { return binary(KAPY_EW_MINNUMF, lhs, rhs); }
+  Value create_remf(Value lhs, Value rhs) { return binary(KAPY_EW_REMF, lhs, rhs); }
   // kapy.clampf(source, low, high, propagateNan) (ir.cc:886-890): min(max(source, low), high); maximumf / minimumf propagate NaNs,
   // the only form the elementwise programs have
   Value create_clampf(Value source, Value low, Value high, bool propagate_nan = true) {
@@ -190,6 +193,10 @@ class OpBuilder {
   Value create_sqrt(Value source) { return unary(KAPY_EW_SQRT, source); }
   Value create_rsqrt(Value source) { return unary(KAPY_EW_RSQRT, source); }
   Value create_erf(Value source) { return unary(KAPY_EW_ERF, source); }
+  Value create_floor(Value source) { return unary(KAPY_EW_FLOOR, source); }
+  Value create_ceil(Value source) { return unary(KAPY_EW_CEIL, source); }
+  Value create_sin(Value source) { return unary(KAPY_EW_SIN, source); }
+  Value create_cos(Value source) { return unary(KAPY_EW_COS, source); }
   // create_elementwise_extern_lib (ir.cc:1168-1174): the library functions the path uses, by name
   Value create_elementwise_extern_lib(const std::string &name, Value source) {
     if (name == "tanh") return unary(KAPY_EW_TANH, source);

@@ -8,6 +8,11 @@
 
 #include "../../include/kapy_hip.h"
 
+// the case labels of every op with two register operands
+#define KAPY_EW_BINARY_CASES                                                                                                          \
+  case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF: case KAPY_EW_MAXNUMF:  \
+  case KAPY_EW_MINNUMF: case KAPY_EW_REMF
+
 namespace kapy {
 
 // Thread-local text of the last failure; the counterpart of the reference's emitOpError

@@ -92,6 +92,9 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
       case KAPY_EW_FMA: r = fma_typed(a, regs[I.b][tid], regs[I.c][tid], dt); break;
       case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
       case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
+      case KAPY_EW_MAXNUMF: r = max_num(a, regs[I.b][tid]); break;
+      case KAPY_EW_MINNUMF: r = min_num(a, regs[I.b][tid]); break;
+      case KAPY_EW_REMF: r = rem_f(a, regs[I.b][tid]); break;
       default: r = apply_unary(I.op, a);
       }
       if (dt != KAPY_F32) r = round_to_dtype(r, dt, true);
@@ -162,6 +165,9 @@ __global__ __launch_bounds__(WAVES * 64) void column_program_kernel(Program P, C
           case KAPY_EW_FMA: r = fma_typed(a, regs[I.b][tid], regs[I.c][tid], dt); break;
           case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
           case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
+          case KAPY_EW_MAXNUMF: r = max_num(a, regs[I.b][tid]); break;
+          case KAPY_EW_MINNUMF: r = min_num(a, regs[I.b][tid]); break;
+          case KAPY_EW_REMF: r = rem_f(a, regs[I.b][tid]); break;
           default: r = apply_unary(I.op, a);
           }
           if (dt != KAPY_F32) r = round_to_dtype(r, dt, true);
@@ -431,7 +437,7 @@ int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *cons
         return fail(KAPY_ERR_VERIFY, "elementwise: operands must have the same element type at %d", k);
       reg_dtype[I.dst] = reg_dtype[I.a];
       break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       if (!reg_ok(I.a) || !reg_ok(I.b)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
       if (reg_dtype[I.a] != reg_dtype[I.b])
         return fail(KAPY_ERR_VERIFY, "elementwise: operands must have the same element type at %d", k);
@@ -483,7 +489,7 @@ bool match_affine_act(const kapy_ew_inst *prog, int n_inst, const kapy_global *c
     case KAPY_EW_FPTOFP: n.a = reg[I.a]; n.dtype = I.dtype; n.rmode = I.rmode; break;
     case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; ++n_store; continue;
     case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       n.a = reg[I.a]; n.b = reg[I.b]; break;
     default: n.a = reg[I.a];
     }
@@ -620,7 +626,7 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     case KAPY_EW_SPLAT: break;
     case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; ++n_store; continue;
     case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       n.a = reg[I.a]; n.b = reg[I.b]; break;
     default: n.a = reg[I.a];
     }
@@ -721,8 +727,8 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
       if (n.dtype != KAPY_F32 && !(id == stored && n.dtype == out->dtype && n.rmode != KAPY_RZ)) push(kCast, 0, n.dtype, n.rmode, d, 0.f);
       return;
     case KAPY_EW_FMA: emit(n.a, d); emit(n.b, d + 1); emit(n.c, d + 2); push(KAPY_EW_FMA, 0, n.dtype, 0, d, 0.f); return;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF: {
-      const bool a_first = std::max(need[n.a], need[n.b] + 1) <= std::max(need[n.b], need[n.a] + 1);
+    KAPY_EW_BINARY_CASES: {
+      const bool a_first = n.op == KAPY_EW_REMF || std::max(need[n.a], need[n.b] + 1) <= std::max(need[n.b], need[n.a] + 1);  // (remf has no reversed form)
       if (a_first) { emit(n.a, d); emit(n.b, d + 1); push(n.op, 0, n.dtype, 0, d, 0.f); }
       else {
         emit(n.b, d); emit(n.a, d + 1);
@@ -797,7 +803,7 @@ int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
     switch (I.op) {
     case KAPY_EW_LD_GLOBAL: case KAPY_EW_SPLAT: break;
     case KAPY_EW_FMA: d |= def_of[I.a] | def_of[I.b] | def_of[I.c]; break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       d |= def_of[I.a] | def_of[I.b];
       break;
     case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX:

@@ -278,7 +278,8 @@ std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig)
     kapy_ew_inst I = prog[k];  // fields an op does not read must not tell two equal programs apart
     const int op = I.op;
     const bool unary_or_cast = !(op == KAPY_EW_LD_GLOBAL || op == KAPY_EW_SPLAT || op == KAPY_EW_FMA || op == KAPY_EW_ADDF || op == KAPY_EW_SUBF ||
-                                 op == KAPY_EW_MULF || op == KAPY_EW_DIVF || op == KAPY_EW_MAXIMUMF || op == KAPY_EW_MINIMUMF);
+                                 op == KAPY_EW_MULF || op == KAPY_EW_DIVF || op == KAPY_EW_MAXIMUMF || op == KAPY_EW_MINIMUMF || op == KAPY_EW_MAXNUMF ||
+                                 op == KAPY_EW_MINNUMF || op == KAPY_EW_REMF);
     if (op == KAPY_EW_SPLAT) I.a = I.b = I.c = 0;
     else I.imm = 0.f;
     if (op == KAPY_EW_LD_GLOBAL) I.b = 0;
@@ -341,7 +342,7 @@ std::vector<Node> build_nodes(const kapy_ew_inst *prog, int n_inst, const int *r
     case KAPY_EW_SPLAT: break;
     case KAPY_EW_ST_GLOBAL: *stored = reg[I.a]; continue;
     case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       n.a = reg[I.a]; n.b = reg[I.b]; break;
     default: n.a = reg[I.a];
     }
@@ -496,6 +497,9 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
     case KAPY_EW_MULF: per_element("__fmul_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
     case KAPY_EW_MAXIMUMF: per_element("max_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
     case KAPY_EW_MINIMUMF: per_element("min_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MAXNUMF: per_element("max_num(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MINNUMF: per_element("min_num(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_REMF: per_element("rem_f(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
     case KAPY_EW_FMA: per_element("fma_typed(" + elem(n.a) + ", " + elem(n.b) + ", " + elem(n.c) + ", " + std::to_string(n.dtype) + ")"); round_result(); break;
     case KAPY_EW_DIVF: {
       const std::string a = as_array(n.a), b = as_array(n.b);
@@ -633,6 +637,9 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
     case KAPY_EW_MULF: assign("__fmul_rn(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
     case KAPY_EW_MAXIMUMF: assign("max_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
     case KAPY_EW_MINIMUMF: assign("min_nan(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MAXNUMF: assign("max_num(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_MINNUMF: assign("min_num(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
+    case KAPY_EW_REMF: assign("rem_f(" + elem(n.a) + ", " + elem(n.b) + ")"); round_result(); break;
     case KAPY_EW_FMA: assign("fma_typed(" + elem(n.a) + ", " + elem(n.b) + ", " + elem(n.c) + ", " + dt + ")"); round_result(); break;
     case KAPY_EW_DIVF:
       if (n.uniform) assign("__fdiv_rn(" + elem(n.a) + ", " + elem(n.b) + ")");

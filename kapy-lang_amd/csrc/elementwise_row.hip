@@ -312,7 +312,7 @@ struct RowBuilder {
       emit_uni(n.a, d, k); emit_uni(n.b, d, k + 1); emit_uni(n.c, d, k + 2);
       push(KAPY_EW_FMA, 0, n.dtype, 0, 0, 0.f, kUniformResult, k);
       break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       emit_uni(n.a, d, k); emit_uni(n.b, d, k + 1);
       push(n.op, 0, n.dtype, 0, 0, 0.f, kUniformResult, k);
       break;
@@ -360,7 +360,7 @@ struct RowBuilder {
       emit_full(n.a, d, k); emit_full(n.b, d + 1, k); emit_full(n.c, d + 2, k);
       push(KAPY_EW_FMA, 0, n.dtype, 0, d, 0.f);
       break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
       if (n.a == n.b) {
         emit_full(n.a, d, k);
         push(n.op, 0, n.dtype, 0, d, 0.f, kSameOperand);
@@ -530,7 +530,8 @@ int run_row_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtyp
     case KAPY_EW_SPLAT: break;
     case KAPY_EW_ST_GLOBAL: B.stored = reg[I.a]; ++n_store; continue;
     case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
-    case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF:
+    KAPY_EW_BINARY_CASES:
+      if (I.op == KAPY_EW_REMF) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: remf in a program with a reduce along rows is served by a compiled kernel only");
       n.a = reg[I.a]; n.b = reg[I.b]; break;
     case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX:
       if (I.b != 1) return fail(KAPY_ERR_UNSUPPORTED, "%s", why);

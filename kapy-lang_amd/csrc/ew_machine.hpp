@@ -65,6 +65,10 @@ __device__ __forceinline__ float apply_unary(int op, float a) {
   case KAPY_EW_TANH: return tanhf(a);
   case KAPY_EW_ERF: return erff(a);
   case KAPY_EW_GELU_TANH: return gelu_tanh_f32(a);
+  case KAPY_EW_FLOOR: return floorf(a);
+  case KAPY_EW_CEIL: return ceilf(a);
+  case KAPY_EW_SIN: return sinf(a);
+  case KAPY_EW_COS: return cosf(a);
   }
   return a;
 }
@@ -72,6 +76,11 @@ __device__ __forceinline__ float apply_unary(int op, float a) {
 // arith.maximumf / minimumf: NaN if either operand is NaN.
 __device__ __forceinline__ float max_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
 __device__ __forceinline__ float min_nan(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+// arith.maxnumf / minnumf: a NaN operand is ignored (NaN only if both are); -0 orders below +0 as above.
+__device__ __forceinline__ float max_num(float a, float b) { return a != a ? b : b != b ? a : fmaxf(a, b); }
+__device__ __forceinline__ float min_num(float a, float b) { return a != a ? b : b != b ? a : fminf(a, b); }
+// arith.remf: a - trunc(a / b) * b computed exactly, sign of a (the frem the reference's BinaryOpConversion emits)
+__device__ __forceinline__ float rem_f(float a, float b) { return fmodf(a, b); }
 
 // ---------------------------------------------------------------------------------------------
 // Stack machine: any program whose expression tree needs at most three live values, on 8
@@ -232,7 +241,8 @@ __device__ __forceinline__ void div8(const float (&x)[8], const float (&y)[8], f
       const float r1 = __builtin_fmaf(__builtin_fmaf(-y[e], r0, 1.0f), r0, r0);
       const float q0 = x[e] * r1;
       const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, y[e], x[e]), r1, q0);
-      q[e] = __builtin_fmaf(__builtin_fmaf(-q1, y[e], x[e]), r1, q1);  // the second correction: without it one quotient in ~10^5 is an ulp off
+      const float q2 = __builtin_fmaf(__builtin_fmaf(-q1, y[e], x[e]), r1, q1);  // the second correction: without it one quotient in ~10^5 is an ulp off
+      q[e] = x[e] == 0.f ? q0 : q2;  // a zero dividend: the corrections add a +0 remainder, which would turn a -0 quotient into +0
     }
   } else {
 #pragma unroll
@@ -337,6 +347,18 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
   case KAPY_EW_MINIMUMF:
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = min_nan(x[e], y[e]);
+    break;
+  case KAPY_EW_MAXNUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = max_num(x[e], y[e]);
+    break;
+  case KAPY_EW_MINNUMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = min_num(x[e], y[e]);
+    break;
+  case KAPY_EW_REMF:
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = rem_f(x[e], y[e]);
     break;
   case KAPY_EW_FMA:
 #pragma unroll

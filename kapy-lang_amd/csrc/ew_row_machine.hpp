@@ -53,6 +53,8 @@ __device__ __forceinline__ float scalar_step(const StackProgram &P, const PostOp
   case kRevDiv: r = __fdiv_rn(y, x); break;
   case KAPY_EW_MAXIMUMF: r = max_nan(x, y); break;
   case KAPY_EW_MINIMUMF: r = min_nan(x, y); break;
+  case KAPY_EW_MAXNUMF: r = max_num(x, y); break;
+  case KAPY_EW_MINNUMF: r = min_num(x, y); break;
   case KAPY_EW_FMA: r = fma_typed(x, y, z, I.dtype); break;
   default: r = apply_unary(I.op, x);
   }
@@ -225,7 +227,7 @@ __device__ __forceinline__ void row_step(const StackProgram &P, const PostOp &I,
         const float q = x * rcp;
         const float rem = __builtin_fmaf(-q, y, x);
         const float q2 = __builtin_fmaf(rem, rcp, q);
-        v[c][D][e] = rem == rem ? q2 : q;
+        v[c][D][e] = (rem == rem && rem != 0.f) ? q2 : q;  // (a zero remainder: q is exact already, and adding +0 would turn a -0 quotient into +0)
       }
       if (I.dtype != KAPY_F32) round8<NARROW>(v[c][D], I.dtype, true);
     }

@@ -990,11 +990,15 @@ struct Interp {
     if (n == "arith.divf") return binary_tensor(op, KAPY_EW_DIVF);
     if (n == "arith.maximumf") return binary_tensor(op, KAPY_EW_MAXIMUMF);
     if (n == "arith.minimumf") return binary_tensor(op, KAPY_EW_MINIMUMF);
+    if (n == "arith.maxnumf") return binary_tensor(op, KAPY_EW_MAXNUMF);
+    if (n == "arith.minnumf") return binary_tensor(op, KAPY_EW_MINNUMF);
+    if (n == "arith.remf") return binary_tensor(op, KAPY_EW_REMF);
     {
       static const struct { const char *name; int ew; } unary[] = {
           {"math.exp", KAPY_EW_EXP}, {"math.exp2", KAPY_EW_EXP2}, {"math.log", KAPY_EW_LOG}, {"math.log2", KAPY_EW_LOG2},
           {"math.sqrt", KAPY_EW_SQRT}, {"math.rsqrt", KAPY_EW_RSQRT}, {"math.tanh", KAPY_EW_TANH}, {"math.erf", KAPY_EW_ERF},
-          {"math.absf", KAPY_EW_ABSF}, {"arith.negf", KAPY_EW_NEGF}};
+          {"math.absf", KAPY_EW_ABSF}, {"arith.negf", KAPY_EW_NEGF}, {"math.floor", KAPY_EW_FLOOR}, {"math.ceil", KAPY_EW_CEIL},
+          {"math.sin", KAPY_EW_SIN}, {"math.cos", KAPY_EW_COS}};
       for (auto &u : unary)
         if (n == u.name) return mapped_tensor(op, 1, u.ew);
     }
@@ -1197,11 +1201,11 @@ const struct OpForm { const char *name; int min_operands, results; } kSupportedO
     {"kapy.return", 0, 0}, {"scf.yield", 0, 0}, {"scf.for", 3, -1}, {"arith.constant", 0, 1}, {"kapy.program_id", 0, 1}, {"kapy.warp_id", 0, 1},
     {"arith.addi", 2, 1}, {"arith.subi", 2, 1}, {"arith.muli", 2, 1}, {"arith.divui", 2, 1}, {"arith.remui", 2, 1}, {"arith.cmpi", 2, 1},
     {"arith.select", 3, 1}, {"arith.addf", 2, 1}, {"arith.subf", 2, 1}, {"arith.mulf", 2, 1}, {"arith.divf", 2, 1}, {"arith.maximumf", 2, 1},
-    {"arith.minimumf", 2, 1}, {"kapy.mk_global", 6, 1}, {"kapy.mk_shared", 0, 1}, {"kapy.sv_global", 5, 1}, {"kapy.sv_shared", 5, 1},
+    {"arith.minimumf", 2, 1}, {"arith.maxnumf", 2, 1}, {"arith.minnumf", 2, 1}, {"arith.remf", 2, 1}, {"kapy.mk_global", 6, 1}, {"kapy.mk_shared", 0, 1}, {"kapy.sv_global", 5, 1}, {"kapy.sv_shared", 5, 1},
     {"kapy.ld_global", 1, 1}, {"kapy.ld_matrix", 1, 1}, {"kapy.ld_shared", 1, 1}, {"kapy.st_global", 2, 0}, {"kapy.st_shared", 2, 0},
     {"kapy.cp_async_global_to_shared", 2, 0}, {"kapy.cp_async_wait_group", 0, 0}, {"kapy.matmul", 3, 1}, {"kapy.reduce", 1, 1},
     {"nvvm.barrier0", 0, 0}, {"math.exp", 1, 1}, {"math.exp2", 1, 1}, {"math.log", 1, 1}, {"math.log2", 1, 1}, {"math.sqrt", 1, 1},
-    {"math.rsqrt", 1, 1}, {"math.tanh", 1, 1}, {"math.erf", 1, 1}, {"math.absf", 1, 1}, {"math.fma", 3, 1}, {"arith.negf", 1, 1},
+    {"math.rsqrt", 1, 1}, {"math.tanh", 1, 1}, {"math.erf", 1, 1}, {"math.absf", 1, 1}, {"math.floor", 1, 1}, {"math.ceil", 1, 1}, {"math.sin", 1, 1}, {"math.cos", 1, 1}, {"math.fma", 3, 1}, {"arith.negf", 1, 1},
     {"arith.extf", 1, 1}, {"arith.truncf", 1, 1}, {"kapy.fptofp", 1, 1}, {"kapy.splat", 1, 1}, {"kapy.broadcast", 1, 1}, {"kapy.transpose", 1, 1}};
 
 // Every op must be one this front-end executes, written with the operands and results it needs; returns the number of ops,

@@ -23,7 +23,7 @@ DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, F8E4M3: 1, F8E5M2: 1, I8: 1, I16: 2, I32
 
 (EW_LD_GLOBAL, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
  EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH,
- EW_ST_GLOBAL, EW_REDUCE_SUM, EW_REDUCE_MAX) = range(24)
+ EW_ST_GLOBAL, EW_REDUCE_SUM, EW_REDUCE_MAX, EW_FLOOR, EW_CEIL, EW_SIN, EW_COS, EW_MAXNUMF, EW_MINNUMF, EW_REMF) = range(31)
 
 EXPORTS = [
     "kapy_version", "kapy_last_error", "kapy_device_info", "kapy_mk_global", "kapy_sv_global",

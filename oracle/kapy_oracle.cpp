@@ -584,7 +584,7 @@ int ko_copy_batched(const ko_global *src, const ko_global *dst, int transpose, i
 enum {
   EW_LD_GLOBAL = 0, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
   EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH, EW_ST_GLOBAL,
-  EW_REDUCE_SUM, EW_REDUCE_MAX,
+  EW_REDUCE_SUM, EW_REDUCE_MAX, EW_FLOOR, EW_CEIL, EW_SIN, EW_COS, EW_MAXNUMF, EW_MINNUMF, EW_REMF,
   EW_NUM_OPS
 };
 enum { EW_MAX_REGS = 16 };
@@ -647,7 +647,7 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
       if (reg_dtype[I.a] != reg_dtype[I.b] || reg_dtype[I.a] != reg_dtype[I.c]) return -10;
       reg_dtype[I.dst] = reg_dtype[I.a];
       break;
-    case EW_ADDF: case EW_SUBF: case EW_MULF: case EW_DIVF: case EW_MAXIMUMF: case EW_MINIMUMF:
+    case EW_ADDF: case EW_SUBF: case EW_MULF: case EW_DIVF: case EW_MAXIMUMF: case EW_MINIMUMF: case EW_MAXNUMF: case EW_MINNUMF: case EW_REMF:
       if (!reg_ok(I.a) || !reg_ok(I.b)) return -6;
       if (reg_dtype[I.a] != reg_dtype[I.b]) return -10;
       reg_dtype[I.dst] = reg_dtype[I.a];
@@ -760,6 +760,17 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
           r = (std::isnan(a) || std::isnan(b)) ? qnan : a == b ? (std::signbit(a) ? a : b) : std::min(a, b);
           break;
         }
+        case EW_MAXNUMF: {  // arith.maxnumf / minnumf: a NaN operand is ignored; -0 below +0 (BinaryOpConversion, ElementwiseOpToLLVM.cpp:1201-1206)
+          const double b = reg[I.b][at];
+          r = std::isnan(a) ? b : std::isnan(b) ? a : a == b ? (std::signbit(a) ? b : a) : std::max(a, b);
+          break;
+        }
+        case EW_MINNUMF: {
+          const double b = reg[I.b][at];
+          r = std::isnan(a) ? b : std::isnan(b) ? a : a == b ? (std::signbit(a) ? a : b) : std::min(a, b);
+          break;
+        }
+        case EW_REMF: r = std::fmod(a, reg[I.b][at]); break;  // arith.remf (frem): exact, sign of the dividend (:1192)
         case EW_NEGF: r = -a; break;
         case EW_ABSF: r = std::fabs(a); break;
         case EW_EXP: r = std::exp(a); break;
@@ -771,6 +782,10 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
         case EW_TANH: r = std::tanh(a); break;
         case EW_ERF: r = std::erf(a); break;
         case EW_GELU_TANH: r = gelu_tanh(a); break;
+        case EW_FLOOR: r = std::floor(a); break;  // math.floor / ceil / sin / cos: UnaryOpConversion, ElementwiseOpToLLVM.cpp:1222-1225
+        case EW_CEIL: r = std::ceil(a); break;
+        case EW_SIN: r = std::sin(a); break;
+        case EW_COS: r = std::cos(a); break;
         case EW_ST_GLOBAL:
           if (in_bounds(out, i, j)) ko_encode(out->ptr, out->dtype, elem_offset(out, i, j), a, KO_RN);
           continue;

@@ -20,7 +20,7 @@ NP_STORAGE = {F16: np.uint16, BF16: np.uint16, F32: np.float32, F8E4M3: np.uint8
 
 (EW_LD_GLOBAL, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
  EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH,
- EW_ST_GLOBAL, EW_REDUCE_SUM, EW_REDUCE_MAX) = range(24)
+ EW_ST_GLOBAL, EW_REDUCE_SUM, EW_REDUCE_MAX, EW_FLOOR, EW_CEIL, EW_SIN, EW_COS, EW_MAXNUMF, EW_MINNUMF, EW_REMF) = range(31)
 
 
 class Global(C.Structure):

@@ -467,3 +467,79 @@ def test_reduces_along_both_axes_in_one_program_are_refused(ko):
     with pytest.raises(kh.KapyError) as e:
         kh.elementwise(kh.program(five), [dglobal(x, m, n, n, 1, kh.F16)], dglobal(dev_zeros(m * n, 2), m, n, n, 1, kh.F16))
     assert e.value.status == -3 and "at most 4" in e.value.message
+
+
+# ---------------------------------------------------------------------------------------------------------
+# The ops of the reference's elementwise list beyond the arithmetic ones: floor, ceil, sin, cos, maxnumf, minnumf, remf.
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16, kh.F32])
+def test_floor_ceil_maxnum_minnum_rem_are_exact(ko, dtype):
+    m, n = 24, 200
+    x = ko.fill_normal(m * n, dtype, 201, 0, 0.0, 6.0).reshape(m, n)
+    y = ko.fill_normal(m * n, dtype, 201, 1, 0.0, 2.0).reshape(m, n)
+    specials = {kh.F16: [0x7e00, 0x3c00, 0x8000, 0x0000, 0x7c00, 0xfc00, 0x4580, 0xc580], kh.BF16: [0x7fc0, 0x3f80, 0x8000, 0x0000, 0x7f80, 0xff80, 0x40b0, 0xc0b0]}
+    others = {kh.F16: [0x4000, 0x7e00, 0x0000, 0x8000, 0x4200, 0x3800, 0x4000, 0x4000], kh.BF16: [0x4000, 0x7fc0, 0x0000, 0x8000, 0x4040, 0x3f00, 0x4000, 0x4000]}
+    if dtype != kh.F32:
+        x.ravel()[:8] = specials[dtype]
+        y.ravel()[:8] = others[dtype]
+    else:
+        x.ravel()[:8] = [np.nan, 1.0, -0.0, 0.0, np.inf, -np.inf, 5.5, -5.5]
+        y.ravel()[:8] = [2.0, np.nan, 0.0, -0.0, 3.0, 0.5, 2.0, 2.0]
+    L0, L1 = dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1)
+    for op in (kh.EW_FLOOR, kh.EW_CEIL):
+        got, want = _run_prog(ko, [L0, dict(op=op, dst=2, a=0), dict(op=kh.EW_ST_GLOBAL, a=2)], [x], [dtype], dtype, m, n)
+        assert _same_bits_or_nan(got, want, dtype), op
+    for op in (kh.EW_MAXNUMF, kh.EW_MINNUMF, kh.EW_REMF):
+        got, want = _run_prog(ko, [L0, L1, dict(op=op, dst=2, a=0, b=1), dict(op=kh.EW_ST_GLOBAL, a=2)], [x, y], [dtype, dtype], dtype, m, n)
+        assert _same_bits_or_nan(got, want, dtype), op
+
+
+def _same_bits_or_nan(got, want, dtype):
+    if dtype == kh.F32:
+        g, w = got.view(np.float32), want.view(np.float32)
+        nan = np.isnan(w)
+        return np.array_equal(np.isnan(g), nan) and np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    nan = np.isnan(_as_f64(want, dtype))
+    return np.array_equal(np.isnan(_as_f64(got, dtype)), nan) and np.array_equal(got[~nan], want[~nan])
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+def test_sin_cos_within_two_ulp(ko, dtype):
+    m, n = 32, 256
+    x = ko.fill_normal(m * n, dtype, 211, 0, 0.0, 4.0).reshape(m, n)
+    for op in (kh.EW_SIN, kh.EW_COS):
+        insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_FPTOFP, dst=1, a=0, dtype=kh.F32), dict(op=op, dst=1, a=1),
+                 dict(op=kh.EW_FPTOFP, dst=2, a=1, dtype=dtype, rmode=kh.RN), dict(op=kh.EW_ST_GLOBAL, a=2)]
+        got, want = _run_prog(ko, insts, [x], [dtype], dtype, m, n)
+        _check_ulp(got, want, dtype)
+
+
+def test_division_keeps_the_sign_of_a_zero_dividend(ko):
+    """-0 / y is -0 for y > 0: the lean division corrects its quotient by the remainder, and adding a +0 remainder would
+    lose the sign.  Through the stack machine, the row machine (division by a per-row value) and a compiled kernel."""
+    m, n = 16, 128
+    x = ko.fill_normal(m * n, kh.F32, 221, 0, 0.0, 1.0).reshape(m, n)
+    x[:, ::3] = -0.0
+    x[:, 1::7] = 0.0
+    y = np.abs(ko.fill_normal(m * n, kh.F32, 221, 1, 0.0, 1.0)).reshape(m, n) + np.float32(0.5)
+    L0, L1, ST = dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1), dict(op=kh.EW_ST_GLOBAL, a=2)
+    insts = [L0, L1, dict(op=kh.EW_DIVF, dst=2, a=0, b=1), ST]
+    got, want = _run_prog(ko, insts, [x, y], [kh.F32, kh.F32], kh.F32, m, n)
+    assert np.array_equal(got, want) and np.array_equal(np.signbit(got.view(np.float32)), np.signbit(x / y))
+    # x / rowmax(y): the row machine's division of a row by one value
+    insts = [L0, L1, dict(op=kh.EW_REDUCE_MAX, dst=1, a=1, b=1), dict(op=kh.EW_DIVF, dst=2, a=0, b=1), ST]
+    got, want = _run_prog(ko, insts, [x, y], [kh.F32, kh.F32], kh.F32, m, n)
+    assert np.array_equal(np.signbit(got.view(np.float32)), np.signbit(want.view(np.float32)))
+    assert np.max(np.abs(got.view(np.float32) - want.view(np.float32))) <= 1e-6
+    # compiled
+    insts = [L0, L1, dict(op=kh.EW_DIVF, dst=2, a=0, b=1), dict(op=kh.EW_NEGF, dst=2, a=2), dict(op=kh.EW_NEGF, dst=2, a=2), ST]
+    dx, dy, dz = to_dev(x), to_dev(y), dev_zeros(m * n, 4)
+    g = lambda t: dglobal(t, m, n, n, 1, kh.F32)
+    try:
+        kh.elementwise_specialize(kh.program(insts), [g(dx), g(dy)], g(dz))
+    except kh.KapyError as e:
+        assert e.status == kh.ERR_UNSUPPORTED      # no runtime compiler on this machine
+        return
+    kh.elementwise(kh.program(insts), [g(dx), g(dy)], g(dz))
+    sync()
+    out = to_host(dz, np.float32, (m, n))
+    assert np.array_equal(out, x / y) and np.array_equal(np.signbit(out), np.signbit(x / y))

@@ -12,8 +12,8 @@ from gpu_util import dev_zeros, sync, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
-BINARY = ["arith.addf", "arith.subf", "arith.mulf", "arith.maximumf", "arith.minimumf"]
-UNARY = ["arith.negf", "math.absf", "math.tanh", "math.tanh", "math.erf"]       # bounded, so that long chains stay finite
+BINARY = ["arith.addf", "arith.subf", "arith.mulf", "arith.maximumf", "arith.minimumf", "arith.maxnumf", "arith.minnumf"]
+UNARY = ["arith.negf", "math.absf", "math.tanh", "math.tanh", "math.erf", "math.sin", "math.cos", "math.floor", "math.ceil"]   # bounded, so that long chains stay finite
 
 
 def random_program(rng, rows_per_warp, cols, warps):

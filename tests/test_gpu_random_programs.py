@@ -1,4 +1,4 @@
-"""Seeded random elementwise programs built from exactly rounded ops only (add, sub, mul, div, max, min, fma, neg, abs, sqrt and
+"""Seeded random elementwise programs built from exactly rounded ops only (add, sub, mul, div, rem, max, min, maxnum, minnum, fma, neg, abs, sqrt, floor, ceil and
 casts between every float type), over random operand kinds (full, column-major, row, column, scalar) and shapes: the machines
 and the compiled kernels must both reproduce the oracle bit for bit (NaNs compared as NaNs)."""
 import numpy as np
@@ -27,8 +27,8 @@ def _random_case(rng):
             insts.append(dict(op=CAST, dst=r, a=r, dtype=compute, rmode=kh.RN if rng.randint(2) or (in_dtypes[k] == kh.BF16 and False) else kh.RZ))
         regs.append(r)
         r += 1
-    binary = [kh.EW_ADDF, kh.EW_SUBF, kh.EW_MULF, kh.EW_DIVF, kh.EW_MAXIMUMF, kh.EW_MINIMUMF]
-    unary = [kh.EW_NEGF, kh.EW_ABSF, kh.EW_SQRT]
+    binary = [kh.EW_ADDF, kh.EW_SUBF, kh.EW_MULF, kh.EW_DIVF, kh.EW_MAXIMUMF, kh.EW_MINIMUMF, kh.EW_MAXNUMF, kh.EW_MINNUMF, kh.EW_REMF]
+    unary = [kh.EW_NEGF, kh.EW_ABSF, kh.EW_SQRT, kh.EW_FLOOR, kh.EW_CEIL]
     for _ in range(2 + rng.randint(7)):
         pick = lambda: regs[rng.randint(len(regs))]
         kind = rng.randint(10)

@@ -324,3 +324,42 @@ def test_f32_fma_rounds_once(ko):
         exact = Fraction(float(aa[k])) * Fraction(float(bb[k])) + Fraction(float(cc[k]))
         lo, hi = np.nextafter(out[k], np.float32(-np.inf)), np.nextafter(out[k], np.float32(np.inf))
         assert abs(Fraction(float(out[k])) - exact) <= min(abs(Fraction(float(lo)) - exact), abs(Fraction(float(hi)) - exact))
+
+
+def test_floor_ceil_sin_cos_maxnum_minnum_rem_vs_numpy(ko):
+    """The ops of the reference's elementwise list beyond the arithmetic ones (ElementwiseOpToLLVM.cpp:1192-1225): against numpy
+    in float64 rounded once to the register type; maxnumf / minnumf ignore a NaN operand and order -0 below +0; remf is exact
+    and keeps the dividend's sign."""
+    import kapy_hip as kh
+    m, n = 8, 96
+    x = ko.fill_normal(m * n, ko.F32, 31, 0, 0.0, 6.0).reshape(m, n)
+    y = ko.fill_normal(m * n, ko.F32, 31, 1, 0.0, 2.0).reshape(m, n)
+    x[0, :6] = [np.nan, 1.0, -0.0, 0.0, np.inf, -np.inf]
+    y[0, :6] = [2.0, np.nan, 0.0, -0.0, 3.0, 0.5]
+    x[1, :4] = [5.5, -5.5, 7.0, 1.0]
+    y[1, :4] = [2.0, 2.0, 0.0, np.inf]
+    out = np.zeros((m, n), np.float32)
+    g = lambda a: ko.mk_global(a, m, n, n, 1, ko.F32)
+    L, ST = dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_ST_GLOBAL, a=2)
+    with np.errstate(invalid="ignore"):
+        for op, ref in ((ko.EW_FLOOR, np.floor), (ko.EW_CEIL, np.ceil), (ko.EW_SIN, np.sin), (ko.EW_COS, np.cos)):
+            assert ko.elementwise(ko.program([L, dict(op=op, dst=2, a=0), ST]), [g(x)], g(out)) == 0
+            want = ref(x.astype(np.float64)).astype(np.float32)
+            assert np.array_equal(np.isnan(out), np.isnan(want)) and np.array_equal(out[~np.isnan(want)], want[~np.isnan(want)]), op
+        L1 = dict(op=ko.EW_LD_GLOBAL, dst=1, a=1)
+        for op, ref in ((ko.EW_MAXNUMF, np.fmax), (ko.EW_MINNUMF, np.fmin), (ko.EW_REMF, np.fmod)):
+            assert ko.elementwise(ko.program([L, L1, dict(op=op, dst=2, a=0, b=1), ST]), [g(x), g(y)], g(out)) == 0
+            want = ref(x.astype(np.float64), y.astype(np.float64)).astype(np.float32)
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(out), nan) and np.array_equal(out[~nan], want[~nan]), op
+            if op != ko.EW_REMF:      # numpy's fmax / fmin do not order the zeros; the ops do
+                assert np.signbit(out[0, 2]) == (op == ko.EW_MINNUMF) and np.signbit(out[0, 3]) == (op == ko.EW_MINNUMF)
+                assert out[0, 0] == 2.0 and out[0, 1] == 1.0
+            else:
+                assert out[1, 0] == 1.5 and out[1, 1] == -1.5 and np.isnan(out[1, 2]) and out[1, 3] == 1.0 and np.isnan(out[0, 2])
+    # f16 registers: the result is rounded once to f16
+    xh = ko.fill_normal(m * n, ko.F16, 32, 0, 0.0, 3.0).reshape(m, n)
+    oh = np.zeros((m, n), np.uint16)
+    gh = lambda a: ko.mk_global(a, m, n, n, 1, ko.F16)
+    assert ko.elementwise(ko.program([L, dict(op=ko.EW_SIN, dst=2, a=0), ST]), [gh(xh)], gh(oh)) == 0
+    assert np.array_equal(oh.view(np.float16), np.sin(xh.view(np.float16).astype(np.float64)).astype(np.float16))

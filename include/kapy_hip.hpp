@@ -168,10 +168,10 @@ class OpBuilder {
   Value create_maxnumf(Value lhs, Value rhs) { return binary(KAPY_EW_MAXNUMF, lhs, rhs); }
   Value create_minnumf(Value lhs, Value rhs) { return binary(KAPY_EW_MINNUMF, lhs, rhs); }
   Value create_remf(Value lhs, Value rhs) { return binary(KAPY_EW_REMF, lhs, rhs); }
-  // kapy.clampf(source, low, high, propagateNan) (ir.cc:886-890): min(max(source, low), high); maximumf / minimumf propagate NaNs,
-  // the only form the elementwise programs have
+  // kapy.clampf(source, low, high, propagateNan) (ir.cc:886-890; ClampFOpConversion, ElementwiseOpToLLVM.cpp:699-728):
+  // min(max(source, low), high) with maximumf / minimumf when NaNs propagate, maxnumf / minnumf when they do not
   Value create_clampf(Value source, Value low, Value high, bool propagate_nan = true) {
-    if (!propagate_nan) throw Error(KAPY_ERR_UNSUPPORTED, "clampf: only the NaN-propagating form is implemented");
+    if (!propagate_nan) return create_minnumf(create_maxnumf(source, low), high);
     return create_minimumf(create_maximumf(source, low), high);
   }
   Value create_fma(Value a, Value b, Value c) {

@@ -53,6 +53,10 @@ static int run_cpu() {
   for (const kapy_ew_inst &I : prog) EXPECT(I.dst >= 0 && I.dst < 16);
   prog = b.program_of(b.create_clampf(lx, b.create_splat(-1.f, KAPY_F16), b.create_splat(1.f, KAPY_F16)));
   EXPECT(prog.size() == 6 && prog[2].op == KAPY_EW_MAXIMUMF && prog[4].op == KAPY_EW_MINIMUMF);
+  prog = b.program_of(b.create_clampf(lx, b.create_splat(-1.f, KAPY_F16), b.create_splat(1.f, KAPY_F16), false));   // NaNs do not propagate: maxnumf / minnumf
+  EXPECT(prog.size() == 6 && prog[2].op == KAPY_EW_MAXNUMF && prog[4].op == KAPY_EW_MINNUMF);
+  prog = b.program_of(b.create_remf(b.create_floor(b.create_sin(lx)), b.create_ceil(b.create_cos(lx))));
+  EXPECT(prog.size() == 7 && prog.back().op == KAPY_EW_ST_GLOBAL && prog[5].op == KAPY_EW_REMF);
   // the verifier's refusal arrives as an exception with the reference's wording
   try {
     kapy::Value h = b.create_ld_global(x), w = b.create_ld_global(b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_BF16));

@@ -54,14 +54,24 @@ struct TileLayout {
   static constexpr Swizzle kSwizzle = first_swizzle(kAccess, {kS.m, kS.k * T::kBytes}, ROWBYTES, 1, 8, 1024);
   static_assert(kSwizzle.bank_param == 4, "MFMA operand reads are 16-byte: the search must return 16-byte atoms");
   static constexpr int kLineParam = kSwizzle.line_param;
+  // The 16x16x128 operand reads (a lane: row lane % 16, the two 16-byte chunks 2 * (lane / 16) and + 1 of a 128-byte row)
+  // pass the search's model - which looks at the 16 lanes of one phase - with (4, 8), but the LDS serves them at two thirds
+  // of its rate (SQ_LDS_BANK_CONFLICT on half of its active cycles).  Measured conflict-free: the same XOR of the chunk
+  // index with three bits of the line index, taken in rotated order (line bits 0, 1, 2 -> chunk bits 1, 2, 0).
+  static constexpr bool kRotatedKey = kS.m == 16 && kS.kpack * T::kBytes == 32 && ROWBYTES == 128;
+  static_assert(!kRotatedKey || kLineParam == 8, "the rotated key replaces the (4, 8) swizzle");
+  static __device__ __forceinline__ uint32_t key_of(uint32_t o) {
+    const uint32_t line = (o >> 8) & (kLineParam - 1);
+    return kRotatedKey ? (((line & 3) << 1) | (line >> 2)) : line;
+  }
   // byte offset of 16-byte chunk `chunk` of row `row`
   static __device__ __forceinline__ uint32_t offset(uint32_t row, uint32_t chunk) {
     uint32_t o = row * kRowBytes + chunk * 16;
-    return o ^ (((o >> 8) & (kLineParam - 1)) << 4);
+    return o ^ (key_of(o) << 4);
   }
   // inverse on a linear LDS byte offset: which (row, chunk) of the tile lives there
   static __device__ __forceinline__ void locate(uint32_t lds_off, uint32_t &row, uint32_t &chunk) {
-    uint32_t o = lds_off ^ (((lds_off >> 8) & (kLineParam - 1)) << 4);
+    uint32_t o = lds_off ^ (key_of(lds_off) << 4);
     row = o / kRowBytes;
     chunk = (o % kRowBytes) / 16;
   }
@@ -588,14 +598,25 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     // instruction and no vector ALU work.  Ring positions repeat every five tiles; the steady-state
     // loop is unrolled by five so that every LDS address is a constant.
     static_assert(BM == BN && WM == 2 && WN == 2, "the unit ring assumes equal lhs / rhs halves and 2 x 2 wavefronts");
-    static_assert(KK >= 2 && KK % 2 == 0, "needs an even number of K-slices per tile");
+    // A tile step runs in kPhases phases with the barrier before the last one.  Normally a phase is a K-slice (all
+    // kTm x kTn blocks with the fragments of that slice, the next slice's fragments fetched meanwhile).  An instruction whose
+    // K extent is the whole tile (16x16x128 on 128-byte rows: KK == 1) has 2 x 8 fragment registers per block pair, too many
+    // to double-buffer whole; its tile runs as two passes over the halves of the rhs blocks instead: the lhs fragments stay
+    // for both passes (double-buffered across tiles), the rhs halves alternate between two buffers.
+    constexpr bool kNPass = KK == 1;
+    static_assert(kNPass || KK % 2 == 0, "needs an even number of K-slices per tile");
+    static_assert(!kNPass || C::kTn % 2 == 0, "two passes over halves of the rhs blocks");
+    constexpr int kPhases = kNPass ? 2 : KK, kPhaseMfmas = kNPass ? kMfmas / 2 : kMfmas, kHalfTn = C::kTn / 2;
     constexpr int kUnit = C::kUnitBytes, kHalf = kLoadsPerTile / 2;  // loads per wavefront per operand
     static_assert(C::kLoadsAPerWave == kHalf && C::kLoadsBPerWave == kHalf && kHalf % 2 == 0, "two equal units per operand");
     constexpr int kPerUnit = kHalf / 2;
-    constexpr int kEven = (KK * kMfmas) / kLoadsPerTile;
+    constexpr int kEven = (kPhases * kPhaseMfmas) / kLoadsPerTile;
     constexpr int kLoadSpacing = kEven < 1 ? 1 : kEven;
-    constexpr int kEarly = kMfmas / kLoadSpacing < kLoadsPerTile ? kMfmas / kLoadSpacing : kLoadsPerTile;
-    static_assert((kLoadsPerTile - kEarly) * kLoadSpacing <= (KK - 1) * kMfmas, "late loads must go out before the barrier that waits for them");
+    constexpr int kEarly = kPhaseMfmas / kLoadSpacing < kLoadsPerTile ? kPhaseMfmas / kLoadSpacing : kLoadsPerTile;
+    static_assert((kLoadsPerTile - kEarly) * kLoadSpacing <= (kPhases - 1) * kPhaseMfmas, "late loads must go out before the barrier that waits for them");
+    // reads and loads in different gaps, where a phase has enough gaps without a load for its reads at one per gap
+    constexpr int kFreeGaps = kPhaseMfmas - (kPhaseMfmas + kLoadSpacing - 1) / kLoadSpacing;
+    constexpr bool kSpread = kLoadSpacing > 1 && (kNPass ? (kLoadSpacing == kHalfTn && CH <= kHalfTn - 2 && kHalfTn * CH <= kFreeGaps) : kReads <= kFreeGaps);
     // The descriptors must sit in scalar registers (a descriptor in vector registers makes every load
     // a loop over its distinct values): pin the workgroup-uniform tile pointers with readfirstlane.
     auto uniform_ptr = [](const char *ptr) {
@@ -614,6 +635,14 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(b_tile), 0, __builtin_amdgcn_readfirstlane(bytes_left(p.N - n0, p.b_sn)), 0x00020000);
     const int wave_lds = wave * 1024;
     auto wrap = [](auto pos) { return pos >= 20 ? pos - 20 : (pos >= 10 ? pos - 10 : pos); };
+    // ring position `pos` + D, keeping a compile-time position (an integral_constant) a compile-time position
+    auto ring_add = [&](auto pos, auto d) {
+      if constexpr (std::is_integral_v<decltype(pos)>) return wrap(pos + decltype(d)::value);
+      else return std::integral_constant<int, (decltype(pos)::value + decltype(d)::value) % 10>{};
+    };
+    using Plus2 = std::integral_constant<int, 2>;
+    using Plus4 = std::integral_constant<int, 4>;
+    using Plus6 = std::integral_constant<int, 6>;
     // K need not be a multiple of BK (only of the 16 bytes of a chunk): the last tile is then partial, and the lanes
     // whose chunk lies past K ask for an offset beyond any descriptor, which the hardware answers with zeros in LDS.
     // Which chunk of a row a lane fetches is the same for every load it issues (the swizzle only mixes in the bit of
@@ -627,6 +656,17 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     }
     constexpr int kTailFlag = (int)0x80000000;
     // (only the KTAIL build of the kernel pays the select and the mask: they cost 2 % of the aligned case)
+    // Two passes: the per-lane offsets of load idx differ from load 0's by idx x (32 rows) only (the swizzle mixes in no bit of
+    // the load index beyond the wavefront's own); they are formed at the load from one register per operand - through an
+    // opaque add, or the compiler would keep all of them alive again - which leaves the registers to the fragments.
+    auto offset_of = [&](const uint32_t(&goff)[kHalf], int idx, uint32_t row_pitch_bytes) -> uint32_t {
+      if constexpr (!kNPass) return goff[idx];
+      if (idx == 0) return goff[0];
+      uint32_t r;
+      const uint32_t delta = (uint32_t)idx * 32u * row_pitch_bytes;
+      asm volatile("v_add_u32 %0, %1, %2" : "=v"(r) : "v"(goff[0]), "s"(delta));
+      return r;
+    };
 #define KAPY_VOFF(g) ((KTAIL && soff < 0 && lane_past_k) ? kTailFlag : (int)(g))
 #define KAPY_SOFF (KTAIL ? (soff & ~kTailFlag) : soff)
     // scalar byte offset of K-tile j in a row, clamped to the last real tile; the sign bit marks a partial tile
@@ -634,15 +674,16 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       const int jj = min(j, KT - 1);
       return jj * (BK * EB) | ((KTAIL && jj == KT - 1 && k_last + BK > p.K) ? kTailFlag : 0);
     };
+    const uint32_t a_pitch_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(p.a_sm * EB)), b_pitch_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(p.b_sn * EB));
     auto load_a = [&](int idx, int pos_of_unit0, int soff) {  // idx: 0 .. kHalf-1, unit idx / kPerUnit
       const int u = idx / kPerUnit, i = idx % kPerUnit;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + wrap(pos_of_unit0 + u) * kUnit + i * C::kWaves * 1024 + wave_lds),
-                                               16, KAPY_VOFF(a_goff[idx]), KAPY_SOFF, 0, 0);
+                                               16, KAPY_VOFF(offset_of(a_goff, idx, a_pitch_bytes)), KAPY_SOFF, 0, 0);
     };
     auto load_b = [&](int idx, int pos_of_unit2, int soff) {
       const int u = idx / kPerUnit, i = idx % kPerUnit;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + wrap(pos_of_unit2 + u) * kUnit + i * C::kWaves * 1024 + wave_lds),
-                                               16, KAPY_VOFF(b_goff[idx]), KAPY_SOFF, 0, 0);
+                                               16, KAPY_VOFF(offset_of(b_goff, idx, b_pitch_bytes)), KAPY_SOFF, 0, 0);
     };
 #undef KAPY_VOFF
 #undef KAPY_SOFF
@@ -653,7 +694,36 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
       if (slot < kHalf) load_b(slot, pos0, soff_b);
       else load_a(slot - kHalf, pos0 + 2, soff_a);
     };
-    Frag af[2][C::kTm], bf[2][C::kTn];
+    Frag af[kNPass ? 1 : 2][C::kTm], bf[2][kNPass ? kHalfTn : C::kTn];
+    // A matrix instruction every 16 (32) clocks leaves the wave 12 (28) clocks to issue anything else before the matrix
+    // pipe runs dry, and a vector ALU instruction takes 8 of them, a scalar or LDS or memory instruction 4 to 8.  The
+    // steady-state loop therefore computes no address: a read at a compile-time ring position is one of three copies of the
+    // lane's fragment offset (the 160 KiB ring seen as 64 KiB windows, the reach of a read's immediate) plus an immediate.
+    constexpr int kWindows = (C::kLdsBytes + 65535) / 65536;
+    // (a tile's units start at an even ring position, so the wave's own unit - wm for the lhs, wn for the rhs - never
+    // wraps on its own and can sit in the register part: one set of copies per operand)
+    uint32_t frag_win[2][kWindows][KK][CH];
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+      for (int w = 0; w < kWindows; ++w)
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+          for (int c = 0; c < CH; ++c) {
+            uint32_t v = (uint32_t)(uintptr_t)lds + frag_off[kk][c] + (uint32_t)(o ? wn : wm) * kUnit + (uint32_t)w * 65536u;
+            asm volatile("" : "+v"(v));  // (opaque: registers that stay, not one register and an add at every read)
+            frag_win[o][w][kk][c] = v;
+          }
+    // The 16 bytes of chunk c, slice kk of operand o (0 lhs, 1 rhs) whose unit 0 starts at ring byte `at`, `rows` bytes in.
+    auto read_at = [&](int o, auto at, uint32_t rows, int kk, int c) -> u32x4 {
+      if constexpr (std::is_integral_v<decltype(at)>) {
+        return *(const u32x4 *)(lds + (at + (o ? wn : wm) * kUnit + frag_off[kk][c]) + rows);
+      } else {
+        const uint32_t v = decltype(at)::value + rows;
+        return *(const __attribute__((address_space(3))) u32x4 *)(uintptr_t)(frag_win[o][v >> 16][kk][c] + (v & 65535u));
+      }
+    };
     // prologue: tiles 0 and 1 whole (lhs units first, then rhs, as the tile steps count them)
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -671,8 +741,9 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     __builtin_amdgcn_s_barrier();  // tile 0 published
     {
       const uint32_t a0 = wm * kUnit, b0 = (2 + wn) * kUnit;
+      // (two passes: the lhs blocks and the first half of the rhs blocks)
 #pragma unroll
-      for (int idx = 0; idx < kReads; ++idx) {
+      for (int idx = 0; idx < (kNPass ? (C::kTm + kHalfTn) * CH : kReads); ++idx) {
         const int blk = idx / CH, c = idx % CH;
         if (blk < C::kTm) af[0][blk].c[c] = *(const u32x4 *)(lds + a0 + frag_off[0][c] + blk * KM * C::kRowBytes);
         else bf[0][blk - C::kTm].c[c] = *(const u32x4 *)(lds + b0 + frag_off[0][c] + (blk - C::kTm) * KM * C::kRowBytes);
@@ -682,18 +753,72 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     // sequence after the barrier of tile kt-1 is [rhs of tile kt+1, lhs of tile kt+2]; its first
     // kEarly loads went out in the last slice of tile kt-1, the rest go out in the first slices of
     // tile kt.  (`first`: tile 0, where the prologue has issued the rhs part of that sequence.)
-    auto tile_step = [&](int kt, auto pos, auto first) {
-      const auto prev = wrap(pos + 6), next = wrap(pos + 4);
+    // (`parity`: two passes only - which lhs fragment buffer holds this tile's blocks; it alternates from tile to tile)
+    auto tile_step = [&](int kt, auto pos, auto first, auto parity) {
+      const auto prev = ring_add(pos, Plus6{});
+      const auto next = ring_add(pos, Plus4{});
       // LDS bases of this wave's operand units in this tile and the next one
-      const uint32_t a_cur_base = wrap(pos + wm) * kUnit, b_cur_base = wrap(pos + 2 + wn) * kUnit;
-      const uint32_t a_nxt_base = wrap(next + wm) * kUnit, b_nxt_base = wrap(next + 2 + wn) * kUnit;
+      // (ring bytes of unit 0 of each operand - compile-time constants in the unrolled loop, see read_at)
+      auto unit_base = [&](auto q) {
+        if constexpr (std::is_integral_v<decltype(q)>) return (uint32_t)(q * kUnit);
+        else return std::integral_constant<uint32_t, (uint32_t)(decltype(q)::value * kUnit)>{};
+      };
+      const auto a_cur_base = unit_base(pos);
+      const auto b_cur_base = unit_base(ring_add(pos, Plus2{}));
+      const auto a_nxt_base = unit_base(next);
+      const auto b_nxt_base = unit_base(ring_add(pos, Plus6{}));
       const int soff_late_b = k_off(kt + 1), soff_late_a = k_off(kt + 2);   // sequence of tile kt-1
       const int soff_early_b = k_off(kt + 2), soff_early_a = k_off(kt + 3); // sequence of tile kt
-      auto ring_read = [&](uint32_t a_base, uint32_t b_base, int kk, int idx, Frag *a_dst, Frag *b_dst) {
+      auto ring_read = [&](auto a_base, auto b_base, int kk, int idx, Frag *a_dst, Frag *b_dst) {
         const int blk = idx / CH, c = idx % CH;
-        if (blk < C::kTm) a_dst[blk].c[c] = *(const u32x4 *)(lds + (a_base + frag_off[kk][c]) + blk * KM * C::kRowBytes);
-        else b_dst[blk - C::kTm].c[c] = *(const u32x4 *)(lds + (b_base + frag_off[kk][c]) + (blk - C::kTm) * KM * C::kRowBytes);
+        if (blk < C::kTm) a_dst[blk].c[c] = read_at(0, a_base, blk * KM * C::kRowBytes, kk, c);
+        else b_dst[blk - C::kTm].c[c] = read_at(1, b_base, (blk - C::kTm) * KM * C::kRowBytes, kk, c);
       };
+      if constexpr (kNPass) {
+        (void)parity;
+        Frag *a_cur = af[0];  // one buffer: a block is fetched again (for the next tile) right behind its last use in pass 1
+#pragma unroll
+        for (int ph = 0; ph < 2; ++ph) {
+          Frag *b_cur = bf[ph];  // pass 0: rhs blocks 0 .. kHalfTn-1, pass 1: the others
+          if (ph == 1) {
+            // tile kt+1 has landed once only the kHalf youngest loads (lhs of tile kt+2) are in flight; this wave's reads
+            // of tile kt (the last ones went out in pass 0) have returned
+            __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
+            __builtin_amdgcn_s_barrier();
+          }
+#pragma unroll
+          for (int g = 0; g < kPhaseMfmas; ++g) {
+            const int i = g / kHalfTn, j = g % kHalfTn;  // lhs-block major: block i is used kHalfTn times in a row, then rests
+            T::mfma_in_place(b_cur[j].c, a_cur[i].c, acc[i][ph * kHalfTn + j]);
+            if (g % kLoadSpacing != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
+            // (a read never shares the gap behind a matrix instruction with a load: the two together, with the scalar
+            // instructions a load brings, outlast the instruction, and the matrix pipe would wait for the next one)
+            if (ph == 0) {  // the second half of this tile's rhs blocks, in the first gaps that carry no load
+              const int r = kSpread ? (g % kLoadSpacing ? g - 1 - g / kLoadSpacing : -1) : g;
+              const int blk = r / CH, c = r % CH;
+              if (r >= 0 && blk < kHalfTn) bf[1][blk].c[c] = read_at(1, b_cur_base, (kHalfTn + blk) * KM * C::kRowBytes, 0, c);
+            } else {
+              // the next tile: lhs block i into the registers its last use has just left ...
+              const int jb = kSpread ? j - 1 : j;  // (loads go out behind j == 0 when kSpread)
+              if (j == kHalfTn - 1) {
+#pragma unroll
+                for (int c = 0; c < CH; ++c) a_cur[i].c[c] = read_at(0, a_nxt_base, i * KM * C::kRowBytes, 0, c);
+              } else if (i < kHalfTn && jb >= 0 && jb < CH) {
+                // ... and the first half of its rhs blocks (block i, chunk jb) into the buffer pass 0 has left
+                bf[0][i].c[jb] = read_at(1, b_nxt_base, i * KM * C::kRowBytes, 0, jb);
+              }
+            }
+            if (g % kLoadSpacing == 0) {
+              const int slot = (ph * kPhaseMfmas + g) / kLoadSpacing;
+              if (ph == 1 && g / kLoadSpacing < kEarly) ring_load(pos, g / kLoadSpacing, soff_early_b, soff_early_a);
+              if (ph == 0 && kEarly + slot < kLoadsPerTile && (!first.value || kEarly + slot >= kHalf))
+                ring_load(prev, kEarly + slot, soff_late_b, soff_late_a);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         Frag *a_cur = af[kk & 1], *b_cur = bf[kk & 1], *a_nxt = af[(kk + 1) & 1], *b_nxt = bf[(kk + 1) & 1];
@@ -706,11 +831,12 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
         for (int g = 0; g < kMfmas; ++g) {
           const int i = g / C::kTn, j = g % C::kTn;
           acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
-          __builtin_amdgcn_sched_barrier(0);
+          if (g % kLoadSpacing != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
 #pragma unroll
           for (int t = 0; t < kReadsPerMfma; ++t) {
-            const int idx = g * kReadsPerMfma + t;
-            if (idx < kReads) {
+            // (kSpread: one read per gap, and none in the gaps that carry a load - see the two-pass step)
+            const int idx = kSpread ? (g % kLoadSpacing ? g - 1 - g / kLoadSpacing : -1) : g * kReadsPerMfma + t;
+            if (idx >= 0 && idx < kReads) {
               if (kk + 1 < KK) ring_read(a_cur_base, b_cur_base, kk + 1, idx, a_nxt, b_nxt);
               else ring_read(a_nxt_base, b_nxt_base, 0, idx, a_nxt, b_nxt);
             }
@@ -725,20 +851,27 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
         }
       }
     };
-    tile_step(0, std::integral_constant<int, 0>{}, Yes{});
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
+    tile_step(0, std::integral_constant<int, 0>{}, Yes{}, Even{});
     int kt = 1;
     for (; kt + 5 <= KT; kt += 5) {
-      tile_step(kt, std::integral_constant<int, 4>{}, No{});
-      tile_step(kt + 1, std::integral_constant<int, 8>{}, No{});
-      tile_step(kt + 2, std::integral_constant<int, 2>{}, No{});
-      tile_step(kt + 3, std::integral_constant<int, 6>{}, No{});
-      tile_step(kt + 4, std::integral_constant<int, 0>{}, No{});
+      tile_step(kt, std::integral_constant<int, 4>{}, No{}, Even{});
+      tile_step(kt + 1, std::integral_constant<int, 8>{}, No{}, Even{});
+      tile_step(kt + 2, std::integral_constant<int, 2>{}, No{}, Even{});
+      tile_step(kt + 3, std::integral_constant<int, 6>{}, No{}, Even{});
+      tile_step(kt + 4, std::integral_constant<int, 0>{}, No{}, Even{});
     }
     for (int pos = 4; kt < KT; ++kt) {
-      tile_step(kt, pos, No{});
+      tile_step(kt, pos, No{}, Even{});
       pos = wrap(pos + 4);
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // loads issued for tiles past the end still target this workgroup's LDS
+    if constexpr (kNPass) {
+      // the in-place matrix instructions are opaque to the compiler, which therefore does not count the wait states their
+      // results need before another kind of instruction may read the accumulators (up to 19 for this instruction)
+      asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    }
   } else if constexpr (STAGES == 2) {
     // Two stages (the ring depth of the reference fixture, matmul.mlir:19-22).  The one barrier per
     // tile sits BEFORE the tile's last K-slice: by then every wave has fetched the fragments of that
@@ -1447,11 +1580,11 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s
   // the ring variants take any M, N >= 128 and any K >= 128 of whole 16-byte chunks (their loads are bounded by the
   // operands' ends); 256x256 tiles when there are at least as many of them as CUs, 128x128 (two workgroups per CU) below
   if (p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
-    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<F8, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
     return launch_f8<F8, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
-    return launch_f8<F8, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   if (p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0) return launch_f8<F8, 128, 128, 128, 2, 2, 2>(p, lhs_fmt, rhs_fmt, s);
   return KAPY_ERR_UNSUPPORTED;
 }

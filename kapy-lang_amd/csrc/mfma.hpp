@@ -92,6 +92,17 @@ struct F8M16 {
     i32x8 bv = {(int)b[0][0], (int)b[0][1], (int)b[0][2], (int)b[0][3], (int)b[1][0], (int)b[1][1], (int)b[1][2], (int)b[1][3]};
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, AF, BF, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
   }
+  // The same instruction accumulating in place in an accumulator register: the tiled kernel's 256 accumulators fill that half
+  // of the register file exactly, and left to itself the compiler gives some matrix instructions a destination other than
+  // their accumulator operand, which needs registers that are not there.  cbsz / blgp carry the operand formats.
+  static __device__ __forceinline__ void mfma_in_place(const u32x4 *a, const u32x4 *b, f32x4 &c) {
+    i32x8 av = {(int)a[0][0], (int)a[0][1], (int)a[0][2], (int)a[0][3], (int)a[1][0], (int)a[1][1], (int)a[1][2], (int)a[1][3]};
+    i32x8 bv = {(int)b[0][0], (int)b[0][1], (int)b[0][2], (int)b[0][3], (int)b[1][0], (int)b[1][1], (int)b[1][2], (int)b[1][3]};
+    const int unit_scales = 0x7F7F7F7F;
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0] cbsz:%4 blgp:%5"
+                 : "+a"(c)
+                 : "v"(av), "v"(bv), "v"(unit_scales), "n"(AF), "n"(BF));
+  }
 };
 
 // Where a lane's operand registers sit in an operand block: the row (lhs) or column (rhs) they belong to and

@@ -248,14 +248,27 @@ struct PackedEpilogue {
     const AccLane at = acc_lane(kAccLayout, kBlock, lane);
     const int wrow = at.row, wcol = at.col;                    // this lane's row / first column in an accumulator block
     const int rrow = lane / kChunks, rchunk = lane % kChunks;  // and in a read-back instruction
+    // The lane's scales - of its row in every block of rows, of its columns in every block of columns - are fetched once, up
+    // front and together: fetched where they are used, each load would be waited for by itself (the result stores in between
+    // might alias them, for all the compiler knows), some hundred exposed cache latencies per wavefront.
+    constexpr int kRowBlocks = EPI == 1 ? kStrips * kBlocksPerStrip : 1, kColQuads = EPI == 1 ? kTn * kQuads : 1;
+    float rs_all[kRowBlocks];
+    f32x4 cs_all[kColQuads];
+    if constexpr (EPI == 1) {
+#pragma unroll
+      for (int b = 0; b < kRowBlocks; ++b) rs_all[b] = p.row_scale[min(m_wave + b * KM + wrow, p.M - 1)];  // (rows past M exist only in tiles that hang over the edge; they are not stored)
+#pragma unroll
+      for (int j = 0; j < kTn; ++j)
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) cs_all[j * kQuads + q] = *(const f32x4 *)(p.col_scale + min(n_wave + j * KM + wcol + kQuadStep * q, p.N - 4));
+    }
 #pragma unroll
     for (int i = 0; i < kStrips; ++i) {
       __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
       char *strip = strip0 + (i & 1) * kStrip;
 #pragma unroll
       for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
-        float rs = 1.0f;
-        if constexpr (EPI == 1) rs = p.row_scale[min(m_wave + i * 32 + bi * KM + wrow, p.M - 1)];  // (rows past M exist only in tiles that hang over the edge; they are not stored)
+        const float rs = EPI == 1 ? rs_all[i * kBlocksPerStrip + bi] : 1.0f;
 #pragma unroll
         for (int j = 0; j < kTn; ++j)
 #pragma unroll
@@ -264,7 +277,7 @@ struct PackedEpilogue {
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
             if constexpr (EPI == 1) {
-              const f32x4 cs = *(const f32x4 *)(p.col_scale + min(n_wave + j * KM + wcol + kQuadStep * q, p.N - 4));
+              const f32x4 cs = cs_all[j * kQuads + q];
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
             }

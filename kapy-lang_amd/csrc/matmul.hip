@@ -222,16 +222,15 @@ __device__ __noinline__ void store_block_generic(const GemmParams &p, int32_t m_
 
 // Packed epilogue (16-bit row-major result, 16-byte aligned rows, no accumulator input, RN) of one
 // wavefront's WTM x WTN block of KM x KM accumulator blocks, by 32-row strips through a wave-private
-// LDS area: accumulator quads (four consecutive columns of one row per lane) are narrowed and written
-// 8 bytes at a time, read back 16 bytes per lane along rows, and stored so that one instruction
-// writes whole 128-byte lines (64 / kChunks rows x WTN*2 bytes) - the register layout itself would
-// scatter 8-byte pieces over KM rows per instruction.  Row stride WTN*2 + 16 bytes: both the 8-byte
-// writes down the rows and the 16-byte reads along them then use every LDS bank equally.
+// LDS area: accumulator quads (four consecutive columns of one row per lane) are written as fp32,
+// read back 32 bytes per lane along rows, narrowed and stored so that one instruction writes whole
+// 128-byte lines (64 / (WTN/8) rows x WTN*2 bytes) - the register layout itself would scatter 8-byte
+// pieces over KM rows per instruction.  Row stride WTN*4 + 16 bytes: the 16-byte writes down the rows
+// then use every LDS bank equally.
 // The caller makes sure (barrier) that no other wave still uses the LDS area.
 template <int KM, int WTM, int WTN>
 struct PackedEpilogue {
-  static constexpr int kRowStride = WTN * 2 + 16, kStrip = 32 * kRowStride, kBytesPerWave = 2 * kStrip;
-  static constexpr int kChunks = WTN * 2 / 16, kRowsPerStore = 64 / kChunks, kStores = 32 / kRowsPerStore;
+  static constexpr int kBytesPerWave = 32 * (WTN * 4 + 16);  // one strip of 32 rows of fp32, rows 16 bytes apart in the banks
   static constexpr int kGroups = 64 / KM, kAccRegs = KM * KM / 64;
   static constexpr int kBlocksPerStrip = 32 / KM, kStrips = WTM / 32, kTn = WTN / KM;
   // the accumulator fragments of a KM x KM block (the operand classes share them): a lane's register quads hold 4
@@ -240,62 +239,80 @@ struct PackedEpilogue {
   static constexpr Fragments kAccLayout = mfma_acc_exchanged(kBlock);
   static constexpr int kQuads = kAccRegs / 4, kQuadStep = kQuads > 1 ? acc_lane(kAccLayout, kBlock, 0).qcol : 0;
   static_assert(quads_run_along_rows(kBlock) && acc_lane_describes(kAccLayout, kBlock) && kAccLayout.loop_size({KM, KM}) == kAccRegs, "accumulator fragments");
-  static_assert(WTM % 32 == 0 && 64 % kChunks == 0 && 32 % kRowsPerStore == 0, "strip geometry");
+  static_assert(WTM % 32 == 0, "strip geometry");
 
-  // EPI: 0 = cast only, 1 = row and column scales
+  // EPI: 0 = cast only, 1 = row and column scales.  The strip goes through LDS as fp32: the accumulator registers are
+  // written as they are (an LDS store takes them from the accumulator file; narrowing first would cost a register move
+  // per element), a lane reads back 8 consecutive columns of a row, scales, narrows and stores 16 bytes.  The stores are
+  // buffer stores through a descriptor of the wavefront's part of the result: it ends with the result's last row, so
+  // the rows of a tile that hangs over the edge fall out of range in hardware, and a store costs one add.
   template <bool F16, int EPI, typename Acc>
-  static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
+  static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip, int32_t m_wave, int32_t n_wave, int lane) {
+    constexpr int kRowStrideF = WTN * 4 + 16, kChunksF = WTN / 8, kRowsPerPass = 64 / kChunksF, kPasses = 32 / kRowsPerPass;
+    static_assert(32 * kRowStrideF <= kBytesPerWave && 64 % kChunksF == 0 && 32 % kRowsPerPass == 0, "fp32 strip geometry");
     const AccLane at = acc_lane(kAccLayout, kBlock, lane);
-    const int wrow = at.row, wcol = at.col;                    // this lane's row / first column in an accumulator block
-    const int rrow = lane / kChunks, rchunk = lane % kChunks;  // and in a read-back instruction
-    // The lane's scales - of its row in every block of rows, of its columns in every block of columns - are fetched once, up
-    // front and together: fetched where they are used, each load would be waited for by itself (the result stores in between
-    // might alias them, for all the compiler knows), some hundred exposed cache latencies per wavefront.
-    constexpr int kRowBlocks = EPI == 1 ? kStrips * kBlocksPerStrip : 1, kColQuads = EPI == 1 ? kTn * kQuads : 1;
-    float rs_all[kRowBlocks];
-    f32x4 cs_all[kColQuads];
+    const int wrow = at.row, wcol = at.col;                      // this lane's row / first column in an accumulator block
+    const int rrow = lane / kChunksF, rchunk = lane % kChunksF;  // and in a read-back instruction
+    const int32_t nn = n_wave + rchunk * 8;                      // (N a multiple of 8: a piece of 8 columns is in or out whole)
+    // The lane's scales - of its 8 columns, of its row in every pass of every strip - are fetched once, up front and together:
+    // fetched where they are used, each load would be waited for by itself (the result stores in between might alias
+    // them, for all the compiler knows), some hundred exposed cache latencies per wavefront.
+    constexpr int kRowsPerLane = EPI == 1 ? kStrips * kPasses : 1;
+    float rs_all[kRowsPerLane];
+    f32x4 cs_lo = {1.f, 1.f, 1.f, 1.f}, cs_hi = cs_lo;
     if constexpr (EPI == 1) {
+      const int32_t nc = min(nn, p.N - 8);
+      cs_lo = *(const f32x4 *)(p.col_scale + nc);
+      cs_hi = *(const f32x4 *)(p.col_scale + nc + 4);
 #pragma unroll
-      for (int b = 0; b < kRowBlocks; ++b) rs_all[b] = p.row_scale[min(m_wave + b * KM + wrow, p.M - 1)];  // (rows past M exist only in tiles that hang over the edge; they are not stored)
-#pragma unroll
-      for (int j = 0; j < kTn; ++j)
-#pragma unroll
-        for (int q = 0; q < kQuads; ++q) cs_all[j * kQuads + q] = *(const f32x4 *)(p.col_scale + min(n_wave + j * KM + wcol + kQuadStep * q, p.N - 4));
+      for (int r = 0; r < kRowsPerLane; ++r)  // (rows past M exist only in tiles that hang over the edge; they are not stored)
+        rs_all[r] = p.row_scale[min(m_wave + (r / kPasses) * 32 + (r % kPasses) * kRowsPerPass + rrow, p.M - 1)];
     }
+    const uint32_t pitch = (uint32_t)__builtin_amdgcn_readfirstlane((int)(p.d_sm * 2));
+    const int32_t rows_left = min(WTM, p.M - m_wave), cols_left = min(WTN, p.N - n_wave);
+    const uint64_t bv = (uint64_t)(p.d + ((int64_t)m_wave * p.d_sm + n_wave) * 2);
+    const uint32_t base_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)bv), base_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(bv >> 32));
+    const int32_t records = (rows_left > 0 && cols_left > 0) ? (int32_t)((uint32_t)(rows_left - 1) * pitch + (uint32_t)cols_left * 2u) : 0;
+    const __amdgpu_buffer_rsrc_t d_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)base_hi << 32) | (uint64_t)base_lo), 0, __builtin_amdgcn_readfirstlane(records), 0x00020000);
+    // (a lane whose columns lie past N asks for an offset beyond any descriptor)
+    const uint32_t voff0 = nn < p.N ? (uint32_t)rrow * pitch + (uint32_t)rchunk * 16u : 0x80000000u;
 #pragma unroll
     for (int i = 0; i < kStrips; ++i) {
       __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
-      char *strip = strip0 + (i & 1) * kStrip;
 #pragma unroll
-      for (int bi = 0; bi < kBlocksPerStrip; ++bi) {
-        const float rs = EPI == 1 ? rs_all[i * kBlocksPerStrip + bi] : 1.0f;
+      for (int bi = 0; bi < kBlocksPerStrip; ++bi)
 #pragma unroll
         for (int j = 0; j < kTn; ++j)
 #pragma unroll
           for (int q = 0; q < kQuads; ++q) {
-            float v[4];
+            f32x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = acc[i * kBlocksPerStrip + bi][j][4 * q + e];
-            if constexpr (EPI == 1) {
-              const f32x4 cs = cs_all[j * kQuads + q];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs[e]));
-            }
-            u32x2 w;
-            w[0] = F16 ? pack2_f16_rn(v[0], v[1]) : pack2_bf16_rn(v[0], v[1]);
-            w[1] = F16 ? pack2_f16_rn(v[2], v[3]) : pack2_bf16_rn(v[2], v[3]);
-            *(u32x2 *)(strip + (bi * KM + wrow) * kRowStride + (j * KM + wcol + kQuadStep * q) * 2) = w;
+            *(f32x4 *)(strip + (bi * KM + wrow) * kRowStrideF + (j * KM + wcol + kQuadStep * q) * 4) = v;
           }
-      }
-      // LDS executes a wave's instructions in order: the reads below see the writes above
+      // LDS executes a wave's instructions in order: the reads below see the writes above, and the next strip's writes
+      // come after these reads
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < kStores; ++t) {
-        const int row = t * kRowsPerStore + rrow;
-        const u32x4 w = *(const u32x4 *)(strip + row * kRowStride + rchunk * 16);
-        // a tile may hang over the result's last rows and columns (N a multiple of 8: a 16-byte piece is in or out whole)
-        if (m_wave + i * 32 + row < p.M && n_wave + rchunk * 8 < p.N)
-          *(u32x4 *)(p.d + ((int64_t)(m_wave + i * 32 + row) * p.d_sm + n_wave + rchunk * 8) * 2) = w;
+      for (int t = 0; t < kPasses; ++t) {
+        const int row = t * kRowsPerPass + rrow;
+        const f32x4 lo = *(const f32x4 *)(strip + row * kRowStrideF + rchunk * 32), hi = *(const f32x4 *)(strip + row * kRowStrideF + rchunk * 32 + 16);
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+        if constexpr (EPI == 1) {
+          const float rs = rs_all[i * kPasses + t];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs_lo[e]));
+            v[4 + e] = __fmul_rn(v[4 + e], __fmul_rn(rs, cs_hi[e]));
+          }
+        }
+        u32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = F16 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
+        __builtin_amdgcn_raw_buffer_store_b128(w, d_rsrc, (int)(voff0 + (uint32_t)(i * 32 + t * kRowsPerPass) * pitch), 0, 0);
       }
     }
   }

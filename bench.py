@@ -707,6 +707,47 @@ def bench_ceilings(kh, steps, warmup, cpu):
             wall, ev = _events(lambda i: kh.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr()), 10, 3)
             out["l2_read_tbs"]["%d MiB per XCD, %s" % (window >> 20, "LDS-direct" if to_lds else "to registers")] = round(nb / (ev * 1e-3) / 1e12, 2)
         del buf
+    # what a wave can issue beside its matrix instructions (one wave per SIMD, as in the tiled matmuls): fillers in the gap
+    # behind every instruction, and the reads and loads of the matmuls' steady-state loop on L2-resident data
+    out["issue_tflops"] = {}
+    fsink = torch.empty(1024 * 256, device="cuda", dtype=torch.float32)
+    window = torch.empty(8 * (2 << 20), dtype=torch.uint8, device="cuda")
+    window.random_(0, 120)
+    for name, way, fills in (("bf16 16x16x32", kh.MFMA_16X16X32_16B, ((0, 0), (1, 3), (1, 4), (1, 6), (2, 1), (2, 2), (2, 3), (3, 0))),
+                             ("e4m3 16x16x128", kh.MFMA_16X16X128_F8, ((0, 0), (1, 6), (1, 8), (2, 2), (2, 3), (2, 4), (3, 0)))):
+        row = {}
+        for filler, count in fills:
+            _, flops = kh.probe_issue(way, filler, count, window.data_ptr(), 2000, fsink.data_ptr())
+            wall, ev = _events(lambda i: kh.probe_issue(way, filler, count, window.data_ptr(), 2000, fsink.data_ptr()), 6, 3)
+            label = ("nothing", "%d scalar" % count, "%d vector ALU" % count, "matmul loop: 32 LDS reads + 16 LDS-direct loads per tile")[filler]
+            row[label] = round(flops / (ev * 1e-3) / 1e12, 1)
+        out["issue_tflops"][name] = row
+    del window
+    # the tiled matmuls' cost per launch that does not grow with K (epilogues, prologues, launch), and the rate beyond it:
+    # the C4 / C5 shapes at K and 2K
+    out["gemm_fixed_cost"] = {}
+    for name, m, n, k, f8 in (("C4 bf16 8192 x 8192", 8192, 8192, 4096, False), ("C5 e4m3 4096 x 8192", 4096, 8192, 8192, True)):
+        times = []
+        for kk in (k, 2 * k):
+            if f8:
+                a = torch.randn(m, kk, device="cuda").mul_(100.0).to(torch.float8_e4m3fn).view(torch.uint8)
+                w = torch.randn(n, kk, device="cuda").mul_(100.0).to(torch.float8_e4m3fn).view(torch.uint8)
+                sa, sb = torch.rand(m, device="cuda") * 0.01 + 0.001, torch.rand(n, device="cuda") * 0.01 + 0.001
+                d = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+                ga, gw, gd = kh.mk_global(a.data_ptr(), m, kk, kk, 1, kh.F8E4M3), kh.mk_global(w.data_ptr(), kk, n, 1, kk, kh.F8E4M3), kh.mk_global(d.data_ptr(), m, n, n, 1, kh.BF16)
+                fn = lambda i: kh.matmul_scaled_f8(ga, gw, sa.data_ptr(), sb.data_ptr(), gd)
+            else:
+                a = torch.randn(m, kk, device="cuda", dtype=torch.bfloat16)
+                w = torch.randn(n, kk, device="cuda", dtype=torch.bfloat16)
+                d = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+                ga, gw, gd = kh.mk_global(a.data_ptr(), m, kk, kk, 1, kh.BF16), kh.mk_global(w.data_ptr(), kk, n, 1, kk, kh.BF16), kh.mk_global(d.data_ptr(), m, n, n, 1, kh.BF16)
+                fn = lambda i: kh.matmul(ga, gw, gd)
+            wall, ev = _events(fn, 30, 10)
+            times.append(ev * 1e3)
+            del a, w, d
+        per_k = (times[1] - times[0]) / k   # us per K element beyond the fixed cost
+        out["gemm_fixed_cost"][name] = {"us_at_K=%d" % k: round(times[0], 1), "us_at_K=%d" % (2 * k): round(times[1], 1), "fixed_us": round(times[0] - per_k * k, 1),
+                                        "marginal_tflops": round(2.0 * m * n / per_k / 1e6, 1)}
     return out
 
 

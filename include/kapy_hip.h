@@ -183,6 +183,15 @@ int kapy_probe_mfma(int32_t impl_way, int32_t dtype, const void *operands, int32
 int kapy_probe_copy(const void *src, void *dst, int64_t bytes, int32_t vectors_per_lane, int32_t nt_load, int32_t nt_store, int32_t persistent_per_cu,
                     uint64_t *ticks, int32_t *workgroups, void *stream);
 
+/* kapy_probe_issue: what a wave can issue beside its matrix instructions.  One wave per SIMD (the tiled matmul's occupancy)
+ * runs `iterations` tiles of independent matrix instructions of `impl_way` (KAPY_MFMA_16X16X32_16B: 128 per tile, or
+ * KAPY_MFMA_16X16X128_F8: 64 per tile - 2048 matrix-pipe clocks either way) with, behind every instruction, filler 0: nothing;
+ * 1: `count` (1, 2, 3, 4, 6, 8) scalar instructions; 2: `count` (1 .. 4) vector ALU instructions; 3: the reads and loads of
+ * the tiled matmul's steady-state loop (32 LDS reads of 16 bytes per lane and 16 LDS-direct loads of 1 KiB per wave and
+ * tile, from `src`: 8 windows of 2 MiB, one per XCD, that stay in the L2s).  sink: one float per lane (workgroups * 256,
+ * never written in practice).  Outputs: the workgroups launched and the flops of the launch. */
+int kapy_probe_issue(int32_t impl_way, int32_t filler, int32_t count, const void *src, int32_t iterations, float *sink, int32_t *workgroups, int64_t *flops,
+                     void *stream);
 /* kapy_probe_l2_read: every workgroup (workgroups_per_cu per CU, 256 lanes) reads the window of `src` that belongs to its XCD
  * (src holds 8 windows of window_bytes, one per XCD; a window of a few MiB stays in that XCD's L2) `iterations` x 32 KiB, 16
  * bytes per lane and instruction, as LDS-direct loads (to_lds = 1, the form the tiled matmul kernels use) or into registers.

@@ -202,6 +202,98 @@ __global__ __launch_bounds__(256) void l2_read_kernel(const char *src, int64_t w
   if (sink && (x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[blockIdx.x] = x[0];  // keeps the register form's loads alive
 }
 
+// What a wave can issue beside its matrix instructions.  One wave per SIMD (the tiled matmul's occupancy) runs `iterations`
+// tiles of kTileClocks of independent matrix instructions - 128 x 16x16x32 (16 clocks each) or 64 x 16x16x128 (32 clocks) - and
+// in the gap behind every instruction FILL asks for: 1 = COUNT scalar instructions (s_nop), 2 = COUNT vector ALU instructions
+// (v_mov), 3 = the steady-state loop of the tiled matmul: 32 LDS reads of 16 bytes per lane and 16 LDS-direct loads of 1 KiB
+// per wave and tile, spread evenly and never in the same gap, from a window of 2 MiB per XCD that stays in the L2.
+// MF: 0 = bf16 16x16x32, 1 = e4m3 16x16x128.
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+template <int MF, int FILL, int COUNT>
+__global__ __launch_bounds__(256) void issue_kernel(const char *src, int iterations, float *sink) {
+  __shared__ __attribute__((aligned(1024))) char ring[128 * 1024];  // (with 128 KiB a workgroup has its CU to itself)
+  constexpr int kMfmas = MF ? 64 : 128, kReadEvery = kMfmas / 32, kLoadEvery = kMfmas / 16;
+  constexpr uint32_t kWindow = 2u << 20, kChunksInWindow = kWindow / 1024;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint64_t bv = (uint64_t)(src + (uint64_t)(blockIdx.x % 8) * kWindow);
+  const uint32_t base_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)bv), base_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(bv >> 32));
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)base_hi << 32) | (uint64_t)base_lo), 0, (int)kWindow, 0x00020000);
+  uint32_t at = (uint32_t)(((blockIdx.x / 8) * 4 + wave) * (kChunksInWindow / 128) % kChunksInWindow);
+  f32x4 acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const u32x8 op8 = {0x38383838u + lane, 0x38383838u, 0x38383838u, 0x38383838u, 0x38383838u, 0x38383838u, 0x38383838u, 0x38383838u};
+  const u32x4 op4 = {0x3c003c00u + lane, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+  const uint32_t unit = 0x7f7f7f7fu, lds_rd = (uint32_t)(uintptr_t)ring + wave * 32768 + lane * 16, voff = lane * 16;
+  uint32_t filler = lane;
+  u32x4 r[8];
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int g = 0; g < kMfmas; ++g) {
+      if constexpr (MF) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0] cbsz:0 blgp:0" : "+a"(acc[g % 16]) : "v"(op8), "v"(op8), "v"(unit));
+      else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[g % 16]) : "v"(op4), "v"(op4));
+      if (g % kLoadEvery != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
+      if constexpr (FILL == 1) {
+#pragma unroll
+        for (int f = 0; f < COUNT; ++f) asm volatile("s_nop 0");
+      }
+      if constexpr (FILL == 2) {
+#pragma unroll
+        for (int f = 0; f < COUNT; ++f) asm volatile("v_mov_b32 %0, %1" : "=v"(filler) : "v"(lane));
+      }
+      if constexpr (FILL == 3) {
+        if (g % kReadEvery == 0 && g % kLoadEvery != 0) {  // (the read that would share a load's gap goes one gap on)
+          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r[(g / kReadEvery) % 8]) : "v"(lds_rd), "n"(((g / kReadEvery) % 16) * 1024));
+        } else if (g % kLoadEvery == 1) {
+          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r[(g / kReadEvery) % 8]) : "v"(lds_rd), "n"(((g / kReadEvery) % 16) * 1024));
+        }
+        if (g % kLoadEvery == 0) {
+          const int k = g / kLoadEvery;
+          const uint32_t chunk = at + k < kChunksInWindow ? at + k : at + k - kChunksInWindow;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(ring + wave * 32768 + 16384 + k * 1024), 16, voff,
+                                                   (int)(chunk * 1024), 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (FILL == 3) {
+      at = at + 16 < kChunksInWindow ? at + 16 : at + 16 - kChunksInWindow;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int k = 0; k < 8; ++k) asm volatile("" ::"v"(r[k]));
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (16 & 15) | ((16 >> 4) << 14));  // vmcnt(16): the previous tile's loads have landed
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // (the compiler does not see the in-place matrix instructions' results coming)
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += acc[i];
+  if (s[0] + s[1] + s[2] + s[3] == 12345.f) sink[blockIdx.x * 256 + threadIdx.x] = s[0] + (float)filler;
+}
+
+template <int MF>
+int launch_issue(int filler, int count, const char *src, int iterations, float *sink, int wgs, hipStream_t s) {
+#define KAPY_ISSUE(F, C) issue_kernel<MF, F, C><<<wgs, 256, 0, s>>>(src, iterations, sink)
+  if (filler == 0) KAPY_ISSUE(0, 0);
+  else if (filler == 3) KAPY_ISSUE(3, 0);
+  else if (filler == 1 && count == 1) KAPY_ISSUE(1, 1);
+  else if (filler == 1 && count == 2) KAPY_ISSUE(1, 2);
+  else if (filler == 1 && count == 3) KAPY_ISSUE(1, 3);
+  else if (filler == 1 && count == 4) KAPY_ISSUE(1, 4);
+  else if (filler == 1 && count == 6) KAPY_ISSUE(1, 6);
+  else if (filler == 1 && count == 8) KAPY_ISSUE(1, 8);
+  else if (filler == 2 && count == 1) KAPY_ISSUE(2, 1);
+  else if (filler == 2 && count == 2) KAPY_ISSUE(2, 2);
+  else if (filler == 2 && count == 3) KAPY_ISSUE(2, 3);
+  else if (filler == 2 && count == 4) KAPY_ISSUE(2, 4);
+  else return fail(KAPY_ERR_INVALID, "probe_issue: filler 0 (none), 1 (scalar; count 1, 2, 3, 4, 6 or 8), 2 (vector ALU; count 1 .. 4) or 3 (the tiled matmul's reads and loads)");
+#undef KAPY_ISSUE
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 template <int U>
 int launch_copy_nt(const void *src, void *dst, int64_t n, int nt_load, int nt_store, int persistent_per_cu, uint64_t *ticks, int32_t *workgroups, hipStream_t s) {
   if (nt_load && nt_store) return launch_copy<U, true, true>(src, dst, n, persistent_per_cu, ticks, workgroups, s);
@@ -258,6 +350,20 @@ int kapy_probe_l2_read(const void *src, int64_t window_bytes, int32_t iterations
   else l2_read_kernel<false><<<wgs, 256, 0, (hipStream_t)stream>>>((const char *)src, window_bytes, iterations, sink);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
+}
+
+int kapy_probe_issue(int32_t impl_way, int32_t filler, int32_t count, const void *src, int32_t iterations, float *sink, int32_t *workgroups, int64_t *flops,
+                     void *stream) {
+  if (!sink || iterations <= 0 || (filler == 3 && !src)) return fail(KAPY_ERR_INVALID, "probe_issue: null buffer or no iterations");
+  if (impl_way != KAPY_MFMA_16X16X32_16B && impl_way != KAPY_MFMA_16X16X128_F8) return fail(KAPY_ERR_INVALID, "probe_issue: 16x16x32 (16-bit) or 16x16x128 (f8) only");
+  int rc = ensure_device();
+  if (rc) return rc;
+  const int wgs = device_cus();
+  if (workgroups) *workgroups = wgs;
+  const bool f8 = impl_way == KAPY_MFMA_16X16X128_F8;
+  if (flops) *flops = (int64_t)wgs * 4 * iterations * (f8 ? 64 : 128) * (f8 ? 65536 : 16384);
+  return f8 ? launch_issue<1>(filler, count, (const char *)src, iterations, sink, wgs, (hipStream_t)stream)
+            : launch_issue<0>(filler, count, (const char *)src, iterations, sink, wgs, (hipStream_t)stream);
 }
 
 int kapy_probe_copy_tiled(const void *src, void *dst, int64_t rows, int64_t row_bytes, int32_t through_lds, void *stream) {

@@ -194,7 +194,10 @@ __global__ __launch_bounds__(WAVES * 64) void column_program_kernel(Program P, C
 
 // Throughput of this kernel follows the number of resident waves (each lane walks its program one
 // dependent step at a time), so the 16-bit-only form is held to 64 registers: 8 waves per SIMD.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void stack_kernel_narrow(StackProgram P) { stack_run<true>(P); }
+// (The operations whose code alone overruns 64 registers - remf, sin, cos - are left out of it; a program that holds one
+// runs the same machine without the cap.)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void stack_kernel_narrow(StackProgram P) { stack_run<true, false, true>(P); }
+__global__ __launch_bounds__(256) void stack_kernel_narrow_heavy(StackProgram P) { stack_run<true>(P); }
 __global__ __launch_bounds__(256) void stack_kernel_any(StackProgram P) { stack_run<false>(P); }
 // rows whose width is not a multiple of 8 (row starts still 16-byte aligned): the last vector of a row moves element by element
 __global__ __launch_bounds__(256) void stack_kernel_narrow_ragged(StackProgram P) { stack_run<true, true>(P); }
@@ -936,7 +939,10 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
       bool narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
       for (int k = 0; k < n_ins; ++k) narrow = narrow && (ins[k]->dtype == KAPY_F16 || ins[k]->dtype == KAPY_BF16);
       for (int k = 0; k < n_inst; ++k) narrow = narrow && !is_f8(result_dtype[k]);
+      bool heavy = false;
+      for (int k = 0; k < n_inst; ++k) heavy = heavy || prog[k].op == KAPY_EW_REMF || prog[k].op == KAPY_EW_SIN || prog[k].op == KAPY_EW_COS;
       if (narrow && SP.width) stack_kernel_narrow_ragged<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
+      else if (narrow && heavy) stack_kernel_narrow_heavy<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
       else if (narrow) stack_kernel_narrow<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
       else stack_kernel_any<<<dim3((unsigned)((slots + 255) / 256)), 256, 0, s>>>(SP);
       KAPY_HIP_CHECK(hipGetLastError());

@@ -52,6 +52,8 @@ __device__ __forceinline__ float gelu_tanh_f32(float v) {
   return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
 }
 
+// LEAN: without the operations whose code needs many registers (sin, cos): the register-capped 16-bit stack kernel
+template <bool LEAN = false>
 __device__ __forceinline__ float apply_unary(int op, float a) {
   switch (op) {
   case KAPY_EW_NEGF: return -a;
@@ -67,8 +69,12 @@ __device__ __forceinline__ float apply_unary(int op, float a) {
   case KAPY_EW_GELU_TANH: return gelu_tanh_f32(a);
   case KAPY_EW_FLOOR: return floorf(a);
   case KAPY_EW_CEIL: return ceilf(a);
-  case KAPY_EW_SIN: return sinf(a);
-  case KAPY_EW_COS: return cosf(a);
+  case KAPY_EW_SIN:
+    if constexpr (!LEAN) return sinf(a);
+    break;
+  case KAPY_EW_COS:
+    if constexpr (!LEAN) return cosf(a);
+    break;
   }
   return a;
 }
@@ -251,7 +257,7 @@ __device__ __forceinline__ void div8(const float (&x)[8], const float (&y)[8], f
 }
 
 // x[e] = op(x[e]) for a unary op whose result has element type dtype (rounding to that type is the caller's).
-template <bool NARROW>
+template <bool NARROW, bool LEAN = false>
 __device__ __forceinline__ void unary8(int op, int dtype, float (&x)[8]) {
   if (NARROW && op == KAPY_EW_EXP && dtype == KAPY_F32) {
     // exp(x) = 2^hi * (1 + lo*ln2), hi + lo = x*log2(e) with lo the product's rounding error: within 2 ulp of fp32,
@@ -268,14 +274,15 @@ __device__ __forceinline__ void unary8(int op, int dtype, float (&x)[8]) {
     return;
   }
 #pragma unroll
-  for (int e = 0; e < 8; ++e) x[e] = apply_unary(op, x[e]);
+  for (int e = 0; e < 8; ++e) x[e] = apply_unary<LEAN>(op, x[e]);
 }
 
 // One step with its result (and left operand) in value D, the right operand in value D+1 and the
 // third operand of an fma in value D+2; D is a template parameter so that no register is indexed.
 // NARROW: every operand, every intermediate type and the result are f16 / bf16 / f32-from-16-bit
 // (no fp8, no fp32 in memory): the common case, and it needs far fewer registers.
-template <int D, bool NARROW, bool RAGGED = false>
+// LEAN: without remf, sin and cos (see apply_unary); the host sends programs that hold one of them to a build with them.
+template <int D, bool NARROW, bool RAGGED = false, bool LEAN = false>
 __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &I, int32_t i, int32_t jv, float (&v)[3][8]) {
   constexpr int R = D + 1 < 3 ? D + 1 : 2, T = D + 2 < 3 ? D + 2 : 2;
   float *x = v[D];
@@ -357,19 +364,21 @@ __device__ __forceinline__ void stack_step(const StackProgram &P, const PostOp &
     for (int e = 0; e < 8; ++e) x[e] = min_num(x[e], y[e]);
     break;
   case KAPY_EW_REMF:
+    if constexpr (!LEAN) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = rem_f(x[e], y[e]);
+      for (int e = 0; e < 8; ++e) x[e] = rem_f(x[e], y[e]);
+    }
     break;
   case KAPY_EW_FMA:
 #pragma unroll
     for (int e = 0; e < 8; ++e) x[e] = fma_typed(x[e], y[e], z[e], I.dtype);
     break;
-  default: unary8<NARROW>(I.op, I.dtype, *(float (*)[8])x);
+  default: unary8<NARROW, LEAN>(I.op, I.dtype, *(float (*)[8])x);
   }
   if (I.dtype != KAPY_F32) round8<NARROW>(x, I.dtype, true);
 }
 
-template <bool NARROW, bool RAGGED = false>
+template <bool NARROW, bool RAGGED = false, bool LEAN = false>
 __device__ __forceinline__ void stack_run(const StackProgram &P) {
   const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (slot >= (int64_t)P.rows * P.vec_per_row) return;
@@ -382,9 +391,9 @@ __device__ __forceinline__ void stack_run(const StackProgram &P) {
   for (int pc = 0; pc < P.n_post; ++pc) {
     const PostOp I = P.post[pc];
     switch (I.slot) {
-    case 0: stack_step<0, NARROW, RAGGED>(P, I, i, jv, v); break;
-    case 1: stack_step<1, NARROW, RAGGED>(P, I, i, jv, v); break;
-    default: stack_step<2, NARROW, RAGGED>(P, I, i, jv, v);
+    case 0: stack_step<0, NARROW, RAGGED, LEAN>(P, I, i, jv, v); break;
+    case 1: stack_step<1, NARROW, RAGGED, LEAN>(P, I, i, jv, v); break;
+    default: stack_step<2, NARROW, RAGGED, LEAN>(P, I, i, jv, v);
     }
   }
 }

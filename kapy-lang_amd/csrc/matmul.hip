@@ -246,7 +246,8 @@ struct PackedEpilogue {
   // per element), a lane reads back 8 consecutive columns of a row, scales, narrows and stores 16 bytes.  The stores are
   // buffer stores through a descriptor of the wavefront's part of the result: it ends with the result's last row, so
   // the rows of a tile that hangs over the edge fall out of range in hardware, and a store costs one add.
-  template <bool F16, int EPI, typename Acc>
+  // OUT: the result's element type - 0 bf16, 1 f16, 2 f32 (stored as it is: two 16-byte pieces per lane).
+  template <int OUT, int EPI, typename Acc>
   static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip, int32_t m_wave, int32_t n_wave, int lane) {
     constexpr int kRowStrideF = WTN * 4 + 16, kChunksF = WTN / 8, kRowsPerPass = 64 / kChunksF, kPasses = 32 / kRowsPerPass;
     static_assert(32 * kRowStrideF <= kBytesPerWave && 64 % kChunksF == 0 && 32 % kRowsPerPass == 0, "fp32 strip geometry");
@@ -268,15 +269,16 @@ struct PackedEpilogue {
       for (int r = 0; r < kRowsPerLane; ++r)  // (rows past M exist only in tiles that hang over the edge; they are not stored)
         rs_all[r] = p.row_scale[min(m_wave + (r / kPasses) * 32 + (r % kPasses) * kRowsPerPass + rrow, p.M - 1)];
     }
-    const uint32_t pitch = (uint32_t)__builtin_amdgcn_readfirstlane((int)(p.d_sm * 2));
+    constexpr uint32_t kOutBytes = OUT == 2 ? 4 : 2;
+    const uint32_t pitch = (uint32_t)__builtin_amdgcn_readfirstlane((int)(p.d_sm * kOutBytes));
     const int32_t rows_left = min(WTM, p.M - m_wave), cols_left = min(WTN, p.N - n_wave);
-    const uint64_t bv = (uint64_t)(p.d + ((int64_t)m_wave * p.d_sm + n_wave) * 2);
+    const uint64_t bv = (uint64_t)(p.d + ((int64_t)m_wave * p.d_sm + n_wave) * kOutBytes);
     const uint32_t base_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)bv), base_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(bv >> 32));
-    const int32_t records = (rows_left > 0 && cols_left > 0) ? (int32_t)((uint32_t)(rows_left - 1) * pitch + (uint32_t)cols_left * 2u) : 0;
+    const int32_t records = (rows_left > 0 && cols_left > 0) ? (int32_t)((uint32_t)(rows_left - 1) * pitch + (uint32_t)cols_left * kOutBytes) : 0;
     const __amdgpu_buffer_rsrc_t d_rsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)base_hi << 32) | (uint64_t)base_lo), 0, __builtin_amdgcn_readfirstlane(records), 0x00020000);
     // (a lane whose columns lie past N asks for an offset beyond any descriptor)
-    const uint32_t voff0 = nn < p.N ? (uint32_t)rrow * pitch + (uint32_t)rchunk * 16u : 0x80000000u;
+    const uint32_t voff0 = nn < p.N ? (uint32_t)rrow * pitch + (uint32_t)rchunk * (8u * kOutBytes) : 0x80000000u;
 #pragma unroll
     for (int i = 0; i < kStrips; ++i) {
       __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
@@ -309,10 +311,19 @@ struct PackedEpilogue {
             v[4 + e] = __fmul_rn(v[4 + e], __fmul_rn(rs, cs_hi[e]));
           }
         }
-        u32x4 w;
+        const int voff = (int)(voff0 + (uint32_t)(i * 32 + t * kRowsPerPass) * pitch);
+        if constexpr (OUT == 2) {
+          u32x4 w0, w1;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = F16 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
-        __builtin_amdgcn_raw_buffer_store_b128(w, d_rsrc, (int)(voff0 + (uint32_t)(i * 32 + t * kRowsPerPass) * pitch), 0, 0);
+          for (int e = 0; e < 4; ++e) { w0[e] = __float_as_uint(v[e]); w1[e] = __float_as_uint(v[4 + e]); }
+          __builtin_amdgcn_raw_buffer_store_b128(w0, d_rsrc, voff, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(w1, d_rsrc, voff, 16, 0);  // (the scalar offset is outside the range check: the piece is in or out whole)
+        } else {
+          u32x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = OUT == 1 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
+          __builtin_amdgcn_raw_buffer_store_b128(w, d_rsrc, voff, 0, 0);
+        }
       }
     }
   }
@@ -320,7 +331,7 @@ struct PackedEpilogue {
   // gives up keeping the accumulators in registers, for the whole kernel), so the strip goes through LDS as fp32 - one strip
   // of 32 x (WTN*4 + 16) bytes fits the two 16-bit strips' space - and a rolled loop applies the tail to 8 consecutive
   // columns per lane on the way out, narrows and stores 16 bytes.
-  template <bool F16, typename Acc>
+  template <int OUT, typename Acc>
   static __device__ __forceinline__ void strips_tail(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip, int32_t m_wave, int32_t n_wave, int lane) {
     constexpr int kRowStrideF = WTN * 4 + 16, kChunksF = WTN / 8, kRowsPerPass = 64 / kChunksF, kPasses = 32 / kRowsPerPass;
     static_assert(32 * kRowStrideF <= kBytesPerWave && 64 % kChunksF == 0 && 32 % kRowsPerPass == 0, "fp32 strip geometry");
@@ -358,11 +369,19 @@ struct PackedEpilogue {
 #pragma unroll
         for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
         apply_tail8(p, v, bias);
-        u32x4 w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = F16 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
         // (N a multiple of 8: a piece of 8 columns is in or out whole)
-        if (mm < p.M && nn < p.N) *(u32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 2) = w;
+        if constexpr (OUT == 2) {
+          if (mm < p.M && nn < p.N) {
+            f32x4 *dst = (f32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 4);
+            dst[0] = f32x4{v[0], v[1], v[2], v[3]};
+            dst[1] = f32x4{v[4], v[5], v[6], v[7]};
+          }
+        } else {
+          u32x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = OUT == 1 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
+          if (mm < p.M && nn < p.N) *(u32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 2) = w;
+        }
       }
     }
   }
@@ -371,16 +390,19 @@ struct PackedEpilogue {
   // push the main loop's accumulators out of registers).
   template <bool TAIL = false, typename Acc>
   static __device__ __forceinline__ void run(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip0, int32_t m_wave, int32_t n_wave, int lane) {
-    const bool f16 = p.d_dtype == KAPY_F16;
+    const int out = p.d_dtype == KAPY_F32 ? 2 : p.d_dtype == KAPY_F16 ? 1 : 0;
     if constexpr (TAIL) {
-      if (f16) strips_tail<true>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips_tail<false>(p, acc, strip0, m_wave, n_wave, lane);
+      if (out == 2) strips_tail<2>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips_tail<1>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips_tail<0>(p, acc, strip0, m_wave, n_wave, lane);
     } else if (p.row_scale) {
-      if (f16) strips<true, 1>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips<false, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      if (out == 2) strips<2, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips<1, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<0, 1>(p, acc, strip0, m_wave, n_wave, lane);
     } else {
-      if (f16) strips<true, 0>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips<false, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      if (out == 2) strips<2, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips<1, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<0, 0>(p, acc, strip0, m_wave, n_wave, lane);
     }
   }
 };
@@ -729,7 +751,9 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     // pipe runs dry, and a vector ALU instruction takes 8 of them, a scalar or LDS or memory instruction 4 to 8.  The
     // steady-state loop therefore computes no address: a read at a compile-time ring position is one of three copies of the
     // lane's fragment offset (the 160 KiB ring seen as 64 KiB windows, the reach of a read's immediate) plus an immediate.
-    constexpr int kWindows = (C::kLdsBytes + 65535) / 65536;
+    // (The build for a partial last K-tile has no registers to spare for the copies: it forms the addresses as before.)
+    constexpr bool kUseWindows = !KTAIL;
+    constexpr int kWindows = kUseWindows ? (C::kLdsBytes + 65535) / 65536 : 1;
     // (a tile's units start at an even ring position, so the wave's own unit - wm for the lhs, wn for the rhs - never
     // wraps on its own and can sit in the register part: one set of copies per operand)
     uint32_t frag_win[2][kWindows][KK][CH];
@@ -749,6 +773,8 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     auto read_at = [&](int o, auto at, uint32_t rows, int kk, int c) -> u32x4 {
       if constexpr (std::is_integral_v<decltype(at)>) {
         return *(const u32x4 *)(lds + (at + (o ? wn : wm) * kUnit + frag_off[kk][c]) + rows);
+      } else if constexpr (!kUseWindows) {
+        return *(const u32x4 *)(lds + (decltype(at)::value + (o ? wn : wm) * kUnit + frag_off[kk][c]) + rows);
       } else {
         const uint32_t v = decltype(at)::value + rows;
         return *(const __attribute__((address_space(3))) u32x4 *)(uintptr_t)(frag_win[o][v >> 16][kk][c] + (v & 65535u));
@@ -861,7 +887,7 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
         for (int g = 0; g < kMfmas; ++g) {
           const int i = g / C::kTn, j = g % C::kTn;
           acc[i][j] = T::mfma(b_cur[j].c, a_cur[i].c, acc[i][j]);
-          if (g % kLoadSpacing != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
+          if (KTAIL || g % kLoadSpacing != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
 #pragma unroll
           for (int t = 0; t < kReadsPerMfma; ++t) {
             // (kSpread: one read per gap, and none in the gaps that carry a load - see the two-pass step)
@@ -1381,10 +1407,12 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
 // ---------------------------------------------------------------------------------------------
 // Host side.
 constexpr int kMaxDevices = 64;  // device ordinals that get a slot in the per-device tables below
-// 16-bit row-major result with 16-byte aligned rows, no accumulator input, RN: the packed epilogue.
+// 16-bit (RN) or fp32 row-major result with 16-byte aligned rows, no accumulator input: the packed epilogue.
 bool packed_epilogue(const GemmParams &p) {
-  return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16) && p.d_sn == 1 && p.acc_dtype < 0 && !p.rz &&
-         ((uintptr_t)p.d & 15) == 0 && (p.d_sm * 2) % 16 == 0 && (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
+  const int64_t eb = p.d_dtype == KAPY_F32 ? 4 : 2;
+  return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16 || p.d_dtype == KAPY_F32) && p.d_sn == 1 && p.acc_dtype < 0 && (!p.rz || p.d_dtype == KAPY_F32) &&
+         ((uintptr_t)p.d & 15) == 0 && (p.d_sm * eb) % 16 == 0 && p.d_sm * eb * 256 < (int64_t(1) << 31) &&  // (a wave's rows are addressed with 32-bit offsets)
+         (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool PACKED, bool KTAIL = false, bool TAIL = false>
@@ -1443,7 +1471,7 @@ int launch_staged(GemmParams p, int a_mode, int b_mode, hipStream_t s) {
   p.tiles_n = (p.N + kSBN - 1) / kSBN;
   p.split_k = 1;
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
-  if (packed_epilogue(p)) staged_kernel<T, true><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
+  if (packed_epilogue(p) && p.d_dtype != KAPY_F32) staged_kernel<T, true><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);  // (its packed stores are 16-bit)
   else staged_kernel<T, false><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;

@@ -221,3 +221,26 @@ def test_extents_that_are_not_multiples_of_the_tile_stay_on_the_ring_kernel(ko, 
         kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd2, M, N, N, 1, dt), tile=tile, stages=25)
         sync()
         assert _frob(ko, to_host(dd2, np.uint16), want, dt) <= FROB_TOL, tile
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 512, 256), (513, 264, 192), (257, 256, 72), (1000, 1000, 128), (130, 136, 64)])
+def test_f32_result_takes_the_strip_epilogue_and_writes_nothing_outside(ko, M, N, K):
+    """A row-major fp32 result (16-byte aligned rows, no accumulator input) is stored by the same strips through LDS as a
+    16-bit one, 32 bytes per lane; tiles that hang over the result's last rows and columns must leave the words behind it
+    alone, and a result window inside a wider buffer must leave the columns beside it alone."""
+    dt = kh.BF16
+    a, b = ko.fill_normal(M * K, dt, 11, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 11, 1, 0.0, 0.5)
+    want = np.zeros(M * N, dtype=np.float32)
+    assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, K, 1, dt)), C.byref(ko.mk_global(b, K, N, 1, K, dt)), None,
+                              C.byref(ko.mk_global(want, M, N, N, 1, kh.F32)), kh.RN) == 0
+    da, db = to_dev(a), to_dev(b)
+    for tile, stages in (((0, 0, 0), 0), ((256, 256, 64), 25), ((128, 128, 64), 25)):
+        pitch = N + 16    # the result is a window of a wider buffer
+        dd = dev_zeros(M * pitch + 64, 4, fill=0x12345678)
+        kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd, M, N, pitch, 1, kh.F32), tile=tile, stages=stages)
+        sync()
+        got = to_host(dd, np.uint32)
+        assert np.all(got[M * pitch:] == 0x12345678), tile
+        rows = got[:M * pitch].reshape(M, pitch)
+        assert np.all(rows[:, N:] == 0x12345678), tile
+        assert _frob(ko, np.ascontiguousarray(rows[:, :N]).view(np.float32).reshape(-1), want, kh.F32) <= 1e-5, tile

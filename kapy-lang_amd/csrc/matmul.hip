@@ -247,7 +247,9 @@ struct PackedEpilogue {
   // buffer stores through a descriptor of the wavefront's part of the result: it ends with the result's last row, so
   // the rows of a tile that hangs over the edge fall out of range in hardware, and a store costs one add.
   // OUT: the result's element type - 0 bf16, 1 f16, 2 f32 (stored as it is: two 16-byte pieces per lane).
-  template <int OUT, int EPI, typename Acc>
+  // ACC: an accumulator input added at the end - 0 none, 1 f16, 2 f32 (row-major, rows 16-byte aligned), fetched a strip ahead
+  // of its use through a descriptor bounded like the result's.
+  template <int OUT, int EPI, int ACC, typename Acc>
   static __device__ __forceinline__ void strips(const GemmParams &p, Acc (&acc)[WTM / KM][WTN / KM], char *strip, int32_t m_wave, int32_t n_wave, int lane) {
     constexpr int kRowStrideF = WTN * 4 + 16, kChunksF = WTN / 8, kRowsPerPass = 64 / kChunksF, kPasses = 32 / kRowsPerPass;
     static_assert(32 * kRowStrideF <= kBytesPerWave && 64 % kChunksF == 0 && 32 % kRowsPerPass == 0, "fp32 strip geometry");
@@ -279,9 +281,27 @@ struct PackedEpilogue {
         __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)base_hi << 32) | (uint64_t)base_lo), 0, __builtin_amdgcn_readfirstlane(records), 0x00020000);
     // (a lane whose columns lie past N asks for an offset beyond any descriptor)
     const uint32_t voff0 = nn < p.N ? (uint32_t)rrow * pitch + (uint32_t)rchunk * (8u * kOutBytes) : 0x80000000u;
+    // the accumulator input, if any: the same geometry in its own element size
+    constexpr uint32_t kAccBytes = ACC == 2 ? 4 : 2;
+    const uint32_t apitch = ACC ? (uint32_t)__builtin_amdgcn_readfirstlane((int)(p.acc_sm * kAccBytes)) : 0;
+    const uint64_t av = ACC ? (uint64_t)(p.acc + ((int64_t)m_wave * p.acc_sm + n_wave) * kAccBytes) : 0;
+    const uint32_t abase_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)av), abase_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(av >> 32));
+    const int32_t arecords = (ACC && rows_left > 0 && cols_left > 0) ? (int32_t)((uint32_t)(rows_left - 1) * apitch + (uint32_t)cols_left * kAccBytes) : 0;
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)abase_hi << 32) | (uint64_t)abase_lo), 0, __builtin_amdgcn_readfirstlane(arecords), 0x00020000);
+    const uint32_t avoff0 = nn < p.N ? (uint32_t)rrow * apitch + (uint32_t)rchunk * (8u * kAccBytes) : 0x80000000u;
+    u32x4 acc_in[ACC ? kPasses : 1][ACC == 2 ? 2 : 1];
 #pragma unroll
     for (int i = 0; i < kStrips; ++i) {
       __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
+      if constexpr (ACC != 0) {
+#pragma unroll
+        for (int t = 0; t < kPasses; ++t) {
+          const int avoff = (int)(avoff0 + (uint32_t)(i * 32 + t * kRowsPerPass) * apitch);
+          acc_in[t][0] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, avoff, 0, 0);
+          if constexpr (ACC == 2) acc_in[t][1] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, avoff, 16, 0);
+        }
+      }
 #pragma unroll
       for (int bi = 0; bi < kBlocksPerStrip; ++bi)
 #pragma unroll
@@ -309,6 +329,19 @@ struct PackedEpilogue {
           for (int e = 0; e < 4; ++e) {
             v[e] = __fmul_rn(v[e], __fmul_rn(rs, cs_lo[e]));
             v[4 + e] = __fmul_rn(v[4 + e], __fmul_rn(rs, cs_hi[e]));
+          }
+        }
+        if constexpr (ACC == 2) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = __fadd_rn(v[e], __uint_as_float(acc_in[t][0][e]));
+            v[4 + e] = __fadd_rn(v[4 + e], __uint_as_float(acc_in[t][1][e]));
+          }
+        } else if constexpr (ACC == 1) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[2 * e] = __fadd_rn(v[2 * e], f16_to_f32((uint16_t)(acc_in[t][0][e] & 0xffffu)));
+            v[2 * e + 1] = __fadd_rn(v[2 * e + 1], f16_to_f32((uint16_t)(acc_in[t][0][e] >> 16)));
           }
         }
         const int voff = (int)(voff0 + (uint32_t)(i * 32 + t * kRowsPerPass) * pitch);
@@ -396,13 +429,21 @@ struct PackedEpilogue {
       else if (out == 1) strips_tail<1>(p, acc, strip0, m_wave, n_wave, lane);
       else strips_tail<0>(p, acc, strip0, m_wave, n_wave, lane);
     } else if (p.row_scale) {
-      if (out == 2) strips<2, 1>(p, acc, strip0, m_wave, n_wave, lane);
-      else if (out == 1) strips<1, 1>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips<0, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      if (out == 2) strips<2, 1, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips<1, 1, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<0, 1, 0>(p, acc, strip0, m_wave, n_wave, lane);
+    } else if (p.acc_dtype == KAPY_F32) {
+      if (out == 2) strips<2, 0, 2>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips<1, 0, 2>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<0, 0, 2>(p, acc, strip0, m_wave, n_wave, lane);
+    } else if (p.acc_dtype == KAPY_F16) {
+      if (out == 2) strips<2, 0, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips<1, 0, 1>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<0, 0, 1>(p, acc, strip0, m_wave, n_wave, lane);
     } else {
-      if (out == 2) strips<2, 0>(p, acc, strip0, m_wave, n_wave, lane);
-      else if (out == 1) strips<1, 0>(p, acc, strip0, m_wave, n_wave, lane);
-      else strips<0, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      if (out == 2) strips<2, 0, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else if (out == 1) strips<1, 0, 0>(p, acc, strip0, m_wave, n_wave, lane);
+      else strips<0, 0, 0>(p, acc, strip0, m_wave, n_wave, lane);
     }
   }
 };
@@ -1407,10 +1448,15 @@ __global__ __launch_bounds__(256) void staged_kernel(GemmParams p, int a_mode, i
 // ---------------------------------------------------------------------------------------------
 // Host side.
 constexpr int kMaxDevices = 64;  // device ordinals that get a slot in the per-device tables below
-// 16-bit (RN) or fp32 row-major result with 16-byte aligned rows, no accumulator input: the packed epilogue.
+bool host_has_tail(const GemmParams &p) { return p.bias != nullptr || p.act >= 0 || p.alpha != 1.0f; }
+
+// 16-bit (RN) or fp32 row-major result with 16-byte aligned rows: the packed epilogue.
 bool packed_epilogue(const GemmParams &p) {
-  const int64_t eb = p.d_dtype == KAPY_F32 ? 4 : 2;
-  return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16 || p.d_dtype == KAPY_F32) && p.d_sn == 1 && p.acc_dtype < 0 && (!p.rz || p.d_dtype == KAPY_F32) &&
+  const int64_t eb = p.d_dtype == KAPY_F32 ? 4 : 2, ab = p.acc_dtype == KAPY_F32 ? 4 : 2;
+  // an accumulator input: f16 or f32, row-major with 16-byte aligned rows, and neither scales nor a fused tail beside it
+  const bool acc_ok = p.acc_dtype < 0 || ((p.acc_dtype == KAPY_F16 || p.acc_dtype == KAPY_F32) && p.acc_sn == 1 && ((uintptr_t)p.acc & 15) == 0 &&
+                                          (p.acc_sm * ab) % 16 == 0 && p.acc_sm * ab * 256 < (int64_t(1) << 31) && !p.row_scale && !host_has_tail(p));
+  return (p.d_dtype == KAPY_F16 || p.d_dtype == KAPY_BF16 || p.d_dtype == KAPY_F32) && p.d_sn == 1 && acc_ok && (!p.rz || p.d_dtype == KAPY_F32) &&
          ((uintptr_t)p.d & 15) == 0 && (p.d_sm * eb) % 16 == 0 && p.d_sm * eb * 256 < (int64_t(1) << 31) &&  // (a wave's rows are addressed with 32-bit offsets)
          (!p.row_scale || ((uintptr_t)p.col_scale & 15) == 0);
 }
@@ -1428,7 +1474,6 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
   return KAPY_OK;
 }
 
-bool host_has_tail(const GemmParams &p) { return p.bias != nullptr || p.act >= 0 || p.alpha != 1.0f; }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 int launch_tn(const GemmParams &p, hipStream_t s) {
@@ -1471,7 +1516,7 @@ int launch_staged(GemmParams p, int a_mode, int b_mode, hipStream_t s) {
   p.tiles_n = (p.N + kSBN - 1) / kSBN;
   p.split_k = 1;
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
-  if (packed_epilogue(p) && p.d_dtype != KAPY_F32) staged_kernel<T, true><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);  // (its packed stores are 16-bit)
+  if (packed_epilogue(p) && p.d_dtype != KAPY_F32 && p.acc_dtype < 0) staged_kernel<T, true><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);  // (its packed stores are 16-bit, without accumulator input)
   else staged_kernel<T, false><<<grid, dim3(256), 0, s>>>(p, a_mode, b_mode);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;

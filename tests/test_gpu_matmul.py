@@ -244,3 +244,25 @@ def test_f32_result_takes_the_strip_epilogue_and_writes_nothing_outside(ko, M, N
         rows = got[:M * pitch].reshape(M, pitch)
         assert np.all(rows[:, N:] == 0x12345678), tile
         assert _frob(ko, np.ascontiguousarray(rows[:, :N]).view(np.float32).reshape(-1), want, kh.F32) <= 1e-5, tile
+
+
+@pytest.mark.parametrize("acc_dt,out_dt", [(kh.F32, kh.F32), (kh.F32, kh.BF16), (kh.F16, kh.F16), (kh.F16, kh.F32)])
+@pytest.mark.parametrize("M,N,K", [(512, 512, 256), (300, 264, 192)])
+def test_accumulator_input_through_the_strip_epilogue(ko, acc_dt, out_dt, M, N, K):
+    """result = lhs x rhs + acc with a row-major acc whose rows are 16-byte aligned: the strip epilogue fetches the lane's 8
+    acc values a strip ahead and adds them in fp32 before the final rounding; ragged extents drop out in the descriptors."""
+    dt = kh.F16 if out_dt == kh.F16 or acc_dt == kh.F16 else kh.BF16
+    a, b = ko.fill_normal(M * K, dt, 13, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 13, 1, 0.0, 0.5)
+    acc = ko.fill_normal(M * N, acc_dt, 13, 2)
+    want = np.zeros(M * N, dtype=_np_store(out_dt))
+    assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, K, 1, dt)), C.byref(ko.mk_global(b, K, N, 1, K, dt)), C.byref(ko.mk_global(acc, M, N, N, 1, acc_dt)),
+                              C.byref(ko.mk_global(want, M, N, N, 1, out_dt)), kh.RN) == 0
+    da, db, dacc = to_dev(a), to_dev(b), to_dev(acc)
+    for tile, stages in (((0, 0, 0), 0), ((256, 256, 64), 25), ((128, 128, 64), 25)):
+        dd = dev_zeros(M * N + 64, kh.DTYPE_BYTES[out_dt], fill=0x1234)
+        kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd, M, N, N, 1, out_dt), acc=dglobal(dacc, M, N, N, 1, acc_dt),
+                  tile=tile, stages=stages)
+        sync()
+        got = to_host(dd, want.dtype.type if out_dt != kh.F32 else np.float32)
+        assert np.all(to_host(dd, np.uint16 if out_dt != kh.F32 else np.uint32)[M * N:] == 0x1234), tile
+        assert _frob(ko, got[:M * N], want, out_dt) <= (1e-5 if out_dt == kh.F32 else FROB_TOL), tile

@@ -1266,7 +1266,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
       for (int g = 0; g < kMfmas; ++g) {
         const int i = g / kTn, j = g % kTn;
         const u32x4 b_op = {b_cur.h0[j][0], b_cur.h0[j][1], b_cur.h1[j][0], b_cur.h1[j][1]};
-        acc[i][j] = T::mfma(&b_op, a_cur[i].c, acc[i][j]);
+        T::mfma_in_place(&b_op, a_cur[i].c, acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         if (g < kReads) {
           const int rs = kk + 1 < KK ? stage : next_stage, rk = kk + 1 < KK ? kk + 1 : 0;
@@ -1289,6 +1289,9 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   }
   if (kt < KT) tile_step(kt, P0{});
   __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
+  // the in-place matrix instructions are opaque to the compiler, which therefore does not count the wait states their
+  // results need before another kind of instruction may read the accumulators
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
   __builtin_amdgcn_s_barrier();  // every wave has left the ring: it is reused as staging space by the packed epilogue
   if (p.split_k > 1 && !split_k_meet<256>(p, tm + tn * p.tiles_m, split, acc, m0 + wm * 64, 16, (uint32_t *)lds)) return;
   if constexpr (PACKED) {

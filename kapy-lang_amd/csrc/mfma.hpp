@@ -56,6 +56,12 @@ struct Bf16M16 {
   static __device__ __forceinline__ f32x4 mfma(const u32x4 *a, const u32x4 *b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
   }
+  // The same instruction accumulating in place in an accumulator register (see F8M16::mfma_in_place): where registers are
+  // not scarce the compiler moves accumulators between the two halves of the register file around the instruction,
+  // several vector moves per matrix instruction, which the matrix pipe then waits for.
+  static __device__ __forceinline__ void mfma_in_place(const u32x4 *a, const u32x4 *b, f32x4 &c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a[0]), "v"(b[0]));
+  }
 };
 struct F16M16 {
   static constexpr int kBytes = 2, kSliceK = 32, kChunks = 1, kMfmaClocks = 16, kM = 16;
@@ -63,6 +69,12 @@ struct F16M16 {
   using Acc = f32x4;
   static __device__ __forceinline__ f32x4 mfma(const u32x4 *a, const u32x4 *b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
+  }
+  // The same instruction accumulating in place in an accumulator register (see F8M16::mfma_in_place): where registers are
+  // not scarce the compiler moves accumulators between the two halves of the register file around the instruction,
+  // several vector moves per matrix instruction, which the matrix pipe then waits for.
+  static __device__ __forceinline__ void mfma_in_place(const u32x4 *a, const u32x4 *b, f32x4 &c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a[0]), "v"(b[0]));
   }
 };
 // OCP fp8, v_mfma_scale_f32_32x32x64_f8f6f4 with unit block scales (E8M0 127 = 2^0).  AF / BF are the

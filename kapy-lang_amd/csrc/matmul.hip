@@ -25,6 +25,7 @@
 //                  on the way when an operand is contiguous along M/N.  128x128x32 tiles.
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 #include "common.hpp"
 #include "layout.hpp"
@@ -90,6 +91,14 @@ __device__ __forceinline__ u32x2_lds tr_read_b64(const char *lds_ptr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(r) : "v"(addr));
   return r;
 }
+// The same from LDS byte address `addr` + IMM (below 64 KiB), the immediate in the instruction: no address arithmetic.
+template <uint32_t IMM>
+__device__ __forceinline__ u32x2_lds tr_read_b64_at(uint32_t addr) {
+  static_assert(IMM < 65536, "a DS instruction's offset field has 16 bits");
+  u32x2_lds r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(IMM));
+  return r;
+}
 // Waits for the transposing reads whose results sit in h0[j], h1[j] (j < 4) and hands those registers back as its own results.
 __device__ __forceinline__ void tr_reads_wait(u32x2_lds (&h0)[4], u32x2_lds (&h1)[4]) {
   asm volatile("s_waitcnt lgkmcnt(0)"
@@ -97,6 +106,12 @@ __device__ __forceinline__ void tr_reads_wait(u32x2_lds (&h0)[4], u32x2_lds (&h1
                :
                : "memory");
 }
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose counter is a compile-time constant in the body
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 
 // s_waitcnt immediate that waits only on vmcnt <= n (gfx9 encoding: vmcnt in bits [3:0] and [15:14],
 // expcnt [6:4] and lgkmcnt [11:8] left at "no wait").
@@ -1218,11 +1233,35 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     u32x2_lds h0[kTn], h1[kTn];
   };
   static_assert(kTn == 4, "tr_reads_wait takes the halves of four fragments");
-  auto read_a = [&](int stage, int kk, int i) { return *(const u32x4 *)(lds + stage * kStage + a_off[kk] + i * 16 * kRowA); };
-  auto read_b = [&](int stage, int kk, int j, FragHalves &dst) {
-    const char *base = lds + stage * kStage + b_off[j] + kk * 32 * kRowB;
-    dst.h0[j] = tr_read_b64(base);
-    dst.h1[j] = tr_read_b64(base + 4 * kRowB);
+  // Every operand read of the main loop is `register + immediate`: the stage is a compile-time constant there (the loop is
+  // unrolled over the ring), and where the ring is longer than a read's 64 KiB immediate reaches, the per-lane offsets
+  // are kept once per 64 KiB window (a vector add per read would cost the matrix pipe more than the read itself).
+  constexpr int kWindows = (STAGES * kStage + 65535) / 65536;
+  uint32_t a_win[kWindows][KK], b_win[kWindows][kTn];
+#pragma unroll
+  for (int w = 0; w < kWindows; ++w) {
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      uint32_t v = (uint32_t)(uintptr_t)lds + a_off[kk] + (uint32_t)w * 65536u;
+      asm volatile("" : "+v"(v));  // (opaque: registers that stay, not one register and an add at every read)
+      a_win[w][kk] = v;
+    }
+#pragma unroll
+    for (int j = 0; j < kTn; ++j) {
+      uint32_t v = (uint32_t)(uintptr_t)lds + b_off[j] + (uint32_t)w * 65536u;
+      asm volatile("" : "+v"(v));
+      b_win[w][j] = v;
+    }
+  }
+  auto read_a = [&](auto stage, auto kk, int i) {
+    constexpr uint32_t at = decltype(stage)::value * kStage;
+    const uint32_t c = at + (uint32_t)i * 16 * kRowA;
+    return *(const __attribute__((address_space(3))) u32x4 *)(uintptr_t)(a_win[c >> 16][decltype(kk)::value] + (c & 65535u));
+  };
+  auto read_b = [&](auto stage, auto kk, auto j, FragHalves &dst) {
+    constexpr uint32_t c0 = decltype(stage)::value * kStage + decltype(kk)::value * 32 * kRowB, c1 = c0 + 4 * kRowB;
+    dst.h0[decltype(j)::value] = tr_read_b64_at<(c0 & 65535u)>(b_win[c0 >> 16][decltype(j)::value]);
+    dst.h1[decltype(j)::value] = tr_read_b64_at<(c1 & 65535u)>(b_win[c1 >> 16][decltype(j)::value]);
   };
 
   using Acc = typename T::Acc;
@@ -1240,54 +1279,55 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   __builtin_amdgcn_s_barrier();  // tile 0 published
   Frag af[2][kTm];
   FragHalves bf[2];
-#pragma unroll
-  for (int i = 0; i < kTm; ++i) af[0][i].c[0] = read_a(0, 0, i);
-#pragma unroll
-  for (int j = 0; j < kTn; ++j) read_b(0, 0, j, bf[0]);
+  using Zero = std::integral_constant<int, 0>;
+  static_for<kTm>([&](auto i) { af[0][decltype(i)::value].c[0] = read_a(Zero{}, Zero{}, decltype(i)::value); });
+  static_for<kTn>([&](auto j) { read_b(Zero{}, Zero{}, j, bf[0]); });
 
   constexpr int kReads = kTm + kTn;
   constexpr int kLoadSpacing = (KK * kMfmas) / kLoads;  // matrix instructions between two loads
-  static_assert(kLoadSpacing >= 1, "");
-  int stage = 0;
-  // One K-tile.  `parity` says which fragment buffer holds slice 0 of this tile: with an odd number
-  // of slices per tile it alternates from tile to tile (compile-time, the loop is unrolled by two).
-  auto tile_step = [&](int kt, auto parity) {
-    const int next_stage = stage + 1 == STAGES ? 0 : stage + 1, free_stage = stage == 0 ? STAGES - 1 : stage - 1;
+  static_assert(kLoadSpacing >= 2 && kReads <= kMfmas - (kMfmas + kLoadSpacing - 1) / kLoadSpacing, "a slice has a gap without a load for each of its reads");
+  // One K-tile in ring stage STAGE (a type: every LDS address of the step is then a constant).  `parity` says which
+  // fragment buffer holds slice 0 of this tile: with an odd number of slices per tile it alternates from tile to tile.
+  // What goes behind which matrix instruction follows the tiled kernel's rule: a read never shares a gap with a load,
+  // and a load's gap is left to the scheduler, which moves the M0 write ahead of the matrix instruction.
+  auto tile_step = [&](int kt, auto stage_c, auto parity) {
+    constexpr int stage = decltype(stage_c)::value, par = decltype(parity)::value;
+    constexpr int next_stage = stage + 1 == STAGES ? 0 : stage + 1, free_stage = stage == 0 ? STAGES - 1 : stage - 1;
     // own loads of tile kt+1 have landed once only the younger tiles' loads remain in flight
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kLoads * (STAGES - 3)));
     __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      constexpr int par = decltype(parity)::value;
+    static_for<KK>([&](auto kk_c) {
+      constexpr int kk = decltype(kk_c)::value;
       Frag *a_cur = af[(kk + par) & 1], *a_nxt = af[(kk + par + 1) & 1];
       FragHalves &b_cur = bf[(kk + par) & 1], &b_nxt = bf[(kk + par + 1) & 1];
       tr_reads_wait(b_cur.h0, b_cur.h1);  // the rhs fragments of this slice were requested during the previous one
-#pragma unroll
-      for (int g = 0; g < kMfmas; ++g) {
-        const int i = g / kTn, j = g % kTn;
+      static_for<kMfmas>([&](auto g_c) {
+        constexpr int g = decltype(g_c)::value, i = g / kTn, j = g % kTn;
+        constexpr bool load_here = (kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads;
         const u32x4 b_op = {b_cur.h0[j][0], b_cur.h0[j][1], b_cur.h1[j][0], b_cur.h1[j][1]};
         T::mfma_in_place(&b_op, a_cur[i].c, acc[i][j]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (g < kReads) {
-          const int rs = kk + 1 < KK ? stage : next_stage, rk = kk + 1 < KK ? kk + 1 : 0;
-          if (g < kTm) a_nxt[g].c[0] = read_a(rs, rk, g);
-          else read_b(rs, rk, g - kTm, b_nxt);
+        if constexpr (!load_here) __builtin_amdgcn_sched_barrier(0);
+        constexpr int r = load_here ? -1 : g - (g + 1) / kLoadSpacing;  // this gap's read: the gaps without a load, in order
+        if constexpr (r >= 0 && r < kReads) {
+          using RS = std::integral_constant<int, (kk + 1 < KK ? stage : next_stage)>;
+          using RK = std::integral_constant<int, (kk + 1 < KK ? kk + 1 : 0)>;
+          if constexpr (r < kTm) a_nxt[r].c[0] = read_a(RS{}, RK{}, r);
+          else read_b(RS{}, RK{}, std::integral_constant<int, r - kTm>{}, b_nxt);
         }
-        if ((kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads)
-          issue_load(kt + STAGES - 1, free_stage, (kk * kMfmas + g) / kLoadSpacing);
+        if constexpr (load_here) issue_load(kt + STAGES - 1, free_stage, (kk * kMfmas + g) / kLoadSpacing);
         __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    stage = next_stage;
+      });
+    });
   };
-  using P0 = std::integral_constant<int, 0>;
-  using P1 = std::integral_constant<int, KK & 1>;
+  // the loop is unrolled over the ring (and over the fragment-buffer parity)
+  constexpr int kUnroll = (KK & 1) && (STAGES & 1) ? 2 * STAGES : STAGES;
   int kt = 0;
-  for (; kt + 2 <= KT; kt += 2) {
-    tile_step(kt, P0{});
-    tile_step(kt + 1, P1{});
-  }
-  if (kt < KT) tile_step(kt, P0{});
+  for (; kt + kUnroll <= KT; kt += kUnroll)
+    static_for<kUnroll>([&](auto u) { tile_step(kt + decltype(u)::value, std::integral_constant<int, decltype(u)::value % STAGES>{}, std::integral_constant<int, (decltype(u)::value * KK) & 1>{}); });
+  static_for<kUnroll - 1>([&](auto u) {
+    if (kt + decltype(u)::value < KT)
+      tile_step(kt + decltype(u)::value, std::integral_constant<int, decltype(u)::value % STAGES>{}, std::integral_constant<int, (decltype(u)::value * KK) & 1>{});
+  });
   __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
   // the in-place matrix instructions are opaque to the compiler, which therefore does not count the wait states their
   // results need before another kind of instruction may read the accumulators

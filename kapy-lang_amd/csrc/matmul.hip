@@ -1200,15 +1200,18 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * 2), 0, 0x7fffffff, 0x00020000);
   const int wave_lds = wave * 1024;
   // load `idx` (lhs first, then rhs) of K-tile j into its stage
-  auto issue_load = [&](int j, int stage, int idx) {
-    const int jc = min(j, KT - 1);
+  // (the scalar offsets of K-tile j, clamped to the last tile: loads past the end of K are still issued, into stages nobody reads)
+  auto soff_a_of = [&](int j) { return min(j, KT - 1) * (BK * 2); };
+  auto soff_b_of = [&](int j) { return min(j, KT - 1) * BK * ldb * 2; };
+  auto issue_load_at = [&](int soff_a, int soff_b, int stage, int idx) {
     if (idx < kLoadsA)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + idx * 4096 + wave_lds), 16,
-                                               (int)a_goff[idx], jc * (BK * 2), 0, 0);
+                                               (int)a_goff[idx], soff_a, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + kBytesA + (idx - kLoadsA) * 4096 + wave_lds),
-                                               16, (int)b_goff[idx - kLoadsA], jc * BK * ldb * 2, 0, 0);
+                                               16, (int)b_goff[idx - kLoadsA], soff_b, 0, 0);
   };
+  auto issue_load = [&](int j, int stage, int idx) { issue_load_at(soff_a_of(j), soff_b_of(j), stage, idx); };
 
   // Operand reads, from the operand fragments of the instruction (l16: the lane's row of an lhs block = its column of
   // an rhs block; grp: which 8 of a slice's 32 K positions its registers hold).  lhs: row l16 of each 16-row block,
@@ -1293,6 +1296,9 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   auto tile_step = [&](int kt, auto stage_c, auto parity) {
     constexpr int stage = decltype(stage_c)::value, par = decltype(parity)::value;
     constexpr int next_stage = stage + 1 == STAGES ? 0 : stage + 1, free_stage = stage == 0 ? STAGES - 1 : stage - 1;
+    // (the scalar offsets of this step's loads are formed here, beside the barrier, not in the gaps of the loads)
+    int soff_a = __builtin_amdgcn_readfirstlane(soff_a_of(kt + STAGES - 1)), soff_b = __builtin_amdgcn_readfirstlane(soff_b_of(kt + STAGES - 1));
+    asm volatile("" : "+s"(soff_a), "+s"(soff_b));
     // own loads of tile kt+1 have landed once only the younger tiles' loads remain in flight
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kLoads * (STAGES - 3)));
     __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
@@ -1314,7 +1320,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
           if constexpr (r < kTm) a_nxt[r].c[0] = read_a(RS{}, RK{}, r);
           else read_b(RS{}, RK{}, std::integral_constant<int, r - kTm>{}, b_nxt);
         }
-        if constexpr (load_here) issue_load(kt + STAGES - 1, free_stage, (kk * kMfmas + g) / kLoadSpacing);
+        if constexpr (load_here) issue_load_at(soff_a, soff_b, free_stage, (kk * kMfmas + g) / kLoadSpacing);
         __builtin_amdgcn_sched_barrier(0);
       });
     });

@@ -1156,14 +1156,20 @@ constexpr int kNBM = 128, kNBN = 128;
 // eight to the eight 32-byte bank groups of the 256-byte row.
 __device__ __forceinline__ uint32_t rhs_key(uint32_t row) { return ((row & 3) + 4 * ((row >> 3) & 1)) * 2; }
 
-template <typename T, int BK, int STAGES, bool PACKED>
+// A_TR / B_TR: how each operand lies in memory and in LDS.  false: K-contiguous (a row-major lhs, a column-major rhs): rows
+// of BK elements staged under the tiled kernel's swizzle and read 16 bytes per lane.  true: contiguous along its other
+// extent (a column-major lhs, a row-major rhs): k-rows of 128 elements staged as they lie and read with the transposing
+// read.  <false, true> is the reference fixture's row-major x row-major; <false, false> is the tiled kernel's business.
+template <typename T, int BK, int STAGES, bool PACKED, bool A_TR = false, bool B_TR = true>
 __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   static_assert(T::kM == 16 && T::kBytes == 2 && BK % 32 == 0 && STAGES >= 3, "16x16x32 instruction, 16-bit operands");
+  static_assert(A_TR || B_TR, "two K-contiguous operands are the tiled kernel's");
   using LA = TileLayout<BK * 2, T>;
-  constexpr int kRowA = BK * 2, kRowB = kNBN * 2;
-  constexpr int kBytesA = kNBM * kRowA, kBytesB = BK * kRowB, kStage = kBytesA + kBytesB;
-  constexpr int kLoadsA = kBytesA / 1024 / 4, kLoadsB = kBytesB / 1024 / 4, kLoads = kLoadsA + kLoadsB;  // per wavefront per tile
+  constexpr int kRowKc = BK * 2, kRowTr = 128 * 2;   // bytes per staged row: a row / column of BK elements, or a k-row of 128
+  constexpr int kBytesOp = 128 * BK * 2, kBytesA = kBytesOp, kStage = 2 * kBytesOp;
+  constexpr int kLoadsOp = kBytesOp / 1024 / 4, kLoads = 2 * kLoadsOp;  // per wavefront per tile
   constexpr int KK = BK / 32, kTm = 4, kTn = 4, kMfmas = kTm * kTn;
+  static_assert(kNBM == 128 && kNBN == 128, "both operands stage 128 rows, columns or elements per k-row");
   __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStage];  // static: see tn_kernel
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1172,100 +1178,118 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   tile_of_block(p, tm, tn);
   const int32_t m0 = tm * kNBM, n0 = tn * kNBN;
   const int32_t split = enter_split(p, 2);
-  const int32_t ldb = (int32_t)p.b_sk;  // elements between consecutive k-rows of the rhs
   const int KT = p.K / BK;
+  // elements between neighbours along the staged rows' other extent: between rows (K-contiguous) or between k-rows (transposed)
+  const int32_t a_ld = (int32_t)(A_TR ? p.a_sk : p.a_sm), b_ld = (int32_t)(B_TR ? p.b_sk : p.b_sn);
 
-  uint32_t a_goff[kLoadsA], b_goff[kLoadsB];
-#pragma unroll
-  for (int i = 0; i < kLoadsA; ++i) {
+  // Per-lane global byte offsets of the 16-byte chunks this lane fetches, one per load instruction (instruction q of an operand
+  // fills LDS bytes [q*1024, q*1024 + 1024) of its image).
+  auto goff_of = [&](bool tr, int q, int32_t ld) -> uint32_t {
+    const uint32_t o = (uint32_t)(wave + q * 4) * 1024u + lane * 16u;
     uint32_t row, chunk;
-    LA::locate((uint32_t)(wave + i * 4) * 1024u + lane * 16u, row, chunk);
-    a_goff[i] = (uint32_t)((row * p.a_sm + chunk * 8) * 2);
-  }
+    if (tr) {
+      row = o / kRowTr;
+      chunk = ((o % kRowTr) / 16) ^ rhs_key(row);
+    } else {
+      LA::locate(o, row, chunk);
+    }
+    return (uint32_t)((row * ld + chunk * 8) * 2);
+  };
+  uint32_t a_goff[kLoadsOp], b_goff[kLoadsOp];
 #pragma unroll
-  for (int i = 0; i < kLoadsB; ++i) {
-    const uint32_t o = (uint32_t)(wave + i * 4) * 1024u + lane * 16u, row = o / kRowB, chunk = ((o % kRowB) / 16) ^ rhs_key(row);
-    b_goff[i] = (uint32_t)((row * ldb + chunk * 8) * 2);
+  for (int q = 0; q < kLoadsOp; ++q) {
+    a_goff[q] = goff_of(A_TR, q, a_ld);
+    b_goff[q] = goff_of(B_TR, q, b_ld);
   }
   auto uniform_ptr = [](const char *ptr) {
     const uint64_t v = (uint64_t)ptr;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (void *)(((uint64_t)hi << 32) | lo);
   };
-  // The lhs descriptor ends where the lhs ends: a tile that hangs over its last rows (M not a multiple of 128) gets zeros
-  // for the rows that do not exist (their per-lane offsets are out of range) instead of a fault.
-  const int64_t a_left = ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2;
-  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm * 2), 0,
+  // A K-contiguous lhs descriptor ends where the lhs ends: a tile that hangs over its last rows (M not a multiple of 128) gets
+  // zeros for the rows that do not exist (their per-lane offsets are out of range) instead of a fault.  (In the other forms
+  // the host asks for whole tiles.)
+  const int64_t a_left = A_TR ? 0x7fffffff : ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2;
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * (A_TR ? 1 : p.a_sm) * 2), 0,
                                                                           __builtin_amdgcn_readfirstlane((int)(a_left < 0x7fffffff ? a_left : 0x7fffffff)), 0x00020000);
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * 2), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * (B_TR ? 1 : p.b_sn) * 2), 0, 0x7fffffff, 0x00020000);
   const int wave_lds = wave * 1024;
-  // load `idx` (lhs first, then rhs) of K-tile j into its stage
   // (the scalar offsets of K-tile j, clamped to the last tile: loads past the end of K are still issued, into stages nobody reads)
-  auto soff_a_of = [&](int j) { return min(j, KT - 1) * (BK * 2); };
-  auto soff_b_of = [&](int j) { return min(j, KT - 1) * BK * ldb * 2; };
+  auto soff_a_of = [&](int j) { return min(j, KT - 1) * BK * (A_TR ? a_ld : 1) * 2; };
+  auto soff_b_of = [&](int j) { return min(j, KT - 1) * BK * (B_TR ? b_ld : 1) * 2; };
   auto issue_load_at = [&](int soff_a, int soff_b, int stage, int idx) {
-    if (idx < kLoadsA)
+    if (idx < kLoadsOp)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + idx * 4096 + wave_lds), 16,
                                                (int)a_goff[idx], soff_a, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + kBytesA + (idx - kLoadsA) * 4096 + wave_lds),
-                                               16, (int)b_goff[idx - kLoadsA], soff_b, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + kBytesA + (idx - kLoadsOp) * 4096 + wave_lds),
+                                               16, (int)b_goff[idx - kLoadsOp], soff_b, 0, 0);
   };
   auto issue_load = [&](int j, int stage, int idx) { issue_load_at(soff_a_of(j), soff_b_of(j), stage, idx); };
 
   // Operand reads, from the operand fragments of the instruction (l16: the lane's row of an lhs block = its column of
-  // an rhs block; grp: which 8 of a slice's 32 K positions its registers hold).  lhs: row l16 of each 16-row block,
-  // 16-byte chunk 4*kk + grp.  rhs: the transposing read hands lane j of a 16-lane group column j of the four k-rows
-  // whose 8-byte pieces the group's lanes address, so lane l16 addresses k-row (8*grp + 4*h + l16/4), columns 4*(l16%4)..
+  // an rhs block; grp: which 8 of a slice's 32 K positions its registers hold).  K-contiguous operand: row / column l16 of each
+  // 16-wide block, 16-byte chunk 4*kk + grp.  Transposed operand: the transposing read hands lane j of a 16-lane group element j
+  // of the four k-rows whose 8-byte pieces the group's lanes address, so lane l16 addresses k-row (8*grp + 4*h + l16/4),
+  // elements 4*(l16%4).. of the block.
   const OperandLane frag_at = operand_lane(T::kShape, lane);
   const uint32_t grp = frag_at.k0 / T::kShape.kpack, l16 = frag_at.row;
-  uint32_t a_off[KK];
-#pragma unroll
-  for (int kk = 0; kk < KK; ++kk) a_off[kk] = LA::offset(wm * 64 + l16, 4 * kk + grp);
-  static_assert((16 * kRowA) % (256 * LA::kLineParam) == 0, "an operand block must span whole swizzle periods");
-  const uint32_t b_row = 8 * grp + (l16 >> 2), b_key = rhs_key(b_row);  // the key is the same for every kk and h
-  uint32_t b_off[kTn];
-#pragma unroll
-  for (int j = 0; j < kTn; ++j) b_off[j] = kBytesA + b_row * kRowB + (((wn * 8 + j * 2 + ((l16 & 3) >> 1)) ^ b_key) * 16) + (l16 & 1) * 8;
-  struct Frag {
-    u32x4 c[1];
-  };
-  // an rhs fragment comes out of LDS as two 8-byte halves (k-rows +0..3 and +4..7 of the lane's K-group)
+  static_assert((16 * kRowKc) % (256 * LA::kLineParam) == 0, "an operand block must span whole swizzle periods");
+  const uint32_t tr_row = 8 * grp + (l16 >> 2), tr_key = rhs_key(tr_row);  // the key is the same for every kk and h
+  // Byte offset, inside an operand's image of a stage, of this lane's read for block `blk` (transposed) or slice kk (K-contiguous)
+  // of the wave's half `w` of the operand.
+  auto tr_off = [&](int w, int blk) { return tr_row * kRowTr + (((w * 8 + blk * 2 + ((l16 & 3) >> 1)) ^ tr_key) * 16) + (l16 & 1) * 8; };
+  auto kc_off = [&](int w, int kk) { return LA::offset(w * 64 + l16, 4 * kk + grp); };
+  // a transposed operand's fragment comes out of LDS as two 8-byte halves (k-rows +0..3 and +4..7 of the lane's K-group)
   // (kept as two arrays of halves per fragment buffer, the form the wait for these reads takes its operands in)
-  struct FragHalves {
-    u32x2_lds h0[kTn], h1[kTn];
+  struct Frags {
+    u32x4 c[4];               // K-contiguous operand: one 16-byte read per block
+    u32x2_lds h0[4], h1[4];   // transposed operand
   };
-  static_assert(kTn == 4, "tr_reads_wait takes the halves of four fragments");
+  static_assert(kTm == 4 && kTn == 4, "tr_reads_wait takes the halves of four fragments");
   // Every operand read of the main loop is `register + immediate`: the stage is a compile-time constant there (the loop is
   // unrolled over the ring), and where the ring is longer than a read's 64 KiB immediate reaches, the per-lane offsets
   // are kept once per 64 KiB window (a vector add per read would cost the matrix pipe more than the read itself).
   constexpr int kWindows = (STAGES * kStage + 65535) / 65536;
-  uint32_t a_win[kWindows][KK], b_win[kWindows][kTn];
+  constexpr int kRegsA = A_TR ? kTm : KK, kRegsB = B_TR ? kTn : KK;
+  uint32_t a_win[kWindows][kRegsA], b_win[kWindows][kRegsB];
 #pragma unroll
   for (int w = 0; w < kWindows; ++w) {
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      uint32_t v = (uint32_t)(uintptr_t)lds + a_off[kk] + (uint32_t)w * 65536u;
+    for (int x = 0; x < kRegsA; ++x) {
+      uint32_t v = (uint32_t)(uintptr_t)lds + (A_TR ? tr_off(wm, x) : kc_off(wm, x)) + (uint32_t)w * 65536u;
       asm volatile("" : "+v"(v));  // (opaque: registers that stay, not one register and an add at every read)
-      a_win[w][kk] = v;
+      a_win[w][x] = v;
     }
 #pragma unroll
-    for (int j = 0; j < kTn; ++j) {
-      uint32_t v = (uint32_t)(uintptr_t)lds + b_off[j] + (uint32_t)w * 65536u;
+    for (int x = 0; x < kRegsB; ++x) {
+      uint32_t v = (uint32_t)(uintptr_t)lds + kBytesA + (B_TR ? tr_off(wn, x) : kc_off(wn, x)) + (uint32_t)w * 65536u;
       asm volatile("" : "+v"(v));
-      b_win[w][j] = v;
+      b_win[w][x] = v;
     }
   }
-  auto read_a = [&](auto stage, auto kk, int i) {
-    constexpr uint32_t at = decltype(stage)::value * kStage;
-    const uint32_t c = at + (uint32_t)i * 16 * kRowA;
-    return *(const __attribute__((address_space(3))) u32x4 *)(uintptr_t)(a_win[c >> 16][decltype(kk)::value] + (c & 65535u));
+  // read `r` (0 .. 3) of slice kk of the stage: block r of the operand
+  auto read_op = [&](auto is_b, auto stage, auto kk, auto blk, Frags &dst) {
+    constexpr bool kIsB = decltype(is_b)::value, kTr = kIsB ? B_TR : A_TR;
+    constexpr int b = decltype(blk)::value;
+    auto win = [&](uint32_t w, int x) { if constexpr (kIsB) return b_win[w][x]; else return a_win[w][x]; };
+    if constexpr (kTr) {
+      constexpr uint32_t c0 = decltype(stage)::value * kStage + decltype(kk)::value * 32 * kRowTr, c1 = c0 + 4 * kRowTr;
+      dst.h0[b] = tr_read_b64_at<(c0 & 65535u)>(win(c0 >> 16, b));
+      dst.h1[b] = tr_read_b64_at<(c1 & 65535u)>(win(c1 >> 16, b));
+    } else {
+      constexpr uint32_t c = decltype(stage)::value * kStage + (uint32_t)b * 16 * kRowKc;
+      dst.c[b] = *(const __attribute__((address_space(3))) u32x4 *)(uintptr_t)(win(c >> 16, decltype(kk)::value) + (c & 65535u));
+    }
   };
-  auto read_b = [&](auto stage, auto kk, auto j, FragHalves &dst) {
-    constexpr uint32_t c0 = decltype(stage)::value * kStage + decltype(kk)::value * 32 * kRowB, c1 = c0 + 4 * kRowB;
-    dst.h0[decltype(j)::value] = tr_read_b64_at<(c0 & 65535u)>(b_win[c0 >> 16][decltype(j)::value]);
-    dst.h1[decltype(j)::value] = tr_read_b64_at<(c1 & 65535u)>(b_win[c1 >> 16][decltype(j)::value]);
+  using IsA = std::integral_constant<bool, false>;
+  using IsB = std::integral_constant<bool, true>;
+  auto operand_of = [](auto tr, const Frags &f, int b) -> u32x4 {
+    if constexpr (decltype(tr)::value) return u32x4{f.h0[b][0], f.h0[b][1], f.h1[b][0], f.h1[b][1]};
+    else return f.c[b];
   };
+  using ATr = std::integral_constant<bool, A_TR>;
+  using BTr = std::integral_constant<bool, B_TR>;
 
   using Acc = typename T::Acc;
   Acc acc[kTm][kTn];
@@ -1280,11 +1304,10 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     for (int idx = 0; idx < kLoads; ++idx) issue_load(j, j, idx);
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (STAGES - 2)));
   __builtin_amdgcn_s_barrier();  // tile 0 published
-  Frag af[2][kTm];
-  FragHalves bf[2];
+  Frags af[2], bf[2];
   using Zero = std::integral_constant<int, 0>;
-  static_for<kTm>([&](auto i) { af[0][decltype(i)::value].c[0] = read_a(Zero{}, Zero{}, decltype(i)::value); });
-  static_for<kTn>([&](auto j) { read_b(Zero{}, Zero{}, j, bf[0]); });
+  static_for<kTm>([&](auto i) { read_op(IsA{}, Zero{}, Zero{}, i, af[0]); });
+  static_for<kTn>([&](auto j) { read_op(IsB{}, Zero{}, Zero{}, j, bf[0]); });
 
   constexpr int kReads = kTm + kTn;
   constexpr int kLoadSpacing = (KK * kMfmas) / kLoads;  // matrix instructions between two loads
@@ -1304,21 +1327,23 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
     static_for<KK>([&](auto kk_c) {
       constexpr int kk = decltype(kk_c)::value;
-      Frag *a_cur = af[(kk + par) & 1], *a_nxt = af[(kk + par + 1) & 1];
-      FragHalves &b_cur = bf[(kk + par) & 1], &b_nxt = bf[(kk + par + 1) & 1];
-      tr_reads_wait(b_cur.h0, b_cur.h1);  // the rhs fragments of this slice were requested during the previous one
+      Frags &a_cur = af[(kk + par) & 1], &a_nxt = af[(kk + par + 1) & 1];
+      Frags &b_cur = bf[(kk + par) & 1], &b_nxt = bf[(kk + par + 1) & 1];
+      // the transposed fragments of this slice were requested during the previous one
+      if constexpr (A_TR) tr_reads_wait(a_cur.h0, a_cur.h1);
+      if constexpr (B_TR) tr_reads_wait(b_cur.h0, b_cur.h1);
       static_for<kMfmas>([&](auto g_c) {
         constexpr int g = decltype(g_c)::value, i = g / kTn, j = g % kTn;
         constexpr bool load_here = (kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads;
-        const u32x4 b_op = {b_cur.h0[j][0], b_cur.h0[j][1], b_cur.h1[j][0], b_cur.h1[j][1]};
-        T::mfma_in_place(&b_op, a_cur[i].c, acc[i][j]);
+        const u32x4 a_op = operand_of(ATr{}, a_cur, i), b_op = operand_of(BTr{}, b_cur, j);
+        T::mfma_in_place(&b_op, &a_op, acc[i][j]);
         if constexpr (!load_here) __builtin_amdgcn_sched_barrier(0);
         constexpr int r = load_here ? -1 : g - (g + 1) / kLoadSpacing;  // this gap's read: the gaps without a load, in order
         if constexpr (r >= 0 && r < kReads) {
           using RS = std::integral_constant<int, (kk + 1 < KK ? stage : next_stage)>;
           using RK = std::integral_constant<int, (kk + 1 < KK ? kk + 1 : 0)>;
-          if constexpr (r < kTm) a_nxt[r].c[0] = read_a(RS{}, RK{}, r);
-          else read_b(RS{}, RK{}, std::integral_constant<int, r - kTm>{}, b_nxt);
+          if constexpr (r < kTm) read_op(IsA{}, RS{}, RK{}, std::integral_constant<int, r>{}, a_nxt);
+          else read_op(IsB{}, RS{}, RK{}, std::integral_constant<int, r - kTm>{}, b_nxt);
         }
         if constexpr (load_here) issue_load_at(soff_a, soff_b, free_stage, (kk * kMfmas + g) / kLoadSpacing);
         __builtin_amdgcn_sched_barrier(0);
@@ -1547,14 +1572,14 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
   return packed ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s) : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
 }
 
-template <typename T, int BK, int STAGES>
+template <typename T, int BK, int STAGES, bool A_TR = false, bool B_TR = true>
 int launch_nn(GemmParams p, hipStream_t s) {
-  p.tiles_m = (p.M + kNBM - 1) / kNBM;  // M need not be a multiple of the tile: see the kernel's lhs descriptor
+  p.tiles_m = (p.M + kNBM - 1) / kNBM;  // (a K-contiguous lhs need not have whole tiles of rows: see the kernel's lhs descriptor)
   p.tiles_n = p.N / kNBN;
   const bool packed = packed_epilogue(p) && !host_has_tail(p);  // (a fused tail goes through the element stores here)
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k);
-  if (packed) nn_kernel<T, BK, STAGES, true><<<grid, dim3(256), 0, s>>>(p);
-  else nn_kernel<T, BK, STAGES, false><<<grid, dim3(256), 0, s>>>(p);
+  if (packed) nn_kernel<T, BK, STAGES, true, A_TR, B_TR><<<grid, dim3(256), 0, s>>>(p);
+  else nn_kernel<T, BK, STAGES, false, A_TR, B_TR><<<grid, dim3(256), 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }
@@ -1818,23 +1843,30 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
       return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
     }
   }
-  // Both operands row-major (the reference fixture's layout, matmul.mlir): the transposing-read kernel.
-  bool nn = p.a_sk == 1 && p.b_sn == 1 && vector_bytes(lhs, 1) == 16 && vector_bytes(rhs, 1) == 16 && p.M > 0 && p.N % kNBN == 0 &&
-            p.K > 0 && p.a_sm >= 0 && p.b_sk >= 0 && p.a_sm * 2 * kNBM < (int64_t(1) << 31) && (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31) &&
+  // An operand that is contiguous along its other extent - a row-major rhs (with a row-major lhs: the reference fixture's
+  // layout, matmul.mlir), a column-major lhs - is staged as it lies and read with the transposing read.
+  const bool a_kc = p.a_sk == 1 && vector_bytes(lhs, 1) == 16 && p.a_sm >= 0 && p.a_sm * 2 * kNBM < (int64_t(1) << 31);
+  const bool a_tr = !a_kc && p.a_sm == 1 && vector_bytes(lhs, 0) == 16 && p.a_sk >= 0 && p.M % kNBM == 0 && (int64_t)p.K * p.a_sk * 2 < (int64_t(1) << 31);
+  const bool b_tr = p.b_sn == 1 && vector_bytes(rhs, 1) == 16 && p.b_sk >= 0 && (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31);
+  const bool b_kc = !b_tr && p.b_sk == 1 && vector_bytes(rhs, 0) == 16 && p.b_sn >= 0 && p.b_sn * 2 * kNBN < (int64_t(1) << 31);
+  bool nn = (a_kc || a_tr) && (b_kc || b_tr) && (a_tr || b_tr) && p.M > 0 && p.N % kNBN == 0 && p.K > 0 &&
             c.impl_way != KAPY_MFMA_32X32X16_16B && (!c.tile_m || c.tile_m == kNBM) && (!c.tile_n || c.tile_n == kNBN) && (!c.waves || c.waves == 4);
   if (nn) {
     struct NnVariant {
       int bk, stages;
-      int (*launch_bf16)(GemmParams, hipStream_t);
-      int (*launch_f16)(GemmParams, hipStream_t);
+      int (*launch_bf16[3])(GemmParams, hipStream_t);   // lhs K-contiguous x rhs transposed, both transposed, lhs transposed x rhs K-contiguous
+      int (*launch_f16[3])(GemmParams, hipStream_t);
     };
-    static const NnVariant kNn[] = {{64, 4, launch_nn<Bf16M16, 64, 4>, launch_nn<F16M16, 64, 4>}, {64, 3, launch_nn<Bf16M16, 64, 3>, launch_nn<F16M16, 64, 3>},
-                                    {32, 4, launch_nn<Bf16M16, 32, 4>, launch_nn<F16M16, 32, 4>}};
+#define KAPY_NN(BK, ST) {BK, ST, {launch_nn<Bf16M16, BK, ST, false, true>, launch_nn<Bf16M16, BK, ST, true, true>, launch_nn<Bf16M16, BK, ST, true, false>}, \
+                         {launch_nn<F16M16, BK, ST, false, true>, launch_nn<F16M16, BK, ST, true, true>, launch_nn<F16M16, BK, ST, true, false>}}
+    static const NnVariant kNn[] = {KAPY_NN(64, 4), KAPY_NN(64, 3), KAPY_NN(32, 4)};
+#undef KAPY_NN
+    const int form = !a_tr ? 0 : (b_tr ? 1 : 2);
     for (const NnVariant &v : kNn) {
       if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;
       rc = plan_split_k(p, c, v.bk);
       if (rc) return rc;
-      return bf16 ? v.launch_bf16(p, s) : v.launch_f16(p, s);
+      return bf16 ? v.launch_bf16[form](p, s) : v.launch_f16[form](p, s);
     }
   }
   if ((c.tile_m && c.tile_m != kSBM) || (c.tile_n && c.tile_n != kSBN) || (c.tile_k && c.tile_k != kSBK) || (c.stages && c.stages != 1) ||

@@ -266,3 +266,15 @@ def test_accumulator_input_through_the_strip_epilogue(ko, acc_dt, out_dt, M, N, 
         got = to_host(dd, want.dtype.type if out_dt != kh.F32 else np.float32)
         assert np.all(to_host(dd, np.uint16 if out_dt != kh.F32 else np.uint32)[M * N:] == 0x1234), tile
         assert _frob(ko, got[:M * N], want, out_dt) <= (1e-5 if out_dt == kh.F32 else FROB_TOL), tile
+
+
+@pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("a_rm,b_rm", [(True, True), (False, True), (False, False)])
+@pytest.mark.parametrize("tile_k,stages", [(64, 4), (64, 3), (32, 4)])
+def test_transposing_read_kernel_takes_either_operand_transposed(ko, dt, a_rm, b_rm, tile_k, stages):
+    """A column-major lhs and / or a row-major rhs is staged as it lies and read with the transposing read (row-major x
+    row-major is the reference fixture's layout): every form and ring depth against the oracle, K of several tiles so
+    that the unrolled ring wraps, a last partial round of the unroll, and a result the tiles cover exactly."""
+    for (M, N, K) in ((256, 384, 64 * 9), (128, 128, 64 * 4), (384, 256, 64 * 5)):
+        got, want = _run(ko, dt, M, N, K, a_rm, b_rm, seed=21, tile=(128, 128, tile_k), stages=stages)
+        assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)

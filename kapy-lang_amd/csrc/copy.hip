@@ -326,6 +326,11 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
     }
   } else if (B == 2 && p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16 && p.d0 >= 128 && p.d1 >= 128 &&
              (p.d1 + 127) / 128 <= 65535) {
+    // 256 x 256 tiles where they divide the matrix and still fill the chip (one workgroup per CU: the tile takes 128 KiB of
+    // LDS): a tile side is the length of the contiguous runs the kernel reads and writes, and 512-byte runs move at
+    // 5.7 TB/s where 256-byte runs move at 5.4 (1 KiB runs would reach the plain copy's 6.1, but no tile that big fits).
+    if (p.d0 % 256 == 0 && p.d1 % 256 == 0 && p.sb0 >= p.d0 && p.sb1 >= p.d1 && (int64_t)(p.d0 / 256) * (p.d1 / 256) * batch >= 2 * (int64_t)device_cus())
+      return launch_transpose_lds<256, 256>(p, nt, batch, stream);
     return launch_transpose_lds<128, 128>(p, nt, batch, stream);
   } else if (p.ds1 == 1 && p.es0 == 1 && vb_src == 16 && vb_dst == 16) {
     constexpr int TILE = 8 * (16 / B);

@@ -182,3 +182,20 @@ def test_cache_hints_do_not_change_results(ko):
             kh.copy(dglobal(d_src, m, n, n, 1, kh.F16), dglobal(d_dst, dm, dn, dn, 1, kh.F16), transpose=transpose, cache=cache, evict=evict, volatile=vol)
             sync()
             assert np.array_equal(to_host(d_dst, np.uint16, (dm, dn)), want), (transpose, cache, evict, vol)
+
+
+@pytest.mark.parametrize("rows,cols", [(4096, 8192), (8192, 4096), (6144, 5632)])
+def test_transpose_with_256_tiles_on_windows_of_wider_buffers(ko, rows, cols):
+    """Extents that 256 x 256 tiles divide, with enough tiles to fill the chip, take the large-tile form of the LDS transpose;
+    source and destination are windows of wider buffers (pitches larger than the extents), and the words beside and behind
+    the destination window must stay as they were."""
+    sp, dp = cols + 64, rows + 128
+    src = ko.fill_bits16(rows * sp, 3).reshape(rows, sp)
+    d_src, d_dst = to_dev(src), dev_zeros(cols * dp + 256, 2, fill=0x5A5A)
+    kh.copy(dglobal(d_src, rows, cols, sp, 1, kh.F16), dglobal(d_dst, cols, rows, dp, 1, kh.F16), transpose=True)
+    sync()
+    got = to_host(d_dst, np.uint16)
+    assert np.all(got[cols * dp:] == 0x5A5A)
+    win = got[:cols * dp].reshape(cols, dp)
+    assert np.all(win[:, rows:] == 0x5A5A)
+    assert np.array_equal(win[:, :rows], src[:, :cols].T)

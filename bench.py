@@ -693,6 +693,14 @@ def bench_ceilings(kh, steps, warmup, cpu):
             raise CheckFailed("probe_copy_tiled: result differs from the source")
         wall, ev = _events(lambda i: kh.probe_copy_tiled(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, lds), 40, 5)
         out["copy"]["transpose footprint (128 rows x 256 B per workgroup)%s" % (", through LDS and a barrier" if lds else "")] = round(2 * nbytes / (ev * 1e-3) / 1e9, 0)
+    # ... and by the length of the contiguous runs alone (a transposing kernel's runs are as long as its tile is wide)
+    for run in (256, 512, 1024, 2048, 4096):
+        kh.probe_copy_runs(src[0].data_ptr(), dst[0].data_ptr(), n, n * 2, run)
+        torch.cuda.synchronize()
+        if not torch.equal(src[0], dst[0]):
+            raise CheckFailed("probe_copy_runs: result differs from the source")
+        wall, ev = _events(lambda i: kh.probe_copy_runs(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, run), 40, 5)
+        out["copy"]["runs of %d B (%d rows x %d B per workgroup)" % (run, 32768 // run, run)] = round(2 * nbytes / (ev * 1e-3) / 1e9, 0)
     out["copy_best_gbs"] = round(best, 0)
     out["copy_best_frac_of_peak"] = round(best / HBM_PEAK_GBS, 4)
     # what the L2s hand to the CUs: every CU re-reads a window that stays in its XCD's L2 (2 MiB), that spills to the Infinity

@@ -183,6 +183,10 @@ int kapy_probe_mfma(int32_t impl_way, int32_t dtype, const void *operands, int32
 int kapy_probe_copy(const void *src, void *dst, int64_t bytes, int32_t vectors_per_lane, int32_t nt_load, int32_t nt_store, int32_t persistent_per_cu,
                     uint64_t *ticks, int32_t *workgroups, void *stream);
 
+/* kapy_probe_copy_runs: dst <- src for a [rows][row_bytes] matrix, moved in pieces of run_bytes (256, 512, 1024, 2048 or 4096)
+ * contiguous bytes: a workgroup owns 32 KiB / run_bytes rows of one run each.  What run length alone costs: a transposing
+ * kernel reads and writes runs as long as its tile is wide. */
+int kapy_probe_copy_runs(const void *src, void *dst, int64_t rows, int64_t row_bytes, int32_t run_bytes, void *stream);
 /* kapy_probe_issue: what a wave can issue beside its matrix instructions.  One wave per SIMD (the tiled matmul's occupancy)
  * runs `iterations` tiles of independent matrix instructions of `impl_way` (KAPY_MFMA_16X16X32_16B: 128 per tile, or
  * KAPY_MFMA_16X16X128_F8: 64 per tile - 2048 matrix-pipe clocks either way) with, behind every instruction, filler 0: nothing;

@@ -149,6 +149,23 @@ __global__ __launch_bounds__(256) void copy_tiled_kernel(const char *__restrict_
   }
 }
 
+// The same plain copy in pieces of RUN contiguous bytes: a workgroup owns (32 KiB / RUN) rows x RUN bytes of a [rows][row_bytes]
+// matrix, 8 vectors of 16 bytes per lane.  What the length of the contiguous runs alone costs: a transposing kernel reads
+// and writes runs as long as its tile is wide.
+template <int RUN>
+__global__ __launch_bounds__(256) void copy_runs_kernel(const char *__restrict__ src, char *__restrict__ dst, int64_t row_bytes, uint32_t tiles_x, uint32_t tiles_y) {
+  constexpr int kRows = 32768 / RUN, kLanesPerRow = RUN / 16, kRowsPerPass = 256 / kLanesPerRow;
+  static_assert(kRows % 8 == 0 && kRowsPerPass * 8 == kRows, "8 passes over the workgroup's rows");
+  const int t = threadIdx.x;
+  uint32_t bx = blockIdx.x % tiles_x, by = (blockIdx.x / tiles_x + bx) % tiles_y;  // diagonal walk, as the transpose
+  const int64_t base = ((int64_t)by * kRows + t / kLanesPerRow) * row_bytes + (int64_t)bx * RUN + (t % kLanesPerRow) * 16;
+  vec16 v[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) v[c] = __builtin_nontemporal_load((const vec16 *)(src + base + (int64_t)c * kRowsPerPass * row_bytes));
+#pragma unroll
+  for (int c = 0; c < 8; ++c) __builtin_nontemporal_store(v[c], (vec16 *)(dst + base + (int64_t)c * kRowsPerPass * row_bytes));
+}
+
 template <int U, bool LNT, bool SNT>
 int launch_copy(const void *src, void *dst, int64_t n, int persistent_per_cu, uint64_t *ticks, int32_t *workgroups, hipStream_t s) {
   if (persistent_per_cu > 0) {
@@ -374,6 +391,28 @@ int kapy_probe_copy_tiled(const void *src, void *dst, int64_t rows, int64_t row_
   const uint32_t tx = (uint32_t)(row_bytes / 256), ty = (uint32_t)(rows / 128);
   if (through_lds) copy_tiled_kernel<true><<<tx * ty, 256, 0, (hipStream_t)stream>>>((const char *)src, (char *)dst, row_bytes, tx, ty);
   else copy_tiled_kernel<false><<<tx * ty, 256, 0, (hipStream_t)stream>>>((const char *)src, (char *)dst, row_bytes, tx, ty);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
+int kapy_probe_copy_runs(const void *src, void *dst, int64_t rows, int64_t row_bytes, int32_t run_bytes, void *stream) {
+  if (!src || !dst || rows <= 0 || row_bytes <= 0 || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
+    return fail(KAPY_ERR_INVALID, "probe_copy_runs: null or misaligned buffer, or an empty matrix");
+  if (run_bytes != 256 && run_bytes != 512 && run_bytes != 1024 && run_bytes != 2048 && run_bytes != 4096)
+    return fail(KAPY_ERR_INVALID, "probe_copy_runs: runs of 256, 512, 1024, 2048 or 4096 bytes");
+  if (row_bytes % run_bytes || rows % (32768 / run_bytes))
+    return fail(KAPY_ERR_INVALID, "probe_copy_runs: row_bytes must be a multiple of the run, rows of 32768 / run");
+  int rc = ensure_device();
+  if (rc) return rc;
+  const uint32_t tx = (uint32_t)(row_bytes / run_bytes), ty = (uint32_t)(rows / (32768 / run_bytes));
+  hipStream_t s = (hipStream_t)stream;
+  switch (run_bytes) {
+  case 256: copy_runs_kernel<256><<<tx * ty, 256, 0, s>>>((const char *)src, (char *)dst, row_bytes, tx, ty); break;
+  case 512: copy_runs_kernel<512><<<tx * ty, 256, 0, s>>>((const char *)src, (char *)dst, row_bytes, tx, ty); break;
+  case 1024: copy_runs_kernel<1024><<<tx * ty, 256, 0, s>>>((const char *)src, (char *)dst, row_bytes, tx, ty); break;
+  case 2048: copy_runs_kernel<2048><<<tx * ty, 256, 0, s>>>((const char *)src, (char *)dst, row_bytes, tx, ty); break;
+  default: copy_runs_kernel<4096><<<tx * ty, 256, 0, s>>>((const char *)src, (char *)dst, row_bytes, tx, ty); break;
+  }
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }

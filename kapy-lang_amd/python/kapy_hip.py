@@ -35,7 +35,7 @@ EXPORTS = [
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
     "kapy_mfma_probe", "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
-    "kapy_mk_shared", "kapy_sv_shared", "kapy_shared_address", "kapy_probe_mfma", "kapy_probe_copy", "kapy_probe_copy_tiled", "kapy_probe_l2_read", "kapy_probe_issue",
+    "kapy_mk_shared", "kapy_sv_shared", "kapy_shared_address", "kapy_probe_mfma", "kapy_probe_copy", "kapy_probe_copy_tiled", "kapy_probe_l2_read", "kapy_probe_issue", "kapy_probe_copy_runs",
 ]
 
 
@@ -141,6 +141,7 @@ def lib():
     L.kapy_probe_copy.argtypes = [vp, vp, i64, i32, i32, i32, i32, vp, P(i32), vp]
     L.kapy_probe_copy_tiled.argtypes = [vp, vp, i64, i64, i32, vp]
     L.kapy_probe_l2_read.argtypes = [vp, i64, i32, i32, i32, vp, C.POINTER(C.c_int32), C.POINTER(C.c_int64), vp]
+    L.kapy_probe_copy_runs.argtypes = [vp, vp, i64, i64, i32, vp]
     L.kapy_probe_issue.argtypes = [i32, i32, i32, vp, i32, vp, C.POINTER(C.c_int32), C.POINTER(C.c_int64), vp]
     L.kapy_mk_shared.argtypes = [P(Shared), i64, i32, i32, i32, i32, i32, i32]
     L.kapy_sv_shared.argtypes = [P(Shared), P(Shared), i32, i32, i32, i32]
@@ -484,6 +485,10 @@ def probe_copy(src_ptr, dst_ptr, nbytes, vectors_per_lane=4, nt_load=False, nt_s
 def probe_copy_tiled(src_ptr, dst_ptr, rows, row_bytes, through_lds=False, stream=None):
     check(lib().kapy_probe_copy_tiled(C.c_void_p(src_ptr), C.c_void_p(dst_ptr), rows, row_bytes, int(through_lds),
                                       stream if stream is not None else current_stream()))
+
+
+def probe_copy_runs(src_ptr, dst_ptr, rows, row_bytes, run_bytes, stream=None):
+    check(lib().kapy_probe_copy_runs(C.c_void_p(src_ptr), C.c_void_p(dst_ptr), rows, row_bytes, run_bytes, stream if stream is not None else current_stream()))
 
 
 def probe_issue(impl_way, filler, count, src_ptr, iterations, sink_ptr, stream=None):

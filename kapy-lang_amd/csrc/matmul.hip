@@ -1752,12 +1752,14 @@ int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k) {
   return KAPY_OK;
 }
 
-int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
+int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, int want_tile, hipStream_t s) {
   if (p.a_sm * 256 >= (int64_t(1) << 31) || p.b_sn * 256 >= (int64_t(1) << 31)) return KAPY_ERR_UNSUPPORTED;
   // the ring variants take any M, N >= 128 and any K >= 128 of whole 16-byte chunks (their loads are bounded by the
   // operands' ends); 256x256 tiles when there are at least as many of them as CUs, 128x128 (two workgroups per CU) below
   if (p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
-    if ((int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()) return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    // (want_tile: 0 = the library's choice, 128 or 256 = the caller's, kapy_matmul_cfg.tile_m)
+    if (want_tile == 256 || (want_tile == 0 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()))
+      return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
     return launch_f8<F8, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())

@@ -422,7 +422,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     // an explicit split is a request for the tiled kernel; the library's own choice weighs it against the block kernel
     const int tiled_from = block_ok && c.split_k <= 1 ? (g.split_k > 1 ? kTiledFromMSplit : kTiledFromM) : (g.split_k > 1 ? kTiledFromMSplitNoBlock : kTiledFromMNoBlock);
     if (p.M < tiled_from) rc = KAPY_ERR_UNSUPPORTED;  // few rows: the streaming kernels below
-    else rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), s);
+    else rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), c.tile_m == 256 || c.tile_m == 128 ? c.tile_m : 0, s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
   }
   if (block_ok) {

@@ -41,7 +41,7 @@ constexpr int kMaxSplitK = 8;
 // Tiled LDS-direct MFMA kernel on fp8 operands (both K-contiguous, extents multiples of the tile).
 // lhs_fmt / rhs_fmt: 0 = E4M3, 1 = E5M2.  Returns KAPY_ERR_UNSUPPORTED when no compiled tile fits,
 // without having launched anything.
-int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s);
+int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, int want_tile, hipStream_t s);
 
 // Decides whether a 128 x 128 tiled kernel with K-tiles of tile_k splits K for this problem (kapy_matmul_cfg::split_k,
 // workspace) and sets p.split_k / p.partial / p.counters; KAPY_OK, or the status of a split that was asked for and

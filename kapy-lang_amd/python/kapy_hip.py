@@ -406,9 +406,9 @@ def matmul_fused(lhs, rhs, result, bias=None, alpha=1.0, act=-1, act_operand=0.0
                                   stream if stream is not None else current_stream()))
 
 
-def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, split_k=0, workspace=None, stream=None):
+def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, split_k=0, workspace=None, tile=(0, 0, 0), stream=None):
     ws, ws_bytes = _workspace(workspace)
-    cfg = MatmulCfg(MATMUL_AUTO, 0, 0, 0, RN, 0, 0, split_k, ws, ws_bytes)
+    cfg = MatmulCfg(MATMUL_AUTO, tile[0], tile[1], tile[2], RN, 0, 0, split_k, ws, ws_bytes)
     check(lib().kapy_matmul_scaled_f8(C.byref(a8), C.byref(w8), C.c_void_p(row_scale_ptr), C.c_void_p(col_scale_ptr),
                                       C.byref(result), C.byref(cfg), stream if stream is not None else current_stream()))
 

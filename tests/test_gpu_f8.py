@@ -163,3 +163,39 @@ def test_config5_m4096_sampled(ko):
         num += ((g - w) ** 2).sum()
         den += (w ** 2).sum()
     assert np.sqrt(num / den) <= FROB_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (768, 256, 1280), (300, 520, 256), (1000, 264, 384), (257, 1000, 128), (512, 256, 272), (256, 512, 144),
+                                   (640, 384, 128 * 7)])   # ragged M and N, a partial last K-tile, K-tile counts around the ring's unroll of five
+def test_scaled_f8_256_tiles_on_the_16x16x128_instruction(ko, M, N, K):
+    """The 256 x 256 x 128 ring kernel (two passes per tile on v_mfma_scale_f32_16x16x128_f8f6f4), asked for by tile size on
+    shapes the library would give to the 128-wide tiles: tiles that hang over every edge, and nothing written past the result."""
+    aq, sa, wq, sb = _quantised(ko, M, N, K, seed=5)
+    want = np.zeros((M, N), dtype=np.uint16)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                        vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16))) == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N + 4096, 2, fill=0x1234)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16), tile=(256, 256, 128))
+    sync()
+    got = to_host(dd, np.uint16)
+    assert np.all(got[M * N:] == 0x1234)
+    assert _frob(ko, got[:M * N].reshape(M, N), want) <= FROB_TOL
+
+
+def test_f8_256_tiles_mixed_formats_f32_result(ko):
+    """e4m3 x e5m2 and e5m2 x e4m3 through the 256-wide tiles, fp32 result, no scales: the format selectors of the in-place
+    matrix instruction on both sides."""
+    M, N, K = 512, 256, 384
+    rng = np.random.default_rng(2)
+    e4 = rng.integers(0x20, 0x50, size=(M, K)).astype(np.uint8) | (rng.integers(0, 2, size=(M, K)).astype(np.uint8) << 7)
+    e5 = rng.integers(0x30, 0x48, size=(N, K)).astype(np.uint8) | (rng.integers(0, 2, size=(N, K)).astype(np.uint8) << 7)
+    for (a, adt, b, bdt, m, n) in ((e4, ko.F8E4M3, e5, ko.F8E5M2, M, N), (e5, ko.F8E5M2, e4, ko.F8E4M3, N, M), (e5, ko.F8E5M2, e5, ko.F8E5M2, N, N)):
+        want = np.zeros((m, n), dtype=np.float32)
+        assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, m, K, K, 1, adt)), C.byref(ko.mk_global(b, K, n, 1, K, bdt)), None,
+                                  C.byref(ko.mk_global(want, m, n, n, 1, ko.F32)), ko.RN) == 0
+        da, db, dd = to_dev(a), to_dev(b), dev_zeros(m * n, 4)
+        kh.matmul(dglobal(da, m, K, K, 1, adt), dglobal(db, K, n, 1, K, bdt), dglobal(dd, m, n, n, 1, kh.F32), tile=(256, 256, 128))
+        sync()
+        got = to_host(dd, np.float32, (m, n))
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-4

@@ -1755,10 +1755,11 @@ int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k) {
 int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, int want_tile, hipStream_t s) {
   if (p.a_sm * 256 >= (int64_t(1) << 31) || p.b_sn * 256 >= (int64_t(1) << 31)) return KAPY_ERR_UNSUPPORTED;
   // the ring variants take any M, N >= 128 and any K >= 128 of whole 16-byte chunks (their loads are bounded by the
-  // operands' ends); 256x256 tiles when there are at least as many of them as CUs, 128x128 (two workgroups per CU) below
+  // operands' ends); 256x256 tiles when there are at least 0.55 times as many of them as CUs, 128x128 (two workgroups per CU) below
   if (p.K % 16 == 0 && p.K >= 128 && p.M >= 1 && p.N >= 128) {
     // (want_tile: 0 = the library's choice, 128 or 256 = the caller's, kapy_matmul_cfg.tile_m)
-    if (want_tile == 256 || (want_tile == 0 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) >= device_cus()))
+    // (measured at N = K = 8192: 192 of the large tiles on 256 CUs already beat 768 of the small ones, 128 do not)
+    if (want_tile == 256 || (want_tile == 0 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 >= (int64_t)device_cus() * 55))
       return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
     return launch_f8<F8, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
@@ -1834,8 +1835,9 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
       const bool whole_tiles = p.M % v.bm == 0 && p.N % v.bn == 0;
       const bool whole_k = p.K % v.bk == 0;  // the ring variants also take a partial last K-tile of whole 16-byte chunks
       if ((!whole_k && (v.stages != kRing25 || p.K % 8)) || (!whole_tiles && v.stages != kRing25)) continue;
-      // with a free choice, a 256x256 tiling with fewer tiles than CUs yields to 128x128
-      if (free_choice && v.bm == 256 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) < device_cus()) continue;
+      // with a free choice, a 256x256 tiling with fewer than 0.55 tiles per CU yields to 128x128 (measured: 144 large tiles on
+      // 256 CUs beat 576 small ones - 3072^3: 1009 against 899 TFLOP/s - 128 do not)
+      if (free_choice && v.bm == 256 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 < (int64_t)device_cus() * 55) continue;
       if (v.bm == 128 && v.stages == kRing25) {
         rc = plan_split_k(p, c, v.bk);
         if (rc) return rc;

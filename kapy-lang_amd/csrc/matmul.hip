@@ -938,6 +938,10 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
           // tile kt+1 has landed once only the kHalf youngest loads (lhs of tile kt+2) are in flight
           __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kHalf));
           __builtin_amdgcn_s_barrier();
+        } else if constexpr (!KTAIL) {
+          // this slice's fragments, asked for during the previous slice, have long returned: one wait here, which never
+          // waits, instead of the compiler's own wait in each of the first gaps, where it costs the gap a third of its slots
+          __builtin_amdgcn_s_waitcnt(0xC07F);
         }
 #pragma unroll
         for (int g = 0; g < kMfmas; ++g) {

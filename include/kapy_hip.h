@@ -371,7 +371,7 @@ int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy
  * In kapy terms: matmul (mma f8, f32 acc) -> mulf with broadcast(row_scale [Mx1]) and
  * broadcast(col_scale [1xN]) -> fptofp rn.  Scales are dense fp32 device arrays.
  * cfg (may be NULL): split_k / workspace as for kapy_matmul; tile_m = 128 or 256 asks for that tile of the tiled kernel
- * (0: the library's choice - 256 x 256 x 128 on the 16x16x128 instruction from as many such tiles as CUs, 128 x 128 x 128 below). */
+ * (0: the library's choice - 256 x 256 x 128 on the 16x16x128 instruction from 0.55 such tiles per CU, 128 x 128 x 128 below). */
 int kapy_matmul_scaled_f8(const kapy_global *a8, const kapy_global *w8, const float *row_scale, const float *col_scale,
                           const kapy_global *result, const kapy_matmul_cfg *cfg, void *stream);
 

@@ -622,7 +622,7 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     flops = 2.0 * M * N * K
     nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
     out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192%s" % (M, ", K split across workgroups (workspace given)" if workspace else ""), "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 160 and not workspace)) else "tn_kernel<F8, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8>",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 160 and not workspace)) else "tn_kernel<F8M16, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8>",
            "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
            "checked": True, "check": "%d %dx64 blocks against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" % (n_blocks, min(M, 64), rel, FROB_TOL)}
     out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d" % M) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)

@@ -915,9 +915,13 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
               if (j == kHalfTn - 1) {
 #pragma unroll
                 for (int c = 0; c < CH; ++c) a_cur[i].c[c] = read_at(0, a_nxt_base, i * KM * C::kRowBytes, 0, c);
-              } else if (i < kHalfTn && jb >= 0 && jb < CH) {
+              } else if (kSpread && i < kHalfTn && jb >= 0 && jb < CH) {
                 // ... and the first half of its rhs blocks (block i, chunk jb) into the buffer pass 0 has left
                 bf[0][i].c[jb] = read_at(1, b_nxt_base, i * KM * C::kRowBytes, 0, jb);
+              } else if (!kSpread && i * (kHalfTn - 1) + j < kHalfTn * CH) {
+                // (without the spread placement: the same reads, one in each gap that refills no lhs block, in order)
+                const int q = i * (kHalfTn - 1) + j;
+                bf[0][q / CH].c[q % CH] = read_at(1, b_nxt_base, (q / CH) * KM * C::kRowBytes, 0, q % CH);
               }
             }
             if (g % kLoadSpacing == 0) {
@@ -1765,7 +1769,7 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, int want_tile
     // (measured at N = K = 8192: 192 of the large tiles on 256 CUs already beat 768 of the small ones, 128 do not)
     if (want_tile == 256 || (want_tile == 0 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 >= (int64_t)device_cus() * 55))
       return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
-    return launch_f8<F8, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    return launch_f8<F8M16, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())
     return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);

@@ -306,6 +306,13 @@ struct PackedEpilogue {
         __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)abase_hi << 32) | (uint64_t)abase_lo), 0, __builtin_amdgcn_readfirstlane(arecords), 0x00020000);
     const uint32_t avoff0 = nn < p.N ? (uint32_t)rrow * apitch + (uint32_t)rchunk * (8u * kAccBytes) : 0x80000000u;
     u32x4 acc_in[ACC ? kPasses : 1][ACC == 2 ? 2 : 1];
+    // A result too large to be found in the L2s by whoever reads it next is stored non-temporally, so that it does not push
+    // the operand panels out of them on its way (bf16 8192^3: + 2 %).
+    const bool stream_out = (int64_t)p.M * p.N * kOutBytes >= (int64_t(32) << 20);
+    auto store16 = [&](u32x4 w, int voff, int soff) {
+      if (stream_out) __builtin_amdgcn_raw_buffer_store_b128(w, d_rsrc, voff, soff, 2);  // (cache policy bit 1: non-temporal)
+      else __builtin_amdgcn_raw_buffer_store_b128(w, d_rsrc, voff, soff, 0);
+    };
 #pragma unroll
     for (int i = 0; i < kStrips; ++i) {
       __builtin_amdgcn_sched_barrier(0);  // keep the strips apart: hoisting accumulator reads costs registers
@@ -364,13 +371,13 @@ struct PackedEpilogue {
           u32x4 w0, w1;
 #pragma unroll
           for (int e = 0; e < 4; ++e) { w0[e] = __float_as_uint(v[e]); w1[e] = __float_as_uint(v[4 + e]); }
-          __builtin_amdgcn_raw_buffer_store_b128(w0, d_rsrc, voff, 0, 0);
-          __builtin_amdgcn_raw_buffer_store_b128(w1, d_rsrc, voff, 16, 0);  // (the scalar offset is outside the range check: the piece is in or out whole)
+          store16(w0, voff, 0);
+          store16(w1, voff, 16);  // (the scalar offset is outside the range check: the piece is in or out whole)
         } else {
           u32x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = OUT == 1 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
-          __builtin_amdgcn_raw_buffer_store_b128(w, d_rsrc, voff, 0, 0);
+          store16(w, voff, 0);
         }
       }
     }
@@ -386,6 +393,7 @@ struct PackedEpilogue {
     const AccLane at = acc_lane(kAccLayout, kBlock, lane);
     const int wrow = at.row, wcol = at.col;
     const int rrow = lane / kChunksF, rchunk = lane % kChunksF;
+    const bool stream_out = (int64_t)p.M * p.N * (OUT == 2 ? 4 : 2) >= (int64_t(32) << 20);  // (see strips)
     // the lane's 8 columns are the same in every pass and strip: their bias values are fetched once
     const int32_t nn = n_wave + rchunk * 8;
     float bias[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -421,14 +429,22 @@ struct PackedEpilogue {
         if constexpr (OUT == 2) {
           if (mm < p.M && nn < p.N) {
             f32x4 *dst = (f32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 4);
-            dst[0] = f32x4{v[0], v[1], v[2], v[3]};
-            dst[1] = f32x4{v[4], v[5], v[6], v[7]};
+            if (stream_out) {
+              __builtin_nontemporal_store(f32x4{v[0], v[1], v[2], v[3]}, dst);
+              __builtin_nontemporal_store(f32x4{v[4], v[5], v[6], v[7]}, dst + 1);
+            } else {
+              dst[0] = f32x4{v[0], v[1], v[2], v[3]};
+              dst[1] = f32x4{v[4], v[5], v[6], v[7]};
+            }
           }
         } else {
           u32x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = OUT == 1 ? pack2_f16_rn(v[2 * e], v[2 * e + 1]) : pack2_bf16_rn(v[2 * e], v[2 * e + 1]);
-          if (mm < p.M && nn < p.N) *(u32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 2) = w;
+          if (mm < p.M && nn < p.N) {
+            if (stream_out) __builtin_nontemporal_store(w, (u32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 2));
+            else *(u32x4 *)(p.d + ((int64_t)mm * p.d_sm + nn) * 2) = w;
+          }
         }
       }
     }

@@ -73,7 +73,9 @@ def _events(fn, steps, warmup):
 # same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
 MEASURED_TRAFFIC = {"gelu": 268411308, "transpose": 268449994, "add": 402640502, "expr": 402796218, "softmax": 268466794, "layernorm": 268779749,
                     "expr_compiled": 402621054, "swiglu": 402555636, "l2norm_compiled": 268407520, "gelu_transposed": 268397184, "copy": 268435456,
-                    "permute": 268435456, "reduce": 134292547, "gemm_bf16": 1375346999, "gemm_bf16_gelu": 1755590499, "f8_m4096": 571433744}
+                    "permute": 268435456, "reduce": 134292547, "gemm_bf16": 1764717568, "gemm_bf16_gelu": 1756925952, "f8_m4096": 470365184,
+                    "gemm_f16": 21158853, "gemm_f16_graph": 21158853, "gemm_f16_splitk": 37989900, "f8_m16": 68542669, "f8_m64": 72475557, "f8_m128": 82781536,
+                    "f8_m128_splitk": 111420621}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -625,7 +627,7 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 160 and not workspace)) else "tn_kernel<F8M16, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8>",
            "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
            "checked": True, "check": "%d %dx64 blocks against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" % (n_blocks, min(M, 64), rel, FROB_TOL)}
-    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d" % M) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
+    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d%s" % (M, "_splitk" if workspace else "")) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
     if cpu:
         rows = min(M, 1024)
         hd = np.zeros(M * N, np.uint16)
@@ -798,9 +800,9 @@ def main():
         "permute": lambda s, w: bench_permute(kh, s, w, cpu),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel", key="gemm_bf16"),
         "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True, key="gemm_bf16_gelu"),
-        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform"),
-        "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform"),
-        "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True),
+        "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform", key="gemm_f16"),
+        "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform", key="gemm_f16_graph"),
+        "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True, key="gemm_f16_splitk"),
         "f8_m16": lambda s, w: bench_f8(kh, s, w, cpu, 16),
         "f8_m64": lambda s, w: bench_f8(kh, s, w, False, 64),
         "f8_m128": lambda s, w: bench_f8(kh, s, w, False, 128),

@@ -72,7 +72,10 @@ __device__ __forceinline__ void row_fetch(const char *base, int32_t vpr, u32x4 (
 // work on the current one, so that a workgroup always has a load in flight.  The two exchange areas of a row's two
 // reduces are safe to reuse from row to row: a wave can write one again only after the barrier of the other, which every
 // wave reaches after it has read the first.
-template <int CH, int THREADS>
+// WALK = false: one row per workgroup and as many workgroups as rows (the host's choice for many rows of up to 8192
+// elements: the dispatcher then keeps every CU full to the end and workgroups drift into different phases, which is worth
+// more than the load in flight across rows - 1024 elements 49 -> 44 us, 8192 elements 47.7 -> 46.3 us for 128 MiB).
+template <int CH, int THREADS, bool WALK>
 __global__ __launch_bounds__(THREADS) void softmax_kernel(FusedRow p, int dtype) {
   __shared__ float red[2][16];
   u32x4 raw[CH];
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(FusedRow p, int dtype)
     float f[CH][8];
 #pragma unroll
     for (int c = 0; c < CH; ++c) widen16x8(raw[c], dtype, f[c]);
-    if (i + (int32_t)gridDim.x < p.rows) row_fetch<CH, THREADS, true>(p.x + (int64_t)(i + gridDim.x) * p.x_stride0 * 2, p.vec_per_row, raw);
+    if (WALK && i + (int32_t)gridDim.x < p.rows) row_fetch<CH, THREADS, true>(p.x + (int64_t)(i + gridDim.x) * p.x_stride0 * 2, p.vec_per_row, raw);
     float m = -__builtin_inff();
     bool any_nan = false;
 #pragma unroll
@@ -127,6 +130,7 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(FusedRow p, int dtype)
       const int32_t jv = c * THREADS + threadIdx.x;
       if (jv < p.vec_per_row) store8<true>(p.out, dtype, (int64_t)i * p.out_stride0 + (int64_t)jv * 8, f[c]);
     }
+    if (!WALK) break;
   }
 }
 
@@ -199,7 +203,9 @@ __global__ __launch_bounds__(THREADS) void norm_kernel(FusedRow p, int dtype) {
 
 int launch_fused_row(const FusedRow &p, int dtype, bool softmax, hipStream_t s) {
   const int vpr = p.vec_per_row;
-  const int threads = vpr <= 256 ? 64 : vpr <= 1024 ? 256 : 1024;
+  // one wave per row up to 256 vectors for softmax, up to 128 for the norms (whose 64-lane build with four chunks per lane
+  // needs more registers than the occupancy it is meant to buy: 2048 elements 61 -> 50 us on 256 lanes)
+  const int threads = vpr <= (softmax ? 256 : 128) ? 64 : vpr <= 1024 ? 256 : 1024;
   const int ch = (vpr + threads - 1) / threads;
   // as many workgroups as are resident at once; each walks its share of the rows
 #define KAPY_FUSED(CH_, TH_)                                                           \
@@ -207,11 +213,12 @@ int launch_fused_row(const FusedRow &p, int dtype, bool softmax, hipStream_t s) 
     int per_cu = 1;                                                                    \
     const size_t lds = softmax ? 0 : (size_t)2 * CH_ * TH_ * 16;                       \
     if (lds > 48 * 1024) KAPY_HIP_CHECK(hipFuncSetAttribute((const void *)norm_kernel<CH_, TH_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-    if (softmax) KAPY_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, softmax_kernel<CH_, TH_>, TH_, 0)); \
+    if (softmax) KAPY_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, softmax_kernel<CH_, TH_, true>, TH_, 0)); \
     else KAPY_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, norm_kernel<CH_, TH_>, TH_, lds)); \
     const int64_t resident = (int64_t)device_cus() * (per_cu > 0 ? per_cu : 1);        \
     dim3 grid((unsigned)(p.rows < resident ? p.rows : resident));                      \
-    if (softmax) softmax_kernel<CH_, TH_><<<grid, TH_, 0, s>>>(p, dtype);              \
+    if (softmax && TH_ <= 256 && p.rows >= 4 * resident) softmax_kernel<CH_, TH_, false><<<dim3((unsigned)p.rows), TH_, 0, s>>>(p, dtype); \
+    else if (softmax) softmax_kernel<CH_, TH_, true><<<grid, TH_, 0, s>>>(p, dtype);   \
     else norm_kernel<CH_, TH_><<<grid, TH_, lds, s>>>(p, dtype);                       \
   } while (0)
 #define KAPY_FUSED_CH(TH_)                                                             \

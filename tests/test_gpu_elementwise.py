@@ -308,6 +308,30 @@ def test_softmax_rows_every_launch_shape(ko, row_path, dtype, m, n):
     _check_ulp(got, want, dtype)
 
 
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(60000, 64), (50000, 200), (9000, 1000), (7000, 4096), (6500, 8192), (6200, 5000)])
+def test_softmax_many_rows(ko, dtype, m, n):
+    """With many times more rows than workgroups fit on the device, softmax takes one workgroup per row instead of resident
+    workgroups that walk the rows.  The device computes every row; the checker a spread sample of them (rows are
+    independent), and a second sample is compared against the first rows of a short launch, which takes the walking kernel."""
+    x = ko.fill_normal(m * n, dtype, 58 + n % 89, std=2.0).reshape(m, n)
+    insts = kh.softmax_insts(dtype)
+    dout = dev_zeros(m * n, 2)
+    kh.elementwise(kh.program(insts), [dglobal(to_dev(x), m, n, n, 1, dtype)], dglobal(dout, m, n, n, 1, dtype))
+    sync()
+    got = to_host(dout, np.uint16, (m, n))
+    rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 61)), [m - 1, m - 2, 1]]))
+    xs = np.ascontiguousarray(x[rows])
+    want = np.zeros((len(rows), n), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(xs, len(rows), n, n, 1, dtype)], ko.mk_global(want, len(rows), n, n, 1, dtype)) == 0
+    _check_ulp(got[rows], want, dtype)
+    few = 40
+    dfew = dev_zeros(few * n, 2)
+    kh.elementwise(kh.program(insts), [dglobal(to_dev(np.ascontiguousarray(x[:few])), few, n, n, 1, dtype)], dglobal(dfew, few, n, n, 1, dtype))
+    sync()
+    assert np.array_equal(to_host(dfew, np.uint16, (few, n)), got[:few])
+
+
 def test_softmax_special_rows(ko, row_path):
     m, n = 6, 1024
     x = ko.fill_normal(m * n, kh.F16, 55, std=4.0).reshape(m, n)

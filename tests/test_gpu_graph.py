@@ -76,7 +76,8 @@ def test_every_kernel_family_replays_from_a_graph():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         _calls(bufs, captured)
-    assert kh.elementwise_specialize_stats()[1] == launches_before + 1   # the compiled kernel is part of the graph
+    # the compiled kernel is part of the graph (more than one, if tests that ran earlier in this process compiled other programs of _calls)
+    assert kh.elementwise_specialize_stats()[1] >= launches_before + 1
     for seed in (2, 3, 4):
         _refill(bufs, seed)
         for t in captured.values():

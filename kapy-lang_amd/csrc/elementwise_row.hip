@@ -201,8 +201,110 @@ __global__ __launch_bounds__(THREADS) void norm_kernel(FusedRow p, int dtype) {
   }
 }
 
+// Rows of up to 32 vectors (256 elements): a wave holds 64 / GROUP rows at a time, GROUP lanes each (GROUP = 8, 16, 32: the
+// next power of two from the row's vectors), so that short rows do not leave most lanes of a wave idle (one wave per row of
+// 64 elements: 8 lanes of 64 at work).  A row's reduces are butterflies inside its group of lanes; no LDS, no barrier.
+template <int GROUP, bool MAX>
+__device__ __forceinline__ float group_fold(float acc) {
+#pragma unroll
+  for (int off = GROUP / 2; off >= 1; off >>= 1) {
+    const float other = __shfl_xor(acc, off, 64);
+    acc = MAX ? max_nan(acc, other) : acc + other;
+  }
+  return acc;
+}
+
+template <int GROUP>
+__global__ __launch_bounds__(256) void softmax_short_kernel(FusedRow p, int dtype) {
+  const int64_t i = (int64_t)blockIdx.x * (256 / GROUP) + threadIdx.x / GROUP;
+  const int32_t jv = threadIdx.x % GROUP;
+  const bool active = i < p.rows && jv < p.vec_per_row;
+  u32x4 raw = {0, 0, 0, 0};
+  if (active) raw = __builtin_nontemporal_load((const u32x4 *)(p.x + (i * p.x_stride0 + (int64_t)jv * 8) * 2));
+  float f[8];
+  widen16x8(raw, dtype, f);
+  float m = -__builtin_inff();
+  bool any_nan = false;
+  if (active) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      m = fmaxf(m, f[e]);
+      any_nan |= f[e] != f[e];
+    }
+  }
+  m = group_fold<GROUP, true>(any_nan ? __builtin_nanf("") : m);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {  // (the same steps as softmax_kernel, which explains them)
+    const float x = __fsub_rn(f[e], m);
+    const float hi = x * 1.44269504088896341f;
+    float lo = __builtin_fmaf(x, 1.44269504088896341f, -hi);
+    lo = !(x <= -3e38f) ? lo : 0.f;
+    const float pw = __builtin_amdgcn_exp2f(hi);
+    f[e] = __builtin_fmaf(pw, lo * 0.693147180559945309f, pw);
+  }
+  float sum = active ? ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7])) : 0.f;
+  sum = group_fold<GROUP, false>(sum);
+  const float rcp = __builtin_amdgcn_rcpf(sum);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float q = f[e] * rcp;
+    const float rem = __builtin_fmaf(-q, sum, f[e]);
+    f[e] = __builtin_fmaf(rem, rcp, q);
+  }
+  if (active) store8<true>(p.out, dtype, i * p.out_stride0 + (int64_t)jv * 8, f);
+}
+
+template <int GROUP>
+__global__ __launch_bounds__(256) void norm_short_kernel(FusedRow p, int dtype) {
+  const int64_t i = (int64_t)blockIdx.x * (256 / GROUP) + threadIdx.x / GROUP;
+  const int32_t jv = threadIdx.x % GROUP;
+  const bool active = i < p.rows && jv < p.vec_per_row;
+  u32x4 raw = {0, 0, 0, 0}, graw = {0, 0, 0, 0}, braw = {0, 0, 0, 0};
+  if (active) raw = __builtin_nontemporal_load((const u32x4 *)(p.x + (i * p.x_stride0 + (int64_t)jv * 8) * 2));
+  if (active && p.gamma) graw = *(const u32x4 *)(p.gamma + (int64_t)jv * 16);
+  if (active && p.beta) braw = *(const u32x4 *)(p.beta + (int64_t)jv * 16);
+  float f[8];
+  widen16x8(raw, dtype, f);
+  if (p.centre) {
+    float sum = active ? ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7])) : -0.f;
+    const float mean = __fmul_rn(group_fold<GROUP, false>(sum), p.inv_n);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = __fsub_rn(f[e], mean);
+  }
+  float sq = 0.f;
+  if (active) {
+    float s8[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s8[e] = __fmul_rn(f[e], f[e]);
+    sq = ((s8[0] + s8[1]) + (s8[2] + s8[3])) + ((s8[4] + s8[5]) + (s8[6] + s8[7]));
+  }
+  const float var = __fmul_rn(group_fold<GROUP, false>(sq), p.inv_n);
+  const float rstd = __builtin_amdgcn_rsqf(__fadd_rn(var, p.eps));
+  float g[8], b[8];
+  widen16x8(graw, dtype, g);
+  widen16x8(braw, dtype, b);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float r = __fmul_rn(f[e], rstd);
+    if (p.gamma) r = __fmul_rn(r, g[e]);
+    if (p.beta) r = __fadd_rn(r, b[e]);
+    f[e] = r;
+  }
+  if (active) store8<true>(p.out, dtype, i * p.out_stride0 + (int64_t)jv * 8, f);
+}
+
+template <int GROUP>
+int launch_short_row(const FusedRow &p, int dtype, bool softmax, hipStream_t s) {
+  const int64_t groups = ((int64_t)p.rows + 256 / GROUP - 1) / (256 / GROUP);
+  if (softmax) softmax_short_kernel<GROUP><<<dim3((unsigned)groups), 256, 0, s>>>(p, dtype);
+  else norm_short_kernel<GROUP><<<dim3((unsigned)groups), 256, 0, s>>>(p, dtype);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 int launch_fused_row(const FusedRow &p, int dtype, bool softmax, hipStream_t s) {
   const int vpr = p.vec_per_row;
+  if (vpr <= 32 && p.rows >= 64) return vpr <= 8 ? launch_short_row<8>(p, dtype, softmax, s) : vpr <= 16 ? launch_short_row<16>(p, dtype, softmax, s) : launch_short_row<32>(p, dtype, softmax, s);
   // one wave per row up to 256 vectors for softmax, up to 128 for the norms (whose 64-lane build with four chunks per lane
   // needs more registers than the occupancy it is meant to buy: 2048 elements 61 -> 50 us on 256 lanes)
   const int threads = vpr <= (softmax ? 256 : 128) ? 64 : vpr <= 1024 ? 256 : 1024;

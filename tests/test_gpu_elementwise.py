@@ -309,11 +309,12 @@ def test_softmax_rows_every_launch_shape(ko, row_path, dtype, m, n):
 
 
 @pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
-@pytest.mark.parametrize("m,n", [(60000, 64), (50000, 200), (9000, 1000), (7000, 4096), (6500, 8192), (6200, 5000)])
+@pytest.mark.parametrize("m,n", [(60000, 64), (50000, 200), (3001, 24), (70, 128), (1000, 256), (9000, 1000), (7000, 4096), (6500, 8192), (6200, 5000)])
 def test_softmax_many_rows(ko, dtype, m, n):
     """With many times more rows than workgroups fit on the device, softmax takes one workgroup per row instead of resident
-    workgroups that walk the rows.  The device computes every row; the checker a spread sample of them (rows are
-    independent), and a second sample is compared against the first rows of a short launch, which takes the walking kernel."""
+    workgroups that walk the rows, and rows of up to 256 elements share a wave (8, 16 or 32 lanes per row).  The device
+    computes every row; the checker a spread sample of them (rows are independent), and the first rows are compared
+    against a short launch, which takes the walking kernel (another order of the fp32 sums: within the tolerance)."""
     x = ko.fill_normal(m * n, dtype, 58 + n % 89, std=2.0).reshape(m, n)
     insts = kh.softmax_insts(dtype)
     dout = dev_zeros(m * n, 2)
@@ -329,7 +330,24 @@ def test_softmax_many_rows(ko, dtype, m, n):
     dfew = dev_zeros(few * n, 2)
     kh.elementwise(kh.program(insts), [dglobal(to_dev(np.ascontiguousarray(x[:few])), few, n, n, 1, dtype)], dglobal(dfew, few, n, n, 1, dtype))
     sync()
-    assert np.array_equal(to_host(dfew, np.uint16, (few, n)), got[:few])
+    _check_ulp(to_host(dfew, np.uint16, (few, n)), got[:few], dtype)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(40000, 64), (3001, 24), (70, 128), (5000, 200), (1000, 256)])
+def test_norms_many_short_rows(ko, dtype, m, n):
+    """Layer norm and RMS norm over rows that share a wave, every row against the checker."""
+    got, want = _row_case(ko, kh.layernorm_insts(n, dtype), dtype, m, n, 64, extra=("gamma", "beta"))
+    # x^ * gamma + beta cancels here and there among a million elements, and what another order of the fp32 sums changes
+    # in the last place of x^ * gamma is then many last places of the result: bounded in units of the terms instead
+    g, w = _as_f64(got, dtype), _as_f64(want, dtype)
+    eps = 2.0 ** -10 if dtype == kh.F16 else 2.0 ** -7
+    assert np.array_equal(np.isnan(g), np.isnan(w)) and np.all(np.abs(g - w)[~np.isnan(w)] <= 2 * eps * np.maximum(np.abs(w[~np.isnan(w)]), 1.0))
+    assert np.mean(got == want) > 0.98
+    got, want = _row_case(ko, kh.layernorm_insts(n, dtype, affine=False), dtype, m, n, 65)
+    _check_ulp(got, want, dtype)
+    got, want = _row_case(ko, kh.rmsnorm_insts(n, dtype), dtype, m, n, 66, extra=("gamma",))
+    _check_ulp(got, want, dtype)
 
 
 def test_softmax_special_rows(ko, row_path):

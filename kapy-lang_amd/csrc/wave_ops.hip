@@ -6,6 +6,9 @@
 // lane is shuffled with shfl.sync.idx and a select chain keeps the one whose iv' matches.
 // ReduceOpToLLVM.cpp:51-172 — an in-lane tree over the loop ivs, then shfl.sync.bfly rounds over
 // the lanes that share the reduced axis.  On gfx950 the shuffles are ds_bpermute_b32 over 64 lanes.
+#include <algorithm>
+#include <mutex>
+
 #include "common.hpp"
 #include "layout.hpp"
 #include "numeric.hpp"
@@ -118,31 +121,117 @@ __global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p) {
   if (lane == 0) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
 }
 
-// 16-bit elements, kept axis contiguous: a workgroup of 512 lanes owns 32 kept indices (4 lanes x 8
-// consecutive elements, one 128-bit load each) and splits the reduced axis 128 ways; partial results
-// meet in LDS.
-template <bool BF16, int KIND>
-__global__ __launch_bounds__(512) void reduce_cols_vec_kernel(ReduceParams p) {
-  __shared__ float part[128][32 + 1];
-  const int cl = threadIdx.x & 3, rg = threadIdx.x >> 2;
-  const int64_t keep0 = (int64_t)blockIdx.x * 32 + cl * 8;
+// 16-bit elements, kept axis contiguous: a workgroup of 256 lanes owns a strip of 8 * LPR kept indices - LPR lanes x one
+// 128-bit load per reduced index - and a chunk of the reduced axis, which its 256 / LPR groups of lanes walk with four
+// loads in flight each; the groups' partial results meet in LDS.  With one chunk the strip's results go to the result;
+// with more (few kept indices, many reduced ones: a tall matrix would otherwise keep a handful of CUs busy) every chunk
+// leaves an fp32 partial line and reduce_partials_kernel folds the lines in chunk order.
+template <bool BF16, int KIND, int LPR>
+__global__ __launch_bounds__(256) void reduce_cols_strip_kernel(ReduceParams p, float *partials, int32_t per_chunk) {
+  constexpr int GROUPS = 256 / LPR, COLS = LPR * 8;
+  __shared__ float part[GROUPS][COLS + 1];
+  const int cl = threadIdx.x % LPR, rg = threadIdx.x / LPR;
+  const int64_t keep0 = (int64_t)blockIdx.x * COLS + cl * 8;
+  const int32_t r_begin = blockIdx.y * per_chunk, r_end = min(p.n_red, r_begin + per_chunk);
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = KIND == 0 ? -0.f : -__builtin_inff();
-  for (int32_t r = rg; r < p.n_red; r += 128) {
-    float f[8];
-    widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(p.src + (r * p.s_red + keep0) * 2)), f);
+  if (keep0 < p.n_keep) {  // (whole vectors: n_keep is a multiple of 8)
+    const char *col = p.src + keep0 * 2;
+    constexpr int U = 4;
+    int32_t r = r_begin + rg;
+    for (; r + GROUPS * (U - 1) < r_end; r += GROUPS * U) {
+      u32x4_t x[U];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = combine(acc[e], f[e], KIND);
+      for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)(r + GROUPS * u) * p.s_red * 2));
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float f[8];
+        widen8<BF16>(x[u], f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = combine(acc[e], f[e], KIND);
+      }
+    }
+    for (; r < r_end; r += GROUPS) {
+      float f[8];
+      widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)r * p.s_red * 2)), f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = combine(acc[e], f[e], KIND);
+    }
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) part[rg][cl * 8 + e] = acc[e];
   __syncthreads();
-  if (threadIdx.x < 32) {
+  const int64_t keep = (int64_t)blockIdx.x * COLS + threadIdx.x;
+  if (threadIdx.x < COLS && keep < p.n_keep) {
     float t = KIND == 0 ? -0.f : -__builtin_inff();
-    for (int g = 0; g < 128; ++g) t = combine(t, part[g][threadIdx.x], KIND);
-    store_from_f32(p.dst, p.dst_dtype, ((int64_t)blockIdx.x * 32 + threadIdx.x) * p.d_keep, t);
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) t = combine(t, part[g][threadIdx.x], KIND);
+    if (partials) partials[(int64_t)blockIdx.y * p.n_keep + keep] = t;
+    else store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
   }
+}
+
+// The second pass over `chunks` fp32 partial lines of n_keep values: 64 kept indices per workgroup, 16 groups of lanes
+// share out the lines, folded in chunk order within a group and in group order across them (the same result every run).
+template <int KIND>
+__global__ __launch_bounds__(1024) void reduce_partials_kernel(ReduceParams p, const float *partials, int32_t chunks) {
+  __shared__ float part[16][64 + 1];
+  const int cl = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int64_t keep = (int64_t)blockIdx.x * 64 + cl;
+  float acc = KIND == 0 ? -0.f : -__builtin_inff();
+  if (keep < p.n_keep)
+    for (int32_t c = rg; c < chunks; c += 16) acc = combine(acc, partials[(int64_t)c * p.n_keep + keep], KIND);
+  part[rg][cl] = acc;
+  __syncthreads();
+  if (threadIdx.x < 64 && keep < p.n_keep) {
+    float t = KIND == 0 ? -0.f : -__builtin_inff();
+#pragma unroll
+    for (int g = 0; g < 16; ++g) t = combine(t, part[g][cl], KIND);
+    store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
+  }
+}
+
+// Memory for the partial lines: one block per device, allocated at the first call that wants it and kept.  Calls on one
+// stream use it in turn by stream order; a call on another stream first makes its stream wait for the event that the last
+// user recorded behind its second pass.  The mutex is held from that wait to the new record, so calls from several host
+// threads cannot interleave.  Not available - and then the caller reduces in one pass - while the stream is being
+// captured (an event of another stream's work cannot be waited for inside a capture) or when the allocation fails.
+constexpr int kMaxPartialsDevices = 16;
+constexpr size_t kPartialsBytes = size_t(1) << 20;  // the launch keeps chunks * n_keep * 4 within this
+struct Partials {
+  float *lines = nullptr;
+  hipEvent_t free_again = nullptr;
+  hipStream_t last_stream = nullptr;
+  bool used = false;
+  int state = 0;  // 0 not tried, 1 ready, -1 not available
+};
+std::mutex partials_mutex;
+Partials partials_of[kMaxPartialsDevices];
+
+// Call with partials_mutex held.  The device's block, ready for work on `s`, or nullptr.
+Partials *partials_for(hipStream_t s) {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxPartialsDevices) return nullptr;
+  Partials &P = partials_of[dev];
+  if (P.state == 0) {
+    if (hipMalloc((void **)&P.lines, kPartialsBytes) == hipSuccess && hipEventCreateWithFlags(&P.free_again, hipEventDisableTiming) == hipSuccess) P.state = 1;
+    else {
+      (void)hipGetLastError();
+      P.state = -1;
+    }
+  }
+  if (P.state != 1) return nullptr;
+  if (P.used && P.last_stream != s && hipStreamWaitEvent(s, P.free_again, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return &P;
 }
 
 // One lane per kept index: used when the kept axis is the contiguous one (coalesced as is).
@@ -223,10 +312,48 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     dim3 grid((unsigned)((p.n_keep + 3) / 4));
     if (bf) { if (kind == 0) reduce_rows_vec_kernel<true, 0><<<grid, 256, 0, s>>>(p); else reduce_rows_vec_kernel<true, 1><<<grid, 256, 0, s>>>(p); }
     else { if (kind == 0) reduce_rows_vec_kernel<false, 0><<<grid, 256, 0, s>>>(p); else reduce_rows_vec_kernel<false, 1><<<grid, 256, 0, s>>>(p); }
-  } else if (b16 && aligned && p.s_keep == 1 && p.n_keep % 32 == 0 && (p.s_red * 2) % 16 == 0 && p.n_red >= 128) {
-    dim3 grid((unsigned)(p.n_keep / 32));
-    if (bf) { if (kind == 0) reduce_cols_vec_kernel<true, 0><<<grid, 512, 0, s>>>(p); else reduce_cols_vec_kernel<true, 1><<<grid, 512, 0, s>>>(p); }
-    else { if (kind == 0) reduce_cols_vec_kernel<false, 0><<<grid, 512, 0, s>>>(p); else reduce_cols_vec_kernel<false, 1><<<grid, 512, 0, s>>>(p); }
+  } else if (b16 && aligned && p.s_keep == 1 && p.n_keep % 8 == 0 && (p.s_red * 2) % 16 == 0 && p.n_red >= 32) {
+    // strips of 256 kept indices (512-byte runs per reduced index), of 64 for narrow sources; the reduced axis in as many
+    // chunks as bring the launch to about four workgroups per CU, of at least 128 reduced indices each, as far as their
+    // partial lines fit the block.  Measured for 128 MiB of fp16: 8192 x 8192 46 -> 29 us (64-wide strips: 31, eight
+    // workgroups per CU: 31, eight loads in flight per lane: 30), 1 Mi x 64 4335 -> 34 us.
+    const int lpr = p.n_keep >= 256 ? 32 : 8, cols = lpr * 8;
+    const int64_t strips = ((int64_t)p.n_keep + cols - 1) / cols, want = 4 * (int64_t)device_cus();
+    if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 128, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
+    std::unique_lock<std::mutex> lock(partials_mutex, std::defer_lock);
+    Partials *P = nullptr;
+    if (chunks > 1) {
+      lock.lock();
+      P = partials_for(s);
+      if (!P) lock.unlock();
+    }
+    if (!P) chunks = 1;
+    const int32_t per_chunk = (int32_t)((p.n_red + chunks - 1) / chunks);
+    chunks = (p.n_red + per_chunk - 1) / per_chunk;
+    float *lines = P ? P->lines : nullptr;
+    dim3 grid((unsigned)strips, (unsigned)chunks);
+#define KAPY_STRIP(BF_, KIND_)                                                                                                        \
+  do {                                                                                                                                \
+    if (lpr == 32) reduce_cols_strip_kernel<BF_, KIND_, 32><<<grid, 256, 0, s>>>(p, lines, per_chunk);                                \
+    else reduce_cols_strip_kernel<BF_, KIND_, 8><<<grid, 256, 0, s>>>(p, lines, per_chunk);                                           \
+  } while (0)
+    if (bf) { if (kind == 0) KAPY_STRIP(true, 0); else KAPY_STRIP(true, 1); }
+    else { if (kind == 0) KAPY_STRIP(false, 0); else KAPY_STRIP(false, 1); }
+#undef KAPY_STRIP
+    if (P) {
+      if (kind == 0) reduce_partials_kernel<0><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
+      else reduce_partials_kernel<1><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
+      // whatever was launched reads or writes the block: the next user waits for all of it
+      const hipError_t launched = hipGetLastError(), recorded = hipEventRecord(P->free_again, s);
+      P->last_stream = s;
+      P->used = true;
+      if (launched != hipSuccess) return fail(KAPY_ERR_HIP, "reduce: %s", hipGetErrorString(launched));
+      if (recorded != hipSuccess) {
+        P->state = -1;  // nobody could wait for this call's use of the block: it is not handed out again
+        return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
+      }
+    }
   } else if (p.s_keep == 1 && p.s_red != 1) reduce_lane_kernel<<<(p.n_keep + 255) / 256, 256, 0, s>>>(p);
   else reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());

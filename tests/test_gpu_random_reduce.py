@@ -123,6 +123,64 @@ def test_reduce_of_lines_with_nan_infinities_and_signed_zeros(ko, dtype, m, n, a
             assert np.all(np.abs(pgf[rest] - pwf[rest]) <= 2 * EPS[dtype] * np.abs(pwf[rest]) + 1e-3)
 
 
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(100000, 64), (20000, 200), (5000, 4096), (4097, 72), (300000, 8), (129, 8192)])
+def test_reduce_along_axis0_of_tall_matrices(ko, dtype, m, n):
+    """Few kept indices and many reduced ones: the reduced axis is shared out over workgroups, whose fp32 partial lines a second
+    pass folds in a fixed order.  max bit-exact, sum within the fp32 accumulation bound, twice with the same bits, and the
+    result type's rounding when the result is 16-bit."""
+    x = ko.fill_normal(m * n, dtype, 77 + n, 0)
+    x.reshape(m, n)[m // 3, 5] = 0x7c00 if dtype == kh.F16 else 0x7f80   # one +inf: its column sums and maximises to +inf
+    dx = to_dev(x)
+    for kind in (0, 1):
+        for ddt in (kh.F32, dtype):
+            db = kh.DTYPE_BYTES[ddt]
+            want = np.zeros(n, NP[db])
+            assert ko.lib().ko_reduce(C.byref(ko.mk_global(x, m, n, n, 1, dtype)), C.byref(ko.mk_global(want, 1, n, n, 1, ddt)), 0, kind) == 0
+            runs = []
+            for _ in range(2):
+                dd = to_dev(np.full(n + 16, 0x5A5A, NP[db]))
+                kh.reduce(dglobal(dx, m, n, n, 1, dtype), dglobal(dd, 1, n, n, 1, ddt), 0, kind)
+                sync()
+                runs.append(to_host(dd, NP[db]))
+            got = runs[0]
+            assert np.array_equal(runs[0], runs[1]) and np.all(got[n:] == 0x5A5A)
+            got = got[:n]
+            if kind == 1:
+                assert np.array_equal(got, want)
+                continue
+            g, w = ko.decode(got.view(VALUE[ddt]), ddt), ko.decode(want.view(VALUE[ddt]), ddt)
+            assert np.isinf(w[5]) and g[5] == w[5]
+            mass = np.abs(ko.decode(x.view(VALUE[dtype]), dtype)).reshape(m, n).sum(axis=0)
+            rest = np.isfinite(w)
+            assert np.all(np.abs(g - w)[rest] <= (2.0 ** -22 * mass + 2.0 * EPS[ddt] * np.abs(w) + 1e-30)[rest])
+
+
+def test_tall_reduces_on_two_streams_share_the_partial_lines_in_turn():
+    """The library keeps one block of partial lines per device; calls on different streams must not overlap in it."""
+    import torch
+    m, n = 60000, 64
+    xs = [torch.randn(m, n, device="cuda").half() for _ in range(6)]
+    alone = []
+    for x in xs:
+        d = torch.zeros(n, device="cuda", dtype=torch.float32)
+        kh.reduce(dglobal(x, m, n, n, 1, kh.F16), dglobal(d, 1, n, n, 1, kh.F32), 0, 0)
+        sync()
+        alone.append(d.clone())
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for st in streams:
+        st.wait_stream(torch.cuda.current_stream())
+    for rep in range(5):
+        outs = [torch.zeros(n, device="cuda", dtype=torch.float32) for _ in xs]
+        for k, (x, d) in enumerate(zip(xs, outs)):
+            with torch.cuda.stream(streams[k % 2]):
+                kh.reduce(dglobal(x, m, n, n, 1, kh.F16), dglobal(d, 1, n, n, 1, kh.F32), 0, 0, stream=streams[k % 2].cuda_stream)
+        for st in streams:
+            st.synchronize()
+        for d, a in zip(outs, alone):
+            assert torch.equal(d, a)
+
+
 @pytest.mark.parametrize("seed", range(32))
 def test_random_batched_copy(ko, seed):
     """A b x h grid of tiles moved between two 4-D layouts (any of the two orders of the grid axes on either side), with or

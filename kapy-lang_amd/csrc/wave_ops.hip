@@ -84,16 +84,18 @@ __device__ __forceinline__ void widen8(u32x4_t v, float f[8]) {
     }
   }
 }
+// With few long lines the reduced axis is shared out as well (blockIdx.y = chunk of vecs_per_chunk vectors): every
+// (line, chunk) leaves an fp32 partial result at partials[line * chunks + chunk], which a second launch folds per line.
 template <bool BF16, int KIND>
-__global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p) {
+__global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p, float *partials, int32_t vecs_per_chunk) {
   const int lane = threadIdx.x & 63;
   const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (keep >= p.n_keep) return;
   const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * 2);
-  const int32_t vecs = p.n_red / 8;
+  const int32_t vecs = min(p.n_red / 8, (int32_t)(blockIdx.y + 1) * vecs_per_chunk);
   float acc = KIND == 0 ? -0.f : -__builtin_inff();
   constexpr int U = 4;
-  int32_t v = lane;
+  int32_t v = blockIdx.y * vecs_per_chunk + lane;
   for (; v + 64 * (U - 1) < vecs; v += 64 * U) {
     u32x4_t x[U];
 #pragma unroll
@@ -118,7 +120,30 @@ __global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p) {
     float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(acc)));
     acc = combine(acc, other, KIND);
   }
-  if (lane == 0) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
+  if (lane == 0) {
+    if (partials) partials[keep * gridDim.y + blockIdx.y] = acc;
+    else store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
+  }
+}
+
+// The same for lines of up to 512 elements: a line takes GROUP lanes (8, 16, 32 or 64: the next power of two from its
+// vectors), a wave 64 / GROUP lines at a time, each lane one 128-bit load; the butterfly stays inside the group.
+template <bool BF16, int KIND, int GROUP>
+__global__ __launch_bounds__(256) void reduce_rows_short_kernel(ReduceParams p) {
+  const int64_t keep = (int64_t)blockIdx.x * (256 / GROUP) + threadIdx.x / GROUP;
+  const int32_t jv = threadIdx.x % GROUP;
+  float acc = KIND == 0 ? -0.f : -__builtin_inff();
+  if (keep < p.n_keep && jv < p.n_red / 8) {
+    float f[8];
+    widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(p.src + keep * p.s_keep * 2) + jv), f);
+    acc = combine(combine(combine(f[0], f[1], KIND), combine(f[2], f[3], KIND), KIND), combine(combine(f[4], f[5], KIND), combine(f[6], f[7], KIND), KIND), KIND);
+  }
+#pragma unroll
+  for (int off = GROUP / 2; off >= 1; off >>= 1) {
+    float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute(((threadIdx.x & 63) ^ off) << 2, (int)f32_bits(acc)));
+    acc = combine(acc, other, KIND);
+  }
+  if (jv == 0 && keep < p.n_keep) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
 }
 
 // 16-bit elements, kept axis contiguous: a workgroup of 256 lanes owns a strip of 8 * LPR kept indices - LPR lanes x one
@@ -308,10 +333,59 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
   hipStream_t s = (hipStream_t)stream;
   const bool b16 = src->dtype == KAPY_F16 || src->dtype == KAPY_BF16, bf = src->dtype == KAPY_BF16;
   const bool aligned = ((uintptr_t)p.src & 15) == 0;
-  if (b16 && aligned && p.s_red == 1 && p.n_red % 8 == 0 && (p.s_keep * 2) % 16 == 0 && p.n_red >= 512) {
-    dim3 grid((unsigned)((p.n_keep + 3) / 4));
-    if (bf) { if (kind == 0) reduce_rows_vec_kernel<true, 0><<<grid, 256, 0, s>>>(p); else reduce_rows_vec_kernel<true, 1><<<grid, 256, 0, s>>>(p); }
-    else { if (kind == 0) reduce_rows_vec_kernel<false, 0><<<grid, 256, 0, s>>>(p); else reduce_rows_vec_kernel<false, 1><<<grid, 256, 0, s>>>(p); }
+  std::unique_lock<std::mutex> lock(partials_mutex, std::defer_lock);
+  if (b16 && aligned && p.s_red == 1 && p.n_red % 8 == 0 && (p.s_keep * 2) % 16 == 0 && p.n_red <= 512 && p.n_red >= 8) {
+    const int vecs = p.n_red / 8, group = vecs <= 8 ? 8 : vecs <= 16 ? 16 : vecs <= 32 ? 32 : 64;
+    const int64_t wgs = ((int64_t)p.n_keep + 256 / group - 1) / (256 / group);
+    if (wgs > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 workgroups");
+    dim3 grid((unsigned)wgs);
+#define KAPY_SHORT(BF_, KIND_)                                                                       \
+  do {                                                                                               \
+    if (group == 8) reduce_rows_short_kernel<BF_, KIND_, 8><<<grid, 256, 0, s>>>(p);                 \
+    else if (group == 16) reduce_rows_short_kernel<BF_, KIND_, 16><<<grid, 256, 0, s>>>(p);          \
+    else if (group == 32) reduce_rows_short_kernel<BF_, KIND_, 32><<<grid, 256, 0, s>>>(p);          \
+    else reduce_rows_short_kernel<BF_, KIND_, 64><<<grid, 256, 0, s>>>(p);                           \
+  } while (0)
+    if (bf) { if (kind == 0) KAPY_SHORT(true, 0); else KAPY_SHORT(true, 1); }
+    else { if (kind == 0) KAPY_SHORT(false, 0); else KAPY_SHORT(false, 1); }
+#undef KAPY_SHORT
+  } else if (b16 && aligned && p.s_red == 1 && p.n_red % 8 == 0 && (p.s_keep * 2) % 16 == 0 && p.n_red > 512) {
+    // four lines per workgroup; with fewer workgroups than CUs, chunks of at least 256 vectors of the reduced axis as well,
+    // up to four workgroups per CU (their partial results within the block): 64 lines of 1 Mi elements 312 -> 33 us, 256
+    // lines of 256 Ki 82 -> 30 us.  The second launch costs about 6 us: 1024 lines of 64 Ki elements are faster whole.
+    const int64_t wgs = ((int64_t)p.n_keep + 3) / 4, want = 4 * (int64_t)device_cus(), vecs = p.n_red / 8;
+    int64_t chunks = wgs >= device_cus() ? 1 : std::max<int64_t>(1, std::min<int64_t>({(want + wgs - 1) / wgs, vecs / 256, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
+    Partials *P = nullptr;
+    if (chunks > 1) {
+      lock.lock();
+      P = partials_for(s);
+      if (!P) lock.unlock();
+    }
+    if (!P) chunks = 1;
+    const int32_t vecs_per_chunk = (int32_t)((vecs + chunks - 1) / chunks);
+    chunks = (vecs + vecs_per_chunk - 1) / vecs_per_chunk;
+    float *lines = P ? P->lines : nullptr;
+    dim3 grid((unsigned)wgs, (unsigned)chunks);
+    if (bf) { if (kind == 0) reduce_rows_vec_kernel<true, 0><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); else reduce_rows_vec_kernel<true, 1><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); }
+    else { if (kind == 0) reduce_rows_vec_kernel<false, 0><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); else reduce_rows_vec_kernel<false, 1><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); }
+    if (P) {
+      // the partial results as an fp32 source of n_keep lines of `chunks` values: one wave per line folds them
+      ReduceParams q = p;
+      q.src = (const char *)lines;
+      q.s_keep = chunks;
+      q.s_red = 1;
+      q.n_red = (int32_t)chunks;
+      q.src_dtype = KAPY_F32;
+      reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(q);
+      const hipError_t launched = hipGetLastError(), recorded = hipEventRecord(P->free_again, s);
+      P->last_stream = s;
+      P->used = true;
+      if (launched != hipSuccess) return fail(KAPY_ERR_HIP, "reduce: %s", hipGetErrorString(launched));
+      if (recorded != hipSuccess) {
+        P->state = -1;
+        return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
+      }
+    }
   } else if (b16 && aligned && p.s_keep == 1 && p.n_keep % 8 == 0 && (p.s_red * 2) % 16 == 0 && p.n_red >= 32) {
     // strips of 256 kept indices (512-byte runs per reduced index), of 64 for narrow sources; the reduced axis in as many
     // chunks as bring the launch to about four workgroups per CU, of at least 128 reduced indices each, as far as their
@@ -321,7 +395,6 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     const int64_t strips = ((int64_t)p.n_keep + cols - 1) / cols, want = 4 * (int64_t)device_cus();
     if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
     int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 128, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
-    std::unique_lock<std::mutex> lock(partials_mutex, std::defer_lock);
     Partials *P = nullptr;
     if (chunks > 1) {
       lock.lock();

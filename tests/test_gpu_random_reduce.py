@@ -153,7 +153,39 @@ def test_reduce_along_axis0_of_tall_matrices(ko, dtype, m, n):
             assert np.isinf(w[5]) and g[5] == w[5]
             mass = np.abs(ko.decode(x.view(VALUE[dtype]), dtype)).reshape(m, n).sum(axis=0)
             rest = np.isfinite(w)
-            assert np.all(np.abs(g - w)[rest] <= (2.0 ** -22 * mass + 2.0 * EPS[ddt] * np.abs(w) + 1e-30)[rest])
+            assert np.all(np.abs(g[rest] - w[rest]) <= (2.0 ** -22 * mass + 2.0 * EPS[ddt] * np.abs(w) + 1e-30)[rest])
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(100000, 64), (30000, 200), (1000, 512), (7, 8), (4099, 24), (3, 1 << 20), (64, 65536), (5, 40000), (300, 16384)])
+def test_reduce_along_axis1_of_short_and_of_few_long_lines(ko, dtype, m, n):
+    """Lines of up to 512 elements share a wave; few long lines are shared out over workgroups in chunks whose fp32 partial
+    results a second launch folds.  max bit-exact, sum within the fp32 accumulation bound, twice with the same bits."""
+    x = ko.fill_normal(m * n, dtype, 79 + n, 0)
+    x.reshape(m, n)[m // 2, n // 3] = 0x7c00 if dtype == kh.F16 else 0x7f80
+    dx = to_dev(x)
+    for kind in (0, 1):
+        for ddt in (kh.F32, dtype):
+            db = kh.DTYPE_BYTES[ddt]
+            want = np.zeros(m, NP[db])
+            assert ko.lib().ko_reduce(C.byref(ko.mk_global(x, m, n, n, 1, dtype)), C.byref(ko.mk_global(want, m, 1, 1, 1, ddt)), 1, kind) == 0
+            runs = []
+            for _ in range(2):
+                dd = to_dev(np.full(m + 16, 0x5A5A, NP[db]))
+                kh.reduce(dglobal(dx, m, n, n, 1, dtype), dglobal(dd, m, 1, 1, 1, ddt), 1, kind)
+                sync()
+                runs.append(to_host(dd, NP[db]))
+            got = runs[0]
+            assert np.array_equal(runs[0], runs[1]) and np.all(got[m:] == 0x5A5A)
+            got = got[:m]
+            if kind == 1:
+                assert np.array_equal(got, want)
+                continue
+            g, w = ko.decode(got.view(VALUE[ddt]), ddt), ko.decode(want.view(VALUE[ddt]), ddt)
+            assert np.isinf(w[m // 2]) and g[m // 2] == w[m // 2]
+            mass = np.abs(ko.decode(x.view(VALUE[dtype]), dtype)).reshape(m, n).sum(axis=1)
+            rest = np.isfinite(w)
+            assert np.all(np.abs(g[rest] - w[rest]) <= (2.0 ** -22 * mass + 2.0 * EPS[ddt] * np.abs(w) + 1e-30)[rest])
 
 
 def test_tall_reduces_on_two_streams_share_the_partial_lines_in_turn():

@@ -199,3 +199,19 @@ def test_transpose_with_256_tiles_on_windows_of_wider_buffers(ko, rows, cols):
     win = got[:cols * dp].reshape(cols, dp)
     assert np.all(win[:, rows:] == 0x5A5A)
     assert np.array_equal(win[:, :rows], src[:, :cols].T)
+
+
+@pytest.mark.parametrize("rows,cols", [(136, 200), (3000, 5000), (264, 392), (128, 136), (1032, 128), (8200, 8184)])
+def test_transpose_whose_tiles_hang_over_the_edge_in_whole_blocks(ko, rows, cols):
+    """Extents that are multiples of 8 but not of the tile: the tiles over the edge take the block path with the blocks beyond
+    the edge left out.  Windows of wider buffers, guard words beside and behind the destination window."""
+    sp, dp = cols + 8, rows + 24
+    src = ko.fill_bits16(rows * sp, 5).reshape(rows, sp)
+    d_src, d_dst = to_dev(src), dev_zeros(cols * dp + 256, 2, fill=0x5A5A)
+    kh.copy(dglobal(d_src, rows, cols, sp, 1, kh.F16), dglobal(d_dst, cols, rows, dp, 1, kh.F16), transpose=True)
+    sync()
+    got = to_host(d_dst, np.uint16)
+    assert np.all(got[cols * dp:] == 0x5A5A)
+    win = got[:cols * dp].reshape(cols, dp)
+    assert np.all(win[:, rows:] == 0x5A5A)
+    assert np.array_equal(win[:, :rows], src[:, :cols].T)

@@ -70,12 +70,16 @@ __global__ __launch_bounds__(256) void reduce_wave_kernel(ReduceParams p) {
 // flight), the 8 values of a load combined in the lane first (the in-lane tree over loop ivs of
 // ReduceOpToLLVM.cpp:76-101), then the six butterfly rounds (:104-119).
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-template <bool BF16>
-__device__ __forceinline__ void widen8(u32x4_t v, float f[8]) {
+// SRC: what a 128-bit load holds - 0: 8 x f16, 1: 8 x bf16, 2: 4 x f32.
+template <int SRC>
+constexpr int per_vec() { return SRC == 2 ? 4 : 8; }
+template <int SRC>
+__device__ __forceinline__ void widen(u32x4_t v, float (&f)[per_vec<SRC>()]) {
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
     const uint32_t word = v[w];
-    if (BF16) {
+    if constexpr (SRC == 2) f[w] = bits_f32(word);
+    else if constexpr (SRC == 1) {
       f[2 * w] = bits_f32(word << 16);
       f[2 * w + 1] = bits_f32(word & 0xFFFF0000u);
     } else {
@@ -84,15 +88,20 @@ __device__ __forceinline__ void widen8(u32x4_t v, float f[8]) {
     }
   }
 }
-// With few long lines the reduced axis is shared out as well (blockIdx.y = chunk of vecs_per_chunk vectors): every
-// (line, chunk) leaves an fp32 partial result at partials[line * chunks + chunk], which a second launch folds per line.
-template <bool BF16, int KIND>
+// the values of one load folded as a tree
+template <int SRC>
+__device__ __forceinline__ float fold_vec(const float (&f)[per_vec<SRC>()], int kind) {
+  if constexpr (SRC == 2) return combine(combine(f[0], f[1], kind), combine(f[2], f[3], kind), kind);
+  else return combine(combine(combine(f[0], f[1], kind), combine(f[2], f[3], kind), kind), combine(combine(f[4], f[5], kind), combine(f[6], f[7], kind), kind), kind);
+}
+template <int SRC, int KIND>
 __global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p, float *partials, int32_t vecs_per_chunk) {
   const int lane = threadIdx.x & 63;
   const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (keep >= p.n_keep) return;
-  const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * 2);
-  const int32_t vecs = min(p.n_red / 8, (int32_t)(blockIdx.y + 1) * vecs_per_chunk);
+  constexpr int E = per_vec<SRC>();
+  const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * (16 / E));
+  const int32_t vecs = min(p.n_red / E, (int32_t)(blockIdx.y + 1) * vecs_per_chunk);
   float acc = KIND == 0 ? -0.f : -__builtin_inff();
   constexpr int U = 4;
   int32_t v = blockIdx.y * vecs_per_chunk + lane;
@@ -102,18 +111,17 @@ __global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p, fl
     for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(row + v + 64 * u);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      float f[8];
-      widen8<BF16>(x[u], f);
-      const float t = combine(combine(combine(f[0], f[1], KIND), combine(f[2], f[3], KIND), KIND),
-                              combine(combine(f[4], f[5], KIND), combine(f[6], f[7], KIND), KIND), KIND);
+      float f[E];
+      widen<SRC>(x[u], f);
+      const float t = fold_vec<SRC>(f, KIND);
       acc = combine(acc, t, KIND);
     }
   }
   for (; v < vecs; v += 64) {
-    float f[8];
-    widen8<BF16>(__builtin_nontemporal_load(row + v), f);
+    float f[E];
+    widen<SRC>(__builtin_nontemporal_load(row + v), f);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc = combine(acc, f[e], KIND);
+    for (int e = 0; e < E; ++e) acc = combine(acc, f[e], KIND);
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -128,15 +136,16 @@ __global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p, fl
 
 // The same for lines of up to 512 elements: a line takes GROUP lanes (8, 16, 32 or 64: the next power of two from its
 // vectors), a wave 64 / GROUP lines at a time, each lane one 128-bit load; the butterfly stays inside the group.
-template <bool BF16, int KIND, int GROUP>
+template <int SRC, int KIND, int GROUP>
 __global__ __launch_bounds__(256) void reduce_rows_short_kernel(ReduceParams p) {
   const int64_t keep = (int64_t)blockIdx.x * (256 / GROUP) + threadIdx.x / GROUP;
   const int32_t jv = threadIdx.x % GROUP;
   float acc = KIND == 0 ? -0.f : -__builtin_inff();
-  if (keep < p.n_keep && jv < p.n_red / 8) {
-    float f[8];
-    widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(p.src + keep * p.s_keep * 2) + jv), f);
-    acc = combine(combine(combine(f[0], f[1], KIND), combine(f[2], f[3], KIND), KIND), combine(combine(f[4], f[5], KIND), combine(f[6], f[7], KIND), KIND), KIND);
+  constexpr int E = per_vec<SRC>();
+  if (keep < p.n_keep && jv < p.n_red / E) {
+    float f[E];
+    widen<SRC>(__builtin_nontemporal_load((const u32x4_t *)(p.src + keep * p.s_keep * (16 / E)) + jv), f);
+    acc = fold_vec<SRC>(f, KIND);
   }
 #pragma unroll
   for (int off = GROUP / 2; off >= 1; off >>= 1) {
@@ -151,41 +160,41 @@ __global__ __launch_bounds__(256) void reduce_rows_short_kernel(ReduceParams p) 
 // loads in flight each; the groups' partial results meet in LDS.  With one chunk the strip's results go to the result;
 // with more (few kept indices, many reduced ones: a tall matrix would otherwise keep a handful of CUs busy) every chunk
 // leaves an fp32 partial line and reduce_partials_kernel folds the lines in chunk order.
-template <bool BF16, int KIND, int LPR>
+template <int SRC, int KIND, int LPR>
 __global__ __launch_bounds__(256) void reduce_cols_strip_kernel(ReduceParams p, float *partials, int32_t per_chunk) {
-  constexpr int GROUPS = 256 / LPR, COLS = LPR * 8;
+  constexpr int E = per_vec<SRC>(), EB = 16 / E, GROUPS = 256 / LPR, COLS = LPR * E;
   __shared__ float part[GROUPS][COLS + 1];
   const int cl = threadIdx.x % LPR, rg = threadIdx.x / LPR;
-  const int64_t keep0 = (int64_t)blockIdx.x * COLS + cl * 8;
+  const int64_t keep0 = (int64_t)blockIdx.x * COLS + cl * E;
   const int32_t r_begin = blockIdx.y * per_chunk, r_end = min(p.n_red, r_begin + per_chunk);
-  float acc[8];
+  float acc[E];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = KIND == 0 ? -0.f : -__builtin_inff();
-  if (keep0 < p.n_keep) {  // (whole vectors: n_keep is a multiple of 8)
-    const char *col = p.src + keep0 * 2;
+  for (int e = 0; e < E; ++e) acc[e] = KIND == 0 ? -0.f : -__builtin_inff();
+  if (keep0 < p.n_keep) {  // (whole vectors: n_keep is a multiple of E)
+    const char *col = p.src + keep0 * EB;
     constexpr int U = 4;
     int32_t r = r_begin + rg;
     for (; r + GROUPS * (U - 1) < r_end; r += GROUPS * U) {
       u32x4_t x[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)(r + GROUPS * u) * p.s_red * 2));
+      for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)(r + GROUPS * u) * p.s_red * EB));
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        float f[8];
-        widen8<BF16>(x[u], f);
+        float f[E];
+        widen<SRC>(x[u], f);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = combine(acc[e], f[e], KIND);
+        for (int e = 0; e < E; ++e) acc[e] = combine(acc[e], f[e], KIND);
       }
     }
     for (; r < r_end; r += GROUPS) {
-      float f[8];
-      widen8<BF16>(__builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)r * p.s_red * 2)), f);
+      float f[E];
+      widen<SRC>(__builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)r * p.s_red * EB)), f);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = combine(acc[e], f[e], KIND);
+      for (int e = 0; e < E; ++e) acc[e] = combine(acc[e], f[e], KIND);
     }
   }
 #pragma unroll
-  for (int e = 0; e < 8; ++e) part[rg][cl * 8 + e] = acc[e];
+  for (int e = 0; e < E; ++e) part[rg][cl * E + e] = acc[e];
   __syncthreads();
   const int64_t keep = (int64_t)blockIdx.x * COLS + threadIdx.x;
   if (threadIdx.x < COLS && keep < p.n_keep) {
@@ -303,6 +312,14 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
   return KAPY_OK;
 }
 
+// LAUNCH(source kind, reduce kind) for the call's source type and reduce kind
+#define KAPY_BY_SOURCE(LAUNCH)                                                                  \
+  do {                                                                                          \
+    if (src_kind == 0) { if (kind == 0) LAUNCH(0, 0); else LAUNCH(0, 1); }                      \
+    else if (src_kind == 1) { if (kind == 0) LAUNCH(1, 0); else LAUNCH(1, 1); }                 \
+    else { if (kind == 0) LAUNCH(2, 0); else LAUNCH(2, 1); }                                    \
+  } while (0)
+
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream) {
   int rc = check_global(src, "reduce source");
   if (!rc) rc = check_global(dst, "reduce result");
@@ -331,29 +348,30 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
   p.kind = kind;
   if (p.n_keep == 0) return KAPY_OK;
   hipStream_t s = (hipStream_t)stream;
-  const bool b16 = src->dtype == KAPY_F16 || src->dtype == KAPY_BF16, bf = src->dtype == KAPY_BF16;
+  // the vector kernels: f16, bf16 or f32 source read in 128-bit pieces of E elements
+  const bool vec_ok = src->dtype == KAPY_F16 || src->dtype == KAPY_BF16 || src->dtype == KAPY_F32;
+  const int src_kind = src->dtype == KAPY_F32 ? 2 : src->dtype == KAPY_BF16 ? 1 : 0, E = src_kind == 2 ? 4 : 8, EB = 16 / E;
   const bool aligned = ((uintptr_t)p.src & 15) == 0;
   std::unique_lock<std::mutex> lock(partials_mutex, std::defer_lock);
-  if (b16 && aligned && p.s_red == 1 && p.n_red % 8 == 0 && (p.s_keep * 2) % 16 == 0 && p.n_red <= 512 && p.n_red >= 8) {
-    const int vecs = p.n_red / 8, group = vecs <= 8 ? 8 : vecs <= 16 ? 16 : vecs <= 32 ? 32 : 64;
+  if (vec_ok && aligned && p.s_red == 1 && p.n_red % E == 0 && (p.s_keep * EB) % 16 == 0 && p.n_red <= 64 * E && p.n_red >= E) {
+    const int vecs = p.n_red / E, group = vecs <= 8 ? 8 : vecs <= 16 ? 16 : vecs <= 32 ? 32 : 64;
     const int64_t wgs = ((int64_t)p.n_keep + 256 / group - 1) / (256 / group);
     if (wgs > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 workgroups");
     dim3 grid((unsigned)wgs);
-#define KAPY_SHORT(BF_, KIND_)                                                                       \
+#define KAPY_SHORT(SRC_, KIND_)                                                                      \
   do {                                                                                               \
-    if (group == 8) reduce_rows_short_kernel<BF_, KIND_, 8><<<grid, 256, 0, s>>>(p);                 \
-    else if (group == 16) reduce_rows_short_kernel<BF_, KIND_, 16><<<grid, 256, 0, s>>>(p);          \
-    else if (group == 32) reduce_rows_short_kernel<BF_, KIND_, 32><<<grid, 256, 0, s>>>(p);          \
-    else reduce_rows_short_kernel<BF_, KIND_, 64><<<grid, 256, 0, s>>>(p);                           \
+    if (group == 8) reduce_rows_short_kernel<SRC_, KIND_, 8><<<grid, 256, 0, s>>>(p);                \
+    else if (group == 16) reduce_rows_short_kernel<SRC_, KIND_, 16><<<grid, 256, 0, s>>>(p);         \
+    else if (group == 32) reduce_rows_short_kernel<SRC_, KIND_, 32><<<grid, 256, 0, s>>>(p);         \
+    else reduce_rows_short_kernel<SRC_, KIND_, 64><<<grid, 256, 0, s>>>(p);                          \
   } while (0)
-    if (bf) { if (kind == 0) KAPY_SHORT(true, 0); else KAPY_SHORT(true, 1); }
-    else { if (kind == 0) KAPY_SHORT(false, 0); else KAPY_SHORT(false, 1); }
+    KAPY_BY_SOURCE(KAPY_SHORT);
 #undef KAPY_SHORT
-  } else if (b16 && aligned && p.s_red == 1 && p.n_red % 8 == 0 && (p.s_keep * 2) % 16 == 0 && p.n_red > 512) {
+  } else if (vec_ok && aligned && p.s_red == 1 && p.n_red % E == 0 && (p.s_keep * EB) % 16 == 0 && p.n_red > 64 * E) {
     // four lines per workgroup; with fewer workgroups than CUs, chunks of at least 256 vectors of the reduced axis as well,
     // up to four workgroups per CU (their partial results within the block): 64 lines of 1 Mi elements 312 -> 33 us, 256
     // lines of 256 Ki 82 -> 30 us.  The second launch costs about 6 us: 1024 lines of 64 Ki elements are faster whole.
-    const int64_t wgs = ((int64_t)p.n_keep + 3) / 4, want = 4 * (int64_t)device_cus(), vecs = p.n_red / 8;
+    const int64_t wgs = ((int64_t)p.n_keep + 3) / 4, want = 4 * (int64_t)device_cus(), vecs = p.n_red / E;
     int64_t chunks = wgs >= device_cus() ? 1 : std::max<int64_t>(1, std::min<int64_t>({(want + wgs - 1) / wgs, vecs / 256, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
     Partials *P = nullptr;
     if (chunks > 1) {
@@ -366,8 +384,9 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     chunks = (vecs + vecs_per_chunk - 1) / vecs_per_chunk;
     float *lines = P ? P->lines : nullptr;
     dim3 grid((unsigned)wgs, (unsigned)chunks);
-    if (bf) { if (kind == 0) reduce_rows_vec_kernel<true, 0><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); else reduce_rows_vec_kernel<true, 1><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); }
-    else { if (kind == 0) reduce_rows_vec_kernel<false, 0><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); else reduce_rows_vec_kernel<false, 1><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk); }
+#define KAPY_ROWS(SRC_, KIND_) reduce_rows_vec_kernel<SRC_, KIND_><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk)
+    KAPY_BY_SOURCE(KAPY_ROWS);
+#undef KAPY_ROWS
     if (P) {
       // the partial results as an fp32 source of n_keep lines of `chunks` values: one wave per line folds them
       ReduceParams q = p;
@@ -386,12 +405,12 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
         return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
       }
     }
-  } else if (b16 && aligned && p.s_keep == 1 && p.n_keep % 8 == 0 && (p.s_red * 2) % 16 == 0 && p.n_red >= 32) {
+  } else if (vec_ok && aligned && p.s_keep == 1 && p.n_keep % E == 0 && (p.s_red * EB) % 16 == 0 && p.n_red >= 32) {
     // strips of 256 kept indices (512-byte runs per reduced index), of 64 for narrow sources; the reduced axis in as many
     // chunks as bring the launch to about four workgroups per CU, of at least 128 reduced indices each, as far as their
     // partial lines fit the block.  Measured for 128 MiB of fp16: 8192 x 8192 46 -> 29 us (64-wide strips: 31, eight
     // workgroups per CU: 31, eight loads in flight per lane: 30), 1 Mi x 64 4335 -> 34 us.
-    const int lpr = p.n_keep >= 256 ? 32 : 8, cols = lpr * 8;
+    const int lpr = p.n_keep >= 32 * E ? 32 : 8, cols = lpr * E;
     const int64_t strips = ((int64_t)p.n_keep + cols - 1) / cols, want = 4 * (int64_t)device_cus();
     if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
     int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 128, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
@@ -406,13 +425,12 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     chunks = (p.n_red + per_chunk - 1) / per_chunk;
     float *lines = P ? P->lines : nullptr;
     dim3 grid((unsigned)strips, (unsigned)chunks);
-#define KAPY_STRIP(BF_, KIND_)                                                                                                        \
+#define KAPY_STRIP(SRC_, KIND_)                                                                                                       \
   do {                                                                                                                                \
-    if (lpr == 32) reduce_cols_strip_kernel<BF_, KIND_, 32><<<grid, 256, 0, s>>>(p, lines, per_chunk);                                \
-    else reduce_cols_strip_kernel<BF_, KIND_, 8><<<grid, 256, 0, s>>>(p, lines, per_chunk);                                           \
+    if (lpr == 32) reduce_cols_strip_kernel<SRC_, KIND_, 32><<<grid, 256, 0, s>>>(p, lines, per_chunk);                               \
+    else reduce_cols_strip_kernel<SRC_, KIND_, 8><<<grid, 256, 0, s>>>(p, lines, per_chunk);                                          \
   } while (0)
-    if (bf) { if (kind == 0) KAPY_STRIP(true, 0); else KAPY_STRIP(true, 1); }
-    else { if (kind == 0) KAPY_STRIP(false, 0); else KAPY_STRIP(false, 1); }
+    KAPY_BY_SOURCE(KAPY_STRIP);
 #undef KAPY_STRIP
     if (P) {
       if (kind == 0) reduce_partials_kernel<0><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
@@ -432,5 +450,6 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }
+#undef KAPY_BY_SOURCE
 
 }  // extern "C"

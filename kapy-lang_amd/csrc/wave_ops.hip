@@ -56,7 +56,15 @@ __global__ __launch_bounds__(256) void reduce_wave_kernel(ReduceParams p) {
   const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (keep >= p.n_keep) return;
   float acc = p.kind == 0 ? -0.f : -__builtin_inff();
-  for (int32_t r = lane; r < p.n_red; r += 64) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + r * p.s_red), p.kind);
+  int32_t r = lane;
+  for (; r + 192 < p.n_red; r += 256) {  // four loads in flight
+    float f[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) f[u] = load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)(r + 64 * u) * p.s_red);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc = combine(acc, f[u], p.kind);
+  }
+  for (; r < p.n_red; r += 64) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)r * p.s_red), p.kind);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
     float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(acc)));
@@ -268,13 +276,59 @@ Partials *partials_for(hipStream_t s) {
   return &P;
 }
 
-// One lane per kept index: used when the kept axis is the contiguous one (coalesced as is).
-__global__ __launch_bounds__(256) void reduce_lane_kernel(ReduceParams p) {
-  const int64_t keep = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (keep >= p.n_keep) return;
+// The block for a call that wants `chunks` > 1 partial lines, with `lock` taken - or nullptr, chunks = 1 and no lock.
+Partials *take_partials(int64_t &chunks, std::unique_lock<std::mutex> &lock, hipStream_t s) {
+  Partials *P = nullptr;
+  if (chunks > 1) {
+    lock.lock();
+    P = partials_for(s);
+    if (!P) lock.unlock();
+  }
+  if (!P) chunks = 1;
+  return P;
+}
+
+// After the call's launches (lock still held): whatever was launched reads or writes the block, so the next user waits for
+// all of it.
+int partials_used(Partials *P, hipStream_t s) {
+  const hipError_t launched = hipGetLastError(), recorded = hipEventRecord(P->free_again, s);
+  P->last_stream = s;
+  P->used = true;
+  if (launched != hipSuccess) return fail(KAPY_ERR_HIP, "reduce: %s", hipGetErrorString(launched));
+  if (recorded != hipSuccess) {
+    P->state = -1;  // nobody could wait for this call's use of the block: it is not handed out again
+    return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
+  }
+  return KAPY_OK;
+}
+
+// Any element type, alignment and extents, kept axis contiguous (or at least not the strided one): a workgroup owns 64 kept
+// indices, one per lane of a wave (a wave's loads cover 64 consecutive elements of one reduced index), its four waves share
+// out a chunk of the reduced axis with four loads in flight each and meet in LDS; chunks as in reduce_cols_strip_kernel.
+__global__ __launch_bounds__(256) void reduce_cols_any_kernel(ReduceParams p, float *partials, int32_t per_chunk) {
+  __shared__ float part[4][64];
+  const int cl = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int64_t keep = (int64_t)blockIdx.x * 64 + cl;
+  const int32_t r_begin = blockIdx.y * per_chunk, r_end = min(p.n_red, r_begin + per_chunk);
   float acc = p.kind == 0 ? -0.f : -__builtin_inff();
-  for (int32_t r = 0; r < p.n_red; ++r) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + r * p.s_red), p.kind);
-  store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
+  if (keep < p.n_keep) {
+    int32_t r = r_begin + rg;
+    for (; r + 12 < r_end; r += 16) {
+      float f[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) f[u] = load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)(r + 4 * u) * p.s_red);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc = combine(acc, f[u], p.kind);
+    }
+    for (; r < r_end; r += 4) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)r * p.s_red), p.kind);
+  }
+  part[rg][cl] = acc;
+  __syncthreads();
+  if (rg == 0 && keep < p.n_keep) {
+    float t = combine(combine(part[0][cl], part[1][cl], p.kind), combine(part[2][cl], part[3][cl], p.kind), p.kind);
+    if (partials) partials[(int64_t)blockIdx.y * p.n_keep + keep] = t;
+    else store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
+  }
 }
 
 Fragments to_internal(const kapy_fragments *f) {
@@ -373,13 +427,7 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     // lines of 256 Ki 82 -> 30 us.  The second launch costs about 6 us: 1024 lines of 64 Ki elements are faster whole.
     const int64_t wgs = ((int64_t)p.n_keep + 3) / 4, want = 4 * (int64_t)device_cus(), vecs = p.n_red / E;
     int64_t chunks = wgs >= device_cus() ? 1 : std::max<int64_t>(1, std::min<int64_t>({(want + wgs - 1) / wgs, vecs / 256, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
-    Partials *P = nullptr;
-    if (chunks > 1) {
-      lock.lock();
-      P = partials_for(s);
-      if (!P) lock.unlock();
-    }
-    if (!P) chunks = 1;
+    Partials *P = take_partials(chunks, lock, s);
     const int32_t vecs_per_chunk = (int32_t)((vecs + chunks - 1) / chunks);
     chunks = (vecs + vecs_per_chunk - 1) / vecs_per_chunk;
     float *lines = P ? P->lines : nullptr;
@@ -396,14 +444,7 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
       q.n_red = (int32_t)chunks;
       q.src_dtype = KAPY_F32;
       reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(q);
-      const hipError_t launched = hipGetLastError(), recorded = hipEventRecord(P->free_again, s);
-      P->last_stream = s;
-      P->used = true;
-      if (launched != hipSuccess) return fail(KAPY_ERR_HIP, "reduce: %s", hipGetErrorString(launched));
-      if (recorded != hipSuccess) {
-        P->state = -1;
-        return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
-      }
+      return partials_used(P, s);
     }
   } else if (vec_ok && aligned && p.s_keep == 1 && p.n_keep % E == 0 && (p.s_red * EB) % 16 == 0 && p.n_red >= 32) {
     // strips of 256 kept indices (512-byte runs per reduced index), of 64 for narrow sources; the reduced axis in as many
@@ -414,13 +455,7 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     const int64_t strips = ((int64_t)p.n_keep + cols - 1) / cols, want = 4 * (int64_t)device_cus();
     if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
     int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 128, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
-    Partials *P = nullptr;
-    if (chunks > 1) {
-      lock.lock();
-      P = partials_for(s);
-      if (!P) lock.unlock();
-    }
-    if (!P) chunks = 1;
+    Partials *P = take_partials(chunks, lock, s);
     const int32_t per_chunk = (int32_t)((p.n_red + chunks - 1) / chunks);
     chunks = (p.n_red + per_chunk - 1) / per_chunk;
     float *lines = P ? P->lines : nullptr;
@@ -435,17 +470,23 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
     if (P) {
       if (kind == 0) reduce_partials_kernel<0><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
       else reduce_partials_kernel<1><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
-      // whatever was launched reads or writes the block: the next user waits for all of it
-      const hipError_t launched = hipGetLastError(), recorded = hipEventRecord(P->free_again, s);
-      P->last_stream = s;
-      P->used = true;
-      if (launched != hipSuccess) return fail(KAPY_ERR_HIP, "reduce: %s", hipGetErrorString(launched));
-      if (recorded != hipSuccess) {
-        P->state = -1;  // nobody could wait for this call's use of the block: it is not handed out again
-        return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
-      }
+      return partials_used(P, s);
     }
-  } else if (p.s_keep == 1 && p.s_red != 1) reduce_lane_kernel<<<(p.n_keep + 255) / 256, 256, 0, s>>>(p);
+  } else if (p.s_keep == 1 && p.s_red != 1) {
+    const int64_t strips = ((int64_t)p.n_keep + 63) / 64, want = 4 * (int64_t)device_cus();
+    if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 64, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
+    Partials *P = take_partials(chunks, lock, s);
+    const int32_t per_chunk = (int32_t)((p.n_red + chunks - 1) / chunks);
+    chunks = (p.n_red + per_chunk - 1) / per_chunk;
+    float *lines = P ? P->lines : nullptr;
+    reduce_cols_any_kernel<<<dim3((unsigned)strips, (unsigned)chunks), 256, 0, s>>>(p, lines, per_chunk);
+    if (P) {
+      if (kind == 0) reduce_partials_kernel<0><<<dim3((unsigned)strips), 1024, 0, s>>>(p, lines, (int32_t)chunks);
+      else reduce_partials_kernel<1><<<dim3((unsigned)strips), 1024, 0, s>>>(p, lines, (int32_t)chunks);
+      return partials_used(P, s);
+    }
+  }
   else reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;

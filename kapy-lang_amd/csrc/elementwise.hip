@@ -855,6 +855,7 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
                      const kapy_global *out, void *stream) {
   int result_dtype[kMaxInst];
   kapy_ew_inst normalised[kMaxInst];
+  const kapy_ew_inst *as_given = prog;
   int rc = verify_program(prog, n_inst, ins, n_ins, out, result_dtype, normalised);
   if (rc) return rc;
   prog = normalised;
@@ -870,6 +871,45 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 
   bool has_reduce = false;
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
+
+  // Rows that are not a whole number of 8-element vectors move element by element (or, 16-bit only, with a ragged last
+  // vector per row, and then only from aligned rows).  When the result and every operand are dense matrices of one shape
+  // (pitch = width) or single elements, the program does not care where a row ends: it runs once over the first
+  // 8 * floor(o0 * o1 / 8) elements as one line, in whole vectors, and once over the up to 7 that remain.
+  if (!has_reduce && o0 > 1 && o1 % 8 != 0 && o0 * o1 < (int64_t(1) << 31) - 1024 && n_ins <= kMaxInputs) {
+    auto dense = [&](const kapy_global *g) { return g->stride1 == 1 && g->stride0 == o1 && extent0(g) == o0 && extent1(g) == o1; };
+    auto single = [](const kapy_global *g) { return extent0(g) == 1 && extent1(g) == 1; };
+    bool flat = dense(out);
+    for (int k = 0; k < n_ins; ++k) flat = flat && (dense(ins[k]) || single(ins[k]));
+    if (flat) {
+      const int64_t total = o0 * o1, whole = total / 8 * 8;
+      auto line = [&](const kapy_global *g, int64_t first, int64_t count) {
+        if (single(g)) return *g;
+        kapy_global v = *g;
+        v.ptr = (void *)(view_base(g) + first * dtype_bytes(g->dtype));
+        v.start0 = v.start1 = 0;
+        v.end0 = 1;
+        v.end1 = v.stride0 = (int32_t)count;
+        v.stride1 = 1;
+        v.alignment = 16;
+        while (v.alignment > 1 && ((uintptr_t)v.ptr & (uintptr_t)(v.alignment - 1))) v.alignment >>= 1;
+        return v;
+      };
+      for (int part = 0; part < 2; ++part) {
+        const int64_t first = part ? whole : 0, count = part ? total - whole : whole;
+        if (count == 0) continue;
+        kapy_global views[kMaxInputs], result = line(out, first, count);
+        const kapy_global *ptrs[kMaxInputs];
+        for (int k = 0; k < n_ins; ++k) {
+          views[k] = line(ins[k], first, count);
+          ptrs[k] = &views[k];
+        }
+        rc = kapy_elementwise(as_given, n_inst, ptrs, n_ins, &result, stream);
+        if (rc) return rc;
+      }
+      return KAPY_OK;
+    }
+  }
   if (has_reduce) {
     int along[2] = {0, 0};
     for (int k = 0; k < n_inst; ++k)

@@ -215,3 +215,17 @@ def test_transpose_whose_tiles_hang_over_the_edge_in_whole_blocks(ko, rows, cols
     win = got[:cols * dp].reshape(cols, dp)
     assert np.all(win[:, rows:] == 0x5A5A)
     assert np.array_equal(win[:, :rows], src[:, :cols].T)
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.F32, kh.F8E4M3])
+@pytest.mark.parametrize("rows,cols", [(301, 501), (17, 3), (3001, 5001), (2, 7)])
+def test_dense_copy_with_odd_widths_moves_as_one_line(ko, dtype, rows, cols):
+    """Two dense matrices of one shape are one line of rows * cols elements, whatever the width; guard words intact."""
+    eb = kh.DTYPE_BYTES[dtype]
+    np_t = {1: np.uint8, 2: np.uint16, 4: np.uint32}[eb]
+    src = np.random.RandomState(rows * 7 + cols).randint(0, 2 ** (8 * eb - 1), size=rows * cols).astype(np_t)
+    d_src, d_dst = to_dev(src), dev_zeros(rows * cols + 64, eb, fill=0x5A)
+    kh.copy(dglobal(d_src, rows, cols, cols, 1, dtype), dglobal(d_dst, rows, cols, cols, 1, dtype))
+    sync()
+    got = to_host(d_dst, np_t)
+    assert np.array_equal(got[:rows * cols], src) and np.all(got[rows * cols:] == got[-1]) and got[-1] != 0

@@ -585,3 +585,27 @@ def test_division_keeps_the_sign_of_a_zero_dividend(ko):
     sync()
     out = to_host(dz, np.float32, (m, n))
     assert np.array_equal(out, x / y) and np.array_equal(np.signbit(out), np.signbit(x / y))
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16, kh.F32])
+@pytest.mark.parametrize("m,n", [(301, 501), (17, 3), (2, 7), (64, 1001), (1000, 9)])
+def test_dense_operands_with_odd_widths_run_as_one_line(ko, dtype, m, n):
+    """Dense matrices of one shape whose rows are not whole vectors: the program runs over all elements as one line (and once
+    more over the last few); a scalar operand rides along.  Bit-exact (one rounding per op), guard words intact."""
+    eb = kh.DTYPE_BYTES[dtype]
+    a, b = ko.fill_normal(m * n, dtype, 91, 0), ko.fill_normal(m * n, dtype, 91, 1)
+    c = ko.fill_normal(1, dtype, 92, 0)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1), dict(op=kh.EW_LD_GLOBAL, dst=2, a=2),
+             dict(op=kh.EW_MULF, dst=3, a=0, b=1), dict(op=kh.EW_ADDF, dst=3, a=3, b=2), dict(op=kh.EW_MAXIMUMF, dst=3, a=3, b=1),
+             dict(op=kh.EW_ST_GLOBAL, a=3)]
+    np_t = {2: np.uint16, 4: np.uint32}[eb]
+    want = np.zeros(m * n, np_t)
+    gos = [ko.mk_global(a, m, n, n, 1, dtype), ko.mk_global(b, m, n, n, 1, dtype), ko.mk_global(c, 1, 1, 1, 1, dtype)]
+    assert ko.elementwise(ko.program(insts), gos, ko.mk_global(want, m, n, n, 1, dtype)) == 0
+    da, db_, dc = to_dev(a), to_dev(b), to_dev(c)
+    dout = dev_zeros(m * n + 32, eb, fill=0x5A5A)
+    kh.elementwise(kh.program(insts), [dglobal(da, m, n, n, 1, dtype), dglobal(db_, m, n, n, 1, dtype), dglobal(dc, 1, 1, 1, 1, dtype)],
+                   dglobal(dout, m, n, n, 1, dtype))
+    sync()
+    got = to_host(dout, np_t)
+    assert np.array_equal(got[:m * n], want.view(np_t)) and np.all(got[m * n:] == got[-1]) and got[-1] != 0

@@ -1236,7 +1236,12 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   const int64_t a_left = A_TR ? 0x7fffffff : ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2;
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * (A_TR ? 1 : p.a_sm) * 2), 0,
                                                                           __builtin_amdgcn_readfirstlane((int)(a_left < 0x7fffffff ? a_left : 0x7fffffff)), 0x00020000);
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * (B_TR ? 1 : p.b_sn) * 2), 0, 0x7fffffff, 0x00020000);
+  // The rhs descriptor ends where the rhs ends, too: of a tile that hangs over the last columns (N not a multiple of 128) the
+  // columns that do not exist read zeros or, in a transposed rhs, the first elements of the next k-row; either way they only
+  // reach results that are not stored.
+  const int64_t b_left = B_TR ? ((int64_t)(p.K - 1) * p.b_sk + (p.N - n0)) * 2 : ((int64_t)(p.N - n0 - 1) * p.b_sn + p.K) * 2;
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * (B_TR ? 1 : p.b_sn) * 2), 0,
+                                                                          __builtin_amdgcn_readfirstlane((int)(b_left < 0x7fffffff ? b_left : 0x7fffffff)), 0x00020000);
   const int wave_lds = wave * 1024;
   // (the scalar offsets of K-tile j, clamped to the last tile: loads past the end of K are still issued, into stages nobody reads)
   auto soff_a_of = [&](int j) { return min(j, KT - 1) * BK * (A_TR ? a_ld : 1) * 2; };
@@ -1599,7 +1604,7 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
 template <typename T, int BK, int STAGES, bool A_TR = false, bool B_TR = true>
 int launch_nn(GemmParams p, hipStream_t s) {
   p.tiles_m = (p.M + kNBM - 1) / kNBM;  // (a K-contiguous lhs need not have whole tiles of rows: see the kernel's lhs descriptor)
-  p.tiles_n = p.N / kNBN;
+  p.tiles_n = (p.N + kNBN - 1) / kNBN;  // (nor whole tiles of columns: see its rhs descriptor)
   const bool packed = packed_epilogue(p) && !host_has_tail(p);  // (a fused tail goes through the element stores here)
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k);
   if (packed) nn_kernel<T, BK, STAGES, true, A_TR, B_TR><<<grid, dim3(256), 0, s>>>(p);
@@ -1877,7 +1882,7 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
   const bool a_tr = !a_kc && p.a_sm == 1 && vector_bytes(lhs, 0) == 16 && p.a_sk >= 0 && p.M % kNBM == 0 && (int64_t)p.K * p.a_sk * 2 < (int64_t(1) << 31);
   const bool b_tr = p.b_sn == 1 && vector_bytes(rhs, 1) == 16 && p.b_sk >= 0 && (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31);
   const bool b_kc = !b_tr && p.b_sk == 1 && vector_bytes(rhs, 0) == 16 && p.b_sn >= 0 && p.b_sn * 2 * kNBN < (int64_t(1) << 31);
-  bool nn = (a_kc || a_tr) && (b_kc || b_tr) && (a_tr || b_tr) && p.M > 0 && p.N % kNBN == 0 && p.K > 0 &&
+  bool nn = (a_kc || a_tr) && (b_kc || b_tr) && (a_tr || b_tr) && p.M > 0 && p.N % 8 == 0 && p.K > 0 &&
             c.impl_way != KAPY_MFMA_32X32X16_16B && (!c.tile_m || c.tile_m == kNBM) && (!c.tile_n || c.tile_n == kNBN) && (!c.waves || c.waves == 4);
   if (nn) {
     struct NnVariant {

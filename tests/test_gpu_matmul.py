@@ -278,3 +278,22 @@ def test_transposing_read_kernel_takes_either_operand_transposed(ko, dt, a_rm, b
     for (M, N, K) in ((256, 384, 64 * 9), (128, 128, 64 * 4), (384, 256, 64 * 5)):
         got, want = _run(ko, dt, M, N, K, a_rm, b_rm, seed=21, tile=(128, 128, tile_k), stages=stages)
         assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
+
+
+@pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("a_rm,b_rm", [(True, True), (False, True), (False, False)])
+def test_transposing_read_kernel_with_columns_that_do_not_fill_the_last_tile(ko, dt, a_rm, b_rm):
+    """N a multiple of 8 but not of the 128-wide tile: the rhs descriptor ends with the rhs, the columns beyond it reach no
+    stored result.  Against the oracle, with guard words behind the result; M ragged too where the lhs is row-major."""
+    for (M, N, K, tile_k) in ((256 if not a_rm else 200, 136, 64 * 5, 64), (128, 1000, 32 * 7, 32), (384 if not a_rm else 333, 8, 64 * 4, 64)):
+        a, b = ko.fill_uniform(M * K, dt, 23, 0), ko.fill_uniform(K * N, dt, 23, 1)
+        a_str, b_str = ((K, 1) if a_rm else (1, M)), ((N, 1) if b_rm else (1, K))
+        want = np.zeros(M * N, dtype=np.uint16)
+        assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, *a_str, dt)), C.byref(ko.mk_global(b, K, N, *b_str, dt)), None,
+                                  C.byref(ko.mk_global(want, M, N, N, 1, dt)), kh.RN) == 0
+        da, db, dd = to_dev(a), to_dev(b), dev_zeros(M * N + 256, 2, fill=0x1234)
+        kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(dd, M, N, N, 1, dt), tile=(128, 128, tile_k))
+        sync()
+        got = to_host(dd, np.uint16)
+        assert np.all(got[M * N:] == 0x1234), (M, N, K)
+        assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL, (M, N, K)

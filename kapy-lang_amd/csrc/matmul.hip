@@ -1184,7 +1184,10 @@ __device__ __forceinline__ uint32_t rhs_key(uint32_t row) { return ((row & 3) + 
 // of BK elements staged under the tiled kernel's swizzle and read 16 bytes per lane.  true: contiguous along its other
 // extent (a column-major lhs, a row-major rhs): k-rows of 128 elements staged as they lie and read with the transposing
 // read.  <false, true> is the reference fixture's row-major x row-major; <false, false> is the tiled kernel's business.
-template <typename T, int BK, int STAGES, bool PACKED, bool A_TR = false, bool B_TR = true>
+// KTAIL: K is a multiple of 8 but not of BK.  The loads of the last K-tile are then issued with the per-lane offsets of the
+// 16-byte pieces (K-contiguous operand) or k-rows (transposed operand) beyond K moved out of the descriptor's range, so that
+// zeros arrive in their place; the switch is made once, beside a barrier, when the last tile's loads come up.
+template <typename T, int BK, int STAGES, bool PACKED, bool A_TR = false, bool B_TR = true, bool KTAIL = false>
 __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   static_assert(T::kM == 16 && T::kBytes == 2 && BK % 32 == 0 && STAGES >= 3, "16x16x32 instruction, 16-bit operands");
   static_assert(A_TR || B_TR, "two K-contiguous operands are the tiled kernel's");
@@ -1202,7 +1205,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   tile_of_block(p, tm, tn);
   const int32_t m0 = tm * kNBM, n0 = tn * kNBN;
   const int32_t split = enter_split(p, 2);
-  const int KT = p.K / BK;
+  const int KT = KTAIL ? (p.K + BK - 1) / BK : p.K / BK;
   // elements between neighbours along the staged rows' other extent: between rows (K-contiguous) or between k-rows (transposed)
   const int32_t a_ld = (int32_t)(A_TR ? p.a_sk : p.a_sm), b_ld = (int32_t)(B_TR ? p.b_sk : p.b_sn);
 
@@ -1225,15 +1228,32 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     a_goff[q] = goff_of(A_TR, q, a_ld);
     b_goff[q] = goff_of(B_TR, q, b_ld);
   }
+  // (KTAIL) first K position, within a tile, of the piece that load instruction q of an operand brings this lane
+  auto k_of = [&](bool tr, int q) -> int32_t {
+    const uint32_t o = (uint32_t)(wave + q * 4) * 1024u + lane * 16u;
+    uint32_t row, chunk;
+    if (tr) return (int32_t)(o / kRowTr);
+    LA::locate(o, row, chunk);
+    return (int32_t)chunk * 8;
+  };
+  // From the last K-tile on (the loads past the end of K repeat it): pieces at or beyond K get an offset no descriptor covers.
+  auto enter_k_tail = [&]() {
+    const int32_t k_left = p.K - (KT - 1) * BK;
+#pragma unroll
+    for (int q = 0; q < kLoadsOp; ++q) {
+      a_goff[q] = k_of(A_TR, q) >= k_left ? 0x7fffffffu : a_goff[q];
+      b_goff[q] = k_of(B_TR, q) >= k_left ? 0x7fffffffu : b_goff[q];
+    }
+  };
   auto uniform_ptr = [](const char *ptr) {
     const uint64_t v = (uint64_t)ptr;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (void *)(((uint64_t)hi << 32) | lo);
   };
-  // A K-contiguous lhs descriptor ends where the lhs ends: a tile that hangs over its last rows (M not a multiple of 128) gets
-  // zeros for the rows that do not exist (their per-lane offsets are out of range) instead of a fault.  (In the other forms
-  // the host asks for whole tiles.)
-  const int64_t a_left = A_TR ? 0x7fffffff : ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2;
+  // The lhs descriptor ends where the lhs ends: a tile of a K-contiguous lhs that hangs over its last rows (M not a multiple of
+  // 128) gets zeros for the rows that do not exist (their per-lane offsets are out of range) instead of a fault.  (For a
+  // transposed lhs the host asks for whole tiles of rows; its descriptor is bounded all the same.)
+  const int64_t a_left = A_TR ? ((int64_t)(p.K - 1) * p.a_sk + (p.M - m0)) * 2 : ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2;
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * (A_TR ? 1 : p.a_sm) * 2), 0,
                                                                           __builtin_amdgcn_readfirstlane((int)(a_left < 0x7fffffff ? a_left : 0x7fffffff)), 0x00020000);
   // The rhs descriptor ends where the rhs ends, too: of a tile that hangs over the last columns (N not a multiple of 128) the
@@ -1328,9 +1348,11 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     for (int j = 0; j < kTn; ++j) acc[i][j] = Acc{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
-  for (int j = 0; j < STAGES - 1; ++j)
+  for (int j = 0; j < STAGES - 1; ++j) {
+    if (KTAIL && j == KT - 1) enter_k_tail();
 #pragma unroll
     for (int idx = 0; idx < kLoads; ++idx) issue_load(j, j, idx);
+  }
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(kLoads * (STAGES - 2)));
   __builtin_amdgcn_s_barrier();  // tile 0 published
   Frags af[2], bf[2];
@@ -1351,6 +1373,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     // (the scalar offsets of this step's loads are formed here, beside the barrier, not in the gaps of the loads)
     int soff_a = __builtin_amdgcn_readfirstlane(soff_a_of(kt + STAGES - 1)), soff_b = __builtin_amdgcn_readfirstlane(soff_b_of(kt + STAGES - 1));
     asm volatile("" : "+s"(soff_a), "+s"(soff_b));
+    if (KTAIL && kt + STAGES - 1 == KT - 1) enter_k_tail();
     // own loads of tile kt+1 have landed once only the younger tiles' loads remain in flight
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kLoads * (STAGES - 3)));
     __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
@@ -1601,14 +1624,14 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
   return packed ? launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, true>(p, s) : launch_tn_epi<T, BM, BN, BK, WM, WN, STAGES, false>(p, s);
 }
 
-template <typename T, int BK, int STAGES, bool A_TR = false, bool B_TR = true>
+template <typename T, int BK, int STAGES, bool A_TR = false, bool B_TR = true, bool KTAIL = false>
 int launch_nn(GemmParams p, hipStream_t s) {
   p.tiles_m = (p.M + kNBM - 1) / kNBM;  // (a K-contiguous lhs need not have whole tiles of rows: see the kernel's lhs descriptor)
   p.tiles_n = (p.N + kNBN - 1) / kNBN;  // (nor whole tiles of columns: see its rhs descriptor)
   const bool packed = packed_epilogue(p) && !host_has_tail(p);  // (a fused tail goes through the element stores here)
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k);
-  if (packed) nn_kernel<T, BK, STAGES, true, A_TR, B_TR><<<grid, dim3(256), 0, s>>>(p);
-  else nn_kernel<T, BK, STAGES, false, A_TR, B_TR><<<grid, dim3(256), 0, s>>>(p);
+  if (packed) nn_kernel<T, BK, STAGES, true, A_TR, B_TR, KTAIL><<<grid, dim3(256), 0, s>>>(p);
+  else nn_kernel<T, BK, STAGES, false, A_TR, B_TR, KTAIL><<<grid, dim3(256), 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }
@@ -1900,6 +1923,22 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
       rc = plan_split_k(p, c, v.bk);
       if (rc) return rc;
       return bf16 ? v.launch_bf16[form](p, s) : v.launch_f16[form](p, s);
+    }
+    // K a multiple of 8 that no variant's K-tile divides: the builds with a partial last K-tile (never split)
+    if (p.K % 8 == 0 && !c.stages && c.split_k <= 1) {
+#define KAPY_NN_TAIL(BK) {launch_nn<Bf16M16, BK, 4, false, true, true>, launch_nn<Bf16M16, BK, 4, true, true, true>, launch_nn<Bf16M16, BK, 4, true, false, true>, \
+                          launch_nn<F16M16, BK, 4, false, true, true>, launch_nn<F16M16, BK, 4, true, true, true>, launch_nn<F16M16, BK, 4, true, false, true>}
+      // (with both operands transposed only the 32-deep build: the 64-deep one needs a stack object for its fragments and
+      // gave wrong results)
+      static int (*const kTail64[6])(GemmParams, hipStream_t) = {launch_nn<Bf16M16, 64, 4, false, true, true>, nullptr, launch_nn<Bf16M16, 64, 4, true, false, true>,
+                                                                 launch_nn<F16M16, 64, 4, false, true, true>, nullptr, launch_nn<F16M16, 64, 4, true, false, true>};
+      static int (*const kTail32[6])(GemmParams, hipStream_t) = KAPY_NN_TAIL(32);
+#undef KAPY_NN_TAIL
+      const int bk = c.tile_k ? c.tile_k : (p.K >= 256 && form != 1 ? 64 : 32);
+      if ((bk == 64 && form != 1) || bk == 32) {
+        p.split_k = 1;
+        return (bk == 64 ? kTail64 : kTail32)[(bf16 ? 0 : 3) + form](p, s);
+      }
     }
   }
   if ((c.tile_m && c.tile_m != kSBM) || (c.tile_n && c.tile_n != kSBN) || (c.tile_k && c.tile_k != kSBK) || (c.stages && c.stages != 1) ||

@@ -297,3 +297,23 @@ def test_transposing_read_kernel_with_columns_that_do_not_fill_the_last_tile(ko,
         got = to_host(dd, np.uint16)
         assert np.all(got[M * N:] == 0x1234), (M, N, K)
         assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL, (M, N, K)
+
+
+@pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("a_rm,b_rm", [(True, True), (False, True), (False, False)])
+def test_transposing_read_kernel_with_a_partial_last_k_tile(ko, dt, a_rm, b_rm):
+    """K a multiple of 8 that the K-tile does not divide: the pieces of the last tile beyond K arrive as zeros.  The operands
+    are followed in memory by large finite values and NaNs (a next row, another tensor): none of it may reach a result."""
+    for (M, N, K) in ((128, 256, 1000), (256, 128, 72), (128, 136, 8), (384 if not a_rm else 200, 128, 64 * 5 + 8), (128, 128, 32 * 3 + 24)):
+        a, b = ko.fill_uniform(M * K, dt, 27, 0), ko.fill_uniform(K * N, dt, 27, 1)
+        a_str, b_str = ((K, 1) if a_rm else (1, M)), ((N, 1) if b_rm else (1, K))
+        want = np.zeros(M * N, dtype=np.uint16)
+        assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, *a_str, dt)), C.byref(ko.mk_global(b, K, N, *b_str, dt)), None,
+                                  C.byref(ko.mk_global(want, M, N, N, 1, dt)), kh.RN) == 0
+        poison = np.full(4096, 0x7e00 if dt == kh.F16 else 0x7fc0, np.uint16)       # NaNs behind each operand
+        da, db, dd = to_dev(np.concatenate([a, poison])), to_dev(np.concatenate([b, poison])), dev_zeros(M * N + 256, 2, fill=0x1234)
+        kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(dd, M, N, N, 1, dt))
+        sync()
+        got = to_host(dd, np.uint16)
+        assert np.all(got[M * N:] == 0x1234), (M, N, K)
+        assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL, (M, N, K)

@@ -406,7 +406,10 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   p.d_dtype = result->dtype;
   p.rz = cfg && cfg->rmode == KAPY_RZ;
   if (p.M == 0 || p.N == 0) return KAPY_OK;
-  bool k_contig = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(a, 1) == 16 && vector_bytes(b, 0) == 16 && p.K % 128 == 0 && p.K > 0;
+  // K-contiguous operands with 16-byte aligned rows of whole 16-byte pieces: what the tiled kernel needs (its ring builds take
+  // a partial last K-tile); the streaming kernels below need whole 128-byte K steps
+  const bool k_pieces = p.a_sk == 1 && p.b_sk == 1 && vector_bytes(a, 1) == 16 && vector_bytes(b, 0) == 16 && p.K % 16 == 0 && p.K > 0;
+  const bool k_contig = k_pieces && p.K % 128 == 0;
   // Many rows: the tiled LDS-direct kernel (MFMA-bound).  Few rows: the skinny kernel (HBM-bound).
   // With a workspace the tiled kernel can split K over several workgroups per tile, which fills the device at few rows too.
   kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
@@ -414,7 +417,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   // (offsets inside a workgroup's rows and columns are 32-bit)
   const bool block_ok = k_contig && p.M > 16 && p.K % (4 * kBlockStep) == 0 && p.a_sm * 64 < (int64_t(1) << 31) && p.b_sn * kBlockCols < (int64_t(1) << 31) &&
                         ((int64_t)(p.N + kBlockCols - 1) / kBlockCols + 8) * ((p.M + 31) / 32) < (int64_t(1) << 31);
-  if (k_contig && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
+  if (k_pieces && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
     GemmParams g;
     g.a = (const char *)p.a; g.b = (const char *)p.b; g.acc = nullptr; g.d = p.d;
     g.row_scale = row_scale; g.col_scale = col_scale;
@@ -427,7 +430,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     if (rc) return rc;
     // an explicit split is a request for the tiled kernel; the library's own choice weighs it against the block kernel
     const int tiled_from = block_ok && c.split_k <= 1 ? (g.split_k > 1 ? kTiledFromMSplit : kTiledFromM) : (g.split_k > 1 ? kTiledFromMSplitNoBlock : kTiledFromMNoBlock);
-    if (p.M < tiled_from) rc = KAPY_ERR_UNSUPPORTED;  // few rows: the streaming kernels below
+    if (k_contig && p.M < tiled_from) rc = KAPY_ERR_UNSUPPORTED;  // few rows: the streaming kernels below (which need whole K steps)
     else rc = matmul_f8_tiled(g, fmt_of(a->dtype), fmt_of(b->dtype), c.tile_m == 256 || c.tile_m == 128 ? c.tile_m : 0, s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
   }

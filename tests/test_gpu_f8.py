@@ -199,3 +199,20 @@ def test_f8_256_tiles_mixed_formats_f32_result(ko):
         sync()
         got = to_host(dd, np.float32, (m, n))
         assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-4
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 128, 144), (200, 256, 400), (64, 264, 656), (1000, 1000, 1040), (1, 128, 128 + 16), (300, 520, 8256)])
+def test_scaled_f8_with_k_of_whole_16_byte_pieces_takes_the_tiled_kernel(ko, M, N, K):
+    """K a multiple of 16 but not of 128, any number of rows: the tiled ring kernel with a partial last K-tile (the streaming
+    kernels for few rows need whole 128-byte K steps).  Guard words behind the result."""
+    aq, sa, wq, sb = _quantised(ko, M, N, K, seed=9)
+    want = np.zeros((M, N), dtype=np.uint16)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                        vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16))) == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N + 4096, 2, fill=0x1234)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    got = to_host(dd, np.uint16)
+    assert np.all(got[M * N:] == 0x1234)
+    assert _frob(ko, got[:M * N].reshape(M, N), want) <= FROB_TOL

@@ -385,7 +385,7 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
  * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`.  The elements themselves are folded, as the
  * lowering does (no identity element joins them): a line of only -0 sums to -0; max orders -0 below +0 and a NaN wins.
  * Launches that leave few results per workgroup share the reduced axis out over workgroups and fold fp32 partial results in
- * a second launch, in a fixed order (the same bits every run).  The partial results live in a 1 MiB block the library
+ * a second launch, in a fixed order (the same bits every run).  The partial results live in a 4 MiB block the library
  * allocates once per device at the first such call (hipMalloc: not while `stream` is being captured - then, and if the
  * allocation fails, the reduction runs in one pass); calls on different streams take turns at it through an event. */
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream);

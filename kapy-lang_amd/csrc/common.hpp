@@ -76,6 +76,11 @@ int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_d
                        char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes);
 
 int check_global(const kapy_global *g, const char *what);
+// A block of device memory the library keeps per device for partial results of reductions (wave_ops.hip): acquire hands it
+// out for work on `stream` with a lock held (nullptr, and no lock, while the stream is being captured or without memory),
+// release after the last launch that touches it.
+float *partials_acquire(hipStream_t stream, size_t *bytes);
+int partials_release(hipStream_t stream);
 int ensure_device();
 int device_cus();
 

@@ -202,6 +202,66 @@ __global__ __launch_bounds__(256) void stack_kernel_any(StackProgram P) { stack_
 // rows whose width is not a multiple of 8 (row starts still 16-byte aligned): the last vector of a row moves element by element
 __global__ __launch_bounds__(256) void stack_kernel_narrow_ragged(StackProgram P) { stack_run<true, true>(P); }
 
+// A reduce along axis 0 of a program's value, for the column programs (run_column_program): the stack machine's steps with
+// the store replaced by a fold over rows.  A workgroup owns a strip of 8 * LPR columns (LPR lanes x one vector of 8) and a
+// chunk of the rows, which its 256 / LPR groups of lanes walk; the groups' partial results meet in LDS and every
+// (chunk, column) leaves an fp32 partial result in `lines`, which column_fold_kernel folds in chunk order.
+template <int LPR>
+__global__ __launch_bounds__(256) void stack_colreduce_kernel(StackProgram P, float *lines, int32_t per_chunk, int32_t sum) {
+  constexpr int GROUPS = 256 / LPR, COLS = LPR * 8;
+  __shared__ float part[GROUPS][COLS + 1];
+  const int cl = threadIdx.x % LPR, rg = threadIdx.x / LPR;
+  const int32_t jv = (int32_t)blockIdx.x * LPR + cl;
+  const int32_t r_begin = blockIdx.y * per_chunk, r_end = min(P.rows, r_begin + per_chunk);
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = sum ? -0.f : -__builtin_inff();  // -0: the identity of addition
+  if (jv < P.vec_per_row) {
+    for (int32_t i = r_begin + rg; i < r_end; i += GROUPS) {
+      float v[3][8];
+#pragma unroll
+      for (int d = 0; d < 3; ++d)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[d][e] = 0.f;
+      for (int pc = 0; pc < P.n_post; ++pc) {
+        const PostOp I = P.post[pc];
+        if (I.op == kStore) {  // (the value to fold is at the bottom of the stack)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = sum ? acc[e] + v[0][e] : max_nan(acc[e], v[0][e]);
+          continue;
+        }
+        switch (I.slot) {
+        case 0: stack_step<0, false>(P, I, i, jv, v); break;
+        case 1: stack_step<1, false>(P, I, i, jv, v); break;
+        default: stack_step<2, false>(P, I, i, jv, v);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) part[rg][cl * 8 + e] = acc[e];
+  __syncthreads();
+  const int64_t col = (int64_t)blockIdx.x * COLS + threadIdx.x;
+  if (threadIdx.x < COLS && col < (int64_t)P.vec_per_row * 8) {
+    float t = part[0][threadIdx.x];
+#pragma unroll
+    for (int g = 1; g < GROUPS; ++g) t = sum ? t + part[g][threadIdx.x] : max_nan(t, part[g][threadIdx.x]);
+    lines[(int64_t)blockIdx.y * P.vec_per_row * 8 + col] = t;
+  }
+}
+
+// `chunks` partial lines of n values folded in chunk order, rounded once to the reduce's type, stored as that type.
+__global__ __launch_bounds__(256) void column_fold_kernel(const float *lines, int32_t chunks, int32_t n, int32_t sum, int32_t dtype, void *result) {
+  const int32_t col = (int32_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= n) return;
+  float t = lines[col];
+  for (int32_t c = 1; c < chunks; ++c) {
+    const float x = lines[(int64_t)c * n + col];
+    t = sum ? t + x : max_nan(t, x);
+  }
+  store_from_f32(result, dtype, col, t);
+}
+
 // ---------------------------------------------------------------------------------------------
 // out[i,j] = cast_out( act( f32(x[i,j]) * scale + f32(bias) ) ), x/out contiguous along j.
 enum BiasMode { kNoBias = 0, kBiasRow = 1 /* bias[0,j] */, kBiasCol = 2 /* bias[i,0] */, kBiasFull = 3 };
@@ -786,6 +846,117 @@ DevView to_dev(const kapy_global *g) {
 
 
 // A program whose reduces all run along axis 0, on the column machine.
+bool stream_is_capturing(hipStream_t s);
+
+// The column program as a sequence of launches over the whole device, where its shapes allow: phase p (one per reduce) is an
+// elementwise program of its own - the instructions reduce p depends on, with every earlier reduce replaced by a load of
+// that reduce's per-column results ([1 x n], in the reduce's type) - whose value is folded over rows instead of stored
+// (stack_colreduce_kernel over strips x row chunks, then column_fold_kernel); the last phase is an ordinary
+// kapy_elementwise call with the results as row operands.  The results and the partial lines live in the block of
+// partials_acquire.  Returns 1 when the program ran this way, 0 when it does not fit (the caller then runs the one-launch
+// column machine, which takes any views), a negative status on failure.
+int run_column_phases(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                      const ColumnPlan &C, const Program &P, hipStream_t s) {
+  const int n_reduce = C.n_phases - 1;
+  const int64_t m = extent0(out), n = extent1(out);
+  if (n % 8 != 0 || out->stride1 != 1 || n_ins + n_reduce > kMaxInputs || m < 64 || stream_is_capturing(s)) return 0;
+  // phase programs, built before anything is launched: any that does not fit the stack machine sends the whole call back
+  struct Phase {
+    kapy_ew_inst inst[kMaxInst + 1];
+    int dtype[kMaxInst + 1];
+    int n = 0;
+  };
+  std::vector<Phase> phases(C.n_phases);
+  int reduce_dtype[kMaxColumnReduces] = {0, 0, 0, 0};
+  for (int k = 0; k < n_inst; ++k)
+    if (prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX) reduce_dtype[P.inst[k].c] = result_dtype[k];
+  for (int ph = 0; ph < C.n_phases; ++ph) {
+    Phase &F = phases[ph];
+    for (int k = 0; k < C.stop[ph]; ++k) {
+      if (!((C.need[ph] >> k) & 1)) continue;
+      kapy_ew_inst I = prog[k];
+      if (I.op == KAPY_EW_REDUCE_SUM || I.op == KAPY_EW_REDUCE_MAX) {
+        const int which = P.inst[k].c;
+        I = kapy_ew_inst{};
+        I.op = KAPY_EW_LD_GLOBAL;
+        I.dst = prog[k].dst;
+        I.a = n_ins + which;
+        I.c = KAPY_PAD_ZERO;
+      }
+      F.dtype[F.n] = result_dtype[k];
+      F.inst[F.n++] = I;
+    }
+    if (ph < n_reduce) {  // the value the reduce folds, "stored" (the kernel folds it instead)
+      kapy_ew_inst St{};
+      St.op = KAPY_EW_ST_GLOBAL;
+      St.a = prog[C.stop[ph]].a;
+      F.dtype[F.n] = reduce_dtype[ph];
+      F.inst[F.n++] = St;
+    }
+  }
+  size_t bytes = 0;
+  float *block = partials_acquire(s, &bytes);
+  if (!block) return 0;
+  auto give_up = [&](int rc) {
+    (void)partials_release(s);
+    return rc;
+  };
+  // [results of up to four reduces, 4 bytes per column each][partial lines]
+  const int64_t floats = (int64_t)(bytes / sizeof(float)), left = floats / n - kMaxColumnReduces;
+  if (left < 1) return give_up(0);
+  const int lpr = n >= 256 ? 32 : 8;
+  const int64_t strips = (n / 8 + lpr - 1) / lpr, want = 4 * (int64_t)device_cus();
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, m / 64, 256, left}));
+  const int32_t per_chunk = (int32_t)((m + chunks - 1) / chunks);
+  chunks = (m + per_chunk - 1) / per_chunk;
+  float *lines = block + kMaxColumnReduces * n;
+  kapy_global views[kMaxInputs];
+  const kapy_global *all[kMaxInputs];
+  for (int k = 0; k < n_ins; ++k) all[k] = ins[k];
+  for (int c = 0; c < n_reduce; ++c) {
+    kapy_global &v = views[c];
+    v.ptr = block + c * n;
+    v.start0 = v.start1 = 0;
+    v.end0 = 1;
+    v.end1 = v.stride0 = (int32_t)n;
+    v.stride1 = 1;
+    v.dtype = reduce_dtype[c];
+    v.alignment = 16;
+    all[n_ins + c] = &v;
+  }
+  if (strips > 0x7fffffff || n >= (int64_t(1) << 31)) return give_up(0);
+  // the reduce phases' stack programs (the value type of a phase is its reduce operand's: a pseudo-result of that type)
+  std::vector<StackProgram> SP(n_reduce);
+  for (int ph = 0; ph < n_reduce; ++ph) {
+    kapy_global pseudo = *out;
+    pseudo.ptr = lines;  // (an aligned address; never written)
+    pseudo.start0 = pseudo.start1 = 0;
+    pseudo.end0 = (int32_t)m;
+    pseudo.end1 = pseudo.stride0 = (int32_t)n;
+    pseudo.stride1 = 1;
+    const Phase &F = phases[ph];
+    // the operand's type: that of the instruction that defines the stored register last
+    int operand_dtype = -1;
+    for (int k = 0; k + 1 < F.n; ++k)
+      if (F.inst[k].op != KAPY_EW_ST_GLOBAL && F.inst[k].dst == F.inst[F.n - 1].a) operand_dtype = F.dtype[k];
+    if (operand_dtype < 0) return give_up(0);
+    pseudo.dtype = operand_dtype;
+    if (!build_stack_program(F.inst, F.n, F.dtype, all, n_ins + ph, &pseudo, &SP[ph]) || SP[ph].width) return give_up(0);
+  }
+  for (int ph = 0; ph < n_reduce; ++ph) {
+    const int sum = prog[C.stop[ph]].op == KAPY_EW_REDUCE_SUM;
+    dim3 grid((unsigned)strips, (unsigned)chunks);
+    if (lpr == 32) stack_colreduce_kernel<32><<<grid, 256, 0, s>>>(SP[ph], lines, per_chunk, sum);
+    else stack_colreduce_kernel<8><<<grid, 256, 0, s>>>(SP[ph], lines, per_chunk, sum);
+    column_fold_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(lines, (int32_t)chunks, (int32_t)n, sum, reduce_dtype[ph], block + ph * n);
+  }
+  const Phase &L = phases[n_reduce];
+  int rc = kapy_elementwise(L.inst, L.n, all, n_ins + n_reduce, out, (void *)s);
+  const int released = partials_release(s);
+  if (rc) return rc;
+  return released ? released : 1;
+}
+
 int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
                        hipStream_t s) {
   Program P;
@@ -829,6 +1000,10 @@ int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
   for (int k = 0; k < n_inst; ++k)
     if (prog[k].op == KAPY_EW_LD_GLOBAL) P.in[prog[k].a].pad = padding_word_of(ins[prog[k].a]->dtype, prog[k].c);
   P.out = to_dev(out);
+  {
+    const int fast = run_column_phases(prog, n_inst, result_dtype, ins, n_ins, out, C, P, s);
+    if (fast != 0) return fast < 0 ? fast : KAPY_OK;
+  }
   const int64_t strips = (extent1(out) + 63) / 64;
   if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "elementwise: too many columns for a program with reduces along axis 0");
   // many rows: more waves per strip

@@ -240,7 +240,7 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(ReduceParams p, c
 // threads cannot interleave.  Not available - and then the caller reduces in one pass - while the stream is being
 // captured (an event of another stream's work cannot be waited for inside a capture) or when the allocation fails.
 constexpr int kMaxPartialsDevices = 16;
-constexpr size_t kPartialsBytes = size_t(1) << 20;  // the launch keeps chunks * n_keep * 4 within this
+constexpr size_t kPartialsBytes = size_t(4) << 20;  // the launches keep what they leave there within this
 struct Partials {
   float *lines = nullptr;
   hipEvent_t free_again = nullptr;
@@ -301,6 +301,31 @@ int partials_used(Partials *P, hipStream_t s) {
   }
   return KAPY_OK;
 }
+
+}  // namespace
+
+// The same block for the column programs of kapy_elementwise (elementwise.hip): acquire returns it ready for work on `s`
+// with the mutex held, or nullptr (then nothing is held); release, after the caller's last launch that touches it, records
+// the event the next user waits for and lets go of the mutex.
+float *partials_acquire(hipStream_t s, size_t *bytes) {
+  partials_mutex.lock();
+  Partials *P = partials_for(s);
+  if (!P) {
+    partials_mutex.unlock();
+    return nullptr;
+  }
+  *bytes = kPartialsBytes;
+  return P->lines;
+}
+int partials_release(hipStream_t s) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  const int rc = partials_used(&partials_of[dev], s);
+  partials_mutex.unlock();
+  return rc;
+}
+
+namespace {
 
 // Any element type, alignment and extents, kept axis contiguous (or at least not the strided one): a workgroup owns 64 kept
 // indices, one per lane of a wave (a wave's loads cover 64 consecutive elements of one reduced index), its four waves share

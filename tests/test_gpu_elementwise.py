@@ -432,6 +432,24 @@ def test_softmax_columns_every_launch_shape(ko, dtype, m, n):
     assert np.allclose(sums, 1.0, atol=m * 2.0 ** (-11 if dtype == kh.F16 else -8) * 0.05 + 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(5000, 512), (70000, 64), (64, 2048), (3000, 264), (129, 8)])
+def test_column_programs_run_as_phases_over_the_whole_device(ko, dtype, m, n):
+    """Widths that are multiples of 8 and at least 64 rows: every reduce is a launch of its own over strips x row chunks with
+    its per-column results kept in memory for the phases after it.  Softmax, and a program whose second reduce depends on
+    the first and on a column operand, in 16-bit arithmetic (the per-column results are then 16-bit too)."""
+    got, want = _row_case(ko, _along_columns(kh.softmax_insts(dtype)), dtype, m, n, 160 + n % 97)
+    _check_ulp(got, want, dtype)
+    # y = (x - max_col(x)) * c[row] - max_col((x - max_col(x)) * c[row]), all in `dtype`
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_REDUCE_MAX, dst=1, a=0, b=0), dict(op=kh.EW_SUBF, dst=0, a=0, b=1),
+             dict(op=kh.EW_LD_GLOBAL, dst=2, a=1), dict(op=kh.EW_MULF, dst=0, a=0, b=2), dict(op=kh.EW_REDUCE_MAX, dst=3, a=0, b=0),
+             dict(op=kh.EW_SUBF, dst=0, a=0, b=3), dict(op=kh.EW_ST_GLOBAL, a=0)]
+    x = ko.fill_normal(m * n, dtype, 161, std=2.0).reshape(m, n)
+    c = ko.fill_normal(m, dtype, 162, mean=1.0, std=0.25)
+    got, want = _run_prog(ko, insts, [x, c], [dtype, dtype], dtype, m, n, in_shapes=[(m, n), (m, 1)])
+    assert np.array_equal(got, want)            # max and single roundings only: bit-exact
+
+
 def test_column_program_equals_the_row_program_on_the_transposed_problem(ko):
     # the same numbers through the other machine: transposing the operand and the result turns columns into rows;
     # max is exact and the sums differ by the order of the fp32 additions only

@@ -1047,6 +1047,26 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   bool has_reduce = false;
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
 
+  // A column-major result: the same program on the transposed problem has a row-major one (every view with its axes
+  // swapped - a row operand becomes a column operand and the other way round), which is what the fast kernels are written for.
+  // Operands that are column-major too then read along their rows; the others are no worse off than before.
+  if (!has_reduce && out->stride0 == 1 && out->stride1 != 1 && o1 > 1 && n_ins <= kMaxInputs) {
+    auto swapped = [](const kapy_global *g) {
+      kapy_global v = *g;
+      std::swap(v.start0, v.start1);
+      std::swap(v.end0, v.end1);
+      std::swap(v.stride0, v.stride1);
+      return v;
+    };
+    kapy_global views[kMaxInputs], result = swapped(out);
+    const kapy_global *ptrs[kMaxInputs];
+    for (int k = 0; k < n_ins; ++k) {
+      views[k] = swapped(ins[k]);
+      ptrs[k] = &views[k];
+    }
+    return kapy_elementwise(as_given, n_inst, ptrs, n_ins, &result, stream);
+  }
+
   // Rows that are not a whole number of 8-element vectors move element by element (or, 16-bit only, with a ragged last
   // vector per row, and then only from aligned rows).  When the result and every operand are dense matrices of one shape
   // (pitch = width) or single elements, the program does not care where a row ends: it runs once over the first

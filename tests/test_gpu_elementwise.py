@@ -627,3 +627,27 @@ def test_dense_operands_with_odd_widths_run_as_one_line(ko, dtype, m, n):
     sync()
     got = to_host(dout, np_t)
     assert np.array_equal(got[:m * n], want.view(np_t)) and np.all(got[m * n:] == got[-1]) and got[-1] != 0
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.F32])
+def test_column_major_result_runs_as_the_transposed_problem(ko, dtype):
+    """Result and full operands column-major, a [1 x n] and a [m x 1] operand beside them: the call is the row-major program on
+    the transposed problem (the row operand becomes a column operand and the other way round).  Bit-exact."""
+    m, n = 200, 136
+    eb = kh.DTYPE_BYTES[dtype]
+    np_t = {2: np.uint16, 4: np.uint32}[eb]
+    a, b = ko.fill_normal(m * n, dtype, 95, 0), ko.fill_normal(m * n, dtype, 95, 1)
+    r, c = ko.fill_normal(n, dtype, 96, 0), ko.fill_normal(m, dtype, 96, 1)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_LD_GLOBAL, dst=1, a=1), dict(op=kh.EW_LD_GLOBAL, dst=2, a=2),
+             dict(op=kh.EW_LD_GLOBAL, dst=3, a=3), dict(op=kh.EW_MULF, dst=4, a=0, b=2), dict(op=kh.EW_FMA, dst=4, a=1, b=3, c=4),
+             dict(op=kh.EW_ST_GLOBAL, a=4)]
+    want = np.zeros(m * n, np_t)
+    shapes = [(m, n, 1, m), (m, n, 1, m), (1, n, n, 1), (m, 1, 1, 1)]      # (rows, cols, stride0, stride1): a, b column-major
+    gos = [ko.mk_global(t, *sh, dtype) for t, sh in zip((a, b, r, c), shapes)]
+    assert ko.elementwise(ko.program(insts), gos, ko.mk_global(want, m, n, 1, m, dtype)) == 0
+    devs = [to_dev(t) for t in (a, b, r, c)]
+    dout = dev_zeros(m * n + 32, eb, fill=0x5A5A)
+    kh.elementwise(kh.program(insts), [dglobal(t, *sh, dtype) for t, sh in zip(devs, shapes)], dglobal(dout, m, n, 1, m, dtype))
+    sync()
+    got = to_host(dout, np_t)
+    assert np.array_equal(got[:m * n], want.view(np_t)) and np.all(got[m * n:] == got[-1]) and got[-1] != 0

@@ -77,6 +77,49 @@ __global__ __launch_bounds__(256) void naive_kernel(F8Params p) {
   finish(p, m, n, s);
 }
 
+// What no other kernel takes (operand rows that are not 16-byte aligned, K not a multiple of 16, strided operands): 64 x 64
+// results per workgroup, 4 x 4 per lane, K in steps of 32 whose operand elements are loaded one by one (lanes along K),
+// decoded to fp32 into LDS and multiplied there on the vector ALU.  About fifty times the one-lane-per-result kernel above.
+__global__ __launch_bounds__(256) void tiled_any_kernel(F8Params p) {
+  constexpr int T = 64, KS = 32, PITCH = KS + 1;
+  __shared__ float as[T * PITCH], bs[T * PITCH];
+  const int t = threadIdx.x, ty = t >> 4, tx = t & 15;
+  const int32_t tiles_n = (p.N + T - 1) / T;
+  const int32_t m0 = (int32_t)(blockIdx.x / tiles_n) * T, n0 = (int32_t)(blockIdx.x % tiles_n) * T;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int32_t k0 = 0; k0 < p.K; k0 += KS) {
+#pragma unroll
+    for (int i = 0; i < T * KS / 256; ++i) {
+      const int e = t + 256 * i, row = e / KS, k = e % KS;
+      const bool k_in = k0 + k < p.K;
+      as[row * PITCH + k] = (k_in && m0 + row < p.M) ? load_as_f32(p.a, p.a_dtype, (int64_t)(m0 + row) * p.a_sm + (int64_t)(k0 + k) * p.a_sk) : 0.f;
+      bs[row * PITCH + k] = (k_in && n0 + row < p.N) ? load_as_f32(p.b, p.b_dtype, (int64_t)(n0 + row) * p.b_sn + (int64_t)(k0 + k) * p.b_sk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < KS; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = as[(ty * 4 + i) * PITCH + k];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = bs[(tx * 4 + j) * PITCH + k];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) finish(p, m0 + ty * 4 + i, n0 + tx * 4 + j, acc[i][j]);
+}
+
 // 32 K-contiguous bytes of one row/column as the 8-dword MFMA operand; rows past the end read zero.
 __device__ __forceinline__ i32x8 load_k32(const uint8_t *base, int64_t stride, int32_t row, int32_t rows, int32_t k) {
   i32x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -467,8 +510,9 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
       return KAPY_OK;
     }
   }
-  int64_t total = (int64_t)p.M * p.N;
-  naive_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(p);
+  const int64_t tiles = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
+  if (tiles < (int64_t(1) << 31) && (int64_t)p.M * p.N >= 4096) tiled_any_kernel<<<(unsigned)tiles, 256, 0, s>>>(p);
+  else naive_kernel<<<(unsigned)(((int64_t)p.M * p.N + 255) / 256), 256, 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }

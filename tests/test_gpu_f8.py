@@ -216,3 +216,19 @@ def test_scaled_f8_with_k_of_whole_16_byte_pieces_takes_the_tiled_kernel(ko, M, 
     got = to_host(dd, np.uint16)
     assert np.all(got[M * N:] == 0x1234)
     assert _frob(ko, got[:M * N].reshape(M, N), want) <= FROB_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(100, 200, 100), (64, 64, 8200), (130, 70, 24), (1, 4096, 40), (257, 129, 1000)])
+def test_scaled_f8_with_rows_that_are_not_16_byte_aligned(ko, M, N, K):
+    """K not a multiple of 16: no vector load reaches these rows; the tiled fp32 kernel for everything else.  Guard words."""
+    aq, sa, wq, sb = _quantised(ko, M, N, K, seed=11)
+    want = np.zeros((M, N), dtype=np.uint16)
+    assert ko.lib().ko_matmul_scaled_f8(C.byref(ko.mk_global(aq, M, K, K, 1, ko.F8E4M3)), C.byref(ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)),
+                                        vp(sa), vp(sb), C.byref(ko.mk_global(want, M, N, N, 1, ko.BF16))) == 0
+    da, dw, dsa, dsb, dd = to_dev(aq), to_dev(wq), to_dev(sa), to_dev(sb), dev_zeros(M * N + 4096, 2, fill=0x1234)
+    kh.matmul_scaled_f8(dglobal(da, M, K, K, 1, kh.F8E4M3), dglobal(dw, K, N, 1, K, kh.F8E4M3), dsa.data_ptr(), dsb.data_ptr(),
+                        dglobal(dd, M, N, N, 1, kh.BF16))
+    sync()
+    got = to_host(dd, np.uint16)
+    assert np.all(got[M * N:] == 0x1234)
+    assert _frob(ko, got[:M * N].reshape(M, N), want) <= FROB_TOL

@@ -62,6 +62,33 @@ __device__ __forceinline__ void copy_one(const CopyParams &p, const char *src, c
   *(T *)(dst + (i * p.ds0 + j * p.ds1) * B) = v;
 }
 
+// A transposing move no vector kernel takes (extents that are not multiples of 8, rows that are not 16-byte aligned):
+// 64 x 64 tiles through LDS, element by element, lanes along the source's contiguous axis (i) when reading and along the
+// destination's (j) when writing, so that both sides see runs of 64 elements where generic_kernel strides one of them.
+template <int B>
+__global__ __launch_bounds__(256) void transpose_any_kernel(CopyParams p) {
+  typedef typename ElemOf<B>::type T;
+  __shared__ T tile[64][65];
+  const char *src;
+  char *dst;
+  program_base<B>(p, src, dst);
+  const int32_t ti = blockIdx.x * 64, tj = blockIdx.y * 64;
+  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+#pragma unroll 4
+  for (int r = 0; r < 16; ++r) {
+    const int32_t i = ti + lane, j = tj + q + 4 * r;
+    T v = (T)p.pad;
+    if (i < p.d0 && j < p.d1 && i < p.sb0 && j < p.sb1) v = *(const T *)(src + ((int64_t)i * p.es0 + (int64_t)j * p.es1) * B);
+    tile[q + 4 * r][lane] = v;
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (int r = 0; r < 16; ++r) {
+    const int32_t i = ti + q + 4 * r, j = tj + lane;
+    if (i < p.d0 && j < p.d1) *(T *)(dst + ((int64_t)i * p.ds0 + (int64_t)j * p.ds1) * B) = tile[lane][q + 4 * r];
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 template <int B>
 __global__ __launch_bounds__(256) void generic_kernel(CopyParams p, int j_fastest) {
@@ -349,6 +376,11 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
       KAPY_HIP_CHECK(hipGetLastError());
       return KAPY_OK;
     }
+  }
+  if (p.ds1 == 1 && p.es0 == 1 && p.d0 >= 16 && p.d1 >= 16 && (p.d1 + 63) / 64 <= 65535) {
+    transpose_any_kernel<B><<<dim3((unsigned)((p.d0 + 63) / 64), (unsigned)((p.d1 + 63) / 64), (unsigned)batch), 256, 0, stream>>>(p);
+    KAPY_HIP_CHECK(hipGetLastError());
+    return KAPY_OK;
   }
   int64_t total = (int64_t)p.d0 * p.d1;
   int j_fastest = p.ds1 <= p.ds0;

@@ -229,3 +229,23 @@ def test_dense_copy_with_odd_widths_moves_as_one_line(ko, dtype, rows, cols):
     sync()
     got = to_host(d_dst, np_t)
     assert np.array_equal(got[:rows * cols], src) and np.all(got[rows * cols:] == got[-1]) and got[-1] != 0
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.F32, kh.F8E4M3])
+@pytest.mark.parametrize("rows,cols", [(301, 501), (17, 33), (3001, 5001), (64, 65), (1000, 16)])
+def test_transpose_with_extents_no_vector_reaches(ko, dtype, rows, cols):
+    """Extents that are not multiples of 8 (rows that are not 16-byte aligned): 64 x 64 tiles through LDS element by element.
+    Windows of wider buffers, guard words beside and behind the destination window; against numpy's transpose."""
+    eb = kh.DTYPE_BYTES[dtype]
+    np_t = {1: np.uint8, 2: np.uint16, 4: np.uint32}[eb]
+    sp, dp = cols + 3, rows + 5
+    src = np.random.RandomState(rows * 11 + cols).randint(1, 2 ** (8 * eb - 1), size=rows * sp).astype(np_t).reshape(rows, sp)
+    d_src, d_dst = to_dev(src), dev_zeros(cols * dp + 64, eb, fill=0x5A)
+    kh.copy(dglobal(d_src, rows, cols, sp, 1, dtype), dglobal(d_dst, cols, rows, dp, 1, dtype), transpose=True)
+    sync()
+    got = to_host(d_dst, np_t)
+    guard = got[-1]
+    assert guard != 0 and np.all(got[cols * dp:] == guard)
+    win = got[:cols * dp].reshape(cols, dp)
+    assert np.all(win[:, rows:] == guard)
+    assert np.array_equal(win[:, :rows], src[:, :cols].T)

@@ -75,7 +75,7 @@ MEASURED_TRAFFIC = {"gelu": 268411308, "transpose": 268449994, "add": 402640502,
                     "expr_compiled": 402621054, "swiglu": 402555636, "l2norm_compiled": 268407520, "gelu_transposed": 268397184, "copy": 268435456,
                     "permute": 268435456, "reduce": 134292547, "gemm_bf16": 1764717568, "gemm_bf16_gelu": 1756925952, "f8_m4096": 470365184,
                     "gemm_f16": 21158853, "gemm_f16_graph": 21158853, "gemm_f16_splitk": 37989900, "f8_m16": 68542669, "f8_m64": 72475557, "f8_m128": 82781536,
-                    "f8_m128_splitk": 111420621}
+                    "f8_m128_splitk": 111420621, "reduce_cols": 136388608, "softmax_cols": 542578688}
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -324,6 +324,64 @@ def bench_reduce(kh, steps, warmup, cpu):
     return {"workload": "reduce_sum axis=1 fp16 8192x8192 -> f32 [8192x1]", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "reduce"), "kernel": "reduce_rows_vec_kernel",
             "inputs": "x normal(0,1) seed 0", "checked": True, "check": "every row sum against fp64: max abs error %.2e" % err}
+
+
+def bench_reduce_cols(kh, steps, warmup, cpu):
+    """kapy.reduce along axis 0 (column sums) of the headline shape: strips x row chunks, a second launch folds the chunks."""
+    import numpy as np
+    import torch
+    import ko
+    n, sets = 8192, 4
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]
+    y = torch.empty(n, device="cuda", dtype=torch.float32)
+    gx = [kh.mk_global(x.data_ptr(), n, n, n, 1, kh.F16) for x in xs]
+    gy = kh.mk_global(y.data_ptr(), 1, n, n, 1, kh.F32)
+    kh.reduce(gx[0], gy, 0, 0)
+    torch.cuda.synchronize()
+    hx = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n)
+    want = hx.view(np.float16).astype(np.float64).sum(axis=0)
+    err = float(np.abs(y.cpu().numpy().astype(np.float64) - want).max())
+    if err > 2e-3:
+        raise CheckFailed("reduce along axis 0: max abs error %g" % err)
+    wall, ev = _events(lambda i: kh.reduce(gx[i % sets], gy, 0, 0), steps, warmup)
+    nbytes = n * n * 2 + n * 4
+    return {"workload": "reduce_sum axis=0 fp16 8192x8192 -> f32 [1x8192] (two launches; time of both)", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "reduce_cols"), "kernel": "reduce_cols_strip_kernel + reduce_partials_kernel",
+            "inputs": "x normal(0,1) seed 0", "checked": True, "check": "every column sum against fp64: max abs error %.2e" % err}
+
+
+def bench_softmax_cols(kh, steps, warmup, cpu):
+    """Softmax of every column as one program with two reduces along axis 0: three launches over the matrix (column maxima,
+    column sums of exp, the store), x read three times and y written once."""
+    import numpy as np
+    import torch
+    import ko
+    n, sets = 8192, 2
+    xs = [_dev("normal", n * n, ko.F16, 0, k) for k in range(sets)]
+    ys = [torch.empty(n * n, device="cuda", dtype=torch.int16) for _ in range(sets)]
+    g = lambda t: kh.mk_global(t.data_ptr(), n, n, n, 1, kh.F16)
+    gx, gy = [g(t) for t in xs], [g(t) for t in ys]
+    insts = [dict(i) for i in kh.softmax_insts(kh.F16)]
+    for i in insts:
+        if i["op"] in (kh.EW_REDUCE_MAX, kh.EW_REDUCE_SUM):
+            i["b"] = 0
+    prog = kh.program(insts)
+    kh.elementwise(prog, [gx[0]], gy[0])
+    torch.cuda.synchronize()
+    # gate: 16 columns against the checker (columns are independent)
+    cols = _sample_rows(n, 16)
+    hx = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n)
+    xc, want = np.ascontiguousarray(hx[:, cols]), np.zeros((n, len(cols)), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(xc, n, len(cols), len(cols), 1, ko.F16)], ko.mk_global(want, n, len(cols), len(cols), 1, ko.F16)) == 0
+    worst = int(np.abs(_line16(_download(ys[0], np.uint16, (n, n))[:, cols]) - _line16(want)).max())
+    if worst > ULP_TOL:
+        raise CheckFailed("column softmax: %d ulp against the checker" % worst)
+    wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]], gy[i % sets]), steps, warmup)
+    nbytes = 4 * n * n * 2
+    return {"workload": "softmax of every column, fp16 8192x8192, fp32 arithmetic (program with two reduces along axis 0)", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "softmax_cols"),
+            "kernel": "stack_colreduce_kernel x 2 + column_fold_kernel x 2 + stack_kernel_any", "inputs": "x normal(0,1) seed 0", "checked": True,
+            "check": "16 columns of the timed result against the checker: max %d ulp (tolerance %d); bytes = three reads and one write of the matrix" % (worst, ULP_TOL)}
 
 
 def bench_rowwise(kh, steps, warmup, cpu, which):
@@ -761,7 +819,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
     return out
 
 
-WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
+WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "layernorm", "l2norm_compiled", "gelu_transposed",
              "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
 
 
@@ -794,6 +852,8 @@ def main():
         "transpose": lambda s, w: bench_transpose(kh, s, w, cpu),
         "gelu_transposed": lambda s, w: bench_gelu_transposed(kh, s, w, cpu),
         "reduce": lambda s, w: bench_reduce(kh, s, w, cpu),
+        "reduce_cols": lambda s, w: bench_reduce_cols(kh, s, w, cpu),
+        "softmax_cols": lambda s, w: bench_softmax_cols(kh, s, w, cpu),
         "softmax": lambda s, w: bench_rowwise(kh, s, w, cpu, "softmax"),
         "layernorm": lambda s, w: bench_rowwise(kh, s, w, cpu, "layernorm"),
         "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, cpu, "l2norm_compiled"),

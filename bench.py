@@ -69,13 +69,25 @@ def _events(fn, steps, warmup):
     return wall_ms, start.elapsed_time(end) / steps
 
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the
-# same counter reads for the rows copy of 2 x 128 MiB (workload "copy"); the summaries are under profiles/.
-MEASURED_TRAFFIC = {"gelu": 268411308, "transpose": 268449994, "add": 402640502, "expr": 402796218, "softmax": 268466794, "layernorm": 268779749,
-                    "expr_compiled": 402621054, "swiglu": 402555636, "l2norm_compiled": 268407520, "gelu_transposed": 268397184, "copy": 268435456,
-                    "permute": 268435456, "reduce": 134292547, "gemm_bf16": 1764717568, "gemm_bf16_gelu": 1756925952, "f8_m4096": 470365184,
-                    "gemm_f16": 21158853, "gemm_f16_graph": 21158853, "gemm_f16_splitk": 37989900, "f8_m16": 68542669, "f8_m64": 72475557, "f8_m128": 82781536,
-                    "f8_m128_splitk": 111420621, "reduce_cols": 136388608, "softmax_cols": 542578688}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the same counter reads
+# for the rows copy of 2 x 128 MiB (workload "copy").  The figures are read from the tracked summary of those runs (its
+# lines "traffic_bytes <workload> <bytes>"), which `bench.py --pmc-summary` writes from the profiler's output.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "bench_all_workloads.hbm_traffic_pmc.txt")
+
+
+def _read_traffic(path=TRAFFIC_SUMMARY):
+    out = {}
+    try:
+        for l in open(path):
+            f = l.split()
+            if len(f) == 3 and f[0] == "traffic_bytes":
+                out[f[1]] = int(f[2])
+    except OSError:
+        pass
+    return out
+
+
+MEASURED_TRAFFIC = _read_traffic()
 
 
 def _roof_hbm(bytes_per_launch, ev_ms, key=None):
@@ -531,6 +543,27 @@ def _blocks_frobenius(ko, got, go_a, go_b, M, N, K, out_dtype, count, blk=64, sc
     return float(np.sqrt(num / max(den, 1e-300)))
 
 
+def _whole_frobenius(ko, got, go_a, go_b, M, N, K, out_dtype, scales=None, blocks=16):
+    """Relative Frobenius error of the WHOLE result against the host GEMM of oracle/kapy_baseline.cpp (fp32 over K blocks of 512,
+    the blocks summed in fp64, rounded once), and that host result's own error on `blocks` 64 x 64 blocks against the
+    fp64-accumulated checker, which ties the fast host GEMM to the exact one.  Outside every timed region."""
+    import numpy as np
+    want = np.zeros((M, N), np.uint16)
+    gw = ko.mk_global(want, M, N, N, 1, out_dtype)
+    rs = scales[0].ctypes.data if scales else None
+    cs = scales[1].ctypes.data if scales else None
+    assert ko.lib().ko_baseline_gemm(C.byref(go_a), C.byref(go_b), rs, cs, C.byref(gw), None) == 0
+    host_rel = _blocks_frobenius(ko, want, go_a, go_b, M, N, K, out_dtype, blocks, scales=scales)
+    num = den = 0.0
+    for r0 in range(0, M, 512):    # in slabs: the fp64 images of a 8192 x 8192 result would take 1 GiB
+        g, w = ko.decode(got[r0:r0 + 512], out_dtype), ko.decode(want[r0:r0 + 512], out_dtype)
+        if not np.all(np.isfinite(g)):
+            return float("inf"), host_rel
+        num += float(((g - w) ** 2).sum())
+        den += float((w ** 2).sum())
+    return float(np.sqrt(num / max(den, 1e-300))), host_rel
+
+
 def _cpu_gemm(ko, go_a, go_b, go_d, rows, N, K, scales, what):
     """The packed, register-blocked fp32 GEMM of oracle/kapy_baseline.cpp on the first `rows` rows of the lhs."""
     import numpy as np
@@ -583,6 +616,7 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
     run(0)
     torch.cuda.synchronize()
     got = _download(d, np.uint16, (M, N))
+    host_rel = None
     if fused_gelu:
         # gate: blocks of gelu(c*0.5 + bias) recomputed in fp64 from the checker's fp32-result GEMM of the same blocks
         num = den = 0.0
@@ -602,6 +636,10 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
         n_blocks = 16 if M * N > 1024 * 1024 else 0
         if n_blocks:
             rel = _blocks_frobenius(ko, got, go_a, go_b, M, N, K, dtype, n_blocks)
+            whole, host_rel = _whole_frobenius(ko, got, go_a, go_b, M, N, K, dtype)
+            if not host_rel <= FROB_TOL:
+                raise CheckFailed("%s: the host GEMM itself is off the fp64 checker by %g" % (name, host_rel))
+            rel = max(rel, whole)
         else:   # small enough for the whole result
             want = np.zeros((M, N), np.uint16)
             assert ko.lib().ko_matmul(C.byref(go_a), C.byref(go_b), None, C.byref(ko.mk_global(want, M, N, N, 1, dtype)), ko.RN) == 0
@@ -623,8 +661,10 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
     kind = "bf16" if dtype == kh.BF16 else "f16"
     out = {"workload": name, "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "kernel_ms": ev,
            "dtype": kind, "roofline": _roof_mfma(flops, ev, kind, key), "kernel": kernel, "inputs": what + " (host-generated, as the configuration states)",
-           "checked": True, "check": "%s against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" %
-                                     ("%d 64x64 blocks of the timed result" % n_blocks if n_blocks else "the whole timed result", rel, tol)}
+           "checked": True, "check": "%s: relative Frobenius error %.2e (tolerance %.0e)" %
+                                     ("the whole timed result against the host GEMM (fp64 sums of fp32 K blocks; itself %.1e off the fp64-accumulated checker on 16 blocks) "
+                                      "and %d 64x64 blocks of it against the fp64-accumulated checker, the larger of the two" % (host_rel, n_blocks) if host_rel is not None else
+                                      "%d 64x64 blocks of the timed result against the fp64 checker" % n_blocks if n_blocks else "the whole timed result against the fp64-accumulated checker", rel, tol)}
     if cpu and not graph_of and not fused_gelu:
         rows = min(M, 1024)
         hd = np.zeros(M * N, np.uint16)
@@ -676,6 +716,13 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     go_a, go_w = ko.mk_global(aq, M, K, K, 1, ko.F8E4M3), ko.mk_global(wq, K, N, 1, K, ko.F8E4M3)
     n_blocks = 16
     rel = _blocks_frobenius(ko, got, go_a, go_w, M, N, K, ko.BF16, n_blocks, scales=(sa, sb))
+    whole = "%d %dx64 blocks of the timed result against the fp64-accumulated checker" % (n_blocks, min(M, 64))
+    if M >= 1024:   # the whole result as well, against the host GEMM
+        wrel, host_rel = _whole_frobenius(ko, got, go_a, go_w, M, N, K, ko.BF16, scales=(sa, sb))
+        if not host_rel <= FROB_TOL:
+            raise CheckFailed("f8 M=%d: the host GEMM itself is off the fp64 checker by %g" % (M, host_rel))
+        rel = max(rel, wrel)
+        whole = "the whole timed result against the host GEMM (fp64 sums of fp32 K blocks; itself %.1e off the fp64-accumulated checker on 16 blocks) and %s, the larger of the two" % (host_rel, whole)
     if not rel <= FROB_TOL:
         raise CheckFailed("f8 M=%d: relative Frobenius error %g" % (M, rel))
     wall, ev = _events(lambda i: kh.matmul_scaled_f8(ga, gws[i % sets], dsa.data_ptr(), dsb.data_ptr(), gd, workspace=ws), steps, warmup)
@@ -684,7 +731,7 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192%s" % (M, ", K split across workgroups (workspace given)" if workspace else ""), "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 160 and not workspace)) else "tn_kernel<F8M16, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8>",
            "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
-           "checked": True, "check": "%d %dx64 blocks against the fp64-accumulated checker: relative Frobenius error %.2e (tolerance %.0e)" % (n_blocks, min(M, 64), rel, FROB_TOL)}
+           "checked": True, "check": "%s: relative Frobenius error %.2e (tolerance %.0e)" % (whole, rel, FROB_TOL)}
     out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d%s" % (M, "_splitk" if workspace else "")) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
     if cpu:
         rows = min(M, 1024)
@@ -877,7 +924,7 @@ def main():
         main_res = table[args.workload](args.steps, args.warmup)
     except CheckFailed as e:
         sys.exit("bench.py: correctness gate failed, nothing timed: %s" % e)
-    others = []
+    others, other_names = [], []
     if not args.no_others:
         for name, fn in table.items():
             if name == args.workload or (name == "expr" and args.workload == "expr_compiled"):   # once compiled, the program no longer reaches the machine
@@ -885,6 +932,7 @@ def main():
             if name in [w.strip() for w in args.skip.split(",") if w.strip()]:
                 continue
             torch.cuda.empty_cache()
+            other_names.append(name)
             try:
                 r = fn(min(args.steps, 20), min(args.warmup, 10))
             except kh.KapyError as e:   # e.g. no runtime compiler on this machine for the compiled workloads
@@ -898,17 +946,33 @@ def main():
                 r["ms_per_step"] = round(r["ms_per_step"], 4)
                 r["kernel_ms"] = round(r["kernel_ms"], 4)
             others.append(r)
+    # every benchmark configuration in one compact block inside "config" (a key that records of this line keep), and the long
+    # tables first in the line, so that its end - what a truncated log keeps - holds the configurations and the headline
+    by_name = dict([(args.workload, main_res)] + [(n, r) for n, r in zip(other_names, others)])
+    configs = {}
+    for cfg, name in (("C1", "gemm_f16"), ("C2", "gelu"), ("C3a", "transpose"), ("C3b", "permute"), ("C4", "gemm_bf16"), ("C5_M16", "f8_m16"), ("C5_M4096", "f8_m4096")):
+        r = by_name.get(name)
+        if r is None:
+            continue
+        if "roofline" not in r:
+            configs[cfg] = {"checked": False, "error": r.get("error", "not run")}
+            continue
+        configs[cfg] = {"value": round(r["value"], 2), "unit": r["unit"], "kernel_ms": round(r["kernel_ms"], 4), "bound": r["roofline"]["bound"],
+                        "frac": r["roofline"]["frac"], "checked": r["checked"], "kernel": r["kernel"],
+                        "cpu_baseline": (r.get("cpu_baseline") or {}).get("value"), "cpu_unit": (r.get("cpu_baseline") or {}).get("unit")}
+    others.sort(key=lambda r: 0 if r.get("workload", "").startswith("device ceilings") else 1)
     line = {
+        "other_workloads": others,
         "metric": "GEMM TFLOP/s + % MFMA peak; elementwise/transpose GB/s + % HBM peak (1 GPU)",
         "value": round(main_res["value"], 2), "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(main_res["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic",
         "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "kernel_ms": round(main_res["kernel_ms"], 4),
                    "inputs": main_res["inputs"], "checked": main_res["checked"], "check": main_res["check"],
-                   "buffers": "4 rotating sets (1 GiB) so reads miss the Infinity Cache" if main_res["unit"] == "GB/s" else "single set"},
+                   "buffers": "4 rotating sets (1 GiB) so reads miss the Infinity Cache" if main_res["unit"] == "GB/s" else "single set",
+                   "configs": configs},
         "roofline": main_res["roofline"],
         "cpu_baseline": main_res.get("cpu_baseline"),
-        "other_workloads": others,
     }
     print(json.dumps(line))
 

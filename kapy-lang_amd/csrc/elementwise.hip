@@ -667,8 +667,10 @@ bool prog_padding_nonzero(const kapy_ew_inst *prog, int n_inst, int input) {
 // Postfix form of the program for the stack machine; false when the program does not fit it
 // (a tree deeper than three values, more than kMaxPost steps after unfolding shared values,
 // operands that are not full / row / column / scalar views readable 8 at a time, padding).
+// `folded`: the final value is folded by a reducing kernel instead of stored, so the rounding a store would perform
+// has to be a step of the program.
 bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins,
-                         const kapy_global *out, StackProgram *P) {
+                         const kapy_global *out, StackProgram *P, bool folded = false) {
   struct N {
     int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
     float imm = 0.f;
@@ -787,7 +789,7 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     case KAPY_EW_FPTOFP:
       emit(n.a, d);
       // values are fp32 images of typed values: widening to f32 changes nothing; and the store rounds to nearest itself
-      if (n.dtype != KAPY_F32 && !(id == stored && n.dtype == out->dtype && n.rmode != KAPY_RZ)) push(kCast, 0, n.dtype, n.rmode, d, 0.f);
+      if (n.dtype != KAPY_F32 && !(!folded && id == stored && n.dtype == out->dtype && n.rmode != KAPY_RZ)) push(kCast, 0, n.dtype, n.rmode, d, 0.f);
       return;
     case KAPY_EW_FMA: emit(n.a, d); emit(n.b, d + 1); emit(n.c, d + 2); push(KAPY_EW_FMA, 0, n.dtype, 0, d, 0.f); return;
     KAPY_EW_BINARY_CASES: {
@@ -941,7 +943,7 @@ int run_column_phases(const kapy_ew_inst *prog, int n_inst, const int *result_dt
       if (F.inst[k].op != KAPY_EW_ST_GLOBAL && F.inst[k].dst == F.inst[F.n - 1].a) operand_dtype = F.dtype[k];
     if (operand_dtype < 0) return give_up(0);
     pseudo.dtype = operand_dtype;
-    if (!build_stack_program(F.inst, F.n, F.dtype, all, n_ins + ph, &pseudo, &SP[ph]) || SP[ph].width) return give_up(0);
+    if (!build_stack_program(F.inst, F.n, F.dtype, all, n_ins + ph, &pseudo, &SP[ph], true) || SP[ph].width) return give_up(0);
   }
   for (int ph = 0; ph < n_reduce; ++ph) {
     const int sum = prog[C.stop[ph]].op == KAPY_EW_REDUCE_SUM;

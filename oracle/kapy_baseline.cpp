@@ -118,7 +118,8 @@ void gelu_rows_portable(const uint16_t *x, const uint16_t *bias, float scale, ui
 
 extern "C" {
 
-// result = cast(lhs . rhs [* row_scale[m] * col_scale[n]]), any operand element types and strides; fp32 accumulate.
+// result = cast(lhs . rhs [* row_scale[m] * col_scale[n]]), any operand element types and strides; fp32 accumulate over
+// K blocks of 512, the blocks summed in fp64 (so that the whole result can serve as a gate at benchmark sizes).
 // *multiply_seconds (if not null) gets the time of the multiplication proper: operands already widened to
 // fp32 and packed into panels (the GPU kernels are handed their operands in the layout they want, too),
 // result still fp32.
@@ -130,7 +131,7 @@ int ko_baseline_gemm(const ko_global *lhs, const ko_global *rhs, const float *ro
   const int64_t mp = (M + MR - 1) / MR, np = (N + NR - 1) / NR;
   float *ap = (float *)aligned_alloc(64, (size_t)mp * K * MR * sizeof(float));
   float *bp = (float *)aligned_alloc(64, (size_t)np * K * NR * sizeof(float));
-  float *c = (float *)aligned_alloc(64, (size_t)mp * MR * np * NR * sizeof(float));
+  double *c = (double *)aligned_alloc(64, (size_t)mp * MR * np * NR * sizeof(double));
   if (!ap || !bp || !c) {
     free(ap); free(bp); free(c);
     return -2;
@@ -158,17 +159,23 @@ int ko_baseline_gemm(const ko_global *lhs, const ko_global *rhs, const float *ro
     // a column panel of B (kc x 32 floats, 64 KiB) stays in a core's L2 while the row panels of A stream past it
 #pragma omp parallel for schedule(dynamic, 1)
     for (int64_t jp = 0; jp < np; ++jp)
-      for (int64_t ip = 0; ip < mp; ++ip)
-        micro(ap + (ip * K + k0) * MR, bp + (jp * K + k0) * NR, c + ip * MR * ldc + jp * NR, ldc, kc, k0 == 0);
+      for (int64_t ip = 0; ip < mp; ++ip) {
+        // one K block of an 8 x 32 tile in fp32 registers, the blocks summed in fp64
+        alignas(64) float t[MR * NR];
+        micro(ap + (ip * K + k0) * MR, bp + (jp * K + k0) * NR, t, NR, kc, true);
+        double *cc = c + ip * MR * ldc + jp * NR;
+        for (int i = 0; i < MR; ++i)
+          for (int j = 0; j < NR; ++j) cc[i * ldc + j] = (k0 == 0 ? 0.0 : cc[i * ldc + j]) + (double)t[i * NR + j];
+      }
   }
   const double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
   if (multiply_seconds) *multiply_seconds = dt;
 #pragma omp parallel for schedule(static)
   for (int64_t m = 0; m < M; ++m)
     for (int64_t n = 0; n < N; ++n) {
-      float v = c[m * ldc + n];
-      if (row_scale && col_scale) v *= row_scale[m] * col_scale[n];
-      ko_encode(result->ptr, result->dtype, elem(result, m, n), (double)v, KO_RN);
+      double v = c[m * ldc + n];
+      if (row_scale && col_scale) v *= (double)(row_scale[m] * col_scale[n]);   // the scale product in fp32, as the checker forms it
+      ko_encode(result->ptr, result->dtype, elem(result, m, n), v, KO_RN);
     }
   free(ap); free(bp); free(c);
   return 0;

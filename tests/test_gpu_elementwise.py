@@ -494,6 +494,27 @@ def test_column_reduces_with_broadcast_operands_special_values_and_views(ko):
     assert np.all(got == 0x8000) and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("narrow", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("m,n", [(256, 64), (4096, 512), (40, 64), (256, 65)])
+def test_a_down_cast_right_before_a_column_sum_is_rounded(ko, narrow, m, n):
+    """reduce_sum(fptofp(x, f32 -> 16 bit), axis 0): the sum adds the ROUNDED values, on the launches-per-reduce path (at least
+    64 rows, width a multiple of 8) and on the one-launch column machine alike.  Rows come in pairs +a + e, -a + e with a in
+    [0.5, 1) on the 16-bit grid and e below half a grid step: rounded, every column sums to exactly zero; unrounded, to m * e."""
+    rng = np.random.default_rng(7 + m + n)
+    step = 2.0 ** (-11 if narrow == kh.F16 else -8)
+    a = 0.5 + step * rng.integers(0, int(0.5 / step), size=(m // 2, n))
+    e = step / 8
+    xf = np.concatenate([a + e, -a + e]).astype(np.float32)
+    xf = xf[rng.permutation(m)]
+    assert np.all(np.abs(xf.astype(np.float64)) % step != 0)            # e survives in fp32
+    x = xf.view(np.uint32)
+    insts = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), dict(op=kh.EW_FPTOFP, dst=1, a=0, dtype=narrow, rmode=kh.RN),
+             dict(op=kh.EW_REDUCE_SUM, dst=2, a=1, b=0), dict(op=kh.EW_ST_GLOBAL, a=2)]
+    got, want = _run_prog(ko, insts, [x], [kh.F32], narrow, m, n)
+    assert np.array_equal(got, want)
+    assert not (got & 0x7FFF).any()              # +-0 everywhere: m * e (a 16-bit value of its own) would show
+
+
 def test_column_program_on_strided_views_and_f32(ko):
     # operand and result are windows of wider buffers; f32 throughout
     m, n, ld = 300, 90, 128

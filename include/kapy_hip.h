@@ -35,7 +35,8 @@ typedef enum kapy_status {
 /* Element types of Kapy tensors (include/kapy/Dialect/Kapy/IR/Types.td; f8 = OCP E4M3FN / E5M2). */
 typedef enum kapy_dtype {
   KAPY_F16 = 0, KAPY_BF16 = 1, KAPY_F32 = 2, KAPY_F8E4M3 = 3, KAPY_F8E5M2 = 4,
-  KAPY_I8 = 5, KAPY_I16 = 6, KAPY_I32 = 7
+  KAPY_I8 = 5, KAPY_I16 = 6, KAPY_I32 = 7,
+  KAPY_I1 = 8 /* the result type of cmpi / cmpf and the condition of select; one byte (0 or 1) in memory */
 } kapy_dtype;
 
 /* Enum values equal include/kapy/Dialect/Kapy/IR/Enums.td (python/src/ir.cc:125-156). */
@@ -255,7 +256,7 @@ int kapy_copy_batched(const kapy_global *src, const kapy_global *dst, const kapy
  * of one program must all run along the same axis. */
 typedef enum kapy_ew_op {
   KAPY_EW_LD_GLOBAL = 0, /* dst <- ins[a]            (c = kapy_padding_option)                  */
-  KAPY_EW_SPLAT,         /* dst <- imm as `dtype`    (kapy.splat)                               */
+  KAPY_EW_SPLAT,         /* dst <- imm as `dtype`    (kapy.splat); for an integer `dtype` the value is field a */
   KAPY_EW_FPTOFP,        /* dst <- cast(a) to `dtype`, `rmode` on down-casts (kapy.fptofp/extf/truncf) */
   KAPY_EW_ADDF, KAPY_EW_SUBF, KAPY_EW_MULF, KAPY_EW_DIVF,
   KAPY_EW_FMA,           /* dst <- a*b + c                                                     */
@@ -271,8 +272,36 @@ typedef enum kapy_ew_op {
   KAPY_EW_SIN, KAPY_EW_COS,    /* math.sin / math.cos (create_sin, create_cos; :1224-1225)                          */
   KAPY_EW_MAXNUMF, KAPY_EW_MINNUMF, /* arith.maxnumf / minnumf: a NaN operand is ignored (create_maxnumf, create_minnumf; :1201-1206) */
   KAPY_EW_REMF,          /* arith.remf: the remainder of a / b with the sign of a, exact (create_remf; :1192)   */
+  /* Integer, compare, select and conversion ops on tensors (BinaryOpConversion / UnaryOpConversion over arith ops,
+   * ElementwiseOpToLLVM.cpp:1178-1215; arith.select, SelectOpToLLVM.cpp:21-98; kapy.arange, ArangeOpToLLVM.cpp:22-50;
+   * builders create_addi ... create_select, python/src/ir.cc:730-1167).  Integer registers (i1, i8, i16, i32) are signless
+   * as in MLIR: the op names the signedness, results wrap to the register's width.  Where MLIR leaves a result undefined
+   * this library and its checker define it: x / 0 = 0 and x % 0 = 0, the most negative value divided by -1 wraps (its
+   * remainder is 0), a shift by the width or more gives 0 (shrsi: the sign), fptosi saturates and turns NaN into 0. */
+  KAPY_EW_ADDI, KAPY_EW_SUBI, KAPY_EW_MULI, KAPY_EW_DIVSI, KAPY_EW_DIVUI, KAPY_EW_FLOORDIVSI, KAPY_EW_CEILDIVSI, KAPY_EW_CEILDIVUI,
+  KAPY_EW_REMSI, KAPY_EW_REMUI, KAPY_EW_ANDI, KAPY_EW_ORI, KAPY_EW_XORI, KAPY_EW_SHLI, KAPY_EW_SHRSI, KAPY_EW_SHRUI,
+  KAPY_EW_MAXSI, KAPY_EW_MAXUI, KAPY_EW_MINSI, KAPY_EW_MINUI, /* dst <- a op b, both of one integer type            */
+  KAPY_EW_ABSI,          /* math.absi (create_absi)                                                              */
+  KAPY_EW_CMPI,          /* dst (i1) <- a <pred> b on integers, c = a kapy_cmpi_predicate; create_cmpi_*      */
+  KAPY_EW_CMPF,          /* dst (i1) <- a <pred> b on floats,   c = a kapy_cmpf_predicate; create_cmpf_*      */
+  KAPY_EW_SELECT,        /* dst <- a ? b : c, a an i1 register, b and c of one type (create_select)               */
+  KAPY_EW_TRUNCI, KAPY_EW_EXTSI, KAPY_EW_EXTUI, /* dst <- a as integer type `dtype` (create_intcast)             */
+  KAPY_EW_SITOFP,        /* dst <- the signed integer a as float type `dtype` (f16, bf16, f32), one RN rounding    */
+  KAPY_EW_FPTOSI,        /* dst <- the float a as integer type `dtype`, toward zero                               */
+  KAPY_EW_BITCAST,       /* dst <- the bits of a as type `dtype` of the same width (a NaN may come out quieted)     */
+  KAPY_EW_ARANGE,        /* dst (i32) <- a + the element's index along axis b: kapy.arange broadcast over the other axis */
   KAPY_EW_NUM_OPS
 } kapy_ew_op;
+/* arith.cmpi / arith.cmpf predicates, numbered as in MLIR's ArithBase.td (what create_cmpi_* / create_cmpf_* pass). */
+typedef enum kapy_cmpi_predicate {
+  KAPY_CMPI_EQ = 0, KAPY_CMPI_NE = 1, KAPY_CMPI_SLT = 2, KAPY_CMPI_SLE = 3, KAPY_CMPI_SGT = 4, KAPY_CMPI_SGE = 5,
+  KAPY_CMPI_ULT = 6, KAPY_CMPI_ULE = 7, KAPY_CMPI_UGT = 8, KAPY_CMPI_UGE = 9
+} kapy_cmpi_predicate;
+typedef enum kapy_cmpf_predicate {
+  KAPY_CMPF_FALSE = 0, KAPY_CMPF_OEQ = 1, KAPY_CMPF_OGT = 2, KAPY_CMPF_OGE = 3, KAPY_CMPF_OLT = 4, KAPY_CMPF_OLE = 5, KAPY_CMPF_ONE = 6,
+  KAPY_CMPF_ORD = 7, KAPY_CMPF_UEQ = 8, KAPY_CMPF_UGT = 9, KAPY_CMPF_UGE = 10, KAPY_CMPF_ULT = 11, KAPY_CMPF_ULE = 12, KAPY_CMPF_UNE = 13,
+  KAPY_CMPF_UNO = 14, KAPY_CMPF_TRUE = 15
+} kapy_cmpf_predicate;
 typedef struct kapy_ew_inst {
   int32_t op, dst, a, b, c;
   int32_t dtype, rmode;

@@ -1,9 +1,10 @@
 // kapy_hip.hpp — the host side of the hot path in C++, above the C ABI of kapy_hip.h.
 //
 // kapy::OpBuilder mirrors the part of the reference's KapyOpBuilder that the hot path uses
-// (python/src/ir.cc:744-1181: create_mk_global, create_sv_global, create_ld_global, create_st_global,
-// create_splat, create_broadcast, create_transpose, create_fptofp / extf / truncf, the arith and math
-// builders, create_reduce, create_matmul), with the same names and argument meaning.  Where the reference
+// (python/src/ir.cc:730-1181: create_mk_global, create_sv_global, create_ld_global, create_st_global,
+// create_splat, create_broadcast, create_transpose, create_arange, create_fptofp / extf / truncf / bitcast / sitofp /
+// fptosi / intcast, the float and integer arith builders, the create_cmpi_* / create_cmpf_* families, create_select,
+// the math builders, create_reduce, create_matmul), with the same names and argument meaning.  Where the reference
 // appends an op to a function that is compiled later, this builder records the op in a dataflow graph;
 // create_st_global - the op with the side effect - lowers the graph under its source to ONE library call:
 //   a load (optionally transposed) stored back            -> kapy_copy
@@ -136,6 +137,29 @@ class OpBuilder {
     n.imm = source;
     return push(n);
   }
+  // an integer splat (the reference splats a create_constant_int* scalar): the value wraps to the type's width
+  Value create_splat(int32_t source, kapy_dtype element_type) {
+    if (element_type <= KAPY_F8E5M2) return create_splat((float)source, element_type);
+    Node n;
+    n.kind = Node::kOp;
+    n.op = KAPY_EW_SPLAT;
+    n.dtype = element_type;
+    n.ival = source;
+    return push(n);
+  }
+  // kapy.arange (ir.cc:730-743): i32 values start, start + 1, ... along `axis`, shape [end - start, 1] or [1, end - start];
+  // inside a program it is the element's index along that axis plus start, broadcast over the other axis
+  Value create_arange(unsigned axis, int32_t start, int32_t end) {
+    if (axis > 1) throw Error(KAPY_ERR_INVALID, "program axis must be 0, 1");
+    if (end <= start) throw Error(KAPY_ERR_VERIFY, "arange: end must be greater than start");
+    Node n;
+    n.kind = Node::kOp;
+    n.op = KAPY_EW_ARANGE;
+    n.dtype = KAPY_I32;
+    n.ival = start;
+    n.axis = (int)axis;
+    return push(n);
+  }
   // kapy.broadcast: extents of 1 stretch to the result's.  A load of a [1 x n] or [m x 1] view already is one; the
   // requested shape is checked when the program is verified against its result.
   Value create_broadcast(Value source, const std::vector<int64_t> & /*shape*/) {
@@ -158,7 +182,70 @@ class OpBuilder {
   Value create_extf(Value source, kapy_dtype element_type) { return create_fptofp(source, element_type, KAPY_RN); }
   Value create_truncf(Value source, kapy_dtype element_type) { return create_fptofp(source, element_type, KAPY_RN); }
 
+  // (ir.cc:755-790) arith.bitcast, sitofp, fptosi; create_intcast picks bitcast / trunci / extsi / extui from the widths
+  Value create_bitcast(Value source, kapy_dtype element_type) { return unary(KAPY_EW_BITCAST, source, element_type); }
+  Value create_sitofp(Value source, kapy_dtype element_type) { return unary(KAPY_EW_SITOFP, source, element_type); }
+  Value create_fptosi(Value source, kapy_dtype element_type) { return unary(KAPY_EW_FPTOSI, source, element_type); }
+  Value create_intcast(Value source, kapy_dtype element_type, bool is_signed) {
+    const int from = bits_of(node(source).dtype), to = bits_of(element_type);
+    if (from == to) return create_bitcast(source, element_type);
+    if (from > to) return unary(KAPY_EW_TRUNCI, source, element_type);
+    return unary(is_signed ? KAPY_EW_EXTSI : KAPY_EW_EXTUI, source, element_type);
+  }
+
   // ---- arith / math (ir.cc:791-1157) ---------------------------------------------------------------------
+  Value create_muli(Value lhs, Value rhs) { return binary(KAPY_EW_MULI, lhs, rhs); }
+  Value create_divsi(Value lhs, Value rhs) { return binary(KAPY_EW_DIVSI, lhs, rhs); }
+  Value create_divui(Value lhs, Value rhs) { return binary(KAPY_EW_DIVUI, lhs, rhs); }
+  Value create_remsi(Value lhs, Value rhs) { return binary(KAPY_EW_REMSI, lhs, rhs); }
+  Value create_remui(Value lhs, Value rhs) { return binary(KAPY_EW_REMUI, lhs, rhs); }
+  Value create_addi(Value lhs, Value rhs) { return binary(KAPY_EW_ADDI, lhs, rhs); }
+  Value create_subi(Value lhs, Value rhs) { return binary(KAPY_EW_SUBI, lhs, rhs); }
+  Value create_shli(Value lhs, Value rhs) { return binary(KAPY_EW_SHLI, lhs, rhs); }
+  Value create_shrui(Value lhs, Value rhs) { return binary(KAPY_EW_SHRUI, lhs, rhs); }
+  Value create_shrsi(Value lhs, Value rhs) { return binary(KAPY_EW_SHRSI, lhs, rhs); }
+  Value create_minsi(Value lhs, Value rhs) { return binary(KAPY_EW_MINSI, lhs, rhs); }
+  Value create_minui(Value lhs, Value rhs) { return binary(KAPY_EW_MINUI, lhs, rhs); }
+  Value create_maxsi(Value lhs, Value rhs) { return binary(KAPY_EW_MAXSI, lhs, rhs); }
+  Value create_maxui(Value lhs, Value rhs) { return binary(KAPY_EW_MAXUI, lhs, rhs); }
+  Value create_andi(Value lhs, Value rhs) { return binary(KAPY_EW_ANDI, lhs, rhs); }
+  Value create_ori(Value lhs, Value rhs) { return binary(KAPY_EW_ORI, lhs, rhs); }
+  Value create_xori(Value lhs, Value rhs) { return binary(KAPY_EW_XORI, lhs, rhs); }
+  Value create_absi(Value source) { return unary(KAPY_EW_ABSI, source); }
+  // arith.cmpi / arith.cmpf (ir.cc:891-1000): an i1 tensor
+  Value create_cmpi_sle(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_SLE, lhs, rhs); }
+  Value create_cmpi_slt(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_SLT, lhs, rhs); }
+  Value create_cmpi_sge(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_SGE, lhs, rhs); }
+  Value create_cmpi_sgt(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_SGT, lhs, rhs); }
+  Value create_cmpi_ule(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_ULE, lhs, rhs); }
+  Value create_cmpi_ult(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_ULT, lhs, rhs); }
+  Value create_cmpi_uge(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_UGE, lhs, rhs); }
+  Value create_cmpi_ugt(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_UGT, lhs, rhs); }
+  Value create_cmpi_eq(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_EQ, lhs, rhs); }
+  Value create_cmpi_ne(Value lhs, Value rhs) { return compare(KAPY_EW_CMPI, KAPY_CMPI_NE, lhs, rhs); }
+  Value create_cmpf_olt(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_OLT, lhs, rhs); }
+  Value create_cmpf_ogt(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_OGT, lhs, rhs); }
+  Value create_cmpf_ole(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_OLE, lhs, rhs); }
+  Value create_cmpf_oge(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_OGE, lhs, rhs); }
+  Value create_cmpf_oeq(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_OEQ, lhs, rhs); }
+  Value create_cmpf_one(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_ONE, lhs, rhs); }
+  Value create_cmpf_ult(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_ULT, lhs, rhs); }
+  Value create_cmpf_ugt(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_UGT, lhs, rhs); }
+  Value create_cmpf_ule(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_ULE, lhs, rhs); }
+  Value create_cmpf_uge(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_UGE, lhs, rhs); }
+  Value create_cmpf_ueq(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_UEQ, lhs, rhs); }
+  Value create_cmpf_une(Value lhs, Value rhs) { return compare(KAPY_EW_CMPF, KAPY_CMPF_UNE, lhs, rhs); }
+  // arith.select on tensors (ir.cc:1162-1167; SelectOpToLLVM.cpp:21-98): condition an i1 tensor
+  Value create_select(Value condition, Value true_value, Value false_value) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = KAPY_EW_SELECT;
+    n.a = tensor(condition, "select");
+    n.b = tensor(true_value, "select");
+    n.c = tensor(false_value, "select");
+    n.dtype = node(true_value).dtype;
+    return push(n);
+  }
   Value create_addf(Value lhs, Value rhs) { return binary(KAPY_EW_ADDF, lhs, rhs); }
   Value create_subf(Value lhs, Value rhs) { return binary(KAPY_EW_SUBF, lhs, rhs); }
   Value create_mulf(Value lhs, Value rhs) { return binary(KAPY_EW_MULF, lhs, rhs); }
@@ -237,6 +324,7 @@ class OpBuilder {
     int padding = KAPY_PAD_ZERO, cache = KAPY_CACHE_NONE, evict = KAPY_EVICT_NORMAL, impl_way = KAPY_MATMUL_AUTO;
     bool transposed = false, is_volatile = false;
     float imm = 0.f;
+    int ival = 0, pred = 0;  // an integer splat's value or arange's start; a compare's predicate
   };
   std::vector<Node> nodes_;
   void *stream_;
@@ -267,6 +355,24 @@ class OpBuilder {
     n.a = tensor(source, "elementwise");
     n.dtype = dtype >= 0 ? dtype : node(source).dtype;
     n.rmode = rmode;
+    return push(n);
+  }
+  static int bits_of(int dtype) {
+    switch (dtype) {
+    case KAPY_I1: return 1;
+    case KAPY_F8E4M3: case KAPY_F8E5M2: case KAPY_I8: return 8;
+    case KAPY_F16: case KAPY_BF16: case KAPY_I16: return 16;
+    default: return 32;
+    }
+  }
+  Value compare(int op, int predicate, Value lhs, Value rhs) {
+    Node n;
+    n.kind = Node::kOp;
+    n.op = op;
+    n.a = tensor(lhs, "compare");
+    n.b = tensor(rhs, "compare");
+    n.pred = predicate;
+    n.dtype = KAPY_I1;
     return push(n);
   }
   Value binary(int op, Value lhs, Value rhs) {
@@ -341,6 +447,9 @@ class OpBuilder {
         I.b = n.b >= 0 ? reg[n.b] : 0;
         I.c = n.c >= 0 ? reg[n.c] : 0;
         if (n.op == KAPY_EW_REDUCE_SUM || n.op == KAPY_EW_REDUCE_MAX) I.b = n.axis;
+        if (n.op == KAPY_EW_CMPI || n.op == KAPY_EW_CMPF) I.c = n.pred;
+        if (n.op == KAPY_EW_ARANGE) { I.a = n.ival; I.b = n.axis; }
+        if (n.op == KAPY_EW_SPLAT && n.dtype >= KAPY_I8) I.a = n.ival;
         release(n.a);
         release(n.b);
         release(n.c);

@@ -11,7 +11,10 @@
 // the case labels of every op with two register operands
 #define KAPY_EW_BINARY_CASES                                                                                                          \
   case KAPY_EW_ADDF: case KAPY_EW_SUBF: case KAPY_EW_MULF: case KAPY_EW_DIVF: case KAPY_EW_MAXIMUMF: case KAPY_EW_MINIMUMF: case KAPY_EW_MAXNUMF:  \
-  case KAPY_EW_MINNUMF: case KAPY_EW_REMF
+  case KAPY_EW_MINNUMF: case KAPY_EW_REMF: case KAPY_EW_ADDI: case KAPY_EW_SUBI: case KAPY_EW_MULI: case KAPY_EW_DIVSI: case KAPY_EW_DIVUI:                 \
+  case KAPY_EW_FLOORDIVSI: case KAPY_EW_CEILDIVSI: case KAPY_EW_CEILDIVUI: case KAPY_EW_REMSI: case KAPY_EW_REMUI: case KAPY_EW_ANDI: case KAPY_EW_ORI:      \
+  case KAPY_EW_XORI: case KAPY_EW_SHLI: case KAPY_EW_SHRSI: case KAPY_EW_SHRUI: case KAPY_EW_MAXSI: case KAPY_EW_MAXUI: case KAPY_EW_MINSI:               \
+  case KAPY_EW_MINUI: case KAPY_EW_CMPI: case KAPY_EW_CMPF
 
 namespace kapy {
 
@@ -30,15 +33,16 @@ inline int dtype_bytes(int32_t dtype) {
   switch (dtype) {
   case KAPY_F16: case KAPY_BF16: case KAPY_I16: return 2;
   case KAPY_F32: case KAPY_I32: return 4;
-  case KAPY_F8E4M3: case KAPY_F8E5M2: case KAPY_I8: return 1;
+  case KAPY_F8E4M3: case KAPY_F8E5M2: case KAPY_I8: case KAPY_I1: return 1;
   }
   return 0;
 }
 inline bool is_float(int32_t d) { return d == KAPY_F16 || d == KAPY_BF16 || d == KAPY_F32 || d == KAPY_F8E4M3 || d == KAPY_F8E5M2; }
 inline bool is_f8(int32_t d) { return d == KAPY_F8E4M3 || d == KAPY_F8E5M2; }
+inline bool is_int(int32_t d) { return d == KAPY_I8 || d == KAPY_I16 || d == KAPY_I32 || d == KAPY_I1; }
 inline const char *dtype_name(int32_t d) {
-  static const char *names[] = {"f16", "bf16", "f32", "f8E4M3", "f8E5M2", "i8", "i16", "i32"};
-  return d >= 0 && d < 8 ? names[d] : "?";
+  static const char *names[] = {"f16", "bf16", "f32", "f8E4M3", "f8E5M2", "i8", "i16", "i32", "i1"};
+  return d >= 0 && d < 9 ? names[d] : "?";
 }
 
 inline int64_t extent0(const kapy_global *g) { return int64_t(g->end0) - g->start0; }

@@ -61,7 +61,6 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
   for (int k = 0; k < P.n_inst; ++k) {
     const kapy_ew_inst I = P.inst[k];
     float r = 0.f;
-    const int dt = I.dtype;
     switch (I.op) {
     case KAPY_EW_LD_GLOBAL: {
       const DevView &g = P.in[I.a];
@@ -73,32 +72,10 @@ __global__ __launch_bounds__(256) void interpreter_kernel(Program P, int j_faste
       }
       break;
     }
-    case KAPY_EW_SPLAT:
-      r = round_to_dtype(I.imm, dt, true);
-      break;
-    case KAPY_EW_FPTOFP:
-      r = round_to_dtype(regs[I.a][tid], dt, I.rmode != KAPY_RZ);
-      break;
     case KAPY_EW_ST_GLOBAL:
       if (active) store_from_f32((void *)P.out.base, P.out.dtype, i * P.out.stride0 + j * P.out.stride1, regs[I.a][tid]);
       continue;
-    default: {
-      const float a = regs[I.a][tid];
-      switch (I.op) {
-      case KAPY_EW_ADDF: r = __fadd_rn(a, regs[I.b][tid]); break;
-      case KAPY_EW_SUBF: r = __fsub_rn(a, regs[I.b][tid]); break;
-      case KAPY_EW_MULF: r = __fmul_rn(a, regs[I.b][tid]); break;
-      case KAPY_EW_DIVF: r = __fdiv_rn(a, regs[I.b][tid]); break;
-      case KAPY_EW_FMA: r = fma_typed(a, regs[I.b][tid], regs[I.c][tid], dt); break;
-      case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
-      case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
-      case KAPY_EW_MAXNUMF: r = max_num(a, regs[I.b][tid]); break;
-      case KAPY_EW_MINNUMF: r = min_num(a, regs[I.b][tid]); break;
-      case KAPY_EW_REMF: r = rem_f(a, regs[I.b][tid]); break;
-      default: r = apply_unary(I.op, a);
-      }
-      if (dt != KAPY_F32) r = round_to_dtype(r, dt, true);
-    }
+    default: r = machine_step<256>(I, &regs[0][tid], i, j);
     }
     regs[I.dst][tid] = r;  // regs[*][tid] is private to the lane: no barrier needed
   }
@@ -137,7 +114,6 @@ __global__ __launch_bounds__(WAVES * 64) void column_program_kernel(Program P, C
         if (!((need >> k) & 1)) continue;
         const kapy_ew_inst I = P.inst[k];
         float r = 0.f;
-        const int dt = I.dtype;
         switch (I.op) {
         case KAPY_EW_LD_GLOBAL: {
           const DevView &g = P.in[I.a];
@@ -149,29 +125,11 @@ __global__ __launch_bounds__(WAVES * 64) void column_program_kernel(Program P, C
           }
           break;
         }
-        case KAPY_EW_SPLAT: r = round_to_dtype(I.imm, dt, true); break;
-        case KAPY_EW_FPTOFP: r = round_to_dtype(regs[I.a][tid], dt, I.rmode != KAPY_RZ); break;
         case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX: r = red[I.c][lane]; break;  // I.c: which reduce this is (set by the host)
         case KAPY_EW_ST_GLOBAL:
           if (in_strip) store_from_f32((void *)P.out.base, P.out.dtype, i * P.out.stride0 + j * P.out.stride1, regs[I.a][tid]);
           continue;
-        default: {
-          const float a = regs[I.a][tid];
-          switch (I.op) {
-          case KAPY_EW_ADDF: r = __fadd_rn(a, regs[I.b][tid]); break;
-          case KAPY_EW_SUBF: r = __fsub_rn(a, regs[I.b][tid]); break;
-          case KAPY_EW_MULF: r = __fmul_rn(a, regs[I.b][tid]); break;
-          case KAPY_EW_DIVF: r = __fdiv_rn(a, regs[I.b][tid]); break;
-          case KAPY_EW_FMA: r = fma_typed(a, regs[I.b][tid], regs[I.c][tid], dt); break;
-          case KAPY_EW_MAXIMUMF: r = max_nan(a, regs[I.b][tid]); break;
-          case KAPY_EW_MINIMUMF: r = min_nan(a, regs[I.b][tid]); break;
-          case KAPY_EW_MAXNUMF: r = max_num(a, regs[I.b][tid]); break;
-          case KAPY_EW_MINNUMF: r = min_num(a, regs[I.b][tid]); break;
-          case KAPY_EW_REMF: r = rem_f(a, regs[I.b][tid]); break;
-          default: r = apply_unary(I.op, a);
-          }
-          if (dt != KAPY_F32) r = round_to_dtype(r, dt, true);
-        }
+        default: r = machine_step<WAVES * 64>(I, &regs[0][tid], i, j);
         }
         regs[I.dst][tid] = r;  // regs[*][tid] is private to the lane
       }
@@ -477,10 +435,38 @@ int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *cons
       break;
     }
     case KAPY_EW_SPLAT:
-      if (I.dtype != KAPY_F16 && I.dtype != KAPY_BF16 && I.dtype != KAPY_F32)
-        return fail(KAPY_ERR_VERIFY, "splat: only f16, bf16 and f32 splats are supported");
+      if (I.dtype != KAPY_F16 && I.dtype != KAPY_BF16 && I.dtype != KAPY_F32 && !is_int(I.dtype))
+        return fail(KAPY_ERR_VERIFY, "splat: only f16, bf16, f32 and integer splats are supported");
       reg_dtype[I.dst] = I.dtype;
       break;
+    case KAPY_EW_ARANGE:
+      if (I.b != 0 && I.b != 1) return fail(KAPY_ERR_VERIFY, "arange: axis must be 0 or 1");
+      reg_dtype[I.dst] = KAPY_I32;
+      break;
+    case KAPY_EW_SELECT:
+      if (!reg_ok(I.a) || !reg_ok(I.b) || !reg_ok(I.c)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      if (reg_dtype[I.a] != KAPY_I1) return fail(KAPY_ERR_VERIFY, "select: condition must have i1 element type");
+      if (reg_dtype[I.b] != reg_dtype[I.c]) return fail(KAPY_ERR_VERIFY, "select: true and false values must have the same element type");
+      reg_dtype[I.dst] = reg_dtype[I.b];
+      break;
+    case KAPY_EW_TRUNCI: case KAPY_EW_EXTSI: case KAPY_EW_EXTUI: case KAPY_EW_SITOFP: case KAPY_EW_FPTOSI: case KAPY_EW_BITCAST: {
+      if (!reg_ok(I.a)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      const int sd = reg_dtype[I.a], dd = I.dtype;
+      auto bits = [](int d) { return d == KAPY_I1 ? 1 : 8 * dtype_bytes(d); };
+      const bool arith_float_s = sd == KAPY_F16 || sd == KAPY_BF16 || sd == KAPY_F32, arith_float_d = dd == KAPY_F16 || dd == KAPY_BF16 || dd == KAPY_F32;
+      if (!dtype_bytes(dd)) return fail(KAPY_ERR_INVALID, "elementwise: unknown element type %d at %d", dd, k);
+      if (I.op == KAPY_EW_TRUNCI && !(is_int(sd) && is_int(dd) && bits(dd) < bits(sd)))
+        return fail(KAPY_ERR_VERIFY, "trunci: operand and result must be integers, the result narrower");
+      if ((I.op == KAPY_EW_EXTSI || I.op == KAPY_EW_EXTUI) && !(is_int(sd) && is_int(dd) && bits(dd) > bits(sd)))
+        return fail(KAPY_ERR_VERIFY, "extsi / extui: operand and result must be integers, the result wider");
+      if (I.op == KAPY_EW_SITOFP && !(is_int(sd) && arith_float_d)) return fail(KAPY_ERR_VERIFY, "sitofp: an integer operand and an f16, bf16 or f32 result are required");
+      if (I.op == KAPY_EW_FPTOSI && !(arith_float_s && is_int(dd) && dd != KAPY_I1)) return fail(KAPY_ERR_VERIFY, "fptosi: an f16, bf16 or f32 operand and an i8, i16 or i32 result are required");
+      if (I.op == KAPY_EW_BITCAST && (sd == KAPY_I1 || dd == KAPY_I1 || dtype_bytes(sd) != dtype_bytes(dd)))
+        return fail(KAPY_ERR_VERIFY, "bitcast: operand and result must have the same bit width");
+      if (normalised) normalised[k].rmode = sd;   // the machines read the operand's type here
+      reg_dtype[I.dst] = dd;
+      break;
+    }
     case KAPY_EW_FPTOFP: {
       if (!reg_ok(I.a)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
       int sd = reg_dtype[I.a], dd = I.dtype;
@@ -500,10 +486,23 @@ int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *cons
         return fail(KAPY_ERR_VERIFY, "elementwise: operands must have the same element type at %d", k);
       reg_dtype[I.dst] = reg_dtype[I.a];
       break;
-    KAPY_EW_BINARY_CASES:
+    KAPY_EW_BINARY_CASES: {
       if (!reg_ok(I.a) || !reg_ok(I.b)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
       if (reg_dtype[I.a] != reg_dtype[I.b])
         return fail(KAPY_ERR_VERIFY, "elementwise: operands must have the same element type at %d", k);
+      const bool on_ints = (I.op >= KAPY_EW_ADDI && I.op <= KAPY_EW_MINUI) || I.op == KAPY_EW_CMPI;
+      if (on_ints && !is_int(reg_dtype[I.a])) return fail(KAPY_ERR_VERIFY, "elementwise: integer op on non-integer operands at %d", k);
+      if (I.op == KAPY_EW_CMPI && (I.c < 0 || I.c > KAPY_CMPI_UGE)) return fail(KAPY_ERR_INVALID, "cmpi: unknown predicate %d", I.c);
+      if (I.op == KAPY_EW_CMPF && (I.c < 0 || I.c > KAPY_CMPF_TRUE)) return fail(KAPY_ERR_INVALID, "cmpf: unknown predicate %d", I.c);
+      if (I.op == KAPY_EW_CMPF && reg_dtype[I.a] != KAPY_F16 && reg_dtype[I.a] != KAPY_BF16 && reg_dtype[I.a] != KAPY_F32)
+        return fail(KAPY_ERR_VERIFY, "cmpf: operands must be f16, bf16 or f32");
+      if (normalised && (I.op == KAPY_EW_CMPI || I.op == KAPY_EW_CMPF)) normalised[k].rmode = reg_dtype[I.a];
+      reg_dtype[I.dst] = (I.op == KAPY_EW_CMPI || I.op == KAPY_EW_CMPF) ? (int)KAPY_I1 : reg_dtype[I.a];
+      break;
+    }
+    case KAPY_EW_ABSI:
+      if (!reg_ok(I.a)) return fail(KAPY_ERR_INVALID, "elementwise: use of undefined register at %d", k);
+      if (!is_int(reg_dtype[I.a])) return fail(KAPY_ERR_VERIFY, "absi: operand must be an integer");
       reg_dtype[I.dst] = reg_dtype[I.a];
       break;
     case KAPY_EW_ST_GLOBAL:
@@ -521,7 +520,8 @@ int verify_program(const kapy_ew_inst *prog, int n_inst, const kapy_global *cons
       reg_dtype[I.dst] = reg_dtype[I.a];
     }
     if (result_dtype) result_dtype[k] = I.op == KAPY_EW_ST_GLOBAL ? out->dtype : reg_dtype[I.dst];
-    if (I.op != KAPY_EW_ST_GLOBAL && I.op != KAPY_EW_LD_GLOBAL && I.op != KAPY_EW_FPTOFP) {
+    const bool typed_above = (I.op >= KAPY_EW_ADDI && I.op < KAPY_EW_NUM_OPS) || I.op == KAPY_EW_SPLAT;   // (each checked its own types)
+    if (I.op != KAPY_EW_ST_GLOBAL && I.op != KAPY_EW_LD_GLOBAL && I.op != KAPY_EW_FPTOFP && !typed_above) {
       int d = reg_dtype[I.dst];
       if (d != KAPY_F16 && d != KAPY_BF16 && d != KAPY_F32)
         return fail(KAPY_ERR_VERIFY, "elementwise: arithmetic needs f16, bf16 or f32 operands at %d", k);
@@ -675,6 +675,8 @@ bool build_stack_program(const kapy_ew_inst *prog, int n_inst, const int *result
     int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
     float imm = 0.f;
   };
+  for (int k = 0; k < n_inst; ++k)
+    if (prog[k].op >= KAPY_EW_ADDI || is_int(result_dtype[k])) return false;  // integer registers: the register machines' business
   std::vector<N> nodes;
   int reg[kMaxRegs];
   for (int r = 0; r < kMaxRegs; ++r) reg[r] = -1;
@@ -977,8 +979,8 @@ int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
     I.dtype = result_dtype[k];
     uint64_t d = uint64_t(1) << k;
     switch (I.op) {
-    case KAPY_EW_LD_GLOBAL: case KAPY_EW_SPLAT: break;
-    case KAPY_EW_FMA: d |= def_of[I.a] | def_of[I.b] | def_of[I.c]; break;
+    case KAPY_EW_LD_GLOBAL: case KAPY_EW_SPLAT: case KAPY_EW_ARANGE: break;
+    case KAPY_EW_FMA: case KAPY_EW_SELECT: d |= def_of[I.a] | def_of[I.b] | def_of[I.c]; break;
     KAPY_EW_BINARY_CASES:
       d |= def_of[I.a] | def_of[I.b];
       break;
@@ -1048,11 +1050,19 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 
   bool has_reduce = false;
   for (int k = 0; k < n_inst; ++k) has_reduce |= prog[k].op == KAPY_EW_REDUCE_SUM || prog[k].op == KAPY_EW_REDUCE_MAX;
+  // Integer registers and the ops on them (compare, select, casts, arange) run on the register machines and in compiled
+  // kernels; the hand-written float kernels and the stack machines are not tried for such a program.  A program with an
+  // arange depends on where an element sits, so it is never re-shaped (transposed problem, one-line form) either.
+  bool has_int = is_int(out->dtype), has_arange = false;
+  for (int k = 0; k < n_inst; ++k) {
+    has_int |= prog[k].op >= KAPY_EW_ADDI || is_int(result_dtype[k]);
+    has_arange |= prog[k].op == KAPY_EW_ARANGE;
+  }
 
   // A column-major result: the same program on the transposed problem has a row-major one (every view with its axes
   // swapped - a row operand becomes a column operand and the other way round), which is what the fast kernels are written for.
   // Operands that are column-major too then read along their rows; the others are no worse off than before.
-  if (!has_reduce && out->stride0 == 1 && out->stride1 != 1 && o1 > 1 && n_ins <= kMaxInputs) {
+  if (!has_reduce && !has_arange && out->stride0 == 1 && out->stride1 != 1 && o1 > 1 && n_ins <= kMaxInputs) {
     auto swapped = [](const kapy_global *g) {
       kapy_global v = *g;
       std::swap(v.start0, v.start1);
@@ -1073,7 +1083,7 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
   // vector per row, and then only from aligned rows).  When the result and every operand are dense matrices of one shape
   // (pitch = width) or single elements, the program does not care where a row ends: it runs once over the first
   // 8 * floor(o0 * o1 / 8) elements as one line, in whole vectors, and once over the up to 7 that remain.
-  if (!has_reduce && o0 > 1 && o1 % 8 != 0 && o0 * o1 < (int64_t(1) << 31) - 1024 && n_ins <= kMaxInputs) {
+  if (!has_reduce && !has_arange && o0 > 1 && o1 % 8 != 0 && o0 * o1 < (int64_t(1) << 31) - 1024 && n_ins <= kMaxInputs) {
     auto dense = [&](const kapy_global *g) { return g->stride1 == 1 && g->stride0 == o1 && extent0(g) == o0 && extent1(g) == o1; };
     auto single = [](const kapy_global *g) { return extent0(g) == 1 && extent1(g) == 1; };
     bool flat = dense(out);
@@ -1114,7 +1124,8 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
     if (along[0] && along[1])
       return fail(KAPY_ERR_UNSUPPORTED, "elementwise: the reduces of one program must run along the same axis (reduce the other axis with kapy_reduce first)");
     if (along[0]) return run_column_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
-    rc = run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
+    rc = has_int ? fail(KAPY_ERR_UNSUPPORTED, "elementwise: a program with a reduce along rows and integer registers runs as a compiled kernel only")
+                 : run_row_program(prog, n_inst, result_dtype, ins, n_ins, out, s);
     if (rc != KAPY_ERR_UNSUPPORTED) return rc;
     // What the row machine refuses (a width that is not a multiple of 8, more than three row values in flight) a compiled
     // kernel may still serve: compile one now rather than turn the caller away.  Without the runtime compiler, or for a
@@ -1130,7 +1141,7 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
 
   AffineActParams ap;
   int T = -1;
-  if (match_affine_act(prog, n_inst, ins, out, &ap, &T)) {
+  if (!has_int && match_affine_act(prog, n_inst, ins, out, &ap, &T)) {
     uint32_t slots = (uint32_t)ap.rows * (uint32_t)ap.vec_per_row;
     const bool cols = (ap.bias_mode == kBiasRow || ap.bias_mode == kNoBias) && (ap.rows + 2 - 1) / 2 <= 65535;
     dim3 grid = cols ? dim3((ap.vec_per_row + 255) / 256, (ap.rows + 2 - 1) / 2)
@@ -1168,7 +1179,7 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
     if (rc != 0) return rc < 0 ? rc : KAPY_OK;
   }
 
-  {
+  if (!has_int) {
     StackProgram SP;
     memset(&SP, 0, sizeof SP);
     if (build_stack_program(prog, n_inst, result_dtype, ins, n_ins, out, &SP)) {

@@ -54,7 +54,7 @@ struct JitArgs {
 // The ragged end of a row: only the first `valid` (1..7) elements of vector jv exist; a whole-vector access would reach
 // past the view (and possibly past its allocation), so they move one by one.
 __device__ __forceinline__ Raw8 fetch8_partial(const StackIn &g, int32_t i, int32_t jv, int valid) {
-  const int eb = g.dtype == KAPY_F32 ? 4 : (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16) ? 2 : 1;
+  const int eb = dtype_elem_bytes(g.dtype);
   const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * eb;
   Raw8 r;
   r.lo = r.hi = u32x4{0, 0, 0, 0};
@@ -226,6 +226,7 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
       sig->rowwise = true;
     }
     if (op == KAPY_EW_LD_GLOBAL && prog[k].c != KAPY_PAD_ZERO) return false;
+    if (op == KAPY_EW_ARANGE && out->stride1 != 1) return false;  // (an arange names its axis: no transposed view of it)
     stores += op == KAPY_EW_ST_GLOBAL;
   }
   if (stores != 1) return false;
@@ -233,7 +234,7 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
   if (sig->rowwise && out->stride1 != 1) return false;  // (a reduce names its axis: no transposed view of it)
   const int64_t o0 = vo->e0, o1 = vo->e1;
   const int ob = dtype_bytes(out->dtype);
-  if (!is_float(out->dtype) || vo->s1 != 1) return false;
+  if (!(is_float(out->dtype) || is_int(out->dtype)) || vo->s1 != 1) return false;
   if (((uintptr_t)vo->base % (8 * ob)) || (vo->s0 * ob) % (8 * ob)) return false;
   if (o0 * ((o1 + 7) / 8) >= (int64_t(1) << 31) - 1024) return false;
   sig->ragged = o1 % 8 != 0;
@@ -246,11 +247,11 @@ bool classify(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, con
   sig->n_ins = n_ins;
   sig->out_dtype = out->dtype;
   sig->narrow = out->dtype == KAPY_F16 || out->dtype == KAPY_BF16;
-  for (int k = 0; k < n_inst; ++k) sig->narrow = sig->narrow && !is_f8(result_dtype[k]);
+  for (int k = 0; k < n_inst; ++k) sig->narrow = sig->narrow && !is_f8(result_dtype[k]) && !is_int(result_dtype[k]);
   int staged_bytes = 0;
   for (int k = 0; k < n_ins; ++k) {
     const View &g = vi[k];
-    if (!is_float(g.dtype)) return false;
+    if (!is_float(g.dtype) && !is_int(g.dtype)) return false;
     sig->narrow = sig->narrow && (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16);
     const int eb = dtype_bytes(g.dtype);
     const bool vec_ok = g.s1 == 1 && ((uintptr_t)g.base % (8 * eb)) == 0 && (g.e0 == 1 || (g.s0 * eb) % (8 * eb) == 0);  // (one row: no pitch to align)
@@ -277,16 +278,21 @@ std::string make_key(const kapy_ew_inst *prog, int n_inst, const Signature &sig)
   for (int k = 0; k < n_inst; ++k) {
     kapy_ew_inst I = prog[k];  // fields an op does not read must not tell two equal programs apart
     const int op = I.op;
+    const bool int_binary_op = (op >= KAPY_EW_ADDI && op <= KAPY_EW_MINUI) || op == KAPY_EW_CMPI || op == KAPY_EW_CMPF;
+    const bool int_cast = op >= KAPY_EW_TRUNCI && op <= KAPY_EW_BITCAST;
     const bool unary_or_cast = !(op == KAPY_EW_LD_GLOBAL || op == KAPY_EW_SPLAT || op == KAPY_EW_FMA || op == KAPY_EW_ADDF || op == KAPY_EW_SUBF ||
                                  op == KAPY_EW_MULF || op == KAPY_EW_DIVF || op == KAPY_EW_MAXIMUMF || op == KAPY_EW_MINIMUMF || op == KAPY_EW_MAXNUMF ||
-                                 op == KAPY_EW_MINNUMF || op == KAPY_EW_REMF);
-    if (op == KAPY_EW_SPLAT) I.a = I.b = I.c = 0;
-    else I.imm = 0.f;
+                                 op == KAPY_EW_MINNUMF || op == KAPY_EW_REMF || int_binary_op || op == KAPY_EW_SELECT || op == KAPY_EW_ARANGE);
+    if (op == KAPY_EW_SPLAT) {
+      I.b = I.c = 0;
+      if (is_int(I.dtype)) I.imm = 0.f;   // an integer splat's value is field a
+      else I.a = 0;
+    } else I.imm = 0.f;
     if (op == KAPY_EW_LD_GLOBAL) I.b = 0;
     if (unary_or_cast) I.b = I.c = 0;
-    if (op != KAPY_EW_FMA && !unary_or_cast && op != KAPY_EW_LD_GLOBAL) I.c = 0;
+    if (op != KAPY_EW_FMA && op != KAPY_EW_SELECT && op != KAPY_EW_CMPI && op != KAPY_EW_CMPF && !unary_or_cast && op != KAPY_EW_LD_GLOBAL) I.c = 0;
     if (op != KAPY_EW_FPTOFP) I.rmode = 0;
-    if (op != KAPY_EW_FPTOFP && op != KAPY_EW_SPLAT) I.dtype = 0;
+    if (op != KAPY_EW_FPTOFP && op != KAPY_EW_SPLAT && !int_cast) I.dtype = 0;
     if (op == KAPY_EW_ST_GLOBAL) I.dst = 0;
     key.append((const char *)&I, sizeof I);
   }
@@ -317,6 +323,7 @@ void appendf(std::string &s, const char *fmt, ...) {
 struct Node {
   int op, a = -1, b = -1, c = -1, dtype = -1, rmode = KAPY_RN, input = -1;
   float imm = 0.f;
+  int ia = 0, ib = 0, ic = 0;  // the instruction's integer fields as given (an integer splat's value, arange's start and axis, a predicate)
   bool used = false;
   std::string name;  // the array, register or constant holding the value
   bool is_const = false;
@@ -337,11 +344,14 @@ std::vector<Node> build_nodes(const kapy_ew_inst *prog, int n_inst, const int *r
     n.dtype = result_dtype[k];
     n.rmode = I.rmode;
     n.imm = I.imm;
+    n.ia = I.a;
+    n.ib = I.b;
+    n.ic = I.c;
     switch (I.op) {
     case KAPY_EW_LD_GLOBAL: n.input = I.a; break;
-    case KAPY_EW_SPLAT: break;
+    case KAPY_EW_SPLAT: case KAPY_EW_ARANGE: break;
     case KAPY_EW_ST_GLOBAL: *stored = reg[I.a]; continue;
-    case KAPY_EW_FMA: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
+    case KAPY_EW_FMA: case KAPY_EW_SELECT: n.a = reg[I.a]; n.b = reg[I.b]; n.c = reg[I.c]; break;
     KAPY_EW_BINARY_CASES:
       n.a = reg[I.a]; n.b = reg[I.b]; break;
     default: n.a = reg[I.a];
@@ -382,8 +392,24 @@ void emit_splats(std::string &s, std::vector<Node> &nodes) {
     memcpy(&bits, &n.imm, 4);
     n.name = "c" + std::to_string(id);
     n.is_const = n.uniform = true;
-    appendf(s, "  const float %s = round_to_dtype(bits_f32(0x%08xu), %d, true);\n", n.name.c_str(), bits, n.dtype);
+    if (is_int(n.dtype)) appendf(s, "  const float %s = int_reg(int_canon((int32_t)0x%08xu, %d));\n", n.name.c_str(), (uint32_t)n.ia, n.dtype);
+    else appendf(s, "  const float %s = round_to_dtype(bits_f32(0x%08xu), %d, true);\n", n.name.c_str(), bits, n.dtype);
   }
+}
+
+// The per-element expression of an op on integer registers, or one that makes or consumes them (compare, select, the
+// integer casts, arange), over the operands' expressions A, B, C; idx0 / idx1: the element's position along the two axes.
+// Empty for every other op.
+std::string int_op_expr(const Node &n, const std::vector<Node> &nodes, const std::string &A, const std::string &B, const std::string &C,
+                        const std::string &idx0, const std::string &idx1) {
+  const std::string op = std::to_string(n.op), dt = std::to_string(n.dtype);
+  if (n.op == KAPY_EW_ARANGE) return "int_reg(" + std::to_string(n.ia) + " + " + (n.ib ? idx1 : idx0) + ")";
+  if (n.op == KAPY_EW_SELECT) return "((reg_int(" + A + ") & 1) ? " + B + " : " + C + ")";
+  if (n.op == KAPY_EW_CMPI) return "int_reg(int_compare(" + std::to_string(n.ic) + ", reg_int(" + A + "), reg_int(" + B + "), " + std::to_string(nodes[n.a].dtype) + "))";
+  if (n.op == KAPY_EW_CMPF) return "int_reg(float_compare(" + std::to_string(n.ic) + ", " + A + ", " + B + "))";
+  if (n.op == KAPY_EW_ABSI || (n.op >= KAPY_EW_TRUNCI && n.op <= KAPY_EW_BITCAST)) return "convert_reg(" + op + ", " + A + ", " + std::to_string(nodes[n.a].dtype) + ", " + dt + ")";
+  if (n.op >= KAPY_EW_ADDI && n.op <= KAPY_EW_MINUI) return "int_reg(int_binary(" + op + ", reg_int(" + A + "), reg_int(" + B + "), " + dt + "))";
+  return "";
 }
 
 // A program without a reduce as straight-line code: every value that the store depends on becomes one array of 8 fp32
@@ -473,6 +499,13 @@ std::string generate_flat(const kapy_ew_inst *prog, int n_inst, const int *resul
       appendf(s, "    float %s[8];\n#pragma unroll\n    for (int e = 0; e < 8; ++e) %s[e] = %s;\n", vn, vn, expr.c_str());
     };
     n.name = v;
+    {
+      const std::string ie = int_op_expr(n, nodes, n.a >= 0 ? elem(n.a) : "", n.b >= 0 ? elem(n.b) : "", n.c >= 0 ? elem(n.c) : "", "row[u]", "(jv[u] * 8 + e)");
+      if (!ie.empty()) {
+        per_element(ie);
+        continue;
+      }
+    }
     switch (n.op) {
     case KAPY_EW_LD_GLOBAL: {
       const int k = n.input, kind = sig.in_kind[k];
@@ -584,6 +617,7 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
     const bool reduce = n.op == KAPY_EW_REDUCE_SUM || n.op == KAPY_EW_REDUCE_MAX;
     n.uniform = reduce || ((n.a < 0 || nodes[n.a].uniform) && (n.b < 0 || nodes[n.b].uniform) && (n.c < 0 || nodes[n.c].uniform) && n.op != KAPY_EW_LD_GLOBAL);
     if (n.op == KAPY_EW_LD_GLOBAL) n.uniform = sig.in_kind[n.input] == kCol || sig.in_kind[n.input] == kScalar;
+    if (n.op == KAPY_EW_ARANGE) n.uniform = n.ib == 0;  // along axis 0: the row's index, one value per row
     n.name = (n.uniform ? "u" : "v") + std::to_string(id);
     const char *vn = n.name.c_str();
     const std::string dt = std::to_string(n.dtype);
@@ -596,6 +630,14 @@ std::string generate_rows(const kapy_ew_inst *prog, int n_inst, const int *resul
       if (n.uniform) appendf(s, "    float %s = %s;\n", vn, expr.c_str());
       else appendf(s, "    float %s[CH][8];\n    %s\n#pragma unroll\n      for (int e = 0; e < 8; ++e) %s[c][e] = %s;\n", vn, kChunks, vn, expr.c_str());
     };
+    {
+      const std::string ie = int_op_expr(n, nodes, n.a >= 0 ? elem(n.a) : "", n.b >= 0 ? elem(n.b) : "", n.c >= 0 ? elem(n.c) : "", "i",
+                                         "((c * THREADS + (int32_t)threadIdx.x) * 8 + e)");
+      if (!ie.empty()) {
+        assign(ie);
+        continue;
+      }
+    }
     switch (n.op) {
     case KAPY_EW_LD_GLOBAL: {
       const int k = n.input, kind = sig.in_kind[k];

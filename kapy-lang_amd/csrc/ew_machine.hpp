@@ -88,6 +88,44 @@ __device__ __forceinline__ float min_num(float a, float b) { return a != a ? b :
 // arith.remf: a - trunc(a / b) * b computed exactly, sign of a (the frem the reference's BinaryOpConversion emits)
 __device__ __forceinline__ float rem_f(float a, float b) { return fmodf(a, b); }
 
+// One instruction of the register machines (interpreter, column machine) for one element: everything but loads, stores and
+// reduces.  Register r of the lane is lane_regs[r * STRIDE]; I.dtype is the result's type (written by the host), and for the
+// ops whose operand type differs from it (cmpi, the integer casts, sitofp, bitcast) the host has put the operand's type
+// into I.rmode; (i, j) is the element's position (kapy.arange).
+template <int STRIDE>
+__device__ __forceinline__ float machine_step(const kapy_ew_inst &I, const float *lane_regs, int32_t i, int32_t j) {
+  const int dt = I.dtype;
+  auto R = [&](int r) { return lane_regs[r * STRIDE]; };
+  switch (I.op) {
+  case KAPY_EW_SPLAT: return dtype_is_int(dt) ? int_reg(int_canon(I.a, dt)) : round_to_dtype(I.imm, dt, true);
+  case KAPY_EW_ARANGE: return int_reg(I.a + (I.b ? j : i));
+  case KAPY_EW_FPTOFP: return round_to_dtype(R(I.a), dt, I.rmode != KAPY_RZ);
+  case KAPY_EW_SELECT: return (reg_int(R(I.a)) & 1) ? R(I.b) : R(I.c);
+  case KAPY_EW_CMPI: return int_reg(int_compare(I.c, reg_int(R(I.a)), reg_int(R(I.b)), I.rmode));
+  case KAPY_EW_CMPF: return int_reg(float_compare(I.c, R(I.a), R(I.b)));
+  case KAPY_EW_ABSI: case KAPY_EW_TRUNCI: case KAPY_EW_EXTSI: case KAPY_EW_EXTUI: case KAPY_EW_SITOFP: case KAPY_EW_FPTOSI: case KAPY_EW_BITCAST:
+    return convert_reg(I.op, R(I.a), I.rmode, dt);
+  default: break;
+  }
+  if (I.op >= KAPY_EW_ADDI && I.op <= KAPY_EW_MINUI) return int_reg(int_binary(I.op, reg_int(R(I.a)), reg_int(R(I.b)), dt));
+  const float a = R(I.a);
+  float r;
+  switch (I.op) {
+  case KAPY_EW_ADDF: r = __fadd_rn(a, R(I.b)); break;
+  case KAPY_EW_SUBF: r = __fsub_rn(a, R(I.b)); break;
+  case KAPY_EW_MULF: r = __fmul_rn(a, R(I.b)); break;
+  case KAPY_EW_DIVF: r = __fdiv_rn(a, R(I.b)); break;
+  case KAPY_EW_FMA: r = fma_typed(a, R(I.b), R(I.c), dt); break;
+  case KAPY_EW_MAXIMUMF: r = max_nan(a, R(I.b)); break;
+  case KAPY_EW_MINIMUMF: r = min_nan(a, R(I.b)); break;
+  case KAPY_EW_MAXNUMF: r = max_num(a, R(I.b)); break;
+  case KAPY_EW_MINNUMF: r = min_num(a, R(I.b)); break;
+  case KAPY_EW_REMF: r = rem_f(a, R(I.b)); break;
+  default: r = apply_unary(I.op, a);
+  }
+  return dt != KAPY_F32 ? round_to_dtype(r, dt, true) : r;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Stack machine: any program whose expression tree needs at most three live values, on 8
 // consecutive elements per lane in registers.  The host unfolds the SSA program into postfix form
@@ -130,7 +168,7 @@ struct Raw8 {
   u32x4 lo, hi;
 };
 __device__ __forceinline__ Raw8 fetch8(const StackIn &g, int32_t i, int32_t jv, bool streaming) {
-  const int eb = g.dtype == KAPY_F32 ? 4 : (g.dtype == KAPY_F16 || g.dtype == KAPY_BF16) ? 2 : 1;
+  const int eb = dtype_elem_bytes(g.dtype);
   const char *ptr = g.base + ((g.kind == kInRow ? 0 : i * g.stride0) + (int64_t)jv * 8) * eb;
   Raw8 r;
   r.lo = r.hi = u32x4{0, 0, 0, 0};
@@ -147,7 +185,16 @@ __device__ __forceinline__ Raw8 fetch8(const StackIn &g, int32_t i, int32_t jv, 
 }
 __device__ __forceinline__ void widen8(const Raw8 &r, int dtype, float f[8]) {
   if (dtype == KAPY_F16 || dtype == KAPY_BF16) widen16x8(r.lo, dtype, f);
-  else if (dtype == KAPY_F32) {
+  else if (dtype == KAPY_I16) {  // integers: the sign-extended image in the container's bits
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = int_reg((int32_t)(int16_t)(r.lo[e >> 1] >> (16 * (e & 1))));
+  } else if (dtype == KAPY_I8 || dtype == KAPY_I1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int32_t byte = (int32_t)(int8_t)(r.lo[e >> 2] >> (8 * (e & 3)));
+      f[e] = int_reg(dtype == KAPY_I1 ? (byte & 1) : byte);
+    }
+  } else if (dtype == KAPY_F32 || dtype == KAPY_I32) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const uint32_t a = r.lo[e], b = r.hi[e];
@@ -212,7 +259,19 @@ __device__ __forceinline__ void store8(char *out, int dtype, int64_t elem, const
 #pragma unroll
     for (int w = 0; w < 4; ++w) v[w] = dtype == KAPY_F16 ? pack2_f16_rn(f[2 * w], f[2 * w + 1]) : pack2_bf16_rn(f[2 * w], f[2 * w + 1]);
     __builtin_nontemporal_store(v, (u32x4 *)(out + elem * 2));
-  } else if (dtype == KAPY_F32) {
+  } else if (dtype == KAPY_I16) {
+    u32x4 v;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v[w] = (f32_bits(f[2 * w]) & 0xFFFFu) | (f32_bits(f[2 * w + 1]) << 16);
+    __builtin_nontemporal_store(v, (u32x4 *)(out + elem * 2));
+  } else if (dtype == KAPY_I8 || dtype == KAPY_I1) {
+    const uint32_t mask = dtype == KAPY_I1 ? 1u : 0xFFu;
+    u32x2 v;
+#pragma unroll
+    for (int w = 0; w < 2; ++w)
+      v[w] = (f32_bits(f[4 * w]) & mask) | ((f32_bits(f[4 * w + 1]) & mask) << 8) | ((f32_bits(f[4 * w + 2]) & mask) << 16) | ((f32_bits(f[4 * w + 3]) & mask) << 24);
+    *(u32x2 *)(out + elem) = v;
+  } else if (dtype == KAPY_F32 || dtype == KAPY_I32) {
     u32x4 lo, hi;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {

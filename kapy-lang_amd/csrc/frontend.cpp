@@ -12,12 +12,14 @@
 // fast path: a program costs tens of launches.
 //
 // Supported: func arguments (!kapy.ptr<1>, i32), arith.constant (i32, float scalar, dense tensor), arith
-// addi/subi/muli/divui/remui/cmpi/select, arith addf/subf/mulf/divf/maximumf/minimumf/negf/extf/truncf and math
-// exp/exp2/log/log2/sqrt/rsqrt/tanh/erf/absf/fma on tensors, kapy.fptofp / splat / broadcast / transpose,
+// addi/subi/muli/divui/remui/cmpi/select on scalars, arith addf/subf/mulf/divf/maximumf/minimumf/negf/extf/truncf and math
+// exp/exp2/log/log2/sqrt/rsqrt/tanh/erf/absf/fma on tensors, the integer arith ops (addi ... minui), cmpi / cmpf / select,
+// trunci / extsi / extui / sitofp / fptosi / bitcast, math.absi and kapy.arange on tensors, kapy.fptofp / splat / broadcast / transpose,
 // kapy.program_id / warp_id / mk_global / sv_global / mk_shared / sv_shared / ld_global / st_global /
 // cp_async_global_to_shared / cp_async_wait_group / ld_matrix / matmul / reduce (addf or maximumf
 // lambda) / return, scf.for with iter_args and scf.yield.
 #include <cctype>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <algorithm>
@@ -106,7 +108,28 @@ int dtype_of(const std::string &w) {
   if (w == "f8E4M3" || w == "f8E4M3FN") return KAPY_F8E4M3;
   if (w == "f8E5M2") return KAPY_F8E5M2;
   if (w == "i32") return KAPY_I32;
+  if (w == "i16") return KAPY_I16;
+  if (w == "i8") return KAPY_I8;
+  if (w == "i1") return KAPY_I1;
   return -1;
+}
+
+// A float literal as MLIR prints it: decimal, or the value's bit pattern in hexadecimal (how infinities and NaNs are written).
+double float_literal(const std::string &w, int dtype) {
+  if (w.size() > 2 && w[0] == '0' && (w[1] == 'x' || w[1] == 'X')) {
+    const uint64_t bits = strtoull(w.c_str(), nullptr, 16);
+    if (dtype == KAPY_F16) {
+      const int e = (int)((bits >> 10) & 31);
+      const double m = (double)(bits & 1023), sign = (bits & 0x8000) ? -1.0 : 1.0;
+      if (e == 31) return m != 0 ? (double)NAN : sign * (double)INFINITY;
+      return sign * (e == 0 ? ldexp(m, -24) : ldexp(1024.0 + m, e - 25));
+    }
+    uint32_t u = dtype == KAPY_BF16 ? (uint32_t)bits << 16 : (uint32_t)bits;
+    float f;
+    memcpy(&f, &u, 4);
+    return (double)f;
+  }
+  return atof(w.c_str());
 }
 
 struct Parser {
@@ -156,7 +179,7 @@ struct Parser {
       ty.kind = Type::kPtr;
       return true;
     }
-    if (k.text == "i32" || k.text == "i1" || k.text == "i64" || k.text == "index") { ++p; ty.kind = Type::kInt; ty.dtype = KAPY_I32; return true; }
+    if (k.text == "i32" || k.text == "i1" || k.text == "i8" || k.text == "i16" || k.text == "i64" || k.text == "index") { ++p; ty.kind = Type::kInt; ty.dtype = KAPY_I32; return true; }
     if (dtype_of(k.text) >= 0) { ++p; ty.kind = Type::kFloat; ty.dtype = dtype_of(k.text); return true; }
     return fail_at("unknown type '" + k.text + "'");
   }
@@ -511,6 +534,7 @@ struct Expr {
   int ew = KAPY_EW_LD_GLOBAL;  // KAPY_EW_LD_GLOBAL: a leaf (`leaf` is the computed tensor); -1: the operand itself (broadcast)
   int dtype = 0, rmode = KAPY_RN;
   float imm = 0.f;
+  int32_t ia = 0, ib = 0, ic = 0;  // integer fields of the instruction: an integer splat's value, arange's start and axis, a compare's predicate
   std::shared_ptr<Expr> in[3];
   int n_in = 0;
   kapy_global leaf;
@@ -662,8 +686,10 @@ struct Interp {
       m.prog[m.n++] = {KAPY_EW_LD_GLOBAL, dst, slot, 0, 0, 0, KAPY_RN, 0.f};
     } else if (e->ew == KAPY_EW_REDUCE_SUM || e->ew == KAPY_EW_REDUCE_MAX) {
       m.prog[m.n++] = {e->ew, dst, src[0], e->axis, 0, 0, KAPY_RN, 0.f};
+    } else if (e->ew == KAPY_EW_ARANGE || (e->ew == KAPY_EW_SPLAT && e->dtype >= KAPY_I8)) {
+      m.prog[m.n++] = {e->ew, dst, e->ia, e->ib, 0, e->dtype, KAPY_RN, 0.f};
     } else {
-      m.prog[m.n++] = {e->ew, dst, src[0], src[1], src[2], e->dtype, e->rmode, e->imm};
+      m.prog[m.n++] = {e->ew, dst, src[0], src[1], (e->ew == KAPY_EW_CMPI || e->ew == KAPY_EW_CMPF) ? e->ic : src[2], e->dtype, e->rmode, e->imm};
     }
     return m.reg[e.get()] = dst;
   }
@@ -760,12 +786,13 @@ struct Interp {
   }
   // result <- ew(operands...) without running anything; falls back to computing operands when the chain would outgrow one
   // program, and to computing the result at once when an operand is memory the program can still change
-  int defer(const Op &op, int n_operands, int ew, int dtype, int rmode, float imm) {
+  int defer(const Op &op, int n_operands, int ew, int dtype, int rmode, float imm, int32_t ia = 0, int32_t ib = 0, int32_t ic = 0) {
     if (op.types.empty()) return fail_op(op, "missing result type");
     const Type &ty = op.types.back();
     if (ty.kind != Type::kTensor || ty.shape[0] <= 0 || ty.shape[1] <= 0) return fail_op(op, "result must be a statically shaped tensor");
     auto e = std::make_shared<Expr>();
     e->ew = ew; e->dtype = dtype; e->rmode = rmode; e->imm = imm; e->n_in = n_operands;
+    e->ia = ia; e->ib = ib; e->ic = ic;
     bool at_once = !fuse;
     for (int k = 0; k < n_operands; ++k) {
       if (k >= (int)op.operands.size()) return fail_op(op, "missing operand");
@@ -942,9 +969,13 @@ struct Interp {
         r.i = w == "true" ? 1 : w == "false" ? 0 : atoll(w.c_str());
       } else if (ty.kind == Type::kFloat) {
         r.kind = Value::kFloat;
-        r.f = op.words.empty() ? 0.0 : atof(op.words[0].c_str());
+        r.f = op.words.empty() ? 0.0 : float_literal(op.words[0], ty.dtype);
       } else if (ty.kind == Type::kTensor) {
-        return defer(op, 0, KAPY_EW_SPLAT, ty.dtype, KAPY_RN, op.words.empty() ? 0.f : (float)atof(op.words[0].c_str()));
+        if (ty.dtype >= KAPY_I8) {  // dense<3> : tensor<..xi32>, dense<true> : tensor<..xi1>
+          const std::string &w = op.words.empty() ? std::string("0") : op.words[0];
+          return defer(op, 0, KAPY_EW_SPLAT, ty.dtype, KAPY_RN, 0.f, w == "true" ? 1 : w == "false" ? 0 : (int32_t)atoll(w.c_str()));
+        }
+        return defer(op, 0, KAPY_EW_SPLAT, ty.dtype, KAPY_RN, op.words.empty() ? 0.f : (float)float_literal(op.words[0], ty.dtype));
       } else return fail_op(op, "unsupported constant type");
       env[op.results[0]] = r;
       return KAPY_OK;
@@ -958,6 +989,43 @@ struct Interp {
       return KAPY_OK;
     }
     if (n == "kapy.warp_id") { r.kind = Value::kInt; r.i = warp; env[op.results[0]] = r; return KAPY_OK; }
+    // integer, compare, select and conversion ops on tensors (ElementwiseOpToLLVM.cpp:1178-1215, SelectOpToLLVM.cpp:21-98): one
+    // instruction of a deferred program each; the same ops on scalars are evaluated on the host below
+    const bool on_tensor = !op.operands.empty() && env.count(op.operands[0]) && env[op.operands[0]].kind == Value::kTensor;
+    if (on_tensor) {
+      static const struct { const char *name; int ew; } int_binary[] = {
+          {"arith.addi", KAPY_EW_ADDI}, {"arith.subi", KAPY_EW_SUBI}, {"arith.muli", KAPY_EW_MULI}, {"arith.divsi", KAPY_EW_DIVSI}, {"arith.divui", KAPY_EW_DIVUI},
+          {"arith.floordivsi", KAPY_EW_FLOORDIVSI}, {"arith.ceildivsi", KAPY_EW_CEILDIVSI}, {"arith.ceildivui", KAPY_EW_CEILDIVUI}, {"arith.remsi", KAPY_EW_REMSI},
+          {"arith.remui", KAPY_EW_REMUI}, {"arith.andi", KAPY_EW_ANDI}, {"arith.ori", KAPY_EW_ORI}, {"arith.xori", KAPY_EW_XORI}, {"arith.shli", KAPY_EW_SHLI},
+          {"arith.shrsi", KAPY_EW_SHRSI}, {"arith.shrui", KAPY_EW_SHRUI}, {"arith.maxsi", KAPY_EW_MAXSI}, {"arith.maxui", KAPY_EW_MAXUI}, {"arith.minsi", KAPY_EW_MINSI},
+          {"arith.minui", KAPY_EW_MINUI}};
+      for (auto &u : int_binary)
+        if (n == u.name) return binary_tensor(op, u.ew);
+      if (n == "arith.cmpi" || n == "arith.cmpf") {
+        static const char *const cmpi[] = {"eq", "ne", "slt", "sle", "sgt", "sge", "ult", "ule", "ugt", "uge"};
+        static const char *const cmpf[] = {"false", "oeq", "ogt", "oge", "olt", "ole", "one", "ord", "ueq", "ugt", "uge", "ult", "ule", "une", "uno", "true"};
+        const std::string &pr = op.words.empty() ? std::string("?") : op.words[0];
+        int pred = -1;
+        if (n == "arith.cmpi") { for (int k = 0; k < 10; ++k) if (pr == cmpi[k]) pred = k; }
+        else { for (int k = 0; k < 16; ++k) if (pr == cmpf[k]) pred = k; }
+        if (pred < 0) return fail_op(op, "unknown compare predicate '" + pr + "'");
+        if (op.types.empty()) return fail_op(op, "compare without a type");
+        Op typed = op;  // the type written after a compare is its operands'; the result has that shape with element type i1
+        typed.types.back().dtype = KAPY_I1;
+        return defer(typed, 2, n == "arith.cmpi" ? KAPY_EW_CMPI : KAPY_EW_CMPF, KAPY_I1, KAPY_RN, 0.f, 0, 0, pred);
+      }
+      if (n == "arith.select") return defer(op, 3, KAPY_EW_SELECT, 0, KAPY_RN, 0.f);
+      static const struct { const char *name; int ew; } int_unary[] = {
+          {"arith.trunci", KAPY_EW_TRUNCI}, {"arith.extsi", KAPY_EW_EXTSI}, {"arith.extui", KAPY_EW_EXTUI}, {"arith.sitofp", KAPY_EW_SITOFP},
+          {"arith.fptosi", KAPY_EW_FPTOSI}, {"arith.bitcast", KAPY_EW_BITCAST}, {"math.absi", KAPY_EW_ABSI}};
+      for (auto &u : int_unary)
+        if (n == u.name) return mapped_tensor(op, 1, u.ew, op.types.empty() ? 0 : op.types.back().dtype);
+    }
+    if (n == "kapy.arange") {  // i32 values start, start + 1, ... along `axis` (ArangeOpToLLVM.cpp:22-50)
+      const int axis = op.attrs.count("axis") ? atoi(op.attrs.at("axis").c_str()) : 0, start = op.attrs.count("start") ? atoi(op.attrs.at("start").c_str()) : 0;
+      if (axis != 0 && axis != 1) return fail_op(op, "axis must be 0 or 1");
+      return defer(op, 0, KAPY_EW_ARANGE, KAPY_I32, KAPY_RN, 0.f, start, axis);
+    }
     if (n == "arith.addi" || n == "arith.subi" || n == "arith.muli" || n == "arith.divui" || n == "arith.remui" || n == "arith.cmpi") {
       if (!get(op, 0, Value::kInt, a) || !get(op, 1, Value::kInt, b)) return KAPY_ERR_INVALID;
       r.kind = Value::kInt;
@@ -1013,6 +1081,10 @@ struct Interp {
     }
     if (n == "kapy.splat") {
       Value v;
+      if (!op.operands.empty() && env.count(op.operands[0]) && env[op.operands[0]].kind == Value::kInt && !op.types.empty()) {  // an integer scalar
+        const int64_t i = env[op.operands[0]].i;
+        return defer(op, 0, KAPY_EW_SPLAT, op.types.back().dtype, KAPY_RN, (float)i, (int32_t)i);
+      }
       if (!get(op, 0, Value::kFloat, v) || op.types.empty()) return KAPY_ERR_INVALID;
       return defer(op, 0, KAPY_EW_SPLAT, op.types.back().dtype, KAPY_RN, (float)v.f);
     }
@@ -1206,7 +1278,11 @@ const struct OpForm { const char *name; int min_operands, results; } kSupportedO
     {"kapy.cp_async_global_to_shared", 2, 0}, {"kapy.cp_async_wait_group", 0, 0}, {"kapy.matmul", 3, 1}, {"kapy.reduce", 1, 1},
     {"nvvm.barrier0", 0, 0}, {"math.exp", 1, 1}, {"math.exp2", 1, 1}, {"math.log", 1, 1}, {"math.log2", 1, 1}, {"math.sqrt", 1, 1},
     {"math.rsqrt", 1, 1}, {"math.tanh", 1, 1}, {"math.erf", 1, 1}, {"math.absf", 1, 1}, {"math.floor", 1, 1}, {"math.ceil", 1, 1}, {"math.sin", 1, 1}, {"math.cos", 1, 1}, {"math.fma", 3, 1}, {"arith.negf", 1, 1},
-    {"arith.extf", 1, 1}, {"arith.truncf", 1, 1}, {"kapy.fptofp", 1, 1}, {"kapy.splat", 1, 1}, {"kapy.broadcast", 1, 1}, {"kapy.transpose", 1, 1}};
+    {"arith.extf", 1, 1}, {"arith.truncf", 1, 1}, {"kapy.fptofp", 1, 1}, {"kapy.splat", 1, 1}, {"kapy.broadcast", 1, 1}, {"kapy.transpose", 1, 1},
+    {"arith.divsi", 2, 1}, {"arith.floordivsi", 2, 1}, {"arith.ceildivsi", 2, 1}, {"arith.ceildivui", 2, 1}, {"arith.remsi", 2, 1}, {"arith.andi", 2, 1},
+    {"arith.ori", 2, 1}, {"arith.xori", 2, 1}, {"arith.shli", 2, 1}, {"arith.shrsi", 2, 1}, {"arith.shrui", 2, 1}, {"arith.maxsi", 2, 1}, {"arith.maxui", 2, 1},
+    {"arith.minsi", 2, 1}, {"arith.minui", 2, 1}, {"arith.cmpf", 2, 1}, {"arith.trunci", 1, 1}, {"arith.extsi", 1, 1}, {"arith.extui", 1, 1},
+    {"arith.sitofp", 1, 1}, {"arith.fptosi", 1, 1}, {"arith.bitcast", 1, 1}, {"math.absi", 1, 1}, {"kapy.arange", 0, 1}};
 
 // Every op must be one this front-end executes, written with the operands and results it needs; returns the number of ops,
 // regions included, -1 for an op it does not execute, -2 for one that is malformed.  (The body of a kapy.reduce is only looked at for its combiner: its ops are not executed.)

@@ -135,7 +135,174 @@ __device__ __forceinline__ float fma_typed(float a, float b, float c, int dtype)
   return r;
 }
 
-// Value of element `idx` of a typed buffer as an fp32 (exact for every supported type but i32).
+// ---- integer registers.  A signless iN value travels in the 32 bits of the machines' fp32 container as its sign-extended
+// image (i1: 0 or 1); nothing but moves, LDS and these helpers ever touches such a container, so the bits survive.
+__device__ __forceinline__ int32_t reg_int(float x) { return __builtin_bit_cast(int32_t, x); }
+__device__ __forceinline__ float int_reg(int32_t v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ bool dtype_is_int(int dtype) { return dtype == KAPY_I8 || dtype == KAPY_I16 || dtype == KAPY_I32 || dtype == KAPY_I1; }
+__device__ __forceinline__ int int_width(int dtype) { return dtype == KAPY_I1 ? 1 : dtype == KAPY_I8 ? 8 : dtype == KAPY_I16 ? 16 : 32; }
+// the canonical image of the low bits of v
+__device__ __forceinline__ int32_t int_canon(int32_t v, int dtype) {
+  return dtype == KAPY_I1 ? (v & 1) : dtype == KAPY_I8 ? (int32_t)(int8_t)v : dtype == KAPY_I16 ? (int32_t)(int16_t)v : v;
+}
+// the value read as a signed / as an unsigned number of its width
+__device__ __forceinline__ int32_t int_signed(int32_t v, int dtype) { return dtype == KAPY_I1 ? -(v & 1) : v; }
+__device__ __forceinline__ uint32_t int_unsigned(int32_t v, int dtype) {
+  return dtype == KAPY_I1 ? (uint32_t)(v & 1) : dtype == KAPY_I8 ? (uint32_t)(uint8_t)v : dtype == KAPY_I16 ? (uint32_t)(uint16_t)v : (uint32_t)v;
+}
+
+// arith.addi ... minui on two values of integer type dtype (BinaryOpConversion, ElementwiseOpToLLVM.cpp:1178-1206): wrapping
+// arithmetic; what MLIR leaves undefined is defined here (x / 0 = 0, x % 0 = 0, min / -1 wraps with remainder 0, shifts by
+// the width or more give 0, shrsi the sign).
+__device__ __forceinline__ int32_t int_binary(int op, int32_t av, int32_t bv, int dtype) {
+  const int32_t a = int_signed(av, dtype), b = int_signed(bv, dtype);
+  const uint32_t ua = int_unsigned(av, dtype), ub = int_unsigned(bv, dtype);
+  const uint32_t width = (uint32_t)int_width(dtype);
+  uint32_t r = 0;
+  switch (op) {
+  case KAPY_EW_ADDI: r = ua + ub; break;
+  case KAPY_EW_SUBI: r = ua - ub; break;
+  case KAPY_EW_MULI: r = ua * ub; break;
+  case KAPY_EW_DIVSI: r = b == 0 ? 0u : b == -1 ? 0u - ua : (uint32_t)(a / b); break;
+  case KAPY_EW_DIVUI: r = ub == 0 ? 0u : ua / ub; break;
+  case KAPY_EW_FLOORDIVSI:
+    if (b == 0) r = 0;
+    else if (b == -1) r = 0u - ua;
+    else {
+      const int32_t q = a / b;
+      r = (uint32_t)(q - ((a % b != 0 && ((a < 0) != (b < 0))) ? 1 : 0));
+    }
+    break;
+  case KAPY_EW_CEILDIVSI:
+    if (b == 0) r = 0;
+    else if (b == -1) r = 0u - ua;
+    else {
+      const int32_t q = a / b;
+      r = (uint32_t)(q + ((a % b != 0 && ((a < 0) == (b < 0))) ? 1 : 0));
+    }
+    break;
+  case KAPY_EW_CEILDIVUI: r = (ub == 0 || ua == 0) ? 0u : (ua - 1) / ub + 1; break;
+  case KAPY_EW_REMSI: r = (b == 0 || b == -1) ? 0u : (uint32_t)(a % b); break;
+  case KAPY_EW_REMUI: r = ub == 0 ? 0u : ua % ub; break;
+  case KAPY_EW_ANDI: r = ua & ub; break;
+  case KAPY_EW_ORI: r = ua | ub; break;
+  case KAPY_EW_XORI: r = ua ^ ub; break;
+  case KAPY_EW_SHLI: r = ub >= width ? 0u : ua << ub; break;
+  case KAPY_EW_SHRUI: r = ub >= width ? 0u : ua >> ub; break;
+  case KAPY_EW_SHRSI: r = (uint32_t)(a >> (ub >= width ? width - 1 : ub)); break;
+  case KAPY_EW_MAXSI: r = (uint32_t)(a > b ? a : b); break;
+  case KAPY_EW_MINSI: r = (uint32_t)(a < b ? a : b); break;
+  case KAPY_EW_MAXUI: r = ua > ub ? ua : ub; break;
+  case KAPY_EW_MINUI: r = ua < ub ? ua : ub; break;
+  }
+  return int_canon((int32_t)r, dtype);
+}
+// arith.cmpi with MLIR's predicate numbers
+__device__ __forceinline__ int32_t int_compare(int pred, int32_t av, int32_t bv, int dtype) {
+  const int32_t a = int_signed(av, dtype), b = int_signed(bv, dtype);
+  const uint32_t ua = int_unsigned(av, dtype), ub = int_unsigned(bv, dtype);
+  switch (pred) {
+  case KAPY_CMPI_EQ: return ua == ub;
+  case KAPY_CMPI_NE: return ua != ub;
+  case KAPY_CMPI_SLT: return a < b;
+  case KAPY_CMPI_SLE: return a <= b;
+  case KAPY_CMPI_SGT: return a > b;
+  case KAPY_CMPI_SGE: return a >= b;
+  case KAPY_CMPI_ULT: return ua < ub;
+  case KAPY_CMPI_ULE: return ua <= ub;
+  case KAPY_CMPI_UGT: return ua > ub;
+  default: return ua >= ub;
+  }
+}
+// arith.cmpf: the ordered predicates are false, the unordered ones true, when an operand is NaN
+__device__ __forceinline__ int32_t float_compare(int pred, float a, float b) {
+  const bool uno = a != a || b != b;
+  switch (pred) {
+  case KAPY_CMPF_FALSE: return 0;
+  case KAPY_CMPF_OEQ: return a == b;
+  case KAPY_CMPF_OGT: return a > b;
+  case KAPY_CMPF_OGE: return a >= b;
+  case KAPY_CMPF_OLT: return a < b;
+  case KAPY_CMPF_OLE: return a <= b;
+  case KAPY_CMPF_ONE: return !uno && a != b;
+  case KAPY_CMPF_ORD: return !uno;
+  case KAPY_CMPF_UEQ: return uno || a == b;
+  case KAPY_CMPF_UGT: return uno || a > b;
+  case KAPY_CMPF_UGE: return uno || a >= b;
+  case KAPY_CMPF_ULT: return uno || a < b;
+  case KAPY_CMPF_ULE: return uno || a <= b;
+  case KAPY_CMPF_UNE: return uno || a != b;
+  case KAPY_CMPF_UNO: return uno;
+  default: return 1;
+  }
+}
+// arith.sitofp: one rounding to nearest even from the integer.  f32: the conversion instruction; f16: through f32 (any
+// integer the f32 rounding touches, |v| >= 2^24, is beyond f16's range and becomes infinity either way); bf16: rounded
+// from the integer's own bits (through f32 a value could be rounded twice).  Returns the fp32 image.
+__device__ __forceinline__ float int_to_float(int32_t v, int dtype) {
+  if (dtype == KAPY_F32) return (float)v;
+  if (dtype == KAPY_F16) return f16_to_f32(f32_to_f16_rn((float)v));
+  if (v == 0) return 0.f;
+  const uint32_t sign = v < 0 ? 0x80000000u : 0u, mag = v < 0 ? 0u - (uint32_t)v : (uint32_t)v;
+  const int lz = __builtin_clz(mag);
+  const uint32_t m = mag << lz;                   // bit 31 is the leading one
+  uint32_t keep = m >> 24;                        // 1.7 bits of a bf16 significand
+  const uint32_t rest = m & 0x00FFFFFFu;
+  int exponent = 31 - lz;
+  if (rest > 0x00800000u || (rest == 0x00800000u && (keep & 1))) {
+    if (++keep == 0x100u) { keep = 0x80u; ++exponent; }
+  }
+  return bits_f32(sign | ((uint32_t)(exponent + 127) << 23) | ((keep & 0x7Fu) << 16));
+}
+// arith.fptosi: toward zero; saturating, NaN -> 0 (where MLIR leaves the result undefined), then wrapped to the width
+__device__ __forceinline__ int32_t float_to_int(float x, int dtype) {
+  const int32_t v = x != x ? 0 : x >= 2147483648.f ? 0x7FFFFFFF : x <= -2147483648.f ? (int32_t)0x80000000u : (int32_t)x;
+  return int_canon(v, dtype);
+}
+// arith.bitcast between a float type and the integer type of its width (containers: fp32 image / sign-extended image)
+__device__ __forceinline__ float bitcast_reg(float x, int from, int to) {
+  if (from == to || (dtype_is_int(from) && dtype_is_int(to))) return x;
+  if (dtype_is_int(to)) {  // float -> int
+    switch (from) {
+    case KAPY_F32: return x;
+    case KAPY_F16: return int_reg((int32_t)(int16_t)f32_to_f16_rn(x));
+    case KAPY_BF16: return int_reg((int32_t)(int16_t)f32_to_bf16_rn(x));
+    case KAPY_F8E4M3: return int_reg((int32_t)(int8_t)f32_to_e4m3(x, true));
+    default: return int_reg((int32_t)(int8_t)f32_to_e5m2(x, true));
+    }
+  }
+  const int32_t v = reg_int(x);
+  switch (to) {
+  case KAPY_F32: return x;
+  case KAPY_F16: return f16_to_f32((uint16_t)v);
+  case KAPY_BF16: return bf16_to_f32((uint16_t)v);
+  case KAPY_F8E4M3: return e4m3_to_f32((uint8_t)v);
+  default: return e5m2_to_f32((uint8_t)v);
+  }
+}
+
+// The conversions with one operand whose result type differs from (or, absi, equals) the operand's: math.absi, arith.trunci /
+// extsi / extui, sitofp, fptosi, bitcast, on containers (x of type `from`, the result of type `to`).
+__device__ __forceinline__ float convert_reg(int op, float x, int from, int to) {
+  switch (op) {
+  case KAPY_EW_ABSI: {
+    const int32_t v = int_signed(reg_int(x), to);
+    return int_reg(int_canon(v < 0 ? (int32_t)(0u - (uint32_t)v) : v, to));
+  }
+  case KAPY_EW_TRUNCI: return int_reg(int_canon(reg_int(x), to));
+  case KAPY_EW_EXTSI: return int_reg(int_canon(int_signed(reg_int(x), from), to));
+  case KAPY_EW_EXTUI: return int_reg(int_canon((int32_t)int_unsigned(reg_int(x), from), to));
+  case KAPY_EW_SITOFP: return int_to_float(int_signed(reg_int(x), from), to);
+  case KAPY_EW_FPTOSI: return int_reg(float_to_int(x, to));
+  default: return bitcast_reg(x, from, to);
+  }
+}
+__device__ __forceinline__ int dtype_elem_bytes(int dtype) {
+  return (dtype == KAPY_F32 || dtype == KAPY_I32) ? 4 : (dtype == KAPY_F16 || dtype == KAPY_BF16 || dtype == KAPY_I16) ? 2 : 1;
+}
+
+// Value of element `idx` of a typed buffer in the machines' container: the fp32 image of a float, the sign-extended image
+// (in the container's bits) of an integer.
 __device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t idx) {
   switch (dtype) {
   case KAPY_F16: return f16_to_f32(((const uint16_t *)p)[idx]);
@@ -143,9 +310,10 @@ __device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t i
   case KAPY_F32: return ((const float *)p)[idx];
   case KAPY_F8E4M3: return e4m3_to_f32(((const uint8_t *)p)[idx]);
   case KAPY_F8E5M2: return e5m2_to_f32(((const uint8_t *)p)[idx]);
-  case KAPY_I8: return (float)((const int8_t *)p)[idx];
-  case KAPY_I16: return (float)((const int16_t *)p)[idx];
-  default: return (float)((const int32_t *)p)[idx];
+  case KAPY_I8: return int_reg((int32_t)((const int8_t *)p)[idx]);
+  case KAPY_I16: return int_reg((int32_t)((const int16_t *)p)[idx]);
+  case KAPY_I1: return int_reg((int32_t)(((const uint8_t *)p)[idx] & 1));
+  default: return int_reg(((const int32_t *)p)[idx]);
   }
 }
 
@@ -168,9 +336,10 @@ __device__ __forceinline__ void store_from_f32(void *p, int dtype, int64_t idx, 
   case KAPY_F32: ((float *)p)[idx] = v; break;
   case KAPY_F8E4M3: ((uint8_t *)p)[idx] = f32_to_e4m3(v, true); break;
   case KAPY_F8E5M2: ((uint8_t *)p)[idx] = f32_to_e5m2(v, true); break;
-  case KAPY_I8: ((int8_t *)p)[idx] = (int8_t)v; break;
-  case KAPY_I16: ((int16_t *)p)[idx] = (int16_t)v; break;
-  default: ((int32_t *)p)[idx] = (int32_t)v; break;
+  case KAPY_I8: ((int8_t *)p)[idx] = (int8_t)reg_int(v); break;
+  case KAPY_I16: ((int16_t *)p)[idx] = (int16_t)reg_int(v); break;
+  case KAPY_I1: ((uint8_t *)p)[idx] = (uint8_t)(reg_int(v) & 1); break;
+  default: ((int32_t *)p)[idx] = reg_int(v); break;
   }
 }
 

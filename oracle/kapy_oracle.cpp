@@ -109,7 +109,7 @@ inline int dtype_bytes(int dtype) {
   switch (dtype) {
   case KO_F16: case KO_BF16: case KO_I16: return 2;
   case KO_F32: case KO_I32: return 4;
-  case KO_F8E4M3: case KO_F8E5M2: case KO_I8: return 1;
+  case KO_F8E4M3: case KO_F8E5M2: case KO_I8: case KO_I1: return 1;
   }
   return 0;
 }
@@ -161,6 +161,7 @@ double ko_decode(const void *p, int dtype, int64_t idx) {
   case KO_I8: return (double)((const int8_t *)p)[idx];
   case KO_I16: return (double)((const int16_t *)p)[idx];
   case KO_I32: return (double)((const int32_t *)p)[idx];
+  case KO_I1: return (double)(((const uint8_t *)p)[idx] & 1);
   }
   return 0.0;
 }
@@ -172,9 +173,10 @@ void ko_encode(void *p, int dtype, int64_t idx, double v, int rmode) {
   case KO_F32: ((float *)p)[idx] = f64_to_f32_mode(v, rmode); break;
   case KO_F8E4M3: ((uint8_t *)p)[idx] = (uint8_t)encode_small(v, kE4M3, rmode); break;
   case KO_F8E5M2: ((uint8_t *)p)[idx] = (uint8_t)encode_small(v, kE5M2, rmode); break;
-  case KO_I8: ((int8_t *)p)[idx] = (int8_t)v; break;
-  case KO_I16: ((int16_t *)p)[idx] = (int16_t)v; break;
-  case KO_I32: ((int32_t *)p)[idx] = (int32_t)v; break;
+  case KO_I8: ((int8_t *)p)[idx] = (int8_t)(int64_t)v; break;
+  case KO_I16: ((int16_t *)p)[idx] = (int16_t)(int64_t)v; break;
+  case KO_I32: ((int32_t *)p)[idx] = (int32_t)(int64_t)v; break;
+  case KO_I1: ((uint8_t *)p)[idx] = (uint8_t)((int64_t)v & 1); break;
   }
 }
 
@@ -585,9 +587,96 @@ enum {
   EW_LD_GLOBAL = 0, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
   EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH, EW_ST_GLOBAL,
   EW_REDUCE_SUM, EW_REDUCE_MAX, EW_FLOOR, EW_CEIL, EW_SIN, EW_COS, EW_MAXNUMF, EW_MINNUMF, EW_REMF,
+  // integer, compare, select and conversion ops (BinaryOpConversion / UnaryOpConversion over the arith ops,
+  // ElementwiseOpToLLVM.cpp:1178-1215; arith.select, SelectOpToLLVM.cpp:21-98; kapy.arange, ArangeOpToLLVM.cpp:22-50)
+  EW_ADDI, EW_SUBI, EW_MULI, EW_DIVSI, EW_DIVUI, EW_FLOORDIVSI, EW_CEILDIVSI, EW_CEILDIVUI, EW_REMSI, EW_REMUI, EW_ANDI, EW_ORI, EW_XORI,
+  EW_SHLI, EW_SHRSI, EW_SHRUI, EW_MAXSI, EW_MAXUI, EW_MINSI, EW_MINUI, EW_ABSI, EW_CMPI, EW_CMPF, EW_SELECT, EW_TRUNCI, EW_EXTSI, EW_EXTUI,
+  EW_SITOFP, EW_FPTOSI, EW_BITCAST, EW_ARANGE,
   EW_NUM_OPS
 };
 enum { EW_MAX_REGS = 16 };
+
+// ---- signless integers (MLIR's iN): a register holds the value read as a signed number of its width (i1: 0 or 1) in a
+// double.  What MLIR leaves undefined is defined as the device library defines it: x / 0 = 0, x % 0 = 0, the most negative
+// value over -1 wraps (remainder 0), a shift by the width or more gives 0 (shrsi: all sign bits), fptosi saturates to i32
+// and maps NaN to 0 before wrapping to the result's width.
+static bool is_int_dtype(int d) { return d == KO_I8 || d == KO_I16 || d == KO_I32 || d == KO_I1; }
+static bool is_arith_float(int d) { return d == KO_F16 || d == KO_BF16 || d == KO_F32; }
+static int int_bits(int d) { return d == KO_I1 ? 1 : d == KO_I8 ? 8 : d == KO_I16 ? 16 : 32; }
+static int64_t int_wrap(int64_t v, int d) {  // the low bits of v as the register keeps them
+  const int bits = int_bits(d);
+  const uint64_t low = (uint64_t)v & ((uint64_t(1) << bits) - 1);
+  if (d == KO_I1) return (int64_t)low;
+  return (low >> (bits - 1)) ? (int64_t)low - (int64_t(1) << bits) : (int64_t)low;
+}
+static int64_t int_as_signed(int64_t reg, int d) { return d == KO_I1 ? -reg : reg; }
+static int64_t int_as_unsigned(int64_t reg, int d) { return d == KO_I1 ? reg : (reg < 0 ? reg + (int64_t(1) << int_bits(d)) : reg); }
+static int64_t floor_div(int64_t a, int64_t b) {
+  int64_t q = a / b;
+  if ((a % b != 0) && ((a < 0) != (b < 0))) --q;
+  return q;
+}
+static int64_t int_binary_op(int op, int64_t ra, int64_t rb, int d) {
+  const int64_t a = int_as_signed(ra, d), b = int_as_signed(rb, d), ua = int_as_unsigned(ra, d), ub = int_as_unsigned(rb, d);
+  const int bits = int_bits(d);
+  int64_t r = 0;
+  switch (op) {
+  case EW_ADDI: r = a + b; break;
+  case EW_SUBI: r = a - b; break;
+  case EW_MULI: r = (int64_t)((uint64_t)a * (uint64_t)b); break;
+  case EW_DIVSI: r = b == 0 ? 0 : a / b; break;                      // (64-bit: the most negative value over -1 does not trap, it wraps below)
+  case EW_DIVUI: r = ub == 0 ? 0 : ua / ub; break;
+  case EW_FLOORDIVSI: r = b == 0 ? 0 : floor_div(a, b); break;
+  case EW_CEILDIVSI: r = b == 0 ? 0 : -floor_div(-a, b); break;
+  case EW_CEILDIVUI: r = ub == 0 ? 0 : (ua + ub - 1) / ub; break;
+  case EW_REMSI: r = b == 0 ? 0 : a % b; break;
+  case EW_REMUI: r = ub == 0 ? 0 : ua % ub; break;
+  case EW_ANDI: r = ua & ub; break;
+  case EW_ORI: r = ua | ub; break;
+  case EW_XORI: r = ua ^ ub; break;
+  case EW_SHLI: r = ub >= bits ? 0 : (int64_t)((uint64_t)ua << ub); break;
+  case EW_SHRUI: r = ub >= bits ? 0 : ua >> ub; break;
+  case EW_SHRSI: r = ub >= bits ? (a < 0 ? -1 : 0) : floor_div(a, int64_t(1) << ub); break;
+  case EW_MAXSI: r = std::max(a, b); break;
+  case EW_MINSI: r = std::min(a, b); break;
+  case EW_MAXUI: r = std::max(ua, ub); break;
+  case EW_MINUI: r = std::min(ua, ub); break;
+  }
+  return int_wrap(r, d);
+}
+static int64_t int_compare_op(int pred, int64_t ra, int64_t rb, int d) {
+  const int64_t a = int_as_signed(ra, d), b = int_as_signed(rb, d), ua = int_as_unsigned(ra, d), ub = int_as_unsigned(rb, d);
+  switch (pred) {  // arith.cmpi predicates as MLIR numbers them
+  case 0: return ua == ub;
+  case 1: return ua != ub;
+  case 2: return a < b;
+  case 3: return a <= b;
+  case 4: return a > b;
+  case 5: return a >= b;
+  case 6: return ua < ub;
+  case 7: return ua <= ub;
+  case 8: return ua > ub;
+  default: return ua >= ub;
+  }
+}
+static int64_t float_compare_op(int pred, double a, double b) {
+  const bool unordered = std::isnan(a) || std::isnan(b);
+  if (pred == 0) return 0;
+  if (pred == 15) return 1;
+  if (pred == 7) return !unordered;
+  if (pred == 14) return unordered;
+  const int base = pred >= 8 ? pred - 7 : pred;  // oeq ogt oge olt ole one = 1..6; ueq .. une = 8..13
+  bool ordered_result = false;
+  switch (base) {
+  case 1: ordered_result = a == b; break;
+  case 2: ordered_result = a > b; break;
+  case 3: ordered_result = a >= b; break;
+  case 4: ordered_result = a < b; break;
+  case 5: ordered_result = a <= b; break;
+  case 6: ordered_result = a != b; break;
+  }
+  return unordered ? pred >= 8 : ordered_result;
+}
 
 static double round_to(double v, int dtype) {
   switch (dtype) {
@@ -628,9 +717,47 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
       break;
     }
     case EW_SPLAT:
-      if (I.dtype != KO_F16 && I.dtype != KO_BF16 && I.dtype != KO_F32) return -5;
+      if (!is_arith_float(I.dtype) && !is_int_dtype(I.dtype)) return -5;
       reg_dtype[I.dst] = I.dtype;
       break;
+    case EW_ARANGE:
+      if (I.b != 0 && I.b != 1) return -14;
+      reg_dtype[I.dst] = KO_I32;
+      break;
+    case EW_SELECT:
+      if (!reg_ok(I.a) || !reg_ok(I.b) || !reg_ok(I.c)) return -6;
+      if (reg_dtype[I.a] != KO_I1 || reg_dtype[I.b] != reg_dtype[I.c]) return -10;
+      reg_dtype[I.dst] = reg_dtype[I.b];
+      break;
+    case EW_ADDI: case EW_SUBI: case EW_MULI: case EW_DIVSI: case EW_DIVUI: case EW_FLOORDIVSI: case EW_CEILDIVSI: case EW_CEILDIVUI: case EW_REMSI:
+    case EW_REMUI: case EW_ANDI: case EW_ORI: case EW_XORI: case EW_SHLI: case EW_SHRSI: case EW_SHRUI: case EW_MAXSI: case EW_MAXUI: case EW_MINSI:
+    case EW_MINUI: case EW_CMPI:
+      if (!reg_ok(I.a) || !reg_ok(I.b)) return -6;
+      if (reg_dtype[I.a] != reg_dtype[I.b] || !is_int_dtype(reg_dtype[I.a])) return -10;
+      if (I.op == EW_CMPI && (I.c < 0 || I.c > 9)) return -15;
+      reg_dtype[I.dst] = I.op == EW_CMPI ? (int)KO_I1 : reg_dtype[I.a];
+      break;
+    case EW_CMPF:
+      if (!reg_ok(I.a) || !reg_ok(I.b)) return -6;
+      if (reg_dtype[I.a] != reg_dtype[I.b] || !is_arith_float(reg_dtype[I.a])) return -10;
+      if (I.c < 0 || I.c > 15) return -15;
+      reg_dtype[I.dst] = KO_I1;
+      break;
+    case EW_ABSI:
+      if (!reg_ok(I.a) || !is_int_dtype(reg_dtype[I.a])) return -6;
+      reg_dtype[I.dst] = reg_dtype[I.a];
+      break;
+    case EW_TRUNCI: case EW_EXTSI: case EW_EXTUI: case EW_SITOFP: case EW_FPTOSI: case EW_BITCAST: {
+      if (!reg_ok(I.a)) return -6;
+      const int sd = reg_dtype[I.a], dd = I.dtype;
+      if (I.op == EW_TRUNCI && !(is_int_dtype(sd) && is_int_dtype(dd) && int_bits(dd) < int_bits(sd))) return -16;
+      if ((I.op == EW_EXTSI || I.op == EW_EXTUI) && !(is_int_dtype(sd) && is_int_dtype(dd) && int_bits(dd) > int_bits(sd))) return -16;
+      if (I.op == EW_SITOFP && !(is_int_dtype(sd) && is_arith_float(dd))) return -16;
+      if (I.op == EW_FPTOSI && !(is_arith_float(sd) && is_int_dtype(dd) && dd != KO_I1)) return -16;
+      if (I.op == EW_BITCAST && (sd == KO_I1 || dd == KO_I1 || dtype_bytes(sd) != dtype_bytes(dd) || dtype_bytes(dd) == 0)) return -16;
+      reg_dtype[I.dst] = dd;
+      break;
+    }
     case EW_FPTOFP: {
       if (!reg_ok(I.a)) return -6;
       int sd = reg_dtype[I.a], dd = I.dtype;
@@ -666,10 +793,11 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
       if (!reg_ok(I.a)) return -6;
       reg_dtype[I.dst] = reg_dtype[I.a];
     }
-    if (I.op != EW_ST_GLOBAL && I.op != EW_LD_GLOBAL && I.op != EW_FPTOFP) {
+    if (I.op != EW_ST_GLOBAL && I.op != EW_LD_GLOBAL && I.op != EW_FPTOFP && I.op != EW_SPLAT && I.op < EW_ADDI) {
       int d = reg_dtype[I.dst];
-      if (d != KO_F16 && d != KO_BF16 && d != KO_F32) return -12;  // arithmetic on f8/int registers is not defined
+      if (d != KO_F16 && d != KO_BF16 && d != KO_F32) return -12;  // float arithmetic on f8 / integer registers is not defined
     }
+    if (I.op == EW_FPTOFP && (is_int_dtype(reg_dtype[I.dst]) || is_int_dtype(reg_dtype[I.a] ))) return -12;
   }
   if (!has_store) return -13;
 
@@ -709,15 +837,52 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
     std::vector<double> dstv(I.op == EW_ST_GLOBAL ? 0 : total);
     int dst_dtype = -1;
     if (I.op == EW_LD_GLOBAL) dst_dtype = ins[I.a]->dtype;
-    else if (I.op == EW_SPLAT || I.op == EW_FPTOFP) dst_dtype = I.dtype;
+    else if (I.op == EW_SPLAT || I.op == EW_FPTOFP || (I.op >= EW_TRUNCI && I.op <= EW_BITCAST)) dst_dtype = I.dtype;
+    else if (I.op == EW_ARANGE) dst_dtype = KO_I32;
+    else if (I.op == EW_CMPI || I.op == EW_CMPF) dst_dtype = KO_I1;
+    else if (I.op == EW_SELECT) dst_dtype = rd[I.b];
     else if (I.op != EW_ST_GLOBAL) dst_dtype = rd[I.a];
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < o0; ++i) {
       for (int64_t j = 0; j < o1; ++j) {
         const int64_t at = i * o1 + j;
-        const double a = (I.op != EW_LD_GLOBAL && I.op != EW_SPLAT) ? reg[I.a][at] : 0.0;
+        const double a = (I.op != EW_LD_GLOBAL && I.op != EW_SPLAT && I.op != EW_ARANGE) ? reg[I.a][at] : 0.0;
         double r = 0.0;
+        if (I.op >= EW_ADDI && I.op <= EW_MINUI) {
+          dstv[at] = (double)int_binary_op(I.op, (int64_t)a, (int64_t)reg[I.b][at], dst_dtype);
+          continue;
+        }
         switch (I.op) {
+        case EW_ARANGE: dstv[at] = (double)int_wrap((int64_t)I.a + (I.b ? j : i), KO_I32); continue;
+        case EW_SELECT: dstv[at] = ((int64_t)a & 1) ? reg[I.b][at] : reg[I.c][at]; continue;
+        case EW_CMPI: dstv[at] = (double)int_compare_op(I.c, (int64_t)a, (int64_t)reg[I.b][at], rd[I.a]); continue;
+        case EW_CMPF: dstv[at] = (double)float_compare_op(I.c, a, reg[I.b][at]); continue;
+        case EW_ABSI: {
+          const int64_t v = int_as_signed((int64_t)a, dst_dtype);
+          dstv[at] = (double)int_wrap(v < 0 ? -v : v, dst_dtype);
+          continue;
+        }
+        case EW_TRUNCI: dstv[at] = (double)int_wrap((int64_t)a, dst_dtype); continue;
+        case EW_EXTSI: dstv[at] = (double)int_wrap(int_as_signed((int64_t)a, rd[I.a]), dst_dtype); continue;
+        case EW_EXTUI: dstv[at] = (double)int_wrap(int_as_unsigned((int64_t)a, rd[I.a]), dst_dtype); continue;
+        case EW_SITOFP: {  // one rounding to nearest even of the exact integer (a double holds any i32)
+          uint32_t tmp = 0;
+          ko_encode(&tmp, dst_dtype, 0, (double)int_as_signed((int64_t)a, rd[I.a]), KO_RN);
+          dstv[at] = ko_decode(&tmp, dst_dtype, 0);
+          continue;
+        }
+        case EW_FPTOSI: {
+          const double t = std::isnan(a) ? 0.0 : std::trunc(a);
+          const int64_t v = t >= 2147483647.0 ? 2147483647 : t <= -2147483648.0 ? -2147483648LL : (int64_t)t;
+          dstv[at] = (double)int_wrap(v, dst_dtype);
+          continue;
+        }
+        case EW_BITCAST: {  // through the memory image of the operand
+          uint32_t tmp = 0;
+          ko_encode(&tmp, rd[I.a], 0, a, KO_RN);
+          dstv[at] = ko_decode(&tmp, dst_dtype, 0);
+          continue;
+        }
         case EW_LD_GLOBAL: {
           const ko_global *g = ins[I.a];
           int64_t gi = extent0(g) == 1 && o0 != 1 ? 0 : i, gj = extent1(g) == 1 && o1 != 1 ? 0 : j;
@@ -729,7 +894,7 @@ int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *i
           dstv[at] = r;
           continue;
         }
-        case EW_SPLAT: dstv[at] = round_to((double)I.imm, I.dtype); continue;
+        case EW_SPLAT: dstv[at] = is_int_dtype(I.dtype) ? (double)int_wrap((int64_t)I.a, I.dtype) : round_to((double)I.imm, I.dtype); continue;
         case EW_FPTOFP: {
           bool down = dtype_bytes(I.dtype) < dtype_bytes(rd[I.a]);
           uint32_t tmp = 0;

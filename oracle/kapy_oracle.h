@@ -28,7 +28,7 @@ extern "C" {
 #endif
 
 /* dtype / enum numbering is shared with include/kapy_hip.h (enum values follow Enums.td). */
-enum { KO_F16 = 0, KO_BF16 = 1, KO_F32 = 2, KO_F8E4M3 = 3, KO_F8E5M2 = 4, KO_I8 = 5, KO_I16 = 6, KO_I32 = 7 };
+enum { KO_F16 = 0, KO_BF16 = 1, KO_F32 = 2, KO_F8E4M3 = 3, KO_F8E5M2 = 4, KO_I8 = 5, KO_I16 = 6, KO_I32 = 7, KO_I1 = 8 /* one byte, 0 or 1 */ };
 enum { KO_RZ = 0, KO_RN = 1 };
 enum { KO_PAD_ZERO = 0, KO_PAD_QNAN = 1, KO_PAD_PINF = 2, KO_PAD_NINF = 3 };
 

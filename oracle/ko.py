@@ -11,16 +11,22 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libkapy_oracle.so")
 
-F16, BF16, F32, F8E4M3, F8E5M2, I8, I16, I32 = range(8)
+F16, BF16, F32, F8E4M3, F8E5M2, I8, I16, I32, I1 = range(9)
 RZ, RN = 0, 1
 PAD_ZERO, PAD_QNAN, PAD_PINF, PAD_NINF = range(4)
-DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, F8E4M3: 1, F8E5M2: 1, I8: 1, I16: 2, I32: 4}
+DTYPE_BYTES = {F16: 2, BF16: 2, F32: 4, F8E4M3: 1, F8E5M2: 1, I8: 1, I16: 2, I32: 4, I1: 1}
 NP_STORAGE = {F16: np.uint16, BF16: np.uint16, F32: np.float32, F8E4M3: np.uint8, F8E5M2: np.uint8,
-              I8: np.int8, I16: np.int16, I32: np.int32}
+              I8: np.int8, I16: np.int16, I32: np.int32, I1: np.uint8}
 
 (EW_LD_GLOBAL, EW_SPLAT, EW_FPTOFP, EW_ADDF, EW_SUBF, EW_MULF, EW_DIVF, EW_FMA, EW_MAXIMUMF, EW_MINIMUMF,
  EW_NEGF, EW_ABSF, EW_EXP, EW_EXP2, EW_LOG, EW_LOG2, EW_SQRT, EW_RSQRT, EW_TANH, EW_ERF, EW_GELU_TANH,
  EW_ST_GLOBAL, EW_REDUCE_SUM, EW_REDUCE_MAX, EW_FLOOR, EW_CEIL, EW_SIN, EW_COS, EW_MAXNUMF, EW_MINNUMF, EW_REMF) = range(31)
+(EW_ADDI, EW_SUBI, EW_MULI, EW_DIVSI, EW_DIVUI, EW_FLOORDIVSI, EW_CEILDIVSI, EW_CEILDIVUI, EW_REMSI, EW_REMUI, EW_ANDI, EW_ORI, EW_XORI,
+ EW_SHLI, EW_SHRSI, EW_SHRUI, EW_MAXSI, EW_MAXUI, EW_MINSI, EW_MINUI, EW_ABSI, EW_CMPI, EW_CMPF, EW_SELECT, EW_TRUNCI, EW_EXTSI, EW_EXTUI,
+ EW_SITOFP, EW_FPTOSI, EW_BITCAST, EW_ARANGE) = range(31, 62)
+(CMPI_EQ, CMPI_NE, CMPI_SLT, CMPI_SLE, CMPI_SGT, CMPI_SGE, CMPI_ULT, CMPI_ULE, CMPI_UGT, CMPI_UGE) = range(10)
+(CMPF_FALSE, CMPF_OEQ, CMPF_OGT, CMPF_OGE, CMPF_OLT, CMPF_OLE, CMPF_ONE, CMPF_ORD, CMPF_UEQ, CMPF_UGT, CMPF_UGE, CMPF_ULT, CMPF_ULE, CMPF_UNE,
+ CMPF_UNO, CMPF_TRUE) = range(16)
 
 
 class Global(C.Structure):

@@ -57,6 +57,33 @@ static int run_cpu() {
   EXPECT(prog.size() == 6 && prog[2].op == KAPY_EW_MAXNUMF && prog[4].op == KAPY_EW_MINNUMF);
   prog = b.program_of(b.create_remf(b.create_floor(b.create_sin(lx)), b.create_ceil(b.create_cos(lx))));
   EXPECT(prog.size() == 7 && prog.back().op == KAPY_EW_ST_GLOBAL && prog[5].op == KAPY_EW_REMF);
+  // integer, compare and select builders: a causal mask (column <= row) in front of a select, as a program the library verifies
+  {
+    kapy::Value row = b.create_arange(0, 0, 64), colv = b.create_arange(1, 0, 256);
+    kapy::Value keep = b.create_cmpi_sle(colv, row);
+    kapy::Value masked = b.create_select(keep, lx, b.create_splat(0.f, KAPY_F16));
+    prog = b.program_of(masked, &ins);
+    EXPECT(prog.size() == 7 && ins.size() == 1 && prog[5].op == KAPY_EW_SELECT && prog.back().op == KAPY_EW_ST_GLOBAL);
+    int n_arange = 0, n_cmp = 0;
+    for (const kapy_ew_inst &I : prog) {
+      n_arange += I.op == KAPY_EW_ARANGE;
+      if (I.op == KAPY_EW_CMPI) { ++n_cmp; EXPECT(I.c == KAPY_CMPI_SLE); }
+    }
+    EXPECT(n_arange == 2 && n_cmp == 1);
+    const kapy_global *one[1] = {&ins[0]};
+    EXPECT(kapy_elementwise_source(prog.data(), (int32_t)prog.size(), one, 1, &out, nullptr, 0, &text, nullptr) == KAPY_OK && text > 1000);
+    // create_intcast picks the op from the widths; an integer splat carries its value in field a
+    kapy::Value wide = b.create_intcast(b.create_splat(-3, KAPY_I8), KAPY_I32, true);
+    prog = b.program_of(b.create_sitofp(b.create_addi(wide, b.create_intcast(b.create_splat(300, KAPY_I16), KAPY_I32, false)), KAPY_F16));
+    EXPECT(prog[0].op == KAPY_EW_SPLAT && prog[0].a == -3 && prog[1].op == KAPY_EW_EXTSI && prog[3].op == KAPY_EW_EXTUI && prog[4].op == KAPY_EW_ADDI);
+    EXPECT(kapy_elementwise_source(prog.data(), (int32_t)prog.size(), one, 0, &out, nullptr, 0, &text, nullptr) == KAPY_OK);
+    try {
+      b.create_st_global(b.create_select(lx, lx, lx), y);   // the condition is not an i1 tensor
+      EXPECT(!"a select on a float condition must be refused");
+    } catch (const kapy::Error &e) {
+      EXPECT(e.status == KAPY_ERR_VERIFY && strstr(e.what(), "i1"));
+    }
+  }
   // the verifier's refusal arrives as an exception with the reference's wording
   try {
     kapy::Value h = b.create_ld_global(x), w = b.create_ld_global(b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_BF16));

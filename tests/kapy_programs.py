@@ -222,6 +222,58 @@ def softmax_program(rows_per_warp=2, cols=256, num_warps=2, dtype="f16"):
             "  kapy.func public @softmax_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" + body + "  }\n}\n")
 
 
+def causal_softmax_program(rows_per_warp=2, cols=256, num_warps=2, dtype="f16"):
+    """out[r, :] = softmax over the columns c <= r of x[r, :] (zero elsewhere), in f32: the row index is kapy.arange along
+    axis 0 plus the tile's first row (an integer splat), the column index kapy.arange along axis 1, arith.cmpi sle makes the
+    i1 mask and arith.select puts -inf where it is false; then the softmax chain."""
+    t16, t32 = "tensor<%dx%dx%s" % (rows_per_warp, cols, dtype), "tensor<%dx%dxf32" % (rows_per_warp, cols)
+    ti, tb = "tensor<%dx%dxi32, #values>" % (rows_per_warp, cols), "tensor<%dx%dxi1, #values>" % (rows_per_warp, cols)
+    ri, ci = "tensor<%dx1xi32, #values>" % rows_per_warp, "tensor<1x%dxi32, #values>" % cols
+    c32 = "tensor<%dx1xf32, #values>" % rows_per_warp
+    dyn = "tensor<?x?x%s, #global>" % dtype
+    body = _consts([0, 1, rows_per_warp, rows_per_warp * num_warps, cols])
+    body += """    %pid = kapy.program_id {{axis = 0 : i32}} : i32
+    %warp = kapy.warp_id : i32
+    %p0 = arith.muli %pid, %c{rpp}_i32 : i32
+    %w0 = arith.muli %warp, %c{rpw}_i32 : i32
+    %row0 = arith.addi %p0, %w0 : i32
+    %row1 = arith.addi %row0, %c{rpw}_i32 : i32
+    %gx = kapy.mk_global %x[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %go = kapy.mk_global %out[%c0_i32] [%rows, %c{cols}_i32] [%c{cols}_i32, %c1_i32] : !kapy.ptr<1> -> {dyn}
+    %sx = kapy.sv_global %gx[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %so = kapy.sv_global %go[%row0 : %row1, %c0_i32 : %c{cols}_i32] : {dyn} -> {t16}, #global>
+    %x16 = kapy.ld_global %sx : {t16}, #global> -> {t16}, #values>
+    %xf = kapy.fptofp %x16 : {t16}, #values> to {t32}, #values>
+    %rl = kapy.arange {{axis = 0 : i32, start = 0 : i32, end = {rpw} : i32}} : {ri}
+    %rb = kapy.splat %row0 : i32 -> {ri}
+    %rg = arith.addi %rl, %rb : {ri}
+    %rr = kapy.broadcast %rg : {ri} -> {ti}
+    %cl = kapy.arange {{axis = 1 : i32, start = 0 : i32, end = {cols} : i32}} : {ci}
+    %cc = kapy.broadcast %cl : {ci} -> {ti}
+    %keep = arith.cmpi sle, %cc, %rr : {ti}
+    %ninf = arith.constant dense<0xFF800000> : {t32}, #values>
+    %xm = arith.select %keep, %xf, %ninf : {tb}, {t32}, #values>
+    %m = kapy.reduce %xm {{axis = 1 : i32}} lambda(%lhs: f32, %rhs: f32) {{
+      %r = arith.maximumf %lhs, %rhs : f32
+      kapy.return %r : f32
+    }} : {t32}, #values> -> {c32}
+    %mb = kapy.broadcast %m : {c32} -> {t32}, #values>
+    %d = arith.subf %xm, %mb : {t32}, #values>
+    %e = math.exp %d : {t32}, #values>
+    %s = kapy.reduce %e {{axis = 1 : i32}} lambda(%lhs: f32, %rhs: f32) {{
+      %r = arith.addf %lhs, %rhs : f32
+      kapy.return %r : f32
+    }} : {t32}, #values> -> {c32}
+    %sb = kapy.broadcast %s : {c32} -> {t32}, #values>
+    %q = arith.divf %e, %sb : {t32}, #values>
+    %y = kapy.fptofp %q {{rounding_mode = 1 : i32}} : {t32}, #values> to {t16}, #values>
+    kapy.st_global %y, %so : {t16}, #values>, {t16}, #global>
+    kapy.return
+""".format(rpp=rows_per_warp * num_warps, rpw=rows_per_warp, cols=cols, dyn=dyn, t16=t16, t32=t32, c32=c32, ti=ti, tb=tb, ri=ri, ci=ci)
+    return (HEADER + "module attributes {kapy.num_warps = %d : i64} {\n" % num_warps +
+            "  kapy.func public @causal_softmax_kernel(%x: !kapy.ptr<1>, %out: !kapy.ptr<1>, %rows: i32) {\n" + body + "  }\n}\n")
+
+
 def gated_program(rows_per_warp=4, cols=256, num_warps=2, dtype="f16"):
     """out[r, :] = silu(x[r, :]) * y[r, :] * g[r] in f32, rounded once: two casts up, negf, math.exp, a splat of 1.0, addf,
     divf, mulf, a broadcast of the per-row gate g ([rows x 1]), mulf, a cast down.  Eleven elementwise ops between the loads

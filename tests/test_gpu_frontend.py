@@ -109,6 +109,26 @@ def test_softmax_program_in_kapy_ops_matches_the_oracle_program(ko, monkeypatch,
     assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # in f32, one rounding to f16 at the end
 
 
+@pytest.mark.parametrize("fuse", ["1", "0"])
+def test_causal_masked_softmax_program_with_integer_tensor_ops(ko, monkeypatch, fuse):
+    """kapy.arange, an integer splat, arith.addi, arith.cmpi and arith.select on tensors in front of the softmax chain: fused, one
+    row program with integer registers (compiled on its first use); KAPY_MLIR_FUSE=0 runs every op by itself, the i32 and i1
+    tensors going through memory."""
+    monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+    rows_per_warp, cols, warps, programs = 2, 64, 2, 4
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 55, std=3.0)
+    dx, dout = to_dev(x), dev_zeros(rows * cols, 2, fill=0x7e00)
+    kh.run_mlir(kp.causal_softmax_program(rows_per_warp, cols, warps), [dx, dout, rows], [programs])
+    sync()
+    got = ko.decode(to_host(dout, np.uint16, (rows, cols)), ko.F16)
+    xf = ko.decode(x.reshape(rows, cols), ko.F16)
+    ref = np.where(np.tril(np.ones((rows, cols), bool)), xf, -np.inf)
+    ref = np.exp(ref - ref.max(axis=1, keepdims=True))
+    ref /= ref.sum(axis=1, keepdims=True)
+    assert not np.triu(got, 1).any() and np.abs(got - ref).max() <= 2.0 ** -10
+
+
 def _gated_insts():
     L, CAST, ST = kh.EW_LD_GLOBAL, kh.EW_FPTOFP, kh.EW_ST_GLOBAL
     return [dict(op=L, dst=0, a=0), dict(op=CAST, dst=0, a=0, dtype=kh.F32), dict(op=L, dst=1, a=1), dict(op=CAST, dst=1, a=1, dtype=kh.F32),

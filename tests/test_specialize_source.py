@@ -130,3 +130,23 @@ def test_code_objects_are_kept_in_the_cache_directory(tmp_path, monkeypatch):
     open(tmp_path / files[0], "wb").close()
     _, third = kh.elementwise_source(prog, *args, compile=True)
     assert third == first and os.path.getsize(tmp_path / files[0]) == first
+
+
+@pytest.mark.skipif(not _has_runtime_compiler(), reason="no libhiprtc on this machine")
+def test_integer_compare_select_and_arange_programs_compile():
+    """Programs with integer registers: a flat one over i32 operands with an i1 condition, and a causal-masked softmax (arange,
+    cmpi, select in front of the row reduces) on the row skeleton; both must compile to a gfx950 code object."""
+    flat = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=kh.EW_DIVSI, dst=2, a=0, b=1), dict(op=kh.EW_SHRSI, dst=2, a=2, b=1),
+            dict(op=kh.EW_CMPI, dst=3, a=2, b=0, c=kh.CMPI_ULT), dict(op=kh.EW_SPLAT, dst=4, dtype=kh.I32, a=-7), dict(op=kh.EW_SELECT, dst=5, a=3, b=2, c=4),
+            dict(op=kh.EW_SITOFP, dst=6, a=5, dtype=kh.BF16), dict(op=ST, a=6)]
+    src, code = kh.elementwise_source(kh.program(flat), [_g(16, 256, kh.I32), _g(1, 256, kh.I32)], _g(16, 256, kh.BF16), compile=True)
+    kernel = src[src.index('extern "C" __global__'):]
+    assert "int_binary(%d" % kh.EW_DIVSI in kernel and "int_compare(%d" % kh.CMPI_ULT in kernel and "convert_reg(%d" % kh.EW_SITOFP in kernel
+    assert "constexpr bool NARROW = false" in kernel and code > 0
+    rows = [dict(op=L, dst=0, a=0), dict(op=CAST, dst=1, a=0, dtype=kh.F32), dict(op=kh.EW_ARANGE, dst=2, a=0, b=0), dict(op=kh.EW_ARANGE, dst=3, a=0, b=1),
+            dict(op=kh.EW_CMPI, dst=4, a=3, b=2, c=kh.CMPI_SLE), dict(op=SPL, dst=5, dtype=kh.F32, imm=float("-inf")), dict(op=kh.EW_SELECT, dst=1, a=4, b=1, c=5),
+            dict(op=kh.EW_REDUCE_MAX, dst=6, a=1, b=1), dict(op=kh.EW_SUBF, dst=1, a=1, b=6), dict(op=kh.EW_EXP, dst=1, a=1), dict(op=kh.EW_REDUCE_SUM, dst=6, a=1, b=1),
+            dict(op=DIV, dst=1, a=1, b=6), dict(op=CAST, dst=7, a=1, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=7)]
+    src, code = kh.elementwise_source(kh.program(rows), [_g(64, 1024, kh.F16)], _g(64, 1024, kh.F16), compile=True)
+    kernel = src[src.index('extern "C" __global__'):]
+    assert "void kapy_ew_rows_" in kernel and "int_reg(0 + i)" in kernel and "threadIdx.x) * 8 + e)" in kernel and code > 0

@@ -339,7 +339,8 @@ def bench_reduce(kh, steps, warmup, cpu):
 
 
 def bench_reduce_cols(kh, steps, warmup, cpu):
-    """kapy.reduce along axis 0 (column sums) of the headline shape: strips x row chunks, a second launch folds the chunks."""
+    """kapy.reduce along axis 0 (column sums) of the headline shape: strips x row chunks in one launch, the last workgroup to arrive
+    at a strip folds its chunks."""
     import numpy as np
     import torch
     import ko
@@ -357,14 +358,14 @@ def bench_reduce_cols(kh, steps, warmup, cpu):
         raise CheckFailed("reduce along axis 0: max abs error %g" % err)
     wall, ev = _events(lambda i: kh.reduce(gx[i % sets], gy, 0, 0), steps, warmup)
     nbytes = n * n * 2 + n * 4
-    return {"workload": "reduce_sum axis=0 fp16 8192x8192 -> f32 [1x8192] (two launches; time of both)", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
-            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "reduce_cols"), "kernel": "reduce_cols_strip_kernel + reduce_partials_kernel",
+    return {"workload": "reduce_sum axis=0 fp16 8192x8192 -> f32 [1x8192]", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
+            "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "reduce_cols"), "kernel": "reduce_cols_strip_kernel (one launch: the last workgroup of a strip folds the row chunks)",
             "inputs": "x normal(0,1) seed 0", "checked": True, "check": "every column sum against fp64: max abs error %.2e" % err}
 
 
 def bench_softmax_cols(kh, steps, warmup, cpu):
-    """Softmax of every column as one program with two reduces along axis 0: three launches over the matrix (column maxima,
-    column sums of exp, the store), x read three times and y written once."""
+    """Softmax of every column as one program with two reduces along axis 0: two launches over the matrix (per-column maximum and
+    sum of exp with a running rescale, then the store), x read twice and y written once."""
     import numpy as np
     import torch
     import ko
@@ -389,11 +390,11 @@ def bench_softmax_cols(kh, steps, warmup, cpu):
     if worst > ULP_TOL:
         raise CheckFailed("column softmax: %d ulp against the checker" % worst)
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]], gy[i % sets]), steps, warmup)
-    nbytes = 4 * n * n * 2
+    nbytes = 2 * n * n * 2
     return {"workload": "softmax of every column, fp16 8192x8192, fp32 arithmetic (program with two reduces along axis 0)", "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, "softmax_cols"),
-            "kernel": "stack_colreduce_kernel x 2 + column_fold_kernel x 2 + stack_kernel_any", "inputs": "x normal(0,1) seed 0", "checked": True,
-            "check": "16 columns of the timed result against the checker: max %d ulp (tolerance %d); bytes = three reads and one write of the matrix" % (worst, ULP_TOL)}
+            "kernel": "col_softmax_stats_kernel + col_softmax_apply_kernel", "inputs": "x normal(0,1) seed 0", "checked": True,
+            "check": "16 columns of the timed result against the checker: max %d ulp (tolerance %d); bytes = one read and one write of the matrix (the two launches read it twice)" % (worst, ULP_TOL)}
 
 
 def bench_rowwise(kh, steps, warmup, cpu, which):
@@ -412,6 +413,14 @@ def bench_rowwise(kh, steps, warmup, cpu, which):
     hextra = []
     if which == "softmax":
         insts, extra = kh.softmax_insts(kh.F16), []
+    elif which == "causal_softmax":    # softmax over the columns j <= i of every row: arange, cmpi and select in front of the softmax chain
+        L, ST = kh.EW_LD_GLOBAL, kh.EW_ST_GLOBAL
+        insts, extra = [dict(op=L, dst=0, a=0), dict(op=kh.EW_FPTOFP, dst=1, a=0, dtype=kh.F32),
+                        dict(op=kh.EW_ARANGE, dst=2, a=0, b=0), dict(op=kh.EW_ARANGE, dst=3, a=0, b=1), dict(op=kh.EW_CMPI, dst=4, a=3, b=2, c=kh.CMPI_SLE),
+                        dict(op=kh.EW_SPLAT, dst=5, dtype=kh.F32, imm=float("-inf")), dict(op=kh.EW_SELECT, dst=1, a=4, b=1, c=5),
+                        dict(op=kh.EW_REDUCE_MAX, dst=6, a=1, b=1), dict(op=kh.EW_SUBF, dst=1, a=1, b=6), dict(op=kh.EW_EXP, dst=1, a=1),
+                        dict(op=kh.EW_REDUCE_SUM, dst=6, a=1, b=1), dict(op=kh.EW_DIVF, dst=1, a=1, b=6),
+                        dict(op=kh.EW_FPTOFP, dst=7, a=1, dtype=kh.F16, rmode=kh.RN), dict(op=ST, a=7)], []
     elif which == "l2norm_compiled":   # x / |x| per row: a row program without a hand-written kernel, compiled at run time
         f32 = dict(op=kh.EW_FPTOFP, dst=0, a=0, dtype=kh.F32)
         insts, extra = [dict(op=kh.EW_LD_GLOBAL, dst=0, a=0), f32, dict(op=kh.EW_MULF, dst=1, a=0, b=0), dict(op=kh.EW_REDUCE_SUM, dst=1, a=1, b=1),
@@ -427,15 +436,24 @@ def bench_rowwise(kh, steps, warmup, cpu, which):
     torch.cuda.synchronize()
     rows = _sample_rows(n, 16)
     hx = _host("normal", n * n, ko.F16, 0, 0).reshape(n, n)
-    xr, want = np.ascontiguousarray(hx[rows]), np.zeros((len(rows), n), np.uint16)
-    assert ko.elementwise(ko.program(insts), [ko.mk_global(xr, len(rows), n, n, 1, ko.F16)] + [ko.mk_global(h, 1, n, n, 1, ko.F16) for h in hextra],
-                          ko.mk_global(want, len(rows), n, n, 1, ko.F16)) == 0
+    if which == "causal_softmax":   # the mask depends on the row's index: a band of rows where they lie, through a sub-view of the whole matrix
+        r0 = 5000
+        rows = list(range(r0, r0 + 16))
+        full, want_full = ko.mk_global(hx, n, n, n, 1, ko.F16), np.zeros((n, n), np.uint16)
+        probe = [dict(i, a=r0) if i["op"] == kh.EW_ARANGE and i["b"] == 0 else i for i in insts]   # the band's first row as arange's start
+        assert ko.elementwise(ko.program(probe), [ko.sv_global(full, r0, r0 + 16, 0, n)], ko.sv_global(ko.mk_global(want_full, n, n, n, 1, ko.F16), r0, r0 + 16, 0, n)) == 0
+        want = want_full[rows]
+    else:
+        xr, want = np.ascontiguousarray(hx[rows]), np.zeros((len(rows), n), np.uint16)
+        assert ko.elementwise(ko.program(insts), [ko.mk_global(xr, len(rows), n, n, 1, ko.F16)] + [ko.mk_global(h, 1, n, n, 1, ko.F16) for h in hextra],
+                              ko.mk_global(want, len(rows), n, n, 1, ko.F16)) == 0
     worst = int(np.abs(_line16(_download(ys[0], np.uint16, (n, n))[rows]) - _line16(want)).max())
     if worst > ULP_TOL:
         raise CheckFailed("%s: %d ulp against the checker" % (which, worst))
     wall, ev = _events(lambda i: kh.elementwise(prog, [gx[i % sets]] + extra, gy[i % sets]), steps, warmup)
     nbytes = 2 * n * n * 2
-    name = "x * rsqrt(sum x^2) of every row, compiled at run time" if which == "l2norm_compiled" else "%s of every row" % which
+    name = {"l2norm_compiled": "x * rsqrt(sum x^2) of every row, compiled at run time",
+            "causal_softmax": "causal-masked softmax of every row (arange, cmpi, select + the softmax chain), compiled at run time"}.get(which, "%s of every row" % which)
     return {"workload": "%s, fp16 8192x8192, fp32 arithmetic" % name, "value": nbytes / (wall * 1e-3) / 1e9, "unit": "GB/s",
             "ms_per_step": wall, "kernel_ms": ev, "dtype": "f16", "roofline": _roof_hbm(nbytes, ev, which),
             "kernel": {"softmax": "softmax_kernel", "layernorm": "norm_kernel"}.get(which, "kapy_ew_rows_<hash> (compiled at run time)"),
@@ -866,7 +884,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
     return out
 
 
-WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "layernorm", "l2norm_compiled", "gelu_transposed",
+WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "causal_softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
              "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
 
 
@@ -902,6 +920,7 @@ def main():
         "reduce_cols": lambda s, w: bench_reduce_cols(kh, s, w, cpu),
         "softmax_cols": lambda s, w: bench_softmax_cols(kh, s, w, cpu),
         "softmax": lambda s, w: bench_rowwise(kh, s, w, cpu, "softmax"),
+        "causal_softmax": lambda s, w: bench_rowwise(kh, s, w, cpu, "causal_softmax"),
         "layernorm": lambda s, w: bench_rowwise(kh, s, w, cpu, "layernorm"),
         "l2norm_compiled": lambda s, w: bench_rowwise(kh, s, w, cpu, "l2norm_compiled"),
         "permute": lambda s, w: bench_permute(kh, s, w, cpu),

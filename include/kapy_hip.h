@@ -410,13 +410,42 @@ int kapy_matmul_scaled_f8(const kapy_global *a8, const kapy_global *w8, const fl
 int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const kapy_fragments *dst,
                 const int64_t shape[2], uint32_t *lane_values_out, void *stream);
 
-/* kapy.reduce with an addf / maximumf combiner along `axis` (Ops.td:441-457, ReduceOpToLLVM.cpp:51-172).
- * kind 0 = sum (fp32 accumulate), 1 = max.  dst has extent 1 along `axis`.  The elements themselves are folded, as the
- * lowering does (no identity element joins them): a line of only -0 sums to -0; max orders -0 below +0 and a NaN wins.
- * Launches that leave few results per workgroup share the reduced axis out over workgroups and fold fp32 partial results in
- * a second launch, in a fixed order (the same bits every run).  The partial results live in a 4 MiB block the library
- * allocates once per device at the first such call (hipMalloc: not while `stream` is being captured - then, and if the
- * allocation fails, the reduction runs in one pass); calls on different streams take turns at it through an event. */
+/* kapy.reduce along `axis` (Ops.td:441-457, ReduceOpToLLVM.cpp:51-172).  The op's combiner is a region; the regions that are
+ * one arith op are named here (what create_reduce's callers write: addf, maximumf ... xori).  dst has extent 1 along `axis`.
+ * The elements themselves are folded, as the lowering does (no identity element joins them): a line of only -0 sums to -0;
+ * maximumf / minimumf order -0 below +0 and a NaN wins, maxnumf / minnumf ignore NaNs unless every element is one. */
+typedef enum kapy_reduce_combiner {
+  KAPY_REDUCE_ADDF = 0, KAPY_REDUCE_MAXIMUMF = 1, KAPY_REDUCE_MINIMUMF = 2, KAPY_REDUCE_MULF = 3, KAPY_REDUCE_MAXNUMF = 4, KAPY_REDUCE_MINNUMF = 5,
+  KAPY_REDUCE_ADDI = 6, KAPY_REDUCE_MULI = 7, KAPY_REDUCE_MAXSI = 8, KAPY_REDUCE_MINSI = 9, KAPY_REDUCE_MAXUI = 10, KAPY_REDUCE_MINUI = 11,
+  KAPY_REDUCE_ANDI = 12, KAPY_REDUCE_ORI = 13, KAPY_REDUCE_XORI = 14
+} kapy_reduce_combiner;
+typedef enum kapy_reduce_arithmetic {
+  KAPY_REDUCE_WIDE = 0,      /* float combiners fold in fp32 and round once to dst's type (any of f16, bf16, f32); the order of the
+                                additions is the library's, fixed for a given call (the same bits every run)                   */
+  KAPY_REDUCE_REFERENCE = 1  /* the lowering's own arithmetic on one wavefront's tile: every combiner application is an op on the
+                                ELEMENT type (an f16 addf rounds each partial sum to f16), each lane folds the elements it holds
+                                under `layout` in loop order, then the lanes that share a reduced line fold by butterfly
+                                exchanges at lane distances laneOffset * 2^i, i = 0, 1, ... (ReduceOpToLLVM.cpp:76-119, laneOffset
+                                and the number of rounds from LayoutUtils.cpp:26-49) - on 64 lanes here.  src must be a
+                                power-of-two tile, dst of src's element type                                                  */
+} kapy_reduce_arithmetic;
+typedef struct kapy_reduce_cfg {
+  int32_t combiner;        /* kapy_reduce_combiner; the integer ones need i8 / i16 / i32 tensors, dst of src's type                */
+  int32_t arithmetic;      /* kapy_reduce_arithmetic                                                                              */
+  const kapy_fragments *layout; /* REFERENCE: how the tile sits in the wavefront's registers; NULL = the default layout of
+                                LayoutUtils.cpp:92-110 for a row-major tile on 64 lanes                                          */
+  void *workspace;         /* device memory for partial results and arrival counters of launches that share a reduced axis out over
+                              workgroups, or NULL: then a 4 MiB + 16 KiB array in the library's device image serves, which every
+                              call on that GPU without a workspace shares - such calls must not overlap in time (streams that run
+                              concurrently: give each a workspace).  The first 16 KiB (the counters) must be zero before the
+                              first use; every call leaves them zero                                                            */
+  int64_t workspace_bytes; /* kapy_reduce_workspace_bytes() is enough for any call; with less the library shares out less        */
+} kapy_reduce_cfg;
+/* Everything on `stream`, nothing allocated, no host-side state: a workgroup that owns part of a reduced line leaves an fp32
+ * partial result in the workspace and counts itself; the last to arrive folds the partials in a fixed order. */
+int kapy_reduce_ex(const kapy_global *src, const kapy_global *dst, int32_t axis, const kapy_reduce_cfg *cfg, void *stream);
+int64_t kapy_reduce_workspace_bytes(void);
+/* kapy_reduce_ex with combiner = kind (0 = addf, 1 = maximumf, ...), WIDE arithmetic and the library's own workspace array. */
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream);
 
 /* Static plan of a workgroup's shared memory (lib/Analysis/AllocAnalysis.cpp:187-270): buffers whose live

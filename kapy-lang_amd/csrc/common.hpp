@@ -80,11 +80,12 @@ int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_d
                        char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes);
 
 int check_global(const kapy_global *g, const char *what);
-// A block of device memory the library keeps per device for partial results of reductions (wave_ops.hip): acquire hands it
-// out for work on `stream` with a lock held (nullptr, and no lock, while the stream is being captured or without memory),
-// release after the last launch that touches it.
-float *partials_acquire(hipStream_t stream, size_t *bytes);
-int partials_release(hipStream_t stream);
+// The partial-line part (bytes: its size) of the array in the library's device image that serves reductions without a
+// caller's workspace (wave_ops.hip), or nullptr; calls that use it must not overlap in time on one GPU.
+float *reduce_scratch_lines(size_t *bytes, uint32_t **counters = nullptr);   // counters: the array's arrival counters (4096 words, zero between calls)
+// softmax of every column of a 16-bit row-major matrix in two launches (elementwise_col.hip): 1 = launched, 0 = the shapes
+// are not the kernels', a negative status on failure.
+int run_column_softmax(const kapy_global *x, const kapy_global *out, hipStream_t stream);
 int ensure_device();
 int device_cus();
 

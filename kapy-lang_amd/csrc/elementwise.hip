@@ -856,14 +856,14 @@ bool stream_is_capturing(hipStream_t s);
 // elementwise program of its own - the instructions reduce p depends on, with every earlier reduce replaced by a load of
 // that reduce's per-column results ([1 x n], in the reduce's type) - whose value is folded over rows instead of stored
 // (stack_colreduce_kernel over strips x row chunks, then column_fold_kernel); the last phase is an ordinary
-// kapy_elementwise call with the results as row operands.  The results and the partial lines live in the block of
-// partials_acquire.  Returns 1 when the program ran this way, 0 when it does not fit (the caller then runs the one-launch
+// kapy_elementwise call with the results as row operands.  The results and the partial lines live in the library's own
+// workspace array (reduce_scratch_lines: calls that use it must not overlap in time on one GPU).  Returns 1 when the program ran this way, 0 when it does not fit (the caller then runs the one-launch
 // column machine, which takes any views), a negative status on failure.
 int run_column_phases(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
                       const ColumnPlan &C, const Program &P, hipStream_t s) {
   const int n_reduce = C.n_phases - 1;
   const int64_t m = extent0(out), n = extent1(out);
-  if (n % 8 != 0 || out->stride1 != 1 || n_ins + n_reduce > kMaxInputs || m < 64 || stream_is_capturing(s)) return 0;
+  if (n % 8 != 0 || out->stride1 != 1 || n_ins + n_reduce > kMaxInputs || m < 64) return 0;
   // phase programs, built before anything is launched: any that does not fit the stack machine sends the whole call back
   struct Phase {
     kapy_ew_inst inst[kMaxInst + 1];
@@ -899,12 +899,9 @@ int run_column_phases(const kapy_ew_inst *prog, int n_inst, const int *result_dt
     }
   }
   size_t bytes = 0;
-  float *block = partials_acquire(s, &bytes);
+  float *block = reduce_scratch_lines(&bytes);
   if (!block) return 0;
-  auto give_up = [&](int rc) {
-    (void)partials_release(s);
-    return rc;
-  };
+  auto give_up = [&](int rc) { return rc; };
   // [results of up to four reduces, 4 bytes per column each][partial lines]
   const int64_t floats = (int64_t)(bytes / sizeof(float)), left = floats / n - kMaxColumnReduces;
   if (left < 1) return give_up(0);
@@ -956,13 +953,58 @@ int run_column_phases(const kapy_ew_inst *prog, int n_inst, const int *result_dt
   }
   const Phase &L = phases[n_reduce];
   int rc = kapy_elementwise(L.inst, L.n, all, n_ins + n_reduce, out, (void *)s);
-  const int released = partials_release(s);
-  if (rc) return rc;
-  return released ? released : 1;
+  return rc ? rc : 1;
+}
+
+// st(fptofp_rn[T](divf(E, reduce_sum0(E)))), E = exp(subf(F, reduce_max0(F))), F = extf(ld x): the input's index, or -1
+int match_column_softmax(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *out) {
+  struct N { int op, a = -1, b = -1, dtype = -1, rmode = KAPY_RN, input = -1, axis = 0; };
+  std::vector<N> nodes;
+  int reg[kMaxRegs];
+  for (int r = 0; r < kMaxRegs; ++r) reg[r] = -1;
+  int stored = -1, n_store = 0;
+  for (int k = 0; k < n_inst; ++k) {
+    const kapy_ew_inst &I = prog[k];
+    N n;
+    n.op = I.op;
+    n.dtype = result_dtype[k];
+    n.rmode = I.rmode;
+    switch (I.op) {
+    case KAPY_EW_LD_GLOBAL: n.input = I.a; if (I.c != KAPY_PAD_ZERO) return -1; break;
+    case KAPY_EW_ST_GLOBAL: stored = reg[I.a]; ++n_store; continue;
+    case KAPY_EW_FPTOFP: case KAPY_EW_EXP: n.a = reg[I.a]; break;
+    case KAPY_EW_REDUCE_SUM: case KAPY_EW_REDUCE_MAX: n.a = reg[I.a]; n.axis = I.b; break;
+    case KAPY_EW_SUBF: case KAPY_EW_DIVF: n.a = reg[I.a]; n.b = reg[I.b]; break;
+    default: return -1;
+    }
+    nodes.push_back(n);
+    reg[I.dst] = (int)nodes.size() - 1;
+  }
+  const int T = out->dtype;
+  if (n_store != 1 || stored < 0 || (T != KAPY_F16 && T != KAPY_BF16)) return -1;
+  auto is = [&](int id, int op) { return id >= 0 && nodes[id].op == op && (op == KAPY_EW_LD_GLOBAL || nodes[id].dtype == KAPY_F32); };
+  const N &st = nodes[stored];
+  if (st.op != KAPY_EW_FPTOFP || st.dtype != T || st.rmode == KAPY_RZ || !is(st.a, KAPY_EW_DIVF)) return -1;
+  const int e = nodes[st.a].a, rs = nodes[st.a].b;
+  if (!is(rs, KAPY_EW_REDUCE_SUM) || nodes[rs].axis != 0 || nodes[rs].a != e || !is(e, KAPY_EW_EXP)) return -1;
+  const int sub = nodes[e].a;
+  if (!is(sub, KAPY_EW_SUBF)) return -1;
+  const int f = nodes[sub].a, rm = nodes[sub].b;
+  if (!is(rm, KAPY_EW_REDUCE_MAX) || nodes[rm].axis != 0 || nodes[rm].a != f || !is(f, KAPY_EW_FPTOFP)) return -1;
+  const int ld = nodes[f].a;
+  if (ld < 0 || nodes[ld].op != KAPY_EW_LD_GLOBAL || nodes[ld].dtype != T) return -1;
+  return nodes[ld].input;
 }
 
 int run_column_program(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
                        hipStream_t s) {
+  {  // the softmax of every column has kernels of its own
+    const int x_in = match_column_softmax(prog, n_inst, result_dtype, out);
+    if (x_in >= 0 && x_in < n_ins) {
+      const int ran = run_column_softmax(ins[x_in], out, s);
+      if (ran != 0) return ran < 0 ? ran : KAPY_OK;
+    }
+  }
   Program P;
   memset(&P, 0, sizeof P);
   ColumnPlan C;

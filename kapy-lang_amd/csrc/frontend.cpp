@@ -1198,17 +1198,29 @@ struct Interp {
       return KAPY_OK;
     }
     if (n == "kapy.reduce") {
-      int kind = -1;
+      // the combiner region: one arith op on the two block arguments (what kapy_reduce_combiner names)
+      static const struct { const char *name; int kind; } combiners[] = {
+          {"arith.addf", KAPY_REDUCE_ADDF}, {"arith.maximumf", KAPY_REDUCE_MAXIMUMF}, {"arith.minimumf", KAPY_REDUCE_MINIMUMF}, {"arith.mulf", KAPY_REDUCE_MULF},
+          {"arith.maxnumf", KAPY_REDUCE_MAXNUMF}, {"arith.minnumf", KAPY_REDUCE_MINNUMF}, {"arith.addi", KAPY_REDUCE_ADDI}, {"arith.muli", KAPY_REDUCE_MULI},
+          {"arith.maxsi", KAPY_REDUCE_MAXSI}, {"arith.minsi", KAPY_REDUCE_MINSI}, {"arith.maxui", KAPY_REDUCE_MAXUI}, {"arith.minui", KAPY_REDUCE_MINUI},
+          {"arith.andi", KAPY_REDUCE_ANDI}, {"arith.ori", KAPY_REDUCE_ORI}, {"arith.xori", KAPY_REDUCE_XORI}};
+      int kind = -1, n_ops = 0;
       for (const Op &inner : op.body) {
-        if (inner.name == "arith.addf") kind = 0;
-        if (inner.name == "arith.maximumf") kind = 1;
+        if (inner.name == "kapy.return") continue;
+        ++n_ops;
+        for (auto &c : combiners)
+          if (inner.name == c.name) kind = c.kind;
       }
-      if (kind < 0) return fail_op(op, "only addf and maximumf combiners are supported");
+      if (kind < 0 || n_ops != 1) return fail_op(op, "the combiner must be one arith op (addf, maximumf, minimumf, mulf, maxnumf, minnumf or an integer op)");
       int axis = op.attrs.count("axis") ? atoi(op.attrs.at("axis").c_str()) : 0;
+      // KAPY_MLIR_REDUCE=reference: the lowering's own arithmetic for the warp's tile (partial results on the element type, lane-serial
+      // fold then butterfly, ReduceOpToLLVM.cpp:76-119) instead of fp32 accumulation; such a reduce is a call of its own
+      const char *reduce_mode = getenv("KAPY_MLIR_REDUCE");
+      const bool reference = reduce_mode && std::string(reduce_mode) == "reference";
       // over a register tensor the reduce joins the deferred chain: followed by a broadcast back to the operand's shape it
       // becomes an instruction of the program that consumes it (along rows: the row programs; along columns: the column machine)
       auto src = op.operands.empty() ? env.end() : env.find(op.operands[0]);
-      if (fuse && (axis == 0 || axis == 1) && !op.types.empty() && op.types.back().kind == Type::kTensor && src != env.end() &&
+      if (fuse && !reference && kind <= KAPY_REDUCE_MAXIMUMF && (axis == 0 || axis == 1) && !op.types.empty() && op.types.back().kind == Type::kTensor && src != env.end() &&
           src->second.kind == Value::kTensor && (src->second.lazy || is_register_tensor(src->second.g))) {
         const kapy_global &sg = src->second.g;
         const Type &ty = op.types.back();
@@ -1232,7 +1244,8 @@ struct Interp {
         }
       }
       if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
-      int rc = lib(op, kapy_reduce(&a.g, &r.g, axis, kind, stream));
+      kapy_reduce_cfg rcfg = {kind, reference ? KAPY_REDUCE_REFERENCE : KAPY_REDUCE_WIDE, nullptr, nullptr, 0};
+      int rc = lib(op, kapy_reduce_ex(&a.g, &r.g, axis, &rcfg, stream));
       if (rc) return rc;
       env[op.results[0]] = r;
       return KAPY_OK;

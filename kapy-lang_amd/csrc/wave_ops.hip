@@ -7,7 +7,6 @@
 // ReduceOpToLLVM.cpp:51-172 — an in-lane tree over the loop ivs, then shfl.sync.bfly rounds over
 // the lanes that share the reduced axis.  On gfx950 the shuffles are ds_bpermute_b32 over 64 lanes.
 #include <algorithm>
-#include <mutex>
 
 #include "common.hpp"
 #include "layout.hpp"
@@ -40,35 +39,98 @@ struct ReduceParams {
   int64_t s_keep, s_red;  // source strides along the kept and the reduced axis
   int64_t d_keep;         // result stride along the kept axis
   int32_t n_keep, n_red;
-  int32_t src_dtype, dst_dtype, kind;
+  int32_t src_dtype, dst_dtype, kind;  // kind: kapy_reduce_combiner
 };
 
+// What a fold starts from so that the elements themselves decide the result (ReduceOpToLLVM.cpp:60-101 folds the elements,
+// no identity joins them): -0 for a sum (-0 + x = x for every x, -0 included, so a line of only -0 sums to -0), the
+// infinities for maximumf / minimumf, NaN for maxnumf / minnumf (ignored unless every element is one), 1 for a product;
+// for the integer combiners the usual neutral elements, as containers.
+__device__ __forceinline__ float identity_of(int kind, int dtype) {
+  switch (kind) {
+  case KAPY_REDUCE_ADDF: return -0.f;
+  case KAPY_REDUCE_MAXIMUMF: return -__builtin_inff();
+  case KAPY_REDUCE_MINIMUMF: return __builtin_inff();
+  case KAPY_REDUCE_MULF: return 1.f;
+  case KAPY_REDUCE_MAXNUMF: case KAPY_REDUCE_MINNUMF: return __builtin_nanf("");
+  case KAPY_REDUCE_MULI: return int_reg(int_canon(1, dtype));
+  case KAPY_REDUCE_MAXSI: return int_reg(int_canon(dtype == KAPY_I8 ? -128 : dtype == KAPY_I16 ? -32768 : (int32_t)0x80000000u, dtype));
+  case KAPY_REDUCE_MINSI: return int_reg(int_canon(dtype == KAPY_I8 ? 127 : dtype == KAPY_I16 ? 32767 : 0x7FFFFFFF, dtype));
+  case KAPY_REDUCE_MINUI: case KAPY_REDUCE_ANDI: return int_reg(int_canon(-1, dtype));
+  default: return int_reg(0);  // addi, maxui, ori, xori
+  }
+}
+// float combiners on fp32 values; -0 orders below +0 for the four orderings (fmaxf / fminf do that on this device)
 __device__ __forceinline__ float combine(float a, float b, int kind) {
-  if (kind == 0) return a + b;
-  return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b);
+  switch (kind) {
+  case KAPY_REDUCE_ADDF: return a + b;
+  case KAPY_REDUCE_MAXIMUMF: return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b);
+  case KAPY_REDUCE_MINIMUMF: return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b);
+  case KAPY_REDUCE_MULF: return a * b;
+  case KAPY_REDUCE_MAXNUMF: return a != a ? b : b != b ? a : fmaxf(a, b);
+  default: return a != a ? b : b != b ? a : fminf(a, b);
+  }
+}
+// any combiner, integer ones on containers of element type dtype
+__device__ __forceinline__ float combine_any(float a, float b, int kind, int dtype) {
+  if (kind < KAPY_REDUCE_ADDI) return combine(a, b, kind);
+  constexpr int op_of[] = {KAPY_EW_ADDI, KAPY_EW_MULI, KAPY_EW_MAXSI, KAPY_EW_MINSI, KAPY_EW_MAXUI, KAPY_EW_MINUI, KAPY_EW_ANDI, KAPY_EW_ORI, KAPY_EW_XORI};
+  return int_reg(int_binary(op_of[kind - KAPY_REDUCE_ADDI], reg_int(a), reg_int(b), dtype));
+}
+// the vector kernels are built twice: KIND 0 adds, KIND 1 reads the (float) combiner from the parameters
+template <int KIND>
+__device__ __forceinline__ float combine_t(float a, float b, int kind) { return KIND == 0 ? a + b : combine(a, b, kind); }
+
+// ---- sharing a reduced axis out over workgroups -----------------------------------------------------------------------
+// Every workgroup that owns a chunk of a line leaves fp32 partial results in `lines` and counts itself at the line group's
+// counter; the one that arrives last folds the partials in chunk order (the same bits every run) and stores the result,
+// then sets the counter back to zero.  Nobody waits for anybody.  The partials cross XCDs, whose L2 caches are not coherent
+// with each other: they are written and read with relaxed device-scope accesses (which go past the L2), every lane waits
+// until its stores have been acknowledged before the workgroup counts itself, and the reader starts only after its count
+// has come back.
+constexpr int kCounterBytes = 16 << 10, kMaxGroups = kCounterBytes / 4;
+constexpr size_t kScratchLineBytes = size_t(4) << 20;
+struct Shared {
+  float *lines = nullptr;
+  uint32_t *counters = nullptr;
+  int64_t floats = 0;
+};
+__device__ __forceinline__ void partial_store(float *at, float v) {
+  __hip_atomic_store((uint32_t *)at, f32_bits(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float partial_load(const float *at) {
+  return bits_f32(__hip_atomic_load((const uint32_t *)at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+// true in the workgroup that arrived last of `parts` at `counter` (all lanes get the same answer); `word`: 4 bytes of LDS
+__device__ __forceinline__ bool arrived_last(uint32_t *counter, uint32_t parts, uint32_t *word) {
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this lane's partial results have been acknowledged (lgkmcnt, expcnt: no wait)
+  __syncthreads();
+  if (threadIdx.x == 0) *word = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const bool last = *word == parts - 1;
+  __syncthreads();
+  return last;
 }
 
-// A sum starts from -0, the identity of IEEE addition (-0 + x = x for every x, -0 included): the result is that of folding
-// the elements themselves, as ReduceOpToLLVM.cpp:60-101 does, and a line of only -0 sums to -0.
-// One wavefront per kept index: lanes stride over the reduced axis, then 6 butterfly rounds.
+// One wavefront per kept index: lanes stride over the reduced axis, then 6 butterfly rounds.  Any element type and strides.
 __global__ __launch_bounds__(256) void reduce_wave_kernel(ReduceParams p) {
   const int lane = threadIdx.x & 63;
   const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (keep >= p.n_keep) return;
-  float acc = p.kind == 0 ? -0.f : -__builtin_inff();
+  float acc = identity_of(p.kind, p.src_dtype);
   int32_t r = lane;
   for (; r + 192 < p.n_red; r += 256) {  // four loads in flight
     float f[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) f[u] = load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)(r + 64 * u) * p.s_red);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) acc = combine(acc, f[u], p.kind);
+    for (int u = 0; u < 4; ++u) acc = combine_any(acc, f[u], p.kind, p.src_dtype);
   }
-  for (; r < p.n_red; r += 64) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)r * p.s_red), p.kind);
+  for (; r < p.n_red; r += 64) acc = combine_any(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)r * p.s_red), p.kind, p.src_dtype);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
     float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(acc)));
-    acc = combine(acc, other, p.kind);
+    acc = combine_any(acc, other, p.kind, p.src_dtype);
   }
   if (lane == 0) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
 }
@@ -97,49 +159,68 @@ __device__ __forceinline__ void widen(u32x4_t v, float (&f)[per_vec<SRC>()]) {
   }
 }
 // the values of one load folded as a tree
-template <int SRC>
-__device__ __forceinline__ float fold_vec(const float (&f)[per_vec<SRC>()], int kind) {
-  if constexpr (SRC == 2) return combine(combine(f[0], f[1], kind), combine(f[2], f[3], kind), kind);
-  else return combine(combine(combine(f[0], f[1], kind), combine(f[2], f[3], kind), kind), combine(combine(f[4], f[5], kind), combine(f[6], f[7], kind), kind), kind);
-}
 template <int SRC, int KIND>
-__global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p, float *partials, int32_t vecs_per_chunk) {
+__device__ __forceinline__ float fold_vec(const float (&f)[per_vec<SRC>()], int kind) {
+  if constexpr (SRC == 2) return combine_t<KIND>(combine_t<KIND>(f[0], f[1], kind), combine_t<KIND>(f[2], f[3], kind), kind);
+  else return combine_t<KIND>(combine_t<KIND>(combine_t<KIND>(f[0], f[1], kind), combine_t<KIND>(f[2], f[3], kind), kind),
+                              combine_t<KIND>(combine_t<KIND>(f[4], f[5], kind), combine_t<KIND>(f[6], f[7], kind), kind), kind);
+}
+// Four lines per workgroup, one wave each; gridDim.y > 1: a wave folds one chunk of its line, and the workgroup that is last
+// to arrive for these four lines folds the chunks' partial results (lane c holds chunk c, c + 64, ..., then the butterfly).
+template <int SRC, int KIND>
+__global__ __launch_bounds__(256) void reduce_rows_vec_kernel(ReduceParams p, Shared sh, int32_t vecs_per_chunk) {
+  __shared__ uint32_t word;
   const int lane = threadIdx.x & 63;
   const int64_t keep = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (keep >= p.n_keep) return;
   constexpr int E = per_vec<SRC>();
-  const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * (16 / E));
-  const int32_t vecs = min(p.n_red / E, (int32_t)(blockIdx.y + 1) * vecs_per_chunk);
-  float acc = KIND == 0 ? -0.f : -__builtin_inff();
-  constexpr int U = 4;
-  int32_t v = blockIdx.y * vecs_per_chunk + lane;
-  for (; v + 64 * (U - 1) < vecs; v += 64 * U) {
-    u32x4_t x[U];
+  const int32_t chunks = gridDim.y;
+  float acc = identity_of(p.kind, p.src_dtype);
+  if (keep < p.n_keep) {
+    const u32x4_t *row = (const u32x4_t *)(p.src + keep * p.s_keep * (16 / E));
+    const int32_t vecs = min(p.n_red / E, (int32_t)(blockIdx.y + 1) * vecs_per_chunk);
+    constexpr int U = 4;
+    int32_t v = blockIdx.y * vecs_per_chunk + lane;
+    for (; v + 64 * (U - 1) < vecs; v += 64 * U) {
+      u32x4_t x[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(row + v + 64 * u);
+      for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(row + v + 64 * u);
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+      for (int u = 0; u < U; ++u) {
+        float f[E];
+        widen<SRC>(x[u], f);
+        const float t = fold_vec<SRC, KIND>(f, p.kind);
+        acc = combine_t<KIND>(acc, t, p.kind);
+      }
+    }
+    for (; v < vecs; v += 64) {
       float f[E];
-      widen<SRC>(x[u], f);
-      const float t = fold_vec<SRC>(f, KIND);
-      acc = combine(acc, t, KIND);
+      widen<SRC>(__builtin_nontemporal_load(row + v), f);
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc = combine_t<KIND>(acc, f[e], p.kind);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(acc)));
+      acc = combine_t<KIND>(acc, other, p.kind);
     }
   }
-  for (; v < vecs; v += 64) {
-    float f[E];
-    widen<SRC>(__builtin_nontemporal_load(row + v), f);
+  if (chunks == 1) {
+    if (lane == 0 && keep < p.n_keep) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
+    return;
+  }
+  if (lane == 0 && keep < p.n_keep) partial_store(sh.lines + keep * chunks + blockIdx.y, acc);
+  if (!arrived_last(sh.counters + blockIdx.x, (uint32_t)chunks, &word)) return;
+  if (keep < p.n_keep) {
+    float t = identity_of(p.kind, p.src_dtype);
+    for (int32_t c = lane; c < chunks; c += 64) t = combine_t<KIND>(t, partial_load(sh.lines + keep * chunks + c), p.kind);
 #pragma unroll
-    for (int e = 0; e < E; ++e) acc = combine(acc, f[e], KIND);
+    for (int off = 32; off >= 1; off >>= 1) {
+      float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(t)));
+      t = combine_t<KIND>(t, other, p.kind);
+    }
+    if (lane == 0) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
   }
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ off) << 2, (int)f32_bits(acc)));
-    acc = combine(acc, other, KIND);
-  }
-  if (lane == 0) {
-    if (partials) partials[keep * gridDim.y + blockIdx.y] = acc;
-    else store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
-  }
+  if (threadIdx.x == 0) __hip_atomic_store(sh.counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The same for lines of up to 512 elements: a line takes GROUP lanes (8, 16, 32 or 64: the next power of two from its
@@ -148,36 +229,71 @@ template <int SRC, int KIND, int GROUP>
 __global__ __launch_bounds__(256) void reduce_rows_short_kernel(ReduceParams p) {
   const int64_t keep = (int64_t)blockIdx.x * (256 / GROUP) + threadIdx.x / GROUP;
   const int32_t jv = threadIdx.x % GROUP;
-  float acc = KIND == 0 ? -0.f : -__builtin_inff();
+  float acc = identity_of(p.kind, p.src_dtype);
   constexpr int E = per_vec<SRC>();
   if (keep < p.n_keep && jv < p.n_red / E) {
     float f[E];
     widen<SRC>(__builtin_nontemporal_load((const u32x4_t *)(p.src + keep * p.s_keep * (16 / E)) + jv), f);
-    acc = fold_vec<SRC>(f, KIND);
+    acc = fold_vec<SRC, KIND>(f, p.kind);
   }
 #pragma unroll
   for (int off = GROUP / 2; off >= 1; off >>= 1) {
     float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute(((threadIdx.x & 63) ^ off) << 2, (int)f32_bits(acc)));
-    acc = combine(acc, other, KIND);
+    acc = combine_t<KIND>(acc, other, p.kind);
   }
   if (jv == 0 && keep < p.n_keep) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, acc);
 }
 
-// 16-bit elements, kept axis contiguous: a workgroup of 256 lanes owns a strip of 8 * LPR kept indices - LPR lanes x one
-// 128-bit load per reduced index - and a chunk of the reduced axis, which its 256 / LPR groups of lanes walk with four
+// The last-arrived workgroup's fold of `chunks` partial lines for COLS kept indices starting at keep0: the 256 lanes form
+// 256 / COLS groups that take chunks g, g + groups, ... (sixteen loads in flight per lane), the groups meet in LDS and are
+// folded in group order.  part: [256 / COLS][COLS + 1] floats.
+template <int COLS, int KIND>
+__device__ __forceinline__ void fold_partial_lines(const ReduceParams &p, const Shared &sh, int64_t keep0, int32_t chunks, float *part) {
+  constexpr int GROUPS = 256 / COLS;
+  const int cl = threadIdx.x % COLS, g = threadIdx.x / COLS;
+  const int64_t keep = keep0 + cl;
+  float t = identity_of(p.kind, p.src_dtype);
+  if (keep < p.n_keep) {
+    int32_t c = g;
+    constexpr int U = 16;
+    for (; c + GROUPS * (U - 1) < chunks; c += GROUPS * U) {
+      float x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = partial_load(sh.lines + (int64_t)(c + GROUPS * u) * p.n_keep + keep);
+#pragma unroll
+      for (int u = 0; u < U; ++u) t = combine_t<KIND>(t, x[u], p.kind);
+    }
+    for (; c < chunks; c += GROUPS) t = combine_t<KIND>(t, partial_load(sh.lines + (int64_t)c * p.n_keep + keep), p.kind);
+  }
+  if (GROUPS > 1) {
+    part[g * (COLS + 1) + cl] = t;
+    __syncthreads();
+    if (g == 0) {
+      t = part[cl];
+#pragma unroll
+      for (int k = 1; k < GROUPS; ++k) t = combine_t<KIND>(t, part[k * (COLS + 1) + cl], p.kind);
+    }
+  }
+  if (g == 0 && keep < p.n_keep) store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
+}
+
+// 16-bit or f32 elements, kept axis contiguous: a workgroup of 256 lanes owns a strip of E * LPR kept indices - LPR lanes x
+// one 128-bit load per reduced index - and a chunk of the reduced axis, which its 256 / LPR groups of lanes walk with four
 // loads in flight each; the groups' partial results meet in LDS.  With one chunk the strip's results go to the result;
 // with more (few kept indices, many reduced ones: a tall matrix would otherwise keep a handful of CUs busy) every chunk
-// leaves an fp32 partial line and reduce_partials_kernel folds the lines in chunk order.
+// leaves an fp32 partial line and the strip's last workgroup to arrive folds the lines in chunk order.
 template <int SRC, int KIND, int LPR>
-__global__ __launch_bounds__(256) void reduce_cols_strip_kernel(ReduceParams p, float *partials, int32_t per_chunk) {
+__global__ __launch_bounds__(256) void reduce_cols_strip_kernel(ReduceParams p, Shared sh, int32_t per_chunk) {
   constexpr int E = per_vec<SRC>(), EB = 16 / E, GROUPS = 256 / LPR, COLS = LPR * E;
   __shared__ float part[GROUPS][COLS + 1];
+  __shared__ uint32_t word;
   const int cl = threadIdx.x % LPR, rg = threadIdx.x / LPR;
   const int64_t keep0 = (int64_t)blockIdx.x * COLS + cl * E;
   const int32_t r_begin = blockIdx.y * per_chunk, r_end = min(p.n_red, r_begin + per_chunk);
+  const int32_t chunks = gridDim.y;
   float acc[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) acc[e] = KIND == 0 ? -0.f : -__builtin_inff();
+  for (int e = 0; e < E; ++e) acc[e] = identity_of(p.kind, p.src_dtype);
   if (keep0 < p.n_keep) {  // (whole vectors: n_keep is a multiple of E)
     const char *col = p.src + keep0 * EB;
     constexpr int U = 4;
@@ -191,14 +307,14 @@ __global__ __launch_bounds__(256) void reduce_cols_strip_kernel(ReduceParams p, 
         float f[E];
         widen<SRC>(x[u], f);
 #pragma unroll
-        for (int e = 0; e < E; ++e) acc[e] = combine(acc[e], f[e], KIND);
+        for (int e = 0; e < E; ++e) acc[e] = combine_t<KIND>(acc[e], f[e], p.kind);
       }
     }
     for (; r < r_end; r += GROUPS) {
       float f[E];
       widen<SRC>(__builtin_nontemporal_load((const u32x4_t *)(col + (int64_t)r * p.s_red * EB)), f);
 #pragma unroll
-      for (int e = 0; e < E; ++e) acc[e] = combine(acc[e], f[e], KIND);
+      for (int e = 0; e < E; ++e) acc[e] = combine_t<KIND>(acc[e], f[e], p.kind);
     }
   }
 #pragma unroll
@@ -206,136 +322,30 @@ __global__ __launch_bounds__(256) void reduce_cols_strip_kernel(ReduceParams p, 
   __syncthreads();
   const int64_t keep = (int64_t)blockIdx.x * COLS + threadIdx.x;
   if (threadIdx.x < COLS && keep < p.n_keep) {
-    float t = KIND == 0 ? -0.f : -__builtin_inff();
+    float t = identity_of(p.kind, p.src_dtype);
 #pragma unroll
-    for (int g = 0; g < GROUPS; ++g) t = combine(t, part[g][threadIdx.x], KIND);
-    if (partials) partials[(int64_t)blockIdx.y * p.n_keep + keep] = t;
+    for (int g = 0; g < GROUPS; ++g) t = combine_t<KIND>(t, part[g][threadIdx.x], p.kind);
+    if (chunks > 1) partial_store(sh.lines + (int64_t)blockIdx.y * p.n_keep + keep, t);
     else store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
   }
+  if (chunks == 1) return;
+  if (!arrived_last(sh.counters + blockIdx.x, (uint32_t)chunks, &word)) return;
+  fold_partial_lines<COLS, KIND>(p, sh, (int64_t)blockIdx.x * COLS, chunks, &part[0][0]);
+  if (threadIdx.x == 0) __hip_atomic_store(sh.counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-
-// The second pass over `chunks` fp32 partial lines of n_keep values: 64 kept indices per workgroup, 16 groups of lanes
-// share out the lines, folded in chunk order within a group and in group order across them (the same result every run).
-template <int KIND>
-__global__ __launch_bounds__(1024) void reduce_partials_kernel(ReduceParams p, const float *partials, int32_t chunks) {
-  __shared__ float part[16][64 + 1];
-  const int cl = threadIdx.x & 63, rg = threadIdx.x >> 6;
-  const int64_t keep = (int64_t)blockIdx.x * 64 + cl;
-  float acc = KIND == 0 ? -0.f : -__builtin_inff();
-  if (keep < p.n_keep)
-    for (int32_t c = rg; c < chunks; c += 16) acc = combine(acc, partials[(int64_t)c * p.n_keep + keep], KIND);
-  part[rg][cl] = acc;
-  __syncthreads();
-  if (threadIdx.x < 64 && keep < p.n_keep) {
-    float t = KIND == 0 ? -0.f : -__builtin_inff();
-#pragma unroll
-    for (int g = 0; g < 16; ++g) t = combine(t, part[g][cl], KIND);
-    store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
-  }
-}
-
-// Memory for the partial lines: one block per device, allocated at the first call that wants it and kept.  Calls on one
-// stream use it in turn by stream order; a call on another stream first makes its stream wait for the event that the last
-// user recorded behind its second pass.  The mutex is held from that wait to the new record, so calls from several host
-// threads cannot interleave.  Not available - and then the caller reduces in one pass - while the stream is being
-// captured (an event of another stream's work cannot be waited for inside a capture) or when the allocation fails.
-constexpr int kMaxPartialsDevices = 16;
-constexpr size_t kPartialsBytes = size_t(4) << 20;  // the launches keep what they leave there within this
-struct Partials {
-  float *lines = nullptr;
-  hipEvent_t free_again = nullptr;
-  hipStream_t last_stream = nullptr;
-  bool used = false;
-  int state = 0;  // 0 not tried, 1 ready, -1 not available
-};
-std::mutex partials_mutex;
-Partials partials_of[kMaxPartialsDevices];
-
-// Call with partials_mutex held.  The device's block, ready for work on `s`, or nullptr.
-Partials *partials_for(hipStream_t s) {
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(s, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return nullptr;
-  }
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxPartialsDevices) return nullptr;
-  Partials &P = partials_of[dev];
-  if (P.state == 0) {
-    if (hipMalloc((void **)&P.lines, kPartialsBytes) == hipSuccess && hipEventCreateWithFlags(&P.free_again, hipEventDisableTiming) == hipSuccess) P.state = 1;
-    else {
-      (void)hipGetLastError();
-      P.state = -1;
-    }
-  }
-  if (P.state != 1) return nullptr;
-  if (P.used && P.last_stream != s && hipStreamWaitEvent(s, P.free_again, 0) != hipSuccess) {
-    (void)hipGetLastError();
-    return nullptr;
-  }
-  return &P;
-}
-
-// The block for a call that wants `chunks` > 1 partial lines, with `lock` taken - or nullptr, chunks = 1 and no lock.
-Partials *take_partials(int64_t &chunks, std::unique_lock<std::mutex> &lock, hipStream_t s) {
-  Partials *P = nullptr;
-  if (chunks > 1) {
-    lock.lock();
-    P = partials_for(s);
-    if (!P) lock.unlock();
-  }
-  if (!P) chunks = 1;
-  return P;
-}
-
-// After the call's launches (lock still held): whatever was launched reads or writes the block, so the next user waits for
-// all of it.
-int partials_used(Partials *P, hipStream_t s) {
-  const hipError_t launched = hipGetLastError(), recorded = hipEventRecord(P->free_again, s);
-  P->last_stream = s;
-  P->used = true;
-  if (launched != hipSuccess) return fail(KAPY_ERR_HIP, "reduce: %s", hipGetErrorString(launched));
-  if (recorded != hipSuccess) {
-    P->state = -1;  // nobody could wait for this call's use of the block: it is not handed out again
-    return fail(KAPY_ERR_HIP, "reduce: hipEventRecord: %s", hipGetErrorString(recorded));
-  }
-  return KAPY_OK;
-}
-
-}  // namespace
-
-// The same block for the column programs of kapy_elementwise (elementwise.hip): acquire returns it ready for work on `s`
-// with the mutex held, or nullptr (then nothing is held); release, after the caller's last launch that touches it, records
-// the event the next user waits for and lets go of the mutex.
-float *partials_acquire(hipStream_t s, size_t *bytes) {
-  partials_mutex.lock();
-  Partials *P = partials_for(s);
-  if (!P) {
-    partials_mutex.unlock();
-    return nullptr;
-  }
-  *bytes = kPartialsBytes;
-  return P->lines;
-}
-int partials_release(hipStream_t s) {
-  int dev = 0;
-  (void)hipGetDevice(&dev);
-  const int rc = partials_used(&partials_of[dev], s);
-  partials_mutex.unlock();
-  return rc;
-}
-
-namespace {
 
 // Any element type, alignment and extents, kept axis contiguous (or at least not the strided one): a workgroup owns 64 kept
 // indices, one per lane of a wave (a wave's loads cover 64 consecutive elements of one reduced index), its four waves share
-// out a chunk of the reduced axis with four loads in flight each and meet in LDS; chunks as in reduce_cols_strip_kernel.
-__global__ __launch_bounds__(256) void reduce_cols_any_kernel(ReduceParams p, float *partials, int32_t per_chunk) {
-  __shared__ float part[4][64];
+// out a chunk of the reduced axis with four loads in flight each and meet in LDS; chunks as in reduce_cols_strip_kernel
+// (float combiners only: the partial lines are fp32).
+__global__ __launch_bounds__(256) void reduce_cols_any_kernel(ReduceParams p, Shared sh, int32_t per_chunk) {
+  __shared__ float part[4][64 + 1];
+  __shared__ uint32_t word;
   const int cl = threadIdx.x & 63, rg = threadIdx.x >> 6;
   const int64_t keep = (int64_t)blockIdx.x * 64 + cl;
   const int32_t r_begin = blockIdx.y * per_chunk, r_end = min(p.n_red, r_begin + per_chunk);
-  float acc = p.kind == 0 ? -0.f : -__builtin_inff();
+  const int32_t chunks = gridDim.y;
+  float acc = identity_of(p.kind, p.src_dtype);
   if (keep < p.n_keep) {
     int32_t r = r_begin + rg;
     for (; r + 12 < r_end; r += 16) {
@@ -343,17 +353,109 @@ __global__ __launch_bounds__(256) void reduce_cols_any_kernel(ReduceParams p, fl
 #pragma unroll
       for (int u = 0; u < 4; ++u) f[u] = load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)(r + 4 * u) * p.s_red);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) acc = combine(acc, f[u], p.kind);
+      for (int u = 0; u < 4; ++u) acc = combine_any(acc, f[u], p.kind, p.src_dtype);
     }
-    for (; r < r_end; r += 4) acc = combine(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)r * p.s_red), p.kind);
+    for (; r < r_end; r += 4) acc = combine_any(acc, load_as_f32(p.src, p.src_dtype, keep * p.s_keep + (int64_t)r * p.s_red), p.kind, p.src_dtype);
   }
   part[rg][cl] = acc;
   __syncthreads();
   if (rg == 0 && keep < p.n_keep) {
-    float t = combine(combine(part[0][cl], part[1][cl], p.kind), combine(part[2][cl], part[3][cl], p.kind), p.kind);
-    if (partials) partials[(int64_t)blockIdx.y * p.n_keep + keep] = t;
+    const int k = p.kind, d = p.src_dtype;
+    float t = combine_any(combine_any(part[0][cl], part[1][cl], k, d), combine_any(part[2][cl], part[3][cl], k, d), k, d);
+    if (chunks > 1) partial_store(sh.lines + (int64_t)blockIdx.y * p.n_keep + keep, t);
     else store_from_f32(p.dst, p.dst_dtype, keep * p.d_keep, t);
   }
+  if (chunks == 1) return;
+  if (!arrived_last(sh.counters + blockIdx.x, (uint32_t)chunks, &word)) return;
+  fold_partial_lines<64, 1>(p, sh, (int64_t)blockIdx.x * 64, chunks, &part[0][0]);
+  if (threadIdx.x == 0) __hip_atomic_store(sh.counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// KAPY_REDUCE_REFERENCE: the lowering's own fold of one wavefront's tile (ReduceOpToLLVM.cpp:51-172 on 64 lanes).  A lane
+// holds the elements `layout` gives it (map 1: positions past the tensor wrap, as the reference's own loads replicate them);
+// per kept loop index it folds its elements along the reduced axis in loop order, every application of the combiner an op
+// on the element type; then `rounds` butterfly exchanges at lane distances lane_offset << i; every lane stores what it holds
+// (lanes that hold replicas store the same value).
+__global__ __launch_bounds__(64) void reduce_reference_kernel(ReduceParams p, Fragments layout, Idx2 shape, int axis, int lane_offset, int rounds) {
+  const int lane = threadIdx.x;
+  const Idx2 ls = layout.loop_space(shape);
+  const int64_t n_keep_iv = axis == 1 ? ls.v0 : ls.v1, n_red_iv = axis == 1 ? ls.v1 : ls.v0;
+  const bool is_float = p.kind < KAPY_REDUCE_ADDI;
+  for (int64_t k = 0; k < n_keep_iv; ++k) {
+    float acc = 0.f;
+    Idx2 at{0, 0};
+    for (int64_t r = 0; r < n_red_iv; ++r) {
+      const int64_t iv0 = axis == 1 ? k : r, iv1 = axis == 1 ? r : k;
+      const int64_t iv = layout.row_major() ? iv0 * ls.v1 + iv1 : iv0 + iv1 * ls.v0;
+      const Idx2 e = layout.to_index(shape, lane, iv, true);
+      const float v = load_as_f32(p.src, p.src_dtype, (axis == 1 ? e.v0 : e.v1) * p.s_keep + (axis == 1 ? e.v1 : e.v0) * p.s_red);
+      if (r == 0) { acc = v; at = e; }
+      else {
+        acc = combine_any(acc, v, p.kind, p.src_dtype);
+        if (is_float) acc = round_to_dtype(acc, p.src_dtype, true);
+      }
+    }
+    for (int i = 0; i < rounds; ++i) {
+      const float other = bits_f32((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ (lane_offset << i)) << 2, (int)f32_bits(acc)));
+      acc = combine_any(acc, other, p.kind, p.src_dtype);
+      if (is_float) acc = round_to_dtype(acc, p.src_dtype, true);
+    }
+    store_from_f32(p.dst, p.dst_dtype, (axis == 1 ? at.v0 : at.v1) * p.d_keep, acc);
+  }
+}
+
+}  // namespace
+}  // namespace kapy
+
+// The library's own workspace: 16 KiB of arrival counters (zero when the code object is loaded, and every launch leaves them
+// zero) and 4 MiB of partial lines, one copy per device.  In host code the array's name is a handle, not a device address.
+static __device__ __align__(256) unsigned char reduce_scratch[kapy::kCounterBytes + kapy::kScratchLineBytes];
+
+namespace kapy {
+
+// This device's copy of the array (asked for once per device; a race between two first calls only repeats the query).
+void *reduce_scratch_address() {
+  constexpr int kMaxDevices = 64;
+  static void *on_device[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void *ws = __atomic_load_n(&on_device[dev], __ATOMIC_ACQUIRE);
+  if (!ws) {
+    if (hipGetSymbolAddress(&ws, HIP_SYMBOL(reduce_scratch)) != hipSuccess || !ws) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    __atomic_store_n(&on_device[dev], ws, __ATOMIC_RELEASE);
+  }
+  return ws;
+}
+// The partial-line part of the library's own array for the column programs of kapy_elementwise (elementwise.hip), which
+// run their reduces as launches of their own on the caller's stream: like every call without a workspace they must not
+// overlap in time with another such call on the same GPU.
+float *reduce_scratch_lines(size_t *bytes, uint32_t **counters) {
+  char *ws = (char *)reduce_scratch_address();
+  if (!ws) return nullptr;
+  *bytes = kScratchLineBytes;
+  if (counters) *counters = (uint32_t *)ws;
+  return (float *)(ws + kCounterBytes);
+}
+
+namespace {
+
+// counters and lines of the call: the caller's workspace if it gave one, else the library's array; empty if neither is usable
+Shared shared_of(const kapy_reduce_cfg &cfg) {
+  Shared sh;
+  char *base = (char *)cfg.workspace;
+  int64_t bytes = cfg.workspace_bytes;
+  if (!base) {
+    base = (char *)reduce_scratch_address();
+    bytes = (int64_t)(kCounterBytes + kScratchLineBytes);
+  }
+  if (!base || bytes <= kCounterBytes || ((uintptr_t)base & 15)) return sh;
+  sh.counters = (uint32_t *)base;
+  sh.lines = (float *)(base + kCounterBytes);
+  sh.floats = (bytes - kCounterBytes) / 4;
+  return sh;
 }
 
 Fragments to_internal(const kapy_fragments *f) {
@@ -391,7 +493,7 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
   return KAPY_OK;
 }
 
-// LAUNCH(source kind, reduce kind) for the call's source type and reduce kind
+// LAUNCH(source kind, KIND) for the call's source type; KIND 0: the kernels' compiled-in addf, 1: the combiner read from p.kind
 #define KAPY_BY_SOURCE(LAUNCH)                                                                  \
   do {                                                                                          \
     if (src_kind == 0) { if (kind == 0) LAUNCH(0, 0); else LAUNCH(0, 1); }                      \
@@ -399,18 +501,34 @@ int kapy_change(const uint32_t *lane_values_in, const kapy_fragments *src, const
     else { if (kind == 0) LAUNCH(2, 0); else LAUNCH(2, 1); }                                    \
   } while (0)
 
+int64_t kapy_reduce_workspace_bytes(void) { return (int64_t)(kCounterBytes + kScratchLineBytes); }
+
 int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind, void *stream) {
+  kapy_reduce_cfg cfg = {kind, KAPY_REDUCE_WIDE, nullptr, nullptr, 0};
+  return kapy_reduce_ex(src, dst, axis, &cfg, stream);
+}
+
+int kapy_reduce_ex(const kapy_global *src, const kapy_global *dst, int32_t axis, const kapy_reduce_cfg *cfg_in, void *stream) {
   int rc = check_global(src, "reduce source");
   if (!rc) rc = check_global(dst, "reduce result");
   if (rc) return rc;
+  kapy_reduce_cfg cfg = {KAPY_REDUCE_ADDF, KAPY_REDUCE_WIDE, nullptr, nullptr, 0};
+  if (cfg_in) cfg = *cfg_in;
+  const int kind = cfg.combiner;
   if (axis != 0 && axis != 1) return fail(KAPY_ERR_VERIFY, "reduce: axis must be 0 or 1");
-  if (kind != 0 && kind != 1) return fail(KAPY_ERR_INVALID, "reduce: kind must be 0 (sum) or 1 (max)");
+  if (kind < KAPY_REDUCE_ADDF || kind > KAPY_REDUCE_XORI) return fail(KAPY_ERR_INVALID, "reduce: unknown combiner %d", kind);
+  if (cfg.arithmetic != KAPY_REDUCE_WIDE && cfg.arithmetic != KAPY_REDUCE_REFERENCE) return fail(KAPY_ERR_INVALID, "reduce: unknown arithmetic %d", cfg.arithmetic);
+  if (cfg.workspace && cfg.workspace_bytes < 0) return fail(KAPY_ERR_INVALID, "reduce: negative workspace size");
   const int64_t s0 = extent0(src), s1 = extent1(src);
   // Kapy.cpp ReduceOp::verify: the result keeps the other axis and has one element along `axis`
   if (axis == 1 ? (extent1(dst) != 1 || extent0(dst) != s0) : (extent0(dst) != 1 || extent1(dst) != s1))
     return fail(KAPY_ERR_VERIFY, "reduce: number of elements in result is incorrect");
-  if (!is_float(src->dtype) || is_f8(src->dtype) || !is_float(dst->dtype) || is_f8(dst->dtype))
-    return fail(KAPY_ERR_UNSUPPORTED, "reduce: only f16, bf16 and f32 tensors are supported");
+  const bool on_ints = kind >= KAPY_REDUCE_ADDI;
+  if (on_ints) {
+    if (!is_int(src->dtype) || src->dtype == KAPY_I1 || dst->dtype != src->dtype)
+      return fail(KAPY_ERR_VERIFY, "reduce: an integer combiner needs i8, i16 or i32 tensors, source and result of one type");
+  } else if (!is_float(src->dtype) || is_f8(src->dtype) || !is_float(dst->dtype) || is_f8(dst->dtype))
+    return fail(KAPY_ERR_UNSUPPORTED, "reduce: a float combiner needs f16, bf16 or f32 tensors");
   if (src->start0 < 0 || src->start1 < 0 || dst->start0 < 0 || dst->start1 < 0) return fail(KAPY_ERR_INVALID, "reduce: negative view start");
   rc = ensure_device();
   if (rc) return rc;
@@ -427,11 +545,45 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
   p.kind = kind;
   if (p.n_keep == 0) return KAPY_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (cfg.arithmetic == KAPY_REDUCE_REFERENCE) {
+    if (dst->dtype != src->dtype) return fail(KAPY_ERR_VERIFY, "reduce: in the reference's arithmetic the result has the source's element type");
+    if ((s0 & (s0 - 1)) || (s1 & (s1 - 1))) return fail(KAPY_ERR_VERIFY, "reduce: a wavefront's tile has power-of-two extents");
+    const Idx2 shape{s0, s1};
+    Fragments layout = default_fragments(Idx2{1, 1}, shape, true);
+    if (cfg.layout) {
+      const kapy_fragments *f = cfg.layout;
+      if (f->lane_array[0] * f->lane_array[1] != kWaveSize || f->lane_loops[0] <= 0 || f->lane_loops[1] <= 0 || (f->major_axis != 0 && f->major_axis != 1) ||
+          f->minor_axis != 1 - f->major_axis)
+        return fail(KAPY_ERR_VERIFY, "reduce: malformed fragments layout");
+      layout = to_internal(f);
+    }
+    if (layout.loop_size(shape) > 4096) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 4096 values per lane in the reference's arithmetic");
+    // laneOffset and the number of exchange rounds: LayoutUtils.cpp:26-49
+    const int lane_offset = layout.major == axis ? 1 : (axis == 1 ? layout.a0 : layout.a1);
+    bool seen[kWaveSize] = {false};
+    int distinct = 0;
+    for (int64_t i = 0; i < (axis == 0 ? s0 : s1); ++i) {
+      const int64_t lane = axis == 0 ? layout.to_lane_iv(shape, i, 0).v0 : layout.to_lane_iv(shape, 0, i).v0;
+      if (!seen[lane]) { seen[lane] = true; ++distinct; }
+    }
+    int rounds = 0;
+    while ((1 << (rounds + 1)) <= distinct) ++rounds;
+    reduce_reference_kernel<<<1, 64, 0, s>>>(p, layout, shape, axis, lane_offset, rounds);
+    KAPY_HIP_CHECK(hipGetLastError());
+    return KAPY_OK;
+  }
   // the vector kernels: f16, bf16 or f32 source read in 128-bit pieces of E elements
-  const bool vec_ok = src->dtype == KAPY_F16 || src->dtype == KAPY_BF16 || src->dtype == KAPY_F32;
+  const bool vec_ok = !on_ints && (src->dtype == KAPY_F16 || src->dtype == KAPY_BF16 || src->dtype == KAPY_F32);
   const int src_kind = src->dtype == KAPY_F32 ? 2 : src->dtype == KAPY_BF16 ? 1 : 0, E = src_kind == 2 ? 4 : 8, EB = 16 / E;
   const bool aligned = ((uintptr_t)p.src & 15) == 0;
-  std::unique_lock<std::mutex> lock(partials_mutex, std::defer_lock);
+  // how far a launch may share a reduced axis out: as many chunks as the partial lines of `lines_of` values each and the
+  // counters of `groups` line groups allow (integer combiners: no sharing, the partial lines are fp32)
+  Shared sh;
+  auto chunks_allowed = [&](int64_t groups, int64_t values_per_chunk) -> int64_t {
+    if (on_ints || groups > kMaxGroups) return 1;
+    sh = shared_of(cfg);
+    return sh.lines ? std::max<int64_t>(1, sh.floats / std::max<int64_t>(1, values_per_chunk)) : 1;
+  };
   if (vec_ok && aligned && p.s_red == 1 && p.n_red % E == 0 && (p.s_keep * EB) % 16 == 0 && p.n_red <= 64 * E && p.n_red >= E) {
     const int vecs = p.n_red / E, group = vecs <= 8 ? 8 : vecs <= 16 ? 16 : vecs <= 32 ? 32 : 64;
     const int64_t wgs = ((int64_t)p.n_keep + 256 / group - 1) / (256 / group);
@@ -448,69 +600,43 @@ int kapy_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, in
 #undef KAPY_SHORT
   } else if (vec_ok && aligned && p.s_red == 1 && p.n_red % E == 0 && (p.s_keep * EB) % 16 == 0 && p.n_red > 64 * E) {
     // four lines per workgroup; with fewer workgroups than CUs, chunks of at least 256 vectors of the reduced axis as well,
-    // up to four workgroups per CU (their partial results within the block): 64 lines of 1 Mi elements 312 -> 33 us, 256
-    // lines of 256 Ki 82 -> 30 us.  The second launch costs about 6 us: 1024 lines of 64 Ki elements are faster whole.
+    // up to four workgroups per CU: 64 lines of 1 Mi elements 312 -> 33 us, 256 lines of 256 Ki 82 -> 30 us.
     const int64_t wgs = ((int64_t)p.n_keep + 3) / 4, want = 4 * (int64_t)device_cus(), vecs = p.n_red / E;
-    int64_t chunks = wgs >= device_cus() ? 1 : std::max<int64_t>(1, std::min<int64_t>({(want + wgs - 1) / wgs, vecs / 256, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
-    Partials *P = take_partials(chunks, lock, s);
+    int64_t chunks = wgs >= device_cus() ? 1 : std::max<int64_t>(1, std::min<int64_t>({(want + wgs - 1) / wgs, vecs / 256, 512}));
+    if (chunks > 1) chunks = std::min(chunks, chunks_allowed(wgs, p.n_keep));
     const int32_t vecs_per_chunk = (int32_t)((vecs + chunks - 1) / chunks);
     chunks = (vecs + vecs_per_chunk - 1) / vecs_per_chunk;
-    float *lines = P ? P->lines : nullptr;
     dim3 grid((unsigned)wgs, (unsigned)chunks);
-#define KAPY_ROWS(SRC_, KIND_) reduce_rows_vec_kernel<SRC_, KIND_><<<grid, 256, 0, s>>>(p, lines, vecs_per_chunk)
+#define KAPY_ROWS(SRC_, KIND_) reduce_rows_vec_kernel<SRC_, KIND_><<<grid, 256, 0, s>>>(p, sh, vecs_per_chunk)
     KAPY_BY_SOURCE(KAPY_ROWS);
 #undef KAPY_ROWS
-    if (P) {
-      // the partial results as an fp32 source of n_keep lines of `chunks` values: one wave per line folds them
-      ReduceParams q = p;
-      q.src = (const char *)lines;
-      q.s_keep = chunks;
-      q.s_red = 1;
-      q.n_red = (int32_t)chunks;
-      q.src_dtype = KAPY_F32;
-      reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(q);
-      return partials_used(P, s);
-    }
   } else if (vec_ok && aligned && p.s_keep == 1 && p.n_keep % E == 0 && (p.s_red * EB) % 16 == 0 && p.n_red >= 32) {
     // strips of 256 kept indices (512-byte runs per reduced index), of 64 for narrow sources; the reduced axis in as many
     // chunks as bring the launch to about four workgroups per CU, of at least 128 reduced indices each, as far as their
-    // partial lines fit the block.  Measured for 128 MiB of fp16: 8192 x 8192 46 -> 29 us (64-wide strips: 31, eight
-    // workgroups per CU: 31, eight loads in flight per lane: 30), 1 Mi x 64 4335 -> 34 us.
+    // partial lines fit the workspace.
     const int lpr = p.n_keep >= 32 * E ? 32 : 8, cols = lpr * E;
     const int64_t strips = ((int64_t)p.n_keep + cols - 1) / cols, want = 4 * (int64_t)device_cus();
     if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
-    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 128, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
-    Partials *P = take_partials(chunks, lock, s);
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 128, 512}));
+    if (chunks > 1) chunks = std::min(chunks, chunks_allowed(strips, p.n_keep));
     const int32_t per_chunk = (int32_t)((p.n_red + chunks - 1) / chunks);
     chunks = (p.n_red + per_chunk - 1) / per_chunk;
-    float *lines = P ? P->lines : nullptr;
     dim3 grid((unsigned)strips, (unsigned)chunks);
 #define KAPY_STRIP(SRC_, KIND_)                                                                                                       \
   do {                                                                                                                                \
-    if (lpr == 32) reduce_cols_strip_kernel<SRC_, KIND_, 32><<<grid, 256, 0, s>>>(p, lines, per_chunk);                               \
-    else reduce_cols_strip_kernel<SRC_, KIND_, 8><<<grid, 256, 0, s>>>(p, lines, per_chunk);                                          \
+    if (lpr == 32) reduce_cols_strip_kernel<SRC_, KIND_, 32><<<grid, 256, 0, s>>>(p, sh, per_chunk);                                  \
+    else reduce_cols_strip_kernel<SRC_, KIND_, 8><<<grid, 256, 0, s>>>(p, sh, per_chunk);                                             \
   } while (0)
     KAPY_BY_SOURCE(KAPY_STRIP);
 #undef KAPY_STRIP
-    if (P) {
-      if (kind == 0) reduce_partials_kernel<0><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
-      else reduce_partials_kernel<1><<<dim3((unsigned)((p.n_keep + 63) / 64)), 1024, 0, s>>>(p, lines, (int32_t)chunks);
-      return partials_used(P, s);
-    }
   } else if (p.s_keep == 1 && p.s_red != 1) {
     const int64_t strips = ((int64_t)p.n_keep + 63) / 64, want = 4 * (int64_t)device_cus();
     if (strips > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "reduce: more than 2^31 strips of results");
-    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 64, 512, (int64_t)(kPartialsBytes / sizeof(float)) / p.n_keep}));
-    Partials *P = take_partials(chunks, lock, s);
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>({(want + strips - 1) / strips, (int64_t)p.n_red / 64, 512}));
+    if (chunks > 1) chunks = std::min(chunks, chunks_allowed(strips, p.n_keep));
     const int32_t per_chunk = (int32_t)((p.n_red + chunks - 1) / chunks);
     chunks = (p.n_red + per_chunk - 1) / per_chunk;
-    float *lines = P ? P->lines : nullptr;
-    reduce_cols_any_kernel<<<dim3((unsigned)strips, (unsigned)chunks), 256, 0, s>>>(p, lines, per_chunk);
-    if (P) {
-      if (kind == 0) reduce_partials_kernel<0><<<dim3((unsigned)strips), 1024, 0, s>>>(p, lines, (int32_t)chunks);
-      else reduce_partials_kernel<1><<<dim3((unsigned)strips), 1024, 0, s>>>(p, lines, (int32_t)chunks);
-      return partials_used(P, s);
-    }
+    reduce_cols_any_kernel<<<dim3((unsigned)strips, (unsigned)chunks), 256, 0, s>>>(p, sh, per_chunk);
   }
   else reduce_wave_kernel<<<(p.n_keep + 3) / 4, 256, 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());

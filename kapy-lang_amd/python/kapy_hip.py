@@ -37,7 +37,7 @@ EXPORTS = [
     "kapy_fragments_default", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
     "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
-    "kapy_change", "kapy_reduce", "kapy_run_mlir", "kapy_parse_mlir",
+    "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
     "kapy_mfma_probe", "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
@@ -102,6 +102,16 @@ class MatmulCfg(C.Structure):
     _fields_ = [("impl_way", C.c_int32), ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
                 ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("split_k", C.c_int32),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64)]
+
+
+class ReduceCfg(C.Structure):
+    _fields_ = [("combiner", C.c_int32), ("arithmetic", C.c_int32), ("layout", C.POINTER(Fragments)), ("workspace", C.c_void_p),
+                ("workspace_bytes", C.c_int64)]
+
+
+(REDUCE_ADDF, REDUCE_MAXIMUMF, REDUCE_MINIMUMF, REDUCE_MULF, REDUCE_MAXNUMF, REDUCE_MINNUMF, REDUCE_ADDI, REDUCE_MULI, REDUCE_MAXSI, REDUCE_MINSI,
+ REDUCE_MAXUI, REDUCE_MINUI, REDUCE_ANDI, REDUCE_ORI, REDUCE_XORI) = range(15)
+REDUCE_WIDE, REDUCE_REFERENCE = 0, 1
 
 
 class MatmulEpilogue(C.Structure):
@@ -186,6 +196,9 @@ def lib():
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
     L.kapy_mfma_probe.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp]
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
+    L.kapy_reduce_ex.argtypes = [P(Global), P(Global), i32, P(ReduceCfg), vp]
+    L.kapy_reduce_workspace_bytes.restype = C.c_int64
+    L.kapy_reduce_workspace_bytes.argtypes = []
     L.kapy_smem_plan.restype = i64
     L.kapy_smem_plan.argtypes = [P(SmemBuffer), i32, i64]
     L.kapy_smem_barriers.argtypes = [P(SmemOp), i32, P(SmemAccess), i32, P(i32), P(i32), i32, P(i32)]
@@ -421,6 +434,13 @@ def matmul_scaled_f8(a8, w8, row_scale_ptr, col_scale_ptr, result, split_k=0, wo
 
 def reduce(src, dst, axis, kind=0, stream=None):
     check(lib().kapy_reduce(C.byref(src), C.byref(dst), axis, kind, stream if stream is not None else current_stream()))
+
+
+def reduce_ex(src, dst, axis, combiner=0, arithmetic=REDUCE_WIDE, layout=None, workspace=None, stream=None):
+    """workspace: None, a (pointer, bytes) pair or a torch tensor."""
+    ptr, nbytes = _workspace(workspace)
+    cfg = ReduceCfg(combiner, arithmetic, C.pointer(layout) if layout is not None else None, ptr, nbytes)
+    check(lib().kapy_reduce_ex(C.byref(src), C.byref(dst), axis, C.byref(cfg), stream if stream is not None else current_stream()))
 
 
 def parse_mlir(text, func_name=None):

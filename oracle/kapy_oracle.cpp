@@ -1067,25 +1067,105 @@ void ko_quantize_e4m3(const float *x, int64_t rows, int64_t cols, int64_t row_st
   }
 }
 
-// kapy.reduce (Ops.td:441-457, ReduceOpToLLVM.cpp:51-172) with an add / max combiner.
-// kind 0: sum (fp64 accumulate), 1: max.  dst extent along `axis` is 1.
+// kapy.reduce (Ops.td:441-457, ReduceOpToLLVM.cpp:51-172) with a combiner region that is one arith op.
+// kind (= kapy_reduce_combiner): 0 addf (fp64 accumulate), 1 maximumf, 2 minimumf, 3 mulf, 4 maxnumf, 5 minnumf; 6 addi, 7 muli,
+// 8 maxsi, 9 minsi, 10 maxui, 11 minui, 12 andi, 13 ori, 14 xori on integers (wrapping).  dst extent along `axis` is 1.
+// The elements themselves are folded (no identity joins them): the fold starts from the line's first element.
+static double reduce_step(double acc, double v, int kind, int dtype) {
+  const double qnan = std::numeric_limits<double>::quiet_NaN();
+  auto lower = [](double a, double b) { return a == b ? (std::signbit(a) ? a : b) : std::min(a, b); };   // -0 orders below +0
+  auto upper = [](double a, double b) { return a == b ? (std::signbit(a) ? b : a) : std::max(a, b); };
+  switch (kind) {
+  case 0: return acc + v;
+  case 1: return (std::isnan(acc) || std::isnan(v)) ? qnan : upper(acc, v);
+  case 2: return (std::isnan(acc) || std::isnan(v)) ? qnan : lower(acc, v);
+  case 3: return acc * v;
+  case 4: return std::isnan(acc) ? v : std::isnan(v) ? acc : upper(acc, v);
+  case 5: return std::isnan(acc) ? v : std::isnan(v) ? acc : lower(acc, v);
+  default: {
+    static const int op_of[] = {EW_ADDI, EW_MULI, EW_MAXSI, EW_MINSI, EW_MAXUI, EW_MINUI, EW_ANDI, EW_ORI, EW_XORI};
+    return (double)int_binary_op(op_of[kind - 6], (int64_t)acc, (int64_t)v, dtype);
+  }
+  }
+}
+
 int ko_reduce(const ko_global *src, const ko_global *dst, int axis, int kind) {
   int64_t s0 = extent0(src), s1 = extent1(src);
   int64_t outer = axis == 0 ? s1 : s0, inner = axis == 0 ? s0 : s1;
   if (axis == 0 ? (extent0(dst) != 1 || extent1(dst) != s1) : (extent1(dst) != 1 || extent0(dst) != s0)) return -1;
+  if (kind < 0 || kind > 14 || inner <= 0) return -2;
+  if (kind >= 6 && (!is_int_dtype(src->dtype) || src->dtype == KO_I1 || dst->dtype != src->dtype)) return -3;
 #pragma omp parallel for schedule(static)
   for (int64_t o = 0; o < outer; ++o) {
-    double acc = kind == 0 ? -0.0 : -std::numeric_limits<double>::infinity();  // -0: identity of addition, = folding the elements themselves (ReduceOpToLLVM.cpp:60-101)
+    double acc = 0.0;
     for (int64_t t = 0; t < inner; ++t) {
       int64_t i = axis == 0 ? t : o, j = axis == 0 ? o : t;
       double v = ko_decode(src->ptr, src->dtype, elem_offset(src, i, j));
-      if (kind == 0) acc += v;
-      else if (std::isnan(v) || std::isnan(acc)) acc = std::numeric_limits<double>::quiet_NaN();
-      else if (v == 0.0 && acc == 0.0) acc = (std::signbit(v) && std::signbit(acc)) ? -0.0 : 0.0;  // maximumf orders -0 below +0
-      else acc = std::max(acc, v);
+      acc = t == 0 ? v : reduce_step(acc, v, kind, src->dtype);
     }
     int64_t i = axis == 0 ? 0 : o, j = axis == 0 ? o : 0;
     ko_encode(dst->ptr, dst->dtype, elem_offset(dst, i, j), acc, KO_RN);
+  }
+  return 0;
+}
+
+// The same reduce in the lowering's own arithmetic and order for one wavefront's tile (ReduceOpToLLVM.cpp:51-172): the tile sits in
+// the registers of `lanes` lanes under `layout` (map 1 of Kgpu.cpp:186-251; nullptr: getFragmentsLayout({1, 1}, tile, rowMajor =
+// true), LayoutUtils.cpp:92-110).  Per kept loop index a lane folds its elements along the reduced axis in loop order (:76-101),
+// then the lanes fold by butterfly exchanges at lane distances laneOffset * 2^i for i = 0 .. numShfls - 1 (:104-119; laneOffset
+// and numShfls: LayoutUtils.cpp:26-49).  Every application of the combiner is an op on the ELEMENT type: a float result is
+// rounded to the source's type each time.  dst has the source's element type.
+int ko_reduce_reference(const ko_global *src, const ko_global *dst, int axis, int kind, const ko_fragments *layout, int64_t lanes) {
+  const int64_t shape[2] = {extent0(src), extent1(src)};
+  if (axis == 0 ? (extent0(dst) != 1 || extent1(dst) != shape[1]) : (extent1(dst) != 1 || extent0(dst) != shape[0])) return -1;
+  if (kind < 0 || kind > 14 || dst->dtype != src->dtype) return -2;
+  if (kind >= 6 && (!is_int_dtype(src->dtype) || src->dtype == KO_I1)) return -3;
+  ko_fragments def;
+  if (!layout) {
+    const int64_t ones[2] = {1, 1};
+    ko_fragments_default(ones, shape, 1, lanes, &def);
+    layout = &def;
+  }
+  int64_t warp_loops[2], space[2];
+  ko_fragments_loops(layout, shape, warp_loops, space);
+  const bool row_major = layout->major_axis == 1;
+  const int64_t n_keep_iv = axis == 1 ? space[0] : space[1], n_red_iv = axis == 1 ? space[1] : space[0];
+  const int64_t lane_offset = layout->major_axis == axis ? 1 : layout->lane_array[axis == 1 ? 0 : 1];
+  std::set<int64_t> owners;
+  for (int64_t index = 0; index < shape[axis]; ++index) {
+    int64_t lane, iv;
+    ko_fragments_map3(layout, shape, axis == 0 ? index : 0, axis == 0 ? 0 : index, &lane, &iv);
+    owners.insert(lane);
+  }
+  int64_t rounds = 0;
+  while ((int64_t(1) << (rounds + 1)) <= (int64_t)owners.size()) ++rounds;
+  auto typed = [&](double a, double b) {
+    const double r = reduce_step(a, b, kind, src->dtype);
+    if (kind >= 6) return r;
+    uint32_t tmp = 0;
+    ko_encode(&tmp, src->dtype, 0, r, KO_RN);
+    return ko_decode(&tmp, src->dtype, 0);
+  };
+  std::vector<double> acc((size_t)lanes);
+  std::vector<int64_t> kept((size_t)lanes);
+  for (int64_t k = 0; k < n_keep_iv; ++k) {
+    for (int64_t lane = 0; lane < lanes; ++lane) {
+      for (int64_t r = 0; r < n_red_iv; ++r) {
+        const int64_t iv0 = axis == 1 ? k : r, iv1 = axis == 1 ? r : k;
+        const int64_t iv = row_major ? iv0 * space[1] + iv1 : iv0 + iv1 * space[0];
+        int64_t idx[2];
+        ko_fragments_map12(layout, shape, 1, lane, iv, idx);
+        const double v = ko_decode(src->ptr, src->dtype, elem_offset(src, idx[0], idx[1]));
+        if (r == 0) { acc[lane] = v; kept[lane] = idx[axis == 1 ? 0 : 1]; }
+        else acc[lane] = typed(acc[lane], v);
+      }
+    }
+    for (int64_t i = 0; i < rounds; ++i) {
+      const std::vector<double> before = acc;
+      for (int64_t lane = 0; lane < lanes; ++lane) acc[lane] = typed(before[lane], before[lane ^ (lane_offset << i)]);
+    }
+    for (int64_t lane = 0; lane < lanes; ++lane)
+      ko_encode(dst->ptr, dst->dtype, axis == 1 ? elem_offset(dst, kept[lane], 0) : elem_offset(dst, 0, kept[lane]), acc[lane], KO_RN);
   }
   return 0;
 }

@@ -114,6 +114,7 @@ int ko_matmul_scaled_f8(const ko_global *a, const ko_global *w, const float *row
 void ko_quantize_e4m3(const float *x, int64_t rows, int64_t cols, int64_t row_stride, int64_t col_stride,
                       int along_cols, uint8_t *q, float *scale);
 int ko_reduce(const ko_global *src, const ko_global *dst, int axis, int kind);
+int ko_reduce_reference(const ko_global *src, const ko_global *dst, int axis, int kind, const ko_fragments *layout, int64_t lanes);
 
 int ko_num_threads(void);
 

@@ -121,6 +121,7 @@ def lib():
         L.ko_quantize_e4m3.restype = None
         L.ko_quantize_e4m3.argtypes = [vp, i64, i64, i64, i64, C.c_int, vp, vp]
         L.ko_reduce.restype = C.c_int; L.ko_reduce.argtypes = [P(Global), P(Global), C.c_int, C.c_int]
+        L.ko_reduce_reference.restype = C.c_int; L.ko_reduce_reference.argtypes = [P(Global), P(Global), C.c_int, C.c_int, P(Fragments), i64]
         L.ko_baseline_gemm.restype = C.c_int; L.ko_baseline_gemm.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(dbl)]
         L.ko_baseline_gelu_f16.restype = C.c_int; L.ko_baseline_gelu_f16.argtypes = [vp, vp, C.c_float, vp, i64, i64, i64]
         L.ko_baseline_transpose16.restype = C.c_int; L.ko_baseline_transpose16.argtypes = [vp, vp, i64, i64]

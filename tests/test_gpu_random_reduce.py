@@ -189,8 +189,9 @@ def test_reduce_along_axis1_of_short_and_of_few_long_lines(ko, dtype, m, n):
             assert np.all(np.abs(g[rest] - w[rest]) <= (2.0 ** -22 * mass + 2.0 * EPS[ddt] * np.abs(w) + 1e-30)[rest])
 
 
-def test_tall_reduces_on_two_streams_share_the_partial_lines_in_turn():
-    """The library keeps one block of partial lines per device; calls on different streams must not overlap in it."""
+def test_tall_reduces_on_two_streams_with_a_workspace_each():
+    """Launches that share a reduced axis out over workgroups meet in a workspace; calls that may overlap in time (two streams)
+    get one each.  Every result has the same bits as the call made alone on the library's own array."""
     import torch
     m, n = 60000, 64
     xs = [torch.randn(m, n, device="cuda").half() for _ in range(6)]
@@ -201,17 +202,167 @@ def test_tall_reduces_on_two_streams_share_the_partial_lines_in_turn():
         sync()
         alone.append(d.clone())
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    spaces = [torch.zeros(kh.lib().kapy_reduce_workspace_bytes(), dtype=torch.uint8, device="cuda") for _ in streams]
+    sync()
     for st in streams:
         st.wait_stream(torch.cuda.current_stream())
     for rep in range(5):
         outs = [torch.zeros(n, device="cuda", dtype=torch.float32) for _ in xs]
         for k, (x, d) in enumerate(zip(xs, outs)):
             with torch.cuda.stream(streams[k % 2]):
-                kh.reduce(dglobal(x, m, n, n, 1, kh.F16), dglobal(d, 1, n, n, 1, kh.F32), 0, 0, stream=streams[k % 2].cuda_stream)
+                kh.reduce_ex(dglobal(x, m, n, n, 1, kh.F16), dglobal(d, 1, n, n, 1, kh.F32), 0, kh.REDUCE_ADDF, workspace=spaces[k % 2],
+                             stream=streams[k % 2].cuda_stream)
         for st in streams:
             st.synchronize()
         for d, a in zip(outs, alone):
             assert torch.equal(d, a)
+    for ws in spaces:
+        assert not ws[:16384].any()                    # the arrival counters are back at zero
+
+
+def test_a_captured_reduce_equals_the_eager_call():
+    """Nothing about the call depends on the stream being captured: the graph's replays give the eager call's bits."""
+    import torch
+    for m, n, axis in ((60000, 64, 0), (8192, 2048, 0), (64, 262144, 1)):
+        x = torch.randn(m, n, device="cuda").half()
+        k = n if axis == 0 else m
+        shape, strides = ((1, n), (n, 1)) if axis == 0 else ((m, 1), (1, m))
+        eager = torch.zeros(k, device="cuda", dtype=torch.float32)
+        kh.reduce(dglobal(x, m, n, n, 1, kh.F16), dglobal(eager, shape[0], shape[1], strides[0], strides[1], kh.F32), axis, 0)
+        sync()
+        out = torch.zeros(k, device="cuda", dtype=torch.float32)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                kh.reduce(dglobal(x, m, n, n, 1, kh.F16), dglobal(out, shape[0], shape[1], strides[0], strides[1], kh.F32), axis, 0, stream=side.cuda_stream)
+        for rep in range(3):
+            out.fill_(-1.0)
+            sync()
+            graph.replay()
+            sync()
+            assert torch.equal(out, eager), (m, n, axis, rep)
+
+
+FLOAT_KINDS = [kh.REDUCE_ADDF, kh.REDUCE_MAXIMUMF, kh.REDUCE_MINIMUMF, kh.REDUCE_MULF, kh.REDUCE_MAXNUMF, kh.REDUCE_MINNUMF]
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16, kh.F32])
+@pytest.mark.parametrize("m,n,axis", [(64, 1024, 1), (16, 520, 1), (4, 262144, 1), (300, 128, 0), (20000, 64, 0), (4096, 2048, 0), (33, 33, 0), (7, 100, 1)])
+def test_every_float_combiner_on_every_kernel_shape(ko, dtype, m, n, axis):
+    """minimumf, mulf, maxnumf and minnumf beside addf and maximumf, through the short-line, long-line, shared-out, strip and
+    element kernels; lines with NaNs for the four orderings (bit-exact), products of values near one."""
+    x = ko.fill_normal(m * n, dtype, 700 + m + n, 0, 0.0, 1.0).reshape(m, n)
+    nan = {kh.F16: 0x7e00, kh.BF16: 0x7fc0, kh.F32: np.float32(np.nan)}[dtype]
+    rng = np.random.default_rng(m)
+    if dtype == kh.F32:
+        x = x.copy()
+    x[rng.integers(0, m), rng.integers(0, n)] = nan
+    if axis == 1:
+        x[m // 2, :] = nan
+    else:
+        x[:, n // 2] = nan
+    sb = kh.DTYPE_BYTES[dtype]
+    om, on = (m, 1) if axis == 1 else (1, n)
+    for kind in FLOAT_KINDS:
+        src = x
+        if kind in (kh.REDUCE_ADDF, kh.REDUCE_MULF):                      # finite operands; products of 1 + small
+            src = ko.fill_normal(m * n, dtype, 800 + m, 0, 1.0 if kind == kh.REDUCE_MULF else 0.0, 2.0 ** -9 if kind == kh.REDUCE_MULF else 1.0).reshape(m, n)
+        want = np.zeros(om * on, NP[sb])
+        assert ko.lib().ko_reduce(C.byref(ko.mk_global(src, m, n, n, 1, dtype)), C.byref(ko.mk_global(want, om, on, on, 1, dtype)), axis, kind) == 0
+        d_dst = to_dev(np.zeros(om * on, NP[sb]))
+        kh.reduce_ex(dglobal(to_dev(src), m, n, n, 1, dtype), dglobal(d_dst, om, on, on, 1, dtype), axis, kind)
+        sync()
+        got = to_host(d_dst, NP[sb])
+        if kind in (kh.REDUCE_ADDF, kh.REDUCE_MULF):
+            g, w = ko.decode(got.view(VALUE[dtype]), dtype), ko.decode(want.view(VALUE[dtype]), dtype)
+            scale = np.abs(ko.decode(src.view(VALUE[dtype]), dtype)).sum(axis=axis).ravel() if kind == kh.REDUCE_ADDF else np.abs(w)
+            n_red = n if axis == 1 else m          # a product's rounding errors add up along the line (about their square root on random data)
+            rel = 8.0 * np.sqrt(n_red) * 2.0 ** -24 if kind == kh.REDUCE_MULF else 2.0 ** -22
+            assert np.all(np.abs(g - w) <= rel * scale + 2.0 * EPS[dtype] * np.abs(w) + 1e-30), kind
+        else:
+            gv, wv = got.view(VALUE[dtype]), want.view(VALUE[dtype])
+            same = gv == wv
+            if dtype == kh.F32:
+                same |= np.isnan(gv) & np.isnan(wv)
+            else:
+                both_nan = (ko.decode(gv, dtype) != ko.decode(gv, dtype)) & (ko.decode(wv, dtype) != ko.decode(wv, dtype))
+                same |= both_nan
+            assert np.all(same), "combiner %d: %d results differ" % (kind, int((~same).sum()))
+
+
+@pytest.mark.parametrize("dt,np_t", [(kh.I8, np.int8), (kh.I16, np.int16), (kh.I32, np.int32)])
+@pytest.mark.parametrize("m,n,axis", [(37, 53, 0), (37, 53, 1), (3000, 64, 0), (8, 5000, 1)])
+def test_integer_combiners_are_bit_exact(ko, dt, np_t, m, n, axis):
+    rng = np.random.default_rng(m + n + axis)
+    info = np.iinfo(np_t)
+    x = rng.integers(info.min, info.max + 1, size=(m, n), dtype=np.int64).astype(np_t)
+    om, on = (m, 1) if axis == 1 else (1, n)
+    for kind in range(kh.REDUCE_ADDI, kh.REDUCE_XORI + 1):
+        want = np.zeros((om, on), np_t)
+        assert ko.lib().ko_reduce(C.byref(ko.mk_global(x, m, n, n, 1, dt)), C.byref(ko.mk_global(want, om, on, on, 1, dt)), axis, kind) == 0
+        d_dst = to_dev(np.zeros(om * on, np_t))
+        kh.reduce_ex(dglobal(to_dev(x), m, n, n, 1, dt), dglobal(d_dst, om, on, on, 1, dt), axis, kind)
+        sync()
+        assert np.array_equal(to_host(d_dst, np_t, (om, on)), want), kind
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16, kh.F32])
+@pytest.mark.parametrize("shape,axis,loops,row_major", [((2, 256), 1, None, True), ((4, 512), 1, (1, 8), True), ((64, 8), 0, (1, 1), False),
+                                                          ((128, 16), 0, (2, 1), False), ((16, 64), 1, (1, 2), True), ((32, 32), 0, (1, 1), True),
+                                                          ((1, 4096), 1, (1, 4), True)])
+def test_reference_arithmetic_equals_the_checker_bit_for_bit(ko, dtype, shape, axis, loops, row_major):
+    """KAPY_REDUCE_REFERENCE: partial results rounded to the element type, lane-serial fold then butterfly, on a wavefront's tile
+    under a given fragments layout (None: the default one) - the same bits as the checker's walk of that order, for sums (where
+    the order shows), maxima and an integer fold."""
+    m, n = shape
+    lay = None
+    klay = None
+    if loops is not None:
+        lay = ko.Fragments()
+        ko.lib().ko_fragments_default((C.c_int64 * 2)(*loops), (C.c_int64 * 2)(*shape), 1 if row_major else 0, 64, C.byref(lay))
+        klay = kh.Fragments.make([lay.lane_array[0], lay.lane_array[1]], [lay.lane_loops[0], lay.lane_loops[1]], lay.minor_axis, lay.major_axis)
+    sb = kh.DTYPE_BYTES[dtype]
+    om, on = (m, 1) if axis == 1 else (1, n)
+    x = ko.fill_normal(m * n, dtype, 900 + m, 0, 0.0, 30.0).reshape(m, n)
+    differs = 0
+    for kind in (kh.REDUCE_ADDF, kh.REDUCE_MAXIMUMF, kh.REDUCE_MULF):
+        src = x if kind != kh.REDUCE_MULF else ko.fill_normal(m * n, dtype, 901, 0, 1.0, 0.01).reshape(m, n)
+        want, wide = np.zeros(om * on, NP[sb]), np.zeros(om * on, NP[sb])
+        g, o = ko.mk_global(src, m, n, n, 1, dtype), ko.mk_global(want, om, on, on, 1, dtype)
+        assert ko.lib().ko_reduce_reference(C.byref(g), C.byref(o), axis, kind, C.byref(lay) if lay is not None else None, 64) == 0
+        assert ko.lib().ko_reduce(C.byref(g), C.byref(ko.mk_global(wide, om, on, on, 1, dtype)), axis, kind) == 0
+        d_dst = to_dev(np.zeros(om * on, NP[sb]))
+        kh.reduce_ex(dglobal(to_dev(src), m, n, n, 1, dtype), dglobal(d_dst, om, on, on, 1, dtype), axis, kind, arithmetic=kh.REDUCE_REFERENCE, layout=klay)
+        sync()
+        assert np.array_equal(to_host(d_dst, NP[sb]), want), kind
+        differs += int((want != wide).sum())
+    if dtype != kh.F32 and max(m, n) >= 256:
+        assert differs > 0        # 16-bit partial sums are not the once-rounded sum: the mode is not a no-op
+    xi = (np.arange(m * n, dtype=np.int64).reshape(m, n) * 2654435761 % 65521 - 30000).astype(np.int16)
+    want = np.zeros((om, on), np.int16)
+    assert ko.lib().ko_reduce_reference(C.byref(ko.mk_global(xi, m, n, n, 1, kh.I16)), C.byref(ko.mk_global(want, om, on, on, 1, kh.I16)), axis, kh.REDUCE_ADDI,
+                                        C.byref(lay) if lay is not None else None, 64) == 0
+    d_dst = to_dev(np.zeros(om * on, np.int16))
+    kh.reduce_ex(dglobal(to_dev(xi), m, n, n, 1, kh.I16), dglobal(d_dst, om, on, on, 1, kh.I16), axis, kh.REDUCE_ADDI, arithmetic=kh.REDUCE_REFERENCE, layout=klay)
+    sync()
+    assert np.array_equal(to_host(d_dst, np.int16, (om, on)), want) and np.array_equal(want.ravel(), xi.astype(np.int64).sum(axis=axis).astype(np.int16))
+
+
+def test_reduce_refusals():
+    import torch
+    x = torch.zeros(64 * 64, device="cuda", dtype=torch.int32)
+    g = lambda m, n, dt: dglobal(x, m, n, n, 1, dt)
+    for args, kw, words in (((g(64, 64, kh.F16), g(64, 1, kh.F16), 1, 15), {}, "unknown combiner"),
+                            ((g(64, 64, kh.F16), g(64, 1, kh.F16), 1, kh.REDUCE_ADDI), {}, "integer combiner"),
+                            ((g(64, 64, kh.I32), g(64, 1, kh.I32), 1, kh.REDUCE_ADDF), {}, "float combiner"),
+                            ((g(64, 64, kh.I32), g(64, 1, kh.I16), 1, kh.REDUCE_ADDI), {}, "one type"),
+                            ((g(48, 64, kh.F16), g(48, 1, kh.F16), 1, kh.REDUCE_ADDF), dict(arithmetic=kh.REDUCE_REFERENCE), "power-of-two"),
+                            ((g(64, 64, kh.F16), g(64, 1, kh.F32), 1, kh.REDUCE_ADDF), dict(arithmetic=kh.REDUCE_REFERENCE), "source's element type")):
+        with pytest.raises(kh.KapyError) as e:
+            kh.reduce_ex(*args, **kw)
+        assert words in e.value.message, e.value.message
 
 
 @pytest.mark.parametrize("seed", range(32))

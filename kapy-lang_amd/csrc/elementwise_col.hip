@@ -15,14 +15,10 @@ namespace {
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-// exp(x) = 2^hi * (1 + lo * ln 2), hi + lo = x * log2(e) with lo the product's rounding error: within 2 ulp of fp32
-__device__ __forceinline__ float exp_f32(float x) {
-  const float hi = x * 1.44269504088896341f;
-  float lo = __builtin_fmaf(x, 1.44269504088896341f, -hi);
-  lo = fabsf(x) < 3e38f ? lo : 0.f;
-  const float pw = __builtin_amdgcn_exp2f(hi);
-  return pw > 3e38f ? pw : __builtin_fmaf(pw, lo * 0.693147180559945309f, pw);
-}
+// exp(x) for x <= 0 up to a relative error of about |x| * 1e-7 (the rounding of x * log2 e): the differences from a column's
+// maximum that matter are a few tens at most, so this stays some hundred times below the 16-bit rounding of the result.
+constexpr float kLog2e = 1.44269504088896341f;
+__device__ __forceinline__ float exp_f32(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
 
 template <bool BF16>
 __device__ __forceinline__ void widen16(u32x4_t v, float (&f)[8]) {
@@ -90,8 +86,9 @@ __global__ __launch_bounds__(256) void col_softmax_stats_kernel(ColSoftmax p, in
           top = fmaxf(top, f[u][e]);   // (a NaN element is skipped here; its exp below makes the sum NaN, which marks the column)
         }
         float acc = s[e] * exp_f32(m[e] - top);
+        const float bias = -top * kLog2e;   // exp(x - top) as 2^(x * log2 e - top * log2 e): one fused multiply-add per element
 #pragma unroll
-        for (int u = 0; u < U; ++u) acc += exp_f32(f[u][e] - top);
+        for (int u = 0; u < U; ++u) acc += __builtin_amdgcn_exp2f(__builtin_fmaf(f[u][e], kLog2e, bias));
         s[e] = acc;
         m[e] = top;
       }
@@ -158,18 +155,16 @@ __global__ __launch_bounds__(256) void col_softmax_stats_kernel(ColSoftmax p, in
 }
 
 // y = exp(x - M) / S: a lane owns 8 consecutive columns, keeps their M and 1 / S in registers and walks `rows_per_wg` rows,
-// two in flight.  The quotient is e * (1 / S) corrected once by its remainder (the correctly rounded e / S but for rare
-// last-bit cases, far inside the 16-bit rounding that follows).
+// two in flight.  The quotient is e * (1 / S): within two fp32 ulps of e / S, far inside the 16-bit rounding that follows.
 template <bool BF16>
 __global__ __launch_bounds__(256) void col_softmax_apply_kernel(ColSoftmax p, int32_t rows_per_wg) {
   const int32_t col0 = (blockIdx.x * 256 + threadIdx.x) * 8;
   if (col0 >= p.cols) return;
-  float M[8], S[8], R[8];
+  float M[8], R[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    M[e] = p.stats[col0 + e];
-    S[e] = p.stats[p.cols + col0 + e];
-    R[e] = __builtin_amdgcn_rcpf(S[e]);
+    M[e] = -p.stats[col0 + e] * kLog2e;   // exp(x - M) as 2^(x * log2 e - M * log2 e)
+    R[e] = __builtin_amdgcn_rcpf(p.stats[p.cols + col0 + e]);
   }
   const int32_t r_begin = blockIdx.y * rows_per_wg, r_end = min(p.rows, r_begin + rows_per_wg);
   const char *col = p.x + (int64_t)col0 * 2;
@@ -187,10 +182,7 @@ __global__ __launch_bounds__(256) void col_softmax_apply_kernel(ColSoftmax p, in
       u32x4_t o;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float ex = exp_f32(f[e] - M[e]);
-        float q = ex * R[e];
-        q = __builtin_fmaf(__builtin_fmaf(-q, S[e], ex), R[e], q);
-        f[e] = (S[e] != S[e] || fabsf(S[e]) > 3e38f || q != q) ? __fdiv_rn(ex, S[e]) : q;   // NaN / infinite sums: the plain division's answer
+        f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], kLog2e, M[e])) * R[e];   // (S >= 1 and finite, or NaN, which 1 / S and the product hand on)
       }
 #pragma unroll
       for (int w = 0; w < 4; ++w) o[w] = BF16 ? pack2_bf16_rn(f[2 * w], f[2 * w + 1]) : pack2_f16_rn(f[2 * w], f[2 * w + 1]);

@@ -197,19 +197,23 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 constexpr int kTiledFromM = 161, kTiledFromMSplit = 65;
 constexpr int kTiledFromMNoBlock = 81, kTiledFromMSplitNoBlock = 40;
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
-template <int A_FMT, int B_FMT>
+// NG: groups of 16 columns a wave multiplies with one activation chunk (a stage is then NG weight parts and one activation part
+// of 4 KiB each).  NG = 1 re-reads the whole activation per 16 columns - as many bytes from the L2s as the weight itself at
+// M = 16; NG = 2 halves that with one workgroup of 96 KiB per CU.
+template <int A_FMT, int B_FMT, int NG, int STAGES>
 __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Params p) {
-  __shared__ __attribute__((aligned(1024))) char ring[kStreamWaves * kStreamStages * kStreamStage];
+  constexpr int kPart = 16 * kStreamChunk, kStage = (NG + 1) * kPart, kLoads = 4 * (NG + 1);
+  __shared__ __attribute__((aligned(1024))) char ring[kStreamWaves * STAGES * kStage];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // Workgroup id -> (16-column block, 16-row group).  With more than one row group the workgroups that stream the same
+  // Workgroup id -> (block of 16 * NG columns, 16-row group).  With more than one row group the workgroups that stream the same
   // columns of the weight must meet in one L2: consecutive ids go to the 8 XCDs in turn, so the groups of a column block
   // take ids 8 apart (the same XCD, dispatched back to back) and the second reader of a weight line finds it there.
-  const int32_t col_blocks = (p.N + 15) / 16, groups = (p.M + 15) / 16;
+  const int32_t col_blocks = (p.N + 16 * NG - 1) / (16 * NG), groups = (p.M + 15) / 16;
   const int32_t on_xcd = blockIdx.x / 8, xcd = blockIdx.x % 8;
   const int32_t col_block = (on_xcd / groups) * 8 + xcd;
   if (col_block >= col_blocks) return;  // (the grid is padded to whole rounds of 8)
-  const int32_t n0 = col_block * 16, m0 = (on_xcd % groups) * 16;
+  const int32_t n0 = col_block * 16 * NG, m0 = (on_xcd % groups) * 16;
   const int32_t k_per_wave = p.K / kStreamWaves, chunks = k_per_wave / kStreamChunk;
   auto uniform_ptr = [](const uint8_t *ptr) {
     const uint64_t v = (uint64_t)ptr;
@@ -218,27 +222,30 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
   };
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.b + (int64_t)n0 * p.b_sn + (int64_t)wave * k_per_wave), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm + (int64_t)wave * k_per_wave), 0, 0x7fffffff, 0x00020000);
-  // load instruction i (0..3) of an operand: rows 4i .. 4i+3, this lane row 4i + lane/16, stored chunk lane%16
-  uint32_t w_off[4], a_off[4];
+  // load instruction i (0..3) of a 16-row part: rows 4i .. 4i+3, this lane row 4i + lane/16, stored chunk lane%16
+  uint32_t w_off[NG][4], a_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = 4 * i + (lane >> 4), c = (lane & 15) ^ r;
-    w_off[i] = (uint32_t)(min(r, p.N - 1 - n0) * p.b_sn + c * 16);
+#pragma unroll
+    for (int g = 0; g < NG; ++g) w_off[g][i] = (uint32_t)(min(16 * g + r, p.N - 1 - n0) * p.b_sn + c * 16);
     a_off[i] = (uint32_t)(min(r, p.M - 1 - m0) * p.a_sm + c * 16);
   }
   // A weight that only this workgroup reads (one group of rows) is loaded non-temporally: it then does not push the activation,
   // which every workgroup re-reads, out of the L2 (cache policy bit 1; M = 16: 14.6 -> 13.7 us).
   const bool w_once = groups == 1;
-  char *my_ring = ring + wave * (kStreamStages * kStreamStage);
+  char *my_ring = ring + wave * (STAGES * kStage);
   auto issue_chunk = [&](int chunk, int stage) {
-    char *dst = my_ring + stage * kStreamStage;
+    char *dst = my_ring + stage * kStage;
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (w_once) __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void *)(dst + g * kPart + i * 1024), 16, (int)w_off[g][i], chunk * kStreamChunk, 0, 2);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void *)(dst + g * kPart + i * 1024), 16, (int)w_off[g][i], chunk * kStreamChunk, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (w_once) __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, (int)w_off[i], chunk * kStreamChunk, 0, 2);
-      else __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, (int)w_off[i], chunk * kStreamChunk, 0, 0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + 4096 + i * 1024), 16, (int)a_off[i], chunk * kStreamChunk, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + NG * kPart + i * 1024), 16, (int)a_off[i], chunk * kStreamChunk, 0, 0);
   };
   // operand reads: the lane's row and its 32 K bytes of a 128-byte step: chunks 8*step + 2*group, +1
   const OperandLane frag_at = operand_lane(kF8Shape, lane);
@@ -248,44 +255,59 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
   for (int st = 0; st < 2; ++st)
 #pragma unroll
     for (int h = 0; h < 2; ++h) rd[st][h] = (uint32_t)(r16 * kStreamChunk + (((8 * st + 2 * grp + h) ^ r16) * 16));
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  issue_chunk(0, 0);
-  if (chunks > 1) issue_chunk(1, 1);
+  f32x4 acc[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < STAGES; ++st)
+    if (st < chunks) issue_chunk(st, st);
+  constexpr auto vmcnt = [](int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); };
+  int stage = 0;
   for (int32_t c = 0; c < chunks; ++c) {
-    const int stage = c & 1;
-    if (c + 1 < chunks) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);  // vmcnt(8): this chunk has landed, the next may be in flight
-    else __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
-    const char *src = my_ring + stage * kStreamStage;
-    i32x4 w[2][2], a[2][2];
+    // this chunk has landed; the (up to STAGES - 1) chunks issued after it may still be in flight
+    const int behind = min(STAGES - 1, chunks - 1 - c);
+    if (behind >= 2) __builtin_amdgcn_s_waitcnt(vmcnt(2 * kLoads));
+    else if (behind == 1) __builtin_amdgcn_s_waitcnt(vmcnt(kLoads));
+    else __builtin_amdgcn_s_waitcnt(vmcnt(0));
+    const char *src = my_ring + stage * kStage;
+    i32x4 w[NG][2][2], a[2][2];
 #pragma unroll
     for (int st = 0; st < 2; ++st)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        w[st][h] = *(const i32x4 *)(src + rd[st][h]);
-        a[st][h] = *(const i32x4 *)(src + 4096 + rd[st][h]);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) w[g][st][h] = *(const i32x4 *)(src + g * kPart + rd[st][h]);
+        a[st][h] = *(const i32x4 *)(src + NG * kPart + rd[st][h]);
       }
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the stage has been read, it may be refilled
-    if (c + 2 < chunks) issue_chunk(c + 2, stage);
+    if (c + STAGES < chunks) issue_chunk(c + STAGES, stage);
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const i32x8 av = {a[st][0][0], a[st][0][1], a[st][0][2], a[st][0][3], a[st][1][0], a[st][1][1], a[st][1][2], a[st][1][3]};
-      const i32x8 wv = {w[st][0][0], w[st][0][1], w[st][0][2], w[st][0][3], w[st][1][0], w[st][1][1], w[st][1][2], w[st][1][3]};
-      acc = mfma_f8<A_FMT, B_FMT>(av, wv, acc);
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const i32x8 wv = {w[g][st][0][0], w[g][st][0][1], w[g][st][0][2], w[g][st][0][3], w[g][st][1][0], w[g][st][1][1], w[g][st][1][2], w[g][st][1][3]};
+        acc[g] = mfma_f8<A_FMT, B_FMT>(av, wv, acc[g]);
+      }
     }
   }
   // the four K ranges meet in LDS
   const AccLane acc_at = acc_lane(mfma_acc(kF8Shape), kF8Shape, lane);
   __syncthreads();  // every wave is done with its ring
-  float *partial = (float *)ring;  // [wave][16][17]
+  float *partial = (float *)ring;  // [wave][NG][16][17]
 #pragma unroll
-  for (int v = 0; v < 4; ++v) partial[(wave * 16 + acc_at.row + v) * 17 + acc_at.col] = acc[v];
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) partial[((wave * NG + g) * 16 + acc_at.row + v) * 17 + acc_at.col] = acc[g][v];
   __syncthreads();
-  {
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
     const int m = threadIdx.x >> 4, n = threadIdx.x & 15;
     float sum = 0.f;
 #pragma unroll
-    for (int w2 = 0; w2 < kStreamWaves; ++w2) sum += partial[(w2 * 16 + m) * 17 + n];
-    finish(p, m0 + m, n0 + n, sum);
+    for (int w2 = 0; w2 < kStreamWaves; ++w2) sum += partial[((w2 * NG + g) * 16 + m) * 17 + n];
+    finish(p, m0 + m, n0 + 16 * g + n, sum);
   }
 }
 
@@ -487,13 +509,23 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
       p.b_sn * 16 < (int64_t(1) << 31)) {
     // rows are addressed from the workgroup's first row, so the per-lane offsets stay small
     F8Params q = p;
-    const int64_t col_rounds = ((p.N + 15) / 16 + 7) / 8, groups = (p.M + 15) / 16;
+    // two column groups per wave (half the activation traffic, 96 KiB of LDS per workgroup) where that still gives every CU a workgroup
+    const int64_t groups = (p.M + 15) / 16;
+    const int ng = groups == 1 && (int64_t)(p.N + 31) / 32 >= device_cus() ? 2 : 1;
+    const int64_t col_rounds = ((p.N + 16 * ng - 1) / (16 * ng) + 7) / 8;
     dim3 grid((unsigned)(col_rounds * 8 * groups));
     int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
-    if (fa == 0 && fb == 0) skinny_stream_kernel<0, 0><<<grid, 64 * kStreamWaves, 0, s>>>(q);
-    else if (fa == 0) skinny_stream_kernel<0, 1><<<grid, 64 * kStreamWaves, 0, s>>>(q);
-    else if (fb == 0) skinny_stream_kernel<1, 0><<<grid, 64 * kStreamWaves, 0, s>>>(q);
-    else skinny_stream_kernel<1, 1><<<grid, 64 * kStreamWaves, 0, s>>>(q);
+#define KAPY_STREAM(NG_, ST_)                                                                                    \
+  do {                                                                                                        \
+    if (fa == 0 && fb == 0) skinny_stream_kernel<0, 0, NG_, ST_><<<grid, 64 * kStreamWaves, 0, s>>>(q);       \
+    else if (fa == 0) skinny_stream_kernel<0, 1, NG_, ST_><<<grid, 64 * kStreamWaves, 0, s>>>(q);             \
+    else if (fb == 0) skinny_stream_kernel<1, 0, NG_, ST_><<<grid, 64 * kStreamWaves, 0, s>>>(q);             \
+    else skinny_stream_kernel<1, 1, NG_, ST_><<<grid, 64 * kStreamWaves, 0, s>>>(q);                          \
+  } while (0)
+    // (rings of three stages measured no faster: N = K = 8192, M = 16: 13.3 us with two column groups either way, 14.8 with one)
+    if (ng == 2) KAPY_STREAM(2, kStreamStages);
+    else KAPY_STREAM(1, kStreamStages);
+#undef KAPY_STREAM
     KAPY_HIP_CHECK(hipGetLastError());
     return KAPY_OK;
   }

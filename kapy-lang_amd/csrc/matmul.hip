@@ -1595,6 +1595,26 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
   p.tiles_n = (p.N + BN - 1) / BN;
   constexpr bool kCanSplit = BM == 128 && BN == 128 && STAGES == kRing25;
   if (!kCanSplit) p.split_k = 1;
+  if constexpr (C::kLdsBytes > 64 * 1024) {
+    // A kernel whose LDS-direct loads address more than the 64 KiB every runtime grants: before its first launch on a device,
+    // ask the runtime what it will give it - the code object's static size must be the kernel's own and within the device's
+    // limit per workgroup - and refuse instead of launching loads that would land outside the workgroup's allocation.
+    static int checked[kMaxDevices];  // 0 not asked, 1 fine, -1 refused (a race between two first calls only repeats the query)
+    int dev = -1;
+    KAPY_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(KAPY_ERR_UNSUPPORTED, "matmul: device ordinal %d beyond %d", dev, kMaxDevices);
+    int state = __atomic_load_n(&checked[dev], __ATOMIC_ACQUIRE);
+    if (state == 0) {
+      hipFuncAttributes attr;
+      int limit = 0;
+      const hipError_t e1 = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
+      const hipError_t e2 = hipDeviceGetAttribute(&limit, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
+      state = (e1 == hipSuccess && e2 == hipSuccess && (int64_t)attr.sharedSizeBytes == (int64_t)C::kLdsBytes && limit >= C::kLdsBytes) ? 1 : -1;
+      (void)hipGetLastError();
+      __atomic_store_n(&checked[dev], state, __ATOMIC_RELEASE);
+    }
+    if (state < 0) return fail(KAPY_ERR_HIP, "matmul: the runtime does not give this kernel the %d bytes of LDS it addresses (nothing was launched)", C::kLdsBytes);
+  }
   kernel<<<dim3((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.split_k), dim3(C::kThreads), 0, s>>>(p);
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
@@ -1890,6 +1910,9 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
       // with a free choice, a 256x256 tiling with fewer than 0.55 tiles per CU yields to 128x128 (measured: 144 large tiles on
       // 256 CUs beat 576 small ones - 3072^3: 1009 against 899 TFLOP/s - 128 do not)
       if (free_choice && v.bm == 256 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 < (int64_t)device_cus() * 55) continue;
+      // an explicit split of K is a request for a variant that can split: with a free tile choice the others are passed over
+      // (plan_split_k then honours the split or says why it cannot)
+      if (c.split_k > 1 && !c.tile_m && !(v.bm == 128 && v.stages == kRing25)) continue;
       if (v.bm == 128 && v.stages == kRing25) {
         rc = plan_split_k(p, c, v.bk);
         if (rc) return rc;

@@ -219,8 +219,51 @@ static int run_gpu() {
   return 0;
 }
 
+// The 256 x 256 x 64 ring kernel (all 160 KiB of a CU's LDS, declared statically) launched from a process that never loaded
+// torch: bf16, A row-major, B column-major, through the C ABI with the tile named in the configuration.
+static int run_gpu_large_tile() {
+  const int M = 512, N = 512, K = 256;
+  std::vector<uint16_t> a(M * K), w(N * K), c(M * N);
+  srand(11);
+  auto rnd = [] { return (float)(rand() % 65536) / 65536.f - 0.5f; };
+  for (auto &v : a) v = f2b(rnd());
+  for (auto &v : w) v = f2b(rnd());
+  uint16_t *da, *dw, *dc;
+  HIP_OK(hipMalloc((void **)&da, a.size() * 2)); HIP_OK(hipMalloc((void **)&dw, w.size() * 2)); HIP_OK(hipMalloc((void **)&dc, c.size() * 2));
+  HIP_OK(hipMemcpy(da, a.data(), a.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(dw, w.data(), w.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemset(dc, 0, c.size() * 2));
+  kapy_global ga, gw, gc;
+  EXPECT(kapy_mk_global(&ga, da, 0, M, K, K, 1, KAPY_BF16, 16) == KAPY_OK);
+  EXPECT(kapy_mk_global(&gw, dw, 0, K, N, 1, K, KAPY_BF16, 16) == KAPY_OK);
+  EXPECT(kapy_mk_global(&gc, dc, 0, M, N, N, 1, KAPY_BF16, 16) == KAPY_OK);
+  kapy_matmul_cfg cfg = {KAPY_MATMUL_AUTO, 256, 256, 64, KAPY_RN, 0, 0, 0, nullptr, 0};
+  printf("launching the 256 x 256 x 64 ring kernel (M = N = %d, K = %d)\n", M, K);
+  fflush(stdout);
+  const int rc = kapy_matmul(&ga, &gw, nullptr, &gc, &cfg, nullptr);
+  if (rc != KAPY_OK) {
+    printf("FAILED: kapy status %d: %s\n", rc, kapy_last_error());
+    return 1;
+  }
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(c.data(), dc, c.size() * 2, hipMemcpyDeviceToHost));
+  double err2 = 0, ref2 = 0;
+  for (int i = 0; i < M; ++i)
+    for (int j = 0; j < N; ++j) {
+      double s = 0;
+      for (int k = 0; k < K; ++k) s += (double)b2f(a[i * K + k]) * b2f(w[j * K + k]);
+      const double got = b2f(c[i * N + j]);
+      err2 += (got - s) * (got - s);
+      ref2 += s * s;
+    }
+  EXPECT(sqrt(err2 / ref2) <= 4e-3);
+  printf("builder gpu large tile ok\n");
+  return 0;
+}
+
 int main(int argc, char **argv) {
   try {
+    if (argc > 1 && std::string(argv[1]) == "gpu256") return run_gpu_large_tile();
     return argc > 1 && std::string(argv[1]) == "gpu" ? run_gpu() : run_cpu();
   } catch (const kapy::Error &e) {
     printf("FAILED: kapy status %d: %s\n", e.status, e.what());

@@ -24,3 +24,12 @@ def test_builder_lowers_and_refuses_without_a_device():
 def test_builder_runs_the_graphs_on_the_gpu():
     out = subprocess.run([_binary(), "gpu"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0 and "builder gpu ok" in out.stdout, out.stdout + out.stderr
+
+
+@pytest.mark.gpu
+def test_the_full_lds_ring_kernel_runs_in_a_process_without_torch():
+    """The 256 x 256 x 64 tiles address all 160 KiB of a CU's LDS, declared statically in the code object and checked against the
+    runtime's own figures before the first launch; this C++ process links the system HIP runtime directly."""
+    out = subprocess.run([_binary(), "gpu256"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "builder gpu large tile ok" in out.stdout, out.stdout + out.stderr
+

@@ -153,3 +153,25 @@ def test_split_k_refusals(ko):
         with pytest.raises(kh.KapyError) as e:
             kh.matmul(g, g, g, tile=(128, 128, 64), **kw)
         assert e.value.status == status, kw
+
+
+def test_an_explicit_split_with_a_free_tile_choice_is_honoured(ko):
+    """A problem large enough for the 256 x 256 tiles (which cannot split K): an explicit split_k moves the call to the
+    128 x 128 tiles instead of being dropped; the result equals the unsplit call's within the GEMM bar, and a split the
+    workspace cannot hold is refused, not ignored."""
+    dt, M, N, K = kh.BF16, 4096, 4096, 512
+    a, b = ko.fill_normal(M * K, dt, 41, 0, 0.0, 0.5), ko.fill_normal(N * K, dt, 42, 0, 0.0, 0.5)
+    da, db = to_dev(a), to_dev(b)
+    ga, gb = dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt)
+    plain, split = dev_zeros(M * N, 2), dev_zeros(M * N, 2)
+    kh.matmul(ga, gb, dglobal(plain, M, N, N, 1, dt))
+    ws = _workspace(M, N)
+    kh.matmul(ga, gb, dglobal(split, M, N, N, 1, dt), split_k=2, workspace=ws)
+    sync()
+    p, q = ko.decode(to_host(plain, np.uint16), dt), ko.decode(to_host(split, np.uint16), dt)
+    assert np.linalg.norm(p - q) <= 2e-3 * np.linalg.norm(p) and not np.array_equal(to_host(split, np.uint16), np.zeros(M * N, np.uint16))
+    assert not ws[:16384].any()                                        # the split ran: its counters were used and are back at zero
+    with pytest.raises(kh.KapyError) as e:
+        kh.matmul(ga, gb, dglobal(split, M, N, N, 1, dt), split_k=2, workspace=(ws.data_ptr(), 16384 + 4096))
+    assert e.value.status == kh.ERR_UNSUPPORTED
+

@@ -767,7 +767,8 @@ def bench_ceilings(kh, steps, warmup, cpu):
     import numpy as np
     import torch
     import ko
-    out = {"workload": "device ceilings (the library's probe kernels)", "checked": True, "check": "nothing to check: measurement only", "mfma": {}, "copy": {}}
+    import kapy_probe as kp
+    out = {"workload": "device ceilings (the probe library's kernels)", "checked": True, "check": "nothing to check: measurement only", "mfma": {}, "copy": {}}
     sink = torch.empty(1024 * 256, device="cuda", dtype=torch.float32)
     ticks = torch.zeros(4 * 1024, device="cuda", dtype=torch.int64)
     for name, way, dt, gen, peak in (("bf16 16x16x32", kh.MFMA_16X16X32_16B, kh.BF16, "normal002", 2500.0), ("bf16 32x32x16", kh.MFMA_32X32X16_16B, kh.BF16, "normal002", 2500.0),
@@ -784,8 +785,8 @@ def bench_ceilings(kh, steps, warmup, cpu):
             ko.lib().ko_quantize_e4m3(x.ctypes.data, x.shape[0], x.shape[1], x.shape[1], 1, 1, q.ctypes.data, sc.ctypes.data)
             ops = _upload(q)
         iters = 2000
-        wgs, flops = kh.probe_mfma(way, dt, ops.data_ptr(), iters, sink.data_ptr())
-        wall, ev = _events(lambda i: kh.probe_mfma(way, dt, ops.data_ptr(), iters, sink.data_ptr(), ticks.data_ptr()), max(steps // 2, 5), warmup)
+        wgs, flops = kp.probe_mfma(way, dt, ops.data_ptr(), iters, sink.data_ptr())
+        wall, ev = _events(lambda i: kp.probe_mfma(way, dt, ops.data_ptr(), iters, sink.data_ptr(), ticks.data_ptr()), max(steps // 2, 5), warmup)
         torch.cuda.synchronize()
         t = ticks.cpu().numpy()[:4 * wgs].reshape(wgs, 4).astype(np.float64)
         ghz = float(np.median((t[:, 1] - t[:, 0]) / np.maximum(t[:, 3] - t[:, 2], 1.0)) * 0.1)    # shader ticks per 100 MHz tick
@@ -794,7 +795,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
     nbytes, sets = 128 << 20, 4
     src = [_dev("bits16", nbytes // 2, ko.F16, 0, k) for k in range(sets)]
     dst = [torch.empty(nbytes // 2, device="cuda", dtype=torch.int16) for _ in range(sets)]
-    kh.probe_copy(src[0].data_ptr(), dst[0].data_ptr(), nbytes)
+    kp.probe_copy(src[0].data_ptr(), dst[0].data_ptr(), nbytes)
     torch.cuda.synchronize()
     if not torch.equal(src[0], dst[0]):
         raise CheckFailed("probe_copy: result differs from the source")
@@ -804,7 +805,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
             for pers in (0, 4, 8, 16):
                 if pers and u > 8:
                     continue
-                wall, ev = _events(lambda i: kh.probe_copy(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), nbytes, u, ntl, nts, pers), 20, 3)
+                wall, ev = _events(lambda i: kp.probe_copy(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), nbytes, u, ntl, nts, pers), 20, 3)
                 gbs = 2 * nbytes / (ev * 1e-3) / 1e9
                 best = max(best, gbs)
                 out["copy"]["vec%d ntld%d ntst%d %s" % (u, ntl, nts, "persistent x%d" % pers if pers else "one pass")] = round(gbs, 0)
@@ -812,20 +813,33 @@ def bench_ceilings(kh, steps, warmup, cpu):
     # instruction instead of one contiguous KiB), untransposed: what the transposes can reach
     n = 8192
     for lds in (0, 1):
-        kh.probe_copy_tiled(src[0].data_ptr(), dst[0].data_ptr(), n, n * 2, lds)
+        kp.probe_copy_tiled(src[0].data_ptr(), dst[0].data_ptr(), n, n * 2, lds)
         torch.cuda.synchronize()
         if not torch.equal(src[0], dst[0]):
             raise CheckFailed("probe_copy_tiled: result differs from the source")
-        wall, ev = _events(lambda i: kh.probe_copy_tiled(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, lds), 40, 5)
+        wall, ev = _events(lambda i: kp.probe_copy_tiled(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, lds), 40, 5)
         out["copy"]["transpose footprint (128 rows x 256 B per workgroup)%s" % (", through LDS and a barrier" if lds else "")] = round(2 * nbytes / (ev * 1e-3) / 1e9, 0)
     # ... and by the length of the contiguous runs alone (a transposing kernel's runs are as long as its tile is wide)
     for run in (256, 512, 1024, 2048, 4096):
-        kh.probe_copy_runs(src[0].data_ptr(), dst[0].data_ptr(), n, n * 2, run)
+        kp.probe_copy_runs(src[0].data_ptr(), dst[0].data_ptr(), n, n * 2, run)
         torch.cuda.synchronize()
         if not torch.equal(src[0], dst[0]):
             raise CheckFailed("probe_copy_runs: result differs from the source")
-        wall, ev = _events(lambda i: kh.probe_copy_runs(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, run), 40, 5)
+        wall, ev = _events(lambda i: kp.probe_copy_runs(src[i % sets].data_ptr(), dst[i % sets].data_ptr(), n, n * 2, run), 40, 5)
         out["copy"]["runs of %d B (%d rows x %d B per workgroup)" % (run, 32768 // run, run)] = round(2 * nbytes / (ev * 1e-3) / 1e9, 0)
+    # a read-only stream (the weight matrix of a skinny GEMM, the operand of a reduce): 64 MiB buffers in rotation
+    out["read"] = {}
+    rsink = torch.zeros(1 << 20, dtype=torch.int32, device="cuda")
+    rbytes, best_read = 64 << 20, 0.0
+    for u in (1, 2, 4, 8):
+        for ntl in (0, 1):
+            for pers in (0, 4, 8):
+                wall, ev = _events(lambda i: kp.probe_read(src[i % sets].data_ptr() + (i // sets % 2) * rbytes, rbytes, u, ntl, pers, rsink.data_ptr()), 24, 4)
+                gbs = rbytes / (ev * 1e-3) / 1e9
+                best_read = max(best_read, gbs)
+                out["read"]["vec%d ntld%d %s" % (u, ntl, "persistent x%d" % pers if pers else "one pass")] = round(gbs, 0)
+    out["read_best_gbs"] = round(best_read, 0)
+    out["read_best_frac_of_peak"] = round(best_read / HBM_PEAK_GBS, 4)
     out["copy_best_gbs"] = round(best, 0)
     out["copy_best_frac_of_peak"] = round(best / HBM_PEAK_GBS, 4)
     # what the L2s hand to the CUs: every CU re-reads a window that stays in its XCD's L2 (2 MiB), that spills to the Infinity
@@ -836,8 +850,8 @@ def bench_ceilings(kh, steps, warmup, cpu):
         buf = torch.empty(8 * window, dtype=torch.uint8, device="cuda")
         buf.random_(0, 255)
         for to_lds in (True, False):
-            _, nb = kh.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr())
-            wall, ev = _events(lambda i: kh.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr()), 10, 3)
+            _, nb = kp.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr())
+            wall, ev = _events(lambda i: kp.probe_l2_read(buf.data_ptr(), window, 512, 1, to_lds, sink.data_ptr()), 10, 3)
             out["l2_read_tbs"]["%d MiB per XCD, %s" % (window >> 20, "LDS-direct" if to_lds else "to registers")] = round(nb / (ev * 1e-3) / 1e12, 2)
         del buf
     # what a wave can issue beside its matrix instructions (one wave per SIMD, as in the tiled matmuls): fillers in the gap
@@ -846,13 +860,14 @@ def bench_ceilings(kh, steps, warmup, cpu):
     fsink = torch.empty(1024 * 256, device="cuda", dtype=torch.float32)
     window = torch.empty(8 * (2 << 20), dtype=torch.uint8, device="cuda")
     window.random_(0, 120)
-    for name, way, fills in (("bf16 16x16x32", kh.MFMA_16X16X32_16B, ((0, 0), (1, 3), (1, 4), (1, 6), (2, 1), (2, 2), (2, 3), (3, 0))),
-                             ("e4m3 16x16x128", kh.MFMA_16X16X128_F8, ((0, 0), (1, 6), (1, 8), (2, 2), (2, 3), (2, 4), (3, 0)))):
+    for name, way, fills in (("bf16 16x16x32", kh.MFMA_16X16X32_16B, ((0, 0), (1, 3), (1, 4), (1, 6), (2, 1), (2, 2), (2, 3), (3, 0), (4, 0))),
+                             ("e4m3 16x16x128", kh.MFMA_16X16X128_F8, ((0, 0), (1, 6), (1, 8), (2, 2), (2, 3), (2, 4), (3, 0), (4, 0)))):
         row = {}
         for filler, count in fills:
-            _, flops = kh.probe_issue(way, filler, count, window.data_ptr(), 2000, fsink.data_ptr())
-            wall, ev = _events(lambda i: kh.probe_issue(way, filler, count, window.data_ptr(), 2000, fsink.data_ptr()), 6, 3)
-            label = ("nothing", "%d scalar" % count, "%d vector ALU" % count, "matmul loop: 32 LDS reads + 16 LDS-direct loads per tile")[filler]
+            _, flops = kp.probe_issue(way, filler, count, window.data_ptr(), 2000, fsink.data_ptr())
+            wall, ev = _events(lambda i: kp.probe_issue(way, filler, count, window.data_ptr(), 2000, fsink.data_ptr()), 6, 3)
+            label = ("nothing", "%d scalar" % count, "%d vector ALU" % count, "matmul loop: 32 LDS reads + 16 LDS-direct loads per tile",
+                     "rhs off the LDS: 16 LDS reads + 8 LDS-direct loads + 16 register loads per tile")[filler]
             row[label] = round(flops / (ev * 1e-3) / 1e12, 1)
         out["issue_tflops"][name] = row
     del window

@@ -1744,45 +1744,6 @@ int launch_f8(const GemmParams &p, int lhs_fmt, int rhs_fmt, hipStream_t s) {
   }
 }
 
-// One matrix instruction on one wavefront, registers in and registers out: lhs / rhs hold each lane's operand
-// registers back to back (kpack elements per lane), acc gets each lane's accumulator registers.  The policy is
-// the one the kernels multiply with, so what this shows about register positions holds for them.
-template <typename T, bool EXCHANGED>
-__global__ __launch_bounds__(64) void probe_kernel(const char *lhs, const char *rhs, float *acc) {
-  const int lane = threadIdx.x;
-  constexpr int kLaneBytes = T::kShape.kpack * T::kBytes, kRegs = T::kShape.m * T::kShape.n / 64;
-  static_assert(kLaneBytes == 16 * T::kChunks, "a lane's operand registers are whole 16-byte chunks");
-  u32x4 a[T::kChunks], b[T::kChunks];
-#pragma unroll
-  for (int c = 0; c < T::kChunks; ++c) {
-    a[c] = *(const u32x4 *)(lhs + lane * kLaneBytes + 16 * c);
-    b[c] = *(const u32x4 *)(rhs + lane * kLaneBytes + 16 * c);
-  }
-  typename T::Acc d;
-#pragma unroll
-  for (int v = 0; v < kRegs; ++v) d[v] = 0.f;
-  d = EXCHANGED ? T::mfma(b, a, d) : T::mfma(a, b, d);
-#pragma unroll
-  for (int v = 0; v < kRegs; ++v) acc[lane * kRegs + v] = d[v];
-}
-template <typename T>
-int launch_probe(bool exchanged, const void *lhs, const void *rhs, float *acc, hipStream_t s) {
-  if (exchanged) probe_kernel<T, true><<<1, 64, 0, s>>>((const char *)lhs, (const char *)rhs, acc);
-  else probe_kernel<T, false><<<1, 64, 0, s>>>((const char *)lhs, (const char *)rhs, acc);
-  KAPY_HIP_CHECK(hipGetLastError());
-  return KAPY_OK;
-}
-// FIRST / SECOND: the fp8 formats of the instruction's first / second operand slot
-template <template <int, int> class P>
-int launch_probe_f8(int first_fmt, int second_fmt, bool exchanged, const void *lhs, const void *rhs, float *acc, hipStream_t s) {
-  switch (first_fmt * 2 + second_fmt) {
-  case 0: return launch_probe<P<0, 0>>(exchanged, lhs, rhs, acc, s);
-  case 1: return launch_probe<P<0, 1>>(exchanged, lhs, rhs, acc, s);
-  case 2: return launch_probe<P<1, 0>>(exchanged, lhs, rhs, acc, s);
-  default: return launch_probe<P<1, 1>>(exchanged, lhs, rhs, acc, s);
-  }
-}
-
 }  // namespace
 
 // Decides whether the 128 x 128 tiled kernels split K for this problem and points the parameters at the workspace.
@@ -2035,30 +1996,6 @@ int kapy_matmul_fused(const kapy_global *lhs, const kapy_global *rhs, const kapy
       return fail(KAPY_ERR_VERIFY, "broadcast: the bias must be one contiguous row [1 x N]");
   }
   return matmul_16bit(lhs, rhs, nullptr, result, cfg, epi, stream);
-}
-
-int kapy_mfma_probe(int32_t impl_way, int32_t lhs_dtype, int32_t rhs_dtype, int32_t exchanged, const void *lhs_regs, const void *rhs_regs,
-                    float *acc_regs, void *stream) {
-  if (!lhs_regs || !rhs_regs || !acc_regs) return fail(KAPY_ERR_INVALID, "mfma_probe: null register array");
-  const bool f8 = is_f8(lhs_dtype) && is_f8(rhs_dtype), b16 = (lhs_dtype == KAPY_F16 || lhs_dtype == KAPY_BF16) && rhs_dtype == lhs_dtype;
-  const bool way16 = impl_way == KAPY_MFMA_32X32X16_16B || impl_way == KAPY_MFMA_16X16X32_16B;
-  const bool way8 = impl_way == KAPY_MFMA_16X16X128_F8 || impl_way == KAPY_MFMA_32X32X64_F8;
-  if (!way16 && !way8) return fail(KAPY_ERR_INVALID, "mfma_probe: impl_way must name a matrix instruction of gfx950 (16..19), not %d", impl_way);
-  if ((way16 && !b16) || (way8 && !f8)) return fail(KAPY_ERR_VERIFY, "mfma_probe: operand element types do not fit the instruction");
-  int rc = ensure_device();
-  if (rc) return rc;
-  hipStream_t s = (hipStream_t)stream;
-  const bool ex = exchanged != 0;
-  if (way16) {
-    const bool bf = lhs_dtype == KAPY_BF16;
-    if (impl_way == KAPY_MFMA_32X32X16_16B) return bf ? launch_probe<Bf16>(ex, lhs_regs, rhs_regs, acc_regs, s) : launch_probe<F16>(ex, lhs_regs, rhs_regs, acc_regs, s);
-    return bf ? launch_probe<Bf16M16>(ex, lhs_regs, rhs_regs, acc_regs, s) : launch_probe<F16M16>(ex, lhs_regs, rhs_regs, acc_regs, s);
-  }
-  // exchanged: the rhs fragment sits in the first operand slot, so the first format selector is the rhs's
-  const int lf = lhs_dtype == KAPY_F8E5M2, rf = rhs_dtype == KAPY_F8E5M2;
-  const int first = ex ? rf : lf, second = ex ? lf : rf;
-  if (impl_way == KAPY_MFMA_16X16X128_F8) return launch_probe_f8<F8M16>(first, second, ex, lhs_regs, rhs_regs, acc_regs, s);
-  return launch_probe_f8<F8>(first, second, ex, lhs_regs, rhs_regs, acc_regs, s);
 }
 
 int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling *out) {

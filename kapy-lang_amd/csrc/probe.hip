@@ -9,14 +9,18 @@
 //   kapy_probe_copy   a 16-byte-per-lane copy in the forms a memory-bound kernel can take (vectors per lane, ordinary or
 //                     non-temporal loads and stores, one pass over a big grid or persistent workgroups striding over
 //                     the buffer): the rate a read + write stream reaches on this part.
+//   kapy_probe_read   the same without the stores: what a kernel that streams an operand and writes little can approach.
 //   kapy_probe_l2_read  every CU reads a window that stays in its XCD's L2, over and over: the rate at which the L2s feed
 //                     the CUs, which is what a tiled matmul's global->LDS traffic runs against.
+//   kapy_mfma_probe   one matrix instruction on one wavefront, registers in and out (binds the exported operand layouts to
+//                     the hardware in a test).
 // The first two record per-workgroup shader-clock and constant-rate timer ticks, from which the sustained clock follows.
 //
 // The reference has no counterpart: it emits code and never runs it (its matmul instruction strings:
 // lib/Conversion/KgpuToLLVM/MatmulOpToLLVM.cpp:269-311; its loads and stores: LdGlobalOpToLLVM.cpp:60-145).
 #include "common.hpp"
 #include "mfma.hpp"
+#include "kapy_probe.h"
 
 namespace kapy {
 namespace {
@@ -166,6 +170,37 @@ __global__ __launch_bounds__(256) void copy_runs_kernel(const char *__restrict__
   for (int c = 0; c < 8; ++c) __builtin_nontemporal_store(v[c], (vec16 *)(dst + base + (int64_t)c * kRowsPerPass * row_bytes));
 }
 
+// A read-only stream: every lane folds U vectors of 16 bytes per pass into a word nobody needs (written only for a value the
+// fold never takes), in one pass over a big grid or by persistent workgroups striding over the buffer.  What the memory system
+// delivers when nothing is written: the ceiling of a kernel that streams a large operand and writes little (a skinny GEMM's
+// weight matrix, a reduce).
+template <int U, bool NT>
+__global__ __launch_bounds__(256) void read_kernel(const vec16 *__restrict__ src, int64_t n, uint32_t *sink) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  uint32_t fold = 0;
+  for (int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x; base < n; base += stride * U) {
+    vec16 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * stride;
+      v[u] = vec16{0, 0, 0, 0};
+      if (i < n) v[u] = NT ? __builtin_nontemporal_load(src + i) : src[i];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) fold ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+  }
+  if (fold == 0x9e3779b9u && sink) sink[blockIdx.x] = fold;
+}
+template <int U>
+int launch_read(const void *src, int64_t n, int nt, int persistent_per_cu, uint32_t *sink, int32_t *workgroups, hipStream_t s) {
+  const int64_t grid = persistent_per_cu > 0 ? (int64_t)device_cus() * persistent_per_cu : (n + 256 * U - 1) / (256 * U);
+  if (workgroups) *workgroups = (int32_t)grid;
+  if (nt) read_kernel<U, true><<<(unsigned)grid, 256, 0, s>>>((const vec16 *)src, n, sink);
+  else read_kernel<U, false><<<(unsigned)grid, 256, 0, s>>>((const vec16 *)src, n, sink);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+
 template <int U, bool LNT, bool SNT>
 int launch_copy(const void *src, void *dst, int64_t n, int persistent_per_cu, uint64_t *ticks, int32_t *workgroups, hipStream_t s) {
   if (persistent_per_cu > 0) {
@@ -223,7 +258,8 @@ __global__ __launch_bounds__(256) void l2_read_kernel(const char *src, int64_t w
 // tiles of kTileClocks of independent matrix instructions - 128 x 16x16x32 (16 clocks each) or 64 x 16x16x128 (32 clocks) - and
 // in the gap behind every instruction FILL asks for: 1 = COUNT scalar instructions (s_nop), 2 = COUNT vector ALU instructions
 // (v_mov), 3 = the steady-state loop of the tiled matmul: 32 LDS reads of 16 bytes per lane and 16 LDS-direct loads of 1 KiB
-// per wave and tile, spread evenly and never in the same gap, from a window of 2 MiB per XCD that stays in the L2.
+// per wave and tile, spread evenly and never in the same gap, from a window of 2 MiB per XCD that stays in the L2; 4 = that loop
+// with the rhs kept off the LDS (16 LDS reads, 8 LDS-direct loads and 16 loads of 16 bytes per lane into registers per tile).
 // MF: 0 = bf16 16x16x32, 1 = e4m3 16x16x128.
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 template <int MF, int FILL, int COUNT>
@@ -245,12 +281,13 @@ __global__ __launch_bounds__(256) void issue_kernel(const char *src, int iterati
   const uint32_t unit = 0x7f7f7f7fu, lds_rd = (uint32_t)(uintptr_t)ring + wave * 32768 + lane * 16, voff = lane * 16;
   uint32_t filler = lane;
   u32x4 r[8];
+  [[maybe_unused]] u32x4 regs[16];
   for (int it = 0; it < iterations; ++it) {
 #pragma unroll
     for (int g = 0; g < kMfmas; ++g) {
       if constexpr (MF) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0] cbsz:0 blgp:0" : "+a"(acc[g % 16]) : "v"(op8), "v"(op8), "v"(unit));
       else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[g % 16]) : "v"(op4), "v"(op4));
-      if (g % kLoadEvery != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
+      if (g % (FILL == 4 ? kMfmas / 8 : kLoadEvery) != 0) __builtin_amdgcn_sched_barrier(0);  // (a load's M0 write may move ahead of the matrix instruction)
       if constexpr (FILL == 1) {
 #pragma unroll
         for (int f = 0; f < COUNT; ++f) asm volatile("s_nop 0");
@@ -272,7 +309,33 @@ __global__ __launch_bounds__(256) void issue_kernel(const char *src, int iterati
                                                    (int)(chunk * 1024), 0, 0);
         }
       }
+      if constexpr (FILL == 4) {
+        // one operand off the LDS: 16 LDS reads and 8 LDS-direct loads for the lhs half of the tile, and the wave's 16 rhs
+        // fragments of the tile as 16-byte loads into registers (lane l: row l % 16 of a 16 KiB-pitch panel, bytes
+        // 32 * (l / 16) .. + 32 of a 128-byte piece, as two loads), issued over the first half of the tile
+        constexpr int kDirectEvery = kMfmas / 8, kLdsEvery = kMfmas / 16, kRegEvery = kMfmas / 32;
+        if (g % kDirectEvery == 0) {
+          const int k = g / kDirectEvery;
+          const uint32_t chunk = at + k < kChunksInWindow ? at + k : at + k - kChunksInWindow;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(ring + wave * 32768 + 16384 + k * 1024), 16, voff,
+                                                   (int)(chunk * 1024), 0, 0);
+        } else if (g % kLdsEvery == kLdsEvery / 2) {
+          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r[(g / kLdsEvery) % 8]) : "v"(lds_rd), "n"(((g / kLdsEvery) % 16) * 1024));
+        } else if (g % kRegEvery == 1 && g < kMfmas / 2) {
+          const int j = g / kRegEvery;  // 0 .. 15: row group j / 2, half j % 2
+          regs[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (lane & 15) * 16384 + (lane >> 4) * 32 + (j & 1) * 16,
+                                                          (int)((j >> 1) * 16 * 16384 + (at * 128u) % 16384u), 0);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (FILL == 4) {
+      at = at + 8 < kChunksInWindow ? at + 8 : at + 8 - kChunksInWindow;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int k = 0; k < 8; ++k) asm volatile("" ::"v"(r[k]));
+#pragma unroll
+      for (int j = 0; j < 16; ++j) asm volatile("" ::"v"(regs[j]));  // (the compiler waits here for the register loads; the four LDS-direct loads behind them stay in flight)
     }
     if constexpr (FILL == 3) {
       at = at + 16 < kChunksInWindow ? at + 16 : at + 16 - kChunksInWindow;
@@ -295,6 +358,7 @@ int launch_issue(int filler, int count, const char *src, int iterations, float *
 #define KAPY_ISSUE(F, C) issue_kernel<MF, F, C><<<wgs, 256, 0, s>>>(src, iterations, sink)
   if (filler == 0) KAPY_ISSUE(0, 0);
   else if (filler == 3) KAPY_ISSUE(3, 0);
+  else if (filler == 4) KAPY_ISSUE(4, 0);
   else if (filler == 1 && count == 1) KAPY_ISSUE(1, 1);
   else if (filler == 1 && count == 2) KAPY_ISSUE(1, 2);
   else if (filler == 1 && count == 3) KAPY_ISSUE(1, 3);
@@ -305,7 +369,7 @@ int launch_issue(int filler, int count, const char *src, int iterations, float *
   else if (filler == 2 && count == 2) KAPY_ISSUE(2, 2);
   else if (filler == 2 && count == 3) KAPY_ISSUE(2, 3);
   else if (filler == 2 && count == 4) KAPY_ISSUE(2, 4);
-  else return fail(KAPY_ERR_INVALID, "probe_issue: filler 0 (none), 1 (scalar; count 1, 2, 3, 4, 6 or 8), 2 (vector ALU; count 1 .. 4) or 3 (the tiled matmul's reads and loads)");
+  else return fail(KAPY_ERR_INVALID, "probe_issue: filler 0 (none), 1 (scalar; count 1, 2, 3, 4, 6 or 8), 2 (vector ALU; count 1 .. 4), 3 (the tiled matmul's reads and loads) or 4 (the same with the rhs loaded into registers)");
 #undef KAPY_ISSUE
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
@@ -319,12 +383,76 @@ int launch_copy_nt(const void *src, void *dst, int64_t n, int nt_load, int nt_st
   return launch_copy<U, false, false>(src, dst, n, persistent_per_cu, ticks, workgroups, s);
 }
 
+// One matrix instruction on one wavefront, registers in and registers out: lhs / rhs hold each lane's operand
+// registers back to back (kpack elements per lane), acc gets each lane's accumulator registers.  The policy is
+// the one the kernels multiply with, so what this shows about register positions holds for them.
+template <typename T, bool EXCHANGED>
+__global__ __launch_bounds__(64) void probe_kernel(const char *lhs, const char *rhs, float *acc) {
+  const int lane = threadIdx.x;
+  constexpr int kLaneBytes = T::kShape.kpack * T::kBytes, kRegs = T::kShape.m * T::kShape.n / 64;
+  static_assert(kLaneBytes == 16 * T::kChunks, "a lane's operand registers are whole 16-byte chunks");
+  u32x4 a[T::kChunks], b[T::kChunks];
+#pragma unroll
+  for (int c = 0; c < T::kChunks; ++c) {
+    a[c] = *(const u32x4 *)(lhs + lane * kLaneBytes + 16 * c);
+    b[c] = *(const u32x4 *)(rhs + lane * kLaneBytes + 16 * c);
+  }
+  typename T::Acc d;
+#pragma unroll
+  for (int v = 0; v < kRegs; ++v) d[v] = 0.f;
+  d = EXCHANGED ? T::mfma(b, a, d) : T::mfma(a, b, d);
+#pragma unroll
+  for (int v = 0; v < kRegs; ++v) acc[lane * kRegs + v] = d[v];
+}
+template <typename T>
+int launch_probe(bool exchanged, const void *lhs, const void *rhs, float *acc, hipStream_t s) {
+  if (exchanged) probe_kernel<T, true><<<1, 64, 0, s>>>((const char *)lhs, (const char *)rhs, acc);
+  else probe_kernel<T, false><<<1, 64, 0, s>>>((const char *)lhs, (const char *)rhs, acc);
+  KAPY_HIP_CHECK(hipGetLastError());
+  return KAPY_OK;
+}
+// FIRST / SECOND: the fp8 formats of the instruction's first / second operand slot
+template <template <int, int> class P>
+int launch_probe_f8(int first_fmt, int second_fmt, bool exchanged, const void *lhs, const void *rhs, float *acc, hipStream_t s) {
+  switch (first_fmt * 2 + second_fmt) {
+  case 0: return launch_probe<P<0, 0>>(exchanged, lhs, rhs, acc, s);
+  case 1: return launch_probe<P<0, 1>>(exchanged, lhs, rhs, acc, s);
+  case 2: return launch_probe<P<1, 0>>(exchanged, lhs, rhs, acc, s);
+  default: return launch_probe<P<1, 1>>(exchanged, lhs, rhs, acc, s);
+  }
+}
+
 }  // namespace
 }  // namespace kapy
 
 using namespace kapy;
 
 extern "C" {
+
+int kapy_mfma_probe(int32_t impl_way, int32_t lhs_dtype, int32_t rhs_dtype, int32_t exchanged, const void *lhs_regs, const void *rhs_regs,
+                    float *acc_regs, void *stream) {
+  if (!lhs_regs || !rhs_regs || !acc_regs) return fail(KAPY_ERR_INVALID, "mfma_probe: null register array");
+  const bool f8 = is_f8(lhs_dtype) && is_f8(rhs_dtype), b16 = (lhs_dtype == KAPY_F16 || lhs_dtype == KAPY_BF16) && rhs_dtype == lhs_dtype;
+  const bool way16 = impl_way == KAPY_MFMA_32X32X16_16B || impl_way == KAPY_MFMA_16X16X32_16B;
+  const bool way8 = impl_way == KAPY_MFMA_16X16X128_F8 || impl_way == KAPY_MFMA_32X32X64_F8;
+  if (!way16 && !way8) return fail(KAPY_ERR_INVALID, "mfma_probe: impl_way must name a matrix instruction of gfx950 (16..19), not %d", impl_way);
+  if ((way16 && !b16) || (way8 && !f8)) return fail(KAPY_ERR_VERIFY, "mfma_probe: operand element types do not fit the instruction");
+  int rc = ensure_device();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const bool ex = exchanged != 0;
+  if (way16) {
+    const bool bf = lhs_dtype == KAPY_BF16;
+    if (impl_way == KAPY_MFMA_32X32X16_16B) return bf ? launch_probe<Bf16>(ex, lhs_regs, rhs_regs, acc_regs, s) : launch_probe<F16>(ex, lhs_regs, rhs_regs, acc_regs, s);
+    return bf ? launch_probe<Bf16M16>(ex, lhs_regs, rhs_regs, acc_regs, s) : launch_probe<F16M16>(ex, lhs_regs, rhs_regs, acc_regs, s);
+  }
+  // exchanged: the rhs fragment sits in the first operand slot, so the first format selector is the rhs's
+  const int lf = lhs_dtype == KAPY_F8E5M2, rf = rhs_dtype == KAPY_F8E5M2;
+  const int first = ex ? rf : lf, second = ex ? lf : rf;
+  if (impl_way == KAPY_MFMA_16X16X128_F8) return launch_probe_f8<F8M16>(first, second, ex, lhs_regs, rhs_regs, acc_regs, s);
+  return launch_probe_f8<F8>(first, second, ex, lhs_regs, rhs_regs, acc_regs, s);
+}
+
 
 int kapy_probe_mfma(int32_t impl_way, int32_t dtype, const void *operands, int32_t iterations, float *sink, uint64_t *ticks, int32_t *workgroups,
                     int64_t *flops, void *stream) {
@@ -434,6 +562,25 @@ int kapy_probe_copy(const void *src, void *dst, int64_t bytes, int32_t vectors_p
   case 16: return launch_copy_nt<16>(src, dst, n, nt_load, nt_store, persistent_per_cu, ticks, workgroups, s);
   }
   return fail(KAPY_ERR_INVALID, "probe_copy: vectors per lane must be 1, 2, 4, 8 or 16");
+}
+
+int kapy_probe_read(const void *src, int64_t bytes, int32_t vectors_per_lane, int32_t nt_load, int32_t persistent_per_cu, uint32_t *sink, int32_t *workgroups,
+                    void *stream) {
+  if (!src || bytes <= 0 || bytes % 16 || ((uintptr_t)src & 15)) return fail(KAPY_ERR_INVALID, "probe_read: the buffer must be 16-byte aligned and a whole number of 16-byte vectors long");
+  if (persistent_per_cu < 0 || persistent_per_cu > 64) return fail(KAPY_ERR_INVALID, "probe_read: persistent workgroups per CU must be 0 (one pass) .. 64");
+  int rc = ensure_device();
+  if (rc) return rc;
+  const int64_t n = bytes / 16;
+  if ((n + 255) / 256 > 0x7fffffff) return fail(KAPY_ERR_UNSUPPORTED, "probe_read: buffer too large for one launch");
+  hipStream_t s = (hipStream_t)stream;
+  switch (vectors_per_lane) {
+  case 1: return launch_read<1>(src, n, nt_load, persistent_per_cu, sink, workgroups, s);
+  case 2: return launch_read<2>(src, n, nt_load, persistent_per_cu, sink, workgroups, s);
+  case 4: return launch_read<4>(src, n, nt_load, persistent_per_cu, sink, workgroups, s);
+  case 8: return launch_read<8>(src, n, nt_load, persistent_per_cu, sink, workgroups, s);
+  case 16: return launch_read<16>(src, n, nt_load, persistent_per_cu, sink, workgroups, s);
+  }
+  return fail(KAPY_ERR_INVALID, "probe_read: vectors per lane must be 1, 2, 4, 8 or 16");
 }
 
 }  // extern "C"

@@ -40,8 +40,8 @@ EXPORTS = [
     "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
-    "kapy_mfma_probe", "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
-    "kapy_mk_shared", "kapy_sv_shared", "kapy_shared_address", "kapy_probe_mfma", "kapy_probe_copy", "kapy_probe_copy_tiled", "kapy_probe_l2_read", "kapy_probe_issue", "kapy_probe_copy_runs",
+    "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
+    "kapy_mk_shared", "kapy_sv_shared", "kapy_shared_address",
 ]
 
 
@@ -153,12 +153,6 @@ def lib():
     L.kapy_device_info.argtypes = [P(i32), P(i32), P(i32), C.c_char_p, i32]
     L.kapy_mk_global.argtypes = [P(Global), vp, i32, i32, i32, i32, i32, i32, i32]
     L.kapy_sv_global.argtypes = [P(Global), P(Global), i32, i32, i32, i32]
-    L.kapy_probe_mfma.argtypes = [i32, i32, vp, i32, vp, vp, P(i32), P(i64), vp]
-    L.kapy_probe_copy.argtypes = [vp, vp, i64, i32, i32, i32, i32, vp, P(i32), vp]
-    L.kapy_probe_copy_tiled.argtypes = [vp, vp, i64, i64, i32, vp]
-    L.kapy_probe_l2_read.argtypes = [vp, i64, i32, i32, i32, vp, C.POINTER(C.c_int32), C.POINTER(C.c_int64), vp]
-    L.kapy_probe_copy_runs.argtypes = [vp, vp, i64, i64, i32, vp]
-    L.kapy_probe_issue.argtypes = [i32, i32, i32, vp, i32, vp, C.POINTER(C.c_int32), C.POINTER(C.c_int64), vp]
     L.kapy_mk_shared.argtypes = [P(Shared), i64, i32, i32, i32, i32, i32, i32]
     L.kapy_sv_shared.argtypes = [P(Shared), P(Shared), i32, i32, i32, i32]
     L.kapy_shared_address.restype = i64
@@ -194,7 +188,6 @@ def lib():
     L.kapy_matmul_fused.argtypes = [P(Global), P(Global), P(Global), P(MatmulEpilogue), P(MatmulCfg), vp]
     L.kapy_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global), P(MatmulCfg), vp]
     L.kapy_change.argtypes = [vp, P(Fragments), P(Fragments), A2, vp, vp]
-    L.kapy_mfma_probe.argtypes = [i32, i32, i32, i32, vp, vp, vp, vp]
     L.kapy_reduce.argtypes = [P(Global), P(Global), i32, i32, vp]
     L.kapy_reduce_ex.argtypes = [P(Global), P(Global), i32, P(ReduceCfg), vp]
     L.kapy_reduce_workspace_bytes.restype = C.c_int64
@@ -488,46 +481,3 @@ def matmul_layouts(impl_way, which):
     return f, tuple(mnk)
 
 
-def mfma_probe(impl_way, lhs_dtype, rhs_dtype, exchanged, lhs_ptr, rhs_ptr, acc_ptr, stream=None):
-    check(lib().kapy_mfma_probe(impl_way, lhs_dtype, rhs_dtype, int(exchanged), C.c_void_p(lhs_ptr), C.c_void_p(rhs_ptr), C.c_void_p(acc_ptr),
-                                stream if stream is not None else current_stream()))
-
-
-def probe_mfma(impl_way, dtype, operands_ptr, iterations, sink_ptr, ticks_ptr=None, stream=None):
-    """(workgroups, flops) of one launch of the matrix-instruction loop."""
-    wgs, flops = C.c_int32(0), C.c_int64(0)
-    check(lib().kapy_probe_mfma(impl_way, dtype, C.c_void_p(operands_ptr), iterations, C.c_void_p(sink_ptr), C.c_void_p(ticks_ptr) if ticks_ptr else None,
-                                C.byref(wgs), C.byref(flops), stream if stream is not None else current_stream()))
-    return wgs.value, flops.value
-
-
-def probe_copy(src_ptr, dst_ptr, nbytes, vectors_per_lane=4, nt_load=False, nt_store=False, persistent_per_cu=0, ticks_ptr=None, stream=None):
-    wgs = C.c_int32(0)
-    check(lib().kapy_probe_copy(C.c_void_p(src_ptr), C.c_void_p(dst_ptr), nbytes, vectors_per_lane, int(nt_load), int(nt_store), persistent_per_cu,
-                                C.c_void_p(ticks_ptr) if ticks_ptr else None, C.byref(wgs), stream if stream is not None else current_stream()))
-    return wgs.value
-
-
-def probe_copy_tiled(src_ptr, dst_ptr, rows, row_bytes, through_lds=False, stream=None):
-    check(lib().kapy_probe_copy_tiled(C.c_void_p(src_ptr), C.c_void_p(dst_ptr), rows, row_bytes, int(through_lds),
-                                      stream if stream is not None else current_stream()))
-
-
-def probe_copy_runs(src_ptr, dst_ptr, rows, row_bytes, run_bytes, stream=None):
-    check(lib().kapy_probe_copy_runs(C.c_void_p(src_ptr), C.c_void_p(dst_ptr), rows, row_bytes, run_bytes, stream if stream is not None else current_stream()))
-
-
-def probe_issue(impl_way, filler, count, src_ptr, iterations, sink_ptr, stream=None):
-    """(workgroups, flops) of one launch of the issue probe: matrix instructions with fillers in the gaps between them."""
-    wgs, flops = C.c_int32(0), C.c_int64(0)
-    check(lib().kapy_probe_issue(impl_way, filler, count, C.c_void_p(src_ptr) if src_ptr else None, iterations, C.c_void_p(sink_ptr),
-                                 C.byref(wgs), C.byref(flops), stream if stream is not None else current_stream()))
-    return wgs.value, flops.value
-
-
-def probe_l2_read(src_ptr, window_bytes, iterations, workgroups_per_cu=1, to_lds=True, sink_ptr=None, stream=None):
-    """(workgroups, bytes read) of one launch of the L2 read loop."""
-    wgs, nbytes = C.c_int32(0), C.c_int64(0)
-    check(lib().kapy_probe_l2_read(C.c_void_p(src_ptr), window_bytes, iterations, workgroups_per_cu, int(to_lds), C.c_void_p(sink_ptr) if sink_ptr else None,
-                                   C.byref(wgs), C.byref(nbytes), stream if stream is not None else current_stream()))
-    return wgs.value, nbytes.value

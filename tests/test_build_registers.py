@@ -18,12 +18,13 @@ import pytest
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(os.path.dirname(HERE), "kapy-lang_amd", "lib", "libkapy_hip.so")
+PROBE_LIB = os.path.join(os.path.dirname(HERE), "kapy-lang_amd", "lib", "libkapy_probe.so")
 LLVM = "/opt/rocm/llvm/bin"
 
 
-def _code_objects(tmp_path):
-    fat = str(tmp_path / "fat.bin")
-    subprocess.run([os.path.join(LLVM, "llvm-objcopy"), "--dump-section", ".hip_fatbin=" + fat, LIB, str(tmp_path / "copy.so")], check=True)
+def _code_objects(tmp_path, library=LIB, tag="p"):
+    fat = str(tmp_path / (tag + "fat.bin"))
+    subprocess.run([os.path.join(LLVM, "llvm-objcopy"), "--dump-section", ".hip_fatbin=" + fat, library, str(tmp_path / (tag + "copy.so"))], check=True)
     blob = open(fat, "rb").read()
     magic, pos, out = b"__CLANG_OFFLOAD_BUNDLE__", 0, []
     while True:
@@ -38,7 +39,7 @@ def _code_objects(tmp_path):
             target = blob[p:p + id_len].decode()
             p += id_len
             if "gfx950" in target and size:
-                path = str(tmp_path / ("co_%d.elf" % len(out)))
+                path = str(tmp_path / ("%sco_%d.elf" % (tag, len(out))))
                 open(path, "wb").write(blob[at + offset:at + offset + size])
                 out.append(path)
         pos = at + len(magic)
@@ -49,6 +50,8 @@ def _code_objects(tmp_path):
 def test_no_kernel_spills(tmp_path):
     objects = _code_objects(tmp_path)
     assert objects, "no gfx950 code object found in the library"
+    if os.path.exists(PROBE_LIB):
+        objects += _code_objects(tmp_path, PROBE_LIB, "q")
     seen, bad = 0, []
     for path in objects:
         notes = subprocess.run([os.path.join(LLVM, "llvm-readelf"), "--notes", path], check=True, capture_output=True, text=True).stdout

@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 
 import kapy_hip as kh
+import kapy_probe as kp
 from gpu_util import dev_zeros, sync, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -73,7 +74,7 @@ def test_exported_layouts_describe_the_matrix_instruction(ko, way, lhs_dt, rhs_d
     assert np.array_equal(want, (a_vals @ b_vals).astype(np.float32))
     d_a, d_b = to_dev(_scatter(lhs_l, (m, k), a_bits)), to_dev(_scatter(rhs_l, (k, n), b_bits))
     d_acc = dev_zeros(64 * (m * n // 64), 4)
-    kh.mfma_probe(way, lhs_dt, rhs_dt, exchanged, d_a.data_ptr(), d_b.data_ptr(), d_acc.data_ptr())
+    kp.mfma_probe(way, lhs_dt, rhs_dt, exchanged, d_a.data_ptr(), d_b.data_ptr(), d_acc.data_ptr())
     sync()
     got = _gather(acc_l, (m, n), to_host(d_acc, np.float32, (64, m * n // 64)))
     assert np.array_equal(got, want)
@@ -94,7 +95,7 @@ def test_a_one_hot_element_lands_where_the_layouts_say(ko):
             a[i, kk], b[kk, j] = one, one
             d_a, d_b, d_acc = to_dev(_scatter(lhs_l, (m, k), a)), to_dev(_scatter(rhs_l, (k, n), b)), dev_zeros(m * n, 4)
             for exchanged in (0, 1):
-                kh.mfma_probe(way, dt, dt, exchanged, d_a.data_ptr(), d_b.data_ptr(), d_acc.data_ptr())
+                kp.mfma_probe(way, dt, dt, exchanged, d_a.data_ptr(), d_b.data_ptr(), d_acc.data_ptr())
                 sync()
                 regs = to_host(d_acc, np.float32, (64, m * n // 64))
                 o = kh.A2(0, 0)
@@ -107,8 +108,8 @@ def test_probe_refuses_mismatched_operands():
     d = dev_zeros(64 * 32, 4)
     for way, a, b in ((kh.MFMA_16X16X32_16B, kh.F16, kh.BF16), (kh.MFMA_16X16X32_16B, kh.F8E4M3, kh.F8E4M3), (kh.MFMA_16X16X128_F8, kh.F16, kh.F16)):
         with pytest.raises(kh.KapyError) as e:
-            kh.mfma_probe(way, a, b, 0, d.data_ptr(), d.data_ptr(), d.data_ptr())
+            kp.mfma_probe(way, a, b, 0, d.data_ptr(), d.data_ptr(), d.data_ptr())
         assert e.value.status == kh.ERR_VERIFY
     with pytest.raises(kh.KapyError) as e:
-        kh.mfma_probe(kh.MMA_M16N8K16_F16, kh.F16, kh.F16, 0, d.data_ptr(), d.data_ptr(), d.data_ptr())
+        kp.mfma_probe(kh.MMA_M16N8K16_F16, kh.F16, kh.F16, 0, d.data_ptr(), d.data_ptr(), d.data_ptr())
     assert e.value.status == kh.ERR_INVALID

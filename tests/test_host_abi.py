@@ -14,13 +14,17 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_library_exports_every_declared_symbol():
-    header = open(os.path.join(ROOT, "include", "kapy_hip.h")).read()
-    declared = set(re.findall(r"\b(kapy_[a-z0-9_]+)\s*\(", header))
-    assert declared == set(kh.EXPORTS)
-    L = kh.lib()
-    for name in declared:
-        assert hasattr(L, name), name
-    assert L.kapy_version() >= 100
+    import kapy_probe as kp
+    for header, module in (("kapy_hip.h", kh), ("kapy_probe.h", kp)):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        declared = set(re.findall(r"\b(kapy_[a-z0-9_]+)\s*\(", text))
+        assert declared == set(module.EXPORTS), header
+        L = module.lib()
+        for name in declared:
+            assert hasattr(L, name), name
+    assert kh.lib().kapy_version() >= 100
+    # the measurement kernels are not part of the product library
+    assert not any(hasattr(kh.lib(), name) for name in kp.EXPORTS)
 
 
 def test_struct_layout_matches_header_and_oracle(ko):

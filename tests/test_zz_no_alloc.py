@@ -50,3 +50,33 @@ def test_static_workspace_equals_caller_workspace_on_two_calls_in_a_row(ko):
     with pytest.raises(kh.KapyError) as e:
         kh.matmul(g2, g2, g2, tile=(128, 128, 32), split_k=2, static_workspace=True)
     assert e.value.status == kh.ERR_UNSUPPORTED and "workspace" in e.value.message
+
+
+def test_static_workspace_under_graph_capture_replays_the_eager_bits(ko):
+    """The callers this entry point is for: a first eager call on the device (it asks the runtime where the device's copy of the
+    array lives), then the same call recorded into a graph; every replay, with eager work of another shape in between that dirties
+    the array, gives the eager call's bits."""
+    M, N, K, dt = 512, 384, 4096, kh.BF16
+    a, b = ko.fill_uniform(M * K, dt, 21, 0), ko.fill_uniform(K * N, dt, 21, 1)
+    da, db = to_dev(a), to_dev(b)
+    ga, gb = dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt)
+    eager, out = dev_zeros(M * N, 2), dev_zeros(M * N, 2)
+    kh.matmul(ga, gb, dglobal(eager, M, N, N, 1, dt), tile=(128, 128, 64), split_k=8, static_workspace=True)
+    sync()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            kh.matmul(ga, gb, dglobal(out, M, N, N, 1, dt), tile=(128, 128, 64), split_k=8, static_workspace=True, stream=side.cuda_stream)
+    other = dev_zeros(256 * 256, 2)
+    g_small = dglobal(to_dev(ko.fill_uniform(256 * 2048, kh.F16, 5, 0)), 256, 2048, 2048, 1, kh.F16)
+    g_small_b = dglobal(to_dev(ko.fill_uniform(2048 * 256, kh.F16, 5, 1)), 2048, 256, 256, 1, kh.F16)
+    for rep in range(3):
+        out.fill_(0x7E7E)
+        sync()
+        graph.replay()
+        sync()
+        assert torch.equal(out, eager), rep
+        kh.matmul(g_small, g_small_b, dglobal(other, 256, 256, 256, 1, kh.F16), tile=(128, 128, 64), split_k=4, static_workspace=True)
+        sync()

@@ -306,7 +306,17 @@ typedef struct kapy_matmul_cfg {
                                     16 KiB (the counters) must be zero before its first use and every call leaves them zero;
                                     calls that share a workspace must not overlap in time */
   int64_t workspace_bytes;       /* kapy_matmul_workspace_bytes(m, n) is enough for any split of an [m x n] result */
+  int32_t accumulate;            /* kapy_matmul_accumulate; 0 = fp32 accumulators, one cast at the end */
+  int32_t reserved;              /* 0 */
 } kapy_matmul_cfg;
+/* What the running sum of a matmul is held in.  The reference's instruction for f16 operands and an f16 result carries f16
+ * accumulators (MatmulOpToLLVM.cpp:270-291, mma.sync ... .f16.f16.f16.f16), so its K loop (MatmulOpToLLVM.cpp:207-262) rounds
+ * the sum to f16 once per instruction: every 16 columns of the lhs for mma_m16n8k16_f16, every 8 for mma_m16n8k8_f16.
+ * KAPY_ACCUMULATE_ELEMENT reproduces that (f16 operands, accumulator and result only; cfg->impl_way =
+ * KAPY_MMA_M16N8K8_F16 selects the 8-column cadence, anything else 16; tile, stage, wave and split fields are ignored; a
+ * small kernel for checking programs against the reference's numbers, not a fast path).  KAPY_ACCUMULATE_F32, the
+ * default, is more accurate and what every tuned kernel does. */
+typedef enum kapy_matmul_accumulate { KAPY_ACCUMULATE_F32 = 0, KAPY_ACCUMULATE_ELEMENT = 1 } kapy_matmul_accumulate;
 /* Workspace size that lets the library split K for an [m x n] result whichever way it chooses. */
 int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n);
 

@@ -1192,6 +1192,11 @@ struct Interp {
       const std::string &way = op.words.empty() ? std::string() : op.words[0];
       cfg.impl_way = way == "mma_m16n8k8_f16" ? KAPY_MMA_M16N8K8_F16 : way == "mma_m16n8k16_f16" ? KAPY_MMA_M16N8K16_F16 :
                      way == "mma_m16n8k16_f8" ? KAPY_MMA_M16N8K16_F8 : way == "mma_m16n8k8_tf32" ? KAPY_MMA_M16N8K8_TF32 : KAPY_MATMUL_AUTO;
+      // KAPY_MLIR_MATMUL=reference: f16 x f16 -> f16 products keep f16 accumulators, rounded once per instruction of the named
+      // way, as the reference's .f16.f16.f16.f16 instruction does (MatmulOpToLLVM.cpp:270-291); other types have fp32 accumulators there too
+      const char *matmul_mode = getenv("KAPY_MLIR_MATMUL");
+      if (matmul_mode && std::string(matmul_mode) == "reference" && a.g.dtype == KAPY_F16 && b.g.dtype == KAPY_F16 && c.g.dtype == KAPY_F16 && r.g.dtype == KAPY_F16)
+        cfg.accumulate = KAPY_ACCUMULATE_ELEMENT;
       int rc = lib(op, kapy_matmul(&a.g, &b.g, &c.g, &r.g, &cfg, stream));
       if (rc) return rc;
       env[op.results[0]] = r;

@@ -1817,9 +1817,15 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
   if (c.rmode != KAPY_RN && c.rmode != KAPY_RZ) return fail(KAPY_ERR_INVALID, "matmul: unknown rounding mode %d", c.rmode);
   if (result->dtype != KAPY_F16 && result->dtype != KAPY_BF16 && result->dtype != KAPY_F32)
     return fail(KAPY_ERR_VERIFY, "matmul: result must have f16, bf16 or f32 element type");
+  if (c.accumulate != KAPY_ACCUMULATE_F32 && c.accumulate != KAPY_ACCUMULATE_ELEMENT) return fail(KAPY_ERR_INVALID, "matmul: unknown accumulate mode %d", c.accumulate);
   rc = ensure_device();
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
+  if (c.accumulate == KAPY_ACCUMULATE_ELEMENT) {
+    if (epi) return fail(KAPY_ERR_UNSUPPORTED, "matmul_fused: the fused tail exists with fp32 accumulators only");
+    if (c.rmode != KAPY_RN) return fail(KAPY_ERR_UNSUPPORTED, "matmul: f16 accumulators round to nearest even, as the instruction they restate");
+    return run_matmul_f16acc(lhs, rhs, acc, result, c.impl_way == KAPY_MMA_M16N8K8_F16 ? 8 : 16, s);
+  }
   if (is_f8(lhs->dtype)) {
     if (epi) return fail(KAPY_ERR_UNSUPPORTED, "matmul_fused: fp8 operands take kapy_matmul_scaled_f8");
     return matmul_f8(lhs, rhs, nullptr, nullptr, acc, result, &c, s);

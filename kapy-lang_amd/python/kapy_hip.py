@@ -101,7 +101,10 @@ class EwInst(C.Structure):
 class MatmulCfg(C.Structure):
     _fields_ = [("impl_way", C.c_int32), ("tile_m", C.c_int32), ("tile_n", C.c_int32), ("tile_k", C.c_int32),
                 ("rmode", C.c_int32), ("stages", C.c_int32), ("waves", C.c_int32), ("split_k", C.c_int32),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64)]
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64), ("accumulate", C.c_int32), ("reserved", C.c_int32)]
+
+
+ACCUMULATE_F32, ACCUMULATE_ELEMENT = 0, 1
 
 
 class ReduceCfg(C.Structure):
@@ -400,11 +403,12 @@ def _workspace(workspace):
 
 
 def matmul(lhs, rhs, result, acc=None, impl_way=MATMUL_AUTO, tile=(0, 0, 0), rmode=RN, stages=0, waves=0, split_k=0, workspace=None,
-           static_workspace=False, stream=None):
+           static_workspace=False, accumulate=ACCUMULATE_F32, stream=None):
     """workspace: zero-initialised device memory (a torch tensor or a (pointer, bytes) pair) that lets the library split K;
-    static_workspace: call kapy_matmul_static_workspace instead (the library's own array)."""
+    static_workspace: call kapy_matmul_static_workspace instead (the library's own array); accumulate: ACCUMULATE_ELEMENT keeps
+    f16 accumulators rounded once per instruction of impl_way, the reference's arithmetic for f16 results."""
     ws, ws_bytes = _workspace(workspace)
-    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, split_k, ws, ws_bytes)
+    cfg = MatmulCfg(impl_way, tile[0], tile[1], tile[2], rmode, stages, waves, split_k, ws, ws_bytes, accumulate, 0)
     fn = lib().kapy_matmul_static_workspace if static_workspace else lib().kapy_matmul
     check(fn(C.byref(lhs), C.byref(rhs), C.byref(acc) if acc is not None else None, C.byref(result),
              C.byref(cfg), stream if stream is not None else current_stream()))

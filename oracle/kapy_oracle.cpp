@@ -1011,6 +1011,39 @@ int ko_matmul(const ko_global *lhs, const ko_global *rhs, const ko_global *acc, 
   return 0;
 }
 
+// kapy.matmul in the reference's own arithmetic when the result has f16 element type: the instruction it emits for f16
+// operands then carries f16 accumulators (MatmulOpToLLVM.cpp:270-291: mma.sync ... .f16.f16.f16.f16), one instruction per
+// k_step columns of the lhs (8: mma_m16n8k8_f16, 16: mma_m16n8k16_f16; the loop over K of MatmulOpToLLVM.cpp:207-262 feeds
+// each instruction's result to the next as its accumulator).  Restated: the accumulator is an f16 value; every step adds the
+// exact sum of the step's k_step products to it and rounds once to f16 (nearest even).  What the instruction does INSIDE a
+// step is not published for either vendor's matrix unit; "exact sum, one rounding" is the model, and a device whose unit adds
+// in fp32 can differ from it by one f16 unit in the last place where the exact sum sits within fp32 round-off of a tie.
+int ko_matmul_f16acc(const ko_global *lhs, const ko_global *rhs, const ko_global *acc, const ko_global *result, int k_step) {
+  int rc = matmul_verify(lhs, rhs, acc, result);
+  if (rc) return rc;
+  if (lhs->dtype != KO_F16 || rhs->dtype != KO_F16 || result->dtype != KO_F16 || (acc && acc->dtype != KO_F16)) return -7;
+  if (k_step != 8 && k_step != 16) return -8;
+  int64_t M = extent0(lhs), K = extent1(lhs), N = extent1(rhs);
+  std::vector<double> A((size_t)M * K), Bt((size_t)N * K);
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t k = 0; k < K; ++k) A[i * K + k] = ko_decode(lhs->ptr, lhs->dtype, elem_offset(lhs, i, k));
+  for (int64_t j = 0; j < N; ++j)
+    for (int64_t k = 0; k < K; ++k) Bt[j * K + k] = ko_decode(rhs->ptr, rhs->dtype, elem_offset(rhs, k, j));
+#pragma omp parallel for schedule(dynamic, 4)
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t j = 0; j < N; ++j) {
+      uint16_t held = 0;  // the accumulator register: f16 bits
+      if (acc) ko_encode(&held, KO_F16, 0, ko_decode(acc->ptr, acc->dtype, elem_offset(acc, i, j)), KO_RN);
+      for (int64_t k0 = 0; k0 < K; k0 += k_step) {
+        long double s = (long double)ko_decode(&held, KO_F16, 0);
+        for (int64_t k = k0; k < std::min<int64_t>(K, k0 + k_step); ++k) s += (long double)(A[i * K + k] * Bt[j * K + k]);  // (a product of two f16 values is exact in double)
+        ko_encode(&held, KO_F16, 0, (double)s, KO_RN);
+      }
+      ko_encode(result->ptr, result->dtype, elem_offset(result, i, j), ko_decode(&held, KO_F16, 0), KO_RN);
+    }
+  return 0;
+}
+
 // W8A8: result[m,n] = RN_bf16( (sum_k a8[m,k]·w8[k,n]) · row_scale[m] · col_scale[n] ), fp64 sum.
 // The scale product is formed in fp32 (row_scale*col_scale) as the kapy chain
 // broadcast(row) * broadcast(col) on f32 tensors would.

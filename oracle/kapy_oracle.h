@@ -109,6 +109,9 @@ int ko_copy_batched(const ko_global *src, const ko_global *dst, int transpose, i
 /* ---- compute ops ---- */
 int ko_elementwise(const ko_ew_inst *prog, int n_inst, const ko_global *const *ins, int n_ins, const ko_global *out);
 int ko_matmul(const ko_global *lhs, const ko_global *rhs, const ko_global *acc, const ko_global *result, int rmode);
+/* The same product with f16 accumulators rounded once per k_step (8 or 16) columns of the lhs: the arithmetic of the
+ * reference's f16-result instruction strings (MatmulOpToLLVM.cpp:270-291).  f16 operands, accumulator and result only. */
+int ko_matmul_f16acc(const ko_global *lhs, const ko_global *rhs, const ko_global *acc, const ko_global *result, int k_step);
 int ko_matmul_scaled_f8(const ko_global *a, const ko_global *w, const float *row_scale, const float *col_scale,
                         const ko_global *result);
 void ko_quantize_e4m3(const float *x, int64_t rows, int64_t cols, int64_t row_stride, int64_t col_stride,

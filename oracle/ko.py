@@ -116,6 +116,8 @@ def lib():
         L.ko_elementwise.argtypes = [P(EwInst), C.c_int, P(P(Global)), C.c_int, P(Global)]
         L.ko_matmul.restype = C.c_int
         L.ko_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), C.c_int]
+        L.ko_matmul_f16acc.restype = C.c_int
+        L.ko_matmul_f16acc.argtypes = [P(Global), P(Global), P(Global), P(Global), C.c_int]
         L.ko_matmul_scaled_f8.restype = C.c_int
         L.ko_matmul_scaled_f8.argtypes = [P(Global), P(Global), vp, vp, P(Global)]
         L.ko_quantize_e4m3.restype = None

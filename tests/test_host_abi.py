@@ -31,7 +31,7 @@ def test_struct_layout_matches_header_and_oracle(ko):
     assert C.sizeof(kh.Global) == C.sizeof(ko.Global) == 40
     assert C.sizeof(kh.Fragments) == C.sizeof(ko.Fragments) == 24
     assert C.sizeof(kh.EwInst) == C.sizeof(ko.EwInst) == 32
-    assert C.sizeof(kh.MatmulCfg) == 48 and C.sizeof(kh.Grid2) == 40 and C.sizeof(kh.CopyCfg) == 24 and C.sizeof(kh.Shared) == 48
+    assert C.sizeof(kh.MatmulCfg) == 56 and C.sizeof(kh.Grid2) == 40 and C.sizeof(kh.CopyCfg) == 24 and C.sizeof(kh.Shared) == 48
 
 
 def test_descriptors_match_oracle(ko):

@@ -190,6 +190,7 @@ int kapy_mk_shared(kapy_shared *out, int64_t byte_offset, int32_t size0, int32_t
   out->layout.stride1 = row_major ? 1 : size0;
   out->layout.bank_param = bank_param;
   out->layout.line_param = line_param;
+  out->layout.rotate = 0;
   return KAPY_OK;
 }
 
@@ -212,7 +213,7 @@ int64_t kapy_shared_address(const kapy_shared *tensor, int64_t i0, int64_t i1) {
   // in bounds iff (start + i) <u end on both axes, the unsigned compare of the loads and stores
   const uint32_t a0 = (uint32_t)(tensor->start0 + i0), a1 = (uint32_t)(tensor->start1 + i1);
   if (a0 >= (uint32_t)tensor->end0 || a1 >= (uint32_t)tensor->end1) return KAPY_ERR_VERIFY;
-  const Swizzle sw{tensor->layout.stride0, tensor->layout.stride1, tensor->layout.bank_param, tensor->layout.line_param};
+  const Swizzle sw{tensor->layout.stride0, tensor->layout.stride1, tensor->layout.bank_param, tensor->layout.line_param, tensor->layout.rotate};
   return tensor->offset + sw.offset(b * 8, a0, a1) * b;
 }
 
@@ -346,7 +347,8 @@ int64_t kapy_change_num_shuffles(const kapy_fragments *src, const kapy_fragments
 int64_t kapy_swizzle_offset(const kapy_swizzling *layout, int64_t bits, int64_t i0, int64_t i1) {
   if (!layout || layout->bank_param <= 0 || layout->line_param <= 0 || bits <= 0)
     return fail(KAPY_ERR_INVALID, "swizzle_offset: bad layout");
-  return Swizzle{layout->stride0, layout->stride1, layout->bank_param, layout->line_param}.offset(bits, i0, i1);
+  if (layout->rotate < 0) return fail(KAPY_ERR_INVALID, "swizzle_offset: bad layout");
+  return Swizzle{layout->stride0, layout->stride1, layout->bank_param, layout->line_param, layout->rotate}.offset(bits, i0, i1);
 }
 
 int kapy_swizzle_search(const kapy_fragments *access, const int64_t shape[2], int64_t stride0, int64_t stride1, int64_t bits,
@@ -358,6 +360,18 @@ int kapy_swizzle_search(const kapy_fragments *access, const int64_t shape[2], in
   if (stride0 != 1 && stride1 != 1) return fail(KAPY_ERR_VERIFY, "swizzle search: can not find a contiguous axis");
   return swizzle_search(to_internal(access), {shape[0], shape[1]}, (int32_t)stride0, (int32_t)stride1, bits, alignment, pairs,
                         max_pairs);
+}
+
+int kapy_swizzle_search_gfx950(const kapy_fragments *access, const int64_t shape[2], int64_t stride0, int64_t stride1, int64_t bits,
+                               int64_t alignment, int32_t *triples, int32_t max_triples) {
+  int rc = check_fragments(access, "swizzle search access layout");
+  if (rc) return rc;
+  if (!shape || (max_triples > 0 && !triples)) return fail(KAPY_ERR_INVALID, "swizzle search: null argument");
+  if (stride0 != 1 && stride1 != 1) return fail(KAPY_ERR_VERIFY, "swizzle search: can not find a contiguous axis");
+  if (access->lane_array[0] * access->lane_array[1] != kWaveSize)
+    return fail(KAPY_ERR_VERIFY, "swizzle search: the read phases of gfx950 are phases of a 64-lane wavefront; the access layout has %d lanes",
+                access->lane_array[0] * access->lane_array[1]);
+  return swizzle_search_gfx950(to_internal(access), {shape[0], shape[1]}, (int32_t)stride0, (int32_t)stride1, bits, alignment, triples, max_triples);
 }
 
 int kapy_matmul_layouts(int32_t impl_way, int32_t which, kapy_fragments *out, int32_t mnk[3]) {

@@ -43,28 +43,24 @@ namespace kapy {
 namespace {
 
 // LDS image of an operand tile: [rows][ROWBYTES] bytes, K contiguous, 16-byte chunks XOR-ed with the
-// line index.  The parameters come from the compile-time search (the reference's getSwizzlingLayouts
-// for 64 banks) run on the access layout of the operand reads of the matrix instruction the kernel is
-// built for: the lhs fragments of T::kShape counted in bytes (T::kShape.m lanes down the rows, the K-groups
+// line index.  The parameters come from the compile-time search (the reference's getSwizzlingLayouts for 64 banks,
+// asked of the gfx950 read phases: layout.hpp) run on the access layout of the operand reads of the matrix instruction
+// the kernel is built for: the lhs fragments of T::kShape counted in bytes (T::kShape.m lanes down the rows, the K-groups
 // across, 16 contiguous bytes per lane and read instruction).
-template <int ROWBYTES, typename T>
+// BLOCK_ROWS: a kernel that computes the key once for all blocks of BLOCK_ROWS rows needs a swizzle period that divides such a
+// block; where the hardware search's first hit does not, the layout falls back to the reference model's first hit.
+template <int ROWBYTES, typename T, int BLOCK_ROWS = 0>
 struct TileLayout {
   static constexpr int kRowBytes = ROWBYTES;
   static constexpr MfmaShape kS = T::kShape;
   static constexpr Fragments kAccess{mfma_lhs(kS).a0, mfma_lhs(kS).a1, 1, mfma_lhs(kS).l1 * T::kBytes, mfma_lhs(kS).major};
-  static constexpr Swizzle kSwizzle = first_swizzle(kAccess, {kS.m, kS.k * T::kBytes}, ROWBYTES, 1, 8, 1024);
+  static constexpr Swizzle kSwizzleHw = first_swizzle_gfx950(kAccess, {kS.m, kS.k * T::kBytes}, ROWBYTES, 1, 8, 1024);
+  static constexpr bool kPeriodFits = BLOCK_ROWS == 0 || (BLOCK_ROWS * ROWBYTES) % (256 * kSwizzleHw.line_param) == 0;
+  static constexpr Swizzle kSwizzle = kPeriodFits ? kSwizzleHw : first_swizzle(kAccess, {kS.m, kS.k * T::kBytes}, ROWBYTES, 1, 8, 1024);
   static_assert(kSwizzle.bank_param == 4, "MFMA operand reads are 16-byte: the search must return 16-byte atoms");
   static constexpr int kLineParam = kSwizzle.line_param;
-  // The 16x16x128 operand reads (a lane: row lane % 16, the two 16-byte chunks 2 * (lane / 16) and + 1 of a 128-byte row)
-  // pass the search's model - which looks at the 16 lanes of one phase - with (4, 8), but the LDS serves them at two thirds
-  // of its rate (SQ_LDS_BANK_CONFLICT on half of its active cycles).  Measured conflict-free: the same XOR of the chunk
-  // index with three bits of the line index, taken in rotated order (line bits 0, 1, 2 -> chunk bits 1, 2, 0).
-  static constexpr bool kRotatedKey = kS.m == 16 && kS.kpack * T::kBytes == 32 && ROWBYTES == 128;
-  static_assert(!kRotatedKey || kLineParam == 8, "the rotated key replaces the (4, 8) swizzle");
-  static __device__ __forceinline__ uint32_t key_of(uint32_t o) {
-    const uint32_t line = (o >> 8) & (kLineParam - 1);
-    return kRotatedKey ? (((line & 3) << 1) | (line >> 2)) : line;
-  }
+  // the chunk index is XOR-ed with the line index taken modulo kLineParam and rotated as the search found it
+  static __device__ __forceinline__ uint32_t key_of(uint32_t o) { return (uint32_t)kSwizzle.key((o >> 8) & (kLineParam - 1)); }
   // byte offset of 16-byte chunk `chunk` of row `row`
   static __device__ __forceinline__ uint32_t offset(uint32_t row, uint32_t chunk) {
     uint32_t o = row * kRowBytes + chunk * 16;
@@ -1191,7 +1187,7 @@ template <typename T, int BK, int STAGES, bool PACKED, bool A_TR = false, bool B
 __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   static_assert(T::kM == 16 && T::kBytes == 2 && BK % 32 == 0 && STAGES >= 3, "16x16x32 instruction, 16-bit operands");
   static_assert(A_TR || B_TR, "two K-contiguous operands are the tiled kernel's");
-  using LA = TileLayout<BK * 2, T>;
+  using LA = TileLayout<BK * 2, T, 16>;
   constexpr int kRowKc = BK * 2, kRowTr = 128 * 2;   // bytes per staged row: a row / column of BK elements, or a k-row of 128
   constexpr int kBytesOp = 128 * BK * 2, kBytesA = kBytesOp, kStage = 2 * kBytesOp;
   constexpr int kLoadsOp = kBytesOp / 1024 / 4, kLoads = 2 * kLoadsOp;  // per wavefront per tile
@@ -2010,8 +2006,8 @@ int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling
     return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: only f16 / bf16 operand tiles are described here");
   Swizzle s;
   switch (tile_k) {
-  case 32: s = TileLayout<64, Bf16M16>::kSwizzle; break;   // (f16 and bf16 share the operand layouts; the search gives the
-  case 64: s = TileLayout<128, Bf16M16>::kSwizzle; break;  //  same parameters for the 32x32x16 instruction)
+  case 32: s = TileLayout<64, Bf16>::kSwizzle; break;      // (f16 and bf16 share the operand layouts; the 32-deep tiles are built
+  case 64: s = TileLayout<128, Bf16M16>::kSwizzle; break;  //  on the 32x32x16 instruction, the 64-deep ones on 16x16x32)
   default: return fail(KAPY_ERR_UNSUPPORTED, "matmul_lds_layout: tile_k must be 32 or 64");
   }
   s.stride0 = tile_k;  // the search runs on bytes; report the row stride in elements
@@ -2019,6 +2015,7 @@ int kapy_matmul_lds_layout(int32_t operand_dtype, int32_t tile_k, kapy_swizzling
   out->stride1 = s.stride1;
   out->bank_param = s.bank_param;
   out->line_param = s.line_param;
+  out->rotate = s.rotate;
   return KAPY_OK;
 }
 

@@ -35,7 +35,7 @@ EXPORTS = [
     "kapy_version", "kapy_last_error", "kapy_device_info", "kapy_mk_global", "kapy_sv_global",
     "kapy_fragments_loops", "kapy_fragments_map", "kapy_fragments_transpose", "kapy_fragments_exchange_axes",
     "kapy_fragments_default", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
-    "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
+    "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_swizzle_search_gfx950", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
     "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
@@ -75,7 +75,7 @@ class Fragments(C.Structure):
 
 
 class Swizzling(C.Structure):
-    _fields_ = [("stride0", C.c_int32), ("stride1", C.c_int32), ("bank_param", C.c_int32), ("line_param", C.c_int32)]
+    _fields_ = [("stride0", C.c_int32), ("stride1", C.c_int32), ("bank_param", C.c_int32), ("line_param", C.c_int32), ("rotate", C.c_int32)]
 
 
 class CopyCfg(C.Structure):
@@ -175,6 +175,7 @@ def lib():
     L.kapy_swizzle_offset.restype = i64
     L.kapy_swizzle_offset.argtypes = [P(Swizzling), i64, i64, i64]
     L.kapy_swizzle_search.argtypes = [P(Fragments), A2, i64, i64, i64, i64, P(i32), i32]
+    L.kapy_swizzle_search_gfx950.argtypes = [P(Fragments), A2, i64, i64, i64, i64, P(i32), i32]
     L.kapy_matmul_layouts.argtypes = [i32, i32, P(Fragments), P(i32)]
     L.kapy_matmul_lds_layout.argtypes = [i32, i32, P(Swizzling)]
     L.kapy_copy.argtypes = [P(Global), P(Global), P(CopyCfg), vp]

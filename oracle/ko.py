@@ -101,6 +101,11 @@ def lib():
         L.ko_no_bank_conflict.argtypes = [P(Fragments), A2] + [i64] * 8
         L.ko_swizzle_search.restype = C.c_int
         L.ko_swizzle_search.argtypes = [P(Fragments), A2, i64, i64, i64, i64, i64, i64, P(i64), C.c_int]
+        L.ko_no_bank_conflict_gfx950.restype = C.c_int
+        L.ko_no_bank_conflict_gfx950.argtypes = [P(Fragments), A2] + [i64] * 7
+        L.ko_swizzle_search_gfx950.restype = C.c_int
+        L.ko_swizzle_search_gfx950.argtypes = [P(Fragments), A2, i64, i64, i64, i64, P(i64), C.c_int]
+        L.ko_swizzle_offset_rotated.restype = i64; L.ko_swizzle_offset_rotated.argtypes = [i64] * 8
         L.ko_mk_global.restype = C.c_int
         L.ko_mk_global.argtypes = [P(Global), vp, i32, i32, i32, i32, i32, C.c_int, i32]
         L.ko_sv_global.restype = C.c_int; L.ko_sv_global.argtypes = [P(Global), P(Global), i32, i32, i32, i32]

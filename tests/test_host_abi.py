@@ -168,10 +168,8 @@ def test_swizzle_agrees_with_oracle_and_matmul_layout_is_searched(ko):
             for i0 in range(0, 64, 3):
                 for i1 in range(0, s0, 5):
                     assert L.kapy_swizzle_offset(C.byref(sw), bits, i0, i1) == O.ko_swizzle_offset(i0, i1, s0, 1, bits, bp, lp, 64)
-    # the LDS layout the matmul uses must be the first hit of the reference's search run on the operand layout of the matrix
-    # instruction its kernels are built on (16x16x32 by default; 32x32x16 gives the same parameters)
+    # the reference's search, re-parameterised for 64 banks and lanes, agrees with the checker's restatement of it
     for tile_k in (32, 64):
-        found = []
         for way, want_mnk in ((kh.MFMA_16X16X32_16B, [16, 16, 32]), (kh.MFMA_32X32X16_16B, [32, 32, 16])):
             f, mnk = kh.Fragments(), (C.c_int32 * 3)()
             assert L.kapy_matmul_layouts(way, 0, C.byref(f), mnk) == 0 and list(mnk) == want_mnk
@@ -183,10 +181,22 @@ def test_swizzle_agrees_with_oracle_and_matmul_layout_is_searched(ko):
             assert n == O.ko_swizzle_search(C.byref(g), shape, tile_k, 1, 16, 1024, 64, 64, op, 32) and n > 0
             assert [pairs[i] for i in range(2 * n)] == [op[i] for i in range(2 * n)]
             assert pairs[0] == 4 and (pairs[0], 1) not in {(pairs[2 * i], pairs[2 * i + 1]) for i in range(n)}  # unswizzled conflicts
-            found.append((pairs[0], pairs[1]))
-        sw = kh.Swizzling()
-        assert L.kapy_matmul_lds_layout(kh.BF16, tile_k, C.byref(sw)) == 0
-        assert (sw.stride0, sw.stride1, sw.bank_param, sw.line_param) == (tile_k, 1) + found[0] and found[0] == found[1]
+            # ... and so does the search over the gfx950 read phases (triples with the key's rotation)
+            triples, ot = (C.c_int32 * 300)(), (C.c_int64 * 300)()
+            n = L.kapy_swizzle_search_gfx950(C.byref(f), shape, tile_k, 1, 16, 1024, triples, 100)
+            assert n == O.ko_swizzle_search_gfx950(C.byref(g), shape, tile_k, 1, 16, 1024, ot, 100) and n > 0
+            assert [triples[i] for i in range(3 * n)] == [ot[i] for i in range(3 * n)]
+            if (way == kh.MFMA_16X16X32_16B) == (tile_k == 64):
+                # the LDS layout the matmul uses is that search's first hit for the instruction its kernels of that depth are
+                # built on (32-deep tiles: 32x32x16; 64-deep tiles: 16x16x32)
+                sw = kh.Swizzling()
+                assert L.kapy_matmul_lds_layout(kh.BF16, tile_k, C.byref(sw)) == 0
+                assert (sw.stride0, sw.stride1, sw.bank_param, sw.line_param, sw.rotate) == (tile_k, 1) + tuple(triples[:3])
+    # rotated keys through the offset function
+    for lp, rot in ((8, 1), (16, 3)):
+        sw = kh.Swizzling(128, 1, 4, lp, rot)
+        assert all(L.kapy_swizzle_offset(C.byref(sw), 8, i0, i1) == O.ko_swizzle_offset_rotated(i0, i1, 128, 1, 8, 4, lp, rot)
+                   for i0 in range(0, 40, 3) for i1 in range(0, 128, 5))
 
 
 def test_mfma_layouts_are_consistent_fragments(ko):

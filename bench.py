@@ -903,6 +903,101 @@ WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce",
              "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
 
 
+# ---------------------------------------------------------------- HBM traffic summary from the profiler's counter files
+# Which kernels' dispatches are one launch of which workload: (workload key, label, [(kernel-name pattern, grid size or None)]);
+# the bytes of the listed kernels add up (a workload of two kernels launches each once per step).
+TRAFFIC_KERNELS = [
+    ("gelu", "C2 gelu fp16 8192^2", [(r"affine_act_cols_kernel<.*(GELU|1\)|, 1[,>])", None)]),
+    ("add", "x + y fp16 8192^2", [(r"affine_act_kernel<", None)]),
+    ("expr", "x*y + x fp16 8192^2 (compiled from its second call)", [(r"kapy_ew_flat_", 32768 * 256)]),
+    ("copy", "copy 2 x 128 MiB", [(r"rows_kernel<", None)]),
+    ("permute", "C3b permute", [(r"rows_kernel<", None)]),
+    ("transpose", "C3a transpose fp16 8192^2", [(r"transpose_lds_kernel<", None)]),
+    ("reduce", "row sums fp16 8192^2", [(r"reduce_rows_vec_kernel<", None)]),
+    ("reduce_cols", "column sums fp16 8192^2", [(r"reduce_cols_strip_kernel<", None)]),
+    ("softmax_cols", "column softmax fp16 8192^2", [(r"col_softmax_stats_kernel<", None), (r"col_softmax_apply_kernel<", None)]),
+    ("softmax", "row softmax fp16 8192^2", [(r"softmax_kernel<", None)]),
+    ("layernorm", "layer norm fp16 8192^2", [(r"norm_kernel<", None)]),
+    ("gemm_bf16", "C4 gemm bf16 8192^3", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, false>\(", None)]),
+    ("gemm_bf16_gelu", "C4 gemm bf16 8192^3 + gelu", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, true>\(", None)]),
+    ("f8_m4096", "C5 W8A8 M=4096", [(r"tn_kernel<kapy::F8M16<0, 0>, 256, 256, 128", None)]),
+    ("f8_m16", "C5 W8A8 M=16", [(r"skinny_stream_kernel<", None)]),
+    ("gemm_f16", "C1 gemm fp16 1024^3", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),
+]
+
+
+def pmc_summary(fetch_csv, write_csv):
+    """The tracked HBM-traffic summary from two rocprofv3 counter files (FETCH_SIZE and WRITE_SIZE, KiB per dispatch): per kernel and
+    grid the mean of each counter, the factor that makes the plain copy's counters read its known 128 MiB each way, and one line
+    `traffic_bytes <workload> <bytes>` per workload of TRAFFIC_KERNELS, which is what the benchmark reports as `traffic`."""
+    import collections
+    import csv
+    import re
+    import subprocess
+
+    def means(path, counter):
+        acc = collections.defaultdict(lambda: [0.0, 0])
+        for row in csv.DictReader(open(path)):
+            if row["Counter_Name"] != counter:
+                continue
+            e = acc[(row["Kernel_Name"], int(row["Grid_Size"]))]
+            e[0] += float(row["Counter_Value"])
+            e[1] += 1
+        return {k: (v[0] / v[1], v[1]) for k, v in acc.items()}
+
+    fetch, write = means(fetch_csv, "FETCH_SIZE"), means(write_csv, "WRITE_SIZE")
+    ours = sorted(k for k in set(fetch) | set(write) if "kapy" in k[0])
+    names = {}
+    try:
+        demangled = subprocess.run(["c++filt"], input="\n".join(k[0] for k in ours), capture_output=True, text=True).stdout.split("\n")
+        names = {k: d.replace("void ", "").replace("kapy::(anonymous namespace)::", "") for k, d in zip(ours, demangled)}
+    except OSError:
+        names = {k: k[0] for k in ours}
+
+    def pick(pattern, grid):
+        hits = [k for k in ours if re.search(pattern, names[k]) and (grid is None or k[1] == grid)]
+        if not hits:
+            return None
+        best = max(hits, key=lambda k: fetch.get(k, (0, 0))[1])       # the form launched most often is the timed one
+        return best
+
+    out = ["rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, all bench workloads, one MI355X (gfx950)", "",
+           "commands (two runs, one counter each; from the repository root after `cd /tmp && export TMPDIR=/tmp && cd <repo>`):",
+           "  rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof/pmc_fetch -o pmc_fetch --output-format csv -- python3 bench.py --no-cpu --skip ceilings --steps 3 --warmup 1",
+           "  rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof/pmc_write -o pmc_write --output-format csv -- python3 bench.py --no-cpu --skip ceilings --steps 3 --warmup 1",
+           "  python3 bench.py --pmc-summary <pmc_fetch counter_collection.csv> <pmc_write counter_collection.csv> > profiles/bench_all_workloads.hbm_traffic_pmc.txt",
+           "", "Per-dispatch mean of the counter (rocprofv3 reports KiB), by kernel and grid size (work-items); n = dispatches seen.", "",
+           "%-86s %10s %20s %20s" % ("kernel", "grid", "FETCH_SIZE (n)", "WRITE_SIZE (n)")]
+    for k in ours:
+        f, w = fetch.get(k, (0.0, 0)), write.get(k, (0.0, 0))
+        out.append("%-86s %10d %12.1f (%5d) %12.1f (%5d)" % (names[k][:86], k[1], f[0], f[1], w[0], w[1]))
+    copy = pick(*TRAFFIC_KERNELS[3][2][0])
+    if copy is None or copy not in fetch or copy not in write:
+        raise SystemExit("bench.py --pmc-summary: the copy kernel (rows_kernel) is in neither counter file; nothing to calibrate against")
+    known_kib = 128 * 1024
+    ff, wf = known_kib / fetch[copy][0], known_kib / write[copy][0]
+    out += ["", "Calibration on the plain copy (%s reads exactly %d KiB and writes exactly %d KiB per launch):" % (names[copy][:40], known_kib, known_kib),
+            "  FETCH_SIZE reads %.1f -> factor %.4f" % (fetch[copy][0], ff), "  WRITE_SIZE reads %.1f -> factor %.4f" % (write[copy][0], wf), "",
+            "Scaled HBM-side traffic per launch (fetch x %.4f + write x %.4f, KiB -> bytes):" % (ff, wf)]
+    lines = []
+    for key, label, kernels in TRAFFIC_KERNELS:
+        total, parts, ok = 0.0, [], True
+        for pattern, grid in kernels:
+            k = pick(pattern, grid)
+            if k is None or k not in fetch or k not in write:
+                ok = False
+                break
+            total += (fetch[k][0] * ff + write[k][0] * wf) * 1024.0
+            parts.append("%s: fetch %.0f KiB + write %.0f KiB" % (names[k][:48], fetch[k][0] * ff, write[k][0] * wf))
+        if not ok:
+            out.append("  %-44s (kernel not seen in the counter files)" % label)
+            continue
+        out.append("  %-44s %9.1f MB   %s" % (label, total / 1e6, "; ".join(parts)))
+        lines.append("traffic_bytes %s %d" % (key, round(total)))
+    out += ["", "What bench.py reads (workload key, HBM-side bytes per launch):"] + lines
+    print("\n".join(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -912,7 +1007,11 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="measure only the selected workload")
     ap.add_argument("--skip", default="", help="comma-separated workloads to leave out of the other workloads (e.g. ceilings, whose probe launches reuse the GEMM kernels at other sizes and would mix into a profiler's per-kernel averages)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), help="no measurement: write the HBM-traffic summary that `traffic` is read from, from the counter_collection.csv files of two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE)")
     args = ap.parse_args()
+    if args.pmc_summary:
+        pmc_summary(*args.pmc_summary)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (every path here runs on a single MI355X)" % args.gpus)
     import torch

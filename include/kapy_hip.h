@@ -286,8 +286,10 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
  * that class only.  KAPY_ERR_UNSUPPORTED otherwise, or when the runtime compiler (libhiprtc) is not
  * installed -- kapy_elementwise keeps working either way.  A program that the hand-written kernels already serve
  * with its activation compiled in (act(x*s + bias) with GELU or no activation, plain binary ops) returns KAPY_OK
- * without compiling anything.  Not to be called while a stream is capturing.  With KAPY_EW_AUTO_SPECIALIZE=1 in
- * the environment kapy_elementwise does this by itself for every program that no hand-written kernel matches;
+ * without compiling anything.  Not to be called while a stream is capturing.  kapy_elementwise does this by itself
+ * for a program that no hand-written kernel matches when the program comes back: its first call with an operand signature
+ * runs on the stepwise machines, its second compiles (never while the stream is capturing; a program that does not compile
+ * is not tried again).  KAPY_EW_AUTO_SPECIALIZE=1 in the environment: already on the first call; =0: never.
  * KAPY_EW_CACHE_DIR=<dir> keeps the compiled code objects on disk for later processes. */
 int kapy_elementwise_specialize(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global *const *ins, int32_t n_ins,
                                 const kapy_global *out);

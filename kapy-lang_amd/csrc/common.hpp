@@ -76,6 +76,11 @@ int specialize_program(const kapy_ew_inst *prog, int n_inst, const int *result_d
 int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
                        hipStream_t stream);
 void specialized_stats(int64_t *loaded, int64_t *launches);
+// Counts a call of a program that no hand-written kernel matches; true when it should be compiled now (its from_call-th call of
+// this signature on this device or a later one, and compiling it has not failed before).
+bool unmatched_call_wants_compile(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                                  int from_call);
+void unmatched_compile_failed(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out);
 int specialized_source(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
                        char *source, int64_t capacity, int64_t *source_bytes, int64_t *code_bytes);
 

@@ -1209,16 +1209,22 @@ int kapy_elementwise(const kapy_ew_inst *prog, int32_t n_inst, const kapy_global
     return KAPY_OK;
   }
 
-  // KAPY_EW_AUTO_SPECIALIZE=1: a program no hand-written kernel matches is compiled on its first call instead of running on
-  // the stepwise machines (a fraction of a second once per program and operand signature; off by default so that no call
-  // takes that long unasked).  A program that cannot be compiled, or a machine without the runtime compiler, goes on below.
-  static const bool auto_specialize = [] {
+  // A program that no hand-written kernel matches is compiled when it comes back: from its second call with the same operand
+  // signature (the first runs on the stepwise machines below, so that no single call takes a compile unasked; a compile is a
+  // fraction of a second, the first in a process seconds).  KAPY_EW_AUTO_SPECIALIZE=1: on its first call; =0: never.  Never
+  // while the stream is capturing.  A program that cannot be compiled, or a machine without the runtime compiler, goes on below
+  // and is not tried again.
+  static const int compile_from_call = [] {
     const char *v = getenv("KAPY_EW_AUTO_SPECIALIZE");
-    return v && v[0] == '1';
+    return !v || !v[0] ? 2 : v[0] == '0' ? 0 : v[0] == '1' ? 1 : 2;
   }();
-  if (auto_specialize && !stream_is_capturing(s) && specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK) {
-    rc = launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s);
-    if (rc != 0) return rc < 0 ? rc : KAPY_OK;
+  if (compile_from_call && !stream_is_capturing(s) && unmatched_call_wants_compile(prog, n_inst, result_dtype, ins, n_ins, out, compile_from_call)) {
+    if (specialize_program(prog, n_inst, result_dtype, ins, n_ins, out) == KAPY_OK) {
+      rc = launch_specialized(prog, n_inst, result_dtype, ins, n_ins, out, s);
+      if (rc != 0) return rc < 0 ? rc : KAPY_OK;
+    } else {
+      unmatched_compile_failed(prog, n_inst, result_dtype, ins, n_ins, out);
+    }
   }
 
   if (!has_int) {

@@ -947,6 +947,37 @@ int launch_specialized(const kapy_ew_inst *prog, int n_inst, const int *result_d
   return 1;
 }
 
+// How often an unmatched program of this signature has been called on this device, and whether compiling it has failed before:
+// kapy_elementwise compiles a program that keeps coming back (from its second call by default) and never tries a failed one again.
+namespace {
+struct Seen {
+  int calls = 0;
+  bool failed = false;
+};
+std::map<std::pair<int, std::string>, Seen> g_seen;
+}  // namespace
+bool unmatched_call_wants_compile(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out,
+                                  int from_call) {
+  Signature sig;
+  View vi[kJitInputs], vo;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig, vi, &vo)) return false;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return false;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  Seen &seen = g_seen[{device, make_key(prog, n_inst, sig)}];
+  if (seen.calls < from_call) ++seen.calls;
+  return !seen.failed && seen.calls >= from_call;
+}
+void unmatched_compile_failed(const kapy_ew_inst *prog, int n_inst, const int *result_dtype, const kapy_global *const *ins, int n_ins, const kapy_global *out) {
+  Signature sig;
+  View vi[kJitInputs], vo;
+  if (!classify(prog, n_inst, result_dtype, ins, n_ins, out, &sig, vi, &vo)) return;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g_seen[{device, make_key(prog, n_inst, sig)}].failed = true;
+}
+
 void specialized_stats(int64_t *loaded, int64_t *launches) {
   if (loaded) *loaded = g_count.load();
   if (launches) *launches = g_launches.load();

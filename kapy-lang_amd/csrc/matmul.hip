@@ -1201,7 +1201,9 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   tile_of_block(p, tm, tn);
   const int32_t m0 = tm * kNBM, n0 = tn * kNBN;
   const int32_t split = enter_split(p, 2);
-  const int KT = KTAIL ? (p.K + BK - 1) / BK : p.K / BK;
+  // (a scalar: in the builds whose epilogue calls the element store out of line the parameters live in scratch memory, and a
+  // count read back from there would make every branch on it a vector compare)
+  const int KT = __builtin_amdgcn_readfirstlane(KTAIL ? (p.K + BK - 1) / BK : p.K / BK);
   // elements between neighbours along the staged rows' other extent: between rows (K-contiguous) or between k-rows (transposed)
   const int32_t a_ld = (int32_t)(A_TR ? p.a_sk : p.a_sm), b_ld = (int32_t)(B_TR ? p.b_sk : p.b_sn);
 
@@ -1233,7 +1235,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     return (int32_t)chunk * 8;
   };
   // From the last K-tile on (the loads past the end of K repeat it): pieces at or beyond K get an offset no descriptor covers.
-  auto enter_k_tail = [&]() {
+  auto enter_k_tail = [&]() __attribute__((always_inline)) {
     const int32_t k_left = p.K - (KT - 1) * BK;
 #pragma unroll
     for (int q = 0; q < kLoadsOp; ++q) {
@@ -1262,7 +1264,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   // (the scalar offsets of K-tile j, clamped to the last tile: loads past the end of K are still issued, into stages nobody reads)
   auto soff_a_of = [&](int j) { return min(j, KT - 1) * BK * (A_TR ? a_ld : 1) * 2; };
   auto soff_b_of = [&](int j) { return min(j, KT - 1) * BK * (B_TR ? b_ld : 1) * 2; };
-  auto issue_load_at = [&](int soff_a, int soff_b, int stage, int idx) {
+  auto issue_load_at = [&](int soff_a, int soff_b, int stage, int idx) __attribute__((always_inline)) {
     if (idx < kLoadsOp)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + idx * 4096 + wave_lds), 16,
                                                (int)a_goff[idx], soff_a, 0, 0);
@@ -1270,7 +1272,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (__attribute__((address_space(3))) void *)(lds + stage * kStage + kBytesA + (idx - kLoadsOp) * 4096 + wave_lds),
                                                16, (int)b_goff[idx - kLoadsOp], soff_b, 0, 0);
   };
-  auto issue_load = [&](int j, int stage, int idx) { issue_load_at(soff_a_of(j), soff_b_of(j), stage, idx); };
+  auto issue_load = [&](int j, int stage, int idx) __attribute__((always_inline)) { issue_load_at(soff_a_of(j), soff_b_of(j), stage, idx); };
 
   // Operand reads, from the operand fragments of the instruction (l16: the lane's row of an lhs block = its column of
   // an rhs block; grp: which 8 of a slice's 32 K positions its registers hold).  K-contiguous operand: row / column l16 of each
@@ -1314,7 +1316,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     }
   }
   // read `r` (0 .. 3) of slice kk of the stage: block r of the operand
-  auto read_op = [&](auto is_b, auto stage, auto kk, auto blk, Frags &dst) {
+  auto read_op = [&](auto is_b, auto stage, auto kk, auto blk, Frags &dst) __attribute__((always_inline)) {
     constexpr bool kIsB = decltype(is_b)::value, kTr = kIsB ? B_TR : A_TR;
     constexpr int b = decltype(blk)::value;
     auto win = [&](uint32_t w, int x) { if constexpr (kIsB) return b_win[w][x]; else return a_win[w][x]; };
@@ -1329,7 +1331,7 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   };
   using IsA = std::integral_constant<bool, false>;
   using IsB = std::integral_constant<bool, true>;
-  auto operand_of = [](auto tr, const Frags &f, int b) -> u32x4 {
+  auto operand_of = [](auto tr, const Frags &f, int b) __attribute__((always_inline)) -> u32x4 {
     if constexpr (decltype(tr)::value) return u32x4{f.h0[b][0], f.h0[b][1], f.h1[b][0], f.h1[b][1]};
     else return f.c[b];
   };
@@ -1359,11 +1361,15 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   constexpr int kReads = kTm + kTn;
   constexpr int kLoadSpacing = (KK * kMfmas) / kLoads;  // matrix instructions between two loads
   static_assert(kLoadSpacing >= 2 && kReads <= kMfmas - (kMfmas + kLoadSpacing - 1) / kLoadSpacing, "a slice has a gap without a load for each of its reads");
+  // (Every lambda that touches the fragment buffers is always_inline.  Left to its cost model the compiler once kept tile_step
+  // out of line in one build - both operands transposed, 64-deep, partial last K-tile - and the buffers it captures by
+  // reference then live in scratch memory: registers with a transposing read still pending were stored there before their
+  // data had arrived, and the products were wrong.)
   // One K-tile in ring stage STAGE (a type: every LDS address of the step is then a constant).  `parity` says which
   // fragment buffer holds slice 0 of this tile: with an odd number of slices per tile it alternates from tile to tile.
   // What goes behind which matrix instruction follows the tiled kernel's rule: a read never shares a gap with a load,
   // and a load's gap is left to the scheduler, which moves the M0 write ahead of the matrix instruction.
-  auto tile_step = [&](int kt, auto stage_c, auto parity) {
+  auto tile_step = [&](int kt, auto stage_c, auto parity) __attribute__((always_inline)) {
     constexpr int stage = decltype(stage_c)::value, par = decltype(parity)::value;
     constexpr int next_stage = stage + 1 == STAGES ? 0 : stage + 1, free_stage = stage == 0 ? STAGES - 1 : stage - 1;
     // (the scalar offsets of this step's loads are formed here, beside the barrier, not in the gaps of the loads)
@@ -1373,14 +1379,14 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
     // own loads of tile kt+1 have landed once only the younger tiles' loads remain in flight
     __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(kLoads * (STAGES - 3)));
     __builtin_amdgcn_s_barrier();  // tile kt+1 published; every wave has left tile kt-1
-    static_for<KK>([&](auto kk_c) {
+    static_for<KK>([&](auto kk_c) __attribute__((always_inline)) {
       constexpr int kk = decltype(kk_c)::value;
       Frags &a_cur = af[(kk + par) & 1], &a_nxt = af[(kk + par + 1) & 1];
       Frags &b_cur = bf[(kk + par) & 1], &b_nxt = bf[(kk + par + 1) & 1];
       // the transposed fragments of this slice were requested during the previous one
       if constexpr (A_TR) tr_reads_wait(a_cur.h0, a_cur.h1);
       if constexpr (B_TR) tr_reads_wait(b_cur.h0, b_cur.h1);
-      static_for<kMfmas>([&](auto g_c) {
+      static_for<kMfmas>([&](auto g_c) __attribute__((always_inline)) {
         constexpr int g = decltype(g_c)::value, i = g / kTn, j = g % kTn;
         constexpr bool load_here = (kk * kMfmas + g) % kLoadSpacing == kLoadSpacing - 1 && (kk * kMfmas + g) / kLoadSpacing < kLoads;
         const u32x4 a_op = operand_of(ATr{}, a_cur, i), b_op = operand_of(BTr{}, b_cur, j);
@@ -1402,10 +1408,18 @@ __global__ __launch_bounds__(256) void nn_kernel(GemmParams p) {
   constexpr int kUnroll = (KK & 1) && (STAGES & 1) ? 2 * STAGES : STAGES;
   int kt = 0;
   for (; kt + kUnroll <= KT; kt += kUnroll)
-    static_for<kUnroll>([&](auto u) { tile_step(kt + decltype(u)::value, std::integral_constant<int, decltype(u)::value % STAGES>{}, std::integral_constant<int, (decltype(u)::value * KK) & 1>{}); });
-  static_for<kUnroll - 1>([&](auto u) {
+    static_for<kUnroll>([&](auto u) __attribute__((always_inline)) { tile_step(kt + decltype(u)::value, std::integral_constant<int, decltype(u)::value % STAGES>{}, std::integral_constant<int, (decltype(u)::value * KK) & 1>{}); });
+  // Every step ends with the transposing reads of the NEXT step's first slice in flight, and only that step waits for them.  A
+  // step that does not run (past the last K-tile) waits in its place, first thing, and so does the end of the kernel: the
+  // compiler does not know that those registers are pending and, once nobody reads them any more, hands them out again - a
+  // late result would land on top of the new value.  (These waits name no register: an asm operand may be given another
+  // register than the read's, and the copy into it would itself read the pending one.  That no instruction names a pending
+  // register before its wait is checked on the library's machine code by the build tests.)
+  static_for<kUnroll - 1>([&](auto u) __attribute__((always_inline)) {
     if (kt + decltype(u)::value < KT)
       tile_step(kt + decltype(u)::value, std::integral_constant<int, decltype(u)::value % STAGES>{}, std::integral_constant<int, (decltype(u)::value * KK) & 1>{});
+    else if constexpr (A_TR || B_TR)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   });
   __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(0));
   // the in-place matrix instructions are opaque to the compiler, which therefore does not count the wait states their
@@ -1914,14 +1928,11 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
     if (p.K % 8 == 0 && !c.stages && c.split_k <= 1) {
 #define KAPY_NN_TAIL(BK) {launch_nn<Bf16M16, BK, 4, false, true, true>, launch_nn<Bf16M16, BK, 4, true, true, true>, launch_nn<Bf16M16, BK, 4, true, false, true>, \
                           launch_nn<F16M16, BK, 4, false, true, true>, launch_nn<F16M16, BK, 4, true, true, true>, launch_nn<F16M16, BK, 4, true, false, true>}
-      // (with both operands transposed only the 32-deep build: the 64-deep one needs a stack object for its fragments and
-      // gave wrong results)
-      static int (*const kTail64[6])(GemmParams, hipStream_t) = {launch_nn<Bf16M16, 64, 4, false, true, true>, nullptr, launch_nn<Bf16M16, 64, 4, true, false, true>,
-                                                                 launch_nn<F16M16, 64, 4, false, true, true>, nullptr, launch_nn<F16M16, 64, 4, true, false, true>};
+      static int (*const kTail64[6])(GemmParams, hipStream_t) = KAPY_NN_TAIL(64);
       static int (*const kTail32[6])(GemmParams, hipStream_t) = KAPY_NN_TAIL(32);
 #undef KAPY_NN_TAIL
-      const int bk = c.tile_k ? c.tile_k : (p.K >= 256 && form != 1 ? 64 : 32);
-      if ((bk == 64 && form != 1) || bk == 32) {
+      const int bk = c.tile_k ? c.tile_k : (p.K >= 256 ? 64 : 32);
+      if (bk == 64 || bk == 32) {
         p.split_k = 1;
         return (bk == 64 ? kTail64 : kTail32)[(bf16 ? 0 : 3) + form](p, s);
       }

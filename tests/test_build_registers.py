@@ -64,10 +64,81 @@ def test_no_kernel_spills(tmp_path):
             m = re.search(r"tn_kernel<.*, (true|false), (true|false), (true|false)>", name)
             if m and (m.group(1) == "false" or m.group(2) == "true"):  # element-store epilogue / partial last K-tile
                 continue
-            if re.search(r"nn_kernel<[^,]+, \d+, \d+, false,", name) or "staged_kernel<" in name:    # element-store epilogue (staged_kernel holds both)
+            if "nn_kernel<" in name:
+                # no register of any build may be spilled: a transposing read's result is pending until the kernel's own wait, and a
+                # spill (or a fragment buffer kept in scratch memory) would store it before it has arrived.  The builds with the
+                # element-store epilogue call that store out of line, which takes a private segment and nothing else.
+                packed = re.search(r"nn_kernel<[^,]+, \d+, \d+, true,", name) is not None
+                if int(field("vgpr_spill_count")) or int(field("sgpr_spill_count")) > 64 or int(field("private_segment_fixed_size")) > (0 if packed else 256):
+                    bad.append("%s: %s VGPRs spilled, %s SGPRs spilled, %s bytes of private segment" %
+                               (name[:140], field("vgpr_spill_count"), field("sgpr_spill_count"), field("private_segment_fixed_size")))
+                continue
+            if "staged_kernel<" in name:    # element-store epilogue
                 continue
             if int(field("vgpr_spill_count")) or int(field("sgpr_spill_count")) > 64 or int(field("private_segment_fixed_size")):
                 bad.append("%s: %s VGPRs spilled, %s SGPRs spilled, %s bytes of private segment" %
                            (name[:140], field("vgpr_spill_count"), field("sgpr_spill_count"), field("private_segment_fixed_size")))
     assert seen > 100, "only %d kernels found" % seen
     assert not bad, "\n".join(bad)
+
+
+def _registers(text):
+    """Vector registers named in an operand string: v7, v[4:7]."""
+    regs = set()
+    for lo, hi in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+        regs.update(range(int(lo), int(hi) + 1))
+    regs.update(int(r) for r in re.findall(r"\bv(\d+)\b", text))
+    return regs
+
+
+@pytest.mark.skipif(not os.path.exists(LIB), reason="library not built")
+@pytest.mark.skipif(not all(os.path.exists(os.path.join(LLVM, t)) for t in ("llvm-objcopy", "llvm-objdump")), reason="binary tools not found")
+def test_no_instruction_touches_a_pending_transposing_read(tmp_path):
+    """The kernels issue ds_read_b64_tr_b16 as opaque assembly and wait for the results themselves (s_waitcnt lgkmcnt(0)); the compiler
+    does not know that the destination registers are pending in between.  In the library's own machine code, between such a read
+    and the next wait for LDS results no instruction may name a destination register of the read - not a copy, not a store to
+    scratch memory, not an overwrite - on the straight path and along every forward branch (the pending set travels with a branch
+    to its label)."""
+    seen_reads, bad = 0, []
+    for path in _code_objects(tmp_path):
+        text = subprocess.run([os.path.join(LLVM, "llvm-objdump"), "-d", "--symbolize-operands", "--no-show-raw-insn", path], check=True, capture_output=True, text=True).stdout
+        if "ds_read_b64_tr_b16" not in text:
+            continue
+        kernel, pending, at_label = "?", set(), {}
+        for line in text.split("\n"):
+            m = re.match(r"^[0-9a-f]+ <(.+)>:$", line)
+            if m:
+                if re.fullmatch(r"L\d+", m.group(1)):
+                    pending |= at_label.pop(m.group(1), set())
+                else:
+                    kernel, pending, at_label = m.group(1), set(), {}
+                continue
+            inst = line.split("//")[0].strip()
+            if not inst:
+                continue
+            op, _, operands = inst.partition(" ")
+            if op == "ds_read_b64_tr_b16":
+                seen_reads += 1
+                dst, _, rest = operands.partition(",")
+                if _registers(rest) & pending:
+                    bad.append("%s: %s addresses through a pending register" % (kernel[:100], inst))
+                pending |= _registers(dst)
+                continue
+            if op == "s_waitcnt" and ("lgkmcnt(0)" in operands or re.fullmatch(r"(0x)?0+", operands.strip())):
+                pending = set()
+                continue
+            if op.startswith("s_cbranch") or op == "s_branch":
+                target = operands.strip()
+                if pending and re.fullmatch(r"L\d+", target):
+                    at_label[target] = at_label.get(target, set()) | pending
+                if op == "s_branch":
+                    pending = set()
+                continue
+            if op in ("s_endpgm", "s_setpc_b64", "s_swappc_b64") and pending:
+                bad.append("%s: %s with reads pending" % (kernel[:100], op))
+                pending = set()
+                continue
+            if pending and _registers(operands) & pending:
+                bad.append("%s: '%s' names v%s while a transposing read into it is pending" % (kernel[:100], inst, sorted(_registers(operands) & pending)))
+    assert seen_reads > 1000, "only %d transposing reads found: is the disassembly what this test expects?" % seen_reads
+    assert not bad, "\n".join(bad[:20]) + "\n(%d in all)" % len(bad)

@@ -490,6 +490,64 @@ print("auto ok")
     assert out.returncode == 0 and "auto ok" in out.stdout, out.stdout + out.stderr
 
 
+
+def test_by_default_a_program_is_compiled_when_it_comes_back(ko):
+    """Without the switch (in a process of its own, where nothing was compiled before): the first call of a program outside the
+    hand-written kernels runs on the stepwise machines, the second compiles it, later ones launch the compiled kernel; another
+    operand signature of the same program starts counting again; a captured call never compiles; results equal the oracle's
+    whichever path served the call.  KAPY_EW_AUTO_SPECIALIZE=0: never."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r'''
+import os, sys
+sys.path[:0] = [%r, %r, %r]
+import numpy as np, torch, kapy_hip as kh, ko
+from gpu_util import dev_zeros, dglobal, sync, to_dev, to_host
+never = os.environ.get("KAPY_EW_AUTO_SPECIALIZE") == "0"
+m, n = 64, 512
+a, b = ko.fill_normal(m * n, kh.F16, 5, 0).reshape(m, n), ko.fill_normal(m * n, kh.F16, 5, 1).reshape(m, n)
+L, ADD, MUL, ST = kh.EW_LD_GLOBAL, kh.EW_ADDF, kh.EW_MULF, kh.EW_ST_GLOBAL
+insts = [dict(op=L, dst=0, a=0), dict(op=L, dst=1, a=1), dict(op=MUL, dst=2, a=0, b=1), dict(op=ADD, dst=2, a=2, b=0), dict(op=ST, a=2)]
+want = np.zeros((m, n), np.uint16)
+assert ko.elementwise(ko.program(insts), [ko.mk_global(a, m, n, n, 1, kh.F16), ko.mk_global(b, m, n, n, 1, kh.F16)], ko.mk_global(want, m, n, n, 1, kh.F16)) == 0
+da, db, dz = to_dev(a), to_dev(b), dev_zeros(m * n, 2)
+g = lambda t: dglobal(t, m, n, n, 1, kh.F16)
+expect = [(0, 0), (1, 1), (1, 2), (1, 3)]
+for call in range(4):
+    dz.zero_()
+    kh.elementwise(kh.program(insts), [g(da), g(db)], g(dz)); sync()
+    assert kh.elementwise_specialize_stats() == ((0, 0) if never else expect[call]), (call, kh.elementwise_specialize_stats())
+    assert np.array_equal(to_host(dz, np.uint16, (m, n)), want), call
+if not never:
+    # the same program with a row operand in place of the second full one: another signature, counted from one again
+    grow = dglobal(db, 1, n, n, 1, kh.F16)
+    kh.elementwise(kh.program(insts), [g(da), grow], g(dz)); sync()
+    assert kh.elementwise_specialize_stats() == (1, 3)
+    # under capture nothing is compiled: its second call is recorded on the stepwise machine and replays correctly
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            kh.elementwise(kh.program(insts), [g(da), grow], g(dz), stream=side.cuda_stream)
+    assert kh.elementwise_specialize_stats() == (1, 3)
+    want_row = np.zeros((m, n), np.uint16)
+    assert ko.elementwise(ko.program(insts), [ko.mk_global(a, m, n, n, 1, kh.F16), ko.mk_global(b, 1, n, n, 1, kh.F16)], ko.mk_global(want_row, m, n, n, 1, kh.F16)) == 0
+    for rep in range(2):
+        dz.zero_(); sync(); graph.replay(); sync()
+        assert np.array_equal(to_host(dz, np.uint16, (m, n)), want_row)
+print("default ok")
+''' % (os.path.join(root, "kapy-lang_amd", "python"), os.path.join(root, "oracle"), os.path.join(root, "tests"))
+    for value in (None, "0"):
+        env = {k: v for k, v in os.environ.items() if k != "KAPY_EW_AUTO_SPECIALIZE"}
+        if value is not None:
+            env["KAPY_EW_AUTO_SPECIALIZE"] = value
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+        assert out.returncode == 0 and "default ok" in out.stdout, out.stdout + out.stderr
+
+
 def test_full_size_transpose_fused_with_gelu(ko):
     """y = gelu_tanh(x^T*0.5 + bias) on fp16 8192x8192 through the tiled skeleton: the whole result against the two
     hand-written kernels run one after the other (transpose, then the fused GELU; <= 2 ulp: one contracts x*s + b into an

@@ -907,22 +907,34 @@ WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce",
 # Which kernels' dispatches are one launch of which workload: (workload key, label, [(kernel-name pattern, grid size or None)]);
 # the bytes of the listed kernels add up (a workload of two kernels launches each once per step).
 TRAFFIC_KERNELS = [
-    ("gelu", "C2 gelu fp16 8192^2", [(r"affine_act_cols_kernel<.*(GELU|1\)|, 1[,>])", None)]),
-    ("add", "x + y fp16 8192^2", [(r"affine_act_kernel<", None)]),
-    ("expr", "x*y + x fp16 8192^2 (compiled from its second call)", [(r"kapy_ew_flat_", 32768 * 256)]),
-    ("copy", "copy 2 x 128 MiB", [(r"rows_kernel<", None)]),
+    ("copy", "copy 2 x 128 MiB", [(r"rows_kernel<", None)]),           # (first: the calibration kernel)
     ("permute", "C3b permute", [(r"rows_kernel<", None)]),
+    ("gelu", "C2 gelu fp16 8192^2", [(r"affine_act_cols_kernel", None)]),
+    ("add", "x + y fp16 8192^2", [(r"affine_act_kernel", None)]),
+    # the compiled kernels are named after a hash of their program and operand signature (a changed program shows up here as
+    # "kernel not seen")
+    ("expr", "x*y + x fp16 8192^2 (compiled from its second call)", [(r"kapy_ew_flat_4fe8d22e", None)]),
+    ("expr_compiled", "x*y + x fp16 8192^2, compiled", [(r"kapy_ew_flat_4fe8d22e", None)]),
+    ("swiglu", "silu(x)*y fp16 8192^2, compiled", [(r"kapy_ew_flat_3c2da24d", None)]),
+    ("gelu_transposed", "gelu(x^T*0.5 + bias), compiled", [(r"kapy_ew_flat_b65a1568", None)]),
+    ("l2norm_compiled", "x*rsqrt(sum x^2), compiled", [(r"kapy_ew_rows_7416033f", None)]),
+    ("causal_softmax", "causal-masked softmax, compiled", [(r"kapy_ew_rows_575adad9", None)]),
     ("transpose", "C3a transpose fp16 8192^2", [(r"transpose_lds_kernel<", None)]),
     ("reduce", "row sums fp16 8192^2", [(r"reduce_rows_vec_kernel<", None)]),
     ("reduce_cols", "column sums fp16 8192^2", [(r"reduce_cols_strip_kernel<", None)]),
     ("softmax_cols", "column softmax fp16 8192^2", [(r"col_softmax_stats_kernel<", None), (r"col_softmax_apply_kernel<", None)]),
     ("softmax", "row softmax fp16 8192^2", [(r"softmax_kernel<", None)]),
     ("layernorm", "layer norm fp16 8192^2", [(r"norm_kernel<", None)]),
-    ("gemm_bf16", "C4 gemm bf16 8192^3", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, false>\(", None)]),
-    ("gemm_bf16_gelu", "C4 gemm bf16 8192^3 + gelu", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, true>\(", None)]),
+    ("gemm_bf16", "C4 gemm bf16 8192^3", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, false>[(]", None)]),
+    ("gemm_bf16_gelu", "C4 gemm bf16 8192^3 + gelu", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, true>[(]", None)]),
     ("f8_m4096", "C5 W8A8 M=4096", [(r"tn_kernel<kapy::F8M16<0, 0>, 256, 256, 128", None)]),
     ("f8_m16", "C5 W8A8 M=16", [(r"skinny_stream_kernel<", None)]),
+    ("f8_m64", "W8A8 M=64", [(r"skinny_block_kernel<", 256 * 256)]),
+    ("f8_m128", "W8A8 M=128", [(r"skinny_block_kernel<", 512 * 256)]),
+    ("f8_m128_splitk", "W8A8 M=128, K split over workgroups", [(r"tn_kernel<kapy::F8M16<0, 0>, 128, 128, 128", None)]),
     ("gemm_f16", "C1 gemm fp16 1024^3", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),
+    ("gemm_f16_graph", "C1 gemm fp16 1024^3, replayed from a graph", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),
+    ("gemm_f16_splitk", "C1 gemm fp16 1024^3, K split two ways", [(r"nn_kernel<kapy::F16M16", 128 * 256)]),
 ]
 
 
@@ -949,7 +961,8 @@ def pmc_summary(fetch_csv, write_csv):
     ours = sorted(k for k in set(fetch) | set(write) if "kapy" in k[0])
     names = {}
     try:
-        demangled = subprocess.run(["c++filt"], input="\n".join(k[0] for k in ours), capture_output=True, text=True).stdout.split("\n")
+        tool = "/opt/rocm/llvm/bin/llvm-cxxfilt" if os.path.exists("/opt/rocm/llvm/bin/llvm-cxxfilt") else "c++filt"
+        demangled = subprocess.run([tool], input="\n".join(k[0] for k in ours), capture_output=True, text=True).stdout.split("\n")
         names = {k: d.replace("void ", "").replace("kapy::(anonymous namespace)::", "") for k, d in zip(ours, demangled)}
     except OSError:
         names = {k: k[0] for k in ours}
@@ -971,7 +984,7 @@ def pmc_summary(fetch_csv, write_csv):
     for k in ours:
         f, w = fetch.get(k, (0.0, 0)), write.get(k, (0.0, 0))
         out.append("%-86s %10d %12.1f (%5d) %12.1f (%5d)" % (names[k][:86], k[1], f[0], f[1], w[0], w[1]))
-    copy = pick(*TRAFFIC_KERNELS[3][2][0])
+    copy = pick(*TRAFFIC_KERNELS[0][2][0])
     if copy is None or copy not in fetch or copy not in write:
         raise SystemExit("bench.py --pmc-summary: the copy kernel (rows_kernel) is in neither counter file; nothing to calibrate against")
     known_kib = 128 * 1024

@@ -600,12 +600,15 @@ def _cpu_gemm(ko, go_a, go_b, go_d, rows, N, K, scales, what):
             "sample": "%s; fp32 accumulate, operands widened to fp32 and packed outside the timed multiply; %d repetitions, %.2f s of multiplying" % (what, reps, tot)}
 
 
-def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None, workspace=False):
-    """graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
+def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None, workspace=False, whole=True):
+    """whole: gate the whole result against the host GEMM as well as 16 blocks against the fp64 checker (a second and third large
+    problem of the same shape are gated on the blocks alone: the host GEMM takes its time).
+    graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
     (what a launch-bound shape gains when the host's per-launch cost is taken out).
     fused_gelu: d = gelu_tanh(a.b*0.5 + bias) with the tail in the GEMM's epilogue (kapy_matmul_fused); flops counted are the GEMM's.
     gen: "normal" = normal(0, 0.02) seeds 0 / 1 (C4), "uniform" = uniform[-1,1) seed 0 streams 0 / 1 (C1).
-    workspace: hand the library a workspace, which lets it split K across workgroups when the tiles alone would not fill the device."""
+    workspace: hand the library a workspace, which lets it split K across workgroups when the tiles alone would not fill the device,
+    or turn a large row-major rhs K-contiguous before multiplying."""
     import numpy as np
     import torch
     import ko
@@ -629,7 +632,8 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
         gbias = kh.mk_global(bias.data_ptr(), 1, N, N, 1, dtype)
         run = lambda i: kh.matmul_fused(ga, gb, gd, bias=gbias, alpha=0.5, act=kh.EW_GELU_TANH, tile=tile)
     else:
-        ws = torch.zeros(kh.lib().kapy_matmul_workspace_bytes(M, N), dtype=torch.uint8, device="cuda") if workspace else None
+        ws_bytes = max(kh.lib().kapy_matmul_workspace_bytes(M, N), kh.lib().kapy_matmul_turn_workspace_bytes(ga, gb))
+        ws = torch.zeros(ws_bytes, dtype=torch.uint8, device="cuda") if workspace else None
         run = lambda i: kh.matmul(ga, gb, gd, tile=tile, workspace=ws)
     run(0)
     torch.cuda.synchronize()
@@ -654,10 +658,11 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
         n_blocks = 16 if M * N > 1024 * 1024 else 0
         if n_blocks:
             rel = _blocks_frobenius(ko, got, go_a, go_b, M, N, K, dtype, n_blocks)
-            whole, host_rel = _whole_frobenius(ko, got, go_a, go_b, M, N, K, dtype)
-            if not host_rel <= FROB_TOL:
-                raise CheckFailed("%s: the host GEMM itself is off the fp64 checker by %g" % (name, host_rel))
-            rel = max(rel, whole)
+            if whole:
+                whole_rel, host_rel = _whole_frobenius(ko, got, go_a, go_b, M, N, K, dtype)
+                if not host_rel <= FROB_TOL:
+                    raise CheckFailed("%s: the host GEMM itself is off the fp64 checker by %g" % (name, host_rel))
+                rel = max(rel, whole_rel)
         else:   # small enough for the whole result
             want = np.zeros((M, N), np.uint16)
             assert ko.lib().ko_matmul(C.byref(go_a), C.byref(go_b), None, C.byref(ko.mk_global(want, M, N, N, 1, dtype)), ko.RN) == 0
@@ -900,7 +905,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
 
 
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "causal_softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
 
 
 # ---------------------------------------------------------------- HBM traffic summary from the profiler's counter files
@@ -1053,6 +1058,8 @@ def main():
         "permute": lambda s, w: bench_permute(kh, s, w, cpu),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel", key="gemm_bf16"),
         "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True, key="gemm_bf16_gelu"),
+        "gemm_bf16_nn": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, read in place by transposing LDS reads (128 x 128 tiles)", "nn_kernel", key="gemm_bf16_nn", whole=False),
+        "gemm_bf16_nn_turned": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, workspace given: the rhs is turned K-contiguous first (time and rate include the turn)", "transpose_lds_kernel + tn_kernel", key="gemm_bf16_nn_turned", workspace=True, whole=False),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform", key="gemm_f16"),
         "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform", key="gemm_f16_graph"),
         "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True, key="gemm_f16_splitk"),

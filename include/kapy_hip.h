@@ -316,9 +316,10 @@ typedef struct kapy_matmul_cfg {
   int32_t split_k;               /* workgroups that share one output tile, each multiplying one part of K (powers of two up to 8);
                                     1 = never split; 0 = library's choice: it splits only when a workspace is given and the
                                     result has too few 128 x 128 tiles to occupy the device */
-  void *workspace;               /* device memory for the partial sums and arrival counters of a split K, or NULL.  Its first
+  void *workspace;               /* device memory for the partial sums and arrival counters of a split K (and, when large enough,
+                                    for an operand turned K-contiguous: kapy_matmul_turn_workspace_bytes), or NULL.  Its first
                                     16 KiB (the counters) must be zero before its first use and every call leaves them zero;
-                                    calls that share a workspace must not overlap in time */
+                                    256-byte aligned; calls that share a workspace must not overlap in time */
   int64_t workspace_bytes;       /* kapy_matmul_workspace_bytes(m, n) is enough for any split of an [m x n] result */
   int32_t accumulate;            /* kapy_matmul_accumulate; 0 = fp32 accumulators, one cast at the end */
   int32_t reserved;              /* 0 */
@@ -333,6 +334,14 @@ typedef struct kapy_matmul_cfg {
 typedef enum kapy_matmul_accumulate { KAPY_ACCUMULATE_F32 = 0, KAPY_ACCUMULATE_ELEMENT = 1 } kapy_matmul_accumulate;
 /* Workspace size that lets the library split K for an [m x n] result whichever way it chooses. */
 int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n);
+/* Workspace size with which a LARGE 16-bit problem (at least 6144 rows for a row-major rhs, at least 6144 columns for a
+ * column-major lhs, at least 2048 of the other, K at least 1024, all multiples of 8) is multiplied by first turning that
+ * operand into the workspace (behind the 16 KiB of counters, which stay zero) with the transposing copy and then running
+ * the K-contiguous kernel on 256 x 256 tiles: 1.15 - 1.2 x the rate of the kernel that reads such operands in place on
+ * 128 x 128 tiles, the extra pass over the operand included.  0 when neither operand needs turning.  Used only with a free tile choice and no explicit split; a smaller
+ * workspace, or a smaller problem, is multiplied in place as before.  The turned copy is scratch: nothing reads it after
+ * the call's kernels have run. */
+int64_t kapy_matmul_turn_workspace_bytes(const kapy_global *lhs, const kapy_global *rhs);
 
 /* kapy.matmul — create_matmul(lhs, rhs, acc, implWay), python/src/ir.cc:1101-1105; verifier
  * lib/Dialect/Kapy/IR/Kapy.cpp:451-574; lowering MatmulOpToLLVM.cpp:58-311 with the

@@ -90,6 +90,8 @@ int check_global(const kapy_global *g, const char *what);
 float *reduce_scratch_lines(size_t *bytes, uint32_t **counters = nullptr);   // counters: the array's arrival counters (4096 words, zero between calls)
 // softmax of every column of a 16-bit row-major matrix in two launches (elementwise_col.hip): 1 = launched, 0 = the shapes
 // are not the kernels', a negative status on failure.
+// kapy_copy / kapy_copy_batched (copy.hip); grid may be null.
+int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, const kapy_grid2 *grid, void *stream);
 int run_matmul_f16acc(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result, int k_step, hipStream_t s);
 int run_column_softmax(const kapy_global *x, const kapy_global *out, hipStream_t stream);
 int ensure_device();

@@ -390,6 +390,8 @@ int launch(const CopyParams &p0, int vb_src, int vb_dst, bool nt, int32_t batch,
   return KAPY_OK;
 }
 
+}  // namespace
+
 int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, const kapy_grid2 *grid, void *stream) {
   int rc = check_global(src, "copy source");
   if (!rc) rc = check_global(dst, "copy target");
@@ -480,7 +482,6 @@ int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cf
   }
 }
 
-}  // namespace
 }  // namespace kapy
 
 extern "C" {

@@ -1843,6 +1843,64 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
   if (lhs->dtype != KAPY_F16 && lhs->dtype != KAPY_BF16)
     return fail(KAPY_ERR_UNSUPPORTED, "matmul: %s operands have no matrix instruction on gfx950", dtype_name(lhs->dtype));
 
+  // A large problem with an operand that is contiguous along its OTHER extent (a row-major rhs, a column-major lhs).  The kernel
+  // that reads such operands with transposing LDS reads works on 128 x 128 tiles and reaches 1.05-1.12 PFLOP/s where the
+  // K-contiguous kernel's 256 x 256 tiles reach 1.35-1.55.  Turning the operand first costs one pass of the transposing copy
+  // over it (its bytes read and written once, at 0.68 of the HBM rate) and pays from about six thousand rows on - if the caller's
+  // workspace has room for the turned operand(s) behind the 16 KiB of split-K counters, which stay untouched.
+  if (c.workspace && !c.tile_m && !c.tile_n && !c.tile_k && !c.stages && !c.waves && c.split_k <= 1 && c.impl_way < KAPY_MFMA_32X32X16_16B) {
+    const int64_t M = extent0(lhs), K = extent1(lhs), N = extent1(rhs);
+    const bool a_turn = lhs->stride0 == 1 && lhs->stride1 != 1, b_turn = rhs->stride1 == 1 && rhs->stride0 != 1;
+    const bool a_kc = lhs->stride1 == 1, b_kc = rhs->stride0 == 1;
+    const int64_t a_bytes = a_turn ? ((M * K * 2 + 255) & ~int64_t(255)) : 0, b_bytes = b_turn ? ((K * N * 2 + 255) & ~int64_t(255)) : 0;
+    // (measured, bf16, in place -> turned: 8192^3 1237 -> 1485 TFLOP/s, 8192 x 2048 x 4096 1130 -> 1317, 8192 x 8192 x 1024 924 -> 1106;
+    // 4096^3 and 2048 x 8192 x 4096 the same either way; 2048^2 x K slower by a third: the turn is paid once per operand and
+    // earned back over the rows - or, for a turned lhs, the columns - that use it)
+    if ((a_turn || b_turn) && (a_turn || a_kc) && (b_turn || b_kc) && (!b_turn || M >= 6144) && (!a_turn || N >= 6144) && M >= 2048 && N >= 2048 && K >= 1024 &&
+        M % 8 == 0 && N % 8 == 0 && K % 8 == 0 &&
+        M * K < (int64_t(1) << 31) && K * N < (int64_t(1) << 31) && kSplitCounterBytes + a_bytes + b_bytes <= c.workspace_bytes &&
+        ((uintptr_t)c.workspace & 255) == 0) {
+      char *at = (char *)c.workspace + kSplitCounterBytes;
+      kapy_global a2 = *lhs, b2 = *rhs;
+      const kapy_copy_cfg turn = {1, KAPY_PAD_ZERO, 0, 0, 0, 0};
+      auto dense = [](void *ptr, int64_t rows, int64_t cols, int32_t dtype) {
+        kapy_global g;
+        g.ptr = ptr;
+        g.start0 = g.start1 = 0;
+        g.end0 = (int32_t)rows;
+        g.end1 = (int32_t)cols;
+        g.stride0 = (int32_t)cols;
+        g.stride1 = 1;
+        g.dtype = dtype;
+        g.alignment = 16;
+        return g;
+      };
+      if (b_turn) {  // rhs [K x N] row-major -> [N x K] row-major in the workspace, read back as a [K x N] view with K contiguous
+        const kapy_global turned = dense(at, N, K, rhs->dtype);
+        rc = copy_impl(rhs, &turned, &turn, nullptr, stream);
+        if (rc) return rc;
+        b2 = turned;
+        b2.end0 = (int32_t)K; b2.end1 = (int32_t)N;
+        b2.stride0 = 1; b2.stride1 = (int32_t)K;
+        at += b_bytes;
+      }
+      if (a_turn) {  // lhs [M x K] column-major -> row-major
+        const kapy_global turned = dense(at, M, K, lhs->dtype);
+        kapy_global as_rows = *lhs;  // the same memory seen as the row-major [K x M] it is, which the copy transposes
+        std::swap(as_rows.start0, as_rows.start1);
+        std::swap(as_rows.end0, as_rows.end1);
+        std::swap(as_rows.stride0, as_rows.stride1);
+        rc = copy_impl(&as_rows, &turned, &turn, nullptr, stream);
+        if (rc) return rc;
+        a2 = turned;
+      }
+      kapy_matmul_cfg inner = c;
+      inner.workspace = nullptr;
+      inner.workspace_bytes = 0;
+      return matmul_16bit(&a2, &b2, acc, result, &inner, epi, stream);
+    }
+  }
+
   GemmParams p;
   p.a = view_base(lhs);
   p.b = view_base(rhs);
@@ -1958,6 +2016,14 @@ extern "C" {
 int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                 const kapy_matmul_cfg *cfg, void *stream) {
   return matmul_16bit(lhs, rhs, acc, result, cfg, nullptr, stream);
+}
+
+int64_t kapy_matmul_turn_workspace_bytes(const kapy_global *lhs, const kapy_global *rhs) {
+  if (!lhs || !rhs) return 0;
+  const int64_t M = extent0(lhs), K = extent1(lhs), N = extent1(rhs);
+  const bool a_turn = lhs->stride0 == 1 && lhs->stride1 != 1, b_turn = rhs->stride1 == 1 && rhs->stride0 != 1;
+  if (!a_turn && !b_turn) return 0;
+  return kSplitCounterBytes + (a_turn ? ((M * K * 2 + 255) & ~int64_t(255)) : 0) + (b_turn ? ((K * N * 2 + 255) & ~int64_t(255)) : 0);
 }
 
 int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n) {

@@ -40,7 +40,7 @@ EXPORTS = [
     "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
-    "kapy_matmul_workspace_bytes", "kapy_matmul_static_workspace",
+    "kapy_matmul_workspace_bytes", "kapy_matmul_turn_workspace_bytes", "kapy_matmul_static_workspace",
     "kapy_mk_shared", "kapy_sv_shared", "kapy_shared_address",
 ]
 
@@ -186,6 +186,8 @@ def lib():
     L.kapy_elementwise_source.argtypes = [P(EwInst), i32, P(P(Global)), i32, P(Global), C.c_char_p, i64, P(i64), P(i64)]
     L.kapy_fptofp.argtypes = [P(Global), P(Global), i32, vp]
     L.kapy_matmul.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
+    L.kapy_matmul_turn_workspace_bytes.restype = i64
+    L.kapy_matmul_turn_workspace_bytes.argtypes = [P(Global), P(Global)]
     L.kapy_matmul_static_workspace.argtypes = [P(Global), P(Global), P(Global), P(Global), P(MatmulCfg), vp]
     L.kapy_matmul_workspace_bytes.restype = i64
     L.kapy_matmul_workspace_bytes.argtypes = [i64, i64]
@@ -205,7 +207,7 @@ def lib():
     for name in EXPORTS:
         f = getattr(L, name)
         if name not in ("kapy_last_error", "kapy_smem_plan", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_num_shuffles", "kapy_swizzle_offset",
-                        "kapy_matmul_workspace_bytes", "kapy_shared_address"):
+                        "kapy_matmul_workspace_bytes", "kapy_matmul_turn_workspace_bytes", "kapy_reduce_workspace_bytes", "kapy_shared_address"):
             f.restype = C.c_int
     _lib = L
     return L

@@ -317,3 +317,40 @@ def test_transposing_read_kernel_with_a_partial_last_k_tile(ko, dt, a_rm, b_rm):
         got = to_host(dd, np.uint16)
         assert np.all(got[M * N:] == 0x1234), (M, N, K)
         assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL, (M, N, K)
+
+
+@pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("a_rm,b_rm", [(True, True), (False, True), (False, False)])
+def test_large_problem_with_a_workspace_turns_the_operand_first(ko, dt, a_rm, b_rm):
+    """A row-major rhs / column-major lhs of a large problem, with a workspace of kapy_matmul_turn_workspace_bytes: the operand is
+    turned K-contiguous into the workspace and the K-contiguous kernel multiplies.  Same result as the in-place kernel within the
+    GEMM tolerance (sampled blocks against the checker), the counters at the head of the workspace stay zero, and a workspace
+    that is too small changes nothing."""
+    import torch
+    M, N, K = 6144, 6400, 1024
+    a, b = ko.fill_normal(M * K, dt, 41, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 41, 1, 0.0, 0.5)
+    a_str, b_str = ((K, 1) if a_rm else (1, M)), ((N, 1) if b_rm else (1, K))
+    da, db = to_dev(a), to_dev(b)
+    ga, gb = dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt)
+    need = kh.lib().kapy_matmul_turn_workspace_bytes(C.byref(ga), C.byref(gb))
+    assert need == 16384 + (0 if a_rm else M * K * 2) + (K * N * 2 if b_rm else 0)
+    outs = []
+    for ws_bytes in (0, 4096 + 16384, need):
+        ws = torch.zeros(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
+        dd = dev_zeros(M * N + 256, 2, fill=0x1234)
+        kh.matmul(ga, gb, dglobal(dd, M, N, N, 1, dt), workspace=ws)
+        sync()
+        got = to_host(dd, np.uint16)
+        assert np.all(got[M * N:] == 0x1234)
+        if ws is not None:
+            assert not ws[:16384].any()
+        outs.append(got[:M * N].reshape(M, N))
+    assert np.array_equal(outs[0], outs[1])                      # too small a workspace: the in-place kernel, as without one
+    goa, gob = ko.mk_global(a, M, K, *a_str, dt), ko.mk_global(b, K, N, *b_str, dt)
+    for t in range(6):
+        r0, c0 = (t * 331) % (M - 64), (t * 577) % (N - 64)
+        want = np.zeros((64, 64), np.uint16)
+        assert ko.lib().ko_matmul(C.byref(ko.sv_global(goa, r0, r0 + 64, 0, K)), C.byref(ko.sv_global(gob, 0, K, c0, c0 + 64)), None,
+                                  C.byref(ko.mk_global(want, 64, 64, 64, 1, dt)), kh.RN) == 0
+        for got in (outs[0], outs[2]):
+            assert _frob(ko, np.ascontiguousarray(got[r0:r0 + 64, c0:c0 + 64]).ravel(), want.ravel(), dt) <= FROB_TOL

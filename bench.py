@@ -764,6 +764,62 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     return out
 
 
+def bench_mlir(kh, steps, warmup, cpu):
+    """The reference's three fixture programs (elementwise add, row sum, matmul; test/Conversion/KapyToKgpu/*.mlir) in the op syntax of
+    kapy_programs.py, run through kapy_run_mlir on grids of program instances: per program the time of one call with the
+    instances' stores merged into one call each (the default) and with one instance at a time (KAPY_MLIR_BATCH=0).  A call
+    parses the text, allocates and frees its arena and synchronises: the figures are those of a validation path."""
+    import numpy as np
+    import torch
+    import ko
+    import kapy_programs as kp
+    out = {"workload": "the reference's three fixture programs through kapy_run_mlir", "unit": "GB/s", "dtype": "f16", "kernel": "one call per kapy.st_global over all instances (elementwise, reduce); per instance for the matmul",
+           "inputs": "normal(0,1) seeded, fp16", "programs": {}}
+    rows_per_warp, cols, warps, programs = 4, 1024, 4, 256
+    rows = rows_per_warp * warps * programs
+    x, y = _dev("normal", rows * cols, ko.F16, 11), _dev("normal", rows * cols, ko.F16, 12)
+    d = torch.empty(rows * cols, device="cuda", dtype=torch.int16)
+    # (name, program text, arguments, grid, the tensor the program writes, algorithmic bytes or None)
+    cases = [("x + y [%d x %d], %d programs x %d warps" % (rows, cols, programs, warps), kp.binary_program("arith.addf", rows_per_warp, cols, warps), [x, y, d, rows], [programs], d, 3 * rows * cols * 2),
+             ("row sums [%d x %d], %d programs x %d warps" % (rows, cols, programs, warps), kp.reduce_program("arith.addf", rows_per_warp, cols, warps), [x, d, rows], [programs], d, rows * cols * 2 + rows * 2)]
+    M, N, K = 512, 512, 256
+    a, b = _dev("normal", M * K, ko.F16, 31, std=0.5), _dev("normal", K * N, ko.F16, 32, std=0.5)
+    c = torch.empty(M * N, device="cuda", dtype=torch.int16)
+    cases.append(("matmul %d x %d x %d, 64 x 64 x 16 per warp, f16 accumulator" % (M, N, K), kp.matmul_program(64, 64, 16, "mma_m16n8k8_f16", "f16"), [a, b, c, M, N, K], [(M // 128) * (N // 128)], c, None))
+    checked = True
+    for name, text, args, grid, target, nbytes in cases:
+        row = {}
+        results = []
+        for label, env in (("instances merged", "1"), ("one instance at a time", "0")):
+            os.environ["KAPY_MLIR_BATCH"] = env
+            target.zero_()
+            before = kh.run_mlir_stats()
+            kh.run_mlir(text, args, grid)
+            torch.cuda.synchronize()
+            row[label + ", merged stores per call"] = kh.run_mlir_stats() - before
+            results.append(target.clone())
+            t0 = time.perf_counter()
+            reps = 3
+            for _ in range(reps):
+                kh.run_mlir(text, args, grid)
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / reps
+            row[label + ", ms per call"] = round(ms, 3)
+            if nbytes:
+                row[label + ", GB/s"] = round(nbytes / (ms * 1e-3) / 1e9, 2)
+        os.environ.pop("KAPY_MLIR_BATCH", None)
+        if not torch.equal(results[0], results[1]):
+            checked = False
+        out["programs"][name] = row
+    if not checked:
+        raise CheckFailed("run_mlir: merged and per-instance runs differ")
+    first = out["programs"][cases[0][0]]
+    out.update({"value": first["instances merged, GB/s"], "ms_per_step": first["instances merged, ms per call"], "kernel_ms": first["instances merged, ms per call"],
+                "checked": True, "check": "merged and per-instance runs give the same bits (the programs themselves are compared with the checker in the GPU tests)",
+                "roofline": _roof_hbm(cases[0][5], first["instances merged, ms per call"], None)})
+    return out
+
+
 def bench_ceilings(kh, steps, warmup, cpu):
     """What this device sustains, from the library's own probe kernels: a loop of nothing but matrix instructions per
     instruction shape (operands of the benchmark's distribution; the part is power-limited, so this, not the data-sheet
@@ -905,7 +961,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
 
 
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "causal_softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "ceilings"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "mlir_fixtures", "ceilings"]
 
 
 # ---------------------------------------------------------------- HBM traffic summary from the profiler's counter files
@@ -1058,6 +1114,7 @@ def main():
         "permute": lambda s, w: bench_permute(kh, s, w, cpu),
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel", key="gemm_bf16"),
         "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True, key="gemm_bf16_gelu"),
+        "mlir_fixtures": lambda s, w: bench_mlir(kh, s, w, cpu),
         "gemm_bf16_nn": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, read in place by transposing LDS reads (128 x 128 tiles)", "nn_kernel", key="gemm_bf16_nn", whole=False),
         "gemm_bf16_nn_turned": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, workspace given: the rhs is turned K-contiguous first (time and rate include the turn)", "transpose_lds_kernel + tn_kernel", key="gemm_bf16_nn_turned", workspace=True, whole=False),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform", key="gemm_f16"),
@@ -1123,7 +1180,7 @@ def main():
         "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "kernel_ms": round(main_res["kernel_ms"], 4),
                    "inputs": main_res["inputs"], "checked": main_res["checked"], "check": main_res["check"],
                    "buffers": "4 rotating sets (1 GiB) so reads miss the Infinity Cache" if main_res["unit"] == "GB/s" else "single set",
-                   "configs": configs},
+                   "configs": configs, **({"programs": main_res["programs"]} if "programs" in main_res else {})},
         "roofline": main_res["roofline"],
         "cpu_baseline": main_res.get("cpu_baseline"),
     }

@@ -485,11 +485,19 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * and warps may exchange data through shared memory wherever the program itself is race-free (the barriers
  * kapy_analyze_mlir places are a subset of these).  A loop whose bounds differ between warps runs warp after warp;
  * KAPY_MLIR_IN_STEP=0 in the environment runs every warp to the end before the next one starts.
+ * The program instances of the grid advance in step too, in groups as large as the arena allows (every program its own
+ * shared-memory tensors).  Where all instances and warps in flight reach a kapy.st_global of chains of one form whose views
+ * - the result's and every loaded operand's - tile a rectangle over the same tensors (an operand moves with the tile along
+ * an axis or is a broadcast row, column or scalar), the store runs as ONE call over the union: one launch per op for
+ * the whole grid, as the reference's one kernel per function (FuncOpToLLVM.cpp:72-88).  Chains with register or shared
+ * operands, an arange, or a reduce across the axis the tiles lie along run per instance as before, and so do loads,
+ * copies into shared memory and kapy.matmul.  KAPY_MLIR_BATCH=0: one instance at a time, nothing merged; same results.
  * `args` follow the function's signature: a device pointer (with the size of its allocation in bytes, 0 =
  * unknown, which mk_global is checked against) for !kapy.ptr<1>, an i32 otherwise.  A sub-view that leaves
- * its parent is an error.  func_name NULL = the first function of the module.  The call allocates a 64 MiB
- * device arena for shared-memory and register tensors, synchronises `stream` and frees it before it returns:
- * it is a way to run the reference's programs against this library, not a fast path. */
+ * its parent is an error.  func_name NULL = the first function of the module.  The first call on a device allocates
+ * a 256 MiB arena for shared-memory and register tensors, which the library keeps until the process ends; calls take
+ * turns at it, and a call synchronises `stream` before it returns: it is a way to run the reference's programs against
+ * this library, not a fast path. */
 typedef struct kapy_mlir_arg {
   void *ptr;      /* device pointer, for a !kapy.ptr<1> argument                    */
   int64_t bytes;  /* size of the allocation behind ptr; 0 = unknown (no range check) */
@@ -498,6 +506,9 @@ typedef struct kapy_mlir_arg {
 } kapy_mlir_arg;
 int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_arg *args, int32_t n_args,
                   const int32_t grid[3], void *stream);
+/* How many kapy.st_global ops this process has run as ONE call for all program instances and warps in flight (the instances'
+ * chains had the same form and their views tiled a rectangle): lets a caller check that a program took that path. */
+int kapy_run_mlir_stats(int64_t *merged_stores);
 /* The parsing half of kapy_run_mlir, without a device: KAPY_ERR_INVALID for text that does not parse,
  * KAPY_ERR_UNSUPPORTED for an op outside the set above; otherwise the function's argument count, its number
  * of ops (loop bodies included) and the module's kapy.num_warps.  Out pointers may be NULL. */

@@ -23,9 +23,11 @@
 #include <cstdlib>
 #include <cstring>
 #include <algorithm>
+#include <atomic>
 #include <climits>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <set>
 #include <string>
 #include <vector>
@@ -556,7 +558,9 @@ struct Value {
 
 // Shared-memory tensors take the first part of the arena and live for the whole call; register tensors
 // take the rest and die with their program instance.
-constexpr size_t kSharedArena = size_t(256) << 10, kArena = size_t(64) << 20;
+// A call runs its program instances in groups (all programs of a group and all their warps in step): every program of a group
+// has its own shared part, the group one region for the register tensors of calls merged over instances, every warp its share.
+constexpr size_t kSharedArena = size_t(256) << 10, kArena = size_t(256) << 20, kMergedArena = size_t(64) << 20, kMinShare = size_t(1) << 20;
 
 struct Interp {
   const Func &f;
@@ -572,18 +576,28 @@ struct Interp {
   struct WarpState {
     std::map<std::string, Value> env;
     size_t top = 0, limit = 0;
+    int64_t pid[3] = {0, 0, 0}, warp = 0;  // which program instance, which of its warps
+    size_t shared_base = 0;                // where that program's shared-memory tensors start in the arena
   };
-  std::vector<WarpState> warps;
+  std::vector<WarpState> warps;  // every warp of every program of the group in flight
+  int current = -1;              // the state swapped in
   void enter(int w) {
     std::swap(env, warps[w].env);
     top = warps[w].top;
     limit = warps[w].limit;
-    warp = w;
+    warp = warps[w].warp;
+    for (int k = 0; k < 3; ++k) pid[k] = warps[w].pid[k];
+    shared_base = warps[w].shared_base;
+    current = w;
   }
   void leave(int w) {
     std::swap(env, warps[w].env);
     warps[w].top = top;
+    current = -1;
   }
+  size_t shared_base = 0, register_base = kSharedArena;  // (register_base: where the shared parts of the group end)
+  size_t merged_base = 0, merged_top = 0;                // the group's region for merged calls, and how much of it is taken
+  bool merge = true;                                     // KAPY_MLIR_BATCH=0: no call is merged over instances
   const Analysis *plan = nullptr;  // where each mk_shared lives inside the shared part of the arena
   int64_t pid[3] = {0, 0, 0}, warp = 0;
   std::string err;
@@ -614,7 +628,7 @@ struct Interp {
   bool fuse = true;  // KAPY_MLIR_FUSE=0: every op runs by itself, as one call
   bool is_register_tensor(const kapy_global &g) const {
     const char *p = (const char *)g.ptr;
-    return p >= arena + kSharedArena && p < arena + kArena;
+    return p >= arena + register_base && p < arena + kArena;
   }
   // [first, last] byte of a view (strides are positive: mk_global refuses others)
   static void byte_range(const kapy_global &g, const char **lo, const char **hi) {
@@ -648,7 +662,7 @@ struct Interp {
     };
     int rc = settle(env);
     for (size_t w = 0; rc == KAPY_OK && w < warps.size(); ++w)
-      if ((int64_t)w != warp) rc = settle(warps[w].env);
+      if ((int)w != current) rc = settle(warps[w].env);
     return rc;
   }
   // the operand as an expression: deferred tensors as they are, computed ones as leaves
@@ -837,8 +851,7 @@ struct Interp {
     }
     return true;
   }
-  // a shared-memory tensor sits at its planned offset in the shared part of the arena, the same for every
-  // program and warp
+  // a shared-memory tensor sits at its planned offset in its program's shared part of the arena, the same for every warp
   int mk_shared(const Op &op) {
     const Type &ty = op.types.back();
     for (const SharedBuffer &b : plan->buffers) {
@@ -846,7 +859,7 @@ struct Interp {
       Value r;
       r.kind = Value::kTensor;
       if (ty.kind != Type::kTensor || ty.shape[0] <= 0 || ty.shape[1] <= 0) return fail_op(op, "result must be a statically shaped tensor");
-      int rc = lib(op, kapy_mk_global(&r.g, arena + b.offset, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 128));
+      int rc = lib(op, kapy_mk_global(&r.g, arena + shared_base + b.offset, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 128));
       if (rc == KAPY_OK) env[op.results[0]] = r;
       return rc;
     }
@@ -861,6 +874,171 @@ struct Interp {
   int mapped_tensor(const Op &op, int n_operands, int ew, int dtype = 0, int rmode = KAPY_RN) {
     return defer(op, n_operands, ew, dtype, rmode, 0.f);
   }
+
+  // ---- one call for all instances ----
+  // The instances in flight all execute the same kapy.st_global.  When every one of them stores a deferred chain of the same
+  // form, and their views - the result's and every loaded operand's - are the tiles of a rectangular grid over the same
+  // tensors (an operand either moves with the tile along an axis or has extent 1 there: a broadcast row, column or scalar),
+  // the instances together are ONE program over the union of the tiles, and it runs as one call: what the reference's one
+  // kernel over the whole grid does.  Anything else (register or shared operands, which differ per instance; an arange,
+  // whose values depend on the tile's origin; a reduce across the axis the tiles are laid out along) is left to the
+  // instances one by one.
+  static bool same_bits(float a, float b) { return !memcmp(&a, &b, sizeof a); }
+  static bool is_leaf(const Expr &e) { return e.ew == KAPY_EW_LD_GLOBAL && e.n_in == 0; }
+  // do two chains have the same form (leaves may differ in where their views start)?  pairs: node of a -> node of b
+  bool same_form(const Expr *a, const Expr *b, std::map<const Expr *, const Expr *> &pairs, std::vector<const Expr *> *leaves_b) {
+    auto seen = pairs.find(a);
+    if (seen != pairs.end()) return seen->second == b;
+    if (a->ew != b->ew || a->n_in != b->n_in) return false;
+    if (is_leaf(*a)) {
+      const kapy_global &x = a->leaf, &y = b->leaf;
+      if (x.ptr != y.ptr || x.stride0 != y.stride0 || x.stride1 != y.stride1 || x.dtype != y.dtype || x.alignment != y.alignment ||
+          x.end0 - x.start0 != y.end0 - y.start0 || x.end1 - x.start1 != y.end1 - y.start1 || a->global_leaf != b->global_leaf)
+        return false;
+      if (leaves_b) leaves_b->push_back(b);
+    } else {
+      if (a->dtype != b->dtype || a->rmode != b->rmode || !same_bits(a->imm, b->imm) || a->ia != b->ia || a->ib != b->ib || a->ic != b->ic ||
+          a->rows != b->rows || a->cols != b->cols || a->operand_dtype != b->operand_dtype || a->axis != b->axis)
+        return false;
+    }
+    pairs[a] = b;
+    for (int k = 0; k < a->n_in; ++k)
+      if (!same_form(a->in[k].get(), b->in[k].get(), pairs, leaves_b)) return false;
+    return true;
+  }
+  std::shared_ptr<Expr> clone(const std::shared_ptr<Expr> &e, std::map<const Expr *, std::shared_ptr<Expr>> &made) {
+    auto it = made.find(e.get());
+    if (it != made.end()) return it->second;
+    auto c = std::make_shared<Expr>(*e);
+    made[e.get()] = c;
+    for (int k = 0; k < e->n_in; ++k) c->in[k] = clone(e->in[k], made);
+    return c;
+  }
+  bool try_merged_store(const Op &op) {
+    const int n = (int)warps.size();
+    if (n < 2 || op.operands.size() < 2) return false;
+    std::vector<std::shared_ptr<Expr>> chain(n);
+    std::vector<kapy_global> out(n);
+    for (int w = 0; w < n; ++w) {
+      auto src = warps[w].env.find(op.operands[0]), dst = warps[w].env.find(op.operands[1]);
+      if (src == warps[w].env.end() || dst == warps[w].env.end() || src->second.kind != Value::kTensor || !src->second.lazy ||
+          dst->second.kind != Value::kTensor || dst->second.lazy)
+        return false;
+      out[w] = dst->second.g;
+      const kapy_global &sg = src->second.g, &o = out[w], &o0 = out[0];
+      const char *ptr = (const char *)o.ptr;
+      if (ptr >= arena && ptr < arena + kArena) return false;  // (a shared or register tensor)
+      if (o.end0 - o.start0 != sg.end0 - sg.start0 || o.end1 - o.start1 != sg.end1 - sg.start1 || o.dtype != sg.dtype) return false;
+      if (o.ptr != o0.ptr || o.stride0 != o0.stride0 || o.stride1 != o0.stride1 || o.dtype != o0.dtype || o.alignment != o0.alignment ||
+          o.end0 - o.start0 != o0.end0 - o0.start0 || o.end1 - o.start1 != o0.end1 - o0.start1)
+        return false;
+    }
+    // the grid of tiles, from the result views
+    const int32_t R = out[0].end0 - out[0].start0, C = out[0].end1 - out[0].start1;
+    if (R <= 0 || C <= 0) return false;
+    int32_t o0 = out[0].start0, o1 = out[0].start1;
+    for (int w = 1; w < n; ++w) { o0 = std::min(o0, out[w].start0); o1 = std::min(o1, out[w].start1); }
+    std::vector<int32_t> a(n), b(n);
+    int32_t I = 0, J = 0;
+    std::set<std::pair<int32_t, int32_t>> tiles;
+    for (int w = 0; w < n; ++w) {
+      if ((out[w].start0 - o0) % R || (out[w].start1 - o1) % C) return false;
+      a[w] = (out[w].start0 - o0) / R;
+      b[w] = (out[w].start1 - o1) / C;
+      I = std::max(I, a[w] + 1);
+      J = std::max(J, b[w] + 1);
+      if (!tiles.insert({a[w], b[w]}).second) return false;
+    }
+    if ((int64_t)I * J != n) return false;
+    if ((int64_t)R * I > 0x7fffffff - o0 || (int64_t)C * J > 0x7fffffff - o1) return false;
+    // what a store does first: deferred values that still read the memory it writes are computed - once, for the union of the
+    // instances' views (all their stores stand at this point of the program); a source that this computes is no chain any more
+    kapy_global all = out[0];
+    all.start0 = o0; all.end0 = o0 + R * I;
+    all.start1 = o1; all.end1 = o1 + C * J;
+    // (register tensors made from here on come from the group's own region of the arena, which is never handed out twice
+    // while the group lives: no warp is swapped in, so no warp's share can be used)
+    struct Region {
+      Interp &in;
+      size_t top_was, limit_was;
+      explicit Region(Interp &i) : in(i), top_was(i.top), limit_was(i.limit) {
+        in.top = in.merged_top;
+        in.limit = in.merged_base + kMergedArena;
+      }
+      ~Region() {
+        in.merged_top = in.top;
+        in.top = top_was;
+        in.limit = limit_was;
+      }
+    } region(*this);
+    {
+      const std::string before = err;
+      if (settle_readers(op, all) != KAPY_OK) { err = before; return false; }  // (the instance's own run reports it)
+    }
+    for (int w = 0; w < n; ++w) {
+      auto src = warps[w].env.find(op.operands[0]);
+      if (!src->second.lazy) return false;
+      chain[w] = src->second.lazy;
+    }
+    // the leaves of every instance's chain, in one order
+    std::vector<std::vector<const Expr *>> leaves(n);
+    {
+      std::map<const Expr *, const Expr *> pairs;
+      if (!same_form(chain[0].get(), chain[0].get(), pairs, &leaves[0])) return false;
+    }
+    for (int w = 1; w < n; ++w) {
+      std::map<const Expr *, const Expr *> pairs;
+      if (!same_form(chain[0].get(), chain[w].get(), pairs, &leaves[w]) || leaves[w].size() != leaves[0].size()) return false;
+    }
+    // every leaf: with the tile along an axis, or of extent 1 and the same for all
+    struct Axis { int32_t origin; bool moves; };
+    std::vector<Axis> l0(leaves[0].size()), l1(leaves[0].size());
+    for (size_t k = 0; k < leaves[0].size(); ++k) {
+      const int32_t r = leaves[0][k]->leaf.end0 - leaves[0][k]->leaf.start0, c = leaves[0][k]->leaf.end1 - leaves[0][k]->leaf.start1;
+      int32_t m0 = leaves[0][k]->leaf.start0, m1 = leaves[0][k]->leaf.start1;
+      for (int w = 1; w < n; ++w) { m0 = std::min(m0, leaves[w][k]->leaf.start0); m1 = std::min(m1, leaves[w][k]->leaf.start1); }
+      bool moves0 = true, still0 = true, moves1 = true, still1 = true;
+      for (int w = 0; w < n; ++w) {
+        const int64_t d0 = leaves[w][k]->leaf.start0 - m0, d1 = leaves[w][k]->leaf.start1 - m1;
+        moves0 = moves0 && d0 == (int64_t)a[w] * r;
+        still0 = still0 && d0 == 0;
+        moves1 = moves1 && d1 == (int64_t)b[w] * c;
+        still1 = still1 && d1 == 0;
+      }
+      if (I > 1 ? !((moves0 && r == R) || (still0 && r == 1 && R != 1) || (R == 1 && r == 1 && (moves0 || still0))) : !still0) return false;
+      if (J > 1 ? !((moves1 && c == C) || (still1 && c == 1 && C != 1) || (C == 1 && c == 1 && (moves1 || still1))) : !still1) return false;
+      l0[k] = {m0, I > 1 && moves0 && !(still0)};
+      l1[k] = {m1, J > 1 && moves1 && !(still1)};
+      if ((int64_t)r * I > 0x7fffffff - m0 || (int64_t)c * J > 0x7fffffff - m1) return false;
+    }
+    // the union as one chain
+    std::map<const Expr *, std::shared_ptr<Expr>> made;
+    std::shared_ptr<Expr> whole = clone(chain[0], made);
+    for (size_t k = 0; k < leaves[0].size(); ++k) {
+      kapy_global &g = made[leaves[0][k]]->leaf;
+      const int32_t r = g.end0 - g.start0, c = g.end1 - g.start1;
+      g.start0 = l0[k].origin;
+      g.end0 = g.start0 + (l0[k].moves ? r * I : r);
+      g.start1 = l1[k].origin;
+      g.end1 = g.start1 + (l1[k].moves ? c * J : c);
+    }
+    for (auto &kv : made) {
+      Expr &e = *kv.second;
+      if (e.ew == KAPY_EW_ARANGE) return false;
+      if (is_reduce(e)) {
+        if ((e.axis == 1 && (J > 1 || e.rows != R)) || (e.axis == 0 && (I > 1 || e.cols != C)) || (e.axis != 0 && e.axis != 1)) return false;
+        if (e.axis == 1) e.rows *= I;
+        else e.cols *= J;
+      }
+    }
+    // run it from the group's own region of the arena (reduces that leave the program need register tensors of the union's size)
+    const std::string before = err;
+    const int rc = run_chain(op, whole, &all);
+    if (rc == KAPY_OK) { ++merged_calls; return true; }
+    err = before;  // refused as a whole: the instances run their own stores
+    return false;
+  }
+  int64_t merged_calls = 0;
 
   int run_ops(const std::vector<Op> &ops, std::vector<Value> *yielded) {
     for (const Op &op : ops) {
@@ -879,6 +1057,7 @@ struct Interp {
         if (rc != KAPY_OK) return rc;
         continue;
       }
+      if (merge && fuse && op.name == "kapy.st_global" && try_merged_store(op)) continue;
       for (int w = 0; w < W; ++w) {
         enter(w);
         int rc = run_op(op, yielded ? &(*yielded)[w] : nullptr);
@@ -1375,6 +1554,12 @@ extern "C" int kapy_analyze_mlir(const char *mlir_text, const char *func_name, i
   return KAPY_OK;
 }
 
+static std::atomic<int64_t> g_merged_calls{0};
+extern "C" int kapy_run_mlir_stats(int64_t *merged_stores) {
+  if (merged_stores) *merged_stores = g_merged_calls.load();
+  return KAPY_OK;
+}
+
 extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_arg *args, int32_t n_args, const int32_t grid[3],
                              void *stream) {
   if (!mlir_text || (n_args > 0 && !args) || !grid) return fail(KAPY_ERR_INVALID, "run_mlir: null argument");
@@ -1404,7 +1589,16 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   Interp in(f, (hipStream_t)stream);
   in.plan = &plan;
   if (const char *e = getenv("KAPY_MLIR_FUSE")) in.fuse = atoi(e) != 0;
-  KAPY_HIP_CHECK(hipMalloc((void **)&in.arena, kArena));
+  // The arena is allocated at the first call on a device and kept (a call used to pay an allocation and a release of its own,
+  // several milliseconds); calls take turns at it.
+  static std::mutex arena_mutex;
+  static char *arenas[16] = {};
+  std::lock_guard<std::mutex> arena_lock(arena_mutex);
+  int device = 0;
+  KAPY_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= 16) return fail(KAPY_ERR_UNSUPPORTED, "run_mlir: device ordinal %d beyond 16", device);
+  if (!arenas[device]) KAPY_HIP_CHECK(hipMalloc((void **)&arenas[device], kArena));
+  in.arena = arenas[device];
   rc = KAPY_OK;
   // KAPY_MLIR_IN_STEP=0: the warps of an instance run one after the other to the end instead of in step (the former way;
   // only right for programs whose warps do not exchange data through shared memory)
@@ -1423,35 +1617,62 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
     }
     return (int)KAPY_OK;
   };
-  for (int32_t p2 = 0; p2 < grid[2] && rc == KAPY_OK; ++p2)
-    for (int32_t p1 = 0; p1 < grid[1] && rc == KAPY_OK; ++p1)
-      for (int32_t p0 = 0; p0 < grid[0] && rc == KAPY_OK; ++p0) {
-        in.pid[0] = p0; in.pid[1] = p1; in.pid[2] = p2;
-        if (in_step) {
-          // register tensors of the previous instance are dead; shared tensors stay.  Every warp gets an equal share of the arena.
-          const size_t share = ((kArena - kSharedArena) / W) & ~size_t(255);
-          in.warps.assign(W, Interp::WarpState());
-          for (int w = 0; w < W && rc == KAPY_OK; ++w) {
-            in.warps[w].top = kSharedArena + w * share;
-            in.warps[w].limit = kSharedArena + (w + 1) * share;
-            rc = bind_args(in.warps[w].env);
-          }
-          in.env.clear();
-          if (rc == KAPY_OK) rc = in.run_ops_in_step(f.body, nullptr);
-          continue;
-        }
+  // KAPY_MLIR_BATCH=0: one program instance at a time (its warps in step), no call merged over instances
+  bool batch = true;
+  if (const char *e = getenv("KAPY_MLIR_BATCH")) batch = atoi(e) != 0;
+  in.merge = batch && in_step;
+  const int64_t programs = (int64_t)grid[0] * grid[1] * grid[2];
+  // programs per group: every warp of the group keeps at least kMinShare of the arena for its register tensors
+  int64_t per_group = 1;
+  if (batch && in_step) {
+    per_group = std::max<int64_t>(1, (int64_t)((kArena - kMergedArena) / (kSharedArena + (size_t)W * kMinShare)));
+    per_group = std::min(per_group, programs);
+  }
+  for (int64_t first = 0; first < programs && rc == KAPY_OK; first += per_group) {
+    const int64_t count = std::min(per_group, programs - first);
+    if (in_step) {
+      // register tensors of the previous group are dead.  Layout of the arena: the shared parts of the group's programs, the
+      // region of merged calls, then an equal share per warp.
+      in.register_base = (size_t)count * kSharedArena;
+      in.merged_base = in.merged_top = in.register_base;
+      const size_t shares_at = in.merged_base + kMergedArena;
+      const size_t share = ((kArena - shares_at) / (size_t)(count * W)) & ~size_t(255);
+      in.warps.assign((size_t)(count * W), Interp::WarpState());
+      for (int64_t g = 0; g < count && rc == KAPY_OK; ++g) {
+        const int64_t id = first + g;
         for (int w = 0; w < W && rc == KAPY_OK; ++w) {
-          in.warp = w;
-          in.env.clear();
-          in.top = kSharedArena;
-          in.limit = kArena;
-          rc = bind_args(in.env);
-          if (rc == KAPY_OK) rc = in.run_ops(f.body, nullptr);
+          Interp::WarpState &st = in.warps[(size_t)(g * W + w)];
+          st.pid[0] = id % grid[0];
+          st.pid[1] = id / grid[0] % grid[1];
+          st.pid[2] = id / ((int64_t)grid[0] * grid[1]);
+          st.warp = w;
+          st.shared_base = (size_t)g * kSharedArena;
+          st.top = shares_at + (size_t)(g * W + w) * share;
+          st.limit = st.top + share;
+          rc = bind_args(st.env);
         }
       }
-  // the arena is freed after the work on the stream has finished
+      in.env.clear();
+      if (rc == KAPY_OK) rc = in.run_ops_in_step(f.body, nullptr);
+      continue;
+    }
+    in.pid[0] = first % grid[0];
+    in.pid[1] = first / grid[0] % grid[1];
+    in.pid[2] = first / ((int64_t)grid[0] * grid[1]);
+    in.register_base = kSharedArena;
+    in.shared_base = 0;
+    for (int w = 0; w < W && rc == KAPY_OK; ++w) {
+      in.warp = w;
+      in.env.clear();
+      in.top = kSharedArena;
+      in.limit = kArena;
+      rc = bind_args(in.env);
+      if (rc == KAPY_OK) rc = in.run_ops(f.body, nullptr);
+    }
+  }
+  g_merged_calls.fetch_add(in.merged_calls, std::memory_order_relaxed);
+  // the next call may use the arena once the work on the stream has finished
   hipError_t e = hipStreamSynchronize((hipStream_t)stream);
-  (void)hipFree(in.arena);
   if (rc != KAPY_OK) return fail(rc, "run_mlir: %s", in.err.c_str());
   if (e != hipSuccess) return fail(KAPY_ERR_HIP, "run_mlir: %s", hipGetErrorString(e));
   return KAPY_OK;

@@ -37,7 +37,7 @@ EXPORTS = [
     "kapy_fragments_default", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
     "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_swizzle_search_gfx950", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
-    "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_parse_mlir",
+    "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_run_mlir_stats", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
     "kapy_matmul_workspace_bytes", "kapy_matmul_turn_workspace_bytes", "kapy_matmul_static_workspace",
@@ -203,6 +203,7 @@ def lib():
     L.kapy_smem_barriers.argtypes = [P(SmemOp), i32, P(SmemAccess), i32, P(i32), P(i32), i32, P(i32)]
     L.kapy_analyze_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i64), P(i32), P(i64), i32, P(i32), P(i32), i32]
     L.kapy_run_mlir.argtypes = [C.c_char_p, C.c_char_p, P(MlirArg), i32, i32 * 3, vp]
+    L.kapy_run_mlir_stats.argtypes = [P(i64)]
     L.kapy_parse_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i32), P(i32), P(i32)]
     for name in EXPORTS:
         f = getattr(L, name)
@@ -474,6 +475,13 @@ def run_mlir(text, args, grid, func_name=None, stream=None):
     g = list(grid) + [1] * (3 - len(grid))
     check(lib().kapy_run_mlir(text.encode(), func_name.encode() if func_name else None, arr, len(args), (C.c_int32 * 3)(*g),
                               stream if stream is not None else current_stream()))
+
+
+def run_mlir_stats():
+    """How many kapy.st_global ops this process has run as one call for all instances in flight."""
+    n = C.c_int64(0)
+    check(lib().kapy_run_mlir_stats(C.byref(n)))
+    return n.value
 
 
 def change(in_ptr, src, dst, shape, out_ptr, stream=None):

@@ -1,4 +1,4 @@
-"""Kapy-dialect programs in textual form, written for these tests in the op syntax of the reference's
+"""Kapy-dialect programs in textual form, written for the tests and the benchmark in the op syntax of the reference's
 fixtures (test/Conversion/KapyToKgpu/{elementwise_add,reduce_sum,matmul}.mlir; Ops.td): the same ops and
 the same program structure (per-warp sub-views, a shared-memory double buffer filled with
 cp_async_global_to_shared, ld_matrix fragments, an scf.for carrying the accumulator, arith.select choosing

@@ -204,8 +204,8 @@ def test_deferred_values_carried_by_a_loop(ko, monkeypatch):
 
 def test_fused_chain_is_one_kernel(ko):
     """With KAPY_EW_AUTO_SPECIALIZE=1 (read once per process, so in a process of its own) every program outside the hand-written
-    kernels is compiled when first seen: the chain of eleven ops leaves exactly one compiled kernel behind, launched once per
-    program instance and warp."""
+    kernels is compiled when first seen: the chain of eleven ops leaves exactly one compiled kernel behind, launched ONCE for all
+    program instances and warps (their tiles join into one view; KAPY_MLIR_BATCH=0: once per instance and warp)."""
     import os
     import subprocess
     import sys
@@ -221,7 +221,13 @@ x, y = ko.fill_normal(rows * cols, ko.F16, 61, std=2.0), ko.fill_normal(rows * c
 gate = np.linspace(0.25, 2.0, rows).astype(np.float32)
 dx, dy, dg, dout = to_dev(x), to_dev(y), to_dev(gate), dev_zeros(rows * cols, 2, fill=0x7e00)
 kh.run_mlir(kp.gated_program(rows_per_warp, cols, warps), [dx, dy, dg, dout, rows], [programs]); sync()
-assert kh.elementwise_specialize_stats() == (1, programs * warps), kh.elementwise_specialize_stats()
+assert kh.elementwise_specialize_stats() == (1, 1), kh.elementwise_specialize_stats()
+import os
+os.environ["KAPY_MLIR_BATCH"] = "0"
+d2 = dev_zeros(rows * cols, 2, fill=0x7e00)
+kh.run_mlir(kp.gated_program(rows_per_warp, cols, warps), [dx, dy, dg, d2, rows], [programs]); sync()
+assert kh.elementwise_specialize_stats() == (1, 1 + programs * warps), kh.elementwise_specialize_stats()
+assert np.array_equal(to_host(d2, np.uint16), to_host(dout, np.uint16))
 xf, yf = x.view(np.float16).astype(np.float64).reshape(rows, cols), y.view(np.float16).astype(np.float64).reshape(rows, cols)
 ref = xf / (1 + np.exp(-xf)) * yf * gate[:, None].astype(np.float64)
 got = to_host(dout, np.float16, (rows, cols)).astype(np.float64)
@@ -311,3 +317,47 @@ def test_column_softmax_program_matches_the_oracle_program(ko, monkeypatch, rows
     kh.run_mlir(kp.column_softmax_program(rows, cols_per_warp, warps), [dx, dout, cols], [programs])
     sync()
     assert ulp_diff_f16(to_host(dout, np.uint16), want).max() <= 2     # in f32, one rounding to f16 at the end
+
+
+def test_the_instances_of_a_grid_run_as_one_call_where_their_tiles_join(ko, monkeypatch):
+    """The fixture-shaped programs over a grid: all programs and warps in step, and every kapy.st_global whose chains have one form
+    and whose views tile a rectangle runs as ONE call over the union (counted by kapy_run_mlir_stats).  Results are bit for bit
+    those of running one instance at a time (KAPY_MLIR_BATCH=0), which the tests above compare with the oracle."""
+    def both(run, out_words, merged_stores):
+        outs = []
+        for batch in ("1", "0"):
+            monkeypatch.setenv("KAPY_MLIR_BATCH", batch)
+            dout = dev_zeros(out_words, 2, fill=0x7e00)
+            before = kh.run_mlir_stats()
+            run(dout)
+            sync()
+            assert kh.run_mlir_stats() - before == (merged_stores if batch == "1" else 0), batch
+            outs.append(to_host(dout, np.uint16))
+        assert np.array_equal(outs[0], outs[1])
+        return outs[0]
+
+    # x + y: 6 programs x 2 warps x [4 x 256] tiles stacked along the rows -> one elementwise call over [48 x 256]
+    rows_per_warp, cols, warps, programs = 4, 256, 2, 6
+    rows = rows_per_warp * warps * programs
+    x, y = ko.fill_normal(rows * cols, ko.F16, 11), ko.fill_normal(rows * cols, ko.F16, 12)
+    dx, dy = to_dev(x), to_dev(y)
+    got = both(lambda d: kh.run_mlir(kp.binary_program("arith.addf", rows_per_warp, cols, warps), [dx, dy, d, rows], [programs]), rows * cols, 1)
+    want = np.zeros(rows * cols, np.uint16)
+    prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_LD_GLOBAL, dst=1, a=1), dict(op=ko.EW_ADDF, dst=2, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=2)])
+    g = lambda a: ko.mk_global(a, rows, cols, cols, 1, ko.F16)
+    assert ko.elementwise(prog, [g(x), g(y)], g(want)) == 0
+    assert np.array_equal(got, want)
+    # the row sum of the fixture: the reduce of all instances as one kapy_reduce, its store as one copy
+    rows_per_warp, cols, warps, programs = 2, 256, 2, 8
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 21)
+    dx = to_dev(x)
+    both(lambda d: kh.run_mlir(kp.reduce_program("arith.addf", rows_per_warp, cols, warps), [dx, d, rows], [programs]), rows, 1)
+    # softmax (two reduces along the rows inside the chain): one row program over all rows of the grid
+    rows_per_warp, cols, warps, programs = 2, 256, 2, 5
+    rows = rows_per_warp * warps * programs
+    x = ko.fill_normal(rows * cols, ko.F16, 31)
+    dx = to_dev(x)
+    both(lambda d: kh.run_mlir(kp.softmax_program(rows_per_warp, cols, warps), [dx, d, rows], [programs]), rows * cols, 1)
+    # a causal mask (kapy.arange: values depend on where the tile lies): never merged
+    both(lambda d: kh.run_mlir(kp.causal_softmax_program(rows_per_warp, cols, warps), [dx, d, rows], [programs]), rows * cols, 0)

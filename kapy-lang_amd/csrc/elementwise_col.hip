@@ -86,9 +86,10 @@ __global__ __launch_bounds__(256) void col_softmax_stats_kernel(ColSoftmax p, in
           top = fmaxf(top, f[u][e]);   // (a NaN element is skipped here; its exp below makes the sum NaN, which marks the column)
         }
         float acc = s[e] * exp_f32(m[e] - top);
-        const float bias = -top * kLog2e;   // exp(x - top) as 2^(x * log2 e - top * log2 e): one fused multiply-add per element
+        // (the difference first: folding top * log2 e into a fused multiply-add would put that product's own rounding - half
+        // a unit in ITS last place, which for a top of 6e4 is 0.4 %, and another one per chunk - into every term)
 #pragma unroll
-        for (int u = 0; u < U; ++u) acc += __builtin_amdgcn_exp2f(__builtin_fmaf(f[u][e], kLog2e, bias));
+        for (int u = 0; u < U; ++u) acc += exp_f32(f[u][e] - top);
         s[e] = acc;
         m[e] = top;
       }
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(256) void col_softmax_apply_kernel(ColSoftmax p, in
   float M[8], R[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    M[e] = -p.stats[col0 + e] * kLog2e;   // exp(x - M) as 2^(x * log2 e - M * log2 e)
+    M[e] = p.stats[col0 + e];
     R[e] = __builtin_amdgcn_rcpf(p.stats[p.cols + col0 + e]);
   }
   const int32_t r_begin = blockIdx.y * rows_per_wg, r_end = min(p.rows, r_begin + rows_per_wg);
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(256) void col_softmax_apply_kernel(ColSoftmax p, in
       u32x4_t o;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        f[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[e], kLog2e, M[e])) * R[e];   // (S >= 1 and finite, or NaN, which 1 / S and the product hand on)
+        f[e] = exp_f32(f[e] - M[e]) * R[e];   // (S >= 1 and finite, or NaN, which 1 / S and the product hand on)
       }
 #pragma unroll
       for (int w = 0; w < 4; ++w) o[w] = BF16 ? pack2_bf16_rn(f[2 * w], f[2 * w + 1]) : pack2_f16_rn(f[2 * w], f[2 * w + 1]);

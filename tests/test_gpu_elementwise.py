@@ -672,3 +672,22 @@ def test_column_major_result_runs_as_the_transposed_problem(ko, dtype):
     sync()
     got = to_host(dout, np_t)
     assert np.array_equal(got[:m * n], want.view(np_t)) and np.all(got[m * n:] == got[-1]) and got[-1] != 0
+
+
+@pytest.mark.parametrize("dtype", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("axis", [1, 0])
+def test_softmax_of_large_magnitudes(ko, dtype, axis):
+    """Lines whose maximum is large (6e4 in f16, 1e6 and 3e38 in bf16) and whose other elements lie within a few units of it: the
+    exponent (x - max) * log2(e) must be formed from the difference - a product max * log2(e) of its own carries a rounding of
+    0.4 % (f16) to several per cent, or overflows - through the row kernels and the column kernels alike."""
+    m, n = (64, 2048) if axis == 1 else (2048, 64)
+    rng = np.random.default_rng(axis)
+    top = 60000.0 if dtype == kh.F16 else 1.0e6
+    x = (top - np.abs(rng.standard_normal((m, n))) * (16.0 if dtype == kh.F16 else 3.0e4)).astype(np.float32)
+    if dtype == kh.BF16:
+        line = (slice(None), 3) if axis == 0 else (3, slice(None))
+        x[line] = 3.0e38 - np.abs(rng.standard_normal(x[line].shape)) * 1.0e37     # max * log2(e) overflows fp32
+    bits = ko.fptofp(np.ascontiguousarray(x), ko.F32, dtype).reshape(m, n)
+    insts = kh.softmax_insts(dtype) if axis == 1 else _along_columns(kh.softmax_insts(dtype))
+    got, want = _run_prog(ko, insts, [bits], [dtype], dtype, m, n, in_shapes=[(m, n)])
+    _check_ulp(got, want, dtype)

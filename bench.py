@@ -48,7 +48,9 @@ class CheckFailed(Exception):
 def _events(fn, steps, warmup):
     """Run fn(i) untimed until the clock has settled, then warmup + steps times;
     return (wall ms per step, event ms per launch)."""
+    import gc
     import torch
+    gc.collect()   # (now, not between the warm-up and the timed steps: the device clock falls within a fraction of a second of idling)
     t0, i = time.perf_counter(), 0
     while time.perf_counter() - t0 < PREWARM_S:
         fn(i)
@@ -58,15 +60,29 @@ def _events(fn, steps, warmup):
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    for i in range(steps):
-        fn(i)
-    end.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return wall_ms, start.elapsed_time(end) / steps
+    # The launches are queued back to back between events; an event every fifth of the way, and the per-launch figure is the
+    # median of the fifths: a pause of the launching thread inside the timed region (the collector, a worker pool of a CPU leg
+    # winding down) once put a millisecond of idle queue into a 20-launch average of a 13 us kernel.  The wall clock is over all
+    # steps, pauses included.
+    parts = 5 if steps >= 10 else 1
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(parts + 1)]
+    at = [steps * k // parts for k in range(parts + 1)]
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        marks[0].record()
+        k = 1
+        for i in range(steps):
+            fn(i)
+            if i + 1 == at[k]:
+                marks[k].record()
+                k += 1
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        gc.enable()
+    per_launch = sorted(marks[k].elapsed_time(marks[k + 1]) / (at[k + 1] - at[k]) for k in range(parts))
+    return wall_ms, per_launch[parts // 2]
 
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by what the same counter reads

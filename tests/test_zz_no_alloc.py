@@ -80,3 +80,21 @@ def test_static_workspace_under_graph_capture_replays_the_eager_bits(ko):
         assert torch.equal(out, eager), rep
         kh.matmul(g_small, g_small_b, dglobal(other, 256, 256, 256, 1, kh.F16), tile=(128, 128, 64), split_k=4, static_workspace=True)
         sync()
+
+
+def test_static_workspace_calls_leave_the_device_memory_as_it_was(ko):
+    """After a first call (the runtime loads the kernels' code on first use), calls through the entry point change nothing
+    about how much device memory is free: nothing is allocated and nothing released."""
+    M, N, K, dt = 256, 384, 4096, kh.F16
+    da, db = to_dev(ko.fill_uniform(M * K, dt, 7, 0)), to_dev(ko.fill_uniform(K * N, dt, 7, 1))
+    ga, gb = dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt)
+    out = dev_zeros(M * N, 2)
+    go = dglobal(out, M, N, N, 1, dt)
+    for split in (8, 0):
+        kh.matmul(ga, gb, go, tile=(128, 128, 64), split_k=split, static_workspace=True)
+    sync()
+    free_before = torch.cuda.mem_get_info()[0]
+    for rep in range(20):
+        kh.matmul(ga, gb, go, tile=(128, 128, 64), split_k=8 if rep % 2 else 0, static_workspace=True)
+    sync()
+    assert torch.cuda.mem_get_info()[0] == free_before

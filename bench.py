@@ -25,6 +25,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -1053,8 +1054,8 @@ def pmc_summary(fetch_csv, write_csv):
 
     out = ["rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, all bench workloads, one MI355X (gfx950)", "",
            "commands (two runs, one counter each; from the repository root after `cd /tmp && export TMPDIR=/tmp && cd <repo>`):",
-           "  rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof/pmc_fetch -o pmc_fetch --output-format csv -- python3 bench.py --no-cpu --skip ceilings --steps 3 --warmup 1",
-           "  rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof/pmc_write -o pmc_write --output-format csv -- python3 bench.py --no-cpu --skip ceilings --steps 3 --warmup 1",
+           "  rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof/pmc_fetch -o pmc_fetch --output-format csv -- python3 bench.py --no-cpu --skip ceilings,mlir_fixtures --steps 3 --warmup 1",
+           "  rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof/pmc_write -o pmc_write --output-format csv -- python3 bench.py --no-cpu --skip ceilings,mlir_fixtures --steps 3 --warmup 1",
            "  python3 bench.py --pmc-summary <pmc_fetch counter_collection.csv> <pmc_write counter_collection.csv> > profiles/bench_all_workloads.hbm_traffic_pmc.txt",
            "", "Per-dispatch mean of the counter (rocprofv3 reports KiB), by kernel and grid size (work-items); n = dispatches seen.", "",
            "%-86s %10s %20s %20s" % ("kernel", "grid", "FETCH_SIZE (n)", "WRITE_SIZE (n)")]
@@ -1088,6 +1089,70 @@ def pmc_summary(fetch_csv, write_csv):
     print("\n".join(out))
 
 
+def stats_summary(stats_csv):
+    """The tracked per-kernel summary from a rocprofv3 --kernel-trace --stats run of this script: this library's kernels (and the
+    kernels it compiled at run time), calls, average, minimum and maximum duration in nanoseconds, by total time."""
+    import csv
+    import subprocess
+    rows = [r for r in csv.DictReader(open(stats_csv)) if "kapy" in r["Name"]]
+    tool = "/opt/rocm/llvm/bin/llvm-cxxfilt" if os.path.exists("/opt/rocm/llvm/bin/llvm-cxxfilt") else "c++filt"
+    try:
+        names = subprocess.run([tool], input="\n".join(r["Name"] for r in rows), capture_output=True, text=True).stdout.split("\n")
+    except OSError:
+        names = [r["Name"] for r in rows]
+    def short(n):
+        m = re.match(r"_ZN4kapy12_GLOBAL__N_1(\d+)", n)            # names with _Float16 arguments come back mangled
+        if m:
+            rest = n[m.end():]
+            return rest[:int(m.group(1))] + "<" + rest[int(m.group(1)) + 1:].split("EEv")[0] + "> (mangled arguments)"
+        return n.replace("void ", "").replace("kapy::(anonymous namespace)::", "").replace("kapy::", "").split("(")[0]
+    out = ["rocprofv3 kernel statistics, all bench workloads, one MI355X (gfx950)", "",
+           "commands (from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd <repo>`):",
+           "  rocprofv3 --kernel-trace --stats -d gpurun_out/prof/stats_all -o stats_all --output-format csv -- python3 bench.py --no-cpu --skip ceilings",
+           "  python3 bench.py --stats-summary <stats_all_kernel_stats.csv> > profiles/bench_all_workloads.kernel_stats.txt", "",
+           "Rows of this library's kernels (torch's fill / compare kernels omitted).  Calls include the untimed clock pre-warm launches of",
+           "bench.py.  kapy_ew_flat_* / kapy_ew_rows_* are the kernels kapy_elementwise compiled at run time in that process (the name ends in",
+           "a hash of program and operand signature).  tn_kernel<..., true> (last argument) is the build with the fused tail.", "",
+           "%-96s %8s %12s %10s %10s" % ("kernel", "calls", "avg_ns", "min_ns", "max_ns")]
+    for r, n in sorted(zip(rows, names), key=lambda rn: -float(rn[0]["TotalDurationNs"])):
+        out.append("%-96s %8d %12.0f %10d %10d" % (short(n)[:96], int(r["Calls"]), float(r["AverageNs"]), int(float(r["MinNs"])), int(float(r["MaxNs"]))))
+    print("\n".join(out))
+
+
+def ceilings_summary(bench_json):
+    """The tracked summary of the probe kernels' figures from the JSON line of `bench.py --workload ceilings --no-others`."""
+    line = json.loads(open(bench_json).read().strip().split("\n")[-1])
+    res = next((r for r in [line.get("config", {})] + line.get("other_workloads", []) if "mfma" in r), None)
+    if res is None:
+        res = line
+    out = ["Device ceilings measured by the probe library's kernels (libkapy_probe.so) and the tiled GEMMs' fixed cost per launch, one MI355X (gfx950)", "",
+           "commands (from the repository root):",
+           "  python3 bench.py --no-cpu --no-others --workload ceilings > gpurun_out/ceilings.json",
+           "  python3 bench.py --ceilings-summary gpurun_out/ceilings.json > profiles/device_ceilings.probe_kernels.txt", "",
+           "bench.py's figures in that run (HIP events around back-to-back launches; the shader clock is what the kernel itself reads: s_memtime",
+           "ticks of one wave against the 100 MHz s_memrealtime over the same interval)."]
+
+    def dump(d, indent):
+        for k, v in d.items():
+            if isinstance(v, dict):
+                out.append("%s%s:" % (" " * indent, k))
+                dump(v, indent + 2)
+            else:
+                out.append("%s%-*s %s" % (" " * indent, max(4, 96 - indent), k, v))
+
+    for key, title in (("mfma", "matrix instruction loop (every CU: 4 waves of independent matrix instructions on registers, no memory traffic)"),
+                       ("copy", "plain copy of 128 MiB to another 128 MiB buffer, GB/s read + written (vecN = 16-byte vectors per lane and step, ntld / ntst = non-temporal loads / stores)"),
+                       ("read", "read-only stream of 64 MiB buffers in rotation, GB/s"), ("l2_read_tbs", "reads of a window that stays in the XCD's L2 / the Infinity Cache / neither, TB/s"),
+                       ("issue_tflops", "matrix instructions with fillers in the gaps behind them, TFLOP/s"), ("gemm_fixed_cost", "the tiled GEMMs at K and 2K")):
+        if key in res:
+            out += ["", title]
+            dump(res[key], 2)
+    for key in ("copy_best_gbs", "copy_best_frac_of_peak", "read_best_gbs", "read_best_frac_of_peak"):
+        if key in res:
+            out.append("%-40s %s" % (key, res[key]))
+    print("\n".join(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -1098,9 +1163,17 @@ def main():
     ap.add_argument("--skip", default="", help="comma-separated workloads to leave out of the other workloads (e.g. ceilings, whose probe launches reuse the GEMM kernels at other sizes and would mix into a profiler's per-kernel averages)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), help="no measurement: write the HBM-traffic summary that `traffic` is read from, from the counter_collection.csv files of two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE)")
+    ap.add_argument("--stats-summary", metavar="STATS_CSV", help="no measurement: the per-kernel summary kept under profiles/, from the kernel_stats.csv of a rocprofv3 --kernel-trace --stats run of this script")
+    ap.add_argument("--ceilings-summary", metavar="BENCH_JSON", help="no measurement: the summary of the probe kernels' figures kept under profiles/, from the JSON line of --workload ceilings")
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
+        return
+    if args.stats_summary:
+        stats_summary(args.stats_summary)
+        return
+    if args.ceilings_summary:
+        ceilings_summary(args.ceilings_summary)
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (every path here runs on a single MI355X)" % args.gpus)

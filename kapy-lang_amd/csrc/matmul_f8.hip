@@ -317,9 +317,12 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
 // 16*RG rows, so at N = 8192 there is one workgroup per CU, every weight byte crosses the fabric once, and the activation
 // (M x K bytes, L2-resident) is read N/32 times.  Its 4 waves split K and work alone on private rings of kBlockStages
 // stages; a stage is one 128-byte K step: 32 weight rows and 16*RG activation rows of 128 contiguous bytes, brought in by
-// LDS-direct loads of 8 rows each, 16-byte chunk c of row r stored at chunk c ^ ((r / 2) % 8) - the 16 rows a
-// quarter-wave reads then cover all 64 banks once.  RG x 2 accumulator blocks per wave; the four K ranges meet in LDS.
+// LDS-direct loads of 8 rows each, 16-byte chunk c of row r stored at chunk c ^ block_key(r % 16) - the 16 lanes of a
+// read phase then cover all 64 banks once.  RG x 2 accumulator blocks per wave; the four K ranges meet in LDS.
 constexpr int kBlockStep = 128, kBlockCols = 32;
+// (the lanes of one phase of a 16-byte LDS read are 0-3, 12-15, 20-23, 24-27 and so on: rows r16 = 0-3 and 12-15 of one K
+// group with rows 4-11 of the next; with this key they fall into 16 different groups of four banks)
+__device__ __forceinline__ constexpr int block_key(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 constexpr int block_stages(int) { return 3; }  // (four for 32 rows fits the LDS too and measured no faster)
 constexpr int waitcnt_vm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }  // s_waitcnt vmcnt(n), nothing else waited for
 template <int A_FMT, int B_FMT, int RG>
@@ -349,12 +352,12 @@ __global__ __launch_bounds__(256) void skinny_block_kernel(F8Params p) {
   uint32_t w_off[kLoadsW], a_off[kLoadsA];
 #pragma unroll
   for (int i = 0; i < kLoadsW; ++i) {
-    const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+    const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ block_key(r);
     w_off[i] = (uint32_t)(min(r, p.N - 1 - n0) * p.b_sn + c * 16);
   }
 #pragma unroll
   for (int i = 0; i < kLoadsA; ++i) {
-    const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ ((r >> 1) & 7);
+    const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ block_key(r);
     a_off[i] = (uint32_t)(min(r, p.M - 1 - m0) * p.a_sm + c * 16);
   }
   const bool w_once = row_blocks == 1;  // (see the streaming kernel: non-temporal loads for a weight read once)
@@ -374,7 +377,7 @@ __global__ __launch_bounds__(256) void skinny_block_kernel(F8Params p) {
   const int r16 = frag_at.row, grp = frag_at.k0 / kF8Shape.kpack;
   uint32_t rd[2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) rd[h] = (uint32_t)(r16 * kBlockStep + (((2 * grp + h) ^ ((r16 >> 1) & 7)) * 16));
+  for (int h = 0; h < 2; ++h) rd[h] = (uint32_t)(r16 * kBlockStep + (((2 * grp + h) ^ block_key(r16)) * 16));
   f32x4 acc[RG][2];
 #pragma unroll
   for (int r = 0; r < RG; ++r)

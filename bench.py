@@ -784,8 +784,9 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
 def bench_mlir(kh, steps, warmup, cpu):
     """The reference's three fixture programs (elementwise add, row sum, matmul; test/Conversion/KapyToKgpu/*.mlir) in the op syntax of
     kapy_programs.py, run through kapy_run_mlir on grids of program instances: per program the time of one call with the
-    instances' stores merged into one call each (the default) and with one instance at a time (KAPY_MLIR_BATCH=0).  A call
-    parses the text, allocates and frees its arena and synchronises: the figures are those of a validation path."""
+    instances' stores merged into one call each and with one instance at a time (KAPY_MLIR_BATCH=0), both parsed and
+    interpreted at every call (KAPY_MLIR_PLAN=0), and as the default does it: the device calls of the first run kept and made
+    again.  A call synchronises its stream: the figures are those of a validation path."""
     import numpy as np
     import torch
     import ko
@@ -807,16 +808,21 @@ def bench_mlir(kh, steps, warmup, cpu):
     for name, text, args, grid, target, nbytes in cases:
         row = {}
         results = []
-        for label, env in (("instances merged", "1"), ("one instance at a time", "0")):
+        for label, env, plan in (("instances merged", "1", "0"), ("one instance at a time", "0", "0"), ("instances merged, calls replayed", "1", "1")):
             os.environ["KAPY_MLIR_BATCH"] = env
+            os.environ["KAPY_MLIR_PLAN"] = plan
             target.zero_()
             before = kh.run_mlir_stats()
             kh.run_mlir(text, args, grid)
             torch.cuda.synchronize()
             row[label + ", merged stores per call"] = kh.run_mlir_stats() - before
+            if plan == "1":                      # the result compared is that of a replayed call
+                target.zero_()
+                kh.run_mlir(text, args, grid)
+                torch.cuda.synchronize()
             results.append(target.clone())
             t0 = time.perf_counter()
-            reps = 3
+            reps = 3 if plan == "0" else 10
             for _ in range(reps):
                 kh.run_mlir(text, args, grid)
             torch.cuda.synchronize()
@@ -825,15 +831,17 @@ def bench_mlir(kh, steps, warmup, cpu):
             if nbytes:
                 row[label + ", GB/s"] = round(nbytes / (ms * 1e-3) / 1e9, 2)
         os.environ.pop("KAPY_MLIR_BATCH", None)
-        if not torch.equal(results[0], results[1]):
+        os.environ.pop("KAPY_MLIR_PLAN", None)
+        if not (torch.equal(results[0], results[1]) and torch.equal(results[0], results[2])):
             checked = False
         out["programs"][name] = row
     if not checked:
-        raise CheckFailed("run_mlir: merged and per-instance runs differ")
+        raise CheckFailed("run_mlir: merged, per-instance and replayed runs differ")
     first = out["programs"][cases[0][0]]
-    out.update({"value": first["instances merged, GB/s"], "ms_per_step": first["instances merged, ms per call"], "kernel_ms": first["instances merged, ms per call"],
-                "checked": True, "check": "merged and per-instance runs give the same bits (the programs themselves are compared with the checker in the GPU tests)",
-                "roofline": _roof_hbm(cases[0][5], first["instances merged, ms per call"], None)})
+    key = "instances merged, calls replayed"
+    out.update({"value": first[key + ", GB/s"], "ms_per_step": first[key + ", ms per call"], "kernel_ms": first[key + ", ms per call"],
+                "checked": True, "check": "merged, per-instance and replayed runs give the same bits (the programs themselves are compared with the checker in the GPU tests)",
+                "roofline": _roof_hbm(cases[0][5], first[key + ", ms per call"], None)})
     return out
 
 

@@ -497,7 +497,11 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * its parent is an error.  func_name NULL = the first function of the module.  The first call on a device allocates
  * a 256 MiB arena for shared-memory and register tensors, which the library keeps until the process ends; calls take
  * turns at it, and a call synchronises `stream` before it returns: it is a way to run the reference's programs against
- * this library, not a fast path. */
+ * this library, not a fast path.
+ * The device calls of a run that succeeded are kept (the last 16 runs): a later call with the same text, function name,
+ * grid, argument values (every field of every kapy_mlir_arg), device and KAPY_MLIR_* modes makes the same calls again
+ * without parsing or interpreting - which calls a run makes cannot depend on the tensors' contents.  KAPY_MLIR_PLAN=0 in
+ * the environment turns that off. */
 typedef struct kapy_mlir_arg {
   void *ptr;      /* device pointer, for a !kapy.ptr<1> argument                    */
   int64_t bytes;  /* size of the allocation behind ptr; 0 = unknown (no range check) */
@@ -509,6 +513,9 @@ int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_
 /* How many kapy.st_global ops this process has run as ONE call for all program instances and warps in flight (the instances'
  * chains had the same form and their views tiled a rectangle): lets a caller check that a program took that path. */
 int kapy_run_mlir_stats(int64_t *merged_stores);
+/* How many runs this process has kept the calls of, and how many calls of kapy_run_mlir were served from a kept run
+ * (either pointer may be NULL). */
+int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays);
 /* The parsing half of kapy_run_mlir, without a device: KAPY_ERR_INVALID for text that does not parse,
  * KAPY_ERR_UNSUPPORTED for an op outside the set above; otherwise the function's argument count, its number
  * of ops (loop bodies included) and the module's kapy.num_warps.  Out pointers may be NULL. */

@@ -25,6 +25,7 @@
 #include <algorithm>
 #include <atomic>
 #include <climits>
+#include <deque>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -562,6 +563,20 @@ struct Value {
 // has its own shared part, the group one region for the register tensors of calls merged over instances, every warp its share.
 constexpr size_t kSharedArena = size_t(256) << 10, kArena = size_t(256) << 20, kMergedArena = size_t(64) << 20, kMinShare = size_t(1) << 20;
 
+// A device call of a run, as recorded for the plan cache: which entry point, and copies of everything it was given.
+struct PlannedCall {
+  enum Kind { kCopy, kElementwise, kReduce, kReduceEx, kMatmul } kind;
+  kapy_global g[4];
+  bool has[4] = {false, false, false, false};
+  kapy_copy_cfg copy_cfg;
+  kapy_matmul_cfg matmul_cfg;
+  kapy_reduce_cfg reduce_cfg;
+  bool has_cfg = false;
+  int32_t axis = 0, reduce_kind = 0;
+  std::vector<kapy_ew_inst> prog;
+  std::vector<kapy_global> ins;
+};
+
 struct Interp {
   const Func &f;
   hipStream_t stream;
@@ -732,7 +747,7 @@ struct Interp {
     if (!ptr) return fail_op(op, "register tensors of one program instance exceed the arena");
     kapy_global g;
     rc = lib(op, kapy_mk_global(&g, ptr, 0, kept0, kept1, kept1, 1, r->operand_dtype, 256));
-    if (rc == KAPY_OK) rc = lib(op, kapy_reduce(&operand.g, &g, r->axis, r->ew == KAPY_EW_REDUCE_MAX ? 1 : 0, stream));
+    if (rc == KAPY_OK) rc = lib(op, do_reduce(&operand.g, &g, r->axis, r->ew == KAPY_EW_REDUCE_MAX ? 1 : 0));
     if (rc != KAPY_OK) return rc;
     r->ew = KAPY_EW_LD_GLOBAL;
     r->n_in = 0;
@@ -745,7 +760,7 @@ struct Interp {
     const int r = emit(e, m);
     if (!m.ok) return fail(KAPY_ERR_UNSUPPORTED, "the deferred chain does not fit one program");
     m.prog[m.n++] = {KAPY_EW_ST_GLOBAL, 0, r, 0, 0, 0, KAPY_RN, 0.f};
-    return kapy_elementwise(m.prog, m.n, m.ins, m.n_ins, out, stream);
+    return do_elementwise(m.prog, m.n, m.ins, m.n_ins, out);
   }
   // the chain as one program that stores into `out`.  Reduces stay inside the program when its result has their
   // operand's shape (the row programs of kapy_elementwise: softmax, normalisations); the others, and all of them
@@ -779,7 +794,7 @@ struct Interp {
     int rc = lib(op, kapy_mk_global(&g, ptr, 0, rows, cols, cols, 1, v.g.dtype, 256));
     if (rc == KAPY_OK) {
       // a deferred load by itself is the copy kapy.ld_global always was (any element type, any strides)
-      if (v.lazy->ew == KAPY_EW_LD_GLOBAL && v.lazy->n_in == 0) rc = lib(op, kapy_copy(&v.lazy->leaf, &g, nullptr, stream));
+      if (v.lazy->ew == KAPY_EW_LD_GLOBAL && v.lazy->n_in == 0) rc = lib(op, do_copy(&v.lazy->leaf, &g, nullptr));
       else rc = lib(op, run_chain(op, v.lazy, &g));
     }
     if (rc != KAPY_OK) return rc;
@@ -866,6 +881,67 @@ struct Interp {
     return fail_op(op, "no shared-memory plan for this tensor");
   }
   int lib(const Op &op, int rc) { return rc == KAPY_OK ? KAPY_OK : (fail_op(op, kapy_last_error()), rc); }
+
+  // The device calls of the run.  With `record` set every call that succeeded is kept, with copies of its arguments: a later
+  // run of the same program on the same arguments makes the same calls (nothing in a program can read a tensor's data into
+  // a scalar, so which calls a run makes depends on the text, the grid and the argument values alone).
+  std::vector<PlannedCall> *record = nullptr;
+  int do_copy(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg) {
+    int rc = kapy_copy(src, dst, cfg, stream);
+    if (rc == KAPY_OK && record) {
+      record->emplace_back();
+      PlannedCall &c = record->back();
+      c.kind = PlannedCall::kCopy;
+      c.g[0] = *src; c.g[1] = *dst;
+      if (cfg) { c.copy_cfg = *cfg; c.has_cfg = true; }
+    }
+    return rc;
+  }
+  int do_elementwise(const kapy_ew_inst *prog, int32_t n, const kapy_global *const *ins, int32_t n_ins, const kapy_global *out) {
+    int rc = kapy_elementwise(prog, n, ins, n_ins, out, stream);
+    if (rc == KAPY_OK && record) {
+      record->emplace_back();
+      PlannedCall &c = record->back();
+      c.kind = PlannedCall::kElementwise;
+      c.prog.assign(prog, prog + n);
+      for (int i = 0; i < n_ins; ++i) c.ins.push_back(*ins[i]);
+      c.g[0] = *out;
+    }
+    return rc;
+  }
+  int do_reduce(const kapy_global *src, const kapy_global *dst, int32_t axis, int32_t kind) {
+    int rc = kapy_reduce(src, dst, axis, kind, stream);
+    if (rc == KAPY_OK && record) {
+      record->emplace_back();
+      PlannedCall &c = record->back();
+      c.kind = PlannedCall::kReduce;
+      c.g[0] = *src; c.g[1] = *dst; c.axis = axis; c.reduce_kind = kind;
+    }
+    return rc;
+  }
+  int do_reduce_ex(const kapy_global *src, const kapy_global *dst, int32_t axis, const kapy_reduce_cfg *cfg) {
+    int rc = kapy_reduce_ex(src, dst, axis, cfg, stream);
+    if (rc == KAPY_OK && record) {
+      record->emplace_back();
+      PlannedCall &c = record->back();
+      c.kind = PlannedCall::kReduceEx;
+      c.g[0] = *src; c.g[1] = *dst; c.axis = axis;
+      if (cfg) { c.reduce_cfg = *cfg; c.has_cfg = true; }
+    }
+    return rc;
+  }
+  int do_matmul(const kapy_global *a, const kapy_global *b, const kapy_global *acc, const kapy_global *r, const kapy_matmul_cfg *cfg) {
+    int rc = kapy_matmul(a, b, acc, r, cfg, stream);
+    if (rc == KAPY_OK && record) {
+      record->emplace_back();
+      PlannedCall &c = record->back();
+      c.kind = PlannedCall::kMatmul;
+      c.g[0] = *a; c.g[1] = *b; c.g[3] = *r;
+      if (acc) { c.g[2] = *acc; c.has[2] = true; }
+      if (cfg) { c.matmul_cfg = *cfg; c.has_cfg = true; }
+    }
+    return rc;
+  }
 
   int binary_tensor(const Op &op, int ew) { return defer(op, 2, ew, 0, KAPY_RN, 0.f); }
 
@@ -1272,7 +1348,7 @@ struct Interp {
       kapy_copy_cfg cfg;
       memset(&cfg, 0, sizeof cfg);
       cfg.transpose = 1;
-      int rc = lib(op, kapy_copy(&a.g, &r.g, &cfg, stream));
+      int rc = lib(op, do_copy(&a.g, &r.g, &cfg));
       if (rc) return rc;
       env[op.results[0]] = r;
       return KAPY_OK;
@@ -1334,7 +1410,7 @@ struct Interp {
     }
     if (n == "kapy.ld_global" || n == "kapy.ld_matrix" || n == "kapy.ld_shared") {
       if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
-      int rc = lib(op, kapy_copy(&a.g, &r.g, nullptr, stream));
+      int rc = lib(op, do_copy(&a.g, &r.g, nullptr));
       if (rc) return rc;
       env[op.results[0]] = r;
       return KAPY_OK;
@@ -1358,7 +1434,7 @@ struct Interp {
         }
       }
       if (!get(op, 0, Value::kTensor, a) || !get(op, 1, Value::kTensor, b)) return KAPY_ERR_INVALID;
-      return lib(op, kapy_copy(&a.g, &b.g, nullptr, stream));
+      return lib(op, do_copy(&a.g, &b.g, nullptr));
     }
     if (n == "kapy.cp_async_wait_group" || n == "nvvm.barrier0") return KAPY_OK;  // every op is complete in stream order
     if (n == "kapy.matmul") {
@@ -1376,7 +1452,7 @@ struct Interp {
       const char *matmul_mode = getenv("KAPY_MLIR_MATMUL");
       if (matmul_mode && std::string(matmul_mode) == "reference" && a.g.dtype == KAPY_F16 && b.g.dtype == KAPY_F16 && c.g.dtype == KAPY_F16 && r.g.dtype == KAPY_F16)
         cfg.accumulate = KAPY_ACCUMULATE_ELEMENT;
-      int rc = lib(op, kapy_matmul(&a.g, &b.g, &c.g, &r.g, &cfg, stream));
+      int rc = lib(op, do_matmul(&a.g, &b.g, &c.g, &r.g, &cfg));
       if (rc) return rc;
       env[op.results[0]] = r;
       return KAPY_OK;
@@ -1429,7 +1505,7 @@ struct Interp {
       }
       if (!get(op, 0, Value::kTensor, a) || op.types.empty() || !new_tensor(op, op.types.back(), r)) return KAPY_ERR_INVALID;
       kapy_reduce_cfg rcfg = {kind, reference ? KAPY_REDUCE_REFERENCE : KAPY_REDUCE_WIDE, nullptr, nullptr, 0};
-      int rc = lib(op, kapy_reduce_ex(&a.g, &r.g, axis, &rcfg, stream));
+      int rc = lib(op, do_reduce_ex(&a.g, &r.g, axis, &rcfg));
       if (rc) return rc;
       env[op.results[0]] = r;
       return KAPY_OK;
@@ -1554,15 +1630,99 @@ extern "C" int kapy_analyze_mlir(const char *mlir_text, const char *func_name, i
   return KAPY_OK;
 }
 
-static std::atomic<int64_t> g_merged_calls{0};
+static std::atomic<int64_t> g_merged_calls{0}, g_plans{0}, g_replays{0};
 extern "C" int kapy_run_mlir_stats(int64_t *merged_stores) {
   if (merged_stores) *merged_stores = g_merged_calls.load();
   return KAPY_OK;
 }
+extern "C" int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays) {
+  if (plans) *plans = g_plans.load();
+  if (replays) *replays = g_replays.load();
+  return KAPY_OK;
+}
+
+// The plan cache: the device calls of a run that succeeded, kept under everything that decides them - the text, the function,
+// the grid, the argument values, the device and the modes read from the environment.  A later call with the same key makes
+// those calls again without parsing or interpreting anything (the register tensors they name live in the device's arena, which
+// is kept for the life of the process and laid out the same way every time).
+namespace {
+struct Plan {
+  std::string key;
+  std::vector<PlannedCall> calls;
+  int64_t merged = 0;
+};
+constexpr size_t kMaxPlans = 16, kMaxPlannedCalls = 1u << 20;
+std::deque<std::shared_ptr<Plan>> g_plan_cache;  // (guarded by the arena's mutex: calls take turns anyway)
+
+std::string plan_key(const char *text, const char *func, const kapy_mlir_arg *args, int32_t n_args, const int32_t grid[3], int device) {
+  std::string k(text);
+  k.push_back('\0');
+  if (func) k += func;
+  k.push_back('\0');
+  k.append((const char *)grid, 3 * sizeof(int32_t));
+  k.append((const char *)&device, sizeof device);
+  for (int i = 0; i < n_args; ++i) {
+    // (field by field: the padding of the struct is not part of the key)
+    k.append((const char *)&args[i].ptr, sizeof args[i].ptr);
+    k.append((const char *)&args[i].bytes, sizeof args[i].bytes);
+    k.append((const char *)&args[i].i32, sizeof args[i].i32);
+  }
+  for (const char *name : {"KAPY_MLIR_FUSE", "KAPY_MLIR_IN_STEP", "KAPY_MLIR_BATCH", "KAPY_MLIR_MATMUL", "KAPY_MLIR_REDUCE"}) {
+    const char *v = getenv(name);
+    k += v ? v : "";
+    k.push_back('\0');
+  }
+  return k;
+}
+
+int replay_plan(const Plan &plan, hipStream_t stream) {
+  std::vector<const kapy_global *> ins;
+  for (const PlannedCall &c : plan.calls) {
+    int rc = KAPY_OK;
+    switch (c.kind) {
+      case PlannedCall::kCopy: rc = kapy_copy(&c.g[0], &c.g[1], c.has_cfg ? &c.copy_cfg : nullptr, stream); break;
+      case PlannedCall::kElementwise:
+        ins.clear();
+        for (const kapy_global &g : c.ins) ins.push_back(&g);
+        rc = kapy_elementwise(c.prog.data(), (int32_t)c.prog.size(), ins.data(), (int32_t)ins.size(), &c.g[0], stream);
+        break;
+      case PlannedCall::kReduce: rc = kapy_reduce(&c.g[0], &c.g[1], c.axis, c.reduce_kind, stream); break;
+      case PlannedCall::kReduceEx: rc = kapy_reduce_ex(&c.g[0], &c.g[1], c.axis, c.has_cfg ? &c.reduce_cfg : nullptr, stream); break;
+      case PlannedCall::kMatmul: rc = kapy_matmul(&c.g[0], &c.g[1], c.has[2] ? &c.g[2] : nullptr, &c.g[3], c.has_cfg ? &c.matmul_cfg : nullptr, stream); break;
+    }
+    if (rc != KAPY_OK) return rc;
+  }
+  return KAPY_OK;
+}
+}  // namespace
 
 extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_arg *args, int32_t n_args, const int32_t grid[3],
                              void *stream) {
   if (!mlir_text || (n_args > 0 && !args) || !grid) return fail(KAPY_ERR_INVALID, "run_mlir: null argument");
+  // The arena is allocated at the first call on a device and kept (a call used to pay an allocation and a release of its own,
+  // several milliseconds); calls take turns at it.
+  static std::mutex arena_mutex;
+  static char *arenas[16] = {};
+  std::lock_guard<std::mutex> arena_lock(arena_mutex);
+  // KAPY_MLIR_PLAN=0: every call parses and interprets the text again
+  bool use_plans = true;
+  if (const char *e = getenv("KAPY_MLIR_PLAN")) use_plans = atoi(e) != 0;
+  if (use_plans && !g_plan_cache.empty()) {  // (a kept run means a device has been in use: nothing here is a call's first touch of it)
+    int device = 0;
+    KAPY_HIP_CHECK(hipGetDevice(&device));
+    const std::string key = plan_key(mlir_text, func_name, args, n_args, grid, device);
+    for (const std::shared_ptr<Plan> &plan : g_plan_cache)
+      if (plan->key == key) {
+        int rc = replay_plan(*plan, (hipStream_t)stream);
+        g_merged_calls.fetch_add(plan->merged, std::memory_order_relaxed);
+        g_replays.fetch_add(1, std::memory_order_relaxed);
+        // the next call may use the arena once the work on the stream has finished
+        hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+        if (rc != KAPY_OK) return rc;  // (the entry point that refused has left its message)
+        if (e != hipSuccess) return fail(KAPY_ERR_HIP, "run_mlir: %s", hipGetErrorString(e));
+        return KAPY_OK;
+      }
+  }
   Parser ps;
   ps.t = tokenize(mlir_text);
   Func f;
@@ -1589,16 +1749,13 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   Interp in(f, (hipStream_t)stream);
   in.plan = &plan;
   if (const char *e = getenv("KAPY_MLIR_FUSE")) in.fuse = atoi(e) != 0;
-  // The arena is allocated at the first call on a device and kept (a call used to pay an allocation and a release of its own,
-  // several milliseconds); calls take turns at it.
-  static std::mutex arena_mutex;
-  static char *arenas[16] = {};
-  std::lock_guard<std::mutex> arena_lock(arena_mutex);
   int device = 0;
   KAPY_HIP_CHECK(hipGetDevice(&device));
   if (device < 0 || device >= 16) return fail(KAPY_ERR_UNSUPPORTED, "run_mlir: device ordinal %d beyond 16", device);
   if (!arenas[device]) KAPY_HIP_CHECK(hipMalloc((void **)&arenas[device], kArena));
   in.arena = arenas[device];
+  std::vector<PlannedCall> recorded;
+  if (use_plans) in.record = &recorded;
   rc = KAPY_OK;
   // KAPY_MLIR_IN_STEP=0: the warps of an instance run one after the other to the end instead of in step (the former way;
   // only right for programs whose warps do not exchange data through shared memory)
@@ -1675,5 +1832,14 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
   hipError_t e = hipStreamSynchronize((hipStream_t)stream);
   if (rc != KAPY_OK) return fail(rc, "run_mlir: %s", in.err.c_str());
   if (e != hipSuccess) return fail(KAPY_ERR_HIP, "run_mlir: %s", hipGetErrorString(e));
+  if (use_plans && recorded.size() <= kMaxPlannedCalls) {
+    auto plan = std::make_shared<Plan>();
+    plan->key = plan_key(mlir_text, func_name, args, n_args, grid, device);
+    plan->calls = std::move(recorded);
+    plan->merged = in.merged_calls;
+    if (g_plan_cache.size() >= kMaxPlans) g_plan_cache.pop_front();
+    g_plan_cache.push_back(std::move(plan));
+    g_plans.fetch_add(1, std::memory_order_relaxed);
+  }
   return KAPY_OK;
 }

@@ -37,7 +37,7 @@ EXPORTS = [
     "kapy_fragments_default", "kapy_layout_string", "kapy_access_simd_size", "kapy_change_source", "kapy_change_num_shuffles",
     "kapy_swizzle_offset", "kapy_swizzle_search", "kapy_swizzle_search_gfx950", "kapy_matmul_layouts", "kapy_matmul_lds_layout",
     "kapy_copy", "kapy_copy_batched", "kapy_elementwise", "kapy_fptofp", "kapy_matmul", "kapy_matmul_scaled_f8",
-    "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_run_mlir_stats", "kapy_parse_mlir",
+    "kapy_change", "kapy_reduce", "kapy_reduce_ex", "kapy_reduce_workspace_bytes", "kapy_run_mlir", "kapy_run_mlir_stats", "kapy_run_mlir_plan_stats", "kapy_parse_mlir",
     "kapy_smem_plan", "kapy_smem_barriers", "kapy_analyze_mlir",
     "kapy_elementwise_specialize", "kapy_elementwise_source", "kapy_elementwise_specialize_stats", "kapy_matmul_fused",
     "kapy_matmul_workspace_bytes", "kapy_matmul_turn_workspace_bytes", "kapy_matmul_static_workspace",
@@ -204,6 +204,7 @@ def lib():
     L.kapy_analyze_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i64), P(i32), P(i64), i32, P(i32), P(i32), i32]
     L.kapy_run_mlir.argtypes = [C.c_char_p, C.c_char_p, P(MlirArg), i32, i32 * 3, vp]
     L.kapy_run_mlir_stats.argtypes = [P(i64)]
+    L.kapy_run_mlir_plan_stats.argtypes = [P(i64), P(i64)]
     L.kapy_parse_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i32), P(i32), P(i32)]
     for name in EXPORTS:
         f = getattr(L, name)
@@ -482,6 +483,13 @@ def run_mlir_stats():
     n = C.c_int64(0)
     check(lib().kapy_run_mlir_stats(C.byref(n)))
     return n.value
+
+
+def run_mlir_plan_stats():
+    """(runs whose device calls are kept, calls of run_mlir served from a kept run) of this process."""
+    plans, replays = C.c_int64(0), C.c_int64(0)
+    check(lib().kapy_run_mlir_plan_stats(C.byref(plans), C.byref(replays)))
+    return plans.value, replays.value
 
 
 def change(in_ptr, src, dst, shape, out_ptr, stream=None):

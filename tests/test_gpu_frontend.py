@@ -361,3 +361,65 @@ def test_the_instances_of_a_grid_run_as_one_call_where_their_tiles_join(ko, monk
     both(lambda d: kh.run_mlir(kp.softmax_program(rows_per_warp, cols, warps), [dx, d, rows], [programs]), rows * cols, 1)
     # a causal mask (kapy.arange: values depend on where the tile lies): never merged
     both(lambda d: kh.run_mlir(kp.causal_softmax_program(rows_per_warp, cols, warps), [dx, d, rows], [programs]), rows * cols, 0)
+
+
+def test_a_repeated_call_replays_the_device_calls_of_the_first(ko, monkeypatch):
+    """A second kapy_run_mlir with the same text, grid and argument values makes the device calls the first one made, without
+    parsing or interpreting again (counted by kapy_run_mlir_plan_stats), on whatever the buffers hold by then; anything else
+    in the key (here an i32 argument, then the grid) is a run of its own, and KAPY_MLIR_PLAN=0 turns the cache off."""
+    rows_per_warp, cols, warps, programs = 4, 256, 2, 6
+    rows = rows_per_warp * warps * programs
+    text = kp.binary_program("arith.addf", rows_per_warp, cols, warps)
+    prog = ko.program([dict(op=ko.EW_LD_GLOBAL, dst=0, a=0), dict(op=ko.EW_LD_GLOBAL, dst=1, a=1), dict(op=ko.EW_ADDF, dst=2, a=0, b=1), dict(op=ko.EW_ST_GLOBAL, a=2)])
+    g = lambda a: ko.mk_global(a, rows, cols, cols, 1, ko.F16)
+
+    def want_of(x, y):
+        want = np.zeros(rows * cols, np.uint16)
+        assert ko.elementwise(prog, [g(x), g(y)], g(want)) == 0
+        return want
+    x1, y1 = ko.fill_normal(rows * cols, ko.F16, 11), ko.fill_normal(rows * cols, ko.F16, 12)
+    x2, y2 = ko.fill_normal(rows * cols, ko.F16, 13), ko.fill_normal(rows * cols, ko.F16, 14)
+    dx, dy, dout = to_dev(x1), to_dev(y1), dev_zeros(rows * cols, 2, fill=0x7e00)
+    plans0, replays0 = kh.run_mlir_plan_stats()
+    kh.run_mlir(text, [dx, dy, dout, rows], [programs])
+    sync()
+    assert kh.run_mlir_plan_stats() == (plans0 + 1, replays0)
+    assert np.array_equal(to_host(dout, np.uint16), want_of(x1, y1))
+    # other contents in the same buffers: the kept calls, the new sums
+    dx.copy_(to_dev(x2)); dy.copy_(to_dev(y2)); dout.fill_(0x7e00)
+    merged0 = kh.run_mlir_stats()
+    kh.run_mlir(text, [dx, dy, dout, rows], [programs])
+    sync()
+    assert kh.run_mlir_plan_stats() == (plans0 + 1, replays0 + 1)
+    assert kh.run_mlir_stats() - merged0 == 1     # (the statistics of the kept run count again)
+    assert np.array_equal(to_host(dout, np.uint16), want_of(x2, y2))
+    # fewer rows (an i32 argument) and fewer programs: runs of their own
+    dout.fill_(0x7e00)
+    fewer = rows - rows_per_warp * warps
+    kh.run_mlir(text, [dx, dy, dout, fewer], [programs - 1])
+    sync()
+    assert kh.run_mlir_plan_stats() == (plans0 + 2, replays0 + 1)
+    got = to_host(dout, np.uint16)
+    assert np.array_equal(got[:fewer * cols], want_of(x2, y2)[:fewer * cols]) and np.all(got[fewer * cols:] == 0x7e00)
+    # the cache off: nothing kept, nothing replayed, the same result
+    monkeypatch.setenv("KAPY_MLIR_PLAN", "0")
+    dout.fill_(0x7e00)
+    kh.run_mlir(text, [dx, dy, dout, rows], [programs])
+    sync()
+    assert kh.run_mlir_plan_stats() == (plans0 + 2, replays0 + 1)
+    assert np.array_equal(to_host(dout, np.uint16), want_of(x2, y2))
+    monkeypatch.delenv("KAPY_MLIR_PLAN")
+    # a program with a loop, shared-memory buffers and kapy.matmul (thousands of calls a run): the replay gives the first run's bits
+    M, N, K = 256, 256, 128
+    a, b = ko.fill_normal(M * K, ko.F16, 31, 0, 0.0, 0.5), ko.fill_normal(K * N, ko.F16, 32, 0, 0.0, 0.5)
+    da, db, dc = to_dev(a), to_dev(b), dev_zeros(M * N, 2, fill=0x7e00)
+    mm = kp.matmul_program(64, 64, 16, "mma_m16n8k8_f16", "f16")
+    kh.run_mlir(mm, [da, db, dc, M, N, K], [(M // 128) * (N // 128)])
+    sync()
+    first = to_host(dc, np.uint16).copy()
+    dc.fill_(0x7e00)
+    _, replays1 = kh.run_mlir_plan_stats()
+    kh.run_mlir(mm, [da, db, dc, M, N, K], [(M // 128) * (N // 128)])
+    sync()
+    assert kh.run_mlir_plan_stats()[1] == replays1 + 1
+    assert np.array_equal(to_host(dc, np.uint16), first) and not np.any(first == 0x7e00)

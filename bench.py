@@ -791,7 +791,7 @@ def bench_mlir(kh, steps, warmup, cpu):
     import torch
     import ko
     import kapy_programs as kp
-    out = {"workload": "the reference's three fixture programs through kapy_run_mlir", "unit": "GB/s", "dtype": "f16", "kernel": "one call per kapy.st_global over all instances (elementwise, reduce); per instance for the matmul",
+    out = {"workload": "the reference's three fixture programs through kapy_run_mlir", "unit": "GB/s", "dtype": "f16", "kernel": "one call per kapy.st_global over all instances (elementwise, reduce); in a replayed run also one launch per copy / product of the matmul program over all instances (copy_table_kernel, matmul_table_kernel)",
            "inputs": "normal(0,1) seeded, fp16", "programs": {}}
     rows_per_warp, cols, warps, programs = 4, 1024, 4, 256
     rows = rows_per_warp * warps * programs

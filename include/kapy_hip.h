@@ -500,8 +500,12 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * this library, not a fast path.
  * The device calls of a run that succeeded are kept (the last 16 runs): a later call with the same text, function name,
  * grid, argument values (every field of every kapy_mlir_arg), device and KAPY_MLIR_* modes makes the same calls again
- * without parsing or interpreting - which calls a run makes cannot depend on the tensors' contents.  KAPY_MLIR_PLAN=0 in
- * the environment turns that off. */
+ * without parsing or interpreting - which calls a run makes cannot depend on the tensors' contents.  In a kept run,
+ * consecutive copies, or matrix products of 16-bit row-major operands, that have one shape, lie in different places and do
+ * not touch each other's results - the same kapy.ld_matrix, kapy.cp_async_global_to_shared or kapy.matmul of every
+ * instance and warp in flight - are one launch each over a table of their addresses, with the bits of the calls they
+ * stand for: one launch per op for the whole grid there too.  KAPY_MLIR_PLAN=0 in the environment turns the keeping off,
+ * KAPY_MLIR_PLAN_BATCH=0 the tables. */
 typedef struct kapy_mlir_arg {
   void *ptr;      /* device pointer, for a !kapy.ptr<1> argument                    */
   int64_t bytes;  /* size of the allocation behind ptr; 0 = unknown (no range check) */
@@ -513,9 +517,9 @@ int kapy_run_mlir(const char *mlir_text, const char *func_name, const kapy_mlir_
 /* How many kapy.st_global ops this process has run as ONE call for all program instances and warps in flight (the instances'
  * chains had the same form and their views tiled a rectangle): lets a caller check that a program took that path. */
 int kapy_run_mlir_stats(int64_t *merged_stores);
-/* How many runs this process has kept the calls of, and how many calls of kapy_run_mlir were served from a kept run
- * (either pointer may be NULL). */
-int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays);
+/* How many runs this process has kept the calls of, how many calls of kapy_run_mlir were served from a kept run, and how
+ * many launches over a table of operand addresses those made (any pointer may be NULL). */
+int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays, int64_t *table_launches);
 /* The parsing half of kapy_run_mlir, without a device: KAPY_ERR_INVALID for text that does not parse,
  * KAPY_ERR_UNSUPPORTED for an op outside the set above; otherwise the function's argument count, its number
  * of ops (loop bodies included) and the module's kapy.num_warps.  Out pointers may be NULL. */

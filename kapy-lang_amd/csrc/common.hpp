@@ -94,6 +94,18 @@ float *reduce_scratch_lines(size_t *bytes, uint32_t **counters = nullptr);   // 
 int copy_impl(const kapy_global *src, const kapy_global *dst, const kapy_copy_cfg *cfg, const kapy_grid2 *grid, void *stream);
 int run_matmul_f16acc(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result, int k_step, hipStream_t s);
 int run_column_softmax(const kapy_global *x, const kapy_global *out, hipStream_t stream);
+// Many copies / matrix products of one shape as one launch over a table of base addresses in device memory (batched.hip):
+// n rows of (source, target) or (lhs, rhs, accumulator input or 0, result), the addresses of element (0, 0) of each view.
+struct CopyTableShape {
+  int32_t d0, d1, elem_bytes;
+  int64_t ss0, ss1, ds0, ds1;  // element strides of source and target
+};
+struct MatmulTableShape {
+  int32_t M, N, K, ab_dtype, acc_dtype, d_dtype;
+  int64_t a_sm, b_sk, acc_sm, acc_sn, d_sm, d_sn;  // lhs rows and rhs k-rows contiguous
+};
+int copy_table_launch(const uint64_t *device_table, int32_t n, const CopyTableShape &shape, bool vec16, hipStream_t s);
+int matmul_table_launch(const uint64_t *device_table, int32_t n, const MatmulTableShape &shape, hipStream_t s);
 int ensure_device();
 int device_cus();
 

@@ -1630,14 +1630,15 @@ extern "C" int kapy_analyze_mlir(const char *mlir_text, const char *func_name, i
   return KAPY_OK;
 }
 
-static std::atomic<int64_t> g_merged_calls{0}, g_plans{0}, g_replays{0};
+static std::atomic<int64_t> g_merged_calls{0}, g_plans{0}, g_replays{0}, g_table_launches{0};
 extern "C" int kapy_run_mlir_stats(int64_t *merged_stores) {
   if (merged_stores) *merged_stores = g_merged_calls.load();
   return KAPY_OK;
 }
-extern "C" int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays) {
+extern "C" int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays, int64_t *table_launches) {
   if (plans) *plans = g_plans.load();
   if (replays) *replays = g_replays.load();
+  if (table_launches) *table_launches = g_table_launches.load();
   return KAPY_OK;
 }
 
@@ -1646,11 +1647,249 @@ extern "C" int kapy_run_mlir_plan_stats(int64_t *plans, int64_t *replays) {
 // those calls again without parsing or interpreting anything (the register tensors they name live in the device's arena, which
 // is kept for the life of the process and laid out the same way every time).
 namespace {
+// A step of a kept run: one of its calls as it was made, or a run of consecutive calls that differ only in where their
+// operands lie (the same copy or matrix product of every instance and warp in flight) as ONE launch over a table of base
+// addresses (batched.hip).  The tables of all steps of a run are one device allocation, written when the run is kept.
+struct PlanStep {
+  enum Kind { kCall, kCopyTable, kMatmulTable } kind = kCall;
+  size_t first = 0, count = 1;   // the calls it stands for
+  size_t rows = 0;               // rows of its table (calls that repeat another of the group word for word have none)
+  CopyTableShape copy = {};
+  bool vec16 = false;
+  MatmulTableShape matmul = {};
+  size_t table_at = 0;           // first word of its table
+};
 struct Plan {
   std::string key;
   std::vector<PlannedCall> calls;
+  std::vector<PlanStep> steps;
+  uint64_t *device_table = nullptr;
   int64_t merged = 0;
 };
+
+// The bytes a [rows x cols] walk over a view touches.  exact: rows of contiguous elements, no longer than the pitch - then two
+// regions of one pitch are compared element by element (two column ranges of one buffer interleave without meeting);
+// anything else by its bounding interval.
+struct Region {
+  uintptr_t lo = 0, hi = 0;
+  int64_t pitch = 0, row_bytes = 0, rows = 0;
+  bool exact = false;
+};
+bool region_of(const kapy_global &g, int64_t e0, int64_t e1, Region &out) {
+  if (e0 <= 0 || e1 <= 0 || g.stride0 <= 0 || g.stride1 <= 0) return false;
+  const int64_t b = dtype_bytes(g.dtype);
+  out.lo = (uintptr_t)view_base(&g);
+  out.hi = out.lo + (uintptr_t)(((e0 - 1) * g.stride0 + (e1 - 1) * g.stride1 + 1) * b);
+  out.pitch = g.stride0 * b;
+  out.row_bytes = e1 * b;
+  out.rows = e0;
+  out.exact = g.stride1 == 1 && out.row_bytes <= out.pitch;
+  return true;
+}
+bool regions_overlap(const Region &x, const Region &y) {
+  if (!(x.lo < y.hi && y.lo < x.hi)) return false;
+  if (!(x.exact && y.exact && x.pitch == y.pitch)) return true;
+  const Region &a = x.lo <= y.lo ? x : y, &b = x.lo <= y.lo ? y : x;
+  // b starts q rows and t bytes into a's grid: its rows meet a's where their byte ranges do, in the same or the next row of a
+  const int64_t delta = (int64_t)(b.lo - a.lo), q = delta / a.pitch, t = delta % a.pitch;
+  return (t < a.row_bytes && q < a.rows) || (t + b.row_bytes > a.pitch && q + 1 < a.rows);
+}
+// What a call reads and writes.  known = false: a view this bookkeeping does not describe (the call then stays where it is
+// and nothing moves across it).
+struct Footprint {
+  std::vector<Region> reads;
+  Region write;
+  bool known = false;
+};
+bool add_read(Footprint &fp, const kapy_global &g, int64_t e0, int64_t e1) {
+  Region r;
+  if (!region_of(g, e0, e1, r)) return false;
+  fp.reads.push_back(r);
+  return true;
+}
+Footprint footprint_of(const PlannedCall &c) {
+  Footprint fp;
+  switch (c.kind) {
+    case PlannedCall::kCopy: {
+      // (the source is read where the target's extent, or its own if smaller, reaches)
+      const bool t = c.has_cfg && c.copy_cfg.transpose;
+      const int64_t d0 = extent0(&c.g[1]), d1 = extent1(&c.g[1]);
+      const int64_t r0 = std::min(extent0(&c.g[0]), t ? d1 : d0), r1 = std::min(extent1(&c.g[0]), t ? d0 : d1);
+      fp.known = region_of(c.g[1], d0, d1, fp.write) && (r0 <= 0 || r1 <= 0 || add_read(fp, c.g[0], r0, r1));
+      break;
+    }
+    case PlannedCall::kElementwise: {
+      fp.known = region_of(c.g[0], extent0(&c.g[0]), extent1(&c.g[0]), fp.write);
+      for (const kapy_global &in : c.ins) fp.known = fp.known && add_read(fp, in, extent0(&in), extent1(&in));
+      break;
+    }
+    case PlannedCall::kReduce:
+    case PlannedCall::kReduceEx:
+      fp.known = region_of(c.g[1], extent0(&c.g[1]), extent1(&c.g[1]), fp.write) && add_read(fp, c.g[0], extent0(&c.g[0]), extent1(&c.g[0]));
+      break;
+    case PlannedCall::kMatmul:
+      fp.known = region_of(c.g[3], extent0(&c.g[3]), extent1(&c.g[3]), fp.write) && add_read(fp, c.g[0], extent0(&c.g[0]), extent1(&c.g[0])) &&
+                 add_read(fp, c.g[1], extent0(&c.g[1]), extent1(&c.g[1])) && (!c.has[2] || add_read(fp, c.g[2], extent0(&c.g[2]), extent1(&c.g[2])));
+      break;
+  }
+  return fp;
+}
+// neither writes what the other reads or writes: the two may run in either order, or at once
+bool independent(const Footprint &x, const Footprint &y) {
+  if (regions_overlap(x.write, y.write)) return false;
+  for (const Region &r : y.reads)
+    if (regions_overlap(x.write, r)) return false;
+  for (const Region &r : x.reads)
+    if (regions_overlap(y.write, r)) return false;
+  return true;
+}
+
+// Whether a call is of a kind the table kernels reproduce bit for bit, and its shape.
+bool copy_for_table(const PlannedCall &c, CopyTableShape &sh) {
+  if (c.kind != PlannedCall::kCopy || (c.has_cfg && c.copy_cfg.transpose)) return false;
+  const kapy_global &src = c.g[0], &dst = c.g[1];
+  const int64_t d0 = extent0(&dst), d1 = extent1(&dst);
+  const int b = dtype_bytes(src.dtype);
+  // (nothing to pad: the source view covers the target's extent)
+  if (b != dtype_bytes(dst.dtype) || (b != 1 && b != 2 && b != 4) || d0 <= 0 || d1 <= 0 || extent0(&src) < d0 || extent1(&src) < d1 || d0 > INT32_MAX || d1 > INT32_MAX ||
+      src.stride0 <= 0 || src.stride1 <= 0 || dst.stride0 <= 0 || dst.stride1 <= 0)
+    return false;
+  sh = {(int32_t)d0, (int32_t)d1, b, src.stride0, src.stride1, dst.stride0, dst.stride1};
+  return true;
+}
+bool matmul_for_table(const PlannedCall &c, MatmulTableShape &sh) {
+  if (c.kind != PlannedCall::kMatmul) return false;
+  const kapy_global &a = c.g[0], &b = c.g[1], &acc = c.g[2], &d = c.g[3];
+  if (c.has_cfg) {
+    const kapy_matmul_cfg &m = c.matmul_cfg;
+    if (m.accumulate != KAPY_ACCUMULATE_F32 || m.rmode != KAPY_RN || m.split_k > 1 || m.workspace || m.tile_m || m.tile_n || m.tile_k || m.stages || m.waves ||
+        m.impl_way >= KAPY_MFMA_32X32X16_16B)
+      return false;
+  }
+  const int64_t M = extent0(&a), K = extent1(&a), N = extent1(&b);
+  // the shapes the library multiplies with its kernel for a row-major lhs and a row-major rhs, whose arithmetic
+  // matmul_table_kernel repeats: 16-byte aligned contiguous rows on both, N and K multiples of 8; and small ones only
+  if ((a.dtype != KAPY_F16 && a.dtype != KAPY_BF16) || b.dtype != a.dtype || a.stride1 != 1 || b.stride1 != 1 || a.stride0 <= 0 || b.stride0 <= 0 || extent0(&b) != K ||
+      M <= 0 || N <= 0 || K <= 0 || N % 8 || K % 8 || M > 256 || N > 256 || K > 1024 || vector_bytes(&a, 1) != 16 || vector_bytes(&b, 1) != 16)
+    return false;
+  if ((d.dtype != KAPY_F16 && d.dtype != KAPY_BF16 && d.dtype != KAPY_F32) || extent0(&d) != M || extent1(&d) != N || d.stride0 <= 0 || d.stride1 <= 0) return false;
+  if (c.has[2] && ((acc.dtype != KAPY_F16 && acc.dtype != KAPY_BF16 && acc.dtype != KAPY_F32) || extent0(&acc) != M || extent1(&acc) != N || acc.stride0 <= 0 || acc.stride1 <= 0))
+    return false;
+  sh = {(int32_t)M, (int32_t)N, (int32_t)K, a.dtype, c.has[2] ? acc.dtype : -1, d.dtype, a.stride0, b.stride0,
+        c.has[2] ? acc.stride0 : 0, c.has[2] ? acc.stride1 : 0, d.stride0, d.stride1};
+  return true;
+}
+bool same_shape(const CopyTableShape &x, const CopyTableShape &y) {
+  return x.d0 == y.d0 && x.d1 == y.d1 && x.elem_bytes == y.elem_bytes && x.ss0 == y.ss0 && x.ss1 == y.ss1 && x.ds0 == y.ds0 && x.ds1 == y.ds1;
+}
+bool same_shape(const MatmulTableShape &x, const MatmulTableShape &y) {
+  return x.M == y.M && x.N == y.N && x.K == y.K && x.ab_dtype == y.ab_dtype && x.acc_dtype == y.acc_dtype && x.d_dtype == y.d_dtype && x.a_sm == y.a_sm &&
+         x.b_sk == y.b_sk && x.acc_sm == y.acc_sm && x.acc_sn == y.acc_sn && x.d_sm == y.d_sm && x.d_sn == y.d_sn;
+}
+
+// Groups the calls of a run into steps and writes the tables.  A group starts at a copy or product the table kernels take and
+// collects, from the calls behind it (a window of them), those of the same kind and shape that are independent of every
+// member so far and of every call passed over on the way - such a call may move up in front of those and run with the
+// group; the calls passed over keep their order.  (The instances reach an op one after the other, and some ops make two
+// calls per instance - a deferred value computed, then the product that reads it - so the calls that belong together are
+// not always neighbours.)  A copy from the same place to the same place as a member, with nothing in between that touches
+// either, is dropped: the warps of a program that fetch one tile into one shared buffer.
+constexpr size_t kMaxTableRows = 16384, kPlanWindow = 8192, kMaxOptimisedCalls = 200000;
+void plan_steps(Plan &plan) {
+  bool tables = true;
+  if (const char *e = getenv("KAPY_MLIR_PLAN_BATCH")) tables = atoi(e) != 0;
+  const std::vector<PlannedCall> &calls = plan.calls;
+  auto singles = [&]() {
+    plan.steps.clear();
+    for (size_t i = 0; i < calls.size(); ++i) {
+      PlanStep st;
+      st.first = i;
+      plan.steps.push_back(st);
+    }
+  };
+  if (!tables || calls.size() > kMaxOptimisedCalls) return singles();
+  std::vector<Footprint> fps;
+  fps.reserve(calls.size());
+  for (const PlannedCall &c : calls) fps.push_back(footprint_of(c));
+  std::vector<char> taken(calls.size(), 0);
+  std::vector<uint64_t> words;
+  std::vector<size_t> members, passed;
+  for (size_t i = 0; i < calls.size(); ++i) {
+    if (taken[i]) continue;
+    PlanStep st;
+    st.first = i;
+    CopyTableShape cs = {};
+    MatmulTableShape ms = {};
+    const bool is_copy = fps[i].known && copy_for_table(calls[i], cs), is_matmul = fps[i].known && !is_copy && matmul_for_table(calls[i], ms);
+    if (!is_copy && !is_matmul) {
+      plan.steps.push_back(st);
+      continue;
+    }
+    members.assign(1, i);
+    passed.clear();
+    size_t stood_for = 1;
+    for (size_t j = i + 1; j < calls.size() && j - i < kPlanWindow && members.size() < kMaxTableRows; ++j) {
+      if (taken[j]) continue;
+      if (!fps[j].known) break;
+      CopyTableShape cs2 = {};
+      MatmulTableShape ms2 = {};
+      bool joins = is_copy ? copy_for_table(calls[j], cs2) && same_shape(cs, cs2) : matmul_for_table(calls[j], ms2) && same_shape(ms, ms2);
+      for (size_t k = 0; k < passed.size() && joins; ++k) joins = independent(fps[j], fps[passed[k]]);
+      bool repeated = false;
+      if (joins && is_copy)
+        for (size_t m : members)
+          if (fps[m].write.lo == fps[j].write.lo && fps[m].write.hi == fps[j].write.hi && fps[m].reads[0].lo == fps[j].reads[0].lo) repeated = true;
+      for (size_t k = 0; k < members.size() && joins && !repeated; ++k) joins = independent(fps[j], fps[members[k]]);
+      if (!joins) {
+        passed.push_back(j);
+        continue;
+      }
+      taken[j] = 1;
+      ++stood_for;
+      if (!repeated) members.push_back(j);
+    }
+    st.count = stood_for;
+    st.rows = members.size();
+    if (stood_for >= 2) {
+      st.table_at = words.size();
+      if (is_copy) {
+        st.kind = PlanStep::kCopyTable;
+        st.copy = cs;
+        const int64_t b = cs.elem_bytes;
+        bool vec = cs.ss1 == 1 && cs.ds1 == 1 && (cs.d1 * b) % 16 == 0 && (cs.ss0 * b) % 16 == 0 && (cs.ds0 * b) % 16 == 0;
+        for (size_t m : members) {
+          vec = vec && fps[m].reads[0].lo % 16 == 0 && fps[m].write.lo % 16 == 0;
+          words.push_back((uint64_t)fps[m].reads[0].lo);
+          words.push_back((uint64_t)fps[m].write.lo);
+        }
+        st.vec16 = vec;
+      } else {
+        st.kind = PlanStep::kMatmulTable;
+        st.matmul = ms;
+        for (size_t m : members) {
+          words.push_back((uint64_t)fps[m].reads[0].lo);
+          words.push_back((uint64_t)fps[m].reads[1].lo);
+          words.push_back(fps[m].reads.size() > 2 ? (uint64_t)fps[m].reads[2].lo : 0);
+          words.push_back((uint64_t)fps[m].write.lo);
+        }
+      }
+    }
+    plan.steps.push_back(st);
+  }
+  if (words.empty()) return;
+  // (a run whose tables cannot be placed keeps its calls as they were made)
+  if (hipMalloc((void **)&plan.device_table, words.size() * sizeof(uint64_t)) != hipSuccess ||
+      hipMemcpy(plan.device_table, words.data(), words.size() * sizeof(uint64_t), hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipGetLastError();
+    if (plan.device_table) (void)hipFree(plan.device_table);
+    plan.device_table = nullptr;
+    singles();
+  }
+}
+void release_plan(Plan &plan) {
+  if (plan.device_table) (void)hipFree(plan.device_table);
+  plan.device_table = nullptr;
+}
 constexpr size_t kMaxPlans = 16, kMaxPlannedCalls = 1u << 20;
 std::deque<std::shared_ptr<Plan>> g_plan_cache;  // (guarded by the arena's mutex: calls take turns anyway)
 
@@ -1667,7 +1906,7 @@ std::string plan_key(const char *text, const char *func, const kapy_mlir_arg *ar
     k.append((const char *)&args[i].bytes, sizeof args[i].bytes);
     k.append((const char *)&args[i].i32, sizeof args[i].i32);
   }
-  for (const char *name : {"KAPY_MLIR_FUSE", "KAPY_MLIR_IN_STEP", "KAPY_MLIR_BATCH", "KAPY_MLIR_MATMUL", "KAPY_MLIR_REDUCE"}) {
+  for (const char *name : {"KAPY_MLIR_FUSE", "KAPY_MLIR_IN_STEP", "KAPY_MLIR_BATCH", "KAPY_MLIR_MATMUL", "KAPY_MLIR_REDUCE", "KAPY_MLIR_PLAN_BATCH"}) {
     const char *v = getenv(name);
     k += v ? v : "";
     k.push_back('\0');
@@ -1677,8 +1916,21 @@ std::string plan_key(const char *text, const char *func, const kapy_mlir_arg *ar
 
 int replay_plan(const Plan &plan, hipStream_t stream) {
   std::vector<const kapy_global *> ins;
-  for (const PlannedCall &c : plan.calls) {
+  for (const PlanStep &st : plan.steps) {
     int rc = KAPY_OK;
+    if (st.kind == PlanStep::kCopyTable) {
+      rc = copy_table_launch(plan.device_table + st.table_at, (int32_t)st.rows, st.copy, st.vec16, stream);
+      if (rc != KAPY_OK) return rc;
+      g_table_launches.fetch_add(1, std::memory_order_relaxed);
+      continue;
+    }
+    if (st.kind == PlanStep::kMatmulTable) {
+      rc = matmul_table_launch(plan.device_table + st.table_at, (int32_t)st.rows, st.matmul, stream);
+      if (rc != KAPY_OK) return rc;
+      g_table_launches.fetch_add(1, std::memory_order_relaxed);
+      continue;
+    }
+    const PlannedCall &c = plan.calls[st.first];
     switch (c.kind) {
       case PlannedCall::kCopy: rc = kapy_copy(&c.g[0], &c.g[1], c.has_cfg ? &c.copy_cfg : nullptr, stream); break;
       case PlannedCall::kElementwise:
@@ -1837,7 +2089,11 @@ extern "C" int kapy_run_mlir(const char *mlir_text, const char *func_name, const
     plan->key = plan_key(mlir_text, func_name, args, n_args, grid, device);
     plan->calls = std::move(recorded);
     plan->merged = in.merged_calls;
-    if (g_plan_cache.size() >= kMaxPlans) g_plan_cache.pop_front();
+    plan_steps(*plan);
+    if (g_plan_cache.size() >= kMaxPlans) {
+      release_plan(*g_plan_cache.front());
+      g_plan_cache.pop_front();
+    }
     g_plan_cache.push_back(std::move(plan));
     g_plans.fetch_add(1, std::memory_order_relaxed);
   }

@@ -204,7 +204,7 @@ def lib():
     L.kapy_analyze_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i64), P(i32), P(i64), i32, P(i32), P(i32), i32]
     L.kapy_run_mlir.argtypes = [C.c_char_p, C.c_char_p, P(MlirArg), i32, i32 * 3, vp]
     L.kapy_run_mlir_stats.argtypes = [P(i64)]
-    L.kapy_run_mlir_plan_stats.argtypes = [P(i64), P(i64)]
+    L.kapy_run_mlir_plan_stats.argtypes = [P(i64), P(i64), P(i64)]
     L.kapy_parse_mlir.argtypes = [C.c_char_p, C.c_char_p, P(i32), P(i32), P(i32)]
     for name in EXPORTS:
         f = getattr(L, name)
@@ -486,10 +486,11 @@ def run_mlir_stats():
 
 
 def run_mlir_plan_stats():
-    """(runs whose device calls are kept, calls of run_mlir served from a kept run) of this process."""
-    plans, replays = C.c_int64(0), C.c_int64(0)
-    check(lib().kapy_run_mlir_plan_stats(C.byref(plans), C.byref(replays)))
-    return plans.value, replays.value
+    """(runs whose device calls are kept, calls of run_mlir served from a kept run, launches over a table of operand
+    addresses made by those) of this process."""
+    plans, replays, tables = C.c_int64(0), C.c_int64(0), C.c_int64(0)
+    check(lib().kapy_run_mlir_plan_stats(C.byref(plans), C.byref(replays), C.byref(tables)))
+    return plans.value, replays.value, tables.value
 
 
 def change(in_ptr, src, dst, shape, out_ptr, stream=None):

@@ -380,17 +380,17 @@ def test_a_repeated_call_replays_the_device_calls_of_the_first(ko, monkeypatch):
     x1, y1 = ko.fill_normal(rows * cols, ko.F16, 11), ko.fill_normal(rows * cols, ko.F16, 12)
     x2, y2 = ko.fill_normal(rows * cols, ko.F16, 13), ko.fill_normal(rows * cols, ko.F16, 14)
     dx, dy, dout = to_dev(x1), to_dev(y1), dev_zeros(rows * cols, 2, fill=0x7e00)
-    plans0, replays0 = kh.run_mlir_plan_stats()
+    plans0, replays0, _ = kh.run_mlir_plan_stats()
     kh.run_mlir(text, [dx, dy, dout, rows], [programs])
     sync()
-    assert kh.run_mlir_plan_stats() == (plans0 + 1, replays0)
+    assert kh.run_mlir_plan_stats()[:2] == (plans0 + 1, replays0)
     assert np.array_equal(to_host(dout, np.uint16), want_of(x1, y1))
     # other contents in the same buffers: the kept calls, the new sums
     dx.copy_(to_dev(x2)); dy.copy_(to_dev(y2)); dout.fill_(0x7e00)
     merged0 = kh.run_mlir_stats()
     kh.run_mlir(text, [dx, dy, dout, rows], [programs])
     sync()
-    assert kh.run_mlir_plan_stats() == (plans0 + 1, replays0 + 1)
+    assert kh.run_mlir_plan_stats()[:2] == (plans0 + 1, replays0 + 1)
     assert kh.run_mlir_stats() - merged0 == 1     # (the statistics of the kept run count again)
     assert np.array_equal(to_host(dout, np.uint16), want_of(x2, y2))
     # fewer rows (an i32 argument) and fewer programs: runs of their own
@@ -398,7 +398,7 @@ def test_a_repeated_call_replays_the_device_calls_of_the_first(ko, monkeypatch):
     fewer = rows - rows_per_warp * warps
     kh.run_mlir(text, [dx, dy, dout, fewer], [programs - 1])
     sync()
-    assert kh.run_mlir_plan_stats() == (plans0 + 2, replays0 + 1)
+    assert kh.run_mlir_plan_stats()[:2] == (plans0 + 2, replays0 + 1)
     got = to_host(dout, np.uint16)
     assert np.array_equal(got[:fewer * cols], want_of(x2, y2)[:fewer * cols]) and np.all(got[fewer * cols:] == 0x7e00)
     # the cache off: nothing kept, nothing replayed, the same result
@@ -406,20 +406,49 @@ def test_a_repeated_call_replays_the_device_calls_of_the_first(ko, monkeypatch):
     dout.fill_(0x7e00)
     kh.run_mlir(text, [dx, dy, dout, rows], [programs])
     sync()
-    assert kh.run_mlir_plan_stats() == (plans0 + 2, replays0 + 1)
+    assert kh.run_mlir_plan_stats()[:2] == (plans0 + 2, replays0 + 1)
     assert np.array_equal(to_host(dout, np.uint16), want_of(x2, y2))
     monkeypatch.delenv("KAPY_MLIR_PLAN")
-    # a program with a loop, shared-memory buffers and kapy.matmul (thousands of calls a run): the replay gives the first run's bits
-    M, N, K = 256, 256, 128
-    a, b = ko.fill_normal(M * K, ko.F16, 31, 0, 0.0, 0.5), ko.fill_normal(K * N, ko.F16, 32, 0, 0.0, 0.5)
-    da, db, dc = to_dev(a), to_dev(b), dev_zeros(M * N, 2, fill=0x7e00)
-    mm = kp.matmul_program(64, 64, 16, "mma_m16n8k8_f16", "f16")
-    kh.run_mlir(mm, [da, db, dc, M, N, K], [(M // 128) * (N // 128)])
-    sync()
-    first = to_host(dc, np.uint16).copy()
-    dc.fill_(0x7e00)
-    _, replays1 = kh.run_mlir_plan_stats()
-    kh.run_mlir(mm, [da, db, dc, M, N, K], [(M // 128) * (N // 128)])
-    sync()
-    assert kh.run_mlir_plan_stats()[1] == replays1 + 1
-    assert np.array_equal(to_host(dc, np.uint16), first) and not np.any(first == 0x7e00)
+
+
+@pytest.mark.parametrize("bm,bn,bk,way,acc,dtype,M,N,K", [
+    (64, 64, 16, "mma_m16n8k8_f16", "f16", "f16", 256, 256, 128),    # the fixture's tiling; K steps of half an instruction's 32
+    (64, 64, 32, "mma_m16n8k16_f16", "f32", "f16", 128, 256, 96),
+    (32, 64, 64, "mma_m16n8k16_f16", "f32", "bf16", 128, 128, 192),  # two instructions per step
+    (32, 32, 32, "mma_m16n8k16_f16", "f16", "f16", 64, 128, 32),     # one K step: the loop body never runs
+])
+def test_a_kept_run_makes_the_copies_and_products_of_all_instances_in_one_launch_each(ko, monkeypatch, bm, bn, bk, way, acc, dtype, M, N, K):
+    """A program with a loop, shared-memory buffers and kapy.matmul makes one call per instance, warp and op when it is
+    interpreted (hundreds to thousands a run).  In the kept run the same copy or product of all instances in flight is one
+    launch over a table of their addresses: the replay gives the bits of the first run, which made the calls one by one
+    (and is compared with the oracle by test_matmul_program_matches_oracle), with and without the tables."""
+    kd = ko.F16 if dtype == "f16" else ko.BF16
+    a, b = ko.fill_normal(M * K, kd, 31, 0, 0.0, 0.5), ko.fill_normal(K * N, kd, 32, 0, 0.0, 0.5)
+    acc_bytes = 2 if acc == "f16" else 4
+    grid = [(M // (2 * bm)) * (N // (2 * bn))]
+    mm = kp.matmul_program(bm, bn, bk, way, acc, dtype)
+    outs = {}
+    for tables in ("1", "0"):
+        monkeypatch.setenv("KAPY_MLIR_PLAN_BATCH", tables)
+        da, db, dc = to_dev(a), to_dev(b), dev_zeros(M * N, acc_bytes, fill=0x7e00)
+        kh.run_mlir(mm, [da, db, dc, M, N, K], grid)
+        sync()
+        first = to_host(dc, np.uint8).copy()
+        dc.fill_(0x7e00)
+        _, replays0, tables0 = kh.run_mlir_plan_stats()
+        kh.run_mlir(mm, [da, db, dc, M, N, K], grid)
+        sync()
+        _, replays1, tables1 = kh.run_mlir_plan_stats()
+        assert replays1 == replays0 + 1
+        steps = K // bk
+        # per K step at most: two copies into shared memory, two out of it and a product, each for all instances at once
+        # (fewer where calls of one shape from neighbouring ops join one table, a few more where a group splits); the store of
+        # the result is one more
+        if tables == "1":
+            assert 3 * steps <= tables1 - tables0 <= 6 * steps + 2, (tables1 - tables0, steps)
+        else:
+            assert tables1 == tables0
+        got = to_host(dc, np.uint8)
+        assert np.array_equal(got, first)
+        outs[tables] = got
+    assert np.array_equal(outs["1"], outs["0"])

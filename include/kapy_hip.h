@@ -504,8 +504,9 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * consecutive copies, or matrix products of 16-bit row-major operands, that have one shape, lie in different places and do
  * not touch each other's results - the same kapy.ld_matrix, kapy.cp_async_global_to_shared or kapy.matmul of every
  * instance and warp in flight - are one launch each over a table of their addresses, with the bits of the calls they
- * stand for: one launch per op for the whole grid there too.  KAPY_MLIR_PLAN=0 in the environment turns the keeping off,
- * KAPY_MLIR_PLAN_BATCH=0 the tables. */
+ * stand for: one launch per op for the whole grid there too (a kept run with tables holds them in device memory of its
+ * own, 16 bytes per copy and 32 per product, until it leaves the cache).  KAPY_MLIR_PLAN=0 in the environment turns the
+ * keeping off, KAPY_MLIR_PLAN_BATCH=0 the tables. */
 typedef struct kapy_mlir_arg {
   void *ptr;      /* device pointer, for a !kapy.ptr<1> argument                    */
   int64_t bytes;  /* size of the allocation behind ptr; 0 = unknown (no range check) */

@@ -452,3 +452,82 @@ def test_a_kept_run_makes_the_copies_and_products_of_all_instances_in_one_launch
         assert np.array_equal(got, first)
         outs[tables] = got
     assert np.array_equal(outs["1"], outs["0"])
+
+
+@pytest.mark.parametrize("fuse", ["1", "0"])
+@pytest.mark.parametrize("family", ["exchange", "exchange_narrow", "exchange_loop", "phases", "aliasing", "block_sum", "transpose", "softmax", "column_softmax",
+                                    "causal_softmax", "gated", "reduce"])
+def test_a_replayed_run_has_the_bits_of_the_interpreted_run(ko, monkeypatch, family, fuse):
+    """Every program family of this file twice on the same buffers (inputs and results restored in between): the second call
+    is served from the kept run - calls regrouped, copies of all instances in one launch where they are independent - and
+    must leave what the interpreted first call left; a third pair does the same with the tables switched off.  The programs
+    that exchange tiles through shared memory, overwrite what earlier loads read or update a buffer in place are the ones a
+    wrong dependence test would break.  KAPY_MLIR_FUSE=0 runs every op as a call of its own (many more copies)."""
+    monkeypatch.setenv("KAPY_MLIR_FUSE", fuse)
+    f16 = lambda n, seed: ko.fill_normal(n, ko.F16, seed)
+    if family in ("exchange", "exchange_narrow"):
+        rpw, cols, warps, programs = (16, 64, 4, 3) if family == "exchange" else (8, 40, 2, 3)   # (rows of 80 bytes: no 16-byte pieces)
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 61), np.full(rows * cols, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.exchange_program(rpw, cols, warps), lambda d: [d[0], d[1], rows], [programs], [1]
+    elif family == "exchange_loop":
+        rpw, cols, warps, steps, programs = 8, 64, 4, 3, 2
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 62), np.full(rows * cols, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.exchange_loop_program(rpw, cols, warps, steps), lambda d: [d[0], d[1], rows], [programs], [1]
+    elif family == "phases":
+        bufs = [f16(64 * 64, 41)]
+        text, args, grid, outs = kp.phases_program(), lambda d: [d[0]], [1], [0]
+    elif family == "aliasing":
+        rpw, cols, warps, programs = 4, 128, 2, 3
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 71), f16(rows * cols, 72), np.full(rows * cols, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.aliasing_program(rpw, cols, warps), lambda d: [d[0], d[1], d[2], rows], [programs], [0, 2]
+    elif family == "block_sum":
+        rpw, bc, warps, programs, cols = 4, 64, 2, 3, 256
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 81), np.full(rows * bc, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.block_sum_program(rpw, bc, warps), lambda d: [d[0], d[1], rows, cols], [programs], [1]
+    elif family == "transpose":
+        m, n, tile = 96, 64, 32
+        bufs = [f16(m * n, 52), np.full(m * n, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.scaled_transpose_program(tile, 0.5), lambda d: [d[0], d[1], m, n], [m // tile, n // tile], [1]
+    elif family == "column_softmax":
+        rows, cpw, warps, programs = 64, 64, 2, 3
+        cols = cpw * warps * programs
+        bufs = [f16(rows * cols, 91), np.full(rows * cols, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.column_softmax_program(rows, cpw, warps), lambda d: [d[0], d[1], cols], [programs], [1]
+    elif family == "gated":
+        rpw, cols, warps, programs = 4, 256, 2, 3
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 1), f16(rows * cols, 2), f16(rows * cols, 3), np.full(rows * cols, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.gated_program(rpw, cols, warps), lambda d: [d[0], d[1], d[2], d[3], rows], [programs], [3]
+    elif family == "reduce":
+        rpw, cols, warps, programs = 2, 256, 2, 8
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 21), np.full(rows, 0x7e00, np.uint16)]
+        text, args, grid, outs = kp.reduce_program("arith.addf", rpw, cols, warps), lambda d: [d[0], d[1], rows], [programs], [1]
+    else:
+        rpw, cols, warps, programs = 2, 256, 2, 5
+        rows = rpw * warps * programs
+        bufs = [f16(rows * cols, 31), np.full(rows * cols, 0x7e00, np.uint16)]
+        gen = kp.softmax_program if family == "softmax" else kp.causal_softmax_program
+        text, args, grid, outs = gen(rpw, cols, warps), lambda d: [d[0], d[1], rows], [programs], [1]
+    dev = [to_dev(b) for b in bufs]
+
+    def run():
+        for d, b in zip(dev, bufs):
+            d.copy_(to_dev(b))
+        kh.run_mlir(text, args(dev), grid)
+        sync()
+        return [to_host(dev[k], np.uint16).copy() for k in outs]
+    results = []
+    for tables in ("1", "0"):
+        monkeypatch.setenv("KAPY_MLIR_PLAN_BATCH", tables)
+        plans0, replays0, _ = kh.run_mlir_plan_stats()
+        results.append(run())
+        assert kh.run_mlir_plan_stats()[:2] == (plans0 + 1, replays0)
+        results.append(run())
+        assert kh.run_mlir_plan_stats()[:2] == (plans0 + 1, replays0 + 1)
+    for r in results[1:]:
+        assert all(np.array_equal(x, y) for x, y in zip(r, results[0]))

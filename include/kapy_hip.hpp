@@ -2,9 +2,11 @@
 //
 // kapy::OpBuilder mirrors the part of the reference's KapyOpBuilder that the hot path uses
 // (python/src/ir.cc:730-1181: create_mk_global, create_sv_global, create_ld_global, create_st_global,
-// create_splat, create_broadcast, create_transpose, create_arange, create_fptofp / extf / truncf / bitcast / sitofp /
+// create_constant_* scalars, create_splat, create_broadcast, create_transpose, create_arange, create_fptofp / extf / truncf / bitcast / sitofp /
 // fptosi / intcast, the float and integer arith builders, the create_cmpi_* / create_cmpf_* families, create_select,
-// the math builders, create_reduce, create_matmul), with the same names and argument meaning.  Where the reference
+// the math builders, create_elementwise_extern_lib, create_reduce, create_matmul: 97 of its 112 create_* names - the rest build
+// modules, blocks, control flow and the ids of a program, which a recorded dataflow graph has none of), with the same names and
+// argument meaning.  Where the reference
 // appends an op to a function that is compiled later, this builder records the op in a dataflow graph;
 // create_st_global - the op with the side effect - lowers the graph under its source to ONE library call:
 //   a load (optionally transposed) stored back            -> kapy_copy
@@ -147,6 +149,37 @@ class OpBuilder {
     n.ival = source;
     return push(n);
   }
+  // ---- scalar constants (ir.cc:480-560: create_constant_int1 ... create_constant_float64, create_constant_zero,
+  // create_constant_all_ones).  A scalar here exists to be splat: create_splat(scalar) makes the tensor of the scalar's type
+  // (f64 and i64 scalars have no tensor type in this library and can only be splat to a named narrower type).
+  Value create_constant_int1(bool v) { return scalar_int(v ? 1 : 0, KAPY_I1); }
+  Value create_constant_int8(int8_t v) { return scalar_int(v, KAPY_I8); }
+  Value create_constant_int16(int16_t v) { return scalar_int(v, KAPY_I16); }
+  Value create_constant_int32(int32_t v) { return scalar_int(v, KAPY_I32); }
+  Value create_constant_int64(int64_t v) { return scalar_int(v, -64); }
+  Value create_constant_float8e4m3(float v) { return scalar_float(v, KAPY_F8E4M3); }
+  Value create_constant_float8e5m2(float v) { return scalar_float(v, KAPY_F8E5M2); }
+  Value create_constant_float16(float v) { return scalar_float(v, KAPY_F16); }
+  Value create_constant_bfloat16(float v) { return scalar_float(v, KAPY_BF16); }
+  Value create_constant_float32(float v) { return scalar_float(v, KAPY_F32); }
+  Value create_constant_float64(double v) { return scalar_float(v, -64); }
+  Value create_constant_zero(kapy_dtype type) { return type <= KAPY_F8E5M2 ? scalar_float(0.0, type) : scalar_int(0, type); }
+  Value create_constant_all_ones(kapy_dtype type) {
+    if (type <= KAPY_F8E5M2) throw Error(KAPY_ERR_UNSUPPORTED, "constant_all_ones: integer types only");
+    return scalar_int(-1, type);
+  }
+  // the reference's form of splat: a scalar Value in, a tensor of its type out (element_type: a narrower type for an f64 / i64 scalar)
+  Value create_splat(Value scalar, int element_type = -1) {
+    const Node &sc = node(scalar);
+    if (sc.kind != Node::kScalar) throw Error(KAPY_ERR_VERIFY, "splat: operand must be a scalar constant");
+    const int dt = element_type >= 0 ? element_type : sc.dtype;
+    if (dt < 0) throw Error(KAPY_ERR_UNSUPPORTED, "splat: a 64-bit scalar needs the tensor's element type");
+    const bool to_float = dt <= KAPY_F8E5M2;
+    if (to_float != sc.scalar_is_float) throw Error(KAPY_ERR_VERIFY, "splat: scalar and tensor must both be float or both integer");
+    if (to_float) return create_splat((float)sc.scalar_f, (kapy_dtype)dt);
+    return create_splat((int32_t)sc.scalar_i, (kapy_dtype)dt);
+  }
+
   // kapy.arange (ir.cc:730-743): i32 values start, start + 1, ... along `axis`, shape [end - start, 1] or [1, end - start];
   // inside a program it is the element's index along that axis plus start, broadcast over the other axis
   Value create_arange(unsigned axis, int32_t start, int32_t end) {
@@ -286,8 +319,14 @@ class OpBuilder {
   Value create_cos(Value source) { return unary(KAPY_EW_COS, source); }
   // create_elementwise_extern_lib (ir.cc:1168-1174): the library functions the path uses, by name
   Value create_elementwise_extern_lib(const std::string &name, Value source) {
-    if (name == "tanh") return unary(KAPY_EW_TANH, source);
-    if (name == "gelu" || name == "gelu_tanh") return unary(KAPY_EW_GELU_TANH, source);
+    // (also under the names of the device library the reference links, symName of ir.cc:1168-1174)
+    static const struct { const char *name; int op; } known[] = {
+        {"tanh", KAPY_EW_TANH}, {"__nv_tanhf", KAPY_EW_TANH}, {"gelu", KAPY_EW_GELU_TANH}, {"gelu_tanh", KAPY_EW_GELU_TANH},
+        {"__nv_expf", KAPY_EW_EXP}, {"__nv_exp2f", KAPY_EW_EXP2}, {"__nv_logf", KAPY_EW_LOG}, {"__nv_log2f", KAPY_EW_LOG2}, {"__nv_sqrtf", KAPY_EW_SQRT},
+        {"__nv_rsqrtf", KAPY_EW_RSQRT}, {"__nv_erff", KAPY_EW_ERF}, {"__nv_sinf", KAPY_EW_SIN}, {"__nv_cosf", KAPY_EW_COS}, {"__nv_floorf", KAPY_EW_FLOOR},
+        {"__nv_ceilf", KAPY_EW_CEIL}, {"__nv_fabsf", KAPY_EW_ABSF}};
+    for (const auto &k : known)
+      if (name == k.name) return unary(k.op, source);
     throw Error(KAPY_ERR_UNSUPPORTED, "elementwise_extern_lib: unknown function " + name);
   }
 
@@ -318,13 +357,16 @@ class OpBuilder {
 
  private:
   struct Node {
-    enum Kind { kGlobal, kLoad, kOp, kMatmul } kind = kOp;
+    enum Kind { kGlobal, kLoad, kOp, kMatmul, kScalar } kind = kOp;
     kapy_global global{};
     int op = -1, a = -1, b = -1, c = -1, dtype = KAPY_F32, rmode = KAPY_RN, axis = 1;
     int padding = KAPY_PAD_ZERO, cache = KAPY_CACHE_NONE, evict = KAPY_EVICT_NORMAL, impl_way = KAPY_MATMUL_AUTO;
     bool transposed = false, is_volatile = false;
     float imm = 0.f;
     int ival = 0, pred = 0;  // an integer splat's value or arange's start; a compare's predicate
+    bool scalar_is_float = false;  // kScalar: a constant that create_splat turns into a tensor
+    double scalar_f = 0.0;
+    int64_t scalar_i = 0;
   };
   std::vector<Node> nodes_;
   void *stream_;
@@ -344,7 +386,23 @@ class OpBuilder {
     if (node(v).kind != Node::kGlobal) throw Error(KAPY_ERR_VERIFY, std::string(what) + ": operand must be a global-memory tensor");
     return node(v).global;
   }
+  Value scalar_float(double v, int dtype) {
+    Node n;
+    n.kind = Node::kScalar;
+    n.dtype = dtype;
+    n.scalar_is_float = true;
+    n.scalar_f = v;
+    return push(n);
+  }
+  Value scalar_int(int64_t v, int dtype) {
+    Node n;
+    n.kind = Node::kScalar;
+    n.dtype = dtype;
+    n.scalar_i = v;
+    return push(n);
+  }
   int tensor(Value v, const char *what) const {
+    if (node(v).kind == Node::kScalar) throw Error(KAPY_ERR_VERIFY, std::string(what) + ": operand must be a tensor (splat the scalar first)");
     if (node(v).kind == Node::kGlobal) throw Error(KAPY_ERR_VERIFY, std::string(what) + ": operand must be a register tensor (ld_global it first)");
     return v.id_;
   }

@@ -84,6 +84,27 @@ static int run_cpu() {
       EXPECT(e.status == KAPY_ERR_VERIFY && strstr(e.what(), "i1"));
     }
   }
+  // scalar constants are splat as in the reference (create_constant_* then create_splat), and library functions answer to
+  // the names of the device library the reference links
+  {
+    kapy::Value half = b.create_splat(b.create_constant_float16(0.5f)), three = b.create_splat(b.create_constant_int32(3));
+    prog = b.program_of(b.create_mulf(lx, half));
+    EXPECT(prog.size() == 4 && prog[1].op == KAPY_EW_SPLAT && prog[1].dtype == KAPY_F16 && prog[1].imm == 0.5f && prog[2].op == KAPY_EW_MULF);
+    prog = b.program_of(b.create_sitofp(b.create_addi(three, b.create_splat(b.create_constant_all_ones(KAPY_I32))), KAPY_F16));
+    EXPECT(prog[0].op == KAPY_EW_SPLAT && prog[0].a == 3 && prog[1].op == KAPY_EW_SPLAT && prog[1].a == -1 && prog[2].op == KAPY_EW_ADDI);
+    prog = b.program_of(b.create_addf(lx, b.create_splat(b.create_constant_float64(0.25), KAPY_F16)));   // a 64-bit scalar names its tensor type
+    EXPECT(prog[1].op == KAPY_EW_SPLAT && prog[1].dtype == KAPY_F16 && prog[1].imm == 0.25f);
+    prog = b.program_of(b.create_addf(lx, b.create_splat(b.create_constant_zero(KAPY_F16))));
+    EXPECT(prog[1].op == KAPY_EW_SPLAT && prog[1].imm == 0.f);
+    prog = b.program_of(b.create_elementwise_extern_lib("__nv_tanhf", b.create_elementwise_extern_lib("__nv_expf", lx)));
+    EXPECT(prog.size() == 4 && prog[1].op == KAPY_EW_EXP && prog[2].op == KAPY_EW_TANH);
+    int refused = 0;
+    try { b.create_splat(b.create_constant_int64(1)); } catch (const kapy::Error &e) { refused += e.status == KAPY_ERR_UNSUPPORTED; }
+    try { b.create_splat(b.create_constant_float32(1.f), KAPY_I32); } catch (const kapy::Error &e) { refused += e.status == KAPY_ERR_VERIFY; }
+    try { b.create_addf(lx, b.create_constant_float16(1.f)); } catch (const kapy::Error &e) { refused += e.status == KAPY_ERR_VERIFY; }
+    try { b.create_elementwise_extern_lib("__nv_lgammaf", lx); } catch (const kapy::Error &e) { refused += e.status == KAPY_ERR_UNSUPPORTED; }
+    EXPECT(refused == 4);
+  }
   // the verifier's refusal arrives as an exception with the reference's wording
   try {
     kapy::Value h = b.create_ld_global(x), w = b.create_ld_global(b.create_mk_global(fake, 0, 64, 256, 256, 1, KAPY_BF16));

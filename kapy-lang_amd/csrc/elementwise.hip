@@ -341,7 +341,7 @@ __global__ __launch_bounds__(256) void affine_act_kernel(AffineActParams p) {
       const int valid = RAGGED ? p.width - col[u] : 8;
       xv[u] = load_row16<RAGGED>(p.x + ((int64_t)row[u] * p.x_stride0 + col[u]) * 2, valid, kEwNt);
       if (p.bias_mode == kBiasRow) bv[u] = load_row16<RAGGED>(p.bias + (int64_t)col[u] * 2, valid, false);
-      else if (p.bias_mode == kBiasFull) bv[u] = load_row16<RAGGED>(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2, valid, false);
+      else if (p.bias_mode == kBiasFull) bv[u] = load_row16<RAGGED>(p.bias + ((int64_t)row[u] * p.bias_stride0 + col[u]) * 2, valid, kEwNt);  // (read once, like x)
       else if (p.bias_mode == kBiasCol) {
         uint32_t h = *(const uint16_t *)(p.bias + (int64_t)row[u] * p.bias_stride0 * 2);
         h |= h << 16;

@@ -36,7 +36,9 @@
 
 // Workspace of a split K for callers that cannot bring one (kapy_matmul_static_workspace): arrival counters, then
 // partial sums.  Part of the device image, so every GPU the library runs on holds its own copy until the process ends;
-// zero when the image is loaded, and every kernel that uses the counters leaves them zero.
+// zero when the image is loaded, and every kernel that uses the counters leaves them zero.  (A launch the runtime refuses has
+// not run and leaves them as they were; a kernel that dies on the way takes the process's context with it, array included: there
+// is no state in between for the host to repair.)
 static __device__ __align__(256) unsigned char scratch[kapy::kSplitCounterBytes + (16 << 20)];
 
 namespace kapy {

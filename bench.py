@@ -1015,8 +1015,8 @@ TRAFFIC_KERNELS = [
     ("gemm_bf16_gelu", "C4 gemm bf16 8192^3 + gelu", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, true>[(]", None)]),
     ("f8_m4096", "C5 W8A8 M=4096", [(r"tn_kernel<kapy::F8M16<0, 0>, 256, 256, 128", None)]),
     ("f8_m16", "C5 W8A8 M=16", [(r"skinny_stream_kernel<", None)]),
-    ("f8_m64", "W8A8 M=64", [(r"skinny_block_kernel<", 256 * 256)]),
-    ("f8_m128", "W8A8 M=128", [(r"skinny_block_kernel<", 512 * 256)]),
+    ("f8_m64", "W8A8 M=64", [(r"skinny_block_kernel<0, 0, 4>", None)]),
+    ("f8_m128", "W8A8 M=128", [(r"skinny_block_kernel<0, 0, 8>", None)]),
     ("f8_m128_splitk", "W8A8 M=128, K split over workgroups", [(r"tn_kernel<kapy::F8M16<0, 0>, 128, 128, 128", None)]),
     ("gemm_f16", "C1 gemm fp16 1024^3", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),
     ("gemm_f16_graph", "C1 gemm fp16 1024^3, replayed from a graph", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),

@@ -190,11 +190,12 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 // so that the 16 rows a quarter-wave reads fall into 16 different bank groups.
 // Rows past M / N are clamped to the last valid row (never stored), so nothing is read out of range.
 // Which kernel serves how many rows (thresholds measured at N = K = 8192).  Up to 16 rows: the streaming kernel below.
-// From 17 rows: the block streaming kernel (32 columns x up to 64 rows per workgroup, the weight read once), where K is a
+// From 17 rows: the block streaming kernel (32 columns x up to 128 rows per workgroup, the weight read once), where K is a
 // multiple of 512; it yields to the tiled MFMA kernel from kTiledFromM rows, or from kTiledFromMSplit when the caller's
-// workspace lets the tiled kernel split K across workgroups.  Where the block kernel cannot run, the streaming kernel
+// workspace lets the tiled kernel split K across workgroups (N = K = 8192, M = 65 / 80 / 96 / 112 / 128: block kernel 20.7 /
+// 22.2 / 24.8 / 27.3 / 29.4 us, split tiled kernel 27.7 / 27.7 / 28.3 / 28.3 / 29.0).  Where the block kernel cannot run, the streaming kernel
 // (which reads the weight once per 16 rows) is all there is below the tiled kernel, and the tiled kernel takes over earlier.
-constexpr int kTiledFromM = 161, kTiledFromMSplit = 65;
+constexpr int kTiledFromM = 161, kTiledFromMSplit = 113;
 constexpr int kTiledFromMNoBlock = 81, kTiledFromMSplitNoBlock = 40;
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
 // NG: groups of 16 columns a wave multiplies with one activation chunk (a stage is then NG weight parts and one activation part
@@ -311,10 +312,10 @@ __global__ __launch_bounds__(64 * kStreamWaves) void skinny_stream_kernel(F8Para
   }
 }
 
-// Block streaming kernel: the same idea for 17 .. 64 rows of lhs (and, in blocks of 64 rows, beyond).  Reading the
+// Block streaming kernel: the same idea for 17 .. 128 rows of lhs (and, in blocks of 64 rows, beyond).  Reading the
 // weight once per 16 rows, as the kernel above does, asks the L2 for it M/16 times, and a workgroup of 16 columns re-reads
 // the whole activation: at M = 64 the activation traffic is four times the weight's.  Here a workgroup owns 32 columns and
-// 16*RG rows, so at N = 8192 there is one workgroup per CU, every weight byte crosses the fabric once, and the activation
+// 16*RG rows (RG = 2 .. 8), so at N = 8192 there is one workgroup per CU, every weight byte crosses the fabric once, and the activation
 // (M x K bytes, L2-resident) is read N/32 times.  Its 4 waves split K and work alone on private rings of kBlockStages
 // stages; a stage is one 128-byte K step: 32 weight rows and 16*RG activation rows of 128 contiguous bytes, brought in by
 // LDS-direct loads of 8 rows each, 16-byte chunk c of row r stored at chunk c ^ block_key(r % 16) - the 16 lanes of a
@@ -323,7 +324,7 @@ constexpr int kBlockStep = 128, kBlockCols = 32;
 // (the lanes of one phase of a 16-byte LDS read are 0-3, 12-15, 20-23, 24-27 and so on: rows r16 = 0-3 and 12-15 of one K
 // group with rows 4-11 of the next; with this key they fall into 16 different groups of four banks)
 __device__ __forceinline__ constexpr int block_key(int r) { return (r & 7) ^ ((r >> 3) & 1); }
-constexpr int block_stages(int) { return 3; }  // (four for 32 rows fits the LDS too and measured no faster)
+constexpr int block_stages(int rg) { return rg >= 5 ? 2 : 3; }  // (four for 32 rows fits the LDS too and measured no faster; 80 rows and more leave room for two)
 constexpr int waitcnt_vm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }  // s_waitcnt vmcnt(n), nothing else waited for
 template <int A_FMT, int B_FMT, int RG>
 __global__ __launch_bounds__(256) void skinny_block_kernel(F8Params p) {
@@ -483,7 +484,7 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
   kapy_matmul_cfg c = {KAPY_MATMUL_AUTO, 0, 0, 0, KAPY_RN, 0, 0, 0, nullptr, 0};
   if (cfg) c = *cfg;
   // (offsets inside a workgroup's rows and columns are 32-bit)
-  const bool block_ok = k_contig && p.M > 16 && p.K % (4 * kBlockStep) == 0 && p.a_sm * 64 < (int64_t(1) << 31) && p.b_sn * kBlockCols < (int64_t(1) << 31) &&
+  const bool block_ok = k_contig && p.M > 16 && p.K % (4 * kBlockStep) == 0 && p.a_sm * 128 < (int64_t(1) << 31) && p.b_sn * kBlockCols < (int64_t(1) << 31) &&
                         ((int64_t)(p.N + kBlockCols - 1) / kBlockCols + 8) * ((p.M + 31) / 32) < (int64_t(1) << 31);
   if (k_pieces && !acc && (result->dtype == KAPY_BF16 || result->dtype == KAPY_F16 || result->dtype == KAPY_F32)) {
     GemmParams g;
@@ -506,7 +507,14 @@ int matmul_f8(const kapy_global *a, const kapy_global *b, const float *row_scale
     const int fa = fmt_of(a->dtype), fb = fmt_of(b->dtype);
     if (p.M <= 32) return launch_skinny_block<2>(p, fa, fb, s);
     if (p.M <= 48) return launch_skinny_block<3>(p, fa, fb, s);
-    return launch_skinny_block<4>(p, fa, fb, s);
+    // 65 .. 128 rows: one block of rows per workgroup still (two stages of up to 20 KiB per wave).  Two blocks of 64 rows would
+    // read the weight twice through the L2s and the activation as often; N = K = 8192, M = 80 / 96 / 128: 30.0 / 30.6 / 33.8 us
+    // in blocks of 64 rows, 25.2 / 26.5 / 29.5 in one of 128.  Beyond 128 rows: blocks of 64.
+    if (p.M <= 64 || p.M > 128) return launch_skinny_block<4>(p, fa, fb, s);
+    if (p.M <= 80) return launch_skinny_block<5>(p, fa, fb, s);
+    if (p.M <= 96) return launch_skinny_block<6>(p, fa, fb, s);
+    if (p.M <= 112) return launch_skinny_block<7>(p, fa, fb, s);
+    return launch_skinny_block<8>(p, fa, fb, s);
   }
   if (k_contig && p.K % (kStreamWaves * kStreamChunk) == 0 && (p.M + 15) / 16 <= 65535 && p.a_sm * 16 < (int64_t(1) << 31) &&
       p.b_sn * 16 < (int64_t(1) << 31)) {

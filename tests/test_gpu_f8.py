@@ -44,11 +44,12 @@ def test_scaled_f8_small(ko, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 64, 512), (32, 96, 1024), (33, 100, 1536), (48, 32, 512), (49, 40, 2048), (64, 256, 4096), (24, 1000, 512),
-                                   (64, 8, 512)])
+                                   (64, 8, 512), (65, 64, 512), (80, 96, 1024), (81, 40, 512), (100, 100, 1536), (112, 32, 512), (113, 72, 1024),
+                                   (128, 256, 2048), (129, 64, 512), (160, 48, 1024)])
 @pytest.mark.parametrize("formats", [(0, 0), (1, 0)])
 def test_scaled_f8_block_streaming_kernel(ko, M, N, K, formats):
-    """17 .. 64 rows with K a multiple of 512: 32 columns x 32 / 48 / 64 rows per workgroup (row and column blocks that hang
-    over M and N included), both operand formats in the first slot; and the plain matmul with an f32 result through it."""
+    """17 .. 160 rows with K a multiple of 512: 32 columns x 32 / 48 / ... / 128 rows per workgroup, beyond 128 rows blocks of
+    64 (row and column blocks that hang over M and N included), both operand formats in the first slot."""
     fa = (ko.F8E4M3, ko.F8E5M2)[formats[0]]
     aq, sa, wq, sb = _quantised(ko, M, N, K, seed=7)
     if formats[0]:      # the same values re-encoded as e5m2

@@ -620,12 +620,15 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   for (int i = 0; i < C::kLoadsAPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
+    // (the builds without bounded loads fetch the operand's last row in place of rows past its end: results nobody stores)
+    if constexpr (STAGES != kRing25) row = min(row, (uint32_t)max(p.M - 1 - tm * BM, 0));
     a_goff[i] = (uint32_t)((row * p.a_sm + chunk * (16 / EB)) * EB);
   }
 #pragma unroll
   for (int i = 0; i < C::kLoadsBPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
+    if constexpr (STAGES != kRing25) row = min(row, (uint32_t)max(p.N - 1 - tn * BN, 0));
     b_goff[i] = (uint32_t)((row * p.b_sn + chunk * (16 / EB)) * EB);
   }
   const char *a_tile = p.a + (int64_t)m0 * p.a_sm * EB;
@@ -1636,7 +1639,9 @@ int launch_tn_epi(GemmParams p, hipStream_t s) {
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES>
 int launch_tn(const GemmParams &p, hipStream_t s) {
   // a result that ends inside a 16-byte piece of a row takes the bounds-checked element stores
-  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || (STAGES == kRing25 && p.N % 8 == 0);
+  // (tiles that hang over the edge: the ring builds' loads are bounded, the others fetch the last row again; the strip stores
+  // are bounded for all of them)
+  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || p.N % 8 == 0;
   const bool packed = packed_epilogue(p) && whole_tiles;
   if (host_has_tail(p)) {
     // a fused elementwise tail: the ring kernels on the 16x16 instruction have builds with it in the packed epilogue,
@@ -1806,6 +1811,12 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, int want_tile
     // (measured at N = K = 8192: 192 of the large tiles on 256 CUs already beat 768 of the small ones, 128 do not)
     if (want_tile == 256 || (want_tile == 0 && (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 >= (int64_t)device_cus() * 55))
       return launch_f8<F8M16, 256, 256, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
+    // At most one 128 x 128 tile per CU and K not split: the ring build's 2.5 tiles of loads in flight are sized for two
+    // workgroups per CU, and one alone waits for them (N = K = 8192, 161 .. 512 rows: 50 us whatever M is).  The four-stage
+    // build has three tiles (96 KiB) in flight per workgroup: 35.6 / 36.4 / 40.0 / 41.6 / 44 us at 161 / 192 / 256 / 384 / 512
+    // rows (five stages measured the same).  It fetches the last row again for rows past an operand's end.
+    if (want_tile == 0 && p.split_k <= 1 && p.K % 128 == 0 && (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) <= device_cus())
+      return launch_f8<F8, 128, 128, 128, 2, 2, 4>(p, lhs_fmt, rhs_fmt, s);
     return launch_f8<F8M16, 128, 128, 128, 2, 2, kRing25>(p, lhs_fmt, rhs_fmt, s);
   }
   if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 256) * 2 >= device_cus())

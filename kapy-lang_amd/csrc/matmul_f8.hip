@@ -193,9 +193,10 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_kernel(F8Params p) {
 // From 17 rows: the block streaming kernel (32 columns x up to 128 rows per workgroup, the weight read once), where K is a
 // multiple of 512; it yields to the tiled MFMA kernel from kTiledFromM rows, or from kTiledFromMSplit when the caller's
 // workspace lets the tiled kernel split K across workgroups (N = K = 8192, M = 65 / 80 / 96 / 112 / 128: block kernel 20.7 /
-// 22.2 / 24.8 / 27.3 / 29.4 us, split tiled kernel 27.7 / 27.7 / 28.3 / 28.3 / 29.0).  Where the block kernel cannot run, the streaming kernel
+// 22.2 / 24.8 / 27.3 / 29.4 us, split tiled kernel 27.7 / 27.7 / 28.3 / 28.3 / 29.0; 144 / 160 rows: blocks of 64 rows 44 us,
+// the tiled kernel's four-stage build 35 us).  Where the block kernel cannot run, the streaming kernel
 // (which reads the weight once per 16 rows) is all there is below the tiled kernel, and the tiled kernel takes over earlier.
-constexpr int kTiledFromM = 161, kTiledFromMSplit = 113;
+constexpr int kTiledFromM = 129, kTiledFromMSplit = 113;
 constexpr int kTiledFromMNoBlock = 81, kTiledFromMSplitNoBlock = 40;
 constexpr int kStreamWaves = 4, kStreamChunk = 256, kStreamStage = 2 * 16 * kStreamChunk, kStreamStages = 2;
 // NG: groups of 16 columns a wave multiplies with one activation chunk (a stage is then NG weight parts and one activation part

@@ -67,7 +67,8 @@ def test_scaled_f8_block_streaming_kernel(ko, M, N, K, formats):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 128), (128, 256, 384), (256, 256, 256), (384, 128, 512), (512, 768, 1024), (1024, 2560, 256),
-                                   (300, 520, 256), (1000, 136, 384), (129, 1001, 128), (300, 520, 272), (256, 256, 144)])   # tiles hang over the edges of M, N and K
+                                   (300, 520, 256), (1000, 136, 384), (129, 1001, 128), (300, 520, 272), (256, 256, 144),   # tiles hang over the edges of M, N and K
+                                   (161, 8192, 256), (192, 4096, 512), (320, 2056, 128), (500, 8192, 128)])   # at most one tile per CU: the four-stage build
 def test_scaled_f8_tiled_kernel(ko, M, N, K):
     """Rows >= 128 and extents multiples of the tile: the LDS-direct MFMA kernel (128- and 256-wide tiles)."""
     aq, sa, wq, sb = _quantised(ko, M, N, K, seed=3)

@@ -620,15 +620,16 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
   for (int i = 0; i < C::kLoadsAPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
-    // (the builds without bounded loads fetch the operand's last row in place of rows past its end: results nobody stores)
-    if constexpr (STAGES != kRing25) row = min(row, (uint32_t)max(p.M - 1 - tm * BM, 0));
+    // (the 128-wide builds without bounded loads fetch the operand's last row in place of rows past its end: results nobody
+    // stores; the 256-wide ones are only given whole tiles)
+    if constexpr (STAGES != kRing25 && BM == 128) row = min(row, (uint32_t)max(p.M - 1 - tm * BM, 0));
     a_goff[i] = (uint32_t)((row * p.a_sm + chunk * (16 / EB)) * EB);
   }
 #pragma unroll
   for (int i = 0; i < C::kLoadsBPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
-    if constexpr (STAGES != kRing25) row = min(row, (uint32_t)max(p.N - 1 - tn * BN, 0));
+    if constexpr (STAGES != kRing25 && BN == 128) row = min(row, (uint32_t)max(p.N - 1 - tn * BN, 0));
     b_goff[i] = (uint32_t)((row * p.b_sn + chunk * (16 / EB)) * EB);
   }
   const char *a_tile = p.a + (int64_t)m0 * p.a_sm * EB;
@@ -1641,7 +1642,7 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
   // a result that ends inside a 16-byte piece of a row takes the bounds-checked element stores
   // (tiles that hang over the edge: the ring builds' loads are bounded, the others fetch the last row again; the strip stores
   // are bounded for all of them)
-  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || p.N % 8 == 0;
+  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || ((STAGES == kRing25 || BM == 128) && p.N % 8 == 0);
   const bool packed = packed_epilogue(p) && whole_tiles;
   if (host_has_tail(p)) {
     // a fused elementwise tail: the ring kernels on the 16x16 instruction have builds with it in the packed epilogue,

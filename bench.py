@@ -743,7 +743,7 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     if ("wdev", N, K) not in _dev_cache:
         _dev_cache[("wdev", N, K)] = _upload(wq)
     w0 = _dev_cache[("wdev", N, K)]
-    sets = 6 if M <= 128 else 1                # M<=64 is weight-streaming: 6 x 64 MiB > Infinity Cache (copies of the same weight)
+    sets = 6 if M <= 512 else 1                # few rows: weight-streaming: 6 x 64 MiB > Infinity Cache (copies of the same weight)
     ws = [w0] + [w0.clone() for _ in range(sets - 1)]
     d = torch.empty(M * N, device="cuda", dtype=torch.int16)
     ga = kh.mk_global(a.data_ptr(), M, K, K, 1, kh.F8E4M3)
@@ -769,10 +769,10 @@ def bench_f8(kh, steps, warmup, cpu, M, workspace=False):
     flops = 2.0 * M * N * K
     nbytes = M * K + N * K + M * N * 2 + (M + N) * 4
     out = {"workload": "C5 W8A8 e4m3 M=%d N=K=8192%s" % (M, ", K split across workgroups (workspace given)" if workspace else ""), "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 160 and not workspace)) else "tn_kernel<F8M16, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8>",
+           "ms_per_step": wall, "kernel_ms": ev, "dtype": "f8e4m3", "kernel": "skinny_stream_kernel" if M <= 16 else "skinny_block_kernel" if (M <= 64 or (M <= 128 and not workspace)) else "tn_kernel<F8M16, 128x128x128> split K" if (workspace and M <= 128) else "tn_kernel<F8, 128x128x128, four stages>" if M <= 512 else "tn_kernel<F8>",
            "inputs": "normal(0,1) fp32 (A seed 0, W seed 1) quantised to e4m3 with per-row / per-column scales amax/448 (as the configuration states)",
            "checked": True, "check": "%s: relative Frobenius error %.2e (tolerance %.0e)" % (whole, rel, FROB_TOL)}
-    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d%s" % (M, "_splitk" if workspace else "")) if M <= 128 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
+    out["roofline"] = _roof_hbm(nbytes, ev, "f8_m%d%s" % (M, "_splitk" if workspace else "")) if M <= 512 else _roof_mfma(flops, ev, "f8", "f8_m%d" % M)
     if cpu:
         rows = min(M, 1024)
         hd = np.zeros(M * N, np.uint16)
@@ -986,7 +986,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
 
 
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "causal_softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m4096", "mlir_fixtures", "ceilings"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m256", "f8_m4096", "mlir_fixtures", "ceilings"]
 
 
 # ---------------------------------------------------------------- HBM traffic summary from the profiler's counter files
@@ -1018,6 +1018,7 @@ TRAFFIC_KERNELS = [
     ("f8_m64", "W8A8 M=64", [(r"skinny_block_kernel<0, 0, 4>", None)]),
     ("f8_m128", "W8A8 M=128", [(r"skinny_block_kernel<0, 0, 8>", None)]),
     ("f8_m128_splitk", "W8A8 M=128, K split over workgroups", [(r"tn_kernel<kapy::F8M16<0, 0>, 128, 128, 128", None)]),
+    ("f8_m256", "W8A8 M=256", [(r"tn_kernel<kapy::F8<0, 0>, 128, 128, 128, 2, 2, 4", None)]),
     ("gemm_f16", "C1 gemm fp16 1024^3", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),
     ("gemm_f16_graph", "C1 gemm fp16 1024^3, replayed from a graph", [(r"nn_kernel<kapy::F16M16", 64 * 256)]),
     ("gemm_f16_splitk", "C1 gemm fp16 1024^3, K split two ways", [(r"nn_kernel<kapy::F16M16", 128 * 256)]),
@@ -1221,6 +1222,7 @@ def main():
         "f8_m64": lambda s, w: bench_f8(kh, s, w, False, 64),
         "f8_m128": lambda s, w: bench_f8(kh, s, w, False, 128),
         "f8_m128_splitk": lambda s, w: bench_f8(kh, s, w, False, 128, workspace=True),
+        "f8_m256": lambda s, w: bench_f8(kh, s, w, False, 256),
         "f8_m4096": lambda s, w: bench_f8(kh, s, w, cpu, 4096),
         "ceilings": lambda s, w: bench_ceilings(kh, s, w, cpu),
     }

@@ -1744,7 +1744,7 @@ struct TnVariant {
 const TnVariant kTnVariants[] = {
     KAPY_TN16(256, 256, 64, 2, 2, kRing25), KAPY_TN16(256, 256, 64, 2, 2, 2),
     KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN16(128, 128, 64, 2, 2, kRing25),
-    KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4),
+    KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 4),
 };
 
 int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
@@ -1965,6 +1965,12 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
       if (v.bm == 128 && v.stages == kRing25) {
         rc = plan_split_k(p, c, v.bk);
         if (rc) return rc;
+        // Tiles for at most half the CUs and K not split: a workgroup alone on its CU waits for the ring's 2.5 tiles of loads.
+        // The four-stage build on the 32-row instruction keeps three tiles in flight: bf16 N = K = 8192, 128 / 256 rows
+        // 54 / 55 -> 48 / 52 us (level at 384 rows, behind from 512; the same depth on the 16-row instruction: 71 us).
+        if (free_choice && p.split_k <= 1 && !host_has_tail(p) && p.K % 64 == 0 && p.N % 8 == 0 &&
+            (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * 2 <= device_cus())
+          return bf16 ? launch_tn<Bf16, 128, 128, 64, 2, 2, 4>(p, s) : launch_tn<F16, 128, 128, 64, 2, 2, 4>(p, s);
       } else if (c.split_k > 1 && c.tile_m) {
         return fail(KAPY_ERR_UNSUPPORTED, "matmul: only the 128 x 128 tiles split K");
       }

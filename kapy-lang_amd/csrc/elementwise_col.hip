@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void col_softmax_stats_kernel(ColSoftmax p, in
   for (int e = 0; e < 8; ++e) { m[e] = -__builtin_inff(); s[e] = 0.f; }
   if (col0 < p.cols) {
     const char *col = p.x + (int64_t)col0 * 2;
-    constexpr int U = 4;
+    constexpr int U = 8;
     int32_t r = r_begin + rg;
     for (; r + kRowGroups * (U - 1) < r_end; r += kRowGroups * U) {
       u32x4_t v[U];

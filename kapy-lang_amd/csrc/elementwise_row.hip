@@ -85,18 +85,16 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(FusedRow p, int dtype)
 #pragma unroll
     for (int c = 0; c < CH; ++c) widen16x8(raw[c], dtype, f[c]);
     if (WALK && i + (int32_t)gridDim.x < p.rows) row_fetch<CH, THREADS, true>(p.x + (int64_t)(i + gridDim.x) * p.x_stride0 * 2, p.vec_per_row, raw);
+    // (a NaN is skipped by the maximum; its exponential below is NaN, so is the row's sum, and with it every quotient of the
+    // row - what a NaN maximum would have made of them)
     float m = -__builtin_inff();
-    bool any_nan = false;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
       if (c * THREADS + (int)threadIdx.x < p.vec_per_row) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          m = fmaxf(m, f[c][e]);
-          any_nan |= f[c][e] != f[c][e];
-        }
+        for (int e = 0; e < 8; ++e) m = fmaxf(m, f[c][e]);
       }
-    m = row_fold<THREADS, true>(any_nan ? __builtin_nanf("") : m, red[0]);
+    m = row_fold<THREADS, true>(m, red[0]);
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {

@@ -617,7 +617,7 @@ def _cpu_gemm(ko, go_a, go_b, go_d, rows, N, K, scales, what):
             "sample": "%s; fp32 accumulate, operands widened to fp32 and packed outside the timed multiply; %d repetitions, %.2f s of multiplying" % (what, reps, tot)}
 
 
-def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None, workspace=False, whole=True):
+def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel, tile=(0, 0, 0), graph_of=0, fused_gelu=False, gen="normal", key=None, workspace=False, whole=True, a_col_major=False):
     """whole: gate the whole result against the host GEMM as well as 16 blocks against the fp64 checker (a second and third large
     problem of the same shape are gated on the blocks alone: the host GEMM takes its time).
     graph_of > 0: that many back-to-back launches recorded once into a HIP graph; a step is one replay, figures are per launch
@@ -639,10 +639,11 @@ def bench_gemm(kh, steps, warmup, cpu, M, N, K, dtype, b_col_major, name, kernel
         what = "A normal(0,0.02) seed 0, B normal(0,0.02) seed 1"
     d = torch.empty(M * N, device="cuda", dtype=torch.int16)
     b_str = (1, K) if b_col_major else (N, 1)
-    ga = kh.mk_global(a.data_ptr(), M, K, K, 1, dtype)
+    a_str = (1, M) if a_col_major else (K, 1)
+    ga = kh.mk_global(a.data_ptr(), M, K, a_str[0], a_str[1], dtype)
     gb = kh.mk_global(b.data_ptr(), K, N, b_str[0], b_str[1], dtype)
     gd = kh.mk_global(d.data_ptr(), M, N, N, 1, dtype)
-    go_a, go_b = ko.mk_global(ha, M, K, K, 1, dtype), ko.mk_global(hb, K, N, b_str[0], b_str[1], dtype)
+    go_a, go_b = ko.mk_global(ha, M, K, a_str[0], a_str[1], dtype), ko.mk_global(hb, K, N, b_str[0], b_str[1], dtype)
     if fused_gelu:
         hbias = _host("normal", N, dtype, 2)
         bias = _dev("normal", N, dtype, 2)
@@ -1213,8 +1214,8 @@ def main():
         "gemm_bf16": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 A row-major B col-major", "tn_kernel", key="gemm_bf16"),
         "gemm_bf16_gelu": lambda s, w: bench_gemm(kh, s, w, cpu, 8192, 8192, 8192, kh.BF16, True, "C4 gemm bf16 8192^3 with gelu_tanh(c*0.5 + bias) fused into the epilogue", "tn_kernel", fused_gelu=True, key="gemm_bf16_gelu"),
         "mlir_fixtures": lambda s, w: bench_mlir(kh, s, w, cpu),
-        "gemm_bf16_nn": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, read in place by transposing LDS reads (128 x 128 tiles)", "nn_kernel", key="gemm_bf16_nn", whole=False),
-        "gemm_bf16_nn_turned": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, workspace given: the rhs is turned K-contiguous first (time and rate include the turn)", "transpose_lds_kernel + tn_kernel", key="gemm_bf16_nn_turned", workspace=True, whole=False),
+        "gemm_bf16_nn": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, the rhs read in place by transposing LDS reads (256 x 256 tiles)", "nn256_kernel", key="gemm_bf16_nn", whole=False),
+        "gemm_bf16_nn_turned": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, True, "gemm bf16 8192^3, lhs column-major, rhs column-major, workspace given: the lhs is turned K-contiguous first (time and rate include the turn)", "transpose_lds_kernel + tn_kernel", key="gemm_bf16_nn_turned", workspace=True, whole=False, a_col_major=True),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform", key="gemm_f16"),
         "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform", key="gemm_f16_graph"),
         "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True, key="gemm_f16_splitk"),

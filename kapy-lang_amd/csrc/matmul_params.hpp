@@ -48,4 +48,9 @@ int matmul_f8_tiled(const GemmParams &p, int lhs_fmt, int rhs_fmt, int want_tile
 // cannot be honoured.
 int plan_split_k(GemmParams &p, const kapy_matmul_cfg &c, int tile_k);
 
+// 256 x 256 x 64 tiles for a row-major lhs and a row-major rhs (matmul_nn256.hip): whether the kernel serves the problem
+// (the strip epilogue's own conditions are the caller's to check), and its launch.
+bool nn256_serves(const GemmParams &p);
+int launch_nn256(GemmParams p, bool bf16, hipStream_t s);
+
 }  // namespace kapy

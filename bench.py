@@ -1014,6 +1014,7 @@ TRAFFIC_KERNELS = [
     ("layernorm", "layer norm fp16 8192^2", [(r"norm_kernel<", None)]),
     ("gemm_bf16", "C4 gemm bf16 8192^3", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, false>[(]", None)]),
     ("gemm_bf16_gelu", "C4 gemm bf16 8192^3 + gelu", [(r"tn_kernel<kapy::Bf16M16, 256, 256, 64, .*, true>[(]", None)]),
+    ("gemm_bf16_nn", "gemm bf16 8192^3, both operands row-major", [(r"nn256_kernel<kapy::Bf16M16", None)]),
     ("f8_m4096", "C5 W8A8 M=4096", [(r"tn_kernel<kapy::F8M16<0, 0>, 256, 256, 128", None)]),
     ("f8_m16", "C5 W8A8 M=16", [(r"skinny_stream_kernel<", None)]),
     ("f8_m64", "W8A8 M=64", [(r"skinny_block_kernel<0, 0, 4>", None)]),

@@ -32,7 +32,8 @@ __device__ __forceinline__ void tr_reads_wait8(u32x2_lds (&h0)[8], u32x2_lds (&h
                : "memory");
 }
 
-template <typename T>
+// TAIL: the build for calls with a fused elementwise tail (scale, bias, activation in the strip epilogue).
+template <typename T, bool TAIL = false>
 __global__ __launch_bounds__(256) void nn256_kernel(GemmParams p) {
   static_assert(T::kM == 16 && T::kBytes == 2, "16x16x32 instruction, 16-bit operands");
   using LA = TileLayout<kBK * 2, T, 16>;
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(256) void nn256_kernel(GemmParams p) {
   asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
   __builtin_amdgcn_s_barrier();  // every wave has left the stages: they are reused as staging space by the strip epilogue
   static_assert(PackedEpilogue<16, 128, 128>::kBytesPerWave * 4 <= 2 * kStageBytes, "a strip per wavefront must fit the stages");
-  PackedEpilogue<16, 128, 128>::run(p, acc, lds + wave * PackedEpilogue<16, 128, 128>::kBytesPerWave, m0 + wm * 128, n0 + wn * 128, lane);
+  PackedEpilogue<16, 128, 128>::template run<TAIL>(p, acc, lds + wave * PackedEpilogue<16, 128, 128>::kBytesPerWave, m0 + wm * 128, n0 + wn * 128, lane);
 }
 
 }  // namespace
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(256) void nn256_kernel(GemmParams p) {
 bool nn256_serves(const GemmParams &p) {
   return p.a_sk == 1 && p.b_sn == 1 && p.M % kBM == 0 && p.N % kBN == 0 && p.K % kBK == 0 && p.K >= 2 * kBK && p.a_sm % 8 == 0 && p.b_sk % 8 == 0 &&
          ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.a_sm > 0 && p.b_sk > 0 && p.a_sm * 2 * kBM < (int64_t(1) << 31) &&
-         (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31) && p.bias == nullptr && p.act < 0 && p.alpha == 1.0f;
+         (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31);
 }
 
 int launch_nn256(GemmParams p, bool bf16, hipStream_t s) {
@@ -230,8 +231,14 @@ int launch_nn256(GemmParams p, bool bf16, hipStream_t s) {
   }
   if (state < 0) return fail(KAPY_ERR_HIP, "matmul: the runtime does not give this kernel the %d bytes of LDS it addresses (nothing was launched)", 2 * kStageBytes);
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1);
-  if (bf16) nn256_kernel<Bf16M16><<<grid, 256, 0, s>>>(p);
-  else nn256_kernel<F16M16><<<grid, 256, 0, s>>>(p);
+  const bool tail = p.bias != nullptr || p.act >= 0 || p.alpha != 1.0f;
+  if (tail) {
+    if (bf16) nn256_kernel<Bf16M16, true><<<grid, 256, 0, s>>>(p);
+    else nn256_kernel<F16M16, true><<<grid, 256, 0, s>>>(p);
+  } else {
+    if (bf16) nn256_kernel<Bf16M16><<<grid, 256, 0, s>>>(p);
+    else nn256_kernel<F16M16><<<grid, 256, 0, s>>>(p);
+  }
   KAPY_HIP_CHECK(hipGetLastError());
   return KAPY_OK;
 }

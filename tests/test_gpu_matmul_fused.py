@@ -76,6 +76,46 @@ def test_every_epilogue_path_carries_the_tail(ko, M, N, K, b_row_major, tile):
     _case(ko, kh.F16, M, N, K, b_row_major, kh.F32, 2.0, MAX, 0.0, tile=tile)
 
 
+@pytest.mark.parametrize("dt,bias_dt,alpha,act", [(kh.BF16, kh.BF16, 1.0, kh.EW_GELU_TANH), (kh.F16, kh.F32, 0.5, MAX), (kh.BF16, None, 2.0, -1)])
+def test_the_tail_on_256_wide_tiles_of_row_major_operands(ko, dt, bias_dt, alpha, act):
+    """Large row-major x row-major with a tail: the 256-wide kernel's build with the tail in its strip epilogue.  Against the
+    128-wide kernel (which applies the tail in its element stores; same accumulation order) <= 2 ulp, and sampled 64 x 64 blocks
+    against the checker's matmul + tail program."""
+    M, N, K = 3072, 3072, 192
+    a, b = ko.fill_normal(M * K, dt, 9, 0, 0.0, 0.25), ko.fill_normal(K * N, dt, 9, 1, 0.0, 0.25)
+    bias = ko.fill_normal(N, bias_dt, 9, 2, 0.0, 1.0) if bias_dt is not None else None
+    da, db = to_dev(a), to_dev(b)
+    dbias = to_dev(bias) if bias is not None else None
+    gb = dglobal(dbias, 1, N, N, 1, bias_dt) if bias is not None else None
+    outs = []
+    for tile in ((0, 0, 0), (128, 128, 64)):
+        dd = dev_zeros(M * N + 64, 2, fill=0x1234)
+        kh.matmul_fused(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt), dglobal(dd, M, N, N, 1, dt), bias=gb, alpha=alpha, act=act,
+                        act_operand=0.0, tile=tile)
+        sync()
+        got = to_host(dd, np.uint16)
+        assert np.all(got[M * N:] == 0x1234)
+        outs.append(got[:M * N].reshape(M, N))
+    assert np.all(np.isfinite(ko.decode(outs[0].ravel(), dt)))
+    assert ulp_diff_f16(outs[0].ravel(), outs[1].ravel()).max() <= 2
+    insts = _tail_program(dt, bias_dt, alpha, act, 0.0)
+    goa, gob = ko.mk_global(a, M, K, K, 1, dt), ko.mk_global(b, K, N, N, 1, dt)
+    for t in range(6):
+        r0, c0 = (t * 331 + 37 * (t % 4) * 16) % (M - 64), ((t * 577 + 128 * (t % 2)) % (N - 64)) // 8 * 8
+        c32 = np.zeros(64 * 64, np.float32)
+        assert ko.lib().ko_matmul(C.byref(ko.sv_global(goa, r0, r0 + 64, 0, K)), C.byref(ko.sv_global(gob, 0, K, c0, c0 + 64)), None,
+                                  C.byref(ko.mk_global(c32, 64, 64, 64, 1, kh.F32)), kh.RN) == 0
+        want = np.zeros(64 * 64, np.uint16)
+        o_ins = [ko.mk_global(c32.view(np.uint32), 64, 64, 64, 1, kh.F32)]
+        if bias is not None:
+            piece = np.ascontiguousarray(bias[c0:c0 + 64])
+            o_ins.append(ko.mk_global(piece, 1, 64, 64, 1, bias_dt))
+        assert ko.elementwise(ko.program(insts), o_ins, ko.mk_global(want, 64, 64, 64, 1, dt)) == 0
+        g, w = ko.decode(np.ascontiguousarray(outs[0][r0:r0 + 64, c0:c0 + 64]).ravel(), dt), ko.decode(want, dt)
+        rel = np.linalg.norm(g - w) / max(np.linalg.norm(w), 1e-30)
+        assert rel <= 1e-3, (t, rel)
+
+
 def test_parts_of_the_tail_alone_and_relu_really_clamps(ko):
     _case(ko, kh.BF16, 256, 256, 128, False, None, 0.125, -1)                  # scale only
     _case(ko, kh.BF16, 256, 256, 128, False, kh.BF16, 1.0, -1)                 # bias only

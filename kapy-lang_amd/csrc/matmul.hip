@@ -1331,6 +1331,25 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
   if (lhs->dtype != KAPY_F16 && lhs->dtype != KAPY_BF16)
     return fail(KAPY_ERR_UNSUPPORTED, "matmul: %s operands have no matrix instruction on gfx950", dtype_name(lhs->dtype));
 
+  // A column-major result: D^T = B^T . A^T is the same problem with a row-major result, which the strip epilogues store (a
+  // column-major one goes element by element).  Every dot product sums the same products in the same order, so the bits are
+  // those of the problem as given.  (A bias row would turn into a bias column, which no epilogue adds: such calls stay.)
+  if (result->stride0 == 1 && result->stride1 != 1 && extent0(result) > 1 && !(epi && epi->bias)) {
+    auto turned = [](const kapy_global &g) {
+      kapy_global t = g;
+      std::swap(t.start0, t.start1);
+      std::swap(t.end0, t.end1);
+      std::swap(t.stride0, t.stride1);
+      return t;
+    };
+    const kapy_global at = turned(*lhs), bt = turned(*rhs), dt = turned(*result);
+    kapy_global acct;
+    if (acc) acct = turned(*acc);
+    kapy_matmul_cfg inner = c;
+    std::swap(inner.tile_m, inner.tile_n);
+    return matmul_16bit(&bt, &at, acc ? &acct : nullptr, &dt, &inner, epi, stream);
+  }
+
   // A large problem with an operand that is contiguous along its OTHER extent (a row-major rhs, a column-major lhs).  The kernel
   // that reads such operands with transposing LDS reads works on 128 x 128 tiles and reaches 1.05-1.12 PFLOP/s where the
   // K-contiguous kernel's 256 x 256 tiles reach 1.35-1.55.  Turning the operand first costs one pass of the transposing copy
@@ -1347,7 +1366,7 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
     // (a row-major rhs beside a row-major lhs in whole 256 x 256 x 64 tiles is read in place by the 256-wide kernel of
     // matmul_nn256.hip, faster than turn and product together: 8192^3 bf16 0.683 ms against 0.727)
     const bool wide_in_place = b_turn && !a_turn && a_kc && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (M / 256) * (N / 256) * 100 >= (int64_t)device_cus() * 55 &&
-                               !epi && c.rmode == KAPY_RN;
+                               c.rmode == KAPY_RN;
     if (!wide_in_place && (a_turn || b_turn) && (a_turn || a_kc) && (b_turn || b_kc) && (!b_turn || M >= 6144) && (!a_turn || N >= 6144) && M >= 2048 && N >= 2048 && K >= 1024 &&
         M % 8 == 0 && N % 8 == 0 && K % 8 == 0 &&
         M * K < (int64_t(1) << 31) && K * N < (int64_t(1) << 31) && kSplitCounterBytes + a_bytes + b_bytes <= c.workspace_bytes &&

@@ -142,6 +142,43 @@ def test_accumulator_input_f32_out_and_column_major_result(ko):
     assert _frob(ko, got, want, kh.BF16) <= 2e-3   # RZ against RZ oracle; accumulation order differs
 
 
+@pytest.mark.parametrize("dt", [kh.F16, kh.BF16])
+@pytest.mark.parametrize("a_rm,b_rm", [(True, True), (True, False), (False, True), (False, False)])
+def test_column_major_result_is_the_transposed_problem(ko, dt, a_rm, b_rm):
+    """A column-major result is computed as D^T = B^T . A^T with a row-major result: against the checker, and bit for bit the
+    row-major result of the same call (every dot product sums the same products in the same order), with and without a
+    column-major fp32 accumulator input, on whole tiles and on ragged extents, and an explicit tile turned with the problem."""
+    for (M, N, K, tile) in ((256, 384, 128, (0, 0, 0)), (200, 136, 72, (0, 0, 0)), (130, 264, 104, (0, 0, 0)), (512, 256, 192, (128, 128, 64))):
+        if tile != (0, 0, 0) and not (a_rm and not b_rm):
+            continue   # (the explicit tile names the K-contiguous kernel)
+        a, b = ko.fill_normal(M * K, dt, 13, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 13, 1, 0.0, 0.5)
+        acc = ko.fill_normal(M * N, kh.F32, 13, 2, 0.0, 0.5)            # read as column-major [M x N] and as row-major [M x N] below
+        a_str, b_str = ((K, 1) if a_rm else (1, M)), ((N, 1) if b_rm else (1, K))
+        da, db, dacc = to_dev(a), to_dev(b), to_dev(acc)
+        acc_t = np.ascontiguousarray(acc.reshape(N, M).T).ravel()      # the same accumulator values laid out row-major
+        dacc_t = to_dev(acc_t)
+        for with_acc in (False, True):
+            out_dt = kh.F32 if with_acc else dt
+            ob = kh.DTYPE_BYTES[out_dt]
+            want = np.zeros(M * N, dtype=_np_store(out_dt))
+            assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, *a_str, dt)), C.byref(ko.mk_global(b, K, N, *b_str, dt)),
+                                      C.byref(ko.mk_global(acc, M, N, 1, M, kh.F32)) if with_acc else None,
+                                      C.byref(ko.mk_global(want, M, N, 1, M, out_dt)), kh.RN) == 0
+            d_col, d_row = dev_zeros(M * N + 64, ob, fill=0x1234), dev_zeros(M * N, ob)
+            kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(d_col, M, N, 1, M, out_dt),
+                      acc=dglobal(dacc, M, N, 1, M, kh.F32) if with_acc else None, tile=tile)
+            kh.matmul(dglobal(da, M, K, *a_str, dt), dglobal(db, K, N, *b_str, dt), dglobal(d_row, M, N, N, 1, out_dt),
+                      acc=dglobal(dacc_t, M, N, N, 1, kh.F32) if with_acc else None, tile=tile)
+            sync()
+            got = to_host(d_col, want.dtype)
+            bits = np.uint32 if ob == 4 else np.uint16
+            assert np.all(got[M * N:].view(bits) == 0x1234), (M, N, K)
+            got = got[:M * N]
+            assert _frob(ko, got, want, out_dt) <= (1e-5 if out_dt == kh.F32 else FROB_TOL), (M, N, K, with_acc)
+            row = to_host(d_row, want.dtype).reshape(M, N)
+            assert np.array_equal(got.reshape(N, M).T.view(bits), row.view(bits)), (M, N, K, with_acc)
+
+
 def test_subview_operands(ko):
     """matmul on sv_global views of larger buffers (start offsets, same strides)."""
     M, N, K = 128, 128, 96

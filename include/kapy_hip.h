@@ -334,8 +334,9 @@ typedef struct kapy_matmul_cfg {
 typedef enum kapy_matmul_accumulate { KAPY_ACCUMULATE_F32 = 0, KAPY_ACCUMULATE_ELEMENT = 1 } kapy_matmul_accumulate;
 /* Workspace size that lets the library split K for an [m x n] result whichever way it chooses. */
 int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n);
-/* Workspace size with which a LARGE 16-bit problem (at least 6144 rows for a row-major rhs, at least 6144 columns for a
- * column-major lhs, at least 2048 of the other, K at least 1024, all multiples of 8) is multiplied by first turning that
+/* Workspace size with which a LARGE 16-bit problem (at least 6144 rows for a row-major rhs - unless the lhs is row-major
+ * too and the sizes are whole 256 x 256 x 64 tiles, which a kernel of its own multiplies in place -, at least 6144 columns
+ * for a column-major lhs, at least 2048 of the other, K at least 1024, all multiples of 8) is multiplied by first turning that
  * operand into the workspace (behind the 16 KiB of counters, which stay zero) with the transposing copy and then running
  * the K-contiguous kernel on 256 x 256 tiles: 1.15 - 1.2 x the rate of the kernel that reads such operands in place on
  * 128 x 128 tiles, the extra pass over the operand included.  0 when neither operand needs turning.  Used only with a free tile choice and no explicit split; a smaller
@@ -347,7 +348,9 @@ int64_t kapy_matmul_turn_workspace_bytes(const kapy_global *lhs, const kapy_glob
  * lib/Dialect/Kapy/IR/Kapy.cpp:451-574; lowering MatmulOpToLLVM.cpp:58-311 with the
  * cp_async/ld_matrix pipeline of CpAsyncOpToLLVM.cpp and LdMatrixOpToLLVM.cpp.
  * result[M,N] = lhs[M,K]·rhs[K,N] (+ acc[M,N]), fp32 accumulate, one final cast to result->dtype.
- * Operand layouts come from the descriptor strides (row- or column-major, either operand).
+ * Operand layouts come from the descriptor strides (row- or column-major, either operand).  A column-major result is
+ * computed as the transposed problem (result^T = rhs^T . lhs^T, cfg->tile_m and tile_n exchanged with it): the same bits,
+ * through the row-major store path.
  * acc may be NULL (zero).  cfg may be NULL. */
 int kapy_matmul(const kapy_global *lhs, const kapy_global *rhs, const kapy_global *acc, const kapy_global *result,
                 const kapy_matmul_cfg *cfg, void *stream);

@@ -498,7 +498,7 @@ int kapy_smem_barriers(const kapy_smem_op *ops, int32_t n_ops, const kapy_smem_a
  * `args` follow the function's signature: a device pointer (with the size of its allocation in bytes, 0 =
  * unknown, which mk_global is checked against) for !kapy.ptr<1>, an i32 otherwise.  A sub-view that leaves
  * its parent is an error.  func_name NULL = the first function of the module.  The first call on a device allocates
- * a 256 MiB arena for shared-memory and register tensors, which the library keeps until the process ends; calls take
+ * a 2 GiB arena for shared-memory and register tensors (about 360 four-warp program instances advance in step in it), which the library keeps until the process ends; calls take
  * turns at it, and a call synchronises `stream` before it returns: it is a way to run the reference's programs against
  * this library, not a fast path.
  * The device calls of a run that succeeded are kept (the last 16 runs): a later call with the same text, function name,

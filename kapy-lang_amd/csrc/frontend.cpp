@@ -561,7 +561,7 @@ struct Value {
 // take the rest and die with their program instance.
 // A call runs its program instances in groups (all programs of a group and all their warps in step): every program of a group
 // has its own shared part, the group one region for the register tensors of calls merged over instances, every warp its share.
-constexpr size_t kSharedArena = size_t(256) << 10, kArena = size_t(256) << 20, kMergedArena = size_t(64) << 20, kMinShare = size_t(1) << 20;
+constexpr size_t kSharedArena = size_t(256) << 10, kArena = size_t(2048) << 20, kMergedArena = size_t(512) << 20, kMinShare = size_t(1) << 20;
 
 // A device call of a run, as recorded for the plan cache: which entry point, and copies of everything it was given.
 struct PlannedCall {
@@ -666,10 +666,17 @@ struct Interp {
   }
   // before a store into `dst`: every deferred value that still has to read that memory is computed now
   // (the values of every warp: another warp's deferred load stands earlier in program order than this store, too)
+  // (with a thousand warps in step, a store per warp that looks through every warp's values is a million looks: a scan that
+  // met no deferred value at all holds until the next one is made - copies of values cannot make one out of none)
+  int64_t lazy_made = 0, none_lazy_at = -1;
   int settle_readers(const Op &op, const kapy_global &dst) {
+    if (none_lazy_at == lazy_made) return KAPY_OK;
+    bool any_lazy = false;
     auto settle = [&](std::map<std::string, Value> &values) {
       for (auto &kv : values)
-        if (kv.second.kind == Value::kTensor && kv.second.lazy && reads_under(kv.second.lazy, dst)) {
+        if (kv.second.kind == Value::kTensor && kv.second.lazy) {
+          any_lazy = true;
+          if (!reads_under(kv.second.lazy, dst)) continue;
           int rc = force(op, kv.second);
           if (rc != KAPY_OK) return rc;
         }
@@ -678,6 +685,7 @@ struct Interp {
     int rc = settle(env);
     for (size_t w = 0; rc == KAPY_OK && w < warps.size(); ++w)
       if ((int)w != current) rc = settle(warps[w].env);
+    if (rc == KAPY_OK && !any_lazy) none_lazy_at = lazy_made;
     return rc;
   }
   // the operand as an expression: deferred tensors as they are, computed ones as leaves
@@ -844,6 +852,7 @@ struct Interp {
     Value r;
     r.kind = Value::kTensor;
     r.lazy = e;
+    ++lazy_made;
     memset(&r.g, 0, sizeof r.g);
     if (kapy_mk_global(&r.g, arena, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 16) != KAPY_OK)
       return fail_op(op, kapy_last_error());
@@ -1401,6 +1410,7 @@ struct Interp {
         e->global_leaf = true;
         r.kind = Value::kTensor;
         r.lazy = e;
+        ++lazy_made;
         memset(&r.g, 0, sizeof r.g);
         int rc = lib(op, kapy_mk_global(&r.g, arena, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 16));
         if (rc) return rc;
@@ -1495,6 +1505,7 @@ struct Interp {
           if (fits(e)) {
             r.kind = Value::kTensor;
             r.lazy = e;
+            ++lazy_made;
             memset(&r.g, 0, sizeof r.g);
             int rc = lib(op, kapy_mk_global(&r.g, arena, 0, (int32_t)ty.shape[0], (int32_t)ty.shape[1], (int32_t)ty.shape[1], 1, ty.dtype, 16));
             if (rc) return rc;

@@ -335,7 +335,7 @@ typedef enum kapy_matmul_accumulate { KAPY_ACCUMULATE_F32 = 0, KAPY_ACCUMULATE_E
 /* Workspace size that lets the library split K for an [m x n] result whichever way it chooses. */
 int64_t kapy_matmul_workspace_bytes(int64_t m, int64_t n);
 /* Workspace size with which a LARGE 16-bit problem (at least 6144 rows for a row-major rhs - unless the lhs is row-major
- * too and the sizes are whole 256 x 256 x 64 tiles, which a kernel of its own multiplies in place -, at least 6144 columns
+ * too and K a multiple of 64, which a kernel of its own multiplies in place -, at least 6144 columns
  * for a column-major lhs, at least 2048 of the other, K at least 1024, all multiples of 8) is multiplied by first turning that
  * operand into the workspace (behind the 16 KiB of counters, which stay zero) with the transposing copy and then running
  * the K-contiguous kernel on 256 x 256 tiles: 1.15 - 1.2 x the rate of the kernel that reads such operands in place on

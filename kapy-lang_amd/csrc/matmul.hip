@@ -1363,9 +1363,9 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
     // (measured, bf16, in place -> turned: 8192^3 1237 -> 1485 TFLOP/s, 8192 x 2048 x 4096 1130 -> 1317, 8192 x 8192 x 1024 924 -> 1106;
     // 4096^3 and 2048 x 8192 x 4096 the same either way; 2048^2 x K slower by a third: the turn is paid once per operand and
     // earned back over the rows - or, for a turned lhs, the columns - that use it)
-    // (a row-major rhs beside a row-major lhs in whole 256 x 256 x 64 tiles is read in place by the 256-wide kernel of
+    // (a row-major rhs beside a row-major lhs with K in whole tiles of 64 is read in place by the 256-wide kernel of
     // matmul_nn256.hip, faster than turn and product together: 8192^3 bf16 0.683 ms against 0.727)
-    const bool wide_in_place = b_turn && !a_turn && a_kc && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (M / 256) * (N / 256) * 100 >= (int64_t)device_cus() * 55 &&
+    const bool wide_in_place = b_turn && !a_turn && a_kc && N % 8 == 0 && K % 64 == 0 && ((M + 255) / 256) * ((N + 255) / 256) * 100 >= (int64_t)device_cus() * 55 &&
                                c.rmode == KAPY_RN;
     if (!wide_in_place && (a_turn || b_turn) && (a_turn || a_kc) && (b_turn || b_kc) && (!b_turn || M >= 6144) && (!a_turn || N >= 6144) && M >= 2048 && N >= 2048 && K >= 1024 &&
         M % 8 == 0 && N % 8 == 0 && K % 8 == 0 &&
@@ -1497,7 +1497,7 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
     // form, half the LDS bytes per flop of the 128-wide tiles below.
     static const bool wide = !(getenv("KAPY_NN256") && getenv("KAPY_NN256")[0] == '0');
     if (wide && form == 0 && !c.tile_m && !c.tile_n && !c.tile_k && !c.stages && !c.waves && c.split_k <= 1 && !p.rz && nn256_serves(p) && packed_epilogue(p) &&
-        (int64_t)(p.M / 256) * (p.N / 256) * 100 >= (int64_t)device_cus() * 55)
+        (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 >= (int64_t)device_cus() * 55)
       return launch_nn256(p, bf16, s);
     for (const NnVariant &v : kNn) {
       if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;

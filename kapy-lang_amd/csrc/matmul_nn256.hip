@@ -67,7 +67,8 @@ __global__ __launch_bounds__(256) void nn256_kernel(GemmParams p) {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (void *)(((uint64_t)hi << 32) | lo);
   };
-  // (the descriptors end where the operands end; the host hands over whole tiles, so nothing of a tile lies beyond)
+  // (the descriptors end where the operands end: what a tile has beyond the last row of the lhs, or beyond the last k-row's
+  // N columns of the rhs, reads as zeros)
   const int64_t a_left = ((int64_t)(p.M - m0 - 1) * p.a_sm + p.K) * 2, b_left = ((int64_t)(p.K - 1) * p.b_sk + (p.N - n0)) * 2;
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.a + (int64_t)m0 * p.a_sm * 2), 0,
                                                                           __builtin_amdgcn_readfirstlane((int)(a_left < 0x7fffffff ? a_left : 0x7fffffff)), 0x00020000);
@@ -203,16 +204,19 @@ __global__ __launch_bounds__(256) void nn256_kernel(GemmParams p) {
 }  // namespace
 
 // Whether nn256_kernel serves the problem (the caller has checked the strip epilogue's own conditions): both operands with
-// contiguous, 16-byte aligned rows of whole 16-byte pieces and whole tiles.
+// contiguous, 16-byte aligned rows of whole 16-byte pieces and whole K-tiles.  Tiles may hang over the last rows and columns:
+// the lhs descriptor ends with the operand's last row (rows beyond it read as zeros), rhs columns beyond N are whatever
+// follows in memory up to the end of the last k-row (zeros beyond) and only reach result columns that are never stored, and
+// the strip stores are bounded by the result's extents.
 bool nn256_serves(const GemmParams &p) {
-  return p.a_sk == 1 && p.b_sn == 1 && p.M % kBM == 0 && p.N % kBN == 0 && p.K % kBK == 0 && p.K >= 2 * kBK && p.a_sm % 8 == 0 && p.b_sk % 8 == 0 &&
+  return p.a_sk == 1 && p.b_sn == 1 && p.M > 0 && p.N > 0 && p.N % 8 == 0 && p.K % kBK == 0 && p.K >= 2 * kBK && p.a_sm % 8 == 0 && p.b_sk % 8 == 0 &&
          ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.a_sm > 0 && p.b_sk > 0 && p.a_sm * 2 * kBM < (int64_t(1) << 31) &&
          (int64_t)p.K * p.b_sk * 2 < (int64_t(1) << 31);
 }
 
 int launch_nn256(GemmParams p, bool bf16, hipStream_t s) {
-  p.tiles_m = p.M / kBM;
-  p.tiles_n = p.N / kBN;
+  p.tiles_m = (p.M + kBM - 1) / kBM;
+  p.tiles_n = (p.N + kBN - 1) / kBN;
   p.split_k = 1;
   // Before the first launch on a device: the runtime must give the kernel the 128 KiB of LDS its loads address.
   static int checked[64];  // 0 not asked, 1 fine, -1 refused (a race between two first calls only repeats the query)

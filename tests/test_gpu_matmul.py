@@ -356,19 +356,21 @@ def test_transposing_read_kernel_with_a_partial_last_k_tile(ko, dt, a_rm, b_rm):
         assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL, (M, N, K)
 
 
+@pytest.mark.parametrize("M,N", [(3072, 3072), (3001, 3016)])   # (the second: tiles that hang over the last rows and columns)
 @pytest.mark.parametrize("dt,acc_dt,out_dt", [("BF16", None, "BF16"), ("F16", None, "F16"), ("BF16", "F32", "F32"), ("F16", "F16", "F16")])
-def test_large_row_major_operands_on_256_wide_tiles(ko, monkeypatch, dt, acc_dt, out_dt):
+def test_large_row_major_operands_on_256_wide_tiles(ko, monkeypatch, dt, acc_dt, out_dt, M, N):
     """Row-major x row-major with at least 0.55 tiles of 256 x 256 per CU: the 256-wide kernel that stages the rhs as it lies and
     transposes it on the way out of LDS.  Sampled blocks against the checker (spread over the tile: every wavefront's part and
     both column halves of the rhs image), nothing written past the result, and the bits of the 128-wide kernel's result where no
     accumulator order differs - both sum K in ascending slices of 32 from zero - i.e. everywhere."""
     dt, out_dt = getattr(ko, dt), getattr(ko, out_dt)
     acc_dt = getattr(ko, acc_dt) if acc_dt else None
-    M, N, K = 3072, 3072, 192
+    K = 192
     ob = 4 if out_dt == ko.F32 else 2
     a, b = ko.fill_normal(M * K, dt, 51, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 51, 1, 0.0, 0.5)
     acc = ko.fill_normal(M * N, acc_dt, 51, 2, 0.0, 0.5) if acc_dt is not None else None
-    da, db = to_dev(a), to_dev(b)
+    poison = np.full(8192, 0x7e00 if dt == ko.F16 else 0x7fc0, np.uint16)       # NaNs behind each operand
+    da, db = to_dev(np.concatenate([a, poison])), to_dev(np.concatenate([b, poison]))
     dacc = to_dev(acc) if acc is not None else None
     ga, gb = dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, N, 1, dt)
     gacc = dglobal(dacc, M, N, N, 1, acc_dt) if acc is not None else None
@@ -386,6 +388,8 @@ def test_large_row_major_operands_on_256_wide_tiles(ko, monkeypatch, dt, acc_dt,
     goacc = ko.mk_global(acc, M, N, N, 1, acc_dt) if acc is not None else None
     for t in range(8):
         r0, c0 = (t * 331 + 37 * (t % 4) * 16) % (M - 64), (t * 577 + 128 * (t % 2)) % (N - 64)
+        if t == 7:
+            r0, c0 = M - 64, N - 64   # (the corner of the last tile)
         want = np.zeros((64, 64), _np_store(out_dt))
         assert ko.lib().ko_matmul(C.byref(ko.sv_global(goa, r0, r0 + 64, 0, K)), C.byref(ko.sv_global(gob, 0, K, c0, c0 + 64)),
                                   C.byref(ko.sv_global(goacc, r0, r0 + 64, c0, c0 + 64)) if goacc is not None else None,

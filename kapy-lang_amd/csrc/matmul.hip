@@ -96,14 +96,14 @@ __global__ __launch_bounds__(64 * WM * WN) void tn_kernel(GemmParams p) {
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
     // (the 128-wide builds without bounded loads fetch the operand's last row in place of rows past its end: results nobody
     // stores; the 256-wide ones are only given whole tiles)
-    if constexpr (STAGES != kRing25 && BM == 128) row = min(row, (uint32_t)max(p.M - 1 - tm * BM, 0));
+    if constexpr (STAGES != kRing25 && BM <= 128) row = min(row, (uint32_t)max(p.M - 1 - tm * BM, 0));
     a_goff[i] = (uint32_t)((row * p.a_sm + chunk * (16 / EB)) * EB);
   }
 #pragma unroll
   for (int i = 0; i < C::kLoadsBPerWave; ++i) {
     uint32_t row, chunk;
     L::locate((uint32_t)(wave + i * C::kWaves) * 1024u + lane * 16u, row, chunk);
-    if constexpr (STAGES != kRing25 && BN == 128) row = min(row, (uint32_t)max(p.N - 1 - tn * BN, 0));
+    if constexpr (STAGES != kRing25 && BN <= 128) row = min(row, (uint32_t)max(p.N - 1 - tn * BN, 0));
     b_goff[i] = (uint32_t)((row * p.b_sn + chunk * (16 / EB)) * EB);
   }
   const char *a_tile = p.a + (int64_t)m0 * p.a_sm * EB;
@@ -1116,7 +1116,7 @@ int launch_tn(const GemmParams &p, hipStream_t s) {
   // a result that ends inside a 16-byte piece of a row takes the bounds-checked element stores
   // (tiles that hang over the edge: the ring builds' loads are bounded, the others fetch the last row again; the strip stores
   // are bounded for all of them)
-  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || ((STAGES == kRing25 || BM == 128) && p.N % 8 == 0);
+  const bool whole_tiles = (p.M % BM == 0 && p.N % BN == 0) || ((STAGES == kRing25 || BM <= 128) && p.N % 8 == 0);
   const bool packed = packed_epilogue(p) && whole_tiles;
   if (host_has_tail(p)) {
     // a fused elementwise tail: the ring kernels on the 16x16 instruction have builds with it in the packed epilogue,
@@ -1219,6 +1219,7 @@ const TnVariant kTnVariants[] = {
     KAPY_TN16(256, 256, 64, 2, 2, kRing25), KAPY_TN16(256, 256, 64, 2, 2, 2),
     KAPY_TN(256, 256, 64, 2, 2, kRing25), KAPY_TN(256, 256, 64, 2, 2, 2), KAPY_TN(256, 256, 32, 2, 2, 4), KAPY_TN16(128, 128, 64, 2, 2, kRing25),
     KAPY_TN(128, 128, 64, 2, 2, 2), KAPY_TN(128, 128, 32, 2, 2, 4), KAPY_TN(128, 128, 64, 2, 2, 4),
+    KAPY_TN(128, 64, 64, 2, 2, 4), KAPY_TN(64, 64, 128, 2, 2, 4),
 };
 
 int operand_mode(int64_t s_row, int64_t s_k) { return s_k == 1 ? kKContig : (s_row == 1 ? kRowContig : kStrided); }
@@ -1465,6 +1466,16 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
         // Tiles for at most half the CUs and K not split: a workgroup alone on its CU waits for the ring's 2.5 tiles of loads.
         // The four-stage build on the 32-row instruction keeps three tiles in flight: bf16 N = K = 8192, 128 / 256 rows
         // 54 / 55 -> 48 / 52 us (level at 384 rows, behind from 512; the same depth on the 16-row instruction: 71 us).
+        // Fewer still: smaller tiles put every CU to work on the operand streams.  bf16 N = K = 8192, 64 / 128 rows on
+        // 64 x 64 x 128 tiles 48 / 47 -> 30 / 30 us, 256 rows on 128 x 64 x 64 tiles 47.5 -> 43; from 384 rows on (more small
+        // tiles than CUs) they lose to the 128 x 128 ring.
+        if (free_choice && p.split_k <= 1 && !host_has_tail(p) && p.N % 8 == 0) {
+          const int64_t n64 = (p.N + 63) / 64;
+          if (p.K % 128 == 0 && (int64_t)((p.M + 63) / 64) * n64 <= device_cus())
+            return bf16 ? launch_tn<Bf16, 64, 64, 128, 2, 2, 4>(p, s) : launch_tn<F16, 64, 64, 128, 2, 2, 4>(p, s);
+          if (p.K % 64 == 0 && (int64_t)((p.M + 127) / 128) * n64 <= device_cus())
+            return bf16 ? launch_tn<Bf16, 128, 64, 64, 2, 2, 4>(p, s) : launch_tn<F16, 128, 64, 64, 2, 2, 4>(p, s);
+        }
         if (free_choice && p.split_k <= 1 && !host_has_tail(p) && p.K % 64 == 0 && p.N % 8 == 0 &&
             (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * 2 <= device_cus())
           return bf16 ? launch_tn<Bf16, 128, 128, 64, 2, 2, 4>(p, s) : launch_tn<F16, 128, 128, 64, 2, 2, 4>(p, s);

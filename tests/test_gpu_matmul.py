@@ -83,7 +83,8 @@ def test_all_operand_layouts_and_ragged_shapes(ko, dt, a_rm, b_rm):
 
 MFMA16, MFMA32 = 17, 16   # KAPY_MFMA_16X16X32_16B, KAPY_MFMA_32X32X16_16B
 TN_VARIANTS = [((256, 256, 64), 25, MFMA16), ((256, 256, 64), 2, MFMA16), ((256, 256, 64), 25, MFMA32), ((256, 256, 64), 2, MFMA32),
-               ((256, 256, 32), 4, MFMA32), ((128, 128, 64), 25, MFMA16), ((128, 128, 64), 2, MFMA32), ((128, 128, 32), 4, MFMA32)]
+               ((256, 256, 32), 4, MFMA32), ((128, 128, 64), 25, MFMA16), ((128, 128, 64), 2, MFMA32), ((128, 128, 32), 4, MFMA32),
+               ((128, 128, 64), 4, MFMA32), ((128, 64, 64), 4, MFMA32), ((64, 64, 128), 4, MFMA32)]
 
 
 @pytest.mark.parametrize("tile,stages,impl_way", TN_VARIANTS)
@@ -97,6 +98,24 @@ def test_tn_roofline_kernel_every_variant(ko, tile, stages, impl_way):
             assert _frob(ko, got, want, dt) <= FROB_TOL, (M, N, K)
     got32, want32 = _run(ko, kh.BF16, 2 * bm, 2 * bn, 8 * bk, True, False, out_dtype=kh.F32, seed=5, tile=tile, stages=stages, impl_way=impl_way)
     assert _frob(ko, got32, want32, kh.F32) <= 1e-5
+
+
+@pytest.mark.parametrize("dt", [kh.BF16, kh.F16])
+def test_few_tiles_take_smaller_tiles(ko, dt):
+    """K-contiguous operands whose 64 x 64 (or 128 x 64) tiles number no more than the CUs: the four-stage builds on those tiles,
+    with tiles that hang over the last rows and columns, K of one to many K-tiles, NaNs behind the operands."""
+    for (M, N, K) in ((100, 520, 512), (192, 1024, 384), (256, 2048, 320), (130, 264, 192), (1, 64, 128), (64, 4096, 1024), (250, 72, 64)):
+        a, b = ko.fill_normal(M * K, dt, 17, 0, 0.0, 0.5), ko.fill_normal(K * N, dt, 17, 1, 0.0, 0.5)
+        want = np.zeros(M * N, np.uint16)
+        assert ko.lib().ko_matmul(C.byref(ko.mk_global(a, M, K, K, 1, dt)), C.byref(ko.mk_global(b, K, N, 1, K, dt)), None,
+                                  C.byref(ko.mk_global(want, M, N, N, 1, dt)), kh.RN) == 0
+        poison = np.full(4096, 0x7e00 if dt == kh.F16 else 0x7fc0, np.uint16)
+        da, db, dd = to_dev(np.concatenate([a, poison])), to_dev(np.concatenate([b, poison])), dev_zeros(M * N + 256, 2, fill=0x1234)
+        kh.matmul(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd, M, N, N, 1, dt))
+        sync()
+        got = to_host(dd, np.uint16)
+        assert np.all(got[M * N:] == 0x1234), (M, N, K)
+        assert _frob(ko, got[:M * N], want, dt) <= FROB_TOL, (M, N, K)
 
 
 def test_tn_default_choice(ko):

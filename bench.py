@@ -989,7 +989,7 @@ def bench_ceilings(kh, steps, warmup, cpu):
 
 
 WORKLOADS = ["gelu", "add", "expr", "expr_compiled", "swiglu", "copy", "reduce", "reduce_cols", "softmax", "softmax_cols", "causal_softmax", "layernorm", "l2norm_compiled", "gelu_transposed",
-             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m256", "f8_m4096", "mlir_fixtures", "ceilings"]
+             "transpose", "permute", "gemm_bf16", "gemm_bf16_gelu", "gemm_bf16_nn", "gemm_bf16_nn_turned", "gemm_bf16_m128", "gemm_f16", "gemm_f16_splitk", "gemm_f16_graph", "f8_m16", "f8_m64", "f8_m128", "f8_m128_splitk", "f8_m256", "f8_m4096", "mlir_fixtures", "ceilings"]
 
 
 # ---------------------------------------------------------------- HBM traffic summary from the profiler's counter files
@@ -1219,6 +1219,7 @@ def main():
         "mlir_fixtures": lambda s, w: bench_mlir(kh, s, w, cpu),
         "gemm_bf16_nn": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, False, "gemm bf16 8192^3, both operands row-major, the rhs read in place by transposing LDS reads (256 x 256 tiles)", "nn256_kernel", key="gemm_bf16_nn", whole=False),
         "gemm_bf16_nn_turned": lambda s, w: bench_gemm(kh, s, w, False, 8192, 8192, 8192, kh.BF16, True, "gemm bf16 8192^3, lhs column-major, rhs column-major, workspace given: the lhs is turned K-contiguous first (time and rate include the turn)", "transpose_lds_kernel + tn_kernel", key="gemm_bf16_nn_turned", workspace=True, whole=False, a_col_major=True),
+        "gemm_bf16_m128": lambda s, w: bench_gemm(kh, s, w, False, 128, 8192, 8192, kh.BF16, True, "gemm bf16 128 x 8192 x 8192, rhs column-major: one 64 x 64 x 128 tile per CU (a weight-streaming shape: its 138 MB in 31 us are 4.4 TB/s of HBM reads, whatever the matrix-pipe fraction says)", "tn_kernel, 64 x 64 x 128 tiles, four stages", key="gemm_bf16_m128"),
         "gemm_f16": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles", "nn_kernel", tile=(128, 128, 32), gen="uniform", key="gemm_f16"),
         "gemm_f16_graph": lambda s, w: bench_gemm(kh, s, w, cpu, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3, 20 launches replayed from a HIP graph (per launch)", "nn_kernel", tile=(128, 128, 32), graph_of=20, gen="uniform", key="gemm_f16_graph"),
         "gemm_f16_splitk": lambda s, w: bench_gemm(kh, s, w, False, 1024, 1024, 1024, kh.F16, False, "C1 gemm fp16 1024^3 row-major 128x128x32 tiles, K split across workgroups (workspace given)", "nn_kernel, split K", tile=(128, 128, 32), gen="uniform", workspace=True, key="gemm_f16_splitk"),

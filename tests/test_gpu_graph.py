@@ -90,6 +90,54 @@ def test_every_kernel_family_replays_from_a_graph():
         assert int((captured["soft"] != 0x1111).sum()) > 0
 
 
+def test_matmul_layouts_and_tile_choices_replay_from_a_graph():
+    """The matmul kernels behind the layout and tile rules - row-major x row-major on 256-wide tiles, the same with a fused tail, a
+    column-major result (the transposed problem), few tiles on 64 x 64 and 128 x 64 tiles - recorded once and replayed with fresh
+    operands: every replay has the bits of the eager calls."""
+    M, N, K = 3072, 3072, 128
+    i16 = lambda count: torch.zeros(count, dtype=torch.int16, device="cuda")
+    a, b, bias = i16(M * K), i16(K * N), i16(N)
+
+    def calls(out):
+        ga, gb = dglobal(a, M, K, K, 1, kh.BF16), dglobal(b, K, N, N, 1, kh.BF16)
+        kh.matmul(ga, gb, dglobal(out["wide"], M, N, N, 1, kh.BF16))
+        kh.matmul_fused(ga, gb, dglobal(out["wide_tail"], M, N, N, 1, kh.BF16), bias=dglobal(bias, 1, N, N, 1, kh.BF16), alpha=0.5, act=kh.EW_GELU_TANH)
+        # K-contiguous operands cut from the same buffers: [256 x 1024] . [1024 x 384]^T-stored, column-major result
+        kh.matmul(dglobal(a, 256, 1024, 1024, 1, kh.BF16), dglobal(b, 1024, 384, 1, 1024, kh.BF16), dglobal(out["col"], 256, 384, 1, 256, kh.BF16))
+        kh.matmul(dglobal(a, 64, 1024, 1024, 1, kh.BF16), dglobal(b, 1024, 384, 1, 1024, kh.BF16), dglobal(out["t64"], 64, 384, 384, 1, kh.BF16))
+        kh.matmul(dglobal(a, 250, 320, 320, 1, kh.BF16), dglobal(b, 320, 1024, 1, 320, kh.BF16), dglobal(out["t128x64"], 250, 1024, 1024, 1, kh.BF16))
+
+    outputs = lambda: {"wide": i16(M * N), "wide_tail": i16(M * N), "col": i16(256 * 384), "t64": i16(64 * 384), "t128x64": i16(250 * 1024)}
+
+    def refill(seed):
+        gen = torch.Generator(device="cuda").manual_seed(seed)
+        a.copy_((0.1 * torch.randn(M * K, generator=gen, device="cuda")).bfloat16().view(torch.int16))
+        b.copy_((0.1 * torch.randn(K * N, generator=gen, device="cuda")).bfloat16().view(torch.int16))
+        bias.copy_(torch.randn(N, generator=gen, device="cuda").bfloat16().view(torch.int16))
+
+    captured, eager = outputs(), outputs()
+    refill(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):           # one eager pass first: attribute queries happen outside the capture
+        calls(eager)
+    torch.cuda.current_stream().wait_stream(side)
+    sync()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        calls(captured)
+    for seed in (2, 3, 4):
+        refill(seed)
+        for t in captured.values():
+            t.fill_(0x1111)
+        graph.replay()
+        calls(eager)
+        sync()
+        for name in captured:
+            assert torch.equal(captured[name], eager[name]), "replay with seed %d differs from the eager call in %s" % (seed, name)
+            assert int((captured[name] != 0x1111).sum()) > captured[name].numel() // 2
+
+
 def test_nothing_is_compiled_or_loaded_while_a_stream_is_captured():
     """A row program the row machine refuses (a width that is no multiple of 8) is normally served by compiling a kernel on its
     first call.  Inside a capture that must not happen (compiling and loading a module are not stream work): the call is refused

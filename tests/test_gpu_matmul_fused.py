@@ -116,6 +116,32 @@ def test_the_tail_on_256_wide_tiles_of_row_major_operands(ko, dt, bias_dt, alpha
         assert rel <= 1e-3, (t, rel)
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_a_column_major_result_carries_the_tail(ko, with_bias):
+    """Scale and activation commute with the transposition, so a column-major result without a bias is the transposed problem
+    (bit for bit the row-major result); with a bias row the call stays as it is and goes through the element stores."""
+    dt, M, N, K = kh.BF16, 320, 264, 192
+    a, b = ko.fill_normal(M * K, dt, 7, 0, 0.0, 0.25), ko.fill_normal(K * N, dt, 7, 1, 0.0, 0.25)
+    bias = ko.fill_normal(N, dt, 7, 2, 0.0, 1.0)   # (the operands of _case)
+    da, db, dbias = to_dev(a), to_dev(b), to_dev(bias)
+    gb = dglobal(dbias, 1, N, N, 1, dt) if with_bias else None
+    d_col, d_row = dev_zeros(M * N + 64, 2, fill=0x1234), dev_zeros(M * N, 2)
+    for dd, strides in ((d_col, (1, M)), (d_row, (N, 1))):
+        kh.matmul_fused(dglobal(da, M, K, K, 1, dt), dglobal(db, K, N, 1, K, dt), dglobal(dd, M, N, *strides, dt), bias=gb, alpha=0.5, act=kh.EW_GELU_TANH)
+    sync()
+    col = to_host(d_col, np.uint16)
+    assert np.all(col[M * N:] == 0x1234)
+    col_as_rows = np.ascontiguousarray(col[:M * N].reshape(N, M).T).ravel()
+    row = to_host(d_row, np.uint16)
+    assert np.all(np.isfinite(ko.decode(col_as_rows, dt)))
+    if with_bias:
+        assert ulp_diff_f16(col_as_rows, row).max() <= 2
+    else:
+        assert np.array_equal(col_as_rows, row)
+    got_row, want = _case(ko, dt, M, N, K, False, dt if with_bias else None, 0.5, kh.EW_GELU_TANH)
+    assert np.array_equal(got_row, row)
+
+
 def test_parts_of_the_tail_alone_and_relu_really_clamps(ko):
     _case(ko, kh.BF16, 256, 256, 128, False, None, 0.125, -1)                  # scale only
     _case(ko, kh.BF16, 256, 256, 128, False, kh.BF16, 1.0, -1)                 # bias only

@@ -282,9 +282,53 @@ static int run_gpu_large_tile() {
   return 0;
 }
 
+// The 256-wide kernel for row-major x row-major operands (128 KiB of LDS, declared statically) from a process that never
+// loaded torch: the library picks it from 0.55 tiles of 256 x 256 per CU; 64 sampled rows against a double-precision sum.
+static int run_gpu_row_major_wide() {
+  const int M = 3072, N = 3072, K = 128;
+  std::vector<uint16_t> a((size_t)M * K), w((size_t)K * N), c((size_t)M * N);
+  srand(13);
+  auto rnd = [] { return (float)(rand() % 65536) / 65536.f - 0.5f; };
+  for (auto &v : a) v = f2b(rnd());
+  for (auto &v : w) v = f2b(rnd());
+  uint16_t *da, *dw, *dc;
+  HIP_OK(hipMalloc((void **)&da, a.size() * 2)); HIP_OK(hipMalloc((void **)&dw, w.size() * 2)); HIP_OK(hipMalloc((void **)&dc, c.size() * 2));
+  HIP_OK(hipMemcpy(da, a.data(), a.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(dw, w.data(), w.size() * 2, hipMemcpyHostToDevice));
+  HIP_OK(hipMemset(dc, 0, c.size() * 2));
+  kapy_global ga, gw, gc;
+  EXPECT(kapy_mk_global(&ga, da, 0, M, K, K, 1, KAPY_BF16, 16) == KAPY_OK);
+  EXPECT(kapy_mk_global(&gw, dw, 0, K, N, N, 1, KAPY_BF16, 16) == KAPY_OK);
+  EXPECT(kapy_mk_global(&gc, dc, 0, M, N, N, 1, KAPY_BF16, 16) == KAPY_OK);
+  printf("launching the row-major x row-major matmul (M = N = %d, K = %d)\n", M, K);
+  fflush(stdout);
+  const int rc = kapy_matmul(&ga, &gw, nullptr, &gc, nullptr, nullptr);
+  if (rc != KAPY_OK) {
+    printf("FAILED: kapy status %d: %s\n", rc, kapy_last_error());
+    return 1;
+  }
+  HIP_OK(hipDeviceSynchronize());
+  HIP_OK(hipMemcpy(c.data(), dc, c.size() * 2, hipMemcpyDeviceToHost));
+  double err2 = 0, ref2 = 0;
+  for (int t = 0; t < 64; ++t) {
+    const int i = (t * 331 + 7) % M;
+    for (int j = 0; j < N; ++j) {
+      double s = 0;
+      for (int k = 0; k < K; ++k) s += (double)b2f(a[(size_t)i * K + k]) * b2f(w[(size_t)k * N + j]);
+      const double got = b2f(c[(size_t)i * N + j]);
+      err2 += (got - s) * (got - s);
+      ref2 += s * s;
+    }
+  }
+  EXPECT(ref2 > 0 && sqrt(err2 / ref2) <= 4e-3);
+  printf("builder gpu row-major wide ok\n");
+  return 0;
+}
+
 int main(int argc, char **argv) {
   try {
     if (argc > 1 && std::string(argv[1]) == "gpu256") return run_gpu_large_tile();
+    if (argc > 1 && std::string(argv[1]) == "gpunn256") return run_gpu_row_major_wide();
     return argc > 1 && std::string(argv[1]) == "gpu" ? run_gpu() : run_cpu();
   } catch (const kapy::Error &e) {
     printf("FAILED: kapy status %d: %s\n", e.status, e.what());

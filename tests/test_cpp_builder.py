@@ -33,3 +33,11 @@ def test_the_full_lds_ring_kernel_runs_in_a_process_without_torch():
     out = subprocess.run([_binary(), "gpu256"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0 and "builder gpu large tile ok" in out.stdout, out.stdout + out.stderr
 
+
+
+@pytest.mark.gpu
+def test_the_wide_row_major_kernel_runs_in_a_process_without_torch():
+    """Row-major x row-major on 256-wide tiles (128 KiB of statically declared LDS, the runtime's figures checked before the first
+    launch), picked by the library's own rule, from the C++ process."""
+    out = subprocess.run([_binary(), "gpunn256"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "builder gpu row-major wide ok" in out.stdout, out.stdout + out.stderr

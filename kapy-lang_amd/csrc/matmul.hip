@@ -1507,8 +1507,10 @@ int matmul_16bit(const kapy_global *lhs, const kapy_global *rhs, const kapy_glob
     // Row-major x row-major with enough 256 x 256 tiles for the device (the rule of the K-contiguous kernel): the 256-wide
     // form, half the LDS bytes per flop of the 128-wide tiles below.
     static const bool wide = !(getenv("KAPY_NN256") && getenv("KAPY_NN256")[0] == '0');
+    // (KAPY_NN256_FROM: the least number of 256 x 256 tiles per 100 CUs, for measurements)
+    static const int wide_from_pct = getenv("KAPY_NN256_FROM") ? atoi(getenv("KAPY_NN256_FROM")) : 55;
     if (wide && form == 0 && !c.tile_m && !c.tile_n && !c.tile_k && !c.stages && !c.waves && c.split_k <= 1 && !p.rz && nn256_serves(p) && packed_epilogue(p) &&
-        (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 >= (int64_t)device_cus() * 55)
+        (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * 100 >= (int64_t)device_cus() * wide_from_pct)
       return launch_nn256(p, bf16, s);
     for (const NnVariant &v : kNn) {
       if ((c.tile_k && c.tile_k != v.bk) || (c.stages && c.stages != v.stages) || p.K % v.bk) continue;
